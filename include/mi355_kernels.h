@@ -1,0 +1,170 @@
+/*
+ * C ABI of the MI355X (gfx950) kernel library for llama.cpp's quantized-inference hot
+ * path.  Plain pointers and sizes only.  All data pointers are DEVICE addresses unless a
+ * parameter says "host".  `stream` is a hipStream_t passed as void* (NULL = default
+ * stream).  Every entry point returns 0 on success or a negative MI355_ERR_* code and
+ * launches asynchronously on `stream`; nothing here allocates device memory unless its
+ * comment says so.
+ *
+ * Each entry point names the reference function it stands in for (paths relative to the
+ * llama.cpp tree).  Element types use the reference's enum values
+ * (ggml/include/ggml.h:351-392): F32 0, F16 1, Q4_0 2, Q8_0 8, Q8_1 9, Q4_K 12, Q6_K 14, I32 26.
+ */
+#ifndef MI355_KERNELS_H
+#define MI355_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_OK            0
+#define MI355_ERR_ARG      -1   /* unsupported type, shape or alignment */
+#define MI355_ERR_HIP      -2   /* a HIP runtime call failed; see mi355_last_error() */
+#define MI355_ERR_WORKSPACE -3  /* workspace too small */
+
+enum mi355_type {
+    MI355_F32 = 0, MI355_F16 = 1, MI355_Q4_0 = 2, MI355_Q8_0 = 8, MI355_Q8_1 = 9,
+    MI355_Q4_K = 12, MI355_Q6_K = 14, MI355_I32 = 26,
+};
+
+/* Library / device ------------------------------------------------------------------ */
+
+/* Version of this ABI (bumped on incompatible change). */
+int mi355_abi_version(void);
+/* Text of the last error on the calling thread ("" if none). */
+const char *mi355_last_error(void);
+/* 1 if `device` is a gfx950 GPU this library can run on, 0 if not, <0 on HIP error.
+ * Counterpart of a backend's score function (ggml/src/ggml-backend-impl.h:212-214). */
+int mi355_device_supported(int device);
+
+/* Weight storage -------------------------------------------------------------------- *
+ * Quantized weight rows are kept in HBM in a per-row "device layout" that makes every
+ * load a 16-byte aligned, coalesced access:
+ *   Q4_K : unchanged (144-byte super-blocks are already 16-byte multiples)
+ *   Q4_0 : [nb x 16 B nibbles][nb x fp16 d]
+ *   Q8_0 : [nb x 32 B int8   ][nb x fp16 d]
+ *   Q6_K : [nb x 128 B ql][nb x 64 B qh][nb x 16 B scales][nb x fp16 d]
+ * A row occupies exactly the same number of bytes as in the reference's block layout
+ * (ggml/src/ggml-common.h:161-166, 203-208, 279-290, 314-320); the mapping is a byte
+ * permutation inside each row.  These two entry points apply it / undo it for the byte
+ * range [offset, offset+size) of a tensor of `nrows` rows of `k` elements, so partial
+ * uploads and read-back return the reference's bytes
+ * (ggml_backend_buffer_i::set_tensor / get_tensor, ggml/src/ggml-backend-impl.h:52-53).
+ * `raw` holds only the `size` bytes of the range; `dev` is the base of the whole tensor. */
+int mi355_weights_scatter(void *stream, int type, const void *raw, void *dev, int64_t k, int64_t nrows,
+                          size_t offset, size_t size);
+int mi355_weights_gather(void *stream, int type, const void *dev, void *raw, int64_t k, int64_t nrows,
+                         size_t offset, size_t size);
+
+/* Activation quantization ------------------------------------------------------------ *
+ * quantize_row_q8_1_ref (ggml/src/ggml-quants.c:220-253), bit-exact: x is f32, row r at
+ * x + r*x_stride (elements); y receives nrows * k/32 block_q8_1 (36 bytes each,
+ * ggml/src/ggml-common.h:210-221), rows contiguous. */
+int mi355_quantize_q8_1(void *stream, const float *x, void *y, int64_t k, int64_t nrows, int64_t x_stride);
+
+/* Same quantizer writing the split layout the matrix kernels read:
+ *   int8 q[nrows][k]  followed by  {float d; int32 sum_q;} ds[nrows][k/32]
+ * where d is the fp16-rounded block scale widened to f32.  mi355_act_bytes() gives the size. */
+size_t mi355_act_bytes(int64_t k, int64_t nrows);
+int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64_t nrows, int64_t x_stride);
+
+/* MUL_MAT --------------------------------------------------------------------------- *
+ * ggml_compute_forward_mul_mat (ggml/src/ggml-cpu/ggml-cpu.c:7443-7635) for quantized
+ * src0 and f32 src1:  dst[b*dst_stride + n] = sum_k W[n][k] * x[b*x_stride + k].
+ * W: N rows of K elements of `type` in device layout.  x, dst f32.
+ * B <= 8 runs the bandwidth-bound GEMV (per-block integer dots of the weights against
+ * Q8_1 activations); larger B runs the int8-MFMA tile kernel.
+ * `ws` is scratch of at least mi355_mul_mat_ws_bytes(K, B) bytes. */
+size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
+int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
+                  int64_t x_stride, int64_t dst_stride, void *ws, size_t ws_bytes);
+
+/* The two halves of mi355_mul_mat for callers that reuse one quantized activation for
+ * several weight matrices (Q/K/V or gate/up projections): `act` from mi355_quantize_act. */
+int mi355_mul_mat_vec_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
+                        int64_t B, int64_t dst_stride);
+int mi355_mul_mat_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                    int64_t dst_stride);
+
+/* Integer sub-block dots, for parity checking the kernels' inner products bit-for-bit
+ * against ggml_vec_dot_q4_0_q8_0 / q8_0_q8_0 / q4_K_q8_K / q6_K_q8_K
+ * (ggml/src/ggml-cpu/ggml-cpu-quants.c:2492-2506, 3919-3927, 6817-6848, 8262-8283).
+ * a: ONE activation row in the split layout written by mi355_quantize_act (the same bytes
+ * the GEMV reads).  out: int32 [N][k/g], g = 32 (16 for Q6_K); the weight level has its
+ * fixed offset removed (Q4_0: nibble-8, Q6_K: q-32, Q4_K: nibble). */
+int mi355_block_dots_q8_1(void *stream, int type, const void *W, const void *a, int32_t *out, int64_t N, int64_t K);
+
+/* MUL_MAT_ID ------------------------------------------------------------------------ *
+ * ggml_compute_forward_mul_mat_id (ggml/src/ggml-cpu/ggml-cpu.c:7717-7895; semantics
+ * ggml/src/ggml.c:2723-2759): as = n_expert matrices of N rows x K in device layout, back
+ * to back; b f32 [K, nb1, T] contiguous; ids int32, element (e,t) at ids[t*ids_stride + e];
+ * dst f32 [N, n_used, T] contiguous.  dst[:,e,t] = as[ids[e,t]] . b[:, e % nb1, t].
+ * Expert bucketing is done on the device (no host synchronisation).
+ * ws: at least mi355_mul_mat_id_ws_bytes(...) bytes. */
+size_t mi355_mul_mat_id_ws_bytes(int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T);
+int mi355_mul_mat_id(void *stream, int type, const void *as, const float *b, const int32_t *ids, int64_t ids_stride,
+                     float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T,
+                     void *ws, size_t ws_bytes);
+
+/* Second half of mi355_mul_mat_id: `act` holds the nb1*T rows of b quantized by
+ * mi355_quantize_act (row t*nb1 + j). */
+int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride,
+                         float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T);
+
+/* FLASH_ATTN_EXT -------------------------------------------------------------------- *
+ * ggml_compute_forward_flash_attn_ext_f16 (ggml/src/ggml-cpu/ggml-cpu.c:10916-11129).
+ * q f32 [D, Nq, Hq] with byte strides q_nb1 (query) and q_nb2 (head); k, v f16
+ * [D, Nkv, Hkv] with byte strides *_nb1 (kv cell) and *_nb2 (kv head); mask f16
+ * [Nkv, >=Nq] contiguous rows of mask_nb1 bytes, or NULL; dst f32 [D, Hq, Nq]
+ * contiguous.  Hq % Hkv == 0 (grouped-query).  -inf mask entries are skipped.
+ * D must be 64, 80, 96, 112, 128 or 256.  ws: mi355_flash_attn_ws_bytes(...) bytes. */
+size_t mi355_flash_attn_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq);
+int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
+                         int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
+                         size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
+                         float max_bias, float logit_softcap, void *ws, size_t ws_bytes);
+
+/* Glue operators -------------------------------------------------------------------- *
+ * A strided f32/f16/i32 operand: up to 4 dimensions, ne[] elements, nb[] byte strides
+ * (the fields of struct ggml_tensor, ggml/include/ggml.h:576-608). */
+typedef struct mi355_tensor {
+    void   *data;
+    int     type;
+    int64_t ne[4];
+    size_t  nb[4];
+} mi355_tensor;
+
+/* ggml_compute_forward_rms_norm_f32 (ggml-cpu.c:7015-7061); rows along ne[0], row strides honoured */
+int mi355_rms_norm(void *stream, const mi355_tensor *src, const mi355_tensor *dst, float eps);
+/* ggml_compute_forward_{add,sub,mul,div}_f32 (ggml-cpu.c:4067-4140, 5142-5305): src1 broadcast over src0. op: 0 add 1 sub 2 mul 3 div */
+int mi355_bin_bcast(void *stream, int op, const mi355_tensor *src0, const mi355_tensor *src1, const mi355_tensor *dst);
+/* ggml_compute_forward_unary (ggml-cpu.c:6646-6683 for silu).  op: ggml_unary_op value
+ * (ggml/include/ggml.h:530-547); supported: ABS SGN NEG STEP TANH ELU RELU SIGMOID GELU GELU_QUICK SILU HARDSWISH HARDSIGMOID EXP */
+int mi355_unary(void *stream, int op, const mi355_tensor *src, const mi355_tensor *dst);
+/* ggml_compute_forward_scale_f32 (ggml-cpu.c:8158) */
+int mi355_scale(void *stream, const mi355_tensor *src, const mi355_tensor *dst, float s);
+/* ggml_compute_forward_dup (CPY/CONT/DUP, ggml-cpu.c:3519-3830): f32<->f16, f32->f32, f16->f16, i32->i32; any strides, same element count */
+int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
+/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, ids i32 [n, b2, b3]; dst f32 */
+int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ids, const mi355_tensor *dst);
+/* ggml_compute_forward_soft_max_f32 (ggml-cpu.c:8959-9055): mask f32 or f16 or NULL */
+int mi355_soft_max(void *stream, const mi355_tensor *src, const mi355_tensor *mask, const mi355_tensor *dst, float scale,
+                   float max_bias);
+/* ggml_compute_forward_rope_f32 (ggml-cpu.c:9366-9549): mode 0 (adjacent pairs) and 2 (NeoX); pos i32 [ne2]; freq_factors f32 or NULL */
+int mi355_rope(void *stream, const mi355_tensor *src, const int32_t *pos, const float *freq_factors,
+               const mi355_tensor *dst, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+               float ext_factor, float attn_factor, float beta_fast, float beta_slow);
+/* ggml_compute_forward_sum_rows_f32 (ggml-cpu.c:5678) */
+int mi355_sum_rows(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
+/* ggml_compute_forward_argsort_f32 (ggml-cpu.c:10857): order 0 ascending, 1 descending; ne[0] <= 1024 */
+int mi355_argsort(void *stream, const mi355_tensor *src, const mi355_tensor *dst, int order);
+/* MUL_MAT with f32 or f16 src0 and f32 src1 (router / small dense matrices): dst[b][n] = sum_k W[n][k] x[b][k], strides honoured, ne2/ne3 broadcast */
+int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *src1, const mi355_tensor *dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_KERNELS_H */

@@ -1,0 +1,120 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/mi355_kernels.h"
+
+namespace mi355 {
+
+typedef unsigned int u32;
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int WAVE = 64;
+
+// ---- block geometry (ggml/src/ggml-common.h:161-166, 203-221, 279-290, 314-320)
+constexpr int QK = 32;     // elements per Q4_0 / Q8_0 / Q8_1 block
+constexpr int QKK = 256;   // elements per K-quant super-block
+constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q8_1_BYTES = 36, Q4_K_BYTES = 144, Q6_K_BYTES = 210;
+
+__host__ __device__ inline int type_block_elems(int t) {
+    switch (t) {
+        case MI355_Q4_0: case MI355_Q8_0: case MI355_Q8_1: return QK;
+        case MI355_Q4_K: case MI355_Q6_K: return QKK;
+        case MI355_F32: case MI355_F16: case MI355_I32: return 1;
+        default: return 0;
+    }
+}
+__host__ __device__ inline int type_block_bytes(int t) {
+    switch (t) {
+        case MI355_Q4_0: return Q4_0_BYTES;
+        case MI355_Q8_0: return Q8_0_BYTES;
+        case MI355_Q8_1: return Q8_1_BYTES;
+        case MI355_Q4_K: return Q4_K_BYTES;
+        case MI355_Q6_K: return Q6_K_BYTES;
+        case MI355_F32: case MI355_I32: return 4;
+        case MI355_F16: return 2;
+        default: return 0;
+    }
+}
+__host__ __device__ inline bool is_weight_type(int t) {
+    return t == MI355_Q4_0 || t == MI355_Q8_0 || t == MI355_Q4_K || t == MI355_Q6_K;
+}
+
+// ---- activation workspace: int8 q[nrows][k] then {float d; int sum;} ds[nrows][k/32]
+struct act_ds {
+    float d;    // fp16-rounded block scale, widened
+    int sum;    // integer sum of the 32 levels
+};
+
+// ---- small device helpers
+__device__ __forceinline__ float half_bits_to_float(unsigned short h) {
+    union { unsigned short u; _Float16 f; } c;
+    c.u = h;
+    return (float)c.f;
+}
+__device__ __forceinline__ unsigned short float_to_half_bits(float f) {
+    union { unsigned short u; _Float16 h; } c;
+    c.h = (_Float16)f;   // v_cvt_f16_f32: round to nearest even
+    return c.u;
+}
+__device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
+
+// streaming (read-once) 16-byte load: keeps weights from evicting activations out of L2
+__device__ __forceinline__ u32x4 load_stream16(const void *p) {
+    return __builtin_nontemporal_load((const u32x4 *)p);
+}
+__device__ __forceinline__ u32x4 load16(const void *p) { return *(const u32x4 *)p; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// ---- host-side error plumbing
+void set_error(const char *fmt, ...);
+
+#define MI355_CHECK_HIP(expr)                                                              \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            mi355::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return MI355_ERR_HIP;                                                          \
+        }                                                                                  \
+    } while (0)
+
+#define MI355_REQUIRE(cond, ...)          \
+    do {                                  \
+        if (!(cond)) {                    \
+            mi355::set_error(__VA_ARGS__); \
+            return MI355_ERR_ARG;         \
+        }                                 \
+    } while (0)
+
+inline int launch_status(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("launch of %s failed: %s", what, hipGetErrorString(e));
+        return MI355_ERR_HIP;
+    }
+    return MI355_OK;
+}
+
+}  // namespace mi355

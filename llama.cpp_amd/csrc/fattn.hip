@@ -1,0 +1,295 @@
+// FLASH_ATTN_EXT over an f16 KV cache with grouped-query heads.
+//
+// k_fattn_vec: the HBM-bound form (decode, and any query count as a fallback).  A group
+// works on one (kv head, query token, kv split).  A K or V row of D halves is read by
+// D/8 neighbouring lanes with one 16-byte load each, so a wave streams 64/LPR cache cells
+// per step and all R = Hq/Hkv query heads that share the kv head are served from the same
+// bytes (each K/V byte leaves HBM once per query token).  q.k uses v_dot2_f32_f16 on q
+// rounded to f16 (as the reference does before its f16 dot), the LPR partial sums are
+// folded with DPP row operations, and every lane group keeps its own online-softmax state
+// (running max, sum, R x 8 output slice); the states are merged through LDS, and across kv
+// splits by k_fattn_combine.  -inf mask entries are skipped, as in the reference.
+#include "common.hpp"
+
+#include <float.h>
+
+namespace mi355 {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// sum over aligned groups of LPR lanes (8, 16 or 32); every lane of the group gets the sum
+template <int LPR>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_mov<0xB1>(v);    // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);    // quad_perm [2,3,0,1]
+    v += dpp_mov<0x141>(v);   // row_half_mirror: 8 lanes
+    if constexpr (LPR >= 16) v += dpp_mov<0x140>(v);   // row_mirror: 16 lanes
+    if constexpr (LPR >= 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
+__device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        s = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a[i]), __builtin_bit_cast(f16x2, b[i]), s, false);
+    return s;
+}
+
+struct fattn_args {
+    const uint8_t *q, *k, *v, *mask;
+    float *dst;      // [D, Hq, Nq]
+    float *ws;       // partial results when n_splits > 1: [Nq][Hq][n_splits][D + 2]
+    int64_t Nq, Nkv, Hq, Hkv;
+    size_t q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1;
+    float scale, max_bias, softcap;
+    float m0, m1;
+    unsigned n_head_log2;
+    int n_splits;
+    int groups;      // head groups of R per kv head: Hq / Hkv == R * groups
+    int64_t cells_per_split;
+};
+
+template <int D, int R>
+__global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
+    constexpr int LPR = D <= 64 ? 8 : (D <= 128 ? 16 : 32);   // lanes per K/V row
+    constexpr int CPW = 64 / LPR;                               // cells per wave step
+    constexpr int SLOTS = 4 * CPW;                              // independent softmax states per group
+    constexpr float NEG = -FLT_MAX / 2;
+
+    __shared__ float s_m[SLOTS][R], s_l[SLOTS][R];
+    __shared__ float s_o[SLOTS][R][D];
+
+    const int split = blockIdx.x;
+    const int64_t hk = blockIdx.y / a.groups, hg = blockIdx.y % a.groups, iq = blockIdx.z;
+    const int64_t head0 = (hk * a.groups + hg) * R;   // first of this group's R query heads
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane % LPR, slot = wave * CPW + lane / LPR;
+    const int d0 = sub * 8;
+    const bool active = d0 < D;
+
+    // q slices, rounded to f16 (ggml-cpu.c:11037-11040 converts q to the K type before the dot)
+    u32x4 qh[R];
+    float slope[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int64_t head = head0 + r;
+        const float *qp = (const float *)(a.q + iq * a.q_nb1 + head * a.q_nb2) + d0;
+        f32x4 x0 = {0, 0, 0, 0}, x1 = {0, 0, 0, 0};
+        if (active) {
+            x0 = *(const f32x4 *)qp;
+            x1 = *(const f32x4 *)(qp + 4);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            f16x2 p0 = {(_Float16)x0[2 * i], (_Float16)x0[2 * i + 1]};
+            f16x2 p1 = {(_Float16)x1[2 * i], (_Float16)x1[2 * i + 1]};
+            qh[r][i] = __builtin_bit_cast(u32, p0);
+            qh[r][2 + i] = __builtin_bit_cast(u32, p1);
+        }
+        // ALiBi slope of this head (ggml-cpu.c:10998-11003)
+        slope[r] = 1.0f;
+        if (a.max_bias > 0.0f) {
+            const unsigned h = (unsigned)head;
+            slope[r] = h < a.n_head_log2 ? powf(a.m0, (float)(h + 1)) : powf(a.m1, (float)(2 * (h - a.n_head_log2) + 1));
+        }
+    }
+
+    float m[R], l[R], acc[R][8];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        m[r] = NEG;
+        l[r] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[r][i] = 0.0f;
+    }
+
+    const int64_t c_begin = (int64_t)split * a.cells_per_split;
+    const int64_t c_end = c_begin + a.cells_per_split < a.Nkv ? c_begin + a.cells_per_split : a.Nkv;
+    const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
+    const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
+
+    for (int64_t cb = c_begin; cb < c_end; cb += SLOTS) {
+        const int64_t c = cb + slot;
+        const bool in_range = c < c_end;
+        float mv = 0.0f;
+        if (mrow && in_range) mv = half_bits_to_float(mrow[c]);
+        const bool valid = in_range && mv != -INFINITY;
+        if (__ballot(valid) == 0) continue;   // whole wave masked: skip the K/V traffic (wave-uniform)
+        u32x4 kk = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+        if (valid && active) {
+            kk = load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2);
+            vv = load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2);
+        }
+        float vf[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const f16x2 h2 = __builtin_bit_cast(f16x2, vv[i]);
+            vf[2 * i] = (float)h2[0];
+            vf[2 * i + 1] = (float)h2[1];
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float s = group_sum<LPR>(dot8_f16(qh[r], kk)) * scale;
+            if (a.softcap != 0.0f) s = a.softcap * tanhf(s);
+            s += slope[r] * mv;
+            if (valid) {
+                if (s > m[r]) {
+                    const float f = __expf(m[r] - s);
+                    l[r] *= f;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc[r][i] *= f;
+                    m[r] = s;
+                }
+                const float p = __expf(s - m[r]);
+                l[r] += p;
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[r][i] += p * vf[i];
+            }
+        }
+    }
+
+    // merge the SLOTS states of this group
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (sub == 0) {
+            s_m[slot][r] = m[r];
+            s_l[slot][r] = l[r];
+        }
+        if (active) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) s_o[slot][r][d0 + i] = acc[r][i];
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < R * D; idx += 256) {
+        const int r = idx / D, d = idx % D;
+        float M = NEG;
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) M = fmaxf(M, s_m[s][r]);
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            const float f = __expf(s_m[s][r] - M);
+            L += s_l[s][r] * f;
+            O += s_o[s][r][d] * f;
+        }
+        const int64_t head = head0 + r;
+        if (a.n_splits == 1) {
+            a.dst[(iq * a.Hq + head) * D + d] = O / L;
+        } else {
+            float *p = a.ws + ((iq * a.Hq + head) * a.n_splits + split) * (D + 2);
+            p[d] = O;
+            if (d == 0) {
+                p[D] = M;
+                p[D + 1] = L;
+            }
+        }
+    }
+}
+
+template <int D>
+__global__ void k_fattn_combine(const float *__restrict__ ws, float *__restrict__ dst, int n_splits) {
+    const int64_t row = blockIdx.x;   // iq * Hq + head
+    const float *p = ws + row * n_splits * (D + 2);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float M = -FLT_MAX / 2;
+        for (int s = 0; s < n_splits; s++) M = fmaxf(M, p[s * (D + 2) + D]);
+        float L = 0.0f, O = 0.0f;
+        for (int s = 0; s < n_splits; s++) {
+            const float f = __expf(p[s * (D + 2) + D] - M);
+            L += p[s * (D + 2) + D + 1] * f;
+            O += p[s * (D + 2) + d] * f;
+        }
+        dst[row * D + d] = O / L;
+    }
+}
+
+static int pick_splits(int64_t Nkv, int64_t Hkv, int64_t Nq) {
+    int64_t by_len = (Nkv + 255) / 256;
+    int64_t by_fill = 2048 / (Hkv * Nq > 0 ? Hkv * Nq : 1);
+    int64_t n = by_len < by_fill ? by_len : by_fill;
+    if (n < 1) n = 1;
+    if (n > 256) n = 256;
+    return (int)n;
+}
+
+template <int D, int R>
+static int launch_vec(hipStream_t s, fattn_args &a) {
+    a.groups = (int)(a.Hq / a.Hkv) / R;
+    const dim3 grid((unsigned)a.n_splits, (unsigned)(a.Hkv * a.groups), (unsigned)a.Nq);
+    hipLaunchKernelGGL((k_fattn_vec<D, R>), grid, dim3(256), 0, s, a);
+    int rc = launch_status("k_fattn_vec");
+    if (rc != MI355_OK) return rc;
+    if (a.n_splits > 1) {
+        hipLaunchKernelGGL(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(D <= 128 ? 128 : 256), 0, s, a.ws, a.dst, a.n_splits);
+        rc = launch_status("k_fattn_combine");
+    }
+    return rc;
+}
+
+template <int D>
+static int launch_vec_r(hipStream_t s, fattn_args &a, int R) {
+    // R = query heads served per group from one pass over the kv head's bytes
+    if (R % 4 == 0) return launch_vec<D, 4>(s, a);
+    if (R % 2 == 0) return launch_vec<D, 2>(s, a);
+    return launch_vec<D, 1>(s, a);
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+size_t mi355_flash_attn_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq) {
+    // worst case: 256 kv splits
+    (void)Nkv;
+    return (size_t)Nq * (size_t)Hq * 256 * (size_t)(D + 2) * sizeof(float);
+}
+
+int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
+                         int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
+                         size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
+                         float max_bias, float logit_softcap, void *ws, size_t ws_bytes) {
+    MI355_REQUIRE(D > 0 && D % 8 == 0 && D <= 256, "flash_attn: head size %lld not supported", (long long)D);
+    MI355_REQUIRE(Nq > 0 && Nkv > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "flash_attn: bad shape");
+    MI355_REQUIRE(Nq <= 65535 && Hq <= 65535, "flash_attn: too many query rows or heads for one launch");
+    MI355_REQUIRE(((uintptr_t)q & 15) == 0 && q_nb1 % 16 == 0 && q_nb2 % 16 == 0, "flash_attn: q rows must be 16-byte aligned");
+    MI355_REQUIRE(((uintptr_t)k & 15) == 0 && k_nb1 % 16 == 0 && k_nb2 % 16 == 0, "flash_attn: k rows must be 16-byte aligned");
+    MI355_REQUIRE(((uintptr_t)v & 15) == 0 && v_nb1 % 16 == 0 && v_nb2 % 16 == 0, "flash_attn: v rows must be 16-byte aligned");
+    MI355_REQUIRE(max_bias <= 0.0f || mask != nullptr, "flash_attn: max_bias needs a mask");
+    fattn_args a;
+    a.q = (const uint8_t *)q; a.k = (const uint8_t *)k; a.v = (const uint8_t *)v; a.mask = (const uint8_t *)mask;
+    a.dst = dst; a.ws = (float *)ws;
+    a.Nq = Nq; a.Nkv = Nkv; a.Hq = Hq; a.Hkv = Hkv;
+    a.q_nb1 = q_nb1; a.q_nb2 = q_nb2; a.k_nb1 = k_nb1; a.k_nb2 = k_nb2; a.v_nb1 = v_nb1; a.v_nb2 = v_nb2; a.mask_nb1 = mask_nb1;
+    a.scale = scale; a.max_bias = max_bias; a.softcap = logit_softcap;
+    // ALiBi base slopes, ggml-cpu.c:10986-10990
+    unsigned n2 = 1;
+    while (n2 * 2 <= (unsigned)Hq) n2 *= 2;
+    a.n_head_log2 = n2;
+    a.m0 = powf(2.0f, -(max_bias) / n2);
+    a.m1 = powf(2.0f, -(max_bias / 2.0f) / n2);
+    a.n_splits = pick_splits(Nkv, Hkv, Nq);
+    if (a.n_splits > 1) {
+        const size_t need = (size_t)Nq * (size_t)Hq * (size_t)a.n_splits * (size_t)(D + 2) * sizeof(float);
+        if (ws == nullptr || ws_bytes < need) a.n_splits = 1;   // no scratch: run unsplit
+    }
+    a.cells_per_split = (Nkv + a.n_splits - 1) / a.n_splits;
+    const int R = (int)(Hq / Hkv);
+    hipStream_t s = (hipStream_t)stream;
+    switch (D) {
+        case 64: return launch_vec_r<64>(s, a, R);
+        case 80: return launch_vec_r<80>(s, a, R);
+        case 96: return launch_vec_r<96>(s, a, R);
+        case 112: return launch_vec_r<112>(s, a, R);
+        case 128: return launch_vec_r<128>(s, a, R);
+        case 256: return launch_vec_r<256>(s, a, R);
+        default: set_error("flash_attn: head size %lld not supported", (long long)D); return MI355_ERR_ARG;
+    }
+}
+
+}  // extern "C"

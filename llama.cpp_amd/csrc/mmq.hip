@@ -1,0 +1,353 @@
+// Batched quantized GEMM on the int8 matrix cores (B > 8):
+//   dst[b][n] = sum_k W[n][k] * x[b][k],  W block-quantized, x quantized to Q8_1 on the device.
+//
+// A 256-thread group (4 waves, 2 x 2) owns a 128 (weight rows) x BN (activation rows)
+// tile of dst and walks K in stages of 128 elements.  Per stage the weight rows are
+// unpacked from their 4/6/8-bit blocks to int8 in LDS (16-byte streaming loads from HBM,
+// each weight byte is unpacked once per group and reused for BN activation rows), the
+// activation int8 rows are copied to LDS, and each wave contracts its 64 x (BN/2)
+// sub-tile with v_mfma_i32_32x32x32_i8, one instruction per 32-element quantization block,
+// so every MFMA result is an exact per-block integer dot.  Block results are scaled by
+// (weight block scale) x (activation block scale) and accumulated in f32 registers.
+//
+//   Q4_0 : level - 8 as int8, scale d                    (one MFMA per block)
+//   Q8_0 : level as int8, scale d
+//   Q4_K : level 0..15 as int8, scale d*sc; the "- dmin*m*sum(q)" term of all blocks is
+//          added with one v_mfma_f32_32x32x16_f16 per stage on (fp16 dx*sum(q)) x (fp16 dmin*m)
+//   Q6_K : level - 32 as int8, scale d*sc per 16 elements (v_mfma_i32_32x32x16_i8, two per block)
+//
+// MFMA operand mapping used here (A = activations, B = weights, D[i][j], i = activation
+// row, j = weight row): lane l supplies row/column l % 32 and the k bytes
+// [16*(l/32), 16*(l/32)+16) of the 32-wide step (8-byte halves for the 16-wide step);
+// D register r of lane l is element i = 8*(r/4) + 4*(l/32) + r%4, j = l % 32.  Both
+// operands use the same k split, so the contraction is independent of how the hardware
+// numbers k internally.
+//
+// Group ids are remapped so that the groups sharing one weight panel run on the same XCD
+// (ids are dealt round-robin over the 8 XCDs) and hit its L2 instead of HBM.
+#include "common.hpp"
+#include "qdot.hpp"
+
+namespace mi355 {
+
+constexpr int MMQ_BM = 128;          // weight rows per group
+constexpr int MMQ_BK = 128;          // K elements per stage
+constexpr int MMQ_LDK = MMQ_BK + 16; // LDS row pitch in bytes (pad to spread banks)
+
+template <int TYPE> struct mmq_cfg {
+    static constexpr int G = TYPE == MI355_Q6_K ? 16 : 32;   // elements per weight scale
+    static constexpr int NG = MMQ_BK / G;                    // weight scales per row per stage
+};
+
+// ---- stage loaders: global (device layout) -> int8 rows + scales in LDS ----------------
+// sW  : int8 [MMQ_BM][MMQ_LDK]
+// sWs : float [NG][MMQ_BM]   (scale g of row r at sWs[g*MMQ_BM + r])
+// sWo : fp16  [MMQ_BM][4]    (Q4_K only: dmin*m of the 4 sub-blocks of the stage)
+template <int TYPE>
+__device__ __forceinline__ void load_weight_stage(const uint8_t *__restrict__ W, const row_layout &L, int64_t row0,
+                                                  int64_t N, int64_t k0, int8_t *sW, float *sWs, _Float16 *sWo) {
+    const int tid = threadIdx.x;
+    if constexpr (TYPE == MI355_Q4_0) {
+        // 128 rows x 4 blocks of 16 B
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 2, b = idx & 3;
+            const int64_t row = row0 + r < N ? row0 + r : N - 1;
+            const uint8_t *wrow = W + row * L.row_bytes;
+            const int64_t blk = (k0 >> 5) + b;
+            const u32x4 q = load_stream16(wrow + blk * 16);
+            u32x4 lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                // nibble - 8 per byte without cross-byte borrow
+                lo[i] = (((q[i] & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+                hi[i] = ((((q[i] >> 4) & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+            }
+            *(u32x4 *)(sW + r * MMQ_LDK + b * 32) = lo;
+            *(u32x4 *)(sW + r * MMQ_LDK + b * 32 + 16) = hi;
+            sWs[b * MMQ_BM + r] = half_bits_to_float(*(const unsigned short *)(wrow + L.off_b + blk * 2));
+        }
+    } else if constexpr (TYPE == MI355_Q8_0) {
+        // 128 rows x 4 blocks x 2 halves of 16 B
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 3, c = idx & 7;   // c: 16-byte piece of the stage
+            const int64_t row = row0 + r < N ? row0 + r : N - 1;
+            const uint8_t *wrow = W + row * L.row_bytes;
+            const u32x4 q = load_stream16(wrow + k0 + c * 16);
+            *(u32x4 *)(sW + r * MMQ_LDK + c * 16) = q;
+            if ((c & 1) == 0) {
+                const int b = c >> 1;
+                sWs[b * MMQ_BM + r] = half_bits_to_float(*(const unsigned short *)(wrow + L.off_b + ((k0 >> 5) + b) * 2));
+            }
+        }
+    } else if constexpr (TYPE == MI355_Q4_K) {
+        // stage = half a super-block: sub-blocks j0..j0+3, 64 B of qs per row = 4 pieces of 16 B
+        const int64_t sb = k0 >> 8;
+        const int half = (int)((k0 >> 7) & 1);
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 2, p = idx & 3;          // p: piece -> group gl = p>>1 of the stage, half h = p&1
+            const int gl = p >> 1, h = p & 1;
+            const int64_t row = row0 + r < N ? row0 + r : N - 1;
+            const uint8_t *blk = W + row * L.row_bytes + sb * Q4_K_BYTES;
+            const u32x4 q = load_stream16(blk + 16 + (half * 2 + gl) * 32 + h * 16);
+            u32x4 lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                lo[i] = q[i] & 0x0F0F0F0Fu;
+                hi[i] = (q[i] >> 4) & 0x0F0F0F0Fu;
+            }
+            *(u32x4 *)(sW + r * MMQ_LDK + (2 * gl) * 32 + h * 16) = lo;
+            *(u32x4 *)(sW + r * MMQ_LDK + (2 * gl + 1) * 32 + h * 16) = hi;
+            // this thread also owns the (scale, min) of sub-block p of the stage
+            const u32x4 hdr = load16(blk);
+            const float d = half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu));
+            const float dmin = half_bits_to_float((unsigned short)(hdr[0] >> 16));
+            int sc, mn;
+            q4k_scale_min(hdr[1], hdr[2], hdr[3], half * 4 + p, sc, mn);
+            sWs[p * MMQ_BM + r] = d * (float)sc;
+            sWo[r * 4 + p] = (_Float16)(dmin * (float)mn);
+        }
+    } else {   // Q6_K: stage = half hf of a super-block: 64 B ql + 32 B qh, 8 scales
+        const int64_t sb = k0 >> 8;
+        const int hf = (int)((k0 >> 7) & 1);
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 2, p = idx & 3;          // p: 16-byte piece of this half's ql
+            const int l0 = 16 * (p & 1), qa = p >> 1;
+            const int64_t row = row0 + r < N ? row0 + r : N - 1;
+            const uint8_t *wrow = W + row * L.row_bytes;
+            const u32x4 ql = load_stream16(wrow + sb * 128 + hf * 64 + p * 16);
+            const u32x4 qh = load_stream16(wrow + L.off_b + sb * 64 + hf * 32 + l0);
+            u32x4 vA, vB;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 a = (ql[i] & 0x0F0F0F0Fu) | (((qh[i] >> (2 * qa)) & 0x03030303u) << 4);
+                const u32 b = ((ql[i] >> 4) & 0x0F0F0F0Fu) | (((qh[i] >> (2 * qa + 4)) & 0x03030303u) << 4);
+                // level - 32 per byte: flip bit 5, then sign-extend it into bits 6..7
+                const u32 ta = a ^ 0x20202020u, tb = b ^ 0x20202020u;
+                const u32 ma = ta & 0x20202020u, mb = tb & 0x20202020u;
+                vA[i] = ta | (ma << 1) | (ma << 2);
+                vB[i] = tb | (mb << 1) | (mb << 2);
+            }
+            *(u32x4 *)(sW + r * MMQ_LDK + qa * 32 + l0) = vA;
+            *(u32x4 *)(sW + r * MMQ_LDK + (qa + 2) * 32 + l0) = vB;
+            // scales of 16-element groups 2p and 2p+1 of the stage
+            const float d = half_bits_to_float(*(const unsigned short *)(wrow + L.off_d + sb * 2));
+            const int8_t *sc = (const int8_t *)(wrow + L.off_c + sb * 16 + hf * 8);
+            sWs[(2 * p) * MMQ_BM + r] = d * (float)sc[2 * p];
+            sWs[(2 * p + 1) * MMQ_BM + r] = d * (float)sc[2 * p + 1];
+        }
+    }
+}
+
+// sA  : int8 [BN][MMQ_LDK];  sAd : float [4][BN] block scales;  sAs : fp16 [BN][4]  dx*sum(q) (Q4_K)
+template <int TYPE, int BN>
+__device__ __forceinline__ void load_act_stage(const int8_t *__restrict__ aq, const act_ds *__restrict__ ads,
+                                               int64_t col0, int64_t B, int64_t K, int64_t k0, int8_t *sA, float *sAd,
+                                               _Float16 *sAs) {
+    const int tid = threadIdx.x;
+    const int64_t nblk = K >> 5;
+    // BN rows x 8 pieces of 16 B
+#pragma unroll
+    for (int it = 0; it < BN * 8 / 256; it++) {
+        const int idx = tid + it * 256;
+        const int r = idx >> 3, c = idx & 7;
+        const int64_t col = col0 + r < B ? col0 + r : B - 1;
+        *(u32x4 *)(sA + r * MMQ_LDK + c * 16) = load16(aq + col * K + k0 + c * 16);
+    }
+    // BN rows x 4 block scales
+#pragma unroll
+    for (int it = 0; it < (BN * 4 + 255) / 256; it++) {
+        const int idx = tid + it * 256;
+        if (idx < BN * 4) {
+            const int r = idx >> 2, b = idx & 3;
+            const int64_t col = col0 + r < B ? col0 + r : B - 1;
+            const act_ds s = ads[col * nblk + (k0 >> 5) + b];
+            sAd[b * BN + r] = s.d;
+            if constexpr (TYPE == MI355_Q4_K) sAs[r * 4 + b] = (_Float16)(s.d * (float)s.sum);
+        }
+    }
+}
+
+template <int TYPE, int TN>
+__global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
+                                             const act_ds *__restrict__ ads, float *__restrict__ dst, int64_t N,
+                                             int64_t K, int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles,
+                                             int n_groups, int n_groups_padded) {
+    typedef mmq_cfg<TYPE> C;
+    constexpr int BN = 64 * TN;
+    __shared__ __attribute__((aligned(16))) int8_t sW[MMQ_BM * MMQ_LDK];
+    __shared__ __attribute__((aligned(16))) int8_t sA[BN * MMQ_LDK];
+    __shared__ __attribute__((aligned(16))) float sWs[C::NG * MMQ_BM];
+    __shared__ __attribute__((aligned(16))) float sAd[4 * BN];
+    __shared__ __attribute__((aligned(16))) _Float16 sWo[TYPE == MI355_Q4_K ? MMQ_BM * 4 : 4];
+    __shared__ __attribute__((aligned(16))) _Float16 sAs[TYPE == MI355_Q4_K ? BN * 4 : 4];
+
+    // XCD-aware id: hardware deals group ids round-robin over 8 XCDs; make logical neighbours share an XCD
+    const int per_xcd = n_groups_padded >> 3;
+    const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (lid >= n_groups) return;   // uniform for the whole group
+    const int64_t row0 = (int64_t)(lid / n_col_tiles) * MMQ_BM;
+    const int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int wrow0 = (wave & 1) * 64;           // weight rows of this wave inside the tile
+    const int wcol0 = (wave >> 1) * (32 * TN);   // activation rows of this wave inside the tile
+
+    f32x16 acc[TN][2];
+#pragma unroll
+    for (int tb = 0; tb < TN; tb++)
+#pragma unroll
+        for (int tw = 0; tw < 2; tw++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[tb][tw][r] = 0.0f;
+
+    for (int64_t k0 = 0; k0 < K; k0 += MMQ_BK) {
+        __syncthreads();
+        load_weight_stage<TYPE>(W, L, row0, N, k0, sW, sWs, sWo);
+        load_act_stage<TYPE, BN>(aq, ads, col0, B, K, k0, sA, sAd, sAs);
+        __syncthreads();
+
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {   // one Q8_1 block per step
+            // activation block scales for this lane's 16 D rows: i = 8*(r/4) + 4*lhi + r%4
+            f32x4 dx[TN][4];
+#pragma unroll
+            for (int tb = 0; tb < TN; tb++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) dx[tb][q] = *(const f32x4 *)(sAd + ks * BN + wcol0 + tb * 32 + 8 * q + 4 * lhi);
+
+            if constexpr (C::G == 32) {
+                i32x4 af[TN], bf[2];
+#pragma unroll
+                for (int tb = 0; tb < TN; tb++) af[tb] = *(const i32x4 *)(sA + (wcol0 + tb * 32 + l32) * MMQ_LDK + ks * 32 + 16 * lhi);
+#pragma unroll
+                for (int tw = 0; tw < 2; tw++) bf[tw] = *(const i32x4 *)(sW + (wrow0 + tw * 32 + l32) * MMQ_LDK + ks * 32 + 16 * lhi);
+#pragma unroll
+                for (int tw = 0; tw < 2; tw++) {
+                    const float dw = sWs[ks * MMQ_BM + wrow0 + tw * 32 + l32];
+#pragma unroll
+                    for (int tb = 0; tb < TN; tb++) {
+                        i32x16 z;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) z[r] = 0;
+                        const i32x16 I = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tb], bf[tw], z, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[tb][tw][r] += (float)I[r] * (dw * dx[tb][r >> 2][r & 3]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int hs = 0; hs < 2; hs++) {   // two 16-element scale groups per block
+                    long af[TN], bf[2];
+#pragma unroll
+                    for (int tb = 0; tb < TN; tb++) af[tb] = *(const long *)(sA + (wcol0 + tb * 32 + l32) * MMQ_LDK + ks * 32 + hs * 16 + 8 * lhi);
+#pragma unroll
+                    for (int tw = 0; tw < 2; tw++) bf[tw] = *(const long *)(sW + (wrow0 + tw * 32 + l32) * MMQ_LDK + ks * 32 + hs * 16 + 8 * lhi);
+#pragma unroll
+                    for (int tw = 0; tw < 2; tw++) {
+                        const float dw = sWs[(ks * 2 + hs) * MMQ_BM + wrow0 + tw * 32 + l32];
+#pragma unroll
+                        for (int tb = 0; tb < TN; tb++) {
+                            i32x16 z;
+#pragma unroll
+                            for (int r = 0; r < 16; r++) z[r] = 0;
+                            const i32x16 I = __builtin_amdgcn_mfma_i32_32x32x16_i8(af[tb], bf[tw], z, 0, 0, 0);
+#pragma unroll
+                            for (int r = 0; r < 16; r++) acc[tb][tw][r] += (float)I[r] * (dw * dx[tb][r >> 2][r & 3]);
+                        }
+                    }
+                }
+            }
+        }
+
+        if constexpr (TYPE == MI355_Q4_K) {
+            // acc -= sum_b (dx*sum q)[i][b] * (dmin*m)[j][b] over the 4 blocks of the stage:
+            // a 32x32x16 f16 MFMA whose k slots 0..3 hold the blocks (lanes 32..63 and slots 4..7 are zero)
+            f16x8 af[TN], bf[2];
+#pragma unroll
+            for (int tb = 0; tb < TN; tb++) {
+                const f16x4 v = *(const f16x4 *)(sAs + (wcol0 + tb * 32 + l32) * 4);
+#pragma unroll
+                for (int i = 0; i < 8; i++) af[tb][i] = (i < 4 && lhi == 0) ? (_Float16)(-(float)v[i & 3]) : (_Float16)0.0f;
+            }
+#pragma unroll
+            for (int tw = 0; tw < 2; tw++) {
+                const f16x4 v = *(const f16x4 *)(sWo + (wrow0 + tw * 32 + l32) * 4);
+#pragma unroll
+                for (int i = 0; i < 8; i++) bf[tw][i] = (i < 4 && lhi == 0) ? v[i & 3] : (_Float16)0.0f;
+            }
+#pragma unroll
+            for (int tb = 0; tb < TN; tb++)
+#pragma unroll
+                for (int tw = 0; tw < 2; tw++) acc[tb][tw] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tb], bf[tw], acc[tb][tw], 0, 0, 0);
+        }
+    }
+
+    // store: lane holds weight row j = l32 of each 32-wide tile, 16 activation rows
+#pragma unroll
+    for (int tb = 0; tb < TN; tb++)
+#pragma unroll
+        for (int tw = 0; tw < 2; tw++) {
+            const int64_t n = row0 + wrow0 + tw * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                if (n < N && b < B) dst[b * dst_stride + n] = acc[tb][tw][r];
+            }
+        }
+}
+
+template <int TYPE, int TN>
+static void launch_mmq(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                       int64_t dst_stride) {
+    constexpr int BN = 64 * TN;
+    const row_layout L = make_row_layout(TYPE, K);
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + B * K);
+    const int n_row_tiles = (int)((N + MMQ_BM - 1) / MMQ_BM);
+    const int n_col_tiles = (int)((B + BN - 1) / BN);
+    const int n_groups = n_row_tiles * n_col_tiles;
+    const int n_groups_padded = (n_groups + 7) & ~7;
+    hipLaunchKernelGGL((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
+                       dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded);
+}
+
+template <int TYPE>
+static void launch_mmq_tn(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                          int64_t dst_stride) {
+    if (B <= 64) launch_mmq<TYPE, 1>(s, W, act, dst, N, K, B, dst_stride);
+    else launch_mmq<TYPE, 2>(s, W, act, dst, N, K, B, dst_stride);
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_mul_mat_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
+                               int64_t B, int64_t dst_stride) {
+    MI355_REQUIRE(is_weight_type(type), "mul_mat_q: unsupported weight type %d", type);
+    MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
+    MI355_REQUIRE(K % MMQ_BK == 0 && K % type_block_elems(type) == 0, "mul_mat_q: K=%lld must be a multiple of 128 and of the block size", (long long)K);
+    MI355_REQUIRE(dst_stride >= N, "mul_mat_q: dst_stride < N");
+    const row_layout L = make_row_layout(type, K);
+    MI355_REQUIRE(((uintptr_t)W & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0,
+                  "mul_mat_q: weight rows are not 16-byte aligned (K=%lld)", (long long)K);
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_q: activation workspace is not 16-byte aligned");
+    MI355_REQUIRE((N + MMQ_BM - 1) / MMQ_BM * ((B + 63) / 64) < (1 << 30), "mul_mat_q: too many tiles");
+    hipStream_t s = (hipStream_t)stream;
+    switch (type) {
+        case MI355_Q4_0: launch_mmq_tn<MI355_Q4_0>(s, W, act, dst, N, K, B, dst_stride); break;
+        case MI355_Q8_0: launch_mmq_tn<MI355_Q8_0>(s, W, act, dst, N, K, B, dst_stride); break;
+        case MI355_Q4_K: launch_mmq_tn<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride); break;
+        default: launch_mmq_tn<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride); break;
+    }
+    return launch_status("k_mmq");
+}

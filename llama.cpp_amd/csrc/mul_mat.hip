@@ -1,0 +1,117 @@
+// MUL_MAT host entry: quantize activations to Q8_1 on the device, then dispatch to the
+// GEMV (B <= 8) or the int8-MFMA tile kernel (B > 8).  Also the unaligned fallback.
+#include "common.hpp"
+#include "qdot.hpp"
+
+namespace mi355 {
+
+// Dequantized weight element e of a row stored in device layout.  Byte loads only, so it
+// works for rows that are not 16-byte aligned (K not a multiple of 256 for Q4_0/Q8_0, of
+// 2048 for Q6_K).  Semantics: dequantize_row_* of ggml/src/ggml-quants.c:255-273, 349-363,
+// 1280-1302, 1690-1719.
+template <int TYPE>
+__device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, const row_layout &L, int64_t e) {
+    if constexpr (TYPE == MI355_Q4_0) {
+        const int64_t b = e >> 5;
+        const int j = (int)(e & 31);
+        const uint8_t byte = row[b * 16 + (j & 15)];
+        const int n = j < 16 ? (byte & 0x0F) : (byte >> 4);
+        const unsigned short dh = (unsigned short)(row[L.off_b + 2 * b] | (row[L.off_b + 2 * b + 1] << 8));
+        return half_bits_to_float(dh) * (float)(n - 8);
+    } else if constexpr (TYPE == MI355_Q8_0) {
+        const int64_t b = e >> 5;
+        const int8_t q = (int8_t)row[b * 32 + (e & 31)];
+        const unsigned short dh = (unsigned short)(row[L.off_b + 2 * b] | (row[L.off_b + 2 * b + 1] << 8));
+        return half_bits_to_float(dh) * (float)q;
+    } else if constexpr (TYPE == MI355_Q4_K) {
+        const int64_t sb = e >> 8;
+        const int r = (int)(e & 255), j = r >> 5, l = r & 31;
+        const uint8_t *blk = row + sb * Q4_K_BYTES;
+        const unsigned short dh = (unsigned short)(blk[0] | (blk[1] << 8)), mh = (unsigned short)(blk[2] | (blk[3] << 8));
+        const uint8_t *p = blk + 4;
+        int sc, mn;
+        if (j < 4) { sc = p[j] & 63; mn = p[j + 4] & 63; }
+        else { sc = (p[j + 4] & 0x0F) | ((p[j - 4] >> 6) << 4); mn = (p[j + 4] >> 4) | ((p[j] >> 6) << 4); }
+        const uint8_t byte = blk[16 + 32 * (j >> 1) + l];
+        const int n = (j & 1) ? (byte >> 4) : (byte & 0x0F);
+        return half_bits_to_float(dh) * (float)sc * (float)n - half_bits_to_float(mh) * (float)mn;
+    } else {
+        const int64_t sb = e >> 8;
+        const int r = (int)(e & 255), hf = r >> 7, quad = (r & 127) >> 5, l = r & 31;
+        const uint8_t lo = row[sb * 128 + 64 * hf + 32 * (quad & 1) + l];
+        const int nib = quad < 2 ? (lo & 0x0F) : (lo >> 4);
+        const int hi = (row[L.off_b + sb * 64 + 32 * hf + l] >> (2 * quad)) & 3;
+        const int8_t sc = (int8_t)row[L.off_c + sb * 16 + (r >> 4)];
+        const unsigned short dh = (unsigned short)(row[L.off_d + 2 * sb] | (row[L.off_d + 2 * sb + 1] << 8));
+        return half_bits_to_float(dh) * (float)sc * (float)((nib | (hi << 4)) - 32);
+    }
+}
+
+// one wave per (row, activation row); any K that is a multiple of the block size
+template <int TYPE>
+__global__ void __launch_bounds__(64) k_gemv_unaligned(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
+                                                       const act_ds *__restrict__ ads, float *__restrict__ dst,
+                                                       int64_t N, int64_t K, int64_t dst_stride, row_layout L) {
+    const int64_t row = blockIdx.x, col = blockIdx.y;
+    const uint8_t *wrow = W + row * L.row_bytes;
+    const int8_t *q = aq + col * K;
+    const act_ds *ds = ads + col * (K >> 5);
+    float acc = 0.0f;
+    for (int64_t e = threadIdx.x; e < K; e += 64) acc += weight_value<TYPE>(wrow, L, e) * (ds[e >> 5].d * (float)q[e]);
+    acc = wave_sum(acc);
+    if (threadIdx.x == 0) dst[col * dst_stride + row] = acc;
+}
+
+static bool rows_aligned(int type, const void *W, int64_t K) {
+    const row_layout L = make_row_layout(type, K);
+    return ((uintptr_t)W & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0;
+}
+
+static int gemv_unaligned(hipStream_t s, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
+                          int64_t B, int64_t dst_stride) {
+    const row_layout L = make_row_layout(type, K);
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + B * K);
+    MI355_REQUIRE(B <= 65535, "mul_mat: batch %lld too large for the unaligned path", (long long)B);
+    const dim3 grid((unsigned)N, (unsigned)B);
+    switch (type) {
+        case MI355_Q4_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
+        case MI355_Q8_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
+        case MI355_Q4_K: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
+        default: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
+    }
+    return launch_status("k_gemv_unaligned");
+}
+
+// act holds B quantized rows; runs the right kernel for any B
+int mul_mat_from_act(hipStream_t s, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
+                     int64_t B, int64_t dst_stride) {
+    if (!rows_aligned(type, W, K) || (B > 8 && K % 128 != 0)) return gemv_unaligned(s, type, W, act, dst, N, K, B, dst_stride);
+    if (B <= 8) return mi355_mul_mat_vec_q(s, type, W, act, dst, N, K, B, dst_stride);
+    return mi355_mul_mat_q(s, type, W, act, dst, N, K, B, dst_stride);
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B) { return (mi355_act_bytes(K, B) + 255) & ~(size_t)255; }
+
+int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
+                  int64_t x_stride, int64_t dst_stride, void *ws, size_t ws_bytes) {
+    MI355_REQUIRE(is_weight_type(type), "mul_mat: unsupported weight type %d", type);
+    MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
+    MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat: K=%lld is not a multiple of the block size", (long long)K);
+    MI355_REQUIRE(dst_stride >= N, "mul_mat: dst_stride < N");
+    if (ws_bytes < mi355_mul_mat_ws_bytes(K, B) || ws == nullptr) {
+        set_error("mul_mat: workspace of %zu bytes, need %zu", ws_bytes, mi355_mul_mat_ws_bytes(K, B));
+        return MI355_ERR_WORKSPACE;
+    }
+    int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
+    if (rc != MI355_OK) return rc;
+    return mul_mat_from_act((hipStream_t)stream, type, W, ws, dst, N, K, B, dst_stride);
+}
+
+}  // extern "C"

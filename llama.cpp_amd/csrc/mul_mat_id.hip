@@ -1,0 +1,32 @@
+// MUL_MAT_ID host entry: quantize the nb1*T rows of b once, then route every
+// (token, expert slot) pair to its expert's weights on the device.
+#include "common.hpp"
+#include "qdot.hpp"
+
+using namespace mi355;
+
+extern "C" {
+
+size_t mi355_mul_mat_id_ws_bytes(int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T) {
+    (void)n_expert;
+    (void)n_used;
+    return (mi355_act_bytes(K, nb1 * T) + 255) & ~(size_t)255;
+}
+
+int mi355_mul_mat_id(void *stream, int type, const void *as, const float *b, const int32_t *ids, int64_t ids_stride,
+                     float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T,
+                     void *ws, size_t ws_bytes) {
+    MI355_REQUIRE(is_weight_type(type), "mul_mat_id: unsupported weight type %d", type);
+    MI355_REQUIRE(N > 0 && K > 0 && n_expert > 0 && n_used > 0 && nb1 > 0 && T > 0, "mul_mat_id: bad shape");
+    MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_id: K=%lld is not a multiple of the block size", (long long)K);
+    MI355_REQUIRE(ids_stride >= n_used, "mul_mat_id: ids_stride < n_used");
+    if (ws == nullptr || ws_bytes < mi355_mul_mat_id_ws_bytes(K, n_expert, n_used, nb1, T)) {
+        set_error("mul_mat_id: workspace of %zu bytes, need %zu", ws_bytes, mi355_mul_mat_id_ws_bytes(K, n_expert, n_used, nb1, T));
+        return MI355_ERR_WORKSPACE;
+    }
+    int rc = mi355_quantize_act(stream, b, ws, K, nb1 * T, K);
+    if (rc != MI355_OK) return rc;
+    return mi355_mul_mat_id_vec(stream, type, as, ws, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T);
+}
+
+}  // extern "C"

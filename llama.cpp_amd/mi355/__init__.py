@@ -1,0 +1,214 @@
+"""Python view of the MI355X kernel library (ctypes over include/mi355_kernels.h).
+
+PyTorch is used only to own device memory and streams; every operator below goes through
+the C ABI of libmi355_kernels.so.  There is no CPU fallback: loading fails loudly when the
+library has not been built.
+"""
+import ctypes as C
+import os
+
+from . import build as _build
+
+F32, F16, Q4_0, Q8_0, Q8_1, Q4_K, Q6_K, I32 = 0, 1, 2, 8, 9, 12, 14, 26
+WEIGHT_TYPES = {"q4_0": Q4_0, "q8_0": Q8_0, "q4_K": Q4_K, "q6_K": Q6_K}
+BLOCK = {F32: (1, 4), F16: (1, 2), I32: (1, 4), Q4_0: (32, 18), Q8_0: (32, 34), Q8_1: (32, 36), Q4_K: (256, 144),
+         Q6_K: (256, 210)}
+
+_p, _i64, _sz, _f, _int = C.c_void_p, C.c_int64, C.c_size_t, C.c_float, C.c_int
+
+
+class Tensor(C.Structure):
+    """struct mi355_tensor"""
+    _fields_ = [("data", _p), ("type", _int), ("ne", _i64 * 4), ("nb", _sz * 4)]
+
+
+_SIGNATURES = {
+    "mi355_abi_version": (_int, []),
+    "mi355_last_error": (C.c_char_p, []),
+    "mi355_device_supported": (_int, [_int]),
+    "mi355_weights_scatter": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
+    "mi355_weights_gather": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
+    "mi355_quantize_q8_1": (_int, [_p, _p, _p, _i64, _i64, _i64]),
+    "mi355_act_bytes": (_sz, [_i64, _i64]),
+    "mi355_quantize_act": (_int, [_p, _p, _p, _i64, _i64, _i64]),
+    "mi355_mul_mat_ws_bytes": (_sz, [_i64, _i64]),
+    "mi355_mul_mat": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_vec_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_mul_mat_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_block_dots_q8_1": (_int, [_p, _int, _p, _p, _p, _i64, _i64]),
+    "mi355_mul_mat_id_ws_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
+    "mi355_mul_mat_id": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_id_vec": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64]),
+    "mi355_flash_attn_ws_bytes": (_sz, [_i64, _i64, _i64, _i64]),
+    "mi355_flash_attn_ext": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _sz, _sz,
+                                    _sz, _f, _f, _f, _p, _sz]),
+    "mi355_rms_norm": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), _f]),
+    "mi355_bin_bcast": (_int, [_p, _int, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]),
+    "mi355_unary": (_int, [_p, _int, C.POINTER(Tensor), C.POINTER(Tensor)]),
+    "mi355_scale": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), _f]),
+    "mi355_cpy": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor)]),
+    "mi355_get_rows": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]),
+    "mi355_soft_max": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor), _f, _f]),
+    "mi355_rope": (_int, [_p, C.POINTER(Tensor), _p, _p, C.POINTER(Tensor), _int, _int, _int, _f, _f, _f, _f, _f, _f]),
+    "mi355_sum_rows": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor)]),
+    "mi355_argsort": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), _int]),
+    "mi355_mul_mat_f": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]),
+}
+
+_lib = None
+
+
+def lib_path():
+    return _build.kernels_lib_path()
+
+
+def load():
+    """dlopen libmi355_kernels.so (already-built file only; see build.build_kernels)."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: run `python __graft_entry__.py` (build()) first" % path)
+        lib = C.CDLL(path)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)   # AttributeError if the library lacks a declared symbol
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+class Mi355Error(RuntimeError):
+    pass
+
+
+def check(rc):
+    if rc != 0:
+        raise Mi355Error("mi355 error %d: %s" % (rc, load().mi355_last_error().decode()))
+
+
+def row_bytes(t, k):
+    be, bb = BLOCK[t]
+    assert k % be == 0
+    return k // be * bb
+
+
+# ---------------------------------------------------------------- torch-facing helpers
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+_TORCH_TYPES = None
+
+
+def tensor_desc(t):
+    """mi355_tensor for a torch tensor; ggml order: ne[0] is the fastest (last torch) dimension."""
+    import torch
+    global _TORCH_TYPES
+    if _TORCH_TYPES is None:
+        _TORCH_TYPES = {torch.float32: F32, torch.float16: F16, torch.int32: I32}
+    d = Tensor()
+    d.data = t.data_ptr()
+    d.type = _TORCH_TYPES[t.dtype]
+    shape = list(t.shape)[::-1]
+    strides = [s * t.element_size() for s in t.stride()][::-1]
+    assert len(shape) <= 4
+    for i in range(4):
+        d.ne[i] = shape[i] if i < len(shape) else 1
+        d.nb[i] = strides[i] if i < len(shape) else (d.nb[i - 1] * d.ne[i - 1] if i > 0 else t.element_size())
+    return d
+
+
+def upload_weights(t, raw):
+    """raw: torch.uint8 CUDA tensor [nrows, row_bytes] in the reference block layout -> device layout copy"""
+    import torch
+    nrows, rb = raw.shape
+    k = rb // BLOCK[t][1] * BLOCK[t][0]
+    out = torch.empty_like(raw)
+    check(load().mi355_weights_scatter(_stream(), t, _ptr(raw), _ptr(out), k, nrows, 0, raw.numel()))
+    return out
+
+
+def download_weights(t, dev):
+    import torch
+    nrows, rb = dev.shape
+    k = rb // BLOCK[t][1] * BLOCK[t][0]
+    out = torch.empty_like(dev)
+    check(load().mi355_weights_gather(_stream(), t, _ptr(dev), _ptr(out), k, nrows, 0, dev.numel()))
+    return out
+
+
+def quantize_q8_1(x):
+    """x f32 [nrows, k] -> uint8 [nrows, k/32*36] (block_q8_1)"""
+    import torch
+    nrows, k = x.shape
+    y = torch.empty((nrows, k // 32 * 36), dtype=torch.uint8, device=x.device)
+    check(load().mi355_quantize_q8_1(_stream(), _ptr(x), _ptr(y), k, nrows, x.stride(0)))
+    return y
+
+
+def quantize_act(x):
+    import torch
+    nrows, k = x.shape
+    ws = torch.empty(load().mi355_act_bytes(k, nrows), dtype=torch.uint8, device=x.device)
+    check(load().mi355_quantize_act(_stream(), _ptr(x), _ptr(ws), k, nrows, x.stride(0)))
+    return ws
+
+
+def mul_mat(t, W, x, ws=None):
+    """W: device-layout uint8 [N, row_bytes]; x f32 [B, K] -> f32 [B, N]"""
+    import torch
+    B, K = x.shape
+    N = W.shape[0]
+    need = load().mi355_mul_mat_ws_bytes(K, B)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    dst = torch.empty((B, N), dtype=torch.float32, device=x.device)
+    check(load().mi355_mul_mat(_stream(), t, _ptr(W), _ptr(x), _ptr(dst), N, K, B, x.stride(0), N, _ptr(ws), ws.numel()))
+    return dst
+
+
+def block_dots(t, W, x_row):
+    """integer granule dots of every row of W against the Q8_1 quantization of x_row (f32 [K])"""
+    import torch
+    K = x_row.numel()
+    N = W.shape[0]
+    act = quantize_act(x_row.reshape(1, K))
+    g = 16 if t == Q6_K else 32
+    out = torch.empty((N, K // g), dtype=torch.int32, device=W.device)
+    check(load().mi355_block_dots_q8_1(_stream(), t, _ptr(W), _ptr(act), _ptr(out), N, K))
+    return out
+
+
+def mul_mat_id(t, as_dev, b, ids, n_used):
+    """as_dev uint8 [n_expert, N, row_bytes] device layout; b f32 [T, nb1, K]; ids int32 [T, >=n_used] (row-strided)
+    -> f32 [T, n_used, N]"""
+    import torch
+    n_expert, N, _ = as_dev.shape
+    T, nb1, K = b.shape
+    need = load().mi355_mul_mat_id_ws_bytes(K, n_expert, n_used, nb1, T)
+    ws = torch.empty(need, dtype=torch.uint8, device=b.device)
+    dst = torch.empty((T, n_used, N), dtype=torch.float32, device=b.device)
+    check(load().mi355_mul_mat_id(_stream(), t, _ptr(as_dev), _ptr(b), _ptr(ids), ids.stride(0), _ptr(dst), N, K,
+                                  n_expert, n_used, nb1, T, _ptr(ws), ws.numel()))
+    return dst
+
+
+def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, softcap=0.0):
+    """q f32 [Hq, Nq, D] (any head/row strides), k,v f16 [Hkv, Nkv, D], mask f16 [>=Nq, Nkv] or None -> f32 [Nq, Hq, D]"""
+    import torch
+    Hq, Nq, D = q.shape
+    Hkv, Nkv, _ = k.shape
+    assert q.stride(2) == 1 and k.stride(2) == 1 and v.stride(2) == 1
+    need = load().mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq)
+    ws = torch.empty(min(need, 1 << 28), dtype=torch.uint8, device=q.device)
+    dst = torch.empty((Nq, Hq, D), dtype=torch.float32, device=q.device)
+    check(load().mi355_flash_attn_ext(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(mask), _ptr(dst), D, Nq, Nkv, Hq, Hkv,
+                                      q.stride(1) * 4, q.stride(0) * 4, k.stride(1) * 2, k.stride(0) * 2,
+                                      v.stride(1) * 2, v.stride(0) * 2, mask.stride(0) * 2 if mask is not None else 0,
+                                      scale, max_bias, softcap, _ptr(ws), ws.numel()))
+    return dst

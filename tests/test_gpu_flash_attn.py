@@ -1,0 +1,93 @@
+"""GPU parity of FLASH_ATTN_EXT against the oracle's restatement of the reference CPU kernel,
+the textbook f64 form (which pins grouped-query heads), and the reference CPU backend."""
+import numpy as np
+import pytest
+
+import orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(rng, D, Nq, Nkv, Hq, Hkv, causal=True, rand_mask=False):
+    q = rng.standard_normal((Hq, Nq, D)).astype(np.float32)
+    k = rng.standard_normal((Hkv, Nkv, D)).astype(np.float16)
+    v = rng.standard_normal((Hkv, Nkv, D)).astype(np.float16)
+    nq_pad = (Nq + 63) // 64 * 64
+    mask = np.zeros((nq_pad, Nkv), dtype=np.float32)
+    if causal:
+        j = np.arange(Nkv)[None, :]
+        i = np.arange(nq_pad)[:, None]
+        mask = np.where(j <= Nkv - Nq + i, 0.0, -np.inf).astype(np.float32)
+        mask[Nq:] = -np.inf
+    if rand_mask:
+        mask = mask + rng.uniform(-1, 1, mask.shape).astype(np.float32)
+    return q, k, v, mask.astype(np.float16)
+
+
+def _run(dev, q, k, v, mask, scale, max_bias=0.0, softcap=0.0, llama_layout=False):
+    import torch
+    import mi355
+    Hq, Nq, D = q.shape
+    Hkv, Nkv, _ = k.shape
+    if llama_layout:
+        # q as permute(0,2,1,3) of [D, Hq, Nq]; k/v as views of a [cell][kv head][D] cache
+        qd = torch.from_numpy(np.ascontiguousarray(q.transpose(1, 0, 2))).to(dev).permute(1, 0, 2)
+        kd = torch.from_numpy(np.ascontiguousarray(k.transpose(1, 0, 2))).to(dev).permute(1, 0, 2)
+        vd = torch.from_numpy(np.ascontiguousarray(v.transpose(1, 0, 2))).to(dev).permute(1, 0, 2)
+    else:
+        qd, kd, vd = (torch.from_numpy(a).to(dev) for a in (q, k, v))
+    md = torch.from_numpy(mask).to(dev) if mask is not None else None
+    return mi355.flash_attn_ext(qd, kd, vd, md, scale, max_bias, softcap).cpu().numpy()
+
+
+@pytest.mark.parametrize("D", [64, 80, 128, 256])
+@pytest.mark.parametrize("Nq,Nkv", [(1, 512), (3, 96), (35, 1024)])
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (8, 2), (6, 3)])
+def test_small_shapes_vs_oracle(dev, D, Nq, Nkv, Hq, Hkv):
+    rng = np.random.default_rng(D + Nq + Nkv + Hq)
+    q, k, v, mask = _inputs(rng, D, Nq, Nkv, Hq, Hkv, causal=True, rand_mask=True)
+    scale = 1.0 / np.sqrt(D)
+    got = _run(dev, q, k, v, mask, scale)
+    f64 = orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale)
+    cpu = orc.flash_attn("cpu", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale)
+    assert orc.nmse(got, f64) < 1e-5          # only q's f16 rounding separates the two
+    assert orc.nmse(got, cpu) <= 5e-4         # tests/test-backend-ops.cpp:3137
+    if orc.ref is not None:
+        assert orc.nmse(got, orc.flash_attn("ref", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale)) <= 5e-4
+
+
+@pytest.mark.parametrize("max_bias,softcap", [(8.0, 0.0), (0.0, 10.0)])
+def test_alibi_and_softcap(dev, max_bias, softcap):
+    rng = np.random.default_rng(17)
+    q, k, v, mask = _inputs(rng, 128, 4, 256, 8, 8, causal=False, rand_mask=True)
+    scale = 1.0 / np.sqrt(128)
+    got = _run(dev, q, k, v, mask, scale, max_bias, softcap)
+    f64 = orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale, max_bias, softcap)
+    assert orc.nmse(got, f64) < 1e-5
+
+
+def test_no_mask(dev):
+    rng = np.random.default_rng(19)
+    q, k, v, _ = _inputs(rng, 128, 2, 300, 4, 1)
+    got = _run(dev, q, k, v, None, 0.1)
+    assert orc.nmse(got, orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), None, 0.1)) < 1e-5
+
+
+@pytest.mark.parametrize("Nq,Nkv", [(1, 512), (1, 4096), (1, 32768), (512, 512), (512, 4096)])
+def test_llama3_shapes(dev, Nq, Nkv):
+    """BASELINE config 2: 32 query heads over 8 kv heads, head size 128, causal, llama's strided layouts.
+    The oracle is evaluated on a slice of heads/queries (it is scalar C); GQA grouping is pinned by
+    the f64 form, which repeats each kv head over its 4 query heads."""
+    rng = np.random.default_rng(Nq + Nkv)
+    q, k, v, mask = _inputs(rng, 128, Nq, Nkv, 32, 8, causal=True)
+    scale = 1.0 / np.sqrt(128)
+    got = _run(dev, q, k, v, mask, scale, llama_layout=True)      # [Nq, 32, 128]
+    assert np.isfinite(got).all()
+    heads = [0, 5, 31]
+    rows = sorted(set([0, Nq // 2, Nq - 1]))
+    for h in heads:
+        qs = q[h:h + 1][:, rows]
+        ms = mask[rows]
+        ms = np.concatenate([ms, np.full((64 - len(rows), Nkv), -np.inf, dtype=np.float16)])
+        f64 = orc.flash_attn("f64", qs, k[h // 4:h // 4 + 1].view(np.uint16), v[h // 4:h // 4 + 1].view(np.uint16), ms.view(np.uint16), scale)
+        assert orc.nmse(got[rows][:, h:h + 1], f64) < 1e-5
