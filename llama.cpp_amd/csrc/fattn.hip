@@ -33,8 +33,11 @@ __device__ __forceinline__ float group_sum(float v) {
 __device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
     float s = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-        s = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a[i]), __builtin_bit_cast(f16x2, b[i]), s, false);
+    for (int i = 0; i < 4; i++) {
+        // copy the lanes out first: bit-casting a vector element expression directly reads element 0
+        const u32 ai = a[i], bi = b[i];
+        s = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, ai), __builtin_bit_cast(f16x2, bi), s, false);
+    }
     return s;
 }
 
@@ -126,7 +129,8 @@ __global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
         float vf[8];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const f16x2 h2 = __builtin_bit_cast(f16x2, vv[i]);
+            const u32 vi = vv[i];
+            const f16x2 h2 = __builtin_bit_cast(f16x2, vi);
             vf[2 * i] = (float)h2[0];
             vf[2 * i + 1] = (float)h2[1];
         }

@@ -135,4 +135,5 @@ def test_unaligned_rows_fallback(dev, name, t):
         x = rng.standard_normal((B, K)).astype(np.float32)
         Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
         got = mi355.mul_mat(t, Wd, _to_dev(dev, x)).cpu().numpy()
-        assert orc.nmse(got, orc.mul_mat("q8_1", t, Wq, x)) < 1e-9
+        # B > 8 with K % 128 == 0 takes the MFMA kernel, whose Q4_K min term goes through fp16 operands
+        assert orc.nmse(got, orc.mul_mat("q8_1", t, Wq, x)) < (1e-6 if (t == orc.Q4_K and B > 8) else 1e-9)
