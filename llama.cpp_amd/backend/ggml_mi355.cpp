@@ -1,0 +1,697 @@
+// ggml backend plug-in for one AMD Instinct MI355X (gfx950).
+//
+// This file is the drop-in boundary: it fills the five vtables of
+// ggml/src/ggml-backend-impl.h:17-207 (buffer type, buffer, backend, device, reg) and
+// exports ggml_backend_init / ggml_backend_score, the two symbols the registry dlsym()s
+// (ggml/src/ggml-backend-reg.cpp:229-245).  It is loaded through GGML_BACKEND_PATH or by
+// sitting next to the executable as libggml-<name>.so, so test-backend-ops, llama-bench and
+// llama-cli run on it unmodified.  All arithmetic lives behind the C ABI of
+// include/mi355_kernels.h; this file only routes ggml tensors to it.
+//
+// Conventions kept from the reference's backends:
+//  * work is declined in supports_op, never inside graph_compute;
+//  * tensor->data is a device address: get_base() + allocator offset, views included;
+//  * buffer set/get_tensor synchronise the device first, because the scheduler may read a
+//    result right after an asynchronous graph_compute (ggml/src/ggml-backend.cpp:243-252).
+//
+// Quantized tensors of type Q4_0 / Q8_0 / Q6_K live in HBM in the 16-byte-aligned row layout
+// described in mi355_kernels.h; set_tensor applies that byte permutation and get_tensor
+// undoes it, so every caller sees the reference's bytes.
+
+#include "ggml-backend-impl.h"
+#include "ggml-impl.h"
+#include "ggml.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "mi355_kernels.h"
+
+#define MI355_HIP_OK(expr)                                                                                      \
+    do {                                                                                                        \
+        hipError_t e_ = (expr);                                                                                 \
+        if (e_ != hipSuccess) GGML_ABORT("MI355: %s failed: %s", #expr, hipGetErrorString(e_));                 \
+    } while (0)
+
+#define MI355_K_OK(expr)                                                                                        \
+    do {                                                                                                        \
+        int rc_ = (expr);                                                                                       \
+        if (rc_ != MI355_OK) GGML_ABORT("MI355: %s failed (%d): %s", #expr, rc_, mi355_last_error());           \
+    } while (0)
+
+namespace {
+
+// ------------------------------------------------------------------------------- helpers
+bool is_repacked_type(ggml_type t) { return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K; }
+bool is_weight_type(ggml_type t) { return is_repacked_type(t) || t == GGML_TYPE_Q4_K; }
+
+int to_mi355_type(ggml_type t) {
+    switch (t) {
+        case GGML_TYPE_F32: return MI355_F32;
+        case GGML_TYPE_F16: return MI355_F16;
+        case GGML_TYPE_I32: return MI355_I32;
+        case GGML_TYPE_Q4_0: return MI355_Q4_0;
+        case GGML_TYPE_Q8_0: return MI355_Q8_0;
+        case GGML_TYPE_Q4_K: return MI355_Q4_K;
+        case GGML_TYPE_Q6_K: return MI355_Q6_K;
+        default: return -1;
+    }
+}
+
+mi355_tensor desc(const ggml_tensor * t) {
+    mi355_tensor d;
+    d.data = t->data;
+    d.type = to_mi355_type(t->type);
+    for (int i = 0; i < 4; i++) {
+        d.ne[i] = t->ne[i];
+        d.nb[i] = t->nb[i];
+    }
+    return d;
+}
+
+bool strides_mult16(const ggml_tensor * t) { return t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0; }
+
+// ------------------------------------------------------------------------------- device state
+struct device_ctx {
+    int device = 0;
+    std::string name;
+    std::string description;
+};
+
+struct backend_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    void * ws = nullptr;   // scratch for quantized activations / attention partials
+    size_t ws_size = 0;
+    std::string name;
+
+    void * workspace(size_t need) {
+        if (need > ws_size) {
+            if (ws) {
+                MI355_HIP_OK(hipStreamSynchronize(stream));   // kernels in flight may still read the old one
+                MI355_HIP_OK(hipFree(ws));
+            }
+            ws_size = (need + (size_t(32) << 20)) & ~((size_t(1) << 20) - 1);
+            MI355_HIP_OK(hipMalloc(&ws, ws_size));
+        }
+        return ws;
+    }
+};
+
+struct buffer_ctx {
+    int device = 0;
+    void * base = nullptr;
+    size_t size = 0;
+};
+
+ggml_backend_buffer_type_t mi355_buffer_type(int device);
+ggml_guid_t mi355_guid() {
+    static ggml_guid guid = { 0x4d, 0x49, 0x33, 0x35, 0x35, 0x58, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35, 0x30, 0x2d, 0x30, 0x31 };
+    return &guid;
+}
+
+// one staging buffer for layout-permuted uploads / read-backs (guarded: the model loader and the
+// compute thread may both call into buffers)
+struct staging {
+    std::mutex mu;
+    void * ptr = nullptr;
+    size_t size = 0;
+    void * get(size_t need) {
+        if (need > size) {
+            if (ptr) MI355_HIP_OK(hipFree(ptr));
+            size = (need + (size_t(1) << 20)) & ~((size_t(1) << 20) - 1);
+            MI355_HIP_OK(hipMalloc(&ptr, size));
+        }
+        return ptr;
+    }
+};
+staging & stage() {
+    static staging s;
+    return s;
+}
+
+// ------------------------------------------------------------------------------- buffer
+void buffer_free(ggml_backend_buffer_t buffer) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipDeviceSynchronize());
+    if (ctx->base) MI355_HIP_OK(hipFree(ctx->base));
+    delete ctx;
+}
+
+void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) buffer->context)->base; }
+
+// number of rows / elements per row of a tensor whose rows are contiguous blocks
+int64_t tensor_nrows(const ggml_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
+
+void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipDeviceSynchronize());
+    if (size == 0) return;
+    if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+        std::lock_guard<std::mutex> lock(stage().mu);
+        void * tmp = stage().get(size);
+        MI355_HIP_OK(hipMemcpy(tmp, data, size, hipMemcpyHostToDevice));
+        MI355_K_OK(mi355_weights_scatter(nullptr, to_mi355_type(tensor->type), tmp, tensor->data, tensor->ne[0], tensor_nrows(tensor), offset, size));
+        MI355_HIP_OK(hipDeviceSynchronize());
+    } else {
+        MI355_HIP_OK(hipMemcpy((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice));
+    }
+}
+
+void buffer_get_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * tensor, void * data, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipDeviceSynchronize());
+    if (size == 0) return;
+    if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+        std::lock_guard<std::mutex> lock(stage().mu);
+        void * tmp = stage().get(size);
+        MI355_K_OK(mi355_weights_gather(nullptr, to_mi355_type(tensor->type), tensor->data, tmp, tensor->ne[0], tensor_nrows(tensor), offset, size));
+        MI355_HIP_OK(hipMemcpy(data, tmp, size, hipMemcpyDeviceToHost));
+    } else {
+        MI355_HIP_OK(hipMemcpy(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost));
+    }
+}
+
+void buffer_memset_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, uint8_t value, size_t offset, size_t size) {
+    if (size == 0) return;
+    if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+        std::vector<uint8_t> host(size, value);   // rare path: route through the layout permutation
+        buffer_set_tensor(buffer, tensor, host.data(), offset, size);
+        return;
+    }
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipDeviceSynchronize());
+    MI355_HIP_OK(hipMemset((char *) tensor->data + offset, value, size));
+    MI355_HIP_OK(hipDeviceSynchronize());
+}
+
+bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, ggml_tensor * dst) {
+    // same buffer type on both sides: identical layouts (device layout included), plain device copy
+    if (src->buffer == nullptr || src->buffer->buft != buffer->buft) return false;
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipDeviceSynchronize());
+    MI355_HIP_OK(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyDeviceToDevice));
+    MI355_HIP_OK(hipDeviceSynchronize());
+    return true;
+}
+
+void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipDeviceSynchronize());
+    MI355_HIP_OK(hipMemset(ctx->base, value, ctx->size));
+    MI355_HIP_OK(hipDeviceSynchronize());
+}
+
+const ggml_backend_buffer_i buffer_iface = {
+    /* .free_buffer   = */ buffer_free,
+    /* .get_base      = */ buffer_get_base,
+    /* .init_tensor   = */ nullptr,
+    /* .memset_tensor = */ buffer_memset_tensor,
+    /* .set_tensor    = */ buffer_set_tensor,
+    /* .get_tensor    = */ buffer_get_tensor,
+    /* .cpy_tensor    = */ buffer_cpy_tensor,
+    /* .clear         = */ buffer_clear,
+    /* .reset         = */ nullptr,
+};
+
+// ------------------------------------------------------------------------------- buffer type
+const char * buft_get_name(ggml_backend_buffer_type_t buft) { return ((device_ctx *) buft->device->context)->name.c_str(); }
+
+ggml_backend_buffer_t buft_alloc_buffer(ggml_backend_buffer_type_t buft, size_t size) {
+    device_ctx * dctx = (device_ctx *) buft->device->context;
+    if (hipSetDevice(dctx->device) != hipSuccess) return nullptr;
+    buffer_ctx * ctx = new buffer_ctx;
+    ctx->device = dctx->device;
+    ctx->size = size;
+    // a little slack so 16-byte loads at the very end of the last tensor stay inside the allocation
+    hipError_t err = hipMalloc(&ctx->base, size + 256);
+    if (err != hipSuccess) {
+        (void) hipGetLastError();
+        GGML_LOG_ERROR("MI355: allocating %.2f MiB on device %d failed: %s\n", size / 1024.0 / 1024.0, dctx->device, hipGetErrorString(err));
+        delete ctx;
+        return nullptr;
+    }
+    return ggml_backend_buffer_init(buft, buffer_iface, ctx, size);
+}
+
+size_t buft_get_alignment(ggml_backend_buffer_type_t) { return 256; }
+
+size_t buft_get_max_size(ggml_backend_buffer_type_t buft) {
+    device_ctx * dctx = (device_ctx *) buft->device->context;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dctx->device) != hipSuccess) return SIZE_MAX;
+    return prop.totalGlobalMem;
+}
+
+const ggml_backend_buffer_type_i buft_iface = {
+    /* .get_name       = */ buft_get_name,
+    /* .alloc_buffer   = */ buft_alloc_buffer,
+    /* .get_alignment  = */ buft_get_alignment,
+    /* .get_max_size   = */ buft_get_max_size,
+    /* .get_alloc_size = */ nullptr,   // ggml_nbytes: the device layout keeps every tensor's footprint
+    /* .is_host        = */ nullptr,
+};
+
+// ------------------------------------------------------------------------------- op support
+bool f32_rows(const ggml_tensor * t) { return t->type == GGML_TYPE_F32 && t->nb[0] == sizeof(float); }
+
+bool supports_mul_mat(const ggml_tensor * op) {
+    const ggml_tensor * a = op->src[0];
+    const ggml_tensor * b = op->src[1];
+    if (op->type != GGML_TYPE_F32 || !ggml_is_contiguous(op)) return false;
+    if (b->type != GGML_TYPE_F32) return false;
+    if (is_weight_type(a->type)) {
+        // quantized weights: whole contiguous matrices; activations as 16-byte aligned f32 rows
+        if (!ggml_is_contiguous(a)) return false;
+        if (b->nb[0] != sizeof(float) || !strides_mult16(b)) return false;
+        if (b->ne[2] % a->ne[2] != 0 || b->ne[3] % a->ne[3] != 0) return false;
+        return b->ne[1] <= 65535;
+    }
+    if (a->type == GGML_TYPE_F32 || a->type == GGML_TYPE_F16) {
+        // dense weights (MoE router and other small matrices): any strides
+        if (b->ne[2] % a->ne[2] != 0 || b->ne[3] % a->ne[3] != 0) return false;
+        return op->ne[1] <= 65535 && op->ne[2] * op->ne[3] <= 65535;
+    }
+    return false;
+}
+
+bool supports_mul_mat_id(const ggml_tensor * op) {
+    const ggml_tensor * as = op->src[0];
+    const ggml_tensor * b = op->src[1];
+    const ggml_tensor * ids = op->src[2];
+    if (!is_weight_type(as->type) || !ggml_is_contiguous(as)) return false;
+    if (b->type != GGML_TYPE_F32 || !ggml_is_contiguous(b)) return false;
+    if (ids->type != GGML_TYPE_I32 || ids->nb[0] != sizeof(int32_t) || ids->nb[1] % sizeof(int32_t) != 0) return false;
+    if (op->type != GGML_TYPE_F32 || !ggml_is_contiguous(op)) return false;
+    if (as->ne[3] != 1 || b->ne[3] != 1 || ids->ne[2] != 1 || ids->ne[3] != 1) return false;
+    if (as->ne[0] % 4 != 0) return false;
+    return ids->ne[0] * ids->ne[1] <= 65535;
+}
+
+bool supports_flash_attn(const ggml_tensor * op) {
+    const ggml_tensor * q = op->src[0];
+    const ggml_tensor * k = op->src[1];
+    const ggml_tensor * v = op->src[2];
+    const ggml_tensor * mask = op->src[3];
+    if (q->type != GGML_TYPE_F32 || k->type != GGML_TYPE_F16 || v->type != GGML_TYPE_F16) return false;
+    if (q->nb[0] != 4 || k->nb[0] != 2 || v->nb[0] != 2) return false;
+    const int64_t D = q->ne[0];
+    if (!(D == 64 || D == 80 || D == 96 || D == 112 || D == 128 || D == 256) || k->ne[0] != D || v->ne[0] != D) return false;
+    if (!strides_mult16(q) || !strides_mult16(k) || !strides_mult16(v)) return false;
+    if (q->ne[2] % k->ne[2] != 0 || k->ne[2] != v->ne[2] || k->ne[1] != v->ne[1]) return false;
+    if (q->ne[3] != k->ne[3] || q->ne[3] != v->ne[3]) return false;
+    if (mask && (mask->type != GGML_TYPE_F16 || !ggml_is_contiguous(mask) || mask->ne[0] != k->ne[1])) return false;
+    if (!ggml_is_contiguous(op)) return false;
+    return q->ne[1] <= 65535 && q->ne[2] <= 65535;
+}
+
+bool device_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
+    switch (op->op) {
+        case GGML_OP_NONE:
+        case GGML_OP_RESHAPE:
+        case GGML_OP_VIEW:
+        case GGML_OP_PERMUTE:
+        case GGML_OP_TRANSPOSE:
+            return true;
+        case GGML_OP_MUL_MAT:
+            return supports_mul_mat(op);
+        case GGML_OP_MUL_MAT_ID:
+            return supports_mul_mat_id(op);
+        case GGML_OP_FLASH_ATTN_EXT:
+            return supports_flash_attn(op);
+        case GGML_OP_RMS_NORM:
+            return f32_rows(op->src[0]) && f32_rows(op);
+        case GGML_OP_ADD:
+        case GGML_OP_SUB:
+        case GGML_OP_MUL:
+        case GGML_OP_DIV:
+            return op->src[0]->type == GGML_TYPE_F32 && op->src[1]->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32;
+        case GGML_OP_UNARY:
+            if (op->src[0]->type != GGML_TYPE_F32 || op->type != GGML_TYPE_F32) return false;
+            switch (ggml_get_unary_op(op)) {
+                case GGML_UNARY_OP_ABS: case GGML_UNARY_OP_SGN: case GGML_UNARY_OP_NEG: case GGML_UNARY_OP_STEP:
+                case GGML_UNARY_OP_TANH: case GGML_UNARY_OP_ELU: case GGML_UNARY_OP_RELU: case GGML_UNARY_OP_SIGMOID:
+                case GGML_UNARY_OP_GELU: case GGML_UNARY_OP_GELU_QUICK: case GGML_UNARY_OP_SILU:
+                case GGML_UNARY_OP_HARDSWISH: case GGML_UNARY_OP_HARDSIGMOID: case GGML_UNARY_OP_EXP:
+                    return true;
+                default:
+                    return false;
+            }
+        case GGML_OP_SCALE:
+            return op->src[0]->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32;
+        case GGML_OP_CPY:
+        case GGML_OP_DUP:
+        case GGML_OP_CONT: {
+            const ggml_type st = op->src[0]->type;
+            const ggml_type dt = op->op == GGML_OP_CPY ? op->src[1]->type : op->type;
+            const bool sf = st == GGML_TYPE_F32 || st == GGML_TYPE_F16, df = dt == GGML_TYPE_F32 || dt == GGML_TYPE_F16;
+            return (sf && df) || (st == GGML_TYPE_I32 && dt == GGML_TYPE_I32);
+        }
+        case GGML_OP_GET_ROWS:
+            return (op->src[0]->type == GGML_TYPE_F32 || op->src[0]->type == GGML_TYPE_F16) && op->src[1]->type == GGML_TYPE_I32 &&
+                   op->type == GGML_TYPE_F32 && op->src[1]->ne[3] == 1;
+        case GGML_OP_SOFT_MAX: {
+            const ggml_tensor * mask = op->src[1];
+            if (!f32_rows(op->src[0]) || !ggml_is_contiguous(op)) return false;
+            if (mask && ((mask->type != GGML_TYPE_F32 && mask->type != GGML_TYPE_F16) || !ggml_is_contiguous(mask))) return false;
+            return true;
+        }
+        case GGML_OP_ROPE: {
+            const int mode = ((const int32_t *) op->op_params)[2];
+            if (mode != 0 && mode != GGML_ROPE_TYPE_NEOX) return false;   // no mrope / vision
+            if (!f32_rows(op->src[0]) || !f32_rows(op) || op->src[1]->type != GGML_TYPE_I32) return false;
+            if (op->src[2] && op->src[2]->type != GGML_TYPE_F32) return false;
+            return op->src[0]->ne[0] % 2 == 0;
+        }
+        case GGML_OP_SUM_ROWS:
+            return f32_rows(op->src[0]) && op->type == GGML_TYPE_F32;
+        case GGML_OP_ARGSORT:
+            return f32_rows(op->src[0]) && op->src[0]->ne[0] <= 1024 && ggml_is_contiguous(op);
+        default:
+            return false;
+    }
+}
+
+// ------------------------------------------------------------------------------- op execution
+void compute_mul_mat(backend_ctx * ctx, ggml_tensor * dst) {
+    const ggml_tensor * a = dst->src[0];
+    const ggml_tensor * b = dst->src[1];
+    if (!is_weight_type(a->type)) {
+        mi355_tensor da = desc(a), db = desc(b), dd = desc(dst);
+        MI355_K_OK(mi355_mul_mat_f(ctx->stream, &da, &db, &dd));
+        return;
+    }
+    const int64_t K = a->ne[0], N = a->ne[1], B = b->ne[1];
+    const int64_t r2 = b->ne[2] / a->ne[2], r3 = b->ne[3] / a->ne[3];
+    const size_t ws_bytes = mi355_mul_mat_ws_bytes(K, B);
+    void * ws = ctx->workspace(ws_bytes);
+    for (int64_t i3 = 0; i3 < b->ne[3]; i3++) {
+        for (int64_t i2 = 0; i2 < b->ne[2]; i2++) {
+            const char * W = (const char *) a->data + (i2 / r2) * a->nb[2] + (i3 / r3) * a->nb[3];
+            const float * x = (const float *) ((const char *) b->data + i2 * b->nb[2] + i3 * b->nb[3]);
+            float * y = (float *) ((char *) dst->data + i2 * dst->nb[2] + i3 * dst->nb[3]);
+            MI355_K_OK(mi355_mul_mat(ctx->stream, to_mi355_type(a->type), W, x, y, N, K, B, (int64_t) (b->nb[1] / sizeof(float)),
+                                     (int64_t) (dst->nb[1] / sizeof(float)), ws, ws_bytes));
+        }
+    }
+}
+
+void compute_mul_mat_id(backend_ctx * ctx, ggml_tensor * dst) {
+    const ggml_tensor * as = dst->src[0];
+    const ggml_tensor * b = dst->src[1];
+    const ggml_tensor * ids = dst->src[2];
+    const int64_t K = as->ne[0], N = as->ne[1], n_expert = as->ne[2];
+    const int64_t nb1 = b->ne[1], T = b->ne[2], n_used = ids->ne[0];
+    const size_t ws_bytes = mi355_mul_mat_id_ws_bytes(K, n_expert, n_used, nb1, T);
+    void * ws = ctx->workspace(ws_bytes);
+    MI355_K_OK(mi355_mul_mat_id(ctx->stream, to_mi355_type(as->type), as->data, (const float *) b->data, (const int32_t *) ids->data,
+                                (int64_t) (ids->nb[1] / sizeof(int32_t)), (float *) dst->data, N, K, n_expert, n_used, nb1, T, ws, ws_bytes));
+}
+
+void compute_flash_attn(backend_ctx * ctx, ggml_tensor * dst) {
+    const ggml_tensor * q = dst->src[0];
+    const ggml_tensor * k = dst->src[1];
+    const ggml_tensor * v = dst->src[2];
+    const ggml_tensor * mask = dst->src[3];
+    float scale, max_bias, softcap;
+    memcpy(&scale, (const float *) dst->op_params + 0, sizeof(float));
+    memcpy(&max_bias, (const float *) dst->op_params + 1, sizeof(float));
+    memcpy(&softcap, (const float *) dst->op_params + 2, sizeof(float));
+    const int64_t D = q->ne[0], Nq = q->ne[1], Hq = q->ne[2], Nkv = k->ne[1], Hkv = k->ne[2];
+    const size_t ws_bytes = mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq) < (size_t(256) << 20) ? mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq) : (size_t(256) << 20);
+    void * ws = ctx->workspace(ws_bytes);
+    for (int64_t i3 = 0; i3 < q->ne[3]; i3++) {
+        MI355_K_OK(mi355_flash_attn_ext(ctx->stream, (const float *) ((const char *) q->data + i3 * q->nb[3]), (const char *) k->data + i3 * k->nb[3],
+                                        (const char *) v->data + i3 * v->nb[3], mask ? mask->data : nullptr,
+                                        (float *) ((char *) dst->data + i3 * dst->nb[3]), D, Nq, Nkv, Hq, Hkv, q->nb[1], q->nb[2], k->nb[1], k->nb[2],
+                                        v->nb[1], v->nb[2], mask ? mask->nb[1] : 0, scale, max_bias, softcap, ws, ws_bytes));
+    }
+}
+
+void compute_node(backend_ctx * ctx, ggml_tensor * node) {
+    hipStream_t s = ctx->stream;
+    switch (node->op) {
+        case GGML_OP_MUL_MAT: compute_mul_mat(ctx, node); break;
+        case GGML_OP_MUL_MAT_ID: compute_mul_mat_id(ctx, node); break;
+        case GGML_OP_FLASH_ATTN_EXT: compute_flash_attn(ctx, node); break;
+        case GGML_OP_RMS_NORM: {
+            float eps;
+            memcpy(&eps, node->op_params, sizeof(float));
+            mi355_tensor a = desc(node->src[0]), d = desc(node);
+            MI355_K_OK(mi355_rms_norm(s, &a, &d, eps));
+        } break;
+        case GGML_OP_ADD: case GGML_OP_SUB: case GGML_OP_MUL: case GGML_OP_DIV: {
+            const int op = node->op == GGML_OP_ADD ? 0 : node->op == GGML_OP_SUB ? 1 : node->op == GGML_OP_MUL ? 2 : 3;
+            mi355_tensor a = desc(node->src[0]), b = desc(node->src[1]), d = desc(node);
+            MI355_K_OK(mi355_bin_bcast(s, op, &a, &b, &d));
+        } break;
+        case GGML_OP_UNARY: {
+            mi355_tensor a = desc(node->src[0]), d = desc(node);
+            MI355_K_OK(mi355_unary(s, (int) ggml_get_unary_op(node), &a, &d));
+        } break;
+        case GGML_OP_SCALE: {
+            float f;
+            memcpy(&f, node->op_params, sizeof(float));
+            mi355_tensor a = desc(node->src[0]), d = desc(node);
+            MI355_K_OK(mi355_scale(s, &a, &d, f));
+        } break;
+        case GGML_OP_CPY: {
+            mi355_tensor a = desc(node->src[0]), d = desc(node->src[1]);
+            MI355_K_OK(mi355_cpy(s, &a, &d));
+        } break;
+        case GGML_OP_DUP: case GGML_OP_CONT: {
+            mi355_tensor a = desc(node->src[0]), d = desc(node);
+            MI355_K_OK(mi355_cpy(s, &a, &d));
+        } break;
+        case GGML_OP_GET_ROWS: {
+            mi355_tensor a = desc(node->src[0]), i = desc(node->src[1]), d = desc(node);
+            MI355_K_OK(mi355_get_rows(s, &a, &i, &d));
+        } break;
+        case GGML_OP_SOFT_MAX: {
+            float scale, max_bias;
+            memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
+            memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
+            mi355_tensor a = desc(node->src[0]), d = desc(node), m;
+            if (node->src[1]) m = desc(node->src[1]);
+            MI355_K_OK(mi355_soft_max(s, &a, node->src[1] ? &m : nullptr, &d, scale, max_bias));
+        } break;
+        case GGML_OP_ROPE: {
+            const int32_t * p = (const int32_t *) node->op_params;
+            float freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
+            memcpy(&freq_base, p + 5, sizeof(float));
+            memcpy(&freq_scale, p + 6, sizeof(float));
+            memcpy(&ext_factor, p + 7, sizeof(float));
+            memcpy(&attn_factor, p + 8, sizeof(float));
+            memcpy(&beta_fast, p + 9, sizeof(float));
+            memcpy(&beta_slow, p + 10, sizeof(float));
+            mi355_tensor a = desc(node->src[0]), d = desc(node);
+            MI355_K_OK(mi355_rope(s, &a, (const int32_t *) node->src[1]->data, node->src[2] ? (const float *) node->src[2]->data : nullptr, &d,
+                                  p[1], p[2], p[4], freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow));
+        } break;
+        case GGML_OP_SUM_ROWS: {
+            mi355_tensor a = desc(node->src[0]), d = desc(node);
+            MI355_K_OK(mi355_sum_rows(s, &a, &d));
+        } break;
+        case GGML_OP_ARGSORT: {
+            mi355_tensor a = desc(node->src[0]), d = desc(node);
+            MI355_K_OK(mi355_argsort(s, &a, &d, ((const int32_t *) node->op_params)[0] == GGML_SORT_ORDER_DESC ? 1 : 0));
+        } break;
+        default:
+            GGML_ABORT("MI355: op %s reached graph_compute but is not supported (supports_op should have declined it)", ggml_op_name(node->op));
+    }
+}
+
+// ------------------------------------------------------------------------------- backend (stream)
+const char * backend_get_name(ggml_backend_t backend) { return ((backend_ctx *) backend->context)->name.c_str(); }
+
+void backend_free(ggml_backend_t backend) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    (void) hipSetDevice(ctx->device);
+    (void) hipStreamSynchronize(ctx->stream);
+    if (ctx->ws) (void) hipFree(ctx->ws);
+    if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
+    delete ctx;
+    delete backend;
+}
+
+void backend_synchronize(ggml_backend_t backend) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
+}
+
+ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    const int n = ggml_graph_n_nodes(cgraph);
+    for (int i = 0; i < n; i++) {
+        ggml_tensor * node = ggml_graph_node(cgraph, i);
+        if (ggml_is_empty(node)) continue;
+        switch (node->op) {
+            case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
+                continue;
+            default:
+                break;
+        }
+        compute_node(ctx, node);
+    }
+    return GGML_STATUS_SUCCESS;   // asynchronous: completion is observed through synchronize()
+}
+
+const ggml_backend_i backend_iface = {
+    /* .get_name           = */ backend_get_name,
+    /* .free               = */ backend_free,
+    /* .set_tensor_async   = */ nullptr,
+    /* .get_tensor_async   = */ nullptr,
+    /* .cpy_tensor_async   = */ nullptr,
+    /* .synchronize        = */ backend_synchronize,
+    /* .graph_plan_create  = */ nullptr,
+    /* .graph_plan_free    = */ nullptr,
+    /* .graph_plan_update  = */ nullptr,
+    /* .graph_plan_compute = */ nullptr,
+    /* .graph_compute      = */ backend_graph_compute,
+    /* .event_record       = */ nullptr,
+    /* .event_wait         = */ nullptr,
+};
+
+// ------------------------------------------------------------------------------- device
+const char * device_get_name(ggml_backend_dev_t dev) { return ((device_ctx *) dev->context)->name.c_str(); }
+const char * device_get_description(ggml_backend_dev_t dev) { return ((device_ctx *) dev->context)->description.c_str(); }
+
+void device_get_memory(ggml_backend_dev_t dev, size_t * free, size_t * total) {
+    device_ctx * ctx = (device_ctx *) dev->context;
+    *free = *total = 0;
+    if (hipSetDevice(ctx->device) == hipSuccess) (void) hipMemGetInfo(free, total);
+}
+
+enum ggml_backend_dev_type device_get_type(ggml_backend_dev_t) { return GGML_BACKEND_DEVICE_TYPE_GPU; }
+
+void device_get_props(ggml_backend_dev_t dev, ggml_backend_dev_props * props) {
+    props->name = device_get_name(dev);
+    props->description = device_get_description(dev);
+    props->type = GGML_BACKEND_DEVICE_TYPE_GPU;
+    device_get_memory(dev, &props->memory_free, &props->memory_total);
+    props->caps = { /* async */ false, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false };
+}
+
+ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
+    device_ctx * dctx = (device_ctx *) dev->context;
+    if (hipSetDevice(dctx->device) != hipSuccess) return nullptr;
+    backend_ctx * ctx = new backend_ctx;
+    ctx->device = dctx->device;
+    ctx->name = dctx->name;
+    if (hipStreamCreate(&ctx->stream) != hipSuccess) {   // default priority, blocking w.r.t. the null stream
+        delete ctx;
+        return nullptr;
+    }
+    return new ggml_backend{ mi355_guid(), backend_iface, dev, ctx };
+}
+
+ggml_backend_buffer_type_t device_get_buffer_type(ggml_backend_dev_t dev) { return mi355_buffer_type(((device_ctx *) dev->context)->device); }
+
+bool device_supports_buft(ggml_backend_dev_t dev, ggml_backend_buffer_type_t buft) {
+    return buft->iface.get_name == buft_get_name && buft->device == dev;
+}
+
+const ggml_backend_device_i device_iface = {
+    /* .get_name             = */ device_get_name,
+    /* .get_description      = */ device_get_description,
+    /* .get_memory           = */ device_get_memory,
+    /* .get_type             = */ device_get_type,
+    /* .get_props            = */ device_get_props,
+    /* .init_backend         = */ device_init_backend,
+    /* .get_buffer_type      = */ device_get_buffer_type,
+    /* .get_host_buffer_type = */ nullptr,
+    /* .buffer_from_host_ptr = */ nullptr,
+    /* .supports_op          = */ device_supports_op,
+    /* .supports_buft        = */ device_supports_buft,
+    /* .offload_op           = */ nullptr,
+    /* .event_new            = */ nullptr,
+    /* .event_free           = */ nullptr,
+    /* .event_synchronize    = */ nullptr,
+};
+
+// ------------------------------------------------------------------------------- reg
+struct reg_ctx {
+    std::vector<ggml_backend_device *> devices;
+    std::vector<ggml_backend_buffer_type *> bufts;
+};
+
+const char * reg_get_name(ggml_backend_reg_t) { return "MI355X"; }
+size_t reg_get_device_count(ggml_backend_reg_t reg) { return ((reg_ctx *) reg->context)->devices.size(); }
+ggml_backend_dev_t reg_get_device(ggml_backend_reg_t reg, size_t index) {
+    reg_ctx * ctx = (reg_ctx *) reg->context;
+    GGML_ASSERT(index < ctx->devices.size());
+    return ctx->devices[index];
+}
+void * reg_get_proc_address(ggml_backend_reg_t, const char *) { return nullptr; }
+
+const ggml_backend_reg_i reg_iface = {
+    /* .get_name         = */ reg_get_name,
+    /* .get_device_count = */ reg_get_device_count,
+    /* .get_device       = */ reg_get_device,
+    /* .get_proc_address = */ reg_get_proc_address,
+};
+
+// One GPU only: the first gfx950 device.  Lifetime of these objects is the process (the registry never unloads).
+ggml_backend_reg * the_reg() {
+    static ggml_backend_reg reg;
+    static reg_ctx ctx;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        int count = 0;
+        if (hipGetDeviceCount(&count) != hipSuccess) count = 0;
+        for (int d = 0; d < count && ctx.devices.empty(); d++) {
+            if (mi355_device_supported(d) != 1) continue;
+            hipDeviceProp_t prop;
+            if (hipGetDeviceProperties(&prop, d) != hipSuccess) continue;
+            device_ctx * dctx = new device_ctx;
+            dctx->device = d;
+            dctx->name = "MI355X" + std::to_string(ctx.devices.size());
+            dctx->description = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+            ggml_backend_device * dev = new ggml_backend_device{ device_iface, &reg, dctx };
+            ctx.devices.push_back(dev);
+            ctx.bufts.push_back(new ggml_backend_buffer_type{ buft_iface, dev, nullptr });
+        }
+        reg.api_version = GGML_BACKEND_API_VERSION;
+        reg.iface = reg_iface;
+        reg.context = &ctx;
+    });
+    return &reg;
+}
+
+ggml_backend_buffer_type_t mi355_buffer_type(int device) {
+    reg_ctx * ctx = (reg_ctx *) the_reg()->context;
+    for (size_t i = 0; i < ctx->devices.size(); i++)
+        if (((device_ctx *) ctx->devices[i]->context)->device == device) return ctx->bufts[i];
+    return nullptr;
+}
+
+}  // namespace
+
+// The two symbols the registry looks up (ggml/src/ggml-backend-reg.cpp:229-245); prototypes in include/ggml_mi355.h
+extern "C" {
+
+GGML_BACKEND_API ggml_backend_reg_t ggml_backend_init(void) { return the_reg(); }
+
+// 0 = "not supported on this system" (no gfx950 GPU visible); higher scores win among variants
+GGML_BACKEND_API int ggml_backend_score(void) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess) return 0;
+    for (int d = 0; d < count; d++)
+        if (mi355_device_supported(d) == 1) return 100;
+    return 0;
+}
+
+}
