@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Headline benchmark: llama-bench-style tg128 (and pp512) on a Llama-3-8B-shaped Q4_K_M model,
+all operators on one MI355X through the kernel C ABI (llama.cpp_amd/mi355/llama_graph.py issues
+the node sequence of llama.cpp's build_llama).
+
+One step = one decoded token (batch 1): upload of the token embedding, the 32-layer graph, the
+128256-wide logits and their read-back, then a device synchronise - what llama-bench's test_gen
+times per token (examples/llama-bench/llama-bench.cpp:1454-1468).  Weights are resident in HBM
+before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "llama.cpp_amd"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(n_threads, budget_s=20.0):
+    """ggml-cpu (the reference's own CPU backend, built by oracle/Makefile) timed on this host:
+    batch-1 MUL_MAT over the weight shapes of one Q4_K_M layer plus the output projection, scaled to
+    32 layers -> tokens/s of the matmul part of tg (the rest of the graph is a few percent on CPU)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import numpy as np
+    import orc
+    if orc.ref is None:
+        return None
+    rng = np.random.default_rng(1234)
+    shapes = [("wq", 4096, 4096, orc.Q4_K, 32), ("wk", 1024, 4096, orc.Q4_K, 32), ("wv", 1024, 4096, orc.Q4_K, 16),
+              ("wv6", 1024, 4096, orc.Q6_K, 16), ("wo", 4096, 4096, orc.Q4_K, 32), ("gate", 14336, 4096, orc.Q4_K, 32),
+              ("up", 14336, 4096, orc.Q4_K, 32), ("down", 4096, 14336, orc.Q4_K, 16), ("down6", 4096, 14336, orc.Q6_K, 16),
+              ("output", 128256, 4096, orc.Q6_K, 1)]
+    t_token = 0.0
+    t0 = time.time()
+    for name, N, K, t, count in shapes:
+        # random blocks with sane scales: the CPU kernels' time does not depend on the values
+        rb = orc.row_bytes(t, K)
+        W = rng.integers(0, 256, (N, rb), dtype=np.uint8)
+        bb = orc.BLOCK[t][1]
+        Wv = W.reshape(N, -1, bb)
+        h = np.array([1e-4], dtype=np.float16).view(np.uint8)
+        if t == orc.Q4_K:
+            Wv[:, :, 0:2] = h
+            Wv[:, :, 2:4] = h
+        else:
+            Wv[:, :, 208:210] = h
+        x = rng.standard_normal((1, K)).astype(np.float32)
+        out = np.zeros((1, N), dtype=np.float32)
+        reps = 3 if N > 20000 else 10
+        sec = orc.ref.ref_mul_mat(t, orc._ptr(W), orc._ptr(x), orc._ptr(out), N, K, 1, n_threads, reps)
+        t_token += sec * count
+        if time.time() - t0 > budget_s * 2:
+            break
+    return {"value": round(1.0 / t_token, 2), "unit": "tokens/s", "cores": n_threads, "kind": "reference",
+            "sample": "ggml-cpu (AVX2 build) batch-1 MUL_MAT over the 10 distinct weight shapes/types of the Q4_K_M model "
+                      "(3-10 runs each), summed with their per-token multiplicities (32 layers + output); matmuls only"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--no-graph", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not available" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import mi355
+    from mi355 import llama_graph as lg
+    lib = mi355.load()   # raises if the HIP library is missing: there is no CPU path to fall back to
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    cfg = lg.LlamaConfig()
+    n_ctx = max(512, (args.warmup + args.steps + 255) // 256 * 256, args.pp)
+    cfg.n_ctx = n_ctx
+    weights = lg.LlamaWeights(cfg, dev)
+    run = lg.LlamaRunner(weights, max_tokens=max(args.pp, 8))
+    emb = torch.randn(max(args.pp, 8), cfg.n_embd).pin_memory()
+    logits_host = torch.empty(cfg.n_vocab, dtype=torch.float32).pin_memory()
+    stream = torch.cuda.Stream()          # default priority; graph capture needs a non-default stream
+    torch.cuda.synchronize()
+
+    # ------------------------------------------------------------------ tg: K decode steps
+    graphs = {}
+
+    def decode_step(pos):
+        n_kv = (pos + 1 + 255) // 256 * 256          # llama.cpp pads n_kv to 256 with flash attention (src/llama.cpp:8565)
+        with torch.cuda.stream(stream):
+            run.x[:1].copy_(emb[pos % emb.shape[0]:pos % emb.shape[0] + 1], non_blocking=True)
+            run.pos[:1].fill_(pos)
+            run.mask[0, pos:pos + 1].fill_(0.0)
+            if args.no_graph:
+                run.forward(1, n_kv)
+            else:
+                g = graphs.get(n_kv)
+                if g is None:
+                    run.forward(1, n_kv)                 # warm every kernel once outside capture
+                    stream.synchronize()
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g, stream=stream):
+                        run.forward(1, n_kv)
+                    graphs[n_kv] = g
+                g.replay()
+            logits_host.copy_(run.logits[0], non_blocking=True)
+        stream.synchronize()
+
+    run.mask.fill_(float("-inf"))
+    for p in range(args.warmup):
+        decode_step(p)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for p in range(args.warmup, args.warmup + args.steps):
+        decode_step(p)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tg = args.steps / dt
+    finite = bool(torch.isfinite(logits_host).all())
+
+    # ------------------------------------------------------------------ pp512: one prefill batch
+    pp = None
+    if args.pp > 0:
+        T = args.pp
+        n_kv = (T + 255) // 256 * 256
+        with torch.cuda.stream(stream):
+            run.set_inputs(emb, 0, T, n_kv)
+            run.forward(T, n_kv)
+            stream.synchronize()
+            reps = 3
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                run.x[:T].copy_(emb[:T], non_blocking=True)
+                run.forward(T, n_kv)
+                logits_host.copy_(run.logits[0], non_blocking=True)
+                stream.synchronize()
+            pp = T * reps / (time.perf_counter() - t0)
+
+    # ------------------------------------------------------------------ roofline of the dominant kernel
+    # k_gemv_q<Q4_K, batch 1> on ffn_gate/ffn_up (14336 x 4096): 64 of the 226 matrices and 46% of the
+    # bytes of a decoded token.  Timed with HIP events on its own stream over the 64 distinct matrices
+    # (2.1 GB, so neither L2 nor the 256 MB Infinity Cache can serve them).
+    N, K = cfg.n_ff, cfg.n_embd
+    mats = [L[k][1] for L in weights.layers for k in ("gate", "up")]
+    x = torch.randn(1, K, device=dev)
+    act = mi355.quantize_act(x)
+    out = torch.empty(1, N, device=dev)
+    with torch.cuda.stream(stream):
+        for W in mats[:4]:
+            mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, mi355.Q4_K, W.data_ptr(), act.data_ptr(), out.data_ptr(), N, K, 1, N))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        nrep = 4
+        e0.record(stream)
+        for _ in range(nrep):
+            for W in mats:
+                mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, mi355.Q4_K, W.data_ptr(), act.data_ptr(), out.data_ptr(), N, K, 1, N))
+        e1.record(stream)
+        stream.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (nrep * len(mats))
+    alg_bytes = N * K * 144 // 256 + 4 * K + 4 * N          # weights + f32 activation + f32 output
+    achieved = alg_bytes / us / 1e3                          # GB/s
+    roofline = {"kernel": "k_gemv_q<Q4_K, ncols 1> 14336x4096 (ffn_gate / ffn_up)", "bound": "hbm", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "us_per_launch": round(us, 3), "algorithmic_bytes_per_launch": alg_bytes}
+
+    cpu = None
+    if not args.no_cpu:
+        try:
+            cpu = cpu_baseline(min(16, os.cpu_count() or 1))
+        except Exception as e:   # the baseline is a reported extra; never let it take the GPU numbers down
+            cpu = {"error": repr(e)}
+
+    weight_bytes = weights.matmul_bytes()
+    result = {
+        "metric": "tg128 tokens/s (Llama-3-8B-shaped Q4_K_M, batch 1, flash attention, all ops on device)",
+        "value": round(tg, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 block dots (Q4_K/Q6_K weights x Q8_1 activations), f32 accumulate, f16 KV cache",
+        "data": "synthetic: random Q4_K/Q6_K blocks scaled like N(0,0.02) weights, random embeddings",
+        "config": {"workload": "configs[3]: Llama-3-8B-shaped Q4_K_M decode (32 layers, d_model 4096, ffn 14336, 32/8 heads, "
+                               "head_dim 128, vocab 128256), KV positions %d..%d, n_kv padded to 256" % (args.warmup, args.warmup + args.steps - 1),
+                   "launch": "host" if args.no_graph else "hip-graph replay", "weight_bytes_per_token": weight_bytes,
+                   "hbm_fraction_of_step": round(weight_bytes / (ms_per_step * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)},
+        "pp512_tokens_per_s": round(pp, 1) if pp else None,
+        "outputs_finite": finite,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -148,6 +148,11 @@ int mi355_unary(void *stream, int op, const mi355_tensor *src, const mi355_tenso
 int mi355_scale(void *stream, const mi355_tensor *src, const mi355_tensor *dst, float s);
 /* ggml_compute_forward_dup (CPY/CONT/DUP, ggml-cpu.c:3519-3830): f32<->f16, f32->f32, f16->f16, i32->i32; any strides, same element count */
 int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
+/* KV-cache store: dst[:, rows[i], j] = convert(src[:, i, j]); src f32 [ne0, n, ne2], rows int32 [n] in DEVICE memory,
+ * dst f32/f16 [ne0, *, ne2].  Same result as the CPY into a view of the cache at row kv_head that llm_build_kv_store
+ * emits (src/llama.cpp:157-199; ggml_compute_forward_dup_f32, ggml-cpu.c:3519-3830), with the row taken from device
+ * memory so that a captured launch sequence does not change as the cache fills. */
+int mi355_set_rows(void *stream, const mi355_tensor *src, const int32_t *rows, const mi355_tensor *dst);
 /* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, ids i32 [n, b2, b3]; dst f32 */
 int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ids, const mi355_tensor *dst);
 /* ggml_compute_forward_soft_max_f32 (ggml-cpu.c:8959-9055): mask f32 or f16 or NULL */

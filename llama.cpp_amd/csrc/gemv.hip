@@ -87,6 +87,25 @@ __global__ void __launch_bounds__(256) k_gemv_id(const uint8_t *__restrict__ as,
     gemv_body<TYPE, 1, RPW>(as + ex * N * L.row_bytes, aq + arow * K, ads + arow * (K >> 5), dst + slot * N, N, K, N, L);
 }
 
+// Same routing for weight rows that are not 16-byte aligned (byte loads): one wave per (row, slot).
+template <int TYPE>
+__global__ void __launch_bounds__(64) k_gemv_id_unaligned(const uint8_t *__restrict__ as, const int8_t *__restrict__ aq,
+                                                          const act_ds *__restrict__ ads, const int32_t *__restrict__ ids,
+                                                          int64_t ids_stride, float *__restrict__ dst, int64_t N, int64_t K,
+                                                          int64_t n_expert, int64_t n_used, int64_t nb1, row_layout L) {
+    const int64_t row = blockIdx.x, slot = blockIdx.y, t = slot / n_used, e = slot % n_used;
+    int64_t ex = ids[t * ids_stride + e];
+    ex = ex < 0 ? 0 : (ex >= n_expert ? n_expert - 1 : ex);
+    const int64_t arow = t * nb1 + e % nb1;
+    const uint8_t *wrow = as + (ex * N + row) * L.row_bytes;
+    const int8_t *q = aq + arow * K;
+    const act_ds *ds = ads + arow * (K >> 5);
+    float acc = 0.0f;
+    for (int64_t i = threadIdx.x; i < K; i += 64) acc += weight_value<TYPE>(wrow, L, i) * (ds[i >> 5].d * (float)q[i]);
+    acc = wave_sum(acc);
+    if (threadIdx.x == 0) dst[slot * N + row] = acc;
+}
+
 // Parity dump of the integer granule dots (one wave per row, activation row 0).
 template <int TYPE>
 __global__ void __launch_bounds__(64) k_block_dots(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
@@ -214,11 +233,19 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
     MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_id: K=%lld is not a multiple of the block size", (long long)K);
     MI355_REQUIRE(n_used * T <= 65535, "mul_mat_id: too many expert slots for one launch");
     const row_layout L = make_row_layout(type, K);
-    MI355_REQUIRE(((uintptr_t)as & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0,
-                  "mul_mat_id: weight rows are not 16-byte aligned (K=%lld)", (long long)K);
     hipStream_t s = (hipStream_t)stream;
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + nb1 * T * K);
+    if (!(((uintptr_t)as & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0)) {
+        const dim3 ugrid((unsigned)N, (unsigned)(n_used * T));
+        switch (type) {
+            case MI355_Q4_0: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q4_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            case MI355_Q8_0: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q8_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            case MI355_Q4_K: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q4_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            default: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q6_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+        }
+        return launch_status("k_gemv_id_unaligned");
+    }
     const int rpw = pick_rpw(N) > 2 ? 2 : pick_rpw(N);
     const dim3 grid((unsigned)((N + 4 * rpw - 1) / (4 * rpw)), (unsigned)(n_used * T));
 #define MI355_ID_LAUNCH(TY)                                                                                           \

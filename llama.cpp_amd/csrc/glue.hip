@@ -156,6 +156,19 @@ __global__ void k_get_rows(tens src, tens ids, tens dst, int64_t n) {
     *(float *)(dst.data + i0 * dst.nb[0] + i1 * dst.nb[1] + i2 * dst.nb[2] + i3 * dst.nb[3]) = (float)v;
 }
 
+// ---------------------------------------------------------------- scatter rows (KV-cache store)
+// dst[:, rows[i1], i2] = convert(src[:, i1, i2]).  The KV-cache write of llm_build_kv_store
+// (src/llama.cpp:157-199) is a CPY into a view of the cache at row kv_head; here the target row
+// comes from device memory so a captured launch sequence stays valid as the cache fills.
+template <typename TD>
+__global__ void k_set_rows(tens src, const int32_t *__restrict__ rows, tens dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t i0 = i % src.ne[0], i1 = (i / src.ne[0]) % src.ne[1], i2 = i / (src.ne[0] * src.ne[1]);
+    const float v = *(const float *)(src.data + i0 * src.nb[0] + i1 * src.nb[1] + i2 * src.nb[2]);
+    *(TD *)(dst.data + i0 * dst.nb[0] + (int64_t)rows[i1] * dst.nb[1] + i2 * dst.nb[2]) = (TD)v;
+}
+
 // ---------------------------------------------------------------- SOFT_MAX
 // ggml_compute_forward_soft_max_f32, ggml-cpu.c:8959-9055.  mask row = row % ne1, contiguous.
 template <typename TM>
@@ -381,6 +394,17 @@ int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *id
     if (src->type == MI355_F32) hipLaunchKernelGGL(k_get_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
     else hipLaunchKernelGGL(k_get_rows<_Float16>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
     return launch_status("k_get_rows");
+}
+
+int mi355_set_rows(void *stream, const mi355_tensor *src, const int32_t *rows, const mi355_tensor *dst) {
+    MI355_REQUIRE(src->type == MI355_F32 && (dst->type == MI355_F32 || dst->type == MI355_F16), "set_rows: f32 -> f32/f16 only");
+    MI355_REQUIRE(src->ne[0] == dst->ne[0] && src->ne[2] == dst->ne[2] && src->ne[3] == 1 && dst->ne[3] == 1, "set_rows: shapes do not match");
+    const int64_t n = nelements(src);
+    if (n == 0) return MI355_OK;
+    const dim3 grid(grid1d(n, 256)), block(256);
+    if (dst->type == MI355_F16) hipLaunchKernelGGL(k_set_rows<_Float16>, grid, block, 0, (hipStream_t)stream, to_tens(src), rows, to_tens(dst), n);
+    else hipLaunchKernelGGL(k_set_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), rows, to_tens(dst), n);
+    return launch_status("k_set_rows");
 }
 
 int mi355_soft_max(void *stream, const mi355_tensor *src, const mi355_tensor *mask, const mi355_tensor *dst, float scale,

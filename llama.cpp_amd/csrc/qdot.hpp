@@ -240,6 +240,48 @@ __device__ __forceinline__ float combine_q6_K(const wchunk_q6_K &w, const act_ch
     return w.d * (w.scA * (A.d0 * (float)r.i0) + w.scB * (A.d1 * (float)r.i1));
 }
 
+// Dequantized weight element e of a row stored in device layout.  Byte loads only, so it
+// works for rows that are not 16-byte aligned (K not a multiple of 256 for Q4_0/Q8_0, of
+// 2048 for Q6_K).  Semantics: dequantize_row_* of ggml/src/ggml-quants.c:255-273, 349-363,
+// 1280-1302, 1690-1719.
+template <int TYPE>
+__device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, const row_layout &L, int64_t e) {
+    if constexpr (TYPE == MI355_Q4_0) {
+        const int64_t b = e >> 5;
+        const int j = (int)(e & 31);
+        const uint8_t byte = row[b * 16 + (j & 15)];
+        const int n = j < 16 ? (byte & 0x0F) : (byte >> 4);
+        const unsigned short dh = (unsigned short)(row[L.off_b + 2 * b] | (row[L.off_b + 2 * b + 1] << 8));
+        return half_bits_to_float(dh) * (float)(n - 8);
+    } else if constexpr (TYPE == MI355_Q8_0) {
+        const int64_t b = e >> 5;
+        const int8_t q = (int8_t)row[b * 32 + (e & 31)];
+        const unsigned short dh = (unsigned short)(row[L.off_b + 2 * b] | (row[L.off_b + 2 * b + 1] << 8));
+        return half_bits_to_float(dh) * (float)q;
+    } else if constexpr (TYPE == MI355_Q4_K) {
+        const int64_t sb = e >> 8;
+        const int r = (int)(e & 255), j = r >> 5, l = r & 31;
+        const uint8_t *blk = row + sb * Q4_K_BYTES;
+        const unsigned short dh = (unsigned short)(blk[0] | (blk[1] << 8)), mh = (unsigned short)(blk[2] | (blk[3] << 8));
+        const uint8_t *p = blk + 4;
+        int sc, mn;
+        if (j < 4) { sc = p[j] & 63; mn = p[j + 4] & 63; }
+        else { sc = (p[j + 4] & 0x0F) | ((p[j - 4] >> 6) << 4); mn = (p[j + 4] >> 4) | ((p[j] >> 6) << 4); }
+        const uint8_t byte = blk[16 + 32 * (j >> 1) + l];
+        const int n = (j & 1) ? (byte >> 4) : (byte & 0x0F);
+        return half_bits_to_float(dh) * (float)sc * (float)n - half_bits_to_float(mh) * (float)mn;
+    } else {
+        const int64_t sb = e >> 8;
+        const int r = (int)(e & 255), hf = r >> 7, quad = (r & 127) >> 5, l = r & 31;
+        const uint8_t lo = row[sb * 128 + 64 * hf + 32 * (quad & 1) + l];
+        const int nib = quad < 2 ? (lo & 0x0F) : (lo >> 4);
+        const int hi = (row[L.off_b + sb * 64 + 32 * hf + l] >> (2 * quad)) & 3;
+        const int8_t sc = (int8_t)row[L.off_c + sb * 16 + (r >> 4)];
+        const unsigned short dh = (unsigned short)(row[L.off_d + 2 * sb] | (row[L.off_d + 2 * sb + 1] << 8));
+        return half_bits_to_float(dh) * (float)sc * (float)((nib | (hi << 4)) - 32);
+    }
+}
+
 // ---------------------------------------------------------------- type dispatch
 template <int TYPE> struct wq;
 template <> struct wq<MI355_Q4_0> {

@@ -47,6 +47,7 @@ _SIGNATURES = {
     "mi355_unary": (_int, [_p, _int, C.POINTER(Tensor), C.POINTER(Tensor)]),
     "mi355_scale": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), _f]),
     "mi355_cpy": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor)]),
+    "mi355_set_rows": (_int, [_p, C.POINTER(Tensor), _p, C.POINTER(Tensor)]),
     "mi355_get_rows": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]),
     "mi355_soft_max": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor), _f, _f]),
     "mi355_rope": (_int, [_p, C.POINTER(Tensor), _p, _p, C.POINTER(Tensor), _int, _int, _int, _f, _f, _f, _f, _f, _f]),

@@ -1,0 +1,196 @@
+"""The llama decoder layer stack as llama.cpp's build_llama emits it (src/llama.cpp:1476-1640,
+llm_build_kv :157-199/:540-662, llm_build_ffn :200-330), driven straight through the kernel
+C ABI.  Measurement and parity harness: it issues, node for node, the kernel sequence the ggml
+backend plug-in issues for the same graph, without needing a GGUF file or the llama.cpp host.
+
+Weights are synthetic: random quantized blocks whose scales make the dequantized values look
+like N(0, 0.02) (generated on the device; kernel time does not depend on the values).
+The Q4_K_M tensor mix follows src/llama-quant.cpp:122-340: attn_v and ffn_down are Q6_K in the
+layers selected by use_more_bits(), the output projection is Q6_K, everything else Q4_K.
+"""
+import ctypes as C
+import math
+
+import torch
+
+from . import (F16, F32, I32, Q4_K, Q6_K, Q4_0, Q8_0, BLOCK, Tensor, check, load, row_bytes, tensor_desc, upload_weights,
+               _ptr, _stream)
+
+
+def use_more_bits(i_layer, n_layer):
+    """src/llama-quant.cpp:129-131"""
+    return i_layer < n_layer // 8 or i_layer >= 7 * n_layer // 8 or (i_layer - n_layer // 8) % 3 == 2
+
+
+class LlamaConfig:
+    def __init__(self, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, head_dim=128, n_vocab=128256,
+                 rope_theta=500000.0, rms_eps=1e-5, n_ctx=4096):
+        self.n_layer, self.n_embd, self.n_ff, self.n_head, self.n_head_kv = n_layer, n_embd, n_ff, n_head, n_head_kv
+        self.head_dim, self.n_vocab, self.rope_theta, self.rms_eps, self.n_ctx = head_dim, n_vocab, rope_theta, rms_eps, n_ctx
+
+
+def random_quantized(t, nrows, k, device, gen):
+    """Random blocks of type t in the reference block layout ([nrows, row_bytes] uint8), values ~ N(0, 0.02)-like."""
+    be, bb = BLOCK[t]
+    nb = k // be
+    raw = torch.randint(0, 256, (nrows, nb, bb), dtype=torch.uint8, device=device, generator=gen)
+
+    def put_half(col, value):
+        h = torch.tensor([value], dtype=torch.float16).view(torch.uint8)
+        raw[:, :, col] = h[0].item()
+        raw[:, :, col + 1] = h[1].item()
+
+    if t == Q4_K:      # w = d*sc*n - dmin*m, sc,m ~ U[0,63], n ~ U[0,15]
+        put_half(0, 0.02 / (31.5 * 4.6))
+        put_half(2, 0.02 / (31.5 * 4.6) * 7.5)
+    elif t == Q6_K:    # w = d*sc*(q-32), sc int8
+        put_half(208, 0.02 / (74.0 * 18.5))
+    elif t == Q4_0:    # w = d*(n-8)
+        put_half(0, 0.02 / 4.6)
+    elif t == Q8_0:
+        put_half(0, 0.02 / 74.0)
+    return raw.reshape(nrows, nb * bb)
+
+
+class LlamaWeights:
+    """device-layout weights of a Q4_K_M (or single-type) llama"""
+
+    def __init__(self, cfg, device, seed=1234, ftype="q4_k_m"):
+        gen = torch.Generator(device=device)
+        gen.manual_seed(seed)
+        self.cfg = cfg
+        E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
+        base = {"q4_k_m": Q4_K, "q4_0": Q4_0, "q8_0": Q8_0, "q4_k": Q4_K, "q6_k": Q6_K}[ftype]
+
+        def mk(t, n, k):
+            return t, upload_weights(t, random_quantized(t, n, k, device, gen))
+
+        self.layers = []
+        for il in range(cfg.n_layer):
+            more = ftype == "q4_k_m" and use_more_bits(il, cfg.n_layer)
+            L = {
+                "attn_norm": torch.ones(E, device=device) + 0.01 * torch.randn(E, device=device, generator=gen),
+                "ffn_norm": torch.ones(E, device=device) + 0.01 * torch.randn(E, device=device, generator=gen),
+                "wq": mk(base, H * D, E), "wk": mk(base, HK * D, E),
+                "wv": mk(Q6_K if more else base, HK * D, E), "wo": mk(base, E, H * D),
+                "gate": mk(base, F, E), "up": mk(base, F, E), "down": mk(Q6_K if more else base, E, F),
+            }
+            self.layers.append(L)
+        self.output_norm = torch.ones(E, device=device)
+        self.output = mk(Q6_K if ftype == "q4_k_m" else base, cfg.n_vocab, E)
+
+    def matmul_bytes(self):
+        """algorithmic weight bytes streamed per decoded token"""
+        n = 0
+        for L in self.layers:
+            for k in ("wq", "wk", "wv", "wo", "gate", "up", "down"):
+                n += L[k][1].numel()
+        return n + self.output[1].numel()
+
+
+class LlamaRunner:
+    """One sequence, f16 KV cache of n_ctx cells laid out [cell][kv head][head_dim] as llama-kv-cache.cpp:80-112."""
+
+    def __init__(self, weights, max_tokens=512):
+        self.w = weights
+        cfg = self.cfg = weights.cfg
+        dev = self.dev = weights.output[1].device
+        self.lib = load()
+        E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
+        T = self.max_tokens = max_tokens
+        f32 = dict(dtype=torch.float32, device=dev)
+        self.x = torch.zeros(T, E, **f32)          # residual stream / layer input
+        self.t0 = torch.zeros(T, E, **f32)
+        self.t1 = torch.zeros(T, E, **f32)
+        self.q = torch.zeros(T, H * D, **f32)
+        self.k = torch.zeros(T, HK * D, **f32)
+        self.v = torch.zeros(T, HK * D, **f32)
+        self.attn = torch.zeros(T, H * D, **f32)
+        self.gate = torch.zeros(T, F, **f32)
+        self.up = torch.zeros(T, F, **f32)
+        self.logits = torch.zeros(T, cfg.n_vocab, **f32)
+        self.kcache = [torch.zeros(cfg.n_ctx, HK, D, dtype=torch.float16, device=dev) for _ in range(cfg.n_layer)]
+        self.vcache = [torch.zeros(cfg.n_ctx, HK, D, dtype=torch.float16, device=dev) for _ in range(cfg.n_layer)]
+        self.pos = torch.zeros(T, dtype=torch.int32, device=dev)
+        self.mask = torch.zeros((T + 63) // 64 * 64, cfg.n_ctx, dtype=torch.float16, device=dev)
+        kmax = max(E, F, H * D)
+        self.ws = torch.empty(int(self.lib.mi355_mul_mat_ws_bytes(kmax, T)) + 256, dtype=torch.uint8, device=dev)
+        self.fa_ws = torch.empty(min(int(self.lib.mi355_flash_attn_ws_bytes(D, T, cfg.n_ctx, H)), 256 << 20), dtype=torch.uint8, device=dev)
+
+    # ---- single operators over the C ABI -------------------------------------------------------
+    def _mm(self, w, x, out, T):
+        t, W = w
+        N, K = out.shape[1], x.shape[1]
+        check(self.lib.mi355_mul_mat(_stream(), t, _ptr(W), _ptr(x), _ptr(out), N, K, T, x.stride(0), out.stride(0), _ptr(self.ws), self.ws.numel()))
+
+    def _norm(self, x, w, out, T):
+        dx, do, dw = tensor_desc(x[:T]), tensor_desc(out[:T]), tensor_desc(w)
+        check(self.lib.mi355_rms_norm(_stream(), C.byref(dx), C.byref(do), self.cfg.rms_eps))
+        check(self.lib.mi355_bin_bcast(_stream(), 2, C.byref(do), C.byref(dw), C.byref(do)))
+
+    def _bin(self, op, a, b, out):
+        da, db, do = tensor_desc(a), tensor_desc(b), tensor_desc(out)
+        check(self.lib.mi355_bin_bcast(_stream(), op, C.byref(da), C.byref(db), C.byref(do)))
+
+    def _rope(self, x, heads, T):
+        cfg = self.cfg
+        v = x[:T].view(T, heads, cfg.head_dim)
+        d = tensor_desc(v)
+        check(self.lib.mi355_rope(_stream(), C.byref(d), _ptr(self.pos), None, C.byref(d), cfg.head_dim, 0, cfg.n_ctx, cfg.rope_theta,
+                                  1.0, 0.0, 1.0, 32.0, 1.0))
+
+    def _kv_store(self, src, cache, T):
+        cfg = self.cfg
+        s = tensor_desc(src[:T].view(T, cfg.n_head_kv * cfg.head_dim))
+        d = tensor_desc(cache.view(cfg.n_ctx, cfg.n_head_kv * cfg.head_dim))
+        check(self.lib.mi355_set_rows(_stream(), C.byref(s), _ptr(self.pos), C.byref(d)))
+
+    def _attn(self, il, T, n_kv):
+        cfg = self.cfg
+        H, HK, D = cfg.n_head, cfg.n_head_kv, cfg.head_dim
+        q = self.q[:T].view(T, H, D)
+        kc, vc = self.kcache[il], self.vcache[il]
+        check(self.lib.mi355_flash_attn_ext(_stream(), _ptr(q), _ptr(kc), _ptr(vc), _ptr(self.mask), _ptr(self.attn), D, T, n_kv, H, HK,
+                                            q.stride(0) * 4, q.stride(1) * 4, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2,
+                                            vc.stride(1) * 2, self.mask.stride(0) * 2, 1.0 / math.sqrt(D), 0.0, 0.0, _ptr(self.fa_ws),
+                                            self.fa_ws.numel()))
+
+    # ---- one forward pass over T tokens whose inputs (x, pos, mask) are already on the device --
+    def forward(self, T, n_kv, last_only=True):
+        cfg, w = self.cfg, self.w
+        x = self.x
+        for il, L in enumerate(w.layers):
+            self._norm(x, L["attn_norm"], self.t0, T)
+            self._mm(L["wq"], self.t0[:T], self.q[:T], T)
+            self._mm(L["wk"], self.t0[:T], self.k[:T], T)
+            self._mm(L["wv"], self.t0[:T], self.v[:T], T)
+            self._rope(self.q, cfg.n_head, T)
+            self._rope(self.k, cfg.n_head_kv, T)
+            self._kv_store(self.k, self.kcache[il], T)
+            self._kv_store(self.v, self.vcache[il], T)
+            self._attn(il, T, n_kv)
+            self._mm(L["wo"], self.attn[:T], self.t1[:T], T)
+            self._bin(0, self.t1[:T], x[:T], x[:T])                      # ffn_inp = attn_out + inpSA
+            self._norm(x, L["ffn_norm"], self.t0, T)
+            self._mm(L["gate"], self.t0[:T], self.gate[:T], T)
+            self._mm(L["up"], self.t0[:T], self.up[:T], T)
+            dg = tensor_desc(self.gate[:T])
+            check(self.lib.mi355_unary(_stream(), 10, C.byref(dg), C.byref(dg)))     # SILU
+            self._bin(2, self.gate[:T], self.up[:T], self.gate[:T])
+            self._mm(L["down"], self.gate[:T], self.t1[:T], T)
+            self._bin(0, self.t1[:T], x[:T], x[:T])
+        To = 1 if last_only else T
+        xo = x[T - 1:T] if last_only else x[:T]
+        self._norm(xo, w.output_norm, self.t0, To)
+        self._mm(w.output, self.t0[:To], self.logits[:To], To)
+        return self.logits[:To]
+
+    # ---- host-side inputs, as llama_set_inputs fills them (src/llama-context.cpp:61-200) --------
+    def set_inputs(self, emb_host, pos0, T, n_kv):
+        """emb_host: pinned f32 [T, n_embd]; tokens occupy cache cells pos0 .. pos0+T-1"""
+        self.x[:T].copy_(emb_host[:T], non_blocking=True)
+        self.pos[:T].copy_(torch.arange(pos0, pos0 + T, dtype=torch.int32), non_blocking=False)
+        m = torch.full((self.mask.shape[0], n_kv), float("-inf"), dtype=torch.float16)
+        for i in range(T):
+            m[i, :pos0 + i + 1] = 0.0
+        self.mask[:, :n_kv].copy_(m, non_blocking=False)
