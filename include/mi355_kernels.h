@@ -89,6 +89,21 @@ int mi355_mul_mat_vec_q(void *stream, int type, const void *W, const void *act, 
 int mi355_mul_mat_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
                     int64_t dst_stride);
 
+/* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
+ * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE
+ * launch, each optionally adding a residual in its epilogue (the ggml_add that follows the wo and
+ * ffn_down products, src/llama.cpp:1566, :1609): dst_i[b][n] = W_i[n] . x[b] (+ residual_i[b][n]).
+ * residual has dst's shape and stride and may alias dst.  B <= 8. */
+typedef struct mi355_gemv_mat {
+    int          type;        /* weight type of this matrix */
+    const void  *W;           /* N rows x K, device layout */
+    int64_t      N;
+    float       *dst;
+    int64_t      dst_stride;
+    const float *residual;    /* NULL for none */
+} mi355_gemv_mat;
+int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B);
+
 /* Integer sub-block dots, for parity checking the kernels' inner products bit-for-bit
  * against ggml_vec_dot_q4_0_q8_0 / q8_0_q8_0 / q4_K_q8_K / q6_K_q8_K
  * (ggml/src/ggml-cpu/ggml-cpu-quants.c:2492-2506, 3919-3927, 6817-6848, 8262-8283).
@@ -166,6 +181,26 @@ int mi355_rope(void *stream, const mi355_tensor *src, const int32_t *pos, const 
 int mi355_sum_rows(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
 /* ggml_compute_forward_argsort_f32 (ggml-cpu.c:10857): order 0 ascending, 1 descending; ne[0] <= 1024 */
 int mi355_argsort(void *stream, const mi355_tensor *src, const mi355_tensor *dst, int order);
+/* Fused node sequences --------------------------------------------------------------- *
+ * Each does the work of the consecutive graph nodes named, with the same arithmetic; where the
+ * consumer is a quantized MUL_MAT the Q8_1 activation (split layout of mi355_quantize_act,
+ * quantize_row_q8_1_ref arithmetic) is produced in the same pass.  y and act are optional (NULL). */
+
+/* llm_build_norm: RMS_NORM then MUL by the norm weight (src/llama.cpp:1499-1503; ggml-cpu.c:7015-7061, 5142-5211).
+ * x f32 rows of k (row stride x_stride elements), w f32 [k] or NULL, y f32 rows (y_stride). k <= 16384. */
+int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride,
+                             void *act, int64_t k, int64_t nrows, float eps);
+/* llm_build_ffn LLM_FFN_SILU + LLM_FFN_PAR: UNARY(SILU)(gate) then MUL by up (src/llama.cpp:280-320; ggml-cpu.c:6646-6683). */
+int mi355_swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
+                       int64_t k, int64_t nrows);
+/* ROPE(q), ROPE(k), CPY(k -> K cache), CPY(v -> V cache) of build_llama + llm_build_kv_store (src/llama.cpp:1535-1548, :157-199;
+ * ggml-cpu.c:9366-9549, 3519-3830).  q f32 [T][H][D] is rotated in place; k, v f32 [T][HK][D] are read; the f16 caches are addressed
+ * as cell*nb1 + head*nb2 + 2*d with the cell of token t taken from cells[t] and its rope position from pos[t] (both DEVICE int32). */
+int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, void *kcache, void *vcache, const int32_t *pos,
+                        const int32_t *cells, const float *freq_factors, int64_t T, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
+                        size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                        float ext_factor, float attn_factor, float beta_fast, float beta_slow);
+
 /* MUL_MAT with f32 or f16 src0 and f32 src1 (router / small dense matrices): dst[b][n] = sum_k W[n][k] x[b][k], strides honoured, ne2/ne3 broadcast */
 int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *src1, const mi355_tensor *dst);
 

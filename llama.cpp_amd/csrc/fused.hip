@@ -1,0 +1,229 @@
+// Fused forms of the glue sequences llama.cpp's graph emits between the matrix products.
+// A decoded token is ~800 graph nodes whose useful work is a few microseconds each; what they
+// cost is launches and HBM round trips of 16 KB vectors.  Each kernel here does the work of two
+// to four consecutive nodes and, where the consumer is a quantized MUL_MAT, also emits the
+// Q8_1 activation (same arithmetic as k_quantize_q8_1, i.e. quantize_row_q8_1_ref), so the
+// separate quantization launch disappears:
+//   RMS_NORM -> MUL(weight) [-> Q8_1]            k_rms_norm_mul_quant
+//   UNARY(SILU) -> MUL(up)  [-> Q8_1]            k_swiglu_quant
+//   ROPE(q), ROPE(k), CPY(k -> cache), CPY(v -> cache)   k_rope_kv_store
+#include "common.hpp"
+
+namespace mi355 {
+
+// Q8_1 of the 4 values held by each of 8 neighbouring lanes (one 32-element block); writes the
+// split activation layout.  Mirrors k_quantize_q8_1 (quantize.hip) instruction for instruction.
+__device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, int8_t *__restrict__ qplane, act_ds *__restrict__ ds,
+                                                    int64_t row, int64_t k, int64_t e0) {
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    int q[4];
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        q[i] = (int)roundf(v[i] * id);
+        sum += q[i];
+    }
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (!live) return;
+    const u32 packed = (u32)(q[0] & 0xFF) | ((u32)(q[1] & 0xFF) << 8) | ((u32)(q[2] & 0xFF) << 16) | ((u32)(q[3] & 0xFF) << 24);
+    *(u32 *)(qplane + row * k + e0) = packed;
+    if (((e0 >> 2) & 7) == 0) {
+        act_ds o;
+        o.d = half_bits_to_float(float_to_half_bits(d));
+        o.sum = sum;
+        ds[row * (k >> 5) + (e0 >> 5)] = o;
+    }
+}
+
+// one 256-thread group per row; each thread keeps its NV float4 of the row in registers
+template <int NV>
+__global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restrict__ x, int64_t x_stride, const float *__restrict__ w,
+                                                            float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k,
+                                                            int64_t nrows, float eps) {
+    __shared__ float sh[4];
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const float *xr = x + row * x_stride;
+    f32x4 v[NV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int it = 0; it < NV; it++) {
+        const int64_t e0 = ((int64_t)it * 256 + tid) * 4;
+        v[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (e0 < k) v[it] = *(const f32x4 *)(xr + e0);
+        ss += v[it][0] * v[it][0] + v[it][1] * v[it][1] + v[it][2] * v[it][2] + v[it][3] * v[it][3];
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) sh[tid >> 6] = ss;
+    __syncthreads();
+    ss = sh[0] + sh[1] + sh[2] + sh[3];
+    const float scale = 1.0f / sqrtf(ss / (float)k + eps);
+    int8_t *qplane = (int8_t *)act;
+    act_ds *ds = (act_ds *)(qplane + nrows * k);
+#pragma unroll
+    for (int it = 0; it < NV; it++) {
+        const int64_t e0 = ((int64_t)it * 256 + tid) * 4;
+        const bool live = e0 < k;
+        f32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = v[it][i] * scale;
+        if (w && live) {
+            const f32x4 ww = *(const f32x4 *)(w + e0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = o[i] * ww[i];
+        }
+        if (y && live) *(f32x4 *)(y + row * y_stride + e0) = o;
+        if (act) quantize_block_lane(o, live, qplane, ds, row, k, e0);
+    }
+}
+
+// h = silu(gate) * up, optional f32 output, optional Q8_1 output; one lane per 4 elements
+__global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ gate, const float *__restrict__ up, int64_t in_stride,
+                                                      float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k,
+                                                      int64_t nrows) {
+    const int64_t row = blockIdx.y;
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const bool live = e0 < k;
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        const f32x4 g = *(const f32x4 *)(gate + row * in_stride + e0);
+        const f32x4 u = *(const f32x4 *)(up + row * in_stride + e0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = (g[i] / (1.0f + expf(-g[i]))) * u[i];
+        if (y) *(f32x4 *)(y + row * y_stride + e0) = o;
+    }
+    if (act) {
+        int8_t *qplane = (int8_t *)act;
+        quantize_block_lane(o, live, qplane, (act_ds *)(qplane + nrows * k), row, k, e0);
+    }
+}
+
+struct rope_kv_args {
+    float *q;               // [T][H][D] f32, rotated in place
+    const float *k;         // [T][HK][D] f32
+    const float *v;         // [T][HK][D] f32
+    uint8_t *kcache, *vcache;   // f16; element (cell, head, d) at cell*nb1 + head*nb2 + 2*d
+    const int32_t *pos;     // [T] rope positions
+    const int32_t *cells;   // [T] cache cell of each token
+    const float *ff;        // rope frequency factors [n_dims/2] or null
+    int64_t k_nb1, k_nb2, v_nb1, v_nb2;
+    int T, H, HK, D, n_dims, mode;
+    float theta_scale, freq_scale, ext_factor, attn_factor, corr0, corr1;
+};
+
+// rope_yarn + rotation as in k_rope (glue.hip) / ggml-cpu.c:9268-9306
+__device__ __forceinline__ void rope_pair(const rope_kv_args &a, int pos, int pair, float x0, float x1, float &y0, float &y1) {
+    const float theta_extrap = (float)pos * powf(a.theta_scale, (float)pair) / (a.ff ? a.ff[pair] : 1.0f);
+    const float theta_interp = a.freq_scale * theta_extrap;
+    float theta = theta_interp, mscale = a.attn_factor;
+    if (a.ext_factor != 0.0f) {
+        const float yv = ((float)pair - a.corr0) / fmaxf(0.001f, a.corr1 - a.corr0);
+        const float ramp = (1.0f - fminf(1.0f, fmaxf(0.0f, yv))) * a.ext_factor;
+        theta = theta_interp * (1.0f - ramp) + theta_extrap * ramp;
+        mscale *= 1.0f + 0.1f * logf(1.0f / a.freq_scale);
+    }
+    const float c = cosf(theta) * mscale, s = sinf(theta) * mscale;
+    y0 = x0 * c - x1 * s;
+    y1 = x0 * s + x1 * c;
+}
+
+// grid (H + 2*HK, T), D/2 threads: heads [0,H) rotate q in place, [H,H+HK) rotate k into the cache,
+// [H+HK, H+2HK) copy v into the cache
+__global__ void k_rope_kv_store(rope_kv_args a) {
+    const int t = blockIdx.y, h = blockIdx.x, pair = threadIdx.x;
+    const int D = a.D;
+    if (2 * pair >= D) return;
+    const bool neox = (a.mode & 2) != 0;
+    const int i0 = 2 * pair;
+    const bool rot = i0 < a.n_dims;
+    const int ia = (rot && neox) ? pair : i0, ib = (rot && neox) ? pair + a.n_dims / 2 : i0 + 1;
+    if (h < a.H) {
+        float *p = a.q + ((int64_t)t * a.H + h) * D;
+        const float x0 = p[ia], x1 = p[ib];
+        float y0 = x0, y1 = x1;
+        if (rot) rope_pair(a, a.pos[t], pair, x0, x1, y0, y1);
+        p[ia] = y0;
+        p[ib] = y1;
+    } else if (h < a.H + a.HK) {
+        const int hk = h - a.H;
+        const float *p = a.k + ((int64_t)t * a.HK + hk) * D;
+        const float x0 = p[ia], x1 = p[ib];
+        float y0 = x0, y1 = x1;
+        if (rot) rope_pair(a, a.pos[t], pair, x0, x1, y0, y1);
+        _Float16 *c = (_Float16 *)(a.kcache + (int64_t)a.cells[t] * a.k_nb1 + (int64_t)hk * a.k_nb2);
+        c[ia] = (_Float16)y0;
+        c[ib] = (_Float16)y1;
+    } else {
+        const int hk = h - a.H - a.HK;
+        const float *p = a.v + ((int64_t)t * a.HK + hk) * D;
+        _Float16 *c = (_Float16 *)(a.vcache + (int64_t)a.cells[t] * a.v_nb1 + (int64_t)hk * a.v_nb2);
+        c[i0] = (_Float16)p[i0];
+        c[i0 + 1] = (_Float16)p[i0 + 1];
+    }
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
+                             int64_t k, int64_t nrows, float eps) {
+    MI355_REQUIRE(k > 0 && k % 32 == 0 && k <= 16384, "rms_norm_mul_quant: k=%lld must be a multiple of 32 and at most 16384", (long long)k);
+    MI355_REQUIRE(nrows >= 0 && nrows < 0x7fffffff, "rms_norm_mul_quant: bad row count");
+    MI355_REQUIRE(((uintptr_t)x & 15) == 0 && x_stride % 4 == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0 && y_stride % 4 == 0 &&
+                  ((uintptr_t)act & 15) == 0, "rms_norm_mul_quant: operands must be 16-byte aligned");
+    MI355_REQUIRE(y != nullptr || act != nullptr, "rms_norm_mul_quant: no output requested");
+    if (nrows == 0) return MI355_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)nrows), block(256);
+    if (k <= 4096) hipLaunchKernelGGL(k_rms_norm_mul_quant<4>, grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);
+    else if (k <= 8192) hipLaunchKernelGGL(k_rms_norm_mul_quant<8>, grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);
+    else hipLaunchKernelGGL(k_rms_norm_mul_quant<16>, grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);
+    return launch_status("k_rms_norm_mul_quant");
+}
+
+int mi355_swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
+                       int64_t k, int64_t nrows) {
+    MI355_REQUIRE(k > 0 && k % 32 == 0, "swiglu_quant: k=%lld must be a multiple of 32", (long long)k);
+    MI355_REQUIRE(nrows >= 0 && nrows <= 65535, "swiglu_quant: bad row count");
+    MI355_REQUIRE(((uintptr_t)gate & 15) == 0 && ((uintptr_t)up & 15) == 0 && in_stride % 4 == 0 && ((uintptr_t)y & 15) == 0 && y_stride % 4 == 0 &&
+                  ((uintptr_t)act & 15) == 0, "swiglu_quant: operands must be 16-byte aligned");
+    MI355_REQUIRE(y != nullptr || act != nullptr, "swiglu_quant: no output requested");
+    if (nrows == 0) return MI355_OK;
+    hipLaunchKernelGGL(k_swiglu_quant, dim3((unsigned)((k + 1023) / 1024), (unsigned)nrows), dim3(256), 0, (hipStream_t)stream, gate, up,
+                       in_stride, y, y_stride, act, k, nrows);
+    return launch_status("k_swiglu_quant");
+}
+
+int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, void *kcache, void *vcache, const int32_t *pos,
+                        const int32_t *cells, const float *freq_factors, int64_t T, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
+                        size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                        float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
+    MI355_REQUIRE(T > 0 && T <= 65535 && H > 0 && HK > 0 && D > 0 && D % 2 == 0 && D <= 2048, "rope_kv_store: bad shape");
+    MI355_REQUIRE(mode == 0 || mode == 2, "rope_kv_store: mode %d not supported (0 = adjacent pairs, 2 = NeoX)", mode);
+    MI355_REQUIRE(n_dims > 0 && n_dims % 2 == 0 && n_dims <= D, "rope_kv_store: bad n_dims");
+    rope_kv_args a;
+    a.q = q; a.k = k; a.v = v; a.kcache = (uint8_t *)kcache; a.vcache = (uint8_t *)vcache;
+    a.pos = pos; a.cells = cells; a.ff = freq_factors;
+    a.k_nb1 = (int64_t)k_nb1; a.k_nb2 = (int64_t)k_nb2; a.v_nb1 = (int64_t)v_nb1; a.v_nb2 = (int64_t)v_nb2;
+    a.T = (int)T; a.H = (int)H; a.HK = (int)HK; a.D = (int)D; a.n_dims = n_dims; a.mode = mode;
+    a.theta_scale = powf(freq_base, -2.0f / n_dims);
+    a.freq_scale = freq_scale; a.ext_factor = ext_factor; a.attn_factor = attn_factor;
+    const float pi = 3.14159265358979323846f;   // ggml_rope_yarn_corr_dims, ggml/src/ggml.c:3695-3707
+    const float c0 = floorf(n_dims * logf(n_ctx_orig / (beta_fast * 2 * pi)) / (2 * logf(freq_base)));
+    const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
+    a.corr0 = c0 > 0 ? c0 : 0;
+    a.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
+    const int threads = (int)((D / 2 + 63) / 64 * 64);
+    hipLaunchKernelGGL(k_rope_kv_store, dim3((unsigned)(H + 2 * HK), (unsigned)T), dim3(threads), 0, (hipStream_t)stream, a);
+    return launch_status("k_rope_kv_store");
+}
+
+}  // extern "C"

@@ -1,11 +1,14 @@
-// Bandwidth-bound quantized GEMV (batch 1..8): dst[b][n] = sum_k W[n][k] * x[b][k].
+// Bandwidth-bound quantized GEMV (batch 1..8): dst[b][n] = sum_k W[n][k] * x[b][k] (+ residual).
 //
-// One wave owns RPW consecutive weight rows and walks them in steps of 64 chunks
-// (2048 elements): every lane issues one or two 16-byte streaming loads per row per step,
-// to consecutive addresses across the wave, so HBM sees long linear bursts.  The
-// activation chunk (already Q8_1-quantized, L2 resident) is loaded once per step and
-// reused for all RPW rows and all NCOLS activation rows.  Integer dots use v_dot4_i32_i8;
-// scales are applied in f32; the wave reduces with cross-lane shuffles.
+// One wave owns RPW consecutive weight rows and walks them in steps of 64 chunks: every lane
+// issues 16-byte streaming loads to consecutive addresses across the wave, so HBM sees long
+// linear bursts.  The activation chunk (already Q8_1-quantized, L2 resident) is loaded once
+// per step and reused for all RPW rows and all NCOLS activation rows.  Integer dots use
+// v_dot4_i32_i8; scales are applied in f32; the wave reduces with cross-lane shuffles.
+//
+// One launch can serve up to four weight matrices that share the activation (Q/K/V, gate/up):
+// the groups of all matrices are laid end to end in the grid, which turns three short launches
+// into one long enough to fill the chip.  An optional residual is added in the epilogue.
 #include "common.hpp"
 #include "qdot.hpp"
 
@@ -13,24 +16,38 @@
 
 namespace mi355 {
 
+struct gemv_item {
+    const uint8_t *W;
+    float *dst;
+    const float *residual;   // may be null; same shape/stride as dst; may alias dst
+    int64_t N;
+    int64_t dst_stride;
+    int type;
+    int first_group;         // index of this matrix's first group in the launch
+};
+struct gemv_batch {
+    gemv_item it[4];
+    int n;
+};
+
 template <int TYPE, int NCOLS, int RPW>
-__device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
-                                          const act_ds *__restrict__ ads, float *__restrict__ dst, int64_t N,
-                                          int64_t K, int64_t dst_stride, const row_layout &L) {
+__device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const int8_t *__restrict__ aq,
+                                          const act_ds *__restrict__ ads, int K) {
     typedef wq<TYPE> T;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * RPW;
-    if (row0 >= N) return;   // whole wave exits together
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t row0 = ((int64_t)group * 4 + wave) * RPW;
+    if (row0 >= m.N) return;   // whole wave exits together
 
-    const int64_t nchunks = K >> 5;
-    const int64_t nblk = K >> 5;   // Q8_1 blocks per activation row
+    const row_layout L = make_row_layout(TYPE, K);
+    const int nchunks = K / T::CHUNK;
+    const int nblk = K >> 5;   // Q8_1 blocks per activation row
 
     const uint8_t *rows[RPW];
 #pragma unroll
     for (int r = 0; r < RPW; r++) {
-        const int64_t row = row0 + r < N ? row0 + r : N - 1;   // clamp: tail rows recompute the last row, never stored
-        rows[r] = W + row * L.row_bytes;
+        const int64_t row = row0 + r < m.N ? row0 + r : m.N - 1;   // clamp: tail rows recompute the last row, never stored
+        rows[r] = m.W + row * L.row_bytes;
     }
 
     float acc[RPW][NCOLS];
@@ -39,15 +56,15 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, const i
 #pragma unroll
         for (int c = 0; c < NCOLS; c++) acc[r][c] = 0.0f;
 
-    for (int64_t c0 = 0; c0 < nchunks; c0 += 64) {
-        const int64_t c = c0 + lane;
+    for (int c0 = 0; c0 < nchunks; c0 += 64) {
+        const int c = c0 + lane;
         if (c < nchunks) {
             typename T::chunk w[RPW];
 #pragma unroll
-            for (int r = 0; r < RPW; r++) w[r] = T::load(rows[r], L, c);
+            for (int r = 0; r < RPW; r++) w[r] = T::load_w(rows[r], L, c);
 #pragma unroll
             for (int col = 0; col < NCOLS; col++) {
-                const act_chunk A = load_act_chunk<TYPE>(aq + col * K, ads + col * nblk, c);
+                const typename T::act A = T::load_a(aq + (int64_t)col * K, ads + col * nblk, c);
 #pragma unroll
                 for (int r = 0; r < RPW; r++) {
                     const chunk_dots d = T::dots(w[r], A);
@@ -62,15 +79,39 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ W, const i
 #pragma unroll
         for (int c = 0; c < NCOLS; c++) {
             const float s = wave_sum(acc[r][c]);
-            if (lane == 0 && row0 + r < N) dst[c * dst_stride + row0 + r] = s;
+            if (lane == 0 && row0 + r < m.N) {
+                const int64_t o = c * m.dst_stride + row0 + r;
+                m.dst[o] = m.residual ? s + m.residual[o] : s;
+            }
         }
 }
 
+template <int NCOLS, int RPW>
+__device__ __forceinline__ void gemv_dispatch(const gemv_item &m, int group, const int8_t *__restrict__ aq,
+                                              const act_ds *__restrict__ ads, int K) {
+    switch (m.type) {   // uniform over the group
+        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, RPW>(m, group, aq, ads, K); break;
+        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW>(m, group, aq, ads, K); break;
+        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW>(m, group, aq, ads, K); break;
+        default: gemv_body<MI355_Q6_K, NCOLS, RPW>(m, group, aq, ads, K); break;
+    }
+}
+
+// single matrix, type known at compile time (smallest code, used by mi355_mul_mat_vec_q)
 template <int TYPE, int NCOLS, int RPW>
-__global__ void __launch_bounds__(256) k_gemv_q(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
-                                                const act_ds *__restrict__ ads, float *__restrict__ dst, int64_t N,
-                                                int64_t K, int64_t dst_stride, row_layout L) {
-    gemv_body<TYPE, NCOLS, RPW>(W, aq, ads, dst, N, K, dst_stride, L);
+__global__ void __launch_bounds__(256) k_gemv_q(gemv_item m, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K) {
+    gemv_body<TYPE, NCOLS, RPW>(m, blockIdx.x, aq, ads, K);
+}
+
+// several matrices sharing one activation
+template <int NCOLS, int RPW>
+__global__ void __launch_bounds__(256) k_gemv_multi(gemv_batch b, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K) {
+    const int g = blockIdx.x;
+    int i = 0;
+#pragma unroll
+    for (int j = 1; j < 4; j++)
+        if (j < b.n && g >= b.it[j].first_group) i = j;
+    gemv_dispatch<NCOLS, RPW>(b.it[i], g - b.it[i].first_group, aq, ads, K);
 }
 
 // MUL_MAT_ID, one activation row per expert slot: blockIdx.y = slot = t * n_used + e.  The
@@ -78,13 +119,22 @@ __global__ void __launch_bounds__(256) k_gemv_q(const uint8_t *__restrict__ W, c
 template <int TYPE, int RPW>
 __global__ void __launch_bounds__(256) k_gemv_id(const uint8_t *__restrict__ as, const int8_t *__restrict__ aq,
                                                  const act_ds *__restrict__ ads, const int32_t *__restrict__ ids,
-                                                 int64_t ids_stride, float *__restrict__ dst, int64_t N, int64_t K,
-                                                 int64_t n_expert, int64_t n_used, int64_t nb1, row_layout L) {
+                                                 int64_t ids_stride, float *__restrict__ dst, int64_t N, int K,
+                                                 int64_t n_expert, int64_t n_used, int64_t nb1) {
     const int64_t slot = blockIdx.y, t = slot / n_used, e = slot % n_used;
     int64_t ex = ids[t * ids_stride + e];
     ex = ex < 0 ? 0 : (ex >= n_expert ? n_expert - 1 : ex);   // never index outside the expert stack
     const int64_t arow = t * nb1 + e % nb1;
-    gemv_body<TYPE, 1, RPW>(as + ex * N * L.row_bytes, aq + arow * K, ads + arow * (K >> 5), dst + slot * N, N, K, N, L);
+    const row_layout L = make_row_layout(TYPE, K);
+    gemv_item m;
+    m.W = as + ex * N * L.row_bytes;
+    m.dst = dst + slot * N;
+    m.residual = nullptr;
+    m.N = N;
+    m.dst_stride = N;
+    m.type = TYPE;
+    m.first_group = 0;
+    gemv_body<TYPE, 1, RPW>(m, blockIdx.x, aq + arow * K, ads + arow * (K >> 5), K);
 }
 
 // Same routing for weight rows that are not 16-byte aligned (byte loads): one wave per (row, slot).
@@ -109,93 +159,85 @@ __global__ void __launch_bounds__(64) k_gemv_id_unaligned(const uint8_t *__restr
 // Parity dump of the integer granule dots (one wave per row, activation row 0).
 template <int TYPE>
 __global__ void __launch_bounds__(64) k_block_dots(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
-                                                   const act_ds *__restrict__ ads, int32_t *__restrict__ out, int64_t N,
-                                                   int64_t K, row_layout L) {
+                                                   const act_ds *__restrict__ ads, int32_t *__restrict__ out, int64_t N, int K) {
     typedef wq<TYPE> T;
     const int lane = threadIdx.x;
     const int64_t row = blockIdx.x;
-    const int64_t nchunks = K >> 5;
-    const uint8_t *wrow = W + row * L.row_bytes;
-    for (int64_t c0 = 0; c0 < nchunks; c0 += 64) {
-        const int64_t c = c0 + lane;
-        const bool live = c < nchunks;
-        const int64_t cc = live ? c : 0;
-        const typename T::chunk w = T::load(wrow, L, cc);
-        act_chunk A = load_act_chunk<TYPE>(aq, ads, cc);
-        const chunk_dots d = T::dots(w, A);
-        if constexpr (TYPE == MI355_Q4_0 || TYPE == MI355_Q8_0) {
-            if (live) out[row * nchunks + c] = d.i0;
-        } else if constexpr (TYPE == MI355_Q4_K) {
-            // two lanes hold the halves of sub-blocks 2g and 2g+1
-            const int o0 = d.i0 + __shfl_xor(d.i0, 1, 64);
-            const int o1 = d.i1 + __shfl_xor(d.i1, 1, 64);
-            if (live && (c & 1) == 0) {
-                const int64_t sb = c >> 3;
-                const int g = (int)(c & 7) >> 1;
-                out[row * nchunks + sb * 8 + 2 * g] = o0;
-                out[row * nchunks + sb * 8 + 2 * g + 1] = o1;
-            }
-        } else {   // Q6_K: 16 granules per super-block
-            if (live) {
-                const int64_t sb = c >> 3;
-                const int ccc = (int)(c & 7), hf = ccc >> 2, r = ccc & 3;
-                const int gi = 8 * hf + 2 * (r >> 1) + (r & 1);
-                out[row * (nchunks * 2) + sb * 16 + gi] = d.i0;
-                out[row * (nchunks * 2) + sb * 16 + gi + 4] = d.i1;
-            }
-        }
-    }
-}
-
-template <int TYPE, int NCOLS, int RPW>
-static void launch_gemv(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
-                        int64_t dst_stride) {
     const row_layout L = make_row_layout(TYPE, K);
-    const int8_t *aq = (const int8_t *)act;
-    const act_ds *ads = (const act_ds *)(aq + B * K);
-    const int64_t rows_per_group = 4 * RPW;
-    const unsigned grid = (unsigned)((N + rows_per_group - 1) / rows_per_group);
-    hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, RPW>), dim3(grid), dim3(256), 0, s, (const uint8_t *)W, aq, ads, dst, N, K,
-                       dst_stride, L);
-}
-
-template <int TYPE, int NCOLS>
-static void launch_gemv_rpw(int rpw, hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K,
-                            int64_t B, int64_t dst_stride) {
-    switch (rpw) {
-        case 1: launch_gemv<TYPE, NCOLS, 1>(s, W, act, dst, N, K, B, dst_stride); break;
-        case 2: launch_gemv<TYPE, NCOLS, 2>(s, W, act, dst, N, K, B, dst_stride); break;
-        default: launch_gemv<TYPE, NCOLS, 4>(s, W, act, dst, N, K, B, dst_stride); break;
-    }
-}
-
-template <int TYPE>
-static void launch_gemv_cols(int rpw, hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K,
-                             int64_t B, int64_t dst_stride) {
-    switch (B) {
-        case 1: launch_gemv_rpw<TYPE, 1>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case 2: launch_gemv_rpw<TYPE, 2>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case 3: launch_gemv_rpw<TYPE, 3>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case 4: launch_gemv_rpw<TYPE, 4>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case 5: launch_gemv_rpw<TYPE, 5>(rpw > 2 ? 2 : rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case 6: launch_gemv_rpw<TYPE, 6>(rpw > 2 ? 2 : rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case 7: launch_gemv_rpw<TYPE, 7>(rpw > 2 ? 2 : rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        default: launch_gemv_rpw<TYPE, 8>(rpw > 2 ? 2 : rpw, s, W, act, dst, N, K, B, dst_stride); break;
+    const int nchunks = K / T::CHUNK;
+    const int ngran = TYPE == MI355_Q6_K ? K / 16 : K / 32;
+    const uint8_t *wrow = W + row * L.row_bytes;
+    for (int c0 = 0; c0 < nchunks; c0 += 64) {
+        const int c = c0 + lane;
+        const bool live = c < nchunks;
+        const int cc = live ? c : 0;
+        const typename T::chunk w = T::load_w(wrow, L, cc);
+        const typename T::act A = T::load_a(aq, ads, cc);
+        const chunk_dots d = T::dots(w, A);
+        if (!live) continue;
+        if constexpr (TYPE == MI355_Q4_0 || TYPE == MI355_Q8_0) {
+            out[row * ngran + c] = d.i0;
+        } else if constexpr (TYPE == MI355_Q4_K) {   // chunk c = sub-blocks 2c and 2c+1 of the row
+            out[row * ngran + 2 * c] = d.i0;
+            out[row * ngran + 2 * c + 1] = d.i1;
+        } else {   // Q6_K: 16 granules per super-block
+            const int sb = c >> 3, ccc = c & 7, hf = ccc >> 2, r = ccc & 3;
+            const int gi = 8 * hf + 2 * (r >> 1) + (r & 1);
+            out[row * ngran + sb * 16 + gi] = d.i0;
+            out[row * ngran + sb * 16 + gi + 4] = d.i1;
+        }
     }
 }
 
 // rows per wave: enough waves to cover every SIMD a few times over, then amortise the
 // activation reads over more rows.  MI355_GEMV_RPW overrides (tuning aid).
-static int pick_rpw(int64_t N) {
+static int pick_rpw(int64_t total_rows) {
     static int forced = -1;
     if (forced < 0) {
         const char *e = getenv("MI355_GEMV_RPW");
         forced = e ? atoi(e) : 0;
     }
     if (forced == 1 || forced == 2 || forced == 4) return forced;
-    if (N >= 32768) return 4;
-    if (N >= 8192) return 2;
+    if (total_rows >= 32768) return 4;
+    if (total_rows >= 8192) return 2;
     return 1;
+}
+
+template <int NCOLS>
+static void launch_multi(int rpw, hipStream_t s, const gemv_batch &b, unsigned grid, const int8_t *aq, const act_ds *ads, int K) {
+    if (rpw == 1) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 1>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 2>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    else hipLaunchKernelGGL((k_gemv_multi<NCOLS, 4>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+}
+
+template <int TYPE, int NCOLS>
+static void launch_single(int rpw, hipStream_t s, const gemv_item &m, unsigned grid, const int8_t *aq, const act_ds *ads, int K) {
+    if (rpw == 1) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 1>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 2>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    else hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 4>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+}
+
+template <int TYPE>
+static void launch_single_cols(int rpw, int64_t B, hipStream_t s, const gemv_item &m, unsigned grid, const int8_t *aq, const act_ds *ads, int K) {
+    switch (B) {
+        case 1: launch_single<TYPE, 1>(rpw, s, m, grid, aq, ads, K); break;
+        case 2: launch_single<TYPE, 2>(rpw, s, m, grid, aq, ads, K); break;
+        case 3: launch_single<TYPE, 3>(rpw, s, m, grid, aq, ads, K); break;
+        case 4: launch_single<TYPE, 4>(rpw, s, m, grid, aq, ads, K); break;
+        case 5: launch_single<TYPE, 5>(rpw, s, m, grid, aq, ads, K); break;
+        case 6: launch_single<TYPE, 6>(rpw, s, m, grid, aq, ads, K); break;
+        case 7: launch_single<TYPE, 7>(rpw, s, m, grid, aq, ads, K); break;
+        default: launch_single<TYPE, 8>(rpw, s, m, grid, aq, ads, K); break;
+    }
+}
+
+static int check_gemv_args(const char *who, int type, const void *W, int64_t N, int64_t K, int64_t dst_stride) {
+    MI355_REQUIRE(is_weight_type(type), "%s: unsupported weight type %d", who, type);
+    MI355_REQUIRE(N > 0 && K > 0 && K < (int64_t(1) << 30), "%s: bad shape N=%lld K=%lld", who, (long long)N, (long long)K);
+    MI355_REQUIRE(K % type_block_elems(type) == 0, "%s: K=%lld is not a multiple of the block size", who, (long long)K);
+    MI355_REQUIRE(dst_stride >= N, "%s: dst_stride < N", who);
+    MI355_REQUIRE(layout_aligned(W, make_row_layout(type, K)), "%s: weight rows are not 16-byte aligned (K=%lld)", who, (long long)K);
+    return MI355_OK;
 }
 
 }  // namespace mi355
@@ -206,37 +248,91 @@ extern "C" {
 
 int mi355_mul_mat_vec_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
                         int64_t B, int64_t dst_stride) {
-    MI355_REQUIRE(is_weight_type(type), "mul_mat_vec_q: unsupported weight type %d", type);
-    MI355_REQUIRE(N > 0 && K > 0 && B >= 1 && B <= 8, "mul_mat_vec_q: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
-    MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_vec_q: K=%lld is not a multiple of the block size", (long long)K);
-    MI355_REQUIRE(dst_stride >= N, "mul_mat_vec_q: dst_stride < N");
-    const row_layout L = make_row_layout(type, K);
-    MI355_REQUIRE(((uintptr_t)W & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0,
-                  "mul_mat_vec_q: weight rows are not 16-byte aligned (K=%lld)", (long long)K);
+    mi355_gemv_mat m = {type, W, N, dst, dst_stride, nullptr};
+    return mi355_mul_mat_vec_q_multi(stream, 1, &m, act, K, B);
+}
+
+int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B) {
+    MI355_REQUIRE(n_mats >= 1 && n_mats <= 4, "mul_mat_vec_q_multi: 1..4 matrices per launch, got %d", n_mats);
+    MI355_REQUIRE(B >= 1 && B <= 8, "mul_mat_vec_q: batch %lld outside 1..8", (long long)B);
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_vec_q: activation workspace is not 16-byte aligned");
-    hipStream_t s = (hipStream_t)stream;
-    const int rpw = pick_rpw(N);
-    switch (type) {
-        case MI355_Q4_0: launch_gemv_cols<MI355_Q4_0>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case MI355_Q8_0: launch_gemv_cols<MI355_Q8_0>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        case MI355_Q4_K: launch_gemv_cols<MI355_Q4_K>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
-        default: launch_gemv_cols<MI355_Q6_K>(rpw, s, W, act, dst, N, K, B, dst_stride); break;
+    int64_t total_rows = 0;
+    bool aligned = true;
+    for (int i = 0; i < n_mats; i++) {
+        MI355_REQUIRE(is_weight_type(mats[i].type) && K > 0 && K % type_block_elems(mats[i].type) == 0, "mul_mat_vec_q: unsupported type %d or K=%lld not a multiple of its block size", mats[i].type, (long long)K);
+        aligned = aligned && layout_aligned(mats[i].W, make_row_layout(mats[i].type, K));
     }
-    return launch_status("k_gemv_q");
+    if (!aligned) {   // tiny / odd shapes only: byte-load kernel, one matrix at a time
+        for (int i = 0; i < n_mats; i++) {
+            MI355_REQUIRE(mats[i].N > 0 && mats[i].dst_stride >= mats[i].N, "mul_mat_vec_q: bad shape");
+            int rc = gemv_unaligned((hipStream_t)stream, mats[i].type, mats[i].W, act, mats[i].dst, mats[i].residual, mats[i].N, K, B, mats[i].dst_stride);
+            if (rc != MI355_OK) return rc;
+        }
+        return MI355_OK;
+    }
+    for (int i = 0; i < n_mats; i++) {
+        int rc = check_gemv_args("mul_mat_vec_q", mats[i].type, mats[i].W, mats[i].N, K, mats[i].dst_stride);
+        if (rc != MI355_OK) return rc;
+        total_rows += mats[i].N;
+    }
+    int rpw = pick_rpw(total_rows);
+    if (B > 4 && rpw > 2) rpw = 2;   // keep the accumulator tile in registers
+    gemv_batch b;
+    b.n = n_mats;
+    int64_t groups = 0;
+    for (int i = 0; i < 4; i++) {
+        const mi355_gemv_mat &src = mats[i < n_mats ? i : 0];
+        b.it[i].W = (const uint8_t *)src.W;
+        b.it[i].dst = src.dst;
+        b.it[i].residual = src.residual;
+        b.it[i].N = src.N;
+        b.it[i].dst_stride = src.dst_stride;
+        b.it[i].type = src.type;
+        b.it[i].first_group = (int)groups;
+        if (i < n_mats) groups += (src.N + 4 * rpw - 1) / (4 * rpw);
+    }
+    MI355_REQUIRE(groups < 0x7fffffff, "mul_mat_vec_q: too many rows for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + B * K);
+    if (n_mats == 1) {
+        switch (mats[0].type) {
+            case MI355_Q4_0: launch_single_cols<MI355_Q4_0>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
+            case MI355_Q8_0: launch_single_cols<MI355_Q8_0>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
+            case MI355_Q4_K: launch_single_cols<MI355_Q4_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
+            default: launch_single_cols<MI355_Q6_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
+        }
+        return launch_status("k_gemv_q");
+    }
+    switch (B) {
+        case 1: launch_multi<1>(rpw, s, b, (unsigned)groups, aq, ads, (int)K); break;
+        case 2: launch_multi<2>(rpw, s, b, (unsigned)groups, aq, ads, (int)K); break;
+        case 3: launch_multi<3>(rpw, s, b, (unsigned)groups, aq, ads, (int)K); break;
+        case 4: launch_multi<4>(rpw, s, b, (unsigned)groups, aq, ads, (int)K); break;
+        default:
+            // wider batches: one launch per matrix (register budget of the type switch)
+            for (int i = 0; i < n_mats; i++) {
+                mi355_gemv_mat one = mats[i];
+                int rc = mi355_mul_mat_vec_q_multi(stream, 1, &one, act, K, B);
+                if (rc != MI355_OK) return rc;
+            }
+            return MI355_OK;
+    }
+    return launch_status("k_gemv_multi");
 }
 
 // act: split layout of nb1*T quantized rows of b.  dst [N, n_used, T] contiguous.
 int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride,
                          float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T) {
     MI355_REQUIRE(is_weight_type(type), "mul_mat_id: unsupported weight type %d", type);
-    MI355_REQUIRE(N > 0 && K > 0 && n_expert > 0 && n_used > 0 && nb1 > 0 && T > 0, "mul_mat_id: bad shape");
+    MI355_REQUIRE(N > 0 && K > 0 && K < (int64_t(1) << 30) && n_expert > 0 && n_used > 0 && nb1 > 0 && T > 0, "mul_mat_id: bad shape");
     MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_id: K=%lld is not a multiple of the block size", (long long)K);
     MI355_REQUIRE(n_used * T <= 65535, "mul_mat_id: too many expert slots for one launch");
     const row_layout L = make_row_layout(type, K);
     hipStream_t s = (hipStream_t)stream;
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + nb1 * T * K);
-    if (!(((uintptr_t)as & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0)) {
+    if (!layout_aligned(as, L)) {
         const dim3 ugrid((unsigned)N, (unsigned)(n_used * T));
         switch (type) {
             case MI355_Q4_0: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q4_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
@@ -246,11 +342,11 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
         }
         return launch_status("k_gemv_id_unaligned");
     }
-    const int rpw = pick_rpw(N) > 2 ? 2 : pick_rpw(N);
+    const int rpw = pick_rpw(N * n_used) > 2 ? 2 : pick_rpw(N * n_used);
     const dim3 grid((unsigned)((N + 4 * rpw - 1) / (4 * rpw)), (unsigned)(n_used * T));
 #define MI355_ID_LAUNCH(TY)                                                                                           \
-    if (rpw == 1) hipLaunchKernelGGL((k_gemv_id<TY, 1>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); \
-    else hipLaunchKernelGGL((k_gemv_id<TY, 2>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L);
+    if (rpw == 1) hipLaunchKernelGGL((k_gemv_id<TY, 1>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
+    else hipLaunchKernelGGL((k_gemv_id<TY, 2>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1);
     switch (type) {
         case MI355_Q4_0: MI355_ID_LAUNCH(MI355_Q4_0) break;
         case MI355_Q8_0: MI355_ID_LAUNCH(MI355_Q8_0) break;
@@ -262,21 +358,17 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
 }
 
 int mi355_block_dots_q8_1(void *stream, int type, const void *W, const void *a, int32_t *out, int64_t N, int64_t K) {
-    // `a` is the split activation layout of mi355_quantize_act for ONE row
-    MI355_REQUIRE(is_weight_type(type), "block_dots: unsupported weight type %d", type);
-    MI355_REQUIRE(N > 0 && K > 0 && K % type_block_elems(type) == 0, "block_dots: bad shape");
-    const row_layout L = make_row_layout(type, K);
-    MI355_REQUIRE(((uintptr_t)W & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0,
-                  "block_dots: weight rows are not 16-byte aligned (K=%lld)", (long long)K);
+    int rc = check_gemv_args("block_dots", type, W, N, K, N);
+    if (rc != MI355_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
     const int8_t *aq = (const int8_t *)a;
     const act_ds *ads = (const act_ds *)(aq + K);
     const dim3 grid((unsigned)N);
     switch (type) {
-        case MI355_Q4_0: hipLaunchKernelGGL(k_block_dots<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, K, L); break;
-        case MI355_Q8_0: hipLaunchKernelGGL(k_block_dots<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, K, L); break;
-        case MI355_Q4_K: hipLaunchKernelGGL(k_block_dots<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, K, L); break;
-        default: hipLaunchKernelGGL(k_block_dots<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, K, L); break;
+        case MI355_Q4_0: hipLaunchKernelGGL(k_block_dots<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        case MI355_Q8_0: hipLaunchKernelGGL(k_block_dots<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        case MI355_Q4_K: hipLaunchKernelGGL(k_block_dots<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        default: hipLaunchKernelGGL(k_block_dots<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
     }
     return launch_status("k_block_dots");
 }

@@ -335,11 +335,11 @@ extern "C" int mi355_mul_mat_q(void *stream, int type, const void *W, const void
                                int64_t B, int64_t dst_stride) {
     MI355_REQUIRE(is_weight_type(type), "mul_mat_q: unsupported weight type %d", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
-    MI355_REQUIRE(K % MMQ_BK == 0 && K % type_block_elems(type) == 0, "mul_mat_q: K=%lld must be a multiple of 128 and of the block size", (long long)K);
+    MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_q: K=%lld is not a multiple of the block size", (long long)K);
     MI355_REQUIRE(dst_stride >= N, "mul_mat_q: dst_stride < N");
     const row_layout L = make_row_layout(type, K);
-    MI355_REQUIRE(((uintptr_t)W & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0,
-                  "mul_mat_q: weight rows are not 16-byte aligned (K=%lld)", (long long)K);
+    if (!layout_aligned(W, L) || K % MMQ_BK != 0)   // tiny / odd shapes only
+        return gemv_unaligned((hipStream_t)stream, type, W, act, dst, nullptr, N, K, B, dst_stride);
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_q: activation workspace is not 16-byte aligned");
     MI355_REQUIRE((N + MMQ_BM - 1) / MMQ_BM * ((B + 63) / 64) < (1 << 30), "mul_mat_q: too many tiles");
     hipStream_t s = (hipStream_t)stream;

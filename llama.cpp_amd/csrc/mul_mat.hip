@@ -1,5 +1,6 @@
 // MUL_MAT host entry: quantize activations to Q8_1 on the device, then dispatch to the
-// GEMV (B <= 8) or the int8-MFMA tile kernel (B > 8).  Also the unaligned fallback.
+// GEMV (B <= 8) or the int8-MFMA tile kernel (B > 8).  Also the byte-load fallback for weight
+// rows that are not 16-byte aligned.
 #include "common.hpp"
 #include "qdot.hpp"
 
@@ -9,7 +10,8 @@ namespace mi355 {
 template <int TYPE>
 __global__ void __launch_bounds__(64) k_gemv_unaligned(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
                                                        const act_ds *__restrict__ ads, float *__restrict__ dst,
-                                                       int64_t N, int64_t K, int64_t dst_stride, row_layout L) {
+                                                       const float *__restrict__ residual, int64_t N, int64_t K,
+                                                       int64_t dst_stride, row_layout L) {
     const int64_t row = blockIdx.x, col = blockIdx.y;
     const uint8_t *wrow = W + row * L.row_bytes;
     const int8_t *q = aq + col * K;
@@ -17,36 +19,27 @@ __global__ void __launch_bounds__(64) k_gemv_unaligned(const uint8_t *__restrict
     float acc = 0.0f;
     for (int64_t e = threadIdx.x; e < K; e += 64) acc += weight_value<TYPE>(wrow, L, e) * (ds[e >> 5].d * (float)q[e]);
     acc = wave_sum(acc);
-    if (threadIdx.x == 0) dst[col * dst_stride + row] = acc;
+    if (threadIdx.x == 0) {
+        const int64_t o = col * dst_stride + row;
+        dst[o] = residual ? acc + residual[o] : acc;
+    }
 }
 
-static bool rows_aligned(int type, const void *W, int64_t K) {
-    const row_layout L = make_row_layout(type, K);
-    return ((uintptr_t)W & 15) == 0 && (L.row_bytes & 15) == 0 && (L.off_b & 15) == 0 && (L.off_c & 15) == 0;
-}
-
-static int gemv_unaligned(hipStream_t s, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
-                          int64_t B, int64_t dst_stride) {
+// act: split layout holding B quantized rows of K
+int gemv_unaligned(hipStream_t s, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N,
+                   int64_t K, int64_t B, int64_t dst_stride) {
     const row_layout L = make_row_layout(type, K);
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + B * K);
     MI355_REQUIRE(B <= 65535, "mul_mat: batch %lld too large for the unaligned path", (long long)B);
     const dim3 grid((unsigned)N, (unsigned)B);
     switch (type) {
-        case MI355_Q4_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
-        case MI355_Q8_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
-        case MI355_Q4_K: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
-        default: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, N, K, dst_stride, L); break;
+        case MI355_Q4_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        case MI355_Q8_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        case MI355_Q4_K: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        default: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
     }
     return launch_status("k_gemv_unaligned");
-}
-
-// act holds B quantized rows; runs the right kernel for any B
-int mul_mat_from_act(hipStream_t s, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
-                     int64_t B, int64_t dst_stride) {
-    if (!rows_aligned(type, W, K) || (B > 8 && K % 128 != 0)) return gemv_unaligned(s, type, W, act, dst, N, K, B, dst_stride);
-    if (B <= 8) return mi355_mul_mat_vec_q(s, type, W, act, dst, N, K, B, dst_stride);
-    return mi355_mul_mat_q(s, type, W, act, dst, N, K, B, dst_stride);
 }
 
 }  // namespace mi355
@@ -69,7 +62,8 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
     }
     int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
     if (rc != MI355_OK) return rc;
-    return mul_mat_from_act((hipStream_t)stream, type, W, ws, dst, N, K, B, dst_stride);
+    if (B <= 8) return mi355_mul_mat_vec_q(stream, type, W, ws, dst, N, K, B, dst_stride);
+    return mi355_mul_mat_q(stream, type, W, ws, dst, N, K, B, dst_stride);
 }
 
 }  // extern "C"

@@ -17,6 +17,11 @@ BLOCK = {F32: (1, 4), F16: (1, 2), I32: (1, 4), Q4_0: (32, 18), Q8_0: (32, 34), 
 _p, _i64, _sz, _f, _int = C.c_void_p, C.c_int64, C.c_size_t, C.c_float, C.c_int
 
 
+class GemvMat(C.Structure):
+    """struct mi355_gemv_mat"""
+    _fields_ = [("type", _int), ("W", _p), ("N", _i64), ("dst", _p), ("dst_stride", _i64), ("residual", _p)]
+
+
 class Tensor(C.Structure):
     """struct mi355_tensor"""
     _fields_ = [("data", _p), ("type", _int), ("ne", _i64 * 4), ("nb", _sz * 4)]
@@ -35,6 +40,11 @@ _SIGNATURES = {
     "mi355_mul_mat": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_vec_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
+    "mi355_rms_norm_mul_quant": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
+    "mi355_swiglu_quant": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
+    "mi355_rope_kv_store": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _int, _int, _int,
+                                   _f, _f, _f, _f, _f, _f]),
     "mi355_block_dots_q8_1": (_int, [_p, _int, _p, _p, _p, _i64, _i64]),
     "mi355_mul_mat_id_ws_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_id": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),

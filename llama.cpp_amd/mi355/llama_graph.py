@@ -13,8 +13,8 @@ import math
 
 import torch
 
-from . import (F16, F32, I32, Q4_K, Q6_K, Q4_0, Q8_0, BLOCK, Tensor, check, load, row_bytes, tensor_desc, upload_weights,
-               _ptr, _stream)
+from . import (F16, F32, I32, Q4_K, Q6_K, Q4_0, Q8_0, BLOCK, GemvMat, Tensor, check, load, row_bytes, tensor_desc,
+               upload_weights, _ptr, _stream)
 
 
 def use_more_bits(i_layer, n_layer):
@@ -114,6 +114,8 @@ class LlamaRunner:
         self.pos = torch.zeros(T, dtype=torch.int32, device=dev)
         self.mask = torch.zeros((T + 63) // 64 * 64, cfg.n_ctx, dtype=torch.float16, device=dev)
         kmax = max(E, F, H * D)
+        self.act_a = torch.empty(int(self.lib.mi355_act_bytes(max(E, H * D), T)) + 256, dtype=torch.uint8, device=dev)
+        self.act_b = torch.empty(int(self.lib.mi355_act_bytes(F, T)) + 256, dtype=torch.uint8, device=dev)
         self.ws = torch.empty(int(self.lib.mi355_mul_mat_ws_bytes(kmax, T)) + 256, dtype=torch.uint8, device=dev)
         self.fa_ws = torch.empty(min(int(self.lib.mi355_flash_attn_ws_bytes(D, T, cfg.n_ctx, H)), 256 << 20), dtype=torch.uint8, device=dev)
 
@@ -155,8 +157,53 @@ class LlamaRunner:
                                             vc.stride(1) * 2, self.mask.stride(0) * 2, 1.0 / math.sqrt(D), 0.0, 0.0, _ptr(self.fa_ws),
                                             self.fa_ws.numel()))
 
-    # ---- one forward pass over T tokens whose inputs (x, pos, mask) are already on the device --
+    # ---- fused operators ------------------------------------------------------------------------
+    def _norm_quant(self, x, w, act, T):
+        K = x.shape[1]
+        check(self.lib.mi355_rms_norm_mul_quant(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
+
+    def _mm_act(self, mats, act, K, T, residual=None):
+        """mats: list of ((type, W), out); all consume the quantized activation `act` (T rows of K)"""
+        if T <= 8:
+            arr = (GemvMat * len(mats))()
+            for i, ((t, W), out) in enumerate(mats):
+                arr[i].type, arr[i].W, arr[i].N, arr[i].dst, arr[i].dst_stride = t, W.data_ptr(), out.shape[1], out.data_ptr(), out.stride(0)
+                arr[i].residual = residual.data_ptr() if residual is not None else None
+            check(self.lib.mi355_mul_mat_vec_q_multi(_stream(), len(mats), arr, _ptr(act), K, T))
+        else:
+            for (t, W), out in mats:
+                dst = out if residual is None else self.t1[:T]
+                check(self.lib.mi355_mul_mat_q(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), out.shape[1], K, T, dst.stride(0)))
+                if residual is not None:
+                    self._bin(0, dst, residual, out)
+
     def forward(self, T, n_kv, last_only=True):
+        """fused launch sequence: 10 launches per layer instead of 25, same arithmetic per node"""
+        cfg, w, lib = self.cfg, self.w, self.lib
+        E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
+        x = self.x[:T]
+        for il, L in enumerate(w.layers):
+            self._norm_quant(x, L["attn_norm"], self.act_a, T)
+            self._mm_act([(L["wq"], self.q[:T]), (L["wk"], self.k[:T]), (L["wv"], self.v[:T])], self.act_a, E, T)
+            kc, vc = self.kcache[il], self.vcache[il]
+            check(lib.mi355_rope_kv_store(_stream(), _ptr(self.q), _ptr(self.k), _ptr(self.v), _ptr(kc), _ptr(vc), _ptr(self.pos), _ptr(self.pos),
+                                          None, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2, vc.stride(1) * 2, D, 0,
+                                          cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
+            self._attn(il, T, n_kv)
+            check(lib.mi355_quantize_act(_stream(), _ptr(self.attn), _ptr(self.act_a), H * D, T, H * D))
+            self._mm_act([(L["wo"], x)], self.act_a, H * D, T, residual=x)
+            self._norm_quant(x, L["ffn_norm"], self.act_a, T)
+            self._mm_act([(L["gate"], self.gate[:T]), (L["up"], self.up[:T])], self.act_a, E, T)
+            check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
+            self._mm_act([(L["down"], x)], self.act_b, F, T, residual=x)
+        To = 1 if last_only else T
+        xo = self.x[T - 1:T] if last_only else x
+        self._norm_quant(xo, w.output_norm, self.act_a, To)
+        self._mm_act([(w.output, self.logits[:To])], self.act_a, E, To)
+        return self.logits[:To]
+
+    # ---- the same pass node for node, as the ggml graph lists it (reference for the fused path) --
+    def forward_nodes(self, T, n_kv, last_only=True):
         cfg, w = self.cfg, self.w
         x = self.x
         for il, L in enumerate(w.layers):

@@ -1,0 +1,142 @@
+"""GPU parity of the fused node sequences and the multi-matrix GEMV launch against the oracle, and of
+the fused llama layer stack against the node-for-node one."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(dev, a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _unpack_act(act, K, nrows):
+    """split activation layout -> (int8 [nrows,K], d f32 [nrows,K/32], sum i32 [nrows,K/32])"""
+    a = act.cpu().numpy()
+    q = a[:nrows * K].view(np.int8).reshape(nrows, K)
+    ds = a[nrows * K:nrows * K + nrows * (K // 32) * 8].view(np.int32).reshape(nrows, K // 32, 2)
+    return q, ds[:, :, 0].copy().view(np.float32), ds[:, :, 1]
+
+
+def _check_act_matches_q8_1(act, y, K, nrows):
+    """the activation a fused kernel emits must be quantize_row_q8_1_ref of the f32 values it emits"""
+    q, d, s = _unpack_act(act, K, nrows)
+    ref = orc.quantize("oracle", orc.Q8_1, y).reshape(nrows, K // 32, 36)
+    assert np.array_equal(q.reshape(nrows, K // 32, 32), ref[:, :, 4:].view(np.int8))
+    assert np.array_equal(d.astype(np.float16).view(np.uint16), ref[:, :, 0:2].copy().view(np.uint16).reshape(nrows, K // 32))
+    assert np.array_equal(s, q.reshape(nrows, K // 32, 32).astype(np.int32).sum(axis=2))
+
+
+@pytest.mark.parametrize("K,nrows", [(4096, 1), (4096, 5), (14336, 2), (8192, 3), (96, 4)])
+def test_rms_norm_mul_quant(dev, K, nrows):
+    import torch
+    import mi355
+    rng = np.random.default_rng(K + nrows)
+    x = rng.standard_normal((nrows, K)).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    xd, wd = _t(dev, x), _t(dev, w)
+    yd = torch.empty_like(xd)
+    act = torch.zeros(mi355.load().mi355_act_bytes(K, nrows), dtype=torch.uint8, device=dev)
+    mi355.check(mi355.load().mi355_rms_norm_mul_quant(None, xd.data_ptr(), K, wd.data_ptr(), yd.data_ptr(), K, act.data_ptr(), K, nrows, 1e-5))
+    y = yd.cpu().numpy()
+    want = np.zeros_like(x)
+    orc.oracle.orc_rms_norm(orc._ptr(x), orc._ptr(want), K, nrows, 1e-5)
+    assert orc.nmse(y, want * w) < 1e-7
+    _check_act_matches_q8_1(act, y, K, nrows)
+
+
+@pytest.mark.parametrize("K,nrows", [(14336, 1), (14336, 4), (1024, 7)])
+def test_swiglu_quant(dev, K, nrows):
+    import torch
+    import mi355
+    rng = np.random.default_rng(K + nrows)
+    g = (rng.standard_normal((nrows, K)) * 3).astype(np.float32)
+    u = rng.standard_normal((nrows, K)).astype(np.float32)
+    gd, ud = _t(dev, g), _t(dev, u)
+    yd = torch.empty_like(gd)
+    act = torch.zeros(mi355.load().mi355_act_bytes(K, nrows), dtype=torch.uint8, device=dev)
+    mi355.check(mi355.load().mi355_swiglu_quant(None, gd.data_ptr(), ud.data_ptr(), K, yd.data_ptr(), K, act.data_ptr(), K, nrows))
+    y = yd.cpu().numpy()
+    s = np.zeros_like(g)
+    orc.oracle.orc_silu(orc._ptr(g), orc._ptr(s), g.size)
+    assert orc.nmse(y, s * u) < 1e-7
+    _check_act_matches_q8_1(act, y, K, nrows)
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+def test_rope_kv_store(dev, mode):
+    import torch
+    import mi355
+    rng = np.random.default_rng(3 + mode)
+    T, H, HK, D, n_ctx = 5, 8, 2, 128, 64
+    q = rng.standard_normal((T, H, D)).astype(np.float32)
+    k = rng.standard_normal((T, HK, D)).astype(np.float32)
+    v = rng.standard_normal((T, HK, D)).astype(np.float32)
+    pos = np.array([3, 4, 5, 100, 4000], dtype=np.int32)
+    cells = np.array([10, 11, 12, 0, 63], dtype=np.int32)
+    qd, kd, vd = _t(dev, q), _t(dev, k), _t(dev, v)
+    kc = torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+    vc = torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+    pd, cd = _t(dev, pos), _t(dev, cells)      # keep the device copies alive across the launch
+    mi355.check(mi355.load().mi355_rope_kv_store(None, qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                                 pd.data_ptr(), cd.data_ptr(), None, T, H, HK, D, HK * D * 2, D * 2,
+                                                 HK * D * 2, D * 2, D, mode, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0))
+    qr, kr = np.zeros_like(q), np.zeros_like(k)
+    orc.oracle.orc_rope(orc._ptr(q), orc._ptr(pos), None, orc._ptr(qr), D, H, T, D, mode, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 8192)
+    orc.oracle.orc_rope(orc._ptr(k), orc._ptr(pos), None, orc._ptr(kr), D, HK, T, D, mode, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 8192)
+    assert orc.nmse(qd.cpu().numpy(), qr) < 1e-7
+    kcn, vcn = kc.cpu().numpy().astype(np.float32), vc.cpu().numpy()
+    assert orc.nmse(kcn[cells], kr.astype(np.float16).astype(np.float32)) < 1e-6
+    assert np.array_equal(vcn[cells], v.astype(np.float16))
+    untouched = np.setdiff1d(np.arange(n_ctx), cells)
+    assert not kcn[untouched].any() and not vcn[untouched].any()
+
+
+@pytest.mark.parametrize("B", [1, 3, 8])
+def test_multi_matrix_gemv_with_residual(dev, B):
+    import torch
+    import mi355
+    rng = np.random.default_rng(B)
+    K = 4096
+    specs = [(orc.Q4_K, 1024), (orc.Q4_K, 512), (orc.Q6_K, 256), (orc.Q8_0, 130)]
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    act = mi355.quantize_act(_t(dev, x))
+    arr = (mi355.GemvMat * len(specs))()
+    keep, outs, wants = [], [], []
+    for i, (t, N) in enumerate(specs):
+        Wq = orc.quantize("oracle", t, (rng.standard_normal((N, K)) * 0.02).astype(np.float32))
+        Wd = mi355.upload_weights(t, _t(dev, Wq))
+        res = rng.standard_normal((B, N)).astype(np.float32)
+        out = _t(dev, res.copy())            # residual aliases dst
+        keep += [Wd, out]
+        arr[i].type, arr[i].W, arr[i].N, arr[i].dst, arr[i].dst_stride = t, Wd.data_ptr(), N, out.data_ptr(), N
+        arr[i].residual = out.data_ptr() if i % 2 == 0 else None
+        outs.append(out)
+        base = orc.mul_mat("q8_1", t, Wq, x)
+        wants.append(base + res if i % 2 == 0 else base)
+    mi355.check(mi355.load().mi355_mul_mat_vec_q_multi(None, len(specs), arr, act.data_ptr(), K, B))
+    torch.cuda.synchronize()
+    for out, want in zip(outs, wants):
+        assert orc.nmse(out.cpu().numpy(), want) < 1e-9
+
+
+def test_fused_layer_stack_matches_node_sequence(dev):
+    """two small llama layers: the fused launch sequence and the node-for-node one agree, decode and prefill"""
+    import torch
+    from mi355 import llama_graph as lg
+    cfg = lg.LlamaConfig(n_layer=2, n_embd=1024, n_ff=2048, n_head=8, n_head_kv=2, head_dim=128, n_vocab=512, n_ctx=256)
+    w = lg.LlamaWeights(cfg, dev, seed=7)
+    run = lg.LlamaRunner(w, max_tokens=64)
+    emb = torch.randn(64, cfg.n_embd).pin_memory()
+    for T, pos0 in [(40, 0), (1, 40), (3, 41)]:
+        run.set_inputs(emb, pos0, T, 256)
+        a = run.forward_nodes(T, 256, last_only=False).cpu().numpy().copy()
+        run.set_inputs(emb, pos0, T, 256)
+        b = run.forward(T, 256, last_only=False).cpu().numpy().copy()
+        assert np.isfinite(a).all() and np.isfinite(b).all()
+        assert orc.nmse(b, a) < 1e-5, (T, pos0)
