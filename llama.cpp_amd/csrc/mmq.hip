@@ -56,7 +56,7 @@ __device__ __forceinline__ void load_weight_stage(const uint8_t *__restrict__ W,
             const int64_t row = row0 + r < N ? row0 + r : N - 1;
             const uint8_t *wrow = W + row * L.row_bytes;
             const int64_t blk = (k0 >> 5) + b;
-            const u32x4 q = load_stream16(wrow + blk * 16);
+            const u32x4 q = load16(wrow + blk * 16);
             u32x4 lo, hi;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -76,7 +76,7 @@ __device__ __forceinline__ void load_weight_stage(const uint8_t *__restrict__ W,
             const int r = idx >> 3, c = idx & 7;   // c: 16-byte piece of the stage
             const int64_t row = row0 + r < N ? row0 + r : N - 1;
             const uint8_t *wrow = W + row * L.row_bytes;
-            const u32x4 q = load_stream16(wrow + k0 + c * 16);
+            const u32x4 q = load16(wrow + k0 + c * 16);
             *(u32x4 *)(sW + r * MMQ_LDK + c * 16) = q;
             if ((c & 1) == 0) {
                 const int b = c >> 1;
@@ -94,7 +94,7 @@ __device__ __forceinline__ void load_weight_stage(const uint8_t *__restrict__ W,
             const int gl = p >> 1, h = p & 1;
             const int64_t row = row0 + r < N ? row0 + r : N - 1;
             const uint8_t *blk = W + row * L.row_bytes + sb * Q4_K_BYTES;
-            const u32x4 q = load_stream16(blk + 16 + (half * 2 + gl) * 32 + h * 16);
+            const u32x4 q = load16(blk + 16 + (half * 2 + gl) * 32 + h * 16);
             u32x4 lo, hi;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -122,8 +122,8 @@ __device__ __forceinline__ void load_weight_stage(const uint8_t *__restrict__ W,
             const int l0 = 16 * (p & 1), qa = p >> 1;
             const int64_t row = row0 + r < N ? row0 + r : N - 1;
             const uint8_t *wrow = W + row * L.row_bytes;
-            const u32x4 ql = load_stream16(wrow + sb * 128 + hf * 64 + p * 16);
-            const u32x4 qh = load_stream16(wrow + L.off_b + sb * 64 + hf * 32 + l0);
+            const u32x4 ql = load16(wrow + sb * 128 + hf * 64 + p * 16);
+            const u32x4 qh = load16(wrow + L.off_b + sb * 64 + hf * 32 + l0);
             u32x4 vA, vB;
 #pragma unroll
             for (int i = 0; i < 4; i++) {

@@ -108,8 +108,10 @@ template <> struct wq<MI355_Q8_0> {
     struct act { u32x4 a0, a1; float d; };
     static __device__ __forceinline__ chunk load_w(const uint8_t *__restrict__ row, const row_layout &L, int c) {
         chunk w;
-        w.q0 = load_stream16(row + c * 32);
-        w.q1 = load_stream16(row + c * 32 + 16);
+        // the two loads of a wave interleave 16-byte pieces of the same 128-byte lines: a streaming
+        // (non-temporal) hint would fetch each line from HBM twice, so these stay ordinary loads
+        w.q0 = load16(row + c * 32);
+        w.q1 = load16(row + c * 32 + 16);
         w.d = half_bits_to_float(*(const unsigned short *)(row + L.off_b + c * 2));
         return w;
     }
@@ -144,9 +146,11 @@ template <> struct wq<MI355_Q4_K> {
         chunk w;
         const int sb = c >> 2, g = c & 3;
         const uint8_t *blk = row + sb * Q4_K_BYTES;
-        const u32x4 hdr = load_stream16(blk);   // d, dmin, 12 scale bytes: same address for the 4 lanes of a super-block
-        w.q0 = load_stream16(blk + 16 + g * 32);
-        w.q1 = load_stream16(blk + 32 + g * 32);
+        // header and both qs loads touch the same 128-byte lines from three instructions: ordinary
+        // (temporal) loads, so the line is fetched from HBM once and the other two hit in cache
+        const u32x4 hdr = load16(blk);   // d, dmin, 12 scale bytes: same address for the 4 lanes of a super-block
+        w.q0 = load16(blk + 16 + g * 32);
+        w.q1 = load16(blk + 32 + g * 32);
         w.d = half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu));
         w.dmin = half_bits_to_float((unsigned short)(hdr[0] >> 16));
         // all eight 6-bit (scale, min) pairs at once, branch-free (get_scale_min_k4, ggml-quants.c:631-638)
