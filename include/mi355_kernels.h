@@ -89,6 +89,19 @@ int mi355_mul_mat_vec_q(void *stream, int type, const void *W, const void *act, 
 int mi355_mul_mat_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
                     int64_t dst_stride);
 
+/* K-quant (Q4_K, Q6_K) tile GEMM with the activation format ggml-cpu uses for these weight
+ * types: one f32 scale per 256 elements (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516;
+ * vec_dot_type of type_traits_cpu, ggml/src/ggml-cpu/ggml-cpu.c:252-417), so the integer
+ * sub-scales fold into the int8 operands and the sums of a whole super-block stay integer
+ * (ggml_vec_dot_q4_K_q8_K / ggml_vec_dot_q6_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6817-6848,
+ * 8262-8283).  `act` layout: int8 q[nrows][k]; float d[nrows][k/256] (16-byte padded);
+ * fp16 bs[nrows][k/256][16] = {bsum_j & 63, bsum_j >> 6} of the eight 32-element sub-blocks.
+ * The levels and d are bit-identical to block_q8_K. */
+size_t mi355_act_q8k_bytes(int64_t k, int64_t nrows);
+int mi355_quantize_act_q8k(void *stream, const float *x, void *act, int64_t k, int64_t nrows, int64_t x_stride);
+int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                      int64_t dst_stride);
+
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE
  * launch, each optionally adding a residual in its epilogue (the ggml_add that follows the wo and

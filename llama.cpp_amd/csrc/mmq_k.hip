@@ -1,0 +1,448 @@
+// Batched GEMM for the K-quants (Q4_K, Q6_K) on the int8 matrix cores with integer
+// accumulation over whole 256-element super-blocks (B > 8):
+//   dst[b][n] = sum_k W[n][k] * x[b][k]
+//
+// Activations are quantized per super-block exactly as ggml-cpu does for these weight types
+// (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516: one f32 scale d8 per 256 elements,
+// int8 levels, integer sums per sub-block), so a super-block contributes
+//   Q4_K:  d*d8 * sum_j sc_j * (n . q)_j  -  dmin*d8 * sum_j m_j * bsum_j      (ggml-cpu-quants.c:6817-6848)
+//   Q6_K:  d*d8 * sum_g sc_g * ((l-32) . q)_g                                  (ggml-cpu-quants.c:8262-8283)
+// with every sum an exact integer.  The 6-bit / 8-bit sub-scales are folded into the weight
+// operand when a tile is unpacked to LDS: the integer sc*n (10 bits) or sc*(l-32) (14 bits) is
+// split into two int8 planes, value = R*hi + lo (R = 8 for Q4_K with sc = 8a+b, hi = a*n,
+// lo = b*n; R = 64 for Q6_K with hi = v >> 6, lo = v & 63).  Each plane is contracted with
+// v_mfma_i32_32x32x32_i8 into an int32 accumulator that runs over all 8 blocks of a
+// super-block, so the vector ALU touches a result tile once per 256 elements instead of once
+// per 32.  The Q4_K min term is one v_mfma_f32_32x32x16_f16 per super-block on exact small
+// integers: k slots 0..7 carry (bsum & 63) x m_j, slots 8..15 carry (bsum >> 6) x 64*m_j.
+//
+// A 256-thread group (4 waves, 2 x 2) owns a 64 (weight rows) x 128 (activation rows) tile of
+// dst; each wave a 32 x 64 sub-tile (1 x 2 MFMA tiles).  K is walked in stages of 128 elements; the global loads of
+// stage s+1 are issued before the MFMAs of stage s and unpacked to LDS after them.
+//
+// MFMA operand mapping (A = activations, B = weights, D[i][j]): lane l supplies row l % 32
+// and k bytes [16*(l/32), +16) (f16: k slots [8*(l/32), +8)); D register r of lane l is
+// i = 8*(r/4) + 4*(l/32) + r%4, j = l % 32.
+#include "common.hpp"
+#include "qdot.hpp"
+
+namespace mi355 {
+
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int KQ_BK = 128;            // K elements per stage (half a super-block)
+constexpr int KQ_LDK = KQ_BK + 16;    // LDS row pitch in bytes
+
+// ---- activation layout: int8 q[B][K]; float d8[B][K/256]; fp16 bs[B][K/256][16]
+// bs = {bsum_j & 63 (j = 0..7), bsum_j >> 6 (j = 0..7)} of the eight 32-element sub-blocks
+__host__ __device__ inline size_t q8k_d_offset(int64_t K, int64_t B) { return (size_t)B * (size_t)K; }
+__host__ __device__ inline size_t q8k_bs_offset(int64_t K, int64_t B) {
+    return (q8k_d_offset(K, B) + (size_t)B * (size_t)(K / QKK) * 4 + 15) & ~(size_t)15;   // bs entries are read 16 bytes at a time
+}
+
+// One wave per (row, super-block); 4 super-blocks per group.
+__global__ void __launch_bounds__(256) k_quantize_q8k(const float *__restrict__ x, int8_t *__restrict__ q, float *__restrict__ d8,
+                                                      _Float16 *__restrict__ bs, int64_t K, int64_t x_stride) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = blockIdx.y;
+    const int64_t nsb = K / QKK;
+    if (sb >= nsb) return;   // whole wave
+    const f32x4 v = *(const f32x4 *)(x + row * x_stride + sb * QKK + lane * 4);
+
+    // signed value of the first element with the largest magnitude
+    float amax = 0.0f, vmax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float ax = fabsf(v[i]);
+        if (ax > amax) { amax = ax; vmax = v[i]; }
+    }
+    int who = lane;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float oa = __shfl_xor(amax, off, 64), ov = __shfl_xor(vmax, off, 64);
+        const int ow = __shfl_xor(who, off, 64);
+        if (oa > amax || (oa == amax && ow < who)) { amax = oa; vmax = ov; who = ow; }
+    }
+
+    int lv[4] = {0, 0, 0, 0};
+    float d = 0.0f;
+    if (amax != 0.0f) {
+        const float iscale = -127.0f / vmax;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int n = (int)rintf(iscale * v[i]);
+            lv[i] = n < 127 ? n : 127;
+        }
+        d = 1.0f / iscale;
+    }
+    int sum = lv[0] + lv[1] + lv[2] + lv[3];
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) sum += __shfl_xor(sum, off, 64);
+
+    const u32 packed = (u32)(lv[0] & 0xFF) | ((u32)(lv[1] & 0xFF) << 8) | ((u32)(lv[2] & 0xFF) << 16) | ((u32)(lv[3] & 0xFF) << 24);
+    *(u32 *)(q + row * K + sb * QKK + lane * 4) = packed;
+    if (lane == 0) d8[row * nsb + sb] = d;
+    if ((lane & 7) == 0) {
+        _Float16 *o = bs + (row * nsb + sb) * 16;
+        o[lane >> 3] = (_Float16)(float)(sum & 63);
+        o[8 + (lane >> 3)] = (_Float16)(float)(sum >> 6);
+    }
+}
+
+// ---- per-thread prefetch registers of one stage -------------------------------------------
+// WI / AI: 16-byte weight pieces (of BM rows x 4) and activation pieces (of BN rows x 8) per thread
+template <int TYPE, int WI, int AI> struct kq_regs;
+template <int WI, int AI> struct kq_regs<MI355_Q4_K, WI, AI> {
+    u32x4 q[WI], hdr[WI];
+    u32x4 a[AI];
+};
+template <int WI, int AI> struct kq_regs<MI355_Q6_K, WI, AI> {
+    u32x4 ql[WI], qh[WI];
+    int scA[WI], scB[WI];   // int8 scales of the two 16-element groups of each chunk
+    float d[WI];
+    u32x4 a[AI];
+};
+
+struct kq_smem {
+    int8_t *sW1, *sW0, *sA;     // [128][KQ_LDK] planes
+    float *sWd, *sWn;           // [128] d and dmin of the current super-block
+    _Float16 *sWm;              // [128][16] m_j and 64*m_j (Q4_K)
+    float *sAd;                 // [128] d8
+    _Float16 *sAb;              // [128][16]
+};
+
+template <int TYPE, int WI, int AI>
+__device__ __forceinline__ void kq_fetch(kq_regs<TYPE, WI, AI> &R, const uint8_t *__restrict__ W, const row_layout &L, int64_t row0, int64_t N,
+                                         const int8_t *__restrict__ aq, int64_t col0, int64_t B, int64_t K, int64_t k0) {
+    const int tid = threadIdx.x;
+    const int64_t sb = k0 >> 8;
+    const int half = (int)((k0 >> 7) & 1);
+#pragma unroll
+    for (int it = 0; it < WI; it++) {
+        const int idx = tid + it * 256;
+        const int r = idx >> 2, p = idx & 3;
+        const int64_t row = row0 + r < N ? row0 + r : N - 1;
+        const uint8_t *wrow = W + row * L.row_bytes;
+        if constexpr (TYPE == MI355_Q4_K) {
+            const uint8_t *blk = wrow + sb * Q4_K_BYTES;
+            R.q[it] = load16(blk + 16 + (half * 2 + (p >> 1)) * 32 + (p & 1) * 16);
+            R.hdr[it] = load16(blk);
+        } else {
+            const int l0 = 16 * (p & 1), qa = p >> 1;
+            R.ql[it] = load16(wrow + sb * 128 + half * 64 + p * 16);
+            R.qh[it] = load16(wrow + L.off_b + sb * 64 + half * 32 + l0);
+            const int8_t *sc = (const int8_t *)(wrow + L.off_c + sb * 16 + half * 8 + (l0 >> 4));
+            R.scA[it] = sc[2 * qa];
+            R.scB[it] = sc[2 * qa + 4];
+            R.d[it] = half_bits_to_float(*(const unsigned short *)(wrow + L.off_d + sb * 2));
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < AI; it++) {
+        const int idx = tid + it * 256;
+        const int r = idx >> 3, c = idx & 7;
+        const int64_t col = col0 + r < B ? col0 + r : B - 1;
+        R.a[it] = load16(aq + col * K + k0 + c * 16);
+    }
+}
+
+// 4 packed bytes (each <= 15) times a small factor (<= 7): no byte overflows, so two 16-bit multiplies do it
+__device__ __forceinline__ u32 mul_bytes(u32 x, u32 f) {
+    const u16x2 v = __builtin_bit_cast(u16x2, x);
+    const u16x2 m = {(unsigned short)f, (unsigned short)f};
+    const u16x2 p = v * m;
+    return __builtin_bit_cast(u32, p);
+}
+
+// Q6_K: four unsigned 6-bit levels (bytes of a) -> int8 planes of sc*(level-32): value = 64*hi + lo
+__device__ __forceinline__ void q6k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
+    const i16x2 s = {(short)sc, (short)sc};
+    const i16x2 off = {(short)(-32 * sc), (short)(-32 * sc)};
+    const i16x2 e = __builtin_bit_cast(i16x2, a & 0x00FF00FFu);
+    const i16x2 o = __builtin_bit_cast(i16x2, (a >> 8) & 0x00FF00FFu);
+    const i16x2 pe = e * s + off, po = o * s + off;
+    const i16x2 six = {6, 6};
+    const u32 he = __builtin_bit_cast(u32, pe >> six), ho = __builtin_bit_cast(u32, po >> six);
+    const u32 le = __builtin_bit_cast(u32, pe) & 0x003F003Fu, lo_ = __builtin_bit_cast(u32, po) & 0x003F003Fu;
+    hi = (he & 0x00FF00FFu) | ((ho & 0x00FF00FFu) << 8);
+    lo = le | (lo_ << 8);
+}
+
+template <int TYPE, int WI, int AI>
+__device__ __forceinline__ void kq_commit(const kq_regs<TYPE, WI, AI> &R, const kq_smem &S, int half) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < WI; it++) {
+        const int idx = tid + it * 256;
+        const int r = idx >> 2, p = idx & 3;
+        if constexpr (TYPE == MI355_Q4_K) {
+            const int gl = p >> 1, h = p & 1;
+            const u32x4 hdr = R.hdr[it];
+            int scl, mnl, sch, mnh;
+            q4k_scale_min(hdr[1], hdr[2], hdr[3], half * 4 + 2 * gl, scl, mnl);
+            q4k_scale_min(hdr[1], hdr[2], hdr[3], half * 4 + 2 * gl + 1, sch, mnh);
+            u32x4 l1, l0, h1, h0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 nl = R.q[it][i] & 0x0F0F0F0Fu, nh = (R.q[it][i] >> 4) & 0x0F0F0F0Fu;
+                l1[i] = mul_bytes(nl, (u32)scl >> 3);
+                l0[i] = mul_bytes(nl, (u32)scl & 7u);
+                h1[i] = mul_bytes(nh, (u32)sch >> 3);
+                h0[i] = mul_bytes(nh, (u32)sch & 7u);
+            }
+            const int o = r * KQ_LDK + (2 * gl) * 32 + h * 16;
+            *(u32x4 *)(S.sW1 + o) = l1;
+            *(u32x4 *)(S.sW0 + o) = l0;
+            *(u32x4 *)(S.sW1 + o + 32) = h1;
+            *(u32x4 *)(S.sW0 + o + 32) = h0;
+            if (half == 0 && p == 0) {   // per super-block: d, dmin and the eight mins
+                S.sWd[r] = half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu));
+                S.sWn[r] = half_bits_to_float((unsigned short)(hdr[0] >> 16));
+                f16x8 m1, m64;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    int sc, mn;
+                    q4k_scale_min(hdr[1], hdr[2], hdr[3], j, sc, mn);
+                    m1[j] = (_Float16)(float)mn;
+                    m64[j] = (_Float16)(float)(64 * mn);
+                }
+                *(f16x8 *)(S.sWm + r * 16) = m1;
+                *(f16x8 *)(S.sWm + r * 16 + 8) = m64;
+            }
+        } else {
+            const int l0 = 16 * (p & 1), qa = p >> 1;
+            u32x4 a1, a0, b1, b0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 va = (R.ql[it][i] & 0x0F0F0F0Fu) | (((R.qh[it][i] >> (2 * qa)) & 0x03030303u) << 4);
+                const u32 vb = ((R.ql[it][i] >> 4) & 0x0F0F0F0Fu) | (((R.qh[it][i] >> (2 * qa + 4)) & 0x03030303u) << 4);
+                u32 hi, lo;
+                q6k_planes(va, R.scA[it], hi, lo);
+                a1[i] = hi; a0[i] = lo;
+                q6k_planes(vb, R.scB[it], hi, lo);
+                b1[i] = hi; b0[i] = lo;
+            }
+            const int o = r * KQ_LDK + qa * 32 + l0;
+            *(u32x4 *)(S.sW1 + o) = a1;
+            *(u32x4 *)(S.sW0 + o) = a0;
+            *(u32x4 *)(S.sW1 + o + 64) = b1;
+            *(u32x4 *)(S.sW0 + o + 64) = b0;
+            if (half == 0 && p == 0) S.sWd[r] = R.d[it];
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < AI; it++) {
+        const int idx = tid + it * 256;
+        const int r = idx >> 3, c = idx & 7;
+        *(u32x4 *)(S.sA + r * KQ_LDK + c * 16) = R.a[it];
+    }
+}
+
+// TW x TB: 32 x 32 MFMA tiles per wave along the weight / activation rows; waves are 2 x 2
+template <int TYPE, int TW, int TB, int OCC>
+__global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq, const float *__restrict__ ad8,
+                                                    const _Float16 *__restrict__ abs_, float *__restrict__ dst, int64_t N, int64_t K,
+                                                    int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles, int n_groups,
+                                                    int n_groups_padded) {
+    constexpr bool Q4 = TYPE == MI355_Q4_K;
+    constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
+    constexpr int BM = 64 * TW, BN = 64 * TB;
+    constexpr int WI = BM / 64, AI = BN / 32;
+    __shared__ __attribute__((aligned(16))) int8_t sW1[BM * KQ_LDK];
+    __shared__ __attribute__((aligned(16))) int8_t sW0[BM * KQ_LDK];
+    __shared__ __attribute__((aligned(16))) int8_t sA[BN * KQ_LDK];
+    __shared__ __attribute__((aligned(16))) float sWd[BM];
+    __shared__ __attribute__((aligned(16))) float sWn[Q4 ? BM : 4];
+    __shared__ __attribute__((aligned(16))) _Float16 sWm[Q4 ? BM * 16 : 8];
+    __shared__ __attribute__((aligned(16))) float sAd[BN];
+    __shared__ __attribute__((aligned(16))) _Float16 sAb[Q4 ? BN * 16 : 8];
+    const kq_smem S = {sW1, sW0, sA, sWd, sWn, sWm, sAd, sAb};
+
+    // hardware deals group ids round-robin over 8 XCDs; make logical neighbours (same weight panel) share one
+    const int per_xcd = n_groups_padded >> 3;
+    const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (lid >= n_groups) return;
+    const int64_t row0 = (int64_t)(lid / n_col_tiles) * BM;
+    const int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int wrow0 = (wave & 1) * (32 * TW);    // weight rows of this wave inside the tile
+    const int wcol0 = (wave >> 1) * (32 * TB);   // activation rows of this wave inside the tile
+    const int64_t nsb = K >> 8;
+
+    f32x16 acc[TB][TW];
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int tw = 0; tw < TW; tw++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[tb][tw][r] = 0.0f;
+
+    kq_regs<TYPE, WI, AI> R;
+    kq_fetch<TYPE, WI, AI>(R, W, L, row0, N, aq, col0, B, K, 0);
+
+    for (int64_t sb = 0; sb < nsb; sb++) {
+        i32x16 hi[TB][TW], lo[TB][TW];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int64_t k0 = sb * QKK + half * KQ_BK;
+            __syncthreads();   // everyone is done reading the previous stage
+            kq_commit<TYPE, WI, AI>(R, S, half);
+            if (half == 0 && tid < BN) {   // per super-block activation scale and sub-block sums
+                const int64_t col = col0 + tid < B ? col0 + tid : B - 1;
+                sAd[tid] = ad8[col * nsb + sb];
+                if constexpr (Q4) {
+                    const u32x4 *src = (const u32x4 *)(abs_ + (col * nsb + sb) * 16);
+                    *(u32x4 *)(sAb + tid * 16) = src[0];
+                    *(u32x4 *)(sAb + tid * 16 + 8) = src[1];
+                }
+            }
+            __syncthreads();
+            if (k0 + KQ_BK < K) kq_fetch<TYPE, WI, AI>(R, W, L, row0, N, aq, col0, B, K, k0 + KQ_BK);
+
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                i32x4 af[TB], b1[TW], b0[TW];
+#pragma unroll
+                for (int tb = 0; tb < TB; tb++) af[tb] = *(const i32x4 *)(sA + (wcol0 + tb * 32 + l32) * KQ_LDK + ks * 32 + 16 * lhi);
+#pragma unroll
+                for (int tw = 0; tw < TW; tw++) {
+                    b1[tw] = *(const i32x4 *)(sW1 + (wrow0 + tw * 32 + l32) * KQ_LDK + ks * 32 + 16 * lhi);
+                    b0[tw] = *(const i32x4 *)(sW0 + (wrow0 + tw * 32 + l32) * KQ_LDK + ks * 32 + 16 * lhi);
+                }
+#pragma unroll
+                for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+                    for (int tw = 0; tw < TW; tw++) {
+                        if (half == 0 && ks == 0) {   // first block of the super-block starts the integer sums
+                            i32x16 z;
+#pragma unroll
+                            for (int r = 0; r < 16; r++) z[r] = 0;
+                            hi[tb][tw] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tb], b1[tw], z, 0, 0, 0);
+                            lo[tb][tw] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tb], b0[tw], z, 0, 0, 0);
+                        } else {
+                            hi[tb][tw] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tb], b1[tw], hi[tb][tw], 0, 0, 0);
+                            lo[tb][tw] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tb], b0[tw], lo[tb][tw], 0, 0, 0);
+                        }
+                    }
+            }
+        }
+
+        // end of the super-block: scale the integer sums into the f32 accumulators
+#pragma unroll
+        for (int tb = 0; tb < TB; tb++) {
+            f32x4 d8[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) d8[q] = *(const f32x4 *)(sAd + wcol0 + tb * 32 + 8 * q + 4 * lhi);
+#pragma unroll
+            for (int tw = 0; tw < TW; tw++) {
+                const int wr = wrow0 + tw * 32 + l32;
+                const float dw = sWd[wr];
+                if constexpr (Q4) {
+                    const float dn = sWn[wr];
+                    const f16x8 am = *(const f16x8 *)(sAb + (wcol0 + tb * 32 + l32) * 16 + 8 * lhi);
+                    const f16x8 bm = *(const f16x8 *)(sWm + wr * 16 + 8 * lhi);
+                    f32x16 z;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                    const f32x16 M = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bm, z, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int t = (hi[tb][tw][r] << RADIX_SHIFT) + lo[tb][tw][r];
+                        acc[tb][tw][r] += d8[r >> 2][r & 3] * (dw * (float)t - dn * M[r]);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int t = (hi[tb][tw][r] << RADIX_SHIFT) + lo[tb][tw][r];
+                        acc[tb][tw][r] += d8[r >> 2][r & 3] * (dw * (float)t);
+                    }
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int tb = 0; tb < TB; tb++)
+#pragma unroll
+        for (int tw = 0; tw < TW; tw++) {
+            const int64_t n = row0 + wrow0 + tw * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                if (n < N && b < B) dst[b * dst_stride + n] = acc[tb][tw][r];
+            }
+        }
+}
+
+template <int TYPE, int TW, int TB, int OCC>
+static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                         int64_t dst_stride) {
+    constexpr int BM = 64 * TW, BN = 64 * TB;
+    const row_layout L = make_row_layout(TYPE, K);
+    const int8_t *aq = (const int8_t *)act;
+    const float *ad8 = (const float *)(aq + q8k_d_offset(K, B));
+    const _Float16 *abs_ = (const _Float16 *)(aq + q8k_bs_offset(K, B));
+    const int n_row_tiles = (int)((N + BM - 1) / BM);
+    const int n_col_tiles = (int)((B + BN - 1) / BN);
+    const int n_groups = n_row_tiles * n_col_tiles;
+    const int n_groups_padded = (n_groups + 7) & ~7;
+    hipLaunchKernelGGL((k_mmq_k<TYPE, TW, TB, OCC>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_,
+                       dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded);
+}
+
+// 64 x 128 tiles: 96 accumulator registers per lane leave room for two groups per CU, which
+// measured faster than 128 x 128 tiles at one group per CU
+template <int TYPE>
+static void launch_mmq_k_any(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                             int64_t dst_stride) {
+    launch_mmq_k<TYPE, 1, 2, 2>(s, W, act, dst, N, K, B, dst_stride);
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+size_t mi355_act_q8k_bytes(int64_t k, int64_t nrows) {
+    if (k <= 0 || nrows <= 0 || k % QKK != 0) return 0;
+    return q8k_bs_offset(k, nrows) + (size_t)nrows * (size_t)(k / QKK) * 32;
+}
+
+int mi355_quantize_act_q8k(void *stream, const float *x, void *act, int64_t k, int64_t nrows, int64_t x_stride) {
+    MI355_REQUIRE(k > 0 && k % QKK == 0, "quantize_act_q8k: k=%lld is not a multiple of 256", (long long)k);
+    MI355_REQUIRE(nrows >= 0 && nrows <= 65535, "quantize_act_q8k: nrows=%lld out of range", (long long)nrows);
+    MI355_REQUIRE(x_stride >= k && x_stride % 4 == 0 && ((uintptr_t)x & 15) == 0, "quantize_act_q8k: x must be 16-byte aligned with a row stride that is a multiple of 4 floats");
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0, "quantize_act_q8k: workspace must be 16-byte aligned");
+    if (nrows == 0) return MI355_OK;
+    int8_t *q = (int8_t *)act;
+    float *d8 = (float *)(q + q8k_d_offset(k, nrows));
+    _Float16 *bs = (_Float16 *)(q + q8k_bs_offset(k, nrows));
+    const dim3 grid((unsigned)((k / QKK + 3) / 4), (unsigned)nrows);
+    hipLaunchKernelGGL(k_quantize_q8k, grid, dim3(256), 0, (hipStream_t)stream, x, q, d8, bs, k, x_stride);
+    return launch_status("k_quantize_q8k");
+}
+
+int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                      int64_t dst_stride) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
+    MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k: K=%lld is not a multiple of 256", (long long)K);
+    MI355_REQUIRE(dst_stride >= N, "mul_mat_q8k: dst_stride < N");
+    const row_layout L = make_row_layout(type, K);
+    MI355_REQUIRE(layout_aligned(W, L), "mul_mat_q8k: weight rows are not 16-byte aligned (K=%lld)", (long long)K);
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0 && (q8k_d_offset(K, B) & 15) == 0 && (q8k_bs_offset(K, B) & 15) == 0,
+                  "mul_mat_q8k: activation workspace is not 16-byte aligned");
+    MI355_REQUIRE((N + 63) / 64 * ((B + 63) / 64) < (1 << 30), "mul_mat_q8k: too many tiles");
+    hipStream_t s = (hipStream_t)stream;
+    if (type == MI355_Q4_K) launch_mmq_k_any<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride);
+    else launch_mmq_k_any<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride);
+    return launch_status("k_mmq_k");
+}
+
+}  // extern "C"

@@ -48,7 +48,12 @@ using namespace mi355;
 
 extern "C" {
 
+// the per-super-block activation format of the K-quant tile kernel is smaller than the Q8_1 one
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B) { return (mi355_act_bytes(K, B) + 255) & ~(size_t)255; }
+
+static bool use_q8k_tiles(int type, const void *W, int64_t K, int64_t B) {
+    return B > 8 && (type == MI355_Q4_K || type == MI355_Q6_K) && layout_aligned(W, make_row_layout(type, K));
+}
 
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
                   int64_t x_stride, int64_t dst_stride, void *ws, size_t ws_bytes) {
@@ -59,6 +64,11 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
     if (ws_bytes < mi355_mul_mat_ws_bytes(K, B) || ws == nullptr) {
         set_error("mul_mat: workspace of %zu bytes, need %zu", ws_bytes, mi355_mul_mat_ws_bytes(K, B));
         return MI355_ERR_WORKSPACE;
+    }
+    if (use_q8k_tiles(type, W, K, B)) {
+        int rc = mi355_quantize_act_q8k(stream, x, ws, K, B, x_stride);
+        if (rc != MI355_OK) return rc;
+        return mi355_mul_mat_q8k(stream, type, W, ws, dst, N, K, B, dst_stride);
     }
     int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
     if (rc != MI355_OK) return rc;

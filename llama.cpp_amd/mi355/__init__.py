@@ -40,6 +40,9 @@ _SIGNATURES = {
     "mi355_mul_mat": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_vec_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_act_q8k_bytes": (_sz, [_i64, _i64]),
+    "mi355_quantize_act_q8k": (_int, [_p, _p, _p, _i64, _i64, _i64]),
+    "mi355_mul_mat_q8k": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_rms_norm_mul_quant": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
     "mi355_swiglu_quant": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
@@ -167,6 +170,15 @@ def quantize_act(x):
     nrows, k = x.shape
     ws = torch.empty(load().mi355_act_bytes(k, nrows), dtype=torch.uint8, device=x.device)
     check(load().mi355_quantize_act(_stream(), _ptr(x), _ptr(ws), k, nrows, x.stride(0)))
+    return ws
+
+
+def quantize_act_q8k(x):
+    """x f32 [nrows, k] -> workspace in the per-super-block layout (int8 levels, f32 d per 256, fp16 sub-block sums)"""
+    import torch
+    nrows, k = x.shape
+    ws = torch.empty(load().mi355_act_q8k_bytes(k, nrows), dtype=torch.uint8, device=x.device)
+    check(load().mi355_quantize_act_q8k(_stream(), _ptr(x), _ptr(ws), k, nrows, x.stride(0)))
     return ws
 
 

@@ -158,11 +158,24 @@ class LlamaRunner:
                                             self.fa_ws.numel()))
 
     # ---- fused operators ------------------------------------------------------------------------
-    def _norm_quant(self, x, w, act, T):
-        K = x.shape[1]
-        check(self.lib.mi355_rms_norm_mul_quant(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
+    @staticmethod
+    def _q8k_ok(mats, K):
+        """the super-block tile GEMM serves K-quants whose device rows are 16-byte aligned"""
+        return all(t == Q4_K or (t == Q6_K and K % 2048 == 0) for (t, _), _ in mats)
 
-    def _mm_act(self, mats, act, K, T, residual=None):
+    def _quant(self, src, act, K, T, q8k):
+        fn = self.lib.mi355_quantize_act_q8k if q8k else self.lib.mi355_quantize_act
+        check(fn(_stream(), _ptr(src), _ptr(act), K, T, src.stride(0)))
+
+    def _norm_quant(self, x, w, act, T, q8k=False):
+        K = x.shape[1]
+        if q8k:     # prefill: normalised rows in f32, then one scale per 256 elements
+            check(self.lib.mi355_rms_norm_mul_quant(_stream(), _ptr(x), x.stride(0), _ptr(w), _ptr(self.t0), self.t0.stride(0), None, K, T, self.cfg.rms_eps))
+            self._quant(self.t0, act, K, T, True)
+        else:
+            check(self.lib.mi355_rms_norm_mul_quant(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
+
+    def _mm_act(self, mats, act, K, T, residual=None, q8k=False):
         """mats: list of ((type, W), out); all consume the quantized activation `act` (T rows of K)"""
         if T <= 8:
             arr = (GemvMat * len(mats))()
@@ -171,9 +184,10 @@ class LlamaRunner:
                 arr[i].residual = residual.data_ptr() if residual is not None else None
             check(self.lib.mi355_mul_mat_vec_q_multi(_stream(), len(mats), arr, _ptr(act), K, T))
         else:
+            fn = self.lib.mi355_mul_mat_q8k if q8k else self.lib.mi355_mul_mat_q
             for (t, W), out in mats:
                 dst = out if residual is None else self.t1[:T]
-                check(self.lib.mi355_mul_mat_q(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), out.shape[1], K, T, dst.stride(0)))
+                check(fn(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), out.shape[1], K, T, dst.stride(0)))
                 if residual is not None:
                     self._bin(0, dst, residual, out)
 
@@ -182,24 +196,39 @@ class LlamaRunner:
         cfg, w, lib = self.cfg, self.w, self.lib
         E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
         x = self.x[:T]
+        big = T > 8
         for il, L in enumerate(w.layers):
-            self._norm_quant(x, L["attn_norm"], self.act_a, T)
-            self._mm_act([(L["wq"], self.q[:T]), (L["wk"], self.k[:T]), (L["wv"], self.v[:T])], self.act_a, E, T)
+            qkv = [(L["wq"], self.q[:T]), (L["wk"], self.k[:T]), (L["wv"], self.v[:T])]
+            kq = big and self._q8k_ok(qkv, E)
+            self._norm_quant(x, L["attn_norm"], self.act_a, T, kq)
+            self._mm_act(qkv, self.act_a, E, T, q8k=kq)
             kc, vc = self.kcache[il], self.vcache[il]
             check(lib.mi355_rope_kv_store(_stream(), _ptr(self.q), _ptr(self.k), _ptr(self.v), _ptr(kc), _ptr(vc), _ptr(self.pos), _ptr(self.pos),
                                           None, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2, vc.stride(1) * 2, D, 0,
                                           cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
             self._attn(il, T, n_kv)
-            check(lib.mi355_quantize_act(_stream(), _ptr(self.attn), _ptr(self.act_a), H * D, T, H * D))
-            self._mm_act([(L["wo"], x)], self.act_a, H * D, T, residual=x)
-            self._norm_quant(x, L["ffn_norm"], self.act_a, T)
-            self._mm_act([(L["gate"], self.gate[:T]), (L["up"], self.up[:T])], self.act_a, E, T)
-            check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
-            self._mm_act([(L["down"], x)], self.act_b, F, T, residual=x)
+            wo = [(L["wo"], x)]
+            kq = big and self._q8k_ok(wo, H * D)
+            self._quant(self.attn, self.act_a, H * D, T, kq)
+            self._mm_act(wo, self.act_a, H * D, T, residual=x, q8k=kq)
+            gu = [(L["gate"], self.gate[:T]), (L["up"], self.up[:T])]
+            kq = big and self._q8k_ok(gu, E)
+            self._norm_quant(x, L["ffn_norm"], self.act_a, T, kq)
+            self._mm_act(gu, self.act_a, E, T, q8k=kq)
+            down = [(L["down"], x)]
+            kq = big and self._q8k_ok(down, F)
+            if kq:
+                check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, _ptr(self.gate), F, None, F, T))
+                self._quant(self.gate, self.act_b, F, T, True)
+            else:
+                check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
+            self._mm_act(down, self.act_b, F, T, residual=x, q8k=kq)
         To = 1 if last_only else T
         xo = self.x[T - 1:T] if last_only else x
-        self._norm_quant(xo, w.output_norm, self.act_a, To)
-        self._mm_act([(w.output, self.logits[:To])], self.act_a, E, To)
+        out = [(w.output, self.logits[:To])]
+        kq = To > 8 and self._q8k_ok(out, E)
+        self._norm_quant(xo, w.output_norm, self.act_a, To, kq)
+        self._mm_act(out, self.act_a, E, To, q8k=kq)
         return self.logits[:To]
 
     # ---- the same pass node for node, as the ggml graph lists it (reference for the fused path) --

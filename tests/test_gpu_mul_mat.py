@@ -105,6 +105,41 @@ def test_gemv_matches_oracle(dev, name, t, N, K, B):
     assert orc.nmse(got[:, :cpu.shape[1]], cpu) <= 5e-4      # tests/test-backend-ops.cpp:1916
 
 
+@pytest.mark.parametrize("K", [256, 4096, 14336])
+@pytest.mark.parametrize("dist", ["normal", "special"])
+def test_quantize_q8k_bit_exact(dev, K, dist):
+    """levels and scale equal block_q8_K of the reference; the sub-block sums are its bsums pairwise"""
+    import mi355
+    rng = np.random.default_rng(11 + K)
+    nrows = 6
+    x = rng.standard_normal((nrows, K)).astype(np.float32)
+    if dist == "special":
+        x[0, :256] = 0.0                       # all-zero super-block: d = 0, levels 0
+        x[1, :256] = 0.0
+        x[1, 77] = 2.5                         # single +amax: its level is exactly -127 and d is negative
+        x[2, 3] = 9.0
+        x[2, 200] = -9.0                       # equal magnitudes: the first one decides the sign of the scale
+        x[3, :256] = -1e-30
+        x[4, :256] = 0.0
+        x[4, 0] = -127.0                       # scale exactly 1: the values below are exact .5 ties (round half to even)
+        x[4, 1:202] = np.arange(-100, 101) + 0.5
+    got = mi355.quantize_act_q8k(_to_dev(dev, x)).cpu().numpy()
+    nsb = K // 256
+    q = got[:nrows * K].view(np.int8).reshape(nrows, nsb, 256)
+    d = got[nrows * K:nrows * K + nrows * nsb * 4].view(np.float32).reshape(nrows, nsb)
+    off = (nrows * K + nrows * nsb * 4 + 15) // 16 * 16
+    bs = got[off:off + nrows * nsb * 32].view(np.float16).reshape(nrows, nsb, 16).astype(np.int64)
+    for kind in ["oracle"] + (["ref"] if orc.ref is not None else []):
+        want = orc.quantize(kind, orc.Q8_K, x).reshape(nrows, nsb, 292)
+        wd = np.ascontiguousarray(want[:, :, :4]).view(np.float32).reshape(nrows, nsb)
+        wq = want[:, :, 4:260].view(np.int8)
+        assert np.array_equal(d.view(np.uint32), wd.view(np.uint32))
+        assert np.array_equal(q, wq)
+        sums = wq.astype(np.int64).reshape(nrows, nsb, 8, 32).sum(axis=3)
+        assert np.array_equal(64 * bs[:, :, 8:] + bs[:, :, :8], sums)
+        assert bs[:, :, :8].min() >= 0 and bs[:, :, :8].max() <= 63
+
+
 @pytest.mark.parametrize("name,t", TYPES)
 @pytest.mark.parametrize("N,K,B", [(512, 4096, 64), (384, 2048, 512), (130, 1024, 33), (4096, 4096, 9), (128, 14336, 100)])
 def test_mmq_matches_oracle(dev, name, t, N, K, B):
@@ -115,12 +150,34 @@ def test_mmq_matches_oracle(dev, name, t, N, K, B):
     Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
     got = mi355.mul_mat(t, Wd, _to_dev(dev, x)).cpu().numpy()
     Nt, Bt = min(N, 64), min(B, 24)
-    want = orc.mul_mat("q8_1", t, Wq[:Nt], x[:Bt])
-    tol = 1e-6 if t == orc.Q4_K else 1e-9    # Q4_K adds its min term through fp16 operands
-    assert orc.nmse(got[:Bt, :Nt], want) < tol
+    if B > 8 and (t == orc.Q4_K or (t == orc.Q6_K and K % 2048 == 0)):   # Q6_K rows are 16-byte aligned only then
+        # K-quants take the activation format of the CPU path (one scale per 256): integer sums are the
+        # CPU's own (ggml-cpu-quants.c:6817-6848, 8262-8283), only the f32 summation order differs
+        want = orc.mul_mat("cpu", t, Wq[:Nt], x[:Bt])
+    else:
+        want = orc.mul_mat("q8_1", t, Wq[:Nt], x[:Bt])
+    assert orc.nmse(got[:Bt, :Nt], want) < 1e-9
     if orc.ref is not None:
         cpu = orc.mul_mat("ref", t, Wq, x)
         assert orc.nmse(got, cpu) <= 5e-4
+
+
+@pytest.mark.parametrize("name,t", [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q6_K)])
+@pytest.mark.parametrize("N,K,B", [(256, 4096, 64), (130, 1024, 33)])
+def test_mmq_q8_1_path_for_k_quants(dev, name, t, N, K, B):
+    """the per-32-block tile kernel stays reachable for K-quants through mi355_mul_mat_q"""
+    import mi355
+    import torch
+    rng = np.random.default_rng(N + K + B)
+    Wq = _weights(rng, t, N, K)
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
+    act = mi355.quantize_act(_to_dev(dev, x))
+    dst = torch.empty((B, N), dtype=torch.float32, device=dev)
+    mi355.check(mi355.load().mi355_mul_mat_q(None, t, Wd.data_ptr(), act.data_ptr(), dst.data_ptr(), N, K, B, N))
+    torch.cuda.synchronize()
+    tol = 1e-6 if t == orc.Q4_K else 1e-9    # Q4_K adds its min term through fp16 operands
+    assert orc.nmse(dst.cpu().numpy()[:24, :64], orc.mul_mat("q8_1", t, Wq[:64], x[:24])) < tol
 
 
 @pytest.mark.parametrize("name,t", TYPES)
@@ -135,5 +192,6 @@ def test_unaligned_rows_fallback(dev, name, t):
         x = rng.standard_normal((B, K)).astype(np.float32)
         Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
         got = mi355.mul_mat(t, Wd, _to_dev(dev, x)).cpu().numpy()
-        # B > 8 with K % 128 == 0 takes the MFMA kernel, whose Q4_K min term goes through fp16 operands
-        assert orc.nmse(got, orc.mul_mat("q8_1", t, Wq, x)) < (1e-6 if (t == orc.Q4_K and B > 8) else 1e-9)
+        # Q4_K rows are always aligned, so B > 8 takes the super-block tile kernel and the CPU's activation format
+        want = orc.mul_mat("cpu" if (t == orc.Q4_K and B > 8) else "q8_1", t, Wq, x)
+        assert orc.nmse(got, want) < 1e-9
