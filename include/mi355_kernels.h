@@ -155,6 +155,15 @@ int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void
                          size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
                          float max_bias, float logit_softcap, void *ws, size_t ws_bytes);
 
+/* Same, and also writes the Q8_1 quantization of dst (one activation row of Hq*D elements per
+ * query, layout of mi355_quantize_act) for the attention-output projection that follows it in
+ * llm_build_kv (src/llama.cpp:157-199), saving that MUL_MAT's separate quantization pass.
+ * act may be NULL; D % 32 == 0 is required otherwise. */
+int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
+                         int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
+                         size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
+                         float max_bias, float logit_softcap, void *ws, size_t ws_bytes, void *act);
+
 /* Glue operators -------------------------------------------------------------------- *
  * A strided f32/f16/i32 operand: up to 4 dimensions, ne[] elements, nb[] byte strides
  * (the fields of struct ggml_tensor, ggml/include/ggml.h:576-608). */
@@ -213,6 +222,17 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
                         const int32_t *cells, const float *freq_factors, int64_t T, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
                         size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                         float ext_factor, float attn_factor, float beta_fast, float beta_slow);
+
+/* The Q, K and V projections of build_llama (src/llama.cpp:1514-1533) in ONE bandwidth-bound launch whose epilogue does what the graph
+ * does next: ROPE(q) into q f32 [B][H][D]; ROPE(k) and CPY into the f16 K cache; CPY(v) into the f16 V cache (src/llama.cpp:1535-1548,
+ * llm_build_kv_store :157-199; ggml-cpu.c:9366-9549, 3519-3830).  wq/wk/wv: device-layout rows of K (16-byte aligned rows required);
+ * act from mi355_quantize_act / mi355_rms_norm_mul_quant (B <= 4 rows).  Cache addressing and pos/cells as in mi355_rope_kv_store.
+ * Only the adjacent-pair rope mode (mode 0) is fused: a wave owns output rows 2i and 2i+1. */
+int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, const void *wk, int type_v, const void *wv, const void *act,
+                         float *q, void *kcache, void *vcache, const int32_t *pos, const int32_t *cells, const float *freq_factors,
+                         int64_t K, int64_t B, int64_t H, int64_t HK, int64_t D, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2,
+                         int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
+                         float beta_fast, float beta_slow);
 
 /* MUL_MAT with f32 or f16 src0 and f32 src1 (router / small dense matrices): dst[b][n] = sum_k W[n][k] x[b][k], strides honoured, ne2/ne3 broadcast */
 int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *src1, const mi355_tensor *dst);

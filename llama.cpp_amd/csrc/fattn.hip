@@ -41,9 +41,13 @@ __device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
     return s;
 }
 
+__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e);
+
 struct fattn_args {
     const uint8_t *q, *k, *v, *mask;
     float *dst;      // [D, Hq, Nq]
+    int8_t *act_q;   // optional: Q8_1 of dst rows (Hq*D elements per query) in the split activation layout
+    act_ds *act_s;
     float *ws;       // partial results when n_splits > 1: [Nq][Hq][n_splits][D + 2]
     int64_t Nq, Nkv, Hq, Hkv;
     size_t q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1;
@@ -182,7 +186,9 @@ __global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
         }
         const int64_t head = head0 + r;
         if (a.n_splits == 1) {
-            a.dst[(iq * a.Hq + head) * D + d] = O / L;
+            const float o = O / L;
+            a.dst[(iq * a.Hq + head) * D + d] = o;
+            if (a.act_q) quantize_lane32(o, a.act_q + iq * a.Hq * D, a.act_s + iq * (a.Hq * D / 32), head * D + d);
         } else {
             float *p = a.ws + ((iq * a.Hq + head) * a.n_splits + split) * (D + 2);
             p[d] = O;
@@ -195,7 +201,8 @@ __global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
 }
 
 template <int D>
-__global__ void k_fattn_combine(const float *__restrict__ ws, float *__restrict__ dst, int n_splits) {
+__global__ void k_fattn_combine(const float *__restrict__ ws, float *__restrict__ dst, int n_splits, int8_t *__restrict__ act_q,
+                                act_ds *__restrict__ act_s, int64_t Hq) {
     const int64_t row = blockIdx.x;   // iq * Hq + head
     const float *p = ws + row * n_splits * (D + 2);
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
@@ -207,7 +214,33 @@ __global__ void k_fattn_combine(const float *__restrict__ ws, float *__restrict_
             L += p[s * (D + 2) + D + 1] * f;
             O += p[s * (D + 2) + d] * f;
         }
-        dst[row * D + d] = O / L;
+        const float o = O / L;
+        dst[row * D + d] = o;
+        if (act_q) {
+            const int64_t iq = row / Hq, head = row % Hq;
+            quantize_lane32(o, act_q + iq * Hq * D, act_s + iq * (Hq * D / 32), head * D + d);
+        }
+    }
+}
+
+// Q8_1 of one value per lane, 32 consecutive lanes = one block (quantize_row_q8_1_ref,
+// ggml/src/ggml-quants.c:220-253); e = element index inside the query row of k elements
+__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q = (int)roundf(v * id);
+    int sum = q;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    qrow[e] = (int8_t)q;
+    if ((e & 31) == 0) {
+        act_ds o;
+        o.d = half_bits_to_float(float_to_half_bits(d));
+        o.sum = sum;
+        srow[e >> 5] = o;
     }
 }
 
@@ -228,7 +261,8 @@ static int launch_vec(hipStream_t s, fattn_args &a) {
     int rc = launch_status("k_fattn_vec");
     if (rc != MI355_OK) return rc;
     if (a.n_splits > 1) {
-        hipLaunchKernelGGL(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(D <= 128 ? 128 : 256), 0, s, a.ws, a.dst, a.n_splits);
+        hipLaunchKernelGGL(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(D <= 128 ? 128 : 256), 0, s, a.ws, a.dst, a.n_splits, a.act_q,
+                           a.act_s, a.Hq);
         rc = launch_status("k_fattn_combine");
     }
     return rc;
@@ -254,10 +288,10 @@ size_t mi355_flash_attn_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq)
     return (size_t)Nq * (size_t)Hq * 256 * (size_t)(D + 2) * sizeof(float);
 }
 
-int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
-                         int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
-                         size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
-                         float max_bias, float logit_softcap, void *ws, size_t ws_bytes) {
+int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
+                               int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
+                               size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
+                               float max_bias, float logit_softcap, void *ws, size_t ws_bytes, void *act) {
     MI355_REQUIRE(D > 0 && D % 8 == 0 && D <= 256, "flash_attn: head size %lld not supported", (long long)D);
     MI355_REQUIRE(Nq > 0 && Nkv > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "flash_attn: bad shape");
     MI355_REQUIRE(Nq <= 65535 && Hq <= 65535, "flash_attn: too many query rows or heads for one launch");
@@ -265,7 +299,10 @@ int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void
     MI355_REQUIRE(((uintptr_t)k & 15) == 0 && k_nb1 % 16 == 0 && k_nb2 % 16 == 0, "flash_attn: k rows must be 16-byte aligned");
     MI355_REQUIRE(((uintptr_t)v & 15) == 0 && v_nb1 % 16 == 0 && v_nb2 % 16 == 0, "flash_attn: v rows must be 16-byte aligned");
     MI355_REQUIRE(max_bias <= 0.0f || mask != nullptr, "flash_attn: max_bias needs a mask");
+    MI355_REQUIRE(act == nullptr || (D % 32 == 0 && ((uintptr_t)act & 15) == 0), "flash_attn: quantized output needs head size %% 32 == 0 and a 16-byte aligned buffer");
     fattn_args a;
+    a.act_q = (int8_t *)act;
+    a.act_s = act ? (act_ds *)((int8_t *)act + Nq * Hq * D) : nullptr;
     a.q = (const uint8_t *)q; a.k = (const uint8_t *)k; a.v = (const uint8_t *)v; a.mask = (const uint8_t *)mask;
     a.dst = dst; a.ws = (float *)ws;
     a.Nq = Nq; a.Nkv = Nkv; a.Hq = Hq; a.Hkv = Hkv;
@@ -294,6 +331,14 @@ int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void
         case 256: return launch_vec_r<256>(s, a, R);
         default: set_error("flash_attn: head size %lld not supported", (long long)D); return MI355_ERR_ARG;
     }
+}
+
+int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
+                         int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
+                         size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
+                         float max_bias, float logit_softcap, void *ws, size_t ws_bytes) {
+    return mi355_flash_attn_ext_quant(stream, q, k, v, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1,
+                                      scale, max_bias, logit_softcap, ws, ws_bytes, nullptr);
 }
 
 }  // extern "C"

@@ -12,6 +12,7 @@
 #include "common.hpp"
 #include "qdot.hpp"
 
+#include <math.h>
 #include <stdlib.h>
 
 namespace mi355 {
@@ -24,15 +25,43 @@ struct gemv_item {
     int64_t dst_stride;
     int type;
     int first_group;         // index of this matrix's first group in the launch
+    int epi;                 // EPI_*: what happens to a finished row
+    int64_t nb1, nb2;        // EPI_*_CACHE: byte strides of a cache cell and of a head inside it (dst = cache base)
 };
+enum { EPI_STORE = 0, EPI_ROPE = 1, EPI_ROPE_CACHE = 2, EPI_CACHE = 3 };
+
+// rotary embedding of the Q/K rows produced by the fused QKV launch (mode 0: adjacent pairs)
+struct gemv_rope {
+    const int32_t *pos;      // [B] rope position of each activation row
+    const int32_t *cells;    // [B] cache cell of each activation row
+    const float *ff;         // frequency factors [n_dims/2] or null
+    int D, n_dims;
+    float theta_scale, freq_scale, ext_factor, attn_factor, corr0, corr1;
+};
+
+// rope_yarn + rotation, same roundings as k_rope (glue.hip) and k_rope_kv_store (fused.hip); ggml-cpu.c:9268-9306
+__device__ __forceinline__ void rope_rotate(const gemv_rope &a, int pos, int pair, float x0, float x1, float &y0, float &y1) {
+    const float theta_extrap = (float)pos * powf(a.theta_scale, (float)pair) / (a.ff ? a.ff[pair] : 1.0f);
+    const float theta_interp = a.freq_scale * theta_extrap;
+    float theta = theta_interp, mscale = a.attn_factor;
+    if (a.ext_factor != 0.0f) {
+        const float yv = ((float)pair - a.corr0) / fmaxf(0.001f, a.corr1 - a.corr0);
+        const float ramp = (1.0f - fminf(1.0f, fmaxf(0.0f, yv))) * a.ext_factor;
+        theta = theta_interp * (1.0f - ramp) + theta_extrap * ramp;
+        mscale *= 1.0f + 0.1f * logf(1.0f / a.freq_scale);
+    }
+    const float c = cosf(theta) * mscale, s = sinf(theta) * mscale;
+    y0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
+    y1 = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+}
 struct gemv_batch {
     gemv_item it[4];
     int n;
 };
 
-template <int TYPE, int NCOLS, int RPW>
+template <int TYPE, int NCOLS, int RPW, bool QKV = false>
 __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const int8_t *__restrict__ aq,
-                                          const act_ds *__restrict__ ads, int K) {
+                                          const act_ds *__restrict__ ads, int K, const gemv_rope *rp = nullptr) {
     typedef wq<TYPE> T;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -74,16 +103,44 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
         }
     }
 
-#pragma unroll
-    for (int r = 0; r < RPW; r++)
+    if constexpr (QKV) {
+        // RPW == 2: the wave owns the adjacent rows (row0, row0 + 1) = one rotation pair of one head.
+        // Every lane gets all sums; lane c finishes activation row c.
+        static_assert(RPW == 2, "the rope epilogue pairs the two rows of a wave");
+        float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
         for (int c = 0; c < NCOLS; c++) {
-            const float s = wave_sum(acc[r][c]);
-            if (lane == 0 && row0 + r < m.N) {
-                const int64_t o = c * m.dst_stride + row0 + r;
-                m.dst[o] = m.residual ? s + m.residual[o] : s;
+            const float a0 = wave_sum(acc[0][c]), a1 = wave_sum(acc[1][c]);
+            if (lane == c) { s0 = a0; s1 = a1; }
+        }
+        if (lane < NCOLS && row0 + 1 < m.N) {
+            const gemv_rope &R = *rp;
+            const int64_t head = row0 / R.D;
+            const int d = (int)(row0 % R.D);
+            float y0 = s0, y1 = s1;
+            if (m.epi != EPI_CACHE && d < R.n_dims) rope_rotate(R, R.pos[lane], d >> 1, s0, s1, y0, y1);
+            if (m.epi == EPI_ROPE) {
+                float *o = m.dst + lane * m.dst_stride + row0;
+                o[0] = y0;
+                o[1] = y1;
+            } else {
+                _Float16 *o = (_Float16 *)((uint8_t *)m.dst + (int64_t)R.cells[lane] * m.nb1 + head * m.nb2) + d;
+                o[0] = (_Float16)y0;
+                o[1] = (_Float16)y1;
             }
         }
+    } else {
+#pragma unroll
+        for (int r = 0; r < RPW; r++)
+#pragma unroll
+            for (int c = 0; c < NCOLS; c++) {
+                const float s = wave_sum(acc[r][c]);
+                if (lane == 0 && row0 + r < m.N) {
+                    const int64_t o = c * m.dst_stride + row0 + r;
+                    m.dst[o] = m.residual ? s + m.residual[o] : s;
+                }
+            }
+    }
 }
 
 template <int NCOLS, int RPW>
@@ -94,6 +151,24 @@ __device__ __forceinline__ void gemv_dispatch(const gemv_item &m, int group, con
         case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW>(m, group, aq, ads, K); break;
         case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW>(m, group, aq, ads, K); break;
         default: gemv_body<MI355_Q6_K, NCOLS, RPW>(m, group, aq, ads, K); break;
+    }
+}
+
+// Q, K and V projections in one launch; finished rows are rotated and land in q (f32) or in the f16 KV cache
+template <int NCOLS>
+__global__ void __launch_bounds__(256) k_gemv_qkv(gemv_batch b, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K, gemv_rope rp) {
+    const int g = blockIdx.x;
+    int i = 0;
+#pragma unroll
+    for (int j = 1; j < 3; j++)
+        if (g >= b.it[j].first_group) i = j;
+    const gemv_item &m = b.it[i];
+    const int group = g - m.first_group;
+    switch (m.type) {   // uniform over the group
+        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
+        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
+        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
+        default: gemv_body<MI355_Q6_K, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
     }
 }
 
@@ -289,6 +364,8 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
         b.it[i].dst_stride = src.dst_stride;
         b.it[i].type = src.type;
         b.it[i].first_group = (int)groups;
+        b.it[i].epi = EPI_STORE;
+        b.it[i].nb1 = b.it[i].nb2 = 0;
         if (i < n_mats) groups += (src.N + 4 * rpw - 1) / (4 * rpw);
     }
     MI355_REQUIRE(groups < 0x7fffffff, "mul_mat_vec_q: too many rows for one launch");
@@ -319,6 +396,63 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
             return MI355_OK;
     }
     return launch_status("k_gemv_multi");
+}
+
+int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, const void *wk, int type_v, const void *wv, const void *act,
+                         float *q, void *kcache, void *vcache, const int32_t *pos, const int32_t *cells, const float *freq_factors,
+                         int64_t K, int64_t B, int64_t H, int64_t HK, int64_t D, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2,
+                         int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
+                         float beta_fast, float beta_slow) {
+    MI355_REQUIRE(B >= 1 && B <= 4, "qkv_rope_store: batch %lld outside 1..4", (long long)B);
+    MI355_REQUIRE(H > 0 && HK > 0 && D > 0 && D % 2 == 0 && n_dims > 0 && n_dims <= D && n_dims % 2 == 0, "qkv_rope_store: bad head geometry");
+    MI355_REQUIRE(mode == 0, "qkv_rope_store: only the adjacent-pair rope mode is fused (mode %d)", mode);
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0 && ((uintptr_t)kcache & 1) == 0 && ((uintptr_t)vcache & 1) == 0 && k_nb1 % 2 == 0 && k_nb2 % 2 == 0 &&
+                  v_nb1 % 2 == 0 && v_nb2 % 2 == 0, "qkv_rope_store: misaligned operands");
+    const int types[3] = {type_q, type_k, type_v};
+    const void *Ws[3] = {wq, wk, wv};
+    const int64_t Ns[3] = {H * D, HK * D, HK * D};
+    for (int i = 0; i < 3; i++) {
+        int rc = check_gemv_args("qkv_rope_store", types[i], Ws[i], Ns[i], K, Ns[i]);
+        if (rc != MI355_OK) return rc;
+    }
+    gemv_batch b;
+    b.n = 3;
+    int64_t groups = 0;
+    for (int i = 0; i < 4; i++) {
+        const int j = i < 3 ? i : 0;
+        b.it[i].W = (const uint8_t *)Ws[j];
+        b.it[i].residual = nullptr;
+        b.it[i].N = Ns[j];
+        b.it[i].type = types[j];
+        b.it[i].first_group = (int)groups;
+        if (i < 3) groups += (Ns[j] + 7) / 8;   // 4 waves x 2 rows
+    }
+    b.it[0].dst = q;               b.it[0].dst_stride = H * D; b.it[0].epi = EPI_ROPE;       b.it[0].nb1 = b.it[0].nb2 = 0;
+    b.it[1].dst = (float *)kcache; b.it[1].dst_stride = 0;     b.it[1].epi = EPI_ROPE_CACHE; b.it[1].nb1 = (int64_t)k_nb1; b.it[1].nb2 = (int64_t)k_nb2;
+    b.it[2].dst = (float *)vcache; b.it[2].dst_stride = 0;     b.it[2].epi = EPI_CACHE;      b.it[2].nb1 = (int64_t)v_nb1; b.it[2].nb2 = (int64_t)v_nb2;
+    b.it[3] = b.it[0];
+    b.it[3].first_group = 0x7fffffff;
+    MI355_REQUIRE(groups < 0x7fffffff, "qkv_rope_store: too many rows for one launch");
+    gemv_rope rp;
+    rp.pos = pos; rp.cells = cells; rp.ff = freq_factors;
+    rp.D = (int)D; rp.n_dims = n_dims;
+    rp.theta_scale = powf(freq_base, -2.0f / n_dims);
+    rp.freq_scale = freq_scale; rp.ext_factor = ext_factor; rp.attn_factor = attn_factor;
+    const float pi = 3.14159265358979323846f;   // ggml_rope_yarn_corr_dims, ggml/src/ggml.c:3695-3707
+    const float c0 = floorf(n_dims * logf(n_ctx_orig / (beta_fast * 2 * pi)) / (2 * logf(freq_base)));
+    const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
+    rp.corr0 = c0 > 0 ? c0 : 0;
+    rp.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
+    hipStream_t s = (hipStream_t)stream;
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + B * K);
+    switch (B) {
+        case 1: hipLaunchKernelGGL(k_gemv_qkv<1>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
+        case 2: hipLaunchKernelGGL(k_gemv_qkv<2>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
+        case 3: hipLaunchKernelGGL(k_gemv_qkv<3>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
+        default: hipLaunchKernelGGL(k_gemv_qkv<4>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
+    }
+    return launch_status("k_gemv_qkv");
 }
 
 // act: split layout of nb1*T quantized rows of b.  dst [N, n_used, T] contiguous.

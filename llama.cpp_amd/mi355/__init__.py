@@ -48,6 +48,8 @@ _SIGNATURES = {
     "mi355_swiglu_quant": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
     "mi355_rope_kv_store": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _int, _int, _int,
                                    _f, _f, _f, _f, _f, _f]),
+    "mi355_qkv_rope_store": (_int, [_p, _int, _p, _int, _p, _int, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64,
+                                    _sz, _sz, _sz, _sz, _int, _int, _int, _f, _f, _f, _f, _f, _f]),
     "mi355_block_dots_q8_1": (_int, [_p, _int, _p, _p, _p, _i64, _i64]),
     "mi355_mul_mat_id_ws_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_id": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
@@ -55,6 +57,8 @@ _SIGNATURES = {
     "mi355_flash_attn_ws_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "mi355_flash_attn_ext": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _sz, _sz,
                                     _sz, _f, _f, _f, _p, _sz]),
+    "mi355_flash_attn_ext_quant": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _sz, _sz,
+                                          _sz, _f, _f, _f, _p, _sz, _p]),
     "mi355_rms_norm": (_int, [_p, C.POINTER(Tensor), C.POINTER(Tensor), _f]),
     "mi355_bin_bcast": (_int, [_p, _int, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]),
     "mi355_unary": (_int, [_p, _int, C.POINTER(Tensor), C.POINTER(Tensor)]),
@@ -221,8 +225,9 @@ def mul_mat_id(t, as_dev, b, ids, n_used):
     return dst
 
 
-def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, softcap=0.0):
-    """q f32 [Hq, Nq, D] (any head/row strides), k,v f16 [Hkv, Nkv, D], mask f16 [>=Nq, Nkv] or None -> f32 [Nq, Hq, D]"""
+def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, softcap=0.0, quantized=False):
+    """q f32 [Hq, Nq, D] (any head/row strides), k,v f16 [Hkv, Nkv, D], mask f16 [>=Nq, Nkv] or None -> f32 [Nq, Hq, D]
+    (quantized=True: also returns the Q8_1 activation workspace of the output rows)"""
     import torch
     Hq, Nq, D = q.shape
     Hkv, Nkv, _ = k.shape
@@ -230,8 +235,13 @@ def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, softcap=0.0):
     need = load().mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq)
     ws = torch.empty(min(need, 1 << 28), dtype=torch.uint8, device=q.device)
     dst = torch.empty((Nq, Hq, D), dtype=torch.float32, device=q.device)
-    check(load().mi355_flash_attn_ext(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(mask), _ptr(dst), D, Nq, Nkv, Hq, Hkv,
-                                      q.stride(1) * 4, q.stride(0) * 4, k.stride(1) * 2, k.stride(0) * 2,
-                                      v.stride(1) * 2, v.stride(0) * 2, mask.stride(0) * 2 if mask is not None else 0,
-                                      scale, max_bias, softcap, _ptr(ws), ws.numel()))
+    args = (_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(mask), _ptr(dst), D, Nq, Nkv, Hq, Hkv,
+            q.stride(1) * 4, q.stride(0) * 4, k.stride(1) * 2, k.stride(0) * 2,
+            v.stride(1) * 2, v.stride(0) * 2, mask.stride(0) * 2 if mask is not None else 0,
+            scale, max_bias, softcap, _ptr(ws), ws.numel())
+    if quantized:
+        act = torch.empty(load().mi355_act_bytes(Hq * D, Nq), dtype=torch.uint8, device=q.device)
+        check(load().mi355_flash_attn_ext_quant(*args, _ptr(act)))
+        return dst, act
+    check(load().mi355_flash_attn_ext(*args))
     return dst

@@ -96,6 +96,7 @@ class LlamaRunner:
         cfg = self.cfg = weights.cfg
         dev = self.dev = weights.output[1].device
         self.lib = load()
+        self.fuse_qkv = True    # rows must be 16-byte aligned; set False to use the three-launch sequence
         E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
         T = self.max_tokens = max_tokens
         f32 = dict(dtype=torch.float32, device=dev)
@@ -147,15 +148,16 @@ class LlamaRunner:
         d = tensor_desc(cache.view(cfg.n_ctx, cfg.n_head_kv * cfg.head_dim))
         check(self.lib.mi355_set_rows(_stream(), C.byref(s), _ptr(self.pos), C.byref(d)))
 
-    def _attn(self, il, T, n_kv):
+    def _attn(self, il, T, n_kv, act=None):
+        """act: optional workspace that receives the Q8_1 quantization of the attention output"""
         cfg = self.cfg
         H, HK, D = cfg.n_head, cfg.n_head_kv, cfg.head_dim
         q = self.q[:T].view(T, H, D)
         kc, vc = self.kcache[il], self.vcache[il]
-        check(self.lib.mi355_flash_attn_ext(_stream(), _ptr(q), _ptr(kc), _ptr(vc), _ptr(self.mask), _ptr(self.attn), D, T, n_kv, H, HK,
-                                            q.stride(0) * 4, q.stride(1) * 4, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2,
-                                            vc.stride(1) * 2, self.mask.stride(0) * 2, 1.0 / math.sqrt(D), 0.0, 0.0, _ptr(self.fa_ws),
-                                            self.fa_ws.numel()))
+        check(self.lib.mi355_flash_attn_ext_quant(_stream(), _ptr(q), _ptr(kc), _ptr(vc), _ptr(self.mask), _ptr(self.attn), D, T, n_kv, H, HK,
+                                                  q.stride(0) * 4, q.stride(1) * 4, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2,
+                                                  vc.stride(1) * 2, self.mask.stride(0) * 2, 1.0 / math.sqrt(D), 0.0, 0.0, _ptr(self.fa_ws),
+                                                  self.fa_ws.numel(), _ptr(act) if act is not None else None))
 
     # ---- fused operators ------------------------------------------------------------------------
     @staticmethod
@@ -201,15 +203,24 @@ class LlamaRunner:
             qkv = [(L["wq"], self.q[:T]), (L["wk"], self.k[:T]), (L["wv"], self.v[:T])]
             kq = big and self._q8k_ok(qkv, E)
             self._norm_quant(x, L["attn_norm"], self.act_a, T, kq)
-            self._mm_act(qkv, self.act_a, E, T, q8k=kq)
             kc, vc = self.kcache[il], self.vcache[il]
-            check(lib.mi355_rope_kv_store(_stream(), _ptr(self.q), _ptr(self.k), _ptr(self.v), _ptr(kc), _ptr(vc), _ptr(self.pos), _ptr(self.pos),
-                                          None, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2, vc.stride(1) * 2, D, 0,
-                                          cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
-            self._attn(il, T, n_kv)
+            if T <= 4 and self.fuse_qkv:    # decode: projections, rope and KV store in one launch
+                (tq, Wq), (tk, Wk), (tv, Wv) = L["wq"], L["wk"], L["wv"]
+                check(lib.mi355_qkv_rope_store(_stream(), tq, _ptr(Wq), tk, _ptr(Wk), tv, _ptr(Wv), _ptr(self.act_a), _ptr(self.q), _ptr(kc), _ptr(vc),
+                                               _ptr(self.pos), _ptr(self.pos), None, E, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2,
+                                               vc.stride(0) * 2, vc.stride(1) * 2, D, 0, cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
+            else:
+                self._mm_act(qkv, self.act_a, E, T, q8k=kq)
+                check(lib.mi355_rope_kv_store(_stream(), _ptr(self.q), _ptr(self.k), _ptr(self.v), _ptr(kc), _ptr(vc), _ptr(self.pos), _ptr(self.pos),
+                                              None, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2, vc.stride(1) * 2, D, 0,
+                                              cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
             wo = [(L["wo"], x)]
             kq = big and self._q8k_ok(wo, H * D)
-            self._quant(self.attn, self.act_a, H * D, T, kq)
+            if kq:
+                self._attn(il, T, n_kv)
+                self._quant(self.attn, self.act_a, H * D, T, True)
+            else:
+                self._attn(il, T, n_kv, act=self.act_a)   # attention writes its own Q8_1 output
             self._mm_act(wo, self.act_a, H * D, T, residual=x, q8k=kq)
             gu = [(L["gate"], self.gate[:T]), (L["up"], self.up[:T])]
             kq = big and self._q8k_ok(gu, E)

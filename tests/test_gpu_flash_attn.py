@@ -91,3 +91,18 @@ def test_llama3_shapes(dev, Nq, Nkv):
         ms = np.concatenate([ms, np.full((64 - len(rows), Nkv), -np.inf, dtype=np.float16)])
         f64 = orc.flash_attn("f64", qs, k[h // 4:h // 4 + 1].view(np.uint16), v[h // 4:h // 4 + 1].view(np.uint16), ms.view(np.uint16), scale)
         assert orc.nmse(got[rows][:, h:h + 1], f64) < 1e-5
+
+
+@pytest.mark.parametrize("D,Nq,Nkv,Hq,Hkv", [(128, 1, 256, 32, 8), (128, 1, 4096, 32, 8), (128, 5, 700, 8, 2), (64, 2, 96, 6, 3), (96, 1, 64, 4, 4)])
+def test_quantized_output_matches_separate_quantization(dev, D, Nq, Nkv, Hq, Hkv):
+    """the Q8_1 rows attention emits equal mi355_quantize_act of its own f32 output, bit for bit (kv split or not)"""
+    import torch
+    import mi355
+    rng = np.random.default_rng(D + Nq + Nkv)
+    q, k, v, mask = _inputs(rng, D, Nq, Nkv, Hq, Hkv)
+    qd, kd, vd, md = (torch.from_numpy(a).to(dev) for a in (q, k, v, mask))
+    dst, act = mi355.flash_attn_ext(qd, kd, vd, md, 1.0 / np.sqrt(D), quantized=True)
+    plain = mi355.flash_attn_ext(qd, kd, vd, md, 1.0 / np.sqrt(D))
+    assert torch.equal(dst, plain)
+    want = mi355.quantize_act(dst.reshape(Nq, Hq * D))
+    assert torch.equal(act, want)

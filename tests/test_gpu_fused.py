@@ -143,3 +143,50 @@ def test_fused_layer_stack_matches_node_sequence(dev):
         # last bit, which flips a few activation levels; with one scale per 256 elements a single flip in a
         # row that holds an outlier moves that row by ~1e-5, and two random-weight layers amplify it.
         assert orc.nmse(b, a) < (5e-4 if T > 8 else 1e-6), (T, pos0)
+
+
+@pytest.mark.parametrize("B", [1, 3])
+@pytest.mark.parametrize("tq,tk,tv", [(orc.Q4_K, orc.Q4_K, orc.Q6_K), (orc.Q4_0, orc.Q8_0, orc.Q4_0)])
+def test_qkv_rope_store_equals_three_launch_sequence(dev, B, tq, tk, tv):
+    """projections + rope + KV store in one launch give bit-identical q and cache contents"""
+    import torch
+    import mi355
+    lib = mi355.load()
+    rng = np.random.default_rng(B + tq)
+    K, H, HK, D, n_ctx = 2048, 8, 2, 128, 64
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    act = mi355.quantize_act(_t(dev, x))
+    Ws = []
+    for t, N in ((tq, H * D), (tk, HK * D), (tv, HK * D)):
+        Wq = orc.quantize("oracle", t, (rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+        Ws.append(mi355.upload_weights(t, _t(dev, Wq)))
+    pos = _t(dev, np.array([5, 17, 40][:B], dtype=np.int32))
+    cells = _t(dev, np.array([9, 3, 33][:B], dtype=np.int32))
+    rope = (D, 0, 4096, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+
+    def caches():
+        return (torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev), torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev))
+
+    # reference sequence: multi-matrix GEMV, then the rope + store kernel
+    q0 = torch.zeros(B, H * D, device=dev)
+    k0 = torch.zeros(B, HK * D, device=dev)
+    v0 = torch.zeros(B, HK * D, device=dev)
+    arr = (mi355.GemvMat * 3)()
+    for i, (t, W, out) in enumerate(((tq, Ws[0], q0), (tk, Ws[1], k0), (tv, Ws[2], v0))):
+        arr[i].type, arr[i].W, arr[i].N, arr[i].dst, arr[i].dst_stride, arr[i].residual = t, W.data_ptr(), out.shape[1], out.data_ptr(), out.shape[1], None
+    mi355.check(lib.mi355_mul_mat_vec_q_multi(None, 3, arr, act.data_ptr(), K, B))
+    kc0, vc0 = caches()
+    mi355.check(lib.mi355_rope_kv_store(None, q0.data_ptr(), k0.data_ptr(), v0.data_ptr(), kc0.data_ptr(), vc0.data_ptr(), pos.data_ptr(),
+                                        cells.data_ptr(), None, B, H, HK, D, kc0.stride(0) * 2, kc0.stride(1) * 2, vc0.stride(0) * 2,
+                                        vc0.stride(1) * 2, *rope))
+    # fused launch
+    q1 = torch.zeros(B, H * D, device=dev)
+    kc1, vc1 = caches()
+    mi355.check(lib.mi355_qkv_rope_store(None, tq, Ws[0].data_ptr(), tk, Ws[1].data_ptr(), tv, Ws[2].data_ptr(), act.data_ptr(), q1.data_ptr(),
+                                         kc1.data_ptr(), vc1.data_ptr(), pos.data_ptr(), cells.data_ptr(), None, K, B, H, HK, D,
+                                         kc1.stride(0) * 2, kc1.stride(1) * 2, vc1.stride(0) * 2, vc1.stride(1) * 2, *rope))
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q0)
+    assert torch.equal(kc1, kc0)
+    assert torch.equal(vc1, vc0)
+    assert kc1.abs().sum().item() > 0 and vc1.abs().sum().item() > 0
