@@ -10,6 +10,7 @@
 // (running max, sum, R x 8 output slice); the states are merged through LDS, and across kv
 // splits by k_fattn_combine.  -inf mask entries are skipped, as in the reference.
 #include "common.hpp"
+#include "fattn.hpp"
 
 #include <float.h>
 
@@ -43,21 +44,6 @@ __device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
 
 __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e);
 
-struct fattn_args {
-    const uint8_t *q, *k, *v, *mask;
-    float *dst;      // [D, Hq, Nq]
-    int8_t *act_q;   // optional: Q8_1 of dst rows (Hq*D elements per query) in the split activation layout
-    act_ds *act_s;
-    float *ws;       // partial results when n_splits > 1: [Nq][Hq][n_splits][D + 2]
-    int64_t Nq, Nkv, Hq, Hkv;
-    size_t q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1;
-    float scale, max_bias, softcap;
-    float m0, m1;
-    unsigned n_head_log2;
-    int n_splits;
-    int groups;      // head groups of R per kv head: Hq / Hkv == R * groups
-    int64_t cells_per_split;
-};
 
 template <int D, int R>
 __global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
@@ -200,20 +186,46 @@ __global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
     }
 }
 
+// Merge of the kv splits: threads first turn the per-split (max, sum) pairs into weights in LDS
+// (one split per thread), then every thread owns one output element and sums the partial
+// outputs with independent, coalesced loads.
 template <int D>
-__global__ void k_fattn_combine(const float *__restrict__ ws, float *__restrict__ dst, int n_splits, int8_t *__restrict__ act_q,
-                                act_ds *__restrict__ act_s, int64_t Hq) {
+__global__ void __launch_bounds__(256) k_fattn_combine(const float *__restrict__ ws, float *__restrict__ dst, int n_splits, int8_t *__restrict__ act_q,
+                                                       act_ds *__restrict__ act_s, int64_t Hq) {
+    __shared__ float s_w[256];
+    __shared__ float s_red[8];
     const int64_t row = blockIdx.x;   // iq * Hq + head
     const float *p = ws + row * n_splits * (D + 2);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float M = -FLT_MAX / 2;
-        for (int s = 0; s < n_splits; s++) M = fmaxf(M, p[s * (D + 2) + D]);
-        float L = 0.0f, O = 0.0f;
-        for (int s = 0; s < n_splits; s++) {
-            const float f = __expf(p[s * (D + 2) + D] - M);
-            L += p[s * (D + 2) + D + 1] * f;
-            O += p[s * (D + 2) + d] * f;
+    const int tid = threadIdx.x;
+    const int nw = blockDim.x >> 6;
+    float ms = -FLT_MAX / 2, ls = 0.0f;
+    if (tid < n_splits) {
+        ms = p[tid * (D + 2) + D];
+        ls = p[tid * (D + 2) + D + 1];
+    }
+    float M = wave_max(ms);
+    if ((tid & 63) == 0) s_red[tid >> 6] = M;
+    __syncthreads();
+    M = s_red[0];
+    for (int i = 1; i < nw; i++) M = fmaxf(M, s_red[i]);
+    const float w = tid < n_splits ? __expf(ms - M) : 0.0f;
+    s_w[tid] = w;
+    float L = wave_sum(ls * w);
+    if ((tid & 63) == 0) s_red[4 + (tid >> 6)] = L;
+    __syncthreads();
+    L = s_red[4];
+    for (int i = 1; i < nw; i++) L += s_red[4 + i];
+    for (int d = tid; d < D; d += blockDim.x) {
+        float O = 0.0f;
+        int s = 0;
+        for (; s + 8 <= n_splits; s += 8) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = p[(s + i) * (D + 2) + d];
+#pragma unroll
+            for (int i = 0; i < 8; i++) O += v[i] * s_w[s + i];
         }
+        for (; s < n_splits; s++) O += p[s * (D + 2) + d] * s_w[s];
         const float o = O / L;
         dst[row * D + d] = o;
         if (act_q) {
@@ -261,7 +273,7 @@ static int launch_vec(hipStream_t s, fattn_args &a) {
     int rc = launch_status("k_fattn_vec");
     if (rc != MI355_OK) return rc;
     if (a.n_splits > 1) {
-        hipLaunchKernelGGL(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(D <= 128 ? 128 : 256), 0, s, a.ws, a.dst, a.n_splits, a.act_q,
+        hipLaunchKernelGGL(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(256), 0, s, a.ws, a.dst, a.n_splits, a.act_q,
                            a.act_s, a.Hq);
         rc = launch_status("k_fattn_combine");
     }
@@ -322,6 +334,39 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
     a.cells_per_split = (Nkv + a.n_splits - 1) / a.n_splits;
     const int R = (int)(Hq / Hkv);
     hipStream_t s = (hipStream_t)stream;
+    if (Nq >= 16 && act == nullptr) {   // prefill: f16 matrix cores
+        const int rc = launch_fattn_mma(s, a, D);
+        if (rc <= 0) return rc;
+    }
+    // Decode and small batches over a long context: matrix cores with (token, head) columns, which read a kv head's
+    // bytes once for its whole GQA group.  Short contexts are latency-bound and mostly padding (-inf mask): the
+    // vector kernel, which skips masked cells before touching K/V, is quicker there.
+    if (Nq < 16 && Nkv > 256 && (D == 64 || D == 128) && R <= 32) {
+        fattn_args b = a;
+        // enough splits to put about two groups on every CU; a split is a whole number of 64-cell tiles
+        const int64_t tiles = (Nkv + 63) / 64;
+        const int64_t nt = 32 / R, base = Hkv * ((Nq + nt - 1) / nt);
+        int64_t n = 512 / base;
+        if (n > tiles) n = tiles;
+        if (n > 256) n = 256;
+        if (n < 1) n = 1;
+        if (n > 1 && (ws == nullptr || ws_bytes < (size_t)Nq * (size_t)Hq * (size_t)n * (size_t)(D + 2) * sizeof(float))) n = 1;
+        const int64_t tiles_per_split = (tiles + n - 1) / n;
+        b.cells_per_split = tiles_per_split * 64;
+        b.n_splits = (int)((tiles + tiles_per_split - 1) / tiles_per_split);
+        int rc = launch_fattn_mma_dec(s, b, D);
+        if (rc < 0) return rc;
+        if (rc == 0) {
+            if (b.n_splits > 1) {
+                switch (D) {
+                    case 64: hipLaunchKernelGGL(k_fattn_combine<64>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
+                    default: hipLaunchKernelGGL(k_fattn_combine<128>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
+                }
+                return launch_status("k_fattn_combine");
+            }
+            return MI355_OK;
+        }
+    }
     switch (D) {
         case 64: return launch_vec_r<64>(s, a, R);
         case 80: return launch_vec_r<80>(s, a, R);

@@ -1,0 +1,29 @@
+// Arguments shared by the flash-attention kernels (vector kernel for decode, matrix-core kernel for prefill).
+#pragma once
+
+#include "common.hpp"
+
+namespace mi355 {
+
+struct fattn_args {
+    const uint8_t *q, *k, *v, *mask;
+    float *dst;      // [D, Hq, Nq]
+    int8_t *act_q;   // optional: Q8_1 of dst rows (Hq*D elements per query) in the split activation layout
+    act_ds *act_s;
+    float *ws;       // partial results when n_splits > 1: [Nq][Hq][n_splits][D + 2]
+    int64_t Nq, Nkv, Hq, Hkv;
+    size_t q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1;
+    float scale, max_bias, softcap;
+    float m0, m1;
+    unsigned n_head_log2;
+    int n_splits;
+    int groups;      // head groups of R per kv head: Hq / Hkv == R * groups
+    int64_t cells_per_split;
+};
+
+// f16 matrix-core kernel for many query rows; returns MI355_OK, an error, or 1 when the shape is not served
+int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D);
+// the same for a few query rows (decode): one kv split per group, partials merged by k_fattn_combine
+int launch_fattn_mma_dec(hipStream_t s, fattn_args &a, int64_t D);
+
+}  // namespace mi355

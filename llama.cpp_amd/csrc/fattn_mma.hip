@@ -1,0 +1,516 @@
+// FLASH_ATTN_EXT for many query rows (prefill) on the f16 matrix cores.
+// Semantics: ggml_compute_forward_flash_attn_ext_f16, ggml/src/ggml-cpu/ggml-cpu.c:10916-11129
+// (q rounded to f16, scores scale * q.k [+ softcap] + slope * mask, online softmax in f32,
+// -inf mask entries contribute nothing, GQA by head index division).
+//
+// A 256-thread group serves one kv head: its 4 waves are HPW query heads of that kv head times
+// 4 / HPW tiles of 32 queries, so every K/V tile staged in LDS is used by all four waves.
+// Per wave and 64-cell kv tile, with v_mfma_f32_32x32x16_f16 (D[i][j], lane l supplies row /
+// column l % 32 and k slots [8*(l/32), +8); D register r is i = 8*(r/4) + 4*(l/32) + r%4, j = l%32):
+//   S^T = K Q^T   A = K rows (i = kv cell), B = Q rows (j = query)  -> a lane holds ONE query's
+//                 scores for 16 cells, so softmax row reductions are in-lane plus one xor-32 step
+//   O^T += V^T P^T  A = V^T rows (i = head dim), B = P^T (j = query) -> the B operand is the lane's
+//                 own score registers 8t..8t+7 rounded to f16: no cross-lane data movement.  The
+//                 kv cells those registers stand for, 16t + 8*(s/4) + 4*(l/32) + s%4, fix which
+//                 cells the A operand must supply in k slot s: two 8-byte reads of a V tile that
+//                 was transposed on its way into LDS.
+// Rescaling by exp(m_old - m_new) is one multiply per accumulator register because both
+// accumulators are indexed by query along the lanes.
+#include "fattn.hpp"
+
+#include <float.h>
+
+namespace mi355 {
+
+namespace {
+
+constexpr int FM_BC = 64;            // kv cells per tile
+constexpr float FM_NEG = -FLT_MAX / 2;
+
+// ---- staging of one 64-cell K tile and the matching V tile (transposed) through registers ----
+template <int D, int NTH> struct kv_stage {
+    static constexpr int KP = D + 8;        // f16 pitch of a K row in LDS (16 bytes of padding spread the banks)
+    static constexpr int VP = FM_BC + 4;    // f16 pitch of a V^T row in LDS (keeps 8-byte alignment)
+    static constexpr int KCH = D / 8;       // 16-byte chunks per K/V row
+    static constexpr int KIT = FM_BC * KCH / NTH;         // K chunks per thread per tile
+    static constexpr int VIT = (FM_BC / 2) * KCH / NTH;   // V (cell pair, chunk) units per thread per tile
+    static_assert(D % 32 == 0 && KIT >= 1 && VIT >= 1, "head size not served by this kernel");
+    u32x4 k[KIT], v0[VIT], v1[VIT];
+
+    __device__ __forceinline__ void fetch(const fattn_args &a, int64_t hk, int64_t kv0, int tid) {
+        const int64_t last = a.Nkv - 1;
+#pragma unroll
+        for (int it = 0; it < KIT; it++) {
+            const int unit = tid + it * NTH;
+            const int row = unit / KCH, ch = unit % KCH;
+            const int64_t c = kv0 + row < last ? kv0 + row : last;   // rows past the end repeat the last cell; their scores are dropped
+            k[it] = load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + ch * 16);
+        }
+#pragma unroll
+        for (int it = 0; it < VIT; it++) {
+            const int unit = tid + it * NTH;
+            const int kp = unit & 31, ch = unit >> 5;
+            const int64_t c0 = kv0 + 2 * kp < last ? kv0 + 2 * kp : last;
+            const int64_t c1 = kv0 + 2 * kp + 1 < last ? kv0 + 2 * kp + 1 : last;
+            v0[it] = load16(a.v + c0 * a.v_nb1 + hk * a.v_nb2 + ch * 16);
+            v1[it] = load16(a.v + c1 * a.v_nb1 + hk * a.v_nb2 + ch * 16);
+        }
+    }
+    __device__ __forceinline__ void commit(_Float16 *sK, _Float16 *sVt, int tid) const {
+#pragma unroll
+        for (int it = 0; it < KIT; it++) {
+            const int unit = tid + it * NTH;
+            const int row = unit / KCH, ch = unit % KCH;
+            *(u32x4 *)(sK + row * KP + ch * 8) = k[it];
+        }
+#pragma unroll
+        for (int it = 0; it < VIT; it++) {
+            const int unit = tid + it * NTH;
+            const int kp = unit & 31, ch = unit >> 5;
+            // element e of both cells -> one dword of row (8*ch + e) of V^T, columns 2*kp and 2*kp+1
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 x = v0[it][i], y = v1[it][i];
+                *(u32 *)(sVt + (8 * ch + 2 * i) * VP + 2 * kp) = (x & 0xFFFFu) | (y << 16);
+                *(u32 *)(sVt + (8 * ch + 2 * i + 1) * VP + 2 * kp) = (x >> 16) | (y & 0xFFFF0000u);
+            }
+        }
+    }
+};
+
+// f16 bits of the mask entries of NG groups of 4 consecutive cells, first cell c0 + 8*g.  Loads are
+// unconditional (clamped), so they can be issued with the K/V prefetch and never force a wait.
+template <int NG>
+__device__ __forceinline__ void fetch_mask(u32x2 (&out)[NG], const unsigned short *mrow, bool vec_ok, int64_t c0, int64_t Nkv) {
+    if (mrow == nullptr) {
+#pragma unroll
+        for (int g = 0; g < NG; g++) out[g] = u32x2{0, 0};
+    } else if (vec_ok) {   // uniform: aligned rows and a full tile
+#pragma unroll
+        for (int g = 0; g < NG; g++) out[g] = *(const u32x2 *)(mrow + c0 + 8 * g);
+    } else {
+        const int64_t last = Nkv - 1;
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            u32 h[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int64_t c = c0 + 8 * g + i;
+                h[i] = mrow[c < last ? c : last];
+            }
+            out[g] = u32x2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
+    }
+}
+__device__ __forceinline__ float mask_value(const u32x2 &w, int i) {
+    return half_bits_to_float((unsigned short)((i < 2 ? w[0] : w[1]) >> (16 * (i & 1))));
+}
+
+// scale [+ softcap], add the mask, mark dropped cells with FM_NEG; returns the largest surviving score
+__device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], const fattn_args &a, float scale, float slope,
+                                                int64_t c_first, int lhi, int64_t c_end) {
+    if (a.softcap != 0.0f) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) S[r] = a.softcap * tanhf(S[r] * scale);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) S[r] *= scale;
+    }
+    float mx = FM_NEG;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const int64_t c = c_first + 8 * g + 4 * lhi;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float mv = mask_value(mw[g], i);
+            float s = S[4 * g + i] + slope * mv;
+            const bool valid = c + i < c_end && mv != -INFINITY && s > FM_NEG;   // NaN scores of stale cells drop out too
+            s = valid ? s : FM_NEG;
+            S[4 * g + i] = s;
+            mx = fmaxf(mx, s);
+        }
+    }
+    return mx;
+}
+
+template <int D>
+__device__ __forceinline__ void load_q(f16x8 (&qf)[D / 16], const float *qp, int lhi) {
+#pragma unroll
+    for (int kk = 0; kk < D / 16; kk++) {   // rounded to f16 (ggml-cpu.c:11037-11040)
+        const f32x4 x0 = *(const f32x4 *)(qp + 16 * kk + 8 * lhi);
+        const f32x4 x1 = *(const f32x4 *)(qp + 16 * kk + 8 * lhi + 4);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            qf[kk][i] = (_Float16)x0[i];
+            qf[kk][4 + i] = (_Float16)x1[i];
+        }
+    }
+}
+__device__ __forceinline__ float alibi_slope(const fattn_args &a, int64_t head) {   // ggml-cpu.c:10998-11003
+    if (a.max_bias <= 0.0f) return 1.0f;
+    const unsigned h = (unsigned)head;
+    return h < a.n_head_log2 ? powf(a.m0, (float)(h + 1)) : powf(a.m1, (float)(2 * (h - a.n_head_log2) + 1));
+}
+
+// O^T tiles [DT0, DT0 + NDT) += V^T P^T for the 32 cells of half u whose probabilities sit in S
+template <int D, int NDT>
+__device__ __forceinline__ void accumulate_pv(f32x16 (&o)[NDT], const f32x16 &S, const _Float16 *sVt, int dt0, int u, int l32, int lhi) {
+    constexpr int VP = FM_BC + 4;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        f16x8 pf;
+#pragma unroll
+        for (int i = 0; i < 8; i++) pf[i] = (_Float16)S[8 * t + i];
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) {
+            const _Float16 *vp = sVt + (32 * (dt0 + dt) + l32) * VP + 32 * u + 16 * t + 4 * lhi;
+            const f16x4 v0 = *(const f16x4 *)vp;
+            const f16x4 v1 = *(const f16x4 *)(vp + 8);
+            f16x8 vf;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                vf[i] = v0[i];
+                vf[4 + i] = v1[i];
+            }
+            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, o[dt], 0, 0, 0);
+        }
+    }
+}
+
+template <int D>
+__device__ __forceinline__ f32x16 scores(const f16x8 (&qf)[D / 16], const _Float16 *sK, int u, int l32, int lhi) {
+    constexpr int KP = D + 8;
+    f32x16 S;
+#pragma unroll
+    for (int r = 0; r < 16; r++) S[r] = 0.0f;
+#pragma unroll
+    for (int kk = 0; kk < D / 16; kk++) {
+        const f16x8 kf = *(const f16x8 *)(sK + (32 * u + l32) * KP + 16 * kk + 8 * lhi);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[kk], S, 0, 0, 0);
+    }
+    return S;
+}
+
+// ---- prefill --------------------------------------------------------------------------------
+template <int D, int HPW>
+__global__ void __launch_bounds__(256) k_fattn_mma(fattn_args a) {
+    typedef kv_stage<D, 256> stage_t;
+    constexpr int QTW = 4 / HPW;   // query tiles per group
+    __shared__ __attribute__((aligned(16))) _Float16 sK[FM_BC * stage_t::KP];
+    __shared__ __attribute__((aligned(16))) _Float16 sVt[D * stage_t::VP];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int groups = (int)(a.Hq / a.Hkv) / HPW;
+    const int64_t hk = blockIdx.y / groups, hg = blockIdx.y % groups;
+    const int64_t head = (hk * groups + hg) * HPW + (wave % HPW);
+    const int64_t q0 = ((int64_t)blockIdx.x * QTW + wave / HPW) * 32;
+    const int64_t iq = q0 + l32 < a.Nq ? q0 + l32 : a.Nq - 1;   // clamped: rows past Nq are computed and dropped
+
+    f16x8 qf[D / 16];
+    load_q<D>(qf, (const float *)(a.q + iq * a.q_nb1 + head * a.q_nb2), lhi);
+    const float slope = alibi_slope(a, head);
+    const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
+    const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
+    const bool mask_aligned = (((uintptr_t)a.mask | a.mask_nb1) & 7) == 0;
+
+    f32x16 o[D / 32];
+#pragma unroll
+    for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+    float m = FM_NEG, l = 0.0f;
+
+    stage_t st;
+    u32x2 mnext[2][4];
+    auto prefetch = [&](int64_t kv0) {
+        st.fetch(a, hk, kv0, tid);
+        const bool vec_ok = mask_aligned && kv0 + FM_BC <= a.Nkv;
+        fetch_mask<4>(mnext[0], mrow, vec_ok, kv0 + 4 * lhi, a.Nkv);
+        fetch_mask<4>(mnext[1], mrow, vec_ok, kv0 + 32 + 4 * lhi, a.Nkv);
+    };
+    prefetch(0);
+    for (int64_t kv0 = 0; kv0 < a.Nkv; kv0 += FM_BC) {
+        __syncthreads();   // the previous tile has been consumed
+        st.commit(sK, sVt, tid);
+        u32x2 mcur[2][4];
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) mcur[u][g] = mnext[u][g];
+        __syncthreads();
+        if (kv0 + FM_BC < a.Nkv) prefetch(kv0 + FM_BC);
+
+        // scores of 64 cells for this lane's query: S[u][r] <-> cell kv0 + 32u + 8*(r/4) + 4*lhi + r%4
+        f32x16 S[2];
+        float mx = FM_NEG;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            S[u] = scores<D>(qf, sK, u, l32, lhi);
+            mx = fmaxf(mx, finish_scores(S[u], mcur[u], a, scale, slope, kv0 + 32 * u, lhi, a.Nkv));
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (__ballot(mx > FM_NEG) == 0) continue;   // every cell of the tile is masked for all 32 queries (wave-uniform)
+        const float m_new = fmaxf(m, mx);
+        const float alpha = __expf(m - m_new);
+        float rs = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float p = S[u][r] > FM_NEG ? __expf(S[u][r] - m_new) : 0.0f;
+                S[u][r] = p;
+                rs += p;
+            }
+        rs += __shfl_xor(rs, 32, 64);
+        l = l * alpha + rs;
+        m = m_new;
+        if (__ballot(alpha != 1.0f) != 0) {   // wave-uniform
+#pragma unroll
+            for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) accumulate_pv<D, D / 32>(o, S[u], sVt, 0, u, l32, lhi);
+    }
+
+    if (q0 + l32 < a.Nq) {
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        float *dp = a.dst + ((q0 + l32) * a.Hq + head) * D;
+#pragma unroll
+        for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                f32x4 w;
+#pragma unroll
+                for (int i = 0; i < 4; i++) w[i] = o[dt][4 * g + i] * inv;
+                *(f32x4 *)(dp + 32 * dt + 8 * g + 4 * lhi) = w;
+            }
+    }
+}
+
+template <int D, int HPW>
+int launch(hipStream_t s, const fattn_args &a) {
+    constexpr int QTW = 4 / HPW;
+    const int64_t groups = (a.Hq / a.Hkv) / HPW;
+    const dim3 grid((unsigned)((a.Nq + 32 * QTW - 1) / (32 * QTW)), (unsigned)(a.Hkv * groups));
+    hipLaunchKernelGGL((k_fattn_mma<D, HPW>), grid, dim3(256), 0, s, a);
+    return launch_status("k_fattn_mma");
+}
+
+template <int D>
+int launch_hpw(hipStream_t s, const fattn_args &a) {
+    const int64_t R = a.Hq / a.Hkv;
+    if (R % 4 == 0) return launch<D, 4>(s, a);
+    if (R % 2 == 0) return launch<D, 2>(s, a);
+    return launch<D, 1>(s, a);
+}
+
+// ---- decode / small batches: the 32 MFMA columns are (token, head of the GQA group) pairs -------
+// A 256-thread group owns one kv head, NT = 32 / R tokens and one kv split, so the K/V bytes of
+// a kv head are read once for all R query heads.  Its four waves are (u, h): u picks the 32-cell
+// half of each 64-cell tile the wave scores, h the half of the head dimension it accumulates.
+// States are merged through LDS; a split writes (O, max, sum) partials for k_fattn_combine.
+template <int D>
+__global__ void __launch_bounds__(256, 2) k_fattn_mma_dec(fattn_args a, int R, int NT) {
+    typedef kv_stage<D, 256> stage_t;
+    constexpr int NDT = D / 64;   // 32-row O^T tiles per wave
+    __shared__ __attribute__((aligned(16))) _Float16 sK[FM_BC * stage_t::KP];
+    __shared__ __attribute__((aligned(16))) _Float16 sVt[D * stage_t::VP];
+    float *s_merge = (float *)sK;   // reused after the last tile: per h, [D/2 + 2][32] floats of the u = 1 wave
+    static_assert(sizeof(_Float16) * FM_BC * stage_t::KP >= sizeof(float) * (D + 4) * 32, "merge buffer does not fit the K tile");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int u = wave & 1, h = wave >> 1;
+    const int split = blockIdx.x;
+    const int64_t hk = blockIdx.y;
+    const int col_tok = l32 / R, col_head = l32 % R;
+    const bool col_live = col_tok < NT && (int64_t)blockIdx.z * NT + col_tok < a.Nq;
+    const int64_t iq = col_live ? (int64_t)blockIdx.z * NT + col_tok : a.Nq - 1;
+    const int64_t head = hk * R + (col_live ? col_head : 0);
+
+    f16x8 qf[D / 16];
+    load_q<D>(qf, (const float *)(a.q + iq * a.q_nb1 + head * a.q_nb2), lhi);
+    const float slope = alibi_slope(a, head);
+    const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
+    const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
+    const bool mask_aligned = (((uintptr_t)a.mask | a.mask_nb1) & 7) == 0;
+
+    f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+    float m = FM_NEG, l = 0.0f;
+
+    const int64_t c_begin = (int64_t)split * a.cells_per_split;
+    const int64_t c_end = c_begin + a.cells_per_split < a.Nkv ? c_begin + a.cells_per_split : a.Nkv;
+
+    // two tiles of K/V (and their mask entries) are always in flight: tile i + 2 is requested as soon as the
+    // registers of tile i have been written to LDS
+    stage_t st0, st1;
+    u32x2 mn0[4], mn1[4];
+    auto prefetch = [&](stage_t &st, u32x2 (&mn)[4], int64_t kv0) {
+        st.fetch(a, hk, kv0, tid);
+        fetch_mask<4>(mn, mrow, mask_aligned && kv0 + FM_BC <= a.Nkv, kv0 + 32 * u + 4 * lhi, a.Nkv);
+    };
+    auto tile = [&](stage_t &st, u32x2 (&mn)[4], int64_t kv0) {
+        __syncthreads();   // the previous tile has been consumed
+        st.commit(sK, sVt, tid);
+        u32x2 mcur[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) mcur[g] = mn[g];
+        __syncthreads();
+        if (kv0 + 2 * FM_BC < c_end) prefetch(st, mn, kv0 + 2 * FM_BC);
+        f32x16 S = scores<D>(qf, sK, u, l32, lhi);
+        float mx = finish_scores(S, mcur, a, scale, slope, kv0 + 32 * u, lhi, c_end);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (__ballot(mx > FM_NEG) == 0) return;   // all 32 cells masked for every column (wave-uniform)
+        const float m_new = fmaxf(m, mx);
+        const float alpha = __expf(m - m_new);
+        float rs = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float p = S[r] > FM_NEG ? __expf(S[r] - m_new) : 0.0f;
+            S[r] = p;
+            rs += p;
+        }
+        rs += __shfl_xor(rs, 32, 64);
+        l = l * alpha + rs;
+        m = m_new;
+        if (__ballot(alpha != 1.0f) != 0) {   // wave-uniform: most tiles do not raise any column's maximum
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+        }
+        accumulate_pv<D, NDT>(o, S, sVt, h * NDT, u, l32, lhi);
+    };
+    if (c_begin < c_end) prefetch(st0, mn0, c_begin);
+    if (c_begin + FM_BC < c_end) prefetch(st1, mn1, c_begin + FM_BC);
+    for (int64_t kv0 = c_begin; kv0 < c_end; kv0 += 2 * FM_BC) {
+        tile(st0, mn0, kv0);
+        if (kv0 + FM_BC < c_end) tile(st1, mn1, kv0 + FM_BC);   // uniform over the group
+    }
+
+    // ---- merge the u = 1 wave into the u = 0 wave of the same h
+    float *mg = s_merge + h * (D / 2 + 2) * 32;   // [d_local][col], then max, sum
+    __syncthreads();
+    if (u == 1) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] = o[dt][r];
+        if (lhi == 0) {
+            mg[(D / 2) * 32 + l32] = m;
+            mg[(D / 2 + 1) * 32 + l32] = l;
+        }
+    }
+    __syncthreads();
+    if (u != 0 || !col_live) return;
+    {
+        const float m1 = mg[(D / 2) * 32 + l32], l1 = mg[(D / 2 + 1) * 32 + l32];
+        const float M = fmaxf(m, m1);
+        const float f0 = __expf(m - M), f1 = __expf(m1 - M);
+        l = l * f0 + l1 * f1;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * f0 + mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] * f1;
+        m = M;
+    }
+    const int d_first = h * (D / 2);   // this wave's slice of the head
+    if (a.n_splits == 1) {
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        float *dp = a.dst + (iq * a.Hq + head) * D + d_first;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) {
+            float w[16];
+            float amax = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                w[r] = o[dt][r] * inv;
+                amax = fmaxf(amax, fabsf(w[r]));
+            }
+#pragma unroll
+            for (int g = 0; g < 4; g++) *(f32x4 *)(dp + 32 * dt + 8 * g + 4 * lhi) = f32x4{w[4 * g], w[4 * g + 1], w[4 * g + 2], w[4 * g + 3]};
+            if (a.act_q) {   // Q8_1 of this 32-element block of the head (quantize_row_q8_1_ref, ggml-quants.c:220-253)
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                const float d = amax / 127.0f;
+                const float id = d != 0.0f ? 1.0f / d : 0.0f;
+                int sum = 0;
+                const int64_t e0 = head * D + d_first + 32 * dt;   // first element of the block inside the activation row
+                int8_t *qrow = a.act_q + iq * a.Hq * D + e0;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    u32 packed = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int q = (int)roundf(w[4 * g + i] * id);
+                        sum += q;
+                        packed |= (u32)(q & 0xFF) << (8 * i);
+                    }
+                    *(u32 *)(qrow + 8 * g + 4 * lhi) = packed;
+                }
+                sum += __shfl_xor(sum, 32, 64);
+                if (lhi == 0) {
+                    act_ds e;
+                    e.d = half_bits_to_float(float_to_half_bits(d));
+                    e.sum = sum;
+                    a.act_s[iq * (a.Hq * D / 32) + e0 / 32] = e;
+                }
+            }
+        }
+    } else {
+        float *p = a.ws + ((iq * a.Hq + head) * a.n_splits + split) * (D + 2);
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) p[d_first + 32 * dt + 8 * g + 4 * lhi + i] = o[dt][4 * g + i];
+        if (h == 0 && lhi == 0) {
+            p[D] = m;
+            p[D + 1] = l;
+        }
+    }
+}
+
+template <int D>
+int launch_dec(hipStream_t s, const fattn_args &a) {
+    const int R = (int)(a.Hq / a.Hkv);
+    const int NT = 32 / R;
+    const dim3 grid((unsigned)a.n_splits, (unsigned)a.Hkv, (unsigned)((a.Nq + NT - 1) / NT));
+    hipLaunchKernelGGL(k_fattn_mma_dec<D>, grid, dim3(256), 0, s, a, R, NT);
+    return launch_status("k_fattn_mma_dec");
+}
+
+}  // namespace
+
+int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D) {
+    if (a.Hkv * (a.Hq / a.Hkv) > 65535 || (a.Nq + 31) / 32 > 0x7fffffff) return 1;
+    if ((a.q_nb1 % 16) != 0 || (a.q_nb2 % 16) != 0) return 1;
+    switch (D) {
+        case 64: return launch_hpw<64>(s, a);
+        case 128: return launch_hpw<128>(s, a);
+        default: return 1;   // other head sizes stay on the vector kernel
+    }
+}
+
+// Few query rows: returns 1 when the shape is not served.  a.n_splits / a.cells_per_split (a multiple of 64) are set by the caller.
+int launch_fattn_mma_dec(hipStream_t s, fattn_args &a, int64_t D) {
+    const int64_t R = a.Hq / a.Hkv;
+    if (R > 32 || a.Hkv > 65535 || (a.q_nb1 % 16) != 0 || (a.q_nb2 % 16) != 0 || a.cells_per_split % FM_BC != 0) return 1;
+    if ((a.Nq + (32 / R) - 1) / (32 / R) > 65535) return 1;
+    switch (D) {
+        case 64: return launch_dec<64>(s, a);
+        case 128: return launch_dec<128>(s, a);
+        default: return 1;
+    }
+}
+
+}  // namespace mi355
