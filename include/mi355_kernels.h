@@ -234,6 +234,14 @@ int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, c
                          int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
                          float beta_fast, float beta_slow);
 
+/* The gate and up projections of llm_build_ffn (LLM_FFN_SILU, LLM_FFN_PAR; src/llama.cpp:280-320) in ONE bandwidth-bound launch that
+ * also performs UNARY(SILU)(gate), MUL by up and the Q8_1 quantization the ffn_down product needs (ggml-cpu.c:6646-6683, 5142-5211;
+ * quantize_row_q8_1_ref).  gate/up: f32 [B][out_stride] receive the raw products; act_out: mi355_quantize_act layout of B rows of N.
+ * counters: N/32 zero-initialised DEVICE words that the launch leaves zero (the group that completes a 32-row block finishes it).
+ * B <= 4, N % 32 == 0, 16-byte aligned weight rows. */
+int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, int type_up, const void *w_up, const void *act, float *gate,
+                             float *up, int64_t out_stride, void *act_out, unsigned *counters, int64_t N, int64_t K, int64_t B);
+
 /* MUL_MAT with f32 or f16 src0 and f32 src1 (router / small dense matrices): dst[b][n] = sum_k W[n][k] x[b][k], strides honoured, ne2/ne3 broadcast */
 int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *src1, const mi355_tensor *dst);
 

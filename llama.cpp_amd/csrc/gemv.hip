@@ -59,7 +59,9 @@ struct gemv_batch {
     int n;
 };
 
-template <int TYPE, int NCOLS, int RPW, bool QKV = false>
+// COH: results are stored with device scope (written through to where every XCD sees them), for launches whose last
+// group reads rows produced by other groups
+template <int TYPE, int NCOLS, int RPW, bool QKV = false, bool COH = false>
 __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const int8_t *__restrict__ aq,
                                           const act_ds *__restrict__ ads, int K, const gemv_rope *rp = nullptr) {
     typedef wq<TYPE> T;
@@ -137,20 +139,22 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
                 const float s = wave_sum(acc[r][c]);
                 if (lane == 0 && row0 + r < m.N) {
                     const int64_t o = c * m.dst_stride + row0 + r;
-                    m.dst[o] = m.residual ? s + m.residual[o] : s;
+                    const float v = m.residual ? s + m.residual[o] : s;
+                    if constexpr (COH) __hip_atomic_store(m.dst + o, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    else m.dst[o] = v;
                 }
             }
     }
 }
 
-template <int NCOLS, int RPW>
+template <int NCOLS, int RPW, bool COH = false>
 __device__ __forceinline__ void gemv_dispatch(const gemv_item &m, int group, const int8_t *__restrict__ aq,
                                               const act_ds *__restrict__ ads, int K) {
     switch (m.type) {   // uniform over the group
-        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, RPW>(m, group, aq, ads, K); break;
-        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW>(m, group, aq, ads, K); break;
-        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW>(m, group, aq, ads, K); break;
-        default: gemv_body<MI355_Q6_K, NCOLS, RPW>(m, group, aq, ads, K); break;
+        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
+        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
+        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
+        default: gemv_body<MI355_Q6_K, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
     }
 }
 
@@ -187,6 +191,73 @@ __global__ void __launch_bounds__(256) k_gemv_multi(gemv_batch b, const int8_t *
     for (int j = 1; j < 4; j++)
         if (j < b.n && g >= b.it[j].first_group) i = j;
     gemv_dispatch<NCOLS, RPW>(b.it[i], g - b.it[i].first_group, aq, ads, K);
+}
+
+// ---- a launch whose last-arriving groups also do the nodes that follow the product ------------
+// Every group stores its rows with device scope and waits for those stores (the barrier does), then
+// one thread takes a ticket from the counter of its 32-row block.  The group that draws the last
+// ticket of a block knows that all of the block's rows have been written, reads them back with
+// device-scope loads, finishes the follow-up nodes and re-arms the counter for the next launch.  No
+// cache-wide fence is involved (a device-scope fence per group writes back and invalidates the
+// whole L2 and made a decoded token 10x slower), counters are shared by 8 groups only (one counter
+// for a whole launch serialises ~1000 device-scope atomics), and nobody waits for anybody, so
+// there is nothing that could hang.
+struct gemv_tail {
+    unsigned *counters;     // one per 32-row block; zero before the first launch, left zero by every launch
+    int8_t *act_q;          // quantized output, split activation layout
+    act_ds *act_s;
+    const float *x2;        // rows of the second matrix (up), same stride as the first
+    int n;                  // elements per output row (N of the matrices)
+};
+
+__device__ __forceinline__ float load_coherent(const float *p) {   // bypasses caches that other XCDs cannot invalidate
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Q8_1 of one value per lane over aligned groups of 32 lanes (quantize_row_q8_1_ref, ggml-quants.c:220-253)
+__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q = (int)roundf(v * id);
+    int sum = q;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    qrow[e] = (int8_t)q;
+    if ((e & 31) == 0) {
+        act_ds o;
+        o.d = half_bits_to_float(float_to_half_bits(d));
+        o.sum = sum;
+        srow[e >> 5] = o;
+    }
+}
+
+// gate and up projections (llm_build_ffn, src/llama.cpp:280-320) with UNARY(SILU), MUL and the Q8_1 quantization of
+// the product done per 32-row block by whichever of the block's 8 groups (4 per matrix, 8 rows each) finishes last
+template <int NCOLS>
+__global__ void __launch_bounds__(256) k_gemv_gate_up(gemv_batch b, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K, gemv_tail t) {
+    __shared__ unsigned s_ticket;
+    const int g = blockIdx.x;
+    const int i = g >= b.it[1].first_group ? 1 : 0;
+    const int group = g - b.it[i].first_group;
+    gemv_dispatch<NCOLS, 2, true>(b.it[i], group, aq, ads, K);
+    __syncthreads();   // waits for this group's stores, which were made with device scope
+    const int block = group >> 2;   // 8 rows per group, 32 rows per quantization block
+    if (threadIdx.x == 0) s_ticket = atomicAdd(t.counters + block, 1u);
+    __syncthreads();
+    if (s_ticket != 7u) return;   // uniform over the group
+    if (threadIdx.x == 0) t.counters[block] = 0;
+    const int tid = threadIdx.x;
+    for (int idx = tid; idx < 32 * NCOLS; idx += 256) {   // NCOLS <= 4: whole waves, aligned groups of 32 lanes
+        const int col = idx >> 5, j = idx & 31;
+        const int64_t row = (int64_t)block * 32 + j;
+        const float gv = load_coherent(b.it[0].dst + col * b.it[0].dst_stride + row);
+        const float uv = load_coherent(t.x2 + col * b.it[0].dst_stride + row);
+        const float h = (gv / (1.0f + expf(-gv))) * uv;
+        quantize_lane32(h, t.act_q + (int64_t)col * t.n, t.act_s + (int64_t)col * (t.n >> 5), row);
+    }
 }
 
 // MUL_MAT_ID, one activation row per expert slot: blockIdx.y = slot = t * n_used + e.  The
@@ -453,6 +524,48 @@ int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, c
         default: hipLaunchKernelGGL(k_gemv_qkv<4>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
     }
     return launch_status("k_gemv_qkv");
+}
+
+int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, int type_up, const void *w_up, const void *act, float *gate,
+                             float *up, int64_t out_stride, void *act_out, unsigned *counters, int64_t N, int64_t K, int64_t B) {
+    MI355_REQUIRE(B >= 1 && B <= 4, "ffn_gate_up_swiglu: batch %lld outside 1..4", (long long)B);
+    MI355_REQUIRE(N > 0 && N % 32 == 0 && out_stride >= N, "ffn_gate_up_swiglu: N=%lld must be a positive multiple of 32 and fit the row stride", (long long)N);
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0 && ((uintptr_t)act_out & 15) == 0 && counters != nullptr, "ffn_gate_up_swiglu: misaligned or missing operands");
+    int rc = check_gemv_args("ffn_gate_up_swiglu", type_gate, w_gate, N, K, out_stride);
+    if (rc != MI355_OK) return rc;
+    rc = check_gemv_args("ffn_gate_up_swiglu", type_up, w_up, N, K, out_stride);
+    if (rc != MI355_OK) return rc;
+    const int64_t per = N / 8;   // groups per matrix: 4 waves x 2 rows
+    MI355_REQUIRE(2 * per < 0x7fffffff, "ffn_gate_up_swiglu: too many rows for one launch");
+    gemv_batch b;
+    b.n = 2;
+    for (int i = 0; i < 4; i++) {
+        const int j = i & 1;
+        b.it[i].W = (const uint8_t *)(j ? w_up : w_gate);
+        b.it[i].dst = j ? up : gate;
+        b.it[i].residual = nullptr;
+        b.it[i].N = N;
+        b.it[i].dst_stride = out_stride;
+        b.it[i].type = j ? type_up : type_gate;
+        b.it[i].first_group = (int)(j * per);
+        b.it[i].epi = EPI_STORE;
+        b.it[i].nb1 = b.it[i].nb2 = 0;
+    }
+    gemv_tail t;
+    t.counters = counters; t.x2 = up; t.n = (int)N;
+    t.act_q = (int8_t *)act_out;
+    t.act_s = (act_ds *)(t.act_q + B * N);
+    hipStream_t s = (hipStream_t)stream;
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + B * K);
+    const dim3 grid((unsigned)(2 * per));
+    switch (B) {
+        case 1: hipLaunchKernelGGL(k_gemv_gate_up<1>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
+        case 2: hipLaunchKernelGGL(k_gemv_gate_up<2>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
+        case 3: hipLaunchKernelGGL(k_gemv_gate_up<3>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
+        default: hipLaunchKernelGGL(k_gemv_gate_up<4>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
+    }
+    return launch_status("k_gemv_gate_up");
 }
 
 // act: split layout of nb1*T quantized rows of b.  dst [N, n_used, T] contiguous.

@@ -97,6 +97,7 @@ class LlamaRunner:
         dev = self.dev = weights.output[1].device
         self.lib = load()
         self.fuse_qkv = True    # rows must be 16-byte aligned; set False to use the three-launch sequence
+        self.fuse_tail = True   # swiglu + Q8_1 done by the last group of each 32-row block of the gate/up launch (decode, T <= 4)
         E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
         T = self.max_tokens = max_tokens
         f32 = dict(dtype=torch.float32, device=dev)
@@ -117,6 +118,8 @@ class LlamaRunner:
         kmax = max(E, F, H * D)
         self.act_a = torch.empty(int(self.lib.mi355_act_bytes(max(E, H * D), T)) + 256, dtype=torch.uint8, device=dev)
         self.act_b = torch.empty(int(self.lib.mi355_act_bytes(F, T)) + 256, dtype=torch.uint8, device=dev)
+        self.act_c = torch.empty(int(self.lib.mi355_act_bytes(max(E, H * D), 4)) + 256, dtype=torch.uint8, device=dev)
+        self.tickets = torch.zeros(F // 32 + 64, dtype=torch.int32, device=dev)   # arrival counters of the tail-fused launches
         self.ws = torch.empty(int(self.lib.mi355_mul_mat_ws_bytes(kmax, T)) + 256, dtype=torch.uint8, device=dev)
         self.fa_ws = torch.empty(min(int(self.lib.mi355_flash_attn_ws_bytes(D, T, cfg.n_ctx, H)), 256 << 20), dtype=torch.uint8, device=dev)
 
@@ -198,6 +201,8 @@ class LlamaRunner:
         cfg, w, lib = self.cfg, self.w, self.lib
         E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
         x = self.x[:T]
+        if T <= 4 and self.fuse_qkv and self.fuse_tail and (T == 1 or not last_only):
+            return self._forward_decode(T, n_kv)
         big = T > 8
         for il, L in enumerate(w.layers):
             qkv = [(L["wq"], self.q[:T]), (L["wk"], self.k[:T]), (L["wv"], self.v[:T])]
@@ -241,6 +246,31 @@ class LlamaRunner:
         self._norm_quant(xo, w.output_norm, self.act_a, To, kq)
         self._mm_act(out, self.act_a, E, To, q8k=kq)
         return self.logits[:To]
+
+    def _forward_decode(self, T, n_kv):
+        """decode sequence, 7 launches per layer: [QKV + rope + KV store] [attention + Q8_1] [wo + residual] [norm + Q8_1]
+        [gate/up + SiLU*up + Q8_1] [down + residual] [next norm + Q8_1]; same arithmetic per node as forward_nodes"""
+        cfg, w, lib = self.cfg, self.w, self.lib
+        E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
+        x = self.x[:T]
+        self._norm_quant(x, w.layers[0]["attn_norm"], self.act_a, T)
+        for il, L in enumerate(w.layers):
+            kc, vc = self.kcache[il], self.vcache[il]
+            (tq, Wq), (tk, Wk), (tv, Wv) = L["wq"], L["wk"], L["wv"]
+            check(lib.mi355_qkv_rope_store(_stream(), tq, _ptr(Wq), tk, _ptr(Wk), tv, _ptr(Wv), _ptr(self.act_a), _ptr(self.q), _ptr(kc), _ptr(vc),
+                                           _ptr(self.pos), _ptr(self.pos), None, E, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2,
+                                           vc.stride(0) * 2, vc.stride(1) * 2, D, 0, cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
+            self._attn(il, T, n_kv, act=self.act_a)
+            self._mm_act([(L["wo"], x)], self.act_a, H * D, T, residual=x)
+            self._norm_quant(x, L["ffn_norm"], self.act_c, T)
+            (tg, Wg), (tu, Wu) = L["gate"], L["up"]
+            check(lib.mi355_ffn_gate_up_swiglu(_stream(), tg, _ptr(Wg), tu, _ptr(Wu), _ptr(self.act_c), _ptr(self.gate), _ptr(self.up), F,
+                                               _ptr(self.act_b), _ptr(self.tickets), F, E, T))
+            nxt = w.layers[il + 1]["attn_norm"] if il + 1 < len(w.layers) else w.output_norm
+            self._mm_act([(L["down"], x)], self.act_b, F, T, residual=x)
+            self._norm_quant(x, nxt, self.act_a, T)
+        self._mm_act([(w.output, self.logits[:T])], self.act_a, E, T)
+        return self.logits[:T]
 
     # ---- the same pass node for node, as the ggml graph lists it (reference for the fused path) --
     def forward_nodes(self, T, n_kv, last_only=True):
