@@ -18,6 +18,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "llama.cpp_amd"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the roofline kernel moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of this command,
+# calibrated on the copy kernel below (profiles/gemv_q4k_14336x4096_hbm_traffic.txt)
+GEMV_TRAFFIC_BYTES = 33160200
 
 
 def cpu_baseline(n_threads, budget_s=20.0):
@@ -168,10 +171,20 @@ def main():
         e1.record(stream)
         stream.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / (nrep * len(mats))
+    # reference for the HBM traffic counters: a plain copy kernel of known size (256 MiB read, 256 MiB written) whose
+    # FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit when this command runs under rocprofv3 --pmc
+    import ctypes as C
+    src = torch.empty(16384, 4096, dtype=torch.float32, device=dev).normal_()
+    dst_c = torch.empty_like(src)
+    ds_, dd_ = mi355.tensor_desc(src), mi355.tensor_desc(dst_c)
+    with torch.cuda.stream(stream):
+        mi355.check(lib.mi355_cpy(stream.cuda_stream, C.byref(ds_), C.byref(dd_)))
+        stream.synchronize()
+    del src, dst_c
     alg_bytes = N * K * 144 // 256 + 4 * K + 4 * N          # weights + f32 activation + f32 output
     achieved = alg_bytes / us / 1e3                          # GB/s
     roofline = {"kernel": "k_gemv_q<Q4_K, ncols 1> 14336x4096 (ffn_gate / ffn_up)", "bound": "hbm", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
                 "us_per_launch": round(us, 3), "algorithmic_bytes_per_launch": alg_bytes}
 
     cpu = None
