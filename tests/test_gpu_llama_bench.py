@@ -1,0 +1,50 @@
+"""Drop-in check at model level: the reference's own benchmark program, examples/llama-bench, built unmodified from the
+reference sources (oracle/Makefile, target llamabench), loads libggml-mi355.so through GGML_BACKEND_PATH, offloads every
+layer of a synthetic llama-architecture Q4_K_M model (tests/make_synthetic_gguf.py) and runs prefill and decode with flash
+attention.  The test asserts that the run completes on the plug-in's device and writes the table to gpurun_out/."""
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BENCH = os.path.join(ROOT, "oracle", "_ref", "llama-bench")
+PLUGIN = os.path.join(ROOT, "llama.cpp_amd", "lib", "libggml-mi355.so")
+
+
+def run_llama_bench(model, args, timeout=900):
+    env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN)
+    r = subprocess.run([BENCH, "-m", model, "-ngl", "99", "-fa", "1"] + args, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                       text=True, timeout=timeout, cwd=os.path.dirname(BENCH))
+    return r
+
+
+def parse_table(text):
+    """{test name: tokens/s} from llama-bench's markdown table"""
+    out = {}
+    for line in text.splitlines():
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 3 and re.match(r"^(pp|tg)\d+$", cells[-2]):
+            out[cells[-2]] = float(cells[-1].split()[0])
+    return out
+
+
+def test_llama_bench_runs_on_the_plugin(dev, tmp_path):
+    if not (os.path.exists(BENCH) and os.path.exists(PLUGIN)):
+        pytest.skip("llama-bench or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import make_synthetic_gguf
+    model = str(tmp_path / "small.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=4, n_embd=2048, n_ff=6144, n_head=16, n_head_kv=4, n_vocab=4096)
+    r = run_llama_bench(model, ["-p", "64", "-n", "16", "-r", "2"])
+    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+    with open(os.path.join(ROOT, "gpurun_out", "llama_bench_small.log"), "w") as f:
+        f.write(r.stdout)
+    assert r.returncode == 0, r.stdout[-3000:]
+    assert "MI355X" in r.stdout, "the plug-in's device does not appear in the table:\n" + r.stdout[-3000:]
+    t = parse_table(r.stdout)
+    assert t.get("pp64", 0) > 0 and t.get("tg16", 0) > 0, r.stdout[-3000:]
