@@ -223,6 +223,35 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
                         size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                         float ext_factor, float attn_factor, float beta_fast, float beta_slow);
 
+/* Up to three weight matrices on one quantized activation whose finished rows go through the nodes that follow the projections in
+ * build_llama (src/llama.cpp:1514-1548; llm_build_kv_store :157-199): ROPE (ggml-cpu.c:9366-9549, adjacent-pair mode only) and / or
+ * CPY to an f16 tensor such as a KV-cache view (ggml-cpu.c:3519-3830).  A wave owns output rows 2i and 2i+1, i.e. one rotation pair.
+ *   MI355_EPI_STORE       dst f32 [B][dst_stride]                          plain product
+ *   MI355_EPI_ROPE        dst f32 [B][dst_stride], rows = [head][head_dim]  rotated by pos[b]
+ *   MI355_EPI_ROPE_CACHE  dst f16 at cells[b]*nb1 + head*nb2 + 2*d          rotated, then converted
+ *   MI355_EPI_CACHE       dst f16 at cells[b]*nb1 + head*nb2 + 2*d          converted
+ * pos / cells: DEVICE int32 [B].  B <= 4; 16-byte aligned weight rows. */
+enum { MI355_EPI_STORE = 0, MI355_EPI_ROPE = 1, MI355_EPI_ROPE_CACHE = 2, MI355_EPI_CACHE = 3 };
+typedef struct mi355_gemv_rope_mat {
+    int          type;
+    const void  *W;           /* N rows x K, device layout */
+    int64_t      N;           /* a whole number of heads unless the epilogue is MI355_EPI_STORE */
+    int          epilogue;
+    void        *dst;
+    int64_t      dst_stride;  /* f32 elements between activation rows (STORE, ROPE) */
+    int64_t      nb1, nb2;    /* bytes per cell and per head (ROPE_CACHE, CACHE) */
+} mi355_gemv_rope_mat;
+typedef struct mi355_rope_desc {
+    const int32_t *pos;
+    const int32_t *cells;
+    const float   *freq_factors;   /* [n_dims/2] or NULL */
+    int64_t        head_dim;
+    int            n_dims, mode, n_ctx_orig;
+    float          freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
+} mi355_rope_desc;
+int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat *mats, const void *act, int64_t K, int64_t B,
+                             const mi355_rope_desc *rope);
+
 /* The Q, K and V projections of build_llama (src/llama.cpp:1514-1533) in ONE bandwidth-bound launch whose epilogue does what the graph
  * does next: ROPE(q) into q f32 [B][H][D]; ROPE(k) and CPY into the f16 K cache; CPY(v) into the f16 V cache (src/llama.cpp:1535-1548,
  * llm_build_kv_store :157-199; ggml-cpu.c:9366-9549, 3519-3830).  wq/wk/wv: device-layout rows of K (16-byte aligned rows required);

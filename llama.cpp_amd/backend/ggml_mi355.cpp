@@ -29,6 +29,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "mi355_kernels.h"
@@ -84,12 +85,47 @@ struct device_ctx {
     std::string description;
 };
 
+// Quantized form of an f32 activation tensor, kept while consecutive MUL_MAT nodes consume the same src1
+struct act_cache {
+    const void * src = nullptr;   // data pointer of the f32 tensor this was quantized from (B rows of K, contiguous)
+    int64_t K = 0, B = 0;
+    int format = 0;               // ACT_Q8_1 (32-element blocks, GEMV) or ACT_Q8K (256-element super-blocks, tile GEMM)
+    bool valid = false;
+};
+enum { ACT_Q8_1 = 1, ACT_Q8K = 2 };
+
 struct backend_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     void * ws = nullptr;   // scratch for quantized activations / attention partials
     size_t ws_size = 0;
+    void * act = nullptr;  // quantized activation shared by consecutive matrix products (see act_cache)
+    size_t act_size = 0;
+    act_cache cache;
+    bool fuse = true;      // MI355_NO_FUSION=1 executes the graph node for node
+    int32_t * iota = nullptr;   // device {0, 1, 2, ...}: token t of a batch goes to row t of a KV-cache view
     std::string name;
+
+    // a node is about to write [p, p + bytes): the cached activation dies if that touches the tensor it came from
+    void note_write(const void * p, size_t bytes) {
+        if (!cache.valid) return;
+        const char * a0 = (const char *) cache.src, * a1 = a0 + (size_t) cache.K * (size_t) cache.B * sizeof(float);
+        const char * b0 = (const char *) p, * b1 = b0 + bytes;
+        if (a0 < b1 && b0 < a1) cache.valid = false;
+    }
+
+    void * act_buffer(size_t need) {
+        if (need > act_size) {
+            if (act) {
+                MI355_HIP_OK(hipStreamSynchronize(stream));
+                MI355_HIP_OK(hipFree(act));
+            }
+            act_size = (need + (size_t(4) << 20)) & ~((size_t(1) << 20) - 1);
+            MI355_HIP_OK(hipMalloc(&act, act_size));
+            cache.valid = false;
+        }
+        return act;
+    }
 
     void * workspace(size_t need) {
         if (need > ws_size) {
@@ -521,6 +557,8 @@ void backend_free(ggml_backend_t backend) {
     (void) hipSetDevice(ctx->device);
     (void) hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void) hipFree(ctx->ws);
+    if (ctx->act) (void) hipFree(ctx->act);
+    if (ctx->iota) (void) hipFree(ctx->iota);
     if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     delete backend;
@@ -531,21 +569,320 @@ void backend_synchronize(ggml_backend_t backend) {
     MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
 }
 
+// ------------------------------------------------------------------------------- graph execution with local fusion
+// The graph llama.cpp builds for a token is ~25 small nodes per layer.  The executor looks a few nodes ahead and
+// replaces the sequences below by the fused entry points of the kernel library (each is tested bit-identical to the
+// separate launches).  A pattern only matches when the skipped intermediate has exactly one consumer in this graph
+// and is not a graph output, so nothing observable changes:
+//   RMS_NORM -> MUL(weight)                      one launch, and the Q8_1 form of the result when a quantized MUL_MAT follows
+//   UNARY(SILU) -> MUL                           one launch, same
+//   FLASH_ATTN_EXT (few rows) -> MUL_MAT         attention also writes the Q8_1 form of its output
+//   MUL_MAT, MUL_MAT, ... on the same src1       activation quantized once; up to 4 matrices per GEMV launch
+//   MUL_MAT -> ADD(residual)                     residual added in the GEMV epilogue
+bool is_noop(const ggml_tensor * t) {
+    switch (t->op) {
+        case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE: return true;
+        default: return ggml_is_empty(t);
+    }
+}
+
+struct graph_walk {
+    ggml_cgraph * g;
+    int n;
+    std::vector<int> uses;   // per node index: how many nodes of this graph read it
+    std::vector<const ggml_tensor *> nodes;
+
+    explicit graph_walk(ggml_cgraph * cg) : g(cg), n(ggml_graph_n_nodes(cg)), uses(n, 0), nodes(n) {
+        std::unordered_map<const ggml_tensor *, int> index;
+        index.reserve((size_t) n * 2);
+        for (int i = 0; i < n; i++) {
+            nodes[i] = ggml_graph_node(g, i);
+            index[nodes[i]] = i;
+        }
+        auto count = [&](const ggml_tensor * t) {
+            if (!t) return;
+            auto it = index.find(t);
+            if (it != index.end()) uses[it->second]++;
+        };
+        for (int i = 0; i < n; i++) {   // each distinct tensor a node reads counts once
+            const ggml_tensor * seen[GGML_MAX_SRC + 1];
+            int n_seen = 0;
+            auto once = [&](const ggml_tensor * t) {
+                if (!t) return;
+                for (int k = 0; k < n_seen; k++)
+                    if (seen[k] == t) return;
+                seen[n_seen++] = t;
+                count(t);
+            };
+            for (int s = 0; s < GGML_MAX_SRC; s++) once(nodes[i]->src[s]);
+            once(nodes[i]->view_src);
+        }
+    }
+    int next(int i) const {   // next node that launches work, or n
+        for (i = i + 1; i < n; i++)
+            if (!is_noop(nodes[i])) return i;
+        return n;
+    }
+    bool sole_use(int i) const { return uses[i] == 1 && !(nodes[i]->flags & GGML_TENSOR_FLAG_OUTPUT); }
+};
+
+bool is_quant_gemv_candidate(const ggml_tensor * mm) {
+    // quantized weights in 16-byte aligned rows, one 2-D activation matrix of at most 8 contiguous rows
+    const ggml_tensor * a = mm->src[0];
+    const ggml_tensor * b = mm->src[1];
+    if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
+    if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
+    if (b->ne[1] > 8 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
+    const int64_t K = a->ne[0];
+    if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
+    if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)
+    return ((uintptr_t) a->data & 15) == 0 && ((uintptr_t) b->data & 15) == 0;
+}
+
+bool is_q8k_tile_candidate(const ggml_tensor * mm) {
+    const ggml_tensor * a = mm->src[0];
+    const ggml_tensor * b = mm->src[1];
+    if (mm->op != GGML_OP_MUL_MAT || (a->type != GGML_TYPE_Q4_K && a->type != GGML_TYPE_Q6_K)) return false;
+    if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
+    if (b->ne[1] <= 8 || b->nb[1] % 16 != 0) return false;
+    const int64_t K = a->ne[0];
+    if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;
+    return ((uintptr_t) a->data & 15) == 0 && ((uintptr_t) b->data & 15) == 0;
+}
+
+// does the node after `i` (skipping views) multiply a quantized matrix by the tensor whose data starts at `data`?
+bool feeds_quant_gemv(const graph_walk & w, int i, const void * data, int64_t K, int64_t B) {
+    const int j = w.next(i);
+    if (j >= w.n) return false;
+    const ggml_tensor * mm = w.nodes[j];
+    return is_quant_gemv_candidate(mm) && mm->src[1]->data == data && mm->src[0]->ne[0] == K && mm->src[1]->ne[1] == B;
+}
+
+// Runs node i and possibly a few of its successors; returns the index of the last node consumed.
+int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
+    hipStream_t s = ctx->stream;
+    ggml_tensor * node = (ggml_tensor *) w.nodes[i];
+    const int j = w.next(i);
+    ggml_tensor * nxt = j < w.n ? (ggml_tensor *) w.nodes[j] : nullptr;
+
+    // ---- RMS_NORM -> MUL(weight vector)
+    if (node->op == GGML_OP_RMS_NORM && nxt && nxt->op == GGML_OP_MUL && nxt->src[0] == node && w.sole_use(i)) {
+        const ggml_tensor * x = node->src[0];
+        const ggml_tensor * wt = nxt->src[1];
+        const int64_t K = x->ne[0], rows = ggml_nrows(x);
+        if (ggml_is_contiguous(x) && ggml_is_contiguous(nxt) && wt->type == GGML_TYPE_F32 && ggml_is_contiguous(wt) && ggml_nelements(wt) == K &&
+            K % 32 == 0 && K <= 16384 && x->type == GGML_TYPE_F32 && nxt->type == GGML_TYPE_F32 &&
+            (((uintptr_t) x->data | (uintptr_t) nxt->data | (uintptr_t) wt->data) & 15) == 0) {
+            float eps;
+            memcpy(&eps, node->op_params, sizeof(float));
+            void * act = nullptr;
+            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_buffer(mi355_act_bytes(K, rows));
+            MI355_K_OK(mi355_rms_norm_mul_quant(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
+            ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr};
+            return j;
+        }
+    }
+    // ---- UNARY(SILU) -> MUL
+    if (node->op == GGML_OP_UNARY && ggml_get_unary_op(node) == GGML_UNARY_OP_SILU && nxt && nxt->op == GGML_OP_MUL && w.sole_use(i) &&
+        (nxt->src[0] == node || nxt->src[1] == node)) {
+        const ggml_tensor * gt = node->src[0];
+        const ggml_tensor * up = nxt->src[0] == node ? nxt->src[1] : nxt->src[0];
+        const int64_t K = gt->ne[0], rows = ggml_nrows(gt);
+        if (ggml_is_contiguous(gt) && ggml_is_contiguous(up) && ggml_is_contiguous(nxt) && ggml_are_same_shape(gt, up) && up->type == GGML_TYPE_F32 &&
+            K % 32 == 0 && rows <= 65535 && (((uintptr_t) gt->data | (uintptr_t) up->data | (uintptr_t) nxt->data) & 15) == 0) {
+            void * act = nullptr;
+            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_buffer(mi355_act_bytes(K, rows));
+            MI355_K_OK(mi355_swiglu_quant(s, (const float *) gt->data, (const float *) up->data, K, (float *) nxt->data, K, act, K, rows));
+            ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr};
+            return j;
+        }
+    }
+    // ---- FLASH_ATTN_EXT whose output feeds a quantized product
+    if (node->op == GGML_OP_FLASH_ATTN_EXT) {
+        const ggml_tensor * q = node->src[0];
+        const int64_t D = q->ne[0], Nq = q->ne[1], Hq = q->ne[2];
+        if (q->ne[3] == 1 && Nq <= 8 && D % 32 == 0 && feeds_quant_gemv(w, i, node->data, Hq * D, Nq)) {
+            const ggml_tensor * k = node->src[1];
+            const ggml_tensor * v = node->src[2];
+            const ggml_tensor * mask = node->src[3];
+            float scale, max_bias, softcap;
+            memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
+            memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
+            memcpy(&softcap, (const float *) node->op_params + 2, sizeof(float));
+            const int64_t Nkv = k->ne[1], Hkv = k->ne[2];
+            const size_t full = mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq);
+            const size_t ws_bytes = full < (size_t(256) << 20) ? full : (size_t(256) << 20);
+            void * ws = ctx->workspace(ws_bytes);
+            void * act = ctx->act_buffer(mi355_act_bytes(Hq * D, Nq));
+            MI355_K_OK(mi355_flash_attn_ext_quant(s, (const float *) q->data, k->data, v->data, mask ? mask->data : nullptr, (float *) node->data, D, Nq, Nkv,
+                                                  Hq, Hkv, q->nb[1], q->nb[2], k->nb[1], k->nb[2], v->nb[1], v->nb[2], mask ? mask->nb[1] : 0, scale,
+                                                  max_bias, softcap, ws, ws_bytes, act));
+            ctx->cache = act_cache{node->data, Hq * D, Nq, ACT_Q8_1, true};
+            return i;
+        }
+    }
+    // ---- MUL_MAT -> [RESHAPE] -> ROPE [-> CPY to an f16 view]   and   MUL_MAT -> CPY to an f16 view   (decode, batch <= 4)
+    if (is_quant_gemv_candidate(node) && node->src[1]->ne[1] <= 4 && w.sole_use(i) && nxt && node->ne[0] % 2 == 0) {
+        const ggml_tensor * b = node->src[1];
+        const int64_t K = b->ne[0], B = b->ne[1], N = node->ne[0];
+        // the consumer may read the product through one reshape
+        auto reads_product = [&](const ggml_tensor * t) {
+            if (t == node) return true;
+            return t && t->op == GGML_OP_RESHAPE && t->src[0] == node && ggml_is_contiguous(t);
+        };
+        auto sole_chain = [&](const ggml_tensor * t) {   // a reshape in between must have a single reader too
+            if (t == node) return true;
+            for (int k = i + 1; k < j; k++)
+                if (w.nodes[k] == t) return w.sole_use(k);
+            return false;
+        };
+        mi355_gemv_rope_mat m;
+        m.type = to_mi355_type(node->src[0]->type);
+        m.W = node->src[0]->data;
+        m.N = N;
+        m.dst = nullptr;
+        m.dst_stride = 0;
+        m.nb1 = m.nb2 = 0;
+        mi355_rope_desc rd;
+        memset(&rd, 0, sizeof(rd));
+        rd.cells = ctx->iota;
+        rd.head_dim = N;   // one "head" spanning the row unless a ROPE says otherwise
+        rd.n_dims = 2; rd.n_ctx_orig = 1; rd.freq_base = 10000.0f; rd.freq_scale = 1.0f; rd.attn_factor = 1.0f; rd.beta_fast = 32.0f; rd.beta_slow = 1.0f;
+        int last = -1;
+        auto f16_row_view = [&](const ggml_tensor * d) {   // CPY destination: B rows of N f16, contiguous
+            return d->type == GGML_TYPE_F16 && ggml_is_contiguous(d) && ggml_nelements(d) == N * B && ((uintptr_t) d->data & 1) == 0;
+        };
+        if (nxt->op == GGML_OP_ROPE && reads_product(nxt->src[0]) && sole_chain(nxt->src[0]) && nxt->src[1]->type == GGML_TYPE_I32 &&
+            ggml_is_contiguous(nxt) && nxt->type == GGML_TYPE_F32 && nxt->ne[0] * nxt->ne[1] == N && nxt->ne[2] == B && nxt->ne[3] == 1 &&
+            (!nxt->src[2] || nxt->src[2]->type == GGML_TYPE_F32)) {
+            const int32_t * p = (const int32_t *) nxt->op_params;
+            if (p[2] == 0 && p[1] % 2 == 0 && p[1] > 0 && p[1] <= nxt->ne[0] && nxt->ne[0] % 2 == 0) {
+                rd.pos = (const int32_t *) nxt->src[1]->data;
+                rd.freq_factors = nxt->src[2] ? (const float *) nxt->src[2]->data : nullptr;
+                rd.head_dim = nxt->ne[0];
+                rd.n_dims = p[1];
+                rd.mode = 0;
+                rd.n_ctx_orig = p[4];
+                memcpy(&rd.freq_base, p + 5, sizeof(float));
+                memcpy(&rd.freq_scale, p + 6, sizeof(float));
+                memcpy(&rd.ext_factor, p + 7, sizeof(float));
+                memcpy(&rd.attn_factor, p + 8, sizeof(float));
+                memcpy(&rd.beta_fast, p + 9, sizeof(float));
+                memcpy(&rd.beta_slow, p + 10, sizeof(float));
+                const int jc = w.next(j);
+                const ggml_tensor * cpy = jc < w.n ? w.nodes[jc] : nullptr;
+                if (cpy && cpy->op == GGML_OP_CPY && cpy->src[0] == nxt && w.sole_use(j) && f16_row_view(cpy->src[1])) {
+                    m.epilogue = MI355_EPI_ROPE_CACHE;   // rotated K rows straight into the cache view
+                    m.dst = cpy->src[1]->data;
+                    m.nb1 = N * 2;
+                    m.nb2 = rd.head_dim * 2;
+                    last = jc;
+                } else {
+                    m.epilogue = MI355_EPI_ROPE;         // rotated Q rows into the ROPE node's tensor
+                    m.dst = nxt->data;
+                    m.dst_stride = N;
+                    last = j;
+                }
+            }
+        } else if (nxt->op == GGML_OP_CPY && reads_product(nxt->src[0]) && sole_chain(nxt->src[0]) && f16_row_view(nxt->src[1])) {
+            m.epilogue = MI355_EPI_CACHE;                // V rows converted into the cache view
+            m.dst = nxt->src[1]->data;
+            m.nb1 = N * 2;
+            m.nb2 = 0;
+            last = j;
+        }
+        if (last >= 0) {
+            void * act = ctx->act_buffer(mi355_act_bytes(K, B));
+            if (!(ctx->cache.valid && ctx->cache.src == b->data && ctx->cache.K == K && ctx->cache.B == B && ctx->cache.format == ACT_Q8_1)) {
+                MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, act, K, B, K));
+                ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true};
+            }
+            MI355_K_OK(mi355_mul_mat_vec_q_rope(s, 1, &m, act, K, B, &rd));
+            ctx->note_write(m.dst, (size_t) N * (size_t) B * (m.epilogue == MI355_EPI_ROPE ? sizeof(float) : 2));
+            return last;
+        }
+    }
+    // ---- runs of quantized products on one activation (batch <= 8): one quantization, multi-matrix GEMV, residual epilogue
+    if (is_quant_gemv_candidate(node)) {
+        const ggml_tensor * b = node->src[1];
+        const int64_t K = b->ne[0], B = b->ne[1];
+        int run[4], n_run = 0, last = i;
+        for (int k = i; k < w.n && n_run < (B <= 4 ? 4 : 1); k = w.next(k)) {
+            const ggml_tensor * mm = w.nodes[k];
+            if (!is_quant_gemv_candidate(mm) || mm->src[1]->data != b->data || mm->src[1]->ne[0] != K || mm->src[1]->ne[1] != B) break;
+            run[n_run++] = k;
+            last = k;
+        }
+        void * act = ctx->act_buffer(mi355_act_bytes(K, B));
+        if (!(ctx->cache.valid && ctx->cache.src == b->data && ctx->cache.K == K && ctx->cache.B == B && ctx->cache.format == ACT_Q8_1)) {
+            MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, act, K, B, K));
+            ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true};
+        }
+        mi355_gemv_mat mats[4];
+        for (int r = 0; r < n_run; r++) {
+            ggml_tensor * mm = (ggml_tensor *) w.nodes[run[r]];
+            mats[r].type = to_mi355_type(mm->src[0]->type);
+            mats[r].W = mm->src[0]->data;
+            mats[r].N = mm->src[0]->ne[1];
+            mats[r].dst = (float *) mm->data;
+            mats[r].dst_stride = (int64_t) (mm->nb[1] / sizeof(float));
+            mats[r].residual = nullptr;
+        }
+        if (n_run == 1) {   // MUL_MAT -> ADD(residual): write the sum straight into the ADD's tensor
+            const int ja = w.next(i);
+            ggml_tensor * add = ja < w.n ? (ggml_tensor *) w.nodes[ja] : nullptr;
+            if (add && add->op == GGML_OP_ADD && w.sole_use(i) && (add->src[0] == node || add->src[1] == node)) {
+                const ggml_tensor * res = add->src[0] == node ? add->src[1] : add->src[0];
+                if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, node) && ggml_is_contiguous(res) && ggml_is_contiguous(add) &&
+                    ggml_is_contiguous(node)) {
+                    mats[0].dst = (float *) add->data;
+                    mats[0].dst_stride = (int64_t) (add->nb[1] / sizeof(float));
+                    mats[0].residual = (const float *) res->data;
+                    last = ja;
+                }
+            }
+        }
+        MI355_K_OK(mi355_mul_mat_vec_q_multi(s, n_run, mats, act, K, B));
+        for (int r = 0; r < n_run; r++) ctx->note_write(mats[r].dst, (size_t) mats[r].N * (size_t) B * sizeof(float));
+        return last;
+    }
+    // ---- runs of K-quant products on one activation (batch > 8): one per-super-block quantization
+    if (is_q8k_tile_candidate(node)) {
+        const ggml_tensor * b = node->src[1];
+        const int64_t K = b->ne[0], B = b->ne[1];
+        void * act = ctx->act_buffer(mi355_act_q8k_bytes(K, B));
+        if (!(ctx->cache.valid && ctx->cache.src == b->data && ctx->cache.K == K && ctx->cache.B == B && ctx->cache.format == ACT_Q8K)) {
+            MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, act, K, B, (int64_t) (b->nb[1] / sizeof(float))));
+            ctx->cache = act_cache{b->data, K, B, ACT_Q8K, true};
+        }
+        MI355_K_OK(mi355_mul_mat_q8k(s, to_mi355_type(node->src[0]->type), node->src[0]->data, act, (float *) node->data, node->src[0]->ne[1], K, B,
+                                     (int64_t) (node->nb[1] / sizeof(float))));
+        ctx->note_write(node->data, ggml_nbytes(node));
+        return i;
+    }
+    ctx->note_write(node->op == GGML_OP_CPY ? node->src[1]->data : node->data, ggml_nbytes(node->op == GGML_OP_CPY ? node->src[1] : node));
+    compute_node(ctx, node);
+    return i;
+}
+
 ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
-    const int n = ggml_graph_n_nodes(cgraph);
-    for (int i = 0; i < n; i++) {
-        ggml_tensor * node = ggml_graph_node(cgraph, i);
-        if (ggml_is_empty(node)) continue;
-        switch (node->op) {
-            case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
-                continue;
-            default:
-                break;
+    ctx->cache.valid = false;
+    if (!ctx->fuse) {
+        const int n = ggml_graph_n_nodes(cgraph);
+        for (int i = 0; i < n; i++) {
+            ggml_tensor * node = ggml_graph_node(cgraph, i);
+            if (!is_noop(node)) compute_node(ctx, node);
         }
-        compute_node(ctx, node);
+        return GGML_STATUS_SUCCESS;
     }
+    const graph_walk w(cgraph);
+    for (int i = 0; i < w.n; i++) {
+        if (is_noop(w.nodes[i])) continue;
+        i = compute_fused(ctx, w, i);
+    }
+    ctx->cache.valid = false;
     return GGML_STATUS_SUCCESS;   // asynchronous: completion is observed through synchronize()
 }
 
@@ -591,6 +928,14 @@ ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
     backend_ctx * ctx = new backend_ctx;
     ctx->device = dctx->device;
     ctx->name = dctx->name;
+    const char * nf = getenv("MI355_NO_FUSION");
+    ctx->fuse = !(nf && nf[0] == '1');
+    const int32_t iota_host[8] = {0, 1, 2, 3, 4, 5, 6, 7};
+    if (hipMalloc((void **) &ctx->iota, sizeof(iota_host)) != hipSuccess ||
+        hipMemcpy(ctx->iota, iota_host, sizeof(iota_host), hipMemcpyHostToDevice) != hipSuccess) {
+        delete ctx;
+        return nullptr;
+    }
     if (hipStreamCreate(&ctx->stream) != hipSuccess) {   // default priority, blocking w.r.t. the null stream
         delete ctx;
         return nullptr;

@@ -120,8 +120,8 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
             const int64_t head = row0 / R.D;
             const int d = (int)(row0 % R.D);
             float y0 = s0, y1 = s1;
-            if (m.epi != EPI_CACHE && d < R.n_dims) rope_rotate(R, R.pos[lane], d >> 1, s0, s1, y0, y1);
-            if (m.epi == EPI_ROPE) {
+            if ((m.epi == EPI_ROPE || m.epi == EPI_ROPE_CACHE) && d < R.n_dims) rope_rotate(R, R.pos[lane], d >> 1, s0, s1, y0, y1);
+            if (m.epi == EPI_ROPE || m.epi == EPI_STORE) {
                 float *o = m.dst + lane * m.dst_stride + row0;
                 o[0] = y0;
                 o[1] = y1;
@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(256) k_gemv_qkv(gemv_batch b, const int8_t *__
     int i = 0;
 #pragma unroll
     for (int j = 1; j < 3; j++)
-        if (g >= b.it[j].first_group) i = j;
+        if (g >= b.it[j].first_group) i = j;   // unused items start at INT_MAX
     const gemv_item &m = b.it[i];
     const int group = g - m.first_group;
     switch (m.type) {   // uniform over the group
@@ -469,49 +469,58 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     return launch_status("k_gemv_multi");
 }
 
-int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, const void *wk, int type_v, const void *wv, const void *act,
-                         float *q, void *kcache, void *vcache, const int32_t *pos, const int32_t *cells, const float *freq_factors,
-                         int64_t K, int64_t B, int64_t H, int64_t HK, int64_t D, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2,
-                         int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
-                         float beta_fast, float beta_slow) {
-    MI355_REQUIRE(B >= 1 && B <= 4, "qkv_rope_store: batch %lld outside 1..4", (long long)B);
-    MI355_REQUIRE(H > 0 && HK > 0 && D > 0 && D % 2 == 0 && n_dims > 0 && n_dims <= D && n_dims % 2 == 0, "qkv_rope_store: bad head geometry");
-    MI355_REQUIRE(mode == 0, "qkv_rope_store: only the adjacent-pair rope mode is fused (mode %d)", mode);
-    MI355_REQUIRE(((uintptr_t)act & 15) == 0 && ((uintptr_t)kcache & 1) == 0 && ((uintptr_t)vcache & 1) == 0 && k_nb1 % 2 == 0 && k_nb2 % 2 == 0 &&
-                  v_nb1 % 2 == 0 && v_nb2 % 2 == 0, "qkv_rope_store: misaligned operands");
-    const int types[3] = {type_q, type_k, type_v};
-    const void *Ws[3] = {wq, wk, wv};
-    const int64_t Ns[3] = {H * D, HK * D, HK * D};
-    for (int i = 0; i < 3; i++) {
-        int rc = check_gemv_args("qkv_rope_store", types[i], Ws[i], Ns[i], K, Ns[i]);
-        if (rc != MI355_OK) return rc;
-    }
+int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat *mats, const void *act, int64_t K, int64_t B,
+                             const mi355_rope_desc *rope) {
+    MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr && rope != nullptr, "mul_mat_vec_q_rope: 1..3 matrices per launch");
+    MI355_REQUIRE(B >= 1 && B <= 4, "mul_mat_vec_q_rope: batch %lld outside 1..4", (long long)B);
+    const int64_t D = rope->head_dim;
+    const int n_dims = rope->n_dims;
+    MI355_REQUIRE(D > 0 && D % 2 == 0 && n_dims > 0 && n_dims <= D && n_dims % 2 == 0, "mul_mat_vec_q_rope: bad head geometry");
+    MI355_REQUIRE(rope->mode == 0, "mul_mat_vec_q_rope: only the adjacent-pair rope mode is fused (mode %d)", rope->mode);
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_vec_q_rope: activation workspace is not 16-byte aligned");
     gemv_batch b;
-    b.n = 3;
+    b.n = n_mats;
     int64_t groups = 0;
+    bool needs_pos = false, needs_cells = false;
     for (int i = 0; i < 4; i++) {
-        const int j = i < 3 ? i : 0;
-        b.it[i].W = (const uint8_t *)Ws[j];
+        const mi355_gemv_rope_mat &m = mats[i < n_mats ? i : 0];
+        if (i < n_mats) {
+            int rc = check_gemv_args("mul_mat_vec_q_rope", m.type, m.W, m.N, K, m.N);
+            if (rc != MI355_OK) return rc;
+            MI355_REQUIRE(m.epilogue >= MI355_EPI_STORE && m.epilogue <= MI355_EPI_CACHE && m.dst != nullptr && m.N % 2 == 0,
+                          "mul_mat_vec_q_rope: bad epilogue %d, missing destination or odd row count", m.epilogue);
+            if (m.epilogue == MI355_EPI_STORE || m.epilogue == MI355_EPI_ROPE)
+                MI355_REQUIRE(m.dst_stride >= m.N, "mul_mat_vec_q_rope: dst_stride < N");
+            else
+                MI355_REQUIRE(((uintptr_t)m.dst & 1) == 0 && m.nb1 % 2 == 0 && m.nb2 % 2 == 0, "mul_mat_vec_q_rope: misaligned f16 destination");
+            if (m.epilogue != MI355_EPI_STORE) MI355_REQUIRE(m.N % D == 0, "mul_mat_vec_q_rope: N=%lld is not a whole number of heads", (long long)m.N);
+            needs_pos = needs_pos || m.epilogue == MI355_EPI_ROPE || m.epilogue == MI355_EPI_ROPE_CACHE;
+            needs_cells = needs_cells || m.epilogue == MI355_EPI_ROPE_CACHE || m.epilogue == MI355_EPI_CACHE;
+        }
+        b.it[i].W = (const uint8_t *)m.W;
         b.it[i].residual = nullptr;
-        b.it[i].N = Ns[j];
-        b.it[i].type = types[j];
-        b.it[i].first_group = (int)groups;
-        if (i < 3) groups += (Ns[j] + 7) / 8;   // 4 waves x 2 rows
+        b.it[i].N = m.N;
+        b.it[i].type = m.type;
+        b.it[i].dst = (float *)m.dst;
+        b.it[i].dst_stride = m.dst_stride;
+        b.it[i].nb1 = m.nb1;
+        b.it[i].nb2 = m.nb2;
+        // the kernel's epilogue codes: plain rows take the rope path with no rotation applied to them
+        b.it[i].epi = m.epilogue == MI355_EPI_STORE ? EPI_STORE : m.epilogue == MI355_EPI_ROPE ? EPI_ROPE : m.epilogue == MI355_EPI_ROPE_CACHE ? EPI_ROPE_CACHE : EPI_CACHE;
+        b.it[i].first_group = i < n_mats ? (int)groups : 0x7fffffff;
+        if (i < n_mats) groups += (m.N + 7) / 8;   // 4 waves x 2 rows
     }
-    b.it[0].dst = q;               b.it[0].dst_stride = H * D; b.it[0].epi = EPI_ROPE;       b.it[0].nb1 = b.it[0].nb2 = 0;
-    b.it[1].dst = (float *)kcache; b.it[1].dst_stride = 0;     b.it[1].epi = EPI_ROPE_CACHE; b.it[1].nb1 = (int64_t)k_nb1; b.it[1].nb2 = (int64_t)k_nb2;
-    b.it[2].dst = (float *)vcache; b.it[2].dst_stride = 0;     b.it[2].epi = EPI_CACHE;      b.it[2].nb1 = (int64_t)v_nb1; b.it[2].nb2 = (int64_t)v_nb2;
-    b.it[3] = b.it[0];
-    b.it[3].first_group = 0x7fffffff;
-    MI355_REQUIRE(groups < 0x7fffffff, "qkv_rope_store: too many rows for one launch");
+    MI355_REQUIRE(!needs_pos || rope->pos != nullptr, "mul_mat_vec_q_rope: rope positions missing");
+    MI355_REQUIRE(!needs_cells || rope->cells != nullptr, "mul_mat_vec_q_rope: cache cells missing");
+    MI355_REQUIRE(groups < 0x7fffffff, "mul_mat_vec_q_rope: too many rows for one launch");
     gemv_rope rp;
-    rp.pos = pos; rp.cells = cells; rp.ff = freq_factors;
+    rp.pos = rope->pos; rp.cells = rope->cells; rp.ff = rope->freq_factors;
     rp.D = (int)D; rp.n_dims = n_dims;
-    rp.theta_scale = powf(freq_base, -2.0f / n_dims);
-    rp.freq_scale = freq_scale; rp.ext_factor = ext_factor; rp.attn_factor = attn_factor;
+    rp.theta_scale = powf(rope->freq_base, -2.0f / n_dims);
+    rp.freq_scale = rope->freq_scale; rp.ext_factor = rope->ext_factor; rp.attn_factor = rope->attn_factor;
     const float pi = 3.14159265358979323846f;   // ggml_rope_yarn_corr_dims, ggml/src/ggml.c:3695-3707
-    const float c0 = floorf(n_dims * logf(n_ctx_orig / (beta_fast * 2 * pi)) / (2 * logf(freq_base)));
-    const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
+    const float c0 = floorf(n_dims * logf(rope->n_ctx_orig / (rope->beta_fast * 2 * pi)) / (2 * logf(rope->freq_base)));
+    const float c1 = ceilf(n_dims * logf(rope->n_ctx_orig / (rope->beta_slow * 2 * pi)) / (2 * logf(rope->freq_base)));
     rp.corr0 = c0 > 0 ? c0 : 0;
     rp.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
     hipStream_t s = (hipStream_t)stream;
@@ -524,6 +533,20 @@ int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, c
         default: hipLaunchKernelGGL(k_gemv_qkv<4>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
     }
     return launch_status("k_gemv_qkv");
+}
+
+int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, const void *wk, int type_v, const void *wv, const void *act,
+                         float *q, void *kcache, void *vcache, const int32_t *pos, const int32_t *cells, const float *freq_factors,
+                         int64_t K, int64_t B, int64_t H, int64_t HK, int64_t D, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2,
+                         int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
+                         float beta_fast, float beta_slow) {
+    MI355_REQUIRE(H > 0 && HK > 0 && D > 0, "qkv_rope_store: bad head geometry");
+    mi355_gemv_rope_mat m[3];
+    m[0] = mi355_gemv_rope_mat{type_q, wq, H * D, MI355_EPI_ROPE, q, H * D, 0, 0};
+    m[1] = mi355_gemv_rope_mat{type_k, wk, HK * D, MI355_EPI_ROPE_CACHE, kcache, 0, (int64_t)k_nb1, (int64_t)k_nb2};
+    m[2] = mi355_gemv_rope_mat{type_v, wv, HK * D, MI355_EPI_CACHE, vcache, 0, (int64_t)v_nb1, (int64_t)v_nb2};
+    mi355_rope_desc r = {pos, cells, freq_factors, D, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow};
+    return mi355_mul_mat_vec_q_rope(stream, 3, m, act, K, B, &r);
 }
 
 int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, int type_up, const void *w_up, const void *act, float *gate,

@@ -1,0 +1,54 @@
+// Test infrastructure (not shipped): drives the reference's own model runtime (libllama, built from the reference
+// sources by this directory's Makefile) through its public API and dumps logits, so that a test can compare the
+// reference CPU backend with the plug-in, and the plug-in's fused graph execution with its node-by-node execution,
+// on the same synthetic model and token ids.
+//
+//   llama_logits <model.gguf> <n_gpu_layers> <n_prompt> <n_decode> <out.bin>
+//
+// Tokens are (7 i + 3) mod n_vocab.  Output: float32 rows of n_vocab logits, one for the last prompt token and one per
+// decoded token (the token ids are fixed, the logits are not fed back).
+#include "ggml-backend.h"
+#include "llama.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+int main(int argc, char ** argv) {
+    if (argc != 6) {
+        fprintf(stderr, "usage: %s model.gguf n_gpu_layers n_prompt n_decode out.bin\n", argv[0]);
+        return 2;
+    }
+    const int ngl = atoi(argv[2]), n_prompt = atoi(argv[3]), n_decode = atoi(argv[4]);
+    ggml_backend_load_all();   // honours GGML_BACKEND_PATH, like the reference's example programs
+    llama_backend_init();
+    llama_model_params mp = llama_model_default_params();
+    mp.n_gpu_layers = ngl;
+    llama_model * model = llama_model_load_from_file(argv[1], mp);
+    if (!model) return 1;
+    llama_context_params cp = llama_context_default_params();
+    cp.n_ctx = 1024;
+    cp.n_batch = 512;
+    cp.n_ubatch = 512;
+    cp.flash_attn = true;
+    cp.n_threads = 8;
+    cp.n_threads_batch = 8;
+    llama_context * ctx = llama_init_from_model(model, cp);
+    if (!ctx) return 1;
+    const int n_vocab = llama_vocab_n_tokens(llama_model_get_vocab(model));
+    FILE * f = fopen(argv[5], "wb");
+    if (!f) return 1;
+    std::vector<llama_token> toks(n_prompt);
+    for (int i = 0; i < n_prompt; i++) toks[i] = (7 * i + 3) % n_vocab;
+    if (llama_decode(ctx, llama_batch_get_one(toks.data(), n_prompt)) != 0) return 1;
+    fwrite(llama_get_logits_ith(ctx, -1), sizeof(float), n_vocab, f);
+    for (int i = 0; i < n_decode; i++) {
+        llama_token t = (7 * (n_prompt + i) + 3) % n_vocab;
+        if (llama_decode(ctx, llama_batch_get_one(&t, 1)) != 0) return 1;
+        fwrite(llama_get_logits_ith(ctx, -1), sizeof(float), n_vocab, f);
+    }
+    fclose(f);
+    llama_free(ctx);
+    llama_model_free(model);
+    return 0;
+}
