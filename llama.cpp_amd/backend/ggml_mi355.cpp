@@ -91,6 +91,7 @@ struct act_cache {
     int64_t K = 0, B = 0;
     int format = 0;               // ACT_Q8_1 (32-element blocks, GEMV) or ACT_Q8K (256-element super-blocks, tile GEMM)
     bool valid = false;
+    void * ptr = nullptr;         // where the quantized form lives (one of the two slots of backend_ctx::act)
 };
 enum { ACT_Q8_1 = 1, ACT_Q8K = 2 };
 
@@ -104,6 +105,21 @@ struct backend_ctx {
     act_cache cache;
     bool fuse = true;      // MI355_NO_FUSION=1 executes the graph node for node
     int32_t * iota = nullptr;   // device {0, 1, 2, ...}: token t of a batch goes to row t of a KV-cache view
+    unsigned * tickets = nullptr;   // zeroed arrival counters of the gate/up launch (one per 32 output rows)
+    size_t n_tickets = 0;
+
+    unsigned * ticket_buffer(size_t n) {
+        if (n > n_tickets) {
+            if (tickets) {
+                MI355_HIP_OK(hipStreamSynchronize(stream));
+                MI355_HIP_OK(hipFree(tickets));
+            }
+            n_tickets = (n + 1023) & ~(size_t) 1023;
+            MI355_HIP_OK(hipMalloc((void **) &tickets, n_tickets * sizeof(unsigned)));
+            MI355_HIP_OK(hipMemset(tickets, 0, n_tickets * sizeof(unsigned)));   // every launch leaves them zero again
+        }
+        return tickets;
+    }
     std::string name;
 
     // a node is about to write [p, p + bytes): the cached activation dies if that touches the tensor it came from
@@ -114,17 +130,26 @@ struct backend_ctx {
         if (a0 < b1 && b0 < a1) cache.valid = false;
     }
 
-    void * act_buffer(size_t need) {
+    // two slots, so that a launch can read one quantized activation while it writes the next one
+    void act_reserve(size_t need) {
         if (need > act_size) {
             if (act) {
                 MI355_HIP_OK(hipStreamSynchronize(stream));
                 MI355_HIP_OK(hipFree(act));
             }
             act_size = (need + (size_t(4) << 20)) & ~((size_t(1) << 20) - 1);
-            MI355_HIP_OK(hipMalloc(&act, act_size));
+            MI355_HIP_OK(hipMalloc(&act, 2 * act_size));
             cache.valid = false;
         }
-        return act;
+    }
+    void * act_slot(size_t need, bool keep_cached = false) {   // keep_cached: pick the slot the valid cache does not occupy
+        act_reserve(need);
+        char * s0 = (char *) act, * s1 = s0 + act_size;
+        if (keep_cached && cache.valid && cache.ptr == s0) return s1;
+        return s0;
+    }
+    bool cached(const void * src, int64_t K, int64_t B, int format) const {
+        return cache.valid && cache.src == src && cache.K == K && cache.B == B && cache.format == format;
     }
 
     void * workspace(size_t need) {
@@ -559,6 +584,7 @@ void backend_free(ggml_backend_t backend) {
     if (ctx->ws) (void) hipFree(ctx->ws);
     if (ctx->act) (void) hipFree(ctx->act);
     if (ctx->iota) (void) hipFree(ctx->iota);
+    if (ctx->tickets) (void) hipFree(ctx->tickets);
     if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     delete backend;
@@ -676,9 +702,9 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             float eps;
             memcpy(&eps, node->op_params, sizeof(float));
             void * act = nullptr;
-            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_buffer(mi355_act_bytes(K, rows));
+            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
             MI355_K_OK(mi355_rms_norm_mul_quant(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
-            ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr};
+            ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
             return j;
         }
     }
@@ -691,9 +717,9 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         if (ggml_is_contiguous(gt) && ggml_is_contiguous(up) && ggml_is_contiguous(nxt) && ggml_are_same_shape(gt, up) && up->type == GGML_TYPE_F32 &&
             K % 32 == 0 && rows <= 65535 && (((uintptr_t) gt->data | (uintptr_t) up->data | (uintptr_t) nxt->data) & 15) == 0) {
             void * act = nullptr;
-            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_buffer(mi355_act_bytes(K, rows));
+            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
             MI355_K_OK(mi355_swiglu_quant(s, (const float *) gt->data, (const float *) up->data, K, (float *) nxt->data, K, act, K, rows));
-            ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr};
+            ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
             return j;
         }
     }
@@ -713,12 +739,45 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             const size_t full = mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq);
             const size_t ws_bytes = full < (size_t(256) << 20) ? full : (size_t(256) << 20);
             void * ws = ctx->workspace(ws_bytes);
-            void * act = ctx->act_buffer(mi355_act_bytes(Hq * D, Nq));
+            void * act = ctx->act_slot(mi355_act_bytes(Hq * D, Nq));
             MI355_K_OK(mi355_flash_attn_ext_quant(s, (const float *) q->data, k->data, v->data, mask ? mask->data : nullptr, (float *) node->data, D, Nq, Nkv,
                                                   Hq, Hkv, q->nb[1], q->nb[2], k->nb[1], k->nb[2], v->nb[1], v->nb[2], mask ? mask->nb[1] : 0, scale,
                                                   max_bias, softcap, ws, ws_bytes, act));
-            ctx->cache = act_cache{node->data, Hq * D, Nq, ACT_Q8_1, true};
+            ctx->cache = act_cache{node->data, Hq * D, Nq, ACT_Q8_1, true, act};
             return i;
+        }
+    }
+    // ---- MUL_MAT(gate) -> UNARY(SILU) -> MUL_MAT(up) -> MUL -> [quantized MUL_MAT]: one launch that also leaves the Q8_1 form
+    //      of silu(gate)*up for ffn_down; the f32 product is not materialised (its only reader takes the quantized form)
+    if (is_quant_gemv_candidate(node) && node->src[1]->ne[1] <= 4 && w.sole_use(i) && nxt && nxt->op == GGML_OP_UNARY &&
+        ggml_get_unary_op(nxt) == GGML_UNARY_OP_SILU && nxt->src[0] == node && w.sole_use(j)) {
+        const int ju = w.next(j);
+        const int jm = ju < w.n ? w.next(ju) : w.n;
+        if (jm < w.n) {
+            const ggml_tensor * up = w.nodes[ju];
+            const ggml_tensor * mul = w.nodes[jm];
+            const ggml_tensor * b = node->src[1];
+            const int64_t K = b->ne[0], B = b->ne[1], N = node->ne[0];
+            const bool mul_ok = mul->op == GGML_OP_MUL && ((mul->src[0] == nxt && mul->src[1] == up) || (mul->src[1] == nxt && mul->src[0] == up)) &&
+                                ggml_is_contiguous(mul) && mul->type == GGML_TYPE_F32 && ggml_are_same_shape(mul, node);
+            if (mul_ok && is_quant_gemv_candidate(up) && up->src[1]->data == b->data && up->src[1]->ne[0] == K && up->src[1]->ne[1] == B &&
+                up->ne[0] == N && w.sole_use(ju) && w.sole_use(jm) && N % 32 == 0 && ggml_is_contiguous(node) && ggml_is_contiguous(up) &&
+                feeds_quant_gemv(w, jm, mul->data, N, B)) {
+                // this launch reads one quantized activation and writes the next: the two slots
+                const size_t in_bytes = mi355_act_bytes(K, B), out_bytes = mi355_act_bytes(N, B);
+                ctx->act_reserve(in_bytes > out_bytes ? in_bytes : out_bytes);
+                if (!ctx->cached(b->data, K, B, ACT_Q8_1)) {
+                    void * fresh = ctx->act_slot(in_bytes);
+                    MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
+                    ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
+                }
+                const void * act_in = ctx->cache.ptr;
+                void * act_out = ctx->act_slot(out_bytes, true);
+                MI355_K_OK(mi355_ffn_gate_up_swiglu(s, to_mi355_type(node->src[0]->type), node->src[0]->data, to_mi355_type(up->src[0]->type), up->src[0]->data,
+                                                    act_in, (float *) node->data, (float *) up->data, N, act_out, ctx->ticket_buffer((size_t) (N / 32)), N, K, B));
+                ctx->cache = act_cache{mul->data, N, B, ACT_Q8_1, true, act_out};
+                return jm;
+            }
         }
     }
     // ---- MUL_MAT -> [RESHAPE] -> ROPE [-> CPY to an f16 view]   and   MUL_MAT -> CPY to an f16 view   (decode, batch <= 4)
@@ -792,12 +851,12 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             last = j;
         }
         if (last >= 0) {
-            void * act = ctx->act_buffer(mi355_act_bytes(K, B));
-            if (!(ctx->cache.valid && ctx->cache.src == b->data && ctx->cache.K == K && ctx->cache.B == B && ctx->cache.format == ACT_Q8_1)) {
-                MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, act, K, B, K));
-                ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true};
+            if (!ctx->cached(b->data, K, B, ACT_Q8_1)) {
+                void * fresh = ctx->act_slot(mi355_act_bytes(K, B));
+                MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
+                ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
             }
-            MI355_K_OK(mi355_mul_mat_vec_q_rope(s, 1, &m, act, K, B, &rd));
+            MI355_K_OK(mi355_mul_mat_vec_q_rope(s, 1, &m, ctx->cache.ptr, K, B, &rd));
             ctx->note_write(m.dst, (size_t) N * (size_t) B * (m.epilogue == MI355_EPI_ROPE ? sizeof(float) : 2));
             return last;
         }
@@ -813,11 +872,12 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             run[n_run++] = k;
             last = k;
         }
-        void * act = ctx->act_buffer(mi355_act_bytes(K, B));
-        if (!(ctx->cache.valid && ctx->cache.src == b->data && ctx->cache.K == K && ctx->cache.B == B && ctx->cache.format == ACT_Q8_1)) {
-            MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, act, K, B, K));
-            ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true};
+        if (!ctx->cached(b->data, K, B, ACT_Q8_1)) {
+            void * fresh = ctx->act_slot(mi355_act_bytes(K, B));
+            MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
+            ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
         }
+        const void * act = ctx->cache.ptr;
         mi355_gemv_mat mats[4];
         for (int r = 0; r < n_run; r++) {
             ggml_tensor * mm = (ggml_tensor *) w.nodes[run[r]];
@@ -850,12 +910,12 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     if (is_q8k_tile_candidate(node)) {
         const ggml_tensor * b = node->src[1];
         const int64_t K = b->ne[0], B = b->ne[1];
-        void * act = ctx->act_buffer(mi355_act_q8k_bytes(K, B));
-        if (!(ctx->cache.valid && ctx->cache.src == b->data && ctx->cache.K == K && ctx->cache.B == B && ctx->cache.format == ACT_Q8K)) {
-            MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, act, K, B, (int64_t) (b->nb[1] / sizeof(float))));
-            ctx->cache = act_cache{b->data, K, B, ACT_Q8K, true};
+        if (!ctx->cached(b->data, K, B, ACT_Q8K)) {
+            void * fresh = ctx->act_slot(mi355_act_q8k_bytes(K, B));
+            MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
+            ctx->cache = act_cache{b->data, K, B, ACT_Q8K, true, fresh};
         }
-        MI355_K_OK(mi355_mul_mat_q8k(s, to_mi355_type(node->src[0]->type), node->src[0]->data, act, (float *) node->data, node->src[0]->ne[1], K, B,
+        MI355_K_OK(mi355_mul_mat_q8k(s, to_mi355_type(node->src[0]->type), node->src[0]->data, ctx->cache.ptr, (float *) node->data, node->src[0]->ne[1], K, B,
                                      (int64_t) (node->nb[1] / sizeof(float))));
         ctx->note_write(node->data, ggml_nbytes(node));
         return i;
