@@ -99,7 +99,7 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
 #pragma unroll
                 for (int r = 0; r < RPW; r++) {
                     const chunk_dots d = T::dots(w[r], A);
-                    acc[r][col] += T::combine(w[r], A, d);
+                    acc[r][col] = T::accumulate(acc[r][col], w[r], A, d);
                 }
             }
         }
@@ -112,7 +112,7 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
         float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
         for (int c = 0; c < NCOLS; c++) {
-            const float a0 = wave_sum(acc[0][c]), a1 = wave_sum(acc[1][c]);
+            const float a0 = wave_sum_dpp(acc[0][c]), a1 = wave_sum_dpp(acc[1][c]);
             if (lane == c) { s0 = a0; s1 = a1; }
         }
         if (lane < NCOLS && row0 + 1 < m.N) {
@@ -136,7 +136,7 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
         for (int r = 0; r < RPW; r++)
 #pragma unroll
             for (int c = 0; c < NCOLS; c++) {
-                const float s = wave_sum(acc[r][c]);
+                const float s = wave_sum_dpp(acc[r][c]);
                 if (lane == 0 && row0 + r < m.N) {
                     const int64_t o = c * m.dst_stride + row0 + r;
                     const float v = m.residual ? s + m.residual[o] : s;
@@ -194,7 +194,7 @@ __global__ void __launch_bounds__(256) k_gemv_multi(gemv_batch b, const int8_t *
 }
 
 // ---- a launch whose last-arriving groups also do the nodes that follow the product ------------
-// Every group stores its rows with device scope and waits for those stores (the barrier does), then
+// Every group stores its rows with device scope and waits for those stores (an explicit vmcnt wait), then
 // one thread takes a ticket from the counter of its 32-row block.  The group that draws the last
 // ticket of a block knows that all of the block's rows have been written, reads them back with
 // device-scope loads, finishes the follow-up nodes and re-arms the counter for the next launch.  No
@@ -243,7 +243,11 @@ __global__ void __launch_bounds__(256) k_gemv_gate_up(gemv_batch b, const int8_t
     const int i = g >= b.it[1].first_group ? 1 : 0;
     const int group = g - b.it[i].first_group;
     gemv_dispatch<NCOLS, 2, true>(b.it[i], group, aq, ads, K);
-    __syncthreads();   // waits for this group's stores, which were made with device scope
+    // Every wave waits until its device-scope stores have been acknowledged before it reaches the barrier: the
+    // barrier's own wait covers LDS and scalar loads only, and a ticket that overtakes a row store would let the
+    // last group read that row too early.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     const int block = group >> 2;   // 8 rows per group, 32 rows per quantization block
     if (threadIdx.x == 0) s_ticket = atomicAdd(t.counters + block, 1u);
     __syncthreads();

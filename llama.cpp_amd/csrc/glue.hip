@@ -323,6 +323,14 @@ int mi355_rms_norm(void *stream, const mi355_tensor *src, const mi355_tensor *ds
     const int64_t nr = nrows(src);
     if (nr == 0 || src->ne[0] == 0) return MI355_OK;
     MI355_REQUIRE(nr < 0x7fffffff, "rms_norm: too many rows");
+    // Rows of a contiguous tensor go through the kernel that the fused norm+weight+quantization launch uses, so that a
+    // graph run node for node and the same graph run fused sum the squares in the same order and agree bit for bit.
+    const int64_t n = src->ne[0];
+    auto packed = [n](const mi355_tensor *t) {
+        return t->nb[1] == n * 4 && t->nb[2] == t->nb[1] * t->ne[1] && t->nb[3] == t->nb[2] * t->ne[2] && ((uintptr_t)t->data & 15) == 0;
+    };
+    if (n % 32 == 0 && n <= 16384 && packed(src) && packed(dst))
+        return mi355_rms_norm_mul_quant(stream, (const float *)src->data, n, nullptr, (float *)dst->data, n, nullptr, n, nr, eps);
     hipLaunchKernelGGL(k_rms_norm, dim3((unsigned)nr), dim3(row_threads(src->ne[0])), 0, (hipStream_t)stream, to_tens(src), to_tens(dst), eps);
     return launch_status("k_rms_norm");
 }

@@ -63,6 +63,9 @@ struct chunk_dots {
     int i0, i1;
 };
 
+// wq<TYPE>::accumulate adds one chunk's contribution to a running sum.  Every multiply, add and fused
+// multiply-add is spelled out: left to the compiler, the choice of which product of a sum gets fused
+// differs between kernel instantiations, and launches that must agree bit for bit would not.
 template <int TYPE> struct wq;
 
 // ---------------------------------------------------------------- Q4_0
@@ -96,8 +99,8 @@ template <> struct wq<MI355_Q4_0> {
         chunk_dots r = {s - 8 * A.sum, 0};
         return r;
     }
-    static __device__ __forceinline__ float combine(const chunk &w, const act &A, const chunk_dots &r) {
-        return w.d * (A.d * (float)r.i0);
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        return __builtin_fmaf(w.d, __fmul_rn(A.d, (float)r.i0), acc);
     }
 };
 
@@ -132,8 +135,8 @@ template <> struct wq<MI355_Q8_0> {
         chunk_dots r = {s, 0};
         return r;
     }
-    static __device__ __forceinline__ float combine(const chunk &w, const act &A, const chunk_dots &r) {
-        return w.d * (A.d * (float)r.i0);
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        return __builtin_fmaf(w.d, __fmul_rn(A.d, (float)r.i0), acc);
     }
 };
 
@@ -193,10 +196,10 @@ template <> struct wq<MI355_Q4_K> {
         chunk_dots r = {sA, sB};
         return r;
     }
-    static __device__ __forceinline__ float combine(const chunk &w, const act &A, const chunk_dots &r) {
-        const float pos = w.scA * (A.d0 * (float)r.i0) + w.scB * (A.d1 * (float)r.i1);
-        const float neg = w.mA * A.ds0 + w.mB * A.ds1;
-        return w.d * pos - w.dmin * neg;
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        const float pos = __builtin_fmaf(w.scA, __fmul_rn(A.d0, (float)r.i0), __fmul_rn(w.scB, __fmul_rn(A.d1, (float)r.i1)));
+        const float neg = __builtin_fmaf(w.mA, A.ds0, __fmul_rn(w.mB, A.ds1));
+        return __fadd_rn(acc, __builtin_fmaf(w.d, pos, -__fmul_rn(w.dmin, neg)));
     }
 };
 
@@ -251,8 +254,9 @@ template <> struct wq<MI355_Q6_K> {
         chunk_dots r = {sA - 32 * A.s0, sB - 32 * A.s1};
         return r;
     }
-    static __device__ __forceinline__ float combine(const chunk &w, const act &A, const chunk_dots &r) {
-        return w.d * (w.scA * (A.d0 * (float)r.i0) + w.scB * (A.d1 * (float)r.i1));
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        const float t = __builtin_fmaf(w.scA, __fmul_rn(A.d0, (float)r.i0), __fmul_rn(w.scB, __fmul_rn(A.d1, (float)r.i1)));
+        return __builtin_fmaf(w.d, t, acc);
     }
 };
 
