@@ -137,6 +137,16 @@ int mi355_mul_mat_id(void *stream, int type, const void *as, const float *b, con
                      float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T,
                      void *ws, size_t ws_bytes);
 
+/* mi355_mul_mat_id for many (token, expert slot) pairs and K-quant experts: the slots are sorted by expert on the
+ * device (the row grouping of ggml_compute_forward_mul_mat_id, ggml/src/ggml-cpu/ggml-cpu.c:7805-7820, mmid_row_mapping
+ * :7639-7644) and one tile launch walks all experts, so every expert's matrix is read once.  `act` holds the nb1*T rows
+ * of b in the mi355_quantize_act_q8k layout; route_ws: at least mi355_mul_mat_id_q8k_route_bytes(...) bytes, 16-byte
+ * aligned.  At most 256 experts; mi355_mul_mat_id picks this path from 32 slots on. */
+size_t mi355_mul_mat_id_q8k_route_bytes(int64_t n_expert, int64_t n_used, int64_t T);
+int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride, float *dst,
+                         int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws,
+                         size_t route_ws_bytes);
+
 /* Second half of mi355_mul_mat_id: `act` holds the nb1*T rows of b quantized by
  * mi355_quantize_act (row t*nb1 + j). */
 int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride,

@@ -115,7 +115,7 @@ struct kq_smem {
 
 template <int TYPE, int WI, int AI>
 __device__ __forceinline__ void kq_fetch(kq_regs<TYPE, WI, AI> &R, const uint8_t *__restrict__ W, const row_layout &L, int64_t row0, int64_t N,
-                                         const int8_t *__restrict__ aq, int64_t col0, int64_t B, int64_t K, int64_t k0) {
+                                         const int8_t *__restrict__ aq, const int (&arow)[AI], int64_t K, int64_t k0) {
     const int tid = threadIdx.x;
     const int64_t sb = k0 >> 8;
     const int half = (int)((k0 >> 7) & 1);
@@ -142,11 +142,21 @@ __device__ __forceinline__ void kq_fetch(kq_regs<TYPE, WI, AI> &R, const uint8_t
 #pragma unroll
     for (int it = 0; it < AI; it++) {
         const int idx = tid + it * 256;
-        const int r = idx >> 3, c = idx & 7;
-        const int64_t col = col0 + r < B ? col0 + r : B - 1;
-        R.a[it] = load16(aq + col * K + k0 + c * 16);
+        const int c = idx & 7;
+        R.a[it] = load16(aq + (int64_t)arow[it] * K + k0 + c * 16);
     }
 }
+
+// Routing of a MUL_MAT_ID launch (semantics ggml/src/ggml.c:2723-2759): the (token, expert slot) pairs sorted by expert.
+// Column c of the sorted list reads activation row act_row[c] and writes dst row dst_row[c]; every column tile
+// belongs to one expert: tiles[4*i] = {expert, first column, end column, 0}.
+struct mmq_route {
+    const int32_t *act_row;
+    const int32_t *dst_row;
+    const int32_t *tiles;
+    const int32_t *n_tiles;        // number of column tiles in use (device value)
+    int64_t expert_bytes;          // bytes from one expert's matrix to the next
+};
 
 // 4 packed bytes (each <= 15) times a small factor (<= 7): no byte overflows, so two 16-bit multiplies do it
 __device__ __forceinline__ u32 mul_bytes(u32 x, u32 f) {
@@ -241,11 +251,11 @@ __device__ __forceinline__ void kq_commit(const kq_regs<TYPE, WI, AI> &R, const 
 }
 
 // TW x TB: 32 x 32 MFMA tiles per wave along the weight / activation rows; waves are 2 x 2
-template <int TYPE, int TW, int TB, int OCC>
+template <int TYPE, int TW, int TB, int OCC, bool ID>
 __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq, const float *__restrict__ ad8,
                                                     const _Float16 *__restrict__ abs_, float *__restrict__ dst, int64_t N, int64_t K,
                                                     int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles, int n_groups,
-                                                    int n_groups_padded) {
+                                                    int n_groups_padded, mmq_route route) {
     constexpr bool Q4 = TYPE == MI355_Q4_K;
     constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
     constexpr int BM = 64 * TW, BN = 64 * TB;
@@ -265,7 +275,14 @@ __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ 
     const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
     if (lid >= n_groups) return;
     const int64_t row0 = (int64_t)(lid / n_col_tiles) * BM;
-    const int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+    int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+    if constexpr (ID) {   // the grid covers the worst case; B becomes the end of this expert's columns
+        const int ct = lid % n_col_tiles;
+        if (ct >= *route.n_tiles) return;
+        W += (int64_t)route.tiles[4 * ct] * route.expert_bytes;
+        col0 = route.tiles[4 * ct + 1];
+        B = route.tiles[4 * ct + 2];
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -282,8 +299,22 @@ __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[tb][tw][r] = 0.0f;
 
+    // activation rows of this thread's staging pieces, and of the column whose scales it copies
+    int arow[AI];
+#pragma unroll
+    for (int it = 0; it < AI; it++) {
+        const int r = (tid + it * 256) >> 3;
+        const int64_t col = col0 + r < B ? col0 + r : B - 1;
+        arow[it] = ID ? route.act_row[col] : (int)col;
+    }
+    int srow = 0;
+    if (tid < BN) {
+        const int64_t col = col0 + tid < B ? col0 + tid : B - 1;
+        srow = ID ? route.act_row[col] : (int)col;
+    }
+
     kq_regs<TYPE, WI, AI> R;
-    kq_fetch<TYPE, WI, AI>(R, W, L, row0, N, aq, col0, B, K, 0);
+    kq_fetch<TYPE, WI, AI>(R, W, L, row0, N, aq, arow, K, 0);
 
     for (int64_t sb = 0; sb < nsb; sb++) {
         i32x16 hi[TB][TW], lo[TB][TW];
@@ -293,16 +324,15 @@ __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ 
             __syncthreads();   // everyone is done reading the previous stage
             kq_commit<TYPE, WI, AI>(R, S, half);
             if (half == 0 && tid < BN) {   // per super-block activation scale and sub-block sums
-                const int64_t col = col0 + tid < B ? col0 + tid : B - 1;
-                sAd[tid] = ad8[col * nsb + sb];
+                sAd[tid] = ad8[(int64_t)srow * nsb + sb];
                 if constexpr (Q4) {
-                    const u32x4 *src = (const u32x4 *)(abs_ + (col * nsb + sb) * 16);
+                    const u32x4 *src = (const u32x4 *)(abs_ + ((int64_t)srow * nsb + sb) * 16);
                     *(u32x4 *)(sAb + tid * 16) = src[0];
                     *(u32x4 *)(sAb + tid * 16 + 8) = src[1];
                 }
             }
             __syncthreads();
-            if (k0 + KQ_BK < K) kq_fetch<TYPE, WI, AI>(R, W, L, row0, N, aq, col0, B, K, k0 + KQ_BK);
+            if (k0 + KQ_BK < K) kq_fetch<TYPE, WI, AI>(R, W, L, row0, N, aq, arow, K, k0 + KQ_BK);
 
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
@@ -374,7 +404,7 @@ __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ 
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                if (n < N && b < B) dst[b * dst_stride + n] = acc[tb][tw][r];
+                if (n < N && b < B) dst[(ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n] = acc[tb][tw][r];
             }
         }
 }
@@ -391,8 +421,85 @@ static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *d
     const int n_col_tiles = (int)((B + BN - 1) / BN);
     const int n_groups = n_row_tiles * n_col_tiles;
     const int n_groups_padded = (n_groups + 7) & ~7;
-    hipLaunchKernelGGL((k_mmq_k<TYPE, TW, TB, OCC>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_,
-                       dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded);
+    hipLaunchKernelGGL((k_mmq_k<TYPE, TW, TB, OCC, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_,
+                       dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
+}
+
+// ---- MUL_MAT_ID with many slots: sort the slots by expert, then one tile launch over all experts ----
+constexpr int ROUTE_MAX_EXPERTS = 256;
+
+// One 1024-thread group.  Slot s = t * n_used + e reads activation row t * nb1 + e % nb1 and writes dst row s
+// (ggml_compute_forward_mul_mat_id, ggml-cpu.c:7717-7895).  The order of the slots inside an expert depends on
+// atomic arrival, the result of every slot does not.
+__global__ void __launch_bounds__(1024) k_route_slots(const int32_t *__restrict__ ids, int64_t ids_stride, int64_t n_expert, int64_t n_used,
+                                                      int64_t nb1, int64_t T, int bn, int32_t *__restrict__ act_row,
+                                                      int32_t *__restrict__ dst_row, int32_t *__restrict__ tiles, int32_t *__restrict__ n_tiles) {
+    __shared__ int cnt[ROUTE_MAX_EXPERTS], first[ROUTE_MAX_EXPERTS], cursor[ROUTE_MAX_EXPERTS];
+    const int tid = threadIdx.x;
+    const int64_t S = T * n_used;
+    for (int i = tid; i < n_expert; i += 1024) { cnt[i] = 0; cursor[i] = 0; }
+    __syncthreads();
+    for (int64_t sl = tid; sl < S; sl += 1024) {
+        int64_t ex = ids[(sl / n_used) * ids_stride + sl % n_used];
+        ex = ex < 0 ? 0 : (ex >= n_expert ? n_expert - 1 : ex);
+        atomicAdd(&cnt[ex], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int col = 0, nt = 0;
+        for (int ex = 0; ex < n_expert; ex++) {
+            first[ex] = col;
+            for (int c = 0; c < cnt[ex]; c += bn, nt++) {
+                tiles[4 * nt] = ex;
+                tiles[4 * nt + 1] = col + c;
+                tiles[4 * nt + 2] = col + cnt[ex];
+                tiles[4 * nt + 3] = 0;
+            }
+            col += cnt[ex];
+        }
+        *n_tiles = nt;
+    }
+    __syncthreads();
+    for (int64_t sl = tid; sl < S; sl += 1024) {
+        const int64_t t = sl / n_used, e = sl % n_used;
+        int64_t ex = ids[t * ids_stride + e];
+        ex = ex < 0 ? 0 : (ex >= n_expert ? n_expert - 1 : ex);
+        const int pos = first[ex] + atomicAdd(&cursor[ex], 1);
+        act_row[pos] = (int32_t)(t * nb1 + e % nb1);
+        dst_row[pos] = (int32_t)sl;
+    }
+}
+
+// column tile of the routed launch: 64 while the experts see few slots each, 128 beyond
+__host__ inline int route_bn(int64_t n_expert, int64_t S) { return S <= 48 * n_expert ? 64 : 128; }
+__host__ inline size_t route_max_tiles(int64_t n_expert, int64_t S) { return (size_t)((S + 63) / 64 + n_expert); }
+__host__ inline size_t route_bytes(int64_t n_expert, int64_t S) {
+    const size_t max_tiles = route_max_tiles(n_expert, S);
+    return (2 * (size_t)S + 4 * max_tiles + 4) * sizeof(int32_t);
+}
+
+template <int TYPE>
+static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int64_t act_rows, const int32_t *ids, int64_t ids_stride,
+                            float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws) {
+    const int64_t S = T * n_used;
+    const int bn = route_bn(n_expert, S);
+    const int max_tiles = (int)((S + bn - 1) / bn + n_expert);
+    int32_t *act_row = (int32_t *)route_ws, *dst_row = act_row + S, *tiles = dst_row + S, *n_tiles = tiles + 4 * (int64_t)route_max_tiles(n_expert, S);
+    hipLaunchKernelGGL(k_route_slots, dim3(1), dim3(1024), 0, s, ids, ids_stride, n_expert, n_used, nb1, T, bn, act_row, dst_row, tiles, n_tiles);
+    const row_layout L = make_row_layout(TYPE, K);
+    const int8_t *aq = (const int8_t *)act;
+    const float *ad8 = (const float *)(aq + q8k_d_offset(K, act_rows));
+    const _Float16 *abs_ = (const _Float16 *)(aq + q8k_bs_offset(K, act_rows));
+    const int n_row_tiles = (int)((N + 63) / 64);
+    const int n_groups = n_row_tiles * max_tiles;
+    const int n_groups_padded = (n_groups + 7) & ~7;
+    const mmq_route route = {act_row, dst_row, tiles, n_tiles, N * L.row_bytes};
+    if (bn == 64)
+        hipLaunchKernelGGL((k_mmq_k<TYPE, 1, 1, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
+                           dst, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
+    else
+        hipLaunchKernelGGL((k_mmq_k<TYPE, 1, 2, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
+                           dst, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
 }
 
 // 64 x 128 tiles: 96 accumulator registers per lane leave room for two groups per CU, which
@@ -426,6 +533,33 @@ int mi355_quantize_act_q8k(void *stream, const float *x, void *act, int64_t k, i
     const dim3 grid((unsigned)((k / QKK + 3) / 4), (unsigned)nrows);
     hipLaunchKernelGGL(k_quantize_q8k, grid, dim3(256), 0, (hipStream_t)stream, x, q, d8, bs, k, x_stride);
     return launch_status("k_quantize_q8k");
+}
+
+size_t mi355_mul_mat_id_q8k_route_bytes(int64_t n_expert, int64_t n_used, int64_t T) {
+    if (n_expert <= 0 || n_used <= 0 || T <= 0) return 0;
+    return (route_bytes(n_expert, T * n_used) + 255) & ~(size_t)255;
+}
+
+int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride, float *dst,
+                         int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws,
+                         size_t route_ws_bytes) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_id_q8k: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(N > 0 && K > 0 && n_expert > 0 && n_used > 0 && nb1 > 0 && T > 0, "mul_mat_id_q8k: bad shape");
+    MI355_REQUIRE(K % QKK == 0, "mul_mat_id_q8k: K=%lld is not a multiple of 256", (long long)K);
+    MI355_REQUIRE(n_expert <= ROUTE_MAX_EXPERTS, "mul_mat_id_q8k: more than %d experts", ROUTE_MAX_EXPERTS);
+    MI355_REQUIRE(ids_stride >= n_used, "mul_mat_id_q8k: ids_stride < n_used");
+    MI355_REQUIRE(T * n_used < (1 << 24) && nb1 * T < (1 << 24), "mul_mat_id_q8k: too many slots");
+    const row_layout L = make_row_layout(type, K);
+    MI355_REQUIRE(layout_aligned(as, L) && (N * L.row_bytes) % 16 == 0, "mul_mat_id_q8k: weight rows are not 16-byte aligned (K=%lld)", (long long)K);
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0 && (q8k_d_offset(K, nb1 * T) & 15) == 0, "mul_mat_id_q8k: activation workspace is not 16-byte aligned");
+    if (route_ws == nullptr || route_ws_bytes < route_bytes(n_expert, T * n_used) || ((uintptr_t)route_ws & 15) != 0) {
+        set_error("mul_mat_id_q8k: routing workspace of %zu bytes, need %zu (16-byte aligned)", route_ws_bytes, route_bytes(n_expert, T * n_used));
+        return MI355_ERR_WORKSPACE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (type == MI355_Q4_K) launch_mmq_k_id<MI355_Q4_K>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
+    else launch_mmq_k_id<MI355_Q6_K>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
+    return launch_status("k_mmq_k (routed)");
 }
 
 int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,

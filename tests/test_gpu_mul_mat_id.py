@@ -8,8 +8,30 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("name,t", list(orc.WEIGHT_TYPES.items()))
+def routed(t, n_used, T, K):
+    """mi355_mul_mat_id sorts the slots by expert and uses the K-quant tile kernel (ggml-cpu's Q8_K arithmetic)"""
+    return T * n_used >= 32 and ((t == orc.Q4_K and K % 256 == 0) or (t == orc.Q6_K and K % 2048 == 0))
+
+
+def expected_per_expert(kind, t, Wq, b, ids_full, n_expert, n_used, nb1, N):
+    """every expert's product over the rows routed to it (ggml.c:2723-2759), one mul_mat per expert"""
+    T = b.shape[0]
+    want = np.zeros((T, n_used, N), dtype=np.float32)
+    for ex in range(n_expert):
+        where = [(tt, e) for tt in range(T) for e in range(n_used) if ids_full[tt, e] == ex]
+        if not where:
+            continue
+        rows = np.stack([b[tt, e % nb1] for tt, e in where])
+        out = orc.mul_mat(kind, t, Wq[ex * N:(ex + 1) * N], rows)
+        for (tt, e), o in zip(where, out):
+            want[tt, e] = o
+    return want
+
+
+@pytest.mark.parametrize("name,t", list(orc.WEIGHT_TYPES.items()))
 @pytest.mark.parametrize("n_expert,n_used,nb1_bcast,T,N,K", [(8, 2, True, 1, 512, 4096), (8, 2, False, 5, 256, 2048),
-                                                              (4, 4, True, 32, 128, 2048), (8, 1, False, 3, 64, 4096)])
+                                                              (4, 4, True, 32, 128, 2048), (8, 1, False, 3, 64, 4096),
+                                                              (8, 2, True, 512, 192, 2048), (8, 2, False, 300, 64, 4096)])
 def test_mul_mat_id(dev, name, t, n_expert, n_used, nb1_bcast, T, N, K):
     import torch
     import mi355
@@ -22,12 +44,39 @@ def test_mul_mat_id(dev, name, t, n_expert, n_used, nb1_bcast, T, N, K):
     Wd = mi355.upload_weights(t, torch.from_numpy(Wq).to(dev)).reshape(n_expert, N, -1)
     idd = torch.from_numpy(ids_full).to(dev)[:, :n_used]          # strided view, as ggml_view of the argsort result
     got = mi355.mul_mat_id(t, Wd, torch.from_numpy(b).to(dev), idd, n_used).cpu().numpy()
-    want = np.zeros((T, n_used, N), dtype=np.float32)
-    assert orc.oracle.orc_mul_mat_id_q8_1(t, orc._ptr(Wq), orc._ptr(b), orc._ptr(ids_full), n_expert, orc._ptr(want), N, K,
-                                          n_expert, n_used, nb1, T) == 0
+    if routed(t, n_used, T, K):
+        want = expected_per_expert("cpu", t, Wq, b, ids_full, n_expert, n_used, nb1, N)
+    else:
+        want = np.zeros((T, n_used, N), dtype=np.float32)
+        assert orc.oracle.orc_mul_mat_id_q8_1(t, orc._ptr(Wq), orc._ptr(b), orc._ptr(ids_full), n_expert, orc._ptr(want), N, K,
+                                              n_expert, n_used, nb1, T) == 0
     assert orc.nmse(got, want) < 1e-9
     if orc.ref is not None:
         cpu = np.zeros_like(want)
         assert orc.ref.ref_mul_mat_id(t, orc._ptr(Wq), orc._ptr(b), orc._ptr(ids_full), orc._ptr(cpu), N, K, n_expert, n_used,
                                       nb1, T, 4, 0) >= 0
         assert orc.nmse(got, cpu) <= 5e-4      # tests/test-backend-ops.cpp:2001
+
+
+@pytest.mark.parametrize("name,t", [("q4_k", orc.Q4_K), ("q6_k", orc.Q6_K)])
+@pytest.mark.parametrize("pattern", ["one_expert", "two_of_eight", "out_of_range"])
+def test_mul_mat_id_skewed_routing(dev, name, t, pattern):
+    """experts with no slots, one expert with more slots than a column tile, ids outside [0, n_expert) clamped like the GEMV path"""
+    import torch
+    import mi355
+    n_expert, n_used, T, N, K = 8, 2, 200, 128, 2048
+    rng = np.random.default_rng(5)
+    Wf = (rng.standard_normal((n_expert * N, K)) * 0.02).astype(np.float32)
+    Wq = orc.quantize("ref" if orc.ref is not None else "oracle", t, Wf)
+    b = rng.standard_normal((T, 1, K)).astype(np.float32)
+    if pattern == "one_expert":
+        ids = np.full((T, n_expert), 3, dtype=np.int32)
+    elif pattern == "two_of_eight":
+        ids = np.tile(np.array([[6, 1, 0, 0, 0, 0, 0, 0]], dtype=np.int32), (T, 1))
+    else:
+        ids = rng.integers(-2, n_expert + 2, size=(T, n_expert)).astype(np.int32)
+    Wd = mi355.upload_weights(t, torch.from_numpy(Wq).to(dev)).reshape(n_expert, N, -1)
+    idd = torch.from_numpy(ids).to(dev)[:, :n_used]
+    got = mi355.mul_mat_id(t, Wd, torch.from_numpy(b).to(dev), idd, n_used).cpu().numpy()
+    want = expected_per_expert("cpu", t, Wq, b, np.clip(ids, 0, n_expert - 1), n_expert, n_used, 1, N)
+    assert orc.nmse(got, want) < 1e-9
