@@ -44,11 +44,25 @@ def _kv(key, vtype, value):
     raise ValueError(vtype)
 
 
-def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab):
+def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert=0):
+    """n_expert > 0: mixture-of-experts feed-forward (src/llama-model.cpp:1553-1558) with every quantized tensor Q4_K, the mix
+    of `llama-quantize --pure ... Q4_K`; the router ffn_gate_inp stays f32 (src/llama-quant.cpp:749)"""
     t = [("token_embd.weight", Q4_K, (n_embd, n_vocab))]
     for il in range(n_layer):
-        more = use_more_bits(il, n_layer)
+        more = use_more_bits(il, n_layer) and n_expert == 0
         p = "blk.%d." % il
+        if n_expert > 0:
+            t += [(p + "attn_norm.weight", F32, (n_embd,)),
+                  (p + "attn_q.weight", Q4_K, (n_embd, n_head * head_dim)),
+                  (p + "attn_k.weight", Q4_K, (n_embd, n_head_kv * head_dim)),
+                  (p + "attn_v.weight", Q4_K, (n_embd, n_head_kv * head_dim)),
+                  (p + "attn_output.weight", Q4_K, (n_head * head_dim, n_embd)),
+                  (p + "ffn_norm.weight", F32, (n_embd,)),
+                  (p + "ffn_gate_inp.weight", F32, (n_embd, n_expert)),
+                  (p + "ffn_gate_exps.weight", Q4_K, (n_embd, n_ff, n_expert)),
+                  (p + "ffn_down_exps.weight", Q4_K, (n_ff, n_embd, n_expert)),
+                  (p + "ffn_up_exps.weight", Q4_K, (n_embd, n_ff, n_expert))]
+            continue
         t += [(p + "attn_norm.weight", F32, (n_embd,)),
               (p + "attn_q.weight", Q4_K, (n_embd, n_head * head_dim)),
               (p + "attn_k.weight", Q4_K, (n_embd, n_head_kv * head_dim)),
@@ -58,7 +72,7 @@ def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab):
               (p + "ffn_gate.weight", Q4_K, (n_embd, n_ff)),
               (p + "ffn_up.weight", Q4_K, (n_embd, n_ff)),
               (p + "ffn_down.weight", Q6_K if more else Q4_K, (n_ff, n_embd))]
-    t += [("output_norm.weight", F32, (n_embd,)), ("output.weight", Q6_K, (n_embd, n_vocab))]
+    t += [("output_norm.weight", F32, (n_embd,)), ("output.weight", Q4_K if n_expert > 0 else Q6_K, (n_embd, n_vocab))]
     return t
 
 
@@ -94,9 +108,9 @@ def random_blocks(ttype, n_blocks, rng, pool):
 
 
 def write_model(path, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=128256, n_ctx=8192,
-                rope_theta=500000.0, rms_eps=1e-5, seed=1234):
+                rope_theta=500000.0, rms_eps=1e-5, seed=1234, n_expert=0, n_expert_used=0):
     head_dim = n_embd // n_head
-    tensors = tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab)
+    tensors = tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert)
     align = 32
     kvs = [
         _kv("general.architecture", T_STR, "llama"),
@@ -115,6 +129,8 @@ def write_model(path, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=
         _kv("llama.vocab_size", T_U32, n_vocab),
         _kv("tokenizer.ggml.model", T_STR, "no_vocab"),
     ]
+    if n_expert > 0:
+        kvs += [_kv("llama.expert_count", T_U32, n_expert), _kv("llama.expert_used_count", T_U32, n_expert_used)]
     infos, off = [], 0
     for name, ttype, shape in tensors:
         infos.append(_s(name) + struct.pack("<I", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape) +
@@ -128,7 +144,10 @@ def write_model(path, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=
         f.write(b"\0" * ((-len(header)) % align))
         for name, ttype, shape in tensors:
             if ttype == F32:
-                data = (1.0 + 0.01 * rng.standard_normal(int(np.prod(shape)))).astype(np.float32).tobytes()
+                if len(shape) == 1:   # norm weights
+                    data = (1.0 + 0.01 * rng.standard_normal(int(np.prod(shape)))).astype(np.float32).tobytes()
+                else:                 # router
+                    data = (0.02 * rng.standard_normal(int(np.prod(shape)))).astype(np.float32).tobytes()
                 f.write(data)
                 f.write(b"\0" * ((-len(data)) % align))
                 continue
@@ -151,6 +170,9 @@ if __name__ == "__main__":
     ap.add_argument("--heads", type=int, default=32)
     ap.add_argument("--kv-heads", type=int, default=8)
     ap.add_argument("--vocab", type=int, default=128256)
+    ap.add_argument("--experts", type=int, default=0, help="mixture of experts: number of experts (0 = dense)")
+    ap.add_argument("--experts-used", type=int, default=2)
     a = ap.parse_args()
-    size = write_model(a.path, a.layers, a.embd, a.ff, a.heads, a.kv_heads, a.vocab)
+    size = write_model(a.path, a.layers, a.embd, a.ff, a.heads, a.kv_heads, a.vocab, n_expert=a.experts,
+                       n_expert_used=a.experts_used if a.experts else 0)
     print("wrote %s: %.2f GB of tensor data" % (a.path, size / 1e9))

@@ -87,3 +87,23 @@ def test_model_logits_cpu_vs_plugin_and_fused_vs_nodes(dev, tmp_path, n_prompt):
     assert orc.nmse(fused, nodes) < (1e-6 if n_prompt <= 8 else 5e-4)
     assert orc.nmse(nodes, cpu) < 2e-3
     assert orc.nmse(fused, cpu) < 2e-3
+
+
+@pytest.mark.parametrize("n_prompt", [3, 48])
+def test_moe_model_logits_cpu_vs_plugin(dev, tmp_path, n_prompt):
+    """Mixture-of-experts llama (8 experts, 2 used, Q4_K experts, f32 router): the router, top-k selection, MUL_MAT_ID (per-slot
+    GEMV for a few slots, slots sorted by expert for many) and the weighted sum all run on the plug-in and reproduce the
+    reference CPU backend's logits.  A token whose router scores nearly tie can pick a different expert on the two backends;
+    the weights' scale makes such ties unlikely and the tolerance is that of the dense test."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / "moe.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=2048, n_head=16, n_head_kv=4, n_vocab=2048, n_expert=8, n_expert_used=2)
+    cpu = _logits(model, 0, n_prompt, 4, str(tmp_path / "cpu.bin"))
+    gpu = _logits(model, 99, n_prompt, 4, str(tmp_path / "gpu.bin"))
+    assert cpu.shape == gpu.shape and np.isfinite(gpu).all()
+    assert orc.nmse(gpu, cpu) < 2e-3
