@@ -281,6 +281,21 @@ int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, c
 int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, int type_up, const void *w_up, const void *act, float *gate,
                              float *up, int64_t out_stride, void *act_out, unsigned *counters, int64_t N, int64_t K, int64_t B);
 
+/* Mixture-of-experts glue of llm_build_moe_ffn (src/llama.cpp:417-530), each call the work of the consecutive graph nodes named,
+ * writing every tensor those nodes write, bit-identical to running them one by one.  All operands contiguous.
+ * moe_route: SOFT_MAX (no mask, scale 1) then ARGSORT descending: logits f32 [T][n_expert] -> probs f32, order i32 (ties by index;
+ *   ggml-cpu.c:8959-9055, 10857).  n_expert <= 64.
+ * moe_weights: GET_ROWS of the selected experts' probabilities, SUM_ROWS, DIV (ggml-cpu.c:8590, 5678, 5236-5305):
+ *   ids i32 [T][ids_stride] (first n_used of each row) -> raw f32 [T][n_used], sum f32 [T], norm f32 [T][n_used].
+ * moe_combine: MUL by the weights, the ADD chain over the expert slots and optionally the residual ADD that follows
+ *   (ggml-cpu.c:5142-5211, 4067-4140): experts f32 [T][n_used][n_embd], weights f32 [T][n_used] -> scaled (same shape, may be
+ *   NULL when nothing else reads it), out f32 [T][n_embd] = sum_e scaled[t][e] (+ residual[t]). */
+int mi355_moe_route(void *stream, const float *logits, float *probs, int32_t *order, int64_t n_expert, int64_t T);
+int mi355_moe_weights(void *stream, const float *probs, const int32_t *ids, int64_t ids_stride, float *raw, float *sum, float *norm,
+                      int64_t n_expert, int64_t n_used, int64_t T);
+int mi355_moe_combine(void *stream, const float *experts, const float *weights, float *scaled, const float *residual, float *out,
+                      int64_t n_embd, int64_t n_used, int64_t T);
+
 /* MUL_MAT with f32 or f16 src0 and f32 src1 (router / small dense matrices): dst[b][n] = sum_k W[n][k] x[b][k], strides honoured, ne2/ne3 broadcast */
 int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *src1, const mi355_tensor *dst);
 

@@ -684,6 +684,25 @@ bool feeds_quant_gemv(const graph_walk & w, int i, const void * data, int64_t K,
     return is_quant_gemv_candidate(mm) && mm->src[1]->data == data && mm->src[0]->ne[0] == K && mm->src[1]->ne[1] == B;
 }
 
+// A MUL_MAT_ID with few (token, expert slot) pairs streams each slot's expert through the GEMV on Q8_1 activations; with many
+// slots and K-quant experts it sorts the slots by expert and uses the tile kernel on per-super-block activations.
+bool mmid_uses_tiles(const ggml_tensor * op) {
+    const ggml_tensor * as = op->src[0];
+    const int64_t K = as->ne[0], slots = op->src[2]->ne[0] * op->src[1]->ne[2];
+    if (slots < 32 || as->ne[2] > 256 || K % 256 != 0 || ((uintptr_t) as->data & 15) != 0) return false;
+    return as->type == GGML_TYPE_Q4_K || (as->type == GGML_TYPE_Q6_K && K % 2048 == 0);
+}
+
+// does the node after `i` (skipping views) route the rows of the tensor at `data` through quantized experts by GEMV?
+bool feeds_quant_mmid(const graph_walk & w, int i, const void * data, int64_t K, int64_t rows) {
+    const int j = w.next(i);
+    if (j >= w.n) return false;
+    const ggml_tensor * op = w.nodes[j];
+    if (op->op != GGML_OP_MUL_MAT_ID || mmid_uses_tiles(op)) return false;
+    const ggml_tensor * b = op->src[1];
+    return b->data == data && b->ne[0] == K && b->ne[1] * b->ne[2] == rows && K % 32 == 0;
+}
+
 // Runs node i and possibly a few of its successors; returns the index of the last node consumed.
 int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     hipStream_t s = ctx->stream;
@@ -717,10 +736,122 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         if (ggml_is_contiguous(gt) && ggml_is_contiguous(up) && ggml_is_contiguous(nxt) && ggml_are_same_shape(gt, up) && up->type == GGML_TYPE_F32 &&
             K % 32 == 0 && rows <= 65535 && (((uintptr_t) gt->data | (uintptr_t) up->data | (uintptr_t) nxt->data) & 15) == 0) {
             void * act = nullptr;
-            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
+            if (rows <= 8 && (feeds_quant_gemv(w, j, nxt->data, K, rows) || feeds_quant_mmid(w, j, nxt->data, K, rows)))
+                act = ctx->act_slot(mi355_act_bytes(K, rows));
             MI355_K_OK(mi355_swiglu_quant(s, (const float *) gt->data, (const float *) up->data, K, (float *) nxt->data, K, act, K, rows));
             ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
             return j;
+        }
+    }
+    // ---- MUL_MAT_ID: the quantized rows of src1 are shared by consecutive products (up and gate experts read the same rows)
+    if (node->op == GGML_OP_MUL_MAT_ID) {
+        const ggml_tensor * as = node->src[0];
+        const ggml_tensor * b = node->src[1];
+        const ggml_tensor * ids = node->src[2];
+        const int64_t K = as->ne[0], N = as->ne[1], n_expert = as->ne[2];
+        const int64_t nb1 = b->ne[1], T = b->ne[2], n_used = ids->ne[0], rows = nb1 * T;
+        const int64_t ids_stride = (int64_t) (ids->nb[1] / sizeof(int32_t));
+        if (((uintptr_t) b->data & 15) == 0 && rows <= 65535 && K % 32 == 0) {
+            if (mmid_uses_tiles(node)) {
+                if (!ctx->cached(b->data, K, rows, ACT_Q8K)) {
+                    void * fresh = ctx->act_slot(mi355_act_q8k_bytes(K, rows));
+                    MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, fresh, K, rows, K));
+                    ctx->cache = act_cache{b->data, K, rows, ACT_Q8K, true, fresh};
+                }
+                const size_t route_bytes = mi355_mul_mat_id_q8k_route_bytes(n_expert, n_used, T);
+                void * route = ctx->workspace(route_bytes);
+                MI355_K_OK(mi355_mul_mat_id_q8k(s, to_mi355_type(as->type), as->data, ctx->cache.ptr, (const int32_t *) ids->data, ids_stride,
+                                                (float *) node->data, N, K, n_expert, n_used, nb1, T, route, route_bytes));
+            } else {
+                if (!ctx->cached(b->data, K, rows, ACT_Q8_1)) {
+                    void * fresh = ctx->act_slot(mi355_act_bytes(K, rows));
+                    MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, rows, K));
+                    ctx->cache = act_cache{b->data, K, rows, ACT_Q8_1, true, fresh};
+                }
+                MI355_K_OK(mi355_mul_mat_id_vec(s, to_mi355_type(as->type), as->data, ctx->cache.ptr, (const int32_t *) ids->data, ids_stride,
+                                                (float *) node->data, N, K, n_expert, n_used, nb1, T));
+            }
+            ctx->note_write(node->data, ggml_nbytes(node));
+            return i;
+        }
+    }
+    // ---- SOFT_MAX -> ARGSORT(descending): expert probabilities and their order (llm_build_moe_ffn)
+    if (node->op == GGML_OP_SOFT_MAX && !node->src[1] && nxt && nxt->op == GGML_OP_ARGSORT && nxt->src[0] == node) {
+        float scale, max_bias;
+        memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
+        memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
+        const ggml_tensor * x = node->src[0];
+        if (scale == 1.0f && max_bias == 0.0f && x->ne[0] <= 64 && x->type == GGML_TYPE_F32 && ggml_is_contiguous(x) && ggml_is_contiguous(node) &&
+            ggml_is_contiguous(nxt) && nxt->type == GGML_TYPE_I32 && ((const int32_t *) nxt->op_params)[0] == GGML_SORT_ORDER_DESC) {
+            ctx->note_write(node->data, ggml_nbytes(node));
+            MI355_K_OK(mi355_moe_route(s, (const float *) x->data, (float *) node->data, (int32_t *) nxt->data, x->ne[0], ggml_nrows(x)));
+            return j;
+        }
+    }
+    // ---- GET_ROWS(probabilities of the selected experts) -> SUM_ROWS -> DIV: normalised expert weights
+    if (node->op == GGML_OP_GET_ROWS && nxt && nxt->op == GGML_OP_SUM_ROWS) {
+        const ggml_tensor * probs = node->src[0];   // [1, n_expert, T]
+        const ggml_tensor * ids = node->src[1];     // [n_used, T]
+        const int jd = w.next(j);
+        const ggml_tensor * div = jd < w.n ? w.nodes[jd] : nullptr;
+        const ggml_tensor * w2d = nxt->src[0];       // [n_used, T] reshape of the GET_ROWS result
+        const int64_t n_expert = probs->ne[1], T = probs->ne[2], n_used = ids->ne[0];
+        if (div && div->op == GGML_OP_DIV && div->src[0] == w2d && div->src[1] == nxt && w2d->op == GGML_OP_RESHAPE && w2d->src[0] == node &&
+            probs->type == GGML_TYPE_F32 && probs->ne[0] == 1 && probs->ne[3] == 1 && ggml_is_contiguous(probs) && ids->type == GGML_TYPE_I32 &&
+            ids->nb[0] == sizeof(int32_t) && ids->ne[1] == T && ids->ne[2] == 1 && ids->ne[3] == 1 && n_used <= 64 && n_used <= n_expert &&
+            ggml_is_contiguous(node) && node->ne[0] == 1 && node->ne[1] == n_used && node->ne[2] == T && ggml_is_contiguous(w2d) &&
+            ggml_is_contiguous(nxt) && ggml_is_contiguous(div) && w2d->ne[0] == n_used && w2d->ne[1] == T && ggml_nelements(nxt) == T) {
+            ctx->note_write(node->data, ggml_nbytes(node));
+            ctx->note_write(div->data, ggml_nbytes(div));
+            MI355_K_OK(mi355_moe_weights(s, (const float *) probs->data, (const int32_t *) ids->data, (int64_t) (ids->nb[1] / sizeof(int32_t)),
+                                         (float *) node->data, (float *) nxt->data, (float *) div->data, n_expert, n_used, T));
+            return jd;
+        }
+    }
+    // ---- MUL(expert outputs, weights) -> ADD over the expert slots [-> ADD(residual)]: weighted sum of the selected experts
+    if (node->op == GGML_OP_MUL && node->ne[1] >= 2 && node->ne[1] <= 64 && node->ne[3] == 1 && nxt && nxt->op == GGML_OP_ADD) {
+        const ggml_tensor * ex = node->src[0];
+        const ggml_tensor * wt = node->src[1];
+        const int64_t n_embd = node->ne[0], n_used = node->ne[1], T = node->ne[2];
+        auto slot_view = [&](const ggml_tensor * v, int64_t e) {
+            return v && v->op == GGML_OP_VIEW && v->view_src == node && v->view_offs == (size_t) e * node->nb[1] && v->ne[0] == n_embd && v->ne[1] == T &&
+                   v->ne[2] == 1 && v->ne[3] == 1 && v->nb[1] == node->nb[2] && v->nb[0] == sizeof(float);
+        };
+        bool ok = ex->type == GGML_TYPE_F32 && wt->type == GGML_TYPE_F32 && ggml_are_same_shape(ex, node) && ggml_is_contiguous(ex) && ggml_is_contiguous(node) &&
+                  ggml_is_contiguous(wt) && wt->ne[0] == 1 && wt->ne[1] == n_used && wt->ne[2] == T && wt->ne[3] == 1 && n_embd % 4 == 0 && T <= 65535 &&
+                  (((uintptr_t) ex->data | (uintptr_t) node->data) & 15) == 0;
+        int k = j;   // the ADD chain: ((slot0 + slot1) + slot2) + ...
+        const ggml_tensor * sum = nullptr;
+        for (int64_t e = 1; ok && e < n_used; e++) {
+            const ggml_tensor * add = k < w.n ? w.nodes[k] : nullptr;
+            ok = add && add->op == GGML_OP_ADD && slot_view(add->src[1], e) && (e == 1 ? slot_view(add->src[0], 0) : add->src[0] == sum) &&
+                 ggml_is_contiguous(add) && add->type == GGML_TYPE_F32 && ((uintptr_t) add->data & 15) == 0;
+            if (ok && e + 1 < n_used) ok = w.sole_use(k);   // intermediate sums are not materialised
+            if (ok) {
+                sum = add;
+                if (e + 1 < n_used) k = w.next(k);
+            }
+        }
+        if (ok) {
+            int last = k;
+            const ggml_tensor * out = sum;
+            const float * residual = nullptr;
+            const int jr = w.next(k);
+            const ggml_tensor * radd = jr < w.n ? w.nodes[jr] : nullptr;
+            if (radd && radd->op == GGML_OP_ADD && w.sole_use(k) && (radd->src[0] == sum || radd->src[1] == sum)) {
+                const ggml_tensor * res = radd->src[0] == sum ? radd->src[1] : radd->src[0];
+                if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, sum) && ggml_is_contiguous(res) && ggml_is_contiguous(radd) &&
+                    (((uintptr_t) res->data | (uintptr_t) radd->data) & 15) == 0) {
+                    residual = (const float *) res->data;
+                    out = radd;
+                    last = jr;
+                }
+            }
+            ctx->note_write(node->data, ggml_nbytes(node));
+            ctx->note_write(out->data, ggml_nbytes(out));
+            MI355_K_OK(mi355_moe_combine(s, (const float *) ex->data, (const float *) wt->data, (float *) node->data, residual, (float *) out->data, n_embd,
+                                         n_used, T));
+            return last;
         }
     }
     // ---- FLASH_ATTN_EXT whose output feeds a quantized product
@@ -780,85 +911,132 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             }
         }
     }
-    // ---- MUL_MAT -> [RESHAPE] -> ROPE [-> CPY to an f16 view]   and   MUL_MAT -> CPY to an f16 view   (decode, batch <= 4)
+    // ---- up to three projections of one activation with their ROPE and f16 cache-store nodes in ONE launch (decode, batch <= 4):
+    //      MUL_MAT -> [RESHAPE] -> ROPE [-> CPY to an f16 view]   and   MUL_MAT -> CPY to an f16 view.
+    //      llm_build_kv lists them as  Q, rope(Q), K, rope(K), V, cpy(K), cpy(V): the window below takes nodes while every one
+    //      of them belongs to such a chain, so nothing outside the window is reordered.
     if (is_quant_gemv_candidate(node) && node->src[1]->ne[1] <= 4 && w.sole_use(i) && nxt && node->ne[0] % 2 == 0) {
         const ggml_tensor * b = node->src[1];
-        const int64_t K = b->ne[0], B = b->ne[1], N = node->ne[0];
-        // the consumer may read the product through one reshape
-        auto reads_product = [&](const ggml_tensor * t) {
-            if (t == node) return true;
-            return t && t->op == GGML_OP_RESHAPE && t->src[0] == node && ggml_is_contiguous(t);
-        };
-        auto sole_chain = [&](const ggml_tensor * t) {   // a reshape in between must have a single reader too
-            if (t == node) return true;
-            for (int k = i + 1; k < j; k++)
+        const int64_t K = b->ne[0], B = b->ne[1];
+        struct chain {
+            const ggml_tensor * mm;     // the product
+            const ggml_tensor * out;    // the tensor that currently holds the chain's value (product or its ROPE)
+            int out_index;
+            mi355_gemv_rope_mat m;
+        } ch[3];
+        int n_ch = 0, last = i - 1;
+        mi355_rope_desc rd;
+        memset(&rd, 0, sizeof(rd));
+        bool have_rope = false;
+        auto node_index_sole = [&](const ggml_tensor * t, int from, int to) {   // t is a node in [from, to) with one reader
+            for (int k = from; k < to; k++)
                 if (w.nodes[k] == t) return w.sole_use(k);
             return false;
         };
-        mi355_gemv_rope_mat m;
-        m.type = to_mi355_type(node->src[0]->type);
-        m.W = node->src[0]->data;
-        m.N = N;
-        m.dst = nullptr;
-        m.dst_stride = 0;
-        m.nb1 = m.nb2 = 0;
-        mi355_rope_desc rd;
-        memset(&rd, 0, sizeof(rd));
-        rd.cells = ctx->iota;
-        rd.head_dim = N;   // one "head" spanning the row unless a ROPE says otherwise
-        rd.n_dims = 2; rd.n_ctx_orig = 1; rd.freq_base = 10000.0f; rd.freq_scale = 1.0f; rd.attn_factor = 1.0f; rd.beta_fast = 32.0f; rd.beta_slow = 1.0f;
-        int last = -1;
-        auto f16_row_view = [&](const ggml_tensor * d) {   // CPY destination: B rows of N f16, contiguous
-            return d->type == GGML_TYPE_F16 && ggml_is_contiguous(d) && ggml_nelements(d) == N * B && ((uintptr_t) d->data & 1) == 0;
-        };
-        if (nxt->op == GGML_OP_ROPE && reads_product(nxt->src[0]) && sole_chain(nxt->src[0]) && nxt->src[1]->type == GGML_TYPE_I32 &&
-            ggml_is_contiguous(nxt) && nxt->type == GGML_TYPE_F32 && nxt->ne[0] * nxt->ne[1] == N && nxt->ne[2] == B && nxt->ne[3] == 1 &&
-            (!nxt->src[2] || nxt->src[2]->type == GGML_TYPE_F32)) {
-            const int32_t * p = (const int32_t *) nxt->op_params;
-            if (p[2] == 0 && p[1] % 2 == 0 && p[1] > 0 && p[1] <= nxt->ne[0] && nxt->ne[0] % 2 == 0) {
-                rd.pos = (const int32_t *) nxt->src[1]->data;
-                rd.freq_factors = nxt->src[2] ? (const float *) nxt->src[2]->data : nullptr;
-                rd.head_dim = nxt->ne[0];
-                rd.n_dims = p[1];
-                rd.mode = 0;
-                rd.n_ctx_orig = p[4];
-                memcpy(&rd.freq_base, p + 5, sizeof(float));
-                memcpy(&rd.freq_scale, p + 6, sizeof(float));
-                memcpy(&rd.ext_factor, p + 7, sizeof(float));
-                memcpy(&rd.attn_factor, p + 8, sizeof(float));
-                memcpy(&rd.beta_fast, p + 9, sizeof(float));
-                memcpy(&rd.beta_slow, p + 10, sizeof(float));
-                const int jc = w.next(j);
-                const ggml_tensor * cpy = jc < w.n ? w.nodes[jc] : nullptr;
-                if (cpy && cpy->op == GGML_OP_CPY && cpy->src[0] == nxt && w.sole_use(j) && f16_row_view(cpy->src[1])) {
-                    m.epilogue = MI355_EPI_ROPE_CACHE;   // rotated K rows straight into the cache view
-                    m.dst = cpy->src[1]->data;
-                    m.nb1 = N * 2;
-                    m.nb2 = rd.head_dim * 2;
-                    last = jc;
-                } else {
-                    m.epilogue = MI355_EPI_ROPE;         // rotated Q rows into the ROPE node's tensor
-                    m.dst = nxt->data;
-                    m.dst_stride = N;
-                    last = j;
+        for (int k = i; k < w.n && k < i + 24; k++) {
+            const ggml_tensor * t = w.nodes[k];
+            if (is_noop(t)) continue;
+            if (t->op == GGML_OP_MUL_MAT) {
+                if (n_ch == 3 || !is_quant_gemv_candidate(t) || t->src[1]->data != b->data || t->src[1]->ne[0] != K || t->src[1]->ne[1] != B ||
+                    !w.sole_use(k) || t->ne[0] % 2 != 0 || !ggml_is_contiguous(t))
+                    break;
+                chain & c = ch[n_ch++];
+                c.mm = t; c.out = t; c.out_index = k;
+                c.m.type = to_mi355_type(t->src[0]->type);
+                c.m.W = t->src[0]->data;
+                c.m.N = t->ne[0];
+                c.m.epilogue = MI355_EPI_STORE;
+                c.m.dst = t->data;
+                c.m.dst_stride = t->ne[0];
+                c.m.nb1 = c.m.nb2 = 0;
+                last = k;
+                continue;
+            }
+            if (t->op == GGML_OP_ROPE) {
+                const ggml_tensor * src = t->src[0];
+                chain * c = nullptr;
+                for (int q = 0; q < n_ch; q++) {
+                    if (ch[q].m.epilogue != MI355_EPI_STORE) continue;
+                    if (src == ch[q].mm) c = &ch[q];
+                    else if (src->op == GGML_OP_RESHAPE && src->src[0] == ch[q].mm && ggml_is_contiguous(src) && node_index_sole(src, ch[q].out_index + 1, k)) c = &ch[q];
                 }
+                const int32_t * p = (const int32_t *) t->op_params;
+                const int64_t N = c ? c->m.N : 0;
+                if (!c || t->src[1]->type != GGML_TYPE_I32 || !ggml_is_contiguous(t) || t->type != GGML_TYPE_F32 || t->ne[0] * t->ne[1] != N || t->ne[2] != B ||
+                    t->ne[3] != 1 || (t->src[2] && t->src[2]->type != GGML_TYPE_F32) || p[2] != 0 || p[1] % 2 != 0 || p[1] <= 0 || p[1] > t->ne[0] ||
+                    t->ne[0] % 2 != 0)
+                    break;
+                mi355_rope_desc r;
+                memset(&r, 0, sizeof(r));
+                r.pos = (const int32_t *) t->src[1]->data;
+                r.cells = ctx->iota;
+                r.freq_factors = t->src[2] ? (const float *) t->src[2]->data : nullptr;
+                r.head_dim = t->ne[0];
+                r.n_dims = p[1];
+                r.mode = 0;
+                r.n_ctx_orig = p[4];
+                memcpy(&r.freq_base, p + 5, sizeof(float));
+                memcpy(&r.freq_scale, p + 6, sizeof(float));
+                memcpy(&r.ext_factor, p + 7, sizeof(float));
+                memcpy(&r.attn_factor, p + 8, sizeof(float));
+                memcpy(&r.beta_fast, p + 9, sizeof(float));
+                memcpy(&r.beta_slow, p + 10, sizeof(float));
+                if (have_rope && memcmp(&r, &rd, sizeof(rd)) != 0) break;   // one set of rope parameters per launch
+                rd = r;
+                have_rope = true;
+                c->m.epilogue = MI355_EPI_ROPE;
+                c->m.dst = t->data;
+                c->m.dst_stride = N;
+                c->out = t;
+                c->out_index = k;
+                last = k;
+                continue;
             }
-        } else if (nxt->op == GGML_OP_CPY && reads_product(nxt->src[0]) && sole_chain(nxt->src[0]) && f16_row_view(nxt->src[1])) {
-            m.epilogue = MI355_EPI_CACHE;                // V rows converted into the cache view
-            m.dst = nxt->src[1]->data;
-            m.nb1 = N * 2;
-            m.nb2 = 0;
-            last = j;
+            if (t->op == GGML_OP_CPY) {
+                chain * c = nullptr;
+                for (int q = 0; q < n_ch; q++)
+                    if (t->src[0] == ch[q].out && (ch[q].m.epilogue == MI355_EPI_STORE || ch[q].m.epilogue == MI355_EPI_ROPE)) c = &ch[q];
+                const ggml_tensor * d = t->src[1];
+                if (!c || !w.sole_use(c->out_index) || d->type != GGML_TYPE_F16 || !ggml_is_contiguous(d) || ggml_nelements(d) != c->m.N * B ||
+                    ((uintptr_t) d->data & 1) != 0)
+                    break;
+                c->m.epilogue = c->m.epilogue == MI355_EPI_ROPE ? MI355_EPI_ROPE_CACHE : MI355_EPI_CACHE;
+                c->m.dst = d->data;
+                c->m.dst_stride = 0;
+                c->m.nb1 = c->m.N * 2;
+                c->out = nullptr;
+                last = k;
+                continue;
+            }
+            break;
         }
-        if (last >= 0) {
-            if (!ctx->cached(b->data, K, B, ACT_Q8_1)) {
-                void * fresh = ctx->act_slot(mi355_act_bytes(K, B));
-                MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
-                ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
+        bool any_epilogue = false;
+        for (int q = 0; q < n_ch; q++) any_epilogue = any_epilogue || ch[q].m.epilogue != MI355_EPI_STORE;
+        if (any_epilogue) {
+            if (!have_rope) {   // cache stores only: rows are one "head"; any even divisor of every N serves
+                rd.cells = ctx->iota;
+                rd.head_dim = 2; rd.n_dims = 2; rd.n_ctx_orig = 1; rd.freq_base = 10000.0f; rd.freq_scale = 1.0f; rd.attn_factor = 1.0f; rd.beta_fast = 32.0f; rd.beta_slow = 1.0f;
             }
-            MI355_K_OK(mi355_mul_mat_vec_q_rope(s, 1, &m, ctx->cache.ptr, K, B, &rd));
-            ctx->note_write(m.dst, (size_t) N * (size_t) B * (m.epilogue == MI355_EPI_ROPE ? sizeof(float) : 2));
-            return last;
+            bool heads_ok = true;
+            mi355_gemv_rope_mat mats[3];
+            for (int q = 0; q < n_ch; q++) {
+                mats[q] = ch[q].m;
+                if (mats[q].epilogue != MI355_EPI_STORE) heads_ok = heads_ok && mats[q].N % rd.head_dim == 0;
+                if (mats[q].epilogue == MI355_EPI_ROPE_CACHE || mats[q].epilogue == MI355_EPI_CACHE) mats[q].nb2 = rd.head_dim * 2;
+            }
+            if (heads_ok) {
+                if (!ctx->cached(b->data, K, B, ACT_Q8_1)) {
+                    void * fresh = ctx->act_slot(mi355_act_bytes(K, B));
+                    MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
+                    ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
+                }
+                MI355_K_OK(mi355_mul_mat_vec_q_rope(s, n_ch, mats, ctx->cache.ptr, K, B, &rd));
+                for (int q = 0; q < n_ch; q++) {
+                    const bool f32_out = mats[q].epilogue == MI355_EPI_STORE || mats[q].epilogue == MI355_EPI_ROPE;
+                    ctx->note_write(mats[q].dst, (size_t) mats[q].N * (size_t) B * (f32_out ? sizeof(float) : 2));
+                }
+                return last;
+            }
         }
     }
     // ---- runs of quantized products on one activation (batch <= 8): one quantization, multi-matrix GEMV, residual epilogue
@@ -938,9 +1116,18 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         return GGML_STATUS_SUCCESS;
     }
     const graph_walk w(cgraph);
+    static const bool log_graph = getenv("MI355_LOG_GRAPH") != nullptr;   // node list and the nodes each launch sequence consumed
     for (int i = 0; i < w.n; i++) {
         if (is_noop(w.nodes[i])) continue;
+        const int first = i;
         i = compute_fused(ctx, w, i);
+        if (log_graph) {
+            for (int k = first; k <= i; k++) {
+                const ggml_tensor * t = w.nodes[k];
+                fprintf(stderr, "MI355 graph %s%3d %-14s %-24s [%lld %lld %lld %lld] uses %d\n", k == first ? "*" : " ", k, ggml_op_name(t->op), t->name,
+                        (long long) t->ne[0], (long long) t->ne[1], (long long) t->ne[2], (long long) t->ne[3], w.uses[k]);
+            }
+        }
     }
     ctx->cache.valid = false;
     return GGML_STATUS_SUCCESS;   // asynchronous: completion is observed through synchronize()

@@ -293,18 +293,38 @@ __global__ void k_argsort(tens src, tens dst, int order, int npad) {
 }
 
 // ---------------------------------------------------------------- dense MUL_MAT (f32 / f16 weights)
-// dst[i3][i2][b][n] = sum_k W[i3/r3][i2/r2][n][k] * x[i3][i2][b][k]; one wave per output element
-template <typename TW>
-__global__ void __launch_bounds__(64) k_mul_mat_f(tens w, tens x, tens d) {
+// dst[i3][i2][b][n] = sum_k W[i3/r3][i2/r2][n][k] * x[i3][i2][b][k]; one 256-thread group per output element.
+// VEC: both rows are dense, 16-byte aligned and K is a multiple of 4 (f32) / 8 (f16), so a lane loads 16 bytes at a time.
+template <typename TW, bool VEC>
+__global__ void __launch_bounds__(256) k_mul_mat_f(tens w, tens x, tens d) {
+    __shared__ float sh[16];
     const int64_t n = blockIdx.x, b = blockIdx.y;
     const int64_t i23 = blockIdx.z, i2 = i23 % d.ne[2], i3 = i23 / d.ne[2];
     const int64_t r2 = x.ne[2] / w.ne[2], r3 = x.ne[3] / w.ne[3];
     const uint8_t *wp = w.data + n * w.nb[1] + (i2 / r2) * w.nb[2] + (i3 / r3) * w.nb[3];
     const uint8_t *xp = x.data + b * x.nb[1] + i2 * x.nb[2] + i3 * x.nb[3];
+    const int64_t K = w.ne[0];
     float acc = 0.0f;
-    for (int64_t k = threadIdx.x; k < w.ne[0]; k += 64)
-        acc += (float)*(const TW *)(wp + k * w.nb[0]) * *(const float *)(xp + k * x.nb[0]);
-    acc = wave_sum(acc);
+    if constexpr (VEC) {
+        constexpr int PER = 16 / sizeof(TW);   // weight elements per 16-byte load
+#pragma unroll 4
+        for (int64_t k = (int64_t)threadIdx.x * PER; k < K; k += 256 * PER) {
+            const f32x4 x0 = *(const f32x4 *)(xp + k * 4);
+            if constexpr (sizeof(TW) == 4) {
+                const f32x4 w0 = *(const f32x4 *)(wp + k * 4);
+                acc += w0[0] * x0[0] + w0[1] * x0[1] + w0[2] * x0[2] + w0[3] * x0[3];
+            } else {
+                const f32x4 x1 = *(const f32x4 *)(xp + k * 4 + 16);
+                const f16x8 w0 = *(const f16x8 *)(wp + k * 2);
+                acc += (float)w0[0] * x0[0] + (float)w0[1] * x0[1] + (float)w0[2] * x0[2] + (float)w0[3] * x0[3] +
+                       (float)w0[4] * x1[0] + (float)w0[5] * x1[1] + (float)w0[6] * x1[2] + (float)w0[7] * x1[3];
+            }
+        }
+    } else {
+#pragma unroll 4
+        for (int64_t k = threadIdx.x; k < K; k += 256) acc += (float)*(const TW *)(wp + k * w.nb[0]) * *(const float *)(xp + k * x.nb[0]);
+    }
+    acc = block_sum(acc, sh);
     if (threadIdx.x == 0) *(float *)(d.data + n * d.nb[0] + b * d.nb[1] + i2 * d.nb[2] + i3 * d.nb[3]) = acc;
 }
 
@@ -502,8 +522,20 @@ int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *
     if (nelements(dst) == 0) return MI355_OK;
     MI355_REQUIRE(dst->ne[1] <= 65535 && dst->ne[2] * dst->ne[3] <= 65535, "mul_mat_f: batch too large for one launch");
     const dim3 grid((unsigned)dst->ne[0], (unsigned)dst->ne[1], (unsigned)(dst->ne[2] * dst->ne[3]));
-    if (src0->type == MI355_F32) hipLaunchKernelGGL(k_mul_mat_f<float>, grid, dim3(64), 0, (hipStream_t)stream, to_tens(src0), to_tens(src1), to_tens(dst));
-    else hipLaunchKernelGGL(k_mul_mat_f<_Float16>, grid, dim3(64), 0, (hipStream_t)stream, to_tens(src0), to_tens(src1), to_tens(dst));
+    const int64_t wsz = src0->type == MI355_F32 ? 4 : 2;
+    auto rows16 = [](const mi355_tensor *t, int64_t esz) {
+        return t->nb[0] == (size_t)esz && ((uintptr_t)t->data & 15) == 0 && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
+    };
+    const bool vec = src0->ne[0] % (16 / wsz) == 0 && rows16(src0, wsz) && rows16(src1, 4);
+    const dim3 block(256);
+    hipStream_t s = (hipStream_t)stream;
+    if (src0->type == MI355_F32) {
+        if (vec) hipLaunchKernelGGL((k_mul_mat_f<float, true>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+        else hipLaunchKernelGGL((k_mul_mat_f<float, false>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+    } else {
+        if (vec) hipLaunchKernelGGL((k_mul_mat_f<_Float16, true>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+        else hipLaunchKernelGGL((k_mul_mat_f<_Float16, false>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+    }
     return launch_status("k_mul_mat_f");
 }
 

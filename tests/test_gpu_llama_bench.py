@@ -105,5 +105,7 @@ def test_moe_model_logits_cpu_vs_plugin(dev, tmp_path, n_prompt):
     make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=2048, n_head=16, n_head_kv=4, n_vocab=2048, n_expert=8, n_expert_used=2)
     cpu = _logits(model, 0, n_prompt, 4, str(tmp_path / "cpu.bin"))
     gpu = _logits(model, 99, n_prompt, 4, str(tmp_path / "gpu.bin"))
-    assert cpu.shape == gpu.shape and np.isfinite(gpu).all()
+    nodes = _logits(model, 99, n_prompt, 4, str(tmp_path / "nodes.bin"), fusion=False)
+    assert cpu.shape == gpu.shape == nodes.shape and np.isfinite(gpu).all()
+    assert orc.nmse(gpu, nodes) < (1e-6 if n_prompt <= 8 else 5e-4)
     assert orc.nmse(gpu, cpu) < 2e-3
