@@ -17,8 +17,10 @@
 // integers: k slots 0..7 carry (bsum & 63) x m_j, slots 8..15 carry (bsum >> 6) x 64*m_j.
 //
 // A 256-thread group (4 waves, 2 x 2) owns a 64 (weight rows) x 128 (activation rows) tile of
-// dst; each wave a 32 x 64 sub-tile (1 x 2 MFMA tiles).  K is walked in stages of 128 elements; the global loads of
-// stage s+1 are issued before the MFMAs of stage s and unpacked to LDS after them.
+// dst; each wave a 32 x 64 sub-tile (1 x 2 MFMA tiles).  K is walked in stages of 128 elements.  k_mmq_kp is the kernel
+// of the full-width tile: double-buffered LDS, one barrier per stage, activations by direct global-to-LDS transfers, the
+// weight unpack interleaved with the matrix instructions.  k_mmq_k is the single-buffered kernel (register prefetch, two
+// barriers per stage) kept for the 64 x 64 tile that sparse expert routing uses.
 //
 // MFMA operand mapping (A = activations, B = weights, D[i][j]): lane l supplies row l % 32
 // and k bytes [16*(l/32), +16) (f16: k slots [8*(l/32), +8)); D register r of lane l is
@@ -409,10 +411,314 @@ __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ 
         }
 }
 
-template <int TYPE, int TW, int TB, int OCC>
-static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
-                         int64_t dst_stride) {
-    constexpr int BM = 64 * TW, BN = 64 * TB;
+// ---- pipelined variant of the 64 x 128 tile ---------------------------------------------------------------------------
+// Two LDS buffers per operand, one barrier per 128-element stage.  While the matrix cores work on stage s from
+// buffer s % 2, the same waves unpack the weights of stage s + 1 (fetched to registers during stage s - 1) into the other
+// buffer, and the activations of stage s + 1 go from global memory straight to LDS (global_load_lds, no registers, no
+// vector-ALU work).  LDS rows are 128 bytes without padding; the 16-byte chunk c of row r lives at chunk c ^ ((r >> 1) & 7),
+// which keeps every 16-lane group of a ds_read_b128 on distinct banks.  A super-block is two stages, so the buffer of a
+// stage is its half: every LDS access names its array statically and the compiler can tell the buffer being filled from
+// the one being read.
+constexpr int KP_ROW = 128;
+__device__ __forceinline__ int kp_off(int row, int chunk) { return row * KP_ROW + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+template <int TYPE> struct kp_w;   // the 16-byte weight piece of one stage that this thread unpacks (row tid / 4, piece tid % 4)
+template <> struct kp_w<MI355_Q4_K> { u32x4 q; };
+template <> struct kp_w<MI355_Q6_K> { u32x4 ql, qh; int scA, scB; };
+// per super-block data of this thread's weight row: the Q4_K block header (d, dmin, 12 scale bytes) / the Q6_K d
+template <int TYPE> struct kp_h;
+template <> struct kp_h<MI355_Q4_K> { u32x4 hdr; };
+template <> struct kp_h<MI355_Q6_K> { unsigned short d; };   // raw fp16 bits: converting at the load would wait for it
+
+template <int TYPE>
+__device__ __forceinline__ void kp_fetch_h(kp_h<TYPE> &H, const uint8_t *__restrict__ wrow, const row_layout &L, int64_t sb) {
+    if constexpr (TYPE == MI355_Q4_K) H.hdr = load16(wrow + sb * Q4_K_BYTES);
+    else H.d = *(const unsigned short *)(wrow + L.off_d + sb * 2);
+}
+
+template <int TYPE>
+__device__ __forceinline__ void kp_fetch_w(kp_w<TYPE> &R, const uint8_t *__restrict__ wrow, const row_layout &L, int64_t sb, int half) {
+    const int p = threadIdx.x & 3;
+    if constexpr (TYPE == MI355_Q4_K) {
+        const uint8_t *blk = wrow + sb * Q4_K_BYTES;
+        R.q = load16(blk + 16 + (half * 2 + (p >> 1)) * 32 + (p & 1) * 16);
+    } else {
+        const int l0 = 16 * (p & 1), qa = p >> 1;
+        R.ql = load16(wrow + sb * 128 + half * 64 + p * 16);
+        R.qh = load16(wrow + L.off_b + sb * 64 + half * 32 + l0);
+        const int8_t *sc = (const int8_t *)(wrow + L.off_c + sb * 16 + half * 8 + (l0 >> 4));
+        R.scA = sc[2 * qa];
+        R.scB = sc[2 * qa + 4];
+    }
+}
+
+// unpacked planes of the piece: two 16-byte chunks per plane
+struct kp_planes { u32x4 a1, a0, b1, b0; };
+
+// dword i of the piece -> dword i of the four plane chunks
+template <int TYPE>
+__device__ __forceinline__ void kp_unpack(const kp_w<TYPE> &R, const kp_h<TYPE> &H, int half, int i, kp_planes &P) {
+    const int p = threadIdx.x & 3;
+    if constexpr (TYPE == MI355_Q4_K) {
+        const int gl = p >> 1;
+        int scl, mnl, sch, mnh;
+        q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], half * 4 + 2 * gl, scl, mnl);
+        q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], half * 4 + 2 * gl + 1, sch, mnh);
+        const u32 nl = R.q[i] & 0x0F0F0F0Fu, nh = (R.q[i] >> 4) & 0x0F0F0F0Fu;
+        P.a1[i] = mul_bytes(nl, (u32)scl >> 3);
+        P.a0[i] = mul_bytes(nl, (u32)scl & 7u);
+        P.b1[i] = mul_bytes(nh, (u32)sch >> 3);
+        P.b0[i] = mul_bytes(nh, (u32)sch & 7u);
+    } else {
+        const int qa = p >> 1;
+        const u32 va = (R.ql[i] & 0x0F0F0F0Fu) | (((R.qh[i] >> (2 * qa)) & 0x03030303u) << 4);
+        const u32 vb = ((R.ql[i] >> 4) & 0x0F0F0F0Fu) | (((R.qh[i] >> (2 * qa + 4)) & 0x03030303u) << 4);
+        u32 hi, lo;
+        q6k_planes(va, R.scA, hi, lo);
+        P.a1[i] = hi; P.a0[i] = lo;
+        q6k_planes(vb, R.scB, hi, lo);
+        P.b1[i] = hi; P.b0[i] = lo;
+    }
+}
+
+template <int TYPE>
+__device__ __forceinline__ void kp_store(const kp_planes &P, int8_t *__restrict__ sW1, int8_t *__restrict__ sW0) {
+    const int r = threadIdx.x >> 2, p = threadIdx.x & 3;
+    // Q4_K: low nibbles are sub-block 2*gl, high nibbles sub-block 2*gl + 1 (32 bytes later); Q6_K: the second group is 64 bytes later
+    const int c0 = TYPE == MI355_Q4_K ? 4 * (p >> 1) + (p & 1) : 2 * (p >> 1) + (p & 1);
+    const int c1 = c0 + (TYPE == MI355_Q4_K ? 2 : 4);
+    *(u32x4 *)(sW1 + kp_off(r, c0)) = P.a1;
+    *(u32x4 *)(sW0 + kp_off(r, c0)) = P.a0;
+    *(u32x4 *)(sW1 + kp_off(r, c1)) = P.b1;
+    *(u32x4 *)(sW0 + kp_off(r, c1)) = P.b0;
+}
+
+// activations of one stage: 128 rows x 128 bytes, 4 wave-wide 16-byte transfers per wave
+__device__ __forceinline__ void kp_dma_a(const int8_t *__restrict__ aq, const int (&arow)[4], int64_t K, int64_t k0, int8_t *__restrict__ sA) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int row = (wave * 4 + it) * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);   // the logical chunk that belongs at this lane's position
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(aq + (int64_t)arow[it] * K + k0 + c * 16),
+                                         (void __attribute__((address_space(3))) *)(sA + (wave * 4 + it) * 1024), 16, 0, 0);
+    }
+}
+
+template <int TYPE, bool ID>
+__global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq, const float *__restrict__ ad8,
+                                                   const _Float16 *__restrict__ abs_, float *__restrict__ dst, int64_t N, int64_t K, int64_t B,
+                                                   int64_t dst_stride, row_layout L, int n_col_tiles, int n_groups, int n_groups_padded,
+                                                   mmq_route route) {
+    constexpr bool Q4 = TYPE == MI355_Q4_K;
+    constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
+    constexpr int BM = 64, BN = 128;
+    __shared__ __attribute__((aligned(16))) int8_t sW1a[BM * KP_ROW], sW1b[BM * KP_ROW];
+    __shared__ __attribute__((aligned(16))) int8_t sW0a[BM * KP_ROW], sW0b[BM * KP_ROW];
+    __shared__ __attribute__((aligned(16))) int8_t sAa[BN * KP_ROW], sAb_[BN * KP_ROW];
+    __shared__ __attribute__((aligned(16))) float sWd[2][BM];
+    __shared__ __attribute__((aligned(16))) float sWn[2][Q4 ? BM : 4];
+    __shared__ __attribute__((aligned(16))) _Float16 sWm[2][Q4 ? BM * 16 : 8];
+    __shared__ __attribute__((aligned(16))) float sAd[2][BN];
+    __shared__ __attribute__((aligned(16))) _Float16 sAs[2][Q4 ? BN * 16 : 8];
+
+    const int per_xcd = n_groups_padded >> 3;
+    const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (lid >= n_groups) return;
+    const int64_t row0 = (int64_t)(lid / n_col_tiles) * BM;
+    int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+    if constexpr (ID) {
+        const int ct = lid % n_col_tiles;
+        if (ct >= *route.n_tiles) return;
+        W += (int64_t)route.tiles[4 * ct] * route.expert_bytes;
+        col0 = route.tiles[4 * ct + 1];
+        B = route.tiles[4 * ct + 2];
+    }
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int wrow0 = (wave & 1) * 32;    // weight rows of this wave inside the tile
+    const int wcol0 = (wave >> 1) * 64;   // activation rows of this wave inside the tile
+    const int64_t nsb = K >> 8;
+
+    // this thread's weight row, the activation rows of its four transfers, and the column whose scales it copies
+    const int64_t wr = row0 + (tid >> 2) < N ? row0 + (tid >> 2) : N - 1;
+    const uint8_t *wrow = W + wr * L.row_bytes;
+    int arow[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int64_t col = col0 + (wave * 4 + it) * 8 + (lane >> 3);
+        const int64_t cc = col < B ? col : B - 1;
+        arow[it] = ID ? route.act_row[cc] : (int)cc;
+    }
+    int srow;
+    {
+        const int64_t col = col0 + (tid >> 1);
+        const int64_t cc = col < B ? col : B - 1;
+        srow = ID ? route.act_row[cc] : (int)cc;
+    }
+
+    f32x16 acc[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[tb][r] = 0.0f;
+
+    // per super-block scales of the weights come with the piece (Q4_K header / Q6_K d); those of the activations are fetched
+    // by two threads per column: 16 bytes of the sub-block sums each, the even thread also the scale
+    auto fetch_scales = [&](int64_t sb, float &d8, u32x4 &bs) {
+        d8 = ad8[(int64_t)srow * nsb + sb];
+        if constexpr (Q4) bs = *(const u32x4 *)(abs_ + ((int64_t)srow * nsb + sb) * 16 + 8 * (tid & 1));
+    };
+    auto store_scales = [&](int sbuf, float d8, const u32x4 &bs, const kp_h<TYPE> &H) {
+        sAd[sbuf][tid >> 1] = d8;   // both threads of the column write the same value: an unconditional use keeps the load where it was issued
+        if constexpr (Q4) {
+            *(u32x4 *)(sAs[sbuf] + (tid >> 1) * 16 + 8 * (tid & 1)) = bs;
+            if ((tid & 3) == 0) {
+                const int r = tid >> 2;
+                sWd[sbuf][r] = half_bits_to_float((unsigned short)(H.hdr[0] & 0xFFFFu));
+                sWn[sbuf][r] = half_bits_to_float((unsigned short)(H.hdr[0] >> 16));
+                f16x8 m1, m64;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    int sc, mn;
+                    q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], j, sc, mn);
+                    m1[j] = (_Float16)(float)mn;
+                    m64[j] = (_Float16)(float)(64 * mn);
+                }
+                *(f16x8 *)(sWm[sbuf] + r * 16) = m1;
+                *(f16x8 *)(sWm[sbuf] + r * 16 + 8) = m64;
+            }
+        } else {
+            sWd[sbuf][tid >> 2] = half_bits_to_float(H.d);   // the four threads of a row write the same value
+        }
+    };
+
+    kp_w<TYPE> R0, R1;   // pieces of the even / odd stages
+    kp_h<TYPE> Hc, Hn;   // super-block data in use / of the next super-block
+    float d8n = 0.0f;
+    u32x4 bsn = {0, 0, 0, 0};
+    // prologue: stage 0 into the "a" buffers, pieces of stage 1 in flight
+    kp_fetch_w<TYPE>(R0, wrow, L, 0, 0);
+    kp_fetch_w<TYPE>(R1, wrow, L, 0, 1);
+    kp_fetch_h<TYPE>(Hc, wrow, L, 0);
+    kp_dma_a(aq, arow, K, 0, sAa);
+    fetch_scales(0, d8n, bsn);
+    {
+        kp_planes P;
+#pragma unroll
+        for (int i = 0; i < 4; i++) kp_unpack<TYPE>(R0, Hc, 0, i, P);
+        kp_store<TYPE>(P, sW1a, sW0a);
+        store_scales(0, d8n, bsn, Hc);
+    }
+    Hn = Hc;
+    __syncthreads();
+
+    for (int64_t sb = 0; sb < nsb; sb++) {
+        i32x16 hi[2], lo[2];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int8_t *cA = half == 0 ? sAa : sAb_;
+            const int8_t *cW1 = half == 0 ? sW1a : sW1b;
+            const int8_t *cW0 = half == 0 ? sW0a : sW0b;
+            int8_t *nA = half == 0 ? sAb_ : sAa;
+            int8_t *nW1 = half == 0 ? sW1b : sW1a;
+            int8_t *nW0 = half == 0 ? sW0b : sW0a;
+            kp_w<TYPE> &Rn = half == 0 ? R1 : R0;    // piece of the next stage: unpacked during this one
+            kp_w<TYPE> &Rf = half == 0 ? R0 : R1;    // held this stage's piece (unpacked one stage ago): refilled for the stage after next
+            // Past the end of K the same work is done on the last super-block again and never read: no branches in the stage,
+            // so the compiler schedules it as one block.
+            const int64_t sb1 = sb + 1 < nsb ? sb + 1 : sb;
+            kp_dma_a(aq, arow, K, half == 0 ? sb * QKK + 128 : sb1 * QKK, nA);
+            if (half == 1) fetch_scales(sb1, d8n, bsn);
+            kp_fetch_w<TYPE>(Rf, wrow, L, sb1, half);
+            if (half == 0) kp_fetch_h<TYPE>(Hn, wrow, L, sb1);   // used from the next stage on
+            __builtin_amdgcn_sched_barrier(0);   // the loads stay here, a whole stage ahead of their first use
+
+            kp_planes P;
+            i32x4 af[2][2], b1[2], b0[2];
+            auto load_frags = [&](int ks, int slot) {
+#pragma unroll
+                for (int tb = 0; tb < 2; tb++) af[slot][tb] = *(const i32x4 *)(cA + kp_off(wcol0 + tb * 32 + l32, ks * 2 + lhi));
+                b1[slot] = *(const i32x4 *)(cW1 + kp_off(wrow0 + l32, ks * 2 + lhi));
+                b0[slot] = *(const i32x4 *)(cW0 + kp_off(wrow0 + l32, ks * 2 + lhi));
+            };
+            load_frags(0, 0);
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                if (ks < 3) load_frags(ks + 1, (ks + 1) & 1);   // operands of the next step are in flight during this step's matrix instructions
+                const int sl = ks & 1;
+#pragma unroll
+                for (int tb = 0; tb < 2; tb++) {
+                    if (half == 0 && ks == 0) {
+                        i32x16 z;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) z[r] = 0;
+                        hi[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b1[sl], z, 0, 0, 0);
+                        lo[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b0[sl], z, 0, 0, 0);
+                    } else {
+                        hi[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b1[sl], hi[tb], 0, 0, 0);
+                        lo[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b0[sl], lo[tb], 0, 0, 0);
+                    }
+                }
+                kp_unpack<TYPE>(Rn, half == 0 ? Hc : Hn, half ^ 1, ks, P);   // a quarter of the next stage's piece between the matrix instructions
+            }
+            kp_store<TYPE>(P, nW1, nW0);
+
+            if (half == 1) {   // end of the super-block: scale the integer sums into the f32 accumulators
+                const int sbuf = (int)(sb & 1);
+#pragma unroll
+                for (int tb = 0; tb < 2; tb++) {
+                    f32x4 d8[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) d8[q] = *(const f32x4 *)(sAd[sbuf] + wcol0 + tb * 32 + 8 * q + 4 * lhi);
+                    const int wr_ = wrow0 + l32;
+                    const float dw = sWd[sbuf][wr_];
+                    if constexpr (Q4) {
+                        const float dn = sWn[sbuf][wr_];
+                        const f16x8 am = *(const f16x8 *)(sAs[sbuf] + (wcol0 + tb * 32 + l32) * 16 + 8 * lhi);
+                        const f16x8 bm = *(const f16x8 *)(sWm[sbuf] + wr_ * 16 + 8 * lhi);
+                        f32x16 z;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                        const f32x16 M = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bm, z, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int t = (hi[tb][r] << RADIX_SHIFT) + lo[tb][r];
+                            acc[tb][r] += d8[r >> 2][r & 3] * (dw * (float)t - dn * M[r]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int t = (hi[tb][r] << RADIX_SHIFT) + lo[tb][r];
+                            acc[tb][r] += d8[r >> 2][r & 3] * (dw * (float)t);
+                        }
+                    }
+                }
+            }
+            if (half == 1) {   // last, so that the loads had the whole stage
+                store_scales((int)((sb + 1) & 1), d8n, bsn, Hn);
+                Hc = Hn;
+            }
+            __syncthreads();   // also waits for this stage's transfers and loads (issued a whole stage ago)
+        }
+    }
+
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++) {
+        const int64_t n = row0 + wrow0 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if (n < N && b < B) dst[(ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n] = acc[tb][r];
+        }
+    }
+}
+
+template <int TYPE>
+static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B, int64_t dst_stride) {
+    constexpr int BM = 64, BN = 128;
     const row_layout L = make_row_layout(TYPE, K);
     const int8_t *aq = (const int8_t *)act;
     const float *ad8 = (const float *)(aq + q8k_d_offset(K, B));
@@ -421,8 +727,8 @@ static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *d
     const int n_col_tiles = (int)((B + BN - 1) / BN);
     const int n_groups = n_row_tiles * n_col_tiles;
     const int n_groups_padded = (n_groups + 7) & ~7;
-    hipLaunchKernelGGL((k_mmq_k<TYPE, TW, TB, OCC, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_,
-                       dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
+    hipLaunchKernelGGL((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_, dst, N, K, B,
+                       dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
 }
 
 // ---- MUL_MAT_ID with many slots: sort the slots by expert, then one tile launch over all experts ----
@@ -498,16 +804,8 @@ static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int6
         hipLaunchKernelGGL((k_mmq_k<TYPE, 1, 1, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
                            dst, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
     else
-        hipLaunchKernelGGL((k_mmq_k<TYPE, 1, 2, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
-                           dst, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
-}
-
-// 64 x 128 tiles: 96 accumulator registers per lane leave room for two groups per CU, which
-// measured faster than 128 x 128 tiles at one group per CU
-template <int TYPE>
-static void launch_mmq_k_any(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
-                             int64_t dst_stride) {
-    launch_mmq_k<TYPE, 1, 2, 2>(s, W, act, dst, N, K, B, dst_stride);
+        hipLaunchKernelGGL((k_mmq_kp<TYPE, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_, dst, N, K, S,
+                           N, L, max_tiles, n_groups, n_groups_padded, route);
 }
 
 }  // namespace mi355
@@ -574,8 +872,8 @@ int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, fl
                   "mul_mat_q8k: activation workspace is not 16-byte aligned");
     MI355_REQUIRE((N + 63) / 64 * ((B + 63) / 64) < (1 << 30), "mul_mat_q8k: too many tiles");
     hipStream_t s = (hipStream_t)stream;
-    if (type == MI355_Q4_K) launch_mmq_k_any<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride);
-    else launch_mmq_k_any<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride);
+    if (type == MI355_Q4_K) launch_mmq_k<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride);
+    else launch_mmq_k<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride);
     return launch_status("k_mmq_k");
 }
 
