@@ -19,8 +19,11 @@
 // A 256-thread group (4 waves, 2 x 2) owns a 64 (weight rows) x 128 (activation rows) tile of
 // dst; each wave a 32 x 64 sub-tile (1 x 2 MFMA tiles).  K is walked in stages of 128 elements.  k_mmq_kp is the kernel
 // of the full-width tile: double-buffered LDS, one barrier per stage, activations by direct global-to-LDS transfers, the
-// weight unpack interleaved with the matrix instructions.  k_mmq_k is the single-buffered kernel (register prefetch, two
-// barriers per stage) kept for the 64 x 64 tile that sparse expert routing uses.
+// weight unpack interleaved with the matrix instructions.  (Keeping the unpacked weights in the registers of the lane that
+// feeds them to the matrix cores, with no LDS round trip, measured the same: the unpack is then repeated by the two waves
+// that share rows, and the vector ALU is the limit either way at ~11 instructions per matrix instruction.)  k_mmq_k is
+// the single-buffered kernel (register prefetch, two barriers per stage) kept for the 64 x 64 tile that sparse expert
+// routing uses.
 //
 // MFMA operand mapping (A = activations, B = weights, D[i][j]): lane l supplies row l % 32
 // and k bytes [16*(l/32), +16) (f16: k slots [8*(l/32), +8)); D register r of lane l is
@@ -493,15 +496,16 @@ __device__ __forceinline__ void kp_store(const kp_planes &P, int8_t *__restrict_
     *(u32x4 *)(sW0 + kp_off(r, c1)) = P.b0;
 }
 
-// activations of one stage: 128 rows x 128 bytes, 4 wave-wide 16-byte transfers per wave
-__device__ __forceinline__ void kp_dma_a(const int8_t *__restrict__ aq, const int (&arow)[4], int64_t K, int64_t k0, int8_t *__restrict__ sA) {
+// activations of one stage: 32 * AI rows x 128 bytes, AI wave-wide 16-byte transfers per wave
+template <int AI>
+__device__ __forceinline__ void kp_dma_a(const int8_t *__restrict__ aq, const int (&arow)[AI], int64_t K, int64_t k0, int8_t *__restrict__ sA) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-    for (int it = 0; it < 4; it++) {
-        const int row = (wave * 4 + it) * 8 + (lane >> 3);
+    for (int it = 0; it < AI; it++) {
+        const int row = (wave * AI + it) * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((row >> 1) & 7);   // the logical chunk that belongs at this lane's position
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(aq + (int64_t)arow[it] * K + k0 + c * 16),
-                                         (void __attribute__((address_space(3))) *)(sA + (wave * 4 + it) * 1024), 16, 0, 0);
+                                         (void __attribute__((address_space(3))) *)(sA + (wave * AI + it) * 1024), 16, 0, 0);
     }
 }
 
@@ -603,7 +607,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
     kp_fetch_w<TYPE>(R0, wrow, L, 0, 0);
     kp_fetch_w<TYPE>(R1, wrow, L, 0, 1);
     kp_fetch_h<TYPE>(Hc, wrow, L, 0);
-    kp_dma_a(aq, arow, K, 0, sAa);
+    kp_dma_a<4>(aq, arow, K, 0, sAa);
     fetch_scales(0, d8n, bsn);
     {
         kp_planes P;
@@ -630,7 +634,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
             // Past the end of K the same work is done on the last super-block again and never read: no branches in the stage,
             // so the compiler schedules it as one block.
             const int64_t sb1 = sb + 1 < nsb ? sb + 1 : sb;
-            kp_dma_a(aq, arow, K, half == 0 ? sb * QKK + 128 : sb1 * QKK, nA);
+            kp_dma_a<4>(aq, arow, K, half == 0 ? sb * QKK + 128 : sb1 * QKK, nA);
             if (half == 1) fetch_scales(sb1, d8n, bsn);
             kp_fetch_w<TYPE>(Rf, wrow, L, sb1, half);
             if (half == 0) kp_fetch_h<TYPE>(Hn, wrow, L, sb1);   // used from the next stage on
