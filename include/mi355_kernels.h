@@ -101,6 +101,10 @@ size_t mi355_act_q8k_bytes(int64_t k, int64_t nrows);
 int mi355_quantize_act_q8k(void *stream, const float *x, void *act, int64_t k, int64_t nrows, int64_t x_stride);
 int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
                       int64_t dst_stride);
+/* Same product with the ADD that follows it in the graph (the residual after wo and ffn_down, src/llama.cpp:1566, :1609) done in
+ * the epilogue: dst[b][n] = W[n] . x[b] + residual[b][n].  residual has dst's shape and stride and may be dst itself. */
+int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
+                          int64_t B, int64_t dst_stride);
 
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE
@@ -225,6 +229,12 @@ int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, con
 /* llm_build_ffn LLM_FFN_SILU + LLM_FFN_PAR: UNARY(SILU)(gate) then MUL by up (src/llama.cpp:280-320; ggml-cpu.c:6646-6683). */
 int mi355_swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
                        int64_t k, int64_t nrows);
+/* The two sequences above with `act` in the per-super-block layout of mi355_quantize_act_q8k (what the K-quant tile GEMM reads);
+ * k must be a multiple of 256.  Same levels, scales and sums as quantizing y with mi355_quantize_act_q8k. */
+int mi355_rms_norm_mul_quant_q8k(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride,
+                                 void *act, int64_t k, int64_t nrows, float eps);
+int mi355_swiglu_quant_q8k(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
+                           int64_t k, int64_t nrows);
 /* ROPE(q), ROPE(k), CPY(k -> K cache), CPY(v -> V cache) of build_llama + llm_build_kv_store (src/llama.cpp:1535-1548, :157-199;
  * ggml-cpu.c:9366-9549, 3519-3830).  q f32 [T][H][D] is rotated in place; k, v f32 [T][HK][D] are read; the f16 caches are addressed
  * as cell*nb1 + head*nb2 + 2*d with the cell of token t taken from cells[t] and its rope position from pos[t] (both DEVICE int32). */

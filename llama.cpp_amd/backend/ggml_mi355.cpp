@@ -604,7 +604,7 @@ void backend_synchronize(ggml_backend_t backend) {
 //   UNARY(SILU) -> MUL                           one launch, same
 //   FLASH_ATTN_EXT (few rows) -> MUL_MAT         attention also writes the Q8_1 form of its output
 //   MUL_MAT, MUL_MAT, ... on the same src1       activation quantized once; up to 4 matrices per GEMV launch
-//   MUL_MAT -> ADD(residual)                     residual added in the GEMV epilogue
+//   MUL_MAT -> ADD(residual)                     residual added in the GEMV / tile GEMM epilogue
 bool is_noop(const ggml_tensor * t) {
     switch (t->op) {
         case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE: return true;
@@ -684,6 +684,15 @@ bool feeds_quant_gemv(const graph_walk & w, int i, const void * data, int64_t K,
     return is_quant_gemv_candidate(mm) && mm->src[1]->data == data && mm->src[0]->ne[0] == K && mm->src[1]->ne[1] == B;
 }
 
+// does the node after `i` (skipping views) run the K-quant tile GEMM on the tensor whose data starts at `data`?
+bool feeds_q8k_tiles(const graph_walk & w, int i, const void * data, int64_t K, int64_t B) {
+    const int j = w.next(i);
+    if (j >= w.n || K % 256 != 0 || B > 65535) return false;
+    const ggml_tensor * mm = w.nodes[j];
+    return is_q8k_tile_candidate(mm) && mm->src[1]->data == data && mm->src[0]->ne[0] == K && mm->src[1]->ne[1] == B &&
+           mm->src[1]->nb[1] == (size_t) K * sizeof(float);
+}
+
 // A MUL_MAT_ID with few (token, expert slot) pairs streams each slot's expert through the GEMV on Q8_1 activations; with many
 // slots and K-quant experts it sorts the slots by expert and uses the tile kernel on per-super-block activations.
 bool mmid_uses_tiles(const ggml_tensor * op) {
@@ -721,6 +730,12 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             float eps;
             memcpy(&eps, node->op_params, sizeof(float));
             void * act = nullptr;
+            if (rows > 8 && feeds_q8k_tiles(w, j, nxt->data, K, rows)) {   // prefill: the per-super-block form for the tile GEMM
+                act = ctx->act_slot(mi355_act_q8k_bytes(K, rows));
+                MI355_K_OK(mi355_rms_norm_mul_quant_q8k(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
+                ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8K, true, act};
+                return j;
+            }
             if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
             MI355_K_OK(mi355_rms_norm_mul_quant(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
             ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
@@ -736,6 +751,12 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         if (ggml_is_contiguous(gt) && ggml_is_contiguous(up) && ggml_is_contiguous(nxt) && ggml_are_same_shape(gt, up) && up->type == GGML_TYPE_F32 &&
             K % 32 == 0 && rows <= 65535 && (((uintptr_t) gt->data | (uintptr_t) up->data | (uintptr_t) nxt->data) & 15) == 0) {
             void * act = nullptr;
+            if (rows > 8 && feeds_q8k_tiles(w, j, nxt->data, K, rows)) {
+                act = ctx->act_slot(mi355_act_q8k_bytes(K, rows));
+                MI355_K_OK(mi355_swiglu_quant_q8k(s, (const float *) gt->data, (const float *) up->data, K, (float *) nxt->data, K, act, K, rows));
+                ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8K, true, act};
+                return j;
+            }
             if (rows <= 8 && (feeds_quant_gemv(w, j, nxt->data, K, rows) || feeds_quant_mmid(w, j, nxt->data, K, rows)))
                 act = ctx->act_slot(mi355_act_bytes(K, rows));
             MI355_K_OK(mi355_swiglu_quant(s, (const float *) gt->data, (const float *) up->data, K, (float *) nxt->data, K, act, K, rows));
@@ -1092,6 +1113,17 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             void * fresh = ctx->act_slot(mi355_act_q8k_bytes(K, B));
             MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
             ctx->cache = act_cache{b->data, K, B, ACT_Q8K, true, fresh};
+        }
+        // MUL_MAT -> ADD(residual): the sum goes straight into the ADD's tensor
+        ggml_tensor * add = nxt;
+        if (add && add->op == GGML_OP_ADD && w.sole_use(i) && (add->src[0] == node || add->src[1] == node)) {
+            const ggml_tensor * res = add->src[0] == node ? add->src[1] : add->src[0];
+            if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, node) && ggml_is_contiguous(res) && ggml_is_contiguous(add) && ggml_is_contiguous(node)) {
+                MI355_K_OK(mi355_mul_mat_q8k_add(s, to_mi355_type(node->src[0]->type), node->src[0]->data, ctx->cache.ptr, (float *) add->data,
+                                                 (const float *) res->data, node->src[0]->ne[1], K, B, (int64_t) (add->nb[1] / sizeof(float))));
+                ctx->note_write(add->data, ggml_nbytes(add));
+                return j;
+            }
         }
         MI355_K_OK(mi355_mul_mat_q8k(s, to_mi355_type(node->src[0]->type), node->src[0]->data, ctx->cache.ptr, (float *) node->data, node->src[0]->ne[1], K, B,
                                      (int64_t) (node->nb[1] / sizeof(float))));

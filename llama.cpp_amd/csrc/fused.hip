@@ -4,10 +4,13 @@
 // to four consecutive nodes and, where the consumer is a quantized MUL_MAT, also emits the
 // Q8_1 activation (same arithmetic as k_quantize_q8_1, i.e. quantize_row_q8_1_ref), so the
 // separate quantization launch disappears:
-//   RMS_NORM -> MUL(weight) [-> Q8_1]            k_rms_norm_mul_quant
-//   UNARY(SILU) -> MUL(up)  [-> Q8_1]            k_swiglu_quant
+//   RMS_NORM -> MUL(weight) [-> Q8_1 | Q8_K]     k_rms_norm_mul_quant
+//   UNARY(SILU) -> MUL(up)  [-> Q8_1 | Q8_K]     k_swiglu_quant
+// (Q8_K: the per-super-block form the K-quant tile GEMM reads, same arithmetic as k_quantize_q8k; a wave's 64 lanes hold
+// exactly one 256-element super-block)
 //   ROPE(q), ROPE(k), CPY(k -> cache), CPY(v -> cache)   k_rope_kv_store
 #include "common.hpp"
+#include "q8k.hpp"
 
 namespace mi355 {
 
@@ -41,7 +44,7 @@ __device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, i
 }
 
 // one 256-thread group per row; each thread keeps its NV float4 of the row in registers
-template <int NV>
+template <int NV, bool Q8K>
 __global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restrict__ x, int64_t x_stride, const float *__restrict__ w,
                                                             float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k,
                                                             int64_t nrows, float eps) {
@@ -83,11 +86,21 @@ __global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restr
             for (int i = 0; i < 4; i++) o[i] = o[i] * ww[it][i];
         }
         if (y && live) *(f32x4 *)(y + row * y_stride + e0) = o;
-        if (act) quantize_block_lane(o, live, qplane, ds, row, k, e0);
+        if constexpr (Q8K) {
+            if (act && live) {   // whole wave: k is a multiple of 256
+                const int64_t nsb = k >> 8, sb = e0 >> 8;
+                float *d8 = (float *)(qplane + q8k_d_offset(k, nrows));
+                _Float16 *bs = (_Float16 *)(qplane + q8k_bs_offset(k, nrows));
+                q8k_quantize_wave(o, tid & 63, qplane + row * k + sb * QKK, d8 + row * nsb + sb, bs + (row * nsb + sb) * 16);
+            }
+        } else {
+            if (act) quantize_block_lane(o, live, qplane, ds, row, k, e0);
+        }
     }
 }
 
 // h = silu(gate) * up, optional f32 output, optional Q8_1 output; one lane per 4 elements
+template <bool Q8K>
 __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ gate, const float *__restrict__ up, int64_t in_stride,
                                                       float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k,
                                                       int64_t nrows) {
@@ -104,7 +117,16 @@ __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ 
     }
     if (act) {
         int8_t *qplane = (int8_t *)act;
-        quantize_block_lane(o, live, qplane, (act_ds *)(qplane + nrows * k), row, k, e0);
+        if constexpr (Q8K) {
+            if (live) {   // whole wave: k is a multiple of 256
+                const int64_t nsb = k >> 8, sb = e0 >> 8;
+                float *d8 = (float *)(qplane + q8k_d_offset(k, nrows));
+                _Float16 *bs = (_Float16 *)(qplane + q8k_bs_offset(k, nrows));
+                q8k_quantize_wave(o, threadIdx.x & 63, qplane + row * k + sb * QKK, d8 + row * nsb + sb, bs + (row * nsb + sb) * 16);
+            }
+        } else {
+            quantize_block_lane(o, live, qplane, (act_ds *)(qplane + nrows * k), row, k, e0);
+        }
     }
 }
 
@@ -178,9 +200,10 @@ using namespace mi355;
 
 extern "C" {
 
-int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
-                             int64_t k, int64_t nrows, float eps) {
+static int rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act, int64_t k,
+                              int64_t nrows, float eps, bool q8k) {
     MI355_REQUIRE(k > 0 && k % 32 == 0 && k <= 16384, "rms_norm_mul_quant: k=%lld must be a multiple of 32 and at most 16384", (long long)k);
+    MI355_REQUIRE(!q8k || k % QKK == 0, "rms_norm_mul_quant: k=%lld is not a multiple of 256", (long long)k);
     MI355_REQUIRE(nrows >= 0 && nrows < 0x7fffffff, "rms_norm_mul_quant: bad row count");
     MI355_REQUIRE(((uintptr_t)x & 15) == 0 && x_stride % 4 == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0 && y_stride % 4 == 0 &&
                   ((uintptr_t)act & 15) == 0, "rms_norm_mul_quant: operands must be 16-byte aligned");
@@ -188,23 +211,51 @@ int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, con
     if (nrows == 0) return MI355_OK;
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((unsigned)nrows), block(256);
-    if (k <= 4096) hipLaunchKernelGGL(k_rms_norm_mul_quant<4>, grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);
-    else if (k <= 8192) hipLaunchKernelGGL(k_rms_norm_mul_quant<8>, grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);
-    else hipLaunchKernelGGL(k_rms_norm_mul_quant<16>, grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);
+#define MI355_LAUNCH_NORM(NV)                                                                                                        \
+    do {                                                                                                                              \
+        if (q8k) hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, true>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
+        else hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, false>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);     \
+    } while (0)
+    if (k <= 4096) MI355_LAUNCH_NORM(4);
+    else if (k <= 8192) MI355_LAUNCH_NORM(8);
+    else MI355_LAUNCH_NORM(16);
+#undef MI355_LAUNCH_NORM
     return launch_status("k_rms_norm_mul_quant");
 }
 
-int mi355_swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
-                       int64_t k, int64_t nrows) {
+int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
+                             int64_t k, int64_t nrows, float eps) {
+    return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, false);
+}
+
+int mi355_rms_norm_mul_quant_q8k(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
+                                 int64_t k, int64_t nrows, float eps) {
+    return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, true);
+}
+
+static int swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act, int64_t k,
+                        int64_t nrows, bool q8k) {
     MI355_REQUIRE(k > 0 && k % 32 == 0, "swiglu_quant: k=%lld must be a multiple of 32", (long long)k);
+    MI355_REQUIRE(!q8k || k % QKK == 0, "swiglu_quant: k=%lld is not a multiple of 256", (long long)k);
     MI355_REQUIRE(nrows >= 0 && nrows <= 65535, "swiglu_quant: bad row count");
     MI355_REQUIRE(((uintptr_t)gate & 15) == 0 && ((uintptr_t)up & 15) == 0 && in_stride % 4 == 0 && ((uintptr_t)y & 15) == 0 && y_stride % 4 == 0 &&
                   ((uintptr_t)act & 15) == 0, "swiglu_quant: operands must be 16-byte aligned");
     MI355_REQUIRE(y != nullptr || act != nullptr, "swiglu_quant: no output requested");
     if (nrows == 0) return MI355_OK;
-    hipLaunchKernelGGL(k_swiglu_quant, dim3((unsigned)((k + 1023) / 1024), (unsigned)nrows), dim3(256), 0, (hipStream_t)stream, gate, up,
-                       in_stride, y, y_stride, act, k, nrows);
+    const dim3 grid((unsigned)((k + 1023) / 1024), (unsigned)nrows), block(256);
+    if (q8k) hipLaunchKernelGGL(k_swiglu_quant<true>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
+    else hipLaunchKernelGGL(k_swiglu_quant<false>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
     return launch_status("k_swiglu_quant");
+}
+
+int mi355_swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
+                       int64_t k, int64_t nrows) {
+    return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, false);
+}
+
+int mi355_swiglu_quant_q8k(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
+                           int64_t k, int64_t nrows) {
+    return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, true);
 }
 
 int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, void *kcache, void *vcache, const int32_t *pos,

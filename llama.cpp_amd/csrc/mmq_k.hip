@@ -29,6 +29,7 @@
 // and k bytes [16*(l/32), +16) (f16: k slots [8*(l/32), +8)); D register r of lane l is
 // i = 8*(r/4) + 4*(l/32) + r%4, j = l % 32.
 #include "common.hpp"
+#include "q8k.hpp"
 #include "qdot.hpp"
 
 namespace mi355 {
@@ -39,13 +40,6 @@ typedef short i16x2 __attribute__((ext_vector_type(2)));
 constexpr int KQ_BK = 128;            // K elements per stage (half a super-block)
 constexpr int KQ_LDK = KQ_BK + 16;    // LDS row pitch in bytes
 
-// ---- activation layout: int8 q[B][K]; float d8[B][K/256]; fp16 bs[B][K/256][16]
-// bs = {bsum_j & 63 (j = 0..7), bsum_j >> 6 (j = 0..7)} of the eight 32-element sub-blocks
-__host__ __device__ inline size_t q8k_d_offset(int64_t K, int64_t B) { return (size_t)B * (size_t)K; }
-__host__ __device__ inline size_t q8k_bs_offset(int64_t K, int64_t B) {
-    return (q8k_d_offset(K, B) + (size_t)B * (size_t)(K / QKK) * 4 + 15) & ~(size_t)15;   // bs entries are read 16 bytes at a time
-}
-
 // One wave per (row, super-block); 4 super-blocks per group.
 __global__ void __launch_bounds__(256) k_quantize_q8k(const float *__restrict__ x, int8_t *__restrict__ q, float *__restrict__ d8,
                                                       _Float16 *__restrict__ bs, int64_t K, int64_t x_stride) {
@@ -55,45 +49,7 @@ __global__ void __launch_bounds__(256) k_quantize_q8k(const float *__restrict__ 
     const int64_t nsb = K / QKK;
     if (sb >= nsb) return;   // whole wave
     const f32x4 v = *(const f32x4 *)(x + row * x_stride + sb * QKK + lane * 4);
-
-    // signed value of the first element with the largest magnitude
-    float amax = 0.0f, vmax = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float ax = fabsf(v[i]);
-        if (ax > amax) { amax = ax; vmax = v[i]; }
-    }
-    int who = lane;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float oa = __shfl_xor(amax, off, 64), ov = __shfl_xor(vmax, off, 64);
-        const int ow = __shfl_xor(who, off, 64);
-        if (oa > amax || (oa == amax && ow < who)) { amax = oa; vmax = ov; who = ow; }
-    }
-
-    int lv[4] = {0, 0, 0, 0};
-    float d = 0.0f;
-    if (amax != 0.0f) {
-        const float iscale = -127.0f / vmax;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int n = (int)rintf(iscale * v[i]);
-            lv[i] = n < 127 ? n : 127;
-        }
-        d = 1.0f / iscale;
-    }
-    int sum = lv[0] + lv[1] + lv[2] + lv[3];
-#pragma unroll
-    for (int off = 1; off < 8; off <<= 1) sum += __shfl_xor(sum, off, 64);
-
-    const u32 packed = (u32)(lv[0] & 0xFF) | ((u32)(lv[1] & 0xFF) << 8) | ((u32)(lv[2] & 0xFF) << 16) | ((u32)(lv[3] & 0xFF) << 24);
-    *(u32 *)(q + row * K + sb * QKK + lane * 4) = packed;
-    if (lane == 0) d8[row * nsb + sb] = d;
-    if ((lane & 7) == 0) {
-        _Float16 *o = bs + (row * nsb + sb) * 16;
-        o[lane >> 3] = (_Float16)(float)(sum & 63);
-        o[8 + (lane >> 3)] = (_Float16)(float)(sum >> 6);
-    }
+    q8k_quantize_wave(v, lane, q + row * K + sb * QKK, d8 + row * nsb + sb, bs + (row * nsb + sb) * 16);
 }
 
 // ---- per-thread prefetch registers of one stage -------------------------------------------
@@ -258,9 +214,9 @@ __device__ __forceinline__ void kq_commit(const kq_regs<TYPE, WI, AI> &R, const 
 // TW x TB: 32 x 32 MFMA tiles per wave along the weight / activation rows; waves are 2 x 2
 template <int TYPE, int TW, int TB, int OCC, bool ID>
 __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq, const float *__restrict__ ad8,
-                                                    const _Float16 *__restrict__ abs_, float *__restrict__ dst, int64_t N, int64_t K,
-                                                    int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles, int n_groups,
-                                                    int n_groups_padded, mmq_route route) {
+                                                    const _Float16 *__restrict__ abs_, float *dst, const float *residual,
+                                                    int64_t N, int64_t K, int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles,
+                                                    int n_groups, int n_groups_padded, mmq_route route) {
     constexpr bool Q4 = TYPE == MI355_Q4_K;
     constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
     constexpr int BM = 64 * TW, BN = 64 * TB;
@@ -409,7 +365,10 @@ __global__ void __launch_bounds__(256, OCC) k_mmq_k(const uint8_t *__restrict__ 
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                if (n < N && b < B) dst[(ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n] = acc[tb][tw][r];
+                if (n < N && b < B) {
+                    const int64_t o = (ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n;
+                    dst[o] = residual ? acc[tb][tw][r] + residual[o] : acc[tb][tw][r];
+                }
             }
         }
 }
@@ -511,9 +470,9 @@ __device__ __forceinline__ void kp_dma_a(const int8_t *__restrict__ aq, const in
 
 template <int TYPE, bool ID>
 __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq, const float *__restrict__ ad8,
-                                                   const _Float16 *__restrict__ abs_, float *__restrict__ dst, int64_t N, int64_t K, int64_t B,
-                                                   int64_t dst_stride, row_layout L, int n_col_tiles, int n_groups, int n_groups_padded,
-                                                   mmq_route route) {
+                                                   const _Float16 *__restrict__ abs_, float *dst, const float *residual,
+                                                   int64_t N, int64_t K, int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles,
+                                                   int n_groups, int n_groups_padded, mmq_route route) {
     constexpr bool Q4 = TYPE == MI355_Q4_K;
     constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
     constexpr int BM = 64, BN = 128;
@@ -715,13 +674,17 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-            if (n < N && b < B) dst[(ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n] = acc[tb][r];
+            if (n < N && b < B) {
+                const int64_t o = (ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n;
+                dst[o] = residual ? acc[tb][r] + residual[o] : acc[tb][r];   // residual may be dst itself: one reader and writer per element
+            }
         }
     }
 }
 
 template <int TYPE>
-static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B, int64_t dst_stride) {
+static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
+                         int64_t dst_stride) {
     constexpr int BM = 64, BN = 128;
     const row_layout L = make_row_layout(TYPE, K);
     const int8_t *aq = (const int8_t *)act;
@@ -731,8 +694,8 @@ static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *d
     const int n_col_tiles = (int)((B + BN - 1) / BN);
     const int n_groups = n_row_tiles * n_col_tiles;
     const int n_groups_padded = (n_groups + 7) & ~7;
-    hipLaunchKernelGGL((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_, dst, N, K, B,
-                       dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
+    hipLaunchKernelGGL((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_, dst, residual, N, K,
+                       B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
 }
 
 // ---- MUL_MAT_ID with many slots: sort the slots by expert, then one tile launch over all experts ----
@@ -806,10 +769,10 @@ static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int6
     const mmq_route route = {act_row, dst_row, tiles, n_tiles, N * L.row_bytes};
     if (bn == 64)
         hipLaunchKernelGGL((k_mmq_k<TYPE, 1, 1, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
-                           dst, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
+                           dst, nullptr, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
     else
-        hipLaunchKernelGGL((k_mmq_kp<TYPE, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_, dst, N, K, S,
-                           N, L, max_tiles, n_groups, n_groups_padded, route);
+        hipLaunchKernelGGL((k_mmq_kp<TYPE, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_, dst, nullptr, N, K,
+                           S, N, L, max_tiles, n_groups, n_groups_padded, route);
 }
 
 }  // namespace mi355
@@ -864,8 +827,8 @@ int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act
     return launch_status("k_mmq_k (routed)");
 }
 
-int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
-                      int64_t dst_stride) {
+int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
+                          int64_t B, int64_t dst_stride) {
     MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k: weight type %d is not a K-quant", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k: K=%lld is not a multiple of 256", (long long)K);
@@ -876,9 +839,14 @@ int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, fl
                   "mul_mat_q8k: activation workspace is not 16-byte aligned");
     MI355_REQUIRE((N + 63) / 64 * ((B + 63) / 64) < (1 << 30), "mul_mat_q8k: too many tiles");
     hipStream_t s = (hipStream_t)stream;
-    if (type == MI355_Q4_K) launch_mmq_k<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride);
-    else launch_mmq_k<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride);
+    if (type == MI355_Q4_K) launch_mmq_k<MI355_Q4_K>(s, W, act, dst, residual, N, K, B, dst_stride);
+    else launch_mmq_k<MI355_Q6_K>(s, W, act, dst, residual, N, K, B, dst_stride);
     return launch_status("k_mmq_k");
+}
+
+int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                      int64_t dst_stride) {
+    return mi355_mul_mat_q8k_add(stream, type, W, act, dst, nullptr, N, K, B, dst_stride);
 }
 
 }  // extern "C"

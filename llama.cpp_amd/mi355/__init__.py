@@ -43,9 +43,12 @@ _SIGNATURES = {
     "mi355_act_q8k_bytes": (_sz, [_i64, _i64]),
     "mi355_quantize_act_q8k": (_int, [_p, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_q8k": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_mul_mat_q8k_add": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_rms_norm_mul_quant": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
     "mi355_swiglu_quant": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
+    "mi355_rms_norm_mul_quant_q8k": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
+    "mi355_swiglu_quant_q8k": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
     "mi355_rope_kv_store": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _int, _int, _int,
                                    _f, _f, _f, _f, _f, _f]),
     "mi355_ffn_gate_up_swiglu": (_int, [_p, _int, _p, _int, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64]),

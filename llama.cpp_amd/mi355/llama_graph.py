@@ -174,9 +174,8 @@ class LlamaRunner:
 
     def _norm_quant(self, x, w, act, T, q8k=False):
         K = x.shape[1]
-        if q8k:     # prefill: normalised rows in f32, then one scale per 256 elements
-            check(self.lib.mi355_rms_norm_mul_quant(_stream(), _ptr(x), x.stride(0), _ptr(w), _ptr(self.t0), self.t0.stride(0), None, K, T, self.cfg.rms_eps))
-            self._quant(self.t0, act, K, T, True)
+        if q8k:     # prefill: one scale per 256 elements
+            check(self.lib.mi355_rms_norm_mul_quant_q8k(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
         else:
             check(self.lib.mi355_rms_norm_mul_quant(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
 
@@ -189,10 +188,13 @@ class LlamaRunner:
                 arr[i].residual = residual.data_ptr() if residual is not None else None
             check(self.lib.mi355_mul_mat_vec_q_multi(_stream(), len(mats), arr, _ptr(act), K, T))
         else:
-            fn = self.lib.mi355_mul_mat_q8k if q8k else self.lib.mi355_mul_mat_q
             for (t, W), out in mats:
+                if q8k:     # the residual add is the tile kernel's epilogue
+                    check(self.lib.mi355_mul_mat_q8k_add(_stream(), t, _ptr(W), _ptr(act), _ptr(out), _ptr(residual) if residual is not None else None,
+                                                         out.shape[1], K, T, out.stride(0)))
+                    continue
                 dst = out if residual is None else self.t1[:T]
-                check(fn(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), out.shape[1], K, T, dst.stride(0)))
+                check(self.lib.mi355_mul_mat_q(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), out.shape[1], K, T, dst.stride(0)))
                 if residual is not None:
                     self._bin(0, dst, residual, out)
 
@@ -234,8 +236,7 @@ class LlamaRunner:
             down = [(L["down"], x)]
             kq = big and self._q8k_ok(down, F)
             if kq:
-                check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, _ptr(self.gate), F, None, F, T))
-                self._quant(self.gate, self.act_b, F, T, True)
+                check(lib.mi355_swiglu_quant_q8k(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
             else:
                 check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
             self._mm_act(down, self.act_b, F, T, residual=x, q8k=kq)

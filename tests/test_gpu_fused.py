@@ -221,3 +221,57 @@ def test_tail_fused_launches_equal_separate_kernels(dev, B):
         assert torch.equal(g1, g0) and torch.equal(u1, u0)
         assert torch.equal(a1, a0)
         assert int(tickets.abs().sum().item()) == 0
+
+
+@pytest.mark.parametrize("K,nrows", [(4096, 40), (14336, 9), (2048, 512)])
+def test_q8k_outputs_of_fused_kernels_equal_separate_quantization(dev, K, nrows):
+    """RMS_NORM+MUL and SiLU*up writing the per-super-block activation format directly: same bytes as quantizing their f32 output"""
+    import torch
+    import mi355
+    lib = mi355.load()
+    g = torch.Generator().manual_seed(K + nrows)
+    x = torch.randn(nrows, K, generator=g).to(dev)
+    w = (1.0 + 0.1 * torch.randn(K, generator=g)).to(dev)
+    n = int(lib.mi355_act_q8k_bytes(K, nrows))
+    y = torch.empty_like(x)
+    act = torch.zeros(n + 256, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_rms_norm_mul_quant_q8k(None, mi355._ptr(x), K, mi355._ptr(w), mi355._ptr(y), K, mi355._ptr(act), K, nrows, 1e-5))
+    y2 = torch.empty_like(x)
+    mi355.check(lib.mi355_rms_norm_mul_quant(None, mi355._ptr(x), K, mi355._ptr(w), mi355._ptr(y2), K, None, K, nrows, 1e-5))
+    assert torch.equal(y, y2)
+    want = mi355.quantize_act_q8k(y2)
+    pad = int(K * nrows + nrows * (K // 256) * 4)     # the gap between the scales and the 16-byte aligned sums is not written
+    bs0 = (pad + 15) // 16 * 16
+    assert torch.equal(act[:pad], want[:pad]) and torch.equal(act[bs0:n], want[bs0:n])
+    up = torch.randn(nrows, K, generator=g).to(dev)
+    h = torch.empty_like(x)
+    act2 = torch.zeros(n + 256, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_swiglu_quant_q8k(None, mi355._ptr(x), mi355._ptr(up), K, mi355._ptr(h), K, mi355._ptr(act2), K, nrows))
+    h2 = torch.empty_like(x)
+    mi355.check(lib.mi355_swiglu_quant(None, mi355._ptr(x), mi355._ptr(up), K, mi355._ptr(h2), K, None, K, nrows))
+    assert torch.equal(h, h2)
+    want = mi355.quantize_act_q8k(h2)
+    assert torch.equal(act2[:pad], want[:pad]) and torch.equal(act2[bs0:n], want[bs0:n])
+
+
+@pytest.mark.parametrize("name,t", [("q4_K", orc.Q4_K), ("q6_K", orc.Q6_K)])
+def test_tile_gemm_residual_epilogue(dev, name, t):
+    """MUL_MAT + ADD(residual) in the tile kernel's epilogue, also in place"""
+    import torch
+    import mi355
+    from mi355 import llama_graph as lg
+    lib = mi355.load()
+    N, K, B = 320, 2048, 70
+    gen = torch.Generator(device=dev).manual_seed(3)
+    W = mi355.upload_weights(t, lg.random_quantized(t, N, K, dev, gen))
+    x = torch.randn(B, K, device=dev, generator=gen)
+    res = torch.randn(B, N, device=dev, generator=gen)
+    act = mi355.quantize_act_q8k(x)
+    plain = torch.empty(B, N, device=dev)
+    mi355.check(lib.mi355_mul_mat_q8k(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(plain), N, K, B, N))
+    fused = torch.empty(B, N, device=dev)
+    mi355.check(lib.mi355_mul_mat_q8k_add(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(fused), mi355._ptr(res), N, K, B, N))
+    assert torch.equal(fused, plain + res)
+    inplace = res.clone()
+    mi355.check(lib.mi355_mul_mat_q8k_add(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(inplace), mi355._ptr(inplace), N, K, B, N))
+    assert torch.equal(inplace, plain + res)
