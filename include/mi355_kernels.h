@@ -106,6 +106,21 @@ int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, fl
 int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
                           int64_t B, int64_t dst_stride);
 
+/* Second, unpacked copy of K-quant weights for the tile GEMM: the two int8 planes whose weighted sum R*hi + lo is the integer
+ * sub-scale times the level (sc*n for Q4_K with R = 8, sc*(l-32) for Q6_K with R = 64; dequantize_row_q4_K / _q6_K,
+ * ggml/src/ggml-quants.c:1280-1302, 1690-1719), 2 bytes per weight: int8 hi[rows][K], int8 lo[rows][K], then 48 bytes per
+ * (row, super-block): the eight sub-block mins as f16, the same times 64 as f16, and {d, dmin} as f32 (Q6_K: only d).
+ * Written once per weight matrix (K % 256 == 0, rows 16-byte aligned as for mi355_mul_mat_q8k); mi355_mul_mat_q8k_planes then
+ * streams the planes straight into LDS and computes exactly what mi355_mul_mat_q8k_add computes (same integer sums, same f32
+ * arithmetic, bit-identical dst) without touching the packed rows.  It pays for Q6_K, whose unpack costs the most vector
+ * instructions per weight (about 1.35x the in-kernel-unpack rate at batch 512); for Q4_K the two run at the same speed, so
+ * callers keep planes for Q6_K matrices only.  No counterpart in the reference, which unpacks in its mmq tile loaders
+ * (ggml/src/ggml-cuda/mmq.cuh load_tiles_q6_K). */
+size_t mi355_kq_planes_bytes(int64_t rows, int64_t K);
+int mi355_kq_unpack_planes(void *stream, int type, const void *W, void *planes, int64_t rows, int64_t K);
+int mi355_mul_mat_q8k_planes(void *stream, int type, const void *planes, const void *act, float *dst, const float *residual, int64_t N,
+                             int64_t K, int64_t B, int64_t dst_stride);
+
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE
  * launch, each optionally adding a residual in its epilogue (the ggml_add that follows the wo and

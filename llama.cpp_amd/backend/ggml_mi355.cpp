@@ -197,11 +197,55 @@ staging & stage() {
     return s;
 }
 
+// Unpacked int8 planes of Q6_K weight matrices for the tile GEMM (mi355_kq_unpack_planes), built the first time a matrix in a
+// weights buffer meets a batch above 8 and kept until that buffer is freed or the tensor is written again.  Keyed by the
+// tensor's data address.  MI355_NO_PLANES=1 keeps the packed rows only (2 bytes per Q6_K weight less device memory).
+struct plane_store {
+    std::mutex mu;
+    struct entry { void * planes; int64_t rows, K; };
+    std::unordered_map<const void *, entry> map;
+    bool enabled = getenv("MI355_NO_PLANES") == nullptr;
+
+    const void * get(hipStream_t s, const ggml_tensor * w) {
+        if (!enabled || w->type != GGML_TYPE_Q6_K || w->buffer == nullptr || w->buffer->usage != GGML_BACKEND_BUFFER_USAGE_WEIGHTS) return nullptr;
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = map.find(w->data);
+        if (it != map.end()) return it->second.rows == w->ne[1] && it->second.K == w->ne[0] ? it->second.planes : nullptr;
+        if (!ggml_is_contiguous(w)) return nullptr;
+        void * planes = nullptr;
+        if (hipMalloc(&planes, mi355_kq_planes_bytes(w->ne[1], w->ne[0]) + 256) != hipSuccess) {   // out of memory: stay with the packed rows
+            (void) hipGetLastError();
+            enabled = false;
+            return nullptr;
+        }
+        MI355_K_OK(mi355_kq_unpack_planes(s, to_mi355_type(w->type), w->data, planes, w->ne[1], w->ne[0]));
+        map.emplace(w->data, entry{planes, w->ne[1], w->ne[0]});
+        return planes;
+    }
+    // forget (and free) the planes of tensors whose data lies in [base, base + size); the caller has synchronized the device
+    void drop(const void * base, size_t size) {
+        std::lock_guard<std::mutex> lock(mu);
+        for (auto it = map.begin(); it != map.end();) {
+            if ((const char *) it->first >= (const char *) base && (const char *) it->first < (const char *) base + size) {
+                MI355_HIP_OK(hipFree(it->second.planes));
+                it = map.erase(it);
+            } else {
+                ++it;
+            }
+        }
+    }
+};
+plane_store & planes() {
+    static plane_store p;
+    return p;
+}
+
 // ------------------------------------------------------------------------------- buffer
 void buffer_free(ggml_backend_buffer_t buffer) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
+    planes().drop(ctx->base, ctx->size);
     if (ctx->base) MI355_HIP_OK(hipFree(ctx->base));
     delete ctx;
 }
@@ -216,6 +260,7 @@ void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
     if (size == 0) return;
+    if (tensor->type == GGML_TYPE_Q6_K) planes().drop(tensor->data, ggml_nbytes(tensor));   // rebuilt from the new contents on next use
     if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
         std::lock_guard<std::mutex> lock(stage().mu);
         void * tmp = stage().get(size);
@@ -262,6 +307,7 @@ bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, gg
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
+    if (dst->type == GGML_TYPE_Q6_K) planes().drop(dst->data, ggml_nbytes(dst));
     MI355_HIP_OK(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyDeviceToDevice));
     MI355_HIP_OK(hipDeviceSynchronize());
     return true;
@@ -271,6 +317,7 @@ void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
+    planes().drop(ctx->base, ctx->size);
     MI355_HIP_OK(hipMemset(ctx->base, value, ctx->size));
     MI355_HIP_OK(hipDeviceSynchronize());
 }
@@ -1114,19 +1161,31 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
             ctx->cache = act_cache{b->data, K, B, ACT_Q8K, true, fresh};
         }
+        const void * pl = planes().get(s, node->src[0]);   // Q6_K weights: the unpacked planes, built on first use
+        const int wtype = to_mi355_type(node->src[0]->type);
         // MUL_MAT -> ADD(residual): the sum goes straight into the ADD's tensor
         ggml_tensor * add = nxt;
         if (add && add->op == GGML_OP_ADD && w.sole_use(i) && (add->src[0] == node || add->src[1] == node)) {
             const ggml_tensor * res = add->src[0] == node ? add->src[1] : add->src[0];
             if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, node) && ggml_is_contiguous(res) && ggml_is_contiguous(add) && ggml_is_contiguous(node)) {
-                MI355_K_OK(mi355_mul_mat_q8k_add(s, to_mi355_type(node->src[0]->type), node->src[0]->data, ctx->cache.ptr, (float *) add->data,
-                                                 (const float *) res->data, node->src[0]->ne[1], K, B, (int64_t) (add->nb[1] / sizeof(float))));
+                if (pl) {
+                    MI355_K_OK(mi355_mul_mat_q8k_planes(s, wtype, pl, ctx->cache.ptr, (float *) add->data, (const float *) res->data, node->src[0]->ne[1],
+                                                        K, B, (int64_t) (add->nb[1] / sizeof(float))));
+                } else {
+                    MI355_K_OK(mi355_mul_mat_q8k_add(s, wtype, node->src[0]->data, ctx->cache.ptr, (float *) add->data, (const float *) res->data,
+                                                     node->src[0]->ne[1], K, B, (int64_t) (add->nb[1] / sizeof(float))));
+                }
                 ctx->note_write(add->data, ggml_nbytes(add));
                 return j;
             }
         }
-        MI355_K_OK(mi355_mul_mat_q8k(s, to_mi355_type(node->src[0]->type), node->src[0]->data, ctx->cache.ptr, (float *) node->data, node->src[0]->ne[1], K, B,
-                                     (int64_t) (node->nb[1] / sizeof(float))));
+        if (pl) {
+            MI355_K_OK(mi355_mul_mat_q8k_planes(s, wtype, pl, ctx->cache.ptr, (float *) node->data, nullptr, node->src[0]->ne[1], K, B,
+                                                (int64_t) (node->nb[1] / sizeof(float))));
+        } else {
+            MI355_K_OK(mi355_mul_mat_q8k(s, wtype, node->src[0]->data, ctx->cache.ptr, (float *) node->data, node->src[0]->ne[1], K, B,
+                                         (int64_t) (node->nb[1] / sizeof(float))));
+        }
         ctx->note_write(node->data, ggml_nbytes(node));
         return i;
     }

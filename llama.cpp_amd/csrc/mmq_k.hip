@@ -455,17 +455,22 @@ __device__ __forceinline__ void kp_store(const kp_planes &P, int8_t *__restrict_
     *(u32x4 *)(sW0 + kp_off(r, c1)) = P.b0;
 }
 
-// activations of one stage: 32 * AI rows x 128 bytes, AI wave-wide 16-byte transfers per wave
+// activations of one stage: 32 * AI rows x 128 bytes, AI wave-wide 16-byte transfers per wave.  aofs: per-lane byte offsets of
+// the 16 bytes this lane moves (row * K + swizzled chunk, fixed for the whole kernel); base: uniform pointer to the stage.
 template <int AI>
-__device__ __forceinline__ void kp_dma_a(const int8_t *__restrict__ aq, const int (&arow)[AI], int64_t K, int64_t k0, int8_t *__restrict__ sA) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__device__ __forceinline__ void kp_dma_a(const int8_t *__restrict__ base, const unsigned (&aofs)[AI], int8_t *__restrict__ sA) {
+    const int wave = threadIdx.x >> 6;
 #pragma unroll
-    for (int it = 0; it < AI; it++) {
-        const int row = (wave * AI + it) * 8 + (lane >> 3);
-        const int c = (lane & 7) ^ ((row >> 1) & 7);   // the logical chunk that belongs at this lane's position
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(aq + (int64_t)arow[it] * K + k0 + c * 16),
+    for (int it = 0; it < AI; it++)
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(base + aofs[it]),
                                          (void __attribute__((address_space(3))) *)(sA + (wave * AI + it) * 1024), 16, 0, 0);
-    }
+}
+// row of transfer `it` of this lane and the logical chunk that belongs at the lane's LDS position
+template <int AI>
+__device__ __forceinline__ void kp_dma_slot(int it, int &row, int &chunk) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    row = (wave * AI + it) * 8 + (lane >> 3);
+    chunk = (lane & 7) ^ ((row >> 1) & 7);
 }
 
 template <int TYPE, bool ID>
@@ -484,6 +489,9 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
     __shared__ __attribute__((aligned(16))) _Float16 sWm[2][Q4 ? BM * 16 : 8];
     __shared__ __attribute__((aligned(16))) float sAd[2][BN];
     __shared__ __attribute__((aligned(16))) _Float16 sAs[2][Q4 ? BN * 16 : 8];
+    // sAa / sAb_ are written by global-to-LDS transfers only; a transfer names the wave's first 16 bytes, so to the compiler most
+    // of these arrays is never stored to.  The empty asm makes them memory that unknown code may have written.
+    asm volatile("" ::"v"((void *)sAa), "v"((void *)sAb_) : "memory");
 
     const int per_xcd = n_groups_padded >> 3;
     const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
@@ -508,12 +516,14 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
     // this thread's weight row, the activation rows of its four transfers, and the column whose scales it copies
     const int64_t wr = row0 + (tid >> 2) < N ? row0 + (tid >> 2) : N - 1;
     const uint8_t *wrow = W + wr * L.row_bytes;
-    int arow[4];
+    unsigned aofs[4];
 #pragma unroll
     for (int it = 0; it < 4; it++) {
-        const int64_t col = col0 + (wave * 4 + it) * 8 + (lane >> 3);
+        int r, c;
+        kp_dma_slot<4>(it, r, c);
+        const int64_t col = col0 + r;
         const int64_t cc = col < B ? col : B - 1;
-        arow[it] = ID ? route.act_row[cc] : (int)cc;
+        aofs[it] = (unsigned)((int64_t)(ID ? route.act_row[cc] : (int)cc) * K + c * 16);
     }
     int srow;
     {
@@ -538,21 +548,19 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
         sAd[sbuf][tid >> 1] = d8;   // both threads of the column write the same value: an unconditional use keeps the load where it was issued
         if constexpr (Q4) {
             *(u32x4 *)(sAs[sbuf] + (tid >> 1) * 16 + 8 * (tid & 1)) = bs;
-            if ((tid & 3) == 0) {
-                const int r = tid >> 2;
-                sWd[sbuf][r] = half_bits_to_float((unsigned short)(H.hdr[0] & 0xFFFFu));
-                sWn[sbuf][r] = half_bits_to_float((unsigned short)(H.hdr[0] >> 16));
-                f16x8 m1, m64;
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    int sc, mn;
-                    q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], j, sc, mn);
-                    m1[j] = (_Float16)(float)mn;
-                    m64[j] = (_Float16)(float)(64 * mn);
-                }
-                *(f16x8 *)(sWm[sbuf] + r * 16) = m1;
-                *(f16x8 *)(sWm[sbuf] + r * 16 + 8) = m64;
-            }
+            // the four threads of a row share the work (and all use the header, so its load stays where it was issued):
+            // each writes d, dmin (same values) and the mins of sub-blocks 2p, 2p + 1
+            const int r = tid >> 2, p2 = 2 * (tid & 3);
+            sWd[sbuf][r] = half_bits_to_float((unsigned short)(H.hdr[0] & 0xFFFFu));
+            sWn[sbuf][r] = half_bits_to_float((unsigned short)(H.hdr[0] >> 16));
+            int sc, mn0, mn1;
+            q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], p2, sc, mn0);
+            q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], p2 + 1, sc, mn1);
+            typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+            const f16x2 m1 = {(_Float16)(float)mn0, (_Float16)(float)mn1};
+            const f16x2 m64 = {(_Float16)(float)(64 * mn0), (_Float16)(float)(64 * mn1)};
+            *(f16x2 *)(sWm[sbuf] + r * 16 + p2) = m1;
+            *(f16x2 *)(sWm[sbuf] + r * 16 + 8 + p2) = m64;
         } else {
             sWd[sbuf][tid >> 2] = half_bits_to_float(H.d);   // the four threads of a row write the same value
         }
@@ -566,7 +574,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
     kp_fetch_w<TYPE>(R0, wrow, L, 0, 0);
     kp_fetch_w<TYPE>(R1, wrow, L, 0, 1);
     kp_fetch_h<TYPE>(Hc, wrow, L, 0);
-    kp_dma_a<4>(aq, arow, K, 0, sAa);
+    kp_dma_a<4>(aq, aofs, sAa);
     fetch_scales(0, d8n, bsn);
     {
         kp_planes P;
@@ -593,7 +601,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
             // Past the end of K the same work is done on the last super-block again and never read: no branches in the stage,
             // so the compiler schedules it as one block.
             const int64_t sb1 = sb + 1 < nsb ? sb + 1 : sb;
-            kp_dma_a<4>(aq, arow, K, half == 0 ? sb * QKK + 128 : sb1 * QKK, nA);
+            kp_dma_a<4>(aq + (half == 0 ? sb * QKK + 128 : sb1 * QKK), aofs, nA);
             if (half == 1) fetch_scales(sb1, d8n, bsn);
             kp_fetch_w<TYPE>(Rf, wrow, L, sb1, half);
             if (half == 0) kp_fetch_h<TYPE>(Hn, wrow, L, sb1);   // used from the next stage on
@@ -660,7 +668,327 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
                     }
                 }
             }
-            if (half == 1) {   // last, so that the loads had the whole stage
+            if (half == 1) {   // last, so that the loads had the whole stage (the barrier keeps the scheduler from hoisting the wait)
+                __builtin_amdgcn_sched_barrier(0);
+                store_scales((int)((sb + 1) & 1), d8n, bsn, Hn);
+                Hc = Hn;
+            }
+            __syncthreads();   // also waits for this stage's transfers and loads (issued a whole stage ago)
+        }
+    }
+
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++) {
+        const int64_t n = row0 + wrow0 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if (n < N && b < B) {
+                const int64_t o = (ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n;
+                dst[o] = residual ? acc[tb][r] + residual[o] : acc[tb][r];   // residual may be dst itself: one reader and writer per element
+            }
+        }
+    }
+}
+
+// ---- planes kept in HBM ----------------------------------------------------------------------------------------------------
+// The vector ALU is what limits k_mmq_kp (about 11 instructions per matrix instruction, 4 of them the unpack).  With 288 GB of
+// HBM a second, unpacked copy of the K-quant weights is affordable (2 bytes per weight: the two int8 planes, written once by
+// k_unpack_planes when the weights are uploaded): k_mmq_pl brings both planes of a stage from global memory straight into
+// LDS, like the activations, and spends no vector instruction on the weights.  The packed copy stays the one the GEMV
+// streams.  planes: int8 hi[N][K], int8 lo[N][K], then 48 bytes per (row, super-block): the eight mins as f16, the eight mins
+// times 64 as f16 (the two operand rows of the min-term matrix instruction), and {d, dmin} as f32.
+template <int TYPE>
+__global__ void __launch_bounds__(256) k_unpack_planes(const uint8_t *__restrict__ W, int8_t *__restrict__ planes, int64_t N, int64_t K,
+                                                       row_layout L) {
+    // one thread per 16-byte piece: row, super-block, half, piece = the unpack of k_mmq_kp
+    const int64_t per_row = (K >> 8) * 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= N * per_row) return;
+    const int64_t row = idx / per_row, rem = idx % per_row, sb = rem >> 3;
+    const int half = (int)((rem >> 2) & 1), p = (int)(rem & 3);
+    const uint8_t *wrow = W + row * L.row_bytes;
+    u32x4 a1, a0, b1, b0;
+    int c0, c1;
+    if constexpr (TYPE == MI355_Q4_K) {
+        const uint8_t *blk = wrow + sb * Q4_K_BYTES;
+        const u32x4 q = load16(blk + 16 + (half * 2 + (p >> 1)) * 32 + (p & 1) * 16);
+        const u32x4 hdr = load16(blk);
+        const int gl = p >> 1;
+        int scl, mnl, sch, mnh;
+        q4k_scale_min(hdr[1], hdr[2], hdr[3], half * 4 + 2 * gl, scl, mnl);
+        q4k_scale_min(hdr[1], hdr[2], hdr[3], half * 4 + 2 * gl + 1, sch, mnh);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const u32 nl = q[i] & 0x0F0F0F0Fu, nh = (q[i] >> 4) & 0x0F0F0F0Fu;
+            a1[i] = mul_bytes(nl, (u32)scl >> 3);
+            a0[i] = mul_bytes(nl, (u32)scl & 7u);
+            b1[i] = mul_bytes(nh, (u32)sch >> 3);
+            b0[i] = mul_bytes(nh, (u32)sch & 7u);
+        }
+        c0 = 4 * gl + (p & 1);
+        c1 = c0 + 2;
+    } else {
+        const int l0 = 16 * (p & 1), qa = p >> 1;
+        const u32x4 ql = load16(wrow + sb * 128 + half * 64 + p * 16);
+        const u32x4 qh = load16(wrow + L.off_b + sb * 64 + half * 32 + l0);
+        const int8_t *sc = (const int8_t *)(wrow + L.off_c + sb * 16 + half * 8 + (l0 >> 4));
+        const int scA = sc[2 * qa], scB = sc[2 * qa + 4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const u32 va = (ql[i] & 0x0F0F0F0Fu) | (((qh[i] >> (2 * qa)) & 0x03030303u) << 4);
+            const u32 vb = ((ql[i] >> 4) & 0x0F0F0F0Fu) | (((qh[i] >> (2 * qa + 4)) & 0x03030303u) << 4);
+            u32 hi, lo;
+            q6k_planes(va, scA, hi, lo);
+            a1[i] = hi; a0[i] = lo;
+            q6k_planes(vb, scB, hi, lo);
+            b1[i] = hi; b0[i] = lo;
+        }
+        c0 = 2 * qa + (p & 1);
+        c1 = c0 + 4;
+    }
+    if (half == 0 && p == 0) {   // the row's per-super-block data behind the planes: three 16-byte chunks
+        u32x4 *aux = (u32x4 *)(planes + 2 * N * K) + (row * (K >> 8) + sb) * 3;
+        if constexpr (TYPE == MI355_Q4_K) {
+            const u32x4 hdr = load16(wrow + sb * Q4_K_BYTES);
+            f16x8 m1, m64;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                int sc, mn;
+                q4k_scale_min(hdr[1], hdr[2], hdr[3], j, sc, mn);
+                m1[j] = (_Float16)(float)mn;
+                m64[j] = (_Float16)(float)(64 * mn);
+            }
+            aux[0] = __builtin_bit_cast(u32x4, m1);
+            aux[1] = __builtin_bit_cast(u32x4, m64);
+            const float d = half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu)), dmin = half_bits_to_float((unsigned short)(hdr[0] >> 16));
+            aux[2] = u32x4{__builtin_bit_cast(u32, d), __builtin_bit_cast(u32, dmin), 0u, 0u};
+        } else {
+            const float d = half_bits_to_float(*(const unsigned short *)(wrow + L.off_d + sb * 2));
+            aux[0] = u32x4{0u, 0u, 0u, 0u};
+            aux[1] = u32x4{0u, 0u, 0u, 0u};
+            aux[2] = u32x4{__builtin_bit_cast(u32, d), 0u, 0u, 0u};
+        }
+    }
+    int8_t *hi = planes + row * K + sb * QKK + half * 128, *lo = hi + N * K;
+    *(u32x4 *)(hi + c0 * 16) = a1;
+    *(u32x4 *)(lo + c0 * 16) = a0;
+    *(u32x4 *)(hi + c1 * 16) = b1;
+    *(u32x4 *)(lo + c1 * 16) = b0;
+}
+
+// what a thread of k_mmq_pl moves per super-block from the 48-byte entry k_unpack_planes wrote behind the planes to LDS: thread
+// p of the four that share a row takes the mins of sub-blocks 2p, 2p + 1 (plain and times 64, ready as f16) and {d, dmin}.
+// Only bytes that are used are loaded: a loaded register that is dead gets reused at once, and that write waits for the load.
+template <int TYPE> struct pl_h { u32 v[TYPE == MI355_Q4_K ? 4 : 1]; };
+template <int TYPE>
+__device__ __forceinline__ void pl_fetch_h(pl_h<TYPE> &H, const u32 *__restrict__ aux_row, int64_t sb) {
+    const u32 *a = aux_row + sb * 12;
+    if constexpr (TYPE == MI355_Q4_K) {
+        const int p = threadIdx.x & 3;
+        H.v[0] = a[p];
+        H.v[1] = a[4 + p];
+        H.v[2] = a[8];
+        H.v[3] = a[9];
+    } else {
+        H.v[0] = a[8];
+    }
+}
+
+template <int TYPE, bool ID>
+__global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ planes, const int8_t *__restrict__ aq, const float *__restrict__ ad8,
+                                                   const _Float16 *__restrict__ abs_, float *dst, const float *residual,
+                                                   int64_t N, int64_t K, int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles,
+                                                   int n_groups, int n_groups_padded, mmq_route route, int64_t plane_stride) {
+    constexpr bool Q4 = TYPE == MI355_Q4_K;
+    constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
+    constexpr int BM = 64, BN = 128;
+    __shared__ __attribute__((aligned(16))) int8_t sW1a[BM * KP_ROW], sW1b[BM * KP_ROW];
+    __shared__ __attribute__((aligned(16))) int8_t sW0a[BM * KP_ROW], sW0b[BM * KP_ROW];
+    __shared__ __attribute__((aligned(16))) int8_t sAa[BN * KP_ROW], sAb_[BN * KP_ROW];
+    __shared__ __attribute__((aligned(16))) float sWd[2][BM];
+    __shared__ __attribute__((aligned(16))) float sWn[2][Q4 ? BM : 4];
+    __shared__ __attribute__((aligned(16))) _Float16 sWm[2][Q4 ? BM * 16 : 8];
+    __shared__ __attribute__((aligned(16))) float sAd[2][BN];
+    __shared__ __attribute__((aligned(16))) _Float16 sAs[2][Q4 ? BN * 16 : 8];
+    // The tile buffers are written by global-to-LDS transfers only; a transfer names the wave's first 16 bytes, so to the compiler
+    // most of these arrays is never stored to.  The empty asm makes them memory that unknown code may have written.
+    asm volatile("" ::"v"((void *)sAa), "v"((void *)sAb_), "v"((void *)sW1a), "v"((void *)sW1b), "v"((void *)sW0a), "v"((void *)sW0b) : "memory");
+
+    const int per_xcd = n_groups_padded >> 3;
+    const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (lid >= n_groups) return;
+    const int64_t row0 = (int64_t)(lid / n_col_tiles) * BM;
+    int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+    int64_t plane_base = 0;
+    if constexpr (ID) {
+        const int ct = lid % n_col_tiles;
+        if (ct >= *route.n_tiles) return;
+        plane_base = (int64_t)route.tiles[4 * ct] * N * K;
+        col0 = route.tiles[4 * ct + 1];
+        B = route.tiles[4 * ct + 2];
+    }
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int wrow0 = (wave & 1) * 32;    // weight rows of this wave inside the tile
+    const int wcol0 = (wave >> 1) * 64;   // activation rows of this wave inside the tile
+    const int64_t nsb = K >> 8;
+
+    // this thread's weight row, the activation rows of its four transfers, and the column whose scales it copies
+    const int64_t wr = row0 + (tid >> 2) < N ? row0 + (tid >> 2) : N - 1;
+    const u32 *aux_row = (const u32 *)(planes + 2 * plane_stride) + (plane_base / K + wr) * nsb * 12;   // per-super-block data of the row
+    // per-lane byte offsets of this thread's two plane transfers per stage (row * K + swizzled chunk)
+    unsigned pofs[2];
+#pragma unroll
+    for (int it = 0; it < 2; it++) {
+        int r, c;
+        kp_dma_slot<2>(it, r, c);
+        const int64_t gr = row0 + r < N ? row0 + r : N - 1;
+        pofs[it] = (unsigned)(gr * K + c * 16);
+    }
+    const int8_t *plane1 = planes + plane_base, *plane0 = plane1 + plane_stride;
+    unsigned aofs[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        int r, c;
+        kp_dma_slot<4>(it, r, c);
+        const int64_t col = col0 + r;
+        const int64_t cc = col < B ? col : B - 1;
+        aofs[it] = (unsigned)((int64_t)(ID ? route.act_row[cc] : (int)cc) * K + c * 16);
+    }
+    int srow;
+    {
+        const int64_t col = col0 + (tid >> 1);
+        const int64_t cc = col < B ? col : B - 1;
+        srow = ID ? route.act_row[cc] : (int)cc;
+    }
+
+    f32x16 acc[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[tb][r] = 0.0f;
+
+    // per super-block scales of the weights come with the piece (Q4_K header / Q6_K d); those of the activations are fetched
+    // by two threads per column: 16 bytes of the sub-block sums each, the even thread also the scale
+    auto fetch_scales = [&](int64_t sb, float &d8, u32x4 &bs) {
+        d8 = ad8[(int64_t)srow * nsb + sb];
+        if constexpr (Q4) bs = *(const u32x4 *)(abs_ + ((int64_t)srow * nsb + sb) * 16 + 8 * (tid & 1));
+    };
+    auto store_scales = [&](int sbuf, float d8, const u32x4 &bs, const pl_h<TYPE> &H) {
+        sAd[sbuf][tid >> 1] = d8;   // both threads of the column write the same value: an unconditional use keeps the load where it was issued
+        if constexpr (Q4) {
+            *(u32x4 *)(sAs[sbuf] + (tid >> 1) * 16 + 8 * (tid & 1)) = bs;
+            // the four threads of a row: each writes d, dmin (same values) and the f16 mins of sub-blocks 2p, 2p + 1
+            const int r = tid >> 2, p = tid & 3;
+            ((u32 *)sWm[sbuf])[r * 8 + p] = H.v[0];
+            ((u32 *)sWm[sbuf])[r * 8 + 4 + p] = H.v[1];
+            sWd[sbuf][r] = __builtin_bit_cast(float, H.v[2]);
+            sWn[sbuf][r] = __builtin_bit_cast(float, H.v[3]);
+        } else {
+            sWd[sbuf][tid >> 2] = __builtin_bit_cast(float, H.v[0]);   // the four threads of a row write the same value
+        }
+    };
+
+    pl_h<TYPE> Hc, Hn;   // super-block data in use / of the next super-block
+    float d8n = 0.0f;
+    u32x4 bsn = {0, 0, 0, 0};
+    // both planes of a stage: 64 rows x 128 bytes each, two wave-wide transfers per wave and plane, swizzled like the activations
+    auto dma_w = [&](int64_t k0, int8_t *s1, int8_t *s0) {
+        kp_dma_a<2>(plane1 + k0, pofs, s1);
+        kp_dma_a<2>(plane0 + k0, pofs, s0);
+    };
+    // prologue: stage 0 into the "a" buffers
+    pl_fetch_h<TYPE>(Hc, aux_row, 0);
+    kp_dma_a<4>(aq, aofs, sAa);
+    dma_w(0, sW1a, sW0a);
+    fetch_scales(0, d8n, bsn);
+    store_scales(0, d8n, bsn, Hc);
+    Hn = Hc;
+    __syncthreads();
+
+    for (int64_t sb = 0; sb < nsb; sb++) {
+        i32x16 hi[2], lo[2];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int8_t *cA = half == 0 ? sAa : sAb_;
+            const int8_t *cW1 = half == 0 ? sW1a : sW1b;
+            const int8_t *cW0 = half == 0 ? sW0a : sW0b;
+            int8_t *nA = half == 0 ? sAb_ : sAa;
+            int8_t *nW1 = half == 0 ? sW1b : sW1a;
+            int8_t *nW0 = half == 0 ? sW0b : sW0a;
+            // Past the end of K the same work is done on the last super-block again and never read: no branches in the stage.
+            const int64_t sb1 = sb + 1 < nsb ? sb + 1 : sb;
+            const int64_t k1 = half == 0 ? sb * QKK + 128 : sb1 * QKK;   // the next stage
+            kp_dma_a<4>(aq + k1, aofs, nA);
+            dma_w(k1, nW1, nW0);
+            if (half == 1) fetch_scales(sb1, d8n, bsn);
+            if (half == 0) pl_fetch_h<TYPE>(Hn, aux_row, sb1);   // used from the next stage on
+            __builtin_amdgcn_sched_barrier(0);   // the loads stay here, a whole stage ahead of their first use
+
+            i32x4 af[1][2], b1[1], b0[1];
+            auto load_frags = [&](int ks, int slot) {
+#pragma unroll
+                for (int tb = 0; tb < 2; tb++) af[slot][tb] = *(const i32x4 *)(cA + kp_off(wcol0 + tb * 32 + l32, ks * 2 + lhi));
+                b1[slot] = *(const i32x4 *)(cW1 + kp_off(wrow0 + l32, ks * 2 + lhi));
+                b0[slot] = *(const i32x4 *)(cW0 + kp_off(wrow0 + l32, ks * 2 + lhi));
+            };
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                // one set of operand registers: the second resident group covers the LDS latency, and the registers a second set
+                // would take are what keeps this kernel from spilling
+                const int sl = 0;
+                load_frags(ks, 0);
+#pragma unroll
+                for (int tb = 0; tb < 2; tb++) {
+                    if (half == 0 && ks == 0) {
+                        i32x16 z;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) z[r] = 0;
+                        hi[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b1[sl], z, 0, 0, 0);
+                        lo[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b0[sl], z, 0, 0, 0);
+                    } else {
+                        hi[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b1[sl], hi[tb], 0, 0, 0);
+                        lo[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[sl][tb], b0[sl], lo[tb], 0, 0, 0);
+                    }
+                }
+            }
+
+            if (half == 1) {   // end of the super-block: scale the integer sums into the f32 accumulators
+                const int sbuf = (int)(sb & 1);
+#pragma unroll
+                for (int tb = 0; tb < 2; tb++) {
+                    f32x4 d8[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) d8[q] = *(const f32x4 *)(sAd[sbuf] + wcol0 + tb * 32 + 8 * q + 4 * lhi);
+                    const int wr_ = wrow0 + l32;
+                    const float dw = sWd[sbuf][wr_];
+                    if constexpr (Q4) {
+                        const float dn = sWn[sbuf][wr_];
+                        const f16x8 am = *(const f16x8 *)(sAs[sbuf] + (wcol0 + tb * 32 + l32) * 16 + 8 * lhi);
+                        const f16x8 bm = *(const f16x8 *)(sWm[sbuf] + wr_ * 16 + 8 * lhi);
+                        f32x16 z;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) z[r] = 0.0f;
+                        const f32x16 M = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bm, z, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int t = (hi[tb][r] << RADIX_SHIFT) + lo[tb][r];
+                            acc[tb][r] += d8[r >> 2][r & 3] * (dw * (float)t - dn * M[r]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int t = (hi[tb][r] << RADIX_SHIFT) + lo[tb][r];
+                            acc[tb][r] += d8[r >> 2][r & 3] * (dw * (float)t);
+                        }
+                    }
+                }
+            }
+            if (half == 1) {   // last, so that the loads had the whole stage (the barrier keeps the scheduler from hoisting the wait)
+                __builtin_amdgcn_sched_barrier(0);
                 store_scales((int)((sb + 1) & 1), d8n, bsn, Hn);
                 Hc = Hn;
             }
@@ -825,6 +1153,51 @@ int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act
     if (type == MI355_Q4_K) launch_mmq_k_id<MI355_Q4_K>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
     else launch_mmq_k_id<MI355_Q6_K>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
     return launch_status("k_mmq_k (routed)");
+}
+
+size_t mi355_kq_planes_bytes(int64_t rows, int64_t K) {
+    if (rows <= 0 || K <= 0 || K % QKK != 0) return 0;
+    return 2 * (size_t)rows * (size_t)K + (size_t)rows * (size_t)(K / QKK) * 48;
+}
+
+int mi355_kq_unpack_planes(void *stream, int type, const void *W, void *planes, int64_t rows, int64_t K) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "kq_unpack_planes: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(rows > 0 && K > 0 && K % QKK == 0, "kq_unpack_planes: bad shape rows=%lld K=%lld", (long long)rows, (long long)K);
+    const row_layout L = make_row_layout(type, K);
+    MI355_REQUIRE(layout_aligned(W, L) && ((uintptr_t)planes & 15) == 0, "kq_unpack_planes: rows are not 16-byte aligned (K=%lld)", (long long)K);
+    const int64_t pieces = rows * (K >> 8) * 8;
+    MI355_REQUIRE((pieces + 255) / 256 < 0x7fffffff, "kq_unpack_planes: too many pieces for one launch");
+    const dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
+    if (type == MI355_Q4_K) hipLaunchKernelGGL(k_unpack_planes<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)planes, rows, K, L);
+    else hipLaunchKernelGGL(k_unpack_planes<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)planes, rows, K, L);
+    return launch_status("k_unpack_planes");
+}
+
+int mi355_mul_mat_q8k_planes(void *stream, int type, const void *planes, const void *act, float *dst, const float *residual, int64_t N,
+                             int64_t K, int64_t B, int64_t dst_stride) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k_planes: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k_planes: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
+    MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k_planes: K=%lld is not a multiple of 256", (long long)K);
+    MI355_REQUIRE(N * K < ((int64_t)1 << 32), "mul_mat_q8k_planes: matrix too large for 32-bit plane offsets");
+    MI355_REQUIRE(dst_stride >= N, "mul_mat_q8k_planes: dst_stride < N");
+    MI355_REQUIRE(planes != nullptr && ((uintptr_t)planes & 15) == 0, "mul_mat_q8k_planes: planes are not 16-byte aligned");
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0 && (q8k_d_offset(K, B) & 15) == 0 && (q8k_bs_offset(K, B) & 15) == 0,
+                  "mul_mat_q8k_planes: activation workspace is not 16-byte aligned");
+    MI355_REQUIRE((N + 63) / 64 * ((B + 63) / 64) < (1 << 30), "mul_mat_q8k_planes: too many tiles");
+    const row_layout L = make_row_layout(type, K);
+    const int8_t *aq = (const int8_t *)act;
+    const float *ad8 = (const float *)(aq + q8k_d_offset(K, B));
+    const _Float16 *abs_ = (const _Float16 *)(aq + q8k_bs_offset(K, B));
+    const int n_row_tiles = (int)((N + 63) / 64), n_col_tiles = (int)((B + 127) / 128);
+    const int n_groups = n_row_tiles * n_col_tiles, n_groups_padded = (n_groups + 7) & ~7;
+    hipStream_t s = (hipStream_t)stream;
+    if (type == MI355_Q4_K)
+        hipLaunchKernelGGL((k_mmq_pl<MI355_Q4_K, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, dst,
+                           residual, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
+    else
+        hipLaunchKernelGGL((k_mmq_pl<MI355_Q6_K, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, dst,
+                           residual, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
+    return launch_status("k_mmq_pl");
 }
 
 int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,

@@ -97,6 +97,8 @@ class LlamaRunner:
         dev = self.dev = weights.output[1].device
         self.lib = load()
         self.fuse_qkv = True    # rows must be 16-byte aligned; set False to use the three-launch sequence
+        self.use_planes = True  # prefill: Q6_K matrices go through their unpacked int8 planes (2 bytes per weight more, kept resident)
+        self.planes = {}
         self.fuse_tail = True   # swiglu + Q8_1 done by the last group of each 32-row block of the gate/up launch (decode, T <= 4)
         E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
         T = self.max_tokens = max_tokens
@@ -168,6 +170,15 @@ class LlamaRunner:
         """the super-block tile GEMM serves K-quants whose device rows are 16-byte aligned"""
         return all(t == Q4_K or (t == Q6_K and K % 2048 == 0) for (t, _), _ in mats)
 
+    def _planes(self, t, W, N, K):
+        """the two int8 planes of a K-quant matrix (value = 64 * hi + lo for Q6_K), built on first use and kept"""
+        key = W.data_ptr()
+        if key not in self.planes:
+            buf = torch.empty(int(self.lib.mi355_kq_planes_bytes(N, K)) + 256, dtype=torch.uint8, device=self.dev)
+            check(self.lib.mi355_kq_unpack_planes(_stream(), t, _ptr(W), _ptr(buf), N, K))
+            self.planes[key] = buf
+        return self.planes[key]
+
     def _quant(self, src, act, K, T, q8k):
         fn = self.lib.mi355_quantize_act_q8k if q8k else self.lib.mi355_quantize_act
         check(fn(_stream(), _ptr(src), _ptr(act), K, T, src.stride(0)))
@@ -189,6 +200,10 @@ class LlamaRunner:
             check(self.lib.mi355_mul_mat_vec_q_multi(_stream(), len(mats), arr, _ptr(act), K, T))
         else:
             for (t, W), out in mats:
+                if q8k and t == Q6_K and self.use_planes:   # Q6_K streams its int8 planes, unpacked once per matrix
+                    check(self.lib.mi355_mul_mat_q8k_planes(_stream(), t, _ptr(self._planes(t, W, out.shape[1], K)), _ptr(act), _ptr(out),
+                                                            _ptr(residual) if residual is not None else None, out.shape[1], K, T, out.stride(0)))
+                    continue
                 if q8k:     # the residual add is the tile kernel's epilogue
                     check(self.lib.mi355_mul_mat_q8k_add(_stream(), t, _ptr(W), _ptr(act), _ptr(out), _ptr(residual) if residual is not None else None,
                                                          out.shape[1], K, T, out.stride(0)))

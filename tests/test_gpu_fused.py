@@ -275,3 +275,93 @@ def test_tile_gemm_residual_epilogue(dev, name, t):
     inplace = res.clone()
     mi355.check(lib.mi355_mul_mat_q8k_add(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(inplace), mi355._ptr(inplace), N, K, B, N))
     assert torch.equal(inplace, plain + res)
+
+
+def _kq_integer_levels(t, raw, N, K):
+    """sub-scale times level of every weight, and the per-sub-block mins, d and dmin, decoded in numpy from ggml's block bytes
+    (dequantize_row_q4_K / dequantize_row_q6_K, ggml/src/ggml-quants.c:1280-1302, 1690-1719)"""
+    nsb = K // 256
+    if t == orc.Q4_K:
+        blk = raw.reshape(N, nsb, 144)
+        d = blk[:, :, 0:2].copy().view(np.float16).astype(np.float32)[..., 0]
+        dmin = blk[:, :, 2:4].copy().view(np.float16).astype(np.float32)[..., 0]
+        s = blk[:, :, 4:16].astype(np.int32)
+        sc = np.empty((N, nsb, 8), np.int32)
+        mn = np.empty((N, nsb, 8), np.int32)
+        for j in range(8):
+            if j < 4:
+                sc[..., j], mn[..., j] = s[..., j] & 63, s[..., j + 4] & 63
+            else:
+                sc[..., j] = (s[..., j + 4] & 0xF) | ((s[..., j - 4] >> 6) << 4)
+                mn[..., j] = (s[..., j + 4] >> 4) | ((s[..., j] >> 6) << 4)
+        qs = blk[:, :, 16:144].astype(np.int32).reshape(N, nsb, 4, 32)
+        lev = np.stack([qs & 0xF, qs >> 4], axis=3).reshape(N, nsb, 8, 32)      # sub-blocks 2j (low nibbles), 2j+1 (high)
+        return (lev * sc[..., None]).reshape(N, K), mn, d, dmin
+    blk = raw.reshape(N, nsb, 210)
+    ql = blk[:, :, 0:128].astype(np.int32).reshape(N, nsb, 2, 64)
+    qh = blk[:, :, 128:192].astype(np.int32).reshape(N, nsb, 2, 32)
+    sc = blk[:, :, 192:208].copy().view(np.int8).astype(np.int32).reshape(N, nsb, 2, 8)
+    d = blk[:, :, 208:210].copy().view(np.float16).astype(np.float32)[..., 0]
+    lo4 = [ql[..., 0:32] & 0xF, ql[..., 32:64] & 0xF, ql[..., 0:32] >> 4, ql[..., 32:64] >> 4]
+    lev = np.stack([(lo4[i] | (((qh >> (2 * i)) & 3) << 4)) - 32 for i in range(4)], axis=3)   # [N][nsb][2][4][32]
+    scale = sc.reshape(N, nsb, 2, 4, 2)[..., None].repeat(16, axis=-1).reshape(N, nsb, 2, 4, 32)     # scales[is + 2 i], is = l / 16
+    return (lev * scale).reshape(N, K), None, d, None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,t,R", [("q4_K", orc.Q4_K, 8), ("q6_K", orc.Q6_K, 64)])
+def test_unpacked_planes_hold_the_integer_levels(dev, name, t, R):
+    """R * hi + lo of the unpacked copy is sub-scale times level of each weight; the per-super-block entries hold mins, d, dmin"""
+    import torch
+    import mi355
+    from mi355 import llama_graph as lg
+    lib = mi355.load()
+    N, K = 96, 2048
+    gen = torch.Generator(device=dev).manual_seed(11)
+    be, bb = lg.BLOCK[t]
+    raw = lg.random_quantized(t, N, K, dev, gen).reshape(N, K // be, bb)
+    for col in ([0, 2] if t == orc.Q4_K else [208]):      # a different d (and dmin) in every super-block
+        h = (torch.rand(N, K // be, device=dev, generator=gen) * 1e-3 + 1e-4).to(torch.float16)
+        raw[:, :, col:col + 2] = h.view(torch.uint8).reshape(N, K // be, 2)
+    raw = raw.reshape(N, -1).contiguous()
+    W = mi355.upload_weights(t, raw)
+    planes = torch.zeros(int(lib.mi355_kq_planes_bytes(N, K)), dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_kq_unpack_planes(None, t, mi355._ptr(W), mi355._ptr(planes), N, K))
+    torch.cuda.synchronize()
+    p = planes.cpu().numpy()
+    hi = p[:N * K].view(np.int8).astype(np.int32).reshape(N, K)
+    lo = p[N * K:2 * N * K].view(np.int8).astype(np.int32).reshape(N, K)
+    want, mn, d, dmin = _kq_integer_levels(t, raw.cpu().numpy().reshape(-1), N, K)
+    np.testing.assert_array_equal(R * hi + lo, want)
+    aux = p[2 * N * K:].reshape(N, K // 256, 48)
+    np.testing.assert_array_equal(aux[:, :, 32:36].copy().view(np.float32)[..., 0], d)
+    if t == orc.Q4_K:
+        np.testing.assert_array_equal(aux[:, :, 36:40].copy().view(np.float32)[..., 0], dmin)
+        np.testing.assert_array_equal(aux[:, :, 0:16].copy().view(np.float16).astype(np.int32), mn)
+        np.testing.assert_array_equal(aux[:, :, 16:32].copy().view(np.float16).astype(np.int32), 64 * mn)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,t", [("q4_K", orc.Q4_K), ("q6_K", orc.Q6_K)])
+@pytest.mark.parametrize("N,K,B", [(320, 2048, 70), (1024, 4096, 512), (4096, 2048, 9), (136, 6144, 130)])
+def test_tile_gemm_from_planes_equals_packed(dev, name, t, N, K, B):
+    """the tile GEMM that streams unpacked planes gives the bits of the one that unpacks in the kernel, residual and strided dst included"""
+    import torch
+    import mi355
+    from mi355 import llama_graph as lg
+    lib = mi355.load()
+    gen = torch.Generator(device=dev).manual_seed(5)
+    W = mi355.upload_weights(t, lg.random_quantized(t, N, K, dev, gen))
+    x = torch.randn(B, K, device=dev, generator=gen)
+    res = torch.randn(B, N + 8, device=dev, generator=gen)
+    act = mi355.quantize_act_q8k(x)
+    planes = torch.empty(int(lib.mi355_kq_planes_bytes(N, K)) + 256, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_kq_unpack_planes(None, t, mi355._ptr(W), mi355._ptr(planes), N, K))
+    for residual in (None, res):
+        want = torch.zeros(B, N + 8, device=dev)
+        got = torch.zeros(B, N + 8, device=dev)
+        r = mi355._ptr(residual) if residual is not None else None
+        mi355.check(lib.mi355_mul_mat_q8k_add(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(want), r, N, K, B, N + 8))
+        mi355.check(lib.mi355_mul_mat_q8k_planes(None, t, mi355._ptr(planes), mi355._ptr(act), mi355._ptr(got), r, N, K, B, N + 8))
+        assert torch.equal(got, want)
+        assert got[:, N:].abs().max().item() == 0.0      # nothing written past the row
