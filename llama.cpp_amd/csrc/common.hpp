@@ -77,6 +77,22 @@ __device__ __forceinline__ u32x4 load_stream16(const void *p) {
 }
 __device__ __forceinline__ u32x4 load16(const void *p) { return *(const u32x4 *)p; }
 
+// Single roundings that stay single: the compiler may not merge these into fused multiply-adds, whatever surrounds the call.
+// (The CUDA-style __fmul_rn / __fadd_rn of the HIP headers are plain operators and do get merged.)  For results that several
+// kernels must reproduce bit for bit.
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+    return a * b;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+#pragma clang fp contract(off)
+    return a + b;
+}
+__device__ __forceinline__ float sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+    return a - b;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);

@@ -104,43 +104,61 @@ __global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
     const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
     const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
 
-    for (int64_t cb = c_begin; cb < c_end; cb += SLOTS) {
-        const int64_t c = cb + slot;
-        const bool in_range = c < c_end;
-        float mv = 0.0f;
-        if (mrow && in_range) mv = half_bits_to_float(mrow[c]);
-        const bool valid = in_range && mv != -INFINITY;
-        if (__ballot(valid) == 0) continue;   // whole wave masked: skip the K/V traffic (wave-uniform)
-        u32x4 kk = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-        if (valid && active) {
-            kk = load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2);
-            vv = load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2);
+    // U steps of SLOTS cells at a time: all mask entries, then all K/V rows of the U steps are requested before the first
+    // is used, so a short context costs one round trip to memory instead of one per step.  Cells are still folded into a
+    // slot's state in ascending order.
+    constexpr int U = 4;
+    for (int64_t cb = c_begin; cb < c_end; cb += U * SLOTS) {
+        float mv[U];
+        bool valid[U];
+#pragma unroll
+        for (int j = 0; j < U; j++) {
+            const int64_t c = cb + j * SLOTS + slot;
+            const bool in_range = c < c_end;
+            mv[j] = 0.0f;
+            if (mrow && in_range) mv[j] = half_bits_to_float(mrow[c]);
+            valid[j] = in_range && mv[j] != -INFINITY;
         }
-        float vf[8];
+        u32x4 kk[U], vv[U];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const u32 vi = vv[i];
-            const f16x2 h2 = __builtin_bit_cast(f16x2, vi);
-            vf[2 * i] = (float)h2[0];
-            vf[2 * i + 1] = (float)h2[1];
+        for (int j = 0; j < U; j++) {
+            const int64_t c = cb + j * SLOTS + slot;
+            kk[j] = u32x4{0, 0, 0, 0};
+            vv[j] = u32x4{0, 0, 0, 0};
+            if (valid[j] && active) {   // masked cells cost no K/V traffic
+                kk[j] = load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2);
+                vv[j] = load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2);
+            }
         }
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            float s = group_sum<LPR>(dot8_f16(qh[r], kk)) * scale;
-            if (a.softcap != 0.0f) s = a.softcap * tanhf(s);
-            s += slope[r] * mv;
-            if (valid) {
-                if (s > m[r]) {
-                    const float f = __expf(m[r] - s);
-                    l[r] *= f;
+        for (int j = 0; j < U; j++) {
+            if (__ballot(valid[j]) == 0) continue;   // whole wave masked (wave-uniform)
+            float vf[8];
 #pragma unroll
-                    for (int i = 0; i < 8; i++) acc[r][i] *= f;
-                    m[r] = s;
+            for (int i = 0; i < 4; i++) {
+                const u32 vi = vv[j][i];
+                const f16x2 h2 = __builtin_bit_cast(f16x2, vi);
+                vf[2 * i] = (float)h2[0];
+                vf[2 * i + 1] = (float)h2[1];
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float s = group_sum<LPR>(dot8_f16(qh[r], kk[j])) * scale;
+                if (a.softcap != 0.0f) s = a.softcap * tanhf(s);
+                s += slope[r] * mv[j];
+                if (valid[j]) {
+                    if (s > m[r]) {
+                        const float f = __expf(m[r] - s);
+                        l[r] *= f;
+#pragma unroll
+                        for (int i = 0; i < 8; i++) acc[r][i] *= f;
+                        m[r] = s;
+                    }
+                    const float p = __expf(s - m[r]);
+                    l[r] += p;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc[r][i] += p * vf[i];
                 }
-                const float p = __expf(s - m[r]);
-                l[r] += p;
-#pragma unroll
-                for (int i = 0; i < 8; i++) acc[r][i] += p * vf[i];
             }
         }
     }

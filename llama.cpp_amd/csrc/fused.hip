@@ -155,8 +155,8 @@ __device__ __forceinline__ void rope_pair(const rope_kv_args &a, int pos, int pa
         mscale *= 1.0f + 0.1f * logf(1.0f / a.freq_scale);
     }
     const float c = cosf(theta) * mscale, s = sinf(theta) * mscale;
-    y0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));   // no contraction: bit-identical to k_rope
-    y1 = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+    y0 = sub_rn(mul_rn(x0, c), mul_rn(x1, s));   // no contraction: bit-identical to k_rope
+    y1 = add_rn(mul_rn(x0, s), mul_rn(x1, c));
 }
 
 // grid (H + 2*HK, T), D/2 threads: heads [0,H) rotate q in place, [H,H+HK) rotate k into the cache,

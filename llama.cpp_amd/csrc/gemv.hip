@@ -39,8 +39,8 @@ struct gemv_rope {
     float theta_scale, freq_scale, ext_factor, attn_factor, corr0, corr1;
 };
 
-// rope_yarn + rotation, same roundings as k_rope (glue.hip) and k_rope_kv_store (fused.hip); ggml-cpu.c:9268-9306
-__device__ __forceinline__ void rope_rotate(const gemv_rope &a, int pos, int pair, float x0, float x1, float &y0, float &y1) {
+// rope_yarn, same roundings as k_rope (glue.hip) and k_rope_kv_store (fused.hip); ggml-cpu.c:9268-9306
+__device__ __forceinline__ void rope_coeffs(const gemv_rope &a, int pos, int pair, float &c, float &s) {
     const float theta_extrap = (float)pos * powf(a.theta_scale, (float)pair) / (a.ff ? a.ff[pair] : 1.0f);
     const float theta_interp = a.freq_scale * theta_extrap;
     float theta = theta_interp, mscale = a.attn_factor;
@@ -50,9 +50,12 @@ __device__ __forceinline__ void rope_rotate(const gemv_rope &a, int pos, int pai
         theta = theta_interp * (1.0f - ramp) + theta_extrap * ramp;
         mscale *= 1.0f + 0.1f * logf(1.0f / a.freq_scale);
     }
-    const float c = cosf(theta) * mscale, s = sinf(theta) * mscale;
-    y0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
-    y1 = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+    c = cosf(theta) * mscale;
+    s = sinf(theta) * mscale;
+}
+__device__ __forceinline__ void rope_apply(float c, float s, float x0, float x1, float &y0, float &y1) {
+    y0 = sub_rn(mul_rn(x0, c), mul_rn(x1, s));
+    y1 = add_rn(mul_rn(x0, s), mul_rn(x1, c));
 }
 struct gemv_batch {
     gemv_item it[4];
@@ -87,6 +90,23 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
 #pragma unroll
         for (int c = 0; c < NCOLS; c++) acc[r][c] = 0.0f;
 
+    // QKV: lane c finishes activation row c.  Its rotation and cache cell depend on nothing the product computes, so they are
+    // worked out here, while the weight loads of the first step are in flight (the empty asm keeps them from being moved
+    // behind the loop, next to their use).
+    float rope_c = 1.0f, rope_s = 0.0f;
+    int cell = 0;
+    bool rotate = false;
+    if constexpr (QKV) {
+        if (lane < NCOLS) {
+            const gemv_rope &R = *rp;
+            const int d = (int)(row0 % R.D);
+            rotate = (m.epi == EPI_ROPE || m.epi == EPI_ROPE_CACHE) && d < R.n_dims;
+            if (rotate) rope_coeffs(R, R.pos[lane], d >> 1, rope_c, rope_s);
+            if (m.epi == EPI_ROPE_CACHE || m.epi == EPI_CACHE) cell = R.cells[lane];
+        }
+        asm volatile("" : "+v"(rope_c), "+v"(rope_s), "+v"(cell));
+    }
+
     for (int c0 = 0; c0 < nchunks; c0 += 64) {
         const int c = c0 + lane;
         if (c < nchunks) {
@@ -120,13 +140,13 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
             const int64_t head = row0 / R.D;
             const int d = (int)(row0 % R.D);
             float y0 = s0, y1 = s1;
-            if ((m.epi == EPI_ROPE || m.epi == EPI_ROPE_CACHE) && d < R.n_dims) rope_rotate(R, R.pos[lane], d >> 1, s0, s1, y0, y1);
+            if (rotate) rope_apply(rope_c, rope_s, s0, s1, y0, y1);
             if (m.epi == EPI_ROPE || m.epi == EPI_STORE) {
                 float *o = m.dst + lane * m.dst_stride + row0;
                 o[0] = y0;
                 o[1] = y1;
             } else {
-                _Float16 *o = (_Float16 *)((uint8_t *)m.dst + (int64_t)R.cells[lane] * m.nb1 + head * m.nb2) + d;
+                _Float16 *o = (_Float16 *)((uint8_t *)m.dst + (int64_t)cell * m.nb1 + head * m.nb2) + d;
                 o[0] = (_Float16)y0;
                 o[1] = (_Float16)y1;
             }

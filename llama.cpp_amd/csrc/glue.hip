@@ -237,8 +237,8 @@ __global__ void k_rope(tens src, const int32_t *__restrict__ pos, const float *_
         const int64_t ia = neox ? pair : i0, ib = neox ? pair + p.n_dims / 2 : i0 + 1;
         const float x0 = x[ia], x1 = x[ib];
         // separately rounded products: the fused rope + KV-store kernel rotates with the same four roundings
-        y[ia] = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
-        y[ib] = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+        y[ia] = sub_rn(mul_rn(x0, c), mul_rn(x1, s));
+        y[ib] = add_rn(mul_rn(x0, s), mul_rn(x1, c));
     }
 }
 

@@ -63,18 +63,18 @@ __global__ void __launch_bounds__(256) k_moe_combine(const float *__restrict__ e
         const f32x4 x = *(const f32x4 *)(experts + (t * n_used + e) * n_embd + i0);
         f32x4 y;
 #pragma unroll
-        for (int i = 0; i < 4; i++) y[i] = __fmul_rn(x[i], wt);
+        for (int i = 0; i < 4; i++) y[i] = mul_rn(x[i], wt);
         if (scaled) *(f32x4 *)(scaled + (t * n_used + e) * n_embd + i0) = y;
         if (e == 0) acc = y;
         else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[i] = __fadd_rn(acc[i], y[i]);
+            for (int i = 0; i < 4; i++) acc[i] = add_rn(acc[i], y[i]);
         }
     }
     if (residual) {
         const f32x4 r = *(const f32x4 *)(residual + t * n_embd + i0);
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[i] = __fadd_rn(acc[i], r[i]);
+        for (int i = 0; i < 4; i++) acc[i] = add_rn(acc[i], r[i]);
     }
     *(f32x4 *)(out + t * n_embd + i0) = acc;
 }

@@ -100,7 +100,7 @@ template <> struct wq<MI355_Q4_0> {
         return r;
     }
     static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
-        return __builtin_fmaf(w.d, __fmul_rn(A.d, (float)r.i0), acc);
+        return __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), acc);
     }
 };
 
@@ -136,7 +136,7 @@ template <> struct wq<MI355_Q8_0> {
         return r;
     }
     static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
-        return __builtin_fmaf(w.d, __fmul_rn(A.d, (float)r.i0), acc);
+        return __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), acc);
     }
 };
 
@@ -197,9 +197,9 @@ template <> struct wq<MI355_Q4_K> {
         return r;
     }
     static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
-        const float pos = __builtin_fmaf(w.scA, __fmul_rn(A.d0, (float)r.i0), __fmul_rn(w.scB, __fmul_rn(A.d1, (float)r.i1)));
-        const float neg = __builtin_fmaf(w.mA, A.ds0, __fmul_rn(w.mB, A.ds1));
-        return __fadd_rn(acc, __builtin_fmaf(w.d, pos, -__fmul_rn(w.dmin, neg)));
+        const float pos = __builtin_fmaf(w.scA, mul_rn(A.d0, (float)r.i0), mul_rn(w.scB, mul_rn(A.d1, (float)r.i1)));
+        const float neg = __builtin_fmaf(w.mA, A.ds0, mul_rn(w.mB, A.ds1));
+        return add_rn(acc, __builtin_fmaf(w.d, pos, -mul_rn(w.dmin, neg)));
     }
 };
 
@@ -255,7 +255,7 @@ template <> struct wq<MI355_Q6_K> {
         return r;
     }
     static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
-        const float t = __builtin_fmaf(w.scA, __fmul_rn(A.d0, (float)r.i0), __fmul_rn(w.scB, __fmul_rn(A.d1, (float)r.i1)));
+        const float t = __builtin_fmaf(w.scA, mul_rn(A.d0, (float)r.i0), mul_rn(w.scB, mul_rn(A.d1, (float)r.i1)));
         return __builtin_fmaf(w.d, t, acc);
     }
 };
