@@ -300,7 +300,9 @@ static int launch_vec(hipStream_t s, fattn_args &a) {
 
 template <int D>
 static int launch_vec_r(hipStream_t s, fattn_args &a, int R) {
-    // R = query heads served per group from one pass over the kv head's bytes
+    // R = query heads served per group from one pass over the kv head's bytes.  A short context is not bandwidth-bound but
+    // a serial chain of soft-max updates per (step, head): one head per group then spreads it over R times as many waves.
+    if (a.Nkv <= 1024 && a.n_splits == 1) return launch_vec<D, 1>(s, a);
     if (R % 4 == 0) return launch_vec<D, 4>(s, a);
     if (R % 2 == 0) return launch_vec<D, 2>(s, a);
     return launch_vec<D, 1>(s, a);

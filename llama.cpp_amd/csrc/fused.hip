@@ -10,93 +10,19 @@
 // exactly one 256-element super-block)
 //   ROPE(q), ROPE(k), CPY(k -> cache), CPY(v -> cache)   k_rope_kv_store
 #include "common.hpp"
+#include "norm_quant.hpp"
 #include "q8k.hpp"
 
 namespace mi355 {
 
-// Q8_1 of the 4 values held by each of 8 neighbouring lanes (one 32-element block); writes the
-// split activation layout.  Mirrors k_quantize_q8_1 (quantize.hip) instruction for instruction.
-__device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, int8_t *__restrict__ qplane, act_ds *__restrict__ ds,
-                                                    int64_t row, int64_t k, int64_t e0) {
-    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-#pragma unroll
-    for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-    const float d = amax / 127.0f;
-    const float id = d != 0.0f ? 1.0f / d : 0.0f;
-    int q[4];
-    int sum = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        q[i] = (int)roundf(v[i] * id);
-        sum += q[i];
-    }
-#pragma unroll
-    for (int off = 4; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    if (!live) return;
-    const u32 packed = (u32)(q[0] & 0xFF) | ((u32)(q[1] & 0xFF) << 8) | ((u32)(q[2] & 0xFF) << 16) | ((u32)(q[3] & 0xFF) << 24);
-    *(u32 *)(qplane + row * k + e0) = packed;
-    if (((e0 >> 2) & 7) == 0) {
-        act_ds o;
-        o.d = half_bits_to_float(float_to_half_bits(d));
-        o.sum = sum;
-        ds[row * (k >> 5) + (e0 >> 5)] = o;
-    }
-}
-
-// one 256-thread group per row; each thread keeps its NV float4 of the row in registers
+// one 256-thread group per row
 template <int NV, bool Q8K>
 __global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restrict__ x, int64_t x_stride, const float *__restrict__ w,
                                                             float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k,
                                                             int64_t nrows, float eps) {
     __shared__ float sh[4];
     const int64_t row = blockIdx.x;
-    const int tid = threadIdx.x;
-    const float *xr = x + row * x_stride;
-    f32x4 v[NV], ww[NV];
-    float ss = 0.0f;
-    // the weight does not depend on the reduction: fetch it together with the row, one memory round trip instead of two
-#pragma unroll
-    for (int it = 0; it < NV; it++) {
-        const int64_t e0 = ((int64_t)it * 256 + tid) * 4;
-        v[it] = f32x4{0.f, 0.f, 0.f, 0.f};
-        ww[it] = f32x4{1.f, 1.f, 1.f, 1.f};
-        if (e0 < k) {
-            v[it] = *(const f32x4 *)(xr + e0);
-            if (w) ww[it] = *(const f32x4 *)(w + e0);
-        }
-    }
-#pragma unroll
-    for (int it = 0; it < NV; it++) ss += v[it][0] * v[it][0] + v[it][1] * v[it][1] + v[it][2] * v[it][2] + v[it][3] * v[it][3];
-    ss = wave_sum(ss);
-    if ((tid & 63) == 0) sh[tid >> 6] = ss;
-    __syncthreads();
-    ss = sh[0] + sh[1] + sh[2] + sh[3];
-    const float scale = 1.0f / sqrtf(ss / (float)k + eps);
-    int8_t *qplane = (int8_t *)act;
-    act_ds *ds = (act_ds *)(qplane + nrows * k);
-#pragma unroll
-    for (int it = 0; it < NV; it++) {
-        const int64_t e0 = ((int64_t)it * 256 + tid) * 4;
-        const bool live = e0 < k;
-        f32x4 o;
-#pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = v[it][i] * scale;
-        if (w && live) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = o[i] * ww[it][i];
-        }
-        if (y && live) *(f32x4 *)(y + row * y_stride + e0) = o;
-        if constexpr (Q8K) {
-            if (act && live) {   // whole wave: k is a multiple of 256
-                const int64_t nsb = k >> 8, sb = e0 >> 8;
-                float *d8 = (float *)(qplane + q8k_d_offset(k, nrows));
-                _Float16 *bs = (_Float16 *)(qplane + q8k_bs_offset(k, nrows));
-                q8k_quantize_wave(o, tid & 63, qplane + row * k + sb * QKK, d8 + row * nsb + sb, bs + (row * nsb + sb) * 16);
-            }
-        } else {
-            if (act) quantize_block_lane(o, live, qplane, ds, row, k, e0);
-        }
-    }
+    rms_norm_quant_row<NV, Q8K, false>(x + row * x_stride, w, y ? y + row * y_stride : nullptr, act, row, k, nrows, eps, sh);
 }
 
 // h = silu(gate) * up, optional f32 output, optional Q8_1 output; one lane per 4 elements
