@@ -30,6 +30,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "mi355_kernels.h"
@@ -108,8 +109,38 @@ struct backend_ctx {
     unsigned * tickets = nullptr;   // zeroed arrival counters of the gate/up launch (one per 32 output rows)
     size_t n_tickets = 0;
 
+    // ---- replay of decode graphs as HIP graphs (see backend_graph_compute)
+    struct replay_state {
+        bool enabled = true;          // MI355_NO_GRAPH=1 turns replay off
+        uint64_t seen_sig = 0;        // signature of the last graph that ran launch by launch ...
+        uint64_t seen_gen = 0;        // ... and the scratch-buffer generation it ran with
+        uint64_t bad_sig = 0;         // a graph whose capture did not work out: not tried again
+        uint64_t exec_sig = 0, exec_gen = 0;
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        long replays = 0, captures = 0;
+        double host_us = 0.0;         // host time spent in graph_compute calls that ended in a replay
+    } replay;
+    uint64_t alloc_gen = 1;           // bumped whenever a scratch buffer moves: captured launches hold the old addresses
+    bool capturing = false, capture_broken = false;
+    int32_t * cells = nullptr;        // device {head, head + 1, ...}: cache cell of token t of this graph's batch
+    int64_t cells_head = -1;          // what `cells` holds
+    int64_t kv_head = -1;             // first cache cell this graph stores to, or -1 when its stores do not agree on one
+    int kv_redirected = 0;            // cache stores of this graph that went through `cells`
+
+    // a scratch buffer has to move: impossible while launches are being recorded (they would keep the old address and
+    // nothing may synchronize); the recording is thrown away afterwards and the graph runs launch by launch
+    bool may_allocate() {
+        if (capturing) {
+            capture_broken = true;
+            return false;
+        }
+        alloc_gen++;
+        return true;
+    }
+
     unsigned * ticket_buffer(size_t n) {
-        if (n > n_tickets) {
+        if (n > n_tickets && may_allocate()) {
             if (tickets) {
                 MI355_HIP_OK(hipStreamSynchronize(stream));
                 MI355_HIP_OK(hipFree(tickets));
@@ -132,7 +163,7 @@ struct backend_ctx {
 
     // two slots, so that a launch can read one quantized activation while it writes the next one
     void act_reserve(size_t need) {
-        if (need > act_size) {
+        if (need > act_size && may_allocate()) {
             if (act) {
                 MI355_HIP_OK(hipStreamSynchronize(stream));
                 MI355_HIP_OK(hipFree(act));
@@ -153,7 +184,7 @@ struct backend_ctx {
     }
 
     void * workspace(size_t need) {
-        if (need > ws_size) {
+        if (need > ws_size && may_allocate()) {
             if (ws) {
                 MI355_HIP_OK(hipStreamSynchronize(stream));   // kernels in flight may still read the old one
                 MI355_HIP_OK(hipFree(ws));
@@ -255,13 +286,19 @@ void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) bu
 // number of rows / elements per row of a tensor whose rows are contiguous blocks
 int64_t tensor_nrows(const ggml_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
 
+// Copies through the null stream are ordered against every backend stream of the device (those are created blocking), in both
+// directions, so plain uploads and read-backs need no device-wide synchronization of their own; the paths that reuse the shared
+// staging buffer or free memory keep it.
 void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
-    MI355_HIP_OK(hipDeviceSynchronize());
     if (size == 0) return;
-    if (tensor->type == GGML_TYPE_Q6_K) planes().drop(tensor->data, ggml_nbytes(tensor));   // rebuilt from the new contents on next use
+    if (tensor->type == GGML_TYPE_Q6_K) {
+        MI355_HIP_OK(hipDeviceSynchronize());
+        planes().drop(tensor->data, ggml_nbytes(tensor));   // rebuilt from the new contents on next use
+    }
     if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+        MI355_HIP_OK(hipDeviceSynchronize());
         std::lock_guard<std::mutex> lock(stage().mu);
         void * tmp = stage().get(size);
         MI355_HIP_OK(hipMemcpy(tmp, data, size, hipMemcpyHostToDevice));
@@ -275,9 +312,9 @@ void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const
 void buffer_get_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * tensor, void * data, size_t offset, size_t size) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
-    MI355_HIP_OK(hipDeviceSynchronize());
     if (size == 0) return;
     if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+        MI355_HIP_OK(hipDeviceSynchronize());
         std::lock_guard<std::mutex> lock(stage().mu);
         void * tmp = stage().get(size);
         MI355_K_OK(mi355_weights_gather(nullptr, to_mi355_type(tensor->type), tensor->data, tmp, tensor->ne[0], tensor_nrows(tensor), offset, size));
@@ -371,6 +408,42 @@ const ggml_backend_buffer_type_i buft_iface = {
     /* .get_alloc_size = */ nullptr,   // ggml_nbytes: the device layout keeps every tensor's footprint
     /* .is_host        = */ nullptr,
 };
+
+// ------------------------------------------------------------------------------- pinned host buffer type
+// Host memory the device reaches by DMA without staging (hipHostMalloc): llama.cpp places the logits it reads back and the
+// intermediate tensors its CPU backend hands to the device there (ggml_backend_dev_host_buffer_type, src/llama.cpp:8577,
+// :9468), which makes those copies one DMA each and lets them be asynchronous.  To the CPU it is an ordinary CPU buffer.
+const char * host_buft_get_name(ggml_backend_buffer_type_t) { return "MI355X_Host"; }
+
+void host_buffer_free(ggml_backend_buffer_t buffer) { (void) hipHostFree(buffer->context); }
+
+ggml_backend_buffer_t host_buft_alloc_buffer(ggml_backend_buffer_type_t buft, size_t size) {
+    void * ptr = nullptr;
+    if (getenv("MI355_NO_PINNED") != nullptr || hipHostMalloc(&ptr, size, hipHostMallocDefault) != hipSuccess) {
+        (void) hipGetLastError();
+        return ggml_backend_buft_alloc_buffer(ggml_backend_cpu_buffer_type(), size);   // pageable memory works too, only slower
+    }
+    ggml_backend_buffer_t buffer = ggml_backend_cpu_buffer_from_ptr(ptr, size);
+    buffer->buft = buft;
+    buffer->iface.free_buffer = host_buffer_free;
+    return buffer;
+}
+
+ggml_backend_buffer_type_t mi355_host_buffer_type(ggml_backend_dev_t dev) {
+    static ggml_backend_buffer_type host = {
+        /* .iface   = */ {
+            /* .get_name       = */ host_buft_get_name,
+            /* .alloc_buffer   = */ host_buft_alloc_buffer,
+            /* .get_alignment  = */ ggml_backend_cpu_buffer_type()->iface.get_alignment,
+            /* .get_max_size   = */ nullptr,
+            /* .get_alloc_size = */ ggml_backend_cpu_buffer_type()->iface.get_alloc_size,
+            /* .is_host        = */ ggml_backend_cpu_buffer_type()->iface.is_host,
+        },
+        /* .device  = */ dev,
+        /* .context = */ nullptr,
+    };
+    return &host;
+}
 
 // ------------------------------------------------------------------------------- op support
 bool f32_rows(const ggml_tensor * t) { return t->type == GGML_TYPE_F32 && t->nb[0] == sizeof(float); }
@@ -631,10 +704,43 @@ void backend_free(ggml_backend_t backend) {
     if (ctx->ws) (void) hipFree(ctx->ws);
     if (ctx->act) (void) hipFree(ctx->act);
     if (ctx->iota) (void) hipFree(ctx->iota);
+    if (ctx->cells) (void) hipFree(ctx->cells);
     if (ctx->tickets) (void) hipFree(ctx->tickets);
+    if (ctx->replay.exec) (void) hipGraphExecDestroy(ctx->replay.exec);
+    if (ctx->replay.graph) (void) hipGraphDestroy(ctx->replay.graph);
+    if (getenv("MI355_GRAPH_STATS"))
+        fprintf(stderr, "MI355 graph replay: %ld captures, %ld replays, %.1f us of host time per replay\n", ctx->replay.captures, ctx->replay.replays,
+                ctx->replay.replays ? ctx->replay.host_us / (double) ctx->replay.replays : 0.0);
     if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     delete backend;
+}
+
+// Asynchronous uploads and read-backs on the backend's own stream (ggml_backend_tensor_set_async / _get_async,
+// ggml/src/ggml-backend.cpp:238-262): ordered with the graphs of this backend, complete after synchronize().  Tensors kept in
+// the device row layout go through the synchronous path, which applies the permutation.
+void backend_set_tensor_async(ggml_backend_t backend, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
+    if ((is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) || size == 0) {
+        MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
+        buf->iface.set_tensor(buf, tensor, data, offset, size);
+        return;
+    }
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipMemcpyAsync((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice, ctx->stream));
+}
+
+void backend_get_tensor_async(ggml_backend_t backend, const ggml_tensor * tensor, void * data, size_t offset, size_t size) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
+    if ((is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) || size == 0) {
+        MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
+        buf->iface.get_tensor(buf, tensor, data, offset, size);
+        return;
+    }
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipMemcpyAsync(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost, ctx->stream));
 }
 
 void backend_synchronize(ggml_backend_t backend) {
@@ -991,6 +1097,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             const ggml_tensor * out;    // the tensor that currently holds the chain's value (product or its ROPE)
             int out_index;
             mi355_gemv_rope_mat m;
+            void * cache_base;          // cache stores that start at cell kv_head: the cache tensor's first byte
         } ch[3];
         int n_ch = 0, last = i - 1;
         mi355_rope_desc rd;
@@ -1010,6 +1117,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                     break;
                 chain & c = ch[n_ch++];
                 c.mm = t; c.out = t; c.out_index = k;
+                c.cache_base = nullptr;
                 c.m.type = to_mi355_type(t->src[0]->type);
                 c.m.W = t->src[0]->data;
                 c.m.N = t->ne[0];
@@ -1073,6 +1181,9 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 c->m.dst_stride = 0;
                 c->m.nb1 = c->m.N * 2;
                 c->out = nullptr;
+                if (ctx->kv_head >= 0 && d->view_src && d->view_src->data &&
+                    (const char *) d->data - (const char *) d->view_src->data == (ptrdiff_t) (ctx->kv_head * c->m.N * 2))
+                    c->cache_base = d->view_src->data;
                 last = k;
                 continue;
             }
@@ -1097,6 +1208,20 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                     void * fresh = ctx->act_slot(mi355_act_bytes(K, B));
                     MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
                     ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
+                }
+                // Cache stores that all start at cell kv_head address the cache tensor through the device-side cell list instead
+                // of through the view's own address, so the launch's arguments do not change from token to token.
+                int n_store = 0, n_base = 0;
+                for (int q = 0; q < n_ch; q++) {
+                    if (mats[q].epilogue != MI355_EPI_ROPE_CACHE && mats[q].epilogue != MI355_EPI_CACHE) continue;
+                    n_store++;
+                    if (ch[q].cache_base) n_base++;
+                }
+                if (n_store > 0 && n_base == n_store) {
+                    for (int q = 0; q < n_ch; q++)
+                        if (ch[q].cache_base) mats[q].dst = ch[q].cache_base;
+                    rd.cells = ctx->cells;
+                    ctx->kv_redirected += n_store;
                 }
                 MI355_K_OK(mi355_mul_mat_vec_q_rope(s, n_ch, mats, ctx->cache.ptr, K, B, &rd));
                 for (int q = 0; q < n_ch; q++) {
@@ -1194,18 +1319,94 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     return i;
 }
 
-ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
-    backend_ctx * ctx = (backend_ctx *) backend->context;
-    MI355_HIP_OK(hipSetDevice(ctx->device));
-    ctx->cache.valid = false;
-    if (!ctx->fuse) {
-        const int n = ggml_graph_n_nodes(cgraph);
-        for (int i = 0; i < n; i++) {
-            ggml_tensor * node = ggml_graph_node(cgraph, i);
-            if (!is_noop(node)) compute_node(ctx, node);
-        }
-        return GGML_STATUS_SUCCESS;
+// ---- HIP-graph replay of decode graphs
+// llama.cpp rebuilds the same ~1000-node graph for every decoded token.  Issued launch by launch that is ~230 kernel launches
+// from the host per token; replayed as one HIP graph it is one.  A graph is replayed when nothing a launch depends on has
+// changed since it was recorded: every node's op, type, shape, strides, parameters and data address, and those of its sources
+// (the signature below).  The one thing that does change from token to token is where K and V are stored: the CPY destinations
+// are views into the cache at the current cell.  Those stores address the cache through a small device array of cell numbers
+// (ctx->cells, written by k_fill_cells before the graph starts), so the recorded launches stay valid; the signature covers
+// the cache tensor behind such a view instead of the view's address.  A graph runs launch by launch the first time it is seen
+// (scratch buffers get their size), is recorded the second time, and replayed from then on.  Batches above 4 rows, graphs
+// whose cache stores are not all taken by the fused Q/K/V launch, and MI355_NO_GRAPH=1 stay launch by launch.
+__global__ void k_fill_cells(int32_t * cells, int head) { cells[threadIdx.x] = head + (int) threadIdx.x; }
+
+struct graph_signature {
+    uint64_t hash = 0;
+    bool capturable = false;
+    int64_t kv_head = -1;
+    int kv_stores = 0;
+};
+
+inline uint64_t sig_mix(uint64_t h, uint64_t v) {
+    h ^= v + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2);
+    return h * 0xff51afd7ed558ccdull;
+}
+
+uint64_t sig_tensor(uint64_t h, const ggml_tensor * t, bool through_cache) {
+    h = sig_mix(h, ((uint64_t) t->type << 32) | (uint64_t) t->op);
+    for (int i = 0; i < GGML_MAX_DIMS; i++) {
+        h = sig_mix(h, (uint64_t) t->ne[i]);
+        h = sig_mix(h, (uint64_t) t->nb[i]);
     }
+    return sig_mix(h, (uint64_t) (uintptr_t) (through_cache ? t->view_src->data : t->data));
+}
+
+bool is_cache_store(const ggml_tensor * node) {
+    if (node->op != GGML_OP_CPY) return false;
+    const ggml_tensor * d = node->src[1];
+    return d && d->type == GGML_TYPE_F16 && d->view_src && d->view_src->data && ggml_is_contiguous(d);
+}
+
+graph_signature sign_graph(ggml_cgraph * cgraph, std::vector<uint64_t> * trace = nullptr) {
+    graph_signature g;
+    const int n = ggml_graph_n_nodes(cgraph);
+    // the views that cache stores write through (they are graph nodes themselves, and sources of the CPY nodes)
+    std::unordered_set<const ggml_tensor *> dests;
+    for (int i = 0; i < n; i++) {
+        const ggml_tensor * node = ggml_graph_node(cgraph, i);
+        if (is_cache_store(node)) dests.insert(node->src[1]);
+    }
+    auto through_cache = [&](const ggml_tensor * t) { return dests.count(t) != 0; };
+    uint64_t h = sig_mix(0x6d693335u, (uint64_t) n);
+    int64_t batch = 0;
+    bool heads_agree = true;
+    for (int i = 0; i < n; i++) {
+        const ggml_tensor * node = ggml_graph_node(cgraph, i);
+        const bool store = is_cache_store(node);
+        h = sig_tensor(h, node, through_cache(node) || (store && node->view_src != nullptr && node->data == node->src[1]->data));
+        h = sig_mix(h, (uint64_t) node->flags);
+        if (!through_cache(node)) {   // a view's parameters hold its offset
+            for (size_t k = 0; k < GGML_MAX_OP_PARAMS / sizeof(int32_t); k += 2)
+                h = sig_mix(h, ((uint64_t) (uint32_t) node->op_params[k] << 32) | (uint32_t) node->op_params[k + 1]);
+        }
+        if (trace) trace->push_back(h);
+        for (int k = 0; k < GGML_MAX_SRC; k++) {
+            const ggml_tensor * src = node->src[k];
+            if (!src) continue;
+            // A store destination read by anything but its CPY keeps its own address in the signature.  Sources that are
+            // computed (nodes of this graph, signed in full where they are listed) are identified by their address alone.
+            if (src->op != GGML_OP_NONE && !(store && k == 1)) h = sig_mix(h, ((uint64_t) (uintptr_t) src->data << 3) | (uint64_t) k);
+            else h = sig_tensor(sig_mix(h, (uint64_t) k), src, store && k == 1);
+        }
+        if (node->op == GGML_OP_MUL_MAT && batch == 0) batch = node->src[1]->ne[1] * node->src[1]->ne[2] * node->src[1]->ne[3];
+        if (store) {
+            g.kv_stores++;
+            const ggml_tensor * d = node->src[1];
+            const int64_t off = (const char *) d->data - (const char *) d->view_src->data;
+            const int64_t row = batch > 0 ? (int64_t) ggml_nbytes(d) / batch : 0;
+            if (row <= 0 || off % row != 0 || (g.kv_head >= 0 && g.kv_head != off / row)) heads_agree = false;
+            else g.kv_head = off / row;
+        }
+    }
+    if (!heads_agree) g.kv_head = -1;
+    g.hash = h | 1;   // never 0
+    g.capturable = batch >= 1 && batch <= 4 && (g.kv_stores == 0 || (g.kv_head >= 0 && g.kv_head + 8 < 0x7fffffff));
+    return g;
+}
+
+void run_graph_launches(backend_ctx * ctx, ggml_cgraph * cgraph) {
+    ctx->cache.valid = false;
     const graph_walk w(cgraph);
     static const bool log_graph = getenv("MI355_LOG_GRAPH") != nullptr;   // node list and the nodes each launch sequence consumed
     for (int i = 0; i < w.n; i++) {
@@ -1221,14 +1422,92 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
         }
     }
     ctx->cache.valid = false;
+}
+
+ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    ctx->cache.valid = false;
+    if (!ctx->fuse) {
+        const int n = ggml_graph_n_nodes(cgraph);
+        for (int i = 0; i < n; i++) {
+            ggml_tensor * node = ggml_graph_node(cgraph, i);
+            if (!is_noop(node)) compute_node(ctx, node);
+        }
+        return GGML_STATUS_SUCCESS;
+    }
+    auto & rp = ctx->replay;
+    const int64_t t_start = ggml_time_us();
+    graph_signature sig;
+    static const bool log_replay = getenv("MI355_GRAPH_STATS") != nullptr && getenv("MI355_GRAPH_STATS")[0] == '2';
+    if (rp.enabled && log_replay) {   // also name the first node whose signature differs from the previous graph's
+        static std::vector<uint64_t> prev;
+        std::vector<uint64_t> cur;
+        sig = sign_graph(cgraph, &cur);
+        size_t k = 0;
+        while (k < cur.size() && k < prev.size() && cur[k] == prev[k]) k++;
+        const ggml_tensor * t = k < cur.size() ? ggml_graph_node(cgraph, (int) k) : nullptr;
+        fprintf(stderr, "MI355 graph: %d nodes, signature %016llx, %s, %d cache stores at cell %lld; first change at node %zu %s %s\n",
+                ggml_graph_n_nodes(cgraph), (unsigned long long) sig.hash, sig.capturable ? "replayable" : "launch by launch", sig.kv_stores,
+                (long long) sig.kv_head, k, t ? ggml_op_name(t->op) : "-", t ? t->name : "-");
+        prev.swap(cur);
+    } else if (rp.enabled) {
+        sig = sign_graph(cgraph);
+    }
+    ctx->kv_head = sig.capturable ? sig.kv_head : -1;
+    ctx->kv_redirected = 0;
+    if (ctx->kv_head >= 0 && ctx->cells_head != ctx->kv_head) {
+        hipLaunchKernelGGL(k_fill_cells, dim3(1), dim3(8), 0, ctx->stream, ctx->cells, (int) ctx->kv_head);
+        MI355_HIP_OK(hipGetLastError());
+        ctx->cells_head = ctx->kv_head;
+    }
+    if (sig.capturable && rp.exec && rp.exec_sig == sig.hash && rp.exec_gen == ctx->alloc_gen) {
+        MI355_HIP_OK(hipGraphLaunch(rp.exec, ctx->stream));
+        rp.replays++;
+        rp.host_us += (double) (ggml_time_us() - t_start);
+        return GGML_STATUS_SUCCESS;
+    }
+    const bool record = sig.capturable && sig.hash != rp.bad_sig && rp.seen_sig == sig.hash && rp.seen_gen == ctx->alloc_gen;
+    if (record && hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+        (void) hipGetLastError();
+        rp.bad_sig = sig.hash;
+    } else if (record) {
+        ctx->capturing = true;
+        ctx->capture_broken = false;
+        run_graph_launches(ctx, cgraph);
+        ctx->capturing = false;
+        hipGraph_t graph = nullptr;
+        const hipError_t end = hipStreamEndCapture(ctx->stream, &graph);
+        const bool ok = end == hipSuccess && graph != nullptr && !ctx->capture_broken && ctx->kv_redirected == sig.kv_stores;
+        if (end != hipSuccess) (void) hipGetLastError();
+        hipGraphExec_t exec = nullptr;
+        if (ok && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) == hipSuccess) {
+            if (rp.exec) MI355_HIP_OK(hipGraphExecDestroy(rp.exec));
+            if (rp.graph) MI355_HIP_OK(hipGraphDestroy(rp.graph));
+            rp.exec = exec;
+            rp.graph = graph;
+            rp.exec_sig = sig.hash;
+            rp.exec_gen = ctx->alloc_gen;
+            rp.captures++;
+            MI355_HIP_OK(hipGraphLaunch(rp.exec, ctx->stream));   // nothing has run yet: recording does not execute
+            return GGML_STATUS_SUCCESS;
+        }
+        (void) hipGetLastError();
+        if (graph) (void) hipGraphDestroy(graph);
+        rp.bad_sig = sig.hash;   // run it launch by launch, now and from now on
+        ctx->kv_redirected = 0;
+    }
+    run_graph_launches(ctx, cgraph);
+    rp.seen_sig = sig.hash;
+    rp.seen_gen = ctx->alloc_gen;
     return GGML_STATUS_SUCCESS;   // asynchronous: completion is observed through synchronize()
 }
 
 const ggml_backend_i backend_iface = {
     /* .get_name           = */ backend_get_name,
     /* .free               = */ backend_free,
-    /* .set_tensor_async   = */ nullptr,
-    /* .get_tensor_async   = */ nullptr,
+    /* .set_tensor_async   = */ backend_set_tensor_async,
+    /* .get_tensor_async   = */ backend_get_tensor_async,
     /* .cpy_tensor_async   = */ nullptr,
     /* .synchronize        = */ backend_synchronize,
     /* .graph_plan_create  = */ nullptr,
@@ -1257,7 +1536,7 @@ void device_get_props(ggml_backend_dev_t dev, ggml_backend_dev_props * props) {
     props->description = device_get_description(dev);
     props->type = GGML_BACKEND_DEVICE_TYPE_GPU;
     device_get_memory(dev, &props->memory_free, &props->memory_total);
-    props->caps = { /* async */ false, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false };
+    props->caps = { /* async */ true, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ false };
 }
 
 ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
@@ -1274,6 +1553,13 @@ ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
         delete ctx;
         return nullptr;
     }
+    const char * ng = getenv("MI355_NO_GRAPH");
+    ctx->replay.enabled = ctx->fuse && !(ng && ng[0] == '1');
+    if (hipMalloc((void **) &ctx->cells, sizeof(iota_host)) != hipSuccess) {
+        (void) hipFree(ctx->iota);
+        delete ctx;
+        return nullptr;
+    }
     if (hipStreamCreate(&ctx->stream) != hipSuccess) {   // default priority, blocking w.r.t. the null stream
         delete ctx;
         return nullptr;
@@ -1282,6 +1568,8 @@ ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
 }
 
 ggml_backend_buffer_type_t device_get_buffer_type(ggml_backend_dev_t dev) { return mi355_buffer_type(((device_ctx *) dev->context)->device); }
+
+ggml_backend_buffer_type_t device_get_host_buffer_type(ggml_backend_dev_t dev) { return mi355_host_buffer_type(dev); }
 
 bool device_supports_buft(ggml_backend_dev_t dev, ggml_backend_buffer_type_t buft) {
     return buft->iface.get_name == buft_get_name && buft->device == dev;
@@ -1295,7 +1583,7 @@ const ggml_backend_device_i device_iface = {
     /* .get_props            = */ device_get_props,
     /* .init_backend         = */ device_init_backend,
     /* .get_buffer_type      = */ device_get_buffer_type,
-    /* .get_host_buffer_type = */ nullptr,
+    /* .get_host_buffer_type = */ device_get_host_buffer_type,
     /* .buffer_from_host_ptr = */ nullptr,
     /* .supports_op          = */ device_supports_op,
     /* .supports_buft        = */ device_supports_buft,

@@ -53,16 +53,21 @@ def test_llama_bench_runs_on_the_plugin(dev, tmp_path):
 LOGITS = os.path.join(ROOT, "oracle", "_ref", "llama_logits")
 
 
-def _logits(model, ngl, n_prompt, n_decode, out, fusion=True):
+def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None):
     import numpy as np
-    env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN)
+    env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN, MI355_GRAPH_STATS="1")
     if not fusion:
         env["MI355_NO_FUSION"] = "1"
+    if not graphs:
+        env["MI355_NO_GRAPH"] = "1"
     r = subprocess.run([LOGITS, model, str(ngl), str(n_prompt), str(n_decode), out], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                        text=True, timeout=600, cwd=os.path.dirname(LOGITS))
     assert r.returncode == 0, r.stdout[-3000:]
     if ngl > 0:
         assert "MI355X" in r.stdout, "layers were not offloaded to the plug-in:\n" + r.stdout[-3000:]
+    if stats is not None:
+        m = re.search(r"MI355 graph replay: (\d+) captures, (\d+) replays", r.stdout)
+        stats["captures"], stats["replays"] = (int(m.group(1)), int(m.group(2))) if m else (0, 0)
     return np.fromfile(out, dtype=np.float32)
 
 
@@ -109,3 +114,26 @@ def test_moe_model_logits_cpu_vs_plugin(dev, tmp_path, n_prompt):
     assert cpu.shape == gpu.shape == nodes.shape and np.isfinite(gpu).all()
     assert orc.nmse(gpu, nodes) < (1e-6 if n_prompt <= 8 else 5e-4)
     assert orc.nmse(gpu, cpu) < 2e-3
+
+
+@pytest.mark.parametrize("moe", [False, True])
+def test_decode_graph_replay_equals_launch_by_launch(dev, tmp_path, moe):
+    """Decode graphs replayed as HIP graphs give the bits of the same graphs issued launch by launch, over a run that crosses a
+    256-cell boundary of the attention window (the graph changes there and is recorded again), with the prompt's prefill and
+    the host's synchronizing logits reads between the replays.  Every decoded token's logits are compared."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    model = str(tmp_path / "small.gguf")
+    if moe:
+        make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=2048, n_head=16, n_head_kv=4, n_vocab=2048, n_expert=8, n_expert_used=2)
+    else:
+        make_synthetic_gguf.write_model(model, n_layer=3, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048)
+    st = {}
+    replayed = _logits(model, 99, 249, 14, str(tmp_path / "graph.bin"), stats=st)
+    launched = _logits(model, 99, 249, 14, str(tmp_path / "eager.bin"), graphs=False)
+    assert st["captures"] >= 2 and st["replays"] >= 8, st
+    assert replayed.shape == launched.shape and np.isfinite(replayed).all()
+    assert np.array_equal(replayed, launched)
