@@ -64,14 +64,19 @@ struct gemv_batch {
 
 // COH: results are stored with device scope (written through to where every XCD sees them), for launches whose last
 // group reads rows produced by other groups
-template <int TYPE, int NCOLS, int RPW, bool QKV = false, bool COH = false>
+// LDSA: the group copies the quantized activation (NCOLS rows of K levels, then their scales) into s_act once and its four
+// waves read it from there; otherwise every wave reads it from memory.  On the 14336 x 4096 Q4_K product the activation
+// reads of the 7168 waves (36 MB from L2) outweighed the 33 MB of weights and competed with them: 8.7 -> 7.9 us with the
+// copy in LDS.  The first step's weight loads are issued before the copy, so the copy's round trip hides behind them.
+template <int TYPE, int NCOLS, int RPW, bool QKV = false, bool COH = false, bool LDSA = false>
 __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const int8_t *__restrict__ aq,
-                                          const act_ds *__restrict__ ads, int K, const gemv_rope *rp = nullptr) {
+                                          const act_ds *__restrict__ ads, int K, const gemv_rope *rp = nullptr, uint8_t *s_act = nullptr) {
     typedef wq<TYPE> T;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t row0 = ((int64_t)group * 4 + wave) * RPW;
-    if (row0 >= m.N) return;   // whole wave exits together
+    const bool wave_live = row0 < m.N;   // uniform over the wave
+    if (!LDSA && !wave_live) return;     // with the copy in LDS a wave without rows still takes its share of the copy
 
     const row_layout L = make_row_layout(TYPE, K);
     const int nchunks = K / T::CHUNK;
@@ -107,12 +112,30 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
         asm volatile("" : "+v"(rope_c), "+v"(rope_s), "+v"(cell));
     }
 
+    typename T::chunk w_first[RPW];
+    if constexpr (LDSA) {
+        const int c = lane < nchunks ? lane : nchunks - 1;
+#pragma unroll
+        for (int r = 0; r < RPW; r++) w_first[r] = T::load_w(rows[r], L, c);
+        int8_t *s_q = (int8_t *)s_act;
+        act_ds *s_ds = (act_ds *)(s_act + NCOLS * K);
+        for (int i = threadIdx.x * 16; i < NCOLS * K; i += 256 * 16) *(u32x4 *)(s_q + i) = load16(aq + i);
+        for (int i = threadIdx.x; i < NCOLS * nblk; i += 256) s_ds[i] = ads[i];
+        __syncthreads();
+        if (!wave_live) return;
+        aq = s_q;
+        ads = s_ds;
+    }
+
     for (int c0 = 0; c0 < nchunks; c0 += 64) {
         const int c = c0 + lane;
         if (c < nchunks) {
             typename T::chunk w[RPW];
 #pragma unroll
-            for (int r = 0; r < RPW; r++) w[r] = T::load_w(rows[r], L, c);
+            for (int r = 0; r < RPW; r++) {
+                if (LDSA && c0 == 0) w[r] = w_first[r];
+                else w[r] = T::load_w(rows[r], L, c);
+            }
 #pragma unroll
             for (int col = 0; col < NCOLS; col++) {
                 const typename T::act A = T::load_a(aq + (int64_t)col * K, ads + col * nblk, c);
@@ -167,19 +190,22 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
     }
 }
 
-template <int NCOLS, int RPW, bool COH = false>
+// dynamic LDS of the launches below: the group's copy of the activation (LDSA), act_lds_bytes() bytes
+extern __shared__ __attribute__((aligned(16))) uint8_t s_act_dyn[];
+
+template <int NCOLS, int RPW, bool COH = false, bool LDSA = false>
 __device__ __forceinline__ void gemv_dispatch(const gemv_item &m, int group, const int8_t *__restrict__ aq,
                                               const act_ds *__restrict__ ads, int K) {
     switch (m.type) {   // uniform over the group
-        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
-        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
-        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
-        default: gemv_body<MI355_Q6_K, NCOLS, RPW, false, COH>(m, group, aq, ads, K); break;
+        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
+        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
+        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
+        default: gemv_body<MI355_Q6_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
     }
 }
 
 // Q, K and V projections in one launch; finished rows are rotated and land in q (f32) or in the f16 KV cache
-template <int NCOLS>
+template <int NCOLS, bool LDSA>
 __global__ void __launch_bounds__(256) k_gemv_qkv(gemv_batch b, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K, gemv_rope rp) {
     const int g = blockIdx.x;
     int i = 0;
@@ -189,28 +215,28 @@ __global__ void __launch_bounds__(256) k_gemv_qkv(gemv_batch b, const int8_t *__
     const gemv_item &m = b.it[i];
     const int group = g - m.first_group;
     switch (m.type) {   // uniform over the group
-        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
-        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
-        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
-        default: gemv_body<MI355_Q6_K, NCOLS, 2, true>(m, group, aq, ads, K, &rp); break;
+        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
+        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
+        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
+        default: gemv_body<MI355_Q6_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
     }
 }
 
 // single matrix, type known at compile time (smallest code, used by mi355_mul_mat_vec_q)
-template <int TYPE, int NCOLS, int RPW>
+template <int TYPE, int NCOLS, int RPW, bool LDSA>
 __global__ void __launch_bounds__(256) k_gemv_q(gemv_item m, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K) {
-    gemv_body<TYPE, NCOLS, RPW>(m, blockIdx.x, aq, ads, K);
+    gemv_body<TYPE, NCOLS, RPW, false, false, LDSA>(m, blockIdx.x, aq, ads, K, nullptr, s_act_dyn);
 }
 
 // several matrices sharing one activation
-template <int NCOLS, int RPW>
+template <int NCOLS, int RPW, bool LDSA>
 __global__ void __launch_bounds__(256) k_gemv_multi(gemv_batch b, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K) {
     const int g = blockIdx.x;
     int i = 0;
 #pragma unroll
     for (int j = 1; j < 4; j++)
         if (j < b.n && g >= b.it[j].first_group) i = j;
-    gemv_dispatch<NCOLS, RPW>(b.it[i], g - b.it[i].first_group, aq, ads, K);
+    gemv_dispatch<NCOLS, RPW, false, LDSA>(b.it[i], g - b.it[i].first_group, aq, ads, K);
 }
 
 // ---- a launch whose last-arriving groups also do the nodes that follow the product ------------
@@ -260,13 +286,13 @@ __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qr
 
 // gate and up projections (llm_build_ffn, src/llama.cpp:280-320) with UNARY(SILU), MUL and the Q8_1 quantization of
 // the product done per 32-row block by whichever of the block's 8 groups (4 per matrix, 8 rows each) finishes last
-template <int NCOLS>
+template <int NCOLS, bool LDSA>
 __global__ void __launch_bounds__(256) k_gemv_gate_up(gemv_batch b, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K, gemv_tail t) {
     __shared__ unsigned s_ticket;
     const int g = blockIdx.x;
     const int i = g >= b.it[1].first_group ? 1 : 0;
     const int group = g - b.it[i].first_group;
-    gemv_dispatch<NCOLS, 2, true>(b.it[i], group, aq, ads, K);
+    gemv_dispatch<NCOLS, 2, true, LDSA>(b.it[i], group, aq, ads, K);
     // Every wave waits until its device-scope stores have been acknowledged before it reaches the barrier: the
     // barrier's own wait covers LDS and scalar loads only, and a ticket that overtakes a row store would let the
     // last group read that row too early.
@@ -377,18 +403,46 @@ static int pick_rpw(int64_t total_rows) {
     return 1;
 }
 
+// bytes of LDS for the group's copy of the activation, or 0 when every wave reads it from memory.  The copy pays when the
+// launch has several generations of groups per compute unit (its round trip then hides behind other groups' loads, and the
+// activation reads it saves are the larger part of the launch's L2 traffic): output projection 98.9 -> 77.5 us (6.8 TB/s),
+// 14336 x 4096 8.6 -> 8.0 us.  A launch whose groups are all resident at once (wo, ffn_down, Q/K/V: ~1000 groups) is one
+// dependent chain per wave, and the copy's barrier lengthens it (+0.3 to +0.7 us measured).  Up to four activation rows, and
+// small enough that eight groups still fit a compute unit.  MI355_GEMV_NO_LDS=1 turns the copy off (tuning aid).
+static size_t act_lds_bytes(int ncols, int64_t K, int64_t groups) {
+    static const bool off = getenv("MI355_GEMV_NO_LDS") != nullptr;
+    const int64_t bytes = (int64_t)ncols * (K + K / 4);
+    return (!off && groups >= 1536 && ncols <= 4 && bytes <= 20480) ? (size_t)bytes : 0;
+}
+
 template <int NCOLS>
 static void launch_multi(int rpw, hipStream_t s, const gemv_batch &b, unsigned grid, const int8_t *aq, const act_ds *ads, int K) {
-    if (rpw == 1) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 1>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
-    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 2>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
-    else hipLaunchKernelGGL((k_gemv_multi<NCOLS, 4>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    if constexpr (NCOLS <= 4) {
+        if (const size_t lds = act_lds_bytes(NCOLS, K, grid)) {
+            if (rpw == 1) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 1, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
+            else if (rpw == 2) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 2, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
+            else hipLaunchKernelGGL((k_gemv_multi<NCOLS, 4, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
+            return;
+        }
+    }
+    if (rpw == 1) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 1, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 2, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    else hipLaunchKernelGGL((k_gemv_multi<NCOLS, 4, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
 }
 
 template <int TYPE, int NCOLS>
 static void launch_single(int rpw, hipStream_t s, const gemv_item &m, unsigned grid, const int8_t *aq, const act_ds *ads, int K) {
-    if (rpw == 1) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 1>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
-    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 2>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
-    else hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 4>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    if constexpr (NCOLS <= 4) {
+        if (const size_t lds = act_lds_bytes(NCOLS, K, grid)) {
+            if (rpw == 1) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 1, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
+            else if (rpw == 2) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 2, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
+            else hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 4, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
+            return;
+        }
+    }
+    if (rpw == 1) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 1, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 2, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    else hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 4, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
 }
 
 template <int TYPE>
@@ -554,11 +608,24 @@ int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat
     hipStream_t s = (hipStream_t)stream;
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + B * K);
+    const size_t lds = act_lds_bytes((int)B, K, groups);
     switch (B) {
-        case 1: hipLaunchKernelGGL(k_gemv_qkv<1>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
-        case 2: hipLaunchKernelGGL(k_gemv_qkv<2>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
-        case 3: hipLaunchKernelGGL(k_gemv_qkv<3>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
-        default: hipLaunchKernelGGL(k_gemv_qkv<4>, dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp); break;
+        case 1:
+            if (lds) hipLaunchKernelGGL((k_gemv_qkv<1, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else hipLaunchKernelGGL((k_gemv_qkv<1, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            break;
+        case 2:
+            if (lds) hipLaunchKernelGGL((k_gemv_qkv<2, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else hipLaunchKernelGGL((k_gemv_qkv<2, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            break;
+        case 3:
+            if (lds) hipLaunchKernelGGL((k_gemv_qkv<3, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else hipLaunchKernelGGL((k_gemv_qkv<3, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            break;
+        default:
+            if (lds) hipLaunchKernelGGL((k_gemv_qkv<4, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else hipLaunchKernelGGL((k_gemv_qkv<4, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            break;
     }
     return launch_status("k_gemv_qkv");
 }
@@ -610,11 +677,24 @@ int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, in
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + B * K);
     const dim3 grid((unsigned)(2 * per));
+    const size_t lds = act_lds_bytes((int)B, K, 2 * per);
     switch (B) {
-        case 1: hipLaunchKernelGGL(k_gemv_gate_up<1>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
-        case 2: hipLaunchKernelGGL(k_gemv_gate_up<2>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
-        case 3: hipLaunchKernelGGL(k_gemv_gate_up<3>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
-        default: hipLaunchKernelGGL(k_gemv_gate_up<4>, grid, dim3(256), 0, s, b, aq, ads, (int)K, t); break;
+        case 1:
+            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<1, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else hipLaunchKernelGGL((k_gemv_gate_up<1, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            break;
+        case 2:
+            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<2, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else hipLaunchKernelGGL((k_gemv_gate_up<2, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            break;
+        case 3:
+            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<3, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else hipLaunchKernelGGL((k_gemv_gate_up<3, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            break;
+        default:
+            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<4, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else hipLaunchKernelGGL((k_gemv_gate_up<4, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            break;
     }
     return launch_status("k_gemv_gate_up");
 }

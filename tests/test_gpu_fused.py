@@ -139,6 +139,12 @@ def test_fused_layer_stack_matches_node_sequence(dev):
         run.set_inputs(emb, pos0, T, 256)
         b = run.forward(T, 256, last_only=False).cpu().numpy().copy()
         assert np.isfinite(a).all() and np.isfinite(b).all()
+        if T <= 4:   # decode: SiLU*up by the gate/up launch's last groups, or as a launch of its own - same bits
+            run.fuse_tail = not run.fuse_tail
+            run.set_inputs(emb, pos0, T, 256)
+            c = run.forward(T, 256, last_only=False).cpu().numpy().copy()
+            run.fuse_tail = not run.fuse_tail
+            assert np.array_equal(b, c), (T, pos0)
         # Decode launches the same arithmetic in both sequences.  Prefill rounds the RMS norm differently in the
         # last bit, which flips a few activation levels; with one scale per 256 elements a single flip in a
         # row that holds an outlier moves that row by ~1e-5, and two random-weight layers amplify it.
