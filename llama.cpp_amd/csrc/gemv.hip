@@ -316,7 +316,7 @@ __global__ void __launch_bounds__(256) k_gemv_gate_up(gemv_batch b, const int8_t
 
 // MUL_MAT_ID, one activation row per expert slot: blockIdx.y = slot = t * n_used + e.  The
 // expert id is read on the device, so no host synchronisation is needed to route tokens.
-template <int TYPE, int RPW>
+template <int TYPE, int RPW, bool LDSA>
 __global__ void __launch_bounds__(256) k_gemv_id(const uint8_t *__restrict__ as, const int8_t *__restrict__ aq,
                                                  const act_ds *__restrict__ ads, const int32_t *__restrict__ ids,
                                                  int64_t ids_stride, float *__restrict__ dst, int64_t N, int K,
@@ -334,7 +334,7 @@ __global__ void __launch_bounds__(256) k_gemv_id(const uint8_t *__restrict__ as,
     m.dst_stride = N;
     m.type = TYPE;
     m.first_group = 0;
-    gemv_body<TYPE, 1, RPW>(m, blockIdx.x, aq + arow * K, ads + arow * (K >> 5), K);
+    gemv_body<TYPE, 1, RPW, false, false, LDSA>(m, blockIdx.x, aq + arow * K, ads + arow * (K >> 5), K, nullptr, s_act_dyn);
 }
 
 // Same routing for weight rows that are not 16-byte aligned (byte loads): one wave per (row, slot).
@@ -722,9 +722,13 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
     }
     const int rpw = pick_rpw(N * n_used) > 2 ? 2 : pick_rpw(N * n_used);
     const dim3 grid((unsigned)((N + 4 * rpw - 1) / (4 * rpw)), (unsigned)(n_used * T));
+    // an activation row of the split layout is 16-byte aligned inside the workspace when K % 64 == 0 (levels and scales)
+    const size_t lds = K % 64 == 0 ? act_lds_bytes(1, K, (int64_t)grid.x * grid.y) : 0;
 #define MI355_ID_LAUNCH(TY)                                                                                           \
-    if (rpw == 1) hipLaunchKernelGGL((k_gemv_id<TY, 1>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
-    else hipLaunchKernelGGL((k_gemv_id<TY, 2>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1);
+    if (lds && rpw == 1) hipLaunchKernelGGL((k_gemv_id<TY, 1, true>), grid, dim3(256), lds, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
+    else if (lds) hipLaunchKernelGGL((k_gemv_id<TY, 2, true>), grid, dim3(256), lds, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
+    else if (rpw == 1) hipLaunchKernelGGL((k_gemv_id<TY, 1, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
+    else hipLaunchKernelGGL((k_gemv_id<TY, 2, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1);
     switch (type) {
         case MI355_Q4_0: MI355_ID_LAUNCH(MI355_Q4_0) break;
         case MI355_Q8_0: MI355_ID_LAUNCH(MI355_Q8_0) break;
