@@ -20,7 +20,7 @@ sys.path.insert(0, os.path.join(ROOT, "llama.cpp_amd"))
 HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the roofline kernel moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of this command,
 # calibrated on the copy kernel below (profiles/gemv_q4k_14336x4096_hbm_traffic.txt)
-GEMV_TRAFFIC_BYTES = 33160200
+GEMV_TRAFFIC_BYTES = 33169000
 
 
 def cpu_baseline(n_threads, budget_s=20.0):

@@ -409,6 +409,9 @@ static int pick_rpw(int64_t total_rows) {
 // 14336 x 4096 8.6 -> 8.0 us.  A launch whose groups are all resident at once (wo, ffn_down, Q/K/V: ~1000 groups) is one
 // dependent chain per wave, and the copy's barrier lengthens it (+0.3 to +0.7 us measured).  Up to four activation rows, and
 // small enough that eight groups still fit a compute unit.  MI355_GEMV_NO_LDS=1 turns the copy off (tuning aid).
+// Measured and not adopted: splitting K over the four waves of a group (each wave reads a quarter of the activation, partial
+// sums meet in LDS at the end) - Q4_K 4096 x 4096 4.9 -> 4.3 us and 14336 x 4096 8.2 -> 7.9 us, but Q6_K slower throughout
+// (4096 x 14336 11.2 -> 14.0 us, output projection 80 -> 87 us): its 16-byte pieces per lane then form 256-byte runs.
 static size_t act_lds_bytes(int ncols, int64_t K, int64_t groups) {
     static const bool off = getenv("MI355_GEMV_NO_LDS") != nullptr;
     const int64_t bytes = (int64_t)ncols * (K + K / 4);
