@@ -335,6 +335,7 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
     MI355_REQUIRE(max_bias <= 0.0f || mask != nullptr, "flash_attn: max_bias needs a mask");
     MI355_REQUIRE(act == nullptr || (D % 32 == 0 && ((uintptr_t)act & 15) == 0), "flash_attn: quantized output needs head size %% 32 == 0 and a 16-byte aligned buffer");
     fattn_args a;
+    a.kv_extent = nullptr;
     a.act_q = (int8_t *)act;
     a.act_s = act ? (act_ds *)((int8_t *)act + Nq * Hq * D) : nullptr;
     a.q = (const uint8_t *)q; a.k = (const uint8_t *)k; a.v = (const uint8_t *)v; a.mask = (const uint8_t *)mask;
@@ -357,7 +358,7 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
     const int R = (int)(Hq / Hkv);
     hipStream_t s = (hipStream_t)stream;
     if (Nq >= 16 && act == nullptr) {   // prefill: f16 matrix cores
-        const int rc = launch_fattn_mma(s, a, D);
+        const int rc = launch_fattn_mma(s, a, D, ws_bytes);
         if (rc <= 0) return rc;
     }
     // Decode and small batches over a long context: matrix cores with (token, head) columns, which read a kv head's

@@ -11,6 +11,8 @@ struct fattn_args {
     int8_t *act_q;   // optional: Q8_1 of dst rows (Hq*D elements per query) in the split activation layout
     act_ds *act_s;
     float *ws;       // partial results when n_splits > 1: [Nq][Hq][n_splits][D + 2]
+    const int32_t *kv_extent;   // prefill, optional: per tile of 32 queries, the number of leading cells after which every
+                                // mask entry of the tile's rows is -inf (see k_mask_extent); null = all Nkv cells
     int64_t Nq, Nkv, Hq, Hkv;
     size_t q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1;
     float scale, max_bias, softcap;
@@ -22,7 +24,7 @@ struct fattn_args {
 };
 
 // f16 matrix-core kernel for many query rows; returns MI355_OK, an error, or 1 when the shape is not served
-int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D);
+int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);
 // the same for a few query rows (decode): one kv split per group, partials merged by k_fattn_combine
 int launch_fattn_mma_dec(hipStream_t s, fattn_args &a, int64_t D);
 

@@ -192,8 +192,39 @@ __device__ __forceinline__ f32x16 scores(const f16x8 (&qf)[D / 16], const _Float
 }
 
 // ---- prefill --------------------------------------------------------------------------------
+// How far each tile of 32 queries can see: extent[t] = 1 + the last cell whose mask entry is not -inf in any of the tile's
+// rows (0 when there is none).  With llama.cpp's causal mask the tiles of a prompt see a growing prefix of the cache, and the
+// prefill kernel stops staging K/V tiles at that point instead of loading, scoring and then discarding them.  One group
+// per tile; threads take 8 cells (16 bytes) of each row at a time.  Needs 16-byte aligned mask rows and Nkv % 8 == 0.
+__global__ void __launch_bounds__(256) k_mask_extent(const uint8_t *__restrict__ mask, size_t mask_nb1, int64_t Nq, int64_t Nkv,
+                                                     int32_t *__restrict__ extent) {
+    __shared__ int s_max[4];
+    const int64_t q0 = (int64_t)blockIdx.x * 32;
+    int last = -1;
+    for (int64_t c = (int64_t)threadIdx.x * 8; c < Nkv; c += 256 * 8) {
+        u32x4 any = {0, 0, 0, 0};   // per 16-bit field: non-zero when some row's entry differs from -inf (0xFC00)
+        for (int r = 0; r < 32; r++) {
+            const int64_t iq = q0 + r < Nq ? q0 + r : Nq - 1;
+            const u32x4 m = load16(mask + iq * mask_nb1 + c * 2);
+#pragma unroll
+            for (int i = 0; i < 4; i++) any[i] |= m[i] ^ 0xFC00FC00u;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {   // c grows, so the last assignment is the largest visible cell
+            const u32 w = any[i];
+            if (w & 0x0000FFFFu) last = (int)c + 2 * i;
+            if (w & 0xFFFF0000u) last = (int)c + 2 * i + 1;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
+    if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = last;
+    __syncthreads();
+    if (threadIdx.x == 0) extent[blockIdx.x] = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3])) + 1;
+}
+
 template <int D, int HPW>
-__global__ void __launch_bounds__(256) k_fattn_mma(fattn_args a) {
+__global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
     typedef kv_stage<D, 256> stage_t;
     constexpr int QTW = 4 / HPW;   // query tiles per group
     __shared__ __attribute__((aligned(16))) _Float16 sK[FM_BC * stage_t::KP];
@@ -222,6 +253,18 @@ __global__ void __launch_bounds__(256) k_fattn_mma(fattn_args a) {
         for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
     float m = FM_NEG, l = 0.0f;
 
+    // cells past kv_limit are masked for every query of this group
+    int64_t kv_limit = a.Nkv;
+    if (a.kv_extent) {
+        int e = 0;
+#pragma unroll
+        for (int j = 0; j < QTW; j++) {
+            const int64_t t = (int64_t)blockIdx.x * QTW + j;
+            if (t * 32 < a.Nq) e = max(e, a.kv_extent[t]);
+        }
+        kv_limit = e < a.Nkv ? e : a.Nkv;
+    }
+
     stage_t st;
     u32x2 mnext[2][4];
     auto prefetch = [&](int64_t kv0) {
@@ -230,8 +273,8 @@ __global__ void __launch_bounds__(256) k_fattn_mma(fattn_args a) {
         fetch_mask<4>(mnext[0], mrow, vec_ok, kv0 + 4 * lhi, a.Nkv);
         fetch_mask<4>(mnext[1], mrow, vec_ok, kv0 + 32 + 4 * lhi, a.Nkv);
     };
-    prefetch(0);
-    for (int64_t kv0 = 0; kv0 < a.Nkv; kv0 += FM_BC) {
+    if (kv_limit > 0) prefetch(0);
+    for (int64_t kv0 = 0; kv0 < kv_limit; kv0 += FM_BC) {
         __syncthreads();   // the previous tile has been consumed
         st.commit(sK, sVt, tid);
         u32x2 mcur[2][4];
@@ -240,7 +283,7 @@ __global__ void __launch_bounds__(256) k_fattn_mma(fattn_args a) {
 #pragma unroll
             for (int g = 0; g < 4; g++) mcur[u][g] = mnext[u][g];
         __syncthreads();
-        if (kv0 + FM_BC < a.Nkv) prefetch(kv0 + FM_BC);
+        if (kv0 + FM_BC < kv_limit) prefetch(kv0 + FM_BC);
 
         // scores of 64 cells for this lane's query: S[u][r] <-> cell kv0 + 32u + 8*(r/4) + 4*lhi + r%4
         f32x16 S[2];
@@ -491,9 +534,22 @@ int launch_dec(hipStream_t s, const fattn_args &a) {
 
 }  // namespace
 
-int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D) {
+int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes) {
     if (a.Hkv * (a.Hq / a.Hkv) > 65535 || (a.Nq + 31) / 32 > 0x7fffffff) return 1;
     if ((a.q_nb1 % 16) != 0 || (a.q_nb2 % 16) != 0) return 1;
+    if (D != 64 && D != 128) return 1;
+    a.kv_extent = nullptr;
+    const int64_t n_tiles = (a.Nq + 31) / 32;
+    // The pre-pass pays when there are more groups than the chip holds at once (two per compute unit): then a group that stops
+    // early makes room for the next one.  With fewer groups the launch takes as long as its longest group either way.
+    const int64_t n_groups = n_tiles * a.Hq / 4;
+    if (n_groups > 512 && a.mask && a.ws && ws_bytes >= (size_t)n_tiles * sizeof(int32_t) && (((uintptr_t)a.mask | a.mask_nb1) & 15) == 0 &&
+        a.Nkv % 8 == 0 && a.Nkv >= 2 * FM_BC && a.Nkv < 0x7fffffff) {
+        hipLaunchKernelGGL(k_mask_extent, dim3((unsigned)n_tiles), dim3(256), 0, s, a.mask, a.mask_nb1, a.Nq, a.Nkv, (int32_t *)a.ws);
+        const int rc = launch_status("k_mask_extent");
+        if (rc != MI355_OK) return rc;
+        a.kv_extent = (const int32_t *)a.ws;
+    }
     switch (D) {
         case 64: return launch_hpw<64>(s, a);
         case 128: return launch_hpw<128>(s, a);

@@ -238,7 +238,7 @@ def mul_mat_id(t, as_dev, b, ids, n_used):
     return dst
 
 
-def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, softcap=0.0, quantized=False):
+def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, softcap=0.0, quantized=False, workspace=True):
     """q f32 [Hq, Nq, D] (any head/row strides), k,v f16 [Hkv, Nkv, D], mask f16 [>=Nq, Nkv] or None -> f32 [Nq, Hq, D]
     (quantized=True: also returns the Q8_1 activation workspace of the output rows)"""
     import torch
@@ -246,12 +246,12 @@ def flash_attn_ext(q, k, v, mask, scale, max_bias=0.0, softcap=0.0, quantized=Fa
     Hkv, Nkv, _ = k.shape
     assert q.stride(2) == 1 and k.stride(2) == 1 and v.stride(2) == 1
     need = load().mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq)
-    ws = torch.empty(min(need, 1 << 28), dtype=torch.uint8, device=q.device)
+    ws = torch.empty(min(need, 1 << 28) if workspace else 0, dtype=torch.uint8, device=q.device)   # none: no kv splits, no mask pre-pass
     dst = torch.empty((Nq, Hq, D), dtype=torch.float32, device=q.device)
     args = (_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(mask), _ptr(dst), D, Nq, Nkv, Hq, Hkv,
             q.stride(1) * 4, q.stride(0) * 4, k.stride(1) * 2, k.stride(0) * 2,
             v.stride(1) * 2, v.stride(0) * 2, mask.stride(0) * 2 if mask is not None else 0,
-            scale, max_bias, softcap, _ptr(ws), ws.numel())
+            scale, max_bias, softcap, _ptr(ws) if workspace else None, ws.numel())
     if quantized:
         act = torch.empty(load().mi355_act_bytes(Hq * D, Nq), dtype=torch.uint8, device=q.device)
         check(load().mi355_flash_attn_ext_quant(*args, _ptr(act)))

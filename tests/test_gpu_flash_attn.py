@@ -106,3 +106,43 @@ def test_quantized_output_matches_separate_quantization(dev, D, Nq, Nkv, Hq, Hkv
     assert torch.equal(dst, plain)
     want = mi355.quantize_act(dst.reshape(Nq, Hq * D))
     assert torch.equal(act, want)
+
+
+@pytest.mark.parametrize("kind", ["causal", "window", "holes", "late_cell", "blind_tile"])
+def test_prefill_mask_extent_prepass(dev, kind):
+    """prefill stops staging K/V where the mask pre-pass says no query of the tile can see any further: same bits as the run
+    without the pre-pass (no workspace), for causal, sliding-window and irregular masks, a single visible cell at the very end
+    of one row, and a tile whose 32 queries see nothing"""
+    import torch
+    import mi355
+    rng = np.random.default_rng(len(kind))
+    D, Nq, Nkv, Hq, Hkv = 128, 2100, 2304, 32, 8     # 66 query tiles x 8 kv heads: more groups than the chip holds, so the pre-pass runs
+    q, k, v, mask = _inputs(rng, D, Nq, Nkv, Hq, Hkv, causal=True)
+    mask = mask.astype(np.float32)
+    if kind == "window":
+        j = np.arange(Nkv)[None, :]
+        i = np.arange(mask.shape[0])[:, None]
+        mask = np.where((j <= Nkv - Nq + i) & (j > Nkv - Nq + i - 100), 0.0, -np.inf).astype(np.float32)
+        mask[Nq:] = -np.inf
+    elif kind == "holes":
+        mask[rng.uniform(size=mask.shape) < 0.3] = -np.inf
+        mask[:Nq, 0] = 0.0
+    elif kind == "late_cell":
+        mask[5, Nkv - 1] = 0.0
+    elif kind == "blind_tile":
+        mask[64:96] = -np.inf
+    mask = mask.astype(np.float16)
+    scale = 1.0 / np.sqrt(D)
+    qd, kd, vd = (torch.from_numpy(a).to(dev) for a in (q, k, v))
+    md = torch.from_numpy(mask).to(dev)
+    with_pass = mi355.flash_attn_ext(qd, kd, vd, md, scale).cpu().numpy()
+    without = mi355.flash_attn_ext(qd, kd, vd, md, scale, workspace=False).cpu().numpy()
+    assert np.array_equal(with_pass, without)
+    if kind == "blind_tile":
+        assert np.all(with_pass[64:96] == 0.0)    # a query that sees nothing gets zeros
+    # the textbook form on a slice (the oracle is scalar C): two heads, rows around the special cases
+    rows = [0, 5, 63, 100, 1500, Nq - 1]
+    for h in (0, 21):
+        ms = np.concatenate([mask[rows], np.full((64 - len(rows), Nkv), -np.inf, dtype=np.float16)])
+        f64 = orc.flash_attn("f64", q[h:h + 1][:, rows], k[h // 4:h // 4 + 1].view(np.uint16), v[h // 4:h // 4 + 1].view(np.uint16), ms.view(np.uint16), scale)
+        assert orc.nmse(with_pass[rows][:, h:h + 1], f64) < 1e-5
