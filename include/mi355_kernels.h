@@ -219,7 +219,9 @@ int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
  * emits (src/llama.cpp:157-199; ggml_compute_forward_dup_f32, ggml-cpu.c:3519-3830), with the row taken from device
  * memory so that a captured launch sequence does not change as the cache fills. */
 int mi355_set_rows(void *stream, const mi355_tensor *src, const int32_t *rows, const mi355_tensor *dst);
-/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, ids i32 [n, b2, b3]; dst f32 */
+/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, or whole quantized rows (Q4_0, Q8_0, Q4_K, Q6_K in the
+ * device row layout, nb[1] = row bytes; dequantize_row_*, ggml-quants.c:255-273, 349-363, 1280-1302, 1690-1719), ids i32
+ * [n, b2, b3]; dst f32 */
 int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ids, const mi355_tensor *dst);
 /* ggml_compute_forward_soft_max_f32 (ggml-cpu.c:8959-9055): mask f32 or f16 or NULL */
 int mi355_soft_max(void *stream, const mi355_tensor *src, const mi355_tensor *mask, const mi355_tensor *dst, float scale,

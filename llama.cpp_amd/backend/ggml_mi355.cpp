@@ -540,9 +540,13 @@ bool device_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
             const bool sf = st == GGML_TYPE_F32 || st == GGML_TYPE_F16, df = dt == GGML_TYPE_F32 || dt == GGML_TYPE_F16;
             return (sf && df) || (st == GGML_TYPE_I32 && dt == GGML_TYPE_I32);
         }
-        case GGML_OP_GET_ROWS:
-            return (op->src[0]->type == GGML_TYPE_F32 || op->src[0]->type == GGML_TYPE_F16) && op->src[1]->type == GGML_TYPE_I32 &&
-                   op->type == GGML_TYPE_F32 && op->src[1]->ne[3] == 1;
+        case GGML_OP_GET_ROWS: {
+            const ggml_tensor * a = op->src[0];
+            if (op->src[1]->type != GGML_TYPE_I32 || op->type != GGML_TYPE_F32 || op->src[1]->ne[3] != 1) return false;
+            if (a->type == GGML_TYPE_F32 || a->type == GGML_TYPE_F16) return true;
+            // quantized rows: whole rows in the device layout (views over rows and batches are fine)
+            return is_weight_type(a->type) && a->nb[0] == ggml_type_size(a->type) && a->nb[1] == ggml_row_size(a->type, a->ne[0]);
+        }
         case GGML_OP_SOFT_MAX: {
             const ggml_tensor * mask = op->src[1];
             if (!f32_rows(op->src[0]) || !ggml_is_contiguous(op)) return false;

@@ -5,6 +5,7 @@
 // checks for it.  These are HBM-trivial next to the weight stream, so they are kept simple:
 // one thread per element or one wave/group per row, 16-byte accesses where rows allow.
 #include "common.hpp"
+#include "qdot.hpp"
 
 #include <float.h>
 
@@ -154,6 +155,19 @@ __global__ void k_get_rows(tens src, tens ids, tens dst, int64_t n) {
     const int32_t r = *(const int32_t *)(ids.data + i1 * ids.nb[0] + i2 * ids.nb[1] + i3 * ids.nb[2]);
     const TS v = *(const TS *)(src.data + i0 * src.nb[0] + (int64_t)r * src.nb[1] + i2 * src.nb[2] + i3 * src.nb[3]);
     *(float *)(dst.data + i0 * dst.nb[0] + i1 * dst.nb[1] + i2 * dst.nb[2] + i3 * dst.nb[3]) = (float)v;
+}
+
+// Rows of a quantized matrix (device row layout) as f32: dequantize_row_q4_0 / _q8_0 / _q4_K / _q6_K (ggml/src/ggml-quants.c:255-273,
+// 349-363, 1280-1302, 1690-1719) of the selected rows, ggml_compute_forward_get_rows_q (ggml-cpu.c:8464-8506).  One thread per element.
+template <int TYPE>
+__global__ void k_get_rows_q(tens src, tens ids, tens dst, int64_t n, row_layout L) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t i0 = i % dst.ne[0], i1 = (i / dst.ne[0]) % dst.ne[1], i2 = (i / (dst.ne[0] * dst.ne[1])) % dst.ne[2],
+                  i3 = i / (dst.ne[0] * dst.ne[1] * dst.ne[2]);
+    const int32_t r = *(const int32_t *)(ids.data + i1 * ids.nb[0] + i2 * ids.nb[1] + i3 * ids.nb[2]);
+    const uint8_t *row = src.data + (int64_t)r * src.nb[1] + i2 * src.nb[2] + i3 * src.nb[3];
+    *(float *)(dst.data + i0 * dst.nb[0] + i1 * dst.nb[1] + i2 * dst.nb[2] + i3 * dst.nb[3]) = weight_value<TYPE>(row, L, i0);
 }
 
 // ---------------------------------------------------------------- scatter rows (KV-cache store)
@@ -413,13 +427,27 @@ int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst) {
 }
 
 int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ids, const mi355_tensor *dst) {
-    MI355_REQUIRE((src->type == MI355_F32 || src->type == MI355_F16) && ids->type == MI355_I32 && dst->type == MI355_F32,
-                  "get_rows: src f32/f16, ids i32, dst f32 only");
+    MI355_REQUIRE((src->type == MI355_F32 || src->type == MI355_F16 || is_weight_type(src->type)) && ids->type == MI355_I32 && dst->type == MI355_F32,
+                  "get_rows: src f32/f16/quantized, ids i32, dst f32 only");
     MI355_REQUIRE(dst->ne[0] == src->ne[0] && dst->ne[1] == ids->ne[0] && dst->ne[2] == ids->ne[1] && dst->ne[3] == ids->ne[2],
                   "get_rows: dst shape does not match ids");
     const int64_t n = nelements(dst);
     if (n == 0) return MI355_OK;
     const dim3 grid(grid1d(n, 256)), block(256);
+    if (is_weight_type(src->type)) {
+        const int64_t K = src->ne[0];
+        MI355_REQUIRE(K % type_block_elems(src->type) == 0, "get_rows: row length %lld is not a multiple of the block size", (long long)K);
+        const row_layout L = make_row_layout(src->type, K);
+        MI355_REQUIRE((int64_t)src->nb[1] == L.row_bytes, "get_rows: quantized rows must be whole and contiguous");
+        hipStream_t s = (hipStream_t)stream;
+        switch (src->type) {
+            case MI355_Q4_0: hipLaunchKernelGGL(k_get_rows_q<MI355_Q4_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            case MI355_Q8_0: hipLaunchKernelGGL(k_get_rows_q<MI355_Q8_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            case MI355_Q4_K: hipLaunchKernelGGL(k_get_rows_q<MI355_Q4_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            default: hipLaunchKernelGGL(k_get_rows_q<MI355_Q6_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+        }
+        return launch_status("k_get_rows_q");
+    }
     if (src->type == MI355_F32) hipLaunchKernelGGL(k_get_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
     else hipLaunchKernelGGL(k_get_rows<_Float16>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
     return launch_status("k_get_rows");

@@ -136,6 +136,35 @@ def test_get_rows(dev):
     assert np.array_equal(od.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("name,t", [("q4_0", orc.Q4_0), ("q8_0", orc.Q8_0), ("q4_K", orc.Q4_K), ("q6_K", orc.Q6_K)])
+@pytest.mark.parametrize("K", [256, 4096])
+def test_get_rows_quantized(dev, name, t, K):
+    """rows of a quantized matrix held in the device layout come back as dequantize_row_* of the original blocks, bit for bit
+    against the oracle's restatement (one product and one difference per element, no sums to reorder)"""
+    import ctypes as C
+    import torch
+    import mi355
+    rng = np.random.default_rng(K + t)
+    n_rows, n_get = 40, 23
+    raw = orc.quantize("oracle", t, (rng.standard_normal((n_rows, K)) * 0.1).astype(np.float32))
+    W = mi355.upload_weights(t, _t(dev, raw))
+    ids = rng.integers(0, n_rows, n_get).astype(np.int32)
+    idd = _t(dev, ids)
+    od = torch.zeros((n_get, K), dtype=torch.float32, device=dev)
+    src = mi355.Tensor()
+    src.data, src.type = W.data_ptr(), t
+    rb = raw.shape[1]
+    for i, (ne, nb) in enumerate(((K, rb // (K // mi355.BLOCK[t][0])), (n_rows, rb), (1, rb * n_rows), (1, rb * n_rows))):
+        src.ne[i], src.nb[i] = ne, nb
+    mi355.check(mi355.load().mi355_get_rows(None, C.byref(src), _d(idd), _d(od)))
+    want = orc.dequantize("oracle", t, raw, K)[ids]
+    got = od.cpu().numpy()
+    if t in (orc.Q4_0, orc.Q8_0, orc.Q6_K):
+        assert np.array_equal(got, want)                      # a single product chain per element
+    else:
+        assert np.max(np.abs(got - want)) <= 1e-6 * np.max(np.abs(want))   # d*sc*n - dmin*m: the compiler may fuse the subtraction
+
+
 @pytest.mark.parametrize("ncols,nrows,masked", [(8, 512, False), (1024, 6, True), (33, 5, True)])
 def test_soft_max(dev, ncols, nrows, masked):
     import torch
