@@ -63,6 +63,119 @@ def cpu_baseline(n_threads, budget_s=20.0):
                       "(3-10 runs each), summed with their per-token multiplicities (32 layers + output); matmuls only"}
 
 
+INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA
+F16_PEAK_TFLOPS = 2500.0     # dense f16 MFMA
+
+
+def sweep(kinds):
+    """Per-kernel roofline tables (one JSON line per case): the matrix products at batch 1 (HBM) and batch 64/512 (int8 MFMA) and
+    FLASH_ATTN_EXT for decode (HBM) and prefill (f16 MFMA) on the Llama-3-8B shapes.  HIP events on the launching stream over
+    operands rotated through more memory than the caches hold.  Not part of the default run."""
+    import math
+    import torch
+    import mi355
+    from mi355 import llama_graph as lg
+    lib = mi355.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    stream = torch.cuda.Stream()
+
+    def timed(fn, n_items, reps):
+        # the n_items calls are recorded once and replayed as a HIP graph, so short kernels are not limited by the host's launch rate
+        with torch.cuda.stream(stream):
+            for i in range(n_items):
+                fn(i)
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for i in range(n_items):
+                    fn(i)
+            g.replay()
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                g.replay()
+            e1.record(stream)
+            stream.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * n_items)
+
+    def emit(**kw):
+        print(json.dumps(kw), flush=True)
+
+    bpe = {mi355.Q4_0: 18 / 32, mi355.Q8_0: 34 / 32, mi355.Q4_K: 144 / 256, mi355.Q6_K: 210 / 256}
+    names = {mi355.Q4_0: "Q4_0", mi355.Q8_0: "Q8_0", mi355.Q4_K: "Q4_K", mi355.Q6_K: "Q6_K"}
+    shapes = [(4096, 4096), (14336, 4096), (4096, 14336)]
+    if "gemv" in kinds:
+        for t in (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q6_K):
+            for N, K in shapes + [(128256, 4096)]:
+                wbytes = int(N * K * bpe[t])
+                nm = max(2, min(32, (1 << 31) // wbytes))
+                Ws = [mi355.upload_weights(t, lg.random_quantized(t, N, K, dev, gen)) for _ in range(nm)]
+                act = mi355.quantize_act(torch.randn(1, K, device=dev, generator=gen))
+                out = torch.empty(1, N, device=dev)
+                us = timed(lambda i: mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, t, Ws[i].data_ptr(), act.data_ptr(), out.data_ptr(), N, K, 1, N)), nm, 4)
+                alg = wbytes + 4 * K + 4 * N
+                emit(kernel="MUL_MAT batch 1 (GEMV)", case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
+                     unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg)
+                del Ws
+    if "mmq" in kinds:
+        for t in (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q6_K):
+            for N, K in shapes:
+                for B in (64, 512):
+                    nm = 4
+                    Ws = [mi355.upload_weights(t, lg.random_quantized(t, N, K, dev, gen)) for _ in range(nm)]
+                    x = torch.randn(B, K, device=dev, generator=gen)
+                    out = torch.empty(B, N, device=dev)
+                    ws = torch.empty(int(lib.mi355_mul_mat_ws_bytes(K, B)) + int(lib.mi355_mul_mat_q8k_ws_bytes(N, K, B)) + 256, dtype=torch.uint8, device=dev)
+                    us = timed(lambda i: mi355.check(lib.mi355_mul_mat(stream.cuda_stream, t, Ws[i].data_ptr(), x.data_ptr(), out.data_ptr(), N, K, B, K, N,
+                                                                       ws.data_ptr(), ws.numel())), nm, 5)
+                    ops = 2.0 * N * K * B
+                    emit(kernel="MUL_MAT batch %d (activation quantization + tile GEMM)" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
+                         achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
+                    if t == mi355.Q6_K and B == 512:   # the same product from the unpacked planes (what prefill uses for Q6_K)
+                        planes = [torch.empty(int(lib.mi355_kq_planes_bytes(N, K)) + 256, dtype=torch.uint8, device=dev) for _ in range(nm)]
+                        for W, P in zip(Ws, planes):
+                            mi355.check(lib.mi355_kq_unpack_planes(None, t, W.data_ptr(), P.data_ptr(), N, K))
+                        a8 = mi355.quantize_act_q8k(x)
+                        us = timed(lambda i: mi355.check(lib.mi355_mul_mat_q8k_planes(stream.cuda_stream, t, planes[i].data_ptr(), a8.data_ptr(), out.data_ptr(), None,
+                                                                                      N, K, B, N)), nm, 5)
+                        emit(kernel="tile GEMM from unpacked planes, batch 512", case="Q6_K %dx%d" % (N, K), us=round(us, 2), bound="mfma",
+                             achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
+                        del planes
+                    del Ws
+    if "fattn" in kinds:
+        H, HK, D = 32, 8, 128
+        for Nq, Nkv in [(1, 512), (1, 4096), (1, 32768), (1, 131072), (512, 512), (512, 4096), (2048, 2048), (4096, 4096)]:
+            nrot = max(2, min(16, (1 << 30) // (Nkv * HK * D * 4))) if Nq == 1 else 1
+            q = torch.randn(Nq, H, D, device=dev, generator=gen)
+            ks = [torch.randn(Nkv, HK, D, device=dev, generator=gen).half() for _ in range(nrot)]
+            vs = [torch.randn(Nkv, HK, D, device=dev, generator=gen).half() for _ in range(nrot)]
+            npad = (Nq + 63) // 64 * 64
+            mask = torch.full((npad, Nkv), float("-inf"), dtype=torch.float16, device=dev)
+            rows = torch.arange(npad, device=dev)[:, None]
+            cols = torch.arange(Nkv, device=dev)[None, :]
+            mask[(cols <= Nkv - Nq + rows) & (rows < Nq)] = 0.0
+            dst = torch.empty(Nq, H, D, device=dev)
+            ws = torch.empty(min(int(lib.mi355_flash_attn_ws_bytes(D, Nq, Nkv, H)), 1 << 28), dtype=torch.uint8, device=dev)
+
+            def fa(i):
+                mi355.check(lib.mi355_flash_attn_ext(stream.cuda_stream, q.data_ptr(), ks[i].data_ptr(), vs[i].data_ptr(), mask.data_ptr(), dst.data_ptr(), D, Nq, Nkv, H,
+                                                     HK, H * D * 4, D * 4, HK * D * 2, D * 2, HK * D * 2, D * 2, Nkv * 2, 1 / math.sqrt(D), 0.0, 0.0, ws.data_ptr(),
+                                                     ws.numel()))
+            us = timed(fa, nrot, 4 if Nq == 1 else 10)
+            if Nq == 1:
+                alg = 4 * HK * D * Nkv + 2 * Nkv + 4 * H * D * 2
+                emit(kernel="FLASH_ATTN_EXT decode (all launches of one call)", case="Nkv %d" % Nkv, us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
+                     unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg)
+            else:
+                fl = 4.0 * H * Nq * D * Nkv
+                emit(kernel="FLASH_ATTN_EXT prefill, causal mask (nominal flops, masked cells included)", case="Nq %d Nkv %d" % (Nq, Nkv), us=round(us, 2), bound="mfma",
+                     achieved=round(fl / us / 1e6, 1), unit="TFLOP/s", frac=round(fl / us / 1e6 / F16_PEAK_TFLOPS, 4), flops=fl)
+            del ks, vs
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -71,7 +184,13 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
+    ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, fattn")
     args = ap.parse_args()
+    if args.sweep:
+        if args.gpus != 1:
+            sys.exit("bench.py: one GPU only")
+        sweep([k.strip() for k in args.sweep.split(",") if k.strip()])
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not available" % args.gpus,
               file=sys.stderr)

@@ -106,6 +106,16 @@ int mi355_mul_mat_q8k(void *stream, int type, const void *W, const void *act, fl
 int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
                           int64_t B, int64_t dst_stride);
 
+/* The same product with a workspace for the split along K: a launch with few tiles (N/64 x B/128 < 384, e.g. any matrix at batch
+ * 64 or the 1024-row wk/wv at batch 512) is cut into up to 8 slices of >= 4 super-blocks that run side by side, their partial
+ * sums land in ws and a second launch adds them in fixed order (plus the residual).  ws: mi355_mul_mat_q8k_ws_bytes(N, K, B) bytes,
+ * 16-byte aligned (0 = this shape is not split); with less, or NULL, the product runs unsplit (then bit-identical to
+ * mi355_mul_mat_q8k_add, otherwise equal up to f32 summation order).  mi355_mul_mat uses whatever its own workspace holds beyond
+ * mi355_mul_mat_ws_bytes(K, B) for this.  No counterpart in the reference (its CPU path splits rows over threads). */
+size_t mi355_mul_mat_q8k_ws_bytes(int64_t N, int64_t K, int64_t B);
+int mi355_mul_mat_q8k_ws(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
+                         int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
+
 /* Second, unpacked copy of K-quant weights for the tile GEMM: the two int8 planes whose weighted sum R*hi + lo is the integer
  * sub-scale times the level (sc*n for Q4_K with R = 8, sc*(l-32) for Q6_K with R = 64; dequantize_row_q4_K / _q6_K,
  * ggml/src/ggml-quants.c:1280-1302, 1690-1719), 2 bytes per weight: int8 hi[rows][K], int8 lo[rows][K], then 48 bytes per
@@ -120,6 +130,9 @@ size_t mi355_kq_planes_bytes(int64_t rows, int64_t K);
 int mi355_kq_unpack_planes(void *stream, int type, const void *W, void *planes, int64_t rows, int64_t K);
 int mi355_mul_mat_q8k_planes(void *stream, int type, const void *planes, const void *act, float *dst, const float *residual, int64_t N,
                              int64_t K, int64_t B, int64_t dst_stride);
+/* ... with the split-along-K workspace of mi355_mul_mat_q8k_ws (same slices, so still bit-identical to it) */
+int mi355_mul_mat_q8k_planes_ws(void *stream, int type, const void *planes, const void *act, float *dst, const float *residual, int64_t N,
+                                int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
 
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE

@@ -1304,29 +1304,25 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         }
         const void * pl = planes().get(s, node->src[0]);   // Q6_K weights: the unpacked planes, built on first use
         const int wtype = to_mi355_type(node->src[0]->type);
+        const int64_t N = node->src[0]->ne[1];
+        // products with few tiles are split along K through the scratch buffer (0 bytes: this shape is not split)
+        const size_t split_bytes = mi355_mul_mat_q8k_ws_bytes(N, K, B);
+        void * split_ws = split_bytes ? ctx->workspace(split_bytes) : nullptr;
+        auto product = [&](float * out, const float * residual, int64_t out_stride) {
+            if (pl) MI355_K_OK(mi355_mul_mat_q8k_planes_ws(s, wtype, pl, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
+            else MI355_K_OK(mi355_mul_mat_q8k_ws(s, wtype, node->src[0]->data, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
+        };
         // MUL_MAT -> ADD(residual): the sum goes straight into the ADD's tensor
         ggml_tensor * add = nxt;
         if (add && add->op == GGML_OP_ADD && w.sole_use(i) && (add->src[0] == node || add->src[1] == node)) {
             const ggml_tensor * res = add->src[0] == node ? add->src[1] : add->src[0];
             if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, node) && ggml_is_contiguous(res) && ggml_is_contiguous(add) && ggml_is_contiguous(node)) {
-                if (pl) {
-                    MI355_K_OK(mi355_mul_mat_q8k_planes(s, wtype, pl, ctx->cache.ptr, (float *) add->data, (const float *) res->data, node->src[0]->ne[1],
-                                                        K, B, (int64_t) (add->nb[1] / sizeof(float))));
-                } else {
-                    MI355_K_OK(mi355_mul_mat_q8k_add(s, wtype, node->src[0]->data, ctx->cache.ptr, (float *) add->data, (const float *) res->data,
-                                                     node->src[0]->ne[1], K, B, (int64_t) (add->nb[1] / sizeof(float))));
-                }
+                product((float *) add->data, (const float *) res->data, (int64_t) (add->nb[1] / sizeof(float)));
                 ctx->note_write(add->data, ggml_nbytes(add));
                 return j;
             }
         }
-        if (pl) {
-            MI355_K_OK(mi355_mul_mat_q8k_planes(s, wtype, pl, ctx->cache.ptr, (float *) node->data, nullptr, node->src[0]->ne[1], K, B,
-                                                (int64_t) (node->nb[1] / sizeof(float))));
-        } else {
-            MI355_K_OK(mi355_mul_mat_q8k(s, wtype, node->src[0]->data, ctx->cache.ptr, (float *) node->data, node->src[0]->ne[1], K, B,
-                                         (int64_t) (node->nb[1] / sizeof(float))));
-        }
+        product((float *) node->data, nullptr, (int64_t) (node->nb[1] / sizeof(float)));
         ctx->note_write(node->data, ggml_nbytes(node));
         return i;
     }

@@ -512,6 +512,13 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
     const int wrow0 = (wave & 1) * 32;    // weight rows of this wave inside the tile
     const int wcol0 = (wave >> 1) * 64;   // activation rows of this wave inside the tile
     const int64_t nsb = K >> 8;
+    // split K: group y of gridDim.y walks super-blocks [sb_lo, sb_hi) and writes its sums to its own slice of `dst` (see launch)
+    const int64_t sb_per = (nsb + gridDim.y - 1) / gridDim.y;
+    const int64_t sb_lo = (int64_t)blockIdx.y * sb_per, sb_hi = sb_lo + sb_per < nsb ? sb_lo + sb_per : nsb;
+    if (gridDim.y > 1) {
+        dst += (int64_t)blockIdx.y * B * dst_stride;
+        residual = nullptr;
+    }
 
     // this thread's weight row, the activation rows of its four transfers, and the column whose scales it copies
     const int64_t wr = row0 + (tid >> 2) < N ? row0 + (tid >> 2) : N - 1;
@@ -571,11 +578,11 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
     float d8n = 0.0f;
     u32x4 bsn = {0, 0, 0, 0};
     // prologue: stage 0 into the "a" buffers, pieces of stage 1 in flight
-    kp_fetch_w<TYPE>(R0, wrow, L, 0, 0);
-    kp_fetch_w<TYPE>(R1, wrow, L, 0, 1);
-    kp_fetch_h<TYPE>(Hc, wrow, L, 0);
-    kp_dma_a<4>(aq, aofs, sAa);
-    fetch_scales(0, d8n, bsn);
+    kp_fetch_w<TYPE>(R0, wrow, L, sb_lo, 0);
+    kp_fetch_w<TYPE>(R1, wrow, L, sb_lo, 1);
+    kp_fetch_h<TYPE>(Hc, wrow, L, sb_lo);
+    kp_dma_a<4>(aq + sb_lo * QKK, aofs, sAa);
+    fetch_scales(sb_lo, d8n, bsn);
     {
         kp_planes P;
 #pragma unroll
@@ -586,7 +593,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
     Hn = Hc;
     __syncthreads();
 
-    for (int64_t sb = 0; sb < nsb; sb++) {
+    for (int64_t sb = sb_lo; sb < sb_hi; sb++) {
         i32x16 hi[2], lo[2];
 #pragma unroll
         for (int half = 0; half < 2; half++) {
@@ -600,7 +607,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
             kp_w<TYPE> &Rf = half == 0 ? R0 : R1;    // held this stage's piece (unpacked one stage ago): refilled for the stage after next
             // Past the end of K the same work is done on the last super-block again and never read: no branches in the stage,
             // so the compiler schedules it as one block.
-            const int64_t sb1 = sb + 1 < nsb ? sb + 1 : sb;
+            const int64_t sb1 = sb + 1 < sb_hi ? sb + 1 : sb;
             kp_dma_a<4>(aq + (half == 0 ? sb * QKK + 128 : sb1 * QKK), aofs, nA);
             if (half == 1) fetch_scales(sb1, d8n, bsn);
             kp_fetch_w<TYPE>(Rf, wrow, L, sb1, half);
@@ -638,7 +645,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
             kp_store<TYPE>(P, nW1, nW0);
 
             if (half == 1) {   // end of the super-block: scale the integer sums into the f32 accumulators
-                const int sbuf = (int)(sb & 1);
+                const int sbuf = (int)((sb - sb_lo) & 1);
 #pragma unroll
                 for (int tb = 0; tb < 2; tb++) {
                     f32x4 d8[4];
@@ -670,7 +677,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
             }
             if (half == 1) {   // last, so that the loads had the whole stage (the barrier keeps the scheduler from hoisting the wait)
                 __builtin_amdgcn_sched_barrier(0);
-                store_scales((int)((sb + 1) & 1), d8n, bsn, Hn);
+                store_scales((int)((sb - sb_lo + 1) & 1), d8n, bsn, Hn);
                 Hc = Hn;
             }
             __syncthreads();   // also waits for this stage's transfers and loads (issued a whole stage ago)
@@ -835,6 +842,13 @@ __global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ pl
     const int wrow0 = (wave & 1) * 32;    // weight rows of this wave inside the tile
     const int wcol0 = (wave >> 1) * 64;   // activation rows of this wave inside the tile
     const int64_t nsb = K >> 8;
+    // split K: group y of gridDim.y walks super-blocks [sb_lo, sb_hi) and writes its sums to its own slice of `dst` (see launch)
+    const int64_t sb_per = (nsb + gridDim.y - 1) / gridDim.y;
+    const int64_t sb_lo = (int64_t)blockIdx.y * sb_per, sb_hi = sb_lo + sb_per < nsb ? sb_lo + sb_per : nsb;
+    if (gridDim.y > 1) {
+        dst += (int64_t)blockIdx.y * B * dst_stride;
+        residual = nullptr;
+    }
 
     // this thread's weight row, the activation rows of its four transfers, and the column whose scales it copies
     const int64_t wr = row0 + (tid >> 2) < N ? row0 + (tid >> 2) : N - 1;
@@ -901,15 +915,15 @@ __global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ pl
         kp_dma_a<2>(plane0 + k0, pofs, s0);
     };
     // prologue: stage 0 into the "a" buffers
-    pl_fetch_h<TYPE>(Hc, aux_row, 0);
-    kp_dma_a<4>(aq, aofs, sAa);
-    dma_w(0, sW1a, sW0a);
-    fetch_scales(0, d8n, bsn);
+    pl_fetch_h<TYPE>(Hc, aux_row, sb_lo);
+    kp_dma_a<4>(aq + sb_lo * QKK, aofs, sAa);
+    dma_w(sb_lo * QKK, sW1a, sW0a);
+    fetch_scales(sb_lo, d8n, bsn);
     store_scales(0, d8n, bsn, Hc);
     Hn = Hc;
     __syncthreads();
 
-    for (int64_t sb = 0; sb < nsb; sb++) {
+    for (int64_t sb = sb_lo; sb < sb_hi; sb++) {
         i32x16 hi[2], lo[2];
 #pragma unroll
         for (int half = 0; half < 2; half++) {
@@ -920,7 +934,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ pl
             int8_t *nW1 = half == 0 ? sW1b : sW1a;
             int8_t *nW0 = half == 0 ? sW0b : sW0a;
             // Past the end of K the same work is done on the last super-block again and never read: no branches in the stage.
-            const int64_t sb1 = sb + 1 < nsb ? sb + 1 : sb;
+            const int64_t sb1 = sb + 1 < sb_hi ? sb + 1 : sb;
             const int64_t k1 = half == 0 ? sb * QKK + 128 : sb1 * QKK;   // the next stage
             kp_dma_a<4>(aq + k1, aofs, nA);
             dma_w(k1, nW1, nW0);
@@ -957,7 +971,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ pl
             }
 
             if (half == 1) {   // end of the super-block: scale the integer sums into the f32 accumulators
-                const int sbuf = (int)(sb & 1);
+                const int sbuf = (int)((sb - sb_lo) & 1);
 #pragma unroll
                 for (int tb = 0; tb < 2; tb++) {
                     f32x4 d8[4];
@@ -989,7 +1003,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ pl
             }
             if (half == 1) {   // last, so that the loads had the whole stage (the barrier keeps the scheduler from hoisting the wait)
                 __builtin_amdgcn_sched_barrier(0);
-                store_scales((int)((sb + 1) & 1), d8n, bsn, Hn);
+                store_scales((int)((sb - sb_lo + 1) & 1), d8n, bsn, Hn);
                 Hc = Hn;
             }
             __syncthreads();   // also waits for this stage's transfers and loads (issued a whole stage ago)
@@ -1010,9 +1024,57 @@ __global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ pl
     }
 }
 
+// ---- split K --------------------------------------------------------------------------------------------------------
+// A product with few tiles (wk / wv of a 512-token batch: 64; any matrix at batch 64: N / 64) leaves most of the chip idle
+// while each group walks all of K, one dependent stage after the other.  Such launches are cut along K: grid row y takes a
+// contiguous range of super-blocks and writes its sums to slice y of a workspace, and k_split_sum adds the slices in fixed
+// order (plus the residual).  The same rule serves the kernel that unpacks and the one that reads planes, so they still
+// agree bit for bit.  At least two super-blocks per slice, at most eight slices, at most two groups per compute unit.
+static int split_k_slices(int64_t N, int64_t K, int64_t B) {
+    const int64_t groups = ((N + 63) / 64) * ((B + 127) / 128), nsb = K / QKK;
+    if (groups >= 384) return 1;
+    int64_t n = 512 / groups;
+    if (n > nsb / 2) n = nsb / 2;
+    if (n > 8) n = 8;
+    if (n < 2) return 1;
+    const int64_t per = (nsb + n - 1) / n;
+    return (int)((nsb + per - 1) / per);   // no empty slice
+}
+
+__global__ void __launch_bounds__(256) k_split_sum(const float *__restrict__ part, float *__restrict__ dst, const float *__restrict__ residual,
+                                                   int64_t N, int64_t B, int64_t dst_stride, int n_slices) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;   // N % 4 == 0 here
+    if (i >= N * B) return;
+    const int64_t b = i / N, n = i % N;
+    f32x4 acc = *(const f32x4 *)(part + i);
+    for (int sl = 1; sl < n_slices; sl++) {
+        const f32x4 v = *(const f32x4 *)(part + (int64_t)sl * N * B + i);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = add_rn(acc[j], v[j]);
+    }
+    const int64_t o = b * dst_stride + n;
+    if (residual) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = add_rn(acc[j], residual[o + j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) dst[o + j] = acc[j];
+}
+
+// slices for this product given the workspace at hand (1 = no split)
+static int usable_slices(int64_t N, int64_t K, int64_t B, const void *ws, size_t ws_bytes) {
+    const int n = split_k_slices(N, K, B);
+    if (n < 2 || ws == nullptr || ((uintptr_t)ws & 15) != 0 || N % 4 != 0) return 1;
+    return ws_bytes >= (size_t)n * (size_t)N * (size_t)B * sizeof(float) ? n : 1;
+}
+
+static void launch_split_sum(hipStream_t s, const float *part, float *dst, const float *residual, int64_t N, int64_t B, int64_t dst_stride, int n) {
+    hipLaunchKernelGGL(k_split_sum, dim3((unsigned)((N * B / 4 + 255) / 256)), dim3(256), 0, s, part, dst, residual, N, B, dst_stride, n);
+}
+
 template <int TYPE>
 static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
-                         int64_t dst_stride) {
+                         int64_t dst_stride, void *ws, size_t ws_bytes) {
     constexpr int BM = 64, BN = 128;
     const row_layout L = make_row_layout(TYPE, K);
     const int8_t *aq = (const int8_t *)act;
@@ -1022,6 +1084,13 @@ static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *d
     const int n_col_tiles = (int)((B + BN - 1) / BN);
     const int n_groups = n_row_tiles * n_col_tiles;
     const int n_groups_padded = (n_groups + 7) & ~7;
+    const int n_slices = usable_slices(N, K, B, ws, ws_bytes);
+    if (n_slices > 1) {
+        hipLaunchKernelGGL((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded, (unsigned)n_slices), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_,
+                           (float *)ws, nullptr, N, K, B, N, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
+        launch_split_sum(s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
+        return;
+    }
     hipLaunchKernelGGL((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_, dst, residual, N, K,
                        B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
 }
@@ -1173,8 +1242,19 @@ int mi355_kq_unpack_planes(void *stream, int type, const void *W, void *planes, 
     return launch_status("k_unpack_planes");
 }
 
+size_t mi355_mul_mat_q8k_ws_bytes(int64_t N, int64_t K, int64_t B) {
+    if (N <= 0 || K <= 0 || B <= 0 || K % QKK != 0) return 0;
+    const int n = split_k_slices(N, K, B);
+    return n > 1 && N % 4 == 0 ? (size_t)n * (size_t)N * (size_t)B * sizeof(float) : 0;
+}
+
 int mi355_mul_mat_q8k_planes(void *stream, int type, const void *planes, const void *act, float *dst, const float *residual, int64_t N,
                              int64_t K, int64_t B, int64_t dst_stride) {
+    return mi355_mul_mat_q8k_planes_ws(stream, type, planes, act, dst, residual, N, K, B, dst_stride, nullptr, 0);
+}
+
+int mi355_mul_mat_q8k_planes_ws(void *stream, int type, const void *planes, const void *act, float *dst, const float *residual, int64_t N,
+                                int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
     MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k_planes: weight type %d is not a K-quant", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k_planes: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k_planes: K=%lld is not a multiple of 256", (long long)K);
@@ -1191,17 +1271,28 @@ int mi355_mul_mat_q8k_planes(void *stream, int type, const void *planes, const v
     const int n_row_tiles = (int)((N + 63) / 64), n_col_tiles = (int)((B + 127) / 128);
     const int n_groups = n_row_tiles * n_col_tiles, n_groups_padded = (n_groups + 7) & ~7;
     hipStream_t s = (hipStream_t)stream;
+    const int n_slices = usable_slices(N, K, B, ws, ws_bytes);
+    const dim3 grid((unsigned)n_groups_padded, (unsigned)n_slices);
+    float *out = n_slices > 1 ? (float *)ws : dst;
+    const float *res = n_slices > 1 ? nullptr : residual;
+    const int64_t out_stride = n_slices > 1 ? N : dst_stride;
     if (type == MI355_Q4_K)
-        hipLaunchKernelGGL((k_mmq_pl<MI355_Q4_K, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, dst,
-                           residual, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
+        hipLaunchKernelGGL((k_mmq_pl<MI355_Q4_K, false>), grid, dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, out, res, N, K, B, out_stride, L,
+                           n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
     else
-        hipLaunchKernelGGL((k_mmq_pl<MI355_Q6_K, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, dst,
-                           residual, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
+        hipLaunchKernelGGL((k_mmq_pl<MI355_Q6_K, false>), grid, dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, out, res, N, K, B, out_stride, L,
+                           n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
+    if (n_slices > 1) launch_split_sum(s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
     return launch_status("k_mmq_pl");
 }
 
 int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
                           int64_t B, int64_t dst_stride) {
+    return mi355_mul_mat_q8k_ws(stream, type, W, act, dst, residual, N, K, B, dst_stride, nullptr, 0);
+}
+
+int mi355_mul_mat_q8k_ws(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
+                         int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
     MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k: weight type %d is not a K-quant", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k: K=%lld is not a multiple of 256", (long long)K);
@@ -1212,8 +1303,8 @@ int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act
                   "mul_mat_q8k: activation workspace is not 16-byte aligned");
     MI355_REQUIRE((N + 63) / 64 * ((B + 63) / 64) < (1 << 30), "mul_mat_q8k: too many tiles");
     hipStream_t s = (hipStream_t)stream;
-    if (type == MI355_Q4_K) launch_mmq_k<MI355_Q4_K>(s, W, act, dst, residual, N, K, B, dst_stride);
-    else launch_mmq_k<MI355_Q6_K>(s, W, act, dst, residual, N, K, B, dst_stride);
+    if (type == MI355_Q4_K) launch_mmq_k<MI355_Q4_K>(s, W, act, dst, residual, N, K, B, dst_stride, ws, ws_bytes);
+    else launch_mmq_k<MI355_Q6_K>(s, W, act, dst, residual, N, K, B, dst_stride, ws, ws_bytes);
     return launch_status("k_mmq_k");
 }
 

@@ -68,7 +68,9 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
     if (use_q8k_tiles(type, W, K, B)) {
         int rc = mi355_quantize_act_q8k(stream, x, ws, K, B, x_stride);
         if (rc != MI355_OK) return rc;
-        return mi355_mul_mat_q8k(stream, type, W, ws, dst, N, K, B, dst_stride);
+        // what the workspace holds beyond the quantized activation serves the split along K of products with few tiles
+        const size_t used = mi355_mul_mat_ws_bytes(K, B);
+        return mi355_mul_mat_q8k_ws(stream, type, W, ws, dst, nullptr, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
     }
     int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
     if (rc != MI355_OK) return rc;

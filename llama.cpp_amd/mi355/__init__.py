@@ -46,6 +46,9 @@ _SIGNATURES = {
     "mi355_kq_planes_bytes": (_sz, [_i64, _i64]),
     "mi355_kq_unpack_planes": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_mul_mat_q8k_planes": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_mul_mat_q8k_planes_ws": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_q8k_ws_bytes": (_sz, [_i64, _i64, _i64]),
+    "mi355_mul_mat_q8k_ws": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_q8k_add": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_rms_norm_mul_quant": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),

@@ -99,6 +99,7 @@ class LlamaRunner:
         self.fuse_qkv = True    # rows must be 16-byte aligned; set False to use the three-launch sequence
         self.use_planes = True  # prefill: Q6_K matrices go through their unpacked int8 planes (2 bytes per weight more, kept resident)
         self.planes = {}
+        self.split_ws = None    # partial sums of tile products that are split along K (grown on first use, before any graph capture)
         # decode, T <= 4: SiLU*up + Q8_1 either by the last group of each 32-row block of the gate/up launch (True) or as a launch
         # of their own after a two-matrix product (False).  With the activation staged in LDS the two-launch form is the quicker
         # one (15.9 us against 16.3-16.8 us per layer on the 8B shape); both give the same bits.
@@ -203,13 +204,18 @@ class LlamaRunner:
             check(self.lib.mi355_mul_mat_vec_q_multi(_stream(), len(mats), arr, _ptr(act), K, T))
         else:
             for (t, W), out in mats:
-                if q8k and t == Q6_K and self.use_planes:   # Q6_K streams its int8 planes, unpacked once per matrix
-                    check(self.lib.mi355_mul_mat_q8k_planes(_stream(), t, _ptr(self._planes(t, W, out.shape[1], K)), _ptr(act), _ptr(out),
-                                                            _ptr(residual) if residual is not None else None, out.shape[1], K, T, out.stride(0)))
-                    continue
-                if q8k:     # the residual add is the tile kernel's epilogue
-                    check(self.lib.mi355_mul_mat_q8k_add(_stream(), t, _ptr(W), _ptr(act), _ptr(out), _ptr(residual) if residual is not None else None,
-                                                         out.shape[1], K, T, out.stride(0)))
+                if q8k:     # the residual add is the tile kernel's epilogue; products with few tiles are split along K through split_ws
+                    N = out.shape[1]
+                    need = int(self.lib.mi355_mul_mat_q8k_ws_bytes(N, K, T))
+                    if self.split_ws is None or self.split_ws.numel() < need:
+                        self.split_ws = torch.empty(need + 256, dtype=torch.uint8, device=self.dev)
+                    sw, sn = (_ptr(self.split_ws), self.split_ws.numel()) if need else (None, 0)
+                    res = _ptr(residual) if residual is not None else None
+                    if t == Q6_K and self.use_planes:   # Q6_K streams its int8 planes, unpacked once per matrix
+                        check(self.lib.mi355_mul_mat_q8k_planes_ws(_stream(), t, _ptr(self._planes(t, W, N, K)), _ptr(act), _ptr(out), res, N, K, T,
+                                                                   out.stride(0), sw, sn))
+                    else:
+                        check(self.lib.mi355_mul_mat_q8k_ws(_stream(), t, _ptr(W), _ptr(act), _ptr(out), res, N, K, T, out.stride(0), sw, sn))
                     continue
                 dst = out if residual is None else self.t1[:T]
                 check(self.lib.mi355_mul_mat_q(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), out.shape[1], K, T, dst.stride(0)))

@@ -363,6 +363,9 @@ def test_tile_gemm_from_planes_equals_packed(dev, name, t, N, K, B):
     act = mi355.quantize_act_q8k(x)
     planes = torch.empty(int(lib.mi355_kq_planes_bytes(N, K)) + 256, dtype=torch.uint8, device=dev)
     mi355.check(lib.mi355_kq_unpack_planes(None, t, mi355._ptr(W), mi355._ptr(planes), N, K))
+    need = int(lib.mi355_mul_mat_q8k_ws_bytes(N, K, B))
+    assert need > 0                                        # these shapes have few tiles: with a workspace they are split along K
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
     for residual in (None, res):
         want = torch.zeros(B, N + 8, device=dev)
         got = torch.zeros(B, N + 8, device=dev)
@@ -371,3 +374,16 @@ def test_tile_gemm_from_planes_equals_packed(dev, name, t, N, K, B):
         mi355.check(lib.mi355_mul_mat_q8k_planes(None, t, mi355._ptr(planes), mi355._ptr(act), mi355._ptr(got), r, N, K, B, N + 8))
         assert torch.equal(got, want)
         assert got[:, N:].abs().max().item() == 0.0      # nothing written past the row
+        # split along K: both kernels cut the same slices, so they still agree bit for bit; against the unsplit product only the
+        # order of the f32 sums differs
+        want_s = torch.zeros(B, N + 8, device=dev)
+        got_s = torch.zeros(B, N + 8, device=dev)
+        mi355.check(lib.mi355_mul_mat_q8k_ws(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(want_s), r, N, K, B, N + 8, mi355._ptr(ws), need))
+        mi355.check(lib.mi355_mul_mat_q8k_planes_ws(None, t, mi355._ptr(planes), mi355._ptr(act), mi355._ptr(got_s), r, N, K, B, N + 8, mi355._ptr(ws), need))
+        assert torch.equal(got_s, want_s)
+        assert got_s[:, N:].abs().max().item() == 0.0
+        assert orc.nmse(want_s[:, :N].cpu().numpy(), want[:, :N].cpu().numpy()) < 1e-12
+        # too small a workspace: the product runs unsplit
+        again = torch.zeros(B, N + 8, device=dev)
+        mi355.check(lib.mi355_mul_mat_q8k_ws(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(again), r, N, K, B, N + 8, mi355._ptr(ws), need - 16))
+        assert torch.equal(again, want)
