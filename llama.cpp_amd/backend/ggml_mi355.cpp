@@ -899,26 +899,43 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             return j;
         }
     }
-    // ---- UNARY(SILU) -> MUL
-    if (node->op == GGML_OP_UNARY && ggml_get_unary_op(node) == GGML_UNARY_OP_SILU && nxt && nxt->op == GGML_OP_MUL && w.sole_use(i) &&
-        (nxt->src[0] == node || nxt->src[1] == node)) {
-        const ggml_tensor * gt = node->src[0];
-        const ggml_tensor * up = nxt->src[0] == node ? nxt->src[1] : nxt->src[0];
-        const int64_t K = gt->ne[0], rows = ggml_nrows(gt);
-        if (ggml_is_contiguous(gt) && ggml_is_contiguous(up) && ggml_is_contiguous(nxt) && ggml_are_same_shape(gt, up) && up->type == GGML_TYPE_F32 &&
-            K % 32 == 0 && rows <= 65535 && (((uintptr_t) gt->data | (uintptr_t) up->data | (uintptr_t) nxt->data) & 15) == 0) {
-            void * act = nullptr;
-            if (rows > 8 && feeds_q8k_tiles(w, j, nxt->data, K, rows)) {
-                act = ctx->act_slot(mi355_act_q8k_bytes(K, rows));
-                MI355_K_OK(mi355_swiglu_quant_q8k(s, (const float *) gt->data, (const float *) up->data, K, (float *) nxt->data, K, act, K, rows));
-                ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8K, true, act};
-                return j;
+    // ---- UNARY(SILU) -> MUL, also across the product that supplies the other factor: llm_build_ffn's graph lists
+    //      MUL_MAT(gate), SILU, MUL_MAT(up), MUL; the up product does not read SILU's value, so it runs first and SiLU*up
+    //      (+ the quantized form ffn_down reads) is one launch after it
+    if (node->op == GGML_OP_UNARY && ggml_get_unary_op(node) == GGML_UNARY_OP_SILU && nxt && w.sole_use(i)) {
+        int jm = -1;   // index of the MUL
+        if (nxt->op == GGML_OP_MUL && (nxt->src[0] == node || nxt->src[1] == node)) {
+            jm = j;
+        } else if (nxt->op == GGML_OP_MUL_MAT && nxt->src[0] != node && nxt->src[1] != node) {
+            const int j2 = w.next(j);
+            const ggml_tensor * m = j2 < w.n ? w.nodes[j2] : nullptr;
+            if (m && m->op == GGML_OP_MUL && ((m->src[0] == node && m->src[1] == nxt) || (m->src[1] == node && m->src[0] == nxt))) jm = j2;
+        }
+        if (jm >= 0) {
+            ggml_tensor * mul = (ggml_tensor *) w.nodes[jm];
+            const ggml_tensor * gt = node->src[0];
+            const ggml_tensor * up = mul->src[0] == node ? mul->src[1] : mul->src[0];
+            const int64_t K = gt->ne[0], rows = ggml_nrows(gt);
+            if (ggml_is_contiguous(gt) && ggml_is_contiguous(up) && ggml_is_contiguous(mul) && ggml_are_same_shape(gt, up) && up->type == GGML_TYPE_F32 &&
+                gt->type == GGML_TYPE_F32 && mul->type == GGML_TYPE_F32 && K % 32 == 0 && rows <= 65535 &&
+                (((uintptr_t) gt->data | (uintptr_t) up->data | (uintptr_t) mul->data) & 15) == 0) {
+                if (jm != j) {   // the product first (it may use the activation cached for the gate product)
+                    const int done = compute_fused(ctx, w, j);
+                    GGML_ASSERT(done == j);   // a MUL_MAT followed by MUL takes nothing with it
+                }
+                void * act = nullptr;
+                if (rows > 8 && feeds_q8k_tiles(w, jm, mul->data, K, rows)) {
+                    act = ctx->act_slot(mi355_act_q8k_bytes(K, rows));
+                    MI355_K_OK(mi355_swiglu_quant_q8k(s, (const float *) gt->data, (const float *) up->data, K, (float *) mul->data, K, act, K, rows));
+                    ctx->cache = act_cache{mul->data, K, rows, ACT_Q8K, true, act};
+                    return jm;
+                }
+                if (rows <= 8 && (feeds_quant_gemv(w, jm, mul->data, K, rows) || feeds_quant_mmid(w, jm, mul->data, K, rows)))
+                    act = ctx->act_slot(mi355_act_bytes(K, rows));
+                MI355_K_OK(mi355_swiglu_quant(s, (const float *) gt->data, (const float *) up->data, K, (float *) mul->data, K, act, K, rows));
+                ctx->cache = act_cache{mul->data, K, rows, ACT_Q8_1, act != nullptr, act};
+                return jm;
             }
-            if (rows <= 8 && (feeds_quant_gemv(w, j, nxt->data, K, rows) || feeds_quant_mmid(w, j, nxt->data, K, rows)))
-                act = ctx->act_slot(mi355_act_bytes(K, rows));
-            MI355_K_OK(mi355_swiglu_quant(s, (const float *) gt->data, (const float *) up->data, K, (float *) nxt->data, K, act, K, rows));
-            ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
-            return j;
         }
     }
     // ---- MUL_MAT_ID: the quantized rows of src1 are shared by consecutive products (up and gate experts read the same rows)

@@ -1033,6 +1033,7 @@ __global__ void __launch_bounds__(256, 2) k_mmq_pl(const int8_t *__restrict__ pl
 static int split_k_slices(int64_t N, int64_t K, int64_t B) {
     const int64_t groups = ((N + 63) / 64) * ((B + 127) / 128), nsb = K / QKK;
     if (groups >= 384) return 1;
+    if (groups >= 192 && nsb < 32) return 1;   // about a group per compute unit already: the extra pass over the sums pays only for a long K
     int64_t n = 512 / groups;
     if (n > nsb / 2) n = nsb / 2;
     if (n > 8) n = 8;

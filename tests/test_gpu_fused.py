@@ -349,7 +349,7 @@ def test_unpacked_planes_hold_the_integer_levels(dev, name, t, R):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name,t", [("q4_K", orc.Q4_K), ("q6_K", orc.Q6_K)])
-@pytest.mark.parametrize("N,K,B", [(320, 2048, 70), (1024, 4096, 512), (4096, 2048, 9), (136, 6144, 130)])
+@pytest.mark.parametrize("N,K,B", [(320, 2048, 70), (1024, 4096, 512), (4096, 2048, 9), (136, 6144, 130), (4096, 8192, 500)])
 def test_tile_gemm_from_planes_equals_packed(dev, name, t, N, K, B):
     """the tile GEMM that streams unpacked planes gives the bits of the one that unpacks in the kernel, residual and strided dst included"""
     import torch
