@@ -128,7 +128,8 @@ def sweep(kinds):
                     Ws = [mi355.upload_weights(t, lg.random_quantized(t, N, K, dev, gen)) for _ in range(nm)]
                     x = torch.randn(B, K, device=dev, generator=gen)
                     out = torch.empty(B, N, device=dev)
-                    ws = torch.empty(int(lib.mi355_mul_mat_ws_bytes(K, B)) + int(lib.mi355_mul_mat_q8k_ws_bytes(N, K, B)) + 256, dtype=torch.uint8, device=dev)
+                    ws = torch.empty(int(lib.mi355_mul_mat_ws_bytes(K, B)) + max(int(lib.mi355_mul_mat_q8k_ws_bytes(N, K, B)), int(lib.mi355_mul_mat_q_ws_bytes(N, K, B))) + 256,
+                                     dtype=torch.uint8, device=dev)
                     us = timed(lambda i: mi355.check(lib.mi355_mul_mat(stream.cuda_stream, t, Ws[i].data_ptr(), x.data_ptr(), out.data_ptr(), N, K, B, K, N,
                                                                        ws.data_ptr(), ws.numel())), nm, 5)
                     ops = 2.0 * N * K * B

@@ -88,6 +88,11 @@ int mi355_mul_mat_vec_q(void *stream, int type, const void *W, const void *act, 
                         int64_t B, int64_t dst_stride);
 int mi355_mul_mat_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
                     int64_t dst_stride);
+/* The same with a workspace for the split along K of products with few tiles (as mi355_mul_mat_q8k_ws): ws of
+ * mi355_mul_mat_q_ws_bytes(N, K, B) bytes, 16-byte aligned; with less, or NULL, the product runs unsplit. */
+size_t mi355_mul_mat_q_ws_bytes(int64_t N, int64_t K, int64_t B);
+int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
+                       int64_t dst_stride, void *ws, size_t ws_bytes);
 
 /* K-quant (Q4_K, Q6_K) tile GEMM with the activation format ggml-cpu uses for these weight
  * types: one f32 scale per 256 elements (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516;

@@ -580,7 +580,9 @@ void compute_mul_mat(backend_ctx * ctx, ggml_tensor * dst) {
     }
     const int64_t K = a->ne[0], N = a->ne[1], B = b->ne[1];
     const int64_t r2 = b->ne[2] / a->ne[2], r3 = b->ne[3] / a->ne[3];
-    const size_t ws_bytes = mi355_mul_mat_ws_bytes(K, B);
+    // the quantized activation, and behind it room for the slices of a product that is split along K
+    const size_t split_q = mi355_mul_mat_q_ws_bytes(N, K, B), split_k = mi355_mul_mat_q8k_ws_bytes(N, K, B);
+    const size_t ws_bytes = mi355_mul_mat_ws_bytes(K, B) + (split_q > split_k ? split_q : split_k);
     void * ws = ctx->workspace(ws_bytes);
     for (int64_t i3 = 0; i3 < b->ne[3]; i3++) {
         for (int64_t i2 = 0; i2 < b->ne[2]; i2++) {

@@ -209,7 +209,13 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[tb][tw][r] = 0.0f;
 
-    for (int64_t k0 = 0; k0 < K; k0 += MMQ_BK) {
+    // split K: grid row y walks stages [k_lo, k_hi) and writes its sums to slice y of `dst` (a workspace then, see launch_mmq)
+    const int64_t stages = K / MMQ_BK, st_per = (stages + gridDim.y - 1) / gridDim.y;
+    const int64_t k_lo = (int64_t)blockIdx.y * st_per * MMQ_BK;
+    const int64_t k_hi = k_lo + st_per * MMQ_BK < K ? k_lo + st_per * MMQ_BK : K;
+    if (gridDim.y > 1) dst += (int64_t)blockIdx.y * B * dst_stride;
+
+    for (int64_t k0 = k_lo; k0 < k_hi; k0 += MMQ_BK) {
         __syncthreads();
         load_weight_stage<TYPE>(W, L, row0, N, k0, sW, sWs, sWo);
         load_act_stage<TYPE, BN>(aq, ads, col0, B, K, k0, sA, sAd, sAs);
@@ -305,9 +311,32 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
         }
 }
 
+// A product with few tiles leaves most of the chip idle while each group walks all of K: such launches are cut along K into
+// slices that run side by side and a second launch adds the slices in fixed order.  At least four stages per slice, at most
+// eight slices, at most two groups per compute unit.
+static int mmq_slices(int64_t N, int64_t K, int64_t B) {
+    const int64_t bn = B <= 64 ? 64 : 128;
+    const int64_t groups = ((N + MMQ_BM - 1) / MMQ_BM) * ((B + bn - 1) / bn), stages = K / MMQ_BK;
+    int64_t n = 512 / groups;
+    if (n > stages / 4) n = stages / 4;
+    if (n > 8) n = 8;
+    if (n < 2) return 1;
+    const int64_t per = (stages + n - 1) / n;
+    return (int)((stages + per - 1) / per);   // no empty slice
+}
+
+__global__ void __launch_bounds__(256) k_mmq_split_sum(const float *__restrict__ part, float *__restrict__ dst, int64_t N, int64_t B, int64_t dst_stride,
+                                                       int n_slices) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= N * B) return;
+    float acc = part[i];
+    for (int sl = 1; sl < n_slices; sl++) acc = add_rn(acc, part[(int64_t)sl * N * B + i]);
+    dst[(i / N) * dst_stride + i % N] = acc;
+}
+
 template <int TYPE, int TN>
 static void launch_mmq(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
-                       int64_t dst_stride) {
+                       int64_t dst_stride, void *ws, size_t ws_bytes) {
     constexpr int BN = 64 * TN;
     const row_layout L = make_row_layout(TYPE, K);
     const int8_t *aq = (const int8_t *)act;
@@ -316,23 +345,42 @@ static void launch_mmq(hipStream_t s, const void *W, const void *act, float *dst
     const int n_col_tiles = (int)((B + BN - 1) / BN);
     const int n_groups = n_row_tiles * n_col_tiles;
     const int n_groups_padded = (n_groups + 7) & ~7;
+    int n_slices = mmq_slices(N, K, B);
+    if (n_slices > 1 && (ws == nullptr || ((uintptr_t)ws & 15) != 0 || ws_bytes < (size_t)n_slices * (size_t)N * (size_t)B * sizeof(float))) n_slices = 1;
+    if (n_slices > 1) {
+        hipLaunchKernelGGL((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded, (unsigned)n_slices), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
+                           (float *)ws, N, K, B, N, L, n_col_tiles, n_groups, n_groups_padded);
+        hipLaunchKernelGGL(k_mmq_split_sum, dim3((unsigned)((N * B + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, N, B, dst_stride, n_slices);
+        return;
+    }
     hipLaunchKernelGGL((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
                        dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded);
 }
 
 template <int TYPE>
 static void launch_mmq_tn(hipStream_t s, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
-                          int64_t dst_stride) {
-    if (B <= 64) launch_mmq<TYPE, 1>(s, W, act, dst, N, K, B, dst_stride);
-    else launch_mmq<TYPE, 2>(s, W, act, dst, N, K, B, dst_stride);
+                          int64_t dst_stride, void *ws, size_t ws_bytes) {
+    if (B <= 64) launch_mmq<TYPE, 1>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes);
+    else launch_mmq<TYPE, 2>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes);
 }
 
 }  // namespace mi355
 
 using namespace mi355;
 
+extern "C" size_t mi355_mul_mat_q_ws_bytes(int64_t N, int64_t K, int64_t B) {
+    if (N <= 0 || K <= 0 || B <= 0 || K % MMQ_BK != 0) return 0;
+    const int n = mmq_slices(N, K, B);
+    return n > 1 ? (size_t)n * (size_t)N * (size_t)B * sizeof(float) : 0;
+}
+
 extern "C" int mi355_mul_mat_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
                                int64_t B, int64_t dst_stride) {
+    return mi355_mul_mat_q_ws(stream, type, W, act, dst, N, K, B, dst_stride, nullptr, 0);
+}
+
+extern "C" int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
+                                  int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
     MI355_REQUIRE(is_weight_type(type), "mul_mat_q: unsupported weight type %d", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_q: K=%lld is not a multiple of the block size", (long long)K);
@@ -344,10 +392,10 @@ extern "C" int mi355_mul_mat_q(void *stream, int type, const void *W, const void
     MI355_REQUIRE((N + MMQ_BM - 1) / MMQ_BM * ((B + 63) / 64) < (1 << 30), "mul_mat_q: too many tiles");
     hipStream_t s = (hipStream_t)stream;
     switch (type) {
-        case MI355_Q4_0: launch_mmq_tn<MI355_Q4_0>(s, W, act, dst, N, K, B, dst_stride); break;
-        case MI355_Q8_0: launch_mmq_tn<MI355_Q8_0>(s, W, act, dst, N, K, B, dst_stride); break;
-        case MI355_Q4_K: launch_mmq_tn<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride); break;
-        default: launch_mmq_tn<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride); break;
+        case MI355_Q4_0: launch_mmq_tn<MI355_Q4_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_Q8_0: launch_mmq_tn<MI355_Q8_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_Q4_K: launch_mmq_tn<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        default: launch_mmq_tn<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
     }
     return launch_status("k_mmq");
 }

@@ -75,7 +75,8 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
     int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
     if (rc != MI355_OK) return rc;
     if (B <= 8) return mi355_mul_mat_vec_q(stream, type, W, ws, dst, N, K, B, dst_stride);
-    return mi355_mul_mat_q(stream, type, W, ws, dst, N, K, B, dst_stride);
+    const size_t used = mi355_mul_mat_ws_bytes(K, B);
+    return mi355_mul_mat_q_ws(stream, type, W, ws, dst, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
 }
 
 }  // extern "C"

@@ -40,6 +40,8 @@ _SIGNATURES = {
     "mi355_mul_mat": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_vec_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_mul_mat_q_ws_bytes": (_sz, [_i64, _i64, _i64]),
+    "mi355_mul_mat_q_ws": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_act_q8k_bytes": (_sz, [_i64, _i64]),
     "mi355_quantize_act_q8k": (_int, [_p, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_q8k": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
@@ -202,12 +204,15 @@ def quantize_act_q8k(x):
     return ws
 
 
-def mul_mat(t, W, x, ws=None):
-    """W: device-layout uint8 [N, row_bytes]; x f32 [B, K] -> f32 [B, N]"""
+def mul_mat(t, W, x, ws=None, split=True):
+    """W: device-layout uint8 [N, row_bytes]; x f32 [B, K] -> f32 [B, N].  split: also give the workspace the room that lets a
+    product with few tiles run as slices along K"""
     import torch
     B, K = x.shape
     N = W.shape[0]
     need = load().mi355_mul_mat_ws_bytes(K, B)
+    if split:
+        need += max(load().mi355_mul_mat_q_ws_bytes(N, K, B), load().mi355_mul_mat_q8k_ws_bytes(N, K, B))
     if ws is None or ws.numel() < need:
         ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     dst = torch.empty((B, N), dtype=torch.float32, device=x.device)
