@@ -277,7 +277,6 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
                         const int32_t *cells, const float *freq_factors, int64_t T, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
                         size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                         float ext_factor, float attn_factor, float beta_fast, float beta_slow);
-
 /* Up to three weight matrices on one quantized activation whose finished rows go through the nodes that follow the projections in
  * build_llama (src/llama.cpp:1514-1548; llm_build_kv_store :157-199): ROPE (ggml-cpu.c:9366-9549, adjacent-pair mode only) and / or
  * CPY to an f16 tensor such as a KV-cache view (ggml-cpu.c:3519-3830).  A wave owns output rows 2i and 2i+1, i.e. one rotation pair.

@@ -871,6 +871,17 @@ bool feeds_quant_mmid(const graph_walk & w, int i, const void * data, int64_t K,
     return b->data == data && b->ne[0] == K && b->ne[1] * b->ne[2] == rows && K % 32 == 0;
 }
 
+// Do the bytes of two tensors intersect?  A pattern that runs a node ahead of its place in the graph must check this: the
+// graph allocator reuses the memory of a tensor once its last reader, in graph order, has run, so a node that comes later may
+// write where an earlier, not yet executed node still has to read.
+// (This is also why the prefill sequence ROPE(q), MUL_MAT(k), ROPE(k), MUL_MAT(v), CPY(k), CPY(v) stays four glue launches: the
+// allocator gives the v product the k product's memory and the k product the unrotated q's, so the products cannot move ahead of
+// the rotations, and a single launch would need k and v at once.)
+bool bytes_overlap(const ggml_tensor * a, const ggml_tensor * b) {
+    const char * a0 = (const char *) a->data, * b0 = (const char *) b->data;
+    return a0 < b0 + ggml_nbytes(b) && b0 < a0 + ggml_nbytes(a);
+}
+
 // Runs node i and possibly a few of its successors; returns the index of the last node consumed.
 int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     hipStream_t s = ctx->stream;
@@ -911,7 +922,10 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         } else if (nxt->op == GGML_OP_MUL_MAT && nxt->src[0] != node && nxt->src[1] != node) {
             const int j2 = w.next(j);
             const ggml_tensor * m = j2 < w.n ? w.nodes[j2] : nullptr;
-            if (m && m->op == GGML_OP_MUL && ((m->src[0] == node && m->src[1] == nxt) || (m->src[1] == node && m->src[0] == nxt))) jm = j2;
+            // the product runs ahead of SILU: its result must not land on SILU's input
+            if (m && m->op == GGML_OP_MUL && ((m->src[0] == node && m->src[1] == nxt) || (m->src[1] == node && m->src[0] == nxt)) &&
+                !bytes_overlap(nxt, node->src[0]))
+                jm = j2;
         }
         if (jm >= 0) {
             ggml_tensor * mul = (ggml_tensor *) w.nodes[jm];
@@ -1090,6 +1104,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                                 ggml_is_contiguous(mul) && mul->type == GGML_TYPE_F32 && ggml_are_same_shape(mul, node);
             if (mul_ok && is_quant_gemv_candidate(up) && up->src[1]->data == b->data && up->src[1]->ne[0] == K && up->src[1]->ne[1] == B &&
                 up->ne[0] == N && w.sole_use(ju) && w.sole_use(jm) && N % 32 == 0 && ggml_is_contiguous(node) && ggml_is_contiguous(up) &&
+                !bytes_overlap(node, up) &&   // both products are written before SiLU*up reads them
                 feeds_quant_gemv(w, jm, mul->data, N, B)) {
                 // this launch reads one quantized activation and writes the next: the two slots
                 const size_t in_bytes = mi355_act_bytes(K, B), out_bytes = mi355_act_bytes(N, B);
@@ -1586,7 +1601,7 @@ ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
     }
     const char * ng = getenv("MI355_NO_GRAPH");
     ctx->replay.enabled = ctx->fuse && !(ng && ng[0] == '1');
-    if (hipMalloc((void **) &ctx->cells, sizeof(iota_host)) != hipSuccess) {
+    if (hipMalloc((void **) &ctx->cells, 8 * sizeof(int32_t)) != hipSuccess) {
         (void) hipFree(ctx->iota);
         delete ctx;
         return nullptr;

@@ -57,7 +57,8 @@ __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ 
 }
 
 struct rope_kv_args {
-    float *q;               // [T][H][D] f32, rotated in place
+    const float *q;         // [T][H][D] f32
+    float *q_out;           // rotated q (may be q itself)
     const float *k;         // [T][HK][D] f32
     const float *v;         // [T][HK][D] f32
     uint8_t *kcache, *vcache;   // f16; element (cell, head, d) at cell*nb1 + head*nb2 + 2*d
@@ -96,12 +97,13 @@ __global__ void k_rope_kv_store(rope_kv_args a) {
     const bool rot = i0 < a.n_dims;
     const int ia = (rot && neox) ? pair : i0, ib = (rot && neox) ? pair + a.n_dims / 2 : i0 + 1;
     if (h < a.H) {
-        float *p = a.q + ((int64_t)t * a.H + h) * D;
+        const float *p = a.q + ((int64_t)t * a.H + h) * D;
+        float *o = a.q_out + ((int64_t)t * a.H + h) * D;
         const float x0 = p[ia], x1 = p[ib];
         float y0 = x0, y1 = x1;
         if (rot) rope_pair(a, a.pos[t], pair, x0, x1, y0, y1);
-        p[ia] = y0;
-        p[ib] = y1;
+        o[ia] = y0;
+        o[ib] = y1;
     } else if (h < a.H + a.HK) {
         const int hk = h - a.H;
         const float *p = a.k + ((int64_t)t * a.HK + hk) * D;
@@ -192,7 +194,7 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
     MI355_REQUIRE(mode == 0 || mode == 2, "rope_kv_store: mode %d not supported (0 = adjacent pairs, 2 = NeoX)", mode);
     MI355_REQUIRE(n_dims > 0 && n_dims % 2 == 0 && n_dims <= D, "rope_kv_store: bad n_dims");
     rope_kv_args a;
-    a.q = q; a.k = k; a.v = v; a.kcache = (uint8_t *)kcache; a.vcache = (uint8_t *)vcache;
+    a.q = q; a.q_out = q; a.k = k; a.v = v; a.kcache = (uint8_t *)kcache; a.vcache = (uint8_t *)vcache;
     a.pos = pos; a.cells = cells; a.ff = freq_factors;
     a.k_nb1 = (int64_t)k_nb1; a.k_nb2 = (int64_t)k_nb2; a.v_nb1 = (int64_t)v_nb1; a.v_nb2 = (int64_t)v_nb2;
     a.T = (int)T; a.H = (int)H; a.HK = (int)HK; a.D = (int)D; a.n_dims = n_dims; a.mode = mode;

@@ -58,7 +58,7 @@ _SIGNATURES = {
     "mi355_rms_norm_mul_quant_q8k": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
     "mi355_swiglu_quant_q8k": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
     "mi355_rope_kv_store": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _int, _int, _int,
-                                   _f, _f, _f, _f, _f, _f]),
+                            _f, _f, _f, _f, _f, _f]),
     "mi355_ffn_gate_up_swiglu": (_int, [_p, _int, _p, _int, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q_rope": (_int, [_p, _int, _p, _p, _i64, _i64, _p]),
     "mi355_qkv_rope_store": (_int, [_p, _int, _p, _int, _p, _int, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64,
