@@ -334,6 +334,129 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
     }
 }
 
+// ---- prefill with few query tiles: the two 32-cell halves of every K/V tile go to different waves ----------------------------
+// k_fattn_mma gives a wave 32 queries of one head and the whole 64-cell tile; a batch of a few hundred rows is then fewer groups
+// than compute units, each a serial chain of tiles.  Here a group is two query heads of one kv head x the two halves of the
+// tile: wave (hp, u) scores and accumulates cells [32u, 32u + 32) of each tile for head hp with its own soft-max state, and the
+// u = 1 wave hands its state to the u = 0 wave through LDS at the end.  Twice the groups, half the work per wave and tile.
+template <int D>
+__global__ void __launch_bounds__(256, 2) k_fattn_mma_half(fattn_args a) {
+    typedef kv_stage<D, 256> stage_t;
+    constexpr int NDT = D / 32;
+    constexpr int KV_HALVES = FM_BC * stage_t::KP + D * stage_t::VP;                 // f16 elements of the K tile and the V^T tile
+    constexpr int MERGE_FLOATS = 2 * (D + 2) * 32;                                    // per head: O^T [D][32], max, sum
+    constexpr int SMEM_BYTES = KV_HALVES * 2 > MERGE_FLOATS * 4 ? KV_HALVES * 2 : MERGE_FLOATS * 4;
+    __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM_BYTES];
+    _Float16 *sK = (_Float16 *)smem, *sVt = sK + FM_BC * stage_t::KP;
+    float *s_merge = (float *)smem;   // reused after the last tile
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int u = wave & 1, hp = wave >> 1;
+    const int pairs = (int)(a.Hq / a.Hkv) / 2;   // head pairs per kv head
+    const int64_t hk = blockIdx.y / pairs, hg = blockIdx.y % pairs;
+    const int64_t head = (hk * pairs + hg) * 2 + hp;
+    const int64_t q0 = (int64_t)blockIdx.x * 32;
+    const int64_t iq = q0 + l32 < a.Nq ? q0 + l32 : a.Nq - 1;   // clamped: rows past Nq are computed and dropped
+
+    f16x8 qf[D / 16];
+    load_q<D>(qf, (const float *)(a.q + iq * a.q_nb1 + head * a.q_nb2), lhi);
+    const float slope = alibi_slope(a, head);
+    const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
+    const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
+    const bool mask_aligned = (((uintptr_t)a.mask | a.mask_nb1) & 7) == 0;
+
+    f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] = 0.0f;
+    float m = FM_NEG, l = 0.0f;
+
+    stage_t st;
+    u32x2 mnext[4];
+    auto prefetch = [&](int64_t kv0) {
+        st.fetch(a, hk, kv0, tid);
+        fetch_mask<4>(mnext, mrow, mask_aligned && kv0 + FM_BC <= a.Nkv, kv0 + 32 * u + 4 * lhi, a.Nkv);
+    };
+    prefetch(0);
+    for (int64_t kv0 = 0; kv0 < a.Nkv; kv0 += FM_BC) {
+        __syncthreads();   // the previous tile has been consumed
+        st.commit(sK, sVt, tid);
+        u32x2 mcur[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) mcur[g] = mnext[g];
+        __syncthreads();
+        if (kv0 + FM_BC < a.Nkv) prefetch(kv0 + FM_BC);
+        f32x16 S = scores<D>(qf, sK, u, l32, lhi);
+        float mx = finish_scores(S, mcur, a, scale, slope, kv0 + 32 * u, lhi, a.Nkv);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (__ballot(mx > FM_NEG) == 0) continue;   // all 32 cells masked for all 32 queries (wave-uniform; barriers are at the loop head)
+        const float m_new = fmaxf(m, mx);
+        const float alpha = __expf(m - m_new);
+        float rs = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float p = S[r] > FM_NEG ? __expf(S[r] - m_new) : 0.0f;
+            S[r] = p;
+            rs += p;
+        }
+        rs += __shfl_xor(rs, 32, 64);
+        l = l * alpha + rs;
+        m = m_new;
+        if (__ballot(alpha != 1.0f) != 0) {   // wave-uniform
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+        }
+        accumulate_pv<D, NDT>(o, S, sVt, 0, u, l32, lhi);
+    }
+
+    // ---- the u = 1 wave's state joins the u = 0 wave of the same head
+    float *mg = s_merge + hp * (D + 2) * 32;   // [d][query], then max, sum
+    __syncthreads();
+    if (u == 1) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] = o[dt][r];
+        if (lhi == 0) {
+            mg[D * 32 + l32] = m;
+            mg[(D + 1) * 32 + l32] = l;
+        }
+    }
+    __syncthreads();
+    if (u != 0 || q0 + l32 >= a.Nq) return;
+    const float m1 = mg[D * 32 + l32], l1 = mg[(D + 1) * 32 + l32];
+    const float M = fmaxf(m, m1);
+    const float f0 = __expf(m - M), f1 = __expf(m1 - M);
+    l = l * f0 + l1 * f1;
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    float *dp = a.dst + ((q0 + l32) * a.Hq + head) * D;
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            f32x4 w;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int r = 4 * g + i;
+                w[i] = (o[dt][r] * f0 + mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] * f1) * inv;
+            }
+            *(f32x4 *)(dp + 32 * dt + 8 * g + 4 * lhi) = w;
+        }
+}
+
+template <int D>
+int launch_half(hipStream_t s, const fattn_args &a) {
+    const int64_t pairs = (a.Hq / a.Hkv) / 2;
+    const dim3 grid((unsigned)((a.Nq + 31) / 32), (unsigned)(a.Hkv * pairs));
+    hipLaunchKernelGGL((k_fattn_mma_half<D>), grid, dim3(256), 0, s, a);
+    return launch_status("k_fattn_mma_half");
+}
+
 template <int D, int HPW>
 int launch(hipStream_t s, const fattn_args &a) {
     constexpr int QTW = 4 / HPW;
@@ -549,6 +672,14 @@ int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes) {
         const int rc = launch_status("k_mask_extent");
         if (rc != MI355_OK) return rc;
         a.kv_extent = (const int32_t *)a.ws;
+    }
+    // few query tiles (a batch of a few hundred rows): twice the groups with half a K/V tile per wave, while the chip is not full
+    const int64_t R = a.Hq / a.Hkv;
+    if (R % 2 == 0 && n_tiles * a.Hkv * (R / 2) <= 512) {
+        switch (D) {
+            case 64: return launch_half<64>(s, a);
+            case 128: return launch_half<128>(s, a);
+        }
     }
     switch (D) {
         case 64: return launch_hpw<64>(s, a);
