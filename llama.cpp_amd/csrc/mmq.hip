@@ -175,6 +175,102 @@ __device__ __forceinline__ void load_act_stage(const int8_t *__restrict__ aq, co
     }
 }
 
+// ---- the same stages split into "request" (global -> registers) and "commit" (unpack -> LDS), so that the next stage's bytes
+// travel while the current stage is contracted (Q4_0 / Q8_0, whose per-32 scales keep them on this kernel)
+template <int TYPE> struct mmq_wregs {};
+template <> struct mmq_wregs<MI355_Q4_0> {
+    u32x4 q[2];
+    unsigned short d[2];
+    __device__ __forceinline__ void fetch(const uint8_t *__restrict__ W, const row_layout &L, int64_t row0, int64_t N, int64_t k0, int tid) {
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 2, b = idx & 3;
+            const int64_t row = row0 + r < N ? row0 + r : N - 1;
+            const uint8_t *wrow = W + row * L.row_bytes;
+            const int64_t blk = (k0 >> 5) + b;
+            q[it] = load16(wrow + blk * 16);
+            d[it] = *(const unsigned short *)(wrow + L.off_b + blk * 2);
+        }
+    }
+    __device__ __forceinline__ void commit(int8_t *sW, float *sWs, int tid) const {
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 2, b = idx & 3;
+            u32x4 lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {   // nibble - 8 per byte without cross-byte borrow
+                lo[i] = (((q[it][i] & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+                hi[i] = ((((q[it][i] >> 4) & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+            }
+            *(u32x4 *)(sW + r * MMQ_LDK + b * 32) = lo;
+            *(u32x4 *)(sW + r * MMQ_LDK + b * 32 + 16) = hi;
+            sWs[b * MMQ_BM + r] = half_bits_to_float(d[it]);
+        }
+    }
+};
+template <> struct mmq_wregs<MI355_Q8_0> {
+    u32x4 q[4];
+    unsigned short d[4];
+    __device__ __forceinline__ void fetch(const uint8_t *__restrict__ W, const row_layout &L, int64_t row0, int64_t N, int64_t k0, int tid) {
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 3, c = idx & 7;   // c: 16-byte piece of the stage
+            const int64_t row = row0 + r < N ? row0 + r : N - 1;
+            const uint8_t *wrow = W + row * L.row_bytes;
+            q[it] = load16(wrow + k0 + c * 16);
+            d[it] = *(const unsigned short *)(wrow + L.off_b + ((k0 >> 5) + (c >> 1)) * 2);   // both pieces of a block read its scale
+        }
+    }
+    __device__ __forceinline__ void commit(int8_t *sW, float *sWs, int tid) const {
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 3, c = idx & 7;
+            *(u32x4 *)(sW + r * MMQ_LDK + c * 16) = q[it];
+            if ((c & 1) == 0) sWs[(c >> 1) * MMQ_BM + r] = half_bits_to_float(d[it]);
+        }
+    }
+};
+template <int BN> struct mmq_aregs {
+    static constexpr int NQ = BN * 8 / 256, NS = (BN * 4 + 255) / 256;
+    u32x4 q[NQ];
+    float d[NS];
+    __device__ __forceinline__ void fetch(const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int64_t col0, int64_t B, int64_t K, int64_t k0,
+                                          int tid) {
+        const int64_t nblk = K >> 5;
+#pragma unroll
+        for (int it = 0; it < NQ; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 3, c = idx & 7;
+            const int64_t col = col0 + r < B ? col0 + r : B - 1;
+            q[it] = load16(aq + col * K + k0 + c * 16);
+        }
+#pragma unroll
+        for (int it = 0; it < NS; it++) {
+            const int idx = tid + it * 256;
+            const int r = (idx >> 2) < BN ? (idx >> 2) : BN - 1, b = idx & 3;
+            const int64_t col = col0 + r < B ? col0 + r : B - 1;
+            d[it] = ads[col * nblk + (k0 >> 5) + b].d;
+        }
+    }
+    __device__ __forceinline__ void commit(int8_t *sA, float *sAd, int tid) const {
+#pragma unroll
+        for (int it = 0; it < NQ; it++) {
+            const int idx = tid + it * 256;
+            const int r = idx >> 3, c = idx & 7;
+            *(u32x4 *)(sA + r * MMQ_LDK + c * 16) = q[it];
+        }
+#pragma unroll
+        for (int it = 0; it < NS; it++) {
+            const int idx = tid + it * 256;
+            if (idx < BN * 4) sAd[(idx & 3) * BN + (idx >> 2)] = d[it];
+        }
+    }
+};
+
 template <int TYPE, int TN>
 __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
                                              const act_ds *__restrict__ ads, float *__restrict__ dst, int64_t N,
@@ -215,11 +311,30 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
     const int64_t k_hi = k_lo + st_per * MMQ_BK < K ? k_lo + st_per * MMQ_BK : K;
     if (gridDim.y > 1) dst += (int64_t)blockIdx.y * B * dst_stride;
 
+    constexpr bool PREFETCH = TYPE == MI355_Q4_0 || TYPE == MI355_Q8_0;
+    mmq_wregs<TYPE> wregs;
+    mmq_aregs<BN> aregs;
+    if constexpr (PREFETCH) {
+        wregs.fetch(W, L, row0, N, k_lo, threadIdx.x);
+        aregs.fetch(aq, ads, col0, B, K, k_lo, threadIdx.x);
+    }
     for (int64_t k0 = k_lo; k0 < k_hi; k0 += MMQ_BK) {
         __syncthreads();
-        load_weight_stage<TYPE>(W, L, row0, N, k0, sW, sWs, sWo);
-        load_act_stage<TYPE, BN>(aq, ads, col0, B, K, k0, sA, sAd, sAs);
+        if constexpr (PREFETCH) {
+            wregs.commit(sW, sWs, threadIdx.x);
+            aregs.commit(sA, sAd, threadIdx.x);
+        } else {
+            load_weight_stage<TYPE>(W, L, row0, N, k0, sW, sWs, sWo);
+            load_act_stage<TYPE, BN>(aq, ads, col0, B, K, k0, sA, sAd, sAs);
+        }
         __syncthreads();
+        if constexpr (PREFETCH) {
+            // past the end the last stage is requested again and never committed: no branch, the loads stay here
+            const int64_t k1 = k0 + MMQ_BK < k_hi ? k0 + MMQ_BK : k0;
+            wregs.fetch(W, L, row0, N, k1, threadIdx.x);
+            aregs.fetch(aq, ads, col0, B, K, k1, threadIdx.x);
+            __builtin_amdgcn_sched_barrier(0);   // requested now, a whole stage ahead of their commit
+        }
 
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {   // one Q8_1 block per step
