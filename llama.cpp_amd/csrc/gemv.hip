@@ -508,6 +508,15 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     }
     int rpw = pick_rpw(total_rows);
     if (B > 4 && rpw > 2) rpw = 2;   // keep the accumulator tile in registers
+    if (getenv("MI355_GEMV_RPW") == nullptr) {   // per-type corrections, measured on the 8B shapes (not applied over the tuning override)
+        bool any_q6 = false, all_q4k = true;
+        for (int i = 0; i < n_mats; i++) {
+            any_q6 = any_q6 || mats[i].type == MI355_Q6_K;
+            all_q4k = all_q4k && mats[i].type == MI355_Q4_K;
+        }
+        if (any_q6 && rpw > 2) rpw = 2;                   // 128256 x 4096 Q6_K: 79.5 -> 69.3 us with two rows per wave
+        if (all_q4k && rpw == 1 && K >= 8192) rpw = 2;    // 4096 x 14336 Q4_K: 11.4 -> 10.6 us (half the activation reads)
+    }
     gemv_batch b;
     b.n = n_mats;
     int64_t groups = 0;
