@@ -508,7 +508,7 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     }
     int rpw = pick_rpw(total_rows);
     if (B > 4 && rpw > 2) rpw = 2;   // keep the accumulator tile in registers
-    if (getenv("MI355_GEMV_RPW") == nullptr) {   // per-type corrections, measured on the 8B shapes (not applied over the tuning override)
+    if (getenv("MI355_GEMV_RPW") == nullptr && getenv("MI355_GEMV_PLAIN_RPW") == nullptr) {   // per-type corrections, measured on the 8B shapes (off under either tuning variable)
         bool any_q6 = false, all_q4k = true;
         for (int i = 0; i < n_mats; i++) {
             any_q6 = any_q6 || mats[i].type == MI355_Q6_K;
