@@ -113,12 +113,13 @@ def sweep(kinds):
                 wbytes = int(N * K * bpe[t])
                 nm = max(2, min(32, (1 << 31) // wbytes))
                 Ws = [mi355.upload_weights(t, lg.random_quantized(t, N, K, dev, gen)) for _ in range(nm)]
-                act = mi355.quantize_act(torch.randn(1, K, device=dev, generator=gen))
-                out = torch.empty(1, N, device=dev)
-                us = timed(lambda i: mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, t, Ws[i].data_ptr(), act.data_ptr(), out.data_ptr(), N, K, 1, N)), nm, 4)
-                alg = wbytes + 4 * K + 4 * N
-                emit(kernel="MUL_MAT batch 1 (GEMV)", case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
-                     unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg)
+                for B in (1, 8):
+                    act = mi355.quantize_act(torch.randn(B, K, device=dev, generator=gen))
+                    out = torch.empty(B, N, device=dev)
+                    us = timed(lambda i: mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, t, Ws[i].data_ptr(), act.data_ptr(), out.data_ptr(), N, K, B, N)), nm, 4)
+                    alg = wbytes + B * (4 * K + 4 * N)
+                    emit(kernel="MUL_MAT batch %d (GEMV)" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
+                         unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg)
                 del Ws
     if "mmq" in kinds:
         for t in (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q6_K):

@@ -94,6 +94,17 @@ size_t mi355_mul_mat_q_ws_bytes(int64_t N, int64_t K, int64_t B);
 int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
                        int64_t dst_stride, void *ws, size_t ws_bytes);
 
+/* MUL_MAT for 1..32 activation rows as one weight-streaming launch on the int8 matrix cores (Q4_0, Q8_0, Q4_K; K a
+ * multiple of 256; 16-byte aligned rows: mi355_mul_mat_skinny_supported says whether a product qualifies).  Same operands
+ * as mi355_mul_mat_vec_q (`act` from mi355_quantize_act) plus an optional residual added to the result (may alias dst).
+ * It is what mi355_mul_mat uses between the batch-1 kernels and the tile kernels (ggml's MUL_MAT with src1->ne[1] of
+ * 5..32, ggml_compute_forward_mul_mat, ggml/src/ggml-cpu/ggml-cpu.c:7380-7560).  `ws` of mi355_mul_mat_skinny_ws_bytes
+ * bytes lets products with few rows split K over several groups; with less, or NULL, one group walks the whole of K. */
+int mi355_mul_mat_skinny_supported(int type, const void *W, int64_t K, int64_t B);
+size_t mi355_mul_mat_skinny_ws_bytes(int64_t N, int64_t K, int64_t B);
+int mi355_mul_mat_skinny(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N,
+                         int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
+
 /* K-quant (Q4_K, Q6_K) tile GEMM with the activation format ggml-cpu uses for these weight
  * types: one f32 scale per 256 elements (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516;
  * vec_dot_type of type_traits_cpu, ggml/src/ggml-cpu/ggml-cpu.c:252-417), so the integer

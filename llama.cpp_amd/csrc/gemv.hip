@@ -506,6 +506,18 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
         if (rc != MI355_OK) return rc;
         total_rows += mats[i].N;
     }
+    if (B >= 5) {   // from five activation rows on the matrix-core kernel is ahead wherever it supports the weight type (skinny.hip)
+        static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;
+        bool ok = !no_skinny;
+        for (int i = 0; i < n_mats; i++) ok = ok && mi355_mul_mat_skinny_supported(mats[i].type, mats[i].W, K, B);
+        if (ok) {
+            for (int i = 0; i < n_mats; i++) {
+                int rc = mi355_mul_mat_skinny(stream, mats[i].type, mats[i].W, act, mats[i].dst, mats[i].residual, mats[i].N, K, B, mats[i].dst_stride, nullptr, 0);
+                if (rc != MI355_OK) return rc;
+            }
+            return MI355_OK;
+        }
+    }
     int rpw = pick_rpw(total_rows);
     if (B > 4 && rpw > 2) rpw = 2;   // keep the accumulator tile in registers
     if (getenv("MI355_GEMV_RPW") == nullptr && getenv("MI355_GEMV_PLAIN_RPW") == nullptr) {   // per-type corrections, measured on the 8B shapes (off under either tuning variable)

@@ -51,8 +51,15 @@ extern "C" {
 // the per-super-block activation format of the K-quant tile kernel is smaller than the Q8_1 one
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B) { return (mi355_act_bytes(K, B) + 255) & ~(size_t)255; }
 
+// 5..32 activation rows: the weight-streaming matrix-core kernel (skinny.hip) where it supports the product.
+// MI355_NO_SKINNY=1 sends these batches to the batch-1 kernels (up to 8) and the tile kernels as before (tuning aid).
+static bool use_skinny(int type, const void *W, int64_t K, int64_t B) {
+    static const bool off = getenv("MI355_NO_SKINNY") != nullptr;
+    return !off && B >= 5 && B <= 32 && mi355_mul_mat_skinny_supported(type, W, K, B);
+}
+
 static bool use_q8k_tiles(int type, const void *W, int64_t K, int64_t B) {
-    return B > 8 && (type == MI355_Q4_K || type == MI355_Q6_K) && layout_aligned(W, make_row_layout(type, K));
+    return B > 8 && !use_skinny(type, W, K, B) && (type == MI355_Q4_K || type == MI355_Q6_K) && layout_aligned(W, make_row_layout(type, K));
 }
 
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
@@ -74,8 +81,9 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
     }
     int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
     if (rc != MI355_OK) return rc;
-    if (B <= 8) return mi355_mul_mat_vec_q(stream, type, W, ws, dst, N, K, B, dst_stride);
     const size_t used = mi355_mul_mat_ws_bytes(K, B);
+    if (use_skinny(type, W, K, B)) return mi355_mul_mat_skinny(stream, type, W, ws, dst, nullptr, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
+    if (B <= 8) return mi355_mul_mat_vec_q(stream, type, W, ws, dst, N, K, B, dst_stride);
     return mi355_mul_mat_q_ws(stream, type, W, ws, dst, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
 }
 

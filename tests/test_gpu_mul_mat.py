@@ -150,7 +150,8 @@ def test_mmq_matches_oracle(dev, name, t, N, K, B):
     Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
     got = mi355.mul_mat(t, Wd, _to_dev(dev, x)).cpu().numpy()
     Nt, Bt = min(N, 64), min(B, 24)
-    if B > 8 and (t == orc.Q4_K or (t == orc.Q6_K and K % 2048 == 0)):   # Q6_K rows are 16-byte aligned only then
+    skinny = B <= 32 and t != orc.Q6_K and K % 256 == 0   # up to 32 activation rows: the weight-streaming kernel, Q8_1 activations
+    if B > 8 and not skinny and (t == orc.Q4_K or (t == orc.Q6_K and K % 2048 == 0)):   # Q6_K rows are 16-byte aligned only then
         # K-quants take the activation format of the CPU path (one scale per 256): integer sums are the
         # CPU's own (ggml-cpu-quants.c:6817-6848, 8262-8283), only the f32 summation order differs
         want = orc.mul_mat("cpu", t, Wq[:Nt], x[:Bt])
@@ -160,6 +161,28 @@ def test_mmq_matches_oracle(dev, name, t, N, K, B):
     if orc.ref is not None:
         cpu = orc.mul_mat("ref", t, Wq, x)
         assert orc.nmse(got, cpu) <= 5e-4
+
+
+@pytest.mark.parametrize("name,t", [(n, t) for n, t in TYPES if t != orc.Q6_K])
+@pytest.mark.parametrize("N,K,B", [(100, 256, 5), (257, 1024, 8), (4096, 4096, 13), (1024, 14336, 17), (64, 3584, 24), (333, 2048, 32), (4096, 4096, 1)])
+@pytest.mark.parametrize("split", [False, True])
+def test_skinny_matches_oracle(dev, name, t, N, K, B, split):
+    """the weight-streaming matrix-core kernel for a few activation rows: ragged row and batch counts, K that does not divide
+    evenly over the four waves, with and without slices along K, with a residual"""
+    import mi355
+    rng = np.random.default_rng(N * 5 + K + B)
+    Wq = _weights(rng, t, N, K, "ref")
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    res = rng.standard_normal((B, N)).astype(np.float32)
+    Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
+    got = mi355.mul_mat_skinny(t, Wd, _to_dev(dev, x), split=split).cpu().numpy()
+    got_res = mi355.mul_mat_skinny(t, Wd, _to_dev(dev, x), residual=_to_dev(dev, res), split=split).cpu().numpy()
+    assert np.array_equal(got_res, got + res)
+    Nt, Bt = min(N, 64), min(B, 24)
+    want = orc.mul_mat("q8_1", t, Wq[:Nt], x[:Bt])
+    assert orc.nmse(got[:Bt, :Nt], want) < 1e-9      # exact integer dots; f32 against f64 scale algebra
+    if orc.ref is not None:
+        assert orc.nmse(got, orc.mul_mat("ref", t, Wq, x)) <= 5e-4      # tests/test-backend-ops.cpp:1916
 
 
 @pytest.mark.parametrize("name,t", [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q6_K)])
@@ -187,11 +210,12 @@ def test_unaligned_rows_fallback(dev, name, t):
     rng = np.random.default_rng(5)
     be = orc.BLOCK[t][0]
     K = be * 3
-    for B in (1, 12):
+    for B in (1, 12, 40):
         Wq = _weights(rng, t, 19, K)
         x = rng.standard_normal((B, K)).astype(np.float32)
         Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
         got = mi355.mul_mat(t, Wd, _to_dev(dev, x)).cpu().numpy()
-        # Q4_K rows are always aligned, so B > 8 takes the super-block tile kernel and the CPU's activation format
-        want = orc.mul_mat("cpu" if (t == orc.Q4_K and B > 8) else "q8_1", t, Wq, x)
+        # Q4_K rows are always aligned, so B > 32 takes the super-block tile kernel and the CPU's activation format
+        # (5..32 rows: the weight-streaming kernel with Q8_1 activations)
+        want = orc.mul_mat("cpu" if (t == orc.Q4_K and B > 32) else "q8_1", t, Wq, x)
         assert orc.nmse(got, want) < 1e-9
