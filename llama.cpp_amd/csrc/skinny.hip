@@ -27,6 +27,7 @@ template <int TYPE> struct sk_traits;
 template <> struct sk_traits<MI355_Q4_0> { static constexpr int ROW_BYTES = 128, W_LOADS = 8; };    // per step and weight row
 template <> struct sk_traits<MI355_Q8_0> { static constexpr int ROW_BYTES = 256, W_LOADS = 16; };
 template <> struct sk_traits<MI355_Q4_K> { static constexpr int ROW_BYTES = 128, W_LOADS = 8; };    // qs only; the header goes to registers
+template <> struct sk_traits<MI355_Q6_K> { static constexpr int ROW_BYTES = 128, W_LOADS = 8; };    // ql; qh (64 bytes) is copied beside it
 
 // Orders a wave's own LDS accesses around the point where its lanes exchange data through LDS: the hardware completes
 // them in program order, so all that is needed is that neither the compiler nor the instruction scheduler moves an access
@@ -53,6 +54,8 @@ template <int TYPE, int NI> struct sk_regs {
     static constexpr int NA = 2 * NI;                                   // ... for 8 NI activation rows of 256 bytes
     static constexpr int NT = (NI + 1) / 2;                             // ... for their 8 {d, sum} pairs each
     u32x4 w[NW], a[NA], t[NT], hdr;
+    u32x4 qh[TYPE == MI355_Q6_K ? 2 : 1];   // Q6_K: the high bit pairs, 32 rows x 64 bytes
+    u32 d6;                                 // Q6_K: the f16 super-block scale of the lane's row (hdr holds its 16 int8 scales)
 };
 
 // grid.x = 32-row tiles of the weight matrix, grid.y = slices of K (partial sums to `dst` as [slice][B][dst_stride] then).
@@ -64,8 +67,11 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
     typedef sk_traits<TYPE> T;
     typedef sk_regs<TYPE, NI> R;
     constexpr int WPAD = T::ROW_BYTES + 16;
-    constexpr int W_BYTES = 32 * WPAD, A_BYTES = 8 * NI * SK_APAD, T_BYTES = 8 * 8 * NI * 8;
-    constexpr int WAVE_BYTES = W_BYTES + A_BYTES + T_BYTES;
+    constexpr int QHPAD = 64 + 16;
+    constexpr bool Q6 = TYPE == MI355_Q6_K;
+    constexpr int W_BYTES = 32 * WPAD + (Q6 ? 32 * QHPAD : 0), A_BYTES = 8 * NI * SK_APAD, T_BYTES = 8 * 8 * NI * 8;
+    constexpr int G_BYTES = Q6 ? 16 * 8 * NI * 4 : 0;   // Q6_K: integer sums of the activation levels per 16 elements
+    constexpr int WAVE_BYTES = W_BYTES + A_BYTES + T_BYTES + G_BYTES;
     constexpr int RED_BYTES = 4 * NI * 4 * 64 * 4;
     __shared__ __attribute__((aligned(16))) uint8_t s_mem[4 * WAVE_BYTES > RED_BYTES ? 4 * WAVE_BYTES : RED_BYTES];
     const int lane = threadIdx.x & 63;
@@ -74,6 +80,8 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
     uint8_t *s_w = s_mem + wave * WAVE_BYTES;
     uint8_t *s_a = s_w + W_BYTES;
     float2 *s_t = (float2 *)(s_a + A_BYTES);
+    int *s_g = (int *)(s_a + A_BYTES + T_BYTES);
+    uint8_t *s_qh = s_w + 32 * WPAD;
 
     const row_layout L = make_row_layout(TYPE, K);
     const int nsteps = K >> 8;
@@ -95,6 +103,13 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
         row = row < N ? row : N - 1;   // clamp: rows past the end repeat the last row and are not stored
         w_src[u] = W + row * L.row_bytes + 16 * w_piece + (TYPE == MI355_Q4_K ? 16 : 0);
     }
+    const uint8_t *qh_src[2];   // Q6_K: 4 lanes per row, 16 rows per load
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        int64_t row = row0 + (lane >> 2) + 16 * u;
+        row = row < N ? row : N - 1;
+        qh_src[u] = W + row * L.row_bytes + L.off_b + 16 * (lane & 3);
+    }
     const int64_t my_row = row0 + r < N ? row0 + r : N - 1;
     const uint8_t *w_mine = W + my_row * L.row_bytes;   // the row whose results this lane holds: its scales go to registers
     const int a_piece = lane & 15, a_row = lane >> 4;
@@ -114,11 +129,19 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
 
     auto fetch = [&](int step, R &g) {
         const int s = step < nsteps ? step : nsteps - 1;
-        const int64_t w_off = TYPE == MI355_Q4_0 ? (int64_t)s * 128 : TYPE == MI355_Q8_0 ? (int64_t)s * 256 : (int64_t)s * Q4_K_BYTES;
+        const int64_t w_off = TYPE == MI355_Q8_0 ? (int64_t)s * 256 : TYPE == MI355_Q4_K ? (int64_t)s * Q4_K_BYTES : (int64_t)s * 128;
 #pragma unroll
         for (int u = 0; u < R::NW; u++) g.w[u] = load16(w_src[u] + w_off);
-        if constexpr (TYPE == MI355_Q4_K) g.hdr = load16(w_mine + w_off);
-        else g.hdr = load16(w_mine + L.off_b + s * 16);   // eight f16 block scales
+        if constexpr (TYPE == MI355_Q4_K) {
+            g.hdr = load16(w_mine + w_off);
+        } else if constexpr (Q6) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) g.qh[u] = load16(qh_src[u] + s * 64);
+            g.hdr = load16(w_mine + L.off_c + s * 16);                            // sixteen int8 scales
+            g.d6 = *(const unsigned short *)(w_mine + L.off_d + s * 2);
+        } else {
+            g.hdr = load16(w_mine + L.off_b + s * 16);   // eight f16 block scales
+        }
 #pragma unroll
         for (int u = 0; u < R::NA; u++) g.a[u] = load16(a_src[u] + s * 256);
 #pragma unroll
@@ -139,8 +162,20 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
         // ---- registers -> the wave's LDS
 #pragma unroll
         for (int u = 0; u < R::NW; u++) *(u32x4 *)(s_w + (w_row + u * RPL) * WPAD + 16 * w_piece) = cur.w[u];
+        if constexpr (Q6) {
 #pragma unroll
-        for (int u = 0; u < R::NA; u++) *(u32x4 *)(s_a + (a_row + 4 * u) * SK_APAD + 16 * a_piece) = cur.a[u];
+            for (int u = 0; u < 2; u++) *(u32x4 *)(s_qh + ((lane >> 2) + 16 * u) * QHPAD + 16 * (lane & 3)) = cur.qh[u];
+        }
+#pragma unroll
+        for (int u = 0; u < R::NA; u++) {
+            *(u32x4 *)(s_a + (a_row + 4 * u) * SK_APAD + 16 * a_piece) = cur.a[u];
+            if constexpr (Q6) {   // the lane's 16 bytes are one 16-element group of its activation row
+                int sum = 0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) sum = dot4(0x01010101, (int)cur.a[u][i], sum);
+                s_g[a_piece * (8 * NI) + a_row + 4 * u] = sum;
+            }
+        }
 #pragma unroll
         for (int u = 0; u < R::NT; u++) {
             if (t_row + 16 * u < 8 * NI) {
@@ -158,59 +193,100 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
         }
         wave_lds_sync();
 
-        // ---- per-block weight scales of this lane's row
-        float ws[8], wm[8];
-        if constexpr (TYPE == MI355_Q4_K) {
-            const float d = half_bits_to_float((unsigned short)(cur.hdr[0] & 0xFFFFu));
-            const float dmin = half_bits_to_float((unsigned short)(cur.hdr[0] >> 16));
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                int sc, mn;
-                q4k_scale_min(cur.hdr[1], cur.hdr[2], cur.hdr[3], j, sc, mn);
-                ws[j] = d * (float)sc;
-                wm[j] = -(dmin * (float)mn);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++) ws[j] = f16_of(cur.hdr, j);
-        }
         const int am = r < 8 * NI ? r : r & 7;   // operand rows past the copied ones repeat copied ones; their results are not used
+        if constexpr (Q6) {
+            // 16 groups of 16 levels, each with its own int8 scale: one v_mfma_i32_32x32x16_i8 per group (8 levels per lane).
+            // Group (hf, q, is): levels 128 hf + 32 q + 16 is .. + 16; level l of it = nibble q / 2 of ql byte 64 hf + 32 (q % 2) + 16 is + l
+            // plus bits 2q, 2q + 1 of qh byte 32 hf + 16 is + l, minus 32 (dequantize_row_q6_K, ggml/src/ggml-quants.c:1690-1719).
+            const float d = half_bits_to_float((unsigned short)cur.d6);
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            // operand B: levels 16 kh .. + 16 of block j of weight row r
-            i32x4 wop;
-            if constexpr (TYPE == MI355_Q8_0) {
-                wop = *(const i32x4 *)(s_w + r * WPAD + 32 * j + 16 * kh);
-            } else if constexpr (TYPE == MI355_Q4_0) {   // byte b of the block's 16: level b in the low nibble, level 16 + b in the high one
-                const u32x4 v = *(const u32x4 *)(s_w + r * WPAD + 16 * j);
+            for (int hf = 0; hf < 2; hf++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) wop[i] = (int)((v[i] >> (4 * kh)) & 0x0F0F0F0Fu);
-            } else {   // chunk j / 2: byte b of its 32: level b of sub-block 2 (j / 2) in the low nibble, of the next one in the high nibble
-                const u32x4 v = *(const u32x4 *)(s_w + r * WPAD + 32 * (j >> 1) + 16 * kh);
+                for (int is = 0; is < 2; is++) {
+                    const u32x2 qh8 = *(const u32x2 *)(s_qh + r * QHPAD + 32 * hf + 16 * is + 8 * kh);
 #pragma unroll
-                for (int i = 0; i < 4; i++) wop[i] = (int)((v[i] >> (4 * (j & 1))) & 0x0F0F0F0Fu);
+                    for (int qlo = 0; qlo < 2; qlo++) {
+                        const u32x2 ql8 = *(const u32x2 *)(s_w + r * WPAD + 64 * hf + 32 * qlo + 16 * is + 8 * kh);
+#pragma unroll
+                        for (int qhi = 0; qhi < 2; qhi++) {
+                            const int q = qlo + 2 * qhi;
+                            const int g = 8 * hf + 2 * q + is;   // scale index = position of the group in the super-block
+                            u32x2 lv;
+#pragma unroll
+                            for (int i = 0; i < 2; i++) lv[i] = ((ql8[i] >> (4 * qhi)) & 0x0F0F0F0Fu) | (((qh8[i] >> (2 * q)) & 0x03030303u) << 4);
+                            const u32x2 a8 = *(const u32x2 *)(s_a + am * SK_APAD + 128 * hf + 32 * q + 16 * is + 8 * kh);
+                            i32x16 z;
+#pragma unroll
+                            for (int i = 0; i < 16; i++) z[i] = 0;
+                            const i32x16 D = __builtin_amdgcn_mfma_i32_32x32x16_i8(__builtin_bit_cast(long, a8), __builtin_bit_cast(long, lv), z, 0, 0, 0);
+                            const u32 sc_word = cur.hdr[g >> 2];
+                            const float wsg = d * (float)(int)(signed char)((sc_word >> (8 * (g & 3))) & 0xFFu);
+#pragma unroll
+                            for (int qq = 0; qq < NI; qq++) {
+                                const float4 *e = (const float4 *)(s_t + (4 * hf + q) * (8 * NI) + 8 * qq + 4 * kh);
+                                const float4 e01 = e[0], e23 = e[1];
+                                const float dd[4] = {e01.x, e01.z, e23.x, e23.z};
+                                const i32x4 gs = *(const i32x4 *)(s_g + g * (8 * NI) + 8 * qq + 4 * kh);
+#pragma unroll
+                                for (int i = 0; i < 4; i++) acc[qq][i] = __builtin_fmaf(wsg, dd[i] * (float)(D[4 * qq + i] - 32 * gs[i]), acc[qq][i]);
+                            }
+                        }
+                    }
+                }
+        } else {
+            // ---- per-block weight scales of this lane's row
+            float ws[8], wm[8];
+            if constexpr (TYPE == MI355_Q4_K) {
+                const float d = half_bits_to_float((unsigned short)(cur.hdr[0] & 0xFFFFu));
+                const float dmin = half_bits_to_float((unsigned short)(cur.hdr[0] >> 16));
+    #pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    int sc, mn;
+                    q4k_scale_min(cur.hdr[1], cur.hdr[2], cur.hdr[3], j, sc, mn);
+                    ws[j] = d * (float)sc;
+                    wm[j] = -(dmin * (float)mn);
+                }
+            } else {
+    #pragma unroll
+                for (int j = 0; j < 8; j++) ws[j] = f16_of(cur.hdr, j);
             }
-            const i32x4 aop = *(const i32x4 *)(s_a + am * SK_APAD + 32 * j + 16 * kh);
-            i32x16 z;
-#pragma unroll
-            for (int i = 0; i < 16; i++) z[i] = 0;
-            const i32x16 D = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, wop, z, 0, 0, 0);
-#pragma unroll
-            for (int q = 0; q < NI; q++) {
-                const float4 *e = (const float4 *)(s_t + j * (8 * NI) + 8 * q + 4 * kh);
-                const float4 e01 = e[0], e23 = e[1];
-                const float dd[4] = {e01.x, e01.z, e23.x, e23.z};
-                const float xx[4] = {e01.y, e01.w, e23.y, e23.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float Df = (float)D[4 * q + i];
-                    if constexpr (TYPE == MI355_Q4_0) {
-                        acc[q][i] = __builtin_fmaf(ws[j], __builtin_fmaf(dd[i], Df, xx[i]), acc[q][i]);   // x = -8 d sum
-                    } else if constexpr (TYPE == MI355_Q8_0) {
-                        acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);
-                    } else {
-                        acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);
-                        acc[q][i] = __builtin_fmaf(wm[j], xx[i], acc[q][i]);                              // x = d sum
+    #pragma unroll
+            for (int j = 0; j < 8; j++) {
+                // operand B: levels 16 kh .. + 16 of block j of weight row r
+                i32x4 wop;
+                if constexpr (TYPE == MI355_Q8_0) {
+                    wop = *(const i32x4 *)(s_w + r * WPAD + 32 * j + 16 * kh);
+                } else if constexpr (TYPE == MI355_Q4_0) {   // byte b of the block's 16: level b in the low nibble, level 16 + b in the high one
+                    const u32x4 v = *(const u32x4 *)(s_w + r * WPAD + 16 * j);
+    #pragma unroll
+                    for (int i = 0; i < 4; i++) wop[i] = (int)((v[i] >> (4 * kh)) & 0x0F0F0F0Fu);
+                } else {   // chunk j / 2: byte b of its 32: level b of sub-block 2 (j / 2) in the low nibble, of the next one in the high nibble
+                    const u32x4 v = *(const u32x4 *)(s_w + r * WPAD + 32 * (j >> 1) + 16 * kh);
+    #pragma unroll
+                    for (int i = 0; i < 4; i++) wop[i] = (int)((v[i] >> (4 * (j & 1))) & 0x0F0F0F0Fu);
+                }
+                const i32x4 aop = *(const i32x4 *)(s_a + am * SK_APAD + 32 * j + 16 * kh);
+                i32x16 z;
+    #pragma unroll
+                for (int i = 0; i < 16; i++) z[i] = 0;
+                const i32x16 D = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, wop, z, 0, 0, 0);
+    #pragma unroll
+                for (int q = 0; q < NI; q++) {
+                    const float4 *e = (const float4 *)(s_t + j * (8 * NI) + 8 * q + 4 * kh);
+                    const float4 e01 = e[0], e23 = e[1];
+                    const float dd[4] = {e01.x, e01.z, e23.x, e23.z};
+                    const float xx[4] = {e01.y, e01.w, e23.y, e23.w};
+    #pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float Df = (float)D[4 * q + i];
+                        if constexpr (TYPE == MI355_Q4_0) {
+                            acc[q][i] = __builtin_fmaf(ws[j], __builtin_fmaf(dd[i], Df, xx[i]), acc[q][i]);   // x = -8 d sum
+                        } else if constexpr (TYPE == MI355_Q8_0) {
+                            acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);
+                        } else {
+                            acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);
+                            acc[q][i] = __builtin_fmaf(wm[j], xx[i], acc[q][i]);                              // x = d sum
+                        }
                     }
                 }
             }
@@ -299,7 +375,7 @@ using namespace mi355;
 extern "C" {
 
 int mi355_mul_mat_skinny_supported(int type, const void *W, int64_t K, int64_t B) {
-    return (type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K) && B >= 1 && B <= 32 && K > 0 && K % 256 == 0 && K < (int64_t(1) << 30) &&
+    return is_weight_type(type) && B >= 1 && B <= 32 && K > 0 && K % 256 == 0 && K < (int64_t(1) << 30) &&
            layout_aligned(W, make_row_layout(type, K));
 }
 
@@ -322,7 +398,8 @@ int mi355_mul_mat_skinny(void *stream, int type, const void *W, const void *act,
     switch (type) {
         case MI355_Q4_0: launch_skinny_nt<MI355_Q4_0>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
         case MI355_Q8_0: launch_skinny_nt<MI355_Q8_0>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
-        default: launch_skinny_nt<MI355_Q4_K>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
+        case MI355_Q4_K: launch_skinny_nt<MI355_Q4_K>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
+        default: launch_skinny_nt<MI355_Q6_K>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
     }
     return launch_status("k_mm_skinny");
 }
