@@ -1,6 +1,6 @@
-// MUL_MAT host entry: quantize activations to Q8_1 on the device, then dispatch to the
-// GEMV (B <= 8) or the int8-MFMA tile kernel (B > 8).  Also the byte-load fallback for weight
-// rows that are not 16-byte aligned.
+// MUL_MAT host entry: quantize activations on the device, then dispatch to the GEMV (few activation rows), the
+// weight-streaming matrix-core kernel (up to 32 rows) or the int8-MFMA tile kernels.  Also the byte-load fallback for
+// weight rows that are not 16-byte aligned.
 #include "common.hpp"
 #include "qdot.hpp"
 
@@ -51,11 +51,11 @@ extern "C" {
 // the per-super-block activation format of the K-quant tile kernel is smaller than the Q8_1 one
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B) { return (mi355_act_bytes(K, B) + 255) & ~(size_t)255; }
 
-// 5..32 activation rows: the weight-streaming matrix-core kernel (skinny.hip) where it supports the product.
+// 4 or 5 (Q6_K) to 32 activation rows: the weight-streaming matrix-core kernel (skinny.hip) where it supports the product.
 // MI355_NO_SKINNY=1 sends these batches to the batch-1 kernels (up to 8) and the tile kernels as before (tuning aid).
 static bool use_skinny(int type, const void *W, int64_t K, int64_t B) {
     static const bool off = getenv("MI355_NO_SKINNY") != nullptr;
-    return !off && B >= 5 && B <= 32 && mi355_mul_mat_skinny_supported(type, W, K, B);
+    return !off && B >= (type == MI355_Q6_K ? 5 : 4) && B <= 32 && mi355_mul_mat_skinny_supported(type, W, K, B);
 }
 
 static bool use_q8k_tiles(int type, const void *W, int64_t K, int64_t B) {

@@ -41,7 +41,10 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-constexpr int SK_APAD = 256 + 16;   // LDS row strides (+16: rows 32 apart in banks do not all collide)
+constexpr int SK_APAD = 256 + 16;
+#ifndef SK_AHEAD_MAX_NI
+#define SK_AHEAD_MAX_NI 2
+#endif   // LDS row strides (+16: rows 32 apart in banks do not all collide)
 
 __device__ __forceinline__ float f16_of(const u32x4 &v, int j) {   // j is a compile-time constant after unrolling
     const u32 u = v[j >> 1];
@@ -154,11 +157,19 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[q][i] = 0.0f;
 
+    // up to 16 activation rows the next step's loads are requested before the current step is contracted; beyond, a second
+    // set of load registers would halve the number of resident waves, which hide the latency better than the wave itself
+    constexpr bool AHEAD = NI <= SK_AHEAD_MAX_NI;
     R nxt;
-    fetch(s_lo, nxt);
+    if constexpr (AHEAD) fetch(s_lo, nxt);
     for (int step = s_lo; step < s_hi; step++) {
-        R cur = nxt;
-        if (step + 1 < s_hi) fetch(step + 1, nxt);
+        R cur;
+        if constexpr (AHEAD) {
+            cur = nxt;
+            if (step + 1 < s_hi) fetch(step + 1, nxt);
+        } else {
+            fetch(step, cur);
+        }
         // ---- registers -> the wave's LDS
 #pragma unroll
         for (int u = 0; u < R::NW; u++) *(u32x4 *)(s_w + (w_row + u * RPL) * WPAD + 16 * w_piece) = cur.w[u];
@@ -239,12 +250,16 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
             if constexpr (TYPE == MI355_Q4_K) {
                 const float d = half_bits_to_float((unsigned short)(cur.hdr[0] & 0xFFFFu));
                 const float dmin = half_bits_to_float((unsigned short)(cur.hdr[0] >> 16));
-    #pragma unroll
+                    // all eight 6-bit (scale, min) pairs at once, as the bytes of four words (get_scale_min_k4, ggml-quants.c:631-638)
+                const u32 u0 = cur.hdr[1], u1 = cur.hdr[2], u2 = cur.hdr[3];
+                const u32 s_lo = u0 & 0x3F3F3F3Fu, m_lo = u1 & 0x3F3F3F3Fu;
+                const u32 s_hi = (u2 & 0x0F0F0F0Fu) | (((u0 >> 6) & 0x03030303u) << 4);
+                const u32 m_hi = ((u2 >> 4) & 0x0F0F0F0Fu) | (((u1 >> 6) & 0x03030303u) << 4);
+#pragma unroll
                 for (int j = 0; j < 8; j++) {
-                    int sc, mn;
-                    q4k_scale_min(cur.hdr[1], cur.hdr[2], cur.hdr[3], j, sc, mn);
-                    ws[j] = d * (float)sc;
-                    wm[j] = -(dmin * (float)mn);
+                    const u32 S = j < 4 ? s_lo : s_hi, M = j < 4 ? m_lo : m_hi;
+                    ws[j] = d * (float)((S >> (8 * (j & 3))) & 0xFFu);
+                    wm[j] = -(dmin * (float)((M >> (8 * (j & 3))) & 0xFFu));
                 }
             } else {
     #pragma unroll
