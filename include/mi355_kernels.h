@@ -75,8 +75,9 @@ int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64
  * ggml_compute_forward_mul_mat (ggml/src/ggml-cpu/ggml-cpu.c:7443-7635) for quantized
  * src0 and f32 src1:  dst[b*dst_stride + n] = sum_k W[n][k] * x[b*x_stride + k].
  * W: N rows of K elements of `type` in device layout.  x, dst f32.
- * B <= 8 runs the bandwidth-bound GEMV (per-block integer dots of the weights against
- * Q8_1 activations); larger B runs the int8-MFMA tile kernel.
+ * Up to 4 activation rows (8 where the matrix-core kernels do not support the product) run the
+ * bandwidth-bound GEMV (per-block integer dots of the weights against Q8_1 activations), up to 32
+ * the weight-streaming matrix-core kernel (mi355_mul_mat_skinny), larger B the int8-MFMA tile kernels.
  * `ws` is scratch of at least mi355_mul_mat_ws_bytes(K, B) bytes. */
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
@@ -154,7 +155,8 @@ int mi355_mul_mat_q8k_planes_ws(void *stream, int type, const void *planes, cons
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE
  * launch, each optionally adding a residual in its epilogue (the ggml_add that follows the wo and
  * ffn_down products, src/llama.cpp:1566, :1609): dst_i[b][n] = W_i[n] . x[b] (+ residual_i[b][n]).
- * residual has dst's shape and stride and may alias dst.  B <= 8. */
+ * residual has dst's shape and stride and may alias dst.  B <= 8; up to 32 where every matrix qualifies for
+ * mi355_mul_mat_skinny, which this call then uses from five activation rows on (one launch per matrix). */
 typedef struct mi355_gemv_mat {
     int          type;        /* weight type of this matrix */
     const void  *W;           /* N rows x K, device layout */

@@ -812,12 +812,13 @@ struct graph_walk {
 };
 
 bool is_quant_gemv_candidate(const ggml_tensor * mm) {
-    // quantized weights in 16-byte aligned rows, one 2-D activation matrix of at most 8 contiguous rows
+    // quantized weights in 16-byte aligned rows, one 2-D activation matrix of at most 32 contiguous rows (up to 4: the batch-1
+    // kernels; from there to 32: the weight-streaming matrix-core kernel)
     const ggml_tensor * a = mm->src[0];
     const ggml_tensor * b = mm->src[1];
     if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
-    if (b->ne[1] > 8 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
+    if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
     const int64_t K = a->ne[0];
     if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)
@@ -829,7 +830,7 @@ bool is_q8k_tile_candidate(const ggml_tensor * mm) {
     const ggml_tensor * b = mm->src[1];
     if (mm->op != GGML_OP_MUL_MAT || (a->type != GGML_TYPE_Q4_K && a->type != GGML_TYPE_Q6_K)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
-    if (b->ne[1] <= 8 || b->nb[1] % 16 != 0) return false;
+    if (b->ne[1] <= 32 || b->nb[1] % 16 != 0) return false;
     const int64_t K = a->ne[0];
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;
     return ((uintptr_t) a->data & 15) == 0 && ((uintptr_t) b->data & 15) == 0;
@@ -1282,7 +1283,8 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             }
         }
     }
-    // ---- runs of quantized products on one activation (batch <= 8): one quantization, multi-matrix GEMV, residual epilogue
+    // ---- runs of quantized products on one activation (batch <= 32): one quantization, multi-matrix GEMV (up to 4 rows) or the
+    //      weight-streaming kernel, residual epilogue
     if (is_quant_gemv_candidate(node)) {
         const ggml_tensor * b = node->src[1];
         const int64_t K = b->ne[0], B = b->ne[1];
@@ -1323,7 +1325,15 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 }
             }
         }
-        MI355_K_OK(mi355_mul_mat_vec_q_multi(s, n_run, mats, act, K, B));
+        if (n_run == 1 && B >= 5 && mi355_mul_mat_skinny_supported(mats[0].type, mats[0].W, K, B)) {
+            // with room for the slices along K that products with few rows are split into
+            const size_t split_bytes = mi355_mul_mat_skinny_ws_bytes(mats[0].N, K, B);
+            void * split_ws = split_bytes ? ctx->workspace(split_bytes) : nullptr;
+            MI355_K_OK(mi355_mul_mat_skinny(s, mats[0].type, mats[0].W, act, mats[0].dst, mats[0].residual, mats[0].N, K, B, mats[0].dst_stride, split_ws,
+                                            split_bytes));
+        } else {
+            MI355_K_OK(mi355_mul_mat_vec_q_multi(s, n_run, mats, act, K, B));
+        }
         for (int r = 0; r < n_run; r++) ctx->note_write(mats[r].dst, (size_t) mats[r].N * (size_t) B * sizeof(float));
         return last;
     }

@@ -485,7 +485,7 @@ int mi355_mul_mat_vec_q(void *stream, int type, const void *W, const void *act, 
 
 int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B) {
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 4, "mul_mat_vec_q_multi: 1..4 matrices per launch, got %d", n_mats);
-    MI355_REQUIRE(B >= 1 && B <= 8, "mul_mat_vec_q: batch %lld outside 1..8", (long long)B);
+    MI355_REQUIRE(B >= 1 && B <= 32, "mul_mat_vec_q: batch %lld outside 1..32", (long long)B);
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_vec_q: activation workspace is not 16-byte aligned");
     int64_t total_rows = 0;
     bool aligned = true;
@@ -520,6 +520,7 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
             return MI355_OK;
         }
     }
+    MI355_REQUIRE(B <= 8, "mul_mat_vec_q: batch %lld needs the matrix-core kernel, which does not support this product (K a multiple of 256, aligned rows)", (long long)B);
     int rpw = pick_rpw(total_rows);
     if (B > 4 && rpw > 2) rpw = 2;   // keep the accumulator tile in registers
     if (getenv("MI355_GEMV_RPW") == nullptr && getenv("MI355_GEMV_PLAIN_RPW") == nullptr) {   // per-type corrections, measured on the 8B shapes (off under either tuning variable)

@@ -61,4 +61,4 @@ def test_argument_errors_are_reported_not_crashed():
     assert lib.mi355_mul_mat_vec_q(None, 3, None, None, None, 16, 256, 1, 16) == -1
     assert b"unsupported" in lib.mi355_last_error()
     assert lib.mi355_mul_mat_vec_q(None, 12, None, None, None, 16, 100, 1, 16) == -1
-    assert lib.mi355_mul_mat_vec_q(None, 12, None, None, None, 16, 256, 9, 16) == -1
+    assert lib.mi355_mul_mat_vec_q(None, 12, None, None, None, 16, 256, 33, 16) == -1
