@@ -1,4 +1,4 @@
-// MUL_MAT for a handful of activation rows (5 .. 32): weight-streaming kernel on the int8 matrix cores.
+// MUL_MAT for a handful of activation rows (4 .. 32): weight-streaming kernel on the int8 matrix cores.
 //
 // The batch-1 kernels (gemv.hip) spend eight v_dot4 per weight block and activation row, which binds them to the vector
 // ALUs from about five activation rows on; the tile kernels (mmq.hip, mmq_k.hip) are built around 64..128-row activation
@@ -24,10 +24,10 @@ namespace mi355 {
 namespace {
 
 template <int TYPE> struct sk_traits;
-template <> struct sk_traits<MI355_Q4_0> { static constexpr int ROW_BYTES = 128, W_LOADS = 8; };    // per step and weight row
-template <> struct sk_traits<MI355_Q8_0> { static constexpr int ROW_BYTES = 256, W_LOADS = 16; };
-template <> struct sk_traits<MI355_Q4_K> { static constexpr int ROW_BYTES = 128, W_LOADS = 8; };    // qs only; the header goes to registers
-template <> struct sk_traits<MI355_Q6_K> { static constexpr int ROW_BYTES = 128, W_LOADS = 8; };    // ql; qh (64 bytes) is copied beside it
+template <> struct sk_traits<MI355_Q4_0> { static constexpr int ROW_BYTES = 128; };    // bytes copied to LDS per step and weight row
+template <> struct sk_traits<MI355_Q8_0> { static constexpr int ROW_BYTES = 256; };
+template <> struct sk_traits<MI355_Q4_K> { static constexpr int ROW_BYTES = 128; };    // qs only; the header goes to registers
+template <> struct sk_traits<MI355_Q6_K> { static constexpr int ROW_BYTES = 128; };    // ql; qh (64 bytes) is copied beside it
 
 // Orders a wave's own LDS accesses around the point where its lanes exchange data through LDS: the hardware completes
 // them in program order, so all that is needed is that neither the compiler nor the instruction scheduler moves an access
@@ -41,10 +41,8 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-constexpr int SK_APAD = 256 + 16;
-#ifndef SK_AHEAD_MAX_NI
-#define SK_AHEAD_MAX_NI 2
-#endif   // LDS row strides (+16: rows 32 apart in banks do not all collide)
+constexpr int SK_APAD = 256 + 16;      // LDS row strides (+16: rows 32 apart in banks do not all collide)
+constexpr int SK_AHEAD_MAX_NI = 2;     // load-ahead up to 16 activation rows (see the K loop)
 
 __device__ __forceinline__ float f16_of(const u32x4 &v, int j) {   // j is a compile-time constant after unrolling
     const u32 u = v[j >> 1];
