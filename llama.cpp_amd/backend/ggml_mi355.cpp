@@ -818,7 +818,8 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
     const ggml_tensor * b = mm->src[1];
     if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
-    if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
+    static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;
+    if (b->ne[1] > (no_skinny ? 8 : 32) || b->nb[1] != b->ne[0] * sizeof(float)) return false;
     const int64_t K = a->ne[0];
     if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)
@@ -830,7 +831,8 @@ bool is_q8k_tile_candidate(const ggml_tensor * mm) {
     const ggml_tensor * b = mm->src[1];
     if (mm->op != GGML_OP_MUL_MAT || (a->type != GGML_TYPE_Q4_K && a->type != GGML_TYPE_Q6_K)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
-    if (b->ne[1] <= 32 || b->nb[1] % 16 != 0) return false;
+    static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;
+    if (b->ne[1] <= (no_skinny ? 8 : 32) || b->nb[1] % 16 != 0) return false;
     const int64_t K = a->ne[0];
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;
     return ((uintptr_t) a->data & 15) == 0 && ((uintptr_t) b->data & 15) == 0;
@@ -1325,7 +1327,8 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 }
             }
         }
-        if (n_run == 1 && B >= 5 && mi355_mul_mat_skinny_supported(mats[0].type, mats[0].W, K, B)) {
+        static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;   // tuning aid, as in the kernel library
+        if (n_run == 1 && B >= 5 && !no_skinny && mi355_mul_mat_skinny_supported(mats[0].type, mats[0].W, K, B)) {
             // with room for the slices along K that products with few rows are split into
             const size_t split_bytes = mi355_mul_mat_skinny_ws_bytes(mats[0].N, K, B);
             void * split_ws = split_bytes ? ctx->workspace(split_bytes) : nullptr;
