@@ -6,7 +6,7 @@
 // rows and one quarter of K and never waits for another wave until the end:
 //   * per step of 256 elements the wave copies its weights (32 rows), activation rows and activation scales to its own
 //     part of LDS with fully coalesced 16-byte loads (a lane reads along a row; the loads of the next step are requested
-//     before the current one is contracted), and reads them back in matrix-core operand order.  Nobody else touches that
+//     as soon as the registers are free, before the current step is contracted), and reads them back in matrix-core operand order.  Nobody else touches that
 //     part of LDS, and a wave's LDS accesses complete in program order, so no barrier is involved;
 //   * one v_mfma_i32_32x32x32_i8 per weight block: operand A = 16 levels of an activation row per lane (lane % 32 = row,
 //     lane / 32 = half of the block), operand B = 16 levels of a weight row per lane;
@@ -42,7 +42,6 @@ __device__ __forceinline__ void wave_lds_sync() {
 }
 
 constexpr int SK_APAD = 256 + 16;      // LDS row strides (+16: rows 32 apart in banks do not all collide)
-constexpr int SK_AHEAD_MAX_NI = 2;     // load-ahead up to 16 activation rows (see the K loop)
 
 __device__ __forceinline__ float f16_of(const u32x4 &v, int j) {   // j is a compile-time constant after unrolling
     const u32 u = v[j >> 1];
@@ -128,9 +127,10 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
         t_src[u] = ads + (int64_t)c * nblk + 2 * t_piece;
     }
 
+    // loads of one step into the register set `g`
     auto fetch = [&](int step, R &g) {
         const int s = step < nsteps ? step : nsteps - 1;
-        const int64_t w_off = TYPE == MI355_Q8_0 ? (int64_t)s * 256 : TYPE == MI355_Q4_K ? (int64_t)s * Q4_K_BYTES : (int64_t)s * 128;
+        const int w_off = s * (TYPE == MI355_Q8_0 ? 256 : TYPE == MI355_Q4_K ? Q4_K_BYTES : 128);   // < 2^31: rows are shorter than that
 #pragma unroll
         for (int u = 0; u < R::NW; u++) g.w[u] = load16(w_src[u] + w_off);
         if constexpr (TYPE == MI355_Q4_K) {
@@ -155,19 +155,11 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[q][i] = 0.0f;
 
-    // up to 16 activation rows the next step's loads are requested before the current step is contracted; beyond, a second
-    // set of load registers would halve the number of resident waves, which hide the latency better than the wave itself
-    constexpr bool AHEAD = NI <= SK_AHEAD_MAX_NI;
-    R nxt;
-    if constexpr (AHEAD) fetch(s_lo, nxt);
+    // One set of load registers: as soon as a step's loads have been copied to LDS, the same registers take the next step's
+    // loads, which are then in flight while this step is contracted.  Only the weight scales of the lane's row stay behind.
+    R cur;
+    fetch(s_lo, cur);
     for (int step = s_lo; step < s_hi; step++) {
-        R cur;
-        if constexpr (AHEAD) {
-            cur = nxt;
-            if (step + 1 < s_hi) fetch(step + 1, nxt);
-        } else {
-            fetch(step, cur);
-        }
         // ---- registers -> the wave's LDS
 #pragma unroll
         for (int u = 0; u < R::NW; u++) *(u32x4 *)(s_w + (w_row + u * RPL) * WPAD + 16 * w_piece) = cur.w[u];
@@ -200,14 +192,17 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
                 }
             }
         }
+        const u32x4 hdr = cur.hdr;
+        const u32 d6 = cur.d6;
         wave_lds_sync();
+        if (step + 1 < s_hi) fetch(step + 1, cur);
 
         const int am = r < 8 * NI ? r : r & 7;   // operand rows past the copied ones repeat copied ones; their results are not used
         if constexpr (Q6) {
             // 16 groups of 16 levels, each with its own int8 scale: one v_mfma_i32_32x32x16_i8 per group (8 levels per lane).
             // Group (hf, q, is): levels 128 hf + 32 q + 16 is .. + 16; level l of it = nibble q / 2 of ql byte 64 hf + 32 (q % 2) + 16 is + l
             // plus bits 2q, 2q + 1 of qh byte 32 hf + 16 is + l, minus 32 (dequantize_row_q6_K, ggml/src/ggml-quants.c:1690-1719).
-            const float d = half_bits_to_float((unsigned short)cur.d6);
+            const float d = half_bits_to_float((unsigned short)d6);
 #pragma unroll
             for (int hf = 0; hf < 2; hf++)
 #pragma unroll
@@ -228,7 +223,7 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
 #pragma unroll
                             for (int i = 0; i < 16; i++) z[i] = 0;
                             const i32x16 D = __builtin_amdgcn_mfma_i32_32x32x16_i8(__builtin_bit_cast(long, a8), __builtin_bit_cast(long, lv), z, 0, 0, 0);
-                            const u32 sc_word = cur.hdr[g >> 2];
+                            const u32 sc_word = hdr[g >> 2];
                             const float wsg = d * (float)(int)(signed char)((sc_word >> (8 * (g & 3))) & 0xFFu);
 #pragma unroll
                             for (int qq = 0; qq < NI; qq++) {
@@ -246,10 +241,10 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
             // ---- per-block weight scales of this lane's row
             float ws[8], wm[8];
             if constexpr (TYPE == MI355_Q4_K) {
-                const float d = half_bits_to_float((unsigned short)(cur.hdr[0] & 0xFFFFu));
-                const float dmin = half_bits_to_float((unsigned short)(cur.hdr[0] >> 16));
+                const float d = half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu));
+                const float dmin = half_bits_to_float((unsigned short)(hdr[0] >> 16));
                     // all eight 6-bit (scale, min) pairs at once, as the bytes of four words (get_scale_min_k4, ggml-quants.c:631-638)
-                const u32 u0 = cur.hdr[1], u1 = cur.hdr[2], u2 = cur.hdr[3];
+                const u32 u0 = hdr[1], u1 = hdr[2], u2 = hdr[3];
                 const u32 s_lo = u0 & 0x3F3F3F3Fu, m_lo = u1 & 0x3F3F3F3Fu;
                 const u32 s_hi = (u2 & 0x0F0F0F0Fu) | (((u0 >> 6) & 0x03030303u) << 4);
                 const u32 m_hi = ((u2 >> 4) & 0x0F0F0F0Fu) | (((u1 >> 6) & 0x03030303u) << 4);
@@ -261,7 +256,7 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
                 }
             } else {
     #pragma unroll
-                for (int j = 0; j < 8; j++) ws[j] = f16_of(cur.hdr, j);
+                for (int j = 0; j < 8; j++) ws[j] = f16_of(hdr, j);
             }
     #pragma unroll
             for (int j = 0; j < 8; j++) {
