@@ -6,8 +6,9 @@
 // rows and one quarter of K and never waits for another wave until the end:
 //   * per step of 256 elements the wave copies its weights (32 rows), activation rows and activation scales to its own
 //     part of LDS with fully coalesced 16-byte loads (a lane reads along a row; the loads of the next step are requested
-//     as soon as the registers are free, before the current step is contracted), and reads them back in matrix-core operand order.  Nobody else touches that
-//     part of LDS, and a wave's LDS accesses complete in program order, so no barrier is involved;
+//     as soon as the registers are free, before the current step is contracted), and reads them back in matrix-core
+//     operand order.  Nobody else touches that part of LDS, and a wave's LDS accesses complete in program order, so no
+//     barrier is involved;
 //   * one v_mfma_i32_32x32x32_i8 per weight block: operand A = 16 levels of an activation row per lane (lane % 32 = row,
 //     lane / 32 = half of the block), operand B = 16 levels of a weight row per lane;
 //   * the result puts ONE weight row (lane % 32) and activation rows 4 (lane / 32) + 8 q + 0..3 (q = 0..3) in a lane:
