@@ -152,9 +152,12 @@ def sweep(kinds):
                              achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
                         del planes
                     del Ws
-    if "fattn" in kinds:
+    if "fattn" in kinds or "fattn_long" in kinds:
         H, HK, D = 32, 8, 128
-        for Nq, Nkv in [(1, 512), (1, 4096), (1, 32768), (1, 131072), (512, 512), (512, 4096), (2048, 2048), (4096, 4096)]:
+        cases = [(1, 512), (1, 4096), (1, 32768), (1, 131072), (512, 512), (512, 4096), (2048, 2048), (4096, 4096)]
+        if "fattn" not in kinds:
+            cases = [(1, 131072)]   # the long-context decode kernel alone (for counter collection)
+        for Nq, Nkv in cases:
             nrot = max(2, min(16, (1 << 30) // (Nkv * HK * D * 4))) if Nq == 1 else 1
             q = torch.randn(Nq, H, D, device=dev, generator=gen)
             ks = [torch.randn(Nkv, HK, D, device=dev, generator=gen).half() for _ in range(nrot)]
@@ -191,7 +194,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
-    ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, fattn")
+    ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, fattn, fattn_long (decode over 131072 cells only)")
     args = ap.parse_args()
     if args.sweep:
         if args.gpus != 1:

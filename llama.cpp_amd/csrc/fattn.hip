@@ -370,7 +370,8 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
         // enough splits to put about two groups on every CU; a split is a whole number of 64-cell tiles
         const int64_t tiles = (Nkv + 63) / 64;
         const int64_t nt = 32 / R, base = Hkv * ((Nq + nt - 1) / nt);
-        int64_t n = 512 / base;
+        static const int64_t target_groups = getenv("MI355_FA_DEC_GROUPS") ? atoll(getenv("MI355_FA_DEC_GROUPS")) : 512;   // tuning aid
+        int64_t n = target_groups / base;
         if (n > tiles) n = tiles;
         if (n > 256) n = 256;
         if (n < 1) n = 1;
