@@ -106,7 +106,9 @@ __device__ __forceinline__ float mask_value(const u32x2 &w, int i) {
     return half_bits_to_float((unsigned short)((i < 2 ? w[0] : w[1]) >> (16 * (i & 1))));
 }
 
-// scale [+ softcap], add the mask, mark dropped cells with FM_NEG; returns the largest surviving score
+// scale [+ softcap], add the mask, mark dropped cells with FM_NEG; returns the largest surviving score.
+// A masked cell (-inf; slopes are positive) and a NaN score of a stale cell fail `s > FM_NEG` by themselves; the test against
+// the end of the range is made only in a tile that reaches past it (uniform over the group), on 32-bit offsets.
 __device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], const fattn_args &a, float scale, float slope,
                                                 int64_t c_first, int lhi, int64_t c_end) {
     if (a.softcap != 0.0f) {
@@ -117,18 +119,28 @@ __device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], 
         for (int r = 0; r < 16; r++) S[r] *= scale;
     }
     float mx = FM_NEG;
+    const int64_t room = c_end - c_first;
+    if (room >= 32) {   // every cell of this half tile lies inside the range
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const int64_t c = c_first + 8 * g + 4 * lhi;
+        for (int g = 0; g < 4; g++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float mv = mask_value(mw[g], i);
-            float s = S[4 * g + i] + slope * mv;
-            const bool valid = c + i < c_end && mv != -INFINITY && s > FM_NEG;   // NaN scores of stale cells drop out too
-            s = valid ? s : FM_NEG;
-            S[4 * g + i] = s;
-            mx = fmaxf(mx, s);
-        }
+            for (int i = 0; i < 4; i++) {
+                float s = S[4 * g + i] + slope * mask_value(mw[g], i);
+                s = s > FM_NEG ? s : FM_NEG;
+                S[4 * g + i] = s;
+                mx = fmaxf(mx, s);
+            }
+    } else {
+        const int left = (int)room - 4 * lhi;   // cells of the range from this lane's first one on (may be <= 0)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float s = S[4 * g + i] + slope * mask_value(mw[g], i);
+                s = (8 * g + i < left && s > FM_NEG) ? s : FM_NEG;
+                S[4 * g + i] = s;
+                mx = fmaxf(mx, s);
+            }
     }
     return mx;
 }
