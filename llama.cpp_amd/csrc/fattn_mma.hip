@@ -107,7 +107,7 @@ __device__ __forceinline__ float mask_value(const u32x2 &w, int i) {
 }
 
 // scale [+ softcap], add the mask, mark dropped cells with FM_NEG; returns the largest surviving score.
-// A masked cell (-inf; slopes are positive) and a NaN score of a stale cell fail `s > FM_NEG` by themselves; the test against
+// A masked cell (-inf; slopes are positive) and a NaN score of a stale cell both end as FM_NEG in fmaxf(s, FM_NEG); the test against
 // the end of the range is made only in a tile that reaches past it (uniform over the group), on 32-bit offsets.
 __device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], const fattn_args &a, float scale, float slope,
                                                 int64_t c_first, int lhi, int64_t c_end) {
@@ -126,7 +126,7 @@ __device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], 
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float s = S[4 * g + i] + slope * mask_value(mw[g], i);
-                s = s > FM_NEG ? s : FM_NEG;
+                s = fmaxf(s, FM_NEG);   // -inf and NaN become FM_NEG
                 S[4 * g + i] = s;
                 mx = fmaxf(mx, s);
             }
@@ -137,7 +137,7 @@ __device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], 
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float s = S[4 * g + i] + slope * mask_value(mw[g], i);
-                s = (8 * g + i < left && s > FM_NEG) ? s : FM_NEG;
+                s = 8 * g + i < left ? fmaxf(s, FM_NEG) : FM_NEG;
                 S[4 * g + i] = s;
                 mx = fmaxf(mx, s);
             }
@@ -309,12 +309,15 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
         if (__ballot(mx > FM_NEG) == 0) continue;   // every cell of the tile is masked for all 32 queries (wave-uniform)
         const float m_new = fmaxf(m, mx);
         const float alpha = __expf(m - m_new);
+        // dropped scores are exactly FM_NEG: exp(FM_NEG - m) is 0 for any real maximum; a column that has seen no cell yet
+        // (maximum still FM_NEG) subtracts 0 instead, so its dropped scores give 0 as well and not exp(0)
+        const float m_eff = m_new > FM_NEG ? m_new : 0.0f;
         float rs = 0.0f;
 #pragma unroll
         for (int u = 0; u < 2; u++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const float p = S[u][r] > FM_NEG ? __expf(S[u][r] - m_new) : 0.0f;
+                const float p = __expf(S[u][r] - m_eff);
                 S[u][r] = p;
                 rs += p;
             }
@@ -407,10 +410,13 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_half(fattn_args a) {
         if (__ballot(mx > FM_NEG) == 0) continue;   // all 32 cells masked for all 32 queries (wave-uniform; barriers are at the loop head)
         const float m_new = fmaxf(m, mx);
         const float alpha = __expf(m - m_new);
+        // dropped scores are exactly FM_NEG: exp(FM_NEG - m) is 0 for any real maximum; a column that has seen no cell yet
+        // (maximum still FM_NEG) subtracts 0 instead, so its dropped scores give 0 as well and not exp(0)
+        const float m_eff = m_new > FM_NEG ? m_new : 0.0f;
         float rs = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float p = S[r] > FM_NEG ? __expf(S[r] - m_new) : 0.0f;
+            const float p = __expf(S[r] - m_eff);
             S[r] = p;
             rs += p;
         }
@@ -550,10 +556,13 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_dec(fattn_args a, int R, i
         if (__ballot(mx > FM_NEG) == 0) return;   // all 32 cells masked for every column (wave-uniform)
         const float m_new = fmaxf(m, mx);
         const float alpha = __expf(m - m_new);
+        // dropped scores are exactly FM_NEG: exp(FM_NEG - m) is 0 for any real maximum; a column that has seen no cell yet
+        // (maximum still FM_NEG) subtracts 0 instead, so its dropped scores give 0 as well and not exp(0)
+        const float m_eff = m_new > FM_NEG ? m_new : 0.0f;
         float rs = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float p = S[r] > FM_NEG ? __expf(S[r] - m_new) : 0.0f;
+            const float p = __expf(S[r] - m_eff);
             S[r] = p;
             rs += p;
         }
