@@ -909,7 +909,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8K, true, act};
                 return j;
             }
-            if (rows <= 8 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
+            if (rows <= 32 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
             MI355_K_OK(mi355_rms_norm_mul_quant(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
             ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
             return j;
@@ -949,7 +949,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                     ctx->cache = act_cache{mul->data, K, rows, ACT_Q8K, true, act};
                     return jm;
                 }
-                if (rows <= 8 && (feeds_quant_gemv(w, jm, mul->data, K, rows) || feeds_quant_mmid(w, jm, mul->data, K, rows)))
+                if ((rows <= 32 && feeds_quant_gemv(w, jm, mul->data, K, rows)) || (rows <= 8 && feeds_quant_mmid(w, jm, mul->data, K, rows)))
                     act = ctx->act_slot(mi355_act_bytes(K, rows));
                 MI355_K_OK(mi355_swiglu_quant(s, (const float *) gt->data, (const float *) up->data, K, (float *) mul->data, K, act, K, rows));
                 ctx->cache = act_cache{mul->data, K, rows, ACT_Q8_1, act != nullptr, act};
