@@ -330,6 +330,17 @@ int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, c
                          int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
                          float beta_fast, float beta_slow);
 
+/* The same for ONE activation row, with the RMS_NORM -> MUL(norm weights) -> Q8_1 that precedes the projections in build_llama
+ * (llm_build_norm, src/llama.cpp:1506-1511; ggml_compute_forward_rms_norm_f32, ggml-cpu.c:6741-6805) done by every group for
+ * itself into its LDS copy of the activation: one launch less per decoded token and layer, bit-identical to
+ * mi355_rms_norm_mul_quant followed by mi355_qkv_rope_store.  x: the f32 layer input (K elements), K <= 4096 and a multiple of
+ * 1024; x and norm_w 16-byte aligned. */
+int mi355_rms_norm_qkv_rope_store(void *stream, const float *x, const float *norm_w, float eps, int type_q, const void *wq, int type_k,
+                                  const void *wk, int type_v, const void *wv, float *q, void *kcache, void *vcache, const int32_t *pos,
+                                  const int32_t *cells, const float *freq_factors, int64_t K, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
+                                  size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base,
+                                  float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow);
+
 /* The gate and up projections of llm_build_ffn (LLM_FFN_SILU, LLM_FFN_PAR; src/llama.cpp:280-320) in ONE bandwidth-bound launch that
  * also performs UNARY(SILU)(gate), MUL by up and the Q8_1 quantization the ffn_down product needs (ggml-cpu.c:6646-6683, 5142-5211;
  * quantize_row_q8_1_ref).  gate/up: f32 [B][out_stride] receive the raw products; act_out: mi355_quantize_act layout of B rows of N.

@@ -11,6 +11,7 @@
 // into one long enough to fill the chip.  An optional residual is added in the epilogue.
 #include "common.hpp"
 #include "qdot.hpp"
+#include "norm_quant.hpp"
 
 #include <math.h>
 #include <stdlib.h>
@@ -37,6 +38,8 @@ struct gemv_rope {
     const float *ff;         // frequency factors [n_dims/2] or null
     int D, n_dims;
     float theta_scale, freq_scale, ext_factor, attn_factor, corr0, corr1;
+    const float *nx, *nw;    // NORM: the f32 row to normalise and the norm weights (the group quantizes it into its LDS copy itself)
+    float neps;
 };
 
 // rope_yarn, same roundings as k_rope (glue.hip) and k_rope_kv_store (fused.hip); ggml-cpu.c:9268-9306
@@ -68,7 +71,7 @@ struct gemv_batch {
 // waves read it from there; otherwise every wave reads it from memory.  On the 14336 x 4096 Q4_K product the activation
 // reads of the 7168 waves (36 MB from L2) outweighed the 33 MB of weights and competed with them: 8.7 -> 7.9 us with the
 // copy in LDS.  The first step's weight loads are issued before the copy, so the copy's round trip hides behind them.
-template <int TYPE, int NCOLS, int RPW, bool QKV = false, bool COH = false, bool LDSA = false>
+template <int TYPE, int NCOLS, int RPW, bool QKV = false, bool COH = false, bool LDSA = false, bool NORM = false>
 __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const int8_t *__restrict__ aq,
                                           const act_ds *__restrict__ ads, int K, const gemv_rope *rp = nullptr, uint8_t *s_act = nullptr) {
     typedef wq<TYPE> T;
@@ -119,8 +122,13 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
         for (int r = 0; r < RPW; r++) w_first[r] = T::load_w(rows[r], L, c);
         int8_t *s_q = (int8_t *)s_act;
         act_ds *s_ds = (act_ds *)(s_act + NCOLS * K);
-        for (int i = threadIdx.x * 16; i < NCOLS * K; i += 256 * 16) *(u32x4 *)(s_q + i) = load16(aq + i);
-        for (int i = threadIdx.x; i < NCOLS * nblk; i += 256) s_ds[i] = ads[i];
+        if constexpr (NORM) {   // RMS_NORM -> MUL -> Q8_1 of the one activation row straight into the group's LDS copy
+            __shared__ float s_norm[4];
+            rms_norm_quant_row<4, false, false>(rp->nx, rp->nw, nullptr, s_act, 0, K, 1, rp->neps, s_norm);
+        } else {
+            for (int i = threadIdx.x * 16; i < NCOLS * K; i += 256 * 16) *(u32x4 *)(s_q + i) = load16(aq + i);
+            for (int i = threadIdx.x; i < NCOLS * nblk; i += 256) s_ds[i] = ads[i];
+        }
         __syncthreads();
         if (!wave_live) return;
         aq = s_q;
@@ -226,6 +234,23 @@ __global__ void __launch_bounds__(256) k_gemv_qkv(gemv_batch b, const int8_t *__
 template <int TYPE, int NCOLS, int RPW, bool LDSA>
 __global__ void __launch_bounds__(256) k_gemv_q(gemv_item m, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K) {
     gemv_body<TYPE, NCOLS, RPW, false, false, LDSA>(m, blockIdx.x, aq, ads, K, nullptr, s_act_dyn);
+}
+
+// ... with the RMS norm of the layer input computed by every group for itself (one activation row)
+__global__ void __launch_bounds__(256) k_gemv_qkv_norm(gemv_batch b, int K, gemv_rope rp) {
+    const int g = blockIdx.x;
+    int i = 0;
+#pragma unroll
+    for (int j = 1; j < 3; j++)
+        if (g >= b.it[j].first_group) i = j;
+    const gemv_item &m = b.it[i];
+    const int group = g - m.first_group;
+    switch (m.type) {
+        case MI355_Q4_0: gemv_body<MI355_Q4_0, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
+        case MI355_Q8_0: gemv_body<MI355_Q8_0, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
+        case MI355_Q4_K: gemv_body<MI355_Q4_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
+        default: gemv_body<MI355_Q6_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
+    }
 }
 
 // several matrices sharing one activation
@@ -582,15 +607,18 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     return launch_status("k_gemv_multi");
 }
 
-int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat *mats, const void *act, int64_t K, int64_t B,
-                             const mi355_rope_desc *rope) {
+// nx != null: one activation row that every group normalises and quantizes for itself (act is not read)
+static int vec_q_rope_impl(void *stream, int n_mats, const mi355_gemv_rope_mat *mats, const void *act, int64_t K, int64_t B,
+                             const mi355_rope_desc *rope, const float *nx, const float *nw, float neps) {
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr && rope != nullptr, "mul_mat_vec_q_rope: 1..3 matrices per launch");
     MI355_REQUIRE(B >= 1 && B <= 4, "mul_mat_vec_q_rope: batch %lld outside 1..4", (long long)B);
     const int64_t D = rope->head_dim;
     const int n_dims = rope->n_dims;
     MI355_REQUIRE(D > 0 && D % 2 == 0 && n_dims > 0 && n_dims <= D && n_dims % 2 == 0, "mul_mat_vec_q_rope: bad head geometry");
     MI355_REQUIRE(rope->mode == 0, "mul_mat_vec_q_rope: only the adjacent-pair rope mode is fused (mode %d)", rope->mode);
-    MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_vec_q_rope: activation workspace is not 16-byte aligned");
+    MI355_REQUIRE(nx != nullptr || ((uintptr_t)act & 15) == 0, "mul_mat_vec_q_rope: activation workspace is not 16-byte aligned");
+    MI355_REQUIRE(nx == nullptr || (B == 1 && K <= 4096 && K % 1024 == 0 && ((uintptr_t)nx & 15) == 0 && ((uintptr_t)nw & 15) == 0),
+                  "rms_norm_qkv_rope_store: one row of K <= 4096 (a multiple of 1024), 16-byte aligned x and weights");
     gemv_batch b;
     b.n = n_mats;
     int64_t groups = 0;
@@ -640,6 +668,12 @@ int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + B * K);
     const size_t lds = act_lds_bytes((int)B, K, groups);
+    if (nx != nullptr) {
+        rp.nx = nx; rp.nw = nw; rp.neps = neps;
+        hipLaunchKernelGGL(k_gemv_qkv_norm, dim3((unsigned)groups), dim3(256), (size_t)K + K / 4, s, b, (int)K, rp);
+        return launch_status("k_gemv_qkv_norm");
+    }
+    rp.nx = rp.nw = nullptr; rp.neps = 0.0f;
     switch (B) {
         case 1:
             if (lds) hipLaunchKernelGGL((k_gemv_qkv<1, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
@@ -659,6 +693,25 @@ int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat
             break;
     }
     return launch_status("k_gemv_qkv");
+}
+
+int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat *mats, const void *act, int64_t K, int64_t B,
+                             const mi355_rope_desc *rope) {
+    return vec_q_rope_impl(stream, n_mats, mats, act, K, B, rope, nullptr, nullptr, 0.0f);
+}
+
+int mi355_rms_norm_qkv_rope_store(void *stream, const float *x, const float *norm_w, float eps, int type_q, const void *wq, int type_k,
+                                  const void *wk, int type_v, const void *wv, float *q, void *kcache, void *vcache, const int32_t *pos,
+                                  const int32_t *cells, const float *freq_factors, int64_t K, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
+                                  size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base,
+                                  float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
+    MI355_REQUIRE(H > 0 && HK > 0 && D > 0 && x != nullptr && norm_w != nullptr, "rms_norm_qkv_rope_store: bad head geometry or missing operands");
+    mi355_gemv_rope_mat m[3];
+    m[0] = mi355_gemv_rope_mat{type_q, wq, H * D, MI355_EPI_ROPE, q, H * D, 0, 0};
+    m[1] = mi355_gemv_rope_mat{type_k, wk, HK * D, MI355_EPI_ROPE_CACHE, kcache, 0, (int64_t)k_nb1, (int64_t)k_nb2};
+    m[2] = mi355_gemv_rope_mat{type_v, wv, HK * D, MI355_EPI_CACHE, vcache, 0, (int64_t)v_nb1, (int64_t)v_nb2};
+    mi355_rope_desc r = {pos, cells, freq_factors, D, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow};
+    return vec_q_rope_impl(stream, 3, m, nullptr, K, 1, &r, x, norm_w, eps);
 }
 
 int mi355_qkv_rope_store(void *stream, int type_q, const void *wq, int type_k, const void *wk, int type_v, const void *wv, const void *act,

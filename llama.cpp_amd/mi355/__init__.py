@@ -66,6 +66,8 @@ _SIGNATURES = {
     "mi355_mul_mat_vec_q_rope": (_int, [_p, _int, _p, _p, _i64, _i64, _p]),
     "mi355_qkv_rope_store": (_int, [_p, _int, _p, _int, _p, _int, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64,
                                     _sz, _sz, _sz, _sz, _int, _int, _int, _f, _f, _f, _f, _f, _f]),
+    "mi355_rms_norm_qkv_rope_store": (_int, [_p, _p, _p, _f, _int, _p, _int, _p, _int, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64,
+                                             _sz, _sz, _sz, _sz, _int, _int, _int, _f, _f, _f, _f, _f, _f]),
     "mi355_block_dots_q8_1": (_int, [_p, _int, _p, _p, _p, _i64, _i64]),
     "mi355_mul_mat_id_ws_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_id": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),

@@ -145,6 +145,12 @@ def test_fused_layer_stack_matches_node_sequence(dev):
             c = run.forward(T, 256, last_only=False).cpu().numpy().copy()
             run.fuse_tail = not run.fuse_tail
             assert np.array_equal(b, c), (T, pos0)
+            # one token: the attention norm inside the Q/K/V launch, or as a launch of its own - same bits
+            run.fuse_qkv_norm = not run.fuse_qkv_norm
+            run.set_inputs(emb, pos0, T, 256)
+            c = run.forward(T, 256, last_only=False).cpu().numpy().copy()
+            run.fuse_qkv_norm = not run.fuse_qkv_norm
+            assert np.array_equal(b, c), (T, pos0)
         # Decode launches the same arithmetic in both sequences.  Prefill rounds the RMS norm differently in the
         # last bit, which flips a few activation levels; with one scale per 256 elements a single flip in a
         # row that holds an outlier moves that row by ~1e-5, and two random-weight layers amplify it.
