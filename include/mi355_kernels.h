@@ -83,6 +83,17 @@ size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
                   int64_t x_stride, int64_t dst_stride, void *ws, size_t ws_bytes);
 
+/* mi355_mul_mat for callers that cannot allocate device memory or bring a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The workspace is an array of
+ * mi355_mul_mat_static_max_ws() bytes (16 MiB) that lives inside the library, one copy per GPU that loads it, held until
+ * the process ends; the call performs no hipMalloc / hipFree and calls no allocating library routine.  Products whose
+ * quantized activation does not fit (mi355_mul_mat_ws_bytes(K, B) > the array, e.g. K = 14336 beyond B = 936) are rejected with
+ * MI355_ERR_WORKSPACE.  Same result as mi355_mul_mat with a workspace of that size.  Every call on one GPU shares that
+ * GPU's array: calls that overlap in time on one GPU (different streams or threads) race on it. */
+size_t mi355_mul_mat_static_max_ws(void);
+int mi355_mul_mat_static(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
+                         int64_t x_stride, int64_t dst_stride);
+
 /* The two halves of mi355_mul_mat for callers that reuse one quantized activation for
  * several weight matrices (Q/K/V or gate/up projections): `act` from mi355_quantize_act. */
 int mi355_mul_mat_vec_q(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,

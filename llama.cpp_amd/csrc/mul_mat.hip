@@ -4,6 +4,8 @@
 #include "common.hpp"
 #include "qdot.hpp"
 
+#include <atomic>
+
 namespace mi355 {
 
 // one wave per (row, activation row); any K that is a multiple of the block size
@@ -40,6 +42,32 @@ int gemv_unaligned(hipStream_t s, int type, const void *W, const void *act, floa
         default: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
     }
     return launch_status("k_gemv_unaligned");
+}
+
+// Scratch of the allocation-free entry point: one array per GPU that loads this library, kept until the process ends.
+// Host code never uses the array's name as an address (it is only a host-side handle): the device address is looked up
+// once per device with hipGetSymbolAddress and kept in g_scratch_ptr.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)16 << 20;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+static std::atomic<void *> g_scratch_ptr[MAX_DEVICES];
+
+// device address of this GPU's scratch array (the current device's); nullptr + error text on failure
+static void *static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        set_error("mul_mat_static: no current device");
+        return nullptr;
+    }
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+        set_error("mul_mat_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        return nullptr;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // every thread finds the same address for one device
+    return p;
 }
 
 }  // namespace mi355
@@ -85,6 +113,24 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
     if (use_skinny(type, W, K, B)) return mi355_mul_mat_skinny(stream, type, W, ws, dst, nullptr, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
     if (B <= 8) return mi355_mul_mat_vec_q(stream, type, W, ws, dst, N, K, B, dst_stride);
     return mi355_mul_mat_q_ws(stream, type, W, ws, dst, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
+}
+
+size_t mi355_mul_mat_static_max_ws(void) { return STATIC_SCRATCH_BYTES; }
+
+int mi355_mul_mat_static(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
+                         int64_t x_stride, int64_t dst_stride) {
+    MI355_REQUIRE(K > 0 && B > 0, "mul_mat_static: bad shape K=%lld B=%lld", (long long)K, (long long)B);
+    const size_t need = mi355_mul_mat_ws_bytes(K, B);
+    if (need > STATIC_SCRATCH_BYTES) {
+        set_error("mul_mat_static: K=%lld x B=%lld needs %zu bytes of scratch, the static array holds %zu; use mi355_mul_mat with a workspace",
+                  (long long)K, (long long)B, need, STATIC_SCRATCH_BYTES);
+        return MI355_ERR_WORKSPACE;
+    }
+    void *ws = static_scratch();
+    if (!ws) return MI355_ERR_HIP;
+    // Nothing in the workspace has to start at zero: the quantized activation and the K-slice partial sums are written in
+    // full by this call before anything reads them.
+    return mi355_mul_mat(stream, type, W, x, dst, N, K, B, x_stride, dst_stride, ws, STATIC_SCRATCH_BYTES);
 }
 
 }  // extern "C"

@@ -38,6 +38,8 @@ _SIGNATURES = {
     "mi355_quantize_act": (_int, [_p, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_ws_bytes": (_sz, [_i64, _i64]),
     "mi355_mul_mat": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_static_max_ws": (_sz, []),
+    "mi355_mul_mat_static": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_q_ws_bytes": (_sz, [_i64, _i64, _i64]),
@@ -222,6 +224,14 @@ def mul_mat(t, W, x, ws=None, split=True):
         ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     dst = torch.empty((B, N), dtype=torch.float32, device=x.device)
     check(load().mi355_mul_mat(_stream(), t, _ptr(W), _ptr(x), _ptr(dst), N, K, B, x.stride(0), N, _ptr(ws), ws.numel()))
+    return dst
+
+
+def mul_mat_static(t, W, x, dst):
+    """mi355_mul_mat on the library's own per-GPU scratch array: the call allocates nothing (dst comes from the caller)"""
+    B, K = x.shape
+    N = W.shape[0]
+    check(load().mi355_mul_mat_static(_stream(), t, _ptr(W), _ptr(x), _ptr(dst), N, K, B, x.stride(0), dst.stride(0)))
     return dst
 
 
