@@ -162,6 +162,27 @@ int mi355_mul_mat_q8k_planes(void *stream, int type, const void *planes, const v
 int mi355_mul_mat_q8k_planes_ws(void *stream, int type, const void *planes, const void *act, float *dst, const float *residual, int64_t N,
                                 int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
 
+/* Wide-tile form of the K-quant tile GEMM (128 weight rows x 128 activation rows per 512-thread group).  Both operands are
+ * *tile images*: an int8 matrix cut into tiles of 16 rows x 64 elements = 1 KiB, stored [row block][k block], each tile byte
+ * for byte what the kernel keeps in LDS, so that one wave-wide global-to-LDS transfer moves a tile.
+ *   activations: mi355_quantize_act_q8k_tiled - same levels, scales and sub-block sums as mi355_quantize_act_q8k
+ *                (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516), mi355_act_q8k_tiled_bytes(k, nrows) bytes;
+ *   weights:     mi355_kq_unpack_tiles - the two int8 planes of mi355_kq_unpack_planes (dequantize_row_q4_K / _q6_K,
+ *                ggml/src/ggml-quants.c:1280-1302, 1690-1719) plus per-super-block d, dmin and mins, written once per
+ *                weight matrix, mi355_kq_tiles_bytes(type, rows, K) bytes (about 2 bytes per weight).
+ * mi355_mul_mat_q8k_tiled computes what mi355_mul_mat_q8k_add computes (same integer sums: ggml_vec_dot_q4_K_q8_K /
+ * ggml_vec_dot_q6_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6817-6848, 8262-8283; f32 summation order may differ).
+ * ws: optional workspace of mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) bytes for the split along K of products with few
+ * tiles (NULL or too small: unsplit).  No counterpart in the reference (its CUDA backend unpacks in the tile loaders,
+ * ggml/src/ggml-cuda/mmq.cuh). */
+size_t mi355_act_q8k_tiled_bytes(int64_t k, int64_t nrows);
+int mi355_quantize_act_q8k_tiled(void *stream, const float *x, void *act, int64_t k, int64_t nrows, int64_t x_stride);
+size_t mi355_kq_tiles_bytes(int type, int64_t rows, int64_t K);
+int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, int64_t rows, int64_t K);
+size_t mi355_mul_mat_q8k_tiled_ws_bytes(int64_t N, int64_t K, int64_t B);
+int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N,
+                            int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
+
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE
  * launch, each optionally adding a residual in its epilogue (the ggml_add that follows the wo and
@@ -294,6 +315,11 @@ int mi355_rms_norm_mul_quant_q8k(void *stream, const float *x, int64_t x_stride,
                                  void *act, int64_t k, int64_t nrows, float eps);
 int mi355_swiglu_quant_q8k(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
                            int64_t k, int64_t nrows);
+/* ... and with `act` as the tile images of mi355_quantize_act_q8k_tiled (what mi355_mul_mat_q8k_tiled reads) */
+int mi355_rms_norm_mul_quant_q8k_tiled(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride,
+                                       void *act, int64_t k, int64_t nrows, float eps);
+int mi355_swiglu_quant_q8k_tiled(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
+                                 int64_t k, int64_t nrows);
 /* ROPE(q), ROPE(k), CPY(k -> K cache), CPY(v -> V cache) of build_llama + llm_build_kv_store (src/llama.cpp:1535-1548, :157-199;
  * ggml-cpu.c:9366-9549, 3519-3830).  q f32 [T][H][D] is rotated in place; k, v f32 [T][HK][D] are read; the f16 caches are addressed
  * as cell*nb1 + head*nb2 + 2*d with the cell of token t taken from cells[t] and its rope position from pos[t] (both DEVICE int32). */

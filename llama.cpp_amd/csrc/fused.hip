@@ -12,21 +12,22 @@
 #include "common.hpp"
 #include "norm_quant.hpp"
 #include "q8k.hpp"
+#include "tiles.hpp"
 
 namespace mi355 {
 
 // one 256-thread group per row
-template <int NV, bool Q8K>
+template <int NV, int FMT>
 __global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restrict__ x, int64_t x_stride, const float *__restrict__ w,
                                                             float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k,
                                                             int64_t nrows, float eps) {
     __shared__ float sh[4];
     const int64_t row = blockIdx.x;
-    rms_norm_quant_row<NV, Q8K, false>(x + row * x_stride, w, y ? y + row * y_stride : nullptr, act, row, k, nrows, eps, sh);
+    rms_norm_quant_row<NV, FMT, false>(x + row * x_stride, w, y ? y + row * y_stride : nullptr, act, row, k, nrows, eps, sh);
 }
 
 // h = silu(gate) * up, optional f32 output, optional Q8_1 output; one lane per 4 elements
-template <bool Q8K>
+template <int FMT>
 __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ gate, const float *__restrict__ up, int64_t in_stride,
                                                       float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k,
                                                       int64_t nrows) {
@@ -43,7 +44,9 @@ __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ 
     }
     if (act) {
         int8_t *qplane = (int8_t *)act;
-        if constexpr (Q8K) {
+        if constexpr (FMT == 2) {
+            if (live) q8k_quantize_wave_tiled(o, threadIdx.x & 63, (uint8_t *)act, k, nrows, row, e0 >> 8);   // whole wave: k is a multiple of 256
+        } else if constexpr (FMT == 1) {
             if (live) {   // whole wave: k is a multiple of 256
                 const int64_t nsb = k >> 8, sb = e0 >> 8;
                 float *d8 = (float *)(qplane + q8k_d_offset(k, nrows));
@@ -129,7 +132,8 @@ using namespace mi355;
 extern "C" {
 
 static int rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act, int64_t k,
-                              int64_t nrows, float eps, bool q8k) {
+                              int64_t nrows, float eps, int fmt) {
+    const bool q8k = fmt != 0;
     MI355_REQUIRE(k > 0 && k % 32 == 0 && k <= 16384, "rms_norm_mul_quant: k=%lld must be a multiple of 32 and at most 16384", (long long)k);
     MI355_REQUIRE(!q8k || k % QKK == 0, "rms_norm_mul_quant: k=%lld is not a multiple of 256", (long long)k);
     MI355_REQUIRE(nrows >= 0 && nrows < 0x7fffffff, "rms_norm_mul_quant: bad row count");
@@ -141,8 +145,9 @@ static int rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, co
     const dim3 grid((unsigned)nrows), block(256);
 #define MI355_LAUNCH_NORM(NV)                                                                                                        \
     do {                                                                                                                              \
-        if (q8k) hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, true>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
-        else hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, false>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);     \
+        if (fmt == 2) hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, 2>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
+        else if (fmt == 1) hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, 1>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
+        else hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, 0>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);     \
     } while (0)
     if (k <= 4096) MI355_LAUNCH_NORM(4);
     else if (k <= 8192) MI355_LAUNCH_NORM(8);
@@ -153,16 +158,22 @@ static int rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, co
 
 int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
                              int64_t k, int64_t nrows, float eps) {
-    return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, false);
+    return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, 0);
 }
 
 int mi355_rms_norm_mul_quant_q8k(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
                                  int64_t k, int64_t nrows, float eps) {
-    return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, true);
+    return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, 1);
+}
+
+int mi355_rms_norm_mul_quant_q8k_tiled(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
+                                       int64_t k, int64_t nrows, float eps) {
+    return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, 2);
 }
 
 static int swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act, int64_t k,
-                        int64_t nrows, bool q8k) {
+                        int64_t nrows, int fmt) {
+    const bool q8k = fmt != 0;
     MI355_REQUIRE(k > 0 && k % 32 == 0, "swiglu_quant: k=%lld must be a multiple of 32", (long long)k);
     MI355_REQUIRE(!q8k || k % QKK == 0, "swiglu_quant: k=%lld is not a multiple of 256", (long long)k);
     MI355_REQUIRE(nrows >= 0 && nrows <= 65535, "swiglu_quant: bad row count");
@@ -171,19 +182,25 @@ static int swiglu_quant(void *stream, const float *gate, const float *up, int64_
     MI355_REQUIRE(y != nullptr || act != nullptr, "swiglu_quant: no output requested");
     if (nrows == 0) return MI355_OK;
     const dim3 grid((unsigned)((k + 1023) / 1024), (unsigned)nrows), block(256);
-    if (q8k) hipLaunchKernelGGL(k_swiglu_quant<true>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
-    else hipLaunchKernelGGL(k_swiglu_quant<false>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
+    if (fmt == 2) hipLaunchKernelGGL(k_swiglu_quant<2>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
+    else if (fmt == 1) hipLaunchKernelGGL(k_swiglu_quant<1>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
+    else hipLaunchKernelGGL(k_swiglu_quant<0>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
     return launch_status("k_swiglu_quant");
 }
 
 int mi355_swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
                        int64_t k, int64_t nrows) {
-    return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, false);
+    return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, 0);
 }
 
 int mi355_swiglu_quant_q8k(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
                            int64_t k, int64_t nrows) {
-    return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, true);
+    return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, 1);
+}
+
+int mi355_swiglu_quant_q8k_tiled(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
+                                 int64_t k, int64_t nrows) {
+    return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, 2);
 }
 
 int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, void *kcache, void *vcache, const int32_t *pos,

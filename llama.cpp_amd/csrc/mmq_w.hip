@@ -1,0 +1,560 @@
+// Wide-tile K-quant GEMM on the int8 matrix cores: 128 weight rows x 128 activation rows per 512-thread group, one group per
+// compute unit, both operands streamed from pre-tiled images in HBM straight into LDS (no vector-ALU work on the way).
+//
+// Arithmetic is that of mmq_k.hip (ggml_vec_dot_q4_K_q8_K / ggml_vec_dot_q6_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6817-6848,
+// 8262-8283, on activations quantized by quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516): the integer sub-scales are
+// folded into two int8 operands per weight (value = R*hi + lo, R = 8 for Q4_K, 64 for Q6_K), v_mfma_i32_32x32x32_i8 sums whole
+// super-blocks in int32, the Q4_K min term is one v_mfma_f32_32x32x16_f16 per super-block on exact small integers, and the
+// vector ALU touches a result once per 256 elements.
+//
+// What differs is the data path and the schedule.  Measured on this part, per compute unit: about 22 bytes per clock from L2 into
+// LDS; a wave does not overlap its own vector instructions with its own matrix instructions, two waves of a SIMD do; packed
+// 16-bit integer multiplies run at a quarter of the rate of other vector instructions (which rules out keeping one byte per
+// Q4_K weight in LDS and multiplying by the sub-block scale on the way into the matrix instruction: measured, 35 % slower).
+//  * Both operands live in HBM as *tile images* (tiles.hpp): tiles of 16 rows x 64 elements = 1 KiB, each byte for byte what
+//    LDS holds, so one wave-wide global_load_lds moves a tile and nobody computes an address per element: 384 bytes from L2 per
+//    matrix instruction where a 64 x 128 tile needs 512.
+//  * K is walked in stages of 64 elements through a ring of four LDS buffers = one super-block; transfers run three stages
+//    ahead of their use, one barrier per stage.  Every LDS read (operands, scales) is issued one 32-element step ahead of its use
+//    and waited for once per step; the operand reads are inline assembly, because for reads it can see the compiler waits for
+//    every transfer in flight whose target it cannot tell from the array being read.
+//  * A wave owns 32 weight rows x 64 activation rows.  That leaves registers for a second set of integer accumulators: the sums
+//    of super-block s are scaled into the f32 accumulators in eight pieces placed between the matrix instructions of
+//    super-block s + 1, so the vector ALU of one wave works in the shadow of the other wave's matrix instructions.
+//
+// MFMA operand mapping (A = activations, B = weights, D[i][j]): lane l supplies row l % 32 and k bytes [16*(l/32), +16)
+// (f16: k slots [8*(l/32), +8)); D register r of lane l is i = 8*(r/4) + 4*(l/32) + r%4, j = l % 32.
+#include "common.hpp"
+#include "q8k.hpp"
+#include "qdot.hpp"
+#include "tiles.hpp"
+
+#include <type_traits>
+
+namespace mi355 {
+
+// unpack one 16-byte piece of packed weights into its two planes (same arithmetic as k_unpack_planes of mmq_k.hip) and store
+// the chunks into the tile images; one thread per piece: row, super-block, half, piece
+typedef unsigned short wt_u16x2 __attribute__((ext_vector_type(2)));
+typedef short wt_i16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32 wt_mul_bytes(u32 x, u32 f) {
+    const wt_u16x2 v = __builtin_bit_cast(wt_u16x2, x);
+    const wt_u16x2 m = {(unsigned short)f, (unsigned short)f};
+    const wt_u16x2 p = v * m;
+    return __builtin_bit_cast(u32, p);
+}
+__device__ __forceinline__ void wt_q6k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
+    const wt_i16x2 s = {(short)sc, (short)sc};
+    const wt_i16x2 off = {(short)(-32 * sc), (short)(-32 * sc)};
+    const wt_i16x2 e = __builtin_bit_cast(wt_i16x2, a & 0x00FF00FFu);
+    const wt_i16x2 o = __builtin_bit_cast(wt_i16x2, (a >> 8) & 0x00FF00FFu);
+    const wt_i16x2 pe = e * s + off, po = o * s + off;
+    const wt_i16x2 six = {6, 6};
+    const u32 he = __builtin_bit_cast(u32, pe >> six), ho = __builtin_bit_cast(u32, po >> six);
+    const u32 le = __builtin_bit_cast(u32, pe) & 0x003F003Fu, lo_ = __builtin_bit_cast(u32, po) & 0x003F003Fu;
+    hi = (he & 0x00FF00FFu) | ((ho & 0x00FF00FFu) << 8);
+    lo = le | (lo_ << 8);
+}
+
+template <int TYPE>
+__global__ void __launch_bounds__(256) k_unpack_tiles(const uint8_t *__restrict__ W, int8_t *__restrict__ img, int64_t N, int64_t K, row_layout L) {
+    const int64_t per_row = (K >> 8) * 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n16 = (N + 15) & ~(int64_t)15;
+    if (idx >= n16 * per_row) return;
+    const int64_t row = idx / per_row, rem = idx % per_row, sb = rem >> 3;
+    const int half = (int)((rem >> 2) & 1), p = (int)(rem & 3);
+    uint8_t *aux = (uint8_t *)img + wt_w_aux_offset(N, K);
+    const int64_t n_rb_pad = wt_rb_pad(N);
+    constexpr int W_AUX = wt_w_aux_bytes(TYPE);
+    const bool live = row < N;   // rows that pad the last 16-row block hold zeros
+    const uint8_t *wrow = W + (live ? row : 0) * L.row_bytes;
+    const int64_t k0 = sb * QKK + half * 128;
+    int8_t *hi_img = img, *lo_img = img + n16 * K;
+    u32x4 a1 = {0, 0, 0, 0}, a0 = a1, b1 = a1, b0 = a1;
+    int c0, c1;   // 16-byte chunk index inside the 128-element half
+    if constexpr (TYPE == MI355_Q4_K) {
+        const uint8_t *blk = wrow + sb * Q4_K_BYTES;
+        const u32x4 q = load16(blk + 16 + (half * 2 + (p >> 1)) * 32 + (p & 1) * 16);
+        const u32x4 hdr = load16(blk);
+        const int gl = p >> 1;
+        int scl, mnl, sch, mnh;
+        q4k_scale_min(hdr[1], hdr[2], hdr[3], half * 4 + 2 * gl, scl, mnl);
+        q4k_scale_min(hdr[1], hdr[2], hdr[3], half * 4 + 2 * gl + 1, sch, mnh);
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 nl = q[i] & 0x0F0F0F0Fu, nh = (q[i] >> 4) & 0x0F0F0F0Fu;
+                a1[i] = wt_mul_bytes(nl, (u32)scl >> 3);
+                a0[i] = wt_mul_bytes(nl, (u32)scl & 7u);
+                b1[i] = wt_mul_bytes(nh, (u32)sch >> 3);
+                b0[i] = wt_mul_bytes(nh, (u32)sch & 7u);
+            }
+        }
+        c0 = 4 * gl + (p & 1);
+        c1 = c0 + 2;
+        if (half == 0 && p == 0) {
+            uint8_t *e = aux + (sb * n_rb_pad + (row >> 4)) * W_AUX;
+            const int r = (int)(row & 15);
+            f16x8 m1, m64;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                int sc, mn;
+                q4k_scale_min(hdr[1], hdr[2], hdr[3], j, sc, mn);
+                if (!live) mn = 0;
+                m1[j] = (_Float16)(float)mn;
+                m64[j] = (_Float16)(float)(64 * mn);
+            }
+            *(f16x8 *)(e + r * 32) = m1;
+            *(f16x8 *)(e + r * 32 + 16) = m64;
+            *(float *)(e + 512 + r * 4) = live ? half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu)) : 0.0f;
+            *(float *)(e + 576 + r * 4) = live ? half_bits_to_float((unsigned short)(hdr[0] >> 16)) : 0.0f;
+        }
+    } else {
+        const int l0 = 16 * (p & 1), qa = p >> 1;
+        const u32x4 ql = load16(wrow + sb * 128 + half * 64 + p * 16);
+        const u32x4 qh = load16(wrow + L.off_b + sb * 64 + half * 32 + l0);
+        const int8_t *sc = (const int8_t *)(wrow + L.off_c + sb * 16 + half * 8 + (l0 >> 4));
+        const int scA = sc[2 * qa], scB = sc[2 * qa + 4];
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 va = (ql[i] & 0x0F0F0F0Fu) | (((qh[i] >> (2 * qa)) & 0x03030303u) << 4);
+                const u32 vb = ((ql[i] >> 4) & 0x0F0F0F0Fu) | (((qh[i] >> (2 * qa + 4)) & 0x03030303u) << 4);
+                u32 hi, lo;
+                wt_q6k_planes(va, scA, hi, lo);
+                a1[i] = hi; a0[i] = lo;
+                wt_q6k_planes(vb, scB, hi, lo);
+                b1[i] = hi; b0[i] = lo;
+            }
+        }
+        c0 = 2 * qa + (p & 1);
+        c1 = c0 + 4;
+        if (half == 0 && p == 0) {
+            uint8_t *e = aux + (sb * n_rb_pad + (row >> 4)) * W_AUX;
+            *(float *)(e + (row & 15) * 4) = live ? half_bits_to_float(*(const unsigned short *)(wrow + L.off_d + sb * 2)) : 0.0f;
+        }
+    }
+    *(u32x4 *)(hi_img + wt_tile_off(row, k0 + c0 * 16, K)) = a1;
+    *(u32x4 *)(lo_img + wt_tile_off(row, k0 + c0 * 16, K)) = a0;
+    *(u32x4 *)(hi_img + wt_tile_off(row, k0 + c1 * 16, K)) = b1;
+    *(u32x4 *)(lo_img + wt_tile_off(row, k0 + c1 * 16, K)) = b0;
+}
+
+// One wave per (row, super-block); 4 super-blocks per group.  Rows that pad the last 16-row block get zeros.
+__global__ void __launch_bounds__(256) k_quantize_q8k_tiled(const float *__restrict__ x, uint8_t *__restrict__ act, int64_t K, int64_t B, int64_t x_stride) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = blockIdx.y;
+    if (sb >= (K >> 8)) return;   // whole wave
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (row < B) v = *(const f32x4 *)(x + row * x_stride + sb * QKK + lane * 4);
+    q8k_quantize_wave_tiled(v, lane, act, K, B, row, sb);
+}
+
+constexpr int WT_BM = 128, WT_BN = 128;
+constexpr int WT_A_AUX_TILE = (WT_BN / 16) * WT_A_AUX;       // 4608 bytes of activation scales per tile and super-block
+
+// s_waitcnt that waits until at most n vector-memory operations of this wave are outstanding (nothing else)
+#define WT_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (7 << 4) | (0xF << 8))
+
+template <int TYPE>
+__global__ void __launch_bounds__(512, 1) k_mmq_w(const int8_t *__restrict__ w_img, const int8_t *__restrict__ a_img, float *dst, const float *residual,
+                                                  int64_t N, int64_t K, int64_t B, int64_t dst_stride, int n_col_tiles, int n_groups, int n_groups_padded) {
+    constexpr bool Q4 = TYPE == MI355_Q4_K;
+    constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
+    constexpr int NP = 2;                                                      // weight planes
+    constexpr int W_AUX = wt_w_aux_bytes(TYPE);
+    constexpr int STAGE = (NP * WT_BM + WT_BN) * 64;                           // bytes of one 64-element stage: plane(s), activations
+    constexpr int OFF_LO = WT_BM * 64, OFF_A = NP * WT_BM * 64;
+    constexpr int DPS = NP + 1;                                                // transfers per wave and stage
+    constexpr int N_A_CHUNKS = (WT_A_AUX_TILE + 1023) / 1024;                  // 5, the last one half full
+    constexpr int N_W_CHUNKS = (WT_BM / 16) * W_AUX / 1024;                    // 5 or 1
+    constexpr int N_CHUNKS = N_A_CHUNKS + N_W_CHUNKS;                          // scale transfers per super-block
+    constexpr int AUX_W_OFF = N_A_CHUNKS * 1024;                               // weight entries behind the (padded) activation entries
+    // Ring of stage buffers: 8 (two super-blocks) where they fit, else 4; a stage's transfers are issued DIST stages ahead.
+    // The operand reads from the ring are inline assembly with waits placed by hand: for accesses it can see, the compiler
+    // waits for every transfer in flight whose target it cannot tell from the array being read, and it tells nothing apart
+    // inside one array and at most eight arrays in all.
+    constexpr int NBUF = 4, DIST = NBUF - 1;
+    __shared__ __attribute__((aligned(1024))) int8_t ring_buf[NBUF * STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t aux0[AUX_W_OFF + 5 * 1024], aux1[AUX_W_OFF + 5 * 1024];   // scale entries of a super-block
+    // The buffers are written by global-to-LDS transfers only; the empty asm makes them memory that unknown code may have written.
+    asm volatile("" ::"v"((void *)ring_buf), "v"((void *)aux0), "v"((void *)aux1) : "memory");
+    auto ring = [&](int i) -> int8_t * { return ring_buf + (i & (NBUF - 1)) * STAGE; };
+
+    const int per_xcd = n_groups_padded >> 3;
+    const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (lid >= n_groups) return;
+    const int64_t row0 = (int64_t)(lid / n_col_tiles) * WT_BM;
+    const int64_t col0 = (int64_t)(lid % n_col_tiles) * WT_BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int wrow0 = (wave & 3) * 32;    // weight rows of this wave inside the tile
+    const int wcol0 = (wave >> 2) * 64;   // activation rows of this wave inside the tile
+    const int64_t nsb = K >> 8, nkb = K >> 6;
+    // split K: group y of gridDim.y walks super-blocks [sb_lo, sb_hi) and writes its sums to its own slice of `dst`
+    const int64_t sb_per = (nsb + gridDim.y - 1) / gridDim.y;
+    const int64_t sb_lo = (int64_t)blockIdx.y * sb_per, sb_hi = sb_lo + sb_per < nsb ? sb_lo + sb_per : nsb;
+    if (gridDim.y > 1) {
+        dst += (int64_t)blockIdx.y * B * dst_stride;
+        residual = nullptr;
+    }
+
+    // ---- sources of this wave's transfers per stage: one tile of each weight plane and one activation tile
+    const int64_t n16 = (N + 15) & ~(int64_t)15, b16 = (B + 15) & ~(int64_t)15;
+    const int64_t n_rb = n16 >> 4, n_cb = b16 >> 4;
+    const int64_t n_rb_pad = wt_rb_pad(N), n_cb_pad = wt_cb_pad(B);
+    const int64_t rb0 = row0 >> 4, cb0 = col0 >> 4;
+    const int64_t rbw = rb0 + wave < n_rb ? rb0 + wave : n_rb - 1;
+    const int64_t cba = cb0 + wave < n_cb ? cb0 + wave : n_cb - 1;
+    // wave-uniform bases; the lane's 16 bytes are added at the transfer
+    const unsigned lane16 = (unsigned)lane * 16u;
+    const int8_t *src_w = w_img + rbw * nkb * WT_TILE;
+    const int8_t *src_a = a_img + cba * nkb * WT_TILE;
+    const uint8_t *w_aux = (const uint8_t *)w_img + wt_w_aux_offset(N, K) + rb0 * W_AUX;
+    const uint8_t *a_aux = (const uint8_t *)a_img + b16 * K + cb0 * WT_A_AUX;
+    // aux chunks 2*wave and 2*wave + 1 of the super-block's N_CHUNKS (those past the end repeat the last one)
+    const int ch0 = 2 * wave < N_CHUNKS ? 2 * wave : N_CHUNKS - 1, ch1 = 2 * wave + 1 < N_CHUNKS ? 2 * wave + 1 : N_CHUNKS - 1;
+
+    auto dma = [&](const void *g, void *l) {   // g: wave-uniform
+        // scalar base + 32-bit lane offset; the empty asm keeps the sum from being formed once per lane ahead of the loop, which
+        // would cost two registers per source
+        unsigned off = lane16;
+        asm volatile("" : "+v"(off));
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)((const char *)g + off),
+                                         (void __attribute__((address_space(3))) *)l, 16, 0, 0);
+    };
+    auto dma_stage = [&](int64_t kb, int8_t *buf) {   // kb: absolute 64-element block
+        const int64_t o = kb * WT_TILE;
+        dma(src_w + o, buf + wave * WT_TILE);
+        dma(src_w + n16 * K + o, buf + OFF_LO + wave * WT_TILE);
+        dma(src_a + o, buf + OFF_A + wave * WT_TILE);
+    };
+    // Scale entries of super-block sb into `buf`.  The activation entries of a tile end in the middle of their last chunk: what
+    // follows them in memory comes along and is never read.
+    auto dma_aux_chunk = [&](int64_t sb, int ch, uint8_t *buf) {
+        const uint8_t *src = ch < N_A_CHUNKS ? a_aux + sb * n_cb_pad * WT_A_AUX + ch * 1024 : w_aux + sb * n_rb_pad * W_AUX + (ch - N_A_CHUNKS) * 1024;
+        dma(src, buf + ch * 1024);
+    };
+    auto dma_aux = [&](int64_t sb, uint8_t *buf) {
+        dma_aux_chunk(sb, ch0, buf);
+        dma_aux_chunk(sb, ch1, buf);
+    };
+
+    // ---- per-lane LDS offsets of the operand reads: row l32 of a 32-row tile, logical chunk 2*ks + lhi of the stage
+    int foff[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) foff[ks] = (l32 >> 4) * WT_TILE + (l32 & 15) * 64 + (((2 * ks + lhi) ^ ((l32 >> 2) & 3)) << 4);
+    const int a_base = OFF_A + (wcol0 >> 4) * WT_TILE, w_base = (wrow0 >> 4) * WT_TILE;
+    // scale entries of this lane's weight row and of the activation row it feeds to the min-term matrix instruction
+    const int we_off = AUX_W_OFF + ((wrow0 >> 4) + (l32 >> 4)) * W_AUX;
+    const int ae_off = (wcol0 >> 4) * WT_A_AUX;
+    // Offset of the activation sub-block sums this lane feeds to the min-term matrix instruction (tile 0; tile 1 is two entries on).
+    // The empty asm hides how it is made up: split into a chain of pointer increments by the optimizer, the access loses the
+    // compiler's knowledge of which LDS array it reads, and every such read would then wait for all transfers in flight.
+    int am_off = ae_off + (l32 >> 4) * WT_A_AUX + 64 + (l32 & 15) * 32 + lhi * 16;
+    asm volatile("" : "+v"(am_off));
+
+    f32x16 acc[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[tb][r] = 0.0f;
+    i32x16 hiX[2], loX[2], hiY[2], loY[2];   // integer sums of the even / odd super-blocks of the slice
+
+    // One eighth of the scaling of a finished super-block: registers 4*q .. 4*q+3 of tile tb.  M: the min term of the tile.
+    // activation scales of registers 4*q .. 4*q+3 of tile tb
+    auto load_d8 = [&](const uint8_t *ax, int tb, int q) {
+        return *(const f32x4 *)(ax + (ae_off + (2 * tb + (q >> 1)) * WT_A_AUX + (8 * (q & 1) + 4 * lhi) * 4));
+    };
+    auto scale_piece = [&](const f32x4 &d8, const i32x16 &h, const i32x16 &l, const f32x16 &M, float dw, float dn, int tb, int q) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int r = 4 * q + i;
+            const float f = (float)((h[r] << RADIX_SHIFT) + l[r]);
+            if constexpr (Q4) acc[tb][r] = __builtin_fmaf(d8[i], __builtin_fmaf(-dn, M[r], mul_rn(dw, f)), acc[tb][r]);
+            else acc[tb][r] = __builtin_fmaf(d8[i], mul_rn(dw, f), acc[tb][r]);
+        }
+    };
+    // operands of the min-term matrix instruction: sub-block sums of tile tb's activation rows / mins of the weight rows
+    auto load_am = [&](const uint8_t *ax, int tb) { return *(const f16x8 *)(ax + (am_off + tb * 2 * WT_A_AUX)); };
+    auto load_bm = [&](const uint8_t *ax) { return *(const f16x8 *)(ax + (we_off + (l32 & 15) * 32 + lhi * 16)); };
+    auto min_term = [&](const f16x8 &am, const f16x8 &bm) {
+        f32x16 z;
+#pragma unroll
+        for (int r = 0; r < 16; r++) z[r] = 0.0f;
+        if constexpr (Q4) return __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bm, z, 0, 0, 0);
+        else return z;
+    };
+    // operand registers of one 32-element step: two activation tiles, both planes of the weight tile
+    struct frags { i32x4 a[2], w[2]; };
+    // LDS byte addresses of this lane's reads in ring position 0 (activation / weight tile, first / second step of a stage); the
+    // second pair is 64 KiB on, for the ring positions an instruction's 16-bit offset does not reach from the first
+    const unsigned ring_addr = (unsigned)(size_t)(__attribute__((address_space(3))) int8_t *)ring_buf;
+    unsigned fa[2][2], fw[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            fa[h][ks] = ring_addr + (unsigned)(a_base + foff[ks]) + h * 65536u;
+            fw[h][ks] = ring_addr + (unsigned)(w_base + foff[ks]) + h * 65536u;
+        }
+#define WT_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+    // rs: ring position (compile-time constant after unrolling).  The values are valid after frags_wait.
+    auto load_frags = [&](frags &F, int rs, int ks) {
+        const int o = (rs & (NBUF - 1)) * STAGE, h = o >> 16, ol = o & 65535;
+        // every offset below must fit 16 bits: a stage never straddles a 64 KiB boundary (STAGE divides 64 KiB or ol + STAGE <= 64 KiB)
+        if (h == 0) {
+            WT_DS_READ(F.a[0], fa[0][ks], ol);
+            WT_DS_READ(F.a[1], fa[0][ks], ol + 2 * WT_TILE);
+            WT_DS_READ(F.w[0], fw[0][ks], ol);
+            WT_DS_READ(F.w[1], fw[0][ks], ol + OFF_LO);
+        } else {
+            WT_DS_READ(F.a[0], fa[1][ks], ol);
+            WT_DS_READ(F.a[1], fa[1][ks], ol + 2 * WT_TILE);
+            WT_DS_READ(F.w[0], fw[1][ks], ol);
+            WT_DS_READ(F.w[1], fw[1][ks], ol + OFF_LO);
+        }
+    };
+    // all LDS reads of this wave have returned; the registers pass through the statement so that their users stay behind it
+    auto frags_wait = [&](frags &F) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(F.a[0]), "+v"(F.a[1]), "+v"(F.w[0]), "+v"(F.w[1]));
+    };
+
+    // ---- prologue: scales of the first super-block, stages 0..2 of the slice
+    const int64_t kb_lo = sb_lo * 4, kb_last = sb_hi * 4 - 1;
+    auto clamp_kb = [&](int64_t kb) { return kb < kb_last ? kb : kb_last; };
+#pragma unroll
+    for (int i = 0; i < DIST; i++) dma_stage(clamp_kb(kb_lo + i), ring(i));
+    WT_WAIT_VM((DIST - 1) * DPS);
+    __builtin_amdgcn_s_barrier();
+    frags F0, F1;   // steps with even / odd index
+    load_frags(F0, 0, 0);
+
+    // Scale data of the super-block whose sums are being scaled, read from LDS one step ahead of their use.
+    f32x4 e_d8 = {0.f, 0.f, 0.f, 0.f};                  // activation scales of the next piece
+    f16x8 e_am = {0, 0, 0, 0, 0, 0, 0, 0}, e_bm = e_am;   // min-term operands: next tile's sub-block sums, the weight rows' mins
+    float e_dw = 0.0f, e_dn = 0.0f;                     // d and dmin of this lane's weight row
+    f32x16 e_M;                                         // min term of the tile whose pieces come next
+#pragma unroll
+    for (int r = 0; r < 16; r++) e_M[r] = 0.0f;
+
+    // One super-block.  ODD: parity of its position in the slice (picks accumulator set and scale buffers at compile time);
+    // PREV: the super-block before it exists and is scaled between this one's matrix instructions.
+    // A step first waits for the LDS reads issued during the step before (its operands and scales), then issues the reads of
+    // the step after it, then computes: no read is waited for right after its issue.
+    auto super_block = [&](auto odd_c, auto prev_c, const int64_t sb) {
+        constexpr bool ODD = decltype(odd_c)::value, PREV = decltype(prev_c)::value;
+        i32x16(&hi)[2] = ODD ? hiY : hiX;
+        i32x16(&lo)[2] = ODD ? loY : loX;
+        const i32x16(&phi)[2] = ODD ? hiX : hiY;
+        const i32x16(&plo)[2] = ODD ? loX : loY;
+        uint8_t *ax_cur = ODD ? aux1 : aux0;           // receives this super-block's scale entries
+        const uint8_t *ax_prev = ODD ? aux0 : aux1;    // holds the previous super-block's
+        float dw = e_dw, dn = e_dn;
+        f16x8 bm = e_bm;
+#pragma unroll
+        for (int piece = 0; piece < 8; piece++) {
+            const int st = piece >> 1, ks = piece & 1;
+            const int rs = (ODD ? 4 : 0) + st;              // position of this stage in the ring (the slice starts at 0)
+            int8_t *nxt = ring(rs + DIST);                  // buffer of the stage DIST ahead = of the stage before this one
+            frags &F = ks == 0 ? F0 : F1;
+            frags &Fn = ks == 0 ? F1 : F0;
+            const f32x4 d8 = e_d8;
+            const f16x8 am = e_am;
+            frags_wait(F);   // all LDS reads of this wave have returned
+            if (ks == 0) {
+                // scale entries first: they are then complete a stage earlier
+                if (st == 0) dma_aux(sb, ax_cur);
+                dma_stage(clamp_kb(sb * 4 + st + DIST), nxt);
+                load_frags(Fn, rs, 1);
+            } else {
+                // The next stage's transfers must have landed, and every wave must be done reading this stage, whose buffer the
+                // next transfers overwrite.  Issued since the next stage's: DIST - 1 stages and the scale entries (2 transfers,
+                // ahead of the first stage's) of every super-block that began among them; the first super-block of a slice has
+                // no predecessor that issued any.
+                // (super-block starts among stages s - DIST + 2 .. s, s = this stage)
+                if (st < 2) WT_WAIT_VM((DIST - 1) * DPS + 2);
+                else WT_WAIT_VM((DIST - 1) * DPS);   // the scale entries are complete from here on: they are read at the end of the super-block
+                __builtin_amdgcn_s_barrier();
+                load_frags(Fn, rs + 1, 0);
+            }
+            // scale data of the next step; the min-term operands one step earlier still, so that the min term of a tile is issued
+            // at the end of the step before the tile's first piece and has left the matrix pipe when that piece reads it
+            if (piece == 7) e_d8 = load_d8(ax_cur, 0, 0);   // the next super-block scales this one's sums
+            else if (PREV) e_d8 = load_d8(ax_prev, (piece + 1) >> 2, (piece + 1) & 3);
+            if (piece == 6) {   // this super-block's entries are complete since the barrier of the stage before
+                if constexpr (Q4) {
+                    e_am = load_am(ax_cur, 0);
+                    e_bm = load_bm(ax_cur);
+                    e_dw = *(const float *)(ax_cur + (we_off + 512 + (l32 & 15) * 4));
+                    e_dn = *(const float *)(ax_cur + (we_off + 576 + (l32 & 15) * 4));
+                } else {
+                    e_dw = *(const float *)(ax_cur + (we_off + (l32 & 15) * 4));
+                }
+            }
+            if (Q4 && PREV && piece == 2) e_am = load_am(ax_prev, 1);
+            const i32x4 b1 = F.w[0], b0 = F.w[1];
+#pragma unroll
+            for (int tb = 0; tb < 2; tb++) {
+                if (piece == 0) {   // the first block of a super-block starts the integer sums
+                    i32x16 z;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) z[r] = 0;
+                    hi[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(F.a[tb], b1, z, 0, 0, 0);
+                    lo[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(F.a[tb], b0, z, 0, 0, 0);
+                } else {
+                    hi[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(F.a[tb], b1, hi[tb], 0, 0, 0);
+                    lo[tb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(F.a[tb], b0, lo[tb], 0, 0, 0);
+                }
+            }
+            if (PREV) scale_piece(d8, phi[piece >> 2], plo[piece >> 2], e_M, dw, dn, piece >> 2, piece & 3);
+            if (Q4 && ((PREV && piece == 3) || piece == 7)) e_M = min_term(am, piece == 7 ? e_bm : bm);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    super_block(std::false_type{}, std::false_type{}, sb_lo);
+    for (int64_t sb = sb_lo + 1; sb < sb_hi; sb += 2) {
+        super_block(std::true_type{}, std::true_type{}, sb);
+        if (sb + 1 < sb_hi) super_block(std::false_type{}, std::true_type{}, sb + 1);
+    }
+    // the last super-block's sums; its scale data for the first piece are in the registers
+    {
+        const bool odd = (sb_hi - 1 - sb_lo) & 1;
+        const uint8_t *ax = odd ? aux1 : aux0;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++) {
+            const f32x16 M = tb == 0 ? e_M : min_term(load_am(ax, 1), e_bm);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const f32x4 d8 = tb == 0 && q == 0 ? e_d8 : load_d8(ax, tb, q);
+                if (odd) scale_piece(d8, hiY[tb], loY[tb], M, e_dw, e_dn, tb, q);
+                else scale_piece(d8, hiX[tb], loX[tb], M, e_dw, e_dn, tb, q);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int tb = 0; tb < 2; tb++) {
+        const int64_t n = row0 + wrow0 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if (n < N && b < B) {
+                const int64_t o = b * dst_stride + n;
+                dst[o] = residual ? acc[tb][r] + residual[o] : acc[tb][r];   // residual may be dst itself: one reader and writer per element
+            }
+        }
+    }
+}
+
+// slices along K for products with few 128 x 256 tiles (same idea as mmq_k.hip's split: partial sums to a workspace, then k_split_sum)
+static int wt_split_slices(int64_t N, int64_t K, int64_t B) {
+    const int64_t groups = ((N + WT_BM - 1) / WT_BM) * ((B + WT_BN - 1) / WT_BN), nsb = K / QKK;
+    if (groups >= 160) return 1;
+    int64_t n = 256 / groups;
+    if (n > nsb / 2) n = nsb / 2;
+    if (n > 8) n = 8;
+    if (n < 2) return 1;
+    const int64_t per = (nsb + n - 1) / n;
+    return (int)((nsb + per - 1) / per);
+}
+
+__global__ void __launch_bounds__(256) k_wt_split_sum(const float *__restrict__ part, float *__restrict__ dst, const float *__restrict__ residual,
+                                                      int64_t N, int64_t B, int64_t dst_stride, int n_slices) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;   // N % 4 == 0 here
+    if (i >= N * B) return;
+    const int64_t b = i / N, n = i % N;
+    f32x4 acc = *(const f32x4 *)(part + i);
+    for (int sl = 1; sl < n_slices; sl++) {
+        const f32x4 v = *(const f32x4 *)(part + (int64_t)sl * N * B + i);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = add_rn(acc[j], v[j]);
+    }
+    const int64_t o = b * dst_stride + n;
+    if (residual) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = add_rn(acc[j], residual[o + j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) dst[o + j] = acc[j];
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+size_t mi355_act_q8k_tiled_bytes(int64_t k, int64_t nrows) {
+    if (k <= 0 || nrows <= 0 || k % QKK != 0) return 0;
+    return wt_act_bytes(k, nrows);
+}
+
+int mi355_quantize_act_q8k_tiled(void *stream, const float *x, void *act, int64_t k, int64_t nrows, int64_t x_stride) {
+    MI355_REQUIRE(k > 0 && k % QKK == 0, "quantize_act_q8k_tiled: k=%lld is not a multiple of 256", (long long)k);
+    MI355_REQUIRE(nrows > 0 && nrows <= 65520, "quantize_act_q8k_tiled: nrows=%lld out of range", (long long)nrows);
+    MI355_REQUIRE(x_stride >= k && x_stride % 4 == 0 && ((uintptr_t)x & 15) == 0, "quantize_act_q8k_tiled: x must be 16-byte aligned with a row stride that is a multiple of 4 floats");
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0, "quantize_act_q8k_tiled: workspace must be 16-byte aligned");
+    const int64_t b16 = (nrows + 15) & ~(int64_t)15;
+    const dim3 grid((unsigned)((k / QKK + 3) / 4), (unsigned)b16);
+    hipLaunchKernelGGL(k_quantize_q8k_tiled, grid, dim3(256), 0, (hipStream_t)stream, x, (uint8_t *)act, k, nrows, x_stride);
+    return launch_status("k_quantize_q8k_tiled");
+}
+
+size_t mi355_kq_tiles_bytes(int type, int64_t rows, int64_t K) {
+    if (rows <= 0 || K <= 0 || K % QKK != 0 || (type != MI355_Q4_K && type != MI355_Q6_K)) return 0;
+    return wt_weight_bytes(type, rows, K);
+}
+
+int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, int64_t rows, int64_t K) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "kq_unpack_tiles: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(rows > 0 && K > 0 && K % QKK == 0, "kq_unpack_tiles: bad shape rows=%lld K=%lld", (long long)rows, (long long)K);
+    const row_layout L = make_row_layout(type, K);
+    MI355_REQUIRE(layout_aligned(W, L) && ((uintptr_t)tiles & 15) == 0, "kq_unpack_tiles: rows are not 16-byte aligned (K=%lld)", (long long)K);
+    const int64_t pieces = ((rows + 15) & ~(int64_t)15) * (K >> 8) * 8;
+    MI355_REQUIRE((pieces + 255) / 256 < 0x7fffffff, "kq_unpack_tiles: too many pieces for one launch");
+    const dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
+    if (type == MI355_Q4_K) hipLaunchKernelGGL(k_unpack_tiles<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
+    else hipLaunchKernelGGL(k_unpack_tiles<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
+    return launch_status("k_unpack_tiles");
+}
+
+size_t mi355_mul_mat_q8k_tiled_ws_bytes(int64_t N, int64_t K, int64_t B) {
+    if (N <= 0 || K <= 0 || B <= 0 || K % QKK != 0) return 0;
+    const int n = wt_split_slices(N, K, B);
+    return n > 1 && N % 4 == 0 ? (size_t)n * (size_t)N * (size_t)B * sizeof(float) : 0;
+}
+
+int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N,
+                            int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k_tiled: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
+    MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k_tiled: K=%lld is not a multiple of 256", (long long)K);
+    MI355_REQUIRE(dst_stride >= N, "mul_mat_q8k_tiled: dst_stride < N");
+    MI355_REQUIRE(tiles != nullptr && ((uintptr_t)tiles & 15) == 0 && act != nullptr && ((uintptr_t)act & 15) == 0, "mul_mat_q8k_tiled: operands are not 16-byte aligned");
+    const int n_row_tiles = (int)((N + WT_BM - 1) / WT_BM), n_col_tiles = (int)((B + WT_BN - 1) / WT_BN);
+    MI355_REQUIRE((int64_t)n_row_tiles * n_col_tiles < (1 << 30), "mul_mat_q8k_tiled: too many tiles");
+    const int n_groups = n_row_tiles * n_col_tiles, n_groups_padded = (n_groups + 7) & ~7;
+    hipStream_t s = (hipStream_t)stream;
+    int n_slices = wt_split_slices(N, K, B);
+    if (n_slices < 2 || ws == nullptr || ((uintptr_t)ws & 15) != 0 || N % 4 != 0 || ws_bytes < (size_t)n_slices * (size_t)N * (size_t)B * sizeof(float)) n_slices = 1;
+    const dim3 grid((unsigned)n_groups_padded, (unsigned)n_slices);
+    float *out = n_slices > 1 ? (float *)ws : dst;
+    const float *res = n_slices > 1 ? nullptr : residual;
+    const int64_t out_stride = n_slices > 1 ? N : dst_stride;
+    if (type == MI355_Q4_K)
+        hipLaunchKernelGGL(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
+    else
+        hipLaunchKernelGGL(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
+    if (n_slices > 1)
+        hipLaunchKernelGGL(k_wt_split_sum, dim3((unsigned)((N * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
+    return launch_status("k_mmq_w");
+}
+
+}  // extern "C"

@@ -5,6 +5,7 @@
 #pragma once
 #include "common.hpp"
 #include "q8k.hpp"
+#include "tiles.hpp"
 
 namespace mi355 {
 
@@ -41,7 +42,8 @@ __device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, i
 // Each thread keeps its NV float4 of the row in registers (k <= 1024 * NV).  COH: the row was written by other groups of the
 // same launch with device-scope stores and is read with device-scope loads.  sh: 4 floats of LDS; the caller places a
 // barrier between two calls that share it.
-template <int NV, bool Q8K, bool COH>
+// FMT: activation format written to `act`: 0 Q8_1 (split layout), 1 per-super-block (q8k.hpp), 2 the same as tile images (tiles.hpp)
+template <int NV, int FMT, bool COH>
 __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr, const float *__restrict__ w, float *__restrict__ yr,
                                                    void *__restrict__ act, int64_t row, int64_t k, int64_t nrows, float eps, float *sh) {
     const int tid = threadIdx.x;
@@ -86,7 +88,9 @@ __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr,
             for (int i = 0; i < 4; i++) o[i] = o[i] * ww[it][i];
         }
         if (yr && live) *(f32x4 *)(yr + e0) = o;
-        if constexpr (Q8K) {
+        if constexpr (FMT == 2) {
+            if (act && live) q8k_quantize_wave_tiled(o, tid & 63, (uint8_t *)act, k, nrows, row, e0 >> 8);   // whole wave: k is a multiple of 256
+        } else if constexpr (FMT == 1) {
             if (act && live) {   // whole wave: k is a multiple of 256
                 const int64_t nsb = k >> 8, sb = e0 >> 8;
                 float *d8 = (float *)(qplane + q8k_d_offset(k, nrows));

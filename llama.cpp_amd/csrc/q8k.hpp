@@ -12,8 +12,9 @@ __host__ __device__ inline size_t q8k_bs_offset(int64_t K, int64_t B) {
     return (q8k_d_offset(K, B) + (size_t)B * (size_t)(K / QKK) * 4 + 15) & ~(size_t)15;   // bs entries are read 16 bytes at a time
 }
 
-// One wave quantizes one super-block: lane l holds elements 4l .. 4l+3.  q, d8, bs point at the super-block's entries.
-__device__ __forceinline__ void q8k_quantize_wave(const f32x4 &v, int lane, int8_t *__restrict__ q, float *__restrict__ d8, _Float16 *__restrict__ bs) {
+// One wave quantizes one super-block: lane l holds elements 4l .. 4l+3.  packed: the lane's four int8 levels; d: the super-block's
+// scale (every lane); sum: the integer sum of the lane's 32-element sub-block (every lane of the 8 that share it).
+__device__ __forceinline__ void q8k_quantize_values(const f32x4 &v, int lane, u32 &packed, float &d, int &sum) {
     // signed value of the first element with the largest magnitude
     float amax = 0.0f, vmax = 0.0f;
 #pragma unroll
@@ -30,7 +31,7 @@ __device__ __forceinline__ void q8k_quantize_wave(const f32x4 &v, int lane, int8
     }
 
     int lv[4] = {0, 0, 0, 0};
-    float d = 0.0f;
+    d = 0.0f;
     if (amax != 0.0f) {
         const float iscale = -127.0f / vmax;
 #pragma unroll
@@ -40,11 +41,18 @@ __device__ __forceinline__ void q8k_quantize_wave(const f32x4 &v, int lane, int8
         }
         d = 1.0f / iscale;
     }
-    int sum = lv[0] + lv[1] + lv[2] + lv[3];
+    sum = lv[0] + lv[1] + lv[2] + lv[3];
 #pragma unroll
     for (int off = 1; off < 8; off <<= 1) sum += __shfl_xor(sum, off, 64);
+    packed = (u32)(lv[0] & 0xFF) | ((u32)(lv[1] & 0xFF) << 8) | ((u32)(lv[2] & 0xFF) << 16) | ((u32)(lv[3] & 0xFF) << 24);
+}
 
-    const u32 packed = (u32)(lv[0] & 0xFF) | ((u32)(lv[1] & 0xFF) << 8) | ((u32)(lv[2] & 0xFF) << 16) | ((u32)(lv[3] & 0xFF) << 24);
+// The same, stored: q, d8, bs point at the super-block's entries.
+__device__ __forceinline__ void q8k_quantize_wave(const f32x4 &v, int lane, int8_t *__restrict__ q, float *__restrict__ d8, _Float16 *__restrict__ bs) {
+    u32 packed;
+    float d;
+    int sum;
+    q8k_quantize_values(v, lane, packed, d, sum);
     *(u32 *)(q + lane * 4) = packed;
     if (lane == 0) *d8 = d;
     if ((lane & 7) == 0) {

@@ -57,11 +57,19 @@ _SIGNATURES = {
     "mi355_mul_mat_q8k_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_q8k_ws": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_q8k_add": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64]),
+    "mi355_act_q8k_tiled_bytes": (_sz, [_i64, _i64]),
+    "mi355_quantize_act_q8k_tiled": (_int, [_p, _p, _p, _i64, _i64, _i64]),
+    "mi355_kq_tiles_bytes": (_sz, [_int, _i64, _i64]),
+    "mi355_kq_unpack_tiles": (_int, [_p, _int, _p, _p, _i64, _i64]),
+    "mi355_mul_mat_q8k_tiled_ws_bytes": (_sz, [_i64, _i64, _i64]),
+    "mi355_mul_mat_q8k_tiled": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_rms_norm_mul_quant": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
     "mi355_swiglu_quant": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
     "mi355_rms_norm_mul_quant_q8k": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
     "mi355_swiglu_quant_q8k": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
+    "mi355_rms_norm_mul_quant_q8k_tiled": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
+    "mi355_swiglu_quant_q8k_tiled": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
     "mi355_rope_kv_store": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _int, _int, _int,
                             _f, _f, _f, _f, _f, _f]),
     "mi355_ffn_gate_up_swiglu": (_int, [_p, _int, _p, _int, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64]),
@@ -209,6 +217,37 @@ def quantize_act_q8k(x):
     ws = torch.empty(load().mi355_act_q8k_bytes(k, nrows), dtype=torch.uint8, device=x.device)
     check(load().mi355_quantize_act_q8k(_stream(), _ptr(x), _ptr(ws), k, nrows, x.stride(0)))
     return ws
+
+
+def quantize_act_q8k_tiled(x):
+    """x f32 [nrows, k] -> the tile-image form of the per-super-block activation quantization"""
+    import torch
+    nrows, k = x.shape
+    ws = torch.empty(load().mi355_act_q8k_tiled_bytes(k, nrows), dtype=torch.uint8, device=x.device)
+    check(load().mi355_quantize_act_q8k_tiled(_stream(), _ptr(x), _ptr(ws), k, nrows, x.stride(0)))
+    return ws
+
+
+def kq_unpack_tiles(t, W):
+    """W: device-layout uint8 [N, row_bytes] (Q4_K / Q6_K) -> tile images of its two int8 planes + per-super-block scales"""
+    import torch
+    N, rb = W.shape
+    K = rb // BLOCK[t][1] * BLOCK[t][0]
+    tiles = torch.empty(load().mi355_kq_tiles_bytes(t, N, K), dtype=torch.uint8, device=W.device)
+    check(load().mi355_kq_unpack_tiles(_stream(), t, _ptr(W), _ptr(tiles), N, K))
+    return tiles
+
+
+def mul_mat_q8k_tiled(t, tiles, act, N, K, B, residual=None, split=True, dst=None):
+    """the wide-tile K-quant GEMM: tiles from kq_unpack_tiles, act from quantize_act_q8k_tiled -> f32 [B, N]"""
+    import torch
+    if dst is None:
+        dst = torch.empty((B, N), dtype=torch.float32, device=tiles.device)
+    nws = load().mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) if split else 0
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=tiles.device)
+    check(load().mi355_mul_mat_q8k_tiled(_stream(), t, _ptr(tiles), _ptr(act), _ptr(dst), _ptr(residual) if residual is not None else None,
+                                         N, K, B, dst.stride(0), _ptr(ws) if nws else None, nws))
+    return dst
 
 
 def mul_mat(t, W, x, ws=None, split=True):

@@ -99,6 +99,10 @@ class LlamaRunner:
         self.fuse_qkv = True    # rows must be 16-byte aligned; set False to use the three-launch sequence
         self.use_planes = True  # prefill: Q6_K matrices go through their unpacked int8 planes (2 bytes per weight more, kept resident)
         self.planes = {}
+        # prefill from 33 tokens on: K-quant matrices go through the wide-tile GEMM, which reads tile images of the weights' two
+        # int8 planes (a second copy, 2 bytes per weight, built on first use and kept) and of the quantized activations
+        self.use_tiles = True
+        self.tiles = {}
         self.split_ws = None    # partial sums of tile products that are split along K (grown on first use, before any graph capture)
         # decode, T <= 4: SiLU*up + Q8_1 either by the last group of each 32-row block of the gate/up launch (True) or as a launch
         # of their own after a two-matrix product (False).  With the activation staged in LDS the two-launch form is the quicker
@@ -125,8 +129,9 @@ class LlamaRunner:
         self.pos = torch.zeros(T, dtype=torch.int32, device=dev)
         self.mask = torch.zeros((T + 63) // 64 * 64, cfg.n_ctx, dtype=torch.float16, device=dev)
         kmax = max(E, F, H * D)
-        self.act_a = torch.empty(int(self.lib.mi355_act_bytes(max(E, H * D), T)) + 256, dtype=torch.uint8, device=dev)
-        self.act_b = torch.empty(int(self.lib.mi355_act_bytes(F, T)) + 256, dtype=torch.uint8, device=dev)
+        self.act_a = torch.empty(max(int(self.lib.mi355_act_bytes(max(E, H * D), T)), int(self.lib.mi355_act_q8k_tiled_bytes(max(E, H * D), T))) + 256,
+                                 dtype=torch.uint8, device=dev)
+        self.act_b = torch.empty(max(int(self.lib.mi355_act_bytes(F, T)), int(self.lib.mi355_act_q8k_tiled_bytes(F, T))) + 256, dtype=torch.uint8, device=dev)
         self.act_c = torch.empty(int(self.lib.mi355_act_bytes(max(E, H * D), 4)) + 256, dtype=torch.uint8, device=dev)
         self.tickets = torch.zeros(F // 32 + 64, dtype=torch.int32, device=dev)   # arrival counters of the tail-fused launches
         self.ws = torch.empty(int(self.lib.mi355_mul_mat_ws_bytes(kmax, T)) + 256, dtype=torch.uint8, device=dev)
@@ -186,16 +191,29 @@ class LlamaRunner:
             self.planes[key] = buf
         return self.planes[key]
 
+    def _tiles(self, t, W, N, K):
+        """tile images of a K-quant matrix's two int8 planes + per-super-block scales, built on first use and kept"""
+        key = W.data_ptr()
+        if key not in self.tiles:
+            buf = torch.empty(int(self.lib.mi355_kq_tiles_bytes(t, N, K)) + 256, dtype=torch.uint8, device=self.dev)
+            check(self.lib.mi355_kq_unpack_tiles(_stream(), t, _ptr(W), _ptr(buf), N, K))
+            self.tiles[key] = buf
+        return self.tiles[key]
+
+    def _fmt(self, mats, K, T):
+        """activation format of a product: 0 Q8_1 blocks, 1 one scale per 256 elements (K-quant tile GEMM), 2 the same as tile images"""
+        if T <= 8 or not self._q8k_ok(mats, K):
+            return 0
+        return 2 if (self.use_tiles and T >= 33) else 1
+
     def _quant(self, src, act, K, T, q8k):
-        fn = self.lib.mi355_quantize_act_q8k if q8k else self.lib.mi355_quantize_act
+        fn = (self.lib.mi355_quantize_act, self.lib.mi355_quantize_act_q8k, self.lib.mi355_quantize_act_q8k_tiled)[int(q8k)]
         check(fn(_stream(), _ptr(src), _ptr(act), K, T, src.stride(0)))
 
-    def _norm_quant(self, x, w, act, T, q8k=False):
+    def _norm_quant(self, x, w, act, T, q8k=0):
         K = x.shape[1]
-        if q8k:     # prefill: one scale per 256 elements
-            check(self.lib.mi355_rms_norm_mul_quant_q8k(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
-        else:
-            check(self.lib.mi355_rms_norm_mul_quant(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
+        fn = (self.lib.mi355_rms_norm_mul_quant, self.lib.mi355_rms_norm_mul_quant_q8k, self.lib.mi355_rms_norm_mul_quant_q8k_tiled)[int(q8k)]
+        check(fn(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
 
     def _mm_act(self, mats, act, K, T, residual=None, q8k=False):
         """mats: list of ((type, W), out); all consume the quantized activation `act` (T rows of K)"""
@@ -209,12 +227,15 @@ class LlamaRunner:
             for (t, W), out in mats:
                 if q8k:     # the residual add is the tile kernel's epilogue; products with few tiles are split along K through split_ws
                     N = out.shape[1]
-                    need = int(self.lib.mi355_mul_mat_q8k_ws_bytes(N, K, T))
+                    need = int(self.lib.mi355_mul_mat_q8k_tiled_ws_bytes(N, K, T) if q8k == 2 else self.lib.mi355_mul_mat_q8k_ws_bytes(N, K, T))
                     if self.split_ws is None or self.split_ws.numel() < need:
                         self.split_ws = torch.empty(need + 256, dtype=torch.uint8, device=self.dev)
                     sw, sn = (_ptr(self.split_ws), self.split_ws.numel()) if need else (None, 0)
                     res = _ptr(residual) if residual is not None else None
-                    if t == Q6_K and self.use_planes:   # Q6_K streams its int8 planes, unpacked once per matrix
+                    if q8k == 2:
+                        check(self.lib.mi355_mul_mat_q8k_tiled(_stream(), t, _ptr(self._tiles(t, W, N, K)), _ptr(act), _ptr(out), res, N, K, T,
+                                                               out.stride(0), sw, sn))
+                    elif t == Q6_K and self.use_planes:   # Q6_K streams its int8 planes, unpacked once per matrix
                         check(self.lib.mi355_mul_mat_q8k_planes_ws(_stream(), t, _ptr(self._planes(t, W, N, K)), _ptr(act), _ptr(out), res, N, K, T,
                                                                    out.stride(0), sw, sn))
                     else:
@@ -232,10 +253,9 @@ class LlamaRunner:
         x = self.x[:T]
         if T <= 4 and self.fuse_qkv and (T == 1 or not last_only):
             return self._forward_decode(T, n_kv)
-        big = T > 8
         for il, L in enumerate(w.layers):
             qkv = [(L["wq"], self.q[:T]), (L["wk"], self.k[:T]), (L["wv"], self.v[:T])]
-            kq = big and self._q8k_ok(qkv, E)
+            kq = self._fmt(qkv, E, T)
             self._norm_quant(x, L["attn_norm"], self.act_a, T, kq)
             kc, vc = self.kcache[il], self.vcache[il]
             if T <= 4 and self.fuse_qkv:    # decode: projections, rope and KV store in one launch
@@ -249,28 +269,26 @@ class LlamaRunner:
                                               None, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2, vc.stride(1) * 2, D, 0,
                                               cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
             wo = [(L["wo"], x)]
-            kq = big and self._q8k_ok(wo, H * D)
+            kq = self._fmt(wo, H * D, T)
             if kq:
                 self._attn(il, T, n_kv)
-                self._quant(self.attn, self.act_a, H * D, T, True)
+                self._quant(self.attn, self.act_a, H * D, T, kq)
             else:
                 self._attn(il, T, n_kv, act=self.act_a)   # attention writes its own Q8_1 output
             self._mm_act(wo, self.act_a, H * D, T, residual=x, q8k=kq)
             gu = [(L["gate"], self.gate[:T]), (L["up"], self.up[:T])]
-            kq = big and self._q8k_ok(gu, E)
+            kq = self._fmt(gu, E, T)
             self._norm_quant(x, L["ffn_norm"], self.act_a, T, kq)
             self._mm_act(gu, self.act_a, E, T, q8k=kq)
             down = [(L["down"], x)]
-            kq = big and self._q8k_ok(down, F)
-            if kq:
-                check(lib.mi355_swiglu_quant_q8k(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
-            else:
-                check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
+            kq = self._fmt(down, F, T)
+            fn = (lib.mi355_swiglu_quant, lib.mi355_swiglu_quant_q8k, lib.mi355_swiglu_quant_q8k_tiled)[kq]
+            check(fn(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
             self._mm_act(down, self.act_b, F, T, residual=x, q8k=kq)
         To = 1 if last_only else T
         xo = self.x[T - 1:T] if last_only else x
         out = [(w.output, self.logits[:To])]
-        kq = To > 8 and self._q8k_ok(out, E)
+        kq = self._fmt(out, E, To)
         self._norm_quant(xo, w.output_norm, self.act_a, To, kq)
         self._mm_act(out, self.act_a, E, To, q8k=kq)
         return self.logits[:To]

@@ -222,3 +222,110 @@ def test_unaligned_rows_fallback(dev, name, t):
         # (5..32 rows: the weight-streaming kernel with Q8_1 activations)
         want = orc.mul_mat("cpu" if (t == orc.Q4_K and B > 32) else "q8_1", t, Wq, x)
         assert orc.nmse(got, want) < 1e-9
+
+
+KQ_TYPES = [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q6_K)]
+
+
+def _tile_off(row, k, K):
+    """byte offset of element (row, k) in a tile image (16 rows x 64 elements per 1 KiB tile, chunk c of row r at c ^ ((r >> 2) & 3))"""
+    r, c = row & 15, (k >> 4) & 3
+    return ((row >> 4) * (K >> 6) + (k >> 6)) * 1024 + r * 64 + ((c ^ ((r >> 2) & 3)) << 4) + (k & 15)
+
+
+@pytest.mark.parametrize("K,B", [(256, 5), (4096, 33), (14336, 130)])
+def test_quantize_q8k_tiled_bit_exact(dev, K, B):
+    """the tile-image form holds the same levels, scales and sub-block sums as block_q8_K of the reference"""
+    import mi355
+    rng = np.random.default_rng(23 + K)
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    x[0, :256] = 0.0
+    got = mi355.quantize_act_q8k_tiled(_to_dev(dev, x)).cpu().numpy()
+    nsb, b16 = K // 256, (B + 15) // 16 * 16
+    cb_pad = ((b16 // 16) + 15) // 16 * 16
+    rows, ks = np.meshgrid(np.arange(B), np.arange(K), indexing="ij")
+    q = got[_tile_off(rows, ks, K)].view(np.int8).reshape(B, nsb, 256)
+    aux = got[b16 * K:]
+    want = orc.quantize("oracle", orc.Q8_K, x).reshape(B, nsb, 292)
+    wd = np.ascontiguousarray(want[:, :, :4]).view(np.float32).reshape(B, nsb)
+    wq = want[:, :, 4:260].view(np.int8)
+    assert np.array_equal(q, wq)
+    sums = wq.astype(np.int64).reshape(B, nsb, 8, 32).sum(axis=3)
+    for b in range(B):
+        for sb in range(nsb):
+            e = aux[(sb * cb_pad + b // 16) * 576:][:576]
+            d = e[:64].view(np.float32)[b % 16]
+            bs = e[64:].view(np.float16).reshape(16, 16)[b % 16].astype(np.int64)
+            assert d.view(np.uint32) == wd[b, sb].view(np.uint32)
+            assert np.array_equal(64 * bs[8:] + bs[:8], sums[b, sb])
+    if orc.ref is not None:
+        assert np.array_equal(want, orc.quantize("ref", orc.Q8_K, x).reshape(B, nsb, 292))
+
+
+@pytest.mark.parametrize("name,t", KQ_TYPES)
+@pytest.mark.parametrize("N,K,B", [(512, 4096, 64), (384, 2048, 512), (130, 2048, 33), (128, 14336, 100), (200, 2048, 77), (1000, 6144, 300)])
+@pytest.mark.parametrize("split", [False, True])
+def test_mmq_tiled_matches_oracle(dev, name, t, N, K, B, split):
+    """the wide-tile K-quant GEMM on tile images: the CPU's own integer sums (ggml-cpu-quants.c:6817-6848, 8262-8283), ragged row and
+    batch counts, with and without slices along K, with a residual; against the oracle, ggml-cpu and the 64 x 128 tile kernel"""
+    import torch
+    import mi355
+    rng = np.random.default_rng(N * 7 + K + B)
+    Wq = _weights(rng, t, N, K, "ref")
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    res = rng.standard_normal((B, N)).astype(np.float32)
+    Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
+    tiles = mi355.kq_unpack_tiles(t, Wd)
+    act = mi355.quantize_act_q8k_tiled(_to_dev(dev, x))
+    got = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B, split=split).cpu().numpy()
+    got_res = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B, residual=_to_dev(dev, res), split=split).cpu().numpy()
+    assert np.array_equal(got_res, got + res)
+    Nt, Bt = min(N, 64), min(B, 24)
+    assert orc.nmse(got[:Bt, :Nt], orc.mul_mat("cpu", t, Wq[:Nt], x[:Bt])) < 1e-9
+    # the last rows and columns (partial tiles)
+    assert orc.nmse(got[B - 5:, N - 7:], orc.mul_mat("cpu", t, Wq[N - 7:], x[B - 5:])) < 1e-9
+    old = torch.empty((B, N), dtype=torch.float32, device=dev)
+    a2 = mi355.quantize_act_q8k(_to_dev(dev, x))
+    mi355.check(mi355.load().mi355_mul_mat_q8k(None, t, Wd.data_ptr(), a2.data_ptr(), old.data_ptr(), N, K, B, N))
+    torch.cuda.synchronize()
+    assert orc.nmse(got, old.cpu().numpy()) < 1e-12      # same integer sums, f32 summation order only
+    if orc.ref is not None:
+        assert orc.nmse(got, orc.mul_mat("ref", t, Wq, x)) <= 5e-4      # tests/test-backend-ops.cpp:1916
+
+
+@pytest.mark.parametrize("name,t", KQ_TYPES)
+def test_fused_producers_write_tile_images(dev, name, t):
+    """RMS_NORM+MUL and SiLU*up with the tile-image activation output equal the separate quantization of their f32 result"""
+    import torch
+    import mi355
+    lib = mi355.load()
+    rng = np.random.default_rng(3)
+    B, K = 37, 4096
+    x = _to_dev(dev, rng.standard_normal((B, K)).astype(np.float32))
+    w = _to_dev(dev, rng.standard_normal(K).astype(np.float32))
+    nbytes = lib.mi355_act_q8k_tiled_bytes(K, B)
+    y = torch.empty((B, K), dtype=torch.float32, device=dev)
+    a1 = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_rms_norm_mul_quant_q8k_tiled(None, x.data_ptr(), K, w.data_ptr(), y.data_ptr(), K, a1.data_ptr(), K, B, 1e-5))
+    a2 = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_quantize_act_q8k_tiled(None, y.data_ptr(), a2.data_ptr(), K, B, K))
+    torch.cuda.synchronize()
+    rows, ks = np.meshgrid(np.arange(B), np.arange(K), indexing="ij")
+    sel = _tile_off(rows, ks, K)
+    assert np.array_equal(a1.cpu().numpy()[sel], a2.cpu().numpy()[sel])
+    b16 = (B + 15) // 16 * 16
+    n1, n2 = a1.cpu().numpy()[b16 * K:], a2.cpu().numpy()[b16 * K:]
+    cb_pad = ((b16 // 16) + 15) // 16 * 16
+    for sb in range(K // 256):
+        for cb in range(b16 // 16):
+            nrow = min(16, B - cb * 16)
+            e1, e2 = n1[(sb * cb_pad + cb) * 576:][:576], n2[(sb * cb_pad + cb) * 576:][:576]
+            assert np.array_equal(e1[:4 * nrow], e2[:4 * nrow]) and np.array_equal(e1[64:64 + 32 * nrow], e2[64:64 + 32 * nrow])
+    g = _to_dev(dev, rng.standard_normal((B, K)).astype(np.float32))
+    u = _to_dev(dev, rng.standard_normal((B, K)).astype(np.float32))
+    a3 = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_swiglu_quant_q8k_tiled(None, g.data_ptr(), u.data_ptr(), K, y.data_ptr(), K, a3.data_ptr(), K, B))
+    a4 = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_quantize_act_q8k_tiled(None, y.data_ptr(), a4.data_ptr(), K, B, K))
+    torch.cuda.synchronize()
+    assert np.array_equal(a3.cpu().numpy()[sel], a4.cpu().numpy()[sel])
