@@ -141,7 +141,27 @@ def sweep(kinds):
                     ops = 2.0 * N * K * B
                     emit(kernel="MUL_MAT batch %d (activation quantization + tile GEMM)" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
                          achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
-                    if t == mi355.Q6_K and B == 512:   # the same product from the unpacked planes (what prefill uses for Q6_K)
+                    if t in (mi355.Q4_K, mi355.Q6_K):   # the wide-tile GEMM on tile images (what prefill uses for K-quants), without the quantization
+                        tiles = [mi355.kq_unpack_tiles(t, W) for W in Ws]
+                        a8 = mi355.quantize_act_q8k_tiled(x)
+                        sws = torch.empty(int(lib.mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B)) + 256, dtype=torch.uint8, device=dev)
+                        us = timed(lambda i: mi355.check(lib.mi355_mul_mat_q8k_tiled(stream.cuda_stream, t, tiles[i].data_ptr(), a8.data_ptr(), out.data_ptr(), None,
+                                                                                     N, K, B, N, sws.data_ptr(), sws.numel())), nm, 5)
+                        # the shader clock while this kernel runs back to back: a one-wave probe on a second stream
+                        probe = torch.zeros(2, dtype=torch.int64, device=dev)
+                        side = torch.cuda.Stream()
+                        with torch.cuda.stream(stream):
+                            for _ in range(int(1500 / us) + 8):
+                                mi355.check(lib.mi355_mul_mat_q8k_tiled(stream.cuda_stream, t, tiles[0].data_ptr(), a8.data_ptr(), out.data_ptr(), None, N, K, B, N,
+                                                                        sws.data_ptr(), sws.numel()))
+                        mi355.check(lib.mi355_probe_clock(side.cuda_stream, probe.data_ptr(), 500))
+                        torch.cuda.synchronize()
+                        mhz = float(probe[0]) / max(float(probe[1]), 1.0) * 100.0
+                        emit(kernel="wide-tile GEMM on tile images, batch %d" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
+                             achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops,
+                             shader_clock_mhz=round(mhz), frac_at_measured_clock=round(ops / us / 1e6 / (INT8_PEAK_TOPS * mhz / 2400.0), 4))
+                        del tiles
+                    if t == mi355.Q6_K and B == 512:   # the same product from the unpacked planes (the 64 x 128 tile kernel)
                         planes = [torch.empty(int(lib.mi355_kq_planes_bytes(N, K)) + 256, dtype=torch.uint8, device=dev) for _ in range(nm)]
                         for W, P in zip(Ws, planes):
                             mi355.check(lib.mi355_kq_unpack_planes(None, t, W.data_ptr(), P.data_ptr(), N, K))

@@ -40,6 +40,11 @@ const char *mi355_last_error(void);
  * Counterpart of a backend's score function (ggml/src/ggml-backend-impl.h:212-214). */
 int mi355_device_supported(int device);
 
+/* Measurement aid, no counterpart in the reference: one wave spins for `micros` microseconds on `stream` and writes
+ * out[0] = shader-clock ticks, out[1] = ticks of the constant 100 MHz reference counter that passed meanwhile (DEVICE int64[2]).
+ * Launched on a second stream next to a kernel under test, out[0] / out[1] * 100 is the clock in MHz that kernel gets. */
+int mi355_probe_clock(void *stream, int64_t *out, int64_t micros);
+
 /* Weight storage -------------------------------------------------------------------- *
  * Quantized weight rows are kept in HBM in a per-row "device layout" that makes every
  * load a 16-byte aligned, coalesced access:

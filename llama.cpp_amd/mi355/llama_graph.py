@@ -99,8 +99,9 @@ class LlamaRunner:
         self.fuse_qkv = True    # rows must be 16-byte aligned; set False to use the three-launch sequence
         self.use_planes = True  # prefill: Q6_K matrices go through their unpacked int8 planes (2 bytes per weight more, kept resident)
         self.planes = {}
-        # prefill from 33 tokens on: K-quant matrices go through the wide-tile GEMM, which reads tile images of the weights' two
-        # int8 planes (a second copy, 2 bytes per weight, built on first use and kept) and of the quantized activations
+        # prefill from 192 tokens on: K-quant matrices go through the wide-tile GEMM, which reads tile images of the weights' two
+        # int8 planes (a second copy, 2 bytes per weight, built on first use and kept) and of the quantized activations; below
+        # that the 2 bytes per weight make the product HBM-bound and the kernel that unpacks the 4.5-bit rows wins
         self.use_tiles = True
         self.tiles = {}
         self.split_ws = None    # partial sums of tile products that are split along K (grown on first use, before any graph capture)
@@ -204,7 +205,7 @@ class LlamaRunner:
         """activation format of a product: 0 Q8_1 blocks, 1 one scale per 256 elements (K-quant tile GEMM), 2 the same as tile images"""
         if T <= 8 or not self._q8k_ok(mats, K):
             return 0
-        return 2 if (self.use_tiles and T >= 33) else 1
+        return 2 if (self.use_tiles and T >= 192) else 1
 
     def _quant(self, src, act, K, T, q8k):
         fn = (self.lib.mi355_quantize_act, self.lib.mi355_quantize_act_q8k, self.lib.mi355_quantize_act_q8k_tiled)[int(q8k)]
