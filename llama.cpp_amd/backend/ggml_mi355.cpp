@@ -90,11 +90,11 @@ struct device_ctx {
 struct act_cache {
     const void * src = nullptr;   // data pointer of the f32 tensor this was quantized from (B rows of K, contiguous)
     int64_t K = 0, B = 0;
-    int format = 0;               // ACT_Q8_1 (32-element blocks, GEMV) or ACT_Q8K (256-element super-blocks, tile GEMM)
+    int format = 0;               // ACT_Q8_1 (32-element blocks, GEMV), ACT_Q8K (256-element super-blocks, tile GEMM) or ACT_Q8KT (the same as tile images)
     bool valid = false;
     void * ptr = nullptr;         // where the quantized form lives (one of the two slots of backend_ctx::act)
 };
-enum { ACT_Q8_1 = 1, ACT_Q8K = 2 };
+enum { ACT_Q8_1 = 1, ACT_Q8K = 2, ACT_Q8KT = 3 };
 
 struct backend_ctx {
     int device = 0;
@@ -271,12 +271,61 @@ plane_store & planes() {
     return p;
 }
 
+// Tile images of K-quant weight matrices for the wide-tile GEMM (mi355_kq_unpack_tiles: both int8 planes cut into 1 KiB tiles plus
+// per-super-block scales, 2 bytes per weight), built the first time a matrix in a weights buffer meets a batch of TILE_MIN_BATCH
+// rows or more and kept until that buffer is freed or the tensor is written again.  Keyed by the tensor's data address.
+// MI355_NO_TILES=1 keeps the packed rows only.  Below TILE_MIN_BATCH rows the second copy's 2 bytes per weight make the product
+// HBM-bound and the kernels that unpack the packed rows are quicker.
+constexpr int64_t TILE_MIN_BATCH = 192;
+struct tile_store {
+    std::mutex mu;
+    struct entry { void * tiles; int64_t rows, K; };
+    std::unordered_map<const void *, entry> map;
+    bool enabled = getenv("MI355_NO_TILES") == nullptr;
+
+    const void * get(hipStream_t s, const ggml_tensor * w) {
+        if (!enabled || (w->type != GGML_TYPE_Q4_K && w->type != GGML_TYPE_Q6_K) || w->buffer == nullptr ||
+            w->buffer->usage != GGML_BACKEND_BUFFER_USAGE_WEIGHTS)
+            return nullptr;
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = map.find(w->data);
+        if (it != map.end()) return it->second.rows == w->ne[1] && it->second.K == w->ne[0] ? it->second.tiles : nullptr;
+        if (!ggml_is_contiguous(w)) return nullptr;
+        void * tiles = nullptr;
+        if (hipMalloc(&tiles, mi355_kq_tiles_bytes(to_mi355_type(w->type), w->ne[1], w->ne[0]) + 256) != hipSuccess) {   // out of memory: stay with the packed rows
+            (void) hipGetLastError();
+            enabled = false;
+            return nullptr;
+        }
+        MI355_K_OK(mi355_kq_unpack_tiles(s, to_mi355_type(w->type), w->data, tiles, w->ne[1], w->ne[0]));
+        map.emplace(w->data, entry{tiles, w->ne[1], w->ne[0]});
+        return tiles;
+    }
+    // forget (and free) the images of tensors whose data lies in [base, base + size); the caller has synchronized the device
+    void drop(const void * base, size_t size) {
+        std::lock_guard<std::mutex> lock(mu);
+        for (auto it = map.begin(); it != map.end();) {
+            if ((const char *) it->first >= (const char *) base && (const char *) it->first < (const char *) base + size) {
+                MI355_HIP_OK(hipFree(it->second.tiles));
+                it = map.erase(it);
+            } else {
+                ++it;
+            }
+        }
+    }
+};
+tile_store & tiles() {
+    static tile_store t;
+    return t;
+}
+
 // ------------------------------------------------------------------------------- buffer
 void buffer_free(ggml_backend_buffer_t buffer) {
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
     planes().drop(ctx->base, ctx->size);
+    tiles().drop(ctx->base, ctx->size);
     if (ctx->base) MI355_HIP_OK(hipFree(ctx->base));
     delete ctx;
 }
@@ -293,9 +342,10 @@ void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     if (size == 0) return;
-    if (tensor->type == GGML_TYPE_Q6_K) {
+    if (tensor->type == GGML_TYPE_Q6_K || tensor->type == GGML_TYPE_Q4_K) {
         MI355_HIP_OK(hipDeviceSynchronize());
         planes().drop(tensor->data, ggml_nbytes(tensor));   // rebuilt from the new contents on next use
+        tiles().drop(tensor->data, ggml_nbytes(tensor));
     }
     if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
         MI355_HIP_OK(hipDeviceSynchronize());
@@ -345,6 +395,7 @@ bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, gg
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
     if (dst->type == GGML_TYPE_Q6_K) planes().drop(dst->data, ggml_nbytes(dst));
+    if (dst->type == GGML_TYPE_Q6_K || dst->type == GGML_TYPE_Q4_K) tiles().drop(dst->data, ggml_nbytes(dst));
     MI355_HIP_OK(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyDeviceToDevice));
     MI355_HIP_OK(hipDeviceSynchronize());
     return true;
@@ -355,6 +406,7 @@ void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
     planes().drop(ctx->base, ctx->size);
+    tiles().drop(ctx->base, ctx->size);
     MI355_HIP_OK(hipMemset(ctx->base, value, ctx->size));
     MI355_HIP_OK(hipDeviceSynchronize());
 }
@@ -818,8 +870,7 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
     const ggml_tensor * b = mm->src[1];
     if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
-    static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;
-    if (b->ne[1] > (no_skinny ? 8 : 32) || b->nb[1] != b->ne[0] * sizeof(float)) return false;
+    if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
     const int64_t K = a->ne[0];
     if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)
@@ -831,8 +882,7 @@ bool is_q8k_tile_candidate(const ggml_tensor * mm) {
     const ggml_tensor * b = mm->src[1];
     if (mm->op != GGML_OP_MUL_MAT || (a->type != GGML_TYPE_Q4_K && a->type != GGML_TYPE_Q6_K)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
-    static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;
-    if (b->ne[1] <= (no_skinny ? 8 : 32) || b->nb[1] % 16 != 0) return false;
+    if (b->ne[1] <= 32 || b->nb[1] % 16 != 0) return false;
     const int64_t K = a->ne[0];
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;
     return ((uintptr_t) a->data & 15) == 0 && ((uintptr_t) b->data & 15) == 0;
@@ -853,6 +903,11 @@ bool feeds_q8k_tiles(const graph_walk & w, int i, const void * data, int64_t K, 
     const ggml_tensor * mm = w.nodes[j];
     return is_q8k_tile_candidate(mm) && mm->src[1]->data == data && mm->src[0]->ne[0] == K && mm->src[1]->ne[1] == B &&
            mm->src[1]->nb[1] == (size_t) K * sizeof(float);
+}
+
+// activation format of a K-quant tile product: tile images when the batch is large and the weights have (or can get) theirs
+int q8k_format_for(hipStream_t s, const ggml_tensor * mm) {
+    return mm->src[1]->ne[1] >= TILE_MIN_BATCH && tiles().get(s, mm->src[0]) != nullptr ? ACT_Q8KT : ACT_Q8K;
 }
 
 // A MUL_MAT_ID with few (token, expert slot) pairs streams each slot's expert through the GEMV on Q8_1 activations; with many
@@ -904,9 +959,13 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             memcpy(&eps, node->op_params, sizeof(float));
             void * act = nullptr;
             if (rows > 8 && feeds_q8k_tiles(w, j, nxt->data, K, rows)) {   // prefill: the per-super-block form for the tile GEMM
-                act = ctx->act_slot(mi355_act_q8k_bytes(K, rows));
-                MI355_K_OK(mi355_rms_norm_mul_quant_q8k(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
-                ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8K, true, act};
+                const int fmt = q8k_format_for(s, w.nodes[w.next(j)]);
+                act = ctx->act_slot(fmt == ACT_Q8KT ? mi355_act_q8k_tiled_bytes(K, rows) : mi355_act_q8k_bytes(K, rows));
+                if (fmt == ACT_Q8KT)
+                    MI355_K_OK(mi355_rms_norm_mul_quant_q8k_tiled(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
+                else
+                    MI355_K_OK(mi355_rms_norm_mul_quant_q8k(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
+                ctx->cache = act_cache{nxt->data, K, rows, fmt, true, act};
                 return j;
             }
             if (rows <= 32 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
@@ -944,9 +1003,13 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 }
                 void * act = nullptr;
                 if (rows > 8 && feeds_q8k_tiles(w, jm, mul->data, K, rows)) {
-                    act = ctx->act_slot(mi355_act_q8k_bytes(K, rows));
-                    MI355_K_OK(mi355_swiglu_quant_q8k(s, (const float *) gt->data, (const float *) up->data, K, (float *) mul->data, K, act, K, rows));
-                    ctx->cache = act_cache{mul->data, K, rows, ACT_Q8K, true, act};
+                    const int fmt = q8k_format_for(s, w.nodes[w.next(jm)]);
+                    act = ctx->act_slot(fmt == ACT_Q8KT ? mi355_act_q8k_tiled_bytes(K, rows) : mi355_act_q8k_bytes(K, rows));
+                    if (fmt == ACT_Q8KT)
+                        MI355_K_OK(mi355_swiglu_quant_q8k_tiled(s, (const float *) gt->data, (const float *) up->data, K, (float *) mul->data, K, act, K, rows));
+                    else
+                        MI355_K_OK(mi355_swiglu_quant_q8k(s, (const float *) gt->data, (const float *) up->data, K, (float *) mul->data, K, act, K, rows));
+                    ctx->cache = act_cache{mul->data, K, rows, fmt, true, act};
                     return jm;
                 }
                 if ((rows <= 32 && feeds_quant_gemv(w, jm, mul->data, K, rows)) || (rows <= 8 && feeds_quant_mmid(w, jm, mul->data, K, rows)))
@@ -1119,20 +1182,13 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 }
                 const void * act_in = ctx->cache.ptr;
                 void * act_out = ctx->act_slot(out_bytes, true);
-                // Two launches (two-matrix product, then SiLU*up + Q8_1) are a little quicker than the one whose last groups do
-                // the tail (15.9 us against 16.3-16.8 us on 2 x 14336 x 4096); MI355_FUSED_TAIL=1 selects the latter.  Same bits.
-                static const bool fused_tail = getenv("MI355_FUSED_TAIL") != nullptr;
-                if (fused_tail) {
-                    MI355_K_OK(mi355_ffn_gate_up_swiglu(s, to_mi355_type(node->src[0]->type), node->src[0]->data, to_mi355_type(up->src[0]->type),
-                                                        up->src[0]->data, act_in, (float *) node->data, (float *) up->data, N, act_out,
-                                                        ctx->ticket_buffer((size_t) (N / 32)), N, K, B));
-                } else {
-                    mi355_gemv_mat gu[2];
-                    gu[0] = mi355_gemv_mat{to_mi355_type(node->src[0]->type), node->src[0]->data, N, (float *) node->data, N, nullptr};
-                    gu[1] = mi355_gemv_mat{to_mi355_type(up->src[0]->type), up->src[0]->data, N, (float *) up->data, N, nullptr};
-                    MI355_K_OK(mi355_mul_mat_vec_q_multi(s, 2, gu, act_in, K, B));
-                    MI355_K_OK(mi355_swiglu_quant(s, (const float *) node->data, (const float *) up->data, N, nullptr, 0, act_out, N, B));
-                }
+                // Two launches (two-matrix product, then SiLU*up + Q8_1) are a little quicker than mi355_ffn_gate_up_swiglu, whose
+                // last groups do the tail (15.9 us against 16.3-16.8 us on 2 x 14336 x 4096).  Same bits.
+                mi355_gemv_mat gu[2];
+                gu[0] = mi355_gemv_mat{to_mi355_type(node->src[0]->type), node->src[0]->data, N, (float *) node->data, N, nullptr};
+                gu[1] = mi355_gemv_mat{to_mi355_type(up->src[0]->type), up->src[0]->data, N, (float *) up->data, N, nullptr};
+                MI355_K_OK(mi355_mul_mat_vec_q_multi(s, 2, gu, act_in, K, B));
+                MI355_K_OK(mi355_swiglu_quant(s, (const float *) node->data, (const float *) up->data, N, nullptr, 0, act_out, N, B));
                 ctx->cache = act_cache{mul->data, N, B, ACT_Q8_1, true, act_out};
                 return jm;
             }
@@ -1327,8 +1383,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 }
             }
         }
-        static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;   // tuning aid, as in the kernel library
-        if (n_run == 1 && B >= 5 && !no_skinny && mi355_mul_mat_skinny_supported(mats[0].type, mats[0].W, K, B)) {
+        if (n_run == 1 && B >= 5 && mi355_mul_mat_skinny_supported(mats[0].type, mats[0].W, K, B)) {
             // with room for the slices along K that products with few rows are split into
             const size_t split_bytes = mi355_mul_mat_skinny_ws_bytes(mats[0].N, K, B);
             void * split_ws = split_bytes ? ctx->workspace(split_bytes) : nullptr;
@@ -1344,19 +1399,24 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     if (is_q8k_tile_candidate(node)) {
         const ggml_tensor * b = node->src[1];
         const int64_t K = b->ne[0], B = b->ne[1];
-        if (!ctx->cached(b->data, K, B, ACT_Q8K)) {
-            void * fresh = ctx->act_slot(mi355_act_q8k_bytes(K, B));
-            MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
-            ctx->cache = act_cache{b->data, K, B, ACT_Q8K, true, fresh};
+        // large batches: the wide-tile kernel on tile images of the weights (built on first use) and of the activation
+        const int fmt = q8k_format_for(s, node);
+        const void * tl = fmt == ACT_Q8KT ? tiles().get(s, node->src[0]) : nullptr;
+        if (!ctx->cached(b->data, K, B, fmt)) {
+            void * fresh = ctx->act_slot(fmt == ACT_Q8KT ? mi355_act_q8k_tiled_bytes(K, B) : mi355_act_q8k_bytes(K, B));
+            if (fmt == ACT_Q8KT) MI355_K_OK(mi355_quantize_act_q8k_tiled(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
+            else MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
+            ctx->cache = act_cache{b->data, K, B, fmt, true, fresh};
         }
-        const void * pl = planes().get(s, node->src[0]);   // Q6_K weights: the unpacked planes, built on first use
+        const void * pl = tl ? nullptr : planes().get(s, node->src[0]);   // Q6_K weights: the unpacked planes, built on first use
         const int wtype = to_mi355_type(node->src[0]->type);
         const int64_t N = node->src[0]->ne[1];
         // products with few tiles are split along K through the scratch buffer (0 bytes: this shape is not split)
-        const size_t split_bytes = mi355_mul_mat_q8k_ws_bytes(N, K, B);
+        const size_t split_bytes = tl ? mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) : mi355_mul_mat_q8k_ws_bytes(N, K, B);
         void * split_ws = split_bytes ? ctx->workspace(split_bytes) : nullptr;
         auto product = [&](float * out, const float * residual, int64_t out_stride) {
-            if (pl) MI355_K_OK(mi355_mul_mat_q8k_planes_ws(s, wtype, pl, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
+            if (tl) MI355_K_OK(mi355_mul_mat_q8k_tiled(s, wtype, tl, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
+            else if (pl) MI355_K_OK(mi355_mul_mat_q8k_planes_ws(s, wtype, pl, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
             else MI355_K_OK(mi355_mul_mat_q8k_ws(s, wtype, node->src[0]->data, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
         };
         // MUL_MAT -> ADD(residual): the sum goes straight into the ADD's tensor

@@ -303,7 +303,7 @@ template <int D>
 static int launch_vec_r(hipStream_t s, fattn_args &a, int R) {
     // R = query heads served per group from one pass over the kv head's bytes.  A short context is not bandwidth-bound but
     // a serial chain of soft-max updates per (step, head): one head per group then spreads it over R times as many waves.
-    static const int64_t one_head_max = getenv("MI355_FA_ONE_HEAD_MAX") ? atoll(getenv("MI355_FA_ONE_HEAD_MAX")) : 1024;   // tuning aid
+    constexpr int64_t one_head_max = 1024;
     if (a.Nkv <= one_head_max) return launch_vec<D, 1>(s, a);
     if (R % 4 == 0) return launch_vec<D, 4>(s, a);
     if (R % 2 == 0) return launch_vec<D, 2>(s, a);
@@ -364,13 +364,13 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
     // Decode and small batches over a long context: matrix cores with (token, head) columns, which read a kv head's
     // bytes once for its whole GQA group.  Short contexts are latency-bound and mostly padding (-inf mask): the
     // vector kernel, which skips masked cells before touching K/V, is quicker there.
-    static const int64_t dec_min = getenv("MI355_FA_DEC_MIN") ? atoll(getenv("MI355_FA_DEC_MIN")) : 256;   // tuning aid
+    constexpr int64_t dec_min = 256;
     if (Nq < 16 && Nkv > dec_min && (D == 64 || D == 128) && R <= 32) {
         fattn_args b = a;
         // enough splits to put about two groups on every CU; a split is a whole number of 64-cell tiles
         const int64_t tiles = (Nkv + 63) / 64;
         const int64_t nt = 32 / R, base = Hkv * ((Nq + nt - 1) / nt);
-        static const int64_t target_groups = getenv("MI355_FA_DEC_GROUPS") ? atoll(getenv("MI355_FA_DEC_GROUPS")) : 512;   // tuning aid
+        constexpr int64_t target_groups = 512;
         int64_t n = target_groups / base;
         if (n > tiles) n = tiles;
         if (n > 256) n = 256;

@@ -415,14 +415,8 @@ __global__ void __launch_bounds__(64) k_block_dots(const uint8_t *__restrict__ W
 }
 
 // rows per wave: enough waves to cover every SIMD a few times over, then amortise the
-// activation reads over more rows.  MI355_GEMV_RPW overrides (tuning aid).
+// activation reads over more rows.
 static int pick_rpw(int64_t total_rows) {
-    static int forced = -1;
-    if (forced < 0) {
-        const char *e = getenv("MI355_GEMV_RPW");
-        forced = e ? atoi(e) : 0;
-    }
-    if (forced == 1 || forced == 2 || forced == 4) return forced;
     if (total_rows >= 32768) return 4;
     if (total_rows >= 8192) return 2;
     return 1;
@@ -433,7 +427,7 @@ static int pick_rpw(int64_t total_rows) {
 // activation reads it saves are the larger part of the launch's L2 traffic): output projection 98.9 -> 77.5 us (6.8 TB/s),
 // 14336 x 4096 8.6 -> 8.0 us.  A launch whose groups are all resident at once (wo, ffn_down, Q/K/V: ~1000 groups) is one
 // dependent chain per wave, and the copy's barrier lengthens it (+0.3 to +0.7 us measured).  Up to four activation rows, and
-// small enough that eight groups still fit a compute unit.  MI355_GEMV_NO_LDS=1 turns the copy off (tuning aid).
+// small enough that eight groups still fit a compute unit.
 // Measured and not adopted: splitting K over the four waves of a group (each wave reads a quarter of the activation, partial
 // sums meet in LDS at the end) - Q4_K 4096 x 4096 4.9 -> 4.3 us and 14336 x 4096 8.2 -> 7.9 us, but Q6_K slower throughout
 // (4096 x 14336 11.2 -> 14.0 us, output projection 80 -> 87 us): its 16-byte pieces per lane then form 256-byte runs.
@@ -442,9 +436,8 @@ static int pick_rpw(int64_t total_rows) {
 // 8.3 -> 9.9..10.9 us and the output projection 50.6 -> 61..77 us: many short-lived waves keep more loads in flight than few
 // long-lived ones with one block of look-ahead.
 static size_t act_lds_bytes(int ncols, int64_t K, int64_t groups) {
-    static const bool off = getenv("MI355_GEMV_NO_LDS") != nullptr;
     const int64_t bytes = (int64_t)ncols * (K + K / 4);
-    return (!off && groups >= 1536 && ncols <= 4 && bytes <= 20480) ? (size_t)bytes : 0;
+    return (groups >= 1536 && ncols <= 4 && bytes <= 20480) ? (size_t)bytes : 0;
 }
 
 template <int NCOLS>
@@ -538,8 +531,7 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     // From five activation rows on the matrix-core kernel (skinny.hip) is ahead wherever it supports the product; a single
     // Q4_0/Q8_0/Q4_K matrix already at four (14336 x 4096 Q4_K: 14.3 -> 12.0 us, 4096 x 14336: 18.0 -> 14.6 us).
     if (B >= 5 || (B == 4 && n_mats == 1 && mats[0].type != MI355_Q6_K)) {
-        static const bool no_skinny = getenv("MI355_NO_SKINNY") != nullptr;
-        bool ok = !no_skinny;
+        bool ok = true;
         for (int i = 0; i < n_mats; i++) ok = ok && mi355_mul_mat_skinny_supported(mats[i].type, mats[i].W, K, B);
         if (ok) {
             for (int i = 0; i < n_mats; i++) {
@@ -552,7 +544,7 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     MI355_REQUIRE(B <= 8, "mul_mat_vec_q: batch %lld needs the matrix-core kernel, which does not support this product (K a multiple of 256, aligned rows)", (long long)B);
     int rpw = pick_rpw(total_rows);
     if (B > 4 && rpw > 2) rpw = 2;   // keep the accumulator tile in registers
-    if (getenv("MI355_GEMV_RPW") == nullptr && getenv("MI355_GEMV_PLAIN_RPW") == nullptr) {   // per-type corrections, measured on the 8B shapes (off under either tuning variable)
+    {   // per-type corrections, measured on the 8B shapes
         bool any_q6 = false, all_q4k = true;
         for (int i = 0; i < n_mats; i++) {
             any_q6 = any_q6 || mats[i].type == MI355_Q6_K;

@@ -80,10 +80,8 @@ extern "C" {
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B) { return (mi355_act_bytes(K, B) + 255) & ~(size_t)255; }
 
 // 4 or 5 (Q6_K) to 32 activation rows: the weight-streaming matrix-core kernel (skinny.hip) where it supports the product.
-// MI355_NO_SKINNY=1 sends these batches to the batch-1 kernels (up to 8) and the tile kernels as before (tuning aid).
 static bool use_skinny(int type, const void *W, int64_t K, int64_t B) {
-    static const bool off = getenv("MI355_NO_SKINNY") != nullptr;
-    return !off && B >= (type == MI355_Q6_K ? 5 : 4) && B <= 32 && mi355_mul_mat_skinny_supported(type, W, K, B);
+    return B >= (type == MI355_Q6_K ? 5 : 4) && B <= 32 && mi355_mul_mat_skinny_supported(type, W, K, B);
 }
 
 static bool use_q8k_tiles(int type, const void *W, int64_t K, int64_t B) {

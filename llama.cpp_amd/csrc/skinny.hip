@@ -364,10 +364,7 @@ void launch_skinny_nt(hipStream_t s, const void *W, const int8_t *aq, const act_
 
 // slices of K: launches with fewer than ~1.5 groups per compute unit split K over several groups (and pay a second launch
 // that adds the slices), as long as a slice keeps 4 steps; a short K with at most 8 activation rows is quicker in one go.
-// MI355_SKINNY_SLICES overrides (tuning aid).
 int skinny_slices(int64_t N, int64_t K, int64_t B) {
-    static const int forced = getenv("MI355_SKINNY_SLICES") ? atoi(getenv("MI355_SKINNY_SLICES")) : 0;
-    if (forced >= 1 && forced <= 8) return forced;
     const int64_t tiles = (N + 31) / 32, nsteps = K >> 8;
     if (tiles >= 384 || (B <= 8 && nsteps <= 16)) return 1;
     int s = 1;

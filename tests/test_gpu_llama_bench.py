@@ -71,7 +71,7 @@ def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats
     return np.fromfile(out, dtype=np.float32)
 
 
-@pytest.mark.parametrize("n_prompt", [5, 40])
+@pytest.mark.parametrize("n_prompt", [5, 40, 256])   # 256: the wide-tile GEMM on tile images (from 192 rows on)
 def test_model_logits_cpu_vs_plugin_and_fused_vs_nodes(dev, tmp_path, n_prompt):
     """The reference's model runtime produces the same logits on its CPU backend and on the plug-in (up to the
     activation-quantization noise that random weights amplify), and the plug-in's fused graph execution reproduces its
