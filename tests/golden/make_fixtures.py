@@ -7,6 +7,7 @@ the reference's outputs for them, so the oracle can be pinned where the referenc
   q8_1_special.npz   : hand-made blocks (zeros, single +-amax, .5 ties) and quantize_row_q8_1_ref bytes
   mul_mat_<type>.npz : W bytes [48,512], x f32 [3,512], y = reference CPU MUL_MAT output
   flash_attn.npz     : q,k,v,mask for D=64, Nq=3, Nkv=40, Hq=4, Hkv=2 and the reference CPU output
+  flash_attn_alibi_softcap.npz : 6 query heads over 3 kv heads, the reference CPU outputs with max_bias = 8 and with logit_softcap = 10
   glue.npz           : inputs/outputs of RMS_NORM, SOFT_MAX, ROPE (modes 0 and 2), SILU, ARGSORT
 """
 import os
@@ -55,6 +56,18 @@ def main():
     y = orc.flash_attn("ref", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), 0.125)
     np.savez_compressed(os.path.join(HERE, "flash_attn.npz"), q=q, k=k.view(np.uint16), v=v.view(np.uint16), mask=mask.view(np.uint16),
                         y=y, scale=np.float32(0.125))
+    # the ALiBi (max_bias > 0: per-head slopes on the mask) and logit soft-cap branches of the same kernel; 6 heads make
+    # n_head_log2 = 4 < n_head, so both slope formulas are exercised
+    Hq2, Hkv2 = 6, 3
+    rng2 = np.random.default_rng(20240608)   # its own stream: the fixtures below keep their inputs
+    q2 = rng2.standard_normal((Hq2, Nq, D)).astype(np.float32)
+    k2 = rng2.standard_normal((Hkv2, Nkv, D)).astype(np.float16)
+    v2 = rng2.standard_normal((Hkv2, Nkv, D)).astype(np.float16)
+    y_alibi = orc.flash_attn("ref", q2, k2.view(np.uint16), v2.view(np.uint16), mask.view(np.uint16), 0.125, max_bias=8.0)
+    y_cap = orc.flash_attn("ref", q2, k2.view(np.uint16), v2.view(np.uint16), mask.view(np.uint16), 0.125, softcap=10.0)
+    np.savez_compressed(os.path.join(HERE, "flash_attn_alibi_softcap.npz"), q=q2, k=k2.view(np.uint16), v=v2.view(np.uint16),
+                        mask=mask.view(np.uint16), y_alibi=y_alibi, y_softcap=y_cap, scale=np.float32(0.125), max_bias=np.float32(8.0),
+                        softcap=np.float32(10.0))
 
     g = {}
     x = rng.standard_normal((5, 96)).astype(np.float32)

@@ -64,6 +64,18 @@ def test_alibi_and_softcap(dev, max_bias, softcap):
     got = _run(dev, q, k, v, mask, scale, max_bias, softcap)
     f64 = orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale, max_bias, softcap)
     assert orc.nmse(got, f64) < 1e-5
+    assert orc.nmse(got, orc.flash_attn("cpu", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale, max_bias, softcap)) <= 5e-4
+    if orc.ref is not None:
+        assert orc.nmse(got, orc.flash_attn("ref", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale, max_bias, softcap)) <= 5e-4
+
+
+def test_alibi_and_softcap_golden_fixture(dev):
+    """the committed outputs of the reference CPU backend for max_bias = 8 (6 heads: both slope formulas) and logit_softcap = 10"""
+    import os
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "flash_attn_alibi_softcap.npz"))
+    q, k, v, mask, scale = g["q"], g["k"].view(np.float16), g["v"].view(np.float16), g["mask"].view(np.float16), float(g["scale"])
+    assert orc.nmse(_run(dev, q, k, v, mask, scale, float(g["max_bias"]), 0.0), g["y_alibi"]) <= 5e-4
+    assert orc.nmse(_run(dev, q, k, v, mask, scale, 0.0, float(g["softcap"])), g["y_softcap"]) <= 5e-4
 
 
 def test_no_mask(dev):
@@ -75,22 +87,40 @@ def test_no_mask(dev):
 
 @pytest.mark.parametrize("Nq,Nkv", [(1, 512), (1, 4096), (1, 32768), (512, 512), (512, 4096)])
 def test_llama3_shapes(dev, Nq, Nkv):
-    """BASELINE config 2: 32 query heads over 8 kv heads, head size 128, causal, llama's strided layouts.
-    The oracle is evaluated on a slice of heads/queries (it is scalar C); GQA grouping is pinned by
-    the f64 form, which repeats each kv head over its 4 query heads."""
+    """BASELINE config 2: 32 query heads over 8 kv heads, head size 128, causal, llama's strided layouts.  The WHOLE output is
+    held to the reference CPU backend's (NMSE <= 5e-4, tests/test-backend-ops.cpp:3137) and to the textbook form in f64 (which
+    repeats each kv head over its 4 query heads and so pins the grouping); the scalar C oracle checks a slice of heads and
+    queries."""
     rng = np.random.default_rng(Nq + Nkv)
     q, k, v, mask = _inputs(rng, 128, Nq, Nkv, 32, 8, causal=True)
+    if Nkv == 32768:
+        # 32768 near-equal softmax weights over zero-mean values leave outputs of 0.007 and put the reference's own f16
+        # accumulator 6.7e-4 (NMSE) from the exact result; queries three times larger give the peaked weights of a trained
+        # model, where the reference is 4e-5 from exact and its tolerance means something
+        q = q * 3.0
     scale = 1.0 / np.sqrt(128)
     got = _run(dev, q, k, v, mask, scale, llama_layout=True)      # [Nq, 32, 128]
     assert np.isfinite(got).all()
+    assert orc.ref is not None, "the reference build (oracle/_ref) is the whole-output check of this test"
+    want = orc.flash_attn("ref", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale, n_threads=16)
+    assert orc.nmse(got, want) <= 5e-4
+    # textbook softmax(q k^T * scale + mask) v, every head and query, in f64 with q rounded to f16 as the kernels do
+    qh = q.astype(np.float16).astype(np.float64)
+    mf = mask[:Nq].astype(np.float64)
+    full = np.empty((Nq, 32, 128))
+    for h in range(32):
+        s_ = qh[h] @ k[h // 4].astype(np.float64).T * scale + mf
+        p = np.exp(s_ - s_.max(axis=1, keepdims=True))
+        full[:, h] = (p / p.sum(axis=1, keepdims=True)) @ v[h // 4].astype(np.float64)
+    assert orc.nmse(got, full) < 1e-5
     heads = [0, 5, 31]
     rows = sorted(set([0, Nq // 2, Nq - 1]))
     for h in heads:
         qs = q[h:h + 1][:, rows]
         ms = mask[rows]
         ms = np.concatenate([ms, np.full((64 - len(rows), Nkv), -np.inf, dtype=np.float16)])
-        f64 = orc.flash_attn("f64", qs, k[h // 4:h // 4 + 1].view(np.uint16), v[h // 4:h // 4 + 1].view(np.uint16), ms.view(np.uint16), scale)
-        assert orc.nmse(got[rows][:, h:h + 1], f64) < 1e-5
+        cpu = orc.flash_attn("cpu", qs, k[h // 4:h // 4 + 1].view(np.uint16), v[h // 4:h // 4 + 1].view(np.uint16), ms.view(np.uint16), scale)
+        assert orc.nmse(got[rows][:, h:h + 1], cpu) <= 5e-4
 
 
 @pytest.mark.parametrize("D,Nq,Nkv,Hq,Hkv", [(128, 1, 256, 32, 8), (128, 1, 4096, 32, 8), (128, 5, 700, 8, 2), (64, 2, 96, 6, 3), (96, 1, 64, 4, 4)])

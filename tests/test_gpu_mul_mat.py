@@ -188,6 +188,39 @@ def test_skinny_matches_oracle(dev, name, t, N, K, B, split):
         assert orc.nmse(got, orc.mul_mat("ref", t, Wq, x)) <= 5e-4      # tests/test-backend-ops.cpp:1916
 
 
+@pytest.mark.parametrize("name,t", TYPES)
+@pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
+def test_mmq_llama8b_ffn_shapes(dev, name, t, N, K):
+    """the FFN products of an 8B llama (gate/up 14336 x 4096, down 4096 x 14336) at batch 64 and 512, whole: every output against
+    the reference CPU backend (NMSE <= 5e-4, tests/test-backend-ops.cpp:1916), a 64 x 24 corner and the last rows/columns against
+    the oracle's integer arithmetic; the K-quants additionally through their tile images"""
+    import mi355
+    rng = np.random.default_rng(N + K + t)
+    Wq = _weights(rng, t, N, K, "ref")
+    Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
+    kq = t in (orc.Q4_K, orc.Q6_K)
+    tiles = mi355.kq_unpack_tiles(t, Wd) if kq else None
+    for B in (64, 512):
+        x = rng.standard_normal((B, K)).astype(np.float32)
+        xd = _to_dev(dev, x)
+        got = mi355.mul_mat(t, Wd, xd).cpu().numpy()
+        kind = "cpu" if kq else "q8_1"          # K-quants compute in the CPU path's Q8_K format, the others in Q8_1
+        corner = orc.mul_mat(kind, t, Wq[:64], x[:24])
+        edge = orc.mul_mat(kind, t, Wq[N - 9:], x[B - 3:])
+        assert orc.nmse(got[:24, :64], corner) < 1e-9
+        assert orc.nmse(got[B - 3:, N - 9:], edge) < 1e-9
+        assert orc.ref is not None, "the reference build (oracle/_ref) is the whole-output check of this test"
+        want = orc.mul_mat("ref", t, Wq, x, n_threads=16)
+        assert orc.nmse(got, want) <= 5e-4
+        if kq:
+            act = mi355.quantize_act_q8k_tiled(xd)
+            wide = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B).cpu().numpy()
+            assert orc.nmse(wide[:24, :64], corner) < 1e-9
+            assert orc.nmse(wide[B - 3:, N - 9:], edge) < 1e-9
+            assert orc.nmse(wide, want) <= 5e-4
+            assert orc.nmse(wide, got) < 1e-12      # same integer sums in both tile kernels
+
+
 @pytest.mark.parametrize("name,t", [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q6_K)])
 @pytest.mark.parametrize("N,K,B", [(256, 4096, 64), (130, 1024, 33)])
 def test_mmq_q8_1_path_for_k_quants(dev, name, t, N, K, B):

@@ -7,7 +7,6 @@ import orc
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name,t", list(orc.WEIGHT_TYPES.items()))
 def routed(t, n_used, T, K):
     """mi355_mul_mat_id sorts the slots by expert and uses the K-quant tile kernel (ggml-cpu's Q8_K arithmetic)"""
     return T * n_used >= 32 and ((t == orc.Q4_K and K % 256 == 0) or (t == orc.Q6_K and K % 2048 == 0))

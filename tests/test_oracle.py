@@ -210,6 +210,35 @@ def test_flash_attn_golden_and_textbook():
     assert orc.nmse(f64, out) < 1e-12
 
 
+def test_flash_attn_alibi_and_softcap_golden():
+    """the ALiBi slopes (ggml-cpu.c:10979-10995: m0 / m1 powers by head index) and the logit soft-cap (tanh) of the oracle against
+    outputs of the reference build, and against the textbook form with the slope / cap written out"""
+    g = gold("flash_attn_alibi_softcap.npz")
+    q, k, v, mask, scale = g["q"], g["k"], g["v"], g["mask"], float(g["scale"])
+    Hq, Nq, D = q.shape
+    kf, vf = k.view(np.float16).astype(np.float64), v.view(np.float16).astype(np.float64)
+    mf = mask.view(np.float16).astype(np.float64)
+    rep = Hq // kf.shape[0]
+    for key, max_bias, softcap in (("y_alibi", float(g["max_bias"]), 0.0), ("y_softcap", 0.0, float(g["softcap"]))):
+        cpu = orc.flash_attn("cpu", q, k, v, mask, scale, max_bias, softcap)
+        f64 = orc.flash_attn("f64", q, k, v, mask, scale, max_bias, softcap)
+        assert orc.nmse(cpu, g[key]) < 1e-6
+        assert orc.nmse(f64, g[key]) <= 5e-4
+        n2 = 1 << int(np.floor(np.log2(Hq)))
+        m0, m1 = 2.0 ** (-max_bias / n2), 2.0 ** (-max_bias / 2.0 / n2)
+        out = np.zeros((Nq, Hq, D))
+        for h in range(Hq):
+            slope = 1.0 if max_bias == 0.0 else (m0 ** (h + 1) if h < n2 else m1 ** (2 * (h - n2) + 1))
+            s = q[h].astype(np.float64) @ kf[h // rep].T * scale
+            if softcap != 0.0:
+                s = softcap * np.tanh(s / softcap)
+            s = s + slope * mf[:Nq]
+            p = np.exp(s - s.max(axis=1, keepdims=True))
+            p /= p.sum(axis=1, keepdims=True)
+            out[:, h] = p @ vf[h // rep]
+        assert orc.nmse(f64, out) < 1e-10
+
+
 # ------------------------------------------------------------------ glue ops
 def test_glue_golden():
     g = gold("glue.npz")
