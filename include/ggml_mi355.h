@@ -10,13 +10,18 @@
  * ggml/src/ggml-backend-impl.h:17-207), which the plug-in fills:
  *
  *   reg         get_name "MI355X", get_device_count, get_device, get_proc_address (none)
- *   device      GPU type; get_memory (hipMemGetInfo); init_backend; get_buffer_type;
- *               supports_op / supports_buft; no host buffer type, no events, caps all false
+ *   device      GPU type; get_memory (hipMemGetInfo); init_backend; get_buffer_type; a pinned host
+ *               buffer type (hipHostMalloc) for the tensors the CPU backend hands over;
+ *               supports_op / supports_buft; caps: async and host_buffer true,
+ *               buffer_from_host_ptr and events false
  *   buffer type hipMalloc-backed, alignment 256, alloc size = ggml_nbytes
  *   buffer      set/get/memset/cpy_tensor and clear; set/get apply / undo the 16-byte-aligned
  *               device row layout for Q4_0, Q8_0 and Q6_K tensors
- *   backend     one HIP stream; graph_compute enqueues one kernel sequence per node and returns,
- *               synchronize waits for the stream
+ *   backend     one HIP stream; set/get_tensor_async on it; graph_compute walks the graph once,
+ *               matching runs of nodes (norm -> weight -> products -> rope -> cache store, gate/up
+ *               -> SiLU*up -> down, ...) to one fused kernel each, records the launches of a
+ *               decode-shaped graph into a HIP graph keyed by the graph's signature and replays
+ *               it on later calls; synchronize waits for the stream
  *
  * The library has no link-time dependency on libggml-base: the handful of ggml symbols it calls
  * (ggml_backend_buffer_init, ggml_nbytes, ggml_is_contiguous, ...) resolve against the host

@@ -36,6 +36,9 @@ enum mi355_type {
 int mi355_abi_version(void);
 /* Text of the last error on the calling thread ("" if none). */
 const char *mi355_last_error(void);
+/* Kernel launches this library has issued in this process so far (every entry point counts each of its launches, also while a
+ * stream is being captured).  A host that fuses graph nodes reads it before and after a graph to report launches per graph. */
+uint64_t mi355_launch_count(void);
 /* 1 if `device` is a gfx950 GPU this library can run on, 0 if not, <0 on HIP error.
  * Counterpart of a backend's score function (ggml/src/ggml-backend-impl.h:212-214). */
 int mi355_device_supported(int device);
@@ -360,6 +363,13 @@ typedef struct mi355_rope_desc {
 } mi355_rope_desc;
 int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat *mats, const void *act, int64_t K, int64_t B,
                              const mi355_rope_desc *rope);
+
+/* The same launch for ONE activation row that is still to be normalised: RMS_NORM(x) -> MUL(norm_w) -> Q8_1 (llm_build_norm,
+ * src/llama.cpp:1506-1511; ggml-cpu.c:6741-6805) done by every group for itself, then the products and epilogues of
+ * mi355_mul_mat_vec_q_rope.  Bit-identical to mi355_rms_norm_mul_quant followed by mi355_mul_mat_vec_q_rope; neither the
+ * normalised f32 row nor its Q8_1 form is written to memory.  K <= 4096 and a multiple of 1024; x, norm_w 16-byte aligned. */
+int mi355_rms_norm_mul_mat_vec_q_rope(void *stream, const float *x, const float *norm_w, float eps, int n_mats, const mi355_gemv_rope_mat *mats,
+                                      int64_t K, const mi355_rope_desc *rope);
 
 /* The Q, K and V projections of build_llama (src/llama.cpp:1514-1533) in ONE bandwidth-bound launch whose epilogue does what the graph
  * does next: ROPE(q) into q f32 [B][H][D]; ROPE(k) and CPY into the f16 K cache; CPY(v) into the f16 V cache (src/llama.cpp:1535-1548,

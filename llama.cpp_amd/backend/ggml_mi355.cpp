@@ -27,10 +27,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <unordered_map>
-#include <unordered_set>
 #include <vector>
 
 #include "mi355_kernels.h"
@@ -96,6 +96,8 @@ struct act_cache {
 };
 enum { ACT_Q8_1 = 1, ACT_Q8K = 2, ACT_Q8KT = 3 };
 
+constexpr int IOTA_N = 16384;
+
 struct backend_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -105,7 +107,16 @@ struct backend_ctx {
     size_t act_size = 0;
     act_cache cache;
     bool fuse = true;      // MI355_NO_FUSION=1 executes the graph node for node
-    int32_t * iota = nullptr;   // device {0, 1, 2, ...}: token t of a batch goes to row t of a KV-cache view
+    int32_t * iota = nullptr;   // device {0, 1, 2, ... IOTA_N - 1}: token t of a batch goes to row t of a KV-cache view
+    // products whose result is written somewhere else than into their own tensor (see match_prefill_qkv)
+    const ggml_tensor * redirect_node[2] = {nullptr, nullptr};
+    void * redirect_to[2] = {nullptr, nullptr};
+    int n_redirect = 0;
+    void * out_ptr(const ggml_tensor * t) const {
+        for (int k = 0; k < n_redirect; k++)
+            if (redirect_node[k] == t) return redirect_to[k];
+        return t->data;
+    }
     unsigned * tickets = nullptr;   // zeroed arrival counters of the gate/up launch (one per 32 output rows)
     size_t n_tickets = 0;
 
@@ -231,6 +242,9 @@ staging & stage() {
 // Unpacked int8 planes of Q6_K weight matrices for the tile GEMM (mi355_kq_unpack_planes), built the first time a matrix in a
 // weights buffer meets a batch above 8 and kept until that buffer is freed or the tensor is written again.  Keyed by the
 // tensor's data address.  MI355_NO_PLANES=1 keeps the packed rows only (2 bytes per Q6_K weight less device memory).
+// launches spent on one-time copies of weights (planes, tile images): reported apart from a graph's own launches
+std::atomic<uint64_t> g_prep_launches{0};
+
 struct plane_store {
     std::mutex mu;
     struct entry { void * planes; int64_t rows, K; };
@@ -249,7 +263,9 @@ struct plane_store {
             enabled = false;
             return nullptr;
         }
+        const uint64_t before = mi355_launch_count();
         MI355_K_OK(mi355_kq_unpack_planes(s, to_mi355_type(w->type), w->data, planes, w->ne[1], w->ne[0]));
+        g_prep_launches += mi355_launch_count() - before;
         map.emplace(w->data, entry{planes, w->ne[1], w->ne[0]});
         return planes;
     }
@@ -297,7 +313,9 @@ struct tile_store {
             enabled = false;
             return nullptr;
         }
+        const uint64_t before = mi355_launch_count();
         MI355_K_OK(mi355_kq_unpack_tiles(s, to_mi355_type(w->type), w->data, tiles, w->ne[1], w->ne[0]));
+        g_prep_launches += mi355_launch_count() - before;
         map.emplace(w->data, entry{tiles, w->ne[1], w->ne[0]});
         return tiles;
     }
@@ -500,6 +518,11 @@ ggml_backend_buffer_type_t mi355_host_buffer_type(ggml_backend_dev_t dev) {
 // ------------------------------------------------------------------------------- op support
 bool f32_rows(const ggml_tensor * t) { return t->type == GGML_TYPE_F32 && t->nb[0] == sizeof(float); }
 
+// Buffers are 256-byte aligned and the allocator places tensors on that alignment, so a tensor's address is 16-byte aligned
+// unless it is a view at an odd byte offset into its source (view_offs is relative to the tensor that owns the memory).
+// The kernels that read with 128-bit loads need this; a view that fails it is left to another backend.
+bool base_aligned16(const ggml_tensor * t) { return t->view_src == nullptr || t->view_offs % 16 == 0; }
+
 bool supports_mul_mat(const ggml_tensor * op) {
     const ggml_tensor * a = op->src[0];
     const ggml_tensor * b = op->src[1];
@@ -508,7 +531,7 @@ bool supports_mul_mat(const ggml_tensor * op) {
     if (is_weight_type(a->type)) {
         // quantized weights: whole contiguous matrices; activations as 16-byte aligned f32 rows
         if (!ggml_is_contiguous(a)) return false;
-        if (b->nb[0] != sizeof(float) || !strides_mult16(b)) return false;
+        if (b->nb[0] != sizeof(float) || !strides_mult16(b) || !base_aligned16(b)) return false;
         if (b->ne[2] % a->ne[2] != 0 || b->ne[3] % a->ne[3] != 0) return false;
         return b->ne[1] <= 65535;
     }
@@ -543,6 +566,7 @@ bool supports_flash_attn(const ggml_tensor * op) {
     const int64_t D = q->ne[0];
     if (!(D == 64 || D == 80 || D == 96 || D == 112 || D == 128 || D == 256) || k->ne[0] != D || v->ne[0] != D) return false;
     if (!strides_mult16(q) || !strides_mult16(k) || !strides_mult16(v)) return false;
+    if (!base_aligned16(q) || !base_aligned16(k) || !base_aligned16(v)) return false;
     if (q->ne[2] % k->ne[2] != 0 || k->ne[2] != v->ne[2] || k->ne[1] != v->ne[1]) return false;
     if (q->ne[3] != k->ne[3] || q->ne[3] != v->ne[3]) return false;
     if (mask && (mask->type != GGML_TYPE_F16 || !ggml_is_contiguous(mask) || mask->ne[0] != k->ne[1])) return false;
@@ -640,7 +664,7 @@ void compute_mul_mat(backend_ctx * ctx, ggml_tensor * dst) {
         for (int64_t i2 = 0; i2 < b->ne[2]; i2++) {
             const char * W = (const char *) a->data + (i2 / r2) * a->nb[2] + (i3 / r3) * a->nb[3];
             const float * x = (const float *) ((const char *) b->data + i2 * b->nb[2] + i3 * b->nb[3]);
-            float * y = (float *) ((char *) dst->data + i2 * dst->nb[2] + i3 * dst->nb[3]);
+            float * y = (float *) ((char *) ctx->out_ptr(dst) + i2 * dst->nb[2] + i3 * dst->nb[3]);
             MI355_K_OK(mi355_mul_mat(ctx->stream, to_mi355_type(a->type), W, x, y, N, K, B, (int64_t) (b->nb[1] / sizeof(float)),
                                      (int64_t) (dst->nb[1] / sizeof(float)), ws, ws_bytes));
         }
@@ -940,6 +964,231 @@ bool bytes_overlap(const ggml_tensor * a, const ggml_tensor * b) {
     return a0 < b0 + ggml_nbytes(b) && b0 < a0 + ggml_nbytes(a);
 }
 
+// Up to three projections of one activation with their ROPE and f16 cache-store nodes, to be served by ONE launch (decode,
+// batch <= 4):  MUL_MAT -> [RESHAPE] -> ROPE [-> CPY to an f16 view]   and   MUL_MAT -> CPY to an f16 view.
+// llm_build_kv lists them as  Q, rope(Q), K, rope(K), V, cpy(K), cpy(V): the window takes nodes from `first` on while every
+// one of them belongs to such a chain, so nothing outside the window is reordered.
+struct qkv_window {
+    int n_ch = 0;
+    int last = -1;                  // last node the window consumed
+    mi355_gemv_rope_mat mats[3];
+    mi355_rope_desc rd;
+    int n_store = 0;                // cache stores among the epilogues
+    bool redirect = false;          // every cache store starts at cell kv_head: address the cache through ctx->cells
+    bool ok = false;                // at least one epilogue, whole heads
+};
+
+qkv_window match_qkv_window(backend_ctx * ctx, const graph_walk & w, int first, const void * b_data, int64_t K, int64_t B) {
+    qkv_window win;
+    struct chain {
+        const ggml_tensor * mm;     // the product
+        const ggml_tensor * out;    // the tensor that currently holds the chain's value (product or its ROPE)
+        int out_index;
+        mi355_gemv_rope_mat m;
+        void * cache_base;          // cache stores that start at cell kv_head: the cache tensor's first byte
+    } ch[3];
+    int n_ch = 0, last = first - 1;
+    mi355_rope_desc rd;
+    memset(&rd, 0, sizeof(rd));
+    bool have_rope = false;
+    auto node_index_sole = [&](const ggml_tensor * t, int from, int to) {   // t is a node in [from, to) with one reader
+        for (int k = from; k < to; k++)
+            if (w.nodes[k] == t) return w.sole_use(k);
+        return false;
+    };
+    for (int k = first; k < w.n && k < first + 24; k++) {
+        const ggml_tensor * t = w.nodes[k];
+        if (is_noop(t)) continue;
+        if (t->op == GGML_OP_MUL_MAT) {
+            if (n_ch == 3 || !is_quant_gemv_candidate(t) || t->src[1]->data != b_data || t->src[1]->ne[0] != K || t->src[1]->ne[1] != B ||
+                !w.sole_use(k) || t->ne[0] % 2 != 0 || !ggml_is_contiguous(t))
+                break;
+            chain & c = ch[n_ch++];
+            c.mm = t; c.out = t; c.out_index = k;
+            c.cache_base = nullptr;
+            c.m.type = to_mi355_type(t->src[0]->type);
+            c.m.W = t->src[0]->data;
+            c.m.N = t->ne[0];
+            c.m.epilogue = MI355_EPI_STORE;
+            c.m.dst = t->data;
+            c.m.dst_stride = t->ne[0];
+            c.m.nb1 = c.m.nb2 = 0;
+            last = k;
+            continue;
+        }
+        if (t->op == GGML_OP_ROPE) {
+            const ggml_tensor * src = t->src[0];
+            chain * c = nullptr;
+            for (int q = 0; q < n_ch; q++) {
+                if (ch[q].m.epilogue != MI355_EPI_STORE) continue;
+                if (src == ch[q].mm) c = &ch[q];
+                else if (src->op == GGML_OP_RESHAPE && src->src[0] == ch[q].mm && ggml_is_contiguous(src) && node_index_sole(src, ch[q].out_index + 1, k)) c = &ch[q];
+            }
+            const int32_t * p = (const int32_t *) t->op_params;
+            const int64_t N = c ? c->m.N : 0;
+            if (!c || t->src[1]->type != GGML_TYPE_I32 || !ggml_is_contiguous(t) || t->type != GGML_TYPE_F32 || t->ne[0] * t->ne[1] != N || t->ne[2] != B ||
+                t->ne[3] != 1 || (t->src[2] && t->src[2]->type != GGML_TYPE_F32) || p[2] != 0 || p[1] % 2 != 0 || p[1] <= 0 || p[1] > t->ne[0] ||
+                t->ne[0] % 2 != 0)
+                break;
+            mi355_rope_desc r;
+            memset(&r, 0, sizeof(r));
+            r.pos = (const int32_t *) t->src[1]->data;
+            r.cells = ctx->iota;
+            r.freq_factors = t->src[2] ? (const float *) t->src[2]->data : nullptr;
+            r.head_dim = t->ne[0];
+            r.n_dims = p[1];
+            r.mode = 0;
+            r.n_ctx_orig = p[4];
+            memcpy(&r.freq_base, p + 5, sizeof(float));
+            memcpy(&r.freq_scale, p + 6, sizeof(float));
+            memcpy(&r.ext_factor, p + 7, sizeof(float));
+            memcpy(&r.attn_factor, p + 8, sizeof(float));
+            memcpy(&r.beta_fast, p + 9, sizeof(float));
+            memcpy(&r.beta_slow, p + 10, sizeof(float));
+            if (have_rope && memcmp(&r, &rd, sizeof(rd)) != 0) break;   // one set of rope parameters per launch
+            rd = r;
+            have_rope = true;
+            c->m.epilogue = MI355_EPI_ROPE;
+            c->m.dst = t->data;
+            c->m.dst_stride = N;
+            c->out = t;
+            c->out_index = k;
+            last = k;
+            continue;
+        }
+        if (t->op == GGML_OP_CPY) {
+            chain * c = nullptr;
+            for (int q = 0; q < n_ch; q++)
+                if (t->src[0] == ch[q].out && (ch[q].m.epilogue == MI355_EPI_STORE || ch[q].m.epilogue == MI355_EPI_ROPE)) c = &ch[q];
+            const ggml_tensor * d = t->src[1];
+            if (!c || !w.sole_use(c->out_index) || d->type != GGML_TYPE_F16 || !ggml_is_contiguous(d) || ggml_nelements(d) != c->m.N * B ||
+                ((uintptr_t) d->data & 1) != 0)
+                break;
+            c->m.epilogue = c->m.epilogue == MI355_EPI_ROPE ? MI355_EPI_ROPE_CACHE : MI355_EPI_CACHE;
+            c->m.dst = d->data;
+            c->m.dst_stride = 0;
+            c->m.nb1 = c->m.N * 2;
+            c->out = nullptr;
+            if (ctx->kv_head >= 0 && d->view_src && d->view_src->data &&
+                (const char *) d->data - (const char *) d->view_src->data == (ptrdiff_t) (ctx->kv_head * c->m.N * 2))
+                c->cache_base = d->view_src->data;
+            last = k;
+            continue;
+        }
+        break;
+    }
+    bool any_epilogue = false;
+    for (int q = 0; q < n_ch; q++) any_epilogue = any_epilogue || ch[q].m.epilogue != MI355_EPI_STORE;
+    if (!any_epilogue) return win;
+    if (!have_rope) {   // cache stores only: rows are one "head"; any even divisor of every N serves
+        rd.cells = ctx->iota;
+        rd.head_dim = 2; rd.n_dims = 2; rd.n_ctx_orig = 1; rd.freq_base = 10000.0f; rd.freq_scale = 1.0f; rd.attn_factor = 1.0f; rd.beta_fast = 32.0f; rd.beta_slow = 1.0f;
+    }
+    bool heads_ok = true;
+    int n_base = 0;
+    for (int q = 0; q < n_ch; q++) {
+        win.mats[q] = ch[q].m;
+        if (win.mats[q].epilogue != MI355_EPI_STORE) heads_ok = heads_ok && win.mats[q].N % rd.head_dim == 0;
+        if (win.mats[q].epilogue == MI355_EPI_ROPE_CACHE || win.mats[q].epilogue == MI355_EPI_CACHE) {
+            win.mats[q].nb2 = rd.head_dim * 2;
+            win.n_store++;
+            if (ch[q].cache_base) n_base++;
+        }
+    }
+    if (!heads_ok) return win;
+    // Cache stores that all start at cell kv_head address the cache tensor through the device-side cell list instead
+    // of through the view's own address, so the launch's arguments do not change from token to token.
+    if (win.n_store > 0 && n_base == win.n_store) {
+        for (int q = 0; q < n_ch; q++)
+            if (ch[q].cache_base) win.mats[q].dst = ch[q].cache_base;
+        rd.cells = ctx->cells;
+        win.redirect = true;
+    }
+    win.n_ch = n_ch;
+    win.last = last;
+    win.rd = rd;
+    win.ok = true;
+    return win;
+}
+
+void note_window_writes(backend_ctx * ctx, const qkv_window & win, int64_t B) {
+    if (win.redirect) ctx->kv_redirected += win.n_store;
+    for (int q = 0; q < win.n_ch; q++) {
+        const bool f32_out = win.mats[q].epilogue == MI355_EPI_STORE || win.mats[q].epilogue == MI355_EPI_ROPE;
+        ctx->note_write(win.mats[q].dst, (size_t) win.mats[q].N * (size_t) B * (f32_out ? sizeof(float) : 2));
+    }
+}
+
+// Prefill (more than 4 rows): build_llama lists  MUL_MAT(q), ROPE(q), MUL_MAT(k), ROPE(k), MUL_MAT(v), CPY(k -> cache),
+// CPY(v -> cache).  The window runs the three products and then ONE launch that rotates q in place, rotates k and stores k and v
+// to the f16 cache.  The graph allocator hands the memory of the unrotated q to the k product and that of the unrotated k to
+// the v product, so the rotations cannot simply wait for the products: instead the q and k products write straight into the
+// memory of their ROPE nodes' results, which nothing else can occupy before those results are read (q by attention, k by its
+// cache store), and are rotated there.
+struct prefill_qkv {
+    bool ok = false;
+    int ik = -1, iv = -1, last = -1;
+    const ggml_tensor * rq = nullptr, * rk = nullptr, * mk = nullptr, * mv = nullptr, * ck = nullptr, * cv = nullptr;
+};
+
+prefill_qkv match_prefill_qkv(const graph_walk & w, int i) {
+    prefill_qkv p;
+    const ggml_tensor * mq = w.nodes[i];
+    const ggml_tensor * b = mq->src[1];
+    const int64_t B = b->ne[1];
+    auto product_ok = [&](const ggml_tensor * m, int idx) {
+        return m->op == GGML_OP_MUL_MAT && is_weight_type(m->src[0]->type) && m->src[0]->ne[2] == 1 && m->src[0]->ne[3] == 1 && m->src[1] == b &&
+               b->ne[2] == 1 && b->ne[3] == 1 && ggml_is_contiguous(m) && m->type == GGML_TYPE_F32 && w.sole_use(idx);
+    };
+    // the ROPE that reads product m, directly or through a RESHAPE nobody else reads
+    auto rope_of = [&](const ggml_tensor * r, const ggml_tensor * m, int from, int to) {
+        if (r->op != GGML_OP_ROPE || r->type != GGML_TYPE_F32 || !ggml_is_contiguous(r) || r->ne[3] != 1 || r->ne[2] != B) return false;
+        const ggml_tensor * src = r->src[0];
+        if (src != m) {
+            if (src->op != GGML_OP_RESHAPE || src->src[0] != m || !ggml_is_contiguous(src)) return false;
+            bool sole = false;
+            for (int k = from; k < to; k++)
+                if (w.nodes[k] == src) sole = w.sole_use(k);
+            if (!sole) return false;
+        }
+        const int32_t * q = (const int32_t *) r->op_params;
+        return r->ne[0] * r->ne[1] == m->ne[0] && r->src[1]->type == GGML_TYPE_I32 && (!r->src[2] || r->src[2]->type == GGML_TYPE_F32) &&
+               (q[2] == 0 || q[2] == 2) && q[1] > 0 && q[1] % 2 == 0 && q[1] <= r->ne[0] && r->ne[0] % 2 == 0 && r->ne[0] <= 2048;
+    };
+    if (B <= 4 || B > IOTA_N || !product_ok(mq, i)) return p;
+    const int j1 = w.next(i);
+    if (j1 >= w.n || !rope_of(w.nodes[j1], mq, i + 1, j1)) return p;
+    const int j2 = w.next(j1);
+    if (j2 >= w.n || !product_ok(w.nodes[j2], j2)) return p;
+    const int j3 = w.next(j2);
+    if (j3 >= w.n || !rope_of(w.nodes[j3], w.nodes[j2], j2 + 1, j3) || !w.sole_use(j3)) return p;
+    const int j4 = w.next(j3);
+    if (j4 >= w.n || !product_ok(w.nodes[j4], j4)) return p;
+    const int j5 = w.next(j4), j6 = j5 < w.n ? w.next(j5) : w.n;
+    if (j6 >= w.n) return p;
+    const ggml_tensor * rq = w.nodes[j1], * mk = w.nodes[j2], * rk = w.nodes[j3], * mv = w.nodes[j4], * ck = w.nodes[j5], * cv = w.nodes[j6];
+    auto store_ok = [&](const ggml_tensor * c, const ggml_tensor * src) {
+        const ggml_tensor * d = c->src[1];
+        return c->op == GGML_OP_CPY && c->src[0] == src && d->type == GGML_TYPE_F16 && ggml_is_contiguous(d) && ggml_nelements(d) == ggml_nelements(src) &&
+               ((uintptr_t) d->data & 1) == 0;
+    };
+    if (!store_ok(ck, rk) || !store_ok(cv, mv)) return p;
+    // one set of rope parameters, positions and frequency factors; k and v heads of q's size
+    if (memcmp(rq->op_params, rk->op_params, 11 * sizeof(int32_t)) != 0 || rq->src[1] != rk->src[1] || rq->src[2] != rk->src[2]) return p;
+    if (rq->ne[0] != rk->ne[0] || mv->ne[0] != mk->ne[0]) return p;
+    // what the products write early must not be read or written by anything else inside the window
+    if (bytes_overlap(rq, rk) || bytes_overlap(rq, mv) || bytes_overlap(rk, mv) || bytes_overlap(rq, b) || bytes_overlap(rk, b)) return p;
+    // ... and what the rotations read late must survive the products: in the last layer the allocator gives the memory of the
+    // position vector, whose last reader in graph order is ROPE(k), to the v product
+    for (const ggml_tensor * in : {rq->src[1], rq->src[2]}) {
+        if (in && (bytes_overlap(in, rq) || bytes_overlap(in, rk) || bytes_overlap(in, mv))) return p;
+    }
+    p.ok = true;
+    p.ik = j2; p.iv = j4; p.last = j6;
+    p.rq = rq; p.rk = rk; p.mk = mk; p.mv = mv; p.ck = ck; p.cv = cv;
+    return p;
+}
+
 // Runs node i and possibly a few of its successors; returns the index of the last node consumed.
 int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     hipStream_t s = ctx->stream;
@@ -947,6 +1196,41 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     const int j = w.next(i);
     ggml_tensor * nxt = j < w.n ? (ggml_tensor *) w.nodes[j] : nullptr;
 
+    // ---- prefill: Q, K and V products, then both rotations and both cache stores in one launch (see match_prefill_qkv)
+    if (node->op == GGML_OP_MUL_MAT && ctx->n_redirect == 0 && node->src[1]->ne[1] > 4) {
+        const prefill_qkv p = match_prefill_qkv(w, i);
+        if (p.ok) {
+            ctx->redirect_node[0] = node;  ctx->redirect_to[0] = p.rq->data;
+            ctx->redirect_node[1] = p.mk;  ctx->redirect_to[1] = p.rk->data;
+            ctx->n_redirect = 2;
+            int done = compute_fused(ctx, w, i);
+            GGML_ASSERT(done == i);        // a product followed by its ROPE takes nothing with it
+            done = compute_fused(ctx, w, p.ik);
+            GGML_ASSERT(done == p.ik);
+            done = compute_fused(ctx, w, p.iv);
+            GGML_ASSERT(done == p.iv);
+            ctx->n_redirect = 0;
+            const ggml_tensor * rq = p.rq;
+            const int32_t * op = (const int32_t *) rq->op_params;
+            float freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
+            memcpy(&freq_base, op + 5, sizeof(float));
+            memcpy(&freq_scale, op + 6, sizeof(float));
+            memcpy(&ext_factor, op + 7, sizeof(float));
+            memcpy(&attn_factor, op + 8, sizeof(float));
+            memcpy(&beta_fast, op + 9, sizeof(float));
+            memcpy(&beta_slow, op + 10, sizeof(float));
+            const int64_t D = rq->ne[0], H = rq->ne[1], HK = p.rk->ne[1], T = rq->ne[2];
+            MI355_K_OK(mi355_rope_kv_store(s, (float *) rq->data, (const float *) p.rk->data, (const float *) p.mv->data, p.ck->src[1]->data, p.cv->src[1]->data,
+                                           (const int32_t *) rq->src[1]->data, ctx->iota, rq->src[2] ? (const float *) rq->src[2]->data : nullptr, T, H, HK, D,
+                                           (size_t) (HK * D * 2), (size_t) (D * 2), (size_t) (HK * D * 2), (size_t) (D * 2), op[1], op[2], op[4], freq_base,
+                                           freq_scale, ext_factor, attn_factor, beta_fast, beta_slow));
+            ctx->note_write(rq->data, ggml_nbytes(rq));
+            ctx->note_write(p.rk->data, ggml_nbytes(p.rk));
+            ctx->note_write(p.ck->src[1]->data, ggml_nbytes(p.ck->src[1]));
+            ctx->note_write(p.cv->src[1]->data, ggml_nbytes(p.cv->src[1]));
+            return p.last;
+        }
+    }
     // ---- RMS_NORM -> MUL(weight vector)
     if (node->op == GGML_OP_RMS_NORM && nxt && nxt->op == GGML_OP_MUL && nxt->src[0] == node && w.sole_use(i)) {
         const ggml_tensor * x = node->src[0];
@@ -958,6 +1242,20 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             float eps;
             memcpy(&eps, node->op_params, sizeof(float));
             void * act = nullptr;
+            // one decoded token: the norm goes into the Q/K/V launch when that launch's products are the only readers of the
+            // normalised row (every group normalises and quantizes the row for itself; the f32 row is not materialised)
+            if (rows == 1 && K <= 4096 && K % 1024 == 0 && !(nxt->flags & GGML_TENSOR_FLAG_OUTPUT)) {
+                const int jq = w.next(j);
+                if (jq < w.n && is_quant_gemv_candidate(w.nodes[jq]) && w.nodes[jq]->src[1]->data == nxt->data) {
+                    const qkv_window win = match_qkv_window(ctx, w, jq, nxt->data, K, 1);
+                    if (win.ok && win.n_ch == w.uses[j]) {
+                        MI355_K_OK(mi355_rms_norm_mul_mat_vec_q_rope(s, (const float *) x->data, (const float *) wt->data, eps, win.n_ch, win.mats, K, &win.rd));
+                        note_window_writes(ctx, win, 1);
+                        ctx->cache.valid = false;
+                        return win.last;
+                    }
+                }
+            }
             if (rows > 8 && feeds_q8k_tiles(w, j, nxt->data, K, rows)) {   // prefill: the per-super-block form for the tile GEMM
                 const int fmt = q8k_format_for(s, w.nodes[w.next(j)]);
                 act = ctx->act_slot(fmt == ACT_Q8KT ? mi355_act_q8k_tiled_bytes(K, rows) : mi355_act_q8k_bytes(K, rows));
@@ -1194,151 +1492,20 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             }
         }
     }
-    // ---- up to three projections of one activation with their ROPE and f16 cache-store nodes in ONE launch (decode, batch <= 4):
-    //      MUL_MAT -> [RESHAPE] -> ROPE [-> CPY to an f16 view]   and   MUL_MAT -> CPY to an f16 view.
-    //      llm_build_kv lists them as  Q, rope(Q), K, rope(K), V, cpy(K), cpy(V): the window below takes nodes while every one
-    //      of them belongs to such a chain, so nothing outside the window is reordered.
+    // ---- the Q/K/V window (see match_qkv_window): projections, rotations and cache stores in one launch
     if (is_quant_gemv_candidate(node) && node->src[1]->ne[1] <= 4 && w.sole_use(i) && nxt && node->ne[0] % 2 == 0) {
         const ggml_tensor * b = node->src[1];
         const int64_t K = b->ne[0], B = b->ne[1];
-        struct chain {
-            const ggml_tensor * mm;     // the product
-            const ggml_tensor * out;    // the tensor that currently holds the chain's value (product or its ROPE)
-            int out_index;
-            mi355_gemv_rope_mat m;
-            void * cache_base;          // cache stores that start at cell kv_head: the cache tensor's first byte
-        } ch[3];
-        int n_ch = 0, last = i - 1;
-        mi355_rope_desc rd;
-        memset(&rd, 0, sizeof(rd));
-        bool have_rope = false;
-        auto node_index_sole = [&](const ggml_tensor * t, int from, int to) {   // t is a node in [from, to) with one reader
-            for (int k = from; k < to; k++)
-                if (w.nodes[k] == t) return w.sole_use(k);
-            return false;
-        };
-        for (int k = i; k < w.n && k < i + 24; k++) {
-            const ggml_tensor * t = w.nodes[k];
-            if (is_noop(t)) continue;
-            if (t->op == GGML_OP_MUL_MAT) {
-                if (n_ch == 3 || !is_quant_gemv_candidate(t) || t->src[1]->data != b->data || t->src[1]->ne[0] != K || t->src[1]->ne[1] != B ||
-                    !w.sole_use(k) || t->ne[0] % 2 != 0 || !ggml_is_contiguous(t))
-                    break;
-                chain & c = ch[n_ch++];
-                c.mm = t; c.out = t; c.out_index = k;
-                c.cache_base = nullptr;
-                c.m.type = to_mi355_type(t->src[0]->type);
-                c.m.W = t->src[0]->data;
-                c.m.N = t->ne[0];
-                c.m.epilogue = MI355_EPI_STORE;
-                c.m.dst = t->data;
-                c.m.dst_stride = t->ne[0];
-                c.m.nb1 = c.m.nb2 = 0;
-                last = k;
-                continue;
+        const qkv_window win = match_qkv_window(ctx, w, i, b->data, K, B);
+        if (win.ok) {
+            if (!ctx->cached(b->data, K, B, ACT_Q8_1)) {
+                void * fresh = ctx->act_slot(mi355_act_bytes(K, B));
+                MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
+                ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
             }
-            if (t->op == GGML_OP_ROPE) {
-                const ggml_tensor * src = t->src[0];
-                chain * c = nullptr;
-                for (int q = 0; q < n_ch; q++) {
-                    if (ch[q].m.epilogue != MI355_EPI_STORE) continue;
-                    if (src == ch[q].mm) c = &ch[q];
-                    else if (src->op == GGML_OP_RESHAPE && src->src[0] == ch[q].mm && ggml_is_contiguous(src) && node_index_sole(src, ch[q].out_index + 1, k)) c = &ch[q];
-                }
-                const int32_t * p = (const int32_t *) t->op_params;
-                const int64_t N = c ? c->m.N : 0;
-                if (!c || t->src[1]->type != GGML_TYPE_I32 || !ggml_is_contiguous(t) || t->type != GGML_TYPE_F32 || t->ne[0] * t->ne[1] != N || t->ne[2] != B ||
-                    t->ne[3] != 1 || (t->src[2] && t->src[2]->type != GGML_TYPE_F32) || p[2] != 0 || p[1] % 2 != 0 || p[1] <= 0 || p[1] > t->ne[0] ||
-                    t->ne[0] % 2 != 0)
-                    break;
-                mi355_rope_desc r;
-                memset(&r, 0, sizeof(r));
-                r.pos = (const int32_t *) t->src[1]->data;
-                r.cells = ctx->iota;
-                r.freq_factors = t->src[2] ? (const float *) t->src[2]->data : nullptr;
-                r.head_dim = t->ne[0];
-                r.n_dims = p[1];
-                r.mode = 0;
-                r.n_ctx_orig = p[4];
-                memcpy(&r.freq_base, p + 5, sizeof(float));
-                memcpy(&r.freq_scale, p + 6, sizeof(float));
-                memcpy(&r.ext_factor, p + 7, sizeof(float));
-                memcpy(&r.attn_factor, p + 8, sizeof(float));
-                memcpy(&r.beta_fast, p + 9, sizeof(float));
-                memcpy(&r.beta_slow, p + 10, sizeof(float));
-                if (have_rope && memcmp(&r, &rd, sizeof(rd)) != 0) break;   // one set of rope parameters per launch
-                rd = r;
-                have_rope = true;
-                c->m.epilogue = MI355_EPI_ROPE;
-                c->m.dst = t->data;
-                c->m.dst_stride = N;
-                c->out = t;
-                c->out_index = k;
-                last = k;
-                continue;
-            }
-            if (t->op == GGML_OP_CPY) {
-                chain * c = nullptr;
-                for (int q = 0; q < n_ch; q++)
-                    if (t->src[0] == ch[q].out && (ch[q].m.epilogue == MI355_EPI_STORE || ch[q].m.epilogue == MI355_EPI_ROPE)) c = &ch[q];
-                const ggml_tensor * d = t->src[1];
-                if (!c || !w.sole_use(c->out_index) || d->type != GGML_TYPE_F16 || !ggml_is_contiguous(d) || ggml_nelements(d) != c->m.N * B ||
-                    ((uintptr_t) d->data & 1) != 0)
-                    break;
-                c->m.epilogue = c->m.epilogue == MI355_EPI_ROPE ? MI355_EPI_ROPE_CACHE : MI355_EPI_CACHE;
-                c->m.dst = d->data;
-                c->m.dst_stride = 0;
-                c->m.nb1 = c->m.N * 2;
-                c->out = nullptr;
-                if (ctx->kv_head >= 0 && d->view_src && d->view_src->data &&
-                    (const char *) d->data - (const char *) d->view_src->data == (ptrdiff_t) (ctx->kv_head * c->m.N * 2))
-                    c->cache_base = d->view_src->data;
-                last = k;
-                continue;
-            }
-            break;
-        }
-        bool any_epilogue = false;
-        for (int q = 0; q < n_ch; q++) any_epilogue = any_epilogue || ch[q].m.epilogue != MI355_EPI_STORE;
-        if (any_epilogue) {
-            if (!have_rope) {   // cache stores only: rows are one "head"; any even divisor of every N serves
-                rd.cells = ctx->iota;
-                rd.head_dim = 2; rd.n_dims = 2; rd.n_ctx_orig = 1; rd.freq_base = 10000.0f; rd.freq_scale = 1.0f; rd.attn_factor = 1.0f; rd.beta_fast = 32.0f; rd.beta_slow = 1.0f;
-            }
-            bool heads_ok = true;
-            mi355_gemv_rope_mat mats[3];
-            for (int q = 0; q < n_ch; q++) {
-                mats[q] = ch[q].m;
-                if (mats[q].epilogue != MI355_EPI_STORE) heads_ok = heads_ok && mats[q].N % rd.head_dim == 0;
-                if (mats[q].epilogue == MI355_EPI_ROPE_CACHE || mats[q].epilogue == MI355_EPI_CACHE) mats[q].nb2 = rd.head_dim * 2;
-            }
-            if (heads_ok) {
-                if (!ctx->cached(b->data, K, B, ACT_Q8_1)) {
-                    void * fresh = ctx->act_slot(mi355_act_bytes(K, B));
-                    MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, B, K));
-                    ctx->cache = act_cache{b->data, K, B, ACT_Q8_1, true, fresh};
-                }
-                // Cache stores that all start at cell kv_head address the cache tensor through the device-side cell list instead
-                // of through the view's own address, so the launch's arguments do not change from token to token.
-                int n_store = 0, n_base = 0;
-                for (int q = 0; q < n_ch; q++) {
-                    if (mats[q].epilogue != MI355_EPI_ROPE_CACHE && mats[q].epilogue != MI355_EPI_CACHE) continue;
-                    n_store++;
-                    if (ch[q].cache_base) n_base++;
-                }
-                if (n_store > 0 && n_base == n_store) {
-                    for (int q = 0; q < n_ch; q++)
-                        if (ch[q].cache_base) mats[q].dst = ch[q].cache_base;
-                    rd.cells = ctx->cells;
-                    ctx->kv_redirected += n_store;
-                }
-                MI355_K_OK(mi355_mul_mat_vec_q_rope(s, n_ch, mats, ctx->cache.ptr, K, B, &rd));
-                for (int q = 0; q < n_ch; q++) {
-                    const bool f32_out = mats[q].epilogue == MI355_EPI_STORE || mats[q].epilogue == MI355_EPI_ROPE;
-                    ctx->note_write(mats[q].dst, (size_t) mats[q].N * (size_t) B * (f32_out ? sizeof(float) : 2));
-                }
-                return last;
-            }
+            MI355_K_OK(mi355_mul_mat_vec_q_rope(s, win.n_ch, win.mats, ctx->cache.ptr, K, B, &win.rd));
+            note_window_writes(ctx, win, B);
+            return win.last;
         }
     }
     // ---- runs of quantized products on one activation (batch <= 32): one quantization, multi-matrix GEMV (up to 4 rows) or the
@@ -1365,7 +1532,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             mats[r].type = to_mi355_type(mm->src[0]->type);
             mats[r].W = mm->src[0]->data;
             mats[r].N = mm->src[0]->ne[1];
-            mats[r].dst = (float *) mm->data;
+            mats[r].dst = (float *) ctx->out_ptr(mm);
             mats[r].dst_stride = (int64_t) (mm->nb[1] / sizeof(float));
             mats[r].residual = nullptr;
         }
@@ -1429,8 +1596,8 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 return j;
             }
         }
-        product((float *) node->data, nullptr, (int64_t) (node->nb[1] / sizeof(float)));
-        ctx->note_write(node->data, ggml_nbytes(node));
+        product((float *) ctx->out_ptr(node), nullptr, (int64_t) (node->nb[1] / sizeof(float)));
+        ctx->note_write(ctx->out_ptr(node), ggml_nbytes(node));
         return i;
     }
     ctx->note_write(node->op == GGML_OP_CPY ? node->src[1]->data : node->data, ggml_nbytes(node->op == GGML_OP_CPY ? node->src[1] : node));
@@ -1457,17 +1624,21 @@ struct graph_signature {
     int kv_stores = 0;
 };
 
+// One multiply per word: the signature is computed for every graph of every token, ahead of the launch.
 inline uint64_t sig_mix(uint64_t h, uint64_t v) {
-    h ^= v + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2);
-    return h * 0xff51afd7ed558ccdull;
+    h = (h ^ v) * 0x9E3779B97F4A7C15ull;
+    return h ^ (h >> 29);
 }
+
+// two fields per word (the second spread by an odd multiplier, so that swapping them changes the word)
+inline uint64_t sig_pair(uint64_t a, uint64_t b) { return a + b * 0xff51afd7ed558ccdull; }
 
 uint64_t sig_tensor(uint64_t h, const ggml_tensor * t, bool through_cache) {
     h = sig_mix(h, ((uint64_t) t->type << 32) | (uint64_t) t->op);
-    for (int i = 0; i < GGML_MAX_DIMS; i++) {
-        h = sig_mix(h, (uint64_t) t->ne[i]);
-        h = sig_mix(h, (uint64_t) t->nb[i]);
-    }
+    h = sig_mix(h, sig_pair((uint64_t) t->ne[0], (uint64_t) t->ne[1]));
+    h = sig_mix(h, sig_pair((uint64_t) t->ne[2], (uint64_t) t->ne[3]));
+    h = sig_mix(h, sig_pair((uint64_t) t->nb[0], (uint64_t) t->nb[1]));
+    h = sig_mix(h, sig_pair((uint64_t) t->nb[2], (uint64_t) t->nb[3]));
     return sig_mix(h, (uint64_t) (uintptr_t) (through_cache ? t->view_src->data : t->data));
 }
 
@@ -1480,24 +1651,36 @@ bool is_cache_store(const ggml_tensor * node) {
 graph_signature sign_graph(ggml_cgraph * cgraph, std::vector<uint64_t> * trace = nullptr) {
     graph_signature g;
     const int n = ggml_graph_n_nodes(cgraph);
-    // the views that cache stores write through (they are graph nodes themselves, and sources of the CPY nodes)
-    std::unordered_set<const ggml_tensor *> dests;
+    // the views that cache stores write through (they are graph nodes themselves, and sources of the CPY nodes): two per layer
+    const ggml_tensor * dests[256];
+    int n_dests = 0;
     for (int i = 0; i < n; i++) {
         const ggml_tensor * node = ggml_graph_node(cgraph, i);
-        if (is_cache_store(node)) dests.insert(node->src[1]);
+        if (node->op == GGML_OP_CPY && is_cache_store(node)) {
+            if (n_dests == 256) return g;   // not a graph this path knows: launch by launch (capturable stays false, hash 0)
+            dests[n_dests++] = node->src[1];
+        }
     }
-    auto through_cache = [&](const ggml_tensor * t) { return dests.count(t) != 0; };
+    auto through_cache = [&](const ggml_tensor * t) {
+        if (t->op != GGML_OP_VIEW) return false;   // ggml_view_1d of the cache tensor (llm_build_kv_store)
+        for (int k = 0; k < n_dests; k++)
+            if (dests[k] == t) return true;
+        return false;
+    };
     uint64_t h = sig_mix(0x6d693335u, (uint64_t) n);
     int64_t batch = 0;
     bool heads_agree = true;
     for (int i = 0; i < n; i++) {
         const ggml_tensor * node = ggml_graph_node(cgraph, i);
-        const bool store = is_cache_store(node);
-        h = sig_tensor(h, node, through_cache(node) || (store && node->view_src != nullptr && node->data == node->src[1]->data));
+        const bool store = node->op == GGML_OP_CPY && is_cache_store(node);
+        const bool via_cache = through_cache(node);
+        h = sig_tensor(h, node, via_cache || (store && node->view_src != nullptr && node->data == node->src[1]->data));
         h = sig_mix(h, (uint64_t) node->flags);
-        if (!through_cache(node)) {   // a view's parameters hold its offset
-            for (size_t k = 0; k < GGML_MAX_OP_PARAMS / sizeof(int32_t); k += 2)
-                h = sig_mix(h, ((uint64_t) (uint32_t) node->op_params[k] << 32) | (uint32_t) node->op_params[k + 1]);
+        if (!via_cache) {   // a view's parameters hold its offset
+            for (size_t k = 0; k < GGML_MAX_OP_PARAMS / sizeof(int32_t); k += 2) {
+                const uint64_t pw = ((uint64_t) (uint32_t) node->op_params[k] << 32) | (uint32_t) node->op_params[k + 1];
+                if (pw) h = sig_mix(h, pw + k);   // most nodes have no parameters at all
+            }
         }
         if (trace) trace->push_back(h);
         for (int k = 0; k < GGML_MAX_SRC; k++) {
@@ -1528,6 +1711,7 @@ void run_graph_launches(backend_ctx * ctx, ggml_cgraph * cgraph) {
     ctx->cache.valid = false;
     const graph_walk w(cgraph);
     static const bool log_graph = getenv("MI355_LOG_GRAPH") != nullptr;   // node list and the nodes each launch sequence consumed
+    const uint64_t launches_before = mi355_launch_count(), prep_before = g_prep_launches.load();
     for (int i = 0; i < w.n; i++) {
         if (is_noop(w.nodes[i])) continue;
         const int first = i;
@@ -1539,6 +1723,16 @@ void run_graph_launches(backend_ctx * ctx, ggml_cgraph * cgraph) {
                         (long long) t->ne[0], (long long) t->ne[1], (long long) t->ne[2], (long long) t->ne[3], w.uses[k]);
             }
         }
+    }
+    if (log_graph) {
+        int64_t batch = 0, layers = 0;
+        for (int i = 0; i < w.n; i++) {
+            if (w.nodes[i]->op == GGML_OP_MUL_MAT && batch == 0) batch = w.nodes[i]->src[1]->ne[1];
+            if (w.nodes[i]->op == GGML_OP_FLASH_ATTN_EXT) layers++;
+        }
+        const uint64_t prep = g_prep_launches.load() - prep_before;
+        fprintf(stderr, "MI355 graph launches: %d nodes, batch %lld, %lld attention nodes, %llu kernel launches + %llu for one-time weight copies\n", w.n,
+                (long long) batch, (long long) layers, (unsigned long long) (mi355_launch_count() - launches_before - prep), (unsigned long long) prep);
     }
     ctx->cache.valid = false;
 }
@@ -1666,9 +1860,10 @@ ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
     ctx->name = dctx->name;
     const char * nf = getenv("MI355_NO_FUSION");
     ctx->fuse = !(nf && nf[0] == '1');
-    const int32_t iota_host[8] = {0, 1, 2, 3, 4, 5, 6, 7};
-    if (hipMalloc((void **) &ctx->iota, sizeof(iota_host)) != hipSuccess ||
-        hipMemcpy(ctx->iota, iota_host, sizeof(iota_host), hipMemcpyHostToDevice) != hipSuccess) {
+    std::vector<int32_t> iota_host(IOTA_N);
+    for (int k = 0; k < IOTA_N; k++) iota_host[k] = k;
+    if (hipMalloc((void **) &ctx->iota, IOTA_N * sizeof(int32_t)) != hipSuccess ||
+        hipMemcpy(ctx->iota, iota_host.data(), IOTA_N * sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess) {
         delete ctx;
         return nullptr;
     }
@@ -1680,6 +1875,8 @@ ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
         return nullptr;
     }
     if (hipStreamCreate(&ctx->stream) != hipSuccess) {   // default priority, blocking w.r.t. the null stream
+        (void) hipFree(ctx->iota);
+        (void) hipFree(ctx->cells);
         delete ctx;
         return nullptr;
     }

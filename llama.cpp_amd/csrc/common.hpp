@@ -122,6 +122,14 @@ __device__ __forceinline__ float wave_max(float v) {
 // ---- host-side error plumbing
 void set_error(const char *fmt, ...);
 
+// every kernel launch of the library goes through this macro, which also counts it (mi355_launch_count)
+void count_launch();
+#define MI355_LAUNCH(...)               \
+    do {                                \
+        mi355::count_launch();          \
+        hipLaunchKernelGGL(__VA_ARGS__); \
+    } while (0)
+
 #define MI355_CHECK_HIP(expr)                                                              \
     do {                                                                                   \
         hipError_t e_ = (expr);                                                            \

@@ -288,11 +288,11 @@ template <int D, int R>
 static int launch_vec(hipStream_t s, fattn_args &a) {
     a.groups = (int)(a.Hq / a.Hkv) / R;
     const dim3 grid((unsigned)a.n_splits, (unsigned)(a.Hkv * a.groups), (unsigned)a.Nq);
-    hipLaunchKernelGGL((k_fattn_vec<D, R>), grid, dim3(256), 0, s, a);
+    MI355_LAUNCH((k_fattn_vec<D, R>), grid, dim3(256), 0, s, a);
     int rc = launch_status("k_fattn_vec");
     if (rc != MI355_OK) return rc;
     if (a.n_splits > 1) {
-        hipLaunchKernelGGL(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(256), 0, s, a.ws, a.dst, a.n_splits, a.act_q,
+        MI355_LAUNCH(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(256), 0, s, a.ws, a.dst, a.n_splits, a.act_q,
                            a.act_s, a.Hq);
         rc = launch_status("k_fattn_combine");
     }
@@ -384,8 +384,8 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
         if (rc == 0) {
             if (b.n_splits > 1) {
                 switch (D) {
-                    case 64: hipLaunchKernelGGL(k_fattn_combine<64>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
-                    default: hipLaunchKernelGGL(k_fattn_combine<128>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
+                    case 64: MI355_LAUNCH(k_fattn_combine<64>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
+                    default: MI355_LAUNCH(k_fattn_combine<128>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
                 }
                 return launch_status("k_fattn_combine");
             }

@@ -499,7 +499,7 @@ template <int D>
 int launch_half(hipStream_t s, const fattn_args &a) {
     const int64_t pairs = (a.Hq / a.Hkv) / 2;
     const dim3 grid((unsigned)((a.Nq + 31) / 32), (unsigned)(a.Hkv * pairs));
-    hipLaunchKernelGGL((k_fattn_mma_half<D>), grid, dim3(256), 0, s, a);
+    MI355_LAUNCH((k_fattn_mma_half<D>), grid, dim3(256), 0, s, a);
     return launch_status("k_fattn_mma_half");
 }
 
@@ -508,7 +508,7 @@ int launch(hipStream_t s, const fattn_args &a) {
     constexpr int QTW = 4 / HPW;
     const int64_t groups = (a.Hq / a.Hkv) / HPW;
     const dim3 grid((unsigned)((a.Nq + 32 * QTW - 1) / (32 * QTW)), (unsigned)(a.Hkv * groups));
-    hipLaunchKernelGGL((k_fattn_mma<D, HPW>), grid, dim3(256), 0, s, a);
+    MI355_LAUNCH((k_fattn_mma<D, HPW>), grid, dim3(256), 0, s, a);
     return launch_status("k_fattn_mma");
 }
 
@@ -697,7 +697,7 @@ int launch_dec(hipStream_t s, const fattn_args &a) {
     const int R = (int)(a.Hq / a.Hkv);
     const int NT = 32 / R;
     const dim3 grid((unsigned)a.n_splits, (unsigned)a.Hkv, (unsigned)((a.Nq + NT - 1) / NT));
-    hipLaunchKernelGGL(k_fattn_mma_dec<D>, grid, dim3(256), 0, s, a, R, NT);
+    MI355_LAUNCH(k_fattn_mma_dec<D>, grid, dim3(256), 0, s, a, R, NT);
     return launch_status("k_fattn_mma_dec");
 }
 
@@ -714,7 +714,7 @@ int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes) {
     const int64_t n_groups = n_tiles * a.Hq / 4;
     if (n_groups > 512 && a.mask && a.ws && ws_bytes >= (size_t)n_tiles * sizeof(int32_t) && (((uintptr_t)a.mask | a.mask_nb1) & 15) == 0 &&
         a.Nkv % 8 == 0 && a.Nkv >= 2 * FM_BC && a.Nkv < 0x7fffffff) {
-        hipLaunchKernelGGL(k_mask_extent, dim3((unsigned)n_tiles), dim3(256), 0, s, a.mask, a.mask_nb1, a.Nq, a.Nkv, (int32_t *)a.ws);
+        MI355_LAUNCH(k_mask_extent, dim3((unsigned)n_tiles), dim3(256), 0, s, a.mask, a.mask_nb1, a.Nq, a.Nkv, (int32_t *)a.ws);
         const int rc = launch_status("k_mask_extent");
         if (rc != MI355_OK) return rc;
         a.kv_extent = (const int32_t *)a.ws;

@@ -145,9 +145,9 @@ static int rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, co
     const dim3 grid((unsigned)nrows), block(256);
 #define MI355_LAUNCH_NORM(NV)                                                                                                        \
     do {                                                                                                                              \
-        if (fmt == 2) hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, 2>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
-        else if (fmt == 1) hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, 1>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
-        else hipLaunchKernelGGL((k_rms_norm_mul_quant<NV, 0>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);     \
+        if (fmt == 2) MI355_LAUNCH((k_rms_norm_mul_quant<NV, 2>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
+        else if (fmt == 1) MI355_LAUNCH((k_rms_norm_mul_quant<NV, 1>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);  \
+        else MI355_LAUNCH((k_rms_norm_mul_quant<NV, 0>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps);     \
     } while (0)
     if (k <= 4096) MI355_LAUNCH_NORM(4);
     else if (k <= 8192) MI355_LAUNCH_NORM(8);
@@ -182,9 +182,9 @@ static int swiglu_quant(void *stream, const float *gate, const float *up, int64_
     MI355_REQUIRE(y != nullptr || act != nullptr, "swiglu_quant: no output requested");
     if (nrows == 0) return MI355_OK;
     const dim3 grid((unsigned)((k + 1023) / 1024), (unsigned)nrows), block(256);
-    if (fmt == 2) hipLaunchKernelGGL(k_swiglu_quant<2>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
-    else if (fmt == 1) hipLaunchKernelGGL(k_swiglu_quant<1>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
-    else hipLaunchKernelGGL(k_swiglu_quant<0>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
+    if (fmt == 2) MI355_LAUNCH(k_swiglu_quant<2>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
+    else if (fmt == 1) MI355_LAUNCH(k_swiglu_quant<1>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
+    else MI355_LAUNCH(k_swiglu_quant<0>, grid, block, 0, (hipStream_t)stream, gate, up, in_stride, y, y_stride, act, k, nrows);
     return launch_status("k_swiglu_quant");
 }
 
@@ -223,7 +223,7 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
     a.corr0 = c0 > 0 ? c0 : 0;
     a.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
     const int threads = (int)((D / 2 + 63) / 64 * 64);
-    hipLaunchKernelGGL(k_rope_kv_store, dim3((unsigned)(H + 2 * HK), (unsigned)T), dim3(threads), 0, (hipStream_t)stream, a);
+    MI355_LAUNCH(k_rope_kv_store, dim3((unsigned)(H + 2 * HK), (unsigned)T), dim3(threads), 0, (hipStream_t)stream, a);
     return launch_status("k_rope_kv_store");
 }
 

@@ -444,30 +444,30 @@ template <int NCOLS>
 static void launch_multi(int rpw, hipStream_t s, const gemv_batch &b, unsigned grid, const int8_t *aq, const act_ds *ads, int K) {
     if constexpr (NCOLS <= 4) {
         if (const size_t lds = act_lds_bytes(NCOLS, K, grid)) {
-            if (rpw == 1) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 1, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
-            else if (rpw == 2) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 2, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
-            else hipLaunchKernelGGL((k_gemv_multi<NCOLS, 4, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
+            if (rpw == 1) MI355_LAUNCH((k_gemv_multi<NCOLS, 1, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
+            else if (rpw == 2) MI355_LAUNCH((k_gemv_multi<NCOLS, 2, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
+            else MI355_LAUNCH((k_gemv_multi<NCOLS, 4, true>), dim3(grid), dim3(256), lds, s, b, aq, ads, K);
             return;
         }
     }
-    if (rpw == 1) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 1, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
-    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_multi<NCOLS, 2, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
-    else hipLaunchKernelGGL((k_gemv_multi<NCOLS, 4, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    if (rpw == 1) MI355_LAUNCH((k_gemv_multi<NCOLS, 1, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    else if (rpw == 2) MI355_LAUNCH((k_gemv_multi<NCOLS, 2, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
+    else MI355_LAUNCH((k_gemv_multi<NCOLS, 4, false>), dim3(grid), dim3(256), 0, s, b, aq, ads, K);
 }
 
 template <int TYPE, int NCOLS>
 static void launch_single(int rpw, hipStream_t s, const gemv_item &m, unsigned grid, const int8_t *aq, const act_ds *ads, int K) {
     if constexpr (NCOLS <= 4) {
         if (const size_t lds = act_lds_bytes(NCOLS, K, grid)) {
-            if (rpw == 1) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 1, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
-            else if (rpw == 2) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 2, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
-            else hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 4, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
+            if (rpw == 1) MI355_LAUNCH((k_gemv_q<TYPE, NCOLS, 1, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
+            else if (rpw == 2) MI355_LAUNCH((k_gemv_q<TYPE, NCOLS, 2, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
+            else MI355_LAUNCH((k_gemv_q<TYPE, NCOLS, 4, true>), dim3(grid), dim3(256), lds, s, m, aq, ads, K);
             return;
         }
     }
-    if (rpw == 1) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 1, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
-    else if (rpw == 2) hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 2, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
-    else hipLaunchKernelGGL((k_gemv_q<TYPE, NCOLS, 4, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    if (rpw == 1) MI355_LAUNCH((k_gemv_q<TYPE, NCOLS, 1, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    else if (rpw == 2) MI355_LAUNCH((k_gemv_q<TYPE, NCOLS, 2, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
+    else MI355_LAUNCH((k_gemv_q<TYPE, NCOLS, 4, false>), dim3(grid), dim3(256), 0, s, m, aq, ads, K);
 }
 
 template <int TYPE>
@@ -662,26 +662,26 @@ static int vec_q_rope_impl(void *stream, int n_mats, const mi355_gemv_rope_mat *
     const size_t lds = act_lds_bytes((int)B, K, groups);
     if (nx != nullptr) {
         rp.nx = nx; rp.nw = nw; rp.neps = neps;
-        hipLaunchKernelGGL(k_gemv_qkv_norm, dim3((unsigned)groups), dim3(256), (size_t)K + K / 4, s, b, (int)K, rp);
+        MI355_LAUNCH(k_gemv_qkv_norm, dim3((unsigned)groups), dim3(256), (size_t)K + K / 4, s, b, (int)K, rp);
         return launch_status("k_gemv_qkv_norm");
     }
     rp.nx = rp.nw = nullptr; rp.neps = 0.0f;
     switch (B) {
         case 1:
-            if (lds) hipLaunchKernelGGL((k_gemv_qkv<1, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
-            else hipLaunchKernelGGL((k_gemv_qkv<1, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            if (lds) MI355_LAUNCH((k_gemv_qkv<1, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else MI355_LAUNCH((k_gemv_qkv<1, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
             break;
         case 2:
-            if (lds) hipLaunchKernelGGL((k_gemv_qkv<2, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
-            else hipLaunchKernelGGL((k_gemv_qkv<2, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            if (lds) MI355_LAUNCH((k_gemv_qkv<2, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else MI355_LAUNCH((k_gemv_qkv<2, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
             break;
         case 3:
-            if (lds) hipLaunchKernelGGL((k_gemv_qkv<3, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
-            else hipLaunchKernelGGL((k_gemv_qkv<3, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            if (lds) MI355_LAUNCH((k_gemv_qkv<3, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else MI355_LAUNCH((k_gemv_qkv<3, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
             break;
         default:
-            if (lds) hipLaunchKernelGGL((k_gemv_qkv<4, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
-            else hipLaunchKernelGGL((k_gemv_qkv<4, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
+            if (lds) MI355_LAUNCH((k_gemv_qkv<4, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);
+            else MI355_LAUNCH((k_gemv_qkv<4, false>), dim3((unsigned)groups), dim3(256), 0, s, b, aq, ads, (int)K, rp);
             break;
     }
     return launch_status("k_gemv_qkv");
@@ -690,6 +690,12 @@ static int vec_q_rope_impl(void *stream, int n_mats, const mi355_gemv_rope_mat *
 int mi355_mul_mat_vec_q_rope(void *stream, int n_mats, const mi355_gemv_rope_mat *mats, const void *act, int64_t K, int64_t B,
                              const mi355_rope_desc *rope) {
     return vec_q_rope_impl(stream, n_mats, mats, act, K, B, rope, nullptr, nullptr, 0.0f);
+}
+
+int mi355_rms_norm_mul_mat_vec_q_rope(void *stream, const float *x, const float *norm_w, float eps, int n_mats, const mi355_gemv_rope_mat *mats,
+                                      int64_t K, const mi355_rope_desc *rope) {
+    MI355_REQUIRE(x != nullptr && norm_w != nullptr, "rms_norm_mul_mat_vec_q_rope: missing operands");
+    return vec_q_rope_impl(stream, n_mats, mats, nullptr, K, 1, rope, x, norm_w, eps);
 }
 
 int mi355_rms_norm_qkv_rope_store(void *stream, const float *x, const float *norm_w, float eps, int type_q, const void *wq, int type_k,
@@ -756,20 +762,20 @@ int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, in
     const size_t lds = act_lds_bytes((int)B, K, 2 * per);
     switch (B) {
         case 1:
-            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<1, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
-            else hipLaunchKernelGGL((k_gemv_gate_up<1, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            if (lds) MI355_LAUNCH((k_gemv_gate_up<1, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else MI355_LAUNCH((k_gemv_gate_up<1, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
             break;
         case 2:
-            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<2, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
-            else hipLaunchKernelGGL((k_gemv_gate_up<2, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            if (lds) MI355_LAUNCH((k_gemv_gate_up<2, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else MI355_LAUNCH((k_gemv_gate_up<2, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
             break;
         case 3:
-            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<3, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
-            else hipLaunchKernelGGL((k_gemv_gate_up<3, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            if (lds) MI355_LAUNCH((k_gemv_gate_up<3, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else MI355_LAUNCH((k_gemv_gate_up<3, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
             break;
         default:
-            if (lds) hipLaunchKernelGGL((k_gemv_gate_up<4, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
-            else hipLaunchKernelGGL((k_gemv_gate_up<4, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
+            if (lds) MI355_LAUNCH((k_gemv_gate_up<4, true>), grid, dim3(256), lds, s, b, aq, ads, (int)K, t);
+            else MI355_LAUNCH((k_gemv_gate_up<4, false>), grid, dim3(256), 0, s, b, aq, ads, (int)K, t);
             break;
     }
     return launch_status("k_gemv_gate_up");
@@ -789,10 +795,10 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
     if (!layout_aligned(as, L)) {
         const dim3 ugrid((unsigned)N, (unsigned)(n_used * T));
         switch (type) {
-            case MI355_Q4_0: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q4_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-            case MI355_Q8_0: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q8_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-            case MI355_Q4_K: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q4_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-            default: hipLaunchKernelGGL(k_gemv_id_unaligned<MI355_Q6_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            case MI355_Q4_0: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q4_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            case MI355_Q8_0: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q8_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            case MI355_Q4_K: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q4_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            default: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q6_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
         }
         return launch_status("k_gemv_id_unaligned");
     }
@@ -801,10 +807,10 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
     // an activation row of the split layout is 16-byte aligned inside the workspace when K % 64 == 0 (levels and scales)
     const size_t lds = K % 64 == 0 ? act_lds_bytes(1, K, (int64_t)grid.x * grid.y) : 0;
 #define MI355_ID_LAUNCH(TY)                                                                                           \
-    if (lds && rpw == 1) hipLaunchKernelGGL((k_gemv_id<TY, 1, true>), grid, dim3(256), lds, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
-    else if (lds) hipLaunchKernelGGL((k_gemv_id<TY, 2, true>), grid, dim3(256), lds, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
-    else if (rpw == 1) hipLaunchKernelGGL((k_gemv_id<TY, 1, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
-    else hipLaunchKernelGGL((k_gemv_id<TY, 2, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1);
+    if (lds && rpw == 1) MI355_LAUNCH((k_gemv_id<TY, 1, true>), grid, dim3(256), lds, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
+    else if (lds) MI355_LAUNCH((k_gemv_id<TY, 2, true>), grid, dim3(256), lds, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
+    else if (rpw == 1) MI355_LAUNCH((k_gemv_id<TY, 1, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
+    else MI355_LAUNCH((k_gemv_id<TY, 2, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1);
     switch (type) {
         case MI355_Q4_0: MI355_ID_LAUNCH(MI355_Q4_0) break;
         case MI355_Q8_0: MI355_ID_LAUNCH(MI355_Q8_0) break;
@@ -823,10 +829,10 @@ int mi355_block_dots_q8_1(void *stream, int type, const void *W, const void *a, 
     const act_ds *ads = (const act_ds *)(aq + K);
     const dim3 grid((unsigned)N);
     switch (type) {
-        case MI355_Q4_0: hipLaunchKernelGGL(k_block_dots<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-        case MI355_Q8_0: hipLaunchKernelGGL(k_block_dots<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-        case MI355_Q4_K: hipLaunchKernelGGL(k_block_dots<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-        default: hipLaunchKernelGGL(k_block_dots<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        case MI355_Q4_0: MI355_LAUNCH(k_block_dots<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        case MI355_Q8_0: MI355_LAUNCH(k_block_dots<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        case MI355_Q4_K: MI355_LAUNCH(k_block_dots<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        default: MI355_LAUNCH(k_block_dots<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
     }
     return launch_status("k_block_dots");
 }

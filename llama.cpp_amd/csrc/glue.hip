@@ -365,7 +365,7 @@ int mi355_rms_norm(void *stream, const mi355_tensor *src, const mi355_tensor *ds
     };
     if (n % 32 == 0 && n <= 16384 && packed(src) && packed(dst))
         return mi355_rms_norm_mul_quant(stream, (const float *)src->data, n, nullptr, (float *)dst->data, n, nullptr, n, nr, eps);
-    hipLaunchKernelGGL(k_rms_norm, dim3((unsigned)nr), dim3(row_threads(src->ne[0])), 0, (hipStream_t)stream, to_tens(src), to_tens(dst), eps);
+    MI355_LAUNCH(k_rms_norm, dim3((unsigned)nr), dim3(row_threads(src->ne[0])), 0, (hipStream_t)stream, to_tens(src), to_tens(dst), eps);
     return launch_status("k_rms_norm");
 }
 
@@ -380,10 +380,10 @@ int mi355_bin_bcast(void *stream, int op, const mi355_tensor *src0, const mi355_
     hipStream_t s = (hipStream_t)stream;
     const tens a = to_tens(src0), b = to_tens(src1), d = to_tens(dst);
     switch (op) {
-        case 0: hipLaunchKernelGGL(k_bin_bcast<0>, grid, block, 0, s, a, b, d, n); break;
-        case 1: hipLaunchKernelGGL(k_bin_bcast<1>, grid, block, 0, s, a, b, d, n); break;
-        case 2: hipLaunchKernelGGL(k_bin_bcast<2>, grid, block, 0, s, a, b, d, n); break;
-        default: hipLaunchKernelGGL(k_bin_bcast<3>, grid, block, 0, s, a, b, d, n); break;
+        case 0: MI355_LAUNCH(k_bin_bcast<0>, grid, block, 0, s, a, b, d, n); break;
+        case 1: MI355_LAUNCH(k_bin_bcast<1>, grid, block, 0, s, a, b, d, n); break;
+        case 2: MI355_LAUNCH(k_bin_bcast<2>, grid, block, 0, s, a, b, d, n); break;
+        default: MI355_LAUNCH(k_bin_bcast<3>, grid, block, 0, s, a, b, d, n); break;
     }
     return launch_status("k_bin_bcast");
 }
@@ -393,7 +393,7 @@ static int unary_launch(void *stream, int op, const mi355_tensor *src, const mi3
     MI355_REQUIRE(same_shape(src, dst), "unary: shapes differ");
     const int64_t n = nelements(dst);
     if (n == 0) return MI355_OK;
-    hipLaunchKernelGGL(k_unary, dim3(grid1d(n, 256)), dim3(256), 0, (hipStream_t)stream, op, to_tens(src), to_tens(dst), n, p);
+    MI355_LAUNCH(k_unary, dim3(grid1d(n, 256)), dim3(256), 0, (hipStream_t)stream, op, to_tens(src), to_tens(dst), n, p);
     return launch_status("k_unary");
 }
 
@@ -414,11 +414,11 @@ int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst) {
     hipStream_t s = (hipStream_t)stream;
     const tens a = to_tens(src), d = to_tens(dst);
     const int st = src->type, dt = dst->type;
-    if (st == MI355_F32 && dt == MI355_F32) hipLaunchKernelGGL((k_cpy<float, float>), grid, block, 0, s, a, d, n);
-    else if (st == MI355_F32 && dt == MI355_F16) hipLaunchKernelGGL((k_cpy<float, _Float16>), grid, block, 0, s, a, d, n);
-    else if (st == MI355_F16 && dt == MI355_F16) hipLaunchKernelGGL((k_cpy<_Float16, _Float16>), grid, block, 0, s, a, d, n);
-    else if (st == MI355_F16 && dt == MI355_F32) hipLaunchKernelGGL((k_cpy<_Float16, float>), grid, block, 0, s, a, d, n);
-    else if (st == MI355_I32 && dt == MI355_I32) hipLaunchKernelGGL((k_cpy<int32_t, int32_t>), grid, block, 0, s, a, d, n);
+    if (st == MI355_F32 && dt == MI355_F32) MI355_LAUNCH((k_cpy<float, float>), grid, block, 0, s, a, d, n);
+    else if (st == MI355_F32 && dt == MI355_F16) MI355_LAUNCH((k_cpy<float, _Float16>), grid, block, 0, s, a, d, n);
+    else if (st == MI355_F16 && dt == MI355_F16) MI355_LAUNCH((k_cpy<_Float16, _Float16>), grid, block, 0, s, a, d, n);
+    else if (st == MI355_F16 && dt == MI355_F32) MI355_LAUNCH((k_cpy<_Float16, float>), grid, block, 0, s, a, d, n);
+    else if (st == MI355_I32 && dt == MI355_I32) MI355_LAUNCH((k_cpy<int32_t, int32_t>), grid, block, 0, s, a, d, n);
     else {
         set_error("cpy: type pair %d -> %d not supported", st, dt);
         return MI355_ERR_ARG;
@@ -441,15 +441,15 @@ int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *id
         MI355_REQUIRE((int64_t)src->nb[1] == L.row_bytes, "get_rows: quantized rows must be whole and contiguous");
         hipStream_t s = (hipStream_t)stream;
         switch (src->type) {
-            case MI355_Q4_0: hipLaunchKernelGGL(k_get_rows_q<MI355_Q4_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-            case MI355_Q8_0: hipLaunchKernelGGL(k_get_rows_q<MI355_Q8_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-            case MI355_Q4_K: hipLaunchKernelGGL(k_get_rows_q<MI355_Q4_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-            default: hipLaunchKernelGGL(k_get_rows_q<MI355_Q6_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            case MI355_Q4_0: MI355_LAUNCH(k_get_rows_q<MI355_Q4_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            case MI355_Q8_0: MI355_LAUNCH(k_get_rows_q<MI355_Q8_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            case MI355_Q4_K: MI355_LAUNCH(k_get_rows_q<MI355_Q4_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            default: MI355_LAUNCH(k_get_rows_q<MI355_Q6_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
         }
         return launch_status("k_get_rows_q");
     }
-    if (src->type == MI355_F32) hipLaunchKernelGGL(k_get_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
-    else hipLaunchKernelGGL(k_get_rows<_Float16>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
+    if (src->type == MI355_F32) MI355_LAUNCH(k_get_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
+    else MI355_LAUNCH(k_get_rows<_Float16>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);
     return launch_status("k_get_rows");
 }
 
@@ -459,8 +459,8 @@ int mi355_set_rows(void *stream, const mi355_tensor *src, const int32_t *rows, c
     const int64_t n = nelements(src);
     if (n == 0) return MI355_OK;
     const dim3 grid(grid1d(n, 256)), block(256);
-    if (dst->type == MI355_F16) hipLaunchKernelGGL(k_set_rows<_Float16>, grid, block, 0, (hipStream_t)stream, to_tens(src), rows, to_tens(dst), n);
-    else hipLaunchKernelGGL(k_set_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), rows, to_tens(dst), n);
+    if (dst->type == MI355_F16) MI355_LAUNCH(k_set_rows<_Float16>, grid, block, 0, (hipStream_t)stream, to_tens(src), rows, to_tens(dst), n);
+    else MI355_LAUNCH(k_set_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), rows, to_tens(dst), n);
     return launch_status("k_set_rows");
 }
 
@@ -482,9 +482,9 @@ int mi355_soft_max(void *stream, const mi355_tensor *src, const mi355_tensor *ma
     const dim3 grid((unsigned)nr), block(row_threads(src->ne[0]));
     hipStream_t s = (hipStream_t)stream;
     if (mask && mask->type == MI355_F16)
-        hipLaunchKernelGGL(k_soft_max<_Float16>, grid, block, 0, s, to_tens(src), (const _Float16 *)mask->data, to_tens(dst), scale, max_bias, m0, m1, n2);
+        MI355_LAUNCH(k_soft_max<_Float16>, grid, block, 0, s, to_tens(src), (const _Float16 *)mask->data, to_tens(dst), scale, max_bias, m0, m1, n2);
     else
-        hipLaunchKernelGGL(k_soft_max<float>, grid, block, 0, s, to_tens(src), (const float *)(mask ? mask->data : nullptr), to_tens(dst), scale, max_bias, m0, m1, n2);
+        MI355_LAUNCH(k_soft_max<float>, grid, block, 0, s, to_tens(src), (const float *)(mask ? mask->data : nullptr), to_tens(dst), scale, max_bias, m0, m1, n2);
     return launch_status("k_soft_max");
 }
 
@@ -511,7 +511,7 @@ int mi355_rope(void *stream, const mi355_tensor *src, const int32_t *pos, const 
     const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
     p.corr0 = c0 > 0 ? c0 : 0;
     p.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
-    hipLaunchKernelGGL(k_rope, dim3((unsigned)nr), dim3(64), 0, (hipStream_t)stream, to_tens(src), pos, freq_factors, to_tens(dst), p);
+    MI355_LAUNCH(k_rope, dim3((unsigned)nr), dim3(64), 0, (hipStream_t)stream, to_tens(src), pos, freq_factors, to_tens(dst), p);
     return launch_status("k_rope");
 }
 
@@ -522,7 +522,7 @@ int mi355_sum_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ds
     const int64_t nr = nrows(src);
     if (nr == 0) return MI355_OK;
     MI355_REQUIRE(nr < 0x7fffffff, "sum_rows: too many rows");
-    hipLaunchKernelGGL(k_sum_rows, dim3((unsigned)nr), dim3(row_threads(src->ne[0])), 0, (hipStream_t)stream, to_tens(src), to_tens(dst));
+    MI355_LAUNCH(k_sum_rows, dim3((unsigned)nr), dim3(row_threads(src->ne[0])), 0, (hipStream_t)stream, to_tens(src), to_tens(dst));
     return launch_status("k_sum_rows");
 }
 
@@ -537,7 +537,7 @@ int mi355_argsort(void *stream, const mi355_tensor *src, const mi355_tensor *dst
     int npad = 1;
     while (npad < src->ne[0]) npad *= 2;
     const int threads = npad < 64 ? 64 : (npad > 256 ? 256 : npad);
-    hipLaunchKernelGGL(k_argsort, dim3((unsigned)nr), dim3(threads), npad * sizeof(int), (hipStream_t)stream, to_tens(src), to_tens(dst), order, npad);
+    MI355_LAUNCH(k_argsort, dim3((unsigned)nr), dim3(threads), npad * sizeof(int), (hipStream_t)stream, to_tens(src), to_tens(dst), order, npad);
     return launch_status("k_argsort");
 }
 
@@ -558,11 +558,11 @@ int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *
     const dim3 block(256);
     hipStream_t s = (hipStream_t)stream;
     if (src0->type == MI355_F32) {
-        if (vec) hipLaunchKernelGGL((k_mul_mat_f<float, true>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
-        else hipLaunchKernelGGL((k_mul_mat_f<float, false>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+        if (vec) MI355_LAUNCH((k_mul_mat_f<float, true>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+        else MI355_LAUNCH((k_mul_mat_f<float, false>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
     } else {
-        if (vec) hipLaunchKernelGGL((k_mul_mat_f<_Float16, true>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
-        else hipLaunchKernelGGL((k_mul_mat_f<_Float16, false>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+        if (vec) MI355_LAUNCH((k_mul_mat_f<_Float16, true>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
+        else MI355_LAUNCH((k_mul_mat_f<_Float16, false>), grid, block, 0, s, to_tens(src0), to_tens(src1), to_tens(dst));
     }
     return launch_status("k_mul_mat_f");
 }

@@ -463,12 +463,12 @@ static void launch_mmq(hipStream_t s, const void *W, const void *act, float *dst
     int n_slices = mmq_slices(N, K, B);
     if (n_slices > 1 && (ws == nullptr || ((uintptr_t)ws & 15) != 0 || ws_bytes < (size_t)n_slices * (size_t)N * (size_t)B * sizeof(float))) n_slices = 1;
     if (n_slices > 1) {
-        hipLaunchKernelGGL((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded, (unsigned)n_slices), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
+        MI355_LAUNCH((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded, (unsigned)n_slices), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
                            (float *)ws, N, K, B, N, L, n_col_tiles, n_groups, n_groups_padded);
-        hipLaunchKernelGGL(k_mmq_split_sum, dim3((unsigned)((N * B + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, N, B, dst_stride, n_slices);
+        MI355_LAUNCH(k_mmq_split_sum, dim3((unsigned)((N * B + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, N, B, dst_stride, n_slices);
         return;
     }
-    hipLaunchKernelGGL((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
+    MI355_LAUNCH((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
                        dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded);
 }
 

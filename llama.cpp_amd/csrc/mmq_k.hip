@@ -1070,7 +1070,7 @@ static int usable_slices(int64_t N, int64_t K, int64_t B, const void *ws, size_t
 }
 
 static void launch_split_sum(hipStream_t s, const float *part, float *dst, const float *residual, int64_t N, int64_t B, int64_t dst_stride, int n) {
-    hipLaunchKernelGGL(k_split_sum, dim3((unsigned)((N * B / 4 + 255) / 256)), dim3(256), 0, s, part, dst, residual, N, B, dst_stride, n);
+    MI355_LAUNCH(k_split_sum, dim3((unsigned)((N * B / 4 + 255) / 256)), dim3(256), 0, s, part, dst, residual, N, B, dst_stride, n);
 }
 
 template <int TYPE>
@@ -1087,12 +1087,12 @@ static void launch_mmq_k(hipStream_t s, const void *W, const void *act, float *d
     const int n_groups_padded = (n_groups + 7) & ~7;
     const int n_slices = usable_slices(N, K, B, ws, ws_bytes);
     if (n_slices > 1) {
-        hipLaunchKernelGGL((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded, (unsigned)n_slices), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_,
+        MI355_LAUNCH((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded, (unsigned)n_slices), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_,
                            (float *)ws, nullptr, N, K, B, N, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
         launch_split_sum(s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
         return;
     }
-    hipLaunchKernelGGL((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_, dst, residual, N, K,
+    MI355_LAUNCH((k_mmq_kp<TYPE, false>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ad8, abs_, dst, residual, N, K,
                        B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq_route{});
 }
 
@@ -1156,7 +1156,7 @@ static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int6
     const int bn = route_bn(n_expert, S);
     const int max_tiles = (int)((S + bn - 1) / bn + n_expert);
     int32_t *act_row = (int32_t *)route_ws, *dst_row = act_row + S, *tiles = dst_row + S, *n_tiles = tiles + 4 * (int64_t)route_max_tiles(n_expert, S);
-    hipLaunchKernelGGL(k_route_slots, dim3(1), dim3(1024), 0, s, ids, ids_stride, n_expert, n_used, nb1, T, bn, act_row, dst_row, tiles, n_tiles);
+    MI355_LAUNCH(k_route_slots, dim3(1), dim3(1024), 0, s, ids, ids_stride, n_expert, n_used, nb1, T, bn, act_row, dst_row, tiles, n_tiles);
     const row_layout L = make_row_layout(TYPE, K);
     const int8_t *aq = (const int8_t *)act;
     const float *ad8 = (const float *)(aq + q8k_d_offset(K, act_rows));
@@ -1166,10 +1166,10 @@ static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int6
     const int n_groups_padded = (n_groups + 7) & ~7;
     const mmq_route route = {act_row, dst_row, tiles, n_tiles, N * L.row_bytes};
     if (bn == 64)
-        hipLaunchKernelGGL((k_mmq_k<TYPE, 1, 1, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
+        MI355_LAUNCH((k_mmq_k<TYPE, 1, 1, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
                            dst, nullptr, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
     else
-        hipLaunchKernelGGL((k_mmq_kp<TYPE, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_, dst, nullptr, N, K,
+        MI355_LAUNCH((k_mmq_kp<TYPE, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_, dst, nullptr, N, K,
                            S, N, L, max_tiles, n_groups, n_groups_padded, route);
 }
 
@@ -1194,7 +1194,7 @@ int mi355_quantize_act_q8k(void *stream, const float *x, void *act, int64_t k, i
     float *d8 = (float *)(q + q8k_d_offset(k, nrows));
     _Float16 *bs = (_Float16 *)(q + q8k_bs_offset(k, nrows));
     const dim3 grid((unsigned)((k / QKK + 3) / 4), (unsigned)nrows);
-    hipLaunchKernelGGL(k_quantize_q8k, grid, dim3(256), 0, (hipStream_t)stream, x, q, d8, bs, k, x_stride);
+    MI355_LAUNCH(k_quantize_q8k, grid, dim3(256), 0, (hipStream_t)stream, x, q, d8, bs, k, x_stride);
     return launch_status("k_quantize_q8k");
 }
 
@@ -1238,8 +1238,8 @@ int mi355_kq_unpack_planes(void *stream, int type, const void *W, void *planes, 
     const int64_t pieces = rows * (K >> 8) * 8;
     MI355_REQUIRE((pieces + 255) / 256 < 0x7fffffff, "kq_unpack_planes: too many pieces for one launch");
     const dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
-    if (type == MI355_Q4_K) hipLaunchKernelGGL(k_unpack_planes<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)planes, rows, K, L);
-    else hipLaunchKernelGGL(k_unpack_planes<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)planes, rows, K, L);
+    if (type == MI355_Q4_K) MI355_LAUNCH(k_unpack_planes<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)planes, rows, K, L);
+    else MI355_LAUNCH(k_unpack_planes<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)planes, rows, K, L);
     return launch_status("k_unpack_planes");
 }
 
@@ -1278,10 +1278,10 @@ int mi355_mul_mat_q8k_planes_ws(void *stream, int type, const void *planes, cons
     const float *res = n_slices > 1 ? nullptr : residual;
     const int64_t out_stride = n_slices > 1 ? N : dst_stride;
     if (type == MI355_Q4_K)
-        hipLaunchKernelGGL((k_mmq_pl<MI355_Q4_K, false>), grid, dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, out, res, N, K, B, out_stride, L,
+        MI355_LAUNCH((k_mmq_pl<MI355_Q4_K, false>), grid, dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, out, res, N, K, B, out_stride, L,
                            n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
     else
-        hipLaunchKernelGGL((k_mmq_pl<MI355_Q6_K, false>), grid, dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, out, res, N, K, B, out_stride, L,
+        MI355_LAUNCH((k_mmq_pl<MI355_Q6_K, false>), grid, dim3(256), 0, s, (const int8_t *)planes, aq, ad8, abs_, out, res, N, K, B, out_stride, L,
                            n_col_tiles, n_groups, n_groups_padded, mmq_route{}, N * K);
     if (n_slices > 1) launch_split_sum(s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
     return launch_status("k_mmq_pl");

@@ -503,7 +503,7 @@ int mi355_quantize_act_q8k_tiled(void *stream, const float *x, void *act, int64_
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "quantize_act_q8k_tiled: workspace must be 16-byte aligned");
     const int64_t b16 = (nrows + 15) & ~(int64_t)15;
     const dim3 grid((unsigned)((k / QKK + 3) / 4), (unsigned)b16);
-    hipLaunchKernelGGL(k_quantize_q8k_tiled, grid, dim3(256), 0, (hipStream_t)stream, x, (uint8_t *)act, k, nrows, x_stride);
+    MI355_LAUNCH(k_quantize_q8k_tiled, grid, dim3(256), 0, (hipStream_t)stream, x, (uint8_t *)act, k, nrows, x_stride);
     return launch_status("k_quantize_q8k_tiled");
 }
 
@@ -520,8 +520,8 @@ int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, in
     const int64_t pieces = ((rows + 15) & ~(int64_t)15) * (K >> 8) * 8;
     MI355_REQUIRE((pieces + 255) / 256 < 0x7fffffff, "kq_unpack_tiles: too many pieces for one launch");
     const dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
-    if (type == MI355_Q4_K) hipLaunchKernelGGL(k_unpack_tiles<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
-    else hipLaunchKernelGGL(k_unpack_tiles<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
+    if (type == MI355_Q4_K) MI355_LAUNCH(k_unpack_tiles<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
+    else MI355_LAUNCH(k_unpack_tiles<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
     return launch_status("k_unpack_tiles");
 }
 
@@ -549,11 +549,11 @@ int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const voi
     const float *res = n_slices > 1 ? nullptr : residual;
     const int64_t out_stride = n_slices > 1 ? N : dst_stride;
     if (type == MI355_Q4_K)
-        hipLaunchKernelGGL(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
+        MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
     else
-        hipLaunchKernelGGL(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
+        MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
     if (n_slices > 1)
-        hipLaunchKernelGGL(k_wt_split_sum, dim3((unsigned)((N * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
+        MI355_LAUNCH(k_wt_split_sum, dim3((unsigned)((N * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
     return launch_status("k_mmq_w");
 }
 

@@ -90,7 +90,7 @@ int mi355_moe_route(void *stream, const float *logits, float *probs, int32_t *or
     MI355_REQUIRE(T >= 0 && T < 0x7fffffff, "moe_route: bad token count");
     MI355_REQUIRE(logits && probs && order, "moe_route: null operand");
     if (T == 0) return MI355_OK;
-    hipLaunchKernelGGL(k_moe_route, dim3((unsigned)T), dim3(64), 0, (hipStream_t)stream, logits, probs, order, (int)n_expert);
+    MI355_LAUNCH(k_moe_route, dim3((unsigned)T), dim3(64), 0, (hipStream_t)stream, logits, probs, order, (int)n_expert);
     return launch_status("k_moe_route");
 }
 
@@ -101,7 +101,7 @@ int mi355_moe_weights(void *stream, const float *probs, const int32_t *ids, int6
     MI355_REQUIRE(T >= 0 && T < 0x7fffffff, "moe_weights: bad token count");
     MI355_REQUIRE(probs && ids && raw && sum && norm, "moe_weights: null operand");
     if (T == 0) return MI355_OK;
-    hipLaunchKernelGGL(k_moe_weights, dim3((unsigned)T), dim3(64), 0, (hipStream_t)stream, probs, ids, ids_stride, raw, sum, norm, (int)n_expert,
+    MI355_LAUNCH(k_moe_weights, dim3((unsigned)T), dim3(64), 0, (hipStream_t)stream, probs, ids, ids_stride, raw, sum, norm, (int)n_expert,
                        (int)n_used);
     return launch_status("k_moe_weights");
 }
@@ -114,7 +114,7 @@ int mi355_moe_combine(void *stream, const float *experts, const float *weights, 
     MI355_REQUIRE((((uintptr_t)experts | (uintptr_t)scaled | (uintptr_t)residual | (uintptr_t)out) & 15) == 0, "moe_combine: operands must be 16-byte aligned");
     if (T == 0) return MI355_OK;
     const dim3 grid((unsigned)((n_embd / 4 + 255) / 256), (unsigned)T);
-    hipLaunchKernelGGL(k_moe_combine, grid, dim3(256), 0, (hipStream_t)stream, experts, weights, scaled, residual, out, n_embd, (int)n_used);
+    MI355_LAUNCH(k_moe_combine, grid, dim3(256), 0, (hipStream_t)stream, experts, weights, scaled, residual, out, n_embd, (int)n_used);
     return launch_status("k_moe_combine");
 }
 

@@ -36,10 +36,10 @@ int gemv_unaligned(hipStream_t s, int type, const void *W, const void *act, floa
     MI355_REQUIRE(B <= 65535, "mul_mat: batch %lld too large for the unaligned path", (long long)B);
     const dim3 grid((unsigned)N, (unsigned)B);
     switch (type) {
-        case MI355_Q4_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-        case MI355_Q8_0: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-        case MI355_Q4_K: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-        default: hipLaunchKernelGGL(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        case MI355_Q4_0: MI355_LAUNCH(k_gemv_unaligned<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        case MI355_Q8_0: MI355_LAUNCH(k_gemv_unaligned<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        case MI355_Q4_K: MI355_LAUNCH(k_gemv_unaligned<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        default: MI355_LAUNCH(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
     }
     return launch_status("k_gemv_unaligned");
 }

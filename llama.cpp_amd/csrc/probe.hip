@@ -25,6 +25,6 @@ __global__ void __launch_bounds__(64) k_probe_clock(long long *out, long long re
 
 extern "C" int mi355_probe_clock(void *stream, int64_t *out, int64_t micros) {
     MI355_REQUIRE(out != nullptr && micros > 0 && micros <= 1000000, "probe_clock: bad arguments");
-    hipLaunchKernelGGL(mi355::k_probe_clock, dim3(1), dim3(64), 0, (hipStream_t)stream, (long long *)out, (long long)micros * 100);
+    MI355_LAUNCH(mi355::k_probe_clock, dim3(1), dim3(64), 0, (hipStream_t)stream, (long long *)out, (long long)micros * 100);
     return mi355::launch_status("k_probe_clock");
 }

@@ -2,12 +2,17 @@
 #include "common.hpp"
 #include "qdot.hpp"
 
+#include <atomic>
 #include <stdarg.h>
 #include <string.h>
 
 namespace mi355 {
 
 static thread_local char g_err[512] = "";
+static std::atomic<uint64_t> g_launches{0};
+
+void count_launch() { g_launches.fetch_add(1, std::memory_order_relaxed); }
+uint64_t launches_so_far() { return g_launches.load(std::memory_order_relaxed); }
 
 void set_error(const char *fmt, ...) {
     va_list ap;
@@ -132,10 +137,10 @@ static int weights_permute(bool scatter, void *stream, int type, const void *src
     const size_t nblocks = (size + 255) / 256;
     MI355_REQUIRE(nblocks < 0x7fffffffull, "weights layout: range too large for one launch");
     if (scatter)
-        hipLaunchKernelGGL(k_weights_permute<true>, dim3((unsigned)nblocks), dim3(256), 0, s, type, (const uint8_t *)src,
+        MI355_LAUNCH(k_weights_permute<true>, dim3((unsigned)nblocks), dim3(256), 0, s, type, (const uint8_t *)src,
                            (uint8_t *)dst, nb, row_bytes, offset, size);
     else
-        hipLaunchKernelGGL(k_weights_permute<false>, dim3((unsigned)nblocks), dim3(256), 0, s, type, (const uint8_t *)src,
+        MI355_LAUNCH(k_weights_permute<false>, dim3((unsigned)nblocks), dim3(256), 0, s, type, (const uint8_t *)src,
                            (uint8_t *)dst, nb, row_bytes, offset, size);
     return launch_status("k_weights_permute");
 }
@@ -149,6 +154,7 @@ extern "C" {
 int mi355_abi_version(void) { return 1; }
 
 const char *mi355_last_error(void) { return g_err; }
+uint64_t mi355_launch_count(void) { return launches_so_far(); }
 
 int mi355_device_supported(int device) {
     hipDeviceProp_t prop;
@@ -179,9 +185,9 @@ static int quantize_launch(bool std_layout, void *stream, const float *x, void *
     if (nrows == 0) return MI355_OK;
     const dim3 grid((unsigned)((k + 1023) / 1024), (unsigned)nrows);
     if (std_layout)
-        hipLaunchKernelGGL(k_quantize_q8_1<true>, grid, dim3(256), 0, (hipStream_t)stream, x, y, k, nrows, x_stride);
+        MI355_LAUNCH(k_quantize_q8_1<true>, grid, dim3(256), 0, (hipStream_t)stream, x, y, k, nrows, x_stride);
     else
-        hipLaunchKernelGGL(k_quantize_q8_1<false>, grid, dim3(256), 0, (hipStream_t)stream, x, y, k, nrows, x_stride);
+        MI355_LAUNCH(k_quantize_q8_1<false>, grid, dim3(256), 0, (hipStream_t)stream, x, y, k, nrows, x_stride);
     return launch_status("k_quantize_q8_1");
 }
 

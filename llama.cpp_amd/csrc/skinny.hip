@@ -344,12 +344,12 @@ void launch_skinny(hipStream_t s, const void *W, const int8_t *aq, const act_ds 
     const int steps_per_wave = (steps_per_slice + 3) / 4;
     const dim3 grid((unsigned)((N + 31) / 32), (unsigned)slices);
     if (slices == 1) {
-        hipLaunchKernelGGL((k_mm_skinny<TYPE, NI>), grid, dim3(256), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, B, dst_stride, steps_per_slice,
+        MI355_LAUNCH((k_mm_skinny<TYPE, NI>), grid, dim3(256), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, B, dst_stride, steps_per_slice,
                            steps_per_wave);
     } else {
-        hipLaunchKernelGGL((k_mm_skinny<TYPE, NI>), grid, dim3(256), 0, s, (const uint8_t *)W, aq, ads, part, (const float *)nullptr, N, K, B, N, steps_per_slice,
+        MI355_LAUNCH((k_mm_skinny<TYPE, NI>), grid, dim3(256), 0, s, (const uint8_t *)W, aq, ads, part, (const float *)nullptr, N, K, B, N, steps_per_slice,
                            steps_per_wave);
-        hipLaunchKernelGGL(k_skinny_slices, dim3((unsigned)((N + 255) / 256), (unsigned)B), dim3(256), 0, s, part, dst, residual, N, B, dst_stride, slices);
+        MI355_LAUNCH(k_skinny_slices, dim3((unsigned)((N + 255) / 256), (unsigned)B), dim3(256), 0, s, part, dst, residual, N, B, dst_stride, slices);
     }
 }
 

@@ -30,6 +30,7 @@ class Tensor(C.Structure):
 _SIGNATURES = {
     "mi355_abi_version": (_int, []),
     "mi355_last_error": (C.c_char_p, []),
+    "mi355_launch_count": (C.c_uint64, []),
     "mi355_device_supported": (_int, [_int]),
     "mi355_probe_clock": (_int, [_p, _p, _i64]),
     "mi355_weights_scatter": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),

@@ -137,3 +137,38 @@ def test_decode_graph_replay_equals_launch_by_launch(dev, tmp_path, moe):
     assert st["captures"] >= 2 and st["replays"] >= 8, st
     assert replayed.shape == launched.shape and np.isfinite(replayed).all()
     assert np.array_equal(replayed, launched)
+
+
+def test_launches_per_layer(dev, tmp_path):
+    """What the plug-in launches for the reference's llama graphs, counted by the kernel library itself and reported per graph
+    under MI355_LOG_GRAPH (one-time copies of weights are reported apart): the difference between a 4-layer and a 2-layer
+    model is two layers' worth.  One decoded token takes 7 launches per layer ([norm + Q/K/V + rope + cache stores] [attention]
+    [wo + residual] [norm] [gate/up] [SiLU*up] [down + residual]).  A prompt of 200 tokens (the wide-tile GEMM; decode then
+    stays within 256 cache cells) takes 13 (norm, Q, K, V, [rope, rope, store, store], attention, quantization, wo + residual,
+    norm, gate, up, SiLU*up, down + residual) plus one reduction launch for each product that is split along K because it has
+    fewer tiles than the chip has compute units: Q, K, V, wo and down at this size."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import make_synthetic_gguf
+    counts = {}
+    for n_layer in (2, 4):
+        model = str(tmp_path / ("l%d.gguf" % n_layer))
+        make_synthetic_gguf.write_model(model, n_layer=n_layer, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=2048)
+        env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN, MI355_LOG_GRAPH="1", MI355_NO_GRAPH="1")
+        r = subprocess.run([LOGITS, model, "99", "200", "3", str(tmp_path / "o.bin")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                           text=True, timeout=600, cwd=os.path.dirname(LOGITS))
+        assert r.returncode == 0, r.stdout[-3000:]
+        per_batch = {}
+        for m in re.finditer(r"MI355 graph launches: (\d+) nodes, batch (\d+), (\d+) attention nodes, (\d+) kernel launches \+ (\d+) for one-time", r.stdout):
+            assert int(m.group(3)) == n_layer
+            per_batch[int(m.group(2))] = int(m.group(4))
+        assert 1 in per_batch and 200 in per_batch, r.stdout[-3000:]
+        counts[n_layer] = per_batch
+    decode = (counts[4][1] - counts[2][1]) / 2
+    prefill = (counts[4][200] - counts[2][200]) / 2
+    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+    with open(os.path.join(ROOT, "gpurun_out", "launches_per_layer.txt"), "w") as f:
+        f.write("decode %g launches per layer, prefill(200) %g; totals %r\n" % (decode, prefill, counts))
+    assert decode == 7, counts
+    assert prefill <= 13 + 5, counts
