@@ -76,6 +76,7 @@ _SIGNATURES = {
                             _f, _f, _f, _f, _f, _f]),
     "mi355_ffn_gate_up_swiglu": (_int, [_p, _int, _p, _int, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q_rope": (_int, [_p, _int, _p, _p, _i64, _i64, _p]),
+    "mi355_rms_norm_mul_mat_vec_q_rope": (_int, [_p, _p, _p, _f, _int, _p, _i64, _p]),
     "mi355_qkv_rope_store": (_int, [_p, _int, _p, _int, _p, _int, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64,
                                     _sz, _sz, _sz, _sz, _int, _int, _int, _f, _f, _f, _f, _f, _f]),
     "mi355_rms_norm_qkv_rope_store": (_int, [_p, _p, _p, _f, _int, _p, _int, _p, _int, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64,
