@@ -18,15 +18,116 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "llama.cpp_amd"))
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes one launch of the roofline kernel moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of this command,
-# calibrated on the copy kernel below (profiles/gemv_q4k_14336x4096_hbm_traffic.txt)
-GEMV_TRAFFIC_BYTES = 33169000
+# HBM bytes one launch of the roofline kernel moves: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings of this command, scaled by
+# the readings of the plain copy kernel the run ends with.  `python bench.py --traffic-from <fetch dir> <write dir>` turns the two
+# counter runs into this file, together with the commit they were measured at; the bench line quotes both.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv_gate_up_q4k_hbm_traffic.txt")
+ROOFLINE_KERNEL = "k_gemv_multi"        # as it appears in the profiler's kernel names
+COPY_KERNEL = "k_cpy"
+COPY_BYTES = 16384 * 4096 * 4           # read, and as many written
 
 
-def cpu_baseline(n_threads, budget_s=20.0):
-    """ggml-cpu (the reference's own CPU backend, built by oracle/Makefile) timed on this host:
-    batch-1 MUL_MAT over the weight shapes of one Q4_K_M layer plus the output projection, scaled to
-    32 layers -> tokens/s of the matmul part of tg (the rest of the graph is a few percent on CPU)."""
+def read_traffic():
+    """(bytes per launch or None, commit or None) from the tracked counter summary"""
+    try:
+        text = open(TRAFFIC_FILE).read()
+    except OSError:
+        return None, None
+    val = commit = None
+    for line in text.splitlines():
+        if line.startswith("traffic_bytes_per_launch:"):
+            val = int(line.split(":", 1)[1].strip())
+        if line.startswith("measured_at_commit:"):
+            commit = line.split(":", 1)[1].strip()
+    return val, commit
+
+
+def traffic_from(fetch_dir, write_dir):
+    """Reads the counter_collection.csv files of the two rocprofv3 --pmc runs and rewrites TRAFFIC_FILE.  Runs where the .git
+    directory is (the commit id goes into the file), on the CPU."""
+    import csv
+    import glob
+    import subprocess
+
+    def per_kernel(d, counter):
+        rows = {}
+        files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+        assert files, "no counter_collection.csv under " + d
+        for f in files:
+            for r in csv.DictReader(open(f)):
+                if r.get("Counter_Name") != counter:
+                    continue
+                rows.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return rows
+
+    out = {}
+    for d, counter in ((fetch_dir, "FETCH_SIZE"), (write_dir, "WRITE_SIZE")):
+        rows = per_kernel(d, counter)
+        cpy = [v for k, vs in rows.items() if COPY_KERNEL in k for v in vs]
+        ker = [v for k, vs in rows.items() if ROOFLINE_KERNEL in k for v in vs]
+        assert cpy and ker, "kernels not found in " + d
+        unit = COPY_BYTES / (sum(cpy) / len(cpy))          # bytes per counter unit, from the copy of known size
+        out[counter] = (sum(ker) / len(ker), len(ker), min(ker), max(ker), sum(cpy) / len(cpy), unit)
+    commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], stdout=subprocess.PIPE, text=True).stdout.strip() or "unknown"
+    fetch_b = out["FETCH_SIZE"][0] * out["FETCH_SIZE"][5]
+    write_b = out["WRITE_SIZE"][0] * out["WRITE_SIZE"][5]
+    lines = [
+        "HBM traffic of the roofline kernel of bench.py: k_gemv_multi<1 column, 2 rows per wave, activation copy in LDS> on the ffn_gate + ffn_up",
+        "matrices of one layer (2 x 14336 x 4096 Q4_K) - the launch a decoded token makes 32 times - on one MI355X",
+        "",
+        "commands (from /tmp, TMPDIR=/tmp; counters in their own runs, no trace domains):",
+        "  rocprofv3 --pmc FETCH_SIZE -d <fetch dir> -o f --output-format csv -- python3 bench.py --no-cpu --pp 0 --steps 4 --warmup 2",
+        "  rocprofv3 --pmc WRITE_SIZE -d <write dir> -o w --output-format csv -- python3 bench.py --no-cpu --pp 0 --steps 4 --warmup 2",
+        "  python bench.py --traffic-from <fetch dir> <write dir>        (where the repository is; writes this file)",
+        "",
+        "calibration: the run ends with one launch of the plain copy kernel k_cpy<float, float> on a 16384 x 4096 f32 tensor,",
+        "256 MiB read and 256 MiB written.",
+        "  k_cpy  FETCH_SIZE = %.1f  -> %.4f bytes per counter unit" % (out["FETCH_SIZE"][4], out["FETCH_SIZE"][5]),
+        "  k_cpy  WRITE_SIZE = %.1f  -> %.4f bytes per counter unit" % (out["WRITE_SIZE"][4], out["WRITE_SIZE"][5]),
+        "",
+        "%s, %d dispatches, per dispatch:" % (ROOFLINE_KERNEL, out["FETCH_SIZE"][1]),
+        "  FETCH_SIZE = %.1f units (min %.1f, max %.1f) = %d B read" % (out["FETCH_SIZE"][0], out["FETCH_SIZE"][2], out["FETCH_SIZE"][3], fetch_b),
+        "  WRITE_SIZE = %.1f units (min %.1f, max %.1f) = %d B written" % (out["WRITE_SIZE"][0], out["WRITE_SIZE"][2], out["WRITE_SIZE"][3], write_b),
+        "",
+        "traffic_bytes_per_launch: %d" % int(fetch_b + write_b),
+        "measured_at_commit: %s" % commit,
+        "",
+        "algorithmic bytes per launch: 2 x 14336 x 4096 x 144/256 (weights) + 4096 x 1.25 (Q8_1 activation: levels + scale/sum pairs)",
+        "  + 2 x 4 x 14336 (f32 outputs) = 66,060,288 + 5,120 + 114,688 = 66,180,096 B",
+    ]
+    with open(TRAFFIC_FILE, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    print("\n".join(lines))
+
+
+def physical_cores():
+    """distinct (package, core) pairs among the CPUs this process may run on, capped at the 16-thread share of a one-GPU box"""
+    allowed = os.sched_getaffinity(0)
+    cores = set()
+    cpu = phys = core = None
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("processor"):
+                cpu = int(line.split(":")[1])
+            elif line.startswith("physical id"):
+                phys = int(line.split(":")[1])
+            elif line.startswith("core id"):
+                core = int(line.split(":")[1])
+            elif not line.strip():
+                if cpu in allowed and phys is not None and core is not None:
+                    cores.add((phys, core))
+                cpu = phys = core = None
+    except OSError:
+        pass
+    n = len(cores) or len(allowed)
+    return max(1, min(n, 16)), n
+
+
+def cpu_baseline():
+    """ggml-cpu (the reference's own CPU backend, built by oracle/Makefile) timed on this host: batch-1 MUL_MAT over the weight
+    shapes of one Q4_K_M layer plus the output projection, each shape for at least a second after a warm-up run, summed with
+    the shapes' per-token multiplicities -> tokens/s of the matmul part of tg (the rest of the graph is a few percent on CPU).
+    Once with one thread per physical core of this process's share of the host, once with a single thread."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import numpy as np
     import orc
@@ -37,8 +138,8 @@ def cpu_baseline(n_threads, budget_s=20.0):
               ("wv6", 1024, 4096, orc.Q6_K, 16), ("wo", 4096, 4096, orc.Q4_K, 32), ("gate", 14336, 4096, orc.Q4_K, 32),
               ("up", 14336, 4096, orc.Q4_K, 32), ("down", 4096, 14336, orc.Q4_K, 16), ("down6", 4096, 14336, orc.Q6_K, 16),
               ("output", 128256, 4096, orc.Q6_K, 1)]
-    t_token = 0.0
-    t0 = time.time()
+    n_threads, n_phys = physical_cores()
+    t_token = {n_threads: 0.0, 1: 0.0}
     for name, N, K, t, count in shapes:
         # random blocks with sane scales: the CPU kernels' time does not depend on the values
         rb = orc.row_bytes(t, K)
@@ -53,14 +154,17 @@ def cpu_baseline(n_threads, budget_s=20.0):
             Wv[:, :, 208:210] = h
         x = rng.standard_normal((1, K)).astype(np.float32)
         out = np.zeros((1, N), dtype=np.float32)
-        reps = 3 if N > 20000 else 10
-        sec = orc.ref.ref_mul_mat(t, orc._ptr(W), orc._ptr(x), orc._ptr(out), N, K, 1, n_threads, reps)
-        t_token += sec * count
-        if time.time() - t0 > budget_s * 2:
-            break
-    return {"value": round(1.0 / t_token, 2), "unit": "tokens/s", "cores": n_threads, "kind": "reference",
-            "sample": "ggml-cpu (AVX2 build) batch-1 MUL_MAT over the 10 distinct weight shapes/types of the Q4_K_M model "
-                      "(3-10 runs each), summed with their per-token multiplicities (32 layers + output); matmuls only"}
+        for nt in sorted(t_token):
+            # ref_mul_mat makes one untimed run, then `reps` timed ones: a short probe sizes the >= 1 s loop
+            probe = orc.ref.ref_mul_mat(t, orc._ptr(W), orc._ptr(x), orc._ptr(out), N, K, 1, nt, 2)
+            reps = max(3, int(1.0 / max(probe, 1e-6)) + 1)
+            t_token[nt] += orc.ref.ref_mul_mat(t, orc._ptr(W), orc._ptr(x), orc._ptr(out), N, K, 1, nt, reps) * count
+    return {"value": round(1.0 / t_token[n_threads], 2), "unit": "tokens/s", "cores": n_threads, "kind": "reference",
+            "one_thread": round(1.0 / t_token[1], 2), "physical_cores_available": n_phys,
+            "sample": "ggml-cpu (AVX2 build of the reference sources) batch-1 MUL_MAT over the 10 distinct weight shapes/types of the "
+                      "Q4_K_M model, each timed for >= 1 s after a warm-up run, summed with their per-token multiplicities (32 layers "
+                      "+ output); matmuls only; threads = physical cores in this process's CPU share (at most 16); end-to-end CPU "
+                      "figures of the reference's llama-bench are in profiles/llama_bench_llama8b_q4km_cpu.txt"}
 
 
 INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA
@@ -215,7 +319,12 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
     ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, fattn, fattn_long (decode over 131072 cells only)")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="rewrite the tracked HBM-traffic summary from two rocprofv3 --pmc output directories (no GPU needed)")
     args = ap.parse_args()
+    if args.traffic_from:
+        traffic_from(*args.traffic_from)
+        return
     if args.sweep:
         if args.gpus != 1:
             sys.exit("bench.py: one GPU only")
@@ -300,26 +409,58 @@ def main():
             pp = T * reps / (time.perf_counter() - t0)
 
     # ------------------------------------------------------------------ roofline of the dominant kernel
-    # k_gemv_q<Q4_K, batch 1> on ffn_gate/ffn_up (14336 x 4096): 64 of the 226 matrices and 46% of the
-    # bytes of a decoded token.  Timed with HIP events on its own stream over the 64 distinct matrices
-    # (2.1 GB, so neither L2 nor the 256 MB Infinity Cache can serve them).
+    # k_gemv_multi on ffn_gate + ffn_up (2 x 14336 x 4096 Q4_K in one launch): what the timed step launches 32 times per token,
+    # 46% of the bytes of a decoded token.  Timed with HIP events on its own stream through the runner's own call, over the 32
+    # layers' matrices (2.1 GB, so neither L2 nor the 256 MB Infinity Cache can serve them).
     N, K = cfg.n_ff, cfg.n_embd
-    mats = [L[k][1] for L in weights.layers for k in ("gate", "up")]
-    x = torch.randn(1, K, device=dev)
-    act = mi355.quantize_act(x)
-    out = torch.empty(1, N, device=dev)
+    pairs = [[(L["gate"], run.gate[:1]), (L["up"], run.up[:1])] for L in weights.layers]
     with torch.cuda.stream(stream):
-        for W in mats[:4]:
-            mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, mi355.Q4_K, W.data_ptr(), act.data_ptr(), out.data_ptr(), N, K, 1, N))
+        run._norm_quant(run.x[:1], weights.layers[0]["ffn_norm"], run.act_c, 1)
+        for gu in pairs[:4]:
+            run._mm_act(gu, run.act_c, K, 1)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        nrep = 4
+        nrep = 8
         e0.record(stream)
         for _ in range(nrep):
-            for W in mats:
-                mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, mi355.Q4_K, W.data_ptr(), act.data_ptr(), out.data_ptr(), N, K, 1, N))
+            for gu in pairs:
+                run._mm_act(gu, run.act_c, K, 1)
         e1.record(stream)
         stream.synchronize()
-    us = e0.elapsed_time(e1) * 1e3 / (nrep * len(mats))
+    us = e0.elapsed_time(e1) * 1e3 / (nrep * len(pairs))
+    wtypes = {t for gu in pairs for (t, _), _ in gu}
+    assert wtypes == {mi355.Q4_K}, "the roofline kernel's byte count assumes Q4_K gate/up matrices"
+    alg_bytes = 2 * (N * K * 144 // 256) + (K + K // 4) + 2 * 4 * N      # weights + Q8_1 activation + two f32 outputs
+    achieved = alg_bytes / us / 1e3                                       # GB/s
+    traffic, traffic_commit = read_traffic()
+    roofline = {"kernel": "k_gemv_multi<1 column, 2 rows per wave, activation in LDS> on ffn_gate + ffn_up, 2 x 14336 x 4096 Q4_K (the launch the timed "
+                          "step makes once per layer)", "bound": "hbm", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "traffic_source": "profiles/%s, measured at commit %s" % (os.path.basename(TRAFFIC_FILE), traffic_commit) if traffic else None,
+                "us_per_launch": round(us, 3), "algorithmic_bytes_per_launch": alg_bytes}
+
+    # ------------------------------------------------------------------ ... and of the dominant prefill kernel
+    # k_mmq_w<Q4_K> (wide-tile int8-MFMA GEMM on tile images) on ffn_gate / ffn_up at the prompt's batch: 2 of the 7 products of a
+    # layer and 56% of its multiply-adds.  The same call the prefill pass makes, over the 64 matrices' tile images.
+    roofline_pp = None
+    if args.pp >= 192:
+        T = args.pp
+        with torch.cuda.stream(stream):
+            run._norm_quant(run.x[:T], weights.layers[0]["ffn_norm"], run.act_a, T, 2)
+            mats = [[(L[k], (run.gate if k == "gate" else run.up)[:T])] for L in weights.layers for k in ("gate", "up")]
+            for m in mats[:2]:
+                run._mm_act(m, run.act_a, K, T, q8k=2)
+            p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            p0.record(stream)
+            for m in mats:
+                run._mm_act(m, run.act_a, K, T, q8k=2)
+            p1.record(stream)
+            stream.synchronize()
+        pus = p0.elapsed_time(p1) * 1e3 / len(mats)
+        ops = 2.0 * N * K * T
+        roofline_pp = {"kernel": "k_mmq_w<Q4_K> 14336 x 4096, batch %d (ffn_gate / ffn_up of the prefill pass)" % T, "bound": "mfma",
+                       "achieved": round(ops / pus / 1e6, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops / pus / 1e6 / INT8_PEAK_TOPS, 4),
+                       "traffic": None, "us_per_launch": round(pus, 2), "ops_per_launch": ops}
+
     # reference for the HBM traffic counters: a plain copy kernel of known size (256 MiB read, 256 MiB written) whose
     # FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit when this command runs under rocprofv3 --pmc
     import ctypes as C
@@ -330,22 +471,17 @@ def main():
         mi355.check(lib.mi355_cpy(stream.cuda_stream, C.byref(ds_), C.byref(dd_)))
         stream.synchronize()
     del src, dst_c
-    alg_bytes = N * K * 144 // 256 + 4 * K + 4 * N          # weights + f32 activation + f32 output
-    achieved = alg_bytes / us / 1e3                          # GB/s
-    roofline = {"kernel": "k_gemv_q<Q4_K, ncols 1> 14336x4096 (ffn_gate / ffn_up)", "bound": "hbm", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                "us_per_launch": round(us, 3), "algorithmic_bytes_per_launch": alg_bytes}
 
     cpu = None
     if not args.no_cpu:
         try:
-            cpu = cpu_baseline(min(16, os.cpu_count() or 1))
+            cpu = cpu_baseline()
         except Exception as e:   # the baseline is a reported extra; never let it take the GPU numbers down
             cpu = {"error": repr(e)}
 
     weight_bytes = weights.matmul_bytes()
     result = {
-        "metric": "tg128 tokens/s (Llama-3-8B-shaped Q4_K_M, batch 1, flash attention, all ops on device)",
+        "metric": "tg%d tokens/s (Llama-3-8B-shaped Q4_K_M, batch 1, flash attention, all ops on device)" % args.steps,
         "value": round(tg, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 block dots (Q4_K/Q6_K weights x Q8_1 activations), f32 accumulate, f16 KV cache",
@@ -354,9 +490,10 @@ def main():
                                "head_dim 128, vocab 128256), KV positions %d..%d, n_kv padded to 256" % (args.warmup, args.warmup + args.steps - 1),
                    "launch": "host" if args.no_graph else "hip-graph replay", "weight_bytes_per_token": weight_bytes,
                    "hbm_fraction_of_step": round(weight_bytes / (ms_per_step * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)},
-        "pp512_tokens_per_s": round(pp, 1) if pp else None,
+        "pp%d_tokens_per_s" % args.pp: round(pp, 1) if pp else None,
         "outputs_finite": finite,
         "roofline": roofline,
+        "roofline_pp%d" % args.pp: roofline_pp,
         "cpu_baseline": cpu,
     }
     print(json.dumps(result))
