@@ -230,21 +230,23 @@ def sweep(kinds):
                     emit(kernel="MUL_MAT batch 1 (GEMV)" if B == 1 else "MUL_MAT batch %d (k_mm_skinny)" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
                          unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg)
                 del Ws
-    if "mmq" in kinds:
-        for t in (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q6_K):
-            for N, K in shapes:
-                for B in (64, 512):
+    if "mmq" in kinds or "mmq_wide" in kinds:
+        wide_only = "mmq" not in kinds    # the wide-tile GEMM alone on the gate/up shape (for counter collection)
+        for t in ((mi355.Q4_K, mi355.Q6_K) if wide_only else (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q6_K)):
+            for N, K in ([(14336, 4096)] if wide_only else shapes):
+                for B in ((512,) if wide_only else (64, 512)):
                     nm = 4
                     Ws = [mi355.upload_weights(t, lg.random_quantized(t, N, K, dev, gen)) for _ in range(nm)]
                     x = torch.randn(B, K, device=dev, generator=gen)
                     out = torch.empty(B, N, device=dev)
                     ws = torch.empty(int(lib.mi355_mul_mat_ws_bytes(K, B)) + max(int(lib.mi355_mul_mat_q8k_ws_bytes(N, K, B)), int(lib.mi355_mul_mat_q_ws_bytes(N, K, B))) + 256,
                                      dtype=torch.uint8, device=dev)
-                    us = timed(lambda i: mi355.check(lib.mi355_mul_mat(stream.cuda_stream, t, Ws[i].data_ptr(), x.data_ptr(), out.data_ptr(), N, K, B, K, N,
-                                                                       ws.data_ptr(), ws.numel())), nm, 5)
                     ops = 2.0 * N * K * B
-                    emit(kernel="MUL_MAT batch %d (activation quantization + tile GEMM)" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
-                         achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
+                    if not wide_only:
+                        us = timed(lambda i: mi355.check(lib.mi355_mul_mat(stream.cuda_stream, t, Ws[i].data_ptr(), x.data_ptr(), out.data_ptr(), N, K, B, K, N,
+                                                                           ws.data_ptr(), ws.numel())), nm, 5)
+                        emit(kernel="MUL_MAT batch %d (activation quantization + tile GEMM)" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
+                             achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
                     if t in (mi355.Q4_K, mi355.Q6_K):   # the wide-tile GEMM on tile images (what prefill uses for K-quants), without the quantization
                         tiles = [mi355.kq_unpack_tiles(t, W) for W in Ws]
                         a8 = mi355.quantize_act_q8k_tiled(x)
@@ -265,7 +267,7 @@ def sweep(kinds):
                              achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops,
                              shader_clock_mhz=round(mhz), frac_at_measured_clock=round(ops / us / 1e6 / (INT8_PEAK_TOPS * mhz / 2400.0), 4))
                         del tiles
-                    if t == mi355.Q6_K and B == 512:   # the same product from the unpacked planes (the 64 x 128 tile kernel)
+                    if t == mi355.Q6_K and B == 512 and not wide_only:   # the same product from the unpacked planes (the 64 x 128 tile kernel)
                         planes = [torch.empty(int(lib.mi355_kq_planes_bytes(N, K)) + 256, dtype=torch.uint8, device=dev) for _ in range(nm)]
                         for W, P in zip(Ws, planes):
                             mi355.check(lib.mi355_kq_unpack_planes(None, t, W.data_ptr(), P.data_ptr(), N, K))
@@ -318,7 +320,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
-    ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, fattn, fattn_long (decode over 131072 cells only)")
+    ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, mmq_wide (the wide-tile GEMM on 14336 x 4096 at batch 512 only), fattn, "
+                                          "fattn_long (decode over 131072 cells only)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="rewrite the tracked HBM-traffic summary from two rocprofv3 --pmc output directories (no GPU needed)")
     args = ap.parse_args()
