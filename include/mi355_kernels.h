@@ -401,6 +401,27 @@ int mi355_rms_norm_qkv_rope_store(void *stream, const float *x, const float *nor
 int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, int type_up, const void *w_up, const void *act, float *gate,
                              float *up, int64_t out_stride, void *act_out, unsigned *counters, int64_t N, int64_t K, int64_t B);
 
+/* Quantized KV cache (llama.cpp's -ctk / -ctv q8_0, q4_0).
+ * Where a block lives: with row_blocks = 0 blocks sit where ggml puts them (block g of a tensor at g * block bytes from its data).
+ * A tensor kept in the device row layout of mi355_weights_scatter (all levels of a row, then the row's scales) is addressed through
+ * the tensor that owns the memory: `base` = its data, row_blocks = blocks per row of THAT tensor; block g is then block
+ * g % row_blocks of row g / row_blocks, whatever view (1-D for the store, [D, cells, heads] for attention) is in use.
+ * cpy_f32_quant: CPY of contiguous f32 into n/32 consecutive Q8_0 / Q4_0 blocks starting at block dst_first_block - what
+ *   llm_build_kv_store (src/llama.cpp:157-199) does to k_cur / v_cur; the bytes of quantize_row_q8_0_ref / quantize_row_q4_0_ref
+ *   (ggml/src/ggml-quants.c:39-72, 194-218; ggml-cpu.c:3519-3830 converts row by row with the type's from_float).
+ * flash_attn_ext_kv: mi355_flash_attn_ext_quant over K and V of type MI355_F16, MI355_Q8_0 or MI355_Q4_0 each (ggml-cpu.c:10997-11003,
+ *   11040-11099).  k / v point at the first row in plain ggml addressing (row of (cell, head) at cell * nb1 + head * nb2); k_base /
+ *   v_base = data of the owning tensor (NULL: k / v themselves).  Quantized rows are expanded to f16 (d * level) in an image at the
+ *   end of the workspace and the f16 kernels run on the image; the reference instead quantizes q to Q8_0 and takes integer dots,
+ *   so results agree to the tolerance of the op (NMSE 5e-4), not to the bit.  ws: 256-byte aligned, at least
+ *   mi355_flash_attn_kv_ws_bytes.  D % 32 == 0. */
+int mi355_cpy_f32_quant(void *stream, int type, const float *src, void *dst_base, int64_t dst_first_block, int64_t dst_row_blocks, int64_t n);
+size_t mi355_flash_attn_kv_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, int type_k, int type_v);
+int mi355_flash_attn_ext_kv(void *stream, const float *q, const void *k, int type_k, const void *k_base, int64_t k_row_blocks, const void *v,
+                            int type_v, const void *v_base, int64_t v_row_blocks, const void *mask, float *dst, int64_t D, int64_t Nq, int64_t Nkv,
+                            int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2,
+                            size_t mask_nb1, float scale, float max_bias, float logit_softcap, void *ws, size_t ws_bytes, void *act);
+
 /* Mixture-of-experts glue of llm_build_moe_ffn (src/llama.cpp:417-530), each call the work of the consecutive graph nodes named,
  * writing every tensor those nodes write, bit-identical to running them one by one.  All operands contiguous.
  * moe_route: SOFT_MAX (no mask, scale 1) then ARGSORT descending: logits f32 [T][n_expert] -> probs f32, order i32 (ties by index;

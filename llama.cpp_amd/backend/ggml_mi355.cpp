@@ -79,6 +79,33 @@ mi355_tensor desc(const ggml_tensor * t) {
 
 bool strides_mult16(const ggml_tensor * t) { return t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0; }
 
+// A Q8_0 / Q4_0 tensor that is read or written block by block (a quantized KV cache).  Its memory belongs to `root` (the tensor
+// itself or the one it is a view of), which set_tensor keeps in the device row layout: blocks are addressed through the root's
+// rows, whatever shape the view has.
+struct kv_operand {
+    const void * p = nullptr;      // first byte in plain ggml addressing
+    const void * base = nullptr;   // data of the owning tensor
+    int64_t row_blocks = 0;        // blocks per row of the owning tensor
+    bool ok = false;
+};
+kv_operand kv_operand_of(const ggml_tensor * t) {
+    kv_operand o;
+    o.p = t->data;
+    if (t->type == GGML_TYPE_F16) {
+        o.ok = true;
+        return o;
+    }
+    if (t->type != GGML_TYPE_Q8_0 && t->type != GGML_TYPE_Q4_0) return o;
+    const ggml_tensor * root = t->view_src ? t->view_src : t;
+    const size_t bb = ggml_type_size(t->type);
+    if (root->type != t->type || !ggml_is_contiguous(root) || root->ne[0] % 32 != 0 || t->ne[0] % 32 != 0 || t->nb[0] != bb) return o;
+    if (t->nb[1] % bb != 0 || t->nb[2] % bb != 0 || t->nb[3] % bb != 0 || (t->view_src && t->view_offs % bb != 0)) return o;
+    o.base = root->data;
+    o.row_blocks = root->ne[0] / 32;
+    o.ok = true;
+    return o;
+}
+
 // ------------------------------------------------------------------------------- device state
 struct device_ctx {
     int device = 0;
@@ -353,6 +380,27 @@ void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) bu
 // number of rows / elements per row of a tensor whose rows are contiguous blocks
 int64_t tensor_nrows(const ggml_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
 
+// Q4_0, Q8_0 and Q6_K tensors live in the device row layout, which is defined by the rows of the tensor that owns the memory: a
+// view (a slice of experts, a permuted or 1-D view of a cache) addresses bytes of that tensor, so transfers through a view go
+// through the owner's layout at the view's byte offset.
+struct repack_target {
+    bool yes = false;
+    void * base = nullptr;   // the owner's data
+    int64_t k = 0, nrows = 0;
+    size_t off = 0;          // byte offset of the tensor inside the owner
+};
+repack_target repack_of(const ggml_tensor * t) {
+    repack_target r;
+    const ggml_tensor * owner = t->view_src ? t->view_src : t;
+    if (!is_repacked_type(owner->type) || owner->type != t->type || !ggml_is_contiguous(owner) || owner->data == nullptr) return r;
+    r.yes = true;
+    r.base = owner->data;
+    r.k = owner->ne[0];
+    r.nrows = tensor_nrows(owner);
+    r.off = (size_t) ((const char *) t->data - (const char *) owner->data);
+    return r;
+}
+
 // Copies through the null stream are ordered against every backend stream of the device (those are created blocking), in both
 // directions, so plain uploads and read-backs need no device-wide synchronization of their own; the paths that reuse the shared
 // staging buffer or free memory keep it.
@@ -365,12 +413,12 @@ void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const
         planes().drop(tensor->data, ggml_nbytes(tensor));   // rebuilt from the new contents on next use
         tiles().drop(tensor->data, ggml_nbytes(tensor));
     }
-    if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+    if (const repack_target rt = repack_of(tensor); rt.yes) {
         MI355_HIP_OK(hipDeviceSynchronize());
         std::lock_guard<std::mutex> lock(stage().mu);
         void * tmp = stage().get(size);
         MI355_HIP_OK(hipMemcpy(tmp, data, size, hipMemcpyHostToDevice));
-        MI355_K_OK(mi355_weights_scatter(nullptr, to_mi355_type(tensor->type), tmp, tensor->data, tensor->ne[0], tensor_nrows(tensor), offset, size));
+        MI355_K_OK(mi355_weights_scatter(nullptr, to_mi355_type(tensor->type), tmp, rt.base, rt.k, rt.nrows, rt.off + offset, size));
         MI355_HIP_OK(hipDeviceSynchronize());
     } else {
         MI355_HIP_OK(hipMemcpy((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice));
@@ -381,11 +429,11 @@ void buffer_get_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * tensor,
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     if (size == 0) return;
-    if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+    if (const repack_target rt = repack_of(tensor); rt.yes) {
         MI355_HIP_OK(hipDeviceSynchronize());
         std::lock_guard<std::mutex> lock(stage().mu);
         void * tmp = stage().get(size);
-        MI355_K_OK(mi355_weights_gather(nullptr, to_mi355_type(tensor->type), tensor->data, tmp, tensor->ne[0], tensor_nrows(tensor), offset, size));
+        MI355_K_OK(mi355_weights_gather(nullptr, to_mi355_type(tensor->type), rt.base, tmp, rt.k, rt.nrows, rt.off + offset, size));
         MI355_HIP_OK(hipMemcpy(data, tmp, size, hipMemcpyDeviceToHost));
     } else {
         MI355_HIP_OK(hipMemcpy(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost));
@@ -394,7 +442,7 @@ void buffer_get_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * tensor,
 
 void buffer_memset_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, uint8_t value, size_t offset, size_t size) {
     if (size == 0) return;
-    if (is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) {
+    if (repack_of(tensor).yes) {
         std::vector<uint8_t> host(size, value);   // rare path: route through the layout permutation
         buffer_set_tensor(buffer, tensor, host.data(), offset, size);
         return;
@@ -409,6 +457,8 @@ void buffer_memset_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, ui
 bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, ggml_tensor * dst) {
     // same buffer type on both sides: identical layouts (device layout included), plain device copy
     if (src->buffer == nullptr || src->buffer->buft != buffer->buft) return false;
+    // views of tensors in the device row layout may belong to owners with different rows: leave those to get + set
+    if (is_repacked_type(src->type) && (src->view_src || dst->view_src)) return false;
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
@@ -561,12 +611,17 @@ bool supports_flash_attn(const ggml_tensor * op) {
     const ggml_tensor * k = op->src[1];
     const ggml_tensor * v = op->src[2];
     const ggml_tensor * mask = op->src[3];
-    if (q->type != GGML_TYPE_F32 || k->type != GGML_TYPE_F16 || v->type != GGML_TYPE_F16) return false;
-    if (q->nb[0] != 4 || k->nb[0] != 2 || v->nb[0] != 2) return false;
+    if (q->type != GGML_TYPE_F32 || q->nb[0] != 4) return false;
     const int64_t D = q->ne[0];
     if (!(D == 64 || D == 80 || D == 96 || D == 112 || D == 128 || D == 256) || k->ne[0] != D || v->ne[0] != D) return false;
-    if (!strides_mult16(q) || !strides_mult16(k) || !strides_mult16(v)) return false;
-    if (!base_aligned16(q) || !base_aligned16(k) || !base_aligned16(v)) return false;
+    if (!strides_mult16(q) || !base_aligned16(q)) return false;
+    for (const ggml_tensor * t : {k, v}) {
+        if (t->type == GGML_TYPE_F16) {
+            if (t->nb[0] != 2 || !strides_mult16(t) || !base_aligned16(t)) return false;
+        } else if (!kv_operand_of(t).ok || D % 32 != 0 || q->ne[3] != 1) {   // Q8_0 / Q4_0 cache rows
+            return false;
+        }
+    }
     if (q->ne[2] % k->ne[2] != 0 || k->ne[2] != v->ne[2] || k->ne[1] != v->ne[1]) return false;
     if (q->ne[3] != k->ne[3] || q->ne[3] != v->ne[3]) return false;
     if (mask && (mask->type != GGML_TYPE_F16 || !ggml_is_contiguous(mask) || mask->ne[0] != k->ne[1])) return false;
@@ -614,6 +669,12 @@ bool device_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
             const ggml_type st = op->src[0]->type;
             const ggml_type dt = op->op == GGML_OP_CPY ? op->src[1]->type : op->type;
             const bool sf = st == GGML_TYPE_F32 || st == GGML_TYPE_F16, df = dt == GGML_TYPE_F32 || dt == GGML_TYPE_F16;
+            if (op->op == GGML_OP_CPY && st == GGML_TYPE_F32 && (dt == GGML_TYPE_Q8_0 || dt == GGML_TYPE_Q4_0)) {
+                // the store into a quantized KV cache: contiguous f32 rows into consecutive blocks
+                const ggml_tensor * a = op->src[0], * d = op->src[1];
+                return ggml_is_contiguous(a) && ggml_is_contiguous(d) && a->ne[0] % 32 == 0 && ggml_nelements(a) == ggml_nelements(d) &&
+                       kv_operand_of(d).ok && base_aligned16(a);
+            }
             return (sf && df) || (st == GGML_TYPE_I32 && dt == GGML_TYPE_I32);
         }
         case GGML_OP_GET_ROWS: {
@@ -693,6 +754,17 @@ void compute_flash_attn(backend_ctx * ctx, ggml_tensor * dst) {
     memcpy(&max_bias, (const float *) dst->op_params + 1, sizeof(float));
     memcpy(&softcap, (const float *) dst->op_params + 2, sizeof(float));
     const int64_t D = q->ne[0], Nq = q->ne[1], Hq = q->ne[2], Nkv = k->ne[1], Hkv = k->ne[2];
+    if (k->type != GGML_TYPE_F16 || v->type != GGML_TYPE_F16) {   // quantized cache (one batch: supports_op)
+        const kv_operand ko = kv_operand_of(k), vo = kv_operand_of(v);
+        GGML_ASSERT(ko.ok && vo.ok);
+        const size_t ws_bytes = mi355_flash_attn_kv_ws_bytes(D, Nq, Nkv, Hq, Hkv, to_mi355_type(k->type), to_mi355_type(v->type));
+        void * ws = ctx->workspace(ws_bytes);
+        MI355_K_OK(mi355_flash_attn_ext_kv(ctx->stream, (const float *) q->data, ko.p, to_mi355_type(k->type), ko.base, ko.row_blocks, vo.p,
+                                           to_mi355_type(v->type), vo.base, vo.row_blocks, mask ? mask->data : nullptr, (float *) dst->data, D, Nq, Nkv,
+                                           Hq, Hkv, q->nb[1], q->nb[2], k->nb[1], k->nb[2], v->nb[1], v->nb[2], mask ? mask->nb[1] : 0, scale, max_bias,
+                                           softcap, ws, ws_bytes, nullptr));
+        return;
+    }
     const size_t ws_bytes = mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq) < (size_t(256) << 20) ? mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq) : (size_t(256) << 20);
     void * ws = ctx->workspace(ws_bytes);
     for (int64_t i3 = 0; i3 < q->ne[3]; i3++) {
@@ -731,6 +803,15 @@ void compute_node(backend_ctx * ctx, ggml_tensor * node) {
             MI355_K_OK(mi355_scale(s, &a, &d, f));
         } break;
         case GGML_OP_CPY: {
+            const ggml_tensor * dt = node->src[1];
+            if (dt->type == GGML_TYPE_Q8_0 || dt->type == GGML_TYPE_Q4_0) {
+                const kv_operand o = kv_operand_of(dt);
+                GGML_ASSERT(o.ok);
+                const int64_t first = (int64_t) (((const char *) o.p - (const char *) o.base) / (ptrdiff_t) ggml_type_size(dt->type));
+                MI355_K_OK(mi355_cpy_f32_quant(s, to_mi355_type(dt->type), (const float *) node->src[0]->data, (void *) o.base, first, o.row_blocks,
+                                               ggml_nelements(dt)));
+                break;
+            }
             mi355_tensor a = desc(node->src[0]), d = desc(node->src[1]);
             MI355_K_OK(mi355_cpy(s, &a, &d));
         } break;
@@ -1433,7 +1514,8 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     if (node->op == GGML_OP_FLASH_ATTN_EXT) {
         const ggml_tensor * q = node->src[0];
         const int64_t D = q->ne[0], Nq = q->ne[1], Hq = q->ne[2];
-        if (q->ne[3] == 1 && Nq <= 8 && D % 32 == 0 && feeds_quant_gemv(w, i, node->data, Hq * D, Nq)) {
+        if (q->ne[3] == 1 && Nq <= 8 && D % 32 == 0 && node->src[1]->type == GGML_TYPE_F16 && node->src[2]->type == GGML_TYPE_F16 &&
+            feeds_quant_gemv(w, i, node->data, Hq * D, Nq)) {
             const ggml_tensor * k = node->src[1];
             const ggml_tensor * v = node->src[2];
             const ggml_tensor * mask = node->src[3];

@@ -1,0 +1,227 @@
+// Quantized KV cache: CPY f32 -> Q8_0 / Q4_0 (what llm_build_kv_store does with -ctk / -ctv q8_0, q4_0) and FLASH_ATTN_EXT over
+// such a cache.  The copies are quantize_row_q8_0_ref / quantize_row_q4_0_ref (ggml/src/ggml-quants.c:39-72, 194-218) bit for
+// bit.  Attention first expands the cells it will read into an f16 scratch image ([cell][kv head][D], d * level rounded to
+// f16) and then runs the f16 kernels on that image: every byte of a quantized cache is read once more than with an f16 cache,
+// which is the price of keeping one set of attention kernels.
+//
+// Where a block lives: a caller with a plain ggml cache passes row_blocks = 0 and blocks sit where ggml puts them (block g of the
+// tensor at g * block bytes).  A tensor kept in this library's device row layout (levels of a row first, its scales behind them,
+// mi355_weights_scatter) passes the blocks per row of the tensor that owns the memory: block g is then block g % row_blocks of
+// row g / row_blocks of that tensor, whatever view of it (1-D for the store, [D, cells, heads] for attention) is being used.
+#include "common.hpp"
+#include "fattn.hpp"
+
+namespace mi355 {
+
+
+struct kv_place {
+    int64_t first_block;   // block index, within the owning tensor, of the first block addressed
+    int64_t row_blocks;    // blocks per row of the owning tensor in the device row layout; 0 = plain ggml blocks
+};
+
+// byte offsets (from the owning tensor's data) of the levels and of the f16 scale of block g
+template <int TYPE>
+__device__ __forceinline__ void kv_block_offsets(const kv_place &p, int64_t g, int64_t &levels, int64_t &scale) {
+    constexpr int BB = TYPE == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES;   // block bytes
+    constexpr int LB = TYPE == MI355_Q8_0 ? 32 : 16;                   // bytes of levels per block
+    if (p.row_blocks == 0) {
+        scale = g * BB;
+        levels = scale + 2;
+    } else {
+        const int64_t row = g / p.row_blocks, b = g % p.row_blocks;
+        const int64_t base = row * p.row_blocks * BB;
+        levels = base + b * LB;
+        scale = base + p.row_blocks * LB + b * 2;
+    }
+}
+
+// Eight lanes share one 32-element block (4 consecutive elements each); n is a multiple of 32.
+__global__ void __launch_bounds__(256) k_cpy_f32_q8_0(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, kv_place pl) {
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const bool live = e0 < n;   // a block is all live or all dead
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) v = *(const f32x4 *)(x + e0);
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    if (!live) return;
+    int64_t lv, sc;
+    kv_block_offsets<MI355_Q8_0>(pl, pl.first_block + (e0 >> 5), lv, sc);
+    const int sub = (int)((e0 >> 2) & 7);
+    int q[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) q[i] = (int)roundf(v[i] * id);
+    // plain 34-byte blocks are 2-byte aligned only
+    unsigned short *o = (unsigned short *)(y + lv + 4 * sub);
+    o[0] = (unsigned short)((q[0] & 0xFF) | ((q[1] & 0xFF) << 8));
+    o[1] = (unsigned short)((q[2] & 0xFF) | ((q[3] & 0xFF) << 8));
+    if (sub == 0) *(unsigned short *)(y + sc) = float_to_half_bits(d);
+}
+
+__global__ void __launch_bounds__(256) k_cpy_f32_q4_0(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, kv_place pl) {
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const bool live = e0 < n;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) v = *(const f32x4 *)(x + e0);
+    // the value of largest magnitude, the first one among equals (the reference's loop keeps the earlier on a tie)
+    const int lane8 = threadIdx.x & 7;
+    float amax = 0.0f, vmax = 0.0f;
+    int imax = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (amax < fabsf(v[i])) {
+            amax = fabsf(v[i]);
+            vmax = v[i];
+            imax = lane8 * 4 + i;
+        }
+    }
+    if (amax == 0.0f) imax = 32;   // "no element yet": loses every tie
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) {
+        const float oa = __shfl_xor(amax, off, 64), ov = __shfl_xor(vmax, off, 64);
+        const int oi = __shfl_xor(imax, off, 64);
+        if (oa > amax || (oa == amax && oi < imax)) {
+            amax = oa;
+            vmax = ov;
+            imax = oi;
+        }
+    }
+    const float d = vmax / -8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    unsigned packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int8_t qi = (int8_t)(v[i] * id + 8.5f);
+        const unsigned u = (unsigned)(qi < 15 ? qi : 15) & 0xFu;
+        packed |= u << (8 * i);
+    }
+    // byte j of the block pairs element j (low nibble) with element j + 16 (high nibble): lanes 0..3 take lanes 4..7's levels
+    const unsigned hi = (unsigned)__shfl_down((int)packed, 4, 8);
+    if (!live || lane8 >= 4) return;
+    int64_t lv, sc;
+    kv_block_offsets<MI355_Q4_0>(pl, pl.first_block + (e0 >> 5), lv, sc);
+    const unsigned bytes = packed | (hi << 4);
+    unsigned short *o = (unsigned short *)(y + lv + 4 * lane8);
+    o[0] = (unsigned short)(bytes & 0xFFFFu);
+    o[1] = (unsigned short)(bytes >> 16);
+    if (lane8 == 0) *(unsigned short *)(y + sc) = float_to_half_bits(d);
+}
+
+// dst f16 [cell][head][D] = dequantized rows of a typed cache whose (cell, head) row starts at block cell * cb + head * hb (+ the
+// view's first block); one lane per 4 elements
+template <int TYPE>
+__global__ void __launch_bounds__(256) k_kv_dequant_f16(const uint8_t *__restrict__ src, int64_t cb, int64_t hb, kv_place pl, _Float16 *__restrict__ dst,
+                                                        int D, int HK, int64_t n_quads) {
+    const int64_t qd = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (qd >= n_quads) return;
+    const int per_row = D >> 2;
+    const int64_t rowi = qd / per_row;
+    const int e0 = (int)(qd % per_row) * 4;
+    const int64_t cell = rowi / HK;
+    const int head = (int)(rowi % HK);
+    const int j = e0 & 31;
+    int64_t lv, sc;
+    kv_block_offsets<TYPE>(pl, pl.first_block + cell * cb + (int64_t)head * hb + (e0 >> 5), lv, sc);
+    const float d = half_bits_to_float(*(const unsigned short *)(src + sc));
+    float f[4];
+    if constexpr (TYPE == MI355_Q8_0) {
+        const unsigned short *p = (const unsigned short *)(src + lv + j);
+        const unsigned w = (unsigned)p[0] | ((unsigned)p[1] << 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = (float)(int8_t)((w >> (8 * i)) & 0xFF) * d;
+    } else {
+        const unsigned short *p = (const unsigned short *)(src + lv + (j & 15));
+        const unsigned w = ((unsigned)p[0] | ((unsigned)p[1] << 16)) >> (j >= 16 ? 4 : 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = (float)((int)((w >> (8 * i)) & 0xF) - 8) * d;
+    }
+    _Float16 *o = dst + rowi * D + e0;
+    const f16x2 lo = {(_Float16)f[0], (_Float16)f[1]}, hi = {(_Float16)f[2], (_Float16)f[3]};
+    *(f16x2 *)o = lo;
+    *(f16x2 *)(o + 2) = hi;
+}
+
+static bool kv_type_ok(int t) { return t == MI355_F16 || t == MI355_Q8_0 || t == MI355_Q4_0; }
+static size_t kv_image_bytes(int type, int64_t D, int64_t Nkv, int64_t Hkv) {
+    return type == MI355_F16 ? 0 : (((size_t)Nkv * (size_t)Hkv * (size_t)D * 2 + 255) & ~(size_t)255);
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+int mi355_cpy_f32_quant(void *stream, int type, const float *src, void *dst_base, int64_t dst_first_block, int64_t dst_row_blocks, int64_t n) {
+    MI355_REQUIRE(type == MI355_Q8_0 || type == MI355_Q4_0, "cpy_f32_quant: destination type %d is not Q8_0 or Q4_0", type);
+    MI355_REQUIRE(n >= 0 && n % 32 == 0 && n / 1024 < 0x7fffffff, "cpy_f32_quant: %lld elements are not whole blocks of 32", (long long)n);
+    MI355_REQUIRE(((uintptr_t)src & 15) == 0 && ((uintptr_t)dst_base & 1) == 0 && dst_first_block >= 0 && dst_row_blocks >= 0,
+                  "cpy_f32_quant: source must be 16-byte, destination 2-byte aligned");
+    if (n == 0) return MI355_OK;
+    const kv_place pl = {dst_first_block, dst_row_blocks};
+    const dim3 grid((unsigned)((n / 4 + 255) / 256));
+    if (type == MI355_Q8_0) MI355_LAUNCH(k_cpy_f32_q8_0, grid, dim3(256), 0, (hipStream_t)stream, src, (uint8_t *)dst_base, n, pl);
+    else MI355_LAUNCH(k_cpy_f32_q4_0, grid, dim3(256), 0, (hipStream_t)stream, src, (uint8_t *)dst_base, n, pl);
+    return launch_status("k_cpy_f32_quant");
+}
+
+size_t mi355_flash_attn_kv_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, int type_k, int type_v) {
+    size_t base = mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq);
+    if (base > ((size_t)256 << 20)) base = (size_t)256 << 20;   // the splits use what they are given
+    return ((base + 255) & ~(size_t)255) + kv_image_bytes(type_k, D, Nkv, Hkv) + kv_image_bytes(type_v, D, Nkv, Hkv);
+}
+
+// expands one quantized operand into its f16 image; `p` points at the first row in plain ggml addressing, `base` at the data of
+// the tensor that owns the memory
+static int kv_expand(hipStream_t s, int type, const void *p, const void *base, int64_t row_blocks, size_t nb1, size_t nb2, void *img, int64_t D,
+                     int64_t Nkv, int64_t Hkv) {
+    const int64_t bb = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES;
+    if (base == nullptr) base = p;
+    const int64_t off = (const char *)p - (const char *)base;
+    MI355_REQUIRE(((uintptr_t)base & 1) == 0 && off >= 0 && off % bb == 0 && nb1 % bb == 0 && nb2 % bb == 0 && row_blocks >= 0,
+                  "flash_attn_kv: quantized rows must start on block boundaries");
+    const int64_t n_quads = Nkv * Hkv * (D / 4);
+    MI355_REQUIRE(n_quads / 256 < 0x7fffffff, "flash_attn_kv: cache too large for one launch");
+    const dim3 grid((unsigned)((n_quads + 255) / 256));
+    const kv_place pl = {off / bb, row_blocks};
+    if (type == MI355_Q8_0) MI355_LAUNCH(k_kv_dequant_f16<MI355_Q8_0>, grid, dim3(256), 0, s, (const uint8_t *)base, (int64_t)nb1 / bb, (int64_t)nb2 / bb, pl, (_Float16 *)img, (int)D, (int)Hkv, n_quads);
+    else MI355_LAUNCH(k_kv_dequant_f16<MI355_Q4_0>, grid, dim3(256), 0, s, (const uint8_t *)base, (int64_t)nb1 / bb, (int64_t)nb2 / bb, pl, (_Float16 *)img, (int)D, (int)Hkv, n_quads);
+    return launch_status("k_kv_dequant_f16");
+}
+
+int mi355_flash_attn_ext_kv(void *stream, const float *q, const void *k, int type_k, const void *k_base, int64_t k_row_blocks, const void *v,
+                            int type_v, const void *v_base, int64_t v_row_blocks, const void *mask, float *dst, int64_t D, int64_t Nq, int64_t Nkv,
+                            int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2,
+                            size_t mask_nb1, float scale, float max_bias, float logit_softcap, void *ws, size_t ws_bytes, void *act) {
+    MI355_REQUIRE(kv_type_ok(type_k) && kv_type_ok(type_v), "flash_attn_kv: cache types %d / %d (f16, Q8_0 and Q4_0 are served)", type_k, type_v);
+    if (type_k == MI355_F16 && type_v == MI355_F16)
+        return mi355_flash_attn_ext_quant(stream, q, k, v, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1, scale,
+                                          max_bias, logit_softcap, ws, ws_bytes, act);
+    MI355_REQUIRE(D > 0 && D % 32 == 0 && Nkv > 0 && Hkv > 0, "flash_attn_kv: head size %lld is not a whole number of blocks", (long long)D);
+    const size_t kb = kv_image_bytes(type_k, D, Nkv, Hkv), vb = kv_image_bytes(type_v, D, Nkv, Hkv);
+    MI355_REQUIRE(ws != nullptr && ((uintptr_t)ws & 255) == 0 && ws_bytes >= kb + vb, "flash_attn_kv: the workspace must be 256-byte aligned and hold the f16 images (%zu bytes)", kb + vb);
+    // the images sit at the end of the workspace; what is in front of them serves the kv splits as before
+    const size_t front = (ws_bytes - kb - vb) & ~(size_t)255;
+    uint8_t *kimg = (uint8_t *)ws + front, *vimg = kimg + kb;
+    hipStream_t s = (hipStream_t)stream;
+    if (type_k != MI355_F16) {
+        int rc = kv_expand(s, type_k, k, k_base, k_row_blocks, k_nb1, k_nb2, kimg, D, Nkv, Hkv);
+        if (rc != MI355_OK) return rc;
+        k = kimg;
+        k_nb1 = (size_t)Hkv * D * 2;
+        k_nb2 = (size_t)D * 2;
+    }
+    if (type_v != MI355_F16) {
+        int rc = kv_expand(s, type_v, v, v_base, v_row_blocks, v_nb1, v_nb2, vimg, D, Nkv, Hkv);
+        if (rc != MI355_OK) return rc;
+        v = vimg;
+        v_nb1 = (size_t)Hkv * D * 2;
+        v_nb2 = (size_t)D * 2;
+    }
+    return mi355_flash_attn_ext_quant(stream, q, k, v, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1, scale,
+                                      max_bias, logit_softcap, front ? ws : nullptr, front, act);
+}
+
+}  // extern "C"

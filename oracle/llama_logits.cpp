@@ -3,7 +3,9 @@
 // reference CPU backend with the plug-in, and the plug-in's fused graph execution with its node-by-node execution,
 // on the same synthetic model and token ids.
 //
-//   llama_logits <model.gguf> <n_gpu_layers> <n_prompt> <n_decode> <out.bin>
+//   llama_logits <model.gguf> <n_gpu_layers> <n_prompt> <n_decode> <out.bin> [<type_k> <type_v>]
+//
+// type_k / type_v: f16 (default), q8_0 or q4_0 - the KV cache types of llama.cpp's -ctk / -ctv.
 //
 // Tokens are (7 i + 3) mod n_vocab.  Output: float32 rows of n_vocab logits, one for the last prompt token and one per
 // decoded token (the token ids are fixed, the logits are not fed back).
@@ -12,13 +14,18 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <string>
 #include <vector>
 
 int main(int argc, char ** argv) {
-    if (argc != 6) {
-        fprintf(stderr, "usage: %s model.gguf n_gpu_layers n_prompt n_decode out.bin\n", argv[0]);
+    if (argc != 6 && argc != 8) {
+        fprintf(stderr, "usage: %s model.gguf n_gpu_layers n_prompt n_decode out.bin [type_k type_v]\n", argv[0]);
         return 2;
     }
+    auto cache_type = [](const char * name) {
+        const std::string s = name;
+        return s == "q8_0" ? GGML_TYPE_Q8_0 : s == "q4_0" ? GGML_TYPE_Q4_0 : GGML_TYPE_F16;
+    };
     const int ngl = atoi(argv[2]), n_prompt = atoi(argv[3]), n_decode = atoi(argv[4]);
     ggml_backend_load_all();   // honours GGML_BACKEND_PATH, like the reference's example programs
     llama_backend_init();
@@ -31,6 +38,10 @@ int main(int argc, char ** argv) {
     cp.n_batch = 512;
     cp.n_ubatch = 512;
     cp.flash_attn = true;
+    if (argc == 8) {
+        cp.type_k = cache_type(argv[6]);
+        cp.type_v = cache_type(argv[7]);
+    }
     cp.n_threads = 8;
     cp.n_threads_batch = 8;
     llama_context * ctx = llama_init_from_model(model, cp);

@@ -811,6 +811,93 @@ void orc_flash_attn_cpu(const float *q, const uint16_t *k, const uint16_t *v, co
     free(q16);
 }
 
+/* The same kernel with a quantized KV cache (type_k, type_v each ORC_F16, ORC_Q8_0 or ORC_Q4_0; k, v are [Hkv][Nkv] rows of
+ * D elements in the type's block layout).  ggml-cpu.c:10997-11003: q is converted to K's vec_dot_type - f16 for f16 K, Q8_0
+ * blocks for Q8_0 and Q4_0 K - and the score is the type's vec_dot (ggml-cpu-quants.c:2492-2506 q4_0 x q8_0, :3919-3927
+ * q8_0 x q8_0: per block the integer dot times both scales, summed in float).  :11040-11099: a V of another type than f16 is
+ * dequantized row by row (to_float) into f32 and accumulated with ggml_vec_mad_f32 in an f32 accumulator. */
+int orc_flash_attn_kv_cpu(const float *q, const void *k, int type_k, const void *v, int type_v, const uint16_t *mask, float *dst,
+                          int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, float scale, float max_bias, float softcap) {
+    if ((type_k != ORC_F16 && type_k != ORC_Q8_0 && type_k != ORC_Q4_0) || (type_v != ORC_F16 && type_v != ORC_Q8_0 && type_v != ORC_Q4_0)) return -1;
+    if (D % QK) return -1;
+    if (softcap != 0) scale /= softcap;
+    const size_t krb = type_k == ORC_F16 ? (size_t)D * 2 : orc_row_bytes(type_k, D);
+    const size_t vrb = type_v == ORC_F16 ? (size_t)D * 2 : orc_row_bytes(type_v, D);
+    uint16_t *acc16 = (uint16_t *)malloc((size_t)D * 2);
+    float *acc32 = (float *)malloc((size_t)D * 4);
+    float *v32 = (float *)malloc((size_t)D * 4);
+    float *q16 = (float *)malloc((size_t)D * 4);
+    blk_q8_0 *qq = (blk_q8_0 *)malloc((size_t)(D / QK) * sizeof(blk_q8_0));
+    const int64_t rep = Hq / Hkv;
+    for (int64_t h = 0; h < Hq; h++) {
+        const float slope = alibi_slope(max_bias, (uint32_t)h, (uint32_t)Hq);
+        const int64_t hk = h / rep;
+        for (int64_t i = 0; i < Nq; i++) {
+            const float *qr = q + (h * Nq + i) * D;
+            if (type_k == ORC_F16) for (int64_t d = 0; d < D; d++) q16[d] = orc_f16_to_f32(orc_f32_to_f16(qr[d]));
+            else quantize_row(ORC_Q8_0, qr, qq, D);
+            memset(acc16, 0, (size_t)D * 2);
+            memset(acc32, 0, (size_t)D * 4);
+            float S = 0.0f, M = -INFINITY;
+            for (int64_t c = 0; c < Nkv; c++) {
+                const float mv = mask ? slope * orc_f16_to_f32(mask[i * Nkv + c]) : 0.0f;
+                if (mv == -INFINITY) continue;
+                const char *kr = (const char *)k + (size_t)(hk * Nkv + c) * krb;
+                double dotacc = 0;    /* the reference sums per-block products in float SIMD lanes; order-free stand-in */
+                if (type_k == ORC_F16) {
+                    const uint16_t *kh = (const uint16_t *)kr;
+                    for (int64_t d = 0; d < D; d++) dotacc += (double)orc_f16_to_f32(kh[d]) * (double)q16[d];
+                } else {
+                    for (int64_t b = 0; b < D / QK; b++) {
+                        int sumi = 0;
+                        float dk;
+                        if (type_k == ORC_Q8_0) {
+                            const blk_q8_0 *kb = (const blk_q8_0 *)kr + b;
+                            for (int j = 0; j < QK; j++) sumi += (int)kb->qs[j] * (int)qq[b].qs[j];
+                            dk = orc_f16_to_f32(kb->d);
+                        } else {
+                            const blk_q4_0 *kb = (const blk_q4_0 *)kr + b;
+                            for (int j = 0; j < QK / 2; j++) {
+                                sumi += ((int)(kb->qs[j] & 0x0F) - 8) * (int)qq[b].qs[j];
+                                sumi += ((int)(kb->qs[j] >> 4) - 8) * (int)qq[b].qs[j + QK / 2];
+                            }
+                            dk = orc_f16_to_f32(kb->d);
+                        }
+                        dotacc += (double)((float)sumi * (dk * orc_f16_to_f32(qq[b].d)));
+                    }
+                }
+                float s = (float)dotacc * scale;
+                if (softcap != 0.0f) s = softcap * tanhf(s);
+                s += mv;
+                const float Mold = M;
+                float ms = 1.0f, vs = 1.0f;
+                const char *vr = (const char *)v + (size_t)(hk * Nkv + c) * vrb;
+                if (s > M) {
+                    M = s;
+                    ms = expf(Mold - M);
+                    if (type_v == ORC_F16) for (int64_t d = 0; d < D; d++) acc16[d] = orc_f32_to_f16(orc_f16_to_f32(acc16[d]) * ms);
+                    else for (int64_t d = 0; d < D; d++) acc32[d] *= ms;
+                } else {
+                    vs = expf(s - M);
+                }
+                if (type_v == ORC_F16) {
+                    const uint16_t *vh = (const uint16_t *)vr;
+                    for (int64_t d = 0; d < D; d++) acc16[d] = orc_f32_to_f16(orc_f16_to_f32(acc16[d]) + orc_f16_to_f32(vh[d]) * vs);
+                } else {
+                    dequantize_row(type_v, vr, v32, D);
+                    for (int64_t d = 0; d < D; d++) acc32[d] = fmaf(v32[d], vs, acc32[d]);
+                }
+                S = S * ms + vs;
+            }
+            const float S_inv = 1.0f / S;
+            float *o = dst + (i * Hq + h) * D;
+            for (int64_t d = 0; d < D; d++) o[d] = (type_v == ORC_F16 ? orc_f16_to_f32(acc16[d]) : acc32[d]) * S_inv;
+        }
+    }
+    free(acc16); free(acc32); free(v32); free(q16); free(qq);
+    return 0;
+}
+
 void orc_flash_attn_f64(const float *q, const uint16_t *k, const uint16_t *v, const uint16_t *mask, float *dst,
                         int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, float scale, float max_bias,
                         float softcap) {

@@ -72,6 +72,11 @@ int orc_mul_mat_id_q8_1(int type, const void *as, const float *b, const int32_t 
 void orc_flash_attn_cpu(const float *q, const uint16_t *k, const uint16_t *v, const uint16_t *mask,
                         float *dst, int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv,
                         float scale, float max_bias, float softcap);
+/* _kv_cpu : the same kernel over a typed KV cache (ORC_F16, ORC_Q8_0, ORC_Q4_0 for K and V independently); k, v hold
+ *  [Hkv][Nkv] rows of D elements in the type's block layout.  Returns 0, or -1 for an unsupported type / D. */
+int orc_flash_attn_kv_cpu(const float *q, const void *k, int type_k, const void *v, int type_v, const uint16_t *mask,
+                          float *dst, int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv,
+                          float scale, float max_bias, float softcap);
 void orc_flash_attn_f64(const float *q, const uint16_t *k, const uint16_t *v, const uint16_t *mask,
                         float *dst, int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv,
                         float scale, float max_bias, float softcap);

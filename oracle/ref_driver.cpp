@@ -152,6 +152,41 @@ double ref_flash_attn(const float * q, const uint16_t * k, const uint16_t * v, c
     return t;
 }
 
+// FLASH_ATTN_EXT over a typed KV cache: k, v are [D, Nkv, Hkv] tensors of type_k / type_v (f16 or a quantized type).
+double ref_flash_attn_kv(const float * q, const void * k, int type_k, const void * v, int type_v, const uint16_t * mask, float * dst,
+                         int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, int64_t Nq_pad, float scale,
+                         float max_bias, float softcap, int n_threads, int reps) {
+    cpu_graph g(n_threads);
+    ggml_tensor * tq = ggml_new_tensor_3d(g.ctx, GGML_TYPE_F32, D, Nq, Hq);
+    ggml_tensor * tk = ggml_new_tensor_3d(g.ctx, (ggml_type) type_k, D, Nkv, Hkv);
+    ggml_tensor * tv = ggml_new_tensor_3d(g.ctx, (ggml_type) type_v, D, Nkv, Hkv);
+    ggml_tensor * tm = mask ? ggml_new_tensor_2d(g.ctx, GGML_TYPE_F16, Nkv, Nq_pad) : nullptr;
+    ggml_tensor * out = ggml_flash_attn_ext(g.ctx, tq, tk, tv, tm, scale, max_bias, softcap);
+    ggml_flash_attn_ext_set_prec(out, GGML_PREC_F32);
+    if (!g.alloc()) return -1.0;
+    ggml_backend_tensor_set(tq, q, 0, ggml_nbytes(tq));
+    ggml_backend_tensor_set(tk, k, 0, ggml_nbytes(tk));
+    ggml_backend_tensor_set(tv, v, 0, ggml_nbytes(tv));
+    if (tm) ggml_backend_tensor_set(tm, mask, 0, ggml_nbytes(tm));
+    double t = g.run(out, reps);
+    ggml_backend_tensor_get(out, dst, 0, ggml_nbytes(out));
+    return t;
+}
+
+// CPY of contiguous f32 rows of k elements into a tensor of `type` (what llm_build_kv_store does with a quantized cache):
+// the CPU backend's own conversion (its from_float, which may round differently from quantize_row_*_ref on SIMD builds).
+int ref_cpy_f32_to(int type, const float * x, void * y, int64_t k, int64_t nrows, int n_threads) {
+    cpu_graph g(n_threads);
+    ggml_tensor * a = ggml_new_tensor_2d(g.ctx, GGML_TYPE_F32, k, nrows);
+    ggml_tensor * b = ggml_new_tensor_2d(g.ctx, (ggml_type) type, k, nrows);
+    ggml_tensor * out = ggml_cpy(g.ctx, a, b);
+    if (!g.alloc()) return -1;
+    ggml_backend_tensor_set(a, x, 0, ggml_nbytes(a));
+    g.run(out, 0);
+    ggml_backend_tensor_get(b, y, 0, ggml_nbytes(b));
+    return 0;
+}
+
 int ref_rms_norm(const float * x, float * y, int64_t ncols, int64_t nrows, float eps, int n_threads) {
     cpu_graph g(n_threads);
     ggml_tensor * a = ggml_new_tensor_2d(g.ctx, GGML_TYPE_F32, ncols, nrows);

@@ -8,6 +8,7 @@ the reference's outputs for them, so the oracle can be pinned where the referenc
   mul_mat_<type>.npz : W bytes [48,512], x f32 [3,512], y = reference CPU MUL_MAT output
   flash_attn.npz     : q,k,v,mask for D=64, Nq=3, Nkv=40, Hq=4, Hkv=2 and the reference CPU output
   flash_attn_alibi_softcap.npz : 6 query heads over 3 kv heads, the reference CPU outputs with max_bias = 8 and with logit_softcap = 10
+  flash_attn_kv_types.npz : D=64, 4 query heads over 2 kv heads; reference CPU outputs for K and V each of f16, Q8_0, Q4_0
   glue.npz           : inputs/outputs of RMS_NORM, SOFT_MAX, ROPE (modes 0 and 2), SILU, ARGSORT
 """
 import os
@@ -68,6 +69,19 @@ def main():
     np.savez_compressed(os.path.join(HERE, "flash_attn_alibi_softcap.npz"), q=q2, k=k2.view(np.uint16), v=v2.view(np.uint16),
                         mask=mask.view(np.uint16), y_alibi=y_alibi, y_softcap=y_cap, scale=np.float32(0.125), max_bias=np.float32(8.0),
                         softcap=np.float32(10.0))
+
+    # a quantized KV cache: every pairing of f16, Q8_0 and Q4_0 for K and V (q is quantized to Q8_0 for a quantized K, V rows are
+    # dequantized into an f32 accumulator)
+    rng3 = np.random.default_rng(20240609)
+    D3, Nq3, Nkv3, Hq3, Hkv3 = 64, 3, 40, 4, 2
+    q3 = rng3.standard_normal((Hq3, Nq3, D3)).astype(np.float32)
+    kf3 = rng3.standard_normal((Hkv3, Nkv3, D3)).astype(np.float32)
+    vf3 = rng3.standard_normal((Hkv3, Nkv3, D3)).astype(np.float32)
+    out3 = {"q": q3, "kf": kf3, "vf": vf3, "mask": mask.view(np.uint16), "scale": np.float32(0.125)}
+    for tk in (orc.F16, orc.Q8_0, orc.Q4_0):
+        for tv in (orc.F16, orc.Q8_0, orc.Q4_0):
+            out3["y_%d_%d" % (tk, tv)] = orc.flash_attn_kv("ref", q3, orc.kv_rows(tk, kf3), tk, orc.kv_rows(tv, vf3), tv, mask.view(np.uint16), 0.125)
+    np.savez_compressed(os.path.join(HERE, "flash_attn_kv_types.npz"), **out3)
 
     g = {}
     x = rng.standard_normal((5, 96)).astype(np.float32)

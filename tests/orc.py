@@ -62,6 +62,8 @@ if oracle is not None:
         getattr(oracle, name).restype = None
         getattr(oracle, name).argtypes = [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _f, _f, _f]
     oracle.orc_rms_norm.argtypes = [_p, _p, _i64, _i64, _f]
+    oracle.orc_flash_attn_kv_cpu.restype = _int
+    oracle.orc_flash_attn_kv_cpu.argtypes = [_p, _p, _int, _p, _int, _p, _p, _i64, _i64, _i64, _i64, _i64, _f, _f, _f]
     oracle.orc_silu.argtypes = [_p, _p, _i64]
     oracle.orc_soft_max.argtypes = [_p, _p, _p, _i64, _i64, _f]
     oracle.orc_rope.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _f, _f, _f, _f, _f, _f, _int]
@@ -85,6 +87,11 @@ if ref is not None:
     ref.ref_mul_mat.argtypes = [_int, _p, _p, _p, _i64, _i64, _i64, _int, _int]
     ref.ref_mul_mat_id.restype = C.c_double
     ref.ref_mul_mat_id.argtypes = [_int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int]
+    if hasattr(ref, "ref_flash_attn_kv"):
+        ref.ref_flash_attn_kv.restype = C.c_double
+        ref.ref_flash_attn_kv.argtypes = [_p, _p, _int, _p, _int, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f, _f, _f, _int, _int]
+        ref.ref_cpy_f32_to.restype = _int
+        ref.ref_cpy_f32_to.argtypes = [_int, _p, _p, _i64, _i64, _int]
     ref.ref_flash_attn.restype = C.c_double
     ref.ref_flash_attn.argtypes = [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f, _f, _f, _int, _int]
     ref.ref_rms_norm.argtypes = [_p, _p, _i64, _i64, _f, _int]
@@ -170,6 +177,38 @@ def flash_attn(kind, q, k, v, mask, scale, max_bias=0.0, softcap=0.0, n_threads=
     else:
         getattr(oracle, "orc_flash_attn_" + kind)(_ptr(q), _ptr(k), _ptr(v), _ptr(mask), _ptr(out), D, Nq, Nkv, Hq,
                                                    Hkv, scale, max_bias, softcap)
+    return out
+
+
+F16 = 1
+
+
+def kv_rows(t, x):
+    """f32 [Hkv, Nkv, D] -> the cache bytes of type t (f16 bits as uint8, or quantized blocks by the reference-pinned quantizer)"""
+    x = f32(x)
+    if t == F16:
+        return np.ascontiguousarray(x.astype(np.float16)).view(np.uint8).reshape(x.shape[0], x.shape[1], -1)
+    H, N, D = x.shape
+    return quantize("oracle", t, x.reshape(H * N, D)).reshape(H, N, -1)
+
+
+def flash_attn_kv(kind, q, k, type_k, v, type_v, mask, scale, max_bias=0.0, softcap=0.0, n_threads=4):
+    """q f32 [Hq,Nq,D]; k, v uint8 [Hkv,Nkv,row bytes] of type_k / type_v (see kv_rows); mask uint16 or None -> f32 [Nq,Hq,D]"""
+    Hq, Nq, D = q.shape
+    Hkv, Nkv = k.shape[0], k.shape[1]
+    q = f32(q)
+    k = np.ascontiguousarray(k, dtype=np.uint8)
+    v = np.ascontiguousarray(v, dtype=np.uint8)
+    out = np.zeros((Nq, Hq, D), dtype=np.float32)
+    if mask is not None:
+        mask = np.ascontiguousarray(mask, dtype=np.uint16)
+    if kind == "ref":
+        nq_pad = mask.shape[0] if mask is not None else Nq
+        assert ref.ref_flash_attn_kv(_ptr(q), _ptr(k), type_k, _ptr(v), type_v, _ptr(mask), _ptr(out), D, Nq, Nkv, Hq, Hkv, nq_pad, scale,
+                                     max_bias, softcap, n_threads, 0) >= 0
+    else:
+        assert oracle.orc_flash_attn_kv_cpu(_ptr(q), _ptr(k), type_k, _ptr(v), type_v, _ptr(mask), _ptr(out), D, Nq, Nkv, Hq, Hkv, scale,
+                                            max_bias, softcap) == 0
     return out
 
 

@@ -53,15 +53,15 @@ def test_llama_bench_runs_on_the_plugin(dev, tmp_path):
 LOGITS = os.path.join(ROOT, "oracle", "_ref", "llama_logits")
 
 
-def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None):
+def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None, cache=None):
     import numpy as np
     env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN, MI355_GRAPH_STATS="1")
     if not fusion:
         env["MI355_NO_FUSION"] = "1"
     if not graphs:
         env["MI355_NO_GRAPH"] = "1"
-    r = subprocess.run([LOGITS, model, str(ngl), str(n_prompt), str(n_decode), out], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
-                       text=True, timeout=600, cwd=os.path.dirname(LOGITS))
+    r = subprocess.run([LOGITS, model, str(ngl), str(n_prompt), str(n_decode), out] + (list(cache) if cache else []), env=env, stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True, timeout=600, cwd=os.path.dirname(LOGITS))
     assert r.returncode == 0, r.stdout[-3000:]
     if ngl > 0:
         assert "MI355X" in r.stdout, "layers were not offloaded to the plug-in:\n" + r.stdout[-3000:]
@@ -92,6 +92,28 @@ def test_model_logits_cpu_vs_plugin_and_fused_vs_nodes(dev, tmp_path, n_prompt):
     assert orc.nmse(fused, nodes) < (1e-6 if n_prompt <= 8 else 5e-4)
     assert orc.nmse(nodes, cpu) < 2e-3
     assert orc.nmse(fused, cpu) < 2e-3
+
+
+@pytest.mark.parametrize("cache", [("q8_0", "q8_0"), ("q4_0", "q4_0"), ("q8_0", "f16")])
+@pytest.mark.parametrize("n_prompt", [5, 200])
+def test_model_logits_quantized_kv_cache(dev, tmp_path, cache, n_prompt):
+    """llama.cpp's -ctk / -ctv: the cache tensors are Q8_0 / Q4_0, the stores are CPY f32 -> quantized and FLASH_ATTN_EXT reads quantized
+    K / V.  The reference's runtime on the plug-in reproduces its CPU backend's logits with the same cache types, prefill and decode."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / "small.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048)
+    cpu = _logits(model, 0, n_prompt, 6, str(tmp_path / "cpu.bin"), cache=cache)
+    gpu = _logits(model, 99, n_prompt, 6, str(tmp_path / "gpu.bin"), cache=cache)
+    assert cpu.shape == gpu.shape and np.isfinite(gpu).all()
+    # A 4-bit cache has 16 levels per block: where the two backends' K / V rows differ in the last bits (summation order of the
+    # projections), a value on a rounding boundary lands on another level and moves by 1/8 of the block's range.  A short prompt
+    # has few cells to average that over.  The op-level parity of the stores and of attention is in tests/test_gpu_kv_quant.py.
+    assert orc.nmse(gpu, cpu) < (2e-2 if "q4_0" in cache else 2e-3)
 
 
 @pytest.mark.parametrize("n_prompt", [3, 48])

@@ -239,6 +239,39 @@ def test_flash_attn_alibi_and_softcap_golden():
         assert orc.nmse(f64, out) < 1e-10
 
 
+def test_flash_attn_quantized_kv_golden():
+    """the oracle over a Q8_0 / Q4_0 KV cache (q quantized to Q8_0 and integer block dots for a quantized K, f32 accumulator over
+    dequantized rows for a quantized V; ggml-cpu.c:10997-11003, 11040-11099) against committed outputs of the reference build, and
+    against the textbook form on the dequantized cache (which the q quantization leaves ~2e-5 away)"""
+    g = gold("flash_attn_kv_types.npz")
+    q, kf, vf, mask, scale = g["q"], g["kf"], g["vf"], g["mask"], float(g["scale"])
+    Hq, Nq, D = q.shape
+    Hkv, Nkv = kf.shape[0], kf.shape[1]
+    mf = mask.view(np.float16).astype(np.float64)
+    for tk in (orc.F16, orc.Q8_0, orc.Q4_0):
+        for tv in (orc.F16, orc.Q8_0, orc.Q4_0):
+            k, v = orc.kv_rows(tk, kf), orc.kv_rows(tv, vf)
+            got = orc.flash_attn_kv("cpu", q, k, tk, v, tv, mask, scale)
+            assert orc.nmse(got, g["y_%d_%d" % (tk, tv)]) < 1e-6, (tk, tv)
+
+            def deq(a, t):
+                if t == orc.F16:
+                    return a.view(np.float16).astype(np.float64).reshape(Hkv, Nkv, D)
+                return orc.dequantize("oracle", t, a.reshape(Hkv * Nkv, -1), D).reshape(Hkv, Nkv, D).astype(np.float64)
+            kd, vd = deq(k, tk), deq(v, tv)
+            out = np.zeros((Nq, Hq, D))
+            for h in range(Hq):
+                s = q[h].astype(np.float64) @ kd[h // 2].T * scale + mf[:Nq]
+                p = np.exp(s - s.max(axis=1, keepdims=True))
+                out[:, h] = (p / p.sum(axis=1, keepdims=True)) @ vd[h // 2]
+            assert orc.nmse(got, out) < 2e-4, (tk, tv)
+    # with f16 K and V it is the kernel of orc_flash_attn_cpu
+    k16, v16 = orc.kv_rows(orc.F16, kf), orc.kv_rows(orc.F16, vf)
+    a = orc.flash_attn_kv("cpu", q, k16, orc.F16, v16, orc.F16, mask, scale)
+    b = orc.flash_attn("cpu", q, k16.view(np.uint16).reshape(Hkv, Nkv, D), v16.view(np.uint16).reshape(Hkv, Nkv, D), mask, scale)
+    assert np.array_equal(a, b)
+
+
 # ------------------------------------------------------------------ glue ops
 def test_glue_golden():
     g = gold("glue.npz")
