@@ -280,7 +280,7 @@ def sweep(kinds):
                     del Ws
     if "fattn" in kinds or "fattn_long" in kinds:
         H, HK, D = 32, 8, 128
-        cases = [(1, 512), (1, 4096), (1, 32768), (1, 131072), (512, 512), (512, 4096), (2048, 2048), (4096, 4096)]
+        cases = [(1, 256), (1, 512), (1, 1024), (1, 4096), (1, 32768), (1, 131072), (512, 512), (512, 4096), (2048, 2048), (4096, 4096)]
         if "fattn" not in kinds:
             cases = [(1, 131072)]   # the long-context decode kernel alone (for counter collection)
         for Nq, Nkv in cases:

@@ -46,15 +46,17 @@ __device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
 __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e);
 
 
-template <int D, int R>
-__global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
+// NW: waves per group
+template <int D, int R, int NW = 4>
+__global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     constexpr int LPR = D <= 64 ? 8 : (D <= 128 ? 16 : 32);   // lanes per K/V row
     constexpr int CPW = 64 / LPR;                               // cells per wave step
-    constexpr int SLOTS = 4 * CPW;                              // independent softmax states per group
+    constexpr int SLOTS = NW * CPW;                             // independent softmax states per group
+    constexpr int NT = NW * 64;
     constexpr float NEG = -FLT_MAX / 2;
 
-    __shared__ float s_m[SLOTS][R], s_l[SLOTS][R];
-    __shared__ float s_o[SLOTS][R][D];
+    __shared__ float s_m[NW][R], s_l[NW][R];
+    __shared__ float s_o[NW][R][D];
 
     const int split = blockIdx.x;
     const int64_t hk = blockIdx.y / a.groups, hg = blockIdx.y % a.groups, iq = blockIdx.z;
@@ -131,60 +133,76 @@ __global__ void __launch_bounds__(256) k_fattn_vec(fattn_args a) {
                 vv[j] = load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2);
             }
         }
+        // V rows as floats, then per head: the U scores (independent of each other), ONE new maximum and ONE rescale of the state,
+        // and the U weighted rows - the dependent chain per step is a fraction of folding the cells one by one
+        float vf[U][8];
 #pragma unroll
-        for (int j = 0; j < U; j++) {
-            if (__ballot(valid[j]) == 0) continue;   // whole wave masked (wave-uniform)
-            float vf[8];
+        for (int j = 0; j < U; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const u32 vi = vv[j][i];
                 const f16x2 h2 = __builtin_bit_cast(f16x2, vi);
-                vf[2 * i] = (float)h2[0];
-                vf[2 * i + 1] = (float)h2[1];
+                vf[j][2 * i] = (float)h2[0];
+                vf[j][2 * i + 1] = (float)h2[1];
             }
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                float s = group_sum<LPR>(dot8_f16(qh[r], kk[j])) * scale;
-                if (a.softcap != 0.0f) s = a.softcap * tanhf(s);
-                s += slope[r] * mv[j];
-                if (valid[j]) {
-                    if (s > m[r]) {
-                        const float f = __expf(m[r] - s);
-                        l[r] *= f;
+        for (int r = 0; r < R; r++) {
+            float sj[U];
+            float mn = m[r];
 #pragma unroll
-                        for (int i = 0; i < 8; i++) acc[r][i] *= f;
-                        m[r] = s;
-                    }
-                    const float p = __expf(s - m[r]);
-                    l[r] += p;
+            for (int j = 0; j < U; j++) {
+                float sc = group_sum<LPR>(dot8_f16(qh[r], kk[j])) * scale;
+                if (a.softcap != 0.0f) sc = a.softcap * tanhf(sc);
+                sc += slope[r] * mv[j];
+                sj[j] = valid[j] ? sc : NEG;
+                mn = fmaxf(mn, sj[j]);
+            }
+            const float f = __expf(m[r] - mn);   // 1 when nothing changed (also while the state is still empty)
+            m[r] = mn;
+            l[r] *= f;
 #pragma unroll
-                    for (int i = 0; i < 8; i++) acc[r][i] += p * vf[i];
-                }
+            for (int i = 0; i < 8; i++) acc[r][i] *= f;
+#pragma unroll
+            for (int j = 0; j < U; j++) {
+                const float p = valid[j] ? __expf(sj[j] - mn) : 0.0f;
+                l[r] += p;
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[r][i] += p * vf[j][i];
             }
         }
     }
 
-    // merge the SLOTS states of this group
+    // merge the states: first the CPW lane groups of a wave (cross-lane), then the NW waves through LDS
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        if (sub == 0) {
-            s_m[slot][r] = m[r];
-            s_l[slot][r] = l[r];
-        }
-        if (active) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) s_o[slot][r][d0 + i] = acc[r][i];
+        for (int off = LPR; off < 64; off <<= 1) {
+            const float om = __shfl_xor(m[r], off, 64), ol = __shfl_xor(l[r], off, 64);
+            const float M = fmaxf(m[r], om);
+            const float fa = __expf(m[r] - M), fb = __expf(om - M);
+            l[r] = l[r] * fa + ol * fb;
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[r][i] = acc[r][i] * fa + __shfl_xor(acc[r][i], off, 64) * fb;
+            m[r] = M;
+        }
+        if (lane == 0) {
+            s_m[wave][r] = m[r];
+            s_l[wave][r] = l[r];
+        }
+        if (active && lane < LPR) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) s_o[wave][r][d0 + i] = acc[r][i];
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < R * D; idx += 256) {
+    for (int idx = threadIdx.x; idx < R * D; idx += NT) {
         const int r = idx / D, d = idx % D;
         float M = NEG;
 #pragma unroll
-        for (int s = 0; s < SLOTS; s++) M = fmaxf(M, s_m[s][r]);
+        for (int s = 0; s < NW; s++) M = fmaxf(M, s_m[s][r]);
         float L = 0.0f, O = 0.0f;
 #pragma unroll
-        for (int s = 0; s < SLOTS; s++) {
+        for (int s = 0; s < NW; s++) {
             const float f = __expf(s_m[s][r] - M);
             L += s_l[s][r] * f;
             O += s_o[s][r][d] * f;
@@ -284,11 +302,11 @@ static int pick_splits(int64_t Nkv, int64_t Hkv, int64_t Nq) {
     return (int)n;
 }
 
-template <int D, int R>
+template <int D, int R, int NW = 4>
 static int launch_vec(hipStream_t s, fattn_args &a) {
     a.groups = (int)(a.Hq / a.Hkv) / R;
     const dim3 grid((unsigned)a.n_splits, (unsigned)(a.Hkv * a.groups), (unsigned)a.Nq);
-    MI355_LAUNCH((k_fattn_vec<D, R>), grid, dim3(256), 0, s, a);
+    MI355_LAUNCH((k_fattn_vec<D, R, NW>), grid, dim3(NW * 64), 0, s, a);
     int rc = launch_status("k_fattn_vec");
     if (rc != MI355_OK) return rc;
     if (a.n_splits > 1) {
@@ -303,8 +321,19 @@ template <int D>
 static int launch_vec_r(hipStream_t s, fattn_args &a, int R) {
     // R = query heads served per group from one pass over the kv head's bytes.  A short context is not bandwidth-bound but
     // a serial chain of soft-max updates per (step, head): one head per group then spreads it over R times as many waves.
+    // Up to 1024 cells and few (token, head) pairs: one head per group, eight waves per group (32 cells of a D = 128 head per step,
+    // four steps' loads in flight) and no split of the cells over groups, so no second launch.  Measured per decoded token of
+    // the 8B model at 256 cells: 4 waves 1.897 ms, 8 waves 1.856 ms, 16 waves 1.875 ms; requesting K and V together with the mask
+    // instead of after it (one round trip less per step, but masked cells then cost their bytes) 1.91-1.96 ms.
     constexpr int64_t one_head_max = 1024;
-    if (a.Nkv <= one_head_max) return launch_vec<D, 1>(s, a);
+    if (a.Nkv <= one_head_max) {
+        if (a.Nq * a.Hq <= 512) {   // few (token, head) pairs: the chip is far from full
+            a.n_splits = 1;
+            a.cells_per_split = a.Nkv;
+            return launch_vec<D, 1, 8>(s, a);
+        }
+        return launch_vec<D, 1>(s, a);
+    }
     if (R % 4 == 0) return launch_vec<D, 4>(s, a);
     if (R % 2 == 0) return launch_vec<D, 2>(s, a);
     return launch_vec<D, 1>(s, a);
