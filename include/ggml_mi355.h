@@ -12,12 +12,13 @@
  *   reg         get_name "MI355X", get_device_count, get_device, get_proc_address (none)
  *   device      GPU type; get_memory (hipMemGetInfo); init_backend; get_buffer_type; a pinned host
  *               buffer type (hipHostMalloc) for the tensors the CPU backend hands over;
- *               supports_op / supports_buft; caps: async and host_buffer true,
- *               buffer_from_host_ptr and events false
+ *               supports_op / supports_buft; event_new / event_free / event_synchronize (HIP events
+ *               without timing); caps: async, host_buffer and events true, buffer_from_host_ptr false
  *   buffer type hipMalloc-backed, alignment 256, alloc size = ggml_nbytes
  *   buffer      set/get/memset/cpy_tensor and clear; set/get apply / undo the 16-byte-aligned
  *               device row layout for Q4_0, Q8_0 and Q6_K tensors
- *   backend     one HIP stream; set/get_tensor_async on it; graph_compute walks the graph once,
+ *   backend     one HIP stream; set/get_tensor_async, cpy_tensor_async (host tensors of the CPU backend
+ *               and tensors of this backend) and event_record / event_wait on it; graph_compute walks the graph once,
  *               matching runs of nodes (norm -> weight -> products -> rope -> cache store, gate/up
  *               -> SiLU*up -> down, ...) to one fused kernel each, records the launches of a
  *               decode-shaped graph into a HIP graph keyed by the graph's signature and replays

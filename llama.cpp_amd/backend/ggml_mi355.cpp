@@ -146,6 +146,7 @@ struct backend_ctx {
     }
     unsigned * tickets = nullptr;   // zeroed arrival counters of the gate/up launch (one per 32 output rows)
     size_t n_tickets = 0;
+    long async_uploads = 0, events_recorded = 0;   // reported with MI355_GRAPH_STATS=1
 
     // ---- replay of decode graphs as HIP graphs (see backend_graph_compute)
     struct replay_state {
@@ -296,6 +297,13 @@ struct plane_store {
         map.emplace(w->data, entry{planes, w->ne[1], w->ne[0]});
         return planes;
     }
+    // whether a tensor whose data lies in [base, base + size) has an entry
+    bool any(const void * base, size_t size) {
+        std::lock_guard<std::mutex> lock(mu);
+        for (const auto & kv : map)
+            if ((const char *) kv.first >= (const char *) base && (const char *) kv.first < (const char *) base + size) return true;
+        return false;
+    }
     // forget (and free) the planes of tensors whose data lies in [base, base + size); the caller has synchronized the device
     void drop(const void * base, size_t size) {
         std::lock_guard<std::mutex> lock(mu);
@@ -345,6 +353,13 @@ struct tile_store {
         g_prep_launches += mi355_launch_count() - before;
         map.emplace(w->data, entry{tiles, w->ne[1], w->ne[0]});
         return tiles;
+    }
+    // whether a tensor whose data lies in [base, base + size) has an entry
+    bool any(const void * base, size_t size) {
+        std::lock_guard<std::mutex> lock(mu);
+        for (const auto & kv : map)
+            if ((const char *) kv.first >= (const char *) base && (const char *) kv.first < (const char *) base + size) return true;
+        return false;
     }
     // forget (and free) the images of tensors whose data lies in [base, base + size); the caller has synchronized the device
     void drop(const void * base, size_t size) {
@@ -874,6 +889,8 @@ void backend_free(ggml_backend_t backend) {
     if (getenv("MI355_GRAPH_STATS"))
         fprintf(stderr, "MI355 graph replay: %ld captures, %ld replays, %.1f us of host time per replay\n", ctx->replay.captures, ctx->replay.replays,
                 ctx->replay.replays ? ctx->replay.host_us / (double) ctx->replay.replays : 0.0);
+    if (getenv("MI355_GRAPH_STATS") && (ctx->async_uploads || ctx->events_recorded))
+        fprintf(stderr, "MI355 transfers: %ld uploads on the backend stream, %ld events recorded\n", ctx->async_uploads, ctx->events_recorded);
     if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     delete backend;
@@ -885,19 +902,23 @@ void backend_free(ggml_backend_t backend) {
 void backend_set_tensor_async(ggml_backend_t backend, ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
     ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
-    if ((is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) || size == 0) {
+    // the layout permutation goes through the staging buffer; a K-quant matrix may have int8 planes or tile images to forget
+    const bool has_images = tensor->type == GGML_TYPE_Q4_K &&
+                            (planes().any(tensor->data, ggml_nbytes(tensor)) || tiles().any(tensor->data, ggml_nbytes(tensor)));
+    if (repack_of(tensor).yes || has_images || size == 0) {
         MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
         buf->iface.set_tensor(buf, tensor, data, offset, size);
         return;
     }
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipMemcpyAsync((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice, ctx->stream));
+    ctx->async_uploads++;
 }
 
 void backend_get_tensor_async(ggml_backend_t backend, const ggml_tensor * tensor, void * data, size_t offset, size_t size) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
     ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
-    if ((is_repacked_type(tensor->type) && ggml_is_contiguous(tensor)) || size == 0) {
+    if (repack_of(tensor).yes || size == 0) {
         MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
         buf->iface.get_tensor(buf, tensor, data, offset, size);
         return;
@@ -906,9 +927,52 @@ void backend_get_tensor_async(ggml_backend_t backend, const ggml_tensor * tensor
     MI355_HIP_OK(hipMemcpyAsync(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost, ctx->stream));
 }
 
+// Copies a tensor into one of this backend's tensors on its stream (ggml_backend_tensor_copy_async, ggml-backend.cpp:380-409; the
+// scheduler hands split inputs over this way, :1384).  Served: a source in host memory produced by a backend that computes
+// synchronously (the CPU backend: its result is complete when the scheduler gets here), and a source of this same backend.
+// Anything else returns false and the caller synchronizes and copies.
+bool backend_cpy_tensor_async(ggml_backend_t backend_src, ggml_backend_t backend_dst, const ggml_tensor * src, ggml_tensor * dst) {
+    backend_ctx * ctx = (backend_ctx *) backend_dst->context;
+    ggml_backend_buffer_t dbuf = dst->view_src ? dst->view_src->buffer : dst->buffer;
+    ggml_backend_buffer_t sbuf = src->view_src ? src->view_src->buffer : src->buffer;
+    if (!dbuf || !sbuf || dbuf->buft->iface.get_name != buft_get_name || dbuf->buft->device != backend_dst->device) return false;
+    if (!ggml_is_contiguous(src) || !ggml_is_contiguous(dst) || src->type != dst->type || ggml_nbytes(src) != ggml_nbytes(dst)) return false;
+    if (repack_of(dst).yes || is_repacked_type(src->type)) return false;   // layout permutations take the synchronous path
+    hipMemcpyKind kind;
+    if (ggml_backend_buffer_is_host(sbuf)) {
+        ggml_backend_dev_t sdev = ggml_backend_get_device(backend_src);
+        if (!sdev || ggml_backend_dev_type(sdev) != GGML_BACKEND_DEVICE_TYPE_CPU) return false;
+        kind = hipMemcpyHostToDevice;
+    } else if (backend_src == backend_dst && sbuf->buft == dbuf->buft) {
+        kind = hipMemcpyDeviceToDevice;
+    } else {
+        return false;
+    }
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipMemcpyAsync(dst->data, src->data, ggml_nbytes(src), kind, ctx->stream));
+    ctx->cache.valid = false;
+    return true;
+}
+
 void backend_synchronize(ggml_backend_t backend) {
     backend_ctx * ctx = (backend_ctx *) backend->context;
     MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
+}
+
+// Events (ggml_backend_event_*, ggml/src/ggml-backend.cpp:413-445): a HIP event without timing.  The model loader records one
+// after each chunk it uploads from a pinned buffer and waits for it before refilling that buffer
+// (src/llama-model-loader.cpp:1040-1046); the scheduler uses them between the copies of a pipelined graph (:1370-1438).
+void backend_event_record(ggml_backend_t backend, ggml_backend_event_t event) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipEventRecord((hipEvent_t) event->context, ctx->stream));
+    ctx->events_recorded++;
+}
+
+void backend_event_wait(ggml_backend_t backend, ggml_backend_event_t event) {
+    backend_ctx * ctx = (backend_ctx *) backend->context;
+    MI355_HIP_OK(hipSetDevice(ctx->device));
+    MI355_HIP_OK(hipStreamWaitEvent(ctx->stream, (hipEvent_t) event->context, 0));
 }
 
 // ------------------------------------------------------------------------------- graph execution with local fusion
@@ -1903,15 +1967,15 @@ const ggml_backend_i backend_iface = {
     /* .free               = */ backend_free,
     /* .set_tensor_async   = */ backend_set_tensor_async,
     /* .get_tensor_async   = */ backend_get_tensor_async,
-    /* .cpy_tensor_async   = */ nullptr,
+    /* .cpy_tensor_async   = */ backend_cpy_tensor_async,
     /* .synchronize        = */ backend_synchronize,
     /* .graph_plan_create  = */ nullptr,
     /* .graph_plan_free    = */ nullptr,
     /* .graph_plan_update  = */ nullptr,
     /* .graph_plan_compute = */ nullptr,
     /* .graph_compute      = */ backend_graph_compute,
-    /* .event_record       = */ nullptr,
-    /* .event_wait         = */ nullptr,
+    /* .event_record       = */ backend_event_record,
+    /* .event_wait         = */ backend_event_wait,
 };
 
 // ------------------------------------------------------------------------------- device
@@ -1931,7 +1995,7 @@ void device_get_props(ggml_backend_dev_t dev, ggml_backend_dev_props * props) {
     props->description = device_get_description(dev);
     props->type = GGML_BACKEND_DEVICE_TYPE_GPU;
     device_get_memory(dev, &props->memory_free, &props->memory_total);
-    props->caps = { /* async */ true, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ false };
+    props->caps = { /* async */ true, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ true };
 }
 
 ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
@@ -1973,6 +2037,26 @@ bool device_supports_buft(ggml_backend_dev_t dev, ggml_backend_buffer_type_t buf
     return buft->iface.get_name == buft_get_name && buft->device == dev;
 }
 
+ggml_backend_event_t device_event_new(ggml_backend_dev_t dev) {
+    device_ctx * ctx = (device_ctx *) dev->context;
+    if (hipSetDevice(ctx->device) != hipSuccess) return nullptr;
+    hipEvent_t ev = nullptr;
+    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+        (void) hipGetLastError();
+        return nullptr;
+    }
+    return new ggml_backend_event{ /* .device = */ dev, /* .context = */ ev };
+}
+
+void device_event_free(ggml_backend_dev_t, ggml_backend_event_t event) {
+    (void) hipEventDestroy((hipEvent_t) event->context);
+    delete event;
+}
+
+void device_event_synchronize(ggml_backend_dev_t, ggml_backend_event_t event) {
+    MI355_HIP_OK(hipEventSynchronize((hipEvent_t) event->context));
+}
+
 const ggml_backend_device_i device_iface = {
     /* .get_name             = */ device_get_name,
     /* .get_description      = */ device_get_description,
@@ -1986,9 +2070,9 @@ const ggml_backend_device_i device_iface = {
     /* .supports_op          = */ device_supports_op,
     /* .supports_buft        = */ device_supports_buft,
     /* .offload_op           = */ nullptr,
-    /* .event_new            = */ nullptr,
-    /* .event_free           = */ nullptr,
-    /* .event_synchronize    = */ nullptr,
+    /* .event_new            = */ device_event_new,
+    /* .event_free           = */ device_event_free,
+    /* .event_synchronize    = */ device_event_synchronize,
 };
 
 // ------------------------------------------------------------------------------- reg

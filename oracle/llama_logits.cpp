@@ -6,6 +6,8 @@
 //   llama_logits <model.gguf> <n_gpu_layers> <n_prompt> <n_decode> <out.bin> [<type_k> <type_v>]
 //
 // type_k / type_v: f16 (default), q8_0 or q4_0 - the KV cache types of llama.cpp's -ctk / -ctv.
+// LLAMA_LOGITS_NO_MMAP=1 in the environment loads the file with read() instead of mmap (llama.cpp's --no-mmap), which is the
+// path that uploads through pinned buffers, set_tensor_async and events when the device offers them.
 //
 // Tokens are (7 i + 3) mod n_vocab.  Output: float32 rows of n_vocab logits, one for the last prompt token and one per
 // decoded token (the token ids are fixed, the logits are not fed back).
@@ -31,6 +33,7 @@ int main(int argc, char ** argv) {
     llama_backend_init();
     llama_model_params mp = llama_model_default_params();
     mp.n_gpu_layers = ngl;
+    if (getenv("LLAMA_LOGITS_NO_MMAP")) mp.use_mmap = false;
     llama_model * model = llama_model_load_from_file(argv[1], mp);
     if (!model) return 1;
     llama_context_params cp = llama_context_default_params();

@@ -53,9 +53,11 @@ def test_llama_bench_runs_on_the_plugin(dev, tmp_path):
 LOGITS = os.path.join(ROOT, "oracle", "_ref", "llama_logits")
 
 
-def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None, cache=None):
+def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None, cache=None, mmap=True):
     import numpy as np
     env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN, MI355_GRAPH_STATS="1")
+    if not mmap:
+        env["LLAMA_LOGITS_NO_MMAP"] = "1"
     if not fusion:
         env["MI355_NO_FUSION"] = "1"
     if not graphs:
@@ -68,7 +70,27 @@ def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats
     if stats is not None:
         m = re.search(r"MI355 graph replay: (\d+) captures, (\d+) replays", r.stdout)
         stats["captures"], stats["replays"] = (int(m.group(1)), int(m.group(2))) if m else (0, 0)
+        m = re.findall(r"MI355 transfers: (\d+) uploads on the backend stream, (\d+) events recorded", r.stdout)
+        stats["uploads"], stats["events"] = max((int(a) for a, _ in m), default=0), max((int(b) for _, b in m), default=0)
     return np.fromfile(out, dtype=np.float32)
+
+
+def test_model_logits_async_loader(dev, tmp_path):
+    """Without mmap the reference's loader uploads the weights in 1 MiB chunks from pinned buffers with set_tensor_async and
+    fences the buffers with events (src/llama-model-loader.cpp:926-960, 1033-1046): chunks land at byte offsets inside tensors,
+    also inside those kept in the device row layout.  The logits must be the very ones of the mmap load."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    model = str(tmp_path / "small.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048)
+    mapped = _logits(model, 99, 40, 3, str(tmp_path / "mmap.bin"))
+    stats = {}
+    read = _logits(model, 99, 40, 3, str(tmp_path / "read.bin"), mmap=False, stats=stats)
+    assert stats["events"] > 20 and stats["uploads"] > 20, stats   # the loader did take the asynchronous path
+    assert np.isfinite(mapped).all() and np.array_equal(mapped, read)
 
 
 @pytest.mark.parametrize("n_prompt", [5, 40, 256])   # 256: the wide-tile GEMM on tile images (from 192 rows on)
