@@ -47,6 +47,12 @@ int mi355_device_supported(int device);
  * out[0] = shader-clock ticks, out[1] = ticks of the constant 100 MHz reference counter that passed meanwhile (DEVICE int64[2]).
  * Launched on a second stream next to a kernel under test, out[0] / out[1] * 100 is the clock in MHz that kernel gets. */
 int mi355_probe_clock(void *stream, int64_t *out, int64_t micros);
+/* Measurement aid, no counterpart in the reference: the rate at which compute units fill LDS with the 16-byte-per-lane
+ * global-to-LDS transfers that feed the wide-tile GEMM.  `n_groups` 512-thread groups (one per compute unit when n_groups is the
+ * number of compute units) each move iters * 8 KiB out of their own `region` bytes of `src` (region a multiple of 8 KiB,
+ * n_groups * region <= src_bytes; 64 KiB regions stay in L2, 4 MiB regions stream from HBM), six 1 KiB transfers in flight per
+ * wave.  out[g] (DEVICE int64[n_groups]) = shader-clock ticks group g took. */
+int mi355_probe_lds_fill(void *stream, const void *src, int64_t src_bytes, int64_t region, int n_groups, int iters, int64_t *out);
 
 /* Weight storage -------------------------------------------------------------------- *
  * Quantized weight rows are kept in HBM in a per-row "device layout" that makes every

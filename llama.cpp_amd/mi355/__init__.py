@@ -33,6 +33,7 @@ _SIGNATURES = {
     "mi355_launch_count": (C.c_uint64, []),
     "mi355_device_supported": (_int, [_int]),
     "mi355_probe_clock": (_int, [_p, _p, _i64]),
+    "mi355_probe_lds_fill": (_int, [_p, _p, _i64, _i64, _int, _int, _p]),
     "mi355_weights_scatter": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
     "mi355_weights_gather": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
     "mi355_quantize_q8_1": (_int, [_p, _p, _p, _i64, _i64, _i64]),
