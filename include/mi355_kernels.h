@@ -196,6 +196,22 @@ int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, in
 size_t mi355_mul_mat_q8k_tiled_ws_bytes(int64_t N, int64_t K, int64_t B);
 int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N,
                             int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
+/* One launch for up to three matrices of the same K-quant type that consume the same activation image (gate and up of llm_build_ffn,
+ * src/llama.cpp:280-320; Q, K and V of a layer where their types agree): their tiles fill the compute units together (gate + up at
+ * batch 512: 896 tiles = 3.5 rounds on 256 compute units instead of two launches of 2 rounds; Q + K + V: 192 tiles in one round
+ * instead of three launches cut along K and their three sum launches).  Each matrix computes exactly what
+ * mi355_mul_mat_q8k_tiled computes for it alone without a workspace.  A single matrix is handled as by mi355_mul_mat_q8k_tiled
+ * (ws: mi355_mul_mat_q8k_tiled_multi_ws_bytes(n_mats, Ns, K, B) bytes, 0 for more than one matrix).  residual: as above, per matrix. */
+typedef struct mi355_tiled_mat {
+    const void *tiles;      /* mi355_kq_unpack_tiles image of the matrix */
+    float *dst;             /* [B][dst_stride] */
+    const float *residual;  /* may be NULL; may be dst; same stride as dst */
+    int64_t N;              /* rows of the matrix */
+    int64_t dst_stride;     /* floats between two rows of dst, >= N */
+} mi355_tiled_mat;
+size_t mi355_mul_mat_q8k_tiled_multi_ws_bytes(int n_mats, const int64_t *Ns, int64_t K, int64_t B);
+int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
+                                  void *ws, size_t ws_bytes);
 
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE

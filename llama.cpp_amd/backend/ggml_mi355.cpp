@@ -147,6 +147,7 @@ struct backend_ctx {
     unsigned * tickets = nullptr;   // zeroed arrival counters of the gate/up launch (one per 32 output rows)
     size_t n_tickets = 0;
     long async_uploads = 0, events_recorded = 0;   // reported with MI355_GRAPH_STATS=1
+    const ggml_tensor * done_ahead = nullptr;      // a product that went out with an earlier node's launch (see tiled_multi)
 
     // ---- replay of decode graphs as HIP graphs (see backend_graph_compute)
     struct replay_state {
@@ -1270,6 +1271,48 @@ void note_window_writes(backend_ctx * ctx, const qkv_window & win, int64_t B) {
 // the v product, so the rotations cannot simply wait for the products: instead the q and k products write straight into the
 // memory of their ROPE nodes' results, which nothing else can occupy before those results are read (q by attention, k by its
 // cache store), and are rotated there.
+// Several K-quant products on one activation at a large batch: those of one weight type that have tile images go out as one
+// launch of the wide-tile GEMM, so that their tiles fill the compute units together (mi355_mul_mat_q8k_tiled_multi).  idx: graph
+// positions of the products, all reading the same src1.  Returns the mask of the products done (0 or at least two bits).
+unsigned tiled_multi(backend_ctx * ctx, hipStream_t s, const graph_walk & w, const int * idx, int n) {
+    const ggml_tensor * b = w.nodes[idx[0]]->src[1];
+    const int64_t K = b->ne[0], B = b->ne[1];
+    const void * tl[3] = {nullptr, nullptr, nullptr};
+    int n_of[2] = {0, 0};   // Q4_K, Q6_K
+    for (int k = 0; k < n && k < 3; k++) {
+        const ggml_tensor * mm = w.nodes[idx[k]];
+        if (!is_q8k_tile_candidate(mm) || mm->src[1]->data != b->data || mm->src[1]->ne[0] != K || mm->src[1]->ne[1] != B || mm->src[1]->nb[1] != b->nb[1] ||
+            mm->type != GGML_TYPE_F32 || mm->nb[0] != sizeof(float) || mm->nb[1] % sizeof(float) != 0 || q8k_format_for(s, mm) != ACT_Q8KT)
+            continue;
+        tl[k] = tiles().get(s, mm->src[0]);
+        if (tl[k]) n_of[mm->src[0]->type == GGML_TYPE_Q6_K]++;
+    }
+    const ggml_type type = n_of[1] > n_of[0] ? GGML_TYPE_Q6_K : GGML_TYPE_Q4_K;
+    if (n_of[type == GGML_TYPE_Q6_K] < 2) return 0;
+    if (!ctx->cached(b->data, K, B, ACT_Q8KT)) {
+        void * fresh = ctx->act_slot(mi355_act_q8k_tiled_bytes(K, B));
+        MI355_K_OK(mi355_quantize_act_q8k_tiled(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
+        ctx->cache = act_cache{b->data, K, B, ACT_Q8KT, true, fresh};
+    }
+    mi355_tiled_mat mats[3];
+    unsigned mask = 0;
+    int m = 0;
+    for (int k = 0; k < n && k < 3; k++) {
+        const ggml_tensor * mm = w.nodes[idx[k]];
+        if (!tl[k] || mm->src[0]->type != type) continue;
+        mats[m].tiles = tl[k];
+        mats[m].dst = (float *) ctx->out_ptr(mm);
+        mats[m].residual = nullptr;
+        mats[m].N = mm->src[0]->ne[1];
+        mats[m].dst_stride = (int64_t) (mm->nb[1] / sizeof(float));
+        m++;
+        mask |= 1u << k;
+    }
+    MI355_K_OK(mi355_mul_mat_q8k_tiled_multi(s, to_mi355_type(type), m, mats, ctx->cache.ptr, K, B, nullptr, 0));
+    for (int k = 0; k < m; k++) ctx->note_write(mats[k].dst, (size_t) mats[k].N * (size_t) B * sizeof(float));
+    return mask;
+}
+
 struct prefill_qkv {
     bool ok = false;
     int ik = -1, iv = -1, last = -1;
@@ -1341,6 +1384,10 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     const int j = w.next(i);
     ggml_tensor * nxt = j < w.n ? (ggml_tensor *) w.nodes[j] : nullptr;
 
+    if (node == ctx->done_ahead) {   // went out with an earlier product's launch
+        ctx->done_ahead = nullptr;
+        return i;
+    }
     // ---- prefill: Q, K and V products, then both rotations and both cache stores in one launch (see match_prefill_qkv)
     if (node->op == GGML_OP_MUL_MAT && ctx->n_redirect == 0 && node->src[1]->ne[1] > 4) {
         const prefill_qkv p = match_prefill_qkv(w, i);
@@ -1348,12 +1395,13 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             ctx->redirect_node[0] = node;  ctx->redirect_to[0] = p.rq->data;
             ctx->redirect_node[1] = p.mk;  ctx->redirect_to[1] = p.rk->data;
             ctx->n_redirect = 2;
-            int done = compute_fused(ctx, w, i);
-            GGML_ASSERT(done == i);        // a product followed by its ROPE takes nothing with it
-            done = compute_fused(ctx, w, p.ik);
-            GGML_ASSERT(done == p.ik);
-            done = compute_fused(ctx, w, p.iv);
-            GGML_ASSERT(done == p.iv);
+            const int at[3] = {i, p.ik, p.iv};
+            const unsigned together = tiled_multi(ctx, s, w, at, 3);   // those of one K-quant type in one launch
+            for (int k = 0; k < 3; k++) {
+                if (together & (1u << k)) continue;
+                const int done = compute_fused(ctx, w, at[k]);
+                GGML_ASSERT(done == at[k]);   // a product followed by its ROPE (or by a product, or by the stores) takes nothing with it
+            }
             ctx->n_redirect = 0;
             const ggml_tensor * rq = p.rq;
             const int32_t * op = (const int32_t *) rq->op_params;
@@ -1712,6 +1760,21 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     if (is_q8k_tile_candidate(node)) {
         const ggml_tensor * b = node->src[1];
         const int64_t K = b->ne[0], B = b->ne[1];
+        // MUL_MAT(gate) -> UNARY(SILU) -> MUL_MAT(up) -> MUL: the up product goes out with the gate product (it reads the same
+        // activation and nothing in between writes); its node is then passed over when the walk gets there
+        if (nxt && nxt->op == GGML_OP_UNARY && ggml_get_unary_op(nxt) == GGML_UNARY_OP_SILU && nxt->src[0] == node && w.sole_use(i) && ctx->done_ahead == nullptr &&
+            ctx->n_redirect == 0) {
+            const int ju = w.next(j);
+            const ggml_tensor * up = ju < w.n ? w.nodes[ju] : nullptr;
+            if (up && up->op == GGML_OP_MUL_MAT && up->src[1]->data == b->data && !bytes_overlap(up, node) && !bytes_overlap(up, b) && ggml_is_contiguous(up) &&
+                ggml_is_contiguous(node)) {
+                const int at[2] = {i, ju};
+                if (tiled_multi(ctx, s, w, at, 2) == 3u) {
+                    ctx->done_ahead = up;
+                    return i;
+                }
+            }
+        }
         // large batches: the wide-tile kernel on tile images of the weights (built on first use) and of the activation
         const int fmt = q8k_format_for(s, node);
         const void * tl = fmt == ACT_Q8KT ? tiles().get(s, node->src[0]) : nullptr;
@@ -1855,6 +1918,8 @@ graph_signature sign_graph(ggml_cgraph * cgraph, std::vector<uint64_t> * trace =
 
 void run_graph_launches(backend_ctx * ctx, ggml_cgraph * cgraph) {
     ctx->cache.valid = false;
+    ctx->done_ahead = nullptr;
+    ctx->n_redirect = 0;
     const graph_walk w(cgraph);
     static const bool log_graph = getenv("MI355_LOG_GRAPH") != nullptr;   // node list and the nodes each launch sequence consumed
     const uint64_t launches_before = mi355_launch_count(), prep_before = g_prep_launches.load();

@@ -158,9 +158,28 @@ constexpr int WT_A_AUX_TILE = (WT_BN / 16) * WT_A_AUX;       // 4608 bytes of ac
 // s_waitcnt that waits until at most n vector-memory operations of this wave are outstanding (nothing else)
 #define WT_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (7 << 4) | (0xF << 8))
 
+// One launch: up to three matrices of one type that share the activation.  Their tiles are numbered one matrix after the other,
+// row tile by row tile, so that together they fill rounds of groups that each matrix alone would leave partly empty (gate + up at
+// batch 512: 2 x 448 tiles = 3.5 rounds on 256 compute units instead of 2 x 2).  Cutting the last, partly empty round's tiles
+// along K so that short groups fill it was measured and dropped: 162 us against 160 us uncut for gate + up - with half of the
+// compute units idle the others run faster, so the uncut tail costs less than its group count suggests.
+// gridDim.y > 1 cuts every tile into gridDim.y slices (single matrices with few tiles; partial sums in dst, one N x B slab per
+// slice, added by k_wt_split_sum).
+struct wt_mat {
+    const int8_t *w_img;
+    float *dst;
+    const float *residual;   // may be null; same shape and stride as dst; may be dst itself
+    int64_t N, dst_stride;
+    int first_tile;          // index of this matrix's first tile in the launch (unused entries: INT_MAX)
+};
+struct wt_launch {
+    wt_mat m[3];
+    int n_col_tiles;
+    int n_tiles, n_tiles_padded;   // n_tiles_padded: rounded up to a multiple of 8
+};
+
 template <int TYPE>
-__global__ void __launch_bounds__(512, 1) k_mmq_w(const int8_t *__restrict__ w_img, const int8_t *__restrict__ a_img, float *dst, const float *residual,
-                                                  int64_t N, int64_t K, int64_t B, int64_t dst_stride, int n_col_tiles, int n_groups, int n_groups_padded) {
+__global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__restrict__ a_img, int64_t K, int64_t B) {
     constexpr bool Q4 = TYPE == MI355_Q4_K;
     constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
     constexpr int NP = 2;                                                      // weight planes
@@ -183,11 +202,19 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(const int8_t *__restrict__ w_i
     asm volatile("" ::"v"((void *)ring_buf), "v"((void *)aux0), "v"((void *)aux1) : "memory");
     auto ring = [&](int i) -> int8_t * { return ring_buf + (i & (NBUF - 1)) * STAGE; };
 
-    const int per_xcd = n_groups_padded >> 3;
-    const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-    if (lid >= n_groups) return;
-    const int64_t row0 = (int64_t)(lid / n_col_tiles) * WT_BM;
-    const int64_t col0 = (int64_t)(lid % n_col_tiles) * WT_BN;
+    // groups of one XCD (every eighth group index) take consecutive tiles: the column tiles of a weight row tile meet in one L2
+    const int tile = (int)(blockIdx.x & 7) * (P.n_tiles_padded >> 3) + (int)(blockIdx.x >> 3);
+    if (tile >= P.n_tiles) return;
+    const int mi = (tile >= P.m[1].first_tile ? 1 : 0) + (tile >= P.m[2].first_tile ? 1 : 0);
+    const int8_t *__restrict__ w_img = P.m[mi].w_img;
+    float *dst = P.m[mi].dst;
+    const float *residual = P.m[mi].residual;
+    const int64_t N = P.m[mi].N;
+    const int64_t dst_stride = P.m[mi].dst_stride;
+    const int n_col_tiles = P.n_col_tiles;
+    const int ltile = tile - P.m[mi].first_tile;
+    const int64_t row0 = (int64_t)(ltile / n_col_tiles) * WT_BM;
+    const int64_t col0 = (int64_t)(ltile % n_col_tiles) * WT_BN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -199,8 +226,11 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(const int8_t *__restrict__ w_i
     // split K: group y of gridDim.y walks super-blocks [sb_lo, sb_hi) and writes its sums to its own slice of `dst`
     const int64_t sb_per = (nsb + gridDim.y - 1) / gridDim.y;
     const int64_t sb_lo = (int64_t)blockIdx.y * sb_per, sb_hi = sb_lo + sb_per < nsb ? sb_lo + sb_per : nsb;
+    // where the sums go: element (b, n) of the product at out[(b - col0) * dst_stride + (n - row0)]
+    float *out = dst + col0 * dst_stride + row0;
+    if (residual) residual += col0 * dst_stride + row0;
     if (gridDim.y > 1) {
-        dst += (int64_t)blockIdx.y * B * dst_stride;
+        out += (int64_t)blockIdx.y * B * dst_stride;
         residual = nullptr;
     }
 
@@ -446,8 +476,8 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(const int8_t *__restrict__ w_i
         for (int r = 0; r < 16; r++) {
             const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
             if (n < N && b < B) {
-                const int64_t o = b * dst_stride + n;
-                dst[o] = residual ? acc[tb][r] + residual[o] : acc[tb][r];   // residual may be dst itself: one reader and writer per element
+                const int64_t o = (b - col0) * dst_stride + (n - row0);
+                out[o] = residual ? acc[tb][r] + residual[o] : acc[tb][r];   // residual may be dst itself: one reader and writer per element
             }
         }
     }
@@ -525,36 +555,92 @@ int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, in
     return launch_status("k_unpack_tiles");
 }
 
+// The plan of one launch over n_mats matrices (rows Ns[]) sharing B activation rows; a single matrix with few tiles is cut along K.
+struct wt_plan {
+    int n_col_tiles, n_tiles, first_tile[3];
+    int slices;   // > 1: every tile cut (single matrix only)
+};
+static wt_plan wt_make_plan(int n_mats, const int64_t *Ns, int64_t K, int64_t B, bool have_ws) {
+    wt_plan p;
+    p.n_col_tiles = (int)((B + WT_BN - 1) / WT_BN);
+    p.n_tiles = 0;
+    for (int i = 0; i < 3; i++) {
+        p.first_tile[i] = i < n_mats ? p.n_tiles : 0x7fffffff;
+        if (i < n_mats) p.n_tiles += (int)((Ns[i] + WT_BM - 1) / WT_BM) * p.n_col_tiles;
+    }
+    p.slices = have_ws && n_mats == 1 && Ns[0] % 4 == 0 ? wt_split_slices(Ns[0], K, B) : 1;
+    return p;
+}
+static size_t wt_plan_ws_bytes(const wt_plan &p, const int64_t *Ns, int64_t B) {
+    return p.slices > 1 ? (size_t)p.slices * (size_t)Ns[0] * (size_t)B * sizeof(float) : 0;
+}
+
 size_t mi355_mul_mat_q8k_tiled_ws_bytes(int64_t N, int64_t K, int64_t B) {
     if (N <= 0 || K <= 0 || B <= 0 || K % QKK != 0) return 0;
-    const int n = wt_split_slices(N, K, B);
-    return n > 1 && N % 4 == 0 ? (size_t)n * (size_t)N * (size_t)B * sizeof(float) : 0;
+    return wt_plan_ws_bytes(wt_make_plan(1, &N, K, B, true), &N, B);
+}
+
+size_t mi355_mul_mat_q8k_tiled_multi_ws_bytes(int n_mats, const int64_t *Ns, int64_t K, int64_t B) {
+    if (n_mats < 1 || n_mats > 3 || Ns == nullptr || K <= 0 || B <= 0 || K % QKK != 0) return 0;
+    for (int i = 0; i < n_mats; i++)
+        if (Ns[i] <= 0) return 0;
+    return wt_plan_ws_bytes(wt_make_plan(n_mats, Ns, K, B, true), Ns, B);
+}
+
+int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
+                                  void *ws, size_t ws_bytes) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_q8k_tiled: 1 to 3 matrices per launch, got %d", n_mats);
+    MI355_REQUIRE(K > 0 && B > 0 && K % QKK == 0, "mul_mat_q8k_tiled: bad shape K=%lld B=%lld (K must be a multiple of 256)", (long long)K, (long long)B);
+    MI355_REQUIRE(act != nullptr && ((uintptr_t)act & 15) == 0, "mul_mat_q8k_tiled: the activation image is not 16-byte aligned");
+    int64_t Ns[3] = {0, 0, 0};
+    for (int i = 0; i < n_mats; i++) {
+        MI355_REQUIRE(mats[i].N > 0 && mats[i].dst_stride >= mats[i].N, "mul_mat_q8k_tiled: matrix %d has N=%lld, dst_stride=%lld", i, (long long)mats[i].N,
+                      (long long)mats[i].dst_stride);
+        MI355_REQUIRE(mats[i].tiles != nullptr && ((uintptr_t)mats[i].tiles & 15) == 0 && mats[i].dst != nullptr, "mul_mat_q8k_tiled: matrix %d: bad pointers", i);
+        Ns[i] = mats[i].N;
+    }
+    wt_plan p = wt_make_plan(n_mats, Ns, K, B, ws != nullptr && ((uintptr_t)ws & 15) == 0);
+    if (ws_bytes < wt_plan_ws_bytes(p, Ns, B)) p = wt_make_plan(n_mats, Ns, K, B, false);
+    MI355_REQUIRE((int64_t)p.n_tiles + 8 < (1 << 30), "mul_mat_q8k_tiled: too many tiles");
+    hipStream_t s = (hipStream_t)stream;
+    wt_launch L;
+    for (int i = 0; i < 3; i++) {
+        const int k = i < n_mats ? i : 0;
+        L.m[i].w_img = (const int8_t *)mats[k].tiles;
+        L.m[i].dst = mats[k].dst;
+        L.m[i].residual = mats[k].residual;
+        L.m[i].N = mats[k].N;
+        L.m[i].dst_stride = mats[k].dst_stride;
+        L.m[i].first_tile = p.first_tile[i];
+    }
+    L.n_col_tiles = p.n_col_tiles;
+    L.n_tiles = p.n_tiles;
+    L.n_tiles_padded = (p.n_tiles + 7) & ~7;
+    if (p.slices > 1) {   // partial sums: one N x B slab per slice in the workspace
+        L.m[0].dst = (float *)ws;
+        L.m[0].residual = nullptr;
+        L.m[0].dst_stride = Ns[0];
+    }
+    const dim3 grid((unsigned)L.n_tiles_padded, (unsigned)p.slices);
+    if (type == MI355_Q4_K) MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
+    else MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
+    if (p.slices > 1)
+        MI355_LAUNCH(k_wt_split_sum, dim3((unsigned)((Ns[0] * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B,
+                     mats[0].dst_stride, p.slices);
+    return launch_status("k_mmq_w");
 }
 
 int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N,
                             int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k_tiled: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
-    MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k_tiled: K=%lld is not a multiple of 256", (long long)K);
-    MI355_REQUIRE(dst_stride >= N, "mul_mat_q8k_tiled: dst_stride < N");
-    MI355_REQUIRE(tiles != nullptr && ((uintptr_t)tiles & 15) == 0 && act != nullptr && ((uintptr_t)act & 15) == 0, "mul_mat_q8k_tiled: operands are not 16-byte aligned");
-    const int n_row_tiles = (int)((N + WT_BM - 1) / WT_BM), n_col_tiles = (int)((B + WT_BN - 1) / WT_BN);
-    MI355_REQUIRE((int64_t)n_row_tiles * n_col_tiles < (1 << 30), "mul_mat_q8k_tiled: too many tiles");
-    const int n_groups = n_row_tiles * n_col_tiles, n_groups_padded = (n_groups + 7) & ~7;
-    hipStream_t s = (hipStream_t)stream;
-    int n_slices = wt_split_slices(N, K, B);
-    if (n_slices < 2 || ws == nullptr || ((uintptr_t)ws & 15) != 0 || N % 4 != 0 || ws_bytes < (size_t)n_slices * (size_t)N * (size_t)B * sizeof(float)) n_slices = 1;
-    const dim3 grid((unsigned)n_groups_padded, (unsigned)n_slices);
-    float *out = n_slices > 1 ? (float *)ws : dst;
-    const float *res = n_slices > 1 ? nullptr : residual;
-    const int64_t out_stride = n_slices > 1 ? N : dst_stride;
-    if (type == MI355_Q4_K)
-        MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
-    else
-        MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, (const int8_t *)tiles, (const int8_t *)act, out, res, N, K, B, out_stride, n_col_tiles, n_groups, n_groups_padded);
-    if (n_slices > 1)
-        MI355_LAUNCH(k_wt_split_sum, dim3((unsigned)((N * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, residual, N, B, dst_stride, n_slices);
-    return launch_status("k_mmq_w");
+    mi355_tiled_mat m;
+    m.tiles = tiles;
+    m.dst = dst;
+    m.residual = residual;
+    m.N = N;
+    m.dst_stride = dst_stride;
+    return mi355_mul_mat_q8k_tiled_multi(stream, type, 1, &m, act, K, B, ws, ws_bytes);
 }
 
 }  // extern "C"

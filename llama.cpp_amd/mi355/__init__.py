@@ -17,6 +17,11 @@ BLOCK = {F32: (1, 4), F16: (1, 2), I32: (1, 4), Q4_0: (32, 18), Q8_0: (32, 34), 
 _p, _i64, _sz, _f, _int = C.c_void_p, C.c_int64, C.c_size_t, C.c_float, C.c_int
 
 
+class TiledMat(C.Structure):
+    """struct mi355_tiled_mat"""
+    _fields_ = [("tiles", _p), ("dst", _p), ("residual", _p), ("N", _i64), ("dst_stride", _i64)]
+
+
 class GemvMat(C.Structure):
     """struct mi355_gemv_mat"""
     _fields_ = [("type", _int), ("W", _p), ("N", _i64), ("dst", _p), ("dst_stride", _i64), ("residual", _p)]
@@ -66,6 +71,8 @@ _SIGNATURES = {
     "mi355_kq_unpack_tiles": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_q8k_tiled_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
+    "mi355_mul_mat_q8k_tiled_multi": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_rms_norm_mul_quant": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
     "mi355_swiglu_quant": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
@@ -244,6 +251,24 @@ def kq_unpack_tiles(t, W):
     tiles = torch.empty(load().mi355_kq_tiles_bytes(t, N, K), dtype=torch.uint8, device=W.device)
     check(load().mi355_kq_unpack_tiles(_stream(), t, _ptr(W), _ptr(tiles), N, K))
     return tiles
+
+
+def mul_mat_q8k_tiled_multi(t, tiles_list, act, Ns, K, B, dsts=None, residuals=None):
+    """one launch of the wide-tile K-quant GEMM for up to three matrices of type t that share `act` -> list of f32 [B, N_i]"""
+    import torch
+    n = len(tiles_list)
+    dev = tiles_list[0].device
+    if dsts is None:
+        dsts = [torch.empty((B, Ni), dtype=torch.float32, device=dev) for Ni in Ns]
+    arr = (TiledMat * n)()
+    for i in range(n):
+        arr[i].tiles, arr[i].dst, arr[i].N, arr[i].dst_stride = tiles_list[i].data_ptr(), dsts[i].data_ptr(), Ns[i], dsts[i].stride(0)
+        arr[i].residual = residuals[i].data_ptr() if residuals is not None and residuals[i] is not None else None
+    ns = (C.c_int64 * n)(*Ns)
+    nws = load().mi355_mul_mat_q8k_tiled_multi_ws_bytes(n, ns, K, B)
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+    check(load().mi355_mul_mat_q8k_tiled_multi(_stream(), t, n, arr, _ptr(act), K, B, _ptr(ws) if nws else None, nws))
+    return dsts
 
 
 def mul_mat_q8k_tiled(t, tiles, act, N, K, B, residual=None, split=True, dst=None):

@@ -13,7 +13,7 @@ import math
 
 import torch
 
-from . import (F16, F32, I32, Q4_K, Q6_K, Q4_0, Q8_0, BLOCK, GemvMat, Tensor, check, load, row_bytes, tensor_desc,
+from . import (F16, F32, I32, Q4_K, Q6_K, Q4_0, Q8_0, BLOCK, GemvMat, Tensor, TiledMat, check, load, row_bytes, tensor_desc,
                upload_weights, _ptr, _stream)
 
 
@@ -225,6 +225,19 @@ class LlamaRunner:
                 arr[i].residual = residual.data_ptr() if residual is not None else None
             check(self.lib.mi355_mul_mat_vec_q_multi(_stream(), len(mats), arr, _ptr(act), K, T))
         else:
+            if q8k == 2 and len(mats) > 1:   # matrices of one type go out as one launch of the wide-tile GEMM
+                rest = []
+                for t in sorted({m[0][0] for m in mats}):
+                    same = [m for m in mats if m[0][0] == t]
+                    if len(same) == 1:
+                        rest += same
+                        continue
+                    arr = (TiledMat * len(same))()
+                    for i, ((_, W), out) in enumerate(same):
+                        arr[i].tiles, arr[i].dst, arr[i].N, arr[i].dst_stride = self._tiles(t, W, out.shape[1], K).data_ptr(), out.data_ptr(), out.shape[1], out.stride(0)
+                        arr[i].residual = residual.data_ptr() if residual is not None else None
+                    check(self.lib.mi355_mul_mat_q8k_tiled_multi(_stream(), t, len(same), arr, _ptr(act), K, T, None, 0))
+                mats = rest
             for (t, W), out in mats:
                 if q8k:     # the residual add is the tile kernel's epilogue; products with few tiles are split along K through split_ws
                     N = out.shape[1]

@@ -362,3 +362,35 @@ def test_fused_producers_write_tile_images(dev, name, t):
     mi355.check(lib.mi355_quantize_act_q8k_tiled(None, y.data_ptr(), a4.data_ptr(), K, B, K))
     torch.cuda.synchronize()
     assert np.array_equal(a3.cpu().numpy()[sel], a4.cpu().numpy()[sel])
+
+
+@pytest.mark.parametrize("name,t", KQ_TYPES)
+@pytest.mark.parametrize("Ns,K,B", [((14336, 14336), 4096, 512),       # gate + up of an 8B llama: 896 tiles
+                                    ((4096, 1024, 1024), 4096, 512),    # Q, K, V: 192 tiles in one round
+                                    ((8200, 8300, 130), 2048, 300),     # ragged rows and batch
+                                    ((1000,), 6144, 300)])              # one matrix: cut along K like the single-matrix entry point
+def test_mmq_tiled_multi(dev, name, t, Ns, K, B):
+    """several matrices in one launch of the wide-tile GEMM: every matrix equals its own launch bit for bit, with and without
+    residual (also in place), and the oracle's integer arithmetic at the corners"""
+    import torch
+    import mi355
+    rng = np.random.default_rng(sum(Ns) + K + B + t)
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    act = mi355.quantize_act_q8k_tiled(_to_dev(dev, x))
+    Wq = [_weights(rng, t, N, K, "ref") for N in Ns]
+    tiles = [mi355.kq_unpack_tiles(t, mi355.upload_weights(t, _to_dev(dev, W))) for W in Wq]
+    res = [_to_dev(dev, rng.standard_normal((B, N)).astype(np.float32)) if i != 1 else None for i, N in enumerate(Ns)]
+    alone = [mi355.mul_mat_q8k_tiled(t, tl, act, N, K, B, split=len(Ns) == 1).cpu().numpy() for tl, N in zip(tiles, Ns)]
+    multi = [o.cpu().numpy() for o in mi355.mul_mat_q8k_tiled_multi(t, tiles, act, list(Ns), K, B)]
+    dsts = [torch.empty((B, N + 8 * i), dtype=torch.float32, device=dev)[:, :N] for i, N in enumerate(Ns)]    # a row stride per matrix
+    for i, N in enumerate(Ns):
+        if res[i] is not None:
+            dsts[i].copy_(res[i])     # residual in place: dst is its own residual
+    inplace = mi355.mul_mat_q8k_tiled_multi(t, tiles, act, list(Ns), K, B, dsts=dsts, residuals=[d if r is not None else None for d, r in zip(dsts, res)])
+    for i, N in enumerate(Ns):
+        assert np.array_equal(multi[i], alone[i])
+        want = multi[i] + res[i].cpu().numpy() if res[i] is not None else multi[i]
+        assert np.array_equal(inplace[i].cpu().numpy(), want)
+        Nt, Bt = min(N, 40), min(B, 16)
+        assert orc.nmse(multi[i][:Bt, :Nt], orc.mul_mat("cpu", t, Wq[i][:Nt], x[:Bt])) < 1e-9
+        assert orc.nmse(multi[i][B - 5:, N - 7:], orc.mul_mat("cpu", t, Wq[i][N - 7:], x[B - 5:])) < 1e-9
