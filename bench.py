@@ -477,27 +477,27 @@ def main():
                 "us_per_launch": round(us, 3), "algorithmic_bytes_per_launch": alg_bytes}
 
     # ------------------------------------------------------------------ ... and of the dominant prefill kernel
-    # k_mmq_w<Q4_K> (wide-tile int8-MFMA GEMM on tile images) on ffn_gate / ffn_up at the prompt's batch: 2 of the 7 products of a
-    # layer and 56% of its multiply-adds.  The same call the prefill pass makes, over the 64 matrices' tile images.
+    # k_mmq_w<Q4_K> (wide-tile int8-MFMA GEMM on tile images) on ffn_gate + ffn_up at the prompt's batch, one launch for the pair:
+    # 2 of the 7 products of a layer and 56% of its multiply-adds.  The same call the prefill pass makes, over the 32 layers' tile images.
     roofline_pp = None
     if args.pp >= 192:
         T = args.pp
         with torch.cuda.stream(stream):
             run._norm_quant(run.x[:T], weights.layers[0]["ffn_norm"], run.act_a, T, 2)
-            mats = [[(L[k], (run.gate if k == "gate" else run.up)[:T])] for L in weights.layers for k in ("gate", "up")]
-            for m in mats[:2]:
+            pairs = [[(L["gate"], run.gate[:T]), (L["up"], run.up[:T])] for L in weights.layers]
+            for m in pairs[:2]:
                 run._mm_act(m, run.act_a, K, T, q8k=2)
             p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             p0.record(stream)
-            for m in mats:
+            for m in pairs:
                 run._mm_act(m, run.act_a, K, T, q8k=2)
             p1.record(stream)
             stream.synchronize()
-        pus = p0.elapsed_time(p1) * 1e3 / len(mats)
-        ops = 2.0 * N * K * T
-        roofline_pp = {"kernel": "k_mmq_w<Q4_K> 14336 x 4096, batch %d (ffn_gate / ffn_up of the prefill pass)" % T, "bound": "mfma",
-                       "achieved": round(ops / pus / 1e6, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops / pus / 1e6 / INT8_PEAK_TOPS, 4),
-                       "traffic": None, "us_per_launch": round(pus, 2), "ops_per_launch": ops}
+        pus = p0.elapsed_time(p1) * 1e3 / len(pairs)
+        ops = 2.0 * 2 * N * K * T
+        roofline_pp = {"kernel": "k_mmq_w<Q4_K> on ffn_gate + ffn_up in one launch, 2 x 14336 x 4096, batch %d (the launch the prefill pass makes once per layer)" % T,
+                       "bound": "mfma", "achieved": round(ops / pus / 1e6, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                       "frac": round(ops / pus / 1e6 / INT8_PEAK_TOPS, 4), "traffic": None, "us_per_launch": round(pus, 2), "ops_per_launch": ops}
 
     # reference for the HBM traffic counters: a plain copy kernel of known size (256 MiB read, 256 MiB written) whose
     # FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit when this command runs under rocprofv3 --pmc
