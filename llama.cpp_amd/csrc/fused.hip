@@ -73,8 +73,8 @@ struct rope_kv_args {
     float theta_scale, freq_scale, ext_factor, attn_factor, corr0, corr1;
 };
 
-// rope_yarn + rotation as in k_rope (glue.hip) / ggml-cpu.c:9268-9306
-__device__ __forceinline__ void rope_pair(const rope_kv_args &a, int pos, int pair, float x0, float x1, float &y0, float &y1) {
+// rope_yarn as in k_rope (glue.hip) / ggml-cpu.c:9268-9306: the rotation of pair `pair` at position `pos`
+__device__ __forceinline__ void rope_cos_sin(const rope_kv_args &a, int pos, int pair, float &c, float &s) {
     const float theta_extrap = (float)pos * powf(a.theta_scale, (float)pair) / (a.ff ? a.ff[pair] : 1.0f);
     const float theta_interp = a.freq_scale * theta_extrap;
     float theta = theta_interp, mscale = a.attn_factor;
@@ -84,44 +84,57 @@ __device__ __forceinline__ void rope_pair(const rope_kv_args &a, int pos, int pa
         theta = theta_interp * (1.0f - ramp) + theta_extrap * ramp;
         mscale *= 1.0f + 0.1f * logf(1.0f / a.freq_scale);
     }
-    const float c = cosf(theta) * mscale, s = sinf(theta) * mscale;
-    y0 = sub_rn(mul_rn(x0, c), mul_rn(x1, s));   // no contraction: bit-identical to k_rope
-    y1 = add_rn(mul_rn(x0, s), mul_rn(x1, c));
+    c = cosf(theta) * mscale;
+    s = sinf(theta) * mscale;
 }
 
-// grid (H + 2*HK, T), D/2 threads: heads [0,H) rotate q in place, [H,H+HK) rotate k into the cache,
-// [H+HK, H+2HK) copy v into the cache
-__global__ void k_rope_kv_store(rope_kv_args a) {
-    const int t = blockIdx.y, h = blockIdx.x, pair = threadIdx.x;
-    const int D = a.D;
-    if (2 * pair >= D) return;
+// One 256-thread group per token.  The rotation of a pair depends on the token's position and the pair only, so a wave works it
+// out once per pair (lane = pair) and applies it to every head it is given: the four waves share the H query heads, HK key heads
+// and HK value heads (plain f16 copies) between them, wave w taking slots w, w + 4, ...  Same roundings as k_rope: no contraction.
+__global__ void __launch_bounds__(256) k_rope_kv_store(rope_kv_args a) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int D = a.D, n_slots = a.H + 2 * a.HK;
     const bool neox = (a.mode & 2) != 0;
-    const int i0 = 2 * pair;
-    const bool rot = i0 < a.n_dims;
-    const int ia = (rot && neox) ? pair : i0, ib = (rot && neox) ? pair + a.n_dims / 2 : i0 + 1;
-    if (h < a.H) {
-        const float *p = a.q + ((int64_t)t * a.H + h) * D;
-        float *o = a.q_out + ((int64_t)t * a.H + h) * D;
-        const float x0 = p[ia], x1 = p[ib];
-        float y0 = x0, y1 = x1;
-        if (rot) rope_pair(a, a.pos[t], pair, x0, x1, y0, y1);
-        o[ia] = y0;
-        o[ib] = y1;
-    } else if (h < a.H + a.HK) {
-        const int hk = h - a.H;
-        const float *p = a.k + ((int64_t)t * a.HK + hk) * D;
-        const float x0 = p[ia], x1 = p[ib];
-        float y0 = x0, y1 = x1;
-        if (rot) rope_pair(a, a.pos[t], pair, x0, x1, y0, y1);
-        _Float16 *c = (_Float16 *)(a.kcache + (int64_t)a.cells[t] * a.k_nb1 + (int64_t)hk * a.k_nb2);
-        c[ia] = (_Float16)y0;
-        c[ib] = (_Float16)y1;
-    } else {
-        const int hk = h - a.H - a.HK;
-        const float *p = a.v + ((int64_t)t * a.HK + hk) * D;
-        _Float16 *c = (_Float16 *)(a.vcache + (int64_t)a.cells[t] * a.v_nb1 + (int64_t)hk * a.v_nb2);
-        c[i0] = (_Float16)p[i0];
-        c[i0 + 1] = (_Float16)p[i0 + 1];
+    const int pos = a.pos[t];
+    const int64_t cell = a.cells[t];
+    for (int pair = lane; 2 * pair < D; pair += 64) {
+        const int i0 = 2 * pair;
+        const bool rot = i0 < a.n_dims;
+        const int ia = (rot && neox) ? pair : i0, ib = (rot && neox) ? pair + a.n_dims / 2 : i0 + 1;
+        float c = 1.0f, sn = 0.0f;
+        if (rot) rope_cos_sin(a, pos, pair, c, sn);
+        for (int h = wave; h < n_slots; h += 4) {
+            if (h < a.H) {
+                const float *p = a.q + ((int64_t)t * a.H + h) * D;
+                float *o = a.q_out + ((int64_t)t * a.H + h) * D;
+                const float x0 = p[ia], x1 = p[ib];
+                float y0 = x0, y1 = x1;
+                if (rot) {
+                    y0 = sub_rn(mul_rn(x0, c), mul_rn(x1, sn));
+                    y1 = add_rn(mul_rn(x0, sn), mul_rn(x1, c));
+                }
+                o[ia] = y0;
+                o[ib] = y1;
+            } else if (h < a.H + a.HK) {
+                const int hk = h - a.H;
+                const float *p = a.k + ((int64_t)t * a.HK + hk) * D;
+                const float x0 = p[ia], x1 = p[ib];
+                float y0 = x0, y1 = x1;
+                if (rot) {
+                    y0 = sub_rn(mul_rn(x0, c), mul_rn(x1, sn));
+                    y1 = add_rn(mul_rn(x0, sn), mul_rn(x1, c));
+                }
+                _Float16 *kc = (_Float16 *)(a.kcache + cell * a.k_nb1 + (int64_t)hk * a.k_nb2);
+                kc[ia] = (_Float16)y0;
+                kc[ib] = (_Float16)y1;
+            } else {
+                const int hk = h - a.H - a.HK;
+                const float *p = a.v + ((int64_t)t * a.HK + hk) * D;
+                _Float16 *vc = (_Float16 *)(a.vcache + cell * a.v_nb1 + (int64_t)hk * a.v_nb2);
+                vc[i0] = (_Float16)p[i0];
+                vc[i0 + 1] = (_Float16)p[i0 + 1];
+            }
+        }
     }
 }
 
@@ -222,8 +235,7 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
     const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
     a.corr0 = c0 > 0 ? c0 : 0;
     a.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
-    const int threads = (int)((D / 2 + 63) / 64 * 64);
-    MI355_LAUNCH(k_rope_kv_store, dim3((unsigned)(H + 2 * HK), (unsigned)T), dim3(threads), 0, (hipStream_t)stream, a);
+    MI355_LAUNCH(k_rope_kv_store, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, a);
     return launch_status("k_rope_kv_store");
 }
 
