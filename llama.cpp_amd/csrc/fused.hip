@@ -26,6 +26,21 @@ __global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restr
     rms_norm_quant_row<NV, FMT, false>(x + row * x_stride, w, y ? y + row * y_stride : nullptr, act, row, k, nrows, eps, sh);
 }
 
+// ... of rows that arrive as the slices of a product cut along K (+ residual): the sum launch and the norm launch in one
+template <int NV, int FMT>
+__global__ void __launch_bounds__(256) k_sum_rms_norm_mul_quant(const float *__restrict__ parts, int n_parts, int64_t part_stride, int64_t row_stride,
+                                                                const float *__restrict__ residual, float *__restrict__ sum, int64_t sum_stride,
+                                                                const float *__restrict__ w, void *__restrict__ act, int64_t k, int64_t nrows, float eps) {
+    __shared__ float sh[4];
+    const int64_t row = blockIdx.x;
+    row_parts P;
+    P.n = n_parts;
+    P.part_stride = part_stride;
+    P.res_row = residual ? residual + row * sum_stride : nullptr;
+    P.sum_row = sum + row * sum_stride;
+    rms_norm_quant_row<NV, FMT, false>(parts + row * row_stride, w, nullptr, act, row, k, nrows, eps, sh, P);
+}
+
 // h = silu(gate) * up, optional f32 output, optional Q8_1 output; one lane per 4 elements
 template <int FMT>
 __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ gate, const float *__restrict__ up, int64_t in_stride,
@@ -103,36 +118,42 @@ __global__ void __launch_bounds__(256) k_rope_kv_store(rope_kv_args a) {
         const int ia = (rot && neox) ? pair : i0, ib = (rot && neox) ? pair + a.n_dims / 2 : i0 + 1;
         float c = 1.0f, sn = 0.0f;
         if (rot) rope_cos_sin(a, pos, pair, c, sn);
-        for (int h = wave; h < n_slots; h += 4) {
-            if (h < a.H) {
-                const float *p = a.q + ((int64_t)t * a.H + h) * D;
-                float *o = a.q_out + ((int64_t)t * a.H + h) * D;
-                const float x0 = p[ia], x1 = p[ib];
-                float y0 = x0, y1 = x1;
-                if (rot) {
-                    y0 = sub_rn(mul_rn(x0, c), mul_rn(x1, sn));
-                    y1 = add_rn(mul_rn(x0, sn), mul_rn(x1, c));
+        // four of the wave's slots at a time: all loads first, so that their round trips overlap
+        for (int h0 = wave; h0 < n_slots; h0 += 16) {
+            float x0[4], x1[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int h = h0 + 4 * u;
+                x0[u] = x1[u] = 0.0f;
+                if (h >= n_slots) continue;
+                const float *p = h < a.H ? a.q + ((int64_t)t * a.H + h) * D
+                                 : h < a.H + a.HK ? a.k + ((int64_t)t * a.HK + (h - a.H)) * D : a.v + ((int64_t)t * a.HK + (h - a.H - a.HK)) * D;
+                const bool is_v = h >= a.H + a.HK;
+                x0[u] = p[is_v ? i0 : ia];
+                x1[u] = p[is_v ? i0 + 1 : ib];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int h = h0 + 4 * u;
+                if (h >= n_slots) continue;
+                float y0 = x0[u], y1 = x1[u];
+                if (h < a.H + a.HK && rot) {
+                    y0 = sub_rn(mul_rn(x0[u], c), mul_rn(x1[u], sn));
+                    y1 = add_rn(mul_rn(x0[u], sn), mul_rn(x1[u], c));
                 }
-                o[ia] = y0;
-                o[ib] = y1;
-            } else if (h < a.H + a.HK) {
-                const int hk = h - a.H;
-                const float *p = a.k + ((int64_t)t * a.HK + hk) * D;
-                const float x0 = p[ia], x1 = p[ib];
-                float y0 = x0, y1 = x1;
-                if (rot) {
-                    y0 = sub_rn(mul_rn(x0, c), mul_rn(x1, sn));
-                    y1 = add_rn(mul_rn(x0, sn), mul_rn(x1, c));
+                if (h < a.H) {
+                    float *o = a.q_out + ((int64_t)t * a.H + h) * D;
+                    o[ia] = y0;
+                    o[ib] = y1;
+                } else if (h < a.H + a.HK) {
+                    _Float16 *kc = (_Float16 *)(a.kcache + cell * a.k_nb1 + (int64_t)(h - a.H) * a.k_nb2);
+                    kc[ia] = (_Float16)y0;
+                    kc[ib] = (_Float16)y1;
+                } else {
+                    _Float16 *vc = (_Float16 *)(a.vcache + cell * a.v_nb1 + (int64_t)(h - a.H - a.HK) * a.v_nb2);
+                    vc[i0] = (_Float16)y0;
+                    vc[i0 + 1] = (_Float16)y1;
                 }
-                _Float16 *kc = (_Float16 *)(a.kcache + cell * a.k_nb1 + (int64_t)hk * a.k_nb2);
-                kc[ia] = (_Float16)y0;
-                kc[ib] = (_Float16)y1;
-            } else {
-                const int hk = h - a.H - a.HK;
-                const float *p = a.v + ((int64_t)t * a.HK + hk) * D;
-                _Float16 *vc = (_Float16 *)(a.vcache + cell * a.v_nb1 + (int64_t)hk * a.v_nb2);
-                vc[i0] = (_Float16)p[i0];
-                vc[i0 + 1] = (_Float16)p[i0 + 1];
             }
         }
     }
@@ -182,6 +203,20 @@ int mi355_rms_norm_mul_quant_q8k(void *stream, const float *x, int64_t x_stride,
 int mi355_rms_norm_mul_quant_q8k_tiled(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
                                        int64_t k, int64_t nrows, float eps) {
     return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, 2);
+}
+
+int mi355_sum_rms_norm_mul_quant_q8k_tiled(void *stream, const float *parts, int n_parts, int64_t k, int64_t nrows, const float *residual, float *sum,
+                                           int64_t sum_stride, const float *w, void *act, float eps) {
+    MI355_REQUIRE(k > 0 && k % QKK == 0 && k <= 8192, "sum_rms_norm_mul_quant: k=%lld must be a multiple of 256 and at most 8192", (long long)k);
+    MI355_REQUIRE(n_parts >= 1 && n_parts <= 8 && nrows > 0 && nrows < 0x7fffffff, "sum_rms_norm_mul_quant: bad slice or row count");
+    MI355_REQUIRE(parts != nullptr && sum != nullptr && w != nullptr && act != nullptr && sum_stride >= k && sum_stride % 4 == 0 &&
+                  (((uintptr_t)parts | (uintptr_t)sum | (uintptr_t)residual | (uintptr_t)w | (uintptr_t)act) & 15) == 0,
+                  "sum_rms_norm_mul_quant: operands must be non-null (but residual) and 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)nrows), block(256);
+    if (k <= 4096) MI355_LAUNCH((k_sum_rms_norm_mul_quant<4, 2>), grid, block, 0, s, parts, n_parts, k * nrows, k, residual, sum, sum_stride, w, act, k, nrows, eps);
+    else MI355_LAUNCH((k_sum_rms_norm_mul_quant<8, 2>), grid, block, 0, s, parts, n_parts, k * nrows, k, residual, sum, sum_stride, w, act, k, nrows, eps);
+    return launch_status("k_sum_rms_norm_mul_quant");
 }
 
 static int swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act, int64_t k,
