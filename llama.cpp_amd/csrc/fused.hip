@@ -26,21 +26,6 @@ __global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restr
     rms_norm_quant_row<NV, FMT, false>(x + row * x_stride, w, y ? y + row * y_stride : nullptr, act, row, k, nrows, eps, sh);
 }
 
-// ... of rows that arrive as the slices of a product cut along K (+ residual): the sum launch and the norm launch in one
-template <int NV, int FMT>
-__global__ void __launch_bounds__(256) k_sum_rms_norm_mul_quant(const float *__restrict__ parts, int n_parts, int64_t part_stride, int64_t row_stride,
-                                                                const float *__restrict__ residual, float *__restrict__ sum, int64_t sum_stride,
-                                                                const float *__restrict__ w, void *__restrict__ act, int64_t k, int64_t nrows, float eps) {
-    __shared__ float sh[4];
-    const int64_t row = blockIdx.x;
-    row_parts P;
-    P.n = n_parts;
-    P.part_stride = part_stride;
-    P.res_row = residual ? residual + row * sum_stride : nullptr;
-    P.sum_row = sum + row * sum_stride;
-    rms_norm_quant_row<NV, FMT, false>(parts + row * row_stride, w, nullptr, act, row, k, nrows, eps, sh, P);
-}
-
 // h = silu(gate) * up, optional f32 output, optional Q8_1 output; one lane per 4 elements
 template <int FMT>
 __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ gate, const float *__restrict__ up, int64_t in_stride,
@@ -203,20 +188,6 @@ int mi355_rms_norm_mul_quant_q8k(void *stream, const float *x, int64_t x_stride,
 int mi355_rms_norm_mul_quant_q8k_tiled(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,
                                        int64_t k, int64_t nrows, float eps) {
     return rms_norm_mul_quant(stream, x, x_stride, w, y, y_stride, act, k, nrows, eps, 2);
-}
-
-int mi355_sum_rms_norm_mul_quant_q8k_tiled(void *stream, const float *parts, int n_parts, int64_t k, int64_t nrows, const float *residual, float *sum,
-                                           int64_t sum_stride, const float *w, void *act, float eps) {
-    MI355_REQUIRE(k > 0 && k % QKK == 0 && k <= 8192, "sum_rms_norm_mul_quant: k=%lld must be a multiple of 256 and at most 8192", (long long)k);
-    MI355_REQUIRE(n_parts >= 1 && n_parts <= 8 && nrows > 0 && nrows < 0x7fffffff, "sum_rms_norm_mul_quant: bad slice or row count");
-    MI355_REQUIRE(parts != nullptr && sum != nullptr && w != nullptr && act != nullptr && sum_stride >= k && sum_stride % 4 == 0 &&
-                  (((uintptr_t)parts | (uintptr_t)sum | (uintptr_t)residual | (uintptr_t)w | (uintptr_t)act) & 15) == 0,
-                  "sum_rms_norm_mul_quant: operands must be non-null (but residual) and 16-byte aligned");
-    hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((unsigned)nrows), block(256);
-    if (k <= 4096) MI355_LAUNCH((k_sum_rms_norm_mul_quant<4, 2>), grid, block, 0, s, parts, n_parts, k * nrows, k, residual, sum, sum_stride, w, act, k, nrows, eps);
-    else MI355_LAUNCH((k_sum_rms_norm_mul_quant<8, 2>), grid, block, 0, s, parts, n_parts, k * nrows, k, residual, sum, sum_stride, w, act, k, nrows, eps);
-    return launch_status("k_sum_rms_norm_mul_quant");
 }
 
 static int swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act, int64_t k,
