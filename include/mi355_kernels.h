@@ -8,7 +8,7 @@
  *
  * Each entry point names the reference function it stands in for (paths relative to the
  * llama.cpp tree).  Element types use the reference's enum values
- * (ggml/include/ggml.h:351-392): F32 0, F16 1, Q4_0 2, Q8_0 8, Q8_1 9, Q4_K 12, Q6_K 14, I32 26.
+ * (ggml/include/ggml.h:351-392): F32 0, F16 1, Q4_0 2, Q8_0 8, Q8_1 9, Q4_K 12, Q5_K 13, Q6_K 14, I32 26.
  */
 #ifndef MI355_KERNELS_H
 #define MI355_KERNELS_H
@@ -27,7 +27,7 @@ extern "C" {
 
 enum mi355_type {
     MI355_F32 = 0, MI355_F16 = 1, MI355_Q4_0 = 2, MI355_Q8_0 = 8, MI355_Q8_1 = 9,
-    MI355_Q4_K = 12, MI355_Q6_K = 14, MI355_I32 = 26,
+    MI355_Q4_K = 12, MI355_Q5_K = 13, MI355_Q6_K = 14, MI355_I32 = 26,
 };
 
 /* Library / device ------------------------------------------------------------------ */
@@ -57,7 +57,7 @@ int mi355_probe_lds_fill(void *stream, const void *src, int64_t src_bytes, int64
 /* Weight storage -------------------------------------------------------------------- *
  * Quantized weight rows are kept in HBM in a per-row "device layout" that makes every
  * load a 16-byte aligned, coalesced access:
- *   Q4_K : unchanged (144-byte super-blocks are already 16-byte multiples)
+ *   Q4_K, Q5_K : unchanged (144- and 176-byte super-blocks are already 16-byte multiples)
  *   Q4_0 : [nb x 16 B nibbles][nb x fp16 d]
  *   Q8_0 : [nb x 32 B int8   ][nb x fp16 d]
  *   Q6_K : [nb x 128 B ql][nb x 64 B qh][nb x 16 B scales][nb x fp16 d]

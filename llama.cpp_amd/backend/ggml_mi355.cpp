@@ -51,7 +51,7 @@ namespace {
 
 // ------------------------------------------------------------------------------- helpers
 bool is_repacked_type(ggml_type t) { return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K; }
-bool is_weight_type(ggml_type t) { return is_repacked_type(t) || t == GGML_TYPE_Q4_K; }
+bool is_weight_type(ggml_type t) { return is_repacked_type(t) || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K; }
 
 int to_mi355_type(ggml_type t) {
     switch (t) {
@@ -61,6 +61,7 @@ int to_mi355_type(ggml_type t) {
         case GGML_TYPE_Q4_0: return MI355_Q4_0;
         case GGML_TYPE_Q8_0: return MI355_Q8_0;
         case GGML_TYPE_Q4_K: return MI355_Q4_K;
+        case GGML_TYPE_Q5_K: return MI355_Q5_K;
         case GGML_TYPE_Q6_K: return MI355_Q6_K;
         default: return -1;
     }
@@ -1041,6 +1042,7 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
     if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
     if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
+    if (a->type == GGML_TYPE_Q5_K && b->ne[1] > 8) return false;    // Q5_K: the GEMV only (up to eight rows); more rows take the generic path
     const int64_t K = a->ne[0];
     if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)

@@ -23,15 +23,15 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int WAVE = 64;
 
-// ---- block geometry (ggml/src/ggml-common.h:161-166, 203-221, 279-290, 314-320)
+// ---- block geometry (ggml/src/ggml-common.h:161-166, 203-221, 279-290, 296-308, 314-320)
 constexpr int QK = 32;     // elements per Q4_0 / Q8_0 / Q8_1 block
 constexpr int QKK = 256;   // elements per K-quant super-block
-constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q8_1_BYTES = 36, Q4_K_BYTES = 144, Q6_K_BYTES = 210;
+constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q8_1_BYTES = 36, Q4_K_BYTES = 144, Q5_K_BYTES = 176, Q6_K_BYTES = 210;
 
 __host__ __device__ inline int type_block_elems(int t) {
     switch (t) {
         case MI355_Q4_0: case MI355_Q8_0: case MI355_Q8_1: return QK;
-        case MI355_Q4_K: case MI355_Q6_K: return QKK;
+        case MI355_Q4_K: case MI355_Q5_K: case MI355_Q6_K: return QKK;
         case MI355_F32: case MI355_F16: case MI355_I32: return 1;
         default: return 0;
     }
@@ -42,6 +42,7 @@ __host__ __device__ inline int type_block_bytes(int t) {
         case MI355_Q8_0: return Q8_0_BYTES;
         case MI355_Q8_1: return Q8_1_BYTES;
         case MI355_Q4_K: return Q4_K_BYTES;
+        case MI355_Q5_K: return Q5_K_BYTES;
         case MI355_Q6_K: return Q6_K_BYTES;
         case MI355_F32: case MI355_I32: return 4;
         case MI355_F16: return 2;
@@ -49,7 +50,7 @@ __host__ __device__ inline int type_block_bytes(int t) {
     }
 }
 __host__ __device__ inline bool is_weight_type(int t) {
-    return t == MI355_Q4_0 || t == MI355_Q8_0 || t == MI355_Q4_K || t == MI355_Q6_K;
+    return t == MI355_Q4_0 || t == MI355_Q8_0 || t == MI355_Q4_K || t == MI355_Q5_K || t == MI355_Q6_K;
 }
 
 // ---- activation workspace: int8 q[nrows][k] then {float d; int sum;} ds[nrows][k/32]

@@ -208,6 +208,7 @@ __device__ __forceinline__ void gemv_dispatch(const gemv_item &m, int group, con
         case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
         case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
         case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
+        case MI355_Q5_K: gemv_body<MI355_Q5_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
         default: gemv_body<MI355_Q6_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
     }
 }
@@ -226,6 +227,7 @@ __global__ void __launch_bounds__(256) k_gemv_qkv(gemv_batch b, const int8_t *__
         case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
         case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
         case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
+        case MI355_Q5_K: gemv_body<MI355_Q5_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
         default: gemv_body<MI355_Q6_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
     }
 }
@@ -249,6 +251,7 @@ __global__ void __launch_bounds__(256) k_gemv_qkv_norm(gemv_batch b, int K, gemv
         case MI355_Q4_0: gemv_body<MI355_Q4_0, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
         case MI355_Q8_0: gemv_body<MI355_Q8_0, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
         case MI355_Q4_K: gemv_body<MI355_Q4_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
+        case MI355_Q5_K: gemv_body<MI355_Q5_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
         default: gemv_body<MI355_Q6_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
     }
 }
@@ -402,7 +405,7 @@ __global__ void __launch_bounds__(64) k_block_dots(const uint8_t *__restrict__ W
         if (!live) continue;
         if constexpr (TYPE == MI355_Q4_0 || TYPE == MI355_Q8_0) {
             out[row * ngran + c] = d.i0;
-        } else if constexpr (TYPE == MI355_Q4_K) {   // chunk c = sub-blocks 2c and 2c+1 of the row
+        } else if constexpr (TYPE == MI355_Q4_K || TYPE == MI355_Q5_K) {   // chunk c = sub-blocks 2c and 2c+1 of the row
             out[row * ngran + 2 * c] = d.i0;
             out[row * ngran + 2 * c + 1] = d.i1;
         } else {   // Q6_K: 16 granules per super-block
@@ -578,6 +581,7 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
             case MI355_Q4_0: launch_single_cols<MI355_Q4_0>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
             case MI355_Q8_0: launch_single_cols<MI355_Q8_0>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
             case MI355_Q4_K: launch_single_cols<MI355_Q4_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
+            case MI355_Q5_K: launch_single_cols<MI355_Q5_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
             default: launch_single_cols<MI355_Q6_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
         }
         return launch_status("k_gemv_q");
@@ -798,6 +802,7 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
             case MI355_Q4_0: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q4_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
             case MI355_Q8_0: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q8_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
             case MI355_Q4_K: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q4_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
+            case MI355_Q5_K: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q5_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
             default: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q6_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
         }
         return launch_status("k_gemv_id_unaligned");
@@ -815,6 +820,7 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
         case MI355_Q4_0: MI355_ID_LAUNCH(MI355_Q4_0) break;
         case MI355_Q8_0: MI355_ID_LAUNCH(MI355_Q8_0) break;
         case MI355_Q4_K: MI355_ID_LAUNCH(MI355_Q4_K) break;
+        case MI355_Q5_K: MI355_ID_LAUNCH(MI355_Q5_K) break;
         default: MI355_ID_LAUNCH(MI355_Q6_K) break;
     }
 #undef MI355_ID_LAUNCH
@@ -832,6 +838,7 @@ int mi355_block_dots_q8_1(void *stream, int type, const void *W, const void *a, 
         case MI355_Q4_0: MI355_LAUNCH(k_block_dots<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
         case MI355_Q8_0: MI355_LAUNCH(k_block_dots<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
         case MI355_Q4_K: MI355_LAUNCH(k_block_dots<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
+        case MI355_Q5_K: MI355_LAUNCH(k_block_dots<MI355_Q5_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
         default: MI355_LAUNCH(k_block_dots<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
     }
     return launch_status("k_block_dots");

@@ -444,6 +444,7 @@ int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *id
             case MI355_Q4_0: MI355_LAUNCH(k_get_rows_q<MI355_Q4_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
             case MI355_Q8_0: MI355_LAUNCH(k_get_rows_q<MI355_Q8_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
             case MI355_Q4_K: MI355_LAUNCH(k_get_rows_q<MI355_Q4_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
+            case MI355_Q5_K: MI355_LAUNCH(k_get_rows_q<MI355_Q5_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
             default: MI355_LAUNCH(k_get_rows_q<MI355_Q6_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
         }
         return launch_status("k_get_rows_q");

@@ -39,6 +39,7 @@ int gemv_unaligned(hipStream_t s, int type, const void *W, const void *act, floa
         case MI355_Q4_0: MI355_LAUNCH(k_gemv_unaligned<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
         case MI355_Q8_0: MI355_LAUNCH(k_gemv_unaligned<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
         case MI355_Q4_K: MI355_LAUNCH(k_gemv_unaligned<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
+        case MI355_Q5_K: MI355_LAUNCH(k_gemv_unaligned<MI355_Q5_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
         default: MI355_LAUNCH(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
     }
     return launch_status("k_gemv_unaligned");
@@ -104,6 +105,18 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
         // what the workspace holds beyond the quantized activation serves the split along K of products with few tiles
         const size_t used = mi355_mul_mat_ws_bytes(K, B);
         return mi355_mul_mat_q8k_ws(stream, type, W, ws, dst, nullptr, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
+    }
+    if (type == MI355_Q5_K && B > 8) {
+        // No tile kernel unpacks Q5_K yet: batches go through the GEMV eight activation rows at a time (each pass streams the
+        // matrix once), quantizing every eight rows into the start of the workspace.
+        for (int64_t b0 = 0; b0 < B; b0 += 8) {
+            const int64_t nb = B - b0 < 8 ? B - b0 : 8;
+            int rc = mi355_quantize_act(stream, x + b0 * x_stride, ws, K, nb, x_stride);
+            if (rc != MI355_OK) return rc;
+            rc = mi355_mul_mat_vec_q(stream, type, W, ws, dst + b0 * dst_stride, N, K, nb, dst_stride);
+            if (rc != MI355_OK) return rc;
+        }
+        return MI355_OK;
     }
     int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
     if (rc != MI355_OK) return rc;

@@ -5,6 +5,7 @@
 //   Q4_0 / Q8_0 : chunk = one 32-element block.
 //   Q4_K        : chunk = 32 bytes of qs = sub-blocks 2g (low nibbles) and 2g+1 (high nibbles),
 //                 64 elements; 4 chunks per super-block share its 16-byte header.
+//   Q5_K        : as Q4_K, plus the 32 bytes of qh that carry the fifth bit of all eight sub-blocks.
 //   Q6_K        : chunk = 16 bytes of ql + the matching 16 bytes of qh = two 16-element
 //                 scale groups, 32 elements; 8 chunks per super-block.
 // The same functions feed the GEMV kernels and the parity entry point that dumps the
@@ -204,6 +205,62 @@ template <> struct wq<MI355_Q4_K> {
 };
 
 // ---------------------------------------------------------------- Q6_K
+// Q5_K (block_q5_K, ggml/src/ggml-common.h:296-308: d, dmin, 12 scale bytes, qh[32], qs[128]): the Q4_K arithmetic on levels
+// 0..31 - low nibble from qs, bit 4 of sub-block j from bit j of qh[l] (dequantize_row_q5_K, ggml/src/ggml-quants.c:1482-1507;
+// ggml_vec_dot_q5_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:7539-7592)
+template <> struct wq<MI355_Q5_K> {
+    static constexpr int CHUNK = 64;
+    struct chunk { u32x4 q0, q1, h0, h1; float d, dmin, scA, mA, scB, mB; int g; };
+    typedef wq<MI355_Q4_K>::act act;
+    static __device__ __forceinline__ chunk load_w(const uint8_t *__restrict__ row, const row_layout &, int c) {
+        chunk w;
+        const int sb = c >> 2, g = c & 3;
+        const uint8_t *blk = row + sb * Q5_K_BYTES;
+        const u32x4 hdr = load16(blk);   // d, dmin, 12 scale bytes: same address for the 4 lanes of a super-block
+        w.h0 = load16(blk + 16);         // qh: also shared by the 4 lanes
+        w.h1 = load16(blk + 32);
+        w.q0 = load16(blk + 48 + g * 32);
+        w.q1 = load16(blk + 64 + g * 32);
+        w.g = g;
+        w.d = half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu));
+        w.dmin = half_bits_to_float((unsigned short)(hdr[0] >> 16));
+        const u32 s_lo = hdr[1] & 0x3F3F3F3Fu, m_lo = hdr[2] & 0x3F3F3F3Fu;
+        const u32 s_hi = (hdr[3] & 0x0F0F0F0Fu) | (((hdr[1] >> 6) & 0x03030303u) << 4);
+        const u32 m_hi = ((hdr[3] >> 4) & 0x0F0F0F0Fu) | (((hdr[2] >> 6) & 0x03030303u) << 4);
+        const u32 S = g < 2 ? s_lo : s_hi, M = g < 2 ? m_lo : m_hi;
+        const int sh = 16 * (g & 1);
+        w.scA = (float)((S >> sh) & 0xFFu);
+        w.scB = (float)((S >> (sh + 8)) & 0xFFu);
+        w.mA = (float)((M >> sh) & 0xFFu);
+        w.mB = (float)((M >> (sh + 8)) & 0xFFu);
+        return w;
+    }
+    static __device__ __forceinline__ act load_a(const int8_t *__restrict__ q, const act_ds *__restrict__ ds, int c) { return wq<MI355_Q4_K>::load_a(q, ds, c); }
+    // i0 / i1 = sum level*q over sub-blocks 2g / 2g+1
+    static __device__ __forceinline__ chunk_dots dots(const chunk &w, const act &A) {
+        int sA = 0, sB = 0;
+        const int ba = 2 * w.g, bb = 2 * w.g + 1;   // bits of qh that belong to the two sub-blocks
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const u32 la0 = (w.q0[i] & 0x0F0F0F0Fu) | (((w.h0[i] >> ba) & 0x01010101u) << 4);
+            const u32 la1 = (w.q1[i] & 0x0F0F0F0Fu) | (((w.h1[i] >> ba) & 0x01010101u) << 4);
+            const u32 lb0 = ((w.q0[i] >> 4) & 0x0F0F0F0Fu) | (((w.h0[i] >> bb) & 0x01010101u) << 4);
+            const u32 lb1 = ((w.q1[i] >> 4) & 0x0F0F0F0Fu) | (((w.h1[i] >> bb) & 0x01010101u) << 4);
+            sA = dot4((int)la0, (int)A.a0lo[i], sA);
+            sA = dot4((int)la1, (int)A.a0hi[i], sA);
+            sB = dot4((int)lb0, (int)A.a1lo[i], sB);
+            sB = dot4((int)lb1, (int)A.a1hi[i], sB);
+        }
+        chunk_dots r = {sA, sB};
+        return r;
+    }
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        const float pos = __builtin_fmaf(w.scA, mul_rn(A.d0, (float)r.i0), mul_rn(w.scB, mul_rn(A.d1, (float)r.i1)));
+        const float neg = __builtin_fmaf(w.mA, A.ds0, mul_rn(w.mB, A.ds1));
+        return add_rn(acc, __builtin_fmaf(w.d, pos, -mul_rn(w.dmin, neg)));
+    }
+};
+
 template <> struct wq<MI355_Q6_K> {
     static constexpr int CHUNK = 32;
     struct chunk { u32x4 ql, qh; float d, scA, scB; int shA, shB; };
@@ -264,7 +321,7 @@ template <> struct wq<MI355_Q6_K> {
 // Dequantized weight element e of a row stored in device layout.  Byte loads only, so it
 // works for rows that are not 16-byte aligned (K not a multiple of 256 for Q4_0/Q8_0, of
 // 2048 for Q6_K).  Semantics: dequantize_row_* of ggml/src/ggml-quants.c:255-273, 349-363,
-// 1280-1302, 1690-1719.
+// 1280-1302, 1482-1507, 1690-1719.
 template <int TYPE>
 __device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, const row_layout &L, int64_t e) {
     if constexpr (TYPE == MI355_Q4_0) {
@@ -290,6 +347,18 @@ __device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, c
         else { sc = (p[j + 4] & 0x0F) | ((p[j - 4] >> 6) << 4); mn = (p[j + 4] >> 4) | ((p[j] >> 6) << 4); }
         const uint8_t byte = blk[16 + 32 * (j >> 1) + l];
         const int n = (j & 1) ? (byte >> 4) : (byte & 0x0F);
+        return half_bits_to_float(dh) * (float)sc * (float)n - half_bits_to_float(mh) * (float)mn;
+    } else if constexpr (TYPE == MI355_Q5_K) {
+        const int64_t sb = e >> 8;
+        const int r = (int)(e & 255), j = r >> 5, l = r & 31;
+        const uint8_t *blk = row + sb * Q5_K_BYTES;
+        const unsigned short dh = (unsigned short)(blk[0] | (blk[1] << 8)), mh = (unsigned short)(blk[2] | (blk[3] << 8));
+        const uint8_t *p = blk + 4;
+        int sc, mn;
+        if (j < 4) { sc = p[j] & 63; mn = p[j + 4] & 63; }
+        else { sc = (p[j + 4] & 0x0F) | ((p[j - 4] >> 6) << 4); mn = (p[j + 4] >> 4) | ((p[j] >> 6) << 4); }
+        const uint8_t byte = blk[48 + 32 * (j >> 1) + l];
+        const int n = ((j & 1) ? (byte >> 4) : (byte & 0x0F)) + (((blk[16 + l] >> j) & 1) << 4);
         return half_bits_to_float(dh) * (float)sc * (float)n - half_bits_to_float(mh) * (float)mn;
     } else {
         const int64_t sb = e >> 8;

@@ -13,7 +13,7 @@ import math
 
 import torch
 
-from . import (F16, F32, I32, Q4_K, Q6_K, Q4_0, Q8_0, BLOCK, GemvMat, Tensor, TiledMat, check, load, row_bytes, tensor_desc,
+from . import (F16, F32, I32, Q4_K, Q5_K, Q6_K, Q4_0, Q8_0, BLOCK, GemvMat, Tensor, TiledMat, check, load, row_bytes, tensor_desc,
                upload_weights, _ptr, _stream)
 
 
@@ -43,6 +43,9 @@ def random_quantized(t, nrows, k, device, gen):
     if t == Q4_K:      # w = d*sc*n - dmin*m, sc,m ~ U[0,63], n ~ U[0,15]
         put_half(0, 0.02 / (31.5 * 4.6))
         put_half(2, 0.02 / (31.5 * 4.6) * 7.5)
+    elif t == Q5_K:    # w = d*sc*n - dmin*m, n ~ U[0,31]
+        put_half(0, 0.02 / (31.5 * 9.2))
+        put_half(2, 0.02 / (31.5 * 9.2) * 15.5)
     elif t == Q6_K:    # w = d*sc*(q-32), sc int8
         put_half(208, 0.02 / (74.0 * 18.5))
     elif t == Q4_0:    # w = d*(n-8)

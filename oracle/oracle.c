@@ -31,12 +31,13 @@
 
 /* ------------------------------------------------------------------ block layouts
  * ggml/src/ggml-common.h:161-166 (q4_0), 203-208 (q8_0), 210-221 (q8_1),
- * 279-290 (q4_K), 314-320 (q6_K), 322-328 (q8_K).  All packed, no padding. */
+ * 279-290 (q4_K), 296-308 (q5_K), 314-320 (q6_K), 322-328 (q8_K).  All packed, no padding. */
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[16]; } blk_q4_0;                       /* 18 B  */
 typedef struct { uint16_t d; int8_t qs[32]; } blk_q8_0;                        /* 34 B  */
 typedef struct { uint16_t d; uint16_t s; int8_t qs[32]; } blk_q8_1;            /* 36 B  */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[128]; } blk_q4_K; /* 144 B */
+typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qh[32]; uint8_t qs[128]; } blk_q5_K; /* 176 B */
 typedef struct { uint8_t ql[128]; uint8_t qh[64]; int8_t scales[16]; uint16_t d; } blk_q6_K; /* 210 B */
 typedef struct { float d; int8_t qs[256]; int16_t bsums[16]; } blk_q8_K;       /* 292 B */
 #pragma pack(pop)
@@ -94,7 +95,7 @@ int orc_block_elems(int type) {
     switch (type) {
         case ORC_F32: case ORC_F16: return 1;
         case ORC_Q4_0: case ORC_Q8_0: case ORC_Q8_1: return QK;
-        case ORC_Q4_K: case ORC_Q6_K: case ORC_Q8_K: return QKK;
+        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_Q8_K: return QKK;
         default: return 0;
     }
 }
@@ -106,6 +107,7 @@ size_t orc_block_bytes(int type) {
         case ORC_Q8_0: return sizeof(blk_q8_0);
         case ORC_Q8_1: return sizeof(blk_q8_1);
         case ORC_Q4_K: return sizeof(blk_q4_K);
+        case ORC_Q5_K: return sizeof(blk_q5_K);
         case ORC_Q6_K: return sizeof(blk_q6_K);
         case ORC_Q8_K: return sizeof(blk_q8_K);
         default: return 0;
@@ -150,6 +152,13 @@ static int q4k_level(const blk_q4_K *b, int e) {
     const int grp = e >> 6, r = e & 63;
     const uint8_t byte = b->qs[32 * grp + (r & 31)];
     return (r < 32) ? (byte & 0x0F) : (byte >> 4);
+}
+/* level 0..31 of element e of a Q5_K super-block: low nibble as in Q4_K, bit 4 from qh (dequantize_row_q5_K, ggml-quants.c:1482-1507:
+ * sub-block j = e / 32 takes bit j of qh[e % 32]) */
+static int q5k_level(const blk_q5_K *b, int e) {
+    const int j = e / 32, l = e % 32;
+    const uint8_t q = b->qs[(j / 2) * 32 + l];
+    return ((j & 1) ? (q >> 4) : (q & 0x0F)) + (((b->qh[l] >> j) & 1) ? 16 : 0);
 }
 
 /* ------------------------------------------------------------------ Q4_0
@@ -364,6 +373,77 @@ static void dequant_q4_K(const blk_q4_K *x, float *y, int64_t k) {
     }
 }
 
+/* ------------------------------------------------------------------ Q5_K
+ * quantize_row_q5_K_ref, ggml/src/ggml-quants.c:1395-1480: the Q4_K scheme with 32 levels (search parameters -0.5, 0.1, 15) and the
+ * fifth bit of sub-block j in bit j of qh */
+static void quant_q5_K(const float *x, blk_q5_K *y, int64_t k) {
+    uint8_t L[QKK], Laux[32];
+    float wts[32], mins[8], scales[8];
+    for (int64_t sb = 0; sb < k / QKK; sb++, x += QKK) {
+        float max_scale = 0, max_min = 0;
+        for (int j = 0; j < 8; j++) {
+            float sum_x2 = 0;
+            for (int l = 0; l < 32; l++) sum_x2 += x[32 * j + l] * x[32 * j + l];
+            const float av_x = sqrtf(sum_x2 / 32);
+            for (int l = 0; l < 32; l++) wts[l] = av_x + fabsf(x[32 * j + l]);
+            scales[j] = fit_scale_min(32, 31, x + 32 * j, wts, L + 32 * j, &mins[j], Laux, -0.5f, 0.1f, 15);
+            if (scales[j] > max_scale) max_scale = scales[j];
+            if (mins[j] > max_min) max_min = mins[j];
+        }
+        const float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
+        const float inv_min = max_min > 0 ? 63.f / max_min : 0.f;
+        memset(y[sb].scales, 0, 12);
+        for (int j = 0; j < 8; j++) {
+            uint8_t ls = (uint8_t)near_int(inv_scale * scales[j]);
+            uint8_t lm = (uint8_t)near_int(inv_min * mins[j]);
+            ls = (uint8_t)MINI(63, ls);
+            lm = (uint8_t)MINI(63, lm);
+            if (j < 4) {
+                y[sb].scales[j] = ls;
+                y[sb].scales[j + 4] = lm;
+            } else {
+                y[sb].scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                y[sb].scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                y[sb].scales[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        y[sb].d = orc_f32_to_f16(max_scale / 63.f);
+        y[sb].dmin = orc_f32_to_f16(max_min / 63.f);
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, mn;
+            q4k_scale_min(j, y[sb].scales, &sc, &mn);
+            const float d = orc_f16_to_f32(y[sb].d) * sc;
+            if (!d) continue;
+            const float dm = orc_f16_to_f32(y[sb].dmin) * mn;
+            for (int i = 0; i < 32; i++) {
+                int l = near_int((x[32 * j + i] + dm) / d);
+                L[32 * j + i] = (uint8_t)MAXI(0, MINI(31, l));
+            }
+        }
+        memset(y[sb].qh, 0, 32);
+        for (int j = 0; j < 8; j++)
+            for (int l = 0; l < 32; l++) {
+                const int v = L[32 * j + l];
+                uint8_t *q = &y[sb].qs[(j / 2) * 32 + l];
+                if (j & 1) *q = (uint8_t)((*q & 0x0F) | ((v & 15) << 4));
+                else *q = (uint8_t)(v & 15);
+                if (v > 15) y[sb].qh[l] |= (uint8_t)(1u << j);
+            }
+    }
+}
+/* dequantize_row_q5_K, ggml/src/ggml-quants.c:1482-1507 */
+static void dequant_q5_K(const blk_q5_K *x, float *y, int64_t k) {
+    for (int64_t sb = 0; sb < k / QKK; sb++) {
+        const float d = orc_f16_to_f32(x[sb].d), dmin = orc_f16_to_f32(x[sb].dmin);
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, mn;
+            q4k_scale_min(j, x[sb].scales, &sc, &mn);
+            const float dj = d * sc, mj = dmin * mn;
+            for (int l = 0; l < 32; l++) y[sb * QKK + 32 * j + l] = dj * q5k_level(&x[sb], 32 * j + l) - mj;
+        }
+    }
+}
+
 /* ------------------------------------------------------------------ Q6_K
  * make_qx_quants with rmse_type 1 and no weights, ggml/src/ggml-quants.c:379-446 */
 static float fit_scale_sym(int n, int nmax, const float *x, int8_t *L) {
@@ -497,6 +577,7 @@ static int quantize_row(int type, const float *x, void *y, int64_t k) {
         case ORC_Q8_0: quant_q8_0(x, (blk_q8_0 *)y, k); return 0;
         case ORC_Q8_1: quant_q8_1(x, (blk_q8_1 *)y, k); return 0;
         case ORC_Q4_K: quant_q4_K(x, (blk_q4_K *)y, k); return 0;
+        case ORC_Q5_K: quant_q5_K(x, (blk_q5_K *)y, k); return 0;
         case ORC_Q6_K: quant_q6_K(x, (blk_q6_K *)y, k); return 0;
         case ORC_Q8_K: quant_q8_K(x, (blk_q8_K *)y, k); return 0;
         default: return -1;
@@ -510,6 +591,7 @@ static int dequantize_row(int type, const void *x, float *y, int64_t k) {
         case ORC_Q8_0: dequant_q8_0((const blk_q8_0 *)x, y, k); return 0;
         case ORC_Q8_1: dequant_q8_1((const blk_q8_1 *)x, y, k); return 0;
         case ORC_Q4_K: dequant_q4_K((const blk_q4_K *)x, y, k); return 0;
+        case ORC_Q5_K: dequant_q5_K((const blk_q5_K *)x, y, k); return 0;
         case ORC_Q6_K: dequant_q6_K((const blk_q6_K *)x, y, k); return 0;
         case ORC_Q8_K: dequant_q8_K((const blk_q8_K *)x, y, k); return 0;
         default: return -1;
@@ -545,6 +627,7 @@ static int weight_level(int type, const void *row, int64_t e) {
         }
         case ORC_Q8_0: return ((const blk_q8_0 *)row + e / QK)->qs[e % QK];
         case ORC_Q4_K: return q4k_level((const blk_q4_K *)row + e / QKK, (int)(e % QKK));
+        case ORC_Q5_K: return q5k_level((const blk_q5_K *)row + e / QKK, (int)(e % QKK));
         case ORC_Q6_K: return q6k_level((const blk_q6_K *)row + e / QKK, (int)(e % QKK)) - 32;
         default: return 0;
     }
@@ -552,7 +635,7 @@ static int weight_level(int type, const void *row, int64_t e) {
 static int granule(int type) { return type == ORC_Q6_K ? 16 : 32; }
 
 int orc_block_dots_q8_1(int type, const void *W, const void *a, int64_t nrows, int64_t k, int32_t *out) {
-    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q6_K) return -1;
+    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q5_K && type != ORC_Q6_K) return -1;
     if (k % orc_block_elems(type)) return -1;
     const int g = granule(type);
     const size_t rb = orc_row_bytes(type, k);
@@ -616,6 +699,26 @@ static float dot_q4_K_q8_K(const blk_q4_K *w, const blk_q8_K *a, int64_t k) {   
     for (int l = 0; l < 8; l++) sumf += sums[l];
     return sumf;
 }
+static float dot_q5_K_q8_K(const blk_q5_K *w, const blk_q8_K *a, int64_t k) {   /* ggml-cpu-quants.c:7539-7592: the Q4_K form on 5-bit levels */
+    float sums[8] = {0};
+    float sumf = 0;
+    for (int64_t sb = 0; sb < k / QKK; sb++) {
+        int32_t lane[8] = {0};
+        int summ = 0;
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, mn;
+            q4k_scale_min(j, w[sb].scales, &sc, &mn);
+            summ += (a[sb].bsums[2 * j] + a[sb].bsums[2 * j + 1]) * mn;
+            for (int l = 0; l < 32; l++) lane[l & 7] += sc * (q5k_level(&w[sb], 32 * j + l) * a[sb].qs[32 * j + l]);
+        }
+        const float d = orc_f16_to_f32(w[sb].d) * a[sb].d;
+        for (int l = 0; l < 8; l++) sums[l] += d * lane[l];
+        const float dmin = orc_f16_to_f32(w[sb].dmin) * a[sb].d;
+        sumf -= dmin * summ;
+    }
+    for (int l = 0; l < 8; l++) sumf += sums[l];
+    return sumf;
+}
 static float dot_q6_K_q8_K(const blk_q6_K *w, const blk_q8_K *a, int64_t k) {   /* ggml-cpu-quants.c:8247-8289 */
     float sums[8] = {0};
     float sumf = 0;
@@ -634,7 +737,7 @@ int orc_mul_mat_cpu(int type, const void *W, const float *x, float *dst, int64_t
     int atype;
     switch (type) {
         case ORC_Q4_0: case ORC_Q8_0: atype = ORC_Q8_0; break;
-        case ORC_Q4_K: case ORC_Q6_K: atype = ORC_Q8_K; break;
+        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: atype = ORC_Q8_K; break;
         default: return -1;
     }
     if (K % orc_block_elems(type)) return -1;
@@ -650,6 +753,7 @@ int orc_mul_mat_cpu(int type, const void *W, const float *x, float *dst, int64_t
                 case ORC_Q4_0: r = dot_q4_0_q8_0((const blk_q4_0 *)row, (const blk_q8_0 *)act, K); break;
                 case ORC_Q8_0: r = dot_q8_0_q8_0((const blk_q8_0 *)row, (const blk_q8_0 *)act, K); break;
                 case ORC_Q4_K: r = dot_q4_K_q8_K((const blk_q4_K *)row, (const blk_q8_K *)act, K); break;
+                case ORC_Q5_K: r = dot_q5_K_q8_K((const blk_q5_K *)row, (const blk_q8_K *)act, K); break;
                 default:       r = dot_q6_K_q8_K((const blk_q6_K *)row, (const blk_q8_K *)act, K); break;
             }
             dst[b * N + n] = r;
@@ -685,6 +789,13 @@ static double row_dot_q8_1(int type, const void *row, const blk_q8_1 *act, int64
                 for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
                 acc += dx * ((double)orc_f16_to_f32(w->d) * sc * isum - (double)orc_f16_to_f32(w->dmin) * mn * sumq);
             } break;
+            case ORC_Q5_K: {
+                const blk_q5_K *w = (const blk_q5_K *)row + b / 8;
+                uint8_t sc, mn;
+                q4k_scale_min((int)(b % 8), w->scales, &sc, &mn);
+                for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
+                acc += dx * ((double)orc_f16_to_f32(w->d) * sc * isum - (double)orc_f16_to_f32(w->dmin) * mn * sumq);
+            } break;
             default: { /* Q6_K: two 16-element groups per activation block */
                 const blk_q6_K *w = (const blk_q6_K *)row + b / 8;
                 for (int j = 0; j < 16; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
@@ -698,7 +809,7 @@ static double row_dot_q8_1(int type, const void *row, const blk_q8_1 *act, int64
 }
 
 int orc_mul_mat_q8_1(int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B) {
-    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q6_K) return -1;
+    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q5_K && type != ORC_Q6_K) return -1;
     if (K % orc_block_elems(type)) return -1;
     const size_t wrb = orc_row_bytes(type, K);
     blk_q8_1 *act = (blk_q8_1 *)malloc(orc_row_bytes(ORC_Q8_1, K));
@@ -733,7 +844,7 @@ int orc_mul_mat_f64(int type, const void *W, const float *x, float *dst, int64_t
  * ggml_compute_forward_mul_mat_id, ggml/src/ggml-cpu/ggml-cpu.c:7717-7895 */
 int orc_mul_mat_id_q8_1(int type, const void *as, const float *b, const int32_t *ids, int64_t ids_stride, float *dst,
                         int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T) {
-    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q6_K) return -1;
+    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q5_K && type != ORC_Q6_K) return -1;
     const size_t wrb = orc_row_bytes(type, K);
     blk_q8_1 *act = (blk_q8_1 *)malloc(orc_row_bytes(ORC_Q8_1, K));
     if (!act) return -1;

@@ -23,6 +23,7 @@ enum orc_type {
     ORC_Q8_0 = 8,
     ORC_Q8_1 = 9,
     ORC_Q4_K = 12,
+    ORC_Q5_K = 13,
     ORC_Q6_K = 14,
     ORC_Q8_K = 15,
 };

@@ -25,7 +25,8 @@ def main():
     assert orc.ref is not None, "build oracle/_ref first (make -C oracle ref refdriver)"
     rng = np.random.default_rng(20240607)
     K = 512
-    for name, t in list(orc.WEIGHT_TYPES.items()) + [("q8_1", orc.Q8_1), ("q8_K", orc.Q8_K)]:
+    first_types = [(n, t) for n, t in orc.WEIGHT_TYPES.items() if n in ("q4_0", "q8_0", "q4_K", "q6_K")]   # the stream below was laid out for these
+    for name, t in first_types + [("q8_1", orc.Q8_1), ("q8_K", orc.Q8_K)]:
         x = (rng.standard_normal((4, K)) * (0.02 if name not in ("q8_1", "q8_K") else 1.0)).astype(np.float32)
         x[0, :32] = 0
         q = orc.quantize("ref", t, x)
@@ -41,10 +42,21 @@ def main():
     sp[0, 128:160] = np.linspace(-7e4, 7e4, 32)
     np.savez_compressed(os.path.join(HERE, "q8_1_special.npz"), x=sp, q=orc.quantize("ref", orc.Q8_1, sp))
 
-    for name, t in orc.WEIGHT_TYPES.items():
+    for name, t in first_types:
         W = orc.quantize("ref", t, (rng.standard_normal((48, K)) * 0.02).astype(np.float32))
         x = rng.standard_normal((3, K)).astype(np.float32)
         np.savez_compressed(os.path.join(HERE, "mul_mat_%s.npz" % name), W=W, x=x, y=orc.mul_mat("ref", t, W, x))
+
+    # weight types added later draw from a generator of their own, so that the files above keep their contents
+    for seed, (name, t) in enumerate([(n, t) for n, t in orc.WEIGHT_TYPES.items() if (n, t) not in first_types]):
+        r2 = np.random.default_rng(20240610 + seed)
+        x = (r2.standard_normal((4, K)) * 0.02).astype(np.float32)
+        x[0, :32] = 0
+        q = orc.quantize("ref", t, x)
+        np.savez_compressed(os.path.join(HERE, "quant_%s.npz" % name), x=x, q=q, dq=orc.dequantize("ref", t, q, K))
+        W = orc.quantize("ref", t, (r2.standard_normal((48, K)) * 0.02).astype(np.float32))
+        xa = r2.standard_normal((3, K)).astype(np.float32)
+        np.savez_compressed(os.path.join(HERE, "mul_mat_%s.npz" % name), W=W, x=xa, y=orc.mul_mat("ref", t, W, xa))
 
     D, Nq, Nkv, Hq, Hkv = 64, 3, 40, 4, 2
     q = rng.standard_normal((Hq, Nq, D)).astype(np.float32)

@@ -16,8 +16,8 @@ import struct
 
 import numpy as np
 
-F32, Q4_K, Q6_K = 0, 12, 14
-BLOCK = {Q4_K: (256, 144), Q6_K: (256, 210)}
+F32, Q4_K, Q5_K, Q6_K = 0, 12, 13, 14
+BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
 T_U32, T_F32, T_STR, T_U64 = 4, 6, 8, 10
 
 
@@ -44,35 +44,36 @@ def _kv(key, vtype, value):
     raise ValueError(vtype)
 
 
-def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert=0):
+def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert=0, base=Q4_K):
     """n_expert > 0: mixture-of-experts feed-forward (src/llama-model.cpp:1553-1558) with every quantized tensor Q4_K, the mix
-    of `llama-quantize --pure ... Q4_K`; the router ffn_gate_inp stays f32 (src/llama-quant.cpp:749)"""
-    t = [("token_embd.weight", Q4_K, (n_embd, n_vocab))]
+    of `llama-quantize --pure ... Q4_K`; the router ffn_gate_inp stays f32 (src/llama-quant.cpp:749).
+    base: Q4_K for the Q4_K_M mix, Q5_K for Q5_K_M (the same rules with Q5_K as the default type, src/llama-quant.cpp:122-340)"""
+    t = [("token_embd.weight", base, (n_embd, n_vocab))]
     for il in range(n_layer):
         more = use_more_bits(il, n_layer) and n_expert == 0
         p = "blk.%d." % il
         if n_expert > 0:
             t += [(p + "attn_norm.weight", F32, (n_embd,)),
-                  (p + "attn_q.weight", Q4_K, (n_embd, n_head * head_dim)),
-                  (p + "attn_k.weight", Q4_K, (n_embd, n_head_kv * head_dim)),
-                  (p + "attn_v.weight", Q4_K, (n_embd, n_head_kv * head_dim)),
-                  (p + "attn_output.weight", Q4_K, (n_head * head_dim, n_embd)),
+                  (p + "attn_q.weight", base, (n_embd, n_head * head_dim)),
+                  (p + "attn_k.weight", base, (n_embd, n_head_kv * head_dim)),
+                  (p + "attn_v.weight", base, (n_embd, n_head_kv * head_dim)),
+                  (p + "attn_output.weight", base, (n_head * head_dim, n_embd)),
                   (p + "ffn_norm.weight", F32, (n_embd,)),
                   (p + "ffn_gate_inp.weight", F32, (n_embd, n_expert)),
-                  (p + "ffn_gate_exps.weight", Q4_K, (n_embd, n_ff, n_expert)),
-                  (p + "ffn_down_exps.weight", Q4_K, (n_ff, n_embd, n_expert)),
-                  (p + "ffn_up_exps.weight", Q4_K, (n_embd, n_ff, n_expert))]
+                  (p + "ffn_gate_exps.weight", base, (n_embd, n_ff, n_expert)),
+                  (p + "ffn_down_exps.weight", base, (n_ff, n_embd, n_expert)),
+                  (p + "ffn_up_exps.weight", base, (n_embd, n_ff, n_expert))]
             continue
         t += [(p + "attn_norm.weight", F32, (n_embd,)),
-              (p + "attn_q.weight", Q4_K, (n_embd, n_head * head_dim)),
-              (p + "attn_k.weight", Q4_K, (n_embd, n_head_kv * head_dim)),
-              (p + "attn_v.weight", Q6_K if more else Q4_K, (n_embd, n_head_kv * head_dim)),
-              (p + "attn_output.weight", Q4_K, (n_head * head_dim, n_embd)),
+              (p + "attn_q.weight", base, (n_embd, n_head * head_dim)),
+              (p + "attn_k.weight", base, (n_embd, n_head_kv * head_dim)),
+              (p + "attn_v.weight", Q6_K if more else base, (n_embd, n_head_kv * head_dim)),
+              (p + "attn_output.weight", base, (n_head * head_dim, n_embd)),
               (p + "ffn_norm.weight", F32, (n_embd,)),
-              (p + "ffn_gate.weight", Q4_K, (n_embd, n_ff)),
-              (p + "ffn_up.weight", Q4_K, (n_embd, n_ff)),
-              (p + "ffn_down.weight", Q6_K if more else Q4_K, (n_ff, n_embd))]
-    t += [("output_norm.weight", F32, (n_embd,)), ("output.weight", Q4_K if n_expert > 0 else Q6_K, (n_embd, n_vocab))]
+              (p + "ffn_gate.weight", base, (n_embd, n_ff)),
+              (p + "ffn_up.weight", base, (n_embd, n_ff)),
+              (p + "ffn_down.weight", Q6_K if more else base, (n_ff, n_embd))]
+    t += [("output_norm.weight", F32, (n_embd,)), ("output.weight", base if n_expert > 0 else Q6_K, (n_embd, n_vocab))]
     return t
 
 
@@ -102,20 +103,25 @@ def random_blocks(ttype, n_blocks, rng, pool):
     if ttype == Q4_K:      # w = d*sc*n - dmin*m, sc,m ~ U[0,63], n ~ U[0,15]
         put_half(0, 0.02 / (31.5 * 4.6))
         put_half(2, 0.02 / (31.5 * 4.6) * 7.5)
+    elif ttype == Q5_K:    # the same with n ~ U[0,31]
+        put_half(0, 0.02 / (31.5 * 9.2))
+        put_half(2, 0.02 / (31.5 * 9.2) * 15.5)
     else:                  # Q6_K: w = d*sc*(q-32), sc int8
         put_half(208, 0.02 / (74.0 * 18.5))
     return raw
 
 
 def write_model(path, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=128256, n_ctx=8192,
-                rope_theta=500000.0, rms_eps=1e-5, seed=1234, n_expert=0, n_expert_used=0):
+                rope_theta=500000.0, rms_eps=1e-5, seed=1234, n_expert=0, n_expert_used=0, ftype="q4_k_m"):
+    """ftype: "q4_k_m" or "q5_k_m" - the tensor mix llama-quantize produces for that file type"""
     head_dim = n_embd // n_head
-    tensors = tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert)
+    base = {"q4_k_m": Q4_K, "q5_k_m": Q5_K}[ftype]
+    tensors = tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert, base)
     align = 32
     kvs = [
         _kv("general.architecture", T_STR, "llama"),
-        _kv("general.name", T_STR, "synthetic-llama-q4_k_m"),
-        _kv("general.file_type", T_U32, 15),    # LLAMA_FTYPE_MOSTLY_Q4_K_M
+        _kv("general.name", T_STR, "synthetic-llama-" + ftype),
+        _kv("general.file_type", T_U32, {"q4_k_m": 15, "q5_k_m": 17}[ftype]),    # LLAMA_FTYPE_MOSTLY_Q4_K_M / _Q5_K_M
         _kv("general.alignment", T_U32, align),
         _kv("llama.block_count", T_U32, n_layer),
         _kv("llama.context_length", T_U32, n_ctx),
@@ -172,7 +178,8 @@ if __name__ == "__main__":
     ap.add_argument("--vocab", type=int, default=128256)
     ap.add_argument("--experts", type=int, default=0, help="mixture of experts: number of experts (0 = dense)")
     ap.add_argument("--experts-used", type=int, default=2)
+    ap.add_argument("--ftype", default="q4_k_m", choices=["q4_k_m", "q5_k_m"])
     a = ap.parse_args()
     size = write_model(a.path, a.layers, a.embd, a.ff, a.heads, a.kv_heads, a.vocab, n_expert=a.experts,
-                       n_expert_used=a.experts_used if a.experts else 0)
+                       n_expert_used=a.experts_used if a.experts else 0, ftype=a.ftype)
     print("wrote %s: %.2f GB of tensor data" % (a.path, size / 1e9))

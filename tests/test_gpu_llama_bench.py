@@ -75,6 +75,25 @@ def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats
     return np.fromfile(out, dtype=np.float32)
 
 
+@pytest.mark.parametrize("n_prompt", [5, 40])
+def test_model_logits_q5_k_m(dev, tmp_path, n_prompt):
+    """A Q5_K_M-shaped file (Q5_K everywhere, Q6_K where llama-quantize uses more bits): the reference's runtime on the plug-in
+    reproduces its CPU backend's logits, so Q5_K products (GEMV for decode, the eight-rows-at-a-time path for the prompt) and
+    Q5_K rows of GET_ROWS stay on the device with the reference's arithmetic."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / "q5km.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048, ftype="q5_k_m")
+    cpu = _logits(model, 0, n_prompt, 4, str(tmp_path / "cpu.bin"))
+    dev_out = _logits(model, 99, n_prompt, 4, str(tmp_path / "dev.bin"))
+    assert cpu.shape == dev_out.shape and np.isfinite(dev_out).all()
+    assert orc.nmse(dev_out, cpu) < 2e-3
+
+
 def test_model_logits_async_loader(dev, tmp_path):
     """Without mmap the reference's loader uploads the weights in 1 MiB chunks from pinned buffers with set_tensor_async and
     fences the buffers with events (src/llama-model-loader.cpp:926-960, 1033-1046): chunks land at byte offsets inside tensors,

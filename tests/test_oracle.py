@@ -122,6 +122,14 @@ def _levels(t, W, K):
     if t == orc.Q4_K:
         qs = W.reshape(N, K // 256, 144)[:, :, 16:].reshape(N, K // 256, 4, 32)
         return np.concatenate([(qs & 15), (qs >> 4)], axis=3).astype(np.int32).reshape(N, K)
+    if t == orc.Q5_K:
+        blk = W.reshape(N, K // 256, 176)
+        qs = blk[:, :, 48:].reshape(N, K // 256, 4, 32)
+        qh = blk[:, :, 16:48].reshape(N, K // 256, 1, 32)
+        g = np.arange(4, dtype=np.uint8).reshape(1, 1, 4, 1)
+        lo = (qs & 15) | (((qh >> (2 * g)) & 1) << 4)        # sub-block 2g: bit 2g of qh
+        hi = (qs >> 4) | (((qh >> (2 * g + 1)) & 1) << 4)    # sub-block 2g + 1: bit 2g + 1
+        return np.concatenate([lo, hi], axis=3).astype(np.int32).reshape(N, K)
     blk = W.reshape(N, K // 256, 210)
     ql = blk[:, :, :128].reshape(N, -1, 2, 64)
     qh = blk[:, :, 128:192].reshape(N, -1, 2, 32)
