@@ -330,6 +330,9 @@ plane_store & planes() {
 // MI355_NO_TILES=1 keeps the packed rows only.  Below TILE_MIN_BATCH rows the second copy's 2 bytes per weight make the product
 // HBM-bound and the kernels that unpack the packed rows are quicker.
 constexpr int64_t TILE_MIN_BATCH = 192;
+// Q5_K has no tile kernel on packed rows and no matrix-core kernel for few rows: its images serve every batch above the GEMV's
+constexpr int64_t TILE_MIN_BATCH_Q5_K = 33;
+inline int64_t tile_min_batch(ggml_type t) { return t == GGML_TYPE_Q5_K ? TILE_MIN_BATCH_Q5_K : TILE_MIN_BATCH; }
 struct tile_store {
     std::mutex mu;
     struct entry { void * tiles; int64_t rows, K; };
@@ -337,7 +340,7 @@ struct tile_store {
     bool enabled = getenv("MI355_NO_TILES") == nullptr;
 
     const void * get(hipStream_t s, const ggml_tensor * w) {
-        if (!enabled || (w->type != GGML_TYPE_Q4_K && w->type != GGML_TYPE_Q6_K) || w->buffer == nullptr ||
+        if (!enabled || (w->type != GGML_TYPE_Q4_K && w->type != GGML_TYPE_Q5_K && w->type != GGML_TYPE_Q6_K) || w->buffer == nullptr ||
             w->buffer->usage != GGML_BACKEND_BUFFER_USAGE_WEIGHTS)
             return nullptr;
         std::lock_guard<std::mutex> lock(mu);
@@ -425,7 +428,7 @@ void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     if (size == 0) return;
-    if (tensor->type == GGML_TYPE_Q6_K || tensor->type == GGML_TYPE_Q4_K) {
+    if (tensor->type == GGML_TYPE_Q6_K || tensor->type == GGML_TYPE_Q4_K || tensor->type == GGML_TYPE_Q5_K) {
         MI355_HIP_OK(hipDeviceSynchronize());
         planes().drop(tensor->data, ggml_nbytes(tensor));   // rebuilt from the new contents on next use
         tiles().drop(tensor->data, ggml_nbytes(tensor));
@@ -480,7 +483,7 @@ bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, gg
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
     if (dst->type == GGML_TYPE_Q6_K) planes().drop(dst->data, ggml_nbytes(dst));
-    if (dst->type == GGML_TYPE_Q6_K || dst->type == GGML_TYPE_Q4_K) tiles().drop(dst->data, ggml_nbytes(dst));
+    if (dst->type == GGML_TYPE_Q6_K || dst->type == GGML_TYPE_Q4_K || dst->type == GGML_TYPE_Q5_K) tiles().drop(dst->data, ggml_nbytes(dst));
     MI355_HIP_OK(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyDeviceToDevice));
     MI355_HIP_OK(hipDeviceSynchronize());
     return true;
@@ -905,7 +908,7 @@ void backend_set_tensor_async(ggml_backend_t backend, ggml_tensor * tensor, cons
     backend_ctx * ctx = (backend_ctx *) backend->context;
     ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
     // the layout permutation goes through the staging buffer; a K-quant matrix may have int8 planes or tile images to forget
-    const bool has_images = tensor->type == GGML_TYPE_Q4_K &&
+    const bool has_images = (tensor->type == GGML_TYPE_Q4_K || tensor->type == GGML_TYPE_Q5_K) &&
                             (planes().any(tensor->data, ggml_nbytes(tensor)) || tiles().any(tensor->data, ggml_nbytes(tensor)));
     if (repack_of(tensor).yes || has_images || size == 0) {
         MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
@@ -1052,7 +1055,7 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
 bool is_q8k_tile_candidate(const ggml_tensor * mm) {
     const ggml_tensor * a = mm->src[0];
     const ggml_tensor * b = mm->src[1];
-    if (mm->op != GGML_OP_MUL_MAT || (a->type != GGML_TYPE_Q4_K && a->type != GGML_TYPE_Q6_K)) return false;
+    if (mm->op != GGML_OP_MUL_MAT || (a->type != GGML_TYPE_Q4_K && a->type != GGML_TYPE_Q5_K && a->type != GGML_TYPE_Q6_K)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
     if (b->ne[1] <= 32 || b->nb[1] % 16 != 0) return false;
     const int64_t K = a->ne[0];
@@ -1079,7 +1082,7 @@ bool feeds_q8k_tiles(const graph_walk & w, int i, const void * data, int64_t K, 
 
 // activation format of a K-quant tile product: tile images when the batch is large and the weights have (or can get) theirs
 int q8k_format_for(hipStream_t s, const ggml_tensor * mm) {
-    return mm->src[1]->ne[1] >= TILE_MIN_BATCH && tiles().get(s, mm->src[0]) != nullptr ? ACT_Q8KT : ACT_Q8K;
+    return mm->src[1]->ne[1] >= tile_min_batch(mm->src[0]->type) && tiles().get(s, mm->src[0]) != nullptr ? ACT_Q8KT : ACT_Q8K;
 }
 
 // A MUL_MAT_ID with few (token, expert slot) pairs streams each slot's expert through the GEMV on Q8_1 activations; with many
@@ -1280,17 +1283,22 @@ unsigned tiled_multi(backend_ctx * ctx, hipStream_t s, const graph_walk & w, con
     const ggml_tensor * b = w.nodes[idx[0]]->src[1];
     const int64_t K = b->ne[0], B = b->ne[1];
     const void * tl[3] = {nullptr, nullptr, nullptr};
-    int n_of[2] = {0, 0};   // Q4_K, Q6_K
+    const ggml_type kinds[3] = {GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K};
+    int n_of[3] = {0, 0, 0};
     for (int k = 0; k < n && k < 3; k++) {
         const ggml_tensor * mm = w.nodes[idx[k]];
         if (!is_q8k_tile_candidate(mm) || mm->src[1]->data != b->data || mm->src[1]->ne[0] != K || mm->src[1]->ne[1] != B || mm->src[1]->nb[1] != b->nb[1] ||
             mm->type != GGML_TYPE_F32 || mm->nb[0] != sizeof(float) || mm->nb[1] % sizeof(float) != 0 || q8k_format_for(s, mm) != ACT_Q8KT)
             continue;
         tl[k] = tiles().get(s, mm->src[0]);
-        if (tl[k]) n_of[mm->src[0]->type == GGML_TYPE_Q6_K]++;
+        if (tl[k])
+            for (int t = 0; t < 3; t++) n_of[t] += mm->src[0]->type == kinds[t];
     }
-    const ggml_type type = n_of[1] > n_of[0] ? GGML_TYPE_Q6_K : GGML_TYPE_Q4_K;
-    if (n_of[type == GGML_TYPE_Q6_K] < 2) return 0;
+    int best = 0;
+    for (int t = 1; t < 3; t++)
+        if (n_of[t] > n_of[best]) best = t;
+    const ggml_type type = kinds[best];
+    if (n_of[best] < 2) return 0;
     if (!ctx->cached(b->data, K, B, ACT_Q8KT)) {
         void * fresh = ctx->act_slot(mi355_act_q8k_tiled_bytes(K, B));
         MI355_K_OK(mi355_quantize_act_q8k_tiled(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
@@ -1759,7 +1767,8 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         return last;
     }
     // ---- runs of K-quant products on one activation (batch > 8): one per-super-block quantization
-    if (is_q8k_tile_candidate(node)) {
+    // (a Q5_K matrix without tile images - not in a weights buffer, or no memory for them - takes the generic path below)
+    if (is_q8k_tile_candidate(node) && !(node->src[0]->type == GGML_TYPE_Q5_K && q8k_format_for(s, node) != ACT_Q8KT)) {
         const ggml_tensor * b = node->src[1];
         const int64_t K = b->ne[0], B = b->ne[1];
         // MUL_MAT(gate) -> UNARY(SILU) -> MUL_MAT(up) -> MUL: the up product goes out with the gate product (it reads the same

@@ -56,6 +56,19 @@ __device__ __forceinline__ void wt_q6k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
     lo = le | (lo_ << 8);
 }
 
+// Q5_K: the four levels 0..31 in the bytes of `a` times the sub-block scale 0..63 -> P = 16 * hi + lo with hi <= 122, lo <= 15
+__device__ __forceinline__ void wt_q5k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
+    const wt_u16x2 s = {(unsigned short)sc, (unsigned short)sc};
+    const wt_u16x2 e = __builtin_bit_cast(wt_u16x2, a & 0x00FF00FFu);
+    const wt_u16x2 o = __builtin_bit_cast(wt_u16x2, (a >> 8) & 0x00FF00FFu);
+    const wt_u16x2 pe = e * s, po = o * s;
+    const wt_u16x2 four = {4, 4};
+    const u32 he = __builtin_bit_cast(u32, pe >> four), ho = __builtin_bit_cast(u32, po >> four);
+    const u32 le = __builtin_bit_cast(u32, pe) & 0x000F000Fu, lo_ = __builtin_bit_cast(u32, po) & 0x000F000Fu;
+    hi = (he & 0x00FF00FFu) | ((ho & 0x00FF00FFu) << 8);
+    lo = le | (lo_ << 8);
+}
+
 template <int TYPE>
 __global__ void __launch_bounds__(256) k_unpack_tiles(const uint8_t *__restrict__ W, int8_t *__restrict__ img, int64_t N, int64_t K, row_layout L) {
     const int64_t per_row = (K >> 8) * 8;
@@ -89,6 +102,48 @@ __global__ void __launch_bounds__(256) k_unpack_tiles(const uint8_t *__restrict_
                 a0[i] = wt_mul_bytes(nl, (u32)scl & 7u);
                 b1[i] = wt_mul_bytes(nh, (u32)sch >> 3);
                 b0[i] = wt_mul_bytes(nh, (u32)sch & 7u);
+            }
+        }
+        c0 = 4 * gl + (p & 1);
+        c1 = c0 + 2;
+        if (half == 0 && p == 0) {
+            uint8_t *e = aux + (sb * n_rb_pad + (row >> 4)) * W_AUX;
+            const int r = (int)(row & 15);
+            f16x8 m1, m64;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                int sc, mn;
+                q4k_scale_min(hdr[1], hdr[2], hdr[3], j, sc, mn);
+                if (!live) mn = 0;
+                m1[j] = (_Float16)(float)mn;
+                m64[j] = (_Float16)(float)(64 * mn);
+            }
+            *(f16x8 *)(e + r * 32) = m1;
+            *(f16x8 *)(e + r * 32 + 16) = m64;
+            *(float *)(e + 512 + r * 4) = live ? half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu)) : 0.0f;
+            *(float *)(e + 576 + r * 4) = live ? half_bits_to_float((unsigned short)(hdr[0] >> 16)) : 0.0f;
+        }
+    } else if constexpr (TYPE == MI355_Q5_K) {
+        // the Q4_K geometry (block_q5_K, ggml/src/ggml-common.h:296-308: header, qh[32] at 16, qs[128] at 48); the fifth bit of sub-block j
+        // is bit j of qh[l]; planes at radix 16
+        const uint8_t *blk = wrow + sb * Q5_K_BYTES;
+        const u32x4 q = load16(blk + 48 + (half * 2 + (p >> 1)) * 32 + (p & 1) * 16);
+        const u32x4 qh = load16(blk + 16 + (p & 1) * 16);
+        const u32x4 hdr = load16(blk);
+        const int gl = p >> 1, g = half * 2 + gl;
+        int scl, mnl, sch, mnh;
+        q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * g, scl, mnl);
+        q4k_scale_min(hdr[1], hdr[2], hdr[3], 2 * g + 1, sch, mnh);
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const u32 nl = (q[i] & 0x0F0F0F0Fu) | (((qh[i] >> (2 * g)) & 0x01010101u) << 4);
+                const u32 nh = ((q[i] >> 4) & 0x0F0F0F0Fu) | (((qh[i] >> (2 * g + 1)) & 0x01010101u) << 4);
+                u32 hi, lo;
+                wt_q5k_planes(nl, scl, hi, lo);
+                a1[i] = hi; a0[i] = lo;
+                wt_q5k_planes(nh, sch, hi, lo);
+                b1[i] = hi; b0[i] = lo;
             }
         }
         c0 = 4 * gl + (p & 1);
@@ -180,8 +235,8 @@ struct wt_launch {
 
 template <int TYPE>
 __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__restrict__ a_img, int64_t K, int64_t B) {
-    constexpr bool Q4 = TYPE == MI355_Q4_K;
-    constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
+    constexpr bool Q4 = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K;   // sub-block mins: the min term and its scale records
+    constexpr int RADIX_SHIFT = TYPE == MI355_Q4_K ? 3 : (TYPE == MI355_Q5_K ? 4 : 6);
     constexpr int NP = 2;                                                      // weight planes
     constexpr int W_AUX = wt_w_aux_bytes(TYPE);
     constexpr int STAGE = (NP * WT_BM + WT_BN) * 64;                           // bytes of one 64-element stage: plane(s), activations
@@ -538,12 +593,12 @@ int mi355_quantize_act_q8k_tiled(void *stream, const float *x, void *act, int64_
 }
 
 size_t mi355_kq_tiles_bytes(int type, int64_t rows, int64_t K) {
-    if (rows <= 0 || K <= 0 || K % QKK != 0 || (type != MI355_Q4_K && type != MI355_Q6_K)) return 0;
+    if (rows <= 0 || K <= 0 || K % QKK != 0 || (type != MI355_Q4_K && type != MI355_Q5_K && type != MI355_Q6_K)) return 0;
     return wt_weight_bytes(type, rows, K);
 }
 
 int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, int64_t rows, int64_t K) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "kq_unpack_tiles: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K, "kq_unpack_tiles: weight type %d is not a K-quant", type);
     MI355_REQUIRE(rows > 0 && K > 0 && K % QKK == 0, "kq_unpack_tiles: bad shape rows=%lld K=%lld", (long long)rows, (long long)K);
     const row_layout L = make_row_layout(type, K);
     MI355_REQUIRE(layout_aligned(W, L) && ((uintptr_t)tiles & 15) == 0, "kq_unpack_tiles: rows are not 16-byte aligned (K=%lld)", (long long)K);
@@ -551,6 +606,7 @@ int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, in
     MI355_REQUIRE((pieces + 255) / 256 < 0x7fffffff, "kq_unpack_tiles: too many pieces for one launch");
     const dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
     if (type == MI355_Q4_K) MI355_LAUNCH(k_unpack_tiles<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
+    else if (type == MI355_Q5_K) MI355_LAUNCH(k_unpack_tiles<MI355_Q5_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
     else MI355_LAUNCH(k_unpack_tiles<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
     return launch_status("k_unpack_tiles");
 }
@@ -589,7 +645,7 @@ size_t mi355_mul_mat_q8k_tiled_multi_ws_bytes(int n_mats, const int64_t *Ns, int
 
 int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
                                   void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", type);
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_q8k_tiled: 1 to 3 matrices per launch, got %d", n_mats);
     MI355_REQUIRE(K > 0 && B > 0 && K % QKK == 0, "mul_mat_q8k_tiled: bad shape K=%lld B=%lld (K must be a multiple of 256)", (long long)K, (long long)B);
     MI355_REQUIRE(act != nullptr && ((uintptr_t)act & 15) == 0, "mul_mat_q8k_tiled: the activation image is not 16-byte aligned");
@@ -624,6 +680,7 @@ int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi35
     }
     const dim3 grid((unsigned)L.n_tiles_padded, (unsigned)p.slices);
     if (type == MI355_Q4_K) MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
+    else if (type == MI355_Q5_K) MI355_LAUNCH(k_mmq_w<MI355_Q5_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
     else MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
     if (p.slices > 1)
         MI355_LAUNCH(k_wt_split_sum, dim3((unsigned)((Ns[0] * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B,

@@ -75,11 +75,12 @@ def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats
     return np.fromfile(out, dtype=np.float32)
 
 
-@pytest.mark.parametrize("n_prompt", [5, 40])
+@pytest.mark.parametrize("n_prompt", [5, 20, 40, 256])
 def test_model_logits_q5_k_m(dev, tmp_path, n_prompt):
     """A Q5_K_M-shaped file (Q5_K everywhere, Q6_K where llama-quantize uses more bits): the reference's runtime on the plug-in
-    reproduces its CPU backend's logits, so Q5_K products (GEMV for decode, the eight-rows-at-a-time path for the prompt) and
-    Q5_K rows of GET_ROWS stay on the device with the reference's arithmetic."""
+    reproduces its CPU backend's logits, so Q5_K products (GEMV for decode and up to eight rows, eight rows at a time up to 32, the
+    wide-tile GEMM on Q5_K tile images from 33 rows on) and Q5_K rows of GET_ROWS stay on the device with the reference's
+    arithmetic."""
     if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
         pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))

@@ -258,6 +258,7 @@ def test_unaligned_rows_fallback(dev, name, t):
 
 
 KQ_TYPES = [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q6_K)]
+TILED_TYPES = [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q5_K, orc.Q6_K)]   # types with tile images for the wide-tile GEMM
 
 
 def _tile_off(row, k, K):
@@ -295,7 +296,7 @@ def test_quantize_q8k_tiled_bit_exact(dev, K, B):
         assert np.array_equal(want, orc.quantize("ref", orc.Q8_K, x).reshape(B, nsb, 292))
 
 
-@pytest.mark.parametrize("name,t", KQ_TYPES)
+@pytest.mark.parametrize("name,t", TILED_TYPES)
 @pytest.mark.parametrize("N,K,B", [(512, 4096, 64), (384, 2048, 512), (130, 2048, 33), (128, 14336, 100), (200, 2048, 77), (1000, 6144, 300)])
 @pytest.mark.parametrize("split", [False, True])
 def test_mmq_tiled_matches_oracle(dev, name, t, N, K, B, split):
@@ -317,11 +318,12 @@ def test_mmq_tiled_matches_oracle(dev, name, t, N, K, B, split):
     assert orc.nmse(got[:Bt, :Nt], orc.mul_mat("cpu", t, Wq[:Nt], x[:Bt])) < 1e-9
     # the last rows and columns (partial tiles)
     assert orc.nmse(got[B - 5:, N - 7:], orc.mul_mat("cpu", t, Wq[N - 7:], x[B - 5:])) < 1e-9
-    old = torch.empty((B, N), dtype=torch.float32, device=dev)
-    a2 = mi355.quantize_act_q8k(_to_dev(dev, x))
-    mi355.check(mi355.load().mi355_mul_mat_q8k(None, t, Wd.data_ptr(), a2.data_ptr(), old.data_ptr(), N, K, B, N))
-    torch.cuda.synchronize()
-    assert orc.nmse(got, old.cpu().numpy()) < 1e-12      # same integer sums, f32 summation order only
+    if t != orc.Q5_K:   # the 64 x 128 tile kernel on packed rows does not unpack Q5_K
+        old = torch.empty((B, N), dtype=torch.float32, device=dev)
+        a2 = mi355.quantize_act_q8k(_to_dev(dev, x))
+        mi355.check(mi355.load().mi355_mul_mat_q8k(None, t, Wd.data_ptr(), a2.data_ptr(), old.data_ptr(), N, K, B, N))
+        torch.cuda.synchronize()
+        assert orc.nmse(got, old.cpu().numpy()) < 1e-12      # same integer sums, f32 summation order only
     if orc.ref is not None:
         assert orc.nmse(got, orc.mul_mat("ref", t, Wq, x)) <= 5e-4      # tests/test-backend-ops.cpp:1916
 
@@ -364,7 +366,7 @@ def test_fused_producers_write_tile_images(dev, name, t):
     assert np.array_equal(a3.cpu().numpy()[sel], a4.cpu().numpy()[sel])
 
 
-@pytest.mark.parametrize("name,t", KQ_TYPES)
+@pytest.mark.parametrize("name,t", TILED_TYPES)
 @pytest.mark.parametrize("Ns,K,B", [((14336, 14336), 4096, 512),       # gate + up of an 8B llama: 896 tiles
                                     ((4096, 1024, 1024), 4096, 512),    # Q, K, V: 192 tiles in one round
                                     ((8200, 8300, 130), 2048, 300),     # ragged rows and batch
