@@ -92,6 +92,9 @@ int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64
  * Up to 4 activation rows (8 where the matrix-core kernels do not support the product) run the
  * bandwidth-bound GEMV (per-block integer dots of the weights against Q8_1 activations), up to 32
  * the weight-streaming matrix-core kernel (mi355_mul_mat_skinny), larger B the int8-MFMA tile kernels.
+ * Q5_K (block_q5_K, ggml/src/ggml-common.h:296-308; ggml_vec_dot_q5_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6859-7592) has the
+ * GEMV for up to 8 rows and the wide-tile GEMM on tile images (mi355_kq_unpack_tiles + mi355_mul_mat_q8k_tiled) for batches;
+ * this entry point, which has no tile image to go by, runs Q5_K batches through the GEMV eight rows at a time.
  * `ws` is scratch of at least mi355_mul_mat_ws_bytes(K, B) bytes. */
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
@@ -120,7 +123,7 @@ size_t mi355_mul_mat_q_ws_bytes(int64_t N, int64_t K, int64_t B);
 int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
                        int64_t dst_stride, void *ws, size_t ws_bytes);
 
-/* MUL_MAT for 1..32 activation rows as one weight-streaming launch on the int8 matrix cores (Q4_0, Q8_0, Q4_K; K a
+/* MUL_MAT for 1..32 activation rows as one weight-streaming launch on the int8 matrix cores (Q4_0, Q8_0, Q4_K, Q6_K; K a
  * multiple of 256; 16-byte aligned rows: mi355_mul_mat_skinny_supported says whether a product qualifies).  Same operands
  * as mi355_mul_mat_vec_q (`act` from mi355_quantize_act) plus an optional residual added to the result (may alias dst).
  * It is what mi355_mul_mat uses between the batch-1 kernels and the tile kernels (ggml's MUL_MAT with src1->ne[1] of
@@ -183,9 +186,11 @@ int mi355_mul_mat_q8k_planes_ws(void *stream, int type, const void *planes, cons
  *                (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516), mi355_act_q8k_tiled_bytes(k, nrows) bytes;
  *   weights:     mi355_kq_unpack_tiles - the two int8 planes of mi355_kq_unpack_planes (dequantize_row_q4_K / _q6_K,
  *                ggml/src/ggml-quants.c:1280-1302, 1690-1719) plus per-super-block d, dmin and mins, written once per
- *                weight matrix, mi355_kq_tiles_bytes(type, rows, K) bytes (about 2 bytes per weight).
+ *                weight matrix, mi355_kq_tiles_bytes(type, rows, K) bytes (about 2 bytes per weight).  Also Q5_K
+ *                (dequantize_row_q5_K, :1482-1507): sub-block scale times level 0..31 = 16 * hi + lo.
  * mi355_mul_mat_q8k_tiled computes what mi355_mul_mat_q8k_add computes (same integer sums: ggml_vec_dot_q4_K_q8_K /
- * ggml_vec_dot_q6_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6817-6848, 8262-8283; f32 summation order may differ).
+ * ggml_vec_dot_q6_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6817-6848, 8262-8283; f32 summation order may differ), and for
+ * Q5_K the integer sums of ggml_vec_dot_q5_K_q8_K (:7539-7592).
  * ws: optional workspace of mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) bytes for the split along K of products with few
  * tiles (NULL or too small: unsplit).  No counterpart in the reference (its CUDA backend unpacks in the tile loaders,
  * ggml/src/ggml-cuda/mmq.cuh). */
@@ -230,11 +235,11 @@ typedef struct mi355_gemv_mat {
 int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B);
 
 /* Integer sub-block dots, for parity checking the kernels' inner products bit-for-bit
- * against ggml_vec_dot_q4_0_q8_0 / q8_0_q8_0 / q4_K_q8_K / q6_K_q8_K
- * (ggml/src/ggml-cpu/ggml-cpu-quants.c:2492-2506, 3919-3927, 6817-6848, 8262-8283).
+ * against ggml_vec_dot_q4_0_q8_0 / q8_0_q8_0 / q4_K_q8_K / q5_K_q8_K / q6_K_q8_K
+ * (ggml/src/ggml-cpu/ggml-cpu-quants.c:2492-2506, 3919-3927, 6817-6848, 7539-7592, 8262-8283).
  * a: ONE activation row in the split layout written by mi355_quantize_act (the same bytes
  * the GEMV reads).  out: int32 [N][k/g], g = 32 (16 for Q6_K); the weight level has its
- * fixed offset removed (Q4_0: nibble-8, Q6_K: q-32, Q4_K: nibble). */
+ * fixed offset removed (Q4_0: nibble-8, Q6_K: q-32, Q4_K: nibble, Q5_K: level 0..31). */
 int mi355_block_dots_q8_1(void *stream, int type, const void *W, const void *a, int32_t *out, int64_t N, int64_t K);
 
 /* MUL_MAT_ID ------------------------------------------------------------------------ *
@@ -312,8 +317,8 @@ int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
  * emits (src/llama.cpp:157-199; ggml_compute_forward_dup_f32, ggml-cpu.c:3519-3830), with the row taken from device
  * memory so that a captured launch sequence does not change as the cache fills. */
 int mi355_set_rows(void *stream, const mi355_tensor *src, const int32_t *rows, const mi355_tensor *dst);
-/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, or whole quantized rows (Q4_0, Q8_0, Q4_K, Q6_K in the
- * device row layout, nb[1] = row bytes; dequantize_row_*, ggml-quants.c:255-273, 349-363, 1280-1302, 1690-1719), ids i32
+/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, or whole quantized rows (Q4_0, Q8_0, Q4_K, Q5_K, Q6_K in the
+ * device row layout, nb[1] = row bytes; dequantize_row_*, ggml-quants.c:255-273, 349-363, 1280-1302, 1482-1507, 1690-1719), ids i32
  * [n, b2, b3]; dst f32 */
 int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ids, const mi355_tensor *dst);
 /* ggml_compute_forward_soft_max_f32 (ggml-cpu.c:8959-9055): mask f32 or f16 or NULL */
