@@ -26,8 +26,8 @@ extern "C" {
 #define MI355_ERR_WORKSPACE -3  /* workspace too small */
 
 enum mi355_type {
-    MI355_F32 = 0, MI355_F16 = 1, MI355_Q4_0 = 2, MI355_Q8_0 = 8, MI355_Q8_1 = 9,
-    MI355_Q4_K = 12, MI355_Q5_K = 13, MI355_Q6_K = 14, MI355_I32 = 26,
+    MI355_F32 = 0, MI355_F16 = 1, MI355_Q4_0 = 2, MI355_Q4_1 = 3, MI355_Q5_0 = 6, MI355_Q5_1 = 7, MI355_Q8_0 = 8, MI355_Q8_1 = 9,
+    MI355_Q4_K = 12, MI355_Q5_K = 13, MI355_Q6_K = 14, MI355_IQ4_NL = 20, MI355_I32 = 26,
 };
 
 /* Library / device ------------------------------------------------------------------ */
@@ -58,11 +58,14 @@ int mi355_probe_lds_fill(void *stream, const void *src, int64_t src_bytes, int64
  * Quantized weight rows are kept in HBM in a per-row "device layout" that makes every
  * load a 16-byte aligned, coalesced access:
  *   Q4_K, Q5_K : unchanged (144- and 176-byte super-blocks are already 16-byte multiples)
- *   Q4_0 : [nb x 16 B nibbles][nb x fp16 d]
+ *   Q4_0, IQ4_NL : [nb x 16 B nibbles][nb x fp16 d]
+ *   Q4_1 : [nb x 16 B nibbles][nb x {fp16 d, fp16 m}]
+ *   Q5_0 : [nb x 16 B nibbles][nb x 4 B fifth bits][nb x fp16 d]
+ *   Q5_1 : [nb x 16 B nibbles][nb x 4 B fifth bits][nb x {fp16 d, fp16 m}]
  *   Q8_0 : [nb x 32 B int8   ][nb x fp16 d]
  *   Q6_K : [nb x 128 B ql][nb x 64 B qh][nb x 16 B scales][nb x fp16 d]
  * A row occupies exactly the same number of bytes as in the reference's block layout
- * (ggml/src/ggml-common.h:161-166, 203-208, 279-290, 314-320); the mapping is a byte
+ * (ggml/src/ggml-common.h:161-208, 279-290, 314-320, 399-404); the mapping is a byte
  * permutation inside each row.  These two entry points apply it / undo it for the byte
  * range [offset, offset+size) of a tensor of `nrows` rows of `k` elements, so partial
  * uploads and read-back return the reference's bytes
@@ -95,6 +98,10 @@ int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64
  * Q5_K (block_q5_K, ggml/src/ggml-common.h:296-308; ggml_vec_dot_q5_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6859-7592) has the
  * GEMV for up to 8 rows and the wide-tile GEMM on tile images (mi355_kq_unpack_tiles + mi355_mul_mat_q8k_tiled) for batches;
  * this entry point, which has no tile image to go by, runs Q5_K batches through the GEMV eight rows at a time.
+ * Q4_1, Q5_0, Q5_1 and IQ4_NL (ggml/src/ggml-common.h:168-201, 399-404; ggml_vec_dot_q4_1_q8_1, _q5_0_q8_0, _q5_1_q8_1 and
+ * _iq4_nl_q8_0, ggml/src/ggml-cpu/ggml-cpu-quants.c:2511, 2804, 3159, 11188) have the single-matrix GEMV and batches in the
+ * same eight-rows-at-a-time form; the launches that take several matrices or fuse an epilogue are built for Q4_0, Q8_0, Q4_K,
+ * Q5_K and Q6_K only.
  * `ws` is scratch of at least mi355_mul_mat_ws_bytes(K, B) bytes. */
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,

@@ -14,7 +14,7 @@
 //  * buffer set/get_tensor synchronise the device first, because the scheduler may read a
 //    result right after an asynchronous graph_compute (ggml/src/ggml-backend.cpp:243-252).
 //
-// Quantized tensors of type Q4_0 / Q8_0 / Q6_K live in HBM in the 16-byte-aligned row layout
+// Quantized tensors of type Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / Q8_0 / Q6_K live in HBM in the 16-byte-aligned row layout
 // described in mi355_kernels.h; set_tensor applies that byte permutation and get_tensor
 // undoes it, so every caller sees the reference's bytes.
 
@@ -50,8 +50,14 @@
 namespace {
 
 // ------------------------------------------------------------------------------- helpers
-bool is_repacked_type(ggml_type t) { return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K; }
-bool is_weight_type(ggml_type t) { return is_repacked_type(t) || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K; }
+// types whose products the fused launches (several matrices per launch, epilogues, matrix-core kernels) are built for ...
+bool is_fused_weight_type(ggml_type t) {
+    return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K;
+}
+// ... and those served one product at a time by mi355_mul_mat / mi355_mul_mat_id / mi355_get_rows
+bool is_plain_weight_type(ggml_type t) { return t == GGML_TYPE_Q4_1 || t == GGML_TYPE_Q5_0 || t == GGML_TYPE_Q5_1 || t == GGML_TYPE_IQ4_NL; }
+bool is_repacked_type(ggml_type t) { return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K || is_plain_weight_type(t); }
+bool is_weight_type(ggml_type t) { return is_fused_weight_type(t) || is_plain_weight_type(t); }
 
 int to_mi355_type(ggml_type t) {
     switch (t) {
@@ -59,6 +65,10 @@ int to_mi355_type(ggml_type t) {
         case GGML_TYPE_F16: return MI355_F16;
         case GGML_TYPE_I32: return MI355_I32;
         case GGML_TYPE_Q4_0: return MI355_Q4_0;
+        case GGML_TYPE_Q4_1: return MI355_Q4_1;
+        case GGML_TYPE_Q5_0: return MI355_Q5_0;
+        case GGML_TYPE_Q5_1: return MI355_Q5_1;
+        case GGML_TYPE_IQ4_NL: return MI355_IQ4_NL;
         case GGML_TYPE_Q8_0: return MI355_Q8_0;
         case GGML_TYPE_Q4_K: return MI355_Q4_K;
         case GGML_TYPE_Q5_K: return MI355_Q5_K;
@@ -400,7 +410,7 @@ void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) bu
 // number of rows / elements per row of a tensor whose rows are contiguous blocks
 int64_t tensor_nrows(const ggml_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
 
-// Q4_0, Q8_0 and Q6_K tensors live in the device row layout, which is defined by the rows of the tensor that owns the memory: a
+// Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0 and Q6_K tensors live in the device row layout, which is defined by the rows of the tensor that owns the memory: a
 // view (a slice of experts, a permuted or 1-D view of a cache) addresses bytes of that tensor, so transfers through a view go
 // through the owner's layout at the view's byte offset.
 struct repack_target {
@@ -1042,7 +1052,7 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
     // kernels; from there to 32: the weight-streaming matrix-core kernel)
     const ggml_tensor * a = mm->src[0];
     const ggml_tensor * b = mm->src[1];
-    if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
+    if (mm->op != GGML_OP_MUL_MAT || !is_fused_weight_type(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
     if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
     if (a->type == GGML_TYPE_Q5_K && b->ne[1] > 8) return false;    // Q5_K: the GEMV only (up to eight rows); more rows take the generic path
@@ -1335,7 +1345,7 @@ prefill_qkv match_prefill_qkv(const graph_walk & w, int i) {
     const ggml_tensor * b = mq->src[1];
     const int64_t B = b->ne[1];
     auto product_ok = [&](const ggml_tensor * m, int idx) {
-        return m->op == GGML_OP_MUL_MAT && is_weight_type(m->src[0]->type) && m->src[0]->ne[2] == 1 && m->src[0]->ne[3] == 1 && m->src[1] == b &&
+        return m->op == GGML_OP_MUL_MAT && is_fused_weight_type(m->src[0]->type) && m->src[0]->ne[2] == 1 && m->src[0]->ne[3] == 1 && m->src[1] == b &&
                b->ne[2] == 1 && b->ne[3] == 1 && ggml_is_contiguous(m) && m->type == GGML_TYPE_F32 && w.sole_use(idx);
     };
     // the ROPE that reads product m, directly or through a RESHAPE nobody else reads

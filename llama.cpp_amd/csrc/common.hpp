@@ -23,14 +23,16 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int WAVE = 64;
 
-// ---- block geometry (ggml/src/ggml-common.h:161-166, 203-221, 279-290, 296-308, 314-320)
-constexpr int QK = 32;     // elements per Q4_0 / Q8_0 / Q8_1 block
+// ---- block geometry (ggml/src/ggml-common.h:161-221, 279-290, 296-308, 314-320, 399-404)
+constexpr int QK = 32;     // elements per Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / Q8_0 / Q8_1 block
 constexpr int QKK = 256;   // elements per K-quant super-block
 constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q8_1_BYTES = 36, Q4_K_BYTES = 144, Q5_K_BYTES = 176, Q6_K_BYTES = 210;
+constexpr int Q4_1_BYTES = 20, Q5_0_BYTES = 22, Q5_1_BYTES = 24, IQ4_NL_BYTES = 18;
 
 __host__ __device__ inline int type_block_elems(int t) {
     switch (t) {
         case MI355_Q4_0: case MI355_Q8_0: case MI355_Q8_1: return QK;
+        case MI355_Q4_1: case MI355_Q5_0: case MI355_Q5_1: case MI355_IQ4_NL: return QK;
         case MI355_Q4_K: case MI355_Q5_K: case MI355_Q6_K: return QKK;
         case MI355_F32: case MI355_F16: case MI355_I32: return 1;
         default: return 0;
@@ -39,6 +41,10 @@ __host__ __device__ inline int type_block_elems(int t) {
 __host__ __device__ inline int type_block_bytes(int t) {
     switch (t) {
         case MI355_Q4_0: return Q4_0_BYTES;
+        case MI355_Q4_1: return Q4_1_BYTES;
+        case MI355_Q5_0: return Q5_0_BYTES;
+        case MI355_Q5_1: return Q5_1_BYTES;
+        case MI355_IQ4_NL: return IQ4_NL_BYTES;
         case MI355_Q8_0: return Q8_0_BYTES;
         case MI355_Q8_1: return Q8_1_BYTES;
         case MI355_Q4_K: return Q4_K_BYTES;
@@ -49,9 +55,27 @@ __host__ __device__ inline int type_block_bytes(int t) {
         default: return 0;
     }
 }
-__host__ __device__ inline bool is_weight_type(int t) {
+// types the kernels that choose the weight type at run time (several matrices per launch, fused epilogues) are built for
+__host__ __device__ inline bool is_fused_weight_type(int t) {
     return t == MI355_Q4_0 || t == MI355_Q8_0 || t == MI355_Q4_K || t == MI355_Q5_K || t == MI355_Q6_K;
 }
+// ... and those served by the single-matrix kernels, whose type is a template parameter
+__host__ __device__ inline bool is_weight_type(int t) {
+    return is_fused_weight_type(t) || t == MI355_Q4_1 || t == MI355_Q5_0 || t == MI355_Q5_1 || t == MI355_IQ4_NL;
+}
+// Expands X(TYPE) for the weight type t (checked with is_weight_type before).
+#define MI355_WEIGHT_TYPE_SWITCH(t, X)            \
+    switch (t) {                                  \
+        case MI355_Q4_0: X(MI355_Q4_0) break;     \
+        case MI355_Q4_1: X(MI355_Q4_1) break;     \
+        case MI355_Q5_0: X(MI355_Q5_0) break;     \
+        case MI355_Q5_1: X(MI355_Q5_1) break;     \
+        case MI355_IQ4_NL: X(MI355_IQ4_NL) break; \
+        case MI355_Q8_0: X(MI355_Q8_0) break;     \
+        case MI355_Q4_K: X(MI355_Q4_K) break;     \
+        case MI355_Q5_K: X(MI355_Q5_K) break;     \
+        default: X(MI355_Q6_K) break;             \
+    }
 
 // ---- activation workspace: int8 q[nrows][k] then {float d; int sum;} ds[nrows][k/32]
 struct act_ds {

@@ -403,7 +403,7 @@ __global__ void __launch_bounds__(64) k_block_dots(const uint8_t *__restrict__ W
         const typename T::act A = T::load_a(aq, ads, cc);
         const chunk_dots d = T::dots(w, A);
         if (!live) continue;
-        if constexpr (TYPE == MI355_Q4_0 || TYPE == MI355_Q8_0) {
+        if constexpr (T::CHUNK == 32 && TYPE != MI355_Q6_K) {   // one 32-element block per chunk
             out[row * ngran + c] = d.i0;
         } else if constexpr (TYPE == MI355_Q4_K || TYPE == MI355_Q5_K) {   // chunk c = sub-blocks 2c and 2c+1 of the row
             out[row * ngran + 2 * c] = d.i0;
@@ -487,8 +487,8 @@ static void launch_single_cols(int rpw, int64_t B, hipStream_t s, const gemv_ite
     }
 }
 
-static int check_gemv_args(const char *who, int type, const void *W, int64_t N, int64_t K, int64_t dst_stride) {
-    MI355_REQUIRE(is_weight_type(type), "%s: unsupported weight type %d", who, type);
+static int check_gemv_args(const char *who, int type, const void *W, int64_t N, int64_t K, int64_t dst_stride, bool fused_only = false) {
+    MI355_REQUIRE(fused_only ? is_fused_weight_type(type) : is_weight_type(type), "%s: unsupported weight type %d", who, type);
     MI355_REQUIRE(N > 0 && K > 0 && K < (int64_t(1) << 30), "%s: bad shape N=%lld K=%lld", who, (long long)N, (long long)K);
     MI355_REQUIRE(K % type_block_elems(type) == 0, "%s: K=%lld is not a multiple of the block size", who, (long long)K);
     MI355_REQUIRE(dst_stride >= N, "%s: dst_stride < N", who);
@@ -514,6 +514,17 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_vec_q: activation workspace is not 16-byte aligned");
     int64_t total_rows = 0;
     bool aligned = true;
+    if (n_mats > 1) {   // the launch that walks several matrices chooses the type at run time among the fused set only
+        bool fused = true;
+        for (int i = 0; i < n_mats; i++) fused = fused && is_fused_weight_type(mats[i].type);
+        if (!fused) {
+            for (int i = 0; i < n_mats; i++) {
+                int rc = mi355_mul_mat_vec_q_multi(stream, 1, mats + i, act, K, B);
+                if (rc != MI355_OK) return rc;
+            }
+            return MI355_OK;
+        }
+    }
     for (int i = 0; i < n_mats; i++) {
         MI355_REQUIRE(is_weight_type(mats[i].type) && K > 0 && K % type_block_elems(mats[i].type) == 0, "mul_mat_vec_q: unsupported type %d or K=%lld not a multiple of its block size", mats[i].type, (long long)K);
         aligned = aligned && layout_aligned(mats[i].W, make_row_layout(mats[i].type, K));
@@ -577,13 +588,9 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + B * K);
     if (n_mats == 1) {
-        switch (mats[0].type) {
-            case MI355_Q4_0: launch_single_cols<MI355_Q4_0>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
-            case MI355_Q8_0: launch_single_cols<MI355_Q8_0>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
-            case MI355_Q4_K: launch_single_cols<MI355_Q4_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
-            case MI355_Q5_K: launch_single_cols<MI355_Q5_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
-            default: launch_single_cols<MI355_Q6_K>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K); break;
-        }
+#define MI355_SINGLE_LAUNCH(TY) launch_single_cols<TY>(rpw, B, s, b.it[0], (unsigned)groups, aq, ads, (int)K);
+        MI355_WEIGHT_TYPE_SWITCH(mats[0].type, MI355_SINGLE_LAUNCH)
+#undef MI355_SINGLE_LAUNCH
         return launch_status("k_gemv_q");
     }
     switch (B) {
@@ -622,7 +629,7 @@ static int vec_q_rope_impl(void *stream, int n_mats, const mi355_gemv_rope_mat *
     for (int i = 0; i < 4; i++) {
         const mi355_gemv_rope_mat &m = mats[i < n_mats ? i : 0];
         if (i < n_mats) {
-            int rc = check_gemv_args("mul_mat_vec_q_rope", m.type, m.W, m.N, K, m.N);
+            int rc = check_gemv_args("mul_mat_vec_q_rope", m.type, m.W, m.N, K, m.N, true);
             if (rc != MI355_OK) return rc;
             MI355_REQUIRE(m.epilogue >= MI355_EPI_STORE && m.epilogue <= MI355_EPI_CACHE && m.dst != nullptr && m.N % 2 == 0,
                           "mul_mat_vec_q_rope: bad epilogue %d, missing destination or odd row count", m.epilogue);
@@ -735,9 +742,9 @@ int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, in
     MI355_REQUIRE(B >= 1 && B <= 4, "ffn_gate_up_swiglu: batch %lld outside 1..4", (long long)B);
     MI355_REQUIRE(N > 0 && N % 32 == 0 && out_stride >= N, "ffn_gate_up_swiglu: N=%lld must be a positive multiple of 32 and fit the row stride", (long long)N);
     MI355_REQUIRE(((uintptr_t)act & 15) == 0 && ((uintptr_t)act_out & 15) == 0 && counters != nullptr, "ffn_gate_up_swiglu: misaligned or missing operands");
-    int rc = check_gemv_args("ffn_gate_up_swiglu", type_gate, w_gate, N, K, out_stride);
+    int rc = check_gemv_args("ffn_gate_up_swiglu", type_gate, w_gate, N, K, out_stride, true);
     if (rc != MI355_OK) return rc;
-    rc = check_gemv_args("ffn_gate_up_swiglu", type_up, w_up, N, K, out_stride);
+    rc = check_gemv_args("ffn_gate_up_swiglu", type_up, w_up, N, K, out_stride, true);
     if (rc != MI355_OK) return rc;
     const int64_t per = N / 8;   // groups per matrix: 4 waves x 2 rows
     MI355_REQUIRE(2 * per < 0x7fffffff, "ffn_gate_up_swiglu: too many rows for one launch");
@@ -798,13 +805,9 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
     const act_ds *ads = (const act_ds *)(aq + nb1 * T * K);
     if (!layout_aligned(as, L)) {
         const dim3 ugrid((unsigned)N, (unsigned)(n_used * T));
-        switch (type) {
-            case MI355_Q4_0: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q4_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-            case MI355_Q8_0: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q8_0>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-            case MI355_Q4_K: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q4_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-            case MI355_Q5_K: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q5_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-            default: MI355_LAUNCH(k_gemv_id_unaligned<MI355_Q6_K>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L); break;
-        }
+#define MI355_ID_UNALIGNED_LAUNCH(TY) MI355_LAUNCH(k_gemv_id_unaligned<TY>, ugrid, dim3(64), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, L);
+        MI355_WEIGHT_TYPE_SWITCH(type, MI355_ID_UNALIGNED_LAUNCH)
+#undef MI355_ID_UNALIGNED_LAUNCH
         return launch_status("k_gemv_id_unaligned");
     }
     const int rpw = pick_rpw(N * n_used) > 2 ? 2 : pick_rpw(N * n_used);
@@ -816,13 +819,7 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
     else if (lds) MI355_LAUNCH((k_gemv_id<TY, 2, true>), grid, dim3(256), lds, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
     else if (rpw == 1) MI355_LAUNCH((k_gemv_id<TY, 1, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1); \
     else MI355_LAUNCH((k_gemv_id<TY, 2, false>), grid, dim3(256), 0, s, (const uint8_t *)as, aq, ads, ids, ids_stride, dst, N, (int)K, n_expert, n_used, nb1);
-    switch (type) {
-        case MI355_Q4_0: MI355_ID_LAUNCH(MI355_Q4_0) break;
-        case MI355_Q8_0: MI355_ID_LAUNCH(MI355_Q8_0) break;
-        case MI355_Q4_K: MI355_ID_LAUNCH(MI355_Q4_K) break;
-        case MI355_Q5_K: MI355_ID_LAUNCH(MI355_Q5_K) break;
-        default: MI355_ID_LAUNCH(MI355_Q6_K) break;
-    }
+    MI355_WEIGHT_TYPE_SWITCH(type, MI355_ID_LAUNCH)
 #undef MI355_ID_LAUNCH
     return launch_status("k_gemv_id");
 }
@@ -834,13 +831,9 @@ int mi355_block_dots_q8_1(void *stream, int type, const void *W, const void *a, 
     const int8_t *aq = (const int8_t *)a;
     const act_ds *ads = (const act_ds *)(aq + K);
     const dim3 grid((unsigned)N);
-    switch (type) {
-        case MI355_Q4_0: MI355_LAUNCH(k_block_dots<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-        case MI355_Q8_0: MI355_LAUNCH(k_block_dots<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-        case MI355_Q4_K: MI355_LAUNCH(k_block_dots<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-        case MI355_Q5_K: MI355_LAUNCH(k_block_dots<MI355_Q5_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-        default: MI355_LAUNCH(k_block_dots<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K); break;
-    }
+#define MI355_BLOCK_DOTS_LAUNCH(TY) MI355_LAUNCH(k_block_dots<TY>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, out, N, (int)K);
+    MI355_WEIGHT_TYPE_SWITCH(type, MI355_BLOCK_DOTS_LAUNCH)
+#undef MI355_BLOCK_DOTS_LAUNCH
     return launch_status("k_block_dots");
 }
 

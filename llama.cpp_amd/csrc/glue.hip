@@ -440,13 +440,9 @@ int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *id
         const row_layout L = make_row_layout(src->type, K);
         MI355_REQUIRE((int64_t)src->nb[1] == L.row_bytes, "get_rows: quantized rows must be whole and contiguous");
         hipStream_t s = (hipStream_t)stream;
-        switch (src->type) {
-            case MI355_Q4_0: MI355_LAUNCH(k_get_rows_q<MI355_Q4_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-            case MI355_Q8_0: MI355_LAUNCH(k_get_rows_q<MI355_Q8_0>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-            case MI355_Q4_K: MI355_LAUNCH(k_get_rows_q<MI355_Q4_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-            case MI355_Q5_K: MI355_LAUNCH(k_get_rows_q<MI355_Q5_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-            default: MI355_LAUNCH(k_get_rows_q<MI355_Q6_K>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L); break;
-        }
+#define MI355_GET_ROWS_LAUNCH(TY) MI355_LAUNCH(k_get_rows_q<TY>, grid, block, 0, s, to_tens(src), to_tens(ids), to_tens(dst), n, L);
+        MI355_WEIGHT_TYPE_SWITCH(src->type, MI355_GET_ROWS_LAUNCH)
+#undef MI355_GET_ROWS_LAUNCH
         return launch_status("k_get_rows_q");
     }
     if (src->type == MI355_F32) MI355_LAUNCH(k_get_rows<float>, grid, block, 0, (hipStream_t)stream, to_tens(src), to_tens(ids), to_tens(dst), n);

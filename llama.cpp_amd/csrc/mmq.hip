@@ -496,7 +496,7 @@ extern "C" int mi355_mul_mat_q(void *stream, int type, const void *W, const void
 
 extern "C" int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
                                   int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(is_weight_type(type), "mul_mat_q: unsupported weight type %d", type);
+    MI355_REQUIRE(type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q: unsupported weight type %d", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_q: K=%lld is not a multiple of the block size", (long long)K);
     MI355_REQUIRE(dst_stride >= N, "mul_mat_q: dst_stride < N");

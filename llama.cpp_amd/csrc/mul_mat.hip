@@ -35,13 +35,9 @@ int gemv_unaligned(hipStream_t s, int type, const void *W, const void *act, floa
     const act_ds *ads = (const act_ds *)(aq + B * K);
     MI355_REQUIRE(B <= 65535, "mul_mat: batch %lld too large for the unaligned path", (long long)B);
     const dim3 grid((unsigned)N, (unsigned)B);
-    switch (type) {
-        case MI355_Q4_0: MI355_LAUNCH(k_gemv_unaligned<MI355_Q4_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-        case MI355_Q8_0: MI355_LAUNCH(k_gemv_unaligned<MI355_Q8_0>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-        case MI355_Q4_K: MI355_LAUNCH(k_gemv_unaligned<MI355_Q4_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-        case MI355_Q5_K: MI355_LAUNCH(k_gemv_unaligned<MI355_Q5_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-        default: MI355_LAUNCH(k_gemv_unaligned<MI355_Q6_K>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L); break;
-    }
+#define MI355_UNALIGNED_LAUNCH(TY) MI355_LAUNCH(k_gemv_unaligned<TY>, grid, dim3(64), 0, s, (const uint8_t *)W, aq, ads, dst, residual, N, K, dst_stride, L);
+    MI355_WEIGHT_TYPE_SWITCH(type, MI355_UNALIGNED_LAUNCH)
+#undef MI355_UNALIGNED_LAUNCH
     return launch_status("k_gemv_unaligned");
 }
 
@@ -106,9 +102,9 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
         const size_t used = mi355_mul_mat_ws_bytes(K, B);
         return mi355_mul_mat_q8k_ws(stream, type, W, ws, dst, nullptr, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
     }
-    if (type == MI355_Q5_K && B > 8) {
-        // No tile kernel unpacks Q5_K yet: batches go through the GEMV eight activation rows at a time (each pass streams the
-        // matrix once), quantizing every eight rows into the start of the workspace.
+    if ((type == MI355_Q5_K || !is_fused_weight_type(type)) && B > 8) {
+        // No tile kernel here unpacks Q5_K, Q4_1, Q5_0, Q5_1 or IQ4_NL: batches go through the GEMV eight activation rows at a
+        // time (each pass streams the matrix once), quantizing every eight rows into the start of the workspace.
         for (int64_t b0 = 0; b0 < B; b0 += 8) {
             const int64_t nb = B - b0 < 8 ? B - b0 : 8;
             int rc = mi355_quantize_act(stream, x + b0 * x_stride, ws, K, nb, x_stride);

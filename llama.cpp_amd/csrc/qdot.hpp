@@ -2,7 +2,7 @@
 //
 // Work unit ("chunk"): what one lane consumes per step.  Chunk c of a row is taken by lane
 // c % 64 at step c / 64, so a wave walks a row in consecutive 16-byte, 16-byte-aligned loads.
-//   Q4_0 / Q8_0 : chunk = one 32-element block.
+//   Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL : chunk = one 32-element block.
 //   Q4_K        : chunk = 32 bytes of qs = sub-blocks 2g (low nibbles) and 2g+1 (high nibbles),
 //                 64 elements; 4 chunks per super-block share its 16-byte header.
 //   Q5_K        : as Q4_K, plus the 32 bytes of qh that carry the fifth bit of all eight sub-blocks.
@@ -19,8 +19,8 @@ namespace mi355 {
 // Device layout of one weight row (see mi355_kernels.h): byte offsets of the per-row regions.
 struct row_layout {
     int64_t row_bytes;
-    int off_b;   // Q4_0/Q8_0: fp16 d array.  Q6_K: qh array
-    int off_c;   // Q6_K: scales array
+    int off_b;   // Q4_0/Q8_0/IQ4_NL: fp16 d array.  Q4_1: {fp16 d, fp16 m} array.  Q5_0/Q5_1: fifth-bit words.  Q6_K: qh array
+    int off_c;   // Q5_0: fp16 d array.  Q5_1: {fp16 d, fp16 m} array.  Q6_K: scales array
     int off_d;   // Q6_K: fp16 d array
 };
 
@@ -29,7 +29,8 @@ __host__ __device__ inline row_layout make_row_layout(int type, int64_t k) {
     const int64_t nb = k / type_block_elems(type);
     L.row_bytes = nb * type_block_bytes(type);
     switch (type) {
-        case MI355_Q4_0: L.off_b = (int)(nb * 16); break;
+        case MI355_Q4_0: case MI355_IQ4_NL: case MI355_Q4_1: L.off_b = (int)(nb * 16); break;
+        case MI355_Q5_0: case MI355_Q5_1: L.off_b = (int)(nb * 16); L.off_c = (int)(nb * 20); break;
         case MI355_Q8_0: L.off_b = (int)(nb * 32); break;
         case MI355_Q6_K: L.off_b = (int)(nb * 128); L.off_c = (int)(nb * 192); L.off_d = (int)(nb * 208); break;
         default: break;
@@ -138,6 +139,129 @@ template <> struct wq<MI355_Q8_0> {
     }
     static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
         return __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), acc);
+    }
+};
+
+// ---------------------------------------------------------------- IQ4_NL
+// block_iq4_nl (ggml/src/ggml-common.h:399-404): the Q4_0 bytes, but nibble n stands for kvalues_iq4nl[n]
+// (ggml/src/ggml-cpu/ggml-cpu-quants.c:1672); ggml_vec_dot_iq4_nl_q8_0 (:11188, scalar tail :11368-11377).
+// The sixteen table bytes sit in four dwords; two byte permutes pick among the lower and the upper eight by the low three bits
+// of each nibble, bit 3 then chooses between the two results.
+__device__ __forceinline__ u32 iq4nl_lookup4(u32 nibbles) {   // four nibbles, one per byte -> four table entries
+    constexpr u32 T0 = 0xBFAD9881u, T1 = 0xF6EADDCFu, T2 = 0x26190D01u, T3 = 0x71594535u;   // -127 -104 -83 -65 | -49 -35 -22 -10 | 1 13 25 38 | 53 69 89 113
+    const u32 sel = nibbles & 0x07070707u;
+    const u32 lo = __builtin_amdgcn_perm(T1, T0, sel);
+    const u32 hi = __builtin_amdgcn_perm(T3, T2, sel);
+    const u32 m = ((nibbles >> 3) & 0x01010101u) * 0xFFu;
+    return (lo & ~m) | (hi & m);
+}
+template <> struct wq<MI355_IQ4_NL> {
+    static constexpr int CHUNK = 32;
+    typedef wq<MI355_Q4_0>::chunk chunk;
+    typedef wq<MI355_Q8_0>::act act;
+    static __device__ __forceinline__ chunk load_w(const uint8_t *__restrict__ row, const row_layout &L, int c) { return wq<MI355_Q4_0>::load_w(row, L, c); }
+    static __device__ __forceinline__ act load_a(const int8_t *__restrict__ q, const act_ds *__restrict__ ds, int c) { return wq<MI355_Q8_0>::load_a(q, ds, c); }
+    static __device__ __forceinline__ chunk_dots dots(const chunk &w, const act &A) {
+        int s = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            s = dot4((int)iq4nl_lookup4(w.qs[i] & 0x0F0F0F0Fu), (int)A.a0[i], s);
+            s = dot4((int)iq4nl_lookup4((w.qs[i] >> 4) & 0x0F0F0F0Fu), (int)A.a1[i], s);
+        }
+        chunk_dots r = {s, 0};
+        return r;
+    }
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        return __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), acc);
+    }
+};
+
+// ---------------------------------------------------------------- Q4_1, Q5_0, Q5_1
+// block_q4_1 / q5_0 / q5_1 (ggml/src/ggml-common.h:168-201): value = d * level (+ m), level = nibble (| fifth bit << 4)
+// (- 16 for Q5_0); ggml_vec_dot_q4_1_q8_1, _q5_0_q8_0, _q5_1_q8_1 (ggml/src/ggml-cpu/ggml-cpu-quants.c:2511, 2804, 3159; scalar
+// tails :2784-2799, :3131-3153, :3504-3526).  The block minimum meets the activation through d_a * sum of its levels.
+__device__ __forceinline__ u32 spread4(u32 bits) {   // bits 0..3 -> bit 4 of bytes 0..3
+    return (((bits & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+}
+template <> struct wq<MI355_Q4_1> {
+    static constexpr int CHUNK = 32;
+    struct chunk { u32x4 qs; float d, m; };
+    typedef wq<MI355_Q4_0>::act act;
+    static __device__ __forceinline__ chunk load_w(const uint8_t *__restrict__ row, const row_layout &L, int c) {
+        chunk w;
+        w.qs = load_stream16(row + c * 16);
+        const u32 dm = *(const u32 *)(row + L.off_b + c * 4);
+        w.d = half_bits_to_float((unsigned short)(dm & 0xFFFFu));
+        w.m = half_bits_to_float((unsigned short)(dm >> 16));
+        return w;
+    }
+    static __device__ __forceinline__ act load_a(const int8_t *__restrict__ q, const act_ds *__restrict__ ds, int c) { return wq<MI355_Q4_0>::load_a(q, ds, c); }
+    static __device__ __forceinline__ chunk_dots dots(const chunk &w, const act &A) {
+        int s = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            s = dot4((int)(w.qs[i] & 0x0F0F0F0Fu), (int)A.a0[i], s);
+            s = dot4((int)((w.qs[i] >> 4) & 0x0F0F0F0Fu), (int)A.a1[i], s);
+        }
+        chunk_dots r = {s, 0};
+        return r;
+    }
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        const float t = __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), mul_rn(w.m, mul_rn(A.d, (float)A.sum)));
+        return add_rn(acc, t);
+    }
+};
+template <> struct wq<MI355_Q5_0> {
+    static constexpr int CHUNK = 32;
+    struct chunk { u32x4 qs; u32 qh; float d; };
+    typedef wq<MI355_Q4_0>::act act;
+    static __device__ __forceinline__ chunk load_w(const uint8_t *__restrict__ row, const row_layout &L, int c) {
+        chunk w;
+        w.qs = load_stream16(row + c * 16);
+        w.qh = *(const u32 *)(row + L.off_b + c * 4);
+        w.d = half_bits_to_float(*(const unsigned short *)(row + L.off_c + c * 2));
+        return w;
+    }
+    static __device__ __forceinline__ act load_a(const int8_t *__restrict__ q, const act_ds *__restrict__ ds, int c) { return wq<MI355_Q4_0>::load_a(q, ds, c); }
+    // sum (level - 16) * q: bit j of qh belongs to element j; elements 4i..4i+3 are the low nibbles of dword i, 16+4i.. the high ones
+    static __device__ __forceinline__ int level_dot(const u32x4 &qs, u32 qh, const u32x4 &a0, const u32x4 &a1) {
+        int s = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            s = dot4((int)((qs[i] & 0x0F0F0F0Fu) | spread4(qh >> (4 * i))), (int)a0[i], s);
+            s = dot4((int)(((qs[i] >> 4) & 0x0F0F0F0Fu) | spread4(qh >> (16 + 4 * i))), (int)a1[i], s);
+        }
+        return s;
+    }
+    static __device__ __forceinline__ chunk_dots dots(const chunk &w, const act &A) {
+        chunk_dots r = {level_dot(w.qs, w.qh, A.a0, A.a1) - 16 * A.sum, 0};
+        return r;
+    }
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        return __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), acc);
+    }
+};
+template <> struct wq<MI355_Q5_1> {
+    static constexpr int CHUNK = 32;
+    struct chunk { u32x4 qs; u32 qh; float d, m; };
+    typedef wq<MI355_Q4_0>::act act;
+    static __device__ __forceinline__ chunk load_w(const uint8_t *__restrict__ row, const row_layout &L, int c) {
+        chunk w;
+        w.qs = load_stream16(row + c * 16);
+        w.qh = *(const u32 *)(row + L.off_b + c * 4);
+        const u32 dm = *(const u32 *)(row + L.off_c + c * 4);
+        w.d = half_bits_to_float((unsigned short)(dm & 0xFFFFu));
+        w.m = half_bits_to_float((unsigned short)(dm >> 16));
+        return w;
+    }
+    static __device__ __forceinline__ act load_a(const int8_t *__restrict__ q, const act_ds *__restrict__ ds, int c) { return wq<MI355_Q4_0>::load_a(q, ds, c); }
+    static __device__ __forceinline__ chunk_dots dots(const chunk &w, const act &A) {
+        chunk_dots r = {wq<MI355_Q5_0>::level_dot(w.qs, w.qh, A.a0, A.a1), 0};
+        return r;
+    }
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        const float t = __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), mul_rn(w.m, mul_rn(A.d, (float)A.sum)));
+        return add_rn(acc, t);
     }
 };
 
@@ -320,8 +444,8 @@ template <> struct wq<MI355_Q6_K> {
 // ---------------------------------------------------------------- scalar element access
 // Dequantized weight element e of a row stored in device layout.  Byte loads only, so it
 // works for rows that are not 16-byte aligned (K not a multiple of 256 for Q4_0/Q8_0, of
-// 2048 for Q6_K).  Semantics: dequantize_row_* of ggml/src/ggml-quants.c:255-273, 349-363,
-// 1280-1302, 1482-1507, 1690-1719.
+// 2048 for Q6_K).  Semantics: dequantize_row_* of ggml/src/ggml-quants.c:255-347, 349-363,
+// 1280-1302, 1482-1507, 1690-1719, 2436-2452.
 template <int TYPE>
 __device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, const row_layout &L, int64_t e) {
     if constexpr (TYPE == MI355_Q4_0) {
@@ -331,6 +455,23 @@ __device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, c
         const int n = j < 16 ? (byte & 0x0F) : (byte >> 4);
         const unsigned short dh = (unsigned short)(row[L.off_b + 2 * b] | (row[L.off_b + 2 * b + 1] << 8));
         return half_bits_to_float(dh) * (float)(n - 8);
+    } else if constexpr (TYPE == MI355_IQ4_NL) {
+        constexpr int8_t values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+        const int64_t b = e >> 5;
+        const int j = (int)(e & 31);
+        const uint8_t byte = row[b * 16 + (j & 15)];
+        const unsigned short dh = (unsigned short)(row[L.off_b + 2 * b] | (row[L.off_b + 2 * b + 1] << 8));
+        return half_bits_to_float(dh) * (float)values[j < 16 ? (byte & 0x0F) : (byte >> 4)];
+    } else if constexpr (TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1) {
+        const int64_t b = e >> 5;
+        const int j = (int)(e & 31);
+        const uint8_t byte = row[b * 16 + (j & 15)];
+        int n = j < 16 ? (byte & 0x0F) : (byte >> 4);
+        if constexpr (TYPE != MI355_Q4_1) n |= ((row[L.off_b + 4 * b + (j >> 3)] >> (j & 7)) & 1) << 4;
+        const int64_t so = TYPE == MI355_Q4_1 ? L.off_b + 4 * b : TYPE == MI355_Q5_0 ? L.off_c + 2 * b : L.off_c + 4 * b;
+        const float d = half_bits_to_float((unsigned short)(row[so] | (row[so + 1] << 8)));
+        if constexpr (TYPE == MI355_Q5_0) return d * (float)(n - 16);
+        else return add_rn(mul_rn((float)n, d), half_bits_to_float((unsigned short)(row[so + 2] | (row[so + 3] << 8))));
     } else if constexpr (TYPE == MI355_Q8_0) {
         const int64_t b = e >> 5;
         const int8_t q = (int8_t)row[b * 32 + (e & 31)];

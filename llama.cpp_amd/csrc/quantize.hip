@@ -86,9 +86,23 @@ __global__ void __launch_bounds__(256) k_quantize_q8_1(const float *__restrict__
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ int64_t dev_offset_in_row(int type, int64_t nb, int64_t w) {
     switch (type) {
-        case MI355_Q4_0: {
+        case MI355_Q4_0: case MI355_IQ4_NL: {
             const int64_t b = w / Q4_0_BYTES, o = w % Q4_0_BYTES;
             return o < 2 ? nb * 16 + b * 2 + o : b * 16 + (o - 2);
+        }
+        case MI355_Q4_1: {   // d, m, 16 nibble bytes
+            const int64_t b = w / Q4_1_BYTES, o = w % Q4_1_BYTES;
+            return o < 4 ? nb * 16 + b * 4 + o : b * 16 + (o - 4);
+        }
+        case MI355_Q5_0: {   // d, 4 bytes of fifth bits, 16 nibble bytes
+            const int64_t b = w / Q5_0_BYTES, o = w % Q5_0_BYTES;
+            if (o < 2) return nb * 20 + b * 2 + o;
+            return o < 6 ? nb * 16 + b * 4 + (o - 2) : b * 16 + (o - 6);
+        }
+        case MI355_Q5_1: {   // d, m, 4 bytes of fifth bits, 16 nibble bytes
+            const int64_t b = w / Q5_1_BYTES, o = w % Q5_1_BYTES;
+            if (o < 4) return nb * 20 + b * 4 + o;
+            return o < 8 ? nb * 16 + b * 4 + (o - 4) : b * 16 + (o - 8);
         }
         case MI355_Q8_0: {
             const int64_t b = w / Q8_0_BYTES, o = w % Q8_0_BYTES;
@@ -128,7 +142,7 @@ static int weights_permute(bool scatter, void *stream, int type, const void *src
     MI355_REQUIRE(offset + size <= (size_t)row_bytes * (size_t)nrows, "weights layout: range exceeds tensor");
     if (size == 0) return MI355_OK;
     hipStream_t s = (hipStream_t)stream;
-    if (type == MI355_Q4_K) {   // identity layout
+    if (type == MI355_Q4_K || type == MI355_Q5_K) {   // identity layout
         const void *from = scatter ? src : (const void *)((const uint8_t *)src + offset);
         void *to = scatter ? (void *)((uint8_t *)dst + offset) : dst;
         MI355_CHECK_HIP(hipMemcpyAsync(to, from, size, hipMemcpyDeviceToDevice, s));

@@ -23,7 +23,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-#define QK   32   /* elements per Q4_0/Q8_0/Q8_1 block  (ggml/src/ggml-common.h:161,203,210) */
+#define QK   32   /* elements per Q4_0/Q4_1/Q5_0/Q5_1/Q8_0/Q8_1/IQ4_NL block  (ggml/src/ggml-common.h:161-210, 399) */
 #define QKK 256   /* elements per K-quant super-block   (ggml/src/ggml-common.h:85) */
 
 #define MAXI(a, b) ((a) > (b) ? (a) : (b))
@@ -31,9 +31,14 @@
 
 /* ------------------------------------------------------------------ block layouts
  * ggml/src/ggml-common.h:161-166 (q4_0), 203-208 (q8_0), 210-221 (q8_1),
- * 279-290 (q4_K), 296-308 (q5_K), 314-320 (q6_K), 322-328 (q8_K).  All packed, no padding. */
+ * 279-290 (q4_K), 296-308 (q5_K), 314-320 (q6_K), 322-328 (q8_K), 168-179 (q4_1), 181-187 (q5_0), 189-201 (q5_1),
+ * 399-404 (iq4_nl).  All packed, no padding. */
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[16]; } blk_q4_0;                       /* 18 B  */
+typedef struct { uint16_t d; uint16_t m; uint8_t qs[16]; } blk_q4_1;           /* 20 B  */
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_0;        /* 22 B  */
+typedef struct { uint16_t d; uint16_t m; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_1; /* 24 B */
+typedef struct { uint16_t d; uint8_t qs[16]; } blk_iq4_nl;                     /* 18 B  */
 typedef struct { uint16_t d; int8_t qs[32]; } blk_q8_0;                        /* 34 B  */
 typedef struct { uint16_t d; uint16_t s; int8_t qs[32]; } blk_q8_1;            /* 36 B  */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[128]; } blk_q4_K; /* 144 B */
@@ -94,7 +99,7 @@ void orc_f16_to_f32_row(const uint16_t *x, float *y, int64_t n) { for (int64_t i
 int orc_block_elems(int type) {
     switch (type) {
         case ORC_F32: case ORC_F16: return 1;
-        case ORC_Q4_0: case ORC_Q8_0: case ORC_Q8_1: return QK;
+        case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_IQ4_NL: case ORC_Q8_0: case ORC_Q8_1: return QK;
         case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_Q8_K: return QKK;
         default: return 0;
     }
@@ -104,6 +109,10 @@ size_t orc_block_bytes(int type) {
         case ORC_F32: return 4;
         case ORC_F16: return 2;
         case ORC_Q4_0: return sizeof(blk_q4_0);
+        case ORC_Q4_1: return sizeof(blk_q4_1);
+        case ORC_Q5_0: return sizeof(blk_q5_0);
+        case ORC_Q5_1: return sizeof(blk_q5_1);
+        case ORC_IQ4_NL: return sizeof(blk_iq4_nl);
         case ORC_Q8_0: return sizeof(blk_q8_0);
         case ORC_Q8_1: return sizeof(blk_q8_1);
         case ORC_Q4_K: return sizeof(blk_q4_K);
@@ -188,6 +197,178 @@ static void dequant_q4_0(const blk_q4_0 *x, float *y, int64_t k) {
         for (int j = 0; j < QK / 2; j++) {
             y[b * QK + j] = ((x[b].qs[j] & 0x0F) - 8) * d;
             y[b * QK + j + QK / 2] = ((x[b].qs[j] >> 4) - 8) * d;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ Q4_1, Q5_0, Q5_1
+ * quantize_row_q4_1_ref / q5_0_ref / q5_1_ref, ggml/src/ggml-quants.c:68-103, 105-147, 149-192;
+ * dequantize_row_q4_1 / q5_0 / q5_1, ggml/src/ggml-quants.c:275-294, 296-320, 322-347.
+ * Bit j of qh is the fifth bit of element j of the block (elements 0..15 sit in the low nibbles, 16..31 in the high ones). */
+static uint32_t q5_qh(const uint8_t *qh) { return (uint32_t)qh[0] | ((uint32_t)qh[1] << 8) | ((uint32_t)qh[2] << 16) | ((uint32_t)qh[3] << 24); }
+static int q5_level(const uint8_t *qs, const uint8_t *qh, int j) {
+    const int n = j < 16 ? (qs[j] & 0x0F) : (qs[j - 16] >> 4);
+    return n | (int)(((q5_qh(qh) >> j) & 1u) << 4);
+}
+static void quant_q4_1(const float *x, blk_q4_1 *y, int64_t k) {
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float *xb = x + b * QK;
+        float vmin = 3.402823466e+38f, vmax = -3.402823466e+38f;
+        for (int j = 0; j < QK; j++) {
+            if (xb[j] < vmin) vmin = xb[j];
+            if (xb[j] > vmax) vmax = xb[j];
+        }
+        const float d = (vmax - vmin) / 15;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = orc_f32_to_f16(d);
+        y[b].m = orc_f32_to_f16(vmin);
+        for (int j = 0; j < QK / 2; j++) {
+            const float a0 = (xb[j] - vmin) * id, a1 = (xb[j + QK / 2] - vmin) * id;
+            const uint8_t lo = (uint8_t)MINI(15, (int8_t)(a0 + 0.5f));
+            const uint8_t hi = (uint8_t)MINI(15, (int8_t)(a1 + 0.5f));
+            y[b].qs[j] = (uint8_t)(lo | (hi << 4));
+        }
+    }
+}
+static void dequant_q4_1(const blk_q4_1 *x, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float d = orc_f16_to_f32(x[b].d), m = orc_f16_to_f32(x[b].m);
+        for (int j = 0; j < QK / 2; j++) {
+            y[b * QK + j] = (x[b].qs[j] & 0x0F) * d + m;
+            y[b * QK + j + QK / 2] = (x[b].qs[j] >> 4) * d + m;
+        }
+    }
+}
+static void q5_store(uint8_t *qs, uint8_t *qh, const uint8_t *lv) {   /* 32 levels 0..31 -> nibbles + fifth bits */
+    uint32_t h = 0;
+    for (int j = 0; j < QK / 2; j++) {
+        qs[j] = (uint8_t)((lv[j] & 0x0F) | ((lv[j + QK / 2] & 0x0F) << 4));
+        h |= (uint32_t)((lv[j] & 0x10) >> 4) << j;
+        h |= (uint32_t)((lv[j + QK / 2] & 0x10) >> 4) << (j + QK / 2);
+    }
+    for (int i = 0; i < 4; i++) qh[i] = (uint8_t)(h >> (8 * i));
+}
+static void quant_q5_0(const float *x, blk_q5_0 *y, int64_t k) {
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float *xb = x + b * QK;
+        float amax = 0.0f, vmax = 0.0f;
+        for (int j = 0; j < QK; j++) {
+            if (amax < fabsf(xb[j])) { amax = fabsf(xb[j]); vmax = xb[j]; }
+        }
+        const float d = vmax / -16;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = orc_f32_to_f16(d);
+        uint8_t lv[QK];
+        for (int j = 0; j < QK; j++) lv[j] = (uint8_t)MINI(31, (int8_t)(xb[j] * id + 16.5f));
+        q5_store(y[b].qs, y[b].qh, lv);
+    }
+}
+static void dequant_q5_0(const blk_q5_0 *x, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float d = orc_f16_to_f32(x[b].d);
+        for (int j = 0; j < QK; j++) y[b * QK + j] = (q5_level(x[b].qs, x[b].qh, j) - 16) * d;
+    }
+}
+static void quant_q5_1(const float *x, blk_q5_1 *y, int64_t k) {
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float *xb = x + b * QK;
+        float vmin = 3.402823466e+38f, vmax = -3.402823466e+38f;
+        for (int j = 0; j < QK; j++) {
+            if (xb[j] < vmin) vmin = xb[j];
+            if (xb[j] > vmax) vmax = xb[j];
+        }
+        const float d = (vmax - vmin) / 31;
+        const float id = d ? 1.0f / d : 0.0f;
+        y[b].d = orc_f32_to_f16(d);
+        y[b].m = orc_f32_to_f16(vmin);
+        uint8_t lv[QK];
+        for (int j = 0; j < QK; j++) lv[j] = (uint8_t)((xb[j] - vmin) * id + 0.5f);   /* no clamp in the reference: bits above the fifth are dropped */
+        q5_store(y[b].qs, y[b].qh, lv);
+    }
+}
+static void dequant_q5_1(const blk_q5_1 *x, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float d = orc_f16_to_f32(x[b].d), m = orc_f16_to_f32(x[b].m);
+        for (int j = 0; j < QK; j++) y[b * QK + j] = q5_level(x[b].qs, x[b].qh, j) * d + m;
+    }
+}
+
+/* ------------------------------------------------------------------ IQ4_NL
+ * sixteen non-uniform levels (kvalues_iq4nl, ggml/src/ggml-cpu/ggml-cpu-quants.c:1672); dequantize_row_iq4_nl,
+ * ggml/src/ggml-quants.c:2436-2452.  The quantizer is quantize_iq4_nl without importance weights (ggml/src/ggml-quants.c:
+ * 4684-4704: what ggml_quantize_chunk and the quantize tool run), i.e. quantize_row_iq4_nl_impl (:4573-4682) on one
+ * 32-element block with ntry = 7: a first scale max / -127, then 15 candidate scales, each scored by the weighted
+ * least-squares fit with weights x^2, and the levels re-chosen for the winning scale. */
+static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+static int iq4nl_best_index(float x) {   /* best_index_int8, ggml/src/ggml-quants.c:4562-4571 */
+    const int8_t *val = iq4nl_values;
+    if (x <= val[0]) return 0;
+    if (x >= val[15]) return 15;
+    int ml = 0, mu = 15;
+    while (mu - ml > 1) {
+        const int mav = (ml + mu) / 2;
+        if (x < val[mav]) mu = mav; else ml = mav;
+    }
+    return x - val[mu - 1] < val[mu] - x ? mu - 1 : mu;
+}
+static void quant_iq4_nl(const float *x, blk_iq4_nl *y, int64_t k) {
+    const int ntry = 7;
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float *xb = x + b * QK;
+        uint8_t L[QK];
+        float weight[QK];
+        memset(y[b].qs, 0, 16);
+        y[b].d = orc_f32_to_f16(0.f);
+        for (int j = 0; j < QK; j++) weight[j] = xb[j] * xb[j];
+        float amax = 0, max = 0;
+        for (int j = 0; j < QK; j++) {
+            const float ax = fabsf(xb[j]);
+            if (ax > amax) { amax = ax; max = xb[j]; }
+        }
+        float scale = 0;
+        memset(L, 0, sizeof(L));
+        if (amax >= 1e-15f) {
+            float d = -max / iq4nl_values[0];
+            float id = 1 / d;
+            float sumqx = 0, sumq2 = 0;
+            for (int j = 0; j < QK; j++) {
+                const float al = id * xb[j];
+                const int l = iq4nl_best_index(al);
+                L[j] = (uint8_t)l;
+                const float q = iq4nl_values[l];
+                const float w = weight[j];
+                sumqx += w * q * xb[j];
+                sumq2 += w * q * q;
+            }
+            d = sumqx / sumq2;
+            float best = d * sumqx;
+            for (int itry = -ntry; itry <= ntry; itry++) {
+                id = (itry + iq4nl_values[0]) / max;
+                sumqx = sumq2 = 0;
+                for (int j = 0; j < QK; j++) {
+                    const float al = id * xb[j];
+                    const int l = iq4nl_best_index(al);
+                    const float q = iq4nl_values[l];
+                    const float w = weight[j];
+                    sumqx += w * q * xb[j];
+                    sumq2 += w * q * q;
+                }
+                if (sumq2 > 0 && sumqx * sumqx > best * sumq2) { d = sumqx / sumq2; best = d * sumqx; }
+            }
+            scale = d;
+        }
+        y[b].d = orc_f32_to_f16(scale);
+        const float id = scale ? 1 / scale : 0;
+        for (int j = 0; j < QK; j++) L[j] = (uint8_t)iq4nl_best_index(id * xb[j]);
+        for (int j = 0; j < 16; j++) y[b].qs[j] = (uint8_t)(L[j] | (L[16 + j] << 4));
+    }
+}
+static void dequant_iq4_nl(const blk_iq4_nl *x, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float d = orc_f16_to_f32(x[b].d);
+        for (int j = 0; j < QK / 2; j++) {
+            y[b * QK + j] = d * iq4nl_values[x[b].qs[j] & 0x0F];
+            y[b * QK + j + QK / 2] = d * iq4nl_values[x[b].qs[j] >> 4];
         }
     }
 }
@@ -574,6 +755,10 @@ static int quantize_row(int type, const float *x, void *y, int64_t k) {
         case ORC_F32: memcpy(y, x, (size_t)k * 4); return 0;
         case ORC_F16: orc_f32_to_f16_row(x, (uint16_t *)y, k); return 0;
         case ORC_Q4_0: quant_q4_0(x, (blk_q4_0 *)y, k); return 0;
+        case ORC_Q4_1: quant_q4_1(x, (blk_q4_1 *)y, k); return 0;
+        case ORC_Q5_0: quant_q5_0(x, (blk_q5_0 *)y, k); return 0;
+        case ORC_Q5_1: quant_q5_1(x, (blk_q5_1 *)y, k); return 0;
+        case ORC_IQ4_NL: quant_iq4_nl(x, (blk_iq4_nl *)y, k); return 0;
         case ORC_Q8_0: quant_q8_0(x, (blk_q8_0 *)y, k); return 0;
         case ORC_Q8_1: quant_q8_1(x, (blk_q8_1 *)y, k); return 0;
         case ORC_Q4_K: quant_q4_K(x, (blk_q4_K *)y, k); return 0;
@@ -588,6 +773,10 @@ static int dequantize_row(int type, const void *x, float *y, int64_t k) {
         case ORC_F32: memcpy(y, x, (size_t)k * 4); return 0;
         case ORC_F16: orc_f16_to_f32_row((const uint16_t *)x, y, k); return 0;
         case ORC_Q4_0: dequant_q4_0((const blk_q4_0 *)x, y, k); return 0;
+        case ORC_Q4_1: dequant_q4_1((const blk_q4_1 *)x, y, k); return 0;
+        case ORC_Q5_0: dequant_q5_0((const blk_q5_0 *)x, y, k); return 0;
+        case ORC_Q5_1: dequant_q5_1((const blk_q5_1 *)x, y, k); return 0;
+        case ORC_IQ4_NL: dequant_iq4_nl((const blk_iq4_nl *)x, y, k); return 0;
         case ORC_Q8_0: dequant_q8_0((const blk_q8_0 *)x, y, k); return 0;
         case ORC_Q8_1: dequant_q8_1((const blk_q8_1 *)x, y, k); return 0;
         case ORC_Q4_K: dequant_q4_K((const blk_q4_K *)x, y, k); return 0;
@@ -625,6 +814,18 @@ static int weight_level(int type, const void *row, int64_t e) {
             const int j = (int)(e % QK);
             return (j < 16 ? (b->qs[j] & 0x0F) : (b->qs[j - 16] >> 4)) - 8;
         }
+        case ORC_Q4_1: {   /* unsigned levels; the block minimum enters through the sum of the activation levels */
+            const blk_q4_1 *b = (const blk_q4_1 *)row + e / QK;
+            const int j = (int)(e % QK);
+            return j < 16 ? (b->qs[j] & 0x0F) : (b->qs[j - 16] >> 4);
+        }
+        case ORC_Q5_0: { const blk_q5_0 *b = (const blk_q5_0 *)row + e / QK; return q5_level(b->qs, b->qh, (int)(e % QK)) - 16; }
+        case ORC_Q5_1: { const blk_q5_1 *b = (const blk_q5_1 *)row + e / QK; return q5_level(b->qs, b->qh, (int)(e % QK)); }
+        case ORC_IQ4_NL: {
+            const blk_iq4_nl *b = (const blk_iq4_nl *)row + e / QK;
+            const int j = (int)(e % QK);
+            return iq4nl_values[j < 16 ? (b->qs[j] & 0x0F) : (b->qs[j - 16] >> 4)];
+        }
         case ORC_Q8_0: return ((const blk_q8_0 *)row + e / QK)->qs[e % QK];
         case ORC_Q4_K: return q4k_level((const blk_q4_K *)row + e / QKK, (int)(e % QKK));
         case ORC_Q5_K: return q5k_level((const blk_q5_K *)row + e / QKK, (int)(e % QKK));
@@ -633,9 +834,16 @@ static int weight_level(int type, const void *row, int64_t e) {
     }
 }
 static int granule(int type) { return type == ORC_Q6_K ? 16 : 32; }
+static int is_weight_type(int type) {
+    switch (type) {
+        case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_IQ4_NL: case ORC_Q8_0:
+        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 1;
+        default: return 0;
+    }
+}
 
 int orc_block_dots_q8_1(int type, const void *W, const void *a, int64_t nrows, int64_t k, int32_t *out) {
-    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q5_K && type != ORC_Q6_K) return -1;
+    if (!is_weight_type(type)) return -1;
     if (k % orc_block_elems(type)) return -1;
     const int g = granule(type);
     const size_t rb = orc_row_bytes(type, k);
@@ -667,6 +875,58 @@ static float dot_q4_0_q8_0(const blk_q4_0 *w, const blk_q8_0 *a, int64_t k) {   
             sumi1 += ((w[b].qs[j] >> 4) - 8) * a[b].qs[j + 16];
         }
         sumf += (sumi0 + sumi1) * orc_f16_to_f32(w[b].d) * orc_f16_to_f32(a[b].d);
+    }
+    return sumf;
+}
+/* the per-32 types share one form: sum over blocks of (d_w * d_a) * sumi [+ m_w * s_a]
+ * (ggml_vec_dot_q4_1_q8_1 ggml-cpu-quants.c:2511 ff., scalar tail :2784-2799; q5_0_q8_0 :2804 ff., tail :3131-3153;
+ * q5_1_q8_1 :3159 ff., tail :3504-3526; iq4_nl_q8_0 :11188 ff., tail :11368-11377) */
+static float dot_q4_1_q8_1(const blk_q4_1 *w, const blk_q8_1 *a, int64_t k) {
+    float sumf = 0;
+    for (int64_t b = 0; b < k / QK; b++) {
+        int sumi0 = 0, sumi1 = 0;
+        for (int j = 0; j < 16; j++) {
+            sumi0 += (w[b].qs[j] & 0x0F) * a[b].qs[j];
+            sumi1 += (w[b].qs[j] >> 4) * a[b].qs[j + 16];
+        }
+        sumf += (orc_f16_to_f32(w[b].d) * orc_f16_to_f32(a[b].d)) * (sumi0 + sumi1) + orc_f16_to_f32(w[b].m) * orc_f16_to_f32(a[b].s);
+    }
+    return sumf;
+}
+static float dot_q5_0_q8_0(const blk_q5_0 *w, const blk_q8_0 *a, int64_t k) {
+    float sumf = 0;
+    for (int64_t b = 0; b < k / QK; b++) {
+        int sumi0 = 0, sumi1 = 0;
+        for (int j = 0; j < 16; j++) {
+            sumi0 += (q5_level(w[b].qs, w[b].qh, j) - 16) * a[b].qs[j];
+            sumi1 += (q5_level(w[b].qs, w[b].qh, j + 16) - 16) * a[b].qs[j + 16];
+        }
+        sumf += (orc_f16_to_f32(w[b].d) * orc_f16_to_f32(a[b].d)) * (sumi0 + sumi1);
+    }
+    return sumf;
+}
+static float dot_q5_1_q8_1(const blk_q5_1 *w, const blk_q8_1 *a, int64_t k) {
+    float sumf = 0;
+    for (int64_t b = 0; b < k / QK; b++) {
+        int sumi0 = 0, sumi1 = 0;
+        for (int j = 0; j < 16; j++) {
+            sumi0 += q5_level(w[b].qs, w[b].qh, j) * a[b].qs[j];
+            sumi1 += q5_level(w[b].qs, w[b].qh, j + 16) * a[b].qs[j + 16];
+        }
+        sumf += (orc_f16_to_f32(w[b].d) * orc_f16_to_f32(a[b].d)) * (sumi0 + sumi1) + orc_f16_to_f32(w[b].m) * orc_f16_to_f32(a[b].s);
+    }
+    return sumf;
+}
+static float dot_iq4_nl_q8_0(const blk_iq4_nl *w, const blk_q8_0 *a, int64_t k) {
+    float sumf = 0;
+    for (int64_t b = 0; b < k / QK; b++) {
+        const float d = orc_f16_to_f32(a[b].d) * orc_f16_to_f32(w[b].d);
+        int sumi1 = 0, sumi2 = 0;
+        for (int j = 0; j < 16; j++) {
+            sumi1 += a[b].qs[j] * iq4nl_values[w[b].qs[j] & 0x0F];
+            sumi2 += a[b].qs[j + 16] * iq4nl_values[w[b].qs[j] >> 4];
+        }
+        sumf += d * (sumi1 + sumi2);
     }
     return sumf;
 }
@@ -736,7 +996,8 @@ static float dot_q6_K_q8_K(const blk_q6_K *w, const blk_q8_K *a, int64_t k) {   
 int orc_mul_mat_cpu(int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B) {
     int atype;
     switch (type) {
-        case ORC_Q4_0: case ORC_Q8_0: atype = ORC_Q8_0; break;
+        case ORC_Q4_0: case ORC_Q5_0: case ORC_IQ4_NL: case ORC_Q8_0: atype = ORC_Q8_0; break;
+        case ORC_Q4_1: case ORC_Q5_1: atype = ORC_Q8_1; break;    /* vec_dot_type, ggml-cpu.c:274-296, 384-389 */
         case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: atype = ORC_Q8_K; break;
         default: return -1;
     }
@@ -751,6 +1012,10 @@ int orc_mul_mat_cpu(int type, const void *W, const float *x, float *dst, int64_t
             float r;
             switch (type) {
                 case ORC_Q4_0: r = dot_q4_0_q8_0((const blk_q4_0 *)row, (const blk_q8_0 *)act, K); break;
+                case ORC_Q4_1: r = dot_q4_1_q8_1((const blk_q4_1 *)row, (const blk_q8_1 *)act, K); break;
+                case ORC_Q5_0: r = dot_q5_0_q8_0((const blk_q5_0 *)row, (const blk_q8_0 *)act, K); break;
+                case ORC_Q5_1: r = dot_q5_1_q8_1((const blk_q5_1 *)row, (const blk_q8_1 *)act, K); break;
+                case ORC_IQ4_NL: r = dot_iq4_nl_q8_0((const blk_iq4_nl *)row, (const blk_q8_0 *)act, K); break;
                 case ORC_Q8_0: r = dot_q8_0_q8_0((const blk_q8_0 *)row, (const blk_q8_0 *)act, K); break;
                 case ORC_Q4_K: r = dot_q4_K_q8_K((const blk_q4_K *)row, (const blk_q8_K *)act, K); break;
                 case ORC_Q5_K: r = dot_q5_K_q8_K((const blk_q5_K *)row, (const blk_q8_K *)act, K); break;
@@ -782,6 +1047,17 @@ static double row_dot_q8_1(int type, const void *row, const blk_q8_1 *act, int64
                 for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
                 acc += (double)orc_f16_to_f32(((const blk_q8_0 *)row)[b].d) * dx * isum;
             } break;
+            case ORC_Q5_0: case ORC_IQ4_NL: {   /* d sits first in both blocks */
+                for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
+                const uint16_t dh = type == ORC_Q5_0 ? ((const blk_q5_0 *)row)[b].d : ((const blk_iq4_nl *)row)[b].d;
+                acc += (double)orc_f16_to_f32(dh) * dx * isum;
+            } break;
+            case ORC_Q4_1: case ORC_Q5_1: {     /* value = d * level + m */
+                for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
+                const uint16_t dh = type == ORC_Q4_1 ? ((const blk_q4_1 *)row)[b].d : ((const blk_q5_1 *)row)[b].d;
+                const uint16_t mh = type == ORC_Q4_1 ? ((const blk_q4_1 *)row)[b].m : ((const blk_q5_1 *)row)[b].m;
+                acc += dx * ((double)orc_f16_to_f32(dh) * isum + (double)orc_f16_to_f32(mh) * sumq);
+            } break;
             case ORC_Q4_K: {
                 const blk_q4_K *w = (const blk_q4_K *)row + b / 8;
                 uint8_t sc, mn;
@@ -809,7 +1085,7 @@ static double row_dot_q8_1(int type, const void *row, const blk_q8_1 *act, int64
 }
 
 int orc_mul_mat_q8_1(int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B) {
-    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q5_K && type != ORC_Q6_K) return -1;
+    if (!is_weight_type(type)) return -1;
     if (K % orc_block_elems(type)) return -1;
     const size_t wrb = orc_row_bytes(type, K);
     blk_q8_1 *act = (blk_q8_1 *)malloc(orc_row_bytes(ORC_Q8_1, K));
@@ -844,7 +1120,7 @@ int orc_mul_mat_f64(int type, const void *W, const float *x, float *dst, int64_t
  * ggml_compute_forward_mul_mat_id, ggml/src/ggml-cpu/ggml-cpu.c:7717-7895 */
 int orc_mul_mat_id_q8_1(int type, const void *as, const float *b, const int32_t *ids, int64_t ids_stride, float *dst,
                         int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T) {
-    if (type != ORC_Q4_0 && type != ORC_Q8_0 && type != ORC_Q4_K && type != ORC_Q5_K && type != ORC_Q6_K) return -1;
+    if (!is_weight_type(type)) return -1;
     const size_t wrb = orc_row_bytes(type, K);
     blk_q8_1 *act = (blk_q8_1 *)malloc(orc_row_bytes(ORC_Q8_1, K));
     if (!act) return -1;

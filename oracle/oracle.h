@@ -20,12 +20,16 @@ enum orc_type {
     ORC_F32  = 0,
     ORC_F16  = 1,
     ORC_Q4_0 = 2,
+    ORC_Q4_1 = 3,
+    ORC_Q5_0 = 6,
+    ORC_Q5_1 = 7,
     ORC_Q8_0 = 8,
     ORC_Q8_1 = 9,
     ORC_Q4_K = 12,
     ORC_Q5_K = 13,
     ORC_Q6_K = 14,
     ORC_Q8_K = 15,
+    ORC_IQ4_NL = 20,
 };
 
 /* IEEE binary16 <-> binary32, round to nearest even */

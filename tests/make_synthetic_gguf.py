@@ -16,8 +16,12 @@ import struct
 
 import numpy as np
 
-F32, Q4_K, Q5_K, Q6_K = 0, 12, 13, 14
-BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
+F32, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL = 0, 2, 3, 6, 7, 8, 12, 13, 14, 20
+BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34),
+         IQ4_NL: (32, 18)}
+# file type -> (default tensor type, LLAMA_FTYPE_MOSTLY_* of include/llama.h:146-169)
+FTYPES = {"q4_k_m": (Q4_K, 15), "q5_k_m": (Q5_K, 17), "q4_0": (Q4_0, 2), "q4_1": (Q4_1, 3), "q5_0": (Q5_0, 8), "q5_1": (Q5_1, 9), "q8_0": (Q8_0, 7),
+          "iq4_nl": (IQ4_NL, 25)}
 T_U32, T_F32, T_STR, T_U64 = 4, 6, 8, 10
 
 
@@ -47,10 +51,16 @@ def _kv(key, vtype, value):
 def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert=0, base=Q4_K):
     """n_expert > 0: mixture-of-experts feed-forward (src/llama-model.cpp:1553-1558) with every quantized tensor Q4_K, the mix
     of `llama-quantize --pure ... Q4_K`; the router ffn_gate_inp stays f32 (src/llama-quant.cpp:749).
-    base: Q4_K for the Q4_K_M mix, Q5_K for Q5_K_M (the same rules with Q5_K as the default type, src/llama-quant.cpp:122-340)"""
+    base: Q4_K for the Q4_K_M mix, Q5_K for Q5_K_M (the same rules with Q5_K as the default type, src/llama-quant.cpp:122-340).
+    A per-32-block base (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0) is used for every matrix, as llama-quantize does without an importance
+    matrix, with output.weight Q6_K (Q8_0 stays Q8_0, :166-168); IQ4_NL takes Q5_K for attn_v (grouped-query models, :232-234) and for
+    ffn_down in the first eighth of the layers (:299-301)."""
     t = [("token_embd.weight", base, (n_embd, n_vocab))]
+    kmix = base in (Q4_K, Q5_K)
     for il in range(n_layer):
-        more = use_more_bits(il, n_layer) and n_expert == 0
+        more = kmix and use_more_bits(il, n_layer) and n_expert == 0
+        v_type = Q6_K if more else Q5_K if (base == IQ4_NL and n_head // n_head_kv >= 4) else base
+        down_type = Q6_K if more else Q5_K if (base == IQ4_NL and il < n_layer // 8) else base
         p = "blk.%d." % il
         if n_expert > 0:
             t += [(p + "attn_norm.weight", F32, (n_embd,)),
@@ -67,13 +77,13 @@ def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_e
         t += [(p + "attn_norm.weight", F32, (n_embd,)),
               (p + "attn_q.weight", base, (n_embd, n_head * head_dim)),
               (p + "attn_k.weight", base, (n_embd, n_head_kv * head_dim)),
-              (p + "attn_v.weight", Q6_K if more else base, (n_embd, n_head_kv * head_dim)),
+              (p + "attn_v.weight", v_type, (n_embd, n_head_kv * head_dim)),
               (p + "attn_output.weight", base, (n_head * head_dim, n_embd)),
               (p + "ffn_norm.weight", F32, (n_embd,)),
               (p + "ffn_gate.weight", base, (n_embd, n_ff)),
               (p + "ffn_up.weight", base, (n_embd, n_ff)),
-              (p + "ffn_down.weight", Q6_K if more else base, (n_ff, n_embd))]
-    t += [("output_norm.weight", F32, (n_embd,)), ("output.weight", base if n_expert > 0 else Q6_K, (n_embd, n_vocab))]
+              (p + "ffn_down.weight", down_type, (n_ff, n_embd))]
+    t += [("output_norm.weight", F32, (n_embd,)), ("output.weight", base if (n_expert > 0 or base == Q8_0) else Q6_K, (n_embd, n_vocab))]
     return t
 
 
@@ -106,22 +116,28 @@ def random_blocks(ttype, n_blocks, rng, pool):
     elif ttype == Q5_K:    # the same with n ~ U[0,31]
         put_half(0, 0.02 / (31.5 * 9.2))
         put_half(2, 0.02 / (31.5 * 9.2) * 15.5)
-    else:                  # Q6_K: w = d*sc*(q-32), sc int8
+    elif ttype == Q6_K:    # w = d*sc*(q-32), sc int8
         put_half(208, 0.02 / (74.0 * 18.5))
+    elif ttype in (Q4_0, Q8_0, Q5_0, IQ4_NL):   # w = d * level: levels of spread 4.6 / 74 / 9.2 / 68
+        put_half(0, 0.02 / {Q4_0: 4.6, Q8_0: 74.0, Q5_0: 9.2, IQ4_NL: 68.0}[ttype])
+    else:                  # Q4_1 / Q5_1: w = d * n + m
+        spread, mid = (4.6, 7.5) if ttype == Q4_1 else (9.2, 15.5)
+        put_half(0, 0.02 / spread)
+        put_half(2, -0.02 / spread * mid)
     return raw
 
 
 def write_model(path, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=128256, n_ctx=8192,
                 rope_theta=500000.0, rms_eps=1e-5, seed=1234, n_expert=0, n_expert_used=0, ftype="q4_k_m"):
-    """ftype: "q4_k_m" or "q5_k_m" - the tensor mix llama-quantize produces for that file type"""
+    """ftype: a key of FTYPES - the tensor mix llama-quantize produces for that file type"""
     head_dim = n_embd // n_head
-    base = {"q4_k_m": Q4_K, "q5_k_m": Q5_K}[ftype]
+    base = FTYPES[ftype][0]
     tensors = tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_expert, base)
     align = 32
     kvs = [
         _kv("general.architecture", T_STR, "llama"),
         _kv("general.name", T_STR, "synthetic-llama-" + ftype),
-        _kv("general.file_type", T_U32, {"q4_k_m": 15, "q5_k_m": 17}[ftype]),    # LLAMA_FTYPE_MOSTLY_Q4_K_M / _Q5_K_M
+        _kv("general.file_type", T_U32, FTYPES[ftype][1]),
         _kv("general.alignment", T_U32, align),
         _kv("llama.block_count", T_U32, n_layer),
         _kv("llama.context_length", T_U32, n_ctx),
@@ -157,7 +173,7 @@ def write_model(path, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=
                 f.write(data)
                 f.write(b"\0" * ((-len(data)) % align))
                 continue
-            total = int(np.prod(shape)) // 256
+            total = int(np.prod(shape)) // BLOCK[ttype][0]
             done = 0
             while done < total:   # in slices, to bound memory
                 n = min(total - done, 1 << 18)
@@ -178,7 +194,7 @@ if __name__ == "__main__":
     ap.add_argument("--vocab", type=int, default=128256)
     ap.add_argument("--experts", type=int, default=0, help="mixture of experts: number of experts (0 = dense)")
     ap.add_argument("--experts-used", type=int, default=2)
-    ap.add_argument("--ftype", default="q4_k_m", choices=["q4_k_m", "q5_k_m"])
+    ap.add_argument("--ftype", default="q4_k_m", choices=sorted(FTYPES))
     a = ap.parse_args()
     size = write_model(a.path, a.layers, a.embd, a.ff, a.heads, a.kv_heads, a.vocab, n_expert=a.experts,
                        n_expert_used=a.experts_used if a.experts else 0, ftype=a.ftype)

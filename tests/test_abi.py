@@ -58,7 +58,7 @@ def test_argument_errors_are_reported_not_crashed():
     lib.mi355_mul_mat_vec_q.restype = ctypes.c_int
     lib.mi355_mul_mat_vec_q.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 3 + [ctypes.c_int64] * 4
     # unsupported type and bad shapes are rejected before any launch
-    assert lib.mi355_mul_mat_vec_q(None, 3, None, None, None, 16, 256, 1, 16) == -1
+    assert lib.mi355_mul_mat_vec_q(None, 10, None, None, None, 16, 256, 1, 16) == -1   # 10: Q2_K, no kernel here
     assert b"unsupported" in lib.mi355_last_error()
     assert lib.mi355_mul_mat_vec_q(None, 12, None, None, None, 16, 100, 1, 16) == -1
     assert lib.mi355_mul_mat_vec_q(None, 12, None, None, None, 16, 256, 33, 16) == -1

@@ -95,6 +95,26 @@ def test_model_logits_q5_k_m(dev, tmp_path, n_prompt):
     assert orc.nmse(dev_out, cpu) < 2e-3
 
 
+@pytest.mark.parametrize("ftype", ["q4_1", "q5_0", "q5_1", "iq4_nl"])
+@pytest.mark.parametrize("n_prompt", [5, 40])
+def test_model_logits_per_32_block_types(dev, tmp_path, ftype, n_prompt):
+    """Files of the per-32-block types beyond Q4_0 / Q8_0 (Q4_1, Q5_0, Q5_1, IQ4_NL with the Q5_K / Q6_K tensors llama-quantize
+    mixes in): the reference's runtime on the plug-in reproduces its CPU backend's logits, so their MUL_MAT (single-matrix GEMV,
+    eight activation rows at a time for a prompt) and GET_ROWS stay on the device with the reference's arithmetic."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / (ftype + ".gguf"))
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048, ftype=ftype)
+    cpu = _logits(model, 0, n_prompt, 3, str(tmp_path / "cpu.bin"))
+    dev_out = _logits(model, 99, n_prompt, 3, str(tmp_path / "dev.bin"))
+    assert cpu.shape == dev_out.shape and np.isfinite(dev_out).all()
+    assert orc.nmse(dev_out, cpu) < 2e-3
+
+
 def test_model_logits_async_loader(dev, tmp_path):
     """Without mmap the reference's loader uploads the weights in 1 MiB chunks from pinned buffers with set_tensor_async and
     fences the buffers with events (src/llama-model-loader.cpp:926-960, 1033-1046): chunks land at byte offsets inside tensors,

@@ -163,7 +163,10 @@ def test_mmq_matches_oracle(dev, name, t, N, K, B):
         assert orc.nmse(got, cpu) <= 5e-4
 
 
-@pytest.mark.parametrize("name,t", [(n, t) for n, t in TYPES if n != "q5_K"])   # Q5_K products with few rows stay with the GEMV
+SKINNY_TYPES = [(n, t) for n, t in TYPES if t in (orc.Q4_0, orc.Q8_0, orc.Q4_K, orc.Q6_K)]   # products of the other types with few rows stay with the GEMV
+
+
+@pytest.mark.parametrize("name,t", SKINNY_TYPES)
 @pytest.mark.parametrize("N,K,B", [(100, 256, 5), (257, 1024, 8), (4096, 4096, 13), (1024, 14336, 17), (64, 3584, 24), (333, 2048, 32), (4096, 4096, 1),
                                    (77, 6144, 9)])
 @pytest.mark.parametrize("split", [False, True])

@@ -119,6 +119,17 @@ def _levels(t, W, K):
         return np.concatenate([(b & 15).astype(np.int32) - 8, (b >> 4).astype(np.int32) - 8], axis=2).reshape(N, K)
     if t == orc.Q8_0:
         return W.reshape(N, K // 32, 34)[:, :, 2:].view(np.int8).astype(np.int32).reshape(N, K)
+    if t in (orc.Q4_1, orc.IQ4_NL):
+        b = W.reshape(N, K // 32, orc.BLOCK[t][1])[:, :, -16:]
+        n = np.concatenate([(b & 15), (b >> 4)], axis=2).astype(np.int32).reshape(N, K)
+        return n if t == orc.Q4_1 else np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.int32)[n]
+    if t in (orc.Q5_0, orc.Q5_1):
+        blk = W.reshape(N, K // 32, orc.BLOCK[t][1])
+        b = blk[:, :, -16:]
+        qh = np.ascontiguousarray(blk[:, :, -20:-16]).view("<u4")                        # [N, nb, 1]: bit j = fifth bit of element j
+        bits = ((qh >> np.arange(32, dtype=np.uint32).reshape(1, 1, 32)) & 1).astype(np.int32)
+        n = np.concatenate([(b & 15), (b >> 4)], axis=2).astype(np.int32) + 16 * bits
+        return (n - (16 if t == orc.Q5_0 else 0)).reshape(N, K)
     if t == orc.Q4_K:
         qs = W.reshape(N, K // 256, 144)[:, :, 16:].reshape(N, K // 256, 4, 32)
         return np.concatenate([(qs & 15), (qs >> 4)], axis=3).astype(np.int32).reshape(N, K)
