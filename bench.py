@@ -208,11 +208,15 @@ def sweep(kinds):
     def emit(**kw):
         print(json.dumps(kw), flush=True)
 
-    bpe = {mi355.Q4_0: 18 / 32, mi355.Q8_0: 34 / 32, mi355.Q4_K: 144 / 256, mi355.Q5_K: 176 / 256, mi355.Q6_K: 210 / 256}
-    names = {mi355.Q4_0: "Q4_0", mi355.Q8_0: "Q8_0", mi355.Q4_K: "Q4_K", mi355.Q5_K: "Q5_K", mi355.Q6_K: "Q6_K"}
+    bpe = {mi355.Q4_0: 18 / 32, mi355.Q8_0: 34 / 32, mi355.Q4_K: 144 / 256, mi355.Q5_K: 176 / 256, mi355.Q6_K: 210 / 256,
+           mi355.Q4_1: 20 / 32, mi355.Q5_0: 22 / 32, mi355.Q5_1: 24 / 32, mi355.IQ4_NL: 18 / 32}
+    names = {mi355.Q4_0: "Q4_0", mi355.Q8_0: "Q8_0", mi355.Q4_K: "Q4_K", mi355.Q5_K: "Q5_K", mi355.Q6_K: "Q6_K", mi355.Q4_1: "Q4_1", mi355.Q5_0: "Q5_0",
+             mi355.Q5_1: "Q5_1", mi355.IQ4_NL: "IQ4_NL"}
+    gemv_only = (mi355.Q5_K, mi355.Q4_1, mi355.Q5_0, mi355.Q5_1, mi355.IQ4_NL)   # no weight-streaming matrix-core kernel: the GEMV serves up to eight rows
+    all_types = (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q5_K, mi355.Q6_K, mi355.Q4_1, mi355.Q5_0, mi355.Q5_1, mi355.IQ4_NL)
     shapes = [(4096, 4096), (14336, 4096), (4096, 14336)]
     if "gemv" in kinds:
-        for t in (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q5_K, mi355.Q6_K):
+        for t in all_types:
             for N, K in shapes + [(128256, 4096)]:
                 wbytes = int(N * K * bpe[t])
                 nm = max(2, min(32, (1 << 31) // wbytes))
@@ -220,19 +224,19 @@ def sweep(kinds):
                 for B in (1, 8):
                     act = mi355.quantize_act(torch.randn(B, K, device=dev, generator=gen))
                     out = torch.empty(B, N, device=dev)
-                    if B == 1 or t == mi355.Q5_K:   # Q5_K: the GEMV serves up to eight rows
+                    if B == 1 or t in gemv_only:
                         us = timed(lambda i: mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, t, Ws[i].data_ptr(), act.data_ptr(), out.data_ptr(), N, K, B, N)), nm, 4)
                     else:   # the weight-streaming matrix-core kernel, with the workspace that lets products with few rows split K
                         ws = torch.empty(int(lib.mi355_mul_mat_skinny_ws_bytes(N, K, B)) + 256, dtype=torch.uint8, device=dev)
                         us = timed(lambda i: mi355.check(lib.mi355_mul_mat_skinny(stream.cuda_stream, t, Ws[i].data_ptr(), act.data_ptr(), out.data_ptr(), None, N, K, B, N,
                                                                                   ws.data_ptr(), ws.numel())), nm, 4)
                     alg = wbytes + B * (4 * K + 4 * N)
-                    emit(kernel="MUL_MAT batch 1 (GEMV)" if B == 1 else ("MUL_MAT batch %d (GEMV)" % B if t == mi355.Q5_K else "MUL_MAT batch %d (k_mm_skinny)" % B), case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
+                    emit(kernel="MUL_MAT batch 1 (GEMV)" if B == 1 else ("MUL_MAT batch %d (GEMV)" % B if t in gemv_only else "MUL_MAT batch %d (k_mm_skinny)" % B), case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
                          unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg)
                 del Ws
     if "mmq" in kinds or "mmq_wide" in kinds:
         wide_only = "mmq" not in kinds    # the wide-tile GEMM alone on the gate/up shape (for counter collection)
-        for t in ((mi355.Q4_K, mi355.Q5_K, mi355.Q6_K) if wide_only else (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q5_K, mi355.Q6_K)):
+        for t in ((mi355.Q4_K, mi355.Q5_K, mi355.Q6_K) if wide_only else all_types):
             for N, K in ([(14336, 4096)] if wide_only else shapes):
                 for B in ((512,) if wide_only else (64, 512)):
                     nm = 4

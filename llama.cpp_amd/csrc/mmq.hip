@@ -12,6 +12,9 @@
 //
 //   Q4_0 : level - 8 as int8, scale d                    (one MFMA per block)
 //   Q8_0 : level as int8, scale d
+//   Q5_0 : level - 16 as int8, scale d;  IQ4_NL : the table value of the nibble as int8, scale d
+//   Q4_1, Q5_1 : level 0..15 / 0..31 as int8, scale d; the "+ m * d_x * sum(q)" term of the stage's four blocks is added with one
+//          v_mfma_f32_32x32x16_f16 on (fp16 dx*sum(q), the reference's `s` field of block_q8_1) x (fp16 m)
 //   Q4_K : level 0..15 as int8, scale d*sc; the "- dmin*m*sum(q)" term of all blocks is
 //          added with one v_mfma_f32_32x32x16_f16 per stage on (fp16 dx*sum(q)) x (fp16 dmin*m)
 //   Q6_K : level - 32 as int8, scale d*sc per 16 elements (v_mfma_i32_32x32x16_i8, two per block)
@@ -37,6 +40,11 @@ constexpr int MMQ_LDK = MMQ_BK + 16; // LDS row pitch in bytes (pad to spread ba
 template <int TYPE> struct mmq_cfg {
     static constexpr int G = TYPE == MI355_Q6_K ? 16 : 32;   // elements per weight scale
     static constexpr int NG = MMQ_BK / G;                    // weight scales per row per stage
+    // a per-block offset rides on the sums of the activation levels: - dmin * m (Q4_K), + m (Q4_1, Q5_1)
+    static constexpr bool MIN = TYPE == MI355_Q4_K || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;
+    // 16 bytes of nibbles per block with a per-block scale: one request / commit form serves them all
+    static constexpr bool NIBBLE32 = TYPE == MI355_Q4_0 || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1 || TYPE == MI355_IQ4_NL;
+    static constexpr bool PREFETCH = NIBBLE32 || TYPE == MI355_Q8_0;
 };
 
 // ---- stage loaders: global (device layout) -> int8 rows + scales in LDS ----------------
@@ -177,10 +185,14 @@ __device__ __forceinline__ void load_act_stage(const int8_t *__restrict__ aq, co
 
 // ---- the same stages split into "request" (global -> registers) and "commit" (unpack -> LDS), so that the next stage's bytes
 // travel while the current stage is contracted (Q4_0 / Q8_0, whose per-32 scales keep them on this kernel)
-template <int TYPE> struct mmq_wregs {};
-template <> struct mmq_wregs<MI355_Q4_0> {
+template <int TYPE, bool NIB = mmq_cfg<TYPE>::NIBBLE32> struct mmq_wregs {};
+// Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL: thread t owns blocks (row, b) = (idx >> 2, idx & 3), idx = t and t + 256
+template <int TYPE> struct mmq_wregs<TYPE, true> {
+    static constexpr bool HAS_QH = TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1;
+    static constexpr bool HAS_MIN = TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;
     u32x4 q[2];
-    unsigned short d[2];
+    u32 qh[2];
+    u32 dm[2];   // fp16 d in the low half, fp16 m above it (HAS_MIN)
     __device__ __forceinline__ void fetch(const uint8_t *__restrict__ W, const row_layout &L, int64_t row0, int64_t N, int64_t k0, int tid) {
 #pragma unroll
         for (int it = 0; it < 2; it++) {
@@ -190,27 +202,50 @@ template <> struct mmq_wregs<MI355_Q4_0> {
             const uint8_t *wrow = W + row * L.row_bytes;
             const int64_t blk = (k0 >> 5) + b;
             q[it] = load16(wrow + blk * 16);
-            d[it] = *(const unsigned short *)(wrow + L.off_b + blk * 2);
+            if constexpr (HAS_QH) qh[it] = *(const u32 *)(wrow + L.off_b + blk * 4);
+            const int so = HAS_QH ? L.off_c : L.off_b;   // the scales follow the fifth bits where there are any
+            if constexpr (HAS_MIN) dm[it] = *(const u32 *)(wrow + so + blk * 4);
+            else dm[it] = *(const unsigned short *)(wrow + so + blk * 2);
         }
     }
-    __device__ __forceinline__ void commit(int8_t *sW, float *sWs, int tid) const {
+    __device__ __forceinline__ void commit(int8_t *sW, float *sWs, _Float16 *sWo, int tid) const {
 #pragma unroll
         for (int it = 0; it < 2; it++) {
             const int idx = tid + it * 256;
             const int r = idx >> 2, b = idx & 3;
             u32x4 lo, hi;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {   // nibble - 8 per byte without cross-byte borrow
-                lo[i] = (((q[it][i] & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-                hi[i] = ((((q[it][i] >> 4) & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+            for (int i = 0; i < 4; i++) {
+                u32 a = q[it][i] & 0x0F0F0F0Fu, c = (q[it][i] >> 4) & 0x0F0F0F0Fu;
+                if constexpr (HAS_QH) {   // bit j of qh: element j; dword i holds elements 4i.. (low nibbles) and 16 + 4i.. (high)
+                    a |= spread4(qh[it] >> (4 * i));
+                    c |= spread4(qh[it] >> (16 + 4 * i));
+                }
+                if constexpr (TYPE == MI355_Q4_0) {          // nibble - 8 per byte without cross-byte borrow
+                    a = ((a | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+                    c = ((c | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+                } else if constexpr (TYPE == MI355_Q5_0) {   // level - 16
+                    a = ((a | 0x80808080u) - 0x10101010u) ^ 0x80808080u;
+                    c = ((c | 0x80808080u) - 0x10101010u) ^ 0x80808080u;
+                } else if constexpr (TYPE == MI355_IQ4_NL) {
+                    a = iq4nl_lookup4(a);
+                    c = iq4nl_lookup4(c);
+                }
+                lo[i] = a;
+                hi[i] = c;
             }
             *(u32x4 *)(sW + r * MMQ_LDK + b * 32) = lo;
             *(u32x4 *)(sW + r * MMQ_LDK + b * 32 + 16) = hi;
-            sWs[b * MMQ_BM + r] = half_bits_to_float(d[it]);
+            sWs[b * MMQ_BM + r] = half_bits_to_float((unsigned short)(dm[it] & 0xFFFFu));
+            if constexpr (HAS_MIN) {
+                union { unsigned short u; _Float16 f; } m;
+                m.u = (unsigned short)(dm[it] >> 16);
+                sWo[r * 4 + b] = m.f;
+            }
         }
     }
 };
-template <> struct mmq_wregs<MI355_Q8_0> {
+template <> struct mmq_wregs<MI355_Q8_0, false> {
     u32x4 q[4];
     unsigned short d[4];
     __device__ __forceinline__ void fetch(const uint8_t *__restrict__ W, const row_layout &L, int64_t row0, int64_t N, int64_t k0, int tid) {
@@ -224,7 +259,7 @@ template <> struct mmq_wregs<MI355_Q8_0> {
             d[it] = *(const unsigned short *)(wrow + L.off_b + ((k0 >> 5) + (c >> 1)) * 2);   // both pieces of a block read its scale
         }
     }
-    __device__ __forceinline__ void commit(int8_t *sW, float *sWs, int tid) const {
+    __device__ __forceinline__ void commit(int8_t *sW, float *sWs, _Float16 *, int tid) const {
 #pragma unroll
         for (int it = 0; it < 4; it++) {
             const int idx = tid + it * 256;
@@ -234,10 +269,11 @@ template <> struct mmq_wregs<MI355_Q8_0> {
         }
     }
 };
-template <int BN> struct mmq_aregs {
+template <int BN, bool WITH_SUM> struct mmq_aregs {
     static constexpr int NQ = BN * 8 / 256, NS = (BN * 4 + 255) / 256;
     u32x4 q[NQ];
     float d[NS];
+    int sum[NS];
     __device__ __forceinline__ void fetch(const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int64_t col0, int64_t B, int64_t K, int64_t k0,
                                           int tid) {
         const int64_t nblk = K >> 5;
@@ -253,10 +289,12 @@ template <int BN> struct mmq_aregs {
             const int idx = tid + it * 256;
             const int r = (idx >> 2) < BN ? (idx >> 2) : BN - 1, b = idx & 3;
             const int64_t col = col0 + r < B ? col0 + r : B - 1;
-            d[it] = ads[col * nblk + (k0 >> 5) + b].d;
+            const act_ds e = ads[col * nblk + (k0 >> 5) + b];
+            d[it] = e.d;
+            if constexpr (WITH_SUM) sum[it] = e.sum;
         }
     }
-    __device__ __forceinline__ void commit(int8_t *sA, float *sAd, int tid) const {
+    __device__ __forceinline__ void commit(int8_t *sA, float *sAd, _Float16 *sAs, int tid) const {
 #pragma unroll
         for (int it = 0; it < NQ; it++) {
             const int idx = tid + it * 256;
@@ -266,7 +304,10 @@ template <int BN> struct mmq_aregs {
 #pragma unroll
         for (int it = 0; it < NS; it++) {
             const int idx = tid + it * 256;
-            if (idx < BN * 4) sAd[(idx & 3) * BN + (idx >> 2)] = d[it];
+            if (idx < BN * 4) {
+                sAd[(idx & 3) * BN + (idx >> 2)] = d[it];
+                if constexpr (WITH_SUM) sAs[idx] = (_Float16)(d[it] * (float)sum[it]);   // [row][block of the stage]
+            }
         }
     }
 };
@@ -282,8 +323,8 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
     __shared__ __attribute__((aligned(16))) int8_t sA[BN * MMQ_LDK];
     __shared__ __attribute__((aligned(16))) float sWs[C::NG * MMQ_BM];
     __shared__ __attribute__((aligned(16))) float sAd[4 * BN];
-    __shared__ __attribute__((aligned(16))) _Float16 sWo[TYPE == MI355_Q4_K ? MMQ_BM * 4 : 4];
-    __shared__ __attribute__((aligned(16))) _Float16 sAs[TYPE == MI355_Q4_K ? BN * 4 : 4];
+    __shared__ __attribute__((aligned(16))) _Float16 sWo[C::MIN ? MMQ_BM * 4 : 4];
+    __shared__ __attribute__((aligned(16))) _Float16 sAs[C::MIN ? BN * 4 : 4];
 
     // XCD-aware id: hardware deals group ids round-robin over 8 XCDs; make logical neighbours share an XCD
     const int per_xcd = n_groups_padded >> 3;
@@ -311,9 +352,9 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
     const int64_t k_hi = k_lo + st_per * MMQ_BK < K ? k_lo + st_per * MMQ_BK : K;
     if (gridDim.y > 1) dst += (int64_t)blockIdx.y * B * dst_stride;
 
-    constexpr bool PREFETCH = TYPE == MI355_Q4_0 || TYPE == MI355_Q8_0;
+    constexpr bool PREFETCH = C::PREFETCH;
     mmq_wregs<TYPE> wregs;
-    mmq_aregs<BN> aregs;
+    mmq_aregs<BN, C::MIN> aregs;
     if constexpr (PREFETCH) {
         wregs.fetch(W, L, row0, N, k_lo, threadIdx.x);
         aregs.fetch(aq, ads, col0, B, K, k_lo, threadIdx.x);
@@ -321,8 +362,8 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
     for (int64_t k0 = k_lo; k0 < k_hi; k0 += MMQ_BK) {
         __syncthreads();
         if constexpr (PREFETCH) {
-            wregs.commit(sW, sWs, threadIdx.x);
-            aregs.commit(sA, sAd, threadIdx.x);
+            wregs.commit(sW, sWs, sWo, threadIdx.x);
+            aregs.commit(sA, sAd, sAs, threadIdx.x);
         } else {
             load_weight_stage<TYPE>(W, L, row0, N, k0, sW, sWs, sWo);
             load_act_stage<TYPE, BN>(aq, ads, col0, B, K, k0, sA, sAd, sAs);
@@ -389,15 +430,15 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
             }
         }
 
-        if constexpr (TYPE == MI355_Q4_K) {
-            // acc -= sum_b (dx*sum q)[i][b] * (dmin*m)[j][b] over the 4 blocks of the stage:
+        if constexpr (C::MIN) {
+            // acc -= sum_b (dx*sum q)[i][b] * (dmin*m)[j][b] over the 4 blocks of the stage (Q4_K; Q4_1 and Q5_1: acc += ... * m[j][b]):
             // a 32x32x16 f16 MFMA whose k slots 0..3 hold the blocks (lanes 32..63 and slots 4..7 are zero)
             f16x8 af[TN], bf[2];
 #pragma unroll
             for (int tb = 0; tb < TN; tb++) {
                 const f16x4 v = *(const f16x4 *)(sAs + (wcol0 + tb * 32 + l32) * 4);
 #pragma unroll
-                for (int i = 0; i < 8; i++) af[tb][i] = (i < 4 && lhi == 0) ? (_Float16)(-(float)v[i & 3]) : (_Float16)0.0f;
+                for (int i = 0; i < 8; i++) af[tb][i] = (i < 4 && lhi == 0) ? (TYPE == MI355_Q4_K ? (_Float16)(-(float)v[i & 3]) : v[i & 3]) : (_Float16)0.0f;
             }
 #pragma unroll
             for (int tw = 0; tw < 2; tw++) {
@@ -496,7 +537,7 @@ extern "C" int mi355_mul_mat_q(void *stream, int type, const void *W, const void
 
 extern "C" int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
                                   int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q: unsupported weight type %d", type);
+    MI355_REQUIRE(is_weight_type(type) && type != MI355_Q5_K, "mul_mat_q: unsupported weight type %d", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_q: K=%lld is not a multiple of the block size", (long long)K);
     MI355_REQUIRE(dst_stride >= N, "mul_mat_q: dst_stride < N");
@@ -510,6 +551,10 @@ extern "C" int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const v
         case MI355_Q4_0: launch_mmq_tn<MI355_Q4_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q8_0: launch_mmq_tn<MI355_Q8_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q4_K: launch_mmq_tn<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_Q4_1: launch_mmq_tn<MI355_Q4_1>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_Q5_0: launch_mmq_tn<MI355_Q5_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_Q5_1: launch_mmq_tn<MI355_Q5_1>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_IQ4_NL: launch_mmq_tn<MI355_IQ4_NL>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         default: launch_mmq_tn<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
     }
     return launch_status("k_mmq");
