@@ -138,6 +138,21 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     v = dpp_add<0x143, 0xC>(v);   // row_bcast31 into rows 2 and 3: lane 63 holds the total
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// Maximum over the 64 lanes the same way (rows that a step does not write keep their value)
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_max(float v) {
+    const int b = __builtin_bit_cast(int, v);
+    return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, CTRL, ROWMASK, 0xF, false)));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+    v = dpp_max<0xB1, 0xF>(v);
+    v = dpp_max<0x4E, 0xF>(v);
+    v = dpp_max<0x141, 0xF>(v);
+    v = dpp_max<0x140, 0xF>(v);
+    v = dpp_max<0x142, 0xA>(v);
+    v = dpp_max<0x143, 0xC>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));

@@ -223,46 +223,69 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     }
 }
 
-// Merge of the kv splits: threads first turn the per-split (max, sum) pairs into weights in LDS
-// (one split per thread), then every thread owns one output element and sums the partial
-// outputs with independent, coalesced loads.
+// Merge of the kv splits, one 512-thread group per (token, head).  The partial results were written by other compute units a
+// moment ago, so every load is a trip to memory: a thread asks for its split's (max, sum) pair and for the first sixteen partial
+// outputs of its element before it uses any of them.  Thread tid owns element tid % D and the splits tid / D, tid / D + PARTS, ...
+// (PARTS = 512 / D); the parts are added through LDS.
 template <int D>
-__global__ void __launch_bounds__(256) k_fattn_combine(const float *__restrict__ ws, float *__restrict__ dst, int n_splits, int8_t *__restrict__ act_q,
+__global__ void __launch_bounds__(512) k_fattn_combine(const float *__restrict__ ws, float *__restrict__ dst, int n_splits, int8_t *__restrict__ act_q,
                                                        act_ds *__restrict__ act_s, int64_t Hq) {
+    constexpr int PARTS = 512 / D, U = 16;
     __shared__ float s_w[256];
-    __shared__ float s_red[8];
+    __shared__ float s_red[16];
+    __shared__ float s_o[PARTS][D];
     const int64_t row = blockIdx.x;   // iq * Hq + head
     const float *p = ws + row * n_splits * (D + 2);
-    const int tid = threadIdx.x;
-    const int nw = blockDim.x >> 6;
+    const int tid = threadIdx.x, d = tid % D, part = tid / D;
+    const bool live = part < PARTS;   // head sizes that do not divide 512 leave the last threads without an element
     float ms = -FLT_MAX / 2, ls = 0.0f;
     if (tid < n_splits) {
         ms = p[tid * (D + 2) + D];
         ls = p[tid * (D + 2) + D + 1];
     }
-    float M = wave_max(ms);
+    float v[U];
+#pragma unroll
+    for (int i = 0; i < U; i++) {
+        const int sidx = part + PARTS * i;
+        v[i] = live && sidx < n_splits ? p[sidx * (D + 2) + d] : 0.0f;
+    }
+    float M = wave_max_dpp(ms);
     if ((tid & 63) == 0) s_red[tid >> 6] = M;
     __syncthreads();
     M = s_red[0];
-    for (int i = 1; i < nw; i++) M = fmaxf(M, s_red[i]);
+#pragma unroll
+    for (int i = 1; i < 8; i++) M = fmaxf(M, s_red[i]);
     const float w = tid < n_splits ? __expf(ms - M) : 0.0f;
-    s_w[tid] = w;
-    float L = wave_sum(ls * w);
-    if ((tid & 63) == 0) s_red[4 + (tid >> 6)] = L;
+    if (tid < 256) s_w[tid] = w;
+    float L = wave_sum_dpp(ls * w);
+    if ((tid & 63) == 0) s_red[8 + (tid >> 6)] = L;
     __syncthreads();
-    L = s_red[4];
-    for (int i = 1; i < nw; i++) L += s_red[4 + i];
-    for (int d = tid; d < D; d += blockDim.x) {
-        float O = 0.0f;
-        int s = 0;
-        for (; s + 8 <= n_splits; s += 8) {
-            float v[8];
+    L = s_red[8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = p[(s + i) * (D + 2) + d];
+    for (int i = 1; i < 8; i++) L += s_red[8 + i];
+    float O = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) O += v[i] * s_w[s + i];
+    for (int i = 0; i < U; i++) {
+        const int sidx = part + PARTS * i;
+        if (sidx < n_splits) O += v[i] * s_w[sidx];
+    }
+    for (int s0 = PARTS * U; s0 < n_splits; s0 += PARTS * U) {   // more than PARTS * 16 splits
+#pragma unroll
+        for (int i = 0; i < U; i++) {
+            const int sidx = s0 + part + PARTS * i;
+            v[i] = live && sidx < n_splits ? p[sidx * (D + 2) + d] : 0.0f;
         }
-        for (; s < n_splits; s++) O += p[s * (D + 2) + d] * s_w[s];
+#pragma unroll
+        for (int i = 0; i < U; i++) {
+            const int sidx = s0 + part + PARTS * i;
+            if (sidx < n_splits) O += v[i] * s_w[sidx];
+        }
+    }
+    if (live) s_o[part][d] = O;
+    __syncthreads();
+    if (part == 0) {   // threads 0 .. D - 1: whole 32-lane runs where the output is also quantized (D % 32 == 0 then)
+#pragma unroll
+        for (int i = 1; i < PARTS; i++) O += s_o[i][d];
         const float o = O / L;
         dst[row * D + d] = o;
         if (act_q) {
@@ -310,7 +333,7 @@ static int launch_vec(hipStream_t s, fattn_args &a) {
     int rc = launch_status("k_fattn_vec");
     if (rc != MI355_OK) return rc;
     if (a.n_splits > 1) {
-        MI355_LAUNCH(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(256), 0, s, a.ws, a.dst, a.n_splits, a.act_q,
+        MI355_LAUNCH(k_fattn_combine<D>, dim3((unsigned)(a.Nq * a.Hq)), dim3(512), 0, s, a.ws, a.dst, a.n_splits, a.act_q,
                            a.act_s, a.Hq);
         rc = launch_status("k_fattn_combine");
     }
@@ -394,6 +417,19 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
     // bytes once for its whole GQA group.  Short contexts are latency-bound and mostly padding (-inf mask): the
     // vector kernel, which skips masked cells before touching K/V, is quicker there.
     constexpr int64_t dec_min = 256;
+    // One token over a long cache (head size 128, up to four query heads per kv head): the per-wave streaming kernel.  Measured on
+    // the 32-over-8-head shape: 12.2 us against 13.7 at 4096 cells, 36 against 41 at 32768, 105 against 117 at 131072; below about
+    // 3000 cells fewer than 512 of its 64-cell tiles exist and the kernel below is ahead (10.2 against 11.2 us at 2048).
+    static const int64_t stream_min = getenv("MI355_FA_STREAM_MIN") ? atoll(getenv("MI355_FA_STREAM_MIN")) : 3072;
+    if (Nq == 1 && Nkv > stream_min && D == 128 && R <= 4 && ws != nullptr) {
+        fattn_args b = a;
+        const int rc = launch_fattn_dec_stream(s, b, D, ws_bytes);
+        if (rc < 0) return rc;
+        if (rc == 0) {
+            MI355_LAUNCH(k_fattn_combine<128>, dim3((unsigned)(Nq * Hq)), dim3(512), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq);
+            return launch_status("k_fattn_combine");
+        }
+    }
     if (Nq < 16 && Nkv > dec_min && (D == 64 || D == 128) && R <= 32) {
         fattn_args b = a;
         // enough splits to put about two groups on every CU; a split is a whole number of 64-cell tiles
@@ -413,8 +449,8 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
         if (rc == 0) {
             if (b.n_splits > 1) {
                 switch (D) {
-                    case 64: MI355_LAUNCH(k_fattn_combine<64>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
-                    default: MI355_LAUNCH(k_fattn_combine<128>, dim3((unsigned)(Nq * Hq)), dim3(256), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
+                    case 64: MI355_LAUNCH(k_fattn_combine<64>, dim3((unsigned)(Nq * Hq)), dim3(512), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
+                    default: MI355_LAUNCH(k_fattn_combine<128>, dim3((unsigned)(Nq * Hq)), dim3(512), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq); break;
                 }
                 return launch_status("k_fattn_combine");
             }

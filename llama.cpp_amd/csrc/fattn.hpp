@@ -28,4 +28,8 @@ int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);
 // the same for a few query rows (decode): one kv split per group, partials merged by k_fattn_combine
 int launch_fattn_mma_dec(hipStream_t s, fattn_args &a, int64_t D);
 
+// one query token over a long f16 cache, head size 128, up to four query heads per kv head: per-wave streaming through LDS
+// (fattn_stream.hip); sets a.n_splits for k_fattn_combine; returns 1 when the shape is not served
+int launch_fattn_dec_stream(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);
+
 }  // namespace mi355

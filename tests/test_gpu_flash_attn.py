@@ -123,6 +123,38 @@ def test_llama3_shapes(dev, Nq, Nkv):
         assert orc.nmse(got[rows][:, h:h + 1], cpu) <= 5e-4
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 2), (4, 4), (6, 3), (3, 1)])
+@pytest.mark.parametrize("Nkv", [3073, 3500, 4096, 5000, 40000])
+def test_decode_streaming_kernel(dev, Hq, Hkv, Nkv):
+    """One query token over more than 3072 cells, head size 128, up to four query heads per kv head: the per-wave streaming kernel
+    (global-to-LDS ring, 4 x 4 x 4 matrix instructions with one cell per lane).  Cell counts that are not multiples of the 64-cell
+    tile, masks with -inf holes and finite biases, every head grouping up to four; against the textbook form in f64 and the
+    oracle's restatement of the reference CPU kernel."""
+    rng = np.random.default_rng(Nkv + Hq)
+    q, k, v, mask = _inputs(rng, 128, 1, Nkv, Hq, Hkv, causal=True, rand_mask=True)
+    q = q * 2.0
+    holes = rng.random(Nkv) < 0.2
+    mask[:, holes] = -np.inf
+    mask[:, 64:192] = -np.inf                  # two whole tiles masked
+    scale = 1.0 / np.sqrt(128)
+    got = _run(dev, q, k, v, mask, scale, llama_layout=True)
+    assert np.isfinite(got).all()
+    f64 = orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale)
+    assert orc.nmse(got, f64) < 1e-5
+    if Nkv <= 5000:
+        assert orc.nmse(got, orc.flash_attn("cpu", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale)) <= 5e-4
+
+
+@pytest.mark.parametrize("max_bias,softcap,use_mask", [(8.0, 0.0, True), (0.0, 10.0, True), (0.0, 0.0, False)])
+def test_decode_streaming_kernel_alibi_softcap_no_mask(dev, max_bias, softcap, use_mask):
+    rng = np.random.default_rng(23)
+    q, k, v, mask = _inputs(rng, 128, 1, 3300, 12, 4, causal=False, rand_mask=True)
+    m = mask if use_mask else None
+    got = _run(dev, q, k, v, m, 0.09, max_bias, softcap)
+    f64 = orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), m.view(np.uint16) if use_mask else None, 0.09, max_bias, softcap)
+    assert orc.nmse(got, f64) < 1e-5
+
+
 @pytest.mark.parametrize("D,Nq,Nkv,Hq,Hkv", [(128, 1, 256, 32, 8), (128, 1, 4096, 32, 8), (128, 5, 700, 8, 2), (64, 2, 96, 6, 3), (96, 1, 64, 4, 4)])
 def test_quantized_output_matches_separate_quantization(dev, D, Nq, Nkv, Hq, Hkv):
     """the Q8_1 rows attention emits equal mi355_quantize_act of its own f32 output, bit for bit (kv split or not)"""
