@@ -43,7 +43,6 @@ __device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
     return s;
 }
 
-__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e);
 
 
 // NW: waves per group
@@ -295,27 +294,6 @@ __global__ void __launch_bounds__(512) k_fattn_combine(const float *__restrict__
     }
 }
 
-// Q8_1 of one value per lane, 32 consecutive lanes = one block (quantize_row_q8_1_ref,
-// ggml/src/ggml-quants.c:220-253); e = element index inside the query row of k elements
-__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
-    float amax = fabsf(v);
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-    const float d = amax / 127.0f;
-    const float id = d != 0.0f ? 1.0f / d : 0.0f;
-    const int q = (int)roundf(v * id);
-    int sum = q;
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    qrow[e] = (int8_t)q;
-    if ((e & 31) == 0) {
-        act_ds o;
-        o.d = half_bits_to_float(float_to_half_bits(d));
-        o.sum = sum;
-        srow[e >> 5] = o;
-    }
-}
-
 static int pick_splits(int64_t Nkv, int64_t Hkv, int64_t Nq) {
     int64_t by_len = (Nkv + 255) / 256;
     int64_t by_fill = 2048 / (Hkv * Nq > 0 ? Hkv * Nq : 1);
@@ -421,6 +399,14 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
     // the 32-over-8-head shape: 12.2 us against 13.7 at 4096 cells, 36 against 41 at 32768, 105 against 117 at 131072; below about
     // 3000 cells fewer than 512 of its 64-cell tiles exist and the kernel below is ahead (10.2 against 11.2 us at 2048).
     static const int64_t stream_min = getenv("MI355_FA_STREAM_MIN") ? atoll(getenv("MI355_FA_STREAM_MIN")) : 3072;
+    // 257 .. 512 cells: one launch with a wave per 64 cells (8.4 / 8.6 us at 384 / 512 cells against 9.0 for the split form below
+    // with its merge launch; up to 256 cells the vector kernel further down is ahead, 6.8 against 7.1 us)
+    static const int64_t short_min = getenv("MI355_FA_SHORT_MIN") ? atoll(getenv("MI355_FA_SHORT_MIN")) : 256;
+    static const int64_t short_max = getenv("MI355_FA_SHORT_MAX") ? atoll(getenv("MI355_FA_SHORT_MAX")) : 512;
+    if (Nq == 1 && Nkv > short_min && Nkv <= short_max && D == 128 && R <= 4) {
+        const int rc = launch_fattn_dec_short(s, a, D);
+        if (rc <= 0) return rc;
+    }
     if (Nq == 1 && Nkv > stream_min && D == 128 && R <= 4 && ws != nullptr) {
         fattn_args b = a;
         const int rc = launch_fattn_dec_stream(s, b, D, ws_bytes);

@@ -23,11 +23,35 @@ struct fattn_args {
     int64_t cells_per_split;
 };
 
+// Q8_1 of one value per lane, 32 consecutive lanes = one block (quantize_row_q8_1_ref,
+// ggml/src/ggml-quants.c:220-253); e = element index inside the query row of k elements
+__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q = (int)roundf(v * id);
+    int sum = q;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    qrow[e] = (int8_t)q;
+    if ((e & 31) == 0) {
+        act_ds o;
+        o.d = half_bits_to_float(float_to_half_bits(d));
+        o.sum = sum;
+        srow[e >> 5] = o;
+    }
+}
+
 // f16 matrix-core kernel for many query rows; returns MI355_OK, an error, or 1 when the shape is not served
 int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);
 // the same for a few query rows (decode): one kv split per group, partials merged by k_fattn_combine
 int launch_fattn_mma_dec(hipStream_t s, fattn_args &a, int64_t D);
 
+// one query token over at most 512 cells of an f16 cache, head size 128, up to four query heads per kv head: one launch, one wave
+// per 64 cells, states merged in LDS (fattn_stream.hip); returns 1 when the shape is not served
+int launch_fattn_dec_short(hipStream_t s, fattn_args &a, int64_t D);
 // one query token over a long f16 cache, head size 128, up to four query heads per kv head: per-wave streaming through LDS
 // (fattn_stream.hip); sets a.n_splits for k_fattn_combine; returns 1 when the shape is not served
 int launch_fattn_dec_stream(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);

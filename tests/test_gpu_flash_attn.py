@@ -145,6 +145,25 @@ def test_decode_streaming_kernel(dev, Hq, Hkv, Nkv):
         assert orc.nmse(got, orc.flash_attn("cpu", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale)) <= 5e-4
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (4, 4), (6, 3), (3, 1)])
+@pytest.mark.parametrize("Nkv", [257, 300, 449, 511, 512])
+@pytest.mark.parametrize("max_bias,softcap", [(0.0, 0.0), (8.0, 0.0), (0.0, 10.0)])
+def test_decode_short_kernel(dev, Hq, Hkv, Nkv, max_bias, softcap):
+    """One query token over 257 .. 512 cells, head size 128, up to four query heads per kv head: the one-launch kernel (a wave per
+    64-cell tile, K rows straight into registers, states merged in LDS).  Partial last tiles, -inf holes, finite biases, ALiBi
+    slopes and the logit soft-cap; against the textbook form in f64 and the oracle's restatement of the reference CPU kernel."""
+    rng = np.random.default_rng(Nkv + Hq)
+    q, k, v, mask = _inputs(rng, 128, 1, Nkv, Hq, Hkv, causal=True, rand_mask=True)
+    mask[:, rng.random(Nkv) < 0.3] = -np.inf
+    mask[:, Nkv - 1] = 0.25                # the one cell of a last tile stays live
+    scale = 1.0 / np.sqrt(128)
+    got = _run(dev, q, k, v, mask, scale, max_bias, softcap, llama_layout=True)
+    assert np.isfinite(got).all()
+    f64 = orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale, max_bias, softcap)
+    assert orc.nmse(got, f64) < 1e-5
+    assert orc.nmse(got, orc.flash_attn("cpu", q, k.view(np.uint16), v.view(np.uint16), mask.view(np.uint16), scale, max_bias, softcap)) <= 5e-4
+
+
 @pytest.mark.parametrize("max_bias,softcap,use_mask", [(8.0, 0.0, True), (0.0, 10.0, True), (0.0, 0.0, False)])
 def test_decode_streaming_kernel_alibi_softcap_no_mask(dev, max_bias, softcap, use_mask):
     rng = np.random.default_rng(23)
