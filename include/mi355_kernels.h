@@ -99,9 +99,9 @@ int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64
  * GEMV for up to 8 rows and the wide-tile GEMM on tile images (mi355_kq_unpack_tiles + mi355_mul_mat_q8k_tiled) for batches;
  * this entry point, which has no tile image to go by, runs Q5_K batches through the GEMV eight rows at a time.
  * Q4_1, Q5_0, Q5_1 and IQ4_NL (ggml/src/ggml-common.h:168-201, 399-404; ggml_vec_dot_q4_1_q8_1, _q5_0_q8_0, _q5_1_q8_1 and
- * _iq4_nl_q8_0, ggml/src/ggml-cpu/ggml-cpu-quants.c:2511, 2804, 3159, 11188) have the single-matrix GEMV for up to 8 rows and
- * the per-32-block int8-MFMA tile kernel (mi355_mul_mat_q) beyond; the launches that take several matrices or fuse an epilogue
- * and the weight-streaming kernel for 5..32 rows are built for Q4_0, Q8_0, Q4_K, Q5_K and Q6_K only.
+ * _iq4_nl_q8_0, ggml/src/ggml-cpu/ggml-cpu-quants.c:2511, 2804, 3159, 11188) have the GEMV for up to 8 rows (also in the
+ * launches that take several matrices or fuse an epilogue) and the per-32-block int8-MFMA tile kernel (mi355_mul_mat_q) beyond;
+ * the weight-streaming kernel for 5..32 rows is built for Q4_0, Q8_0, Q4_K and Q6_K only.
  * `ws` is scratch of at least mi355_mul_mat_ws_bytes(K, B) bytes. */
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,

@@ -50,14 +50,13 @@
 namespace {
 
 // ------------------------------------------------------------------------------- helpers
-// types whose products the fused launches (several matrices per launch, epilogues, matrix-core kernels) are built for ...
-bool is_fused_weight_type(ggml_type t) {
-    return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K;
+// types whose batches of 5..32 rows have the weight-streaming matrix-core kernel; the others stay with the GEMV up to 8 rows
+bool has_skinny_kernel(ggml_type t) { return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q6_K; }
+bool is_repacked_type(ggml_type t) {
+    return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K || t == GGML_TYPE_Q4_1 || t == GGML_TYPE_Q5_0 || t == GGML_TYPE_Q5_1 ||
+           t == GGML_TYPE_IQ4_NL;
 }
-// ... and those served one product at a time by mi355_mul_mat / mi355_mul_mat_id / mi355_get_rows
-bool is_plain_weight_type(ggml_type t) { return t == GGML_TYPE_Q4_1 || t == GGML_TYPE_Q5_0 || t == GGML_TYPE_Q5_1 || t == GGML_TYPE_IQ4_NL; }
-bool is_repacked_type(ggml_type t) { return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K || is_plain_weight_type(t); }
-bool is_weight_type(ggml_type t) { return is_fused_weight_type(t) || is_plain_weight_type(t); }
+bool is_weight_type(ggml_type t) { return is_repacked_type(t) || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K; }
 
 int to_mi355_type(ggml_type t) {
     switch (t) {
@@ -1052,10 +1051,10 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
     // kernels; from there to 32: the weight-streaming matrix-core kernel)
     const ggml_tensor * a = mm->src[0];
     const ggml_tensor * b = mm->src[1];
-    if (mm->op != GGML_OP_MUL_MAT || !is_fused_weight_type(a->type)) return false;
+    if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
     if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
-    if (a->type == GGML_TYPE_Q5_K && b->ne[1] > 8) return false;    // Q5_K: the GEMV only (up to eight rows); more rows take the generic path
+    if (!has_skinny_kernel(a->type) && b->ne[1] > 8) return false;    // the GEMV only (up to eight rows); more rows take the generic path
     const int64_t K = a->ne[0];
     if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)
@@ -1345,7 +1344,7 @@ prefill_qkv match_prefill_qkv(const graph_walk & w, int i) {
     const ggml_tensor * b = mq->src[1];
     const int64_t B = b->ne[1];
     auto product_ok = [&](const ggml_tensor * m, int idx) {
-        return m->op == GGML_OP_MUL_MAT && is_fused_weight_type(m->src[0]->type) && m->src[0]->ne[2] == 1 && m->src[0]->ne[3] == 1 && m->src[1] == b &&
+        return m->op == GGML_OP_MUL_MAT && is_weight_type(m->src[0]->type) && m->src[0]->ne[2] == 1 && m->src[0]->ne[3] == 1 && m->src[1] == b &&
                b->ne[2] == 1 && b->ne[3] == 1 && ggml_is_contiguous(m) && m->type == GGML_TYPE_F32 && w.sole_use(idx);
     };
     // the ROPE that reads product m, directly or through a RESHAPE nobody else reads

@@ -55,13 +55,9 @@ __host__ __device__ inline int type_block_bytes(int t) {
         default: return 0;
     }
 }
-// types the kernels that choose the weight type at run time (several matrices per launch, fused epilogues) are built for
-__host__ __device__ inline bool is_fused_weight_type(int t) {
-    return t == MI355_Q4_0 || t == MI355_Q8_0 || t == MI355_Q4_K || t == MI355_Q5_K || t == MI355_Q6_K;
-}
-// ... and those served by the single-matrix kernels, whose type is a template parameter
 __host__ __device__ inline bool is_weight_type(int t) {
-    return is_fused_weight_type(t) || t == MI355_Q4_1 || t == MI355_Q5_0 || t == MI355_Q5_1 || t == MI355_IQ4_NL;
+    return t == MI355_Q4_0 || t == MI355_Q8_0 || t == MI355_Q4_K || t == MI355_Q5_K || t == MI355_Q6_K || t == MI355_Q4_1 || t == MI355_Q5_0 ||
+           t == MI355_Q5_1 || t == MI355_IQ4_NL;
 }
 // Expands X(TYPE) for the weight type t (checked with is_weight_type before).
 #define MI355_WEIGHT_TYPE_SWITCH(t, X)            \

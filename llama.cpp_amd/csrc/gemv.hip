@@ -204,13 +204,9 @@ extern __shared__ __attribute__((aligned(16))) uint8_t s_act_dyn[];
 template <int NCOLS, int RPW, bool COH = false, bool LDSA = false>
 __device__ __forceinline__ void gemv_dispatch(const gemv_item &m, int group, const int8_t *__restrict__ aq,
                                               const act_ds *__restrict__ ads, int K) {
-    switch (m.type) {   // uniform over the group
-        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
-        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
-        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
-        case MI355_Q5_K: gemv_body<MI355_Q5_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
-        default: gemv_body<MI355_Q6_K, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn); break;
-    }
+#define MI355_BODY(TY) gemv_body<TY, NCOLS, RPW, false, COH, LDSA>(m, group, aq, ads, K, nullptr, s_act_dyn);
+    MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)   // uniform over the group
+#undef MI355_BODY
 }
 
 // Q, K and V projections in one launch; finished rows are rotated and land in q (f32) or in the f16 KV cache
@@ -223,13 +219,9 @@ __global__ void __launch_bounds__(256) k_gemv_qkv(gemv_batch b, const int8_t *__
         if (g >= b.it[j].first_group) i = j;   // unused items start at INT_MAX
     const gemv_item &m = b.it[i];
     const int group = g - m.first_group;
-    switch (m.type) {   // uniform over the group
-        case MI355_Q4_0: gemv_body<MI355_Q4_0, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
-        case MI355_Q8_0: gemv_body<MI355_Q8_0, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
-        case MI355_Q4_K: gemv_body<MI355_Q4_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
-        case MI355_Q5_K: gemv_body<MI355_Q5_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
-        default: gemv_body<MI355_Q6_K, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn); break;
-    }
+#define MI355_BODY(TY) gemv_body<TY, NCOLS, 2, true, false, LDSA>(m, group, aq, ads, K, &rp, s_act_dyn);
+    MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)   // uniform over the group
+#undef MI355_BODY
 }
 
 // single matrix, type known at compile time (smallest code, used by mi355_mul_mat_vec_q)
@@ -247,13 +239,9 @@ __global__ void __launch_bounds__(256) k_gemv_qkv_norm(gemv_batch b, int K, gemv
         if (g >= b.it[j].first_group) i = j;
     const gemv_item &m = b.it[i];
     const int group = g - m.first_group;
-    switch (m.type) {
-        case MI355_Q4_0: gemv_body<MI355_Q4_0, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
-        case MI355_Q8_0: gemv_body<MI355_Q8_0, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
-        case MI355_Q4_K: gemv_body<MI355_Q4_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
-        case MI355_Q5_K: gemv_body<MI355_Q5_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
-        default: gemv_body<MI355_Q6_K, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn); break;
-    }
+#define MI355_BODY(TY) gemv_body<TY, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn);
+    MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)
+#undef MI355_BODY
 }
 
 // several matrices sharing one activation
@@ -487,8 +475,8 @@ static void launch_single_cols(int rpw, int64_t B, hipStream_t s, const gemv_ite
     }
 }
 
-static int check_gemv_args(const char *who, int type, const void *W, int64_t N, int64_t K, int64_t dst_stride, bool fused_only = false) {
-    MI355_REQUIRE(fused_only ? is_fused_weight_type(type) : is_weight_type(type), "%s: unsupported weight type %d", who, type);
+static int check_gemv_args(const char *who, int type, const void *W, int64_t N, int64_t K, int64_t dst_stride) {
+    MI355_REQUIRE(is_weight_type(type), "%s: unsupported weight type %d", who, type);
     MI355_REQUIRE(N > 0 && K > 0 && K < (int64_t(1) << 30), "%s: bad shape N=%lld K=%lld", who, (long long)N, (long long)K);
     MI355_REQUIRE(K % type_block_elems(type) == 0, "%s: K=%lld is not a multiple of the block size", who, (long long)K);
     MI355_REQUIRE(dst_stride >= N, "%s: dst_stride < N", who);
@@ -514,17 +502,6 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_vec_q: activation workspace is not 16-byte aligned");
     int64_t total_rows = 0;
     bool aligned = true;
-    if (n_mats > 1) {   // the launch that walks several matrices chooses the type at run time among the fused set only
-        bool fused = true;
-        for (int i = 0; i < n_mats; i++) fused = fused && is_fused_weight_type(mats[i].type);
-        if (!fused) {
-            for (int i = 0; i < n_mats; i++) {
-                int rc = mi355_mul_mat_vec_q_multi(stream, 1, mats + i, act, K, B);
-                if (rc != MI355_OK) return rc;
-            }
-            return MI355_OK;
-        }
-    }
     for (int i = 0; i < n_mats; i++) {
         MI355_REQUIRE(is_weight_type(mats[i].type) && K > 0 && K % type_block_elems(mats[i].type) == 0, "mul_mat_vec_q: unsupported type %d or K=%lld not a multiple of its block size", mats[i].type, (long long)K);
         aligned = aligned && layout_aligned(mats[i].W, make_row_layout(mats[i].type, K));
@@ -629,7 +606,7 @@ static int vec_q_rope_impl(void *stream, int n_mats, const mi355_gemv_rope_mat *
     for (int i = 0; i < 4; i++) {
         const mi355_gemv_rope_mat &m = mats[i < n_mats ? i : 0];
         if (i < n_mats) {
-            int rc = check_gemv_args("mul_mat_vec_q_rope", m.type, m.W, m.N, K, m.N, true);
+            int rc = check_gemv_args("mul_mat_vec_q_rope", m.type, m.W, m.N, K, m.N);
             if (rc != MI355_OK) return rc;
             MI355_REQUIRE(m.epilogue >= MI355_EPI_STORE && m.epilogue <= MI355_EPI_CACHE && m.dst != nullptr && m.N % 2 == 0,
                           "mul_mat_vec_q_rope: bad epilogue %d, missing destination or odd row count", m.epilogue);
@@ -742,9 +719,9 @@ int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, in
     MI355_REQUIRE(B >= 1 && B <= 4, "ffn_gate_up_swiglu: batch %lld outside 1..4", (long long)B);
     MI355_REQUIRE(N > 0 && N % 32 == 0 && out_stride >= N, "ffn_gate_up_swiglu: N=%lld must be a positive multiple of 32 and fit the row stride", (long long)N);
     MI355_REQUIRE(((uintptr_t)act & 15) == 0 && ((uintptr_t)act_out & 15) == 0 && counters != nullptr, "ffn_gate_up_swiglu: misaligned or missing operands");
-    int rc = check_gemv_args("ffn_gate_up_swiglu", type_gate, w_gate, N, K, out_stride, true);
+    int rc = check_gemv_args("ffn_gate_up_swiglu", type_gate, w_gate, N, K, out_stride);
     if (rc != MI355_OK) return rc;
-    rc = check_gemv_args("ffn_gate_up_swiglu", type_up, w_up, N, K, out_stride, true);
+    rc = check_gemv_args("ffn_gate_up_swiglu", type_up, w_up, N, K, out_stride);
     if (rc != MI355_OK) return rc;
     const int64_t per = N / 8;   // groups per matrix: 4 waves x 2 rows
     MI355_REQUIRE(2 * per < 0x7fffffff, "ffn_gate_up_swiglu: too many rows for one launch");

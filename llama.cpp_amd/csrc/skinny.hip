@@ -381,8 +381,8 @@ using namespace mi355;
 extern "C" {
 
 int mi355_mul_mat_skinny_supported(int type, const void *W, int64_t K, int64_t B) {
-    // Q5_K and the types outside the fused set have no operand unpacking in this kernel: their products stay with the GEMV
-    return is_fused_weight_type(type) && type != MI355_Q5_K && B >= 1 && B <= 32 && K > 0 && K % 256 == 0 && K < (int64_t(1) << 30) &&
+    // the other types have no operand unpacking in this kernel: their products stay with the GEMV
+    return (type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K || type == MI355_Q6_K) && B >= 1 && B <= 32 && K > 0 && K % 256 == 0 && K < (int64_t(1) << 30) &&
            layout_aligned(W, make_row_layout(type, K));
 }
 

@@ -98,12 +98,14 @@ def test_rope_kv_store(dev, mode):
 
 
 @pytest.mark.parametrize("B", [1, 3, 8])
-def test_multi_matrix_gemv_with_residual(dev, B):
+@pytest.mark.parametrize("specs", [[(orc.Q4_K, 1024), (orc.Q4_K, 512), (orc.Q6_K, 256), (orc.Q8_0, 130)],
+                                   [(orc.Q5_0, 1024), (orc.IQ4_NL, 512), (orc.Q5_1, 256), (orc.Q4_1, 130)],
+                                   [(orc.IQ4_NL, 2048), (orc.Q5_K, 640)]], ids=["k_quants_q8_0", "per_32_block_types", "iq4_nl_q5_K"])
+def test_multi_matrix_gemv_with_residual(dev, B, specs):
     import torch
     import mi355
     rng = np.random.default_rng(B)
     K = 4096
-    specs = [(orc.Q4_K, 1024), (orc.Q4_K, 512), (orc.Q6_K, 256), (orc.Q8_0, 130)]
     x = rng.standard_normal((B, K)).astype(np.float32)
     act = mi355.quantize_act(_t(dev, x))
     arr = (mi355.GemvMat * len(specs))()
@@ -158,7 +160,8 @@ def test_fused_layer_stack_matches_node_sequence(dev):
 
 
 @pytest.mark.parametrize("B", [1, 3])
-@pytest.mark.parametrize("tq,tk,tv", [(orc.Q4_K, orc.Q4_K, orc.Q6_K), (orc.Q4_0, orc.Q8_0, orc.Q4_0)])
+@pytest.mark.parametrize("tq,tk,tv", [(orc.Q4_K, orc.Q4_K, orc.Q6_K), (orc.Q4_0, orc.Q8_0, orc.Q4_0), (orc.Q5_0, orc.Q5_0, orc.Q5_1), (orc.IQ4_NL, orc.IQ4_NL, orc.Q5_K),
+                                      (orc.Q4_1, orc.Q4_1, orc.Q4_1)])
 def test_qkv_rope_store_equals_three_launch_sequence(dev, B, tq, tk, tv):
     """projections + rope + KV store in one launch give bit-identical q and cache contents"""
     import torch
