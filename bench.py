@@ -250,8 +250,6 @@ def sweep(kinds):
                         us = timed(lambda i: mi355.check(lib.mi355_mul_mat(stream.cuda_stream, t, Ws[i].data_ptr(), x.data_ptr(), out.data_ptr(), N, K, B, K, N,
                                                                            ws.data_ptr(), ws.numel())), nm, 5)
                         label = "MUL_MAT batch %d (activation quantization + tile GEMM)" % B
-                        if t == mi355.Q5_K:   # mi355_mul_mat has no tile image to go by: the GEMV, eight rows at a time
-                            label = "MUL_MAT batch %d (mi355_mul_mat: eight rows at a time through the GEMV)" % B
                         emit(kernel=label, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
                              achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
                     if t in (mi355.Q4_K, mi355.Q5_K, mi355.Q6_K):   # the wide-tile GEMM on tile images (what prefill uses for K-quants), without the quantization

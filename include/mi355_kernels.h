@@ -8,7 +8,7 @@
  *
  * Each entry point names the reference function it stands in for (paths relative to the
  * llama.cpp tree).  Element types use the reference's enum values
- * (ggml/include/ggml.h:351-392): F32 0, F16 1, Q4_0 2, Q8_0 8, Q8_1 9, Q4_K 12, Q5_K 13, Q6_K 14, I32 26.
+ * (ggml/include/ggml.h:351-392): F32 0, F16 1, Q4_0 2, Q4_1 3, Q5_0 6, Q5_1 7, Q8_0 8, Q8_1 9, Q4_K 12, Q5_K 13, Q6_K 14, IQ4_NL 20, I32 26.
  */
 #ifndef MI355_KERNELS_H
 #define MI355_KERNELS_H
@@ -96,8 +96,8 @@ int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64
  * bandwidth-bound GEMV (per-block integer dots of the weights against Q8_1 activations), up to 32
  * the weight-streaming matrix-core kernel (mi355_mul_mat_skinny), larger B the int8-MFMA tile kernels.
  * Q5_K (block_q5_K, ggml/src/ggml-common.h:296-308; ggml_vec_dot_q5_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6859-7592) has the
- * GEMV for up to 8 rows and the wide-tile GEMM on tile images (mi355_kq_unpack_tiles + mi355_mul_mat_q8k_tiled) for batches;
- * this entry point, which has no tile image to go by, runs Q5_K batches through the GEMV eight rows at a time.
+ * GEMV for up to 8 rows, the per-32-block int8-MFMA tile kernel (mi355_mul_mat_q) for batches on packed rows - what this entry
+ * point runs - and the wide-tile GEMM on tile images (mi355_kq_unpack_tiles + mi355_mul_mat_q8k_tiled) for callers that keep images.
  * Q4_1, Q5_0, Q5_1 and IQ4_NL (ggml/src/ggml-common.h:168-201, 399-404; ggml_vec_dot_q4_1_q8_1, _q5_0_q8_0, _q5_1_q8_1 and
  * _iq4_nl_q8_0, ggml/src/ggml-cpu/ggml-cpu-quants.c:2511, 2804, 3159, 11188) have the GEMV for up to 8 rows (also in the
  * launches that take several matrices or fuse an epilogue) and the per-32-block int8-MFMA tile kernel (mi355_mul_mat_q) beyond;
@@ -324,7 +324,7 @@ int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
  * emits (src/llama.cpp:157-199; ggml_compute_forward_dup_f32, ggml-cpu.c:3519-3830), with the row taken from device
  * memory so that a captured launch sequence does not change as the cache fills. */
 int mi355_set_rows(void *stream, const mi355_tensor *src, const int32_t *rows, const mi355_tensor *dst);
-/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, or whole quantized rows (Q4_0, Q8_0, Q4_K, Q5_K, Q6_K in the
+/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, or whole quantized rows (Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0, Q4_K, Q5_K, Q6_K in the
  * device row layout, nb[1] = row bytes; dequantize_row_*, ggml-quants.c:255-273, 349-363, 1280-1302, 1482-1507, 1690-1719), ids i32
  * [n, b2, b3]; dst f32 */
 int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ids, const mi355_tensor *dst);

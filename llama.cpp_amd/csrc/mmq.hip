@@ -15,7 +15,7 @@
 //   Q5_0 : level - 16 as int8, scale d;  IQ4_NL : the table value of the nibble as int8, scale d
 //   Q4_1, Q5_1 : level 0..15 / 0..31 as int8, scale d; the "+ m * d_x * sum(q)" term of the stage's four blocks is added with one
 //          v_mfma_f32_32x32x16_f16 on (fp16 dx*sum(q), the reference's `s` field of block_q8_1) x (fp16 m)
-//   Q4_K : level 0..15 as int8, scale d*sc; the "- dmin*m*sum(q)" term of all blocks is
+//   Q4_K, Q5_K : level 0..15 / 0..31 as int8, scale d*sc; the "- dmin*m*sum(q)" term of all blocks is
 //          added with one v_mfma_f32_32x32x16_f16 per stage on (fp16 dx*sum(q)) x (fp16 dmin*m)
 //   Q6_K : level - 32 as int8, scale d*sc per 16 elements (v_mfma_i32_32x32x16_i8, two per block)
 //
@@ -41,7 +41,7 @@ template <int TYPE> struct mmq_cfg {
     static constexpr int G = TYPE == MI355_Q6_K ? 16 : 32;   // elements per weight scale
     static constexpr int NG = MMQ_BK / G;                    // weight scales per row per stage
     // a per-block offset rides on the sums of the activation levels: - dmin * m (Q4_K), + m (Q4_1, Q5_1)
-    static constexpr bool MIN = TYPE == MI355_Q4_K || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;
+    static constexpr bool MIN = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;
     // 16 bytes of nibbles per block with a per-block scale: one request / commit form serves them all
     static constexpr bool NIBBLE32 = TYPE == MI355_Q4_0 || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1 || TYPE == MI355_IQ4_NL;
     static constexpr bool PREFETCH = NIBBLE32 || TYPE == MI355_Q8_0;
@@ -91,8 +91,10 @@ __device__ __forceinline__ void load_weight_stage(const uint8_t *__restrict__ W,
                 sWs[b * MMQ_BM + r] = half_bits_to_float(*(const unsigned short *)(wrow + L.off_b + ((k0 >> 5) + b) * 2));
             }
         }
-    } else if constexpr (TYPE == MI355_Q4_K) {
-        // stage = half a super-block: sub-blocks j0..j0+3, 64 B of qs per row = 4 pieces of 16 B
+    } else if constexpr (TYPE == MI355_Q4_K || TYPE == MI355_Q5_K) {
+        // stage = half a super-block: sub-blocks j0..j0+3, 64 B of qs per row = 4 pieces of 16 B (Q5_K: bit j of qh[l] is the fifth
+        // bit of element l of sub-block j, dequantize_row_q5_K, ggml/src/ggml-quants.c:1482-1507)
+        constexpr int BB = TYPE == MI355_Q4_K ? Q4_K_BYTES : Q5_K_BYTES, QS = TYPE == MI355_Q4_K ? 16 : 48;
         const int64_t sb = k0 >> 8;
         const int half = (int)((k0 >> 7) & 1);
 #pragma unroll
@@ -101,13 +103,22 @@ __device__ __forceinline__ void load_weight_stage(const uint8_t *__restrict__ W,
             const int r = idx >> 2, p = idx & 3;          // p: piece -> group gl = p>>1 of the stage, half h = p&1
             const int gl = p >> 1, h = p & 1;
             const int64_t row = row0 + r < N ? row0 + r : N - 1;
-            const uint8_t *blk = W + row * L.row_bytes + sb * Q4_K_BYTES;
-            const u32x4 q = load16(blk + 16 + (half * 2 + gl) * 32 + h * 16);
+            const uint8_t *blk = W + row * L.row_bytes + sb * BB;
+            const u32x4 q = load16(blk + QS + (half * 2 + gl) * 32 + h * 16);
             u32x4 lo, hi;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 lo[i] = q[i] & 0x0F0F0F0Fu;
                 hi[i] = (q[i] >> 4) & 0x0F0F0F0Fu;
+            }
+            if constexpr (TYPE == MI355_Q5_K) {
+                const u32x4 qh = load16(blk + 16 + h * 16);
+                const int ja = half * 4 + 2 * gl;         // sub-block of the low nibbles; the high nibbles are the next one
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    lo[i] |= ((qh[i] >> ja) & 0x01010101u) << 4;
+                    hi[i] |= ((qh[i] >> (ja + 1)) & 0x01010101u) << 4;
+                }
             }
             *(u32x4 *)(sW + r * MMQ_LDK + (2 * gl) * 32 + h * 16) = lo;
             *(u32x4 *)(sW + r * MMQ_LDK + (2 * gl + 1) * 32 + h * 16) = hi;
@@ -178,7 +189,7 @@ __device__ __forceinline__ void load_act_stage(const int8_t *__restrict__ aq, co
             const int64_t col = col0 + r < B ? col0 + r : B - 1;
             const act_ds s = ads[col * nblk + (k0 >> 5) + b];
             sAd[b * BN + r] = s.d;
-            if constexpr (TYPE == MI355_Q4_K) sAs[r * 4 + b] = (_Float16)(s.d * (float)s.sum);
+            if constexpr (TYPE == MI355_Q4_K || TYPE == MI355_Q5_K) sAs[r * 4 + b] = (_Float16)(s.d * (float)s.sum);
         }
     }
 }
@@ -438,7 +449,7 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
             for (int tb = 0; tb < TN; tb++) {
                 const f16x4 v = *(const f16x4 *)(sAs + (wcol0 + tb * 32 + l32) * 4);
 #pragma unroll
-                for (int i = 0; i < 8; i++) af[tb][i] = (i < 4 && lhi == 0) ? (TYPE == MI355_Q4_K ? (_Float16)(-(float)v[i & 3]) : v[i & 3]) : (_Float16)0.0f;
+                for (int i = 0; i < 8; i++) af[tb][i] = (i < 4 && lhi == 0) ? (TYPE == MI355_Q4_K || TYPE == MI355_Q5_K ? (_Float16)(-(float)v[i & 3]) : v[i & 3]) : (_Float16)0.0f;
             }
 #pragma unroll
             for (int tw = 0; tw < 2; tw++) {
@@ -537,7 +548,7 @@ extern "C" int mi355_mul_mat_q(void *stream, int type, const void *W, const void
 
 extern "C" int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K,
                                   int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(is_weight_type(type) && type != MI355_Q5_K, "mul_mat_q: unsupported weight type %d", type);
+    MI355_REQUIRE(is_weight_type(type), "mul_mat_q: unsupported weight type %d", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % type_block_elems(type) == 0, "mul_mat_q: K=%lld is not a multiple of the block size", (long long)K);
     MI355_REQUIRE(dst_stride >= N, "mul_mat_q: dst_stride < N");
@@ -551,6 +562,7 @@ extern "C" int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const v
         case MI355_Q4_0: launch_mmq_tn<MI355_Q4_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q8_0: launch_mmq_tn<MI355_Q8_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q4_K: launch_mmq_tn<MI355_Q4_K>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_Q5_K: launch_mmq_tn<MI355_Q5_K>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q4_1: launch_mmq_tn<MI355_Q4_1>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q5_0: launch_mmq_tn<MI355_Q5_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q5_1: launch_mmq_tn<MI355_Q5_1>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;

@@ -102,18 +102,6 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
         const size_t used = mi355_mul_mat_ws_bytes(K, B);
         return mi355_mul_mat_q8k_ws(stream, type, W, ws, dst, nullptr, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
     }
-    if (type == MI355_Q5_K && B > 8) {
-        // No tile kernel unpacks Q5_K from packed rows: batches go through the GEMV eight activation rows at a time (each pass
-        // streams the matrix once), quantizing every eight rows into the start of the workspace.
-        for (int64_t b0 = 0; b0 < B; b0 += 8) {
-            const int64_t nb = B - b0 < 8 ? B - b0 : 8;
-            int rc = mi355_quantize_act(stream, x + b0 * x_stride, ws, K, nb, x_stride);
-            if (rc != MI355_OK) return rc;
-            rc = mi355_mul_mat_vec_q(stream, type, W, ws, dst + b0 * dst_stride, N, K, nb, dst_stride);
-            if (rc != MI355_OK) return rc;
-        }
-        return MI355_OK;
-    }
     int rc = mi355_quantize_act(stream, x, ws, K, B, x_stride);
     if (rc != MI355_OK) return rc;
     const size_t used = mi355_mul_mat_ws_bytes(K, B);
