@@ -78,7 +78,7 @@ def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats
 @pytest.mark.parametrize("n_prompt", [5, 20, 40, 256])
 def test_model_logits_q5_k_m(dev, tmp_path, n_prompt):
     """A Q5_K_M-shaped file (Q5_K everywhere, Q6_K where llama-quantize uses more bits): the reference's runtime on the plug-in
-    reproduces its CPU backend's logits, so Q5_K products (GEMV for decode and up to eight rows, eight rows at a time up to 32, the
+    reproduces its CPU backend's logits, so Q5_K products (GEMV for decode and up to eight rows, the per-32-block tile kernel up to 32, the
     wide-tile GEMM on Q5_K tile images from 33 rows on) and Q5_K rows of GET_ROWS stay on the device with the reference's
     arithmetic."""
     if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
@@ -99,8 +99,8 @@ def test_model_logits_q5_k_m(dev, tmp_path, n_prompt):
 @pytest.mark.parametrize("n_prompt", [5, 40])
 def test_model_logits_per_32_block_types(dev, tmp_path, ftype, n_prompt):
     """Files of the per-32-block types beyond Q4_0 / Q8_0 (Q4_1, Q5_0, Q5_1, IQ4_NL with the Q5_K / Q6_K tensors llama-quantize
-    mixes in): the reference's runtime on the plug-in reproduces its CPU backend's logits, so their MUL_MAT (single-matrix GEMV,
-    eight activation rows at a time for a prompt) and GET_ROWS stay on the device with the reference's arithmetic."""
+    mixes in): the reference's runtime on the plug-in reproduces its CPU backend's logits, so their MUL_MAT (the GEMV launches of
+    decode, the per-32-block tile kernel for a prompt) and GET_ROWS stay on the device with the reference's arithmetic."""
     if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
         pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
