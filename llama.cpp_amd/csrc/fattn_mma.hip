@@ -12,8 +12,8 @@
 //   O^T += V^T P^T  A = V^T rows (i = head dim), B = P^T (j = query) -> the B operand is the lane's
 //                 own score registers 8t..8t+7 rounded to f16: no cross-lane data movement.  The
 //                 kv cells those registers stand for, 16t + 8*(s/4) + 4*(l/32) + s%4, fix which
-//                 cells the A operand must supply in k slot s: two 8-byte reads of a V tile that
-//                 was transposed on its way into LDS.
+//                 cells the A operand must supply in k slot s: four cells at one element of the head, twice -
+//                 two transposing reads (ds_read_b64_tr_b16) of the row-major V tile.
 // Rescaling by exp(m_old - m_new) is one multiply per accumulator register because both
 // accumulators are indexed by query along the lanes.
 #include "fattn.hpp"
@@ -27,15 +27,14 @@ namespace {
 constexpr int FM_BC = 64;            // kv cells per tile
 constexpr float FM_NEG = -FLT_MAX / 2;
 
-// ---- staging of one 64-cell K tile and the matching V tile (transposed) through registers ----
+// ---- staging of one 64-cell K tile and the matching V tile through registers, both row-major ----
 template <int D, int NTH> struct kv_stage {
     static constexpr int KP = D + 8;        // f16 pitch of a K row in LDS (16 bytes of padding spread the banks)
-    static constexpr int VP = FM_BC + 4;    // f16 pitch of a V^T row in LDS (keeps 8-byte alignment)
+    static constexpr int VP = D + 16;       // f16 pitch of a V row in LDS: rows 8 banks apart, so the four rows of a transposing read miss each other
     static constexpr int KCH = D / 8;       // 16-byte chunks per K/V row
-    static constexpr int KIT = FM_BC * KCH / NTH;         // K chunks per thread per tile
-    static constexpr int VIT = (FM_BC / 2) * KCH / NTH;   // V (cell pair, chunk) units per thread per tile
-    static_assert(D % 32 == 0 && KIT >= 1 && VIT >= 1, "head size not served by this kernel");
-    u32x4 k[KIT], v0[VIT], v1[VIT];
+    static constexpr int KIT = FM_BC * KCH / NTH;         // chunks per thread per tile, K and V each
+    static_assert(D % 32 == 0 && KIT >= 1, "head size not served by this kernel");
+    u32x4 k[KIT], v[KIT];
 
     __device__ __forceinline__ void fetch(const fattn_args &a, int64_t hk, int64_t kv0, int tid) {
         const int64_t last = a.Nkv - 1;
@@ -45,35 +44,16 @@ template <int D, int NTH> struct kv_stage {
             const int row = unit / KCH, ch = unit % KCH;
             const int64_t c = kv0 + row < last ? kv0 + row : last;   // rows past the end repeat the last cell; their scores are dropped
             k[it] = load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + ch * 16);
-        }
-#pragma unroll
-        for (int it = 0; it < VIT; it++) {
-            const int unit = tid + it * NTH;
-            const int kp = unit & 31, ch = unit >> 5;
-            const int64_t c0 = kv0 + 2 * kp < last ? kv0 + 2 * kp : last;
-            const int64_t c1 = kv0 + 2 * kp + 1 < last ? kv0 + 2 * kp + 1 : last;
-            v0[it] = load16(a.v + c0 * a.v_nb1 + hk * a.v_nb2 + ch * 16);
-            v1[it] = load16(a.v + c1 * a.v_nb1 + hk * a.v_nb2 + ch * 16);
+            v[it] = load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + ch * 16);
         }
     }
-    __device__ __forceinline__ void commit(_Float16 *sK, _Float16 *sVt, int tid) const {
+    __device__ __forceinline__ void commit(_Float16 *sK, _Float16 *sV, int tid) const {
 #pragma unroll
         for (int it = 0; it < KIT; it++) {
             const int unit = tid + it * NTH;
             const int row = unit / KCH, ch = unit % KCH;
             *(u32x4 *)(sK + row * KP + ch * 8) = k[it];
-        }
-#pragma unroll
-        for (int it = 0; it < VIT; it++) {
-            const int unit = tid + it * NTH;
-            const int kp = unit & 31, ch = unit >> 5;
-            // element e of both cells -> one dword of row (8*ch + e) of V^T, columns 2*kp and 2*kp+1
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const u32 x = v0[it][i], y = v1[it][i];
-                *(u32 *)(sVt + (8 * ch + 2 * i) * VP + 2 * kp) = (x & 0xFFFFu) | (y << 16);
-                *(u32 *)(sVt + (8 * ch + 2 * i + 1) * VP + 2 * kp) = (x >> 16) | (y & 0xFFFF0000u);
-            }
+            *(u32x4 *)(sV + row * VP + ch * 8) = v[it];
         }
     }
 };
@@ -192,10 +172,16 @@ __device__ __forceinline__ float alibi_slope(const fattn_args &a, int64_t head) 
     return h < a.n_head_log2 ? powf(a.m0, (float)(h + 1)) : powf(a.m1, (float)(2 * (h - a.n_head_log2) + 1));
 }
 
-// O^T tiles [DT0, DT0 + NDT) += V^T P^T for the 32 cells of half u whose probabilities sit in S
+// O^T tiles [DT0, DT0 + NDT) += V^T P^T for the 32 cells of half u whose probabilities sit in S.  The A operand of a lane -
+// element 32 dt + l32 of cells c .. c + 3 and c + 8 .. c + 11, c = 32 u + 16 t + 4 lhi - comes from the row-major V tile by two
+// transposing reads: in each group of 16 lanes, lane i receives element i % 4 of the four rows that lanes i / 4, i / 4 + 4, + 8 and
+// + 12 point at, so lane 4 r + q of a group points at row c + r, elements 16 (group % 2) + 4 q .. + 3 of the tile's 32.
 template <int D, int NDT>
-__device__ __forceinline__ void accumulate_pv(f32x16 (&o)[NDT], const f32x16 &S, const _Float16 *sVt, int dt0, int u, int l32, int lhi) {
-    constexpr int VP = FM_BC + 4;
+__device__ __forceinline__ void accumulate_pv(f32x16 (&o)[NDT], const f32x16 &S, const _Float16 *sV, int dt0, int u, int l32, int lhi) {
+    constexpr int VP = D + 16;
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const int li = l32 & 15;
+    const _Float16 *lane_base = sV + (32 * u + 4 * lhi + (li >> 2)) * VP + 16 * (l32 >> 4) + 4 * (li & 3);
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         f16x8 pf;
@@ -203,14 +189,15 @@ __device__ __forceinline__ void accumulate_pv(f32x16 (&o)[NDT], const f32x16 &S,
         for (int i = 0; i < 8; i++) pf[i] = (_Float16)S[8 * t + i];
 #pragma unroll
         for (int dt = 0; dt < NDT; dt++) {
-            const _Float16 *vp = sVt + (32 * (dt0 + dt) + l32) * VP + 32 * u + 16 * t + 4 * lhi;
-            const f16x4 v0 = *(const f16x4 *)vp;
-            const f16x4 v1 = *(const f16x4 *)(vp + 8);
+            const _Float16 *vp = lane_base + 16 * t * VP + 32 * (dt0 + dt);
+            const s16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)vp);
+            const s16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(vp + 8 * VP));
+            const f16x4 h0 = __builtin_bit_cast(f16x4, v0), h1 = __builtin_bit_cast(f16x4, v1);
             f16x8 vf;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                vf[i] = v0[i];
-                vf[4 + i] = v1[i];
+                vf[i] = h0[i];
+                vf[4 + i] = h1[i];
             }
             o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, o[dt], 0, 0, 0);
         }
@@ -268,7 +255,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
     typedef kv_stage<D, 256> stage_t;
     constexpr int QTW = 4 / HPW;   // query tiles per group
     __shared__ __attribute__((aligned(16))) _Float16 sK[FM_BC * stage_t::KP];
-    __shared__ __attribute__((aligned(16))) _Float16 sVt[D * stage_t::VP];
+    __shared__ __attribute__((aligned(16))) _Float16 sVt[FM_BC * stage_t::VP];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -386,7 +373,7 @@ template <int D>
 __global__ void __launch_bounds__(256, 2) k_fattn_mma_half(fattn_args a) {
     typedef kv_stage<D, 256> stage_t;
     constexpr int NDT = D / 32;
-    constexpr int KV_HALVES = FM_BC * stage_t::KP + D * stage_t::VP;                 // f16 elements of the K tile and the V^T tile
+    constexpr int KV_HALVES = FM_BC * stage_t::KP + FM_BC * stage_t::VP;              // f16 elements of the K tile and the V tile
     constexpr int MERGE_FLOATS = 2 * (D + 2) * 32;                                    // per head: O^T [D][32], max, sum
     constexpr int SMEM_BYTES = KV_HALVES * 2 > MERGE_FLOATS * 4 ? KV_HALVES * 2 : MERGE_FLOATS * 4;
     __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM_BYTES];
@@ -530,7 +517,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_dec(fattn_args a, int R, i
     typedef kv_stage<D, 256> stage_t;
     constexpr int NDT = D / 64;   // 32-row O^T tiles per wave
     __shared__ __attribute__((aligned(16))) _Float16 sK[FM_BC * stage_t::KP];
-    __shared__ __attribute__((aligned(16))) _Float16 sVt[D * stage_t::VP];
+    __shared__ __attribute__((aligned(16))) _Float16 sVt[FM_BC * stage_t::VP];
     float *s_merge = (float *)sK;   // reused after the last tile: per h, [D/2 + 2][32] floats of the u = 1 wave
     static_assert(sizeof(_Float16) * FM_BC * stage_t::KP >= sizeof(float) * (D + 4) * 32, "merge buffer does not fit the K tile");
 
