@@ -18,6 +18,7 @@
 // accumulators are indexed by query along the lanes.
 #include "fattn.hpp"
 
+
 #include <float.h>
 
 namespace mi355 {
@@ -28,11 +29,11 @@ constexpr int FM_BC = 64;            // kv cells per tile
 constexpr float FM_NEG = -FLT_MAX / 2;
 
 // ---- staging of one 64-cell K tile and the matching V tile through registers, both row-major ----
-template <int D, int NTH> struct kv_stage {
+template <int D, int NTH, int BC = FM_BC> struct kv_stage {
     static constexpr int KP = D + 8;        // f16 pitch of a K row in LDS (16 bytes of padding spread the banks)
     static constexpr int VP = D + 16;       // f16 pitch of a V row in LDS: rows 8 banks apart, so the four rows of a transposing read miss each other
     static constexpr int KCH = D / 8;       // 16-byte chunks per K/V row
-    static constexpr int KIT = FM_BC * KCH / NTH;         // chunks per thread per tile, K and V each
+    static constexpr int KIT = BC * KCH / NTH;            // chunks per thread per tile, K and V each
     static_assert(D % 32 == 0 && KIT >= 1, "head size not served by this kernel");
     u32x4 k[KIT], v[KIT];
 
@@ -250,6 +251,17 @@ __global__ void __launch_bounds__(256) k_mask_extent(const uint8_t *__restrict__
     if (threadIdx.x == 0) extent[blockIdx.x] = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3])) + 1;
 }
 
+// Groups go to the eight XCDs round-robin by linear index and each XCD has its own L2.  Renumbered so that XCD x works through the
+// x-th eighth of the grid in (head, query tile) order, the groups that read one kv head's K and V run on one XCD and find in its
+// L2 what their neighbours loaded (with 8 kv heads: one head per XCD).  Returns the group's place (x, y) in the launch's grid.
+struct grid_pos { unsigned x, y; };
+__device__ __forceinline__ grid_pos xcd_grid_pos() {
+    const unsigned nx = gridDim.x, total = nx * gridDim.y;
+    unsigned L = blockIdx.x + nx * blockIdx.y;
+    if (total % 8 == 0) L = (L % 8) * (total / 8) + L / 8;
+    return grid_pos{L % nx, L / nx};
+}
+
 template <int D, int HPW>
 __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
     typedef kv_stage<D, 256> stage_t;
@@ -261,9 +273,10 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
     const int groups = (int)(a.Hq / a.Hkv) / HPW;
-    const int64_t hk = blockIdx.y / groups, hg = blockIdx.y % groups;
+    const grid_pos gp = xcd_grid_pos();
+    const int64_t hk = gp.y / groups, hg = gp.y % groups;
     const int64_t head = (hk * groups + hg) * HPW + (wave % HPW);
-    const int64_t q0 = ((int64_t)blockIdx.x * QTW + wave / HPW) * 32;
+    const int64_t q0 = ((int64_t)gp.x * QTW + wave / HPW) * 32;
     const int64_t iq = q0 + l32 < a.Nq ? q0 + l32 : a.Nq - 1;   // clamped: rows past Nq are computed and dropped
 
     f16x8 qf[D / 16];
@@ -286,7 +299,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
         int e = 0;
 #pragma unroll
         for (int j = 0; j < QTW; j++) {
-            const int64_t t = (int64_t)blockIdx.x * QTW + j;
+            const int64_t t = (int64_t)gp.x * QTW + j;
             if (t * 32 < a.Nq) e = max(e, a.kv_extent[t]);
         }
         kv_limit = e < a.Nkv ? e : a.Nkv;
@@ -364,30 +377,35 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
     }
 }
 
-// ---- prefill with few query tiles: the two 32-cell halves of every K/V tile go to different waves ----------------------------
+// ---- prefill with few query tiles: the 32-cell parts of every K/V tile go to different waves -----------------------------------
 // k_fattn_mma gives a wave 32 queries of one head and the whole 64-cell tile; a batch of a few hundred rows is then fewer groups
-// than compute units, each a serial chain of tiles.  Here a group is two query heads of one kv head x the two halves of the
-// tile: wave (hp, u) scores and accumulates cells [32u, 32u + 32) of each tile for head hp with its own soft-max state, and the
-// u = 1 wave hands its state to the u = 0 wave through LDS at the end.  Twice the groups, half the work per wave and tile.
-template <int D>
-__global__ void __launch_bounds__(256, 2) k_fattn_mma_half(fattn_args a) {
-    typedef kv_stage<D, 256> stage_t;
+// than compute units, each a serial chain of tiles.  Here a group is two query heads of one kv head x the NU 32-cell parts of a
+// tile of 32 NU cells: wave (hp, u) scores and accumulates cells [32u, 32u + 32) of each tile for head hp with its own soft-max
+// state, and the states of a head's waves are joined pairwise through LDS at the end.  NU = 2: twice the groups of k_fattn_mma
+// with half the work per wave and tile; NU = 4 (eight waves, 128-cell tiles) when even those leave one group per compute
+// unit: two waves per SIMD, so that one wave's matrix instructions run under the other's soft-max arithmetic, and half the
+// tile steps.
+template <int D, int NU>
+__global__ void __launch_bounds__(128 * NU, NU == 2 ? 2 : 1) k_fattn_mma_half(fattn_args a) {
+    constexpr int NTH = 128 * NU, BC = 32 * NU;
+    typedef kv_stage<D, NTH, BC> stage_t;
     constexpr int NDT = D / 32;
-    constexpr int KV_HALVES = FM_BC * stage_t::KP + FM_BC * stage_t::VP;              // f16 elements of the K tile and the V tile
-    constexpr int MERGE_FLOATS = 2 * (D + 2) * 32;                                    // per head: O^T [D][32], max, sum
+    constexpr int KV_HALVES = BC * stage_t::KP + BC * stage_t::VP;                    // f16 elements of the K tile and the V tile
+    constexpr int MERGE_FLOATS = NU * (D + 2) * 32;                                   // per (head, pair of waves): O^T [D][32], max, sum
     constexpr int SMEM_BYTES = KV_HALVES * 2 > MERGE_FLOATS * 4 ? KV_HALVES * 2 : MERGE_FLOATS * 4;
     __shared__ __attribute__((aligned(16))) uint8_t smem[SMEM_BYTES];
-    _Float16 *sK = (_Float16 *)smem, *sVt = sK + FM_BC * stage_t::KP;
+    _Float16 *sK = (_Float16 *)smem, *sVt = sK + BC * stage_t::KP;
     float *s_merge = (float *)smem;   // reused after the last tile
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
-    const int u = wave & 1, hp = wave >> 1;
+    const int u = wave % NU, hp = wave / NU;
     const int pairs = (int)(a.Hq / a.Hkv) / 2;   // head pairs per kv head
-    const int64_t hk = blockIdx.y / pairs, hg = blockIdx.y % pairs;
+    const grid_pos gp = xcd_grid_pos();
+    const int64_t hk = gp.y / pairs, hg = gp.y % pairs;
     const int64_t head = (hk * pairs + hg) * 2 + hp;
-    const int64_t q0 = (int64_t)blockIdx.x * 32;
+    const int64_t q0 = (int64_t)gp.x * 32;
     const int64_t iq = q0 + l32 < a.Nq ? q0 + l32 : a.Nq - 1;   // clamped: rows past Nq are computed and dropped
 
     f16x8 qf[D / 16];
@@ -408,17 +426,17 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_half(fattn_args a) {
     u32x2 mnext[4];
     auto prefetch = [&](int64_t kv0) {
         st.fetch(a, hk, kv0, tid);
-        fetch_mask<4>(mnext, mrow, mask_aligned && kv0 + FM_BC <= a.Nkv, kv0 + 32 * u + 4 * lhi, a.Nkv);
+        fetch_mask<4>(mnext, mrow, mask_aligned && kv0 + BC <= a.Nkv, kv0 + 32 * u + 4 * lhi, a.Nkv);
     };
     prefetch(0);
-    for (int64_t kv0 = 0; kv0 < a.Nkv; kv0 += FM_BC) {
+    for (int64_t kv0 = 0; kv0 < a.Nkv; kv0 += BC) {
         __syncthreads();   // the previous tile has been consumed
         st.commit(sK, sVt, tid);
         u32x2 mcur[4];
 #pragma unroll
         for (int g = 0; g < 4; g++) mcur[g] = mnext[g];
         __syncthreads();
-        if (kv0 + FM_BC < a.Nkv) prefetch(kv0 + FM_BC);
+        if (kv0 + BC < a.Nkv) prefetch(kv0 + BC);
         f32x16 S = scores<D>(qf, sK, u, l32, lhi);
         float mx = finish_scores(S, mcur, a, scale, slope, kv0 + 32 * u, lhi, a.Nkv);
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -447,25 +465,35 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_half(fattn_args a) {
         accumulate_pv<D, NDT>(o, S, sVt, 0, u, l32, lhi);
     }
 
-    // ---- the u = 1 wave's state joins the u = 0 wave of the same head
-    float *mg = s_merge + hp * (D + 2) * 32;   // [d][query], then max, sum
-    __syncthreads();
-    if (u == 1) {
+    // ---- the states of a head's waves are joined pairwise: u + step hands its state to u (step = 1, then 2)
 #pragma unroll
-        for (int dt = 0; dt < NDT; dt++)
+    for (int step = 1; step < NU; step *= 2) {
+        float *mg = s_merge + (hp * (NU / 2) + (u >> 1) / step) * (D + 2) * 32;   // [d][query], then max, sum
+        __syncthreads();
+        if ((u & (2 * step - 1)) == step) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] = o[dt][r];
-        if (lhi == 0) {
-            mg[D * 32 + l32] = m;
-            mg[(D + 1) * 32 + l32] = l;
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] = o[dt][r];
+            if (lhi == 0) {
+                mg[D * 32 + l32] = m;
+                mg[(D + 1) * 32 + l32] = l;
+            }
+        }
+        __syncthreads();
+        if ((u & (2 * step - 1)) == 0) {
+            const float m1 = mg[D * 32 + l32], l1 = mg[(D + 1) * 32 + l32];
+            const float M = fmaxf(m, m1);
+            const float f0 = __expf(m - M), f1 = __expf(m1 - M);
+            l = l * f0 + l1 * f1;
+            m = M;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[dt][r] = o[dt][r] * f0 + mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] * f1;
         }
     }
-    __syncthreads();
     if (u != 0 || q0 + l32 >= a.Nq) return;
-    const float m1 = mg[D * 32 + l32], l1 = mg[(D + 1) * 32 + l32];
-    const float M = fmaxf(m, m1);
-    const float f0 = __expf(m - M), f1 = __expf(m1 - M);
-    l = l * f0 + l1 * f1;
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
     float *dp = a.dst + ((q0 + l32) * a.Hq + head) * D;
 #pragma unroll
@@ -474,10 +502,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_half(fattn_args a) {
         for (int g = 0; g < 4; g++) {
             f32x4 w;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int r = 4 * g + i;
-                w[i] = (o[dt][r] * f0 + mg[(32 * dt + 8 * (r >> 2) + 4 * lhi + (r & 3)) * 32 + l32] * f1) * inv;
-            }
+            for (int i = 0; i < 4; i++) w[i] = o[dt][4 * g + i] * inv;
             *(f32x4 *)(dp + 32 * dt + 8 * g + 4 * lhi) = w;
         }
 }
@@ -486,7 +511,10 @@ template <int D>
 int launch_half(hipStream_t s, const fattn_args &a) {
     const int64_t pairs = (a.Hq / a.Hkv) / 2;
     const dim3 grid((unsigned)((a.Nq + 31) / 32), (unsigned)(a.Hkv * pairs));
-    MI355_LAUNCH((k_fattn_mma_half<D>), grid, dim3(256), 0, s, a);
+    // at most one group per compute unit and a long cache: eight waves on 128-cell tiles (512 rows: 4096 cells 112 -> 103 us,
+    // 512 cells 24.8 -> 26.2 us)
+    if ((int64_t)grid.x * grid.y <= 256 && a.Nkv >= 1024) MI355_LAUNCH((k_fattn_mma_half<D, 4>), grid, dim3(512), 0, s, a);
+    else MI355_LAUNCH((k_fattn_mma_half<D, 2>), grid, dim3(256), 0, s, a);
     return launch_status("k_fattn_mma_half");
 }
 
