@@ -318,11 +318,12 @@ def sweep(kinds):
                      achieved=round(ops / us / 1e6, 1), unit="TFLOP/s" if dt == torch.float16 else "TOP/s",
                      frac=round(ops / us / 1e6 / (F16_PEAK_TFLOPS if dt == torch.float16 else INT8_PEAK_TOPS), 4), ops=ops)
                 del ws_
-    if "fattn" in kinds or "fattn_long" in kinds or "fattn_prefill" in kinds:
+    if "fattn" in kinds or "fattn_long" in kinds or "fattn_prefill" in kinds or "fattn_prefill_512" in kinds:
         H, HK, D = 32, 8, 128
         cases = [(1, 256), (1, 512), (1, 1024), (1, 4096), (1, 32768), (1, 131072), (512, 512), (512, 4096), (2048, 2048), (4096, 4096)]
         if "fattn" not in kinds:   # one kernel alone (for counter collection): long-context decode and / or the prefill kernel
-            cases = ([(1, 131072)] if "fattn_long" in kinds else []) + ([(4096, 4096)] if "fattn_prefill" in kinds else [])
+            cases = ([(1, 131072)] if "fattn_long" in kinds else []) + ([(4096, 4096)] if "fattn_prefill" in kinds else []) + \
+                    ([(512, 4096)] if "fattn_prefill_512" in kinds else [])
         for Nq, Nkv in cases:
             nrot = max(2, min(16, (1 << 30) // (Nkv * HK * D * 4))) if Nq == 1 else 1
             q = torch.randn(Nq, H, D, device=dev, generator=gen)
@@ -361,7 +362,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
     ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, mmq_wide (the wide-tile GEMM on 14336 x 4096 at batch 512 only), fattn, "
-                                          "fattn_long (decode over 131072 cells only), fattn_prefill (4096 x 4096 prefill only), limits (LDS fill rate of a compute unit and the vendor library's dense GEMMs on the prefill shapes)")
+                                          "fattn_long (decode over 131072 cells only), fattn_prefill (4096 x 4096 prefill only), fattn_prefill_512 (512 rows over 4096 cells only), limits (LDS fill rate of a compute unit and the vendor library's dense GEMMs on the prefill shapes)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="rewrite the tracked HBM-traffic summary from two rocprofv3 --pmc output directories (no GPU needed)")
     args = ap.parse_args()

@@ -87,11 +87,36 @@ __device__ __forceinline__ float mask_value(const u32x2 &w, int i) {
     return half_bits_to_float((unsigned short)((i < 2 ? w[0] : w[1]) >> (16 * (i & 1))));
 }
 
+// Running maximum of the prefill kernels.  The reference point of a column's exponentials moves only when the tile's largest
+// score exceeds it by more than FM_LAZY: any reference point gives the same quotient sum(p v) / sum(p), and while it stays put
+// the 64 output registers are not rescaled (with an exact running maximum some query of a 32-query tile raises its maximum
+// in most tiles of a few thousand cells; this way it happens in the first tiles only).  Probabilities then reach e^FM_LAZY at
+// most, far inside the f16 range of the matrix operand.
+constexpr float FM_LAZY = 8.0f;
+constexpr float FM_LOG2E = 1.4426950408889634f;
+__device__ __forceinline__ float lazy_max(float m, float mx) { return mx > m + FM_LAZY ? mx : m; }
+// exp(s - m) as one multiply-add and one exponential: 2^(s log2(e) - m log2(e)); m2 = m log2(e)
+__device__ __forceinline__ float exp_rel(float s, float m2) { return __builtin_amdgcn_exp2f(fmaf(s, FM_LOG2E, -m2)); }
+
 // scale [+ softcap], add the mask, mark dropped cells with FM_NEG; returns the largest surviving score.
 // A masked cell (-inf; slopes are positive) and a NaN score of a stale cell both end as FM_NEG in fmaxf(s, FM_NEG); the test against
 // the end of the range is made only in a tile that reaches past it (uniform over the group), on 32-bit offsets.
 __device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], const fattn_args &a, float scale, float slope,
                                                 int64_t c_first, int lhi, int64_t c_end) {
+    float mx = FM_NEG;
+    const int64_t room = c_end - c_first;
+    if (a.softcap == 0.0f && slope == 1.0f && room >= 32) {   // the common case in one multiply-add per score: scale * s + mask
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float s = fmaf(S[4 * g + i], scale, mask_value(mw[g], i));
+                s = fmaxf(s, FM_NEG);   // -inf and NaN become FM_NEG
+                S[4 * g + i] = s;
+                mx = fmaxf(mx, s);
+            }
+        return mx;
+    }
     if (a.softcap != 0.0f) {
 #pragma unroll
         for (int r = 0; r < 16; r++) S[r] = a.softcap * tanhf(S[r] * scale);
@@ -99,8 +124,6 @@ __device__ __forceinline__ float finish_scores(f32x16 &S, const u32x2 (&mw)[4], 
 #pragma unroll
         for (int r = 0; r < 16; r++) S[r] *= scale;
     }
-    float mx = FM_NEG;
-    const int64_t room = c_end - c_first;
     if (room >= 32) {   // every cell of this half tile lies inside the range
 #pragma unroll
         for (int g = 0; g < 4; g++)
@@ -253,13 +276,16 @@ __global__ void __launch_bounds__(256) k_mask_extent(const uint8_t *__restrict__
 
 // Groups go to the eight XCDs round-robin by linear index and each XCD has its own L2.  Renumbered so that XCD x works through the
 // x-th eighth of the grid in (head, query tile) order, the groups that read one kv head's K and V run on one XCD and find in its
-// L2 what their neighbours loaded (with 8 kv heads: one head per XCD).  Returns the group's place (x, y) in the launch's grid.
+// L2 what their neighbours loaded (with 8 kv heads: one head per XCD).  Query tiles are taken from the last one down: under a
+// causal mask the last tile sees the most cells, and groups are started in index order, so the long groups start first and the
+// short ones fill the gaps at the end (in ascending order the launch ends with the longest groups running alone: 64 slots
+// and 128 tiles of 1 .. 128 half-steps finish after 96 steps instead of 64.5).  Returns the group's place (x, y) in the grid.
 struct grid_pos { unsigned x, y; };
 __device__ __forceinline__ grid_pos xcd_grid_pos() {
     const unsigned nx = gridDim.x, total = nx * gridDim.y;
     unsigned L = blockIdx.x + nx * blockIdx.y;
     if (total % 8 == 0) L = (L % 8) * (total / 8) + L / 8;
-    return grid_pos{L % nx, L / nx};
+    return grid_pos{nx - 1 - L % nx, L / nx};
 }
 
 template <int D, int HPW>
@@ -335,17 +361,17 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         if (__ballot(mx > FM_NEG) == 0) continue;   // every cell of the tile is masked for all 32 queries (wave-uniform)
-        const float m_new = fmaxf(m, mx);
-        const float alpha = __expf(m - m_new);
+        const float m_new = lazy_max(m, mx);
+        const float alpha = __builtin_amdgcn_exp2f((m - m_new) * FM_LOG2E);   // exactly 1 while the reference point stays
         // dropped scores are exactly FM_NEG: exp(FM_NEG - m) is 0 for any real maximum; a column that has seen no cell yet
         // (maximum still FM_NEG) subtracts 0 instead, so its dropped scores give 0 as well and not exp(0)
-        const float m_eff = m_new > FM_NEG ? m_new : 0.0f;
+        const float m2 = m_new > FM_NEG ? m_new * FM_LOG2E : 0.0f;
         float rs = 0.0f;
 #pragma unroll
         for (int u = 0; u < 2; u++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const float p = __expf(S[u][r] - m_eff);
+                const float p = exp_rel(S[u][r], m2);
                 S[u][r] = p;
                 rs += p;
             }
@@ -441,15 +467,15 @@ __global__ void __launch_bounds__(128 * NU, NU == 2 ? 2 : 1) k_fattn_mma_half(fa
         float mx = finish_scores(S, mcur, a, scale, slope, kv0 + 32 * u, lhi, a.Nkv);
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         if (__ballot(mx > FM_NEG) == 0) continue;   // all 32 cells masked for all 32 queries (wave-uniform; barriers are at the loop head)
-        const float m_new = fmaxf(m, mx);
-        const float alpha = __expf(m - m_new);
+        const float m_new = lazy_max(m, mx);
+        const float alpha = __builtin_amdgcn_exp2f((m - m_new) * FM_LOG2E);   // exactly 1 while the reference point stays
         // dropped scores are exactly FM_NEG: exp(FM_NEG - m) is 0 for any real maximum; a column that has seen no cell yet
         // (maximum still FM_NEG) subtracts 0 instead, so its dropped scores give 0 as well and not exp(0)
-        const float m_eff = m_new > FM_NEG ? m_new : 0.0f;
+        const float m2 = m_new > FM_NEG ? m_new * FM_LOG2E : 0.0f;
         float rs = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float p = __expf(S[r] - m_eff);
+            const float p = exp_rel(S[r], m2);
             S[r] = p;
             rs += p;
         }
