@@ -35,9 +35,25 @@ template <int D, int NTH, int BC = FM_BC> struct kv_stage {
     static constexpr int KCH = D / 8;       // 16-byte chunks per K/V row
     static constexpr int KIT = BC * KCH / NTH;            // chunks per thread per tile, K and V each
     static_assert(D % 32 == 0 && KIT >= 1, "head size not served by this kernel");
+    static_assert(NTH % KCH == 0, "a thread keeps its chunk position over the rows it loads");
     u32x4 k[KIT], v[KIT];
 
+    // A tile that lies inside the cache is addressed as (uniform base of the tile and of the thread's it-th row block) + (one
+    // 32-bit offset per thread, the same for every tile): thread tid loads rows tid / KCH + it * (NTH / KCH), chunk tid % KCH.
+    // The uniform part is scalar arithmetic; per-row 64-bit products in vector registers cost as many instructions per tile
+    // step as the soft-max.  The launcher checks that a tile's span fits 32 bits.  The last, partial tile clamps row by row.
     __device__ __forceinline__ void fetch(const fattn_args &a, int64_t hk, int64_t kv0, int tid) {
+        if (kv0 + BC <= a.Nkv) {   // uniform
+            const unsigned r0 = (unsigned)(tid / KCH), ch16 = (unsigned)(tid % KCH) * 16;
+            const unsigned ko = r0 * (unsigned)a.k_nb1 + ch16, vo = r0 * (unsigned)a.v_nb1 + ch16;
+            const uint8_t *kb = a.k + kv0 * a.k_nb1 + hk * a.k_nb2, *vb = a.v + kv0 * a.v_nb1 + hk * a.v_nb2;
+#pragma unroll
+            for (int it = 0; it < KIT; it++) {
+                k[it] = load16(kb + (size_t)it * (NTH / KCH) * a.k_nb1 + ko);
+                v[it] = load16(vb + (size_t)it * (NTH / KCH) * a.v_nb1 + vo);
+            }
+            return;
+        }
         const int64_t last = a.Nkv - 1;
 #pragma unroll
         for (int it = 0; it < KIT; it++) {
@@ -748,6 +764,7 @@ int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes) {
     if (a.Hkv * (a.Hq / a.Hkv) > 65535 || (a.Nq + 31) / 32 > 0x7fffffff) return 1;
     if ((a.q_nb1 % 16) != 0 || (a.q_nb2 % 16) != 0) return 1;
     if (D != 64 && D != 128) return 1;
+    if (a.k_nb1 >= (size_t(1) << 24) || a.v_nb1 >= (size_t(1) << 24)) return 1;   // kv_stage: a tile's rows within 32-bit offsets
     a.kv_extent = nullptr;
     const int64_t n_tiles = (a.Nq + 31) / 32;
     // The pre-pass pays when there are more groups than the chip holds at once (two per compute unit): then a group that stops
@@ -780,6 +797,7 @@ int launch_fattn_mma_dec(hipStream_t s, fattn_args &a, int64_t D) {
     const int64_t R = a.Hq / a.Hkv;
     if (R > 32 || a.Hkv > 65535 || (a.q_nb1 % 16) != 0 || (a.q_nb2 % 16) != 0 || a.cells_per_split % FM_BC != 0) return 1;
     if ((a.Nq + (32 / R) - 1) / (32 / R) > 65535) return 1;
+    if (a.k_nb1 >= (size_t(1) << 24) || a.v_nb1 >= (size_t(1) << 24)) return 1;   // kv_stage: a tile's rows within 32-bit offsets
     switch (D) {
         case 64: return launch_dec<64>(s, a);
         case 128: return launch_dec<128>(s, a);
