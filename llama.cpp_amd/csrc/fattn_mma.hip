@@ -103,6 +103,18 @@ __device__ __forceinline__ float mask_value(const u32x2 &w, int i) {
     return half_bits_to_float((unsigned short)((i < 2 ? w[0] : w[1]) >> (16 * (i & 1))));
 }
 
+// max / sum of a value over a lane and its partner in the other half of the wave (lane ^ 32), in every lane: one
+// v_permlane32_swap (both halves of one register handed to the other half of a second) instead of a trip through the LDS
+// crossbar, whose latency a wave that is alone on its SIMD waits out.
+__device__ __forceinline__ float half_pair_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_pair_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Running maximum of the prefill kernels.  The reference point of a column's exponentials moves only when the tile's largest
 // score exceeds it by more than FM_LAZY: any reference point gives the same quotient sum(p v) / sum(p), and while it stays put
 // the 64 output registers are not rescaled (with an exact running maximum some query of a 32-query tile raises its maximum
@@ -375,7 +387,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
             S[u] = scores<D>(qf, sK, u, l32, lhi);
             mx = fmaxf(mx, finish_scores(S[u], mcur[u], a, scale, slope, kv0 + 32 * u, lhi, a.Nkv));
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = half_pair_max(mx);
         if (__ballot(mx > FM_NEG) == 0) continue;   // every cell of the tile is masked for all 32 queries (wave-uniform)
         const float m_new = lazy_max(m, mx);
         const float alpha = __builtin_amdgcn_exp2f((m - m_new) * FM_LOG2E);   // exactly 1 while the reference point stays
@@ -391,7 +403,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
                 S[u][r] = p;
                 rs += p;
             }
-        rs += __shfl_xor(rs, 32, 64);
+        rs = half_pair_sum(rs);
         l = l * alpha + rs;
         m = m_new;
         if (__ballot(alpha != 1.0f) != 0) {   // wave-uniform
@@ -481,7 +493,7 @@ __global__ void __launch_bounds__(128 * NU, NU == 2 ? 2 : 1) k_fattn_mma_half(fa
         if (kv0 + BC < a.Nkv) prefetch(kv0 + BC);
         f32x16 S = scores<D>(qf, sK, u, l32, lhi);
         float mx = finish_scores(S, mcur, a, scale, slope, kv0 + 32 * u, lhi, a.Nkv);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = half_pair_max(mx);
         if (__ballot(mx > FM_NEG) == 0) continue;   // all 32 cells masked for all 32 queries (wave-uniform; barriers are at the loop head)
         const float m_new = lazy_max(m, mx);
         const float alpha = __builtin_amdgcn_exp2f((m - m_new) * FM_LOG2E);   // exactly 1 while the reference point stays
@@ -495,7 +507,7 @@ __global__ void __launch_bounds__(128 * NU, NU == 2 ? 2 : 1) k_fattn_mma_half(fa
             S[r] = p;
             rs += p;
         }
-        rs += __shfl_xor(rs, 32, 64);
+        rs = half_pair_sum(rs);
         l = l * alpha + rs;
         m = m_new;
         if (__ballot(alpha != 1.0f) != 0) {   // wave-uniform
@@ -637,7 +649,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_dec(fattn_args a, int R, i
         if (kv0 + 2 * FM_BC < c_end) prefetch(st, mn, kv0 + 2 * FM_BC);
         f32x16 S = scores<D>(qf, sK, u, l32, lhi);
         float mx = finish_scores_dec(S, mcur, a, scale, slope, kv0 + 32 * u, lhi, c_end);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = half_pair_max(mx);
         if (__ballot(mx > FM_NEG) == 0) return;   // all 32 cells masked for every column (wave-uniform)
         const float m_new = fmaxf(m, mx);
         const float alpha = __expf(m - m_new);
@@ -648,7 +660,7 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma_dec(fattn_args a, int R, i
             S[r] = p;
             rs += p;
         }
-        rs += __shfl_xor(rs, 32, 64);
+        rs = half_pair_sum(rs);
         l = l * alpha + rs;
         m = m_new;
         if (__ballot(alpha != 1.0f) != 0) {   // wave-uniform: most tiles do not raise any column's maximum
