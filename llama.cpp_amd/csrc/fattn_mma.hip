@@ -256,12 +256,24 @@ __device__ __forceinline__ void accumulate_pv(f32x16 (&o)[NDT], const f32x16 &S,
     }
 }
 
-template <int D>
+// EAGER: all of the row's fragments are requested before the first matrix instruction (D / 2 more registers), so the chain of
+// dependent instructions does not stop for an LDS round trip after every second one.
+template <int D, bool EAGER = false>
 __device__ __forceinline__ f32x16 scores(const f16x8 (&qf)[D / 16], const _Float16 *sK, int u, int l32, int lhi) {
     constexpr int KP = D + 8;
     f32x16 S;
 #pragma unroll
     for (int r = 0; r < 16; r++) S[r] = 0.0f;
+    if constexpr (EAGER) {
+        f16x8 kf[D / 16];
+#pragma unroll
+        for (int kk = 0; kk < D / 16; kk++) kf[kk] = *(const f16x8 *)(sK + (32 * u + l32) * KP + 16 * kk + 8 * lhi);
+#pragma unroll
+        for (int kk = 0; kk < D / 16; kk++) asm volatile("" : "+v"(kf[kk]));   // keeps the loads ahead of the chain
+#pragma unroll
+        for (int kk = 0; kk < D / 16; kk++) S = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[kk], qf[kk], S, 0, 0, 0);
+        return S;
+    }
 #pragma unroll
     for (int kk = 0; kk < D / 16; kk++) {
         const f16x8 kf = *(const f16x8 *)(sK + (32 * u + l32) * KP + 16 * kk + 8 * lhi);
@@ -491,7 +503,7 @@ __global__ void __launch_bounds__(128 * NU, NU == 2 ? 2 : 1) k_fattn_mma_half(fa
         for (int g = 0; g < 4; g++) mcur[g] = mnext[g];
         __syncthreads();
         if (kv0 + BC < a.Nkv) prefetch(kv0 + BC);
-        f32x16 S = scores<D>(qf, sK, u, l32, lhi);
+        f32x16 S = scores<D, true>(qf, sK, u, l32, lhi);
         float mx = finish_scores(S, mcur, a, scale, slope, kv0 + 32 * u, lhi, a.Nkv);
         mx = half_pair_max(mx);
         if (__ballot(mx > FM_NEG) == 0) continue;   // all 32 cells masked for all 32 queries (wave-uniform; barriers are at the loop head)
