@@ -347,7 +347,9 @@ __global__ void __launch_bounds__(256, 2) k_fattn_mma(fattn_args a) {
 
     f16x8 qf[D / 16];
     load_q<D>(qf, (const float *)(a.q + iq * a.q_nb1 + head * a.q_nb2), lhi);
-    const float slope = alibi_slope(a, head);
+    float slope = alibi_slope(a, head);
+    asm volatile("" : "+v"(slope));   // kept in a vector register also where the head is uniform over the group: a scalar slope makes
+                                      // the compiler build a second copy of the tile loop around "slope == 1", which then spills
     const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
     const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
     const bool mask_aligned = (((uintptr_t)a.mask | a.mask_nb1) & 7) == 0;
