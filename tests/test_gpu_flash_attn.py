@@ -85,7 +85,7 @@ def test_no_mask(dev):
     assert orc.nmse(got, orc.flash_attn("f64", q, k.view(np.uint16), v.view(np.uint16), None, 0.1)) < 1e-5
 
 
-@pytest.mark.parametrize("Nq,Nkv", [(1, 512), (1, 4096), (1, 32768), (512, 512), (512, 4096)])
+@pytest.mark.parametrize("Nq,Nkv", [(1, 512), (1, 4096), (1, 32768), (512, 512), (512, 4096), (2048, 2048)])
 def test_llama3_shapes(dev, Nq, Nkv):
     """BASELINE config 2: 32 query heads over 8 kv heads, head size 128, causal, llama's strided layouts.  The WHOLE output is
     held to the reference CPU backend's (NMSE <= 5e-4, tests/test-backend-ops.cpp:3137) and to the textbook form in f64 (which
