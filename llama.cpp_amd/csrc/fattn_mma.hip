@@ -322,10 +322,11 @@ __global__ void __launch_bounds__(256) k_mask_extent(const uint8_t *__restrict__
 // and 128 tiles of 1 .. 128 half-steps finish after 96 steps instead of 64.5).  Returns the group's place (x, y) in the grid.
 struct grid_pos { unsigned x, y; };
 __device__ __forceinline__ grid_pos xcd_grid_pos() {
-    const unsigned nx = gridDim.x, total = nx * gridDim.y;
-    unsigned L = blockIdx.x + nx * blockIdx.y;
+    const unsigned nx = gridDim.x;
+    const uint64_t total = (uint64_t)nx * gridDim.y;
+    uint64_t L = blockIdx.x + (uint64_t)nx * blockIdx.y;
     if (total % 8 == 0) L = (L % 8) * (total / 8) + L / 8;
-    return grid_pos{nx - 1 - L % nx, L / nx};
+    return grid_pos{nx - 1 - (unsigned)(L % nx), (unsigned)(L / nx)};
 }
 
 template <int D, int HPW>
