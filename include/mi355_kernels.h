@@ -271,6 +271,17 @@ int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act
                          int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws,
                          size_t route_ws_bytes);
 
+/* MUL_MAT_ID with many slots on the wide-tile kernel (ggml_compute_forward_mul_mat_id, ggml-cpu.c:7717-7895; K-quants only).
+ * expert_tiles: the experts' tile images (mi355_kq_unpack_tiles of each expert's N x K matrix), expert e at
+ * expert_tiles + e * expert_tiles_bytes.  b: the f32 activations [T][nb1][K] (16-byte aligned, rows K apart); they are
+ * quantized per 256 elements like mi355_quantize_act_q8k, gathered in expert order into one image with 128 rows per column tile.
+ * dst f32 [T][n_used][N].  ws: mi355_mul_mat_id_q8k_tiled_ws_bytes(...) bytes, 16-byte aligned.  Results equal those of
+ * mi355_mul_mat_q8k_tiled on each expert's rows. */
+size_t mi355_mul_mat_id_q8k_tiled_ws_bytes(int64_t K, int64_t n_expert, int64_t n_used, int64_t T);
+int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles, size_t expert_tiles_bytes, const float *b, const int32_t *ids,
+                               int64_t ids_stride, float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T,
+                               void *ws, size_t ws_bytes);
+
 /* Second half of mi355_mul_mat_id: `act` holds the nb1*T rows of b quantized by
  * mi355_quantize_act (row t*nb1 + j). */
 int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride,

@@ -1149,6 +1149,12 @@ __host__ inline size_t route_bytes(int64_t n_expert, int64_t S) {
     return (2 * (size_t)S + 4 * max_tiles + 4) * sizeof(int32_t);
 }
 
+// the routing kernel for launches built elsewhere (the wide-tile kernel's routed form, mmq_w.hip)
+void launch_route_slots(hipStream_t s, const int32_t *ids, int64_t ids_stride, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, int bn,
+                        int32_t *act_row, int32_t *dst_row, int32_t *tiles, int32_t *n_tiles) {
+    MI355_LAUNCH(k_route_slots, dim3(1), dim3(1024), 0, s, ids, ids_stride, n_expert, n_used, nb1, T, bn, act_row, dst_row, tiles, n_tiles);
+}
+
 template <int TYPE>
 static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int64_t act_rows, const int32_t *ids, int64_t ids_stride,
                             float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws) {

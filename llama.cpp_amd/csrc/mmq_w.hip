@@ -208,6 +208,30 @@ __global__ void __launch_bounds__(256) k_quantize_q8k_tiled(const float *__restr
 }
 
 constexpr int WT_BM = 128, WT_BN = 128;
+
+// MUL_MAT_ID on tile images: column tile ct of the sorted slot list (at most 128 slots of one expert) owns rows
+// [128 ct, 128 ct + 128) of the activation image; rows past the tile's slots are zeros.
+struct wt_route {
+    const int32_t *dst_row;
+    const int32_t *tiles;
+    const int32_t *n_tiles;
+    int64_t expert_img_bytes;   // from one expert's weight images to the next
+};
+__global__ void __launch_bounds__(256) k_quantize_q8k_tiled_routed(const float *__restrict__ x, uint8_t *__restrict__ act, int64_t K, int64_t B_img, int64_t x_stride,
+                                                                   const int32_t *__restrict__ act_row, const int32_t *__restrict__ tiles,
+                                                                   const int32_t *__restrict__ n_tiles) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = blockIdx.y;
+    if (sb >= (K >> 8)) return;   // whole wave
+    const int ct = (int)(row / WT_BN);
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (ct < *n_tiles) {
+        const int c = tiles[4 * ct + 1] + (int)(row % WT_BN);
+        if (c < tiles[4 * ct + 2]) v = *(const f32x4 *)(x + (int64_t)act_row[c] * x_stride + sb * QKK + lane * 4);
+    }
+    q8k_quantize_wave_tiled(v, lane, act, K, B_img, row, sb);
+}
 constexpr int WT_A_AUX_TILE = (WT_BN / 16) * WT_A_AUX;       // 4608 bytes of activation scales per tile and super-block
 
 // s_waitcnt that waits until at most n vector-memory operations of this wave are outstanding (nothing else)
@@ -233,8 +257,10 @@ struct wt_launch {
     int n_tiles, n_tiles_padded;   // n_tiles_padded: rounded up to a multiple of 8
 };
 
-template <int TYPE>
-__global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__restrict__ a_img, int64_t K, int64_t B) {
+// ID: MUL_MAT_ID.  The "matrix" is expert 0's images, the column tiles are those of the sorted slot list (rt), B the rows of the
+// activation image (128 per column tile); a tile's rows go to the dst rows of its slots.
+template <int TYPE, bool ID = false>
+__global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__restrict__ a_img, int64_t K, int64_t B, wt_route rt) {
     constexpr bool Q4 = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K;   // sub-block mins: the min term and its scale records
     constexpr int RADIX_SHIFT = TYPE == MI355_Q4_K ? 3 : (TYPE == MI355_Q5_K ? 4 : 6);
     constexpr int NP = 2;                                                      // weight planes
@@ -270,6 +296,14 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__r
     const int ltile = tile - P.m[mi].first_tile;
     const int64_t row0 = (int64_t)(ltile / n_col_tiles) * WT_BM;
     const int64_t col0 = (int64_t)(ltile % n_col_tiles) * WT_BN;
+    int slot_first = 0, slot_end = 0;   // ID: the tile's columns of the sorted slot list
+    if constexpr (ID) {
+        const int ct = ltile % n_col_tiles;
+        if (ct >= *rt.n_tiles) return;   // the whole group
+        w_img += (int64_t)rt.tiles[4 * ct] * rt.expert_img_bytes;
+        slot_first = rt.tiles[4 * ct + 1];
+        slot_end = rt.tiles[4 * ct + 2];
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -530,6 +564,11 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__r
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if constexpr (ID) {
+                const int c = slot_first + (int)(b - col0);
+                if (n < N && c < slot_end) dst[(int64_t)rt.dst_row[c] * dst_stride + n] = acc[tb][r];
+                continue;
+            }
             if (n < N && b < B) {
                 const int64_t o = (b - col0) * dst_stride + (n - row0);
                 out[o] = residual ? acc[tb][r] + residual[o] : acc[tb][r];   // residual may be dst itself: one reader and writer per element
@@ -679,9 +718,9 @@ int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi35
         L.m[0].dst_stride = Ns[0];
     }
     const dim3 grid((unsigned)L.n_tiles_padded, (unsigned)p.slices);
-    if (type == MI355_Q4_K) MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
-    else if (type == MI355_Q5_K) MI355_LAUNCH(k_mmq_w<MI355_Q5_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
-    else MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B);
+    if (type == MI355_Q4_K) MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
+    else if (type == MI355_Q5_K) MI355_LAUNCH(k_mmq_w<MI355_Q5_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
+    else MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
     if (p.slices > 1)
         MI355_LAUNCH(k_wt_split_sum, dim3((unsigned)((Ns[0] * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B,
                      mats[0].dst_stride, p.slices);
@@ -698,6 +737,59 @@ int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const voi
     m.N = N;
     m.dst_stride = dst_stride;
     return mi355_mul_mat_q8k_tiled_multi(stream, type, 1, &m, act, K, B, ws, ws_bytes);
+}
+
+// ---- MUL_MAT_ID on tile images ------------------------------------------------------------------------------------------------
+static int64_t wt_id_max_tiles(int64_t n_expert, int64_t S) { return (S + WT_BN - 1) / WT_BN + n_expert; }
+
+size_t mi355_mul_mat_id_q8k_tiled_ws_bytes(int64_t K, int64_t n_expert, int64_t n_used, int64_t T) {
+    if (K <= 0 || n_expert <= 0 || n_used <= 0 || T <= 0 || K % QKK != 0) return 0;
+    const int64_t S = T * n_used, max_tiles = wt_id_max_tiles(n_expert, S);
+    const size_t img = (wt_act_bytes(K, max_tiles * WT_BN) + 255) & ~(size_t)255;
+    return img + ((2 * (size_t)S + 4 * (size_t)max_tiles + 4) * sizeof(int32_t) + 255 & ~(size_t)255);
+}
+
+int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles, size_t expert_tiles_bytes, const float *b, const int32_t *ids,
+                               int64_t ids_stride, float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T,
+                               void *ws, size_t ws_bytes) {
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K, "mul_mat_id_q8k_tiled: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(N > 0 && K > 0 && n_expert > 0 && n_expert <= 256 && n_used > 0 && nb1 > 0 && T > 0 && K % QKK == 0, "mul_mat_id_q8k_tiled: bad shape");
+    MI355_REQUIRE(ids_stride >= n_used && T * n_used < (1 << 24) && nb1 * T < (1 << 24), "mul_mat_id_q8k_tiled: bad ids stride or too many slots");
+    MI355_REQUIRE(expert_tiles != nullptr && ((uintptr_t)expert_tiles & 15) == 0 && expert_tiles_bytes % 16 == 0 && expert_tiles_bytes >= wt_weight_bytes(type, N, K),
+                  "mul_mat_id_q8k_tiled: expert images must be 16-byte aligned and %zu bytes or more apart", wt_weight_bytes(type, N, K));
+    MI355_REQUIRE(((uintptr_t)b & 15) == 0, "mul_mat_id_q8k_tiled: b must be 16-byte aligned");
+    if (ws == nullptr || ((uintptr_t)ws & 15) != 0 || ws_bytes < mi355_mul_mat_id_q8k_tiled_ws_bytes(K, n_expert, n_used, T)) {
+        set_error("mul_mat_id_q8k_tiled: workspace of %zu bytes, need %zu (16-byte aligned)", ws_bytes, mi355_mul_mat_id_q8k_tiled_ws_bytes(K, n_expert, n_used, T));
+        return MI355_ERR_WORKSPACE;
+    }
+    const int64_t S = T * n_used, max_tiles = wt_id_max_tiles(n_expert, S), B_img = max_tiles * WT_BN;
+    MI355_REQUIRE(B_img <= 65535, "mul_mat_id_q8k_tiled: too many slots for one launch");
+    uint8_t *img = (uint8_t *)ws;
+    int32_t *act_row = (int32_t *)(img + ((wt_act_bytes(K, B_img) + 255) & ~(size_t)255)), *dst_row = act_row + S, *tiles = dst_row + S, *n_tiles = tiles + 4 * max_tiles;
+    hipStream_t s = (hipStream_t)stream;
+    launch_route_slots(s, ids, ids_stride, n_expert, n_used, nb1, T, WT_BN, act_row, dst_row, tiles, n_tiles);
+    const dim3 qgrid((unsigned)((K / QKK + 3) / 4), (unsigned)B_img);
+    MI355_LAUNCH(k_quantize_q8k_tiled_routed, qgrid, dim3(256), 0, s, b, img, K, B_img, K, act_row, tiles, n_tiles);
+    wt_launch L;
+    for (int i = 0; i < 3; i++) {
+        L.m[i].w_img = (const int8_t *)expert_tiles;
+        L.m[i].dst = dst;
+        L.m[i].residual = nullptr;
+        L.m[i].N = N;
+        L.m[i].dst_stride = N;
+        L.m[i].first_tile = i == 0 ? 0 : 0x7fffffff;
+    }
+    const int64_t n_row_tiles = (N + WT_BM - 1) / WT_BM;
+    MI355_REQUIRE(n_row_tiles * max_tiles + 8 < (1 << 30), "mul_mat_id_q8k_tiled: too many tiles");
+    L.n_col_tiles = (int)max_tiles;
+    L.n_tiles = (int)(n_row_tiles * max_tiles);
+    L.n_tiles_padded = (L.n_tiles + 7) & ~7;
+    const wt_route rt = {dst_row, tiles, n_tiles, (int64_t)expert_tiles_bytes};
+    const dim3 grid((unsigned)L.n_tiles_padded);
+    if (type == MI355_Q4_K) MI355_LAUNCH((k_mmq_w<MI355_Q4_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
+    else if (type == MI355_Q5_K) MI355_LAUNCH((k_mmq_w<MI355_Q5_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
+    else MI355_LAUNCH((k_mmq_w<MI355_Q6_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
+    return launch_status("k_mmq_w (routed)");
 }
 
 }  // extern "C"

@@ -64,4 +64,10 @@ __device__ __forceinline__ void q8k_quantize_wave_tiled(const f32x4 &v, int lane
     }
 }
 
+// MUL_MAT_ID: the (token, expert slot) pairs sorted by expert (k_route_slots, mmq_k.hip).  Column c of the sorted list reads
+// activation row act_row[c] and writes dst row dst_row[c]; tiles[4 i] = {expert, first column, end column of the expert, 0} for
+// column tiles of at most bn columns; *n_tiles tiles are in use.  At most 256 experts.
+void launch_route_slots(hipStream_t s, const int32_t *ids, int64_t ids_stride, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, int bn,
+                        int32_t *act_row, int32_t *dst_row, int32_t *tiles, int32_t *n_tiles);
+
 }  // namespace mi355

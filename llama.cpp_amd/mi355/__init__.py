@@ -71,6 +71,8 @@ _SIGNATURES = {
     "mi355_quantize_act_q8k_tiled": (_int, [_p, _p, _p, _i64, _i64, _i64]),
     "mi355_kq_tiles_bytes": (_sz, [_int, _i64, _i64]),
     "mi355_kq_unpack_tiles": (_int, [_p, _int, _p, _p, _i64, _i64]),
+    "mi355_mul_mat_id_q8k_tiled_ws_bytes": (_sz, [_i64, _i64, _i64, _i64]),
+    "mi355_mul_mat_id_q8k_tiled": (_int, [_p, _int, _p, _sz, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_q8k_tiled_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_q8k_tiled_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
@@ -347,6 +349,31 @@ def mul_mat_id(t, as_dev, b, ids, n_used):
     dst = torch.empty((T, n_used, N), dtype=torch.float32, device=b.device)
     check(load().mi355_mul_mat_id(_stream(), t, _ptr(as_dev), _ptr(b), _ptr(ids), ids.stride(0), _ptr(dst), N, K,
                                   n_expert, n_used, nb1, T, _ptr(ws), ws.numel()))
+    return dst
+
+
+def kq_unpack_expert_tiles(t, as_dev):
+    """as_dev uint8 [n_expert, N, row_bytes] device layout -> uint8 [n_expert, tile image bytes]: every expert's tile images"""
+    import torch
+    n_expert, N, rb = as_dev.shape
+    K = rb // BLOCK[t][1] * BLOCK[t][0]
+    per = (load().mi355_kq_tiles_bytes(t, N, K) + 255) // 256 * 256
+    out = torch.empty((n_expert, per), dtype=torch.uint8, device=as_dev.device)
+    for e in range(n_expert):
+        check(load().mi355_kq_unpack_tiles(_stream(), t, _ptr(as_dev[e]), _ptr(out[e]), N, K))
+    return out
+
+
+def mul_mat_id_tiled(t, expert_tiles, N, b, ids, n_used):
+    """expert_tiles from kq_unpack_expert_tiles; b f32 [T, nb1, K]; ids int32 [T, >=n_used] (row-strided) -> f32 [T, n_used, N]"""
+    import torch
+    n_expert = expert_tiles.shape[0]
+    T, nb1, K = b.shape
+    need = load().mi355_mul_mat_id_q8k_tiled_ws_bytes(K, n_expert, n_used, T)
+    ws = torch.empty(need, dtype=torch.uint8, device=b.device)
+    dst = torch.empty((T, n_used, N), dtype=torch.float32, device=b.device)
+    check(load().mi355_mul_mat_id_q8k_tiled(_stream(), t, _ptr(expert_tiles), expert_tiles.stride(0), _ptr(b), _ptr(ids), ids.stride(0), _ptr(dst), N, K,
+                                            n_expert, n_used, nb1, T, _ptr(ws), ws.numel()))
     return dst
 
 

@@ -79,3 +79,55 @@ def test_mul_mat_id_skewed_routing(dev, name, t, pattern):
     got = mi355.mul_mat_id(t, Wd, torch.from_numpy(b).to(dev), idd, n_used).cpu().numpy()
     want = expected_per_expert("cpu", t, Wq, b, np.clip(ids, 0, n_expert - 1), n_expert, n_used, 1, N)
     assert orc.nmse(got, want) < 1e-9
+
+
+@pytest.mark.parametrize("name,t", [("q4_k", orc.Q4_K), ("q5_k", orc.Q5_K), ("q6_k", orc.Q6_K)])
+@pytest.mark.parametrize("n_expert,n_used,nb1_bcast,T,N,K", [(8, 2, True, 512, 192, 2048), (8, 2, False, 300, 64, 4096), (4, 4, True, 70, 256, 2048),
+                                                              (8, 1, False, 3, 130, 2048)])   # Q6_K rows are 16-byte aligned from K = 2048 on
+def test_mul_mat_id_on_tile_images(dev, name, t, n_expert, n_used, nb1_bcast, T, N, K):
+    """the routed form of the wide-tile kernel: slots sorted by expert, activations gathered into one tile image, rows
+    scattered to their slots; against ggml-cpu's arithmetic per expert (Q8_K activations) and the reference's MUL_MAT_ID"""
+    import torch
+    import mi355
+    rng = np.random.default_rng(n_expert + T + N + K)
+    nb1 = 1 if nb1_bcast else n_used
+    Wf = (rng.standard_normal((n_expert * N, K)) * 0.02).astype(np.float32)
+    Wq = orc.quantize("ref" if orc.ref is not None else "oracle", t, Wf)
+    b = rng.standard_normal((T, nb1, K)).astype(np.float32)
+    ids_full = np.stack([rng.permutation(n_expert) for _ in range(T)]).astype(np.int32)
+    Wd = mi355.upload_weights(t, torch.from_numpy(Wq).to(dev)).reshape(n_expert, N, -1)
+    tiles = mi355.kq_unpack_expert_tiles(t, Wd)
+    idd = torch.from_numpy(ids_full).to(dev)[:, :n_used]
+    got = mi355.mul_mat_id_tiled(t, tiles, N, torch.from_numpy(b).to(dev), idd, n_used).cpu().numpy()
+    want = expected_per_expert("cpu", t, Wq, b, ids_full, n_expert, n_used, nb1, N)
+    assert orc.nmse(got, want) < 1e-9
+    if orc.ref is not None:
+        cpu = np.zeros_like(want)
+        assert orc.ref.ref_mul_mat_id(t, orc._ptr(Wq), orc._ptr(b), orc._ptr(ids_full), orc._ptr(cpu), N, K, n_expert, n_used,
+                                      nb1, T, 4, 0) >= 0
+        assert orc.nmse(got, cpu) <= 5e-4      # tests/test-backend-ops.cpp:2001
+
+
+@pytest.mark.parametrize("pattern", ["one_expert", "two_of_eight", "out_of_range"])
+def test_mul_mat_id_on_tile_images_skewed_routing(dev, pattern):
+    """experts without slots, one expert with more slots than a column tile, ids outside [0, n_expert) clamped"""
+    import torch
+    import mi355
+    t = orc.Q4_K
+    n_expert, n_used, T, N, K = 8, 2, 200, 128, 2048
+    rng = np.random.default_rng(6)
+    Wf = (rng.standard_normal((n_expert * N, K)) * 0.02).astype(np.float32)
+    Wq = orc.quantize("ref" if orc.ref is not None else "oracle", t, Wf)
+    b = rng.standard_normal((T, 1, K)).astype(np.float32)
+    if pattern == "one_expert":
+        ids = np.full((T, n_expert), 3, dtype=np.int32)
+    elif pattern == "two_of_eight":
+        ids = np.tile(np.array([[6, 1, 0, 0, 0, 0, 0, 0]], dtype=np.int32), (T, 1))
+    else:
+        ids = rng.integers(-2, n_expert + 2, size=(T, n_expert)).astype(np.int32)
+    Wd = mi355.upload_weights(t, torch.from_numpy(Wq).to(dev)).reshape(n_expert, N, -1)
+    tiles = mi355.kq_unpack_expert_tiles(t, Wd)
+    idd = torch.from_numpy(ids).to(dev)[:, :n_used]
+    got = mi355.mul_mat_id_tiled(t, tiles, N, torch.from_numpy(b).to(dev), idd, n_used).cpu().numpy()
+    want = expected_per_expert("cpu", t, Wq, b, np.clip(ids, 0, n_expert - 1), n_expert, n_used, 1, N)
+    assert orc.nmse(got, want) < 1e-9
