@@ -140,6 +140,12 @@ __device__ __forceinline__ float dpp_max(float v) {
     const int b = __builtin_bit_cast(int, v);
     return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, CTRL, ROWMASK, 0xF, false)));
 }
+// x / (1 + exp(-x)) for the fused SiLU * up launches: exp as v_exp_f32 of a scaled argument and the quotient as a multiplication
+// by v_rcp_f32 (a few 1e-7 relative from the library forms, which cost ~35 instructions per element and made the 512-row
+// launch compute-bound; the reference's own SiLU is a vectorized approximation, ggml-cpu.c:1868-1911).  The unary SILU node
+// keeps the library forms.
+__device__ __forceinline__ float silu_fast(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+
 __device__ __forceinline__ float wave_max_dpp(float v) {
     v = dpp_max<0xB1, 0xF>(v);
     v = dpp_max<0x4E, 0xF>(v);

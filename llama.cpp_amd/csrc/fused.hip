@@ -39,7 +39,7 @@ __global__ void __launch_bounds__(256) k_swiglu_quant(const float *__restrict__ 
         const f32x4 g = *(const f32x4 *)(gate + row * in_stride + e0);
         const f32x4 u = *(const f32x4 *)(up + row * in_stride + e0);
 #pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = (g[i] / (1.0f + expf(-g[i]))) * u[i];
+        for (int i = 0; i < 4; i++) o[i] = silu_fast(g[i]) * u[i];
         if (y) *(f32x4 *)(y + row * y_stride + e0) = o;
     }
     if (act) {

@@ -325,7 +325,7 @@ __global__ void __launch_bounds__(256) k_gemv_gate_up(gemv_batch b, const int8_t
         const int64_t row = (int64_t)block * 32 + j;
         const float gv = load_coherent(b.it[0].dst + col * b.it[0].dst_stride + row);
         const float uv = load_coherent(t.x2 + col * b.it[0].dst_stride + row);
-        const float h = (gv / (1.0f + expf(-gv))) * uv;
+        const float h = silu_fast(gv) * uv;
         quantize_lane32(h, t.act_q + (int64_t)col * t.n, t.act_s + (int64_t)col * (t.n >> 5), row);
     }
 }
