@@ -258,19 +258,8 @@ def sweep(kinds):
                         sws = torch.empty(int(lib.mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B)) + 256, dtype=torch.uint8, device=dev)
                         us = timed(lambda i: mi355.check(lib.mi355_mul_mat_q8k_tiled(stream.cuda_stream, t, tiles[i].data_ptr(), a8.data_ptr(), out.data_ptr(), None,
                                                                                      N, K, B, N, sws.data_ptr(), sws.numel())), nm, 5)
-                        # the shader clock while this kernel runs back to back: a one-wave probe on a second stream
-                        probe = torch.zeros(2, dtype=torch.int64, device=dev)
-                        side = torch.cuda.Stream()
-                        with torch.cuda.stream(stream):
-                            for _ in range(int(1500 / us) + 8):
-                                mi355.check(lib.mi355_mul_mat_q8k_tiled(stream.cuda_stream, t, tiles[0].data_ptr(), a8.data_ptr(), out.data_ptr(), None, N, K, B, N,
-                                                                        sws.data_ptr(), sws.numel()))
-                        mi355.check(lib.mi355_probe_clock(side.cuda_stream, probe.data_ptr(), 500))
-                        torch.cuda.synchronize()
-                        mhz = float(probe[0]) / max(float(probe[1]), 1.0) * 100.0
                         emit(kernel="wide-tile GEMM on tile images, batch %d" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
-                             achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops,
-                             shader_clock_mhz=round(mhz), frac_at_measured_clock=round(ops / us / 1e6 / (INT8_PEAK_TOPS * mhz / 2400.0), 4))
+                             achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
                         del tiles
                     if t == mi355.Q6_K and B == 512 and not wide_only:   # the same product from the unpacked planes (the 64 x 128 tile kernel)
                         planes = [torch.empty(int(lib.mi355_kq_planes_bytes(N, K)) + 256, dtype=torch.uint8, device=dev) for _ in range(nm)]
@@ -283,41 +272,6 @@ def sweep(kinds):
                              achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
                         del planes
                     del Ws
-    if "limits" in kinds:
-        # What bounds the wide-tile GEMM at batch 512.  (1) The rate at which a compute unit fills LDS from L2 / HBM with the
-        # transfers the kernel uses, against the bytes it needs per matrix instruction.  (2) Yardstick: the vendor library's plain
-        # dense GEMMs (torch.matmul f16, torch._int_mm int8: no quantization scales, one operand plane) on the same shapes.
-        n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
-        src = torch.zeros(n_cu * (4 << 20), dtype=torch.uint8, device=dev)
-        ticks = torch.zeros(n_cu, dtype=torch.int64, device=dev)
-        iters = 4096
-        for region, where in ((64 << 10, "L2-resident (64 KiB per group)"), (4 << 20, "streaming from HBM (4 MiB per group)")):
-            probe = lambda i: mi355.check(lib.mi355_probe_lds_fill(stream.cuda_stream, src.data_ptr(), src.numel(), region, n_cu, iters, ticks.data_ptr()))
-            us = timed(probe, 1, 3)
-            per_group = iters * 8192
-            emit(kernel="global-to-LDS fill rate (k_probe_lds_fill, one 512-thread group per compute unit)", case=where, us=round(us, 1),
-                 aggregate_tb_s=round(per_group * n_cu / us / 1e6, 2), bytes_per_clock_per_cu=round(per_group / float(ticks.double().mean()), 1),
-                 shader_clock_mhz=round(float(ticks.double().mean()) / us),
-                 note="k_mmq_w moves 24.6 KiB of operands + 2.5 KiB of scale records per 64-element stage = 64 matrix instructions of 32 clocks on 4 SIMDs: "
-                      "53 bytes per clock would keep the matrix pipes busy")
-        for N, K in shapes:
-            B = 512
-            ops = 2.0 * N * K * B
-            for dt, nm_ in ((torch.float16, "f16"), (torch.int8, "int8")):
-                if dt == torch.int8:
-                    ws_ = [torch.randint(-100, 100, (K, N), device=dev, dtype=torch.int8) for _ in range(4)]
-                    xi = torch.randint(-100, 100, (B, K), device=dev, dtype=torch.int8)
-                    fn = lambda i: torch._int_mm(xi, ws_[i])
-                else:
-                    ws_ = [torch.randn(N, K, device=dev, dtype=dt) for _ in range(4)]
-                    xi = torch.randn(B, K, device=dev, dtype=dt)
-                    fn = lambda i: torch.matmul(xi, ws_[i].t())
-                with torch.cuda.stream(stream):
-                    us = timed(fn, 4, 5)
-                emit(kernel="yardstick: vendor library dense GEMM, batch 512 (not part of the product)", case="%s %dx%d" % (nm_, N, K), us=round(us, 2), bound="mfma",
-                     achieved=round(ops / us / 1e6, 1), unit="TFLOP/s" if dt == torch.float16 else "TOP/s",
-                     frac=round(ops / us / 1e6 / (F16_PEAK_TFLOPS if dt == torch.float16 else INT8_PEAK_TOPS), 4), ops=ops)
-                del ws_
     if "fattn" in kinds or "fattn_long" in kinds or "fattn_prefill" in kinds or "fattn_prefill_512" in kinds:
         H, HK, D = 32, 8, 128
         cases = [(1, 256), (1, 512), (1, 1024), (1, 4096), (1, 32768), (1, 131072), (512, 512), (512, 4096), (2048, 2048), (4096, 4096)]
@@ -362,7 +316,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
     ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, mmq_wide (the wide-tile GEMM on 14336 x 4096 at batch 512 only), fattn, "
-                                          "fattn_long (decode over 131072 cells only), fattn_prefill (4096 x 4096 prefill only), fattn_prefill_512 (512 rows over 4096 cells only), limits (LDS fill rate of a compute unit and the vendor library's dense GEMMs on the prefill shapes)")
+                                          "fattn_long (decode over 131072 cells only), fattn_prefill (4096 x 4096 prefill only), fattn_prefill_512 (512 rows over 4096 cells only)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="rewrite the tracked HBM-traffic summary from two rocprofv3 --pmc output directories (no GPU needed)")
     args = ap.parse_args()

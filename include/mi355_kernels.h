@@ -43,17 +43,6 @@ uint64_t mi355_launch_count(void);
  * Counterpart of a backend's score function (ggml/src/ggml-backend-impl.h:212-214). */
 int mi355_device_supported(int device);
 
-/* Measurement aid, no counterpart in the reference: one wave spins for `micros` microseconds on `stream` and writes
- * out[0] = shader-clock ticks, out[1] = ticks of the constant 100 MHz reference counter that passed meanwhile (DEVICE int64[2]).
- * Launched on a second stream next to a kernel under test, out[0] / out[1] * 100 is the clock in MHz that kernel gets. */
-int mi355_probe_clock(void *stream, int64_t *out, int64_t micros);
-/* Measurement aid, no counterpart in the reference: the rate at which compute units fill LDS with the 16-byte-per-lane
- * global-to-LDS transfers that feed the wide-tile GEMM.  `n_groups` 512-thread groups (one per compute unit when n_groups is the
- * number of compute units) each move iters * 8 KiB out of their own `region` bytes of `src` (region a multiple of 8 KiB,
- * n_groups * region <= src_bytes; 64 KiB regions stay in L2, 4 MiB regions stream from HBM), six 1 KiB transfers in flight per
- * wave.  out[g] (DEVICE int64[n_groups]) = shader-clock ticks group g took. */
-int mi355_probe_lds_fill(void *stream, const void *src, int64_t src_bytes, int64_t region, int n_groups, int iters, int64_t *out);
-
 /* Weight storage -------------------------------------------------------------------- *
  * Quantized weight rows are kept in HBM in a per-row "device layout" that makes every
  * load a 16-byte aligned, coalesced access:
@@ -113,8 +102,12 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
  * the process ends; the call performs no hipMalloc / hipFree and calls no allocating library routine.  Products whose
  * quantized activation does not fit (mi355_mul_mat_ws_bytes(K, B) > the array, e.g. K = 14336 beyond B = 936) are rejected with
  * MI355_ERR_WORKSPACE.  Same result as mi355_mul_mat with a workspace of that size.  Every call on one GPU shares that
- * GPU's array: calls that overlap in time on one GPU (different streams or threads) race on it. */
+ * GPU's array: calls that overlap in time on one GPU (different streams or threads) race on it.
+ * mi355_mul_mat_static_init() looks the array's device address up for the current device (the first lookup on a device may load
+ * the code object and place the array); call it once per device at set-up, outside any stream capture.  A first
+ * mi355_mul_mat_static call on a device makes the same lookup itself. */
 size_t mi355_mul_mat_static_max_ws(void);
+int mi355_mul_mat_static_init(void);
 int mi355_mul_mat_static(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
                          int64_t x_stride, int64_t dst_stride);
 

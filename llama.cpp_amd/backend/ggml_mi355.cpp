@@ -157,6 +157,13 @@ struct backend_ctx {
     unsigned * tickets = nullptr;   // zeroed arrival counters of the gate/up launch (one per 32 output rows)
     size_t n_tickets = 0;
     long async_uploads = 0, events_recorded = 0;   // reported with MI355_GRAPH_STATS=1
+    // Host-to-device hand-over of split inputs (backend_cpy_tensor_async): the bytes are copied into one of these pinned slots
+    // at the call and uploaded from there, so the upload never reads the caller's memory after the call returns.
+    static constexpr int STAGE_SLOTS = 8;
+    static constexpr size_t STAGE_BYTES = (size_t) 1 << 20;
+    void * stage = nullptr;                 // STAGE_SLOTS x STAGE_BYTES of pinned host memory, allocated at the first use
+    hipEvent_t stage_done[STAGE_SLOTS] = {};   // recorded after the upload that reads slot i
+    int stage_next = 0;
     const ggml_tensor * done_ahead = nullptr;      // a product that went out with an earlier node's launch (see tiled_multi)
 
     // ---- replay of decode graphs as HIP graphs (see backend_graph_compute)
@@ -898,6 +905,9 @@ void backend_free(ggml_backend_t backend) {
     if (ctx->iota) (void) hipFree(ctx->iota);
     if (ctx->cells) (void) hipFree(ctx->cells);
     if (ctx->tickets) (void) hipFree(ctx->tickets);
+    if (ctx->stage) (void) hipHostFree(ctx->stage);
+    for (hipEvent_t e : ctx->stage_done)
+        if (e) (void) hipEventDestroy(e);
     if (ctx->replay.exec) (void) hipGraphExecDestroy(ctx->replay.exec);
     if (ctx->replay.graph) (void) hipGraphDestroy(ctx->replay.graph);
     if (getenv("MI355_GRAPH_STATS"))
@@ -942,8 +952,11 @@ void backend_get_tensor_async(ggml_backend_t backend, const ggml_tensor * tensor
 }
 
 // Copies a tensor into one of this backend's tensors on its stream (ggml_backend_tensor_copy_async, ggml-backend.cpp:380-409; the
-// scheduler hands split inputs over this way, :1384).  Served: a source in host memory produced by a backend that computes
-// synchronously (the CPU backend: its result is complete when the scheduler gets here), and a source of this same backend.
+// scheduler hands split inputs over this way, :1384).  Served: a source of this same backend, and a source in host memory
+// produced by a backend that computes synchronously (the CPU backend: its result is complete when the scheduler gets here) of
+// up to STAGE_BYTES.  A host source is copied into a pinned slot of this backend before the call returns and uploaded from the
+// slot: the scheduler keeps the source alive only until the consuming split starts, and a later CPU split may reuse that
+// memory while an upload that read it directly (a true DMA when the source is pinned) would still be in flight.
 // Anything else returns false and the caller synchronizes and copies.
 bool backend_cpy_tensor_async(ggml_backend_t backend_src, ggml_backend_t backend_dst, const ggml_tensor * src, ggml_tensor * dst) {
     backend_ctx * ctx = (backend_ctx *) backend_dst->context;
@@ -952,18 +965,33 @@ bool backend_cpy_tensor_async(ggml_backend_t backend_src, ggml_backend_t backend
     if (!dbuf || !sbuf || dbuf->buft->iface.get_name != buft_get_name || dbuf->buft->device != backend_dst->device) return false;
     if (!ggml_is_contiguous(src) || !ggml_is_contiguous(dst) || src->type != dst->type || ggml_nbytes(src) != ggml_nbytes(dst)) return false;
     if (repack_of(dst).yes || is_repacked_type(src->type)) return false;   // layout permutations take the synchronous path
-    hipMemcpyKind kind;
+    const size_t n = ggml_nbytes(src);
     if (ggml_backend_buffer_is_host(sbuf)) {
         ggml_backend_dev_t sdev = ggml_backend_get_device(backend_src);
         if (!sdev || ggml_backend_dev_type(sdev) != GGML_BACKEND_DEVICE_TYPE_CPU) return false;
-        kind = hipMemcpyHostToDevice;
+        if (n > backend_ctx::STAGE_BYTES) return false;
+        MI355_HIP_OK(hipSetDevice(ctx->device));
+        if (!ctx->stage) {
+            if (hipHostMalloc(&ctx->stage, backend_ctx::STAGE_SLOTS * backend_ctx::STAGE_BYTES, hipHostMallocDefault) != hipSuccess) {
+                (void) hipGetLastError();
+                ctx->stage = nullptr;
+                return false;
+            }
+            for (hipEvent_t & e : ctx->stage_done) MI355_HIP_OK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        }
+        const int slot = ctx->stage_next;
+        ctx->stage_next = (slot + 1) % backend_ctx::STAGE_SLOTS;
+        MI355_HIP_OK(hipEventSynchronize(ctx->stage_done[slot]));   // the upload that last read this slot (never recorded: returns at once)
+        void * at = (char *) ctx->stage + (size_t) slot * backend_ctx::STAGE_BYTES;
+        memcpy(at, src->data, n);
+        MI355_HIP_OK(hipMemcpyAsync(dst->data, at, n, hipMemcpyHostToDevice, ctx->stream));
+        MI355_HIP_OK(hipEventRecord(ctx->stage_done[slot], ctx->stream));
     } else if (backend_src == backend_dst && sbuf->buft == dbuf->buft) {
-        kind = hipMemcpyDeviceToDevice;
+        MI355_HIP_OK(hipSetDevice(ctx->device));
+        MI355_HIP_OK(hipMemcpyAsync(dst->data, src->data, n, hipMemcpyDeviceToDevice, ctx->stream));
     } else {
         return false;
     }
-    MI355_HIP_OK(hipSetDevice(ctx->device));
-    MI355_HIP_OK(hipMemcpyAsync(dst->data, src->data, ggml_nbytes(src), kind, ctx->stream));
     ctx->cache.valid = false;
     return true;
 }

@@ -398,11 +398,11 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
     // One token over a long cache (head size 128, up to four query heads per kv head): the per-wave streaming kernel.  Measured on
     // the 32-over-8-head shape: 12.2 us against 13.7 at 4096 cells, 36 against 41 at 32768, 105 against 117 at 131072; below about
     // 3000 cells fewer than 512 of its 64-cell tiles exist and the kernel below is ahead (10.2 against 11.2 us at 2048).
-    static const int64_t stream_min = getenv("MI355_FA_STREAM_MIN") ? atoll(getenv("MI355_FA_STREAM_MIN")) : 3072;
+    constexpr int64_t stream_min = 3072;
     // 257 .. 512 cells: one launch with a wave per 64 cells (8.4 / 8.6 us at 384 / 512 cells against 9.0 for the split form below
     // with its merge launch; up to 256 cells the vector kernel further down is ahead, 6.8 against 7.1 us)
-    static const int64_t short_min = getenv("MI355_FA_SHORT_MIN") ? atoll(getenv("MI355_FA_SHORT_MIN")) : 256;
-    static const int64_t short_max = getenv("MI355_FA_SHORT_MAX") ? atoll(getenv("MI355_FA_SHORT_MAX")) : 512;
+    constexpr int64_t short_min = 256;
+    constexpr int64_t short_max = 512;
     if (Nq == 1 && Nkv > short_min && Nkv <= short_max && D == 128 && R <= 4) {
         const int rc = launch_fattn_dec_short(s, a, D);
         if (rc <= 0) return rc;

@@ -112,6 +112,8 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
 
 size_t mi355_mul_mat_static_max_ws(void) { return STATIC_SCRATCH_BYTES; }
 
+int mi355_mul_mat_static_init(void) { return static_scratch() ? MI355_OK : MI355_ERR_HIP; }
+
 int mi355_mul_mat_static(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
                          int64_t x_stride, int64_t dst_stride) {
     MI355_REQUIRE(K > 0 && B > 0, "mul_mat_static: bad shape K=%lld B=%lld", (long long)K, (long long)B);

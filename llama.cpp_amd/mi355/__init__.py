@@ -39,8 +39,6 @@ _SIGNATURES = {
     "mi355_last_error": (C.c_char_p, []),
     "mi355_launch_count": (C.c_uint64, []),
     "mi355_device_supported": (_int, [_int]),
-    "mi355_probe_clock": (_int, [_p, _p, _i64]),
-    "mi355_probe_lds_fill": (_int, [_p, _p, _i64, _i64, _int, _int, _p]),
     "mi355_weights_scatter": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
     "mi355_weights_gather": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
     "mi355_quantize_q8_1": (_int, [_p, _p, _p, _i64, _i64, _i64]),
@@ -49,6 +47,7 @@ _SIGNATURES = {
     "mi355_mul_mat_ws_bytes": (_sz, [_i64, _i64]),
     "mi355_mul_mat": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_static_max_ws": (_sz, []),
+    "mi355_mul_mat_static_init": (_int, []),
     "mi355_mul_mat_static": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
     "mi355_mul_mat_q": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),

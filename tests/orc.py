@@ -127,6 +127,17 @@ def quantize(lib_kind, t, x):
     return out
 
 
+def quantize_mt(lib_kind, t, x, threads=16):
+    """quantize() over row chunks on `threads` host threads (the C calls release the interpreter lock): whole 8B-model matrices"""
+    from concurrent.futures import ThreadPoolExecutor
+    x = f32(x)
+    n = x.shape[0]
+    step = max(64, (n + 4 * threads - 1) // (4 * threads))
+    with ThreadPoolExecutor(max_workers=threads) as ex:
+        parts = list(ex.map(lambda i: quantize(lib_kind, t, x[i:i + step]), range(0, n, step)))
+    return np.concatenate(parts)
+
+
 def dequantize(lib_kind, t, q, k):
     q = np.ascontiguousarray(q, dtype=np.uint8)
     nrows = q.shape[0]

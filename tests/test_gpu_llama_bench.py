@@ -156,6 +156,28 @@ def test_model_logits_cpu_vs_plugin_and_fused_vs_nodes(dev, tmp_path, n_prompt):
     assert orc.nmse(fused, cpu) < 2e-3
 
 
+def test_model_logits_full_width_8b_layers(dev, tmp_path):
+    """Two layers at the full width of BASELINE config 3 (d 4096, ffn 14336, 32 / 8 heads, vocabulary 128256, Q4_K_M mix): the
+    reference's runtime on its CPU backend and on the plug-in.  At this width the decode launches are the instantiations the timed
+    benchmark step uses (gate + up in one launch with two rows per wave and the activation in LDS, the 128256-row output
+    projection), which smaller models never reach."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / "wide.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=128256)
+    for n_prompt in (5, 256):
+        cpu = _logits(model, 0, n_prompt, 4, str(tmp_path / "cpu.bin"))
+        fused = _logits(model, 99, n_prompt, 4, str(tmp_path / "fused.bin"))
+        nodes = _logits(model, 99, n_prompt, 4, str(tmp_path / "nodes.bin"), fusion=False, graphs=False)
+        assert cpu.shape == fused.shape == nodes.shape and cpu.size % 128256 == 0 and np.isfinite(fused).all()
+        assert orc.nmse(fused, nodes) < (1e-6 if n_prompt <= 8 else 5e-4)
+        assert orc.nmse(nodes, cpu) < 2e-3 and orc.nmse(fused, cpu) < 2e-3
+
+
 @pytest.mark.parametrize("cache", [("q8_0", "q8_0"), ("q4_0", "q4_0"), ("q8_0", "f16")])
 @pytest.mark.parametrize("n_prompt", [5, 200])
 def test_model_logits_quantized_kv_cache(dev, tmp_path, cache, n_prompt):

@@ -53,3 +53,36 @@ def test_static_scratch_rejects_oversize(dev):
     dst = torch.zeros((B, 32), dtype=torch.float32, device=dev)
     with pytest.raises(mi355.Mi355Error, match="scratch"):
         mi355.mul_mat_static(mi355.Q4_K, W, x, dst)
+
+
+def test_static_scratch_allocates_nothing_and_runs_under_capture(dev):
+    """after mi355_mul_mat_static_init the calls leave the device's free memory unchanged, and a call recorded into a HIP graph
+    gives the eager result on every replay"""
+    import torch
+    import mi355
+    lib = mi355.load()
+    mi355.check(lib.mi355_mul_mat_static_init())
+    t = mi355.Q4_K
+    cases = [_case(dev, t, N, K, B, 300 + i) + (N, B) for i, (N, K, B) in enumerate([(512, 4096, 320), (256, 2048, 8), (128, 1024, 1)])]
+    outs = [torch.zeros((B, N), dtype=torch.float32, device=dev) for _, _, _, N, B in cases]
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for (W, x, _, _, _), out in zip(cases, outs):
+        mi355.mul_mat_static(t, W, x, out)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    W, x, _, N, B = cases[0]
+    eager = outs[0].clone()
+    out = torch.zeros_like(eager)
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        mi355.mul_mat_static(t, W, x, out)
+    for rep in range(3):
+        out.zero_()
+        mi355.mul_mat_static(t, cases[1][0], cases[1][1], outs[1])     # eager work on the same array between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
