@@ -22,7 +22,7 @@ HBM_PEAK_GBS = 8000.0
 # the readings of the plain copy kernel the run ends with.  `python bench.py --traffic-from <fetch dir> <write dir>` turns the two
 # counter runs into this file, together with the commit they were measured at; the bench line quotes both.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv_gate_up_q4k_hbm_traffic.txt")
-ROOFLINE_KERNEL = "k_gemv_multi"        # as it appears in the profiler's kernel names
+ROOFLINE_KERNEL = "k_gemv_gate_up_blk"        # as it appears in the profiler's kernel names
 COPY_KERNEL = "k_cpy"
 COPY_BYTES = 16384 * 4096 * 4           # read, and as many written
 
@@ -72,8 +72,8 @@ def traffic_from(fetch_dir, write_dir):
     fetch_b = out["FETCH_SIZE"][0] * out["FETCH_SIZE"][5]
     write_b = out["WRITE_SIZE"][0] * out["WRITE_SIZE"][5]
     lines = [
-        "HBM traffic of the roofline kernel of bench.py: k_gemv_multi<1 column, 2 rows per wave, activation copy in LDS> on the ffn_gate + ffn_up",
-        "matrices of one layer (2 x 14336 x 4096 Q4_K) - the launch a decoded token makes 32 times - on one MI355X",
+        "HBM traffic of the roofline kernel of bench.py: k_gemv_gate_up_blk<Q4_K, 1 column, 8 waves, 4 + 4 rows in flight> on the ffn_gate + ffn_up",
+        "matrices of one layer (2 x 14336 x 4096 Q4_K, SiLU * up + Q8_1 inside) - the launch a decoded token makes 32 times - on one MI355X",
         "",
         "commands (from /tmp, TMPDIR=/tmp; counters in their own runs, no trace domains):",
         "  rocprofv3 --pmc FETCH_SIZE -d <fetch dir> -o f --output-format csv -- python3 bench.py --no-cpu --pp 0 --steps 4 --warmup 2",
@@ -93,7 +93,7 @@ def traffic_from(fetch_dir, write_dir):
         "measured_at_commit: %s" % commit,
         "",
         "algorithmic bytes per launch: 2 x 14336 x 4096 x 144/256 (weights) + 4096 x 1.25 (Q8_1 activation: levels + scale/sum pairs)",
-        "  + 2 x 4 x 14336 (f32 outputs) = 66,060,288 + 5,120 + 114,688 = 66,180,096 B",
+        "  + 2 x 4 x 14336 (f32 outputs) + 14336 x 1.25 (Q8_1 of SiLU * up) = 66,060,288 + 5,120 + 114,688 + 17,920 = 66,198,016 B",
     ]
     with open(TRAFFIC_FILE, "w") as f:
         f.write("\n".join(lines) + "\n")
@@ -407,31 +407,38 @@ def main():
             pp = T * reps / (time.perf_counter() - t0)
 
     # ------------------------------------------------------------------ roofline of the dominant kernel
-    # k_gemv_multi on ffn_gate + ffn_up (2 x 14336 x 4096 Q4_K in one launch): what the timed step launches 32 times per token,
-    # 46% of the bytes of a decoded token.  Timed with HIP events on its own stream through the runner's own call, over the 32
-    # layers' matrices (2.1 GB, so neither L2 nor the 256 MB Infinity Cache can serve them).
+    # k_gemv_gate_up_blk on ffn_gate + ffn_up (2 x 14336 x 4096 Q4_K, SiLU * up and its Q8_1 quantization inside the launch): what
+    # the timed step launches 32 times per token, 46% of the bytes of a decoded token.  Timed with HIP events on its own stream
+    # through the runner's own call, over the 32 layers' matrices (2.1 GB, so neither L2 nor the 256 MB Infinity Cache can serve them).
     N, K = cfg.n_ff, cfg.n_embd
-    pairs = [[(L["gate"], run.gate[:1]), (L["up"], run.up[:1])] for L in weights.layers]
+    pairs = [(L["gate"], L["up"]) for L in weights.layers]
+
+    def gate_up(pair):
+        (tg, Wg), (tu, Wu) = pair
+        mi355.check(lib.mi355_ffn_gate_up_swiglu(stream.cuda_stream, tg, Wg.data_ptr(), tu, Wu.data_ptr(), run.act_c.data_ptr(), run.gate.data_ptr(),
+                                                 run.up.data_ptr(), N, run.act_b.data_ptr(), run.tickets.data_ptr(), N, K, 1))
+
     with torch.cuda.stream(stream):
         run._norm_quant(run.x[:1], weights.layers[0]["ffn_norm"], run.act_c, 1)
         for gu in pairs[:4]:
-            run._mm_act(gu, run.act_c, K, 1)
+            gate_up(gu)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         nrep = 8
         e0.record(stream)
         for _ in range(nrep):
             for gu in pairs:
-                run._mm_act(gu, run.act_c, K, 1)
+                gate_up(gu)
         e1.record(stream)
         stream.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / (nrep * len(pairs))
-    wtypes = {t for gu in pairs for (t, _), _ in gu}
+    wtypes = {t for gu in pairs for t, _ in gu}
     assert wtypes == {mi355.Q4_K}, "the roofline kernel's byte count assumes Q4_K gate/up matrices"
-    alg_bytes = 2 * (N * K * 144 // 256) + (K + K // 4) + 2 * 4 * N      # weights + Q8_1 activation + two f32 outputs
+    # weights + Q8_1 activation in + two f32 outputs + Q8_1 activation out
+    alg_bytes = 2 * (N * K * 144 // 256) + (K + K // 4) + 2 * 4 * N + (N + N // 4)
     achieved = alg_bytes / us / 1e3                                       # GB/s
     traffic, traffic_commit = read_traffic()
-    roofline = {"kernel": "k_gemv_multi<1 column, 2 rows per wave, activation in LDS> on ffn_gate + ffn_up, 2 x 14336 x 4096 Q4_K (the launch the timed "
-                          "step makes once per layer)", "bound": "hbm", "achieved": round(achieved, 1),
+    roofline = {"kernel": "k_gemv_gate_up_blk<Q4_K, 1 column, 8 waves, 4 + 4 rows in flight> on ffn_gate + ffn_up with SiLU * up + Q8_1, 2 x 14336 x 4096 "
+                          "(the launch the timed step makes once per layer)", "bound": "hbm", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "traffic_source": "profiles/%s, measured at commit %s" % (os.path.basename(TRAFFIC_FILE), traffic_commit) if traffic else None,
                 "us_per_launch": round(us, 3), "algorithmic_bytes_per_launch": alg_bytes}

@@ -439,6 +439,8 @@ int mi355_rms_norm_qkv_rope_store(void *stream, const float *x, const float *nor
 int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, int type_up, const void *w_up, const void *act, float *gate,
                              float *up, int64_t out_stride, void *act_out, unsigned *counters, int64_t N, int64_t K, int64_t B);
 
+
+
 /* Quantized KV cache (llama.cpp's -ctk / -ctv q8_0, q4_0).
  * Where a block lives: with row_blocks = 0 blocks sit where ggml puts them (block g of a tensor at g * block bytes from its data).
  * A tensor kept in the device row layout of mi355_weights_scatter (all levels of a row, then the row's scales) is addressed through

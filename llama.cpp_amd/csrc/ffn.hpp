@@ -1,0 +1,12 @@
+// Launches of ffn.hip that other translation units call.
+#pragma once
+#include "common.hpp"
+
+namespace mi355 {
+
+// gate + up + SiLU * up + Q8_1 by groups that own whole 32-row blocks of both matrices (both of type `type`); act_out in the
+// mi355_quantize_act layout of B rows of N.  B <= 4, N % 32 == 0, B * 1.25 K bytes of LDS.
+int launch_gate_up_blk(hipStream_t s, int type, const void *w_gate, const void *w_up, const int8_t *aq, const act_ds *ads, int64_t K, int64_t B,
+                       float *gate, float *up, int64_t out_stride, void *act_out, int64_t N);
+
+}  // namespace mi355

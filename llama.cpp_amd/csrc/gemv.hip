@@ -12,6 +12,7 @@
 #include "common.hpp"
 #include "qdot.hpp"
 #include "norm_quant.hpp"
+#include "ffn.hpp"
 
 #include <math.h>
 #include <stdlib.h>
@@ -280,26 +281,6 @@ __device__ __forceinline__ float load_coherent(const float *p) {   // bypasses c
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Q8_1 of one value per lane over aligned groups of 32 lanes (quantize_row_q8_1_ref, ggml-quants.c:220-253)
-__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
-    float amax = fabsf(v);
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-    const float d = amax / 127.0f;
-    const float id = d != 0.0f ? 1.0f / d : 0.0f;
-    const int q = (int)roundf(v * id);
-    int sum = q;
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    qrow[e] = (int8_t)q;
-    if ((e & 31) == 0) {
-        act_ds o;
-        o.d = half_bits_to_float(float_to_half_bits(d));
-        o.sum = sum;
-        srow[e >> 5] = o;
-    }
-}
-
 // gate and up projections (llm_build_ffn, src/llama.cpp:280-320) with UNARY(SILU), MUL and the Q8_1 quantization of
 // the product done per 32-row block by whichever of the block's 8 groups (4 per matrix, 8 rows each) finishes last
 template <int NCOLS, bool LDSA>
@@ -326,7 +307,7 @@ __global__ void __launch_bounds__(256) k_gemv_gate_up(gemv_batch b, const int8_t
         const float gv = load_coherent(b.it[0].dst + col * b.it[0].dst_stride + row);
         const float uv = load_coherent(t.x2 + col * b.it[0].dst_stride + row);
         const float h = silu_fast(gv) * uv;
-        quantize_lane32(h, t.act_q + (int64_t)col * t.n, t.act_s + (int64_t)col * (t.n >> 5), row);
+        quantize_lane32<false>(h, t.act_q + (int64_t)col * t.n, t.act_s + (int64_t)col * (t.n >> 5), row);
     }
 }
 
@@ -723,6 +704,12 @@ int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, in
     if (rc != MI355_OK) return rc;
     rc = check_gemv_args("ffn_gate_up_swiglu", type_up, w_up, N, K, out_stride);
     if (rc != MI355_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + B * K);
+    // both matrices of one type, the activation rows fit in LDS: the launch whose groups own whole Q8_1 blocks (ffn.hip; no counters used)
+    if (type_gate == type_up && B * (K + K / 4) <= 40960 && N / 32 < 0x7fffffff)
+        return launch_gate_up_blk(s, type_gate, w_gate, w_up, aq, ads, K, B, gate, up, out_stride, act_out, N);
     const int64_t per = N / 8;   // groups per matrix: 4 waves x 2 rows
     MI355_REQUIRE(2 * per < 0x7fffffff, "ffn_gate_up_swiglu: too many rows for one launch");
     gemv_batch b;
@@ -743,9 +730,6 @@ int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, in
     t.counters = counters; t.x2 = up; t.n = (int)N;
     t.act_q = (int8_t *)act_out;
     t.act_s = (act_ds *)(t.act_q + B * N);
-    hipStream_t s = (hipStream_t)stream;
-    const int8_t *aq = (const int8_t *)act;
-    const act_ds *ads = (const act_ds *)(aq + B * K);
     const dim3 grid((unsigned)(2 * per));
     const size_t lds = act_lds_bytes((int)B, K, 2 * per);
     switch (B) {

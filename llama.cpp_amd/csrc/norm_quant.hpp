@@ -38,11 +38,46 @@ __device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, i
     }
 }
 
+// Q8_1 of one value per lane over aligned groups of 32 lanes (quantize_row_q8_1_ref, ggml-quants.c:220-253); e = index of the
+// lane's element in the row.  COH: the block is stored with device scope (four levels per store, the {d, sum} pair as one
+// 8-byte store), for rows that other groups of the same launch read after a grid-wide step.
+template <bool COH = false>
+__device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q = (int)roundf(v * id);
+    int sum = q;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    act_ds o;
+    o.d = half_bits_to_float(float_to_half_bits(d));
+    o.sum = sum;
+    if constexpr (COH) {
+        u32 packed = (u32)(q & 0xFF);
+        packed |= ((u32)__shfl_down(q, 1, 64) & 0xFFu) << 8;
+        packed |= ((u32)__shfl_down(q, 2, 64) & 0xFFu) << 16;
+        packed |= ((u32)__shfl_down(q, 3, 64) & 0xFFu) << 24;
+        if ((e & 3) == 0) __hip_atomic_store((u32 *)(qrow + e), packed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((e & 31) == 0) {
+            const unsigned long long bits = (unsigned long long)__builtin_bit_cast(u32, o.d) | ((unsigned long long)(u32)o.sum << 32);
+            __hip_atomic_store((unsigned long long *)(srow + (e >> 5)), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    } else {
+        qrow[e] = (int8_t)q;
+        if ((e & 31) == 0) srow[e >> 5] = o;
+    }
+}
+
 // One row: xr -> y row (optional) and row `row` of the activation workspace `act` (optional), which holds nrows rows of k.
 // Each thread keeps its NV float4 of the row in registers (k <= 1024 * NV).  COH: the row was written by other groups of the
 // same launch with device-scope stores and is read with device-scope loads.  sh: 4 floats of LDS; the caller places a
 // barrier between two calls that share it.
 // FMT: activation format written to `act`: 0 Q8_1 (split layout), 1 per-super-block (q8k.hpp), 2 the same as tile images (tiles.hpp)
+// Called by the first 256 threads of a group; contains exactly one group barrier, which further waves of a larger group must
+// match with a barrier of their own.
 template <int NV, int FMT, bool COH>
 __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr, const float *__restrict__ w, float *__restrict__ yr,
                                                    void *__restrict__ act, int64_t row, int64_t k, int64_t nrows, float eps, float *sh) {

@@ -116,10 +116,10 @@ class LlamaRunner:
         self.use_tiles = True
         self.tiles = {}
         self.split_ws = None    # partial sums of tile products that are split along K (grown on first use, before any graph capture)
-        # decode, T <= 4: SiLU*up + Q8_1 either by the last group of each 32-row block of the gate/up launch (True) or as a launch
-        # of their own after a two-matrix product (False).  With the activation staged in LDS the two-launch form is the quicker
-        # one (15.9 us against 16.3-16.8 us per layer on the 8B shape); both give the same bits.
-        self.fuse_tail = False
+        # decode, T <= 4: SiLU*up + Q8_1 inside the gate/up launch (True: with both matrices of one type a group owns a whole 32-row
+        # block of both and quantizes it itself; otherwise the last group of each block finishes it) or as a launch of their own
+        # after a two-matrix product (False).  8B shape: 1.917 -> 1.832 ms per token with the block-owning launch; same bits.
+        self.fuse_tail = True
         # decode, one token: the attention norm + Q8_1 inside the Q/K/V launch (every group normalises the row for itself:
         # one launch less per layer, 1.935 -> 1.889 ms per token on the 8B shape; same bits)
         self.fuse_qkv_norm = True
@@ -342,15 +342,15 @@ class LlamaRunner:
                                                vc.stride(0) * 2, vc.stride(1) * 2, D, 0, cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
             self._attn(il, T, n_kv, act=self.act_a)
             self._mm_act([(L["wo"], x)], self.act_a, H * D, T, residual=x)
-            self._norm_quant(x, L["ffn_norm"], self.act_c, T)
             (tg, Wg), (tu, Wu) = L["gate"], L["up"]
+            self._norm_quant(x, L["ffn_norm"], self.act_c, T)
+            nxt = w.layers[il + 1]["attn_norm"] if il + 1 < len(w.layers) else w.output_norm
             if self.fuse_tail:
                 check(lib.mi355_ffn_gate_up_swiglu(_stream(), tg, _ptr(Wg), tu, _ptr(Wu), _ptr(self.act_c), _ptr(self.gate), _ptr(self.up), F,
                                                    _ptr(self.act_b), _ptr(self.tickets), F, E, T))
             else:
                 self._mm_act([(L["gate"], self.gate[:T]), (L["up"], self.up[:T])], self.act_c, E, T)
                 check(lib.mi355_swiglu_quant(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
-            nxt = w.layers[il + 1]["attn_norm"] if il + 1 < len(w.layers) else w.output_norm
             self._mm_act([(L["down"], x)], self.act_b, F, T, residual=x)
             if not qkv_norm or il + 1 == len(w.layers):
                 self._norm_quant(x, nxt, self.act_a, T)

@@ -93,6 +93,41 @@ def test_gate_up_one_launch_llama8b(dev, tg, tu):
                 assert np.array_equal(got, _gemv(dev, t, Wd[i], x))
 
 
+@pytest.mark.parametrize("t", [orc.Q4_K, orc.Q6_K, orc.Q4_0])
+def test_gate_up_swiglu_one_launch_llama8b(dev, t):
+    """ffn_gate + ffn_up + SiLU * up + Q8_1 of an 8B llama layer in one launch (mi355_ffn_gate_up_swiglu; a group owns a 32-row block
+    of both matrices): gate and up hold the bits of the two-matrix product launch, the activation the bits of SiLU * up + Q8_1 as
+    their own launch, and the products match the oracle and the reference CPU backend"""
+    import torch
+    import mi355
+    lib = mi355.load()
+    N, K = 14336, 4096
+    rng = np.random.default_rng(100 + t)
+    Wq = [_weights(rng, t, N, K) for _ in range(2)]
+    Wd = [mi355.upload_weights(t, _t(dev, W)) for W in Wq]
+    tickets = torch.zeros(N // 32 + 1, dtype=torch.int32, device=dev)
+    for B in (1, 2, 4):
+        x = rng.standard_normal((B, K)).astype(np.float32)
+        act = mi355.quantize_act(_t(dev, x))
+        g0, u0 = (torch.full((B, N), float("nan"), dtype=torch.float32, device=dev) for _ in range(2))
+        arr = (mi355.GemvMat * 2)()
+        for i, out in enumerate((g0, u0)):
+            arr[i].type, arr[i].W, arr[i].N, arr[i].dst, arr[i].dst_stride, arr[i].residual = t, Wd[i].data_ptr(), N, out.data_ptr(), N, None
+        mi355.check(lib.mi355_mul_mat_vec_q_multi(None, 2, arr, act.data_ptr(), K, B))
+        a0 = torch.zeros(lib.mi355_act_bytes(N, B), dtype=torch.uint8, device=dev)
+        mi355.check(lib.mi355_swiglu_quant(None, g0.data_ptr(), u0.data_ptr(), N, None, 0, a0.data_ptr(), N, B))
+        g1, u1 = (torch.full((B, N), float("nan"), dtype=torch.float32, device=dev) for _ in range(2))
+        a1 = torch.zeros_like(a0)
+        mi355.check(lib.mi355_ffn_gate_up_swiglu(None, t, Wd[0].data_ptr(), t, Wd[1].data_ptr(), act.data_ptr(), g1.data_ptr(), u1.data_ptr(), N,
+                                                 a1.data_ptr(), tickets.data_ptr(), N, K, B))
+        torch.cuda.synchronize()
+        assert torch.equal(g1, g0) and torch.equal(u1, u0) and torch.equal(a1, a0), B
+        for out, W in ((g1, Wq[0]), (u1, Wq[1])):
+            got = out.cpu().numpy()
+            _check_slices(got, t, W, x)
+            assert orc.nmse(got, orc.mul_mat("ref", t, W, x, n_threads=16)) <= 5e-4
+
+
 @pytest.mark.parametrize("tq,tk,tv", [(orc.Q4_K, orc.Q4_K, orc.Q6_K), (orc.Q4_K, orc.Q4_K, orc.Q4_K), (orc.Q4_0, orc.Q4_0, orc.Q8_0)])
 def test_norm_qkv_rope_store_llama8b(dev, tq, tk, tv):
     """attention norm + Q/K/V + ROPE + cache store of an 8B llama layer (d 4096, 32 / 8 heads of 128) in one launch: bit-identical to

@@ -207,30 +207,34 @@ def test_qkv_rope_store_equals_three_launch_sequence(dev, B, tq, tk, tv):
     assert kc1.abs().sum().item() > 0 and vc1.abs().sum().item() > 0
 
 
-@pytest.mark.parametrize("B", [1, 3])
-def test_tail_fused_launches_equal_separate_kernels(dev, B):
+@pytest.mark.parametrize("B", [1, 2, 3, 4])
+@pytest.mark.parametrize("tg,tu,K,N", [(orc.Q4_K, orc.Q6_K, 2048, 1536),       # two types: groups of 8 rows, the last group of a 32-row block finishes it
+                                       (orc.Q4_K, orc.Q4_K, 2048, 1536),       # one type: a group owns a 32-row block in both matrices
+                                       (orc.Q6_K, orc.Q6_K, 2048, 96), (orc.Q8_0, orc.Q8_0, 1024, 160), (orc.Q4_0, orc.Q4_0, 8192, 64),
+                                       (orc.IQ4_NL, orc.IQ4_NL, 1024, 64), (orc.Q5_K, orc.Q5_K, 768, 32), (orc.Q5_1, orc.Q5_1, 4096, 64),
+                                       (orc.Q4_K, orc.Q4_K, 16384, 32)])       # K beyond what the one-type launch keeps in LDS at 3 and 4 rows
+def test_tail_fused_launches_equal_separate_kernels(dev, B, tg, tu, K, N):
     """gate/up + swiglu + Q8_1 in one launch gives the bytes of the separate launches"""
     import torch
     import mi355
     lib = mi355.load()
     rng = np.random.default_rng(40 + B)
-    K, N = 2048, 1536
     x = rng.standard_normal((B, K)).astype(np.float32)
     act = mi355.quantize_act(_t(dev, x))
-    Wg = mi355.upload_weights(orc.Q4_K, _t(dev, orc.quantize("oracle", orc.Q4_K, (rng.standard_normal((N, K)) * 0.05).astype(np.float32))))
-    Wu = mi355.upload_weights(orc.Q6_K, _t(dev, orc.quantize("oracle", orc.Q6_K, (rng.standard_normal((N, K)) * 0.05).astype(np.float32))))
+    Wg = mi355.upload_weights(tg, _t(dev, orc.quantize("oracle", tg, (rng.standard_normal((N, K)) * 0.05).astype(np.float32))))
+    Wu = mi355.upload_weights(tu, _t(dev, orc.quantize("oracle", tu, (rng.standard_normal((N, K)) * 0.05).astype(np.float32))))
     tickets = torch.zeros(N // 32 + 1, dtype=torch.int32, device=dev)
     for rep in range(2):   # second round: the counters must have been re-armed
         g0 = torch.zeros(B, N, device=dev); u0 = torch.zeros(B, N, device=dev)
         arr = (mi355.GemvMat * 2)()
-        for i, (t, W, out) in enumerate(((orc.Q4_K, Wg, g0), (orc.Q6_K, Wu, u0))):
+        for i, (t, W, out) in enumerate(((tg, Wg, g0), (tu, Wu, u0))):
             arr[i].type, arr[i].W, arr[i].N, arr[i].dst, arr[i].dst_stride, arr[i].residual = t, W.data_ptr(), N, out.data_ptr(), N, None
         mi355.check(lib.mi355_mul_mat_vec_q_multi(None, 2, arr, act.data_ptr(), K, B))
         a0 = torch.zeros(lib.mi355_act_bytes(N, B), dtype=torch.uint8, device=dev)
         mi355.check(lib.mi355_swiglu_quant(None, g0.data_ptr(), u0.data_ptr(), N, None, 0, a0.data_ptr(), N, B))
         g1 = torch.zeros(B, N, device=dev); u1 = torch.zeros(B, N, device=dev)
         a1 = torch.zeros_like(a0)
-        mi355.check(lib.mi355_ffn_gate_up_swiglu(None, orc.Q4_K, Wg.data_ptr(), orc.Q6_K, Wu.data_ptr(), act.data_ptr(), g1.data_ptr(), u1.data_ptr(), N,
+        mi355.check(lib.mi355_ffn_gate_up_swiglu(None, tg, Wg.data_ptr(), tu, Wu.data_ptr(), act.data_ptr(), g1.data_ptr(), u1.data_ptr(), N,
                                                  a1.data_ptr(), tickets.data_ptr(), N, K, B))
         torch.cuda.synchronize()
         assert torch.equal(g1, g0) and torch.equal(u1, u0)
