@@ -134,6 +134,17 @@ size_t mi355_mul_mat_skinny_ws_bytes(int64_t N, int64_t K, int64_t B);
 int mi355_mul_mat_skinny(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N,
                          int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
 
+/* The same product for 33..128 activation rows on Q4_K weights (ggml_compute_forward_mul_mat with ggml_vec_dot_q4_K_q8_K,
+ * ggml-cpu.c:7443-7635, ggml-cpu-quants.c:6817-6848): weights streamed once, packed; the 6-bit sub-block scales folded into two
+ * int8 operand planes so that the matrix cores accumulate whole super-blocks in int32 - the CPU path's own integer sums.
+ * act: tile images of the B activation rows (mi355_quantize_act_q8k_tiled: quantize_row_q8_K_ref levels, scales and sums).
+ * Products with few 32-row tiles run as slices of K when `ws` has mi355_mul_mat_mid_ws_bytes(N, K, B) bytes (may be NULL / 0:
+ * one slice).  dst = W x act (+ residual, which may alias dst). */
+int mi355_mul_mat_mid_supported(int type, const void *W, int64_t K, int64_t B);
+size_t mi355_mul_mat_mid_ws_bytes(int64_t N, int64_t K, int64_t B);
+int mi355_mul_mat_mid(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
+                      int64_t dst_stride, void *ws, size_t ws_bytes);
+
 /* K-quant (Q4_K, Q6_K) tile GEMM with the activation format ggml-cpu uses for these weight
  * types: one f32 scale per 256 elements (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516;
  * vec_dot_type of type_traits_cpu, ggml/src/ggml-cpu/ggml-cpu.c:252-417), so the integer

@@ -1117,8 +1117,17 @@ bool feeds_q8k_tiles(const graph_walk & w, int i, const void * data, int64_t K, 
            mm->src[1]->nb[1] == (size_t) K * sizeof(float);
 }
 
+// 33 to 128 activation rows on Q4_K: the weight-streaming matrix-core kernel on the packed rows (mi355_mul_mat_mid), which takes
+// the activations as tile images
+bool takes_mid_kernel(const ggml_tensor * mm) {
+    const int64_t B = mm->src[1]->ne[1];
+    return mm->src[0]->type == GGML_TYPE_Q4_K && B > 32 && B <= 128 &&
+           mi355_mul_mat_mid_supported(MI355_Q4_K, mm->src[0]->data, mm->src[0]->ne[0], B) && (size_t) ggml_nbytes(mm->src[0]) < ((size_t) 1 << 32);
+}
+
 // activation format of a K-quant tile product: tile images when the batch is large and the weights have (or can get) theirs
 int q8k_format_for(hipStream_t s, const ggml_tensor * mm) {
+    if (takes_mid_kernel(mm)) return ACT_Q8KT;
     return mm->src[1]->ne[1] >= tile_min_batch(mm->src[0]->type) && tiles().get(s, mm->src[0]) != nullptr ? ACT_Q8KT : ACT_Q8K;
 }
 
@@ -1325,7 +1334,7 @@ unsigned tiled_multi(backend_ctx * ctx, hipStream_t s, const graph_walk & w, con
     for (int k = 0; k < n && k < 3; k++) {
         const ggml_tensor * mm = w.nodes[idx[k]];
         if (!is_q8k_tile_candidate(mm) || mm->src[1]->data != b->data || mm->src[1]->ne[0] != K || mm->src[1]->ne[1] != B || mm->src[1]->nb[1] != b->nb[1] ||
-            mm->type != GGML_TYPE_F32 || mm->nb[0] != sizeof(float) || mm->nb[1] % sizeof(float) != 0 || q8k_format_for(s, mm) != ACT_Q8KT)
+            mm->type != GGML_TYPE_F32 || mm->nb[0] != sizeof(float) || mm->nb[1] % sizeof(float) != 0 || takes_mid_kernel(mm) || q8k_format_for(s, mm) != ACT_Q8KT)
             continue;
         tl[k] = tiles().get(s, mm->src[0]);
         if (tl[k])
@@ -1835,21 +1844,23 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         }
         // large batches: the wide-tile kernel on tile images of the weights (built on first use) and of the activation
         const int fmt = q8k_format_for(s, node);
-        const void * tl = fmt == ACT_Q8KT ? tiles().get(s, node->src[0]) : nullptr;
+        const bool mid = takes_mid_kernel(node);
+        const void * tl = fmt == ACT_Q8KT && !mid ? tiles().get(s, node->src[0]) : nullptr;
         if (!ctx->cached(b->data, K, B, fmt)) {
             void * fresh = ctx->act_slot(fmt == ACT_Q8KT ? mi355_act_q8k_tiled_bytes(K, B) : mi355_act_q8k_bytes(K, B));
             if (fmt == ACT_Q8KT) MI355_K_OK(mi355_quantize_act_q8k_tiled(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
             else MI355_K_OK(mi355_quantize_act_q8k(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
             ctx->cache = act_cache{b->data, K, B, fmt, true, fresh};
         }
-        const void * pl = tl ? nullptr : planes().get(s, node->src[0]);   // Q6_K weights: the unpacked planes, built on first use
+        const void * pl = tl || mid ? nullptr : planes().get(s, node->src[0]);   // Q6_K weights: the unpacked planes, built on first use
         const int wtype = to_mi355_type(node->src[0]->type);
         const int64_t N = node->src[0]->ne[1];
         // products with few tiles are split along K through the scratch buffer (0 bytes: this shape is not split)
-        const size_t split_bytes = tl ? mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) : mi355_mul_mat_q8k_ws_bytes(N, K, B);
+        const size_t split_bytes = mid ? mi355_mul_mat_mid_ws_bytes(N, K, B) : tl ? mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) : mi355_mul_mat_q8k_ws_bytes(N, K, B);
         void * split_ws = split_bytes ? ctx->workspace(split_bytes) : nullptr;
         auto product = [&](float * out, const float * residual, int64_t out_stride) {
-            if (tl) MI355_K_OK(mi355_mul_mat_q8k_tiled(s, wtype, tl, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
+            if (mid) MI355_K_OK(mi355_mul_mat_mid(s, wtype, node->src[0]->data, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
+            else if (tl) MI355_K_OK(mi355_mul_mat_q8k_tiled(s, wtype, tl, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
             else if (pl) MI355_K_OK(mi355_mul_mat_q8k_planes_ws(s, wtype, pl, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
             else MI355_K_OK(mi355_mul_mat_q8k_ws(s, wtype, node->src[0]->data, ctx->cache.ptr, out, residual, N, K, B, out_stride, split_ws, split_bytes));
         };

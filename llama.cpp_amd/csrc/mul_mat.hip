@@ -74,15 +74,25 @@ using namespace mi355;
 extern "C" {
 
 // the per-super-block activation format of the K-quant tile kernel is smaller than the Q8_1 one
-size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B) { return (mi355_act_bytes(K, B) + 255) & ~(size_t)255; }
+size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B) {
+    size_t n = mi355_act_bytes(K, B);
+    if (B > 32 && B <= 128 && K % 256 == 0) {   // the weight-streaming kernel for 33..128 rows takes tile images of the activations
+        const size_t t = mi355_act_q8k_tiled_bytes(K, B);
+        n = t > n ? t : n;
+    }
+    return (n + 255) & ~(size_t)255;
+}
 
 // 4 or 5 (Q6_K) to 32 activation rows: the weight-streaming matrix-core kernel (skinny.hip) where it supports the product.
 static bool use_skinny(int type, const void *W, int64_t K, int64_t B) {
     return B >= (type == MI355_Q6_K ? 5 : 4) && B <= 32 && mi355_mul_mat_skinny_supported(type, W, K, B);
 }
 
+// 33 to 128 activation rows on Q4_K: the weight-streaming matrix-core kernel with the sub-block scales folded into the operand (mid.hip)
+static bool use_mid(int type, const void *W, int64_t K, int64_t B) { return B > 32 && B <= 128 && mi355_mul_mat_mid_supported(type, W, K, B); }
+
 static bool use_q8k_tiles(int type, const void *W, int64_t K, int64_t B) {
-    return B > 8 && !use_skinny(type, W, K, B) && (type == MI355_Q4_K || type == MI355_Q6_K) && layout_aligned(W, make_row_layout(type, K));
+    return B > 8 && !use_skinny(type, W, K, B) && !use_mid(type, W, K, B) && (type == MI355_Q4_K || type == MI355_Q6_K) && layout_aligned(W, make_row_layout(type, K));
 }
 
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
@@ -94,6 +104,12 @@ int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *
     if (ws_bytes < mi355_mul_mat_ws_bytes(K, B) || ws == nullptr) {
         set_error("mul_mat: workspace of %zu bytes, need %zu", ws_bytes, mi355_mul_mat_ws_bytes(K, B));
         return MI355_ERR_WORKSPACE;
+    }
+    if (use_mid(type, W, K, B)) {
+        int rc = mi355_quantize_act_q8k_tiled(stream, x, ws, K, B, x_stride);
+        if (rc != MI355_OK) return rc;
+        const size_t used = mi355_mul_mat_ws_bytes(K, B);
+        return mi355_mul_mat_mid(stream, type, W, ws, dst, nullptr, N, K, B, dst_stride, (char *)ws + used, ws_bytes - used);
     }
     if (use_q8k_tiles(type, W, K, B)) {
         int rc = mi355_quantize_act_q8k(stream, x, ws, K, B, x_stride);

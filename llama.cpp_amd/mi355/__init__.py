@@ -56,6 +56,9 @@ _SIGNATURES = {
     "mi355_mul_mat_skinny_supported": (_int, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_skinny_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_skinny": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_mid_supported": (_int, [_int, _p, _i64, _i64]),
+    "mi355_mul_mat_mid_ws_bytes": (_sz, [_i64, _i64, _i64]),
+    "mi355_mul_mat_mid": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_act_q8k_bytes": (_sz, [_i64, _i64]),
     "mi355_quantize_act_q8k": (_int, [_p, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_q8k": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
@@ -294,7 +297,8 @@ def mul_mat(t, W, x, ws=None, split=True):
     N = W.shape[0]
     need = load().mi355_mul_mat_ws_bytes(K, B)
     if split:
-        need += max(load().mi355_mul_mat_q_ws_bytes(N, K, B), load().mi355_mul_mat_q8k_ws_bytes(N, K, B), load().mi355_mul_mat_skinny_ws_bytes(N, K, B))
+        need += max(load().mi355_mul_mat_q_ws_bytes(N, K, B), load().mi355_mul_mat_q8k_ws_bytes(N, K, B), load().mi355_mul_mat_skinny_ws_bytes(N, K, B),
+                    load().mi355_mul_mat_mid_ws_bytes(N, K, B))
     if ws is None or ws.numel() < need:
         ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     dst = torch.empty((B, N), dtype=torch.float32, device=x.device)
@@ -322,6 +326,21 @@ def mul_mat_skinny(t, W, x, residual=None, split=True):
     dst = torch.empty((B, N), dtype=torch.float32, device=x.device)
     check(load().mi355_mul_mat_skinny(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), _ptr(residual) if residual is not None else None,
                                       N, K, B, N, _ptr(ws) if nws else None, nws))
+    return dst
+
+
+def mul_mat_mid(t, W, x, residual=None, split=True):
+    """The weight-streaming matrix-core product for 33..128 activation rows (Q4_K): W device layout [N, row_bytes], x f32 [B, K]
+    -> f32 [B, N] (+ residual [B, N]).  split: give it the workspace that lets few rows run as slices along K"""
+    import torch
+    B, K = x.shape
+    N = W.shape[0]
+    act = quantize_act_q8k_tiled(x)
+    nws = load().mi355_mul_mat_mid_ws_bytes(N, K, B) if split else 0
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=x.device)
+    dst = torch.empty((B, N), dtype=torch.float32, device=x.device)
+    check(load().mi355_mul_mat_mid(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), _ptr(residual) if residual is not None else None,
+                                   N, K, B, N, _ptr(ws) if nws else None, nws))
     return dst
 
 

@@ -213,18 +213,22 @@ class LlamaRunner:
         return self.tiles[key]
 
     def _fmt(self, mats, K, T):
-        """activation format of a product: 0 Q8_1 blocks, 1 one scale per 256 elements (K-quant tile GEMM), 2 the same as tile images"""
+        """activation format of a product: 0 Q8_1 blocks, 1 one scale per 256 elements (K-quant tile GEMM), 2 the same as tile images,
+        3 tile images for the 33..128-row kernel on packed Q4_K rows"""
         if T <= 8 or not self._q8k_ok(mats, K):
             return 0
+        if 32 < T <= 128 and all(t == Q4_K for (t, _), _ in mats):
+            return 3     # the weight-streaming kernel for 33..128 rows: activations as tile images, weights packed
         return 2 if (self.use_tiles and T >= 192) else 1
 
     def _quant(self, src, act, K, T, q8k):
-        fn = (self.lib.mi355_quantize_act, self.lib.mi355_quantize_act_q8k, self.lib.mi355_quantize_act_q8k_tiled)[int(q8k)]
+        fn = (self.lib.mi355_quantize_act, self.lib.mi355_quantize_act_q8k, self.lib.mi355_quantize_act_q8k_tiled, self.lib.mi355_quantize_act_q8k_tiled)[int(q8k)]
         check(fn(_stream(), _ptr(src), _ptr(act), K, T, src.stride(0)))
 
     def _norm_quant(self, x, w, act, T, q8k=0):
         K = x.shape[1]
-        fn = (self.lib.mi355_rms_norm_mul_quant, self.lib.mi355_rms_norm_mul_quant_q8k, self.lib.mi355_rms_norm_mul_quant_q8k_tiled)[int(q8k)]
+        fn = (self.lib.mi355_rms_norm_mul_quant, self.lib.mi355_rms_norm_mul_quant_q8k, self.lib.mi355_rms_norm_mul_quant_q8k_tiled,
+              self.lib.mi355_rms_norm_mul_quant_q8k_tiled)[int(q8k)]
         check(fn(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
 
     def _mm_act(self, mats, act, K, T, residual=None, q8k=False):
@@ -250,6 +254,14 @@ class LlamaRunner:
                     check(self.lib.mi355_mul_mat_q8k_tiled_multi(_stream(), t, len(same), arr, _ptr(act), K, T, None, 0))
                 mats = rest
             for (t, W), out in mats:
+                if q8k == 3:
+                    N = out.shape[1]
+                    need = int(self.lib.mi355_mul_mat_mid_ws_bytes(N, K, T))
+                    if self.split_ws is None or self.split_ws.numel() < need:
+                        self.split_ws = torch.empty(need + 256, dtype=torch.uint8, device=self.dev)
+                    check(self.lib.mi355_mul_mat_mid(_stream(), t, _ptr(W), _ptr(act), _ptr(out), _ptr(residual) if residual is not None else None, N, K, T,
+                                                     out.stride(0), _ptr(self.split_ws) if need else None, need))
+                    continue
                 if q8k:     # the residual add is the tile kernel's epilogue; products with few tiles are split along K through split_ws
                     N = out.shape[1]
                     need = int(self.lib.mi355_mul_mat_q8k_tiled_ws_bytes(N, K, T) if q8k == 2 else self.lib.mi355_mul_mat_q8k_ws_bytes(N, K, T))
@@ -307,7 +319,7 @@ class LlamaRunner:
             self._mm_act(gu, self.act_a, E, T, q8k=kq)
             down = [(L["down"], x)]
             kq = self._fmt(down, F, T)
-            fn = (lib.mi355_swiglu_quant, lib.mi355_swiglu_quant_q8k, lib.mi355_swiglu_quant_q8k_tiled)[kq]
+            fn = (lib.mi355_swiglu_quant, lib.mi355_swiglu_quant_q8k, lib.mi355_swiglu_quant_q8k_tiled, lib.mi355_swiglu_quant_q8k_tiled)[kq]
             check(fn(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
             self._mm_act(down, self.act_b, F, T, residual=x, q8k=kq)
         To = 1 if last_only else T

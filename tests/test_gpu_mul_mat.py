@@ -193,6 +193,32 @@ def test_skinny_matches_oracle(dev, name, t, N, K, B, split):
         assert orc.nmse(got, orc.mul_mat("ref", t, Wq, x)) <= 5e-4      # tests/test-backend-ops.cpp:1916
 
 
+@pytest.mark.parametrize("N,K,B", [(100, 256, 33), (257, 1024, 64), (4096, 4096, 50), (1024, 14336, 100), (64, 3584, 128), (333, 2048, 96), (77, 6144, 65),
+                                   (130, 512, 20), (4096, 4096, 128), (512, 4096, 40)])
+@pytest.mark.parametrize("split", [False, True])
+def test_mid_matches_oracle(dev, N, K, B, split):
+    """the weight-streaming matrix-core kernel for 33..128 activation rows on Q4_K (sub-block scales folded into two int8 operand
+    planes): the CPU path's integer sums (ggml-cpu-quants.c:6817-6848) - ragged row and batch counts, both activation halves, K that
+    does not divide evenly over the four waves, with and without slices along K, with a residual"""
+    import mi355
+    t = orc.Q4_K
+    rng = np.random.default_rng(N * 5 + K + B)
+    Wq = _weights(rng, t, N, K, "ref")
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    res = rng.standard_normal((B, N)).astype(np.float32)
+    Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
+    got = mi355.mul_mat_mid(t, Wd, _to_dev(dev, x), split=split).cpu().numpy()
+    got_res = mi355.mul_mat_mid(t, Wd, _to_dev(dev, x), residual=_to_dev(dev, res), split=split).cpu().numpy()
+    assert np.array_equal(got_res, got + res)
+    Nt = min(N, 48)
+    assert orc.nmse(got[:, :Nt], orc.mul_mat("cpu", t, Wq[:Nt], x)) < 1e-9          # every activation row, the first weight rows
+    assert orc.nmse(got[B - 9:, N - 40:], orc.mul_mat("cpu", t, Wq[N - 40:], x[B - 9:])) < 1e-9
+    if orc.ref is not None:
+        assert orc.nmse(got, orc.mul_mat("ref", t, Wq, x)) <= 5e-4      # tests/test-backend-ops.cpp:1916
+    if B > 32:   # mi355_mul_mat takes this kernel for 33..128 rows
+        assert np.array_equal(mi355.mul_mat(t, Wd, _to_dev(dev, x), split=split).cpu().numpy(), got)
+
+
 @pytest.mark.parametrize("name,t", TYPES)
 @pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
 def test_mmq_llama8b_ffn_shapes(dev, name, t, N, K):
