@@ -314,6 +314,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--random-blocks", action="store_true", help="fill the weights with random blocks instead of quantizing N(0, 0.02) values on the device")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
     ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, mmq_wide (the wide-tile GEMM on 14336 x 4096 at batch 512 only), fattn, "
                                           "fattn_long (decode over 131072 cells only), fattn_prefill (4096 x 4096 prefill only), fattn_prefill_512 (512 rows over 4096 cells only)")
@@ -344,7 +345,10 @@ def main():
     cfg = lg.LlamaConfig()
     n_ctx = max(512, (args.warmup + args.steps + 255) // 256 * 256, args.pp)
     cfg.n_ctx = n_ctx
-    weights = lg.LlamaWeights(cfg, dev)
+    tq = time.perf_counter()
+    weights = lg.LlamaWeights(cfg, dev, quantize=not args.random_blocks)     # N(0, 0.02) weights quantized on the device (Q4_K_M mix)
+    torch.cuda.synchronize()
+    quantize_s = time.perf_counter() - tq
     run = lg.LlamaRunner(weights, max_tokens=max(args.pp, 8))
     emb = torch.randn(max(args.pp, 8), cfg.n_embd).pin_memory()
     logits_host = torch.empty(cfg.n_vocab, dtype=torch.float32).pin_memory()
@@ -490,7 +494,9 @@ def main():
         "value": round(tg, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 block dots (Q4_K/Q6_K weights x Q8_1 activations), f32 accumulate, f16 KV cache",
-        "data": "synthetic: random Q4_K/Q6_K blocks scaled like N(0,0.02) weights, random embeddings",
+        "data": ("synthetic: random Q4_K/Q6_K blocks scaled like N(0,0.02) weights, random embeddings" if args.random_blocks else
+                 "synthetic: weights drawn from N(0,0.02) and quantized on the device to the Q4_K_M mix with the reference quantizers' arithmetic "
+                 "(%.1f s for the 8B model), random embeddings" % quantize_s),
         "config": {"workload": "configs[3]: Llama-3-8B-shaped Q4_K_M decode (32 layers, d_model 4096, ffn 14336, 32/8 heads, "
                                "head_dim 128, vocab 128256), KV positions %d..%d, n_kv padded to 256" % (args.warmup, args.warmup + args.steps - 1),
                    "launch": "host" if args.no_graph else "hip-graph replay", "weight_bytes_per_token": weight_bytes,

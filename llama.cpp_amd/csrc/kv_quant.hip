@@ -88,7 +88,10 @@ __global__ void __launch_bounds__(256) k_cpy_f32_q4_0(const float *__restrict__ 
             imax = oi;
         }
     }
-    const float d = vmax / -8.0f;
+    // d = vmax / -8, exact as an eighth with the sign flipped; the stored half takes its sign flip in the half's bits, so that a
+    // zero block keeps the reference's -0.0 (a product converted to half may be fused with a +0.0 addend, which loses that sign)
+    const float eighth = vmax * 0.125f;
+    const float d = -eighth;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     unsigned packed = 0;
 #pragma unroll
@@ -106,7 +109,7 @@ __global__ void __launch_bounds__(256) k_cpy_f32_q4_0(const float *__restrict__ 
     unsigned short *o = (unsigned short *)(y + lv + 4 * lane8);
     o[0] = (unsigned short)(bytes & 0xFFFFu);
     o[1] = (unsigned short)(bytes >> 16);
-    if (lane8 == 0) *(unsigned short *)(y + sc) = float_to_half_bits(d);
+    if (lane8 == 0) *(unsigned short *)(y + sc) = (unsigned short)(float_to_half_bits(eighth) ^ 0x8000u);
 }
 
 // dst f16 [cell][head][D] = dequantized rows of a typed cache whose (cell, head) row starts at block cell * cb + head * hb (+ the

@@ -39,6 +39,8 @@ _SIGNATURES = {
     "mi355_last_error": (C.c_char_p, []),
     "mi355_launch_count": (C.c_uint64, []),
     "mi355_device_supported": (_int, [_int]),
+    "mi355_quantize_weights_supported": (_int, [_int]),
+    "mi355_quantize_weights": (_int, [_p, _int, _p, _p, _i64, _i64]),
     "mi355_weights_scatter": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
     "mi355_weights_gather": (_int, [_p, _int, _p, _p, _i64, _i64, _sz, _sz]),
     "mi355_quantize_q8_1": (_int, [_p, _p, _p, _i64, _i64, _i64]),
@@ -212,6 +214,16 @@ def download_weights(t, dev):
     out = torch.empty_like(dev)
     check(load().mi355_weights_gather(_stream(), t, _ptr(dev), _ptr(out), k, nrows, 0, dev.numel()))
     return out
+
+
+def quantize_weights(t, x):
+    """x: f32 CUDA tensor [nrows, k] -> uint8 [nrows, row_bytes] in the reference block layout (the reference quantizer's bytes)"""
+    import torch
+    x = x.contiguous()
+    nrows, k = x.shape
+    y = torch.empty((nrows, row_bytes(t, k)), dtype=torch.uint8, device=x.device)
+    check(load().mi355_quantize_weights(_stream(), t, _ptr(x), _ptr(y), k, nrows))
+    return y
 
 
 def quantize_q8_1(x):

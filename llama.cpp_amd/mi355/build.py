@@ -20,7 +20,7 @@ BACKEND_SRC = os.path.join(PKG, "backend")
 LIB = os.path.join(PKG, "lib")
 OBJ = os.path.join(LIB, "obj")
 
-KERNEL_SOURCES = ["quantize.hip", "gemv.hip", "ffn.hip", "mul_mat.hip", "skinny.hip", "mid.hip", "mmq.hip", "mmq_k.hip", "mmq_w.hip", "mul_mat_id.hip", "fattn.hip", "fattn_mma.hip", "fattn_stream.hip", "kv_quant.hip", "glue.hip", "fused.hip", "moe.hip"]
+KERNEL_SOURCES = ["quantize.hip", "wquant.hip", "gemv.hip", "ffn.hip", "mul_mat.hip", "skinny.hip", "mid.hip", "mmq.hip", "mmq_k.hip", "mmq_w.hip", "mul_mat_id.hip", "fattn.hip", "fattn_mma.hip", "fattn_stream.hip", "kv_quant.hip", "glue.hip", "fused.hip", "moe.hip"]
 
 # -packed-fp32-ops: keep hipcc from forming packed-FP32 instructions out of scalar float code
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",

@@ -66,14 +66,22 @@ def random_quantized(t, nrows, k, device, gen):
 class LlamaWeights:
     """device-layout weights of a Q4_K_M (or single-type) llama"""
 
-    def __init__(self, cfg, device, seed=1234, ftype="q4_k_m"):
+    def __init__(self, cfg, device, seed=1234, ftype="q4_k_m", quantize=False):
+        """quantize: draw every matrix from N(0, 0.02) in f32 and quantize it on the device with the reference quantizers'
+        arithmetic (mi355_quantize_weights) instead of drawing random blocks"""
         gen = torch.Generator(device=device)
         gen.manual_seed(seed)
         self.cfg = cfg
         E, F, H, HK, D = cfg.n_embd, cfg.n_ff, cfg.n_head, cfg.n_head_kv, cfg.head_dim
         base = {"q4_k_m": Q4_K, "q4_0": Q4_0, "q8_0": Q8_0, "q4_k": Q4_K, "q6_k": Q6_K}[ftype]
+        self.quantized = bool(quantize)
 
         def mk(t, n, k):
+            if quantize:
+                from . import quantize_weights
+                step = max(1, (1 << 28) // (4 * k))      # 256 MiB of f32 at a time
+                parts = [quantize_weights(t, torch.randn((min(step, n - r0), k), device=device, generator=gen) * 0.02) for r0 in range(0, n, step)]
+                return t, upload_weights(t, torch.cat(parts) if len(parts) > 1 else parts[0])
             return t, upload_weights(t, random_quantized(t, n, k, device, gen))
 
         self.layers = []
