@@ -306,6 +306,40 @@ def sweep(kinds):
                      achieved=round(fl / us / 1e6, 1), unit="TFLOP/s", frac=round(fl / us / 1e6 / F16_PEAK_TFLOPS, 4), flops=fl)
             del ks, vs
 
+    if "fattn" in kinds or "fattn_kv" in kinds:
+        # decode over a quantized cache kept as llama.cpp's cache tensors are in a plug-in buffer ([cells][Hkv * D] rows in the device row
+        # layout), filled through the quantizing store; the blocks are read where they lie
+        H, HK, D = 32, 8, 128
+        for tname, t, bb in (("Q8_0", mi355.Q8_0, 34), ("Q4_0", mi355.Q4_0, 18)):
+            for Nkv in (256, 1024, 4096, 32768, 131072):
+                nrot = max(2, min(16, (1 << 29) // (Nkv * HK * D)))
+                rb = HK * D // 32
+                row_bytes = rb * bb
+                q = torch.randn(1, H, D, device=dev, generator=gen)
+                caches = []
+                for _ in range(2 * nrot):
+                    c = torch.empty(Nkv * row_bytes, dtype=torch.uint8, device=dev)
+                    src = torch.randn(Nkv, HK * D, device=dev, generator=gen)
+                    mi355.check(lib.mi355_cpy_f32_quant(stream.cuda_stream, t, src.data_ptr(), c.data_ptr(), 0, rb, Nkv * HK * D))
+                    caches.append(c)
+                torch.cuda.synchronize()
+                mask = torch.zeros((64, Nkv), dtype=torch.float16, device=dev)
+                dst = torch.empty(1, H, D, device=dev)
+                need = int(lib.mi355_flash_attn_ws_bytes(D, 1, Nkv, H))
+                ws = torch.empty(min(need, 1 << 28) + 256, dtype=torch.uint8, device=dev)
+                wp = (ws.data_ptr() + 255) & ~255
+
+                def fa(i):
+                    kc, vc = caches[2 * i], caches[2 * i + 1]
+                    mi355.check(lib.mi355_flash_attn_ext_kv(stream.cuda_stream, q.data_ptr(), kc.data_ptr(), t, kc.data_ptr(), rb, vc.data_ptr(), t, vc.data_ptr(), rb,
+                                                            mask.data_ptr(), dst.data_ptr(), D, 1, Nkv, H, HK, H * D * 4, D * 4, row_bytes, D // 32 * bb, row_bytes,
+                                                            D // 32 * bb, Nkv * 2, 1 / math.sqrt(D), 0.0, 0.0, wp, ws.numel() - 256, None))
+                us = timed(fa, nrot, 4)
+                alg = 2 * Nkv * row_bytes + 2 * Nkv + 4 * H * D * 2
+                emit(kernel="FLASH_ATTN_EXT decode over a %s cache read in place (all launches of one call)" % tname, case="Nkv %d" % Nkv, us=round(us, 2), bound="hbm",
+                     achieved=round(alg / us / 1e3, 1), unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg, cache_bytes=2 * Nkv * row_bytes)
+                del caches
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -317,7 +351,7 @@ def main():
     ap.add_argument("--random-blocks", action="store_true", help="fill the weights with random blocks instead of quantizing N(0, 0.02) values on the device")
     ap.add_argument("--pp", type=int, default=512, help="prompt length of the prefill measurement (0 = skip)")
     ap.add_argument("--sweep", default="", help="comma-separated kernel tables instead of the model run: gemv, mmq, mmq_wide (the wide-tile GEMM on 14336 x 4096 at batch 512 only), fattn, "
-                                          "fattn_long (decode over 131072 cells only), fattn_prefill (4096 x 4096 prefill only), fattn_prefill_512 (512 rows over 4096 cells only)")
+                                          "fattn_long (decode over 131072 cells only), fattn_prefill (4096 x 4096 prefill only), fattn_prefill_512 (512 rows over 4096 cells only), fattn_kv (decode over Q8_0 / Q4_0 caches only)")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="rewrite the tracked HBM-traffic summary from two rocprofv3 --pmc output directories (no GPU needed)")
     args = ap.parse_args()

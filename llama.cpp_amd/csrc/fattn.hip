@@ -1,4 +1,4 @@
-// FLASH_ATTN_EXT over an f16 KV cache with grouped-query heads.
+// FLASH_ATTN_EXT with grouped-query heads over an f16 KV cache; the vector kernel also reads Q8_0 / Q4_0 caches where they lie.
 //
 // k_fattn_vec: the HBM-bound form (decode, and any query count as a fallback).  A group
 // works on one (kv head, query token, kv split).  A K or V row of D halves is read by
@@ -44,6 +44,66 @@ __device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
 }
 
 
+
+// Where this lane's eight elements d0 .. d0 + 7 of the (cell 0, kv head hk) row of a quantized operand lie: their levels (Q4_0: the
+// eight bytes whose low or high nibbles - shift 0 or 4 - they are) and the block's f16 scale; a cell further on is nb1 bytes
+// further on in both.
+struct kv_lane {
+    const uint8_t *lv, *sc;
+    int shift;
+};
+__device__ __forceinline__ kv_lane kv_lane_of(const kv_src &s, int type, int64_t hk, int d0) {
+    const int BB = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES, LB = type == MI355_Q8_0 ? 32 : 16;
+    const int64_t g = s.first_block + hk * s.head_blocks + (d0 >> 5);
+    const int j = d0 & 31;
+    kv_lane o;
+    const uint8_t *lv;
+    if (s.row_blocks == 0) {
+        o.sc = s.base + g * BB;
+        lv = o.sc + 2;
+    } else {
+        const int64_t row = g / s.row_blocks, b = g % s.row_blocks;
+        const uint8_t *rb = s.base + row * s.row_blocks * BB;
+        lv = rb + b * LB;
+        o.sc = rb + s.row_blocks * LB + b * 2;
+    }
+    o.lv = lv + (type == MI355_Q8_0 ? j : (j & 15));
+    o.shift = (type == MI355_Q4_0 && j >= 16) ? 4 : 0;
+    return o;
+}
+// the raw bytes of one cell's eight elements: levels in words 0 and 1, the scale's bits in word 2 (plain blocks are 2-byte aligned)
+__device__ __forceinline__ u32x4 kv_load8(const kv_lane &p, int64_t off) {
+    u32x2 w;
+    __builtin_memcpy(&w, p.lv + off, 8);
+    return u32x4{w[0], w[1], (u32)*(const unsigned short *)(p.sc + off), 0u};
+}
+// d * level of the eight elements (dequantize_row_q8_0 / dequantize_row_q4_0, ggml-quants.c:255-273, 365-380)
+__device__ __forceinline__ void kv_values8(int type, const u32x4 &raw, int shift, float (&f)[8]) {
+    const float d = half_bits_to_float((unsigned short)raw[2]);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const u32 w = raw[i >> 2] >> (8 * (i & 3));
+        f[i] = type == MI355_Q8_0 ? (float)(int8_t)(w & 0xFF) * d : (float)((int)((w >> shift) & 0xF) - 8) * d;
+    }
+}
+// The eight levels as f16 pairs, exact: byte u in the low byte of a half whose high byte is 0x64 reads 1024 + u, and one packed
+// subtraction brings it to the level (Q8_0: u = level + 128 after the sign bit is flipped; Q4_0: u = nibble, level = u - 8).
+// Returns the block's scale; the dot of these levels with q is multiplied by it afterwards.
+__device__ __forceinline__ float kv_levels8_f16(int type, const u32x4 &raw, int shift, u32x4 &out) {
+    const bool q8 = type == MI355_Q8_0;
+    const f16x2 bias = q8 ? f16x2{(_Float16)-1152.0f, (_Float16)-1152.0f} : f16x2{(_Float16)-1032.0f, (_Float16)-1032.0f};
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const u32 w = q8 ? raw[h] ^ 0x80808080u : (raw[h] >> shift) & 0x0F0F0F0Fu;
+        // v_perm_b32 picks bytes of {0x64646464, w}: selector bytes 0..3 = w's bytes, 4..7 = the constant's
+        const u32 lo = __builtin_amdgcn_perm(0x64646464u, w, 0x04010400u);   // halves (0x64, byte 0), (0x64, byte 1)
+        const u32 hi = __builtin_amdgcn_perm(0x64646464u, w, 0x04030402u);   // halves (0x64, byte 2), (0x64, byte 3)
+        const f16x2 a = __builtin_bit_cast(f16x2, lo) + bias, b = __builtin_bit_cast(f16x2, hi) + bias;
+        out[2 * h] = __builtin_bit_cast(u32, a);
+        out[2 * h + 1] = __builtin_bit_cast(u32, b);
+    }
+    return half_bits_to_float((unsigned short)raw[2]);
+}
 
 // NW: waves per group
 template <int D, int R, int NW = 4>
@@ -105,6 +165,11 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     const int64_t c_end = c_begin + a.cells_per_split < a.Nkv ? c_begin + a.cells_per_split : a.Nkv;
     const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
     const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
+    // quantized operands (wave-uniform choice): this lane's place in the rows of kv head hk
+    const bool k_f16 = a.type_k == MI355_F16, v_f16 = a.type_v == MI355_F16;
+    kv_lane kl = {nullptr, nullptr, 0}, vl = {nullptr, nullptr, 0};
+    if (!k_f16 && active) kl = kv_lane_of(a.kq, a.type_k, hk, d0);
+    if (!v_f16 && active) vl = kv_lane_of(a.vq, a.type_v, hk, d0);
 
     // U steps of SLOTS cells at a time: all mask entries, then all K/V rows of the U steps are requested before the first
     // is used, so a short context costs one round trip to memory instead of one per step.  Cells are still folded into a
@@ -128,29 +193,43 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
             kk[j] = u32x4{0, 0, 0, 0};
             vv[j] = u32x4{0, 0, 0, 0};
             if (valid[j] && active) {   // masked cells cost no K/V traffic
-                kk[j] = load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2);
-                vv[j] = load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2);
+                kk[j] = k_f16 ? load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2) : kv_load8(kl, c * (int64_t)a.k_nb1);
+                vv[j] = v_f16 ? load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2) : kv_load8(vl, c * (int64_t)a.v_nb1);
+            }
+        }
+        float kd[U];   // quantized K: the levels as exact f16 values; their dot with q takes the block's scale afterwards
+#pragma unroll
+        for (int j = 0; j < U; j++) {
+            kd[j] = 1.0f;
+            if (!k_f16) {
+                const u32x4 raw = kk[j];
+                kd[j] = kv_levels8_f16(a.type_k, raw, kl.shift, kk[j]);
             }
         }
         // V rows as floats, then per head: the U scores (independent of each other), ONE new maximum and ONE rescale of the state,
         // and the U weighted rows - the dependent chain per step is a fraction of folding the cells one by one
         float vf[U][8];
 #pragma unroll
-        for (int j = 0; j < U; j++)
+        for (int j = 0; j < U; j++) {
+            if (v_f16) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const u32 vi = vv[j][i];
-                const f16x2 h2 = __builtin_bit_cast(f16x2, vi);
-                vf[j][2 * i] = (float)h2[0];
-                vf[j][2 * i + 1] = (float)h2[1];
+                for (int i = 0; i < 4; i++) {
+                    const u32 vi = vv[j][i];
+                    const f16x2 h2 = __builtin_bit_cast(f16x2, vi);
+                    vf[j][2 * i] = (float)h2[0];
+                    vf[j][2 * i + 1] = (float)h2[1];
+                }
+            } else {
+                kv_values8(a.type_v, vv[j], vl.shift, vf[j]);
             }
+        }
 #pragma unroll
         for (int r = 0; r < R; r++) {
             float sj[U];
             float mn = m[r];
 #pragma unroll
             for (int j = 0; j < U; j++) {
-                float sc = group_sum<LPR>(dot8_f16(qh[r], kk[j])) * scale;
+                float sc = group_sum<LPR>(k_f16 ? dot8_f16(qh[r], kk[j]) : dot8_f16(qh[r], kk[j]) * kd[j]) * scale;
                 if (a.softcap != 0.0f) sc = a.softcap * tanhf(sc);
                 sc += slope[r] * mv[j];
                 sj[j] = valid[j] ? sc : NEG;
@@ -327,7 +406,9 @@ static int launch_vec_r(hipStream_t s, fattn_args &a, int R) {
     // the 8B model at 256 cells: 4 waves 1.897 ms, 8 waves 1.856 ms, 16 waves 1.875 ms; requesting K and V together with the mask
     // instead of after it (one round trip less per step, but masked cells then cost their bytes) 1.91-1.96 ms.
     constexpr int64_t one_head_max = 1024;
-    if (a.Nkv <= one_head_max) {
+    // (quantized operands cost more arithmetic per cell: from 257 cells on their cells are split over groups)
+    const bool quantized = a.type_k != MI355_F16 || a.type_v != MI355_F16;
+    if (a.Nkv <= one_head_max && !(quantized && a.Nkv > 256 && a.n_splits > 1)) {
         if (a.Nq * a.Hq <= 512) {   // few (token, head) pairs: the chip is far from full
             a.n_splits = 1;
             a.cells_per_split = a.Nkv;
@@ -340,31 +421,18 @@ static int launch_vec_r(hipStream_t s, fattn_args &a, int R) {
     return launch_vec<D, 1>(s, a);
 }
 
-}  // namespace mi355
-
-using namespace mi355;
-
-extern "C" {
-
-size_t mi355_flash_attn_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq) {
-    // worst case: 256 kv splits
-    (void)Nkv;
-    return (size_t)Nq * (size_t)Hq * 256 * (size_t)(D + 2) * sizeof(float);
-}
-
-int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
-                               int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
-                               size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
-                               float max_bias, float logit_softcap, void *ws, size_t ws_bytes, void *act) {
+// checks shared by the entry points and the argument block of the kernels; quantized operands skip the f16 row checks
+static int fattn_fill(fattn_args &a, const float *q, const void *k, const void *v, const void *mask, float *dst, int64_t D, int64_t Nq, int64_t Nkv,
+                      int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1,
+                      float scale, float max_bias, float logit_softcap, void *ws, size_t ws_bytes, void *act, bool k_f16, bool v_f16) {
     MI355_REQUIRE(D > 0 && D % 8 == 0 && D <= 256, "flash_attn: head size %lld not supported", (long long)D);
     MI355_REQUIRE(Nq > 0 && Nkv > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "flash_attn: bad shape");
     MI355_REQUIRE(Nq <= 65535 && Hq <= 65535, "flash_attn: too many query rows or heads for one launch");
     MI355_REQUIRE(((uintptr_t)q & 15) == 0 && q_nb1 % 16 == 0 && q_nb2 % 16 == 0, "flash_attn: q rows must be 16-byte aligned");
-    MI355_REQUIRE(((uintptr_t)k & 15) == 0 && k_nb1 % 16 == 0 && k_nb2 % 16 == 0, "flash_attn: k rows must be 16-byte aligned");
-    MI355_REQUIRE(((uintptr_t)v & 15) == 0 && v_nb1 % 16 == 0 && v_nb2 % 16 == 0, "flash_attn: v rows must be 16-byte aligned");
+    MI355_REQUIRE(!k_f16 || (((uintptr_t)k & 15) == 0 && k_nb1 % 16 == 0 && k_nb2 % 16 == 0), "flash_attn: k rows must be 16-byte aligned");
+    MI355_REQUIRE(!v_f16 || (((uintptr_t)v & 15) == 0 && v_nb1 % 16 == 0 && v_nb2 % 16 == 0), "flash_attn: v rows must be 16-byte aligned");
     MI355_REQUIRE(max_bias <= 0.0f || mask != nullptr, "flash_attn: max_bias needs a mask");
     MI355_REQUIRE(act == nullptr || (D % 32 == 0 && ((uintptr_t)act & 15) == 0), "flash_attn: quantized output needs head size %% 32 == 0 and a 16-byte aligned buffer");
-    fattn_args a;
     a.kv_extent = nullptr;
     a.act_q = (int8_t *)act;
     a.act_s = act ? (act_ds *)((int8_t *)act + Nq * Hq * D) : nullptr;
@@ -385,6 +453,57 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
         if (ws == nullptr || ws_bytes < need) a.n_splits = 1;   // no scratch: run unsplit
     }
     a.cells_per_split = (Nkv + a.n_splits - 1) / a.n_splits;
+    return MI355_OK;
+}
+
+int fattn_vec_kv(hipStream_t s, const float *q, const void *k, int type_k, const kv_src &kq, const void *v, int type_v, const kv_src &vq,
+                 const void *mask, float *dst, int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2, size_t k_nb1,
+                 size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale, float max_bias, float logit_softcap, void *ws,
+                 size_t ws_bytes, void *act) {
+    fattn_args a;
+    const int frc = fattn_fill(a, q, k, v, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1, scale, max_bias, logit_softcap,
+                               ws, ws_bytes, act, type_k == MI355_F16, type_v == MI355_F16);
+    if (frc != MI355_OK) return frc;
+    a.type_k = type_k;
+    a.type_v = type_v;
+    a.kq = kq;
+    a.vq = vq;
+    return launch_fattn_vec_any(s, a, D);
+}
+
+int launch_fattn_vec_any(hipStream_t s, fattn_args &a, int64_t D) {
+    const int R = (int)(a.Hq / a.Hkv);
+    switch (D) {
+        case 64: return launch_vec_r<64>(s, a, R);
+        case 80: return launch_vec_r<80>(s, a, R);
+        case 96: return launch_vec_r<96>(s, a, R);
+        case 112: return launch_vec_r<112>(s, a, R);
+        case 128: return launch_vec_r<128>(s, a, R);
+        case 256: return launch_vec_r<256>(s, a, R);
+        default: set_error("flash_attn: head size %lld not supported", (long long)D); return MI355_ERR_ARG;
+    }
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+size_t mi355_flash_attn_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq) {
+    // worst case: 256 kv splits
+    (void)Nkv;
+    return (size_t)Nq * (size_t)Hq * 256 * (size_t)(D + 2) * sizeof(float);
+}
+
+int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,
+                               int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2,
+                               size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale,
+                               float max_bias, float logit_softcap, void *ws, size_t ws_bytes, void *act) {
+    fattn_args a;
+    const int frc = fattn_fill(a, q, k, v, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1, scale, max_bias, logit_softcap,
+                               ws, ws_bytes, act, true, true);
+    if (frc != MI355_OK) return frc;
     const int R = (int)(Hq / Hkv);
     hipStream_t s = (hipStream_t)stream;
     if (Nq >= 16 && act == nullptr) {   // prefill: f16 matrix cores
@@ -443,15 +562,7 @@ int mi355_flash_attn_ext_quant(void *stream, const float *q, const void *k, cons
             return MI355_OK;
         }
     }
-    switch (D) {
-        case 64: return launch_vec_r<64>(s, a, R);
-        case 80: return launch_vec_r<80>(s, a, R);
-        case 96: return launch_vec_r<96>(s, a, R);
-        case 112: return launch_vec_r<112>(s, a, R);
-        case 128: return launch_vec_r<128>(s, a, R);
-        case 256: return launch_vec_r<256>(s, a, R);
-        default: set_error("flash_attn: head size %lld not supported", (long long)D); return MI355_ERR_ARG;
-    }
+    return launch_fattn_vec_any(s, a, D);
 }
 
 int mi355_flash_attn_ext(void *stream, const float *q, const void *k, const void *v, const void *mask, float *dst,

@@ -5,8 +5,19 @@
 
 namespace mi355 {
 
+// A Q8_0 / Q4_0 operand of the vector kernel, read block by block where it lies (no f16 copy).  Block g of the owning tensor sits
+// at g * block bytes (row_blocks == 0: plain ggml blocks, the f16 scale in front of the levels) or, for a tensor in the device row
+// layout, in row g / row_blocks at position g % row_blocks (the levels of a row first, its scales behind them).  The (cell, head)
+// row starts at block first_block + cell * (nb1 / block bytes) + head * head_blocks; nb1 is a whole number of rows of the owner.
+struct kv_src {
+    const uint8_t *base;
+    int64_t first_block, row_blocks, head_blocks;
+};
+
 struct fattn_args {
     const uint8_t *q, *k, *v, *mask;
+    int type_k = MI355_F16, type_v = MI355_F16;   // k_fattn_vec only: MI355_Q8_0 / MI355_Q4_0 operands are described by kq / vq
+    kv_src kq = {nullptr, 0, 0, 0}, vq = {nullptr, 0, 0, 0};
     float *dst;      // [D, Hq, Nq]
     int8_t *act_q;   // optional: Q8_1 of dst rows (Hq*D elements per query) in the split activation layout
     act_ds *act_s;
@@ -48,6 +59,16 @@ __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qr
 int launch_fattn_mma(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);
 // the same for a few query rows (decode): one kv split per group, partials merged by k_fattn_combine
 int launch_fattn_mma_dec(hipStream_t s, fattn_args &a, int64_t D);
+
+// the vector kernel on f16 / Q8_0 / Q4_0 operands in any mix (a.type_k, a.type_v, a.kq, a.vq filled in), splits merged by
+// k_fattn_combine; for the shapes the matrix-core kernels do not take, and for every quantized cache read in place
+int launch_fattn_vec_any(hipStream_t s, fattn_args &a, int64_t D);
+// mi355_flash_attn_ext_quant's arguments with typed K / V, served by the vector kernel alone (k, v: the f16 operands' data; a
+// quantized operand is described by kq / vq and its k_nb1 / v_nb1)
+int fattn_vec_kv(hipStream_t s, const float *q, const void *k, int type_k, const kv_src &kq, const void *v, int type_v, const kv_src &vq,
+                 const void *mask, float *dst, int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, size_t q_nb1, size_t q_nb2, size_t k_nb1,
+                 size_t k_nb2, size_t v_nb1, size_t v_nb2, size_t mask_nb1, float scale, float max_bias, float logit_softcap, void *ws,
+                 size_t ws_bytes, void *act);
 
 // one query token over at most 512 cells of an f16 cache, head size 128, up to four query heads per kv head: one launch, one wave
 // per 64 cells, states merged in LDS (fattn_stream.hip); returns 1 when the shape is not served

@@ -1,8 +1,9 @@
 // Quantized KV cache: CPY f32 -> Q8_0 / Q4_0 (what llm_build_kv_store does with -ctk / -ctv q8_0, q4_0) and FLASH_ATTN_EXT over
 // such a cache.  The copies are quantize_row_q8_0_ref / quantize_row_q4_0_ref (ggml/src/ggml-quants.c:39-72, 194-218) bit for
-// bit.  Attention first expands the cells it will read into an f16 scratch image ([cell][kv head][D], d * level rounded to
-// f16) and then runs the f16 kernels on that image: every byte of a quantized cache is read once more than with an f16 cache,
-// which is the price of keeping one set of attention kernels.
+// bit.  Attention with fewer than 16 query rows (decode) reads the blocks where they lie: the vector kernel turns the levels into
+// exact f16 values in its registers and applies the block's scale to the dot / to the weighted row, so every byte of the cache
+// leaves memory once.  With 16 or more query rows the cells are first expanded into an f16 scratch image ([cell][kv head][D],
+// d * level rounded to f16) that the matrix-core kernels then read: the expansion is shared by all rows of the batch.
 //
 // Where a block lives: a caller with a plain ggml cache passes row_blocks = 0 and blocks sit where ggml puts them (block g of the
 // tensor at g * block bytes).  A tensor kept in this library's device row layout (levels of a row first, its scales behind them,
@@ -151,6 +152,25 @@ static size_t kv_image_bytes(int type, int64_t D, int64_t Nkv, int64_t Hkv) {
     return type == MI355_F16 ? 0 : (((size_t)Nkv * (size_t)Hkv * (size_t)D * 2 + 255) & ~(size_t)255);
 }
 
+// From this many query rows on the cache is expanded to f16 once and the matrix-core kernels run on the image (the expansion is
+// shared by all rows); below it the vector kernel dequantizes in its registers.
+constexpr int64_t KV_IMAGE_MIN_ROWS = 16;
+
+// describes a quantized operand for in-place reads; false when its rows do not start on block boundaries or a cell's stride is not
+// a whole number of the owner's rows (then the image path, with its own checks, takes it)
+static bool kv_in_place(int type, const void *p, const void *base, int64_t row_blocks, size_t nb1, size_t nb2, kv_src &o) {
+    const int64_t bb = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES;
+    if (base == nullptr) base = p;
+    const int64_t off = (const char *)p - (const char *)base;
+    if (((uintptr_t)base & 1) != 0 || off < 0 || off % bb != 0 || nb1 % bb != 0 || nb2 % bb != 0 || row_blocks < 0) return false;
+    if (row_blocks > 0 && ((int64_t)(nb1 / bb) % row_blocks) != 0) return false;
+    o.base = (const uint8_t *)base;
+    o.first_block = off / bb;
+    o.row_blocks = row_blocks;
+    o.head_blocks = (int64_t)(nb2 / bb);
+    return true;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -203,12 +223,21 @@ int mi355_flash_attn_ext_kv(void *stream, const float *q, const void *k, int typ
         return mi355_flash_attn_ext_quant(stream, q, k, v, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1, scale,
                                           max_bias, logit_softcap, ws, ws_bytes, act);
     MI355_REQUIRE(D > 0 && D % 32 == 0 && Nkv > 0 && Hkv > 0, "flash_attn_kv: head size %lld is not a whole number of blocks", (long long)D);
+    hipStream_t s = (hipStream_t)stream;
+    // A few query rows (decode): the vector kernel reads the blocks where they lie, each byte of the cache once.
+    if (Nq < KV_IMAGE_MIN_ROWS) {
+        kv_src kq = {nullptr, 0, 0, 0}, vq = {nullptr, 0, 0, 0};
+        const bool k_ok = type_k == MI355_F16 || kv_in_place(type_k, k, k_base, k_row_blocks, k_nb1, k_nb2, kq);
+        const bool v_ok = type_v == MI355_F16 || kv_in_place(type_v, v, v_base, v_row_blocks, v_nb1, v_nb2, vq);
+        if (k_ok && v_ok)
+            return fattn_vec_kv(s, q, k, type_k, kq, v, type_v, vq, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1, scale,
+                                max_bias, logit_softcap, ws, ws_bytes, act);
+    }
     const size_t kb = kv_image_bytes(type_k, D, Nkv, Hkv), vb = kv_image_bytes(type_v, D, Nkv, Hkv);
     MI355_REQUIRE(ws != nullptr && ((uintptr_t)ws & 255) == 0 && ws_bytes >= kb + vb, "flash_attn_kv: the workspace must be 256-byte aligned and hold the f16 images (%zu bytes)", kb + vb);
     // the images sit at the end of the workspace; what is in front of them serves the kv splits as before
     const size_t front = (ws_bytes - kb - vb) & ~(size_t)255;
     uint8_t *kimg = (uint8_t *)ws + front, *vimg = kimg + kb;
-    hipStream_t s = (hipStream_t)stream;
     if (type_k != MI355_F16) {
         int rc = kv_expand(s, type_k, k, k_base, k_row_blocks, k_nb1, k_nb2, kimg, D, Nkv, Hkv);
         if (rc != MI355_OK) return rc;
