@@ -7,10 +7,17 @@
 // super-blocks in int32, the Q4_K min term is one v_mfma_f32_32x32x16_f16 per super-block on exact small integers, and the
 // vector ALU touches a result once per 256 elements.
 //
-// What differs is the data path and the schedule.  Measured on this part, per compute unit: about 22 bytes per clock from L2 into
-// LDS; a wave does not overlap its own vector instructions with its own matrix instructions, two waves of a SIMD do; packed
-// 16-bit integer multiplies run at a quarter of the rate of other vector instructions (which rules out keeping one byte per
-// Q4_K weight in LDS and multiplying by the sub-block scale on the way into the matrix instruction: measured, 35 % slower).
+// What differs is the data path and the schedule.  Measured on this part: about 52 bytes per clock and compute unit from L2 into LDS;
+// one wave per SIMD issues a matrix instruction (32x32x32 i8) every 15.8 ns alone and every 18.2 / 23.7 / 30.5 ns with 4 / 8 / 12
+// independent vector instructions behind each, two waves per SIMD every 14.6 / 15.2 / 19.2 / 23.3 ns: a wave overlaps its own
+// vector and matrix instructions as long as both are there to issue, and two waves issue vector instructions at twice the rate of
+// one (1.3-1.5 ns against 2.3-2.8 ns each).  Keeping one byte per Q4_K weight in LDS and multiplying by the sub-block scale on the
+// way into the matrix instruction was measured 35 % slower than the two planes.
+// A 128 x 256 tile (64 x 64 per wave: 0.75 KiB of operand reads per matrix instruction instead of 1, same arithmetic bit for bit) was
+// built and measured on 14336 x 4096 at batch 512: Q6_K 76.8 us against 76-80 us here, Q4_K 99 us against 82-86 us.  At that wave
+// tile the registers hold one set of integer sums, so a finished super-block is scaled in one burst at the start of the next; both
+// waves of a SIMD reach it together and the matrix pipe waits (all 68.1 us, without the scaling 52.1, matrix instructions alone
+// 41.5, empty loop 11.8).  The second set of sums below is what lets the scaling hide; it fits only at 32 x 64 per wave.
 //  * Both operands live in HBM as *tile images* (tiles.hpp): tiles of 16 rows x 64 elements = 1 KiB, each byte for byte what
 //    LDS holds, so one wave-wide global_load_lds moves a tile and nobody computes an address per element: 384 bytes from L2 per
 //    matrix instruction where a 64 x 128 tile needs 512.

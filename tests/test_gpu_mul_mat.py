@@ -186,6 +186,9 @@ def test_skinny_matches_oracle(dev, name, t, N, K, B, split):
     got = mi355.mul_mat_skinny(t, Wd, _to_dev(dev, x), split=split).cpu().numpy()
     got_res = mi355.mul_mat_skinny(t, Wd, _to_dev(dev, x), residual=_to_dev(dev, res), split=split).cpu().numpy()
     assert np.array_equal(got_res, got + res)
+    if B > 192 and not split:   # the 128 x 256 tile kernel holds the bits of the 128 x 128 one (which a 128-row batch takes)
+        a128 = mi355.quantize_act_q8k_tiled(_to_dev(dev, x[B - 128:]))
+        assert np.array_equal(got[B - 128:], mi355.mul_mat_q8k_tiled(t, tiles, a128, N, K, 128, split=False).cpu().numpy())
     Nt, Bt = min(N, 64), min(B, 24)
     want = orc.mul_mat("q8_1", t, Wq[:Nt], x[:Bt])
     assert orc.nmse(got[:Bt, :Nt], want) < 1e-9      # exact integer dots; f32 against f64 scale algebra
@@ -330,7 +333,8 @@ def test_quantize_q8k_tiled_bit_exact(dev, K, B):
 
 
 @pytest.mark.parametrize("name,t", TILED_TYPES)
-@pytest.mark.parametrize("N,K,B", [(512, 4096, 64), (384, 2048, 512), (130, 2048, 33), (128, 14336, 100), (200, 2048, 77), (1000, 6144, 300)])
+@pytest.mark.parametrize("N,K,B", [(512, 4096, 64), (384, 2048, 512), (130, 2048, 33), (128, 14336, 100), (200, 2048, 77), (1000, 6144, 300),
+                                   (200, 2048, 250), (1000, 6144, 450), (4096, 4096, 512)])     # 193+ rows: 256-row column tiles where the last is over half full
 @pytest.mark.parametrize("split", [False, True])
 def test_mmq_tiled_matches_oracle(dev, name, t, N, K, B, split):
     """the wide-tile K-quant GEMM on tile images: the CPU's own integer sums (ggml-cpu-quants.c:6817-6848, 8262-8283), ragged row and
@@ -347,6 +351,9 @@ def test_mmq_tiled_matches_oracle(dev, name, t, N, K, B, split):
     got = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B, split=split).cpu().numpy()
     got_res = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B, residual=_to_dev(dev, res), split=split).cpu().numpy()
     assert np.array_equal(got_res, got + res)
+    if B > 192 and not split:   # the 128 x 256 tile kernel holds the bits of the 128 x 128 one (which a 128-row batch takes)
+        a128 = mi355.quantize_act_q8k_tiled(_to_dev(dev, x[B - 128:]))
+        assert np.array_equal(got[B - 128:], mi355.mul_mat_q8k_tiled(t, tiles, a128, N, K, 128, split=False).cpu().numpy())
     Nt, Bt = min(N, 64), min(B, 24)
     assert orc.nmse(got[:Bt, :Nt], orc.mul_mat("cpu", t, Wq[:Nt], x[:Bt])) < 1e-9
     # the last rows and columns (partial tiles)
