@@ -468,6 +468,18 @@ int fattn_vec_kv(hipStream_t s, const float *q, const void *k, int type_k, const
     a.type_v = type_v;
     a.kq = kq;
     a.vq = vq;
+    // One token over a long cache with both operands quantized: the streaming kernel (at 1024 cells the 512 waves have two tiles
+    // each; below that the vector kernel's splits are as quick)
+    constexpr int64_t stream_q_min = 1024;
+    if (Nq == 1 && Nkv >= stream_q_min && type_k != MI355_F16 && type_v != MI355_F16) {
+        fattn_args b = a;
+        const int rc = launch_fattn_dec_stream_q(s, b, D, ws_bytes);
+        if (rc < 0) return rc;
+        if (rc == 0) {
+            MI355_LAUNCH(k_fattn_combine<128>, dim3((unsigned)(Nq * Hq)), dim3(512), 0, s, b.ws, b.dst, b.n_splits, b.act_q, b.act_s, b.Hq);
+            return launch_status("k_fattn_combine");
+        }
+    }
     return launch_fattn_vec_any(s, a, D);
 }
 

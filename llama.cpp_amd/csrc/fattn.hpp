@@ -77,4 +77,7 @@ int launch_fattn_dec_short(hipStream_t s, fattn_args &a, int64_t D);
 // (fattn_stream.hip); sets a.n_splits for k_fattn_combine; returns 1 when the shape is not served
 int launch_fattn_dec_stream(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);
 
+// the same over a Q8_0 / Q4_0 cache in the device row layout, read in place (a.type_k, a.type_v, a.kq, a.vq filled in)
+int launch_fattn_dec_stream_q(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes);
+
 }  // namespace mi355

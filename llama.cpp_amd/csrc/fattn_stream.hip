@@ -1,5 +1,6 @@
-// FLASH_ATTN_EXT for one query token over a long f16 KV cache (head size 128, up to four query heads per kv head): the
-// streaming form.
+// FLASH_ATTN_EXT for one query token over a long KV cache (head size 128, up to four query heads per kv head): the streaming
+// form, for f16 caches (k_fattn_dec_stream, described here) and for Q8_0 / Q4_0 caches in the device row layout
+// (k_fattn_dec_stream_q, further down).
 //
 // The kernel is bound by how many bytes of K and V a compute unit keeps in flight, not by arithmetic: a token reads every cell
 // once and does 4 flops per byte.  So a wave owns a contiguous range of 64-cell tiles of one kv head and moves them with
@@ -77,25 +78,15 @@ __device__ __forceinline__ void fs_slopes(const fattn_args &a, int64_t head0, fl
         }
     }
 }
-// Scores of one tile (kc: the 16 chunks of this lane's K row), the soft-max update of the state, and P^T (head, cell) as f16 into
-// the wave's 512 bytes of LDS at p_wr (= base + 2 * lane), where fs_output reads it back as the A operand.  LDS serves a wave's
-// operations in order: those reads see these writes, and the next tile's writes come after them.
-__device__ __forceinline__ void fs_scores(const u32 (&qv)[FS_D / 2], const u32x4 (&kc)[16], float mv, float scale, float softcap, const float (&slope)[4],
-                                          unsigned p_wr, fs_state &S) {
+// The soft-max update of the state with one tile's raw scores (q . k of this lane's cell and the four heads), and P^T (head, cell)
+// as f16 into the wave's 512 bytes of LDS at p_wr (= base + 2 * lane), where fs_output reads it back as the A operand.  LDS serves a
+// wave's operations in order: those reads see these writes, and the next tile's writes come after them.
+__device__ __forceinline__ void fs_softmax(const float (&raw)[4], float mv, float scale, float softcap, const float (&slope)[4], unsigned p_wr, fs_state &S) {
     constexpr float NEG = -FLT_MAX / 2;
-    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int c = 0; c < 16; c++) {
-        const u32 a0 = qv[4 * c], a1 = qv[4 * c + 1], a2 = qv[4 * c + 2], a3 = qv[4 * c + 3];
-        const u32 b0 = kc[c][0], b1 = kc[c][1], b2 = kc[c][2], b3 = kc[c][3];
-        const u32x2 qa = {a0, a1}, qb = {a2, a3}, ka = {b0, b1}, kb2 = {b2, b3};
-        s0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, qa), __builtin_bit_cast(f16x4, ka), s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, qb), __builtin_bit_cast(f16x4, kb2), s1, 0, 0, 0);
-    }
     const bool valid = mv != -INFINITY;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        float sc = (s0[r] + s1[r]) * scale;
+        float sc = raw[r] * scale;
         if (softcap != 0.0f) sc = softcap * tanhf(sc);
         sc += slope[r] * mv;
         sc = valid ? sc : NEG;
@@ -109,6 +100,23 @@ __device__ __forceinline__ void fs_scores(const u32 (&qv)[FS_D / 2], const u32x4
         const u32 ph = float_to_half_bits(p);
         asm volatile("ds_write_b16 %0, %1 offset:%2" ::"v"(p_wr), "v"(ph), "n"(r * FS_TILE * 2) : "memory");
     }
+}
+// Scores of one tile (kc: the 16 chunks of this lane's K row), then fs_softmax.
+__device__ __forceinline__ void fs_scores(const u32 (&qv)[FS_D / 2], const u32x4 (&kc)[16], float mv, float scale, float softcap, const float (&slope)[4],
+                                          unsigned p_wr, fs_state &S) {
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 16; c++) {
+        const u32 a0 = qv[4 * c], a1 = qv[4 * c + 1], a2 = qv[4 * c + 2], a3 = qv[4 * c + 3];
+        const u32 b0 = kc[c][0], b1 = kc[c][1], b2 = kc[c][2], b3 = kc[c][3];
+        const u32x2 qa = {a0, a1}, qb = {a2, a3}, ka = {b0, b1}, kb2 = {b2, b3};
+        s0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, qa), __builtin_bit_cast(f16x4, ka), s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, qb), __builtin_bit_cast(f16x4, kb2), s1, 0, 0, 0);
+    }
+    float raw[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) raw[r] = s0[r] + s1[r];
+    fs_softmax(raw, mv, scale, softcap, slope, p_wr, S);
 }
 // This lane's offset inside a row-major V tile for the transposing reads of fs_output: lane l' = lane % 16 of its 16-lane group
 // g points at row c0 + l' / 4, elements 16 g + 4 (l' % 4) .. + 3
@@ -291,6 +299,372 @@ __global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream(fattn_arg
     }
 }
 
+// ---- the same over a Q8_0 / Q4_0 cache in the device row layout --------------------------------------------------------------
+// A cell's row in such a cache holds the levels of all its kv heads first and their f16 scales behind them, so the levels of one
+// (cell, head) are 128 / 64 contiguous, 16-byte aligned bytes and its four scales 8 bytes: both move by global-to-LDS transfers like
+// the f16 rows above (levels 16 bytes per lane, scales 4), half the bytes or less per cell.
+// Scores follow the reference's arithmetic for a quantized K (ggml-cpu.c:11037-11046: q is quantized to Q8_0, kq_vec_dot is the
+// integer block dot ggml_vec_dot_q8_0_q8_0 / ggml_vec_dot_q4_0_q8_0, ggml-cpu-quants.c): v_mfma_i32_4x4x4_16b_i8 with A = q levels
+// (row = head) and B = this lane's cell, one accumulator per 32-element block, then sum_b d_k d_q sumi in f32.
+// V (ggml-cpu.c:11078-11090 dequantizes the row and accumulates in f32): the wave turns the tile's levels into d * level as f16 -
+// bytes into the low byte of halves whose high byte is 0x64 (1024 + u), minus 1152 or 1032, times the block's scale, all packed
+// f16 operations on exact values until the one rounding of the product - and writes them row-major into its own 16 KiB of LDS,
+// where fs_output finds what it finds for an f16 cache.
+struct fsq_src {
+    const uint8_t *lv, *sc;   // levels / scales of (cell 0, kv head 0); a cell further on is nb1 bytes further on in both
+    int64_t head_lv, head_sc; // bytes from one kv head to the next
+};
+template <int T>
+struct fsq_geo {
+    static constexpr int ROW = T == MI355_Q8_0 ? 128 : 64;   // bytes of levels per (cell, head)
+    static constexpr int CH = ROW / 16;                       // 16-byte chunks per row
+    static constexpr int RPT = 64 / CH;                       // rows per transfer
+    static constexpr int NT = FS_TILE / RPT;                  // level transfers per tile
+    static constexpr int CNT = NT + 2;                        // with the two scale transfers
+};
+constexpr int FSQ_SCALES = FS_TILE * 8;   // bytes of scales per tile and operand
+
+template <int R4>
+__device__ __forceinline__ int quad_bcast_i(int v) { return __builtin_amdgcn_update_dpp(0, v, R4 * 0x55, 0xF, 0xF, true); }
+
+// q of head head0 + lane % 4 as Q8_0 (quantize_row_q8_0_ref, ggml-quants.c:194-218): 32 words of levels, the f16-rounded scales of
+// the four blocks and the sums of their levels; zeros past the R heads of the group
+__device__ __forceinline__ void fsq_load_q(const fattn_args &a, int64_t head0, int R, int lane, u32 (&qw)[32], float (&dq)[4], int (&qs)[4]) {
+    const int hr = lane & 3;
+    const float *qp = (const float *)(a.q + (head0 + (hr < R ? hr : 0)) * a.q_nb2);
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        f32x4 x[8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            x[i] = *(const f32x4 *)(qp + 32 * b + 4 * i);
+            if (hr >= R) x[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; j++) amax = fmaxf(amax, fabsf(x[i][j]));
+        }
+        const float d = amax / 127.0f;
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            u32 w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int q = (int)roundf(x[i][j] * id);
+                sum += q;
+                w |= (u32)(q & 0xFF) << (8 * j);
+            }
+            qw[8 * b + i] = w;
+        }
+        dq[b] = half_bits_to_float(float_to_half_bits(d));
+        qs[b] = sum;
+    }
+}
+
+// raw scores of this lane's cell against the four heads: kc = the chunks of its K row, ksc = its four scales
+template <int TK>
+__device__ __forceinline__ void fsq_scores(const u32 (&qw)[32], const float (&dqa)[4][4], const int (&qsa)[4][4], const u32x4 (&kc)[fsq_geo<TK>::CH], const u32x2 &ksc,
+                                           float (&raw)[4]) {
+    i32x4 ab[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++) ab[b] = i32x4{0, 0, 0, 0};
+    if constexpr (TK == MI355_Q8_0) {
+#pragma unroll
+        for (int c = 0; c < 8; c++)
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const u32 kw = kc[c][w];
+                ab[c >> 1] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)qw[4 * c + w], (int)kw, ab[c >> 1], 0, 0, 0);
+            }
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const u32 kw = kc[c][w];
+                ab[c] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)qw[8 * c + w], (int)(kw & 0x0F0F0F0Fu), ab[c], 0, 0, 0);
+                ab[c] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)qw[8 * c + 4 + w], (int)((kw >> 4) & 0x0F0F0F0Fu), ab[c], 0, 0, 0);
+            }
+    }
+    float dk[4];
+    dk[0] = half_bits_to_float((unsigned short)(ksc[0] & 0xFFFFu));
+    dk[1] = half_bits_to_float((unsigned short)(ksc[0] >> 16));
+    dk[2] = half_bits_to_float((unsigned short)(ksc[1] & 0xFFFFu));
+    dk[3] = half_bits_to_float((unsigned short)(ksc[1] >> 16));
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int sumi = TK == MI355_Q8_0 ? ab[b][r] : ab[b][r] - 8 * qsa[r][b];
+            sum += (float)sumi * (dk[b] * dqa[r][b]);
+        }
+        raw[r] = sum;
+    }
+}
+
+// four bytes u -> the f16 pairs (u0 + bias, u1 + bias) * d and (u2 + bias, u3 + bias) * d; 1024 + u is exact in a half whose high
+// byte is 0x64, and so is the sum with bias = -(1024 + offset of the level)
+__device__ __forceinline__ u32x2 fsq_bytes_to_f16(u32 u, f16x2 bias, f16x2 d2) {
+    const u32 a = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u), b = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+    const f16x2 x = (__builtin_bit_cast(f16x2, a) + bias) * d2, y = (__builtin_bit_cast(f16x2, b) + bias) * d2;
+    return u32x2{__builtin_bit_cast(u32, x), __builtin_bit_cast(u32, y)};
+}
+
+// V levels of a stage (LDS byte address v_lv, scales at v_sc) -> d * level as f16, row-major [64][128], at LDS byte address v_f16
+template <int TV>
+__device__ __forceinline__ void fsq_convert_v(unsigned v_lv, unsigned v_sc, unsigned v_f16, int lane) {
+    typedef fsq_geo<TV> G;
+    constexpr int NJ = FS_TILE * G::CH / 64;   // chunks per lane: 8 (Q8_0, 16 elements each) or 4 (Q4_0, 32 elements each)
+    u32x4 lv[NJ];
+    u32 sc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        const int chunk = j * 64 + lane, row = chunk / G::CH, c = chunk % G::CH;
+        const int blk = TV == MI355_Q8_0 ? c >> 1 : c;
+        asm volatile("ds_read_b128 %0, %1" : "=v"(lv[j]) : "v"(v_lv + (unsigned)chunk * 16u));
+        asm volatile("ds_read_u16 %0, %1" : "=v"(sc[j]) : "v"(v_sc + (unsigned)(row * 8 + blk * 2)));
+    }
+    if constexpr (NJ == 8)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]),
+                       "+v"(sc[3]), "+v"(sc[4]), "+v"(sc[5]), "+v"(sc[6]), "+v"(sc[7]));
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]));
+    const f16x2 bias = TV == MI355_Q8_0 ? f16x2{(_Float16)-1152.0f, (_Float16)-1152.0f} : f16x2{(_Float16)-1032.0f, (_Float16)-1032.0f};
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        const int chunk = j * 64 + lane, row = chunk / G::CH, c = chunk % G::CH;
+        const u32 dd = sc[j] | (sc[j] << 16);
+        const f16x2 d2 = __builtin_bit_cast(f16x2, dd);
+        if constexpr (TV == MI355_Q8_0) {
+            // elements 16 c .. 16 c + 7, .. + 15 of the row
+            const u32 w0 = lv[j][0], w1 = lv[j][1], w2 = lv[j][2], w3 = lv[j][3];
+            const u32x2 e0 = fsq_bytes_to_f16(w0 ^ 0x80808080u, bias, d2), e1 = fsq_bytes_to_f16(w1 ^ 0x80808080u, bias, d2);
+            const u32x2 e2 = fsq_bytes_to_f16(w2 ^ 0x80808080u, bias, d2), e3 = fsq_bytes_to_f16(w3 ^ 0x80808080u, bias, d2);
+            const u32x4 o0 = {e0[0], e0[1], e1[0], e1[1]}, o1 = {e2[0], e2[1], e3[0], e3[1]};
+            const unsigned dst = v_f16 + (unsigned)(row * FS_ROW + c * 32);
+            asm volatile("ds_write_b128 %0, %1" ::"v"(dst), "v"(o0) : "memory");
+            asm volatile("ds_write_b128 %0, %1 offset:16" ::"v"(dst), "v"(o1) : "memory");
+        } else {
+            u32x4 o[4];   // elements 32 c + 0..7, 8..15 (low nibbles), 16..23, 24..31 (high nibbles)
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const u32 wa = lv[j][2 * h], wb = lv[j][2 * h + 1];
+                const u32x2 la = fsq_bytes_to_f16(wa & 0x0F0F0F0Fu, bias, d2), lb = fsq_bytes_to_f16(wb & 0x0F0F0F0Fu, bias, d2);
+                const u32x2 ha = fsq_bytes_to_f16((wa >> 4) & 0x0F0F0F0Fu, bias, d2), hb = fsq_bytes_to_f16((wb >> 4) & 0x0F0F0F0Fu, bias, d2);
+                o[h] = u32x4{la[0], la[1], lb[0], lb[1]};
+                o[2 + h] = u32x4{ha[0], ha[1], hb[0], hb[1]};
+            }
+            const unsigned dst = v_f16 + (unsigned)(row * FS_ROW + c * 64);
+            asm volatile("ds_write_b128 %0, %1" ::"v"(dst), "v"(o[0]) : "memory");
+            asm volatile("ds_write_b128 %0, %1 offset:16" ::"v"(dst), "v"(o[1]) : "memory");
+            asm volatile("ds_write_b128 %0, %1 offset:32" ::"v"(dst), "v"(o[2]) : "memory");
+            asm volatile("ds_write_b128 %0, %1 offset:48" ::"v"(dst), "v"(o[3]) : "memory");
+        }
+    }
+}
+
+template <int TK, int TV>
+__global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream_q(fattn_args a, fsq_src ksrc, fsq_src vsrc, int tiles_per_wave, int n_tiles, int R) {
+    typedef fsq_geo<TK> GK;
+    typedef fsq_geo<TV> GV;
+    constexpr int K_LV = FS_TILE * GK::ROW, V_LV = FS_TILE * GV::ROW;
+    constexpr int OFF_V = K_LV, OFF_KS = K_LV + V_LV, OFF_VS = OFF_KS + FSQ_SCALES;
+    constexpr int STAGE = OFF_VS + FSQ_SCALES;
+    constexpr int CK = GK::CNT, CV = GV::CNT;   // transfers of the K / V part of a tile
+    __shared__ __attribute__((aligned(1024))) uint8_t ring_buf[FS_WAVES * 2 * STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t vf_buf[FS_WAVES * FS_KT];   // the wave's V tile as f16
+    __shared__ __attribute__((aligned(16))) unsigned short pbuf[FS_WAVES][4][FS_TILE];
+    __shared__ __attribute__((aligned(16))) unsigned short mbuf[FS_WAVES][FS_MAX_TILES * FS_TILE];
+    asm volatile("" ::"v"((void *)ring_buf), "v"((void *)vf_buf) : "memory");
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int split = (int)blockIdx.x * FS_WAVES + wave;
+    const int64_t hk = blockIdx.y;
+    const int t_begin = split * tiles_per_wave;
+    const int t_end = t_begin + tiles_per_wave < n_tiles ? t_begin + tiles_per_wave : n_tiles;
+    const int n = t_end > t_begin ? t_end - t_begin : 0;
+    const int64_t c_begin = (int64_t)t_begin * FS_TILE;
+
+    float slope[4];
+    fs_slopes(a, hk * R, slope);
+    uint8_t *ring = ring_buf + wave * (2 * STAGE);
+    const uint8_t *k_lv = ksrc.lv + hk * ksrc.head_lv, *k_sc = ksrc.sc + hk * ksrc.head_sc;
+    const uint8_t *v_lv = vsrc.lv + hk * vsrc.head_lv, *v_sc = vsrc.sc + hk * vsrc.head_sc;
+    // per-lane offsets of the transfers.  K levels: transfer i moves rows RPT i .. + RPT - 1, lane p -> row RPT i + p / CH, LDS position
+    // p % CH, which holds chunk position ^ swz(row) (swz: (row >> 1) & 7 for 128-byte rows, (row >> 2) & 3 for 64-byte rows), so that
+    // the 64 lanes reading chunk c of their own rows hit all banks.  V levels: rows as they are.  Scales: two transfers of 32 rows.
+    unsigned koff[2], voff, ksoff, vsoff;
+    {
+        const unsigned p = (unsigned)lane;
+        if constexpr (TK == MI355_Q8_0) {
+#pragma unroll
+            for (int e = 0; e < 2; e++) koff[e] = (p >> 3) * (unsigned)a.k_nb1 + (((p & 7) ^ ((4 * e + (p >> 4)) & 7)) << 4);
+        } else {
+            koff[0] = koff[1] = (p >> 2) * (unsigned)a.k_nb1 + (((p & 3) ^ ((p >> 4) & 3)) << 4);
+        }
+        voff = TV == MI355_Q8_0 ? (p >> 3) * (unsigned)a.v_nb1 + ((p & 7) << 4) : (p >> 2) * (unsigned)a.v_nb1 + ((p & 3) << 4);
+        ksoff = (p >> 1) * (unsigned)a.k_nb1 + ((p & 1) << 2);
+        vsoff = (p >> 1) * (unsigned)a.v_nb1 + ((p & 1) << 2);
+    }
+    auto dma16 = [&](const uint8_t *g, unsigned off, uint8_t *l) {   // g, l: wave-uniform
+        asm volatile("" : "+v"(off));
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(g + off), (void __attribute__((address_space(3))) *)l, 16, 0, 0);
+    };
+    auto dma4 = [&](const uint8_t *g, unsigned off, uint8_t *l) {
+        asm volatile("" : "+v"(off));
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(g + off), (void __attribute__((address_space(3))) *)l, 4, 0, 0);
+    };
+    // which = 0: K levels and scales of tile t into stage st (CK transfers), 1: V (CV transfers)
+    auto issue = [&](int t, int st, int which) {
+        const int64_t c0 = c_begin + (int64_t)t * FS_TILE;
+        uint8_t *sb = ring + st * STAGE;
+        const int64_t nb1 = which ? (int64_t)a.v_nb1 : (int64_t)a.k_nb1;
+        const uint8_t *lvp = which ? v_lv : k_lv, *scp = which ? v_sc : k_sc;
+        uint8_t *l_lv = sb + (which ? OFF_V : 0), *l_sc = sb + (which ? OFF_VS : OFF_KS);
+        const int NT = which ? GV::NT : GK::NT, RPT = which ? GV::RPT : GK::RPT, CH = which ? GV::CH : GK::CH;
+        if (c0 + FS_TILE <= a.Nkv) {
+            const uint8_t *g = lvp + c0 * nb1;
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (i < NT) dma16(g + (int64_t)(RPT * i) * nb1, which ? voff : koff[i & 1], l_lv + i * 1024);
+            const uint8_t *gs = scp + c0 * nb1;
+            dma4(gs, which ? vsoff : ksoff, l_sc);
+            dma4(gs + 32 * nb1, which ? vsoff : ksoff, l_sc + 256);
+        } else {   // the cache's last, partial tile: rows past the end repeat the last cell (their scores are discarded)
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (i < NT) {
+                    const int row = RPT * i + lane / CH, pos = lane % CH;
+                    int64_t cell = c0 + row;
+                    if (cell >= a.Nkv) cell = a.Nkv - 1;
+                    const int swz = which ? 0 : (TK == MI355_Q8_0 ? (row >> 1) & 7 : (row >> 2) & 3);
+                    const uint8_t *g = lvp + cell * nb1 + ((pos ^ swz) << 4);
+                    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)g, (void __attribute__((address_space(3))) *)(l_lv + i * 1024), 16, 0, 0);
+                }
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                int64_t cell = c0 + 32 * i + (lane >> 1);
+                if (cell >= a.Nkv) cell = a.Nkv - 1;
+                const uint8_t *g = scp + cell * nb1 + ((lane & 1) << 2);
+                __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)g, (void __attribute__((address_space(3))) *)(l_sc + i * 256), 4, 0, 0);
+            }
+        }
+    };
+
+    fs_state S;
+    fs_init(S);
+    const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
+    if (n > 0) {
+        issue(0, 0, 0);
+        issue(0, 0, 1);
+    }
+    if (n > 1) {
+        issue(1, 1, 0);
+        issue(1, 1, 1);
+    }
+    // While the first two tiles travel: q as Q8_0 and this wave's mask values.
+    const int hr = lane & 3;
+    u32 qw[32];
+    float dq[4], dqa[4][4];
+    int qs[4], qsa[4][4];
+    fsq_load_q(a, hk * R, R, lane, qw, dq, qs);
+#pragma unroll
+    for (int b = 0; b < 4; b++) {   // every lane needs the scales and sums of all four heads: lane r of its quad holds head r's
+        const int di = __builtin_bit_cast(int, dq[b]);
+        dqa[0][b] = __builtin_bit_cast(float, quad_bcast_i<0>(di));
+        dqa[1][b] = __builtin_bit_cast(float, quad_bcast_i<1>(di));
+        dqa[2][b] = __builtin_bit_cast(float, quad_bcast_i<2>(di));
+        dqa[3][b] = __builtin_bit_cast(float, quad_bcast_i<3>(di));
+        qsa[0][b] = quad_bcast_i<0>(qs[b]);
+        qsa[1][b] = quad_bcast_i<1>(qs[b]);
+        qsa[2][b] = quad_bcast_i<2>(qs[b]);
+        qsa[3][b] = quad_bcast_i<3>(qs[b]);
+    }
+    unsigned short *mw = mbuf[wave];
+    {
+        const unsigned short *mrow = (const unsigned short *)a.mask;
+        const bool wide = ((uintptr_t)mrow & 15) == 0;
+        u32x4 mc[FS_MAX_TILES / 8];
+#pragma unroll
+        for (int it = 0; it < FS_MAX_TILES / 8; it++) {
+            const int j = it * 64 + lane;
+            const int64_t c = c_begin + (int64_t)j * 8;
+            mc[it] = u32x4{0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u};   // -inf
+            if (j * 8 < n * FS_TILE) {
+                if (mrow && wide && c + 8 <= a.Nkv) {
+                    mc[it] = load16(mrow + c);
+                } else {
+                    unsigned short e[8];
+#pragma unroll
+                    for (int i = 0; i < 8; i++) e[i] = c + i < a.Nkv ? (mrow ? mrow[c + i] : (unsigned short)0) : (unsigned short)0xFC00;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) mc[it][i] = (u32)e[2 * i] | ((u32)e[2 * i + 1] << 16);
+                }
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < FS_MAX_TILES / 8; it++) {
+            const int j = it * 64 + lane;
+            if (j * 8 < n * FS_TILE) *(u32x4 *)(mw + j * 8) = mc[it];
+        }
+    }
+    // From here on LDS is read and written through inline assembly with waits placed by hand (see k_fattn_dec_stream).
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    const unsigned ring_lds = (unsigned)(uintptr_t)(void __attribute__((address_space(3))) *)ring;
+    const unsigned vf_lds = (unsigned)(uintptr_t)(void __attribute__((address_space(3))) *)(vf_buf + wave * FS_KT);
+    const unsigned k_lane = TK == MI355_Q8_0 ? (unsigned)lane * 128u + ((((unsigned)lane >> 1) & 7u) << 4) : (unsigned)lane * 64u + ((((unsigned)lane >> 2) & 3u) << 4);
+    const unsigned m_lane = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned short *)mw + (unsigned)lane * 2;
+    const unsigned p_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned short *)&pbuf[wave][0][0];
+    const unsigned p_wr = p_base + (unsigned)lane * 2, p_rd = p_base + (unsigned)hr * (FS_TILE * 2);
+
+    for (int t = 0; t < n; t++) {
+        const int st = t & 1;
+        // K(t) has landed when at most V(t), K(t + 1), V(t + 1) are still on their way (transfers complete in the order issued)
+        if (t + 1 < n) FS_WAIT_VM(CV + CK + CV);
+        else FS_WAIT_VM(CV);
+        const unsigned sb = ring_lds + (unsigned)st * STAGE;
+        u32x4 kc[GK::CH];
+        u32x2 ksc;
+        u32 mbits;
+        asm volatile("ds_read_u16 %0, %1" : "=v"(mbits) : "v"(m_lane + (unsigned)t * (FS_TILE * 2)));
+        asm volatile("ds_read_b64 %0, %1" : "=v"(ksc) : "v"(sb + (unsigned)OFF_KS + (unsigned)lane * 8u));
+#pragma unroll
+        for (int c = 0; c < GK::CH; c++) asm volatile("ds_read_b128 %0, %1" : "=v"(kc[c]) : "v"(sb + (k_lane ^ (unsigned)(c << 4))));
+        if constexpr (GK::CH == 8)
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(mbits), "+v"(ksc), "+v"(kc[0]), "+v"(kc[1]), "+v"(kc[2]), "+v"(kc[3]), "+v"(kc[4]), "+v"(kc[5]), "+v"(kc[6]), "+v"(kc[7]));
+        else
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(mbits), "+v"(ksc), "+v"(kc[0]), "+v"(kc[1]), "+v"(kc[2]), "+v"(kc[3]));
+        if (t + 2 < n) issue(t + 2, st, 0);   // the K rows are in registers: their part of the stage is free
+        float raw[4];
+        fsq_scores<TK>(qw, dqa, qsa, kc, ksc, raw);
+        fs_softmax(raw, half_bits_to_float((unsigned short)mbits), scale, a.softcap, slope, p_wr, S);
+        // V(t) has landed when at most K(t + 1), V(t + 1), K(t + 2) are outstanding
+        if (t + 2 < n) FS_WAIT_VM(CK + CV + CK);
+        else if (t + 1 < n) FS_WAIT_VM(CK + CV);
+        else FS_WAIT_VM(0);
+        fsq_convert_v<TV>(sb + (unsigned)OFF_V, sb + (unsigned)OFF_VS, vf_lds, lane);
+        // the levels are in registers or already converted: the V part of the stage may be overwritten
+        if (t + 2 < n) issue(t + 2, st, 1);
+        fs_output(vf_lds + fs_v_lane(lane), p_rd, S);
+    }
+
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        if (r < R) {
+            const float L = wave_sum_dpp(S.lsum[r]);
+            float *p = a.ws + (((int64_t)hk * R + r) * a.n_splits + split) * (FS_D + 2);
+            p[lane] = S.o0[r];
+            p[64 + lane] = S.o1[r];
+            if (lane == 0) {
+                p[FS_D] = S.m[r];
+                p[FS_D + 1] = L;
+            }
+        }
+    }
+}
+
 // ---- short caches: at most 512 cells, one launch -------------------------------------------------------------------------------
 // One group per kv head, one wave per 64-cell tile (up to eight).  Nothing here is bound by bytes: the time is one trip to memory
 // plus the arithmetic of one tile, so a wave requests everything at once - its K and V tiles as coalesced 16-byte loads into
@@ -434,6 +808,50 @@ int launch_fattn_dec_stream(hipStream_t s, fattn_args &a, int64_t D, size_t ws_b
     a.n_splits = (int)n_splits;
     MI355_LAUNCH(k_fattn_dec_stream, dim3((unsigned)(n_splits / FS_WAVES), (unsigned)a.Hkv), dim3(FS_WAVES * 64), 0, s, a, (int)tiles_per_wave, (int)n_tiles, (int)R);
     return launch_status("k_fattn_dec_stream");
+}
+
+// fsq_src of a kv_src in the device row layout; false when the operand does not have the shape the kernel moves (whole heads of four
+// blocks inside one row of the owner, levels 16-byte and scales 4-byte aligned)
+static bool fsq_describe(int type, const kv_src &q, int64_t Hkv, size_t nb1, fsq_src &o) {
+    if (q.row_blocks <= 0 || q.base == nullptr) return false;
+    const int64_t BB = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES, LB = type == MI355_Q8_0 ? 32 : 16;
+    const int64_t row0 = q.first_block / q.row_blocks, b0 = q.first_block % q.row_blocks, RB = q.row_blocks * BB;
+    if (q.head_blocks < FS_D / 32 || b0 + (Hkv - 1) * q.head_blocks + FS_D / 32 > q.row_blocks) return false;
+    o.lv = q.base + row0 * RB + b0 * LB;
+    o.sc = q.base + row0 * RB + q.row_blocks * LB + b0 * 2;
+    o.head_lv = q.head_blocks * LB;
+    o.head_sc = q.head_blocks * 2;
+    if (((uintptr_t)o.lv & 15) != 0 || (o.head_lv & 15) != 0 || (nb1 & 15) != 0 || ((uintptr_t)o.sc & 3) != 0 || (o.head_sc & 3) != 0) return false;
+    if (nb1 >= ((size_t)1 << 26)) return false;   // the per-lane offsets are 32-bit
+    return true;
+}
+
+// One query token over a long Q8_0 / Q4_0 cache in the device row layout (a.type_k, a.type_v, a.kq, a.vq filled in), head size 128,
+// R <= 4.  Sets a.n_splits; the caller merges the splits with k_fattn_combine.  Returns 1 when the shape is not served.
+int launch_fattn_dec_stream_q(hipStream_t s, fattn_args &a, int64_t D, size_t ws_bytes) {
+    const int64_t R = a.Hq / a.Hkv;
+    if (D != FS_D || a.Nq != 1 || R > 4 || a.Hkv > 65535 || a.ws == nullptr || (a.q_nb2 % 16) != 0) return 1;
+    if ((a.type_k != MI355_Q8_0 && a.type_k != MI355_Q4_0) || (a.type_v != MI355_Q8_0 && a.type_v != MI355_Q4_0)) return 1;
+    fsq_src ks, vs;
+    if (!fsq_describe(a.type_k, a.kq, a.Hkv, a.k_nb1, ks) || !fsq_describe(a.type_v, a.vq, a.Hkv, a.v_nb1, vs)) return 1;
+    const int64_t n_tiles = (a.Nkv + FS_TILE - 1) / FS_TILE;
+    int64_t waves_per_head = FS_TOTAL_WAVES / a.Hkv;
+    if (waves_per_head < FS_WAVES) waves_per_head = FS_WAVES;
+    if (waves_per_head > 256) waves_per_head = 256;   // k_fattn_combine takes up to 256 splits
+    int64_t tiles_per_wave = (n_tiles + waves_per_head - 1) / waves_per_head;
+    if (tiles_per_wave > FS_MAX_TILES) return 1;
+    int64_t n_splits = (n_tiles + tiles_per_wave - 1) / tiles_per_wave;
+    n_splits = (n_splits + FS_WAVES - 1) / FS_WAVES * FS_WAVES;   // whole groups; a wave without tiles writes an empty partial
+    if (ws_bytes < (size_t)a.Hq * (size_t)n_splits * (size_t)(FS_D + 2) * sizeof(float)) return 1;
+    a.n_splits = (int)n_splits;
+    const dim3 grid((unsigned)(n_splits / FS_WAVES), (unsigned)a.Hkv), block(FS_WAVES * 64);
+#define MI355_FSQ_LAUNCH(TK, TV) MI355_LAUNCH((k_fattn_dec_stream_q<TK, TV>), grid, block, 0, s, a, ks, vs, (int)tiles_per_wave, (int)n_tiles, (int)R)
+    if (a.type_k == MI355_Q8_0 && a.type_v == MI355_Q8_0) MI355_FSQ_LAUNCH(MI355_Q8_0, MI355_Q8_0);
+    else if (a.type_k == MI355_Q8_0) MI355_FSQ_LAUNCH(MI355_Q8_0, MI355_Q4_0);
+    else if (a.type_v == MI355_Q8_0) MI355_FSQ_LAUNCH(MI355_Q4_0, MI355_Q8_0);
+    else MI355_FSQ_LAUNCH(MI355_Q4_0, MI355_Q4_0);
+#undef MI355_FSQ_LAUNCH
+    return launch_status("k_fattn_dec_stream_q");
 }
 
 }  // namespace mi355

@@ -1,8 +1,9 @@
 // Quantized KV cache: CPY f32 -> Q8_0 / Q4_0 (what llm_build_kv_store does with -ctk / -ctv q8_0, q4_0) and FLASH_ATTN_EXT over
 // such a cache.  The copies are quantize_row_q8_0_ref / quantize_row_q4_0_ref (ggml/src/ggml-quants.c:39-72, 194-218) bit for
-// bit.  Attention with fewer than 16 query rows (decode) reads the blocks where they lie: the vector kernel turns the levels into
-// exact f16 values in its registers and applies the block's scale to the dot / to the weighted row, so every byte of the cache
-// leaves memory once.  With 16 or more query rows the cells are first expanded into an f16 scratch image ([cell][kv head][D],
+// bit.  Attention with fewer than 16 query rows (decode) reads the blocks where they lie, every byte of the cache once: one token
+// over 1024 or more cells of a cache in the device row layout takes the streaming kernel (fattn_stream.hip: integer block dots
+// with q as Q8_0, the reference's own arithmetic; V expanded to f16 inside the wave), everything else the vector kernel, which
+// turns the levels into exact f16 values in its registers and applies the block's scale afterwards.  With 16 or more query rows the cells are first expanded into an f16 scratch image ([cell][kv head][D],
 // d * level rounded to f16) that the matrix-core kernels then read: the expansion is shared by all rows of the batch.
 //
 // Where a block lives: a caller with a plain ggml cache passes row_blocks = 0 and blocks sit where ggml puts them (block g of the

@@ -61,8 +61,11 @@ def _case(rng, D, Nq, Nkv, Hq, Hkv):
     return q, kf, vf, mask
 
 
-def _textbook(q, k, tk, v, tv, mask, scale):
+def _textbook(q, k, tk, v, tv, mask, scale, q_as_q8_0=False):
+    """q_as_q8_0: q rounded to Q8_0 first, as ggml-cpu does for a quantized K (its dot is the integer block dot, ggml-cpu.c:11037-11046)"""
     Hq, Nq, D = q.shape
+    if q_as_q8_0:
+        q = orc.dequantize("oracle", orc.Q8_0, orc.quantize("oracle", orc.Q8_0, q.reshape(Hq * Nq, D)), D).reshape(Hq, Nq, D)
     Hkv, Nkv = k.shape[0], k.shape[1]
 
     def deq(a, t):
@@ -126,10 +129,32 @@ def test_flash_attn_quantized_kv(dev, kname, tk, vname, tv, D, Nq, Nkv, Hq, Hkv,
     scale = 1.0 / np.sqrt(D)
     got = _run(dev, q, k, tk, v, tv, mask, scale, device_layout)
     assert np.isfinite(got).all()
-    # exact arithmetic on the dequantized cache: only the f16 rounding of q and of d * level separates the two
-    assert orc.nmse(got, _textbook(q, k, tk, v, tv, mask, scale)) < 1e-5
+    # exact arithmetic on the dequantized cache: only the f16 rounding of q and of d * level separates the two (the streaming kernel,
+    # which one token over 1024+ cells of a fully quantized cache in the device layout takes, rounds q to Q8_0 as ggml-cpu does)
+    streaming = device_layout and Nq == 1 and Nkv >= 1024 and tk != orc.F16 and tv != orc.F16
+    assert orc.nmse(got, _textbook(q, k, tk, v, tv, mask, scale, q_as_q8_0=streaming)) < 1e-5
     # the reference kernel quantizes q to Q8_0 for a quantized K: its own distance from exact is ~2e-5
     if Nq * Nkv * Hq <= 40 * 700 * 8:
         assert orc.nmse(got, orc.flash_attn_kv("cpu", q, k, tk, v, tv, mask.view(np.uint16), scale)) <= 5e-4      # tests/test-backend-ops.cpp:3137
     if orc.ref is not None:
         assert orc.nmse(got, orc.flash_attn_kv("ref", q, k, tk, v, tv, mask.view(np.uint16), scale, n_threads=16)) <= 5e-4
+
+
+@pytest.mark.parametrize("kname,tk", [kt for kt in KV_TYPES if kt[1] != orc.F16])
+@pytest.mark.parametrize("vname,tv", [kt for kt in KV_TYPES if kt[1] != orc.F16])
+@pytest.mark.parametrize("Nkv,Hq,Hkv", [(1024, 32, 8), (4096, 32, 8), (5000, 32, 8), (16421, 32, 8), (2048, 8, 8), (3000, 16, 8), (40000, 8, 2)])
+def test_flash_attn_quantized_kv_streaming(dev, kname, tk, vname, tv, Nkv, Hq, Hkv):
+    """one token over a long quantized cache in the device row layout: the streaming kernel (levels and scales by global-to-LDS transfers,
+    integer block dots of Q8_0-quantized q with K, V expanded to f16 inside the wave).  Held to the reference's arithmetic - exact
+    sums with q rounded to Q8_0 - and, more loosely, to the sums with q unrounded; ragged last tiles, one to four heads per kv head."""
+    D = 128
+    rng = np.random.default_rng(Nkv + Hq + tk * 3 + tv)
+    q, kf, vf, mask = _case(rng, D, 1, Nkv, Hq, Hkv)
+    k, v = orc.kv_rows(tk, kf), orc.kv_rows(tv, vf)
+    scale = 1.0 / np.sqrt(D)
+    got = _run(dev, q, k, tk, v, tv, mask, scale, True)
+    assert np.isfinite(got).all()
+    assert orc.nmse(got, _textbook(q, k, tk, v, tv, mask, scale, q_as_q8_0=True)) < 1e-5
+    assert orc.nmse(got, _textbook(q, k, tk, v, tv, mask, scale)) < 5e-4
+    if orc.ref is not None:   # ggml-cpu itself: same rounding of q, same integer dots; its V sum runs in f16 for f16 V only
+        assert orc.nmse(got, orc.flash_attn_kv("ref", q, k, tk, v, tv, mask.view(np.uint16), scale, n_threads=16)) <= 1e-5
