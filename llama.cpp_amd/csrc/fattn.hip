@@ -105,8 +105,8 @@ __device__ __forceinline__ float kv_levels8_f16(int type, const u32x4 &raw, int 
     return half_bits_to_float((unsigned short)raw[2]);
 }
 
-// NW: waves per group
-template <int D, int R, int NW = 4>
+// NW: waves per group; QUANT: K and / or V may be Q8_0 / Q4_0 (a.type_k, a.type_v), read in place
+template <int D, int R, int NW = 4, bool QUANT = false>
 __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     constexpr int LPR = D <= 64 ? 8 : (D <= 128 ? 16 : 32);   // lanes per K/V row
     constexpr int CPW = 64 / LPR;                               // cells per wave step
@@ -166,7 +166,7 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
     const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
     // quantized operands (wave-uniform choice): this lane's place in the rows of kv head hk
-    const bool k_f16 = a.type_k == MI355_F16, v_f16 = a.type_v == MI355_F16;
+    const bool k_f16 = !QUANT || a.type_k == MI355_F16, v_f16 = !QUANT || a.type_v == MI355_F16;
     kv_lane kl = {nullptr, nullptr, 0}, vl = {nullptr, nullptr, 0};
     if (!k_f16 && active) kl = kv_lane_of(a.kq, a.type_k, hk, d0);
     if (!v_f16 && active) vl = kv_lane_of(a.vq, a.type_v, hk, d0);
@@ -384,9 +384,19 @@ static int pick_splits(int64_t Nkv, int64_t Hkv, int64_t Nq) {
 
 template <int D, int R, int NW = 4>
 static int launch_vec(hipStream_t s, fattn_args &a) {
+    const bool quant = a.type_k != MI355_F16 || a.type_v != MI355_F16;
     a.groups = (int)(a.Hq / a.Hkv) / R;
     const dim3 grid((unsigned)a.n_splits, (unsigned)(a.Hkv * a.groups), (unsigned)a.Nq);
-    MI355_LAUNCH((k_fattn_vec<D, R, NW>), grid, dim3(NW * 64), 0, s, a);
+    if constexpr (D % 32 == 0) {
+        if (quant) MI355_LAUNCH((k_fattn_vec<D, R, NW, true>), grid, dim3(NW * 64), 0, s, a);
+        else MI355_LAUNCH((k_fattn_vec<D, R, NW, false>), grid, dim3(NW * 64), 0, s, a);
+    } else {
+        if (quant) {
+            set_error("flash_attn: head size %d is not a whole number of quantization blocks", D);
+            return MI355_ERR_ARG;
+        }
+        MI355_LAUNCH((k_fattn_vec<D, R, NW, false>), grid, dim3(NW * 64), 0, s, a);
+    }
     int rc = launch_status("k_fattn_vec");
     if (rc != MI355_OK) return rc;
     if (a.n_splits > 1) {

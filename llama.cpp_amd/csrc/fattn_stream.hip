@@ -125,23 +125,24 @@ __device__ __forceinline__ unsigned fs_v_lane(int lane) {
 }
 // Output of one tile: four cells per step, elements lane and 64 + lane; every operand of the tile is requested before the first
 // is used.  v_addr: LDS byte address of the V tile + fs_v_lane; p_rd: the wave's P^T + 128 * (lane % 4).
+template <int NJ = 16>   // steps of four cells: 16 = a whole tile, 8 = half of one
 __device__ __forceinline__ void fs_output(unsigned v_addr, unsigned p_rd, fs_state &S) {
-    u32x2 vlo[16], vhi[16], pa[16];
+    u32x2 vlo[NJ], vhi[NJ], pa[NJ];
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
+    for (int j = 0; j < NJ; j++) {
         const unsigned addr = v_addr + (unsigned)(j * 4 * FS_ROW);
         asm volatile("ds_read_b64 %0, %1" : "=v"(pa[j]) : "v"(p_rd + (unsigned)(j * 8)));
         asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(vlo[j]) : "v"(addr));
         asm volatile("ds_read_b64_tr_b16 %0, %1 offset:128" : "=v"(vhi[j]) : "v"(addr));
     }
 #pragma unroll
-    for (int jb = 0; jb < 16; jb += 8)   // the wait names its registers so that nothing is used ahead of it; 24 operands per statement
+    for (int jb = 0; jb < NJ; jb += 8)   // the wait names its registers so that nothing is used ahead of it; 24 operands per statement
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(vlo[jb]), "+v"(vlo[jb + 1]), "+v"(vlo[jb + 2]), "+v"(vlo[jb + 3]), "+v"(vlo[jb + 4]), "+v"(vlo[jb + 5]), "+v"(vlo[jb + 6]), "+v"(vlo[jb + 7]),
                        "+v"(vhi[jb]), "+v"(vhi[jb + 1]), "+v"(vhi[jb + 2]), "+v"(vhi[jb + 3]), "+v"(vhi[jb + 4]), "+v"(vhi[jb + 5]), "+v"(vhi[jb + 6]), "+v"(vhi[jb + 7]),
                        "+v"(pa[jb]), "+v"(pa[jb + 1]), "+v"(pa[jb + 2]), "+v"(pa[jb + 3]), "+v"(pa[jb + 4]), "+v"(pa[jb + 5]), "+v"(pa[jb + 6]), "+v"(pa[jb + 7]));
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
+    for (int j = 0; j < NJ; j++) {
         S.o0 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, pa[j]), __builtin_bit_cast(f16x4, vlo[j]), S.o0, 0, 0, 0);
         S.o1 = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, pa[j]), __builtin_bit_cast(f16x4, vhi[j]), S.o1, 0, 0, 0);
     }
@@ -412,11 +413,12 @@ __device__ __forceinline__ u32x2 fsq_bytes_to_f16(u32 u, f16x2 bias, f16x2 d2) {
     return u32x2{__builtin_bit_cast(u32, x), __builtin_bit_cast(u32, y)};
 }
 
-// V levels of a stage (LDS byte address v_lv, scales at v_sc) -> d * level as f16, row-major [64][128], at LDS byte address v_f16
+// V levels of 32 cells of a stage (LDS byte addresses of the first cell's levels / scales) -> d * level as f16, row-major
+// [32][128], at LDS byte address v_f16
 template <int TV>
 __device__ __forceinline__ void fsq_convert_v(unsigned v_lv, unsigned v_sc, unsigned v_f16, int lane) {
     typedef fsq_geo<TV> G;
-    constexpr int NJ = FS_TILE * G::CH / 64;   // chunks per lane: 8 (Q8_0, 16 elements each) or 4 (Q4_0, 32 elements each)
+    constexpr int NJ = 32 * G::CH / 64;   // chunks per lane: 4 (Q8_0, 16 elements each) or 2 (Q4_0, 32 elements each)
     u32x4 lv[NJ];
     u32 sc[NJ];
 #pragma unroll
@@ -426,12 +428,10 @@ __device__ __forceinline__ void fsq_convert_v(unsigned v_lv, unsigned v_sc, unsi
         asm volatile("ds_read_b128 %0, %1" : "=v"(lv[j]) : "v"(v_lv + (unsigned)chunk * 16u));
         asm volatile("ds_read_u16 %0, %1" : "=v"(sc[j]) : "v"(v_sc + (unsigned)(row * 8 + blk * 2)));
     }
-    if constexpr (NJ == 8)
-        asm volatile("s_waitcnt lgkmcnt(0)"
-                     : "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(lv[4]), "+v"(lv[5]), "+v"(lv[6]), "+v"(lv[7]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]),
-                       "+v"(sc[3]), "+v"(sc[4]), "+v"(sc[5]), "+v"(sc[6]), "+v"(sc[7]));
-    else
+    if constexpr (NJ == 4)
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lv[0]), "+v"(lv[1]), "+v"(lv[2]), "+v"(lv[3]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]));
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lv[0]), "+v"(lv[1]), "+v"(sc[0]), "+v"(sc[1]));
     const f16x2 bias = TV == MI355_Q8_0 ? f16x2{(_Float16)-1152.0f, (_Float16)-1152.0f} : f16x2{(_Float16)-1032.0f, (_Float16)-1032.0f};
 #pragma unroll
     for (int j = 0; j < NJ; j++) {
@@ -466,21 +466,32 @@ __device__ __forceinline__ void fsq_convert_v(unsigned v_lv, unsigned v_sc, unsi
     }
 }
 
+// Waves per group (= per compute unit): as many as LDS holds - each wave keeps two stages, half a tile of f16 V, its P^T and the mask
+// values of up to FSQ_MAX_TILES tiles.  A wave on its own is one dependent chain (reads, scores, soft-max, conversion, output);
+// more of them per compute unit is what keeps its vector ALUs and its transfers busy.
+constexpr int FSQ_MAX_TILES = 32;
+constexpr int FSQ_VF = 32 * FS_ROW;   // bytes of half a V tile as f16
 template <int TK, int TV>
-__global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream_q(fattn_args a, fsq_src ksrc, fsq_src vsrc, int tiles_per_wave, int n_tiles, int R) {
+constexpr int fsq_waves() { return TK == MI355_Q8_0 && TV == MI355_Q8_0 ? 3 : (TK == MI355_Q4_0 && TV == MI355_Q4_0 ? 5 : 4); }
+static int fsq_waves_rt(int tk, int tv) { return tk == MI355_Q8_0 && tv == MI355_Q8_0 ? 3 : (tk == MI355_Q4_0 && tv == MI355_Q4_0 ? 5 : 4); }
+constexpr int FSQ_TOTAL_GROUPS = 256;
+
+template <int TK, int TV>
+__global__ void __launch_bounds__((fsq_waves<TK, TV>() * 64), 1) k_fattn_dec_stream_q(fattn_args a, fsq_src ksrc, fsq_src vsrc, int tiles_per_wave, int n_tiles, int R) {
     typedef fsq_geo<TK> GK;
     typedef fsq_geo<TV> GV;
+    constexpr int NWV = fsq_waves<TK, TV>();
     constexpr int K_LV = FS_TILE * GK::ROW, V_LV = FS_TILE * GV::ROW;
     constexpr int OFF_V = K_LV, OFF_KS = K_LV + V_LV, OFF_VS = OFF_KS + FSQ_SCALES;
     constexpr int STAGE = OFF_VS + FSQ_SCALES;
     constexpr int CK = GK::CNT, CV = GV::CNT;   // transfers of the K / V part of a tile
-    __shared__ __attribute__((aligned(1024))) uint8_t ring_buf[FS_WAVES * 2 * STAGE];
-    __shared__ __attribute__((aligned(1024))) uint8_t vf_buf[FS_WAVES * FS_KT];   // the wave's V tile as f16
-    __shared__ __attribute__((aligned(16))) unsigned short pbuf[FS_WAVES][4][FS_TILE];
-    __shared__ __attribute__((aligned(16))) unsigned short mbuf[FS_WAVES][FS_MAX_TILES * FS_TILE];
+    __shared__ __attribute__((aligned(1024))) uint8_t ring_buf[NWV * 2 * STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t vf_buf[NWV * FSQ_VF];   // half of the wave's V tile as f16
+    __shared__ __attribute__((aligned(16))) unsigned short pbuf[NWV][4][FS_TILE];
+    __shared__ __attribute__((aligned(16))) unsigned short mbuf[NWV][FSQ_MAX_TILES * FS_TILE];
     asm volatile("" ::"v"((void *)ring_buf), "v"((void *)vf_buf) : "memory");
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int split = (int)blockIdx.x * FS_WAVES + wave;
+    const int split = (int)blockIdx.x * (int)(blockDim.x >> 6) + wave;   // the launch may give a group fewer than NWV waves
     const int64_t hk = blockIdx.y;
     const int t_begin = split * tiles_per_wave;
     const int t_end = t_begin + tiles_per_wave < n_tiles ? t_begin + tiles_per_wave : n_tiles;
@@ -586,9 +597,9 @@ __global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream_q(fattn_a
     {
         const unsigned short *mrow = (const unsigned short *)a.mask;
         const bool wide = ((uintptr_t)mrow & 15) == 0;
-        u32x4 mc[FS_MAX_TILES / 8];
+        u32x4 mc[FSQ_MAX_TILES / 8];
 #pragma unroll
-        for (int it = 0; it < FS_MAX_TILES / 8; it++) {
+        for (int it = 0; it < FSQ_MAX_TILES / 8; it++) {
             const int j = it * 64 + lane;
             const int64_t c = c_begin + (int64_t)j * 8;
             mc[it] = u32x4{0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u};   // -inf
@@ -605,7 +616,7 @@ __global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream_q(fattn_a
             }
         }
 #pragma unroll
-        for (int it = 0; it < FS_MAX_TILES / 8; it++) {
+        for (int it = 0; it < FSQ_MAX_TILES / 8; it++) {
             const int j = it * 64 + lane;
             if (j * 8 < n * FS_TILE) *(u32x4 *)(mw + j * 8) = mc[it];
         }
@@ -613,7 +624,7 @@ __global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream_q(fattn_a
     // From here on LDS is read and written through inline assembly with waits placed by hand (see k_fattn_dec_stream).
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     const unsigned ring_lds = (unsigned)(uintptr_t)(void __attribute__((address_space(3))) *)ring;
-    const unsigned vf_lds = (unsigned)(uintptr_t)(void __attribute__((address_space(3))) *)(vf_buf + wave * FS_KT);
+    const unsigned vf_lds = (unsigned)(uintptr_t)(void __attribute__((address_space(3))) *)(vf_buf + wave * FSQ_VF);
     const unsigned k_lane = TK == MI355_Q8_0 ? (unsigned)lane * 128u + ((((unsigned)lane >> 1) & 7u) << 4) : (unsigned)lane * 64u + ((((unsigned)lane >> 2) & 3u) << 4);
     const unsigned m_lane = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned short *)mw + (unsigned)lane * 2;
     const unsigned p_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned short *)&pbuf[wave][0][0];
@@ -644,10 +655,13 @@ __global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream_q(fattn_a
         if (t + 2 < n) FS_WAIT_VM(CK + CV + CK);
         else if (t + 1 < n) FS_WAIT_VM(CK + CV);
         else FS_WAIT_VM(0);
+        // the tile's V in two halves of 32 cells through the wave's 8 KiB of f16 rows
         fsq_convert_v<TV>(sb + (unsigned)OFF_V, sb + (unsigned)OFF_VS, vf_lds, lane);
+        fs_output<8>(vf_lds + fs_v_lane(lane), p_rd, S);
+        fsq_convert_v<TV>(sb + (unsigned)(OFF_V + 32 * GV::ROW), sb + (unsigned)(OFF_VS + 32 * 8), vf_lds, lane);
         // the levels are in registers or already converted: the V part of the stage may be overwritten
         if (t + 2 < n) issue(t + 2, st, 1);
-        fs_output(vf_lds + fs_v_lane(lane), p_rd, S);
+        fs_output<8>(vf_lds + fs_v_lane(lane), p_rd + 64, S);
     }
 
 #pragma unroll
@@ -835,16 +849,22 @@ int launch_fattn_dec_stream_q(hipStream_t s, fattn_args &a, int64_t D, size_t ws
     fsq_src ks, vs;
     if (!fsq_describe(a.type_k, a.kq, a.Hkv, a.k_nb1, ks) || !fsq_describe(a.type_v, a.vq, a.Hkv, a.v_nb1, vs)) return 1;
     const int64_t n_tiles = (a.Nkv + FS_TILE - 1) / FS_TILE;
-    int64_t waves_per_head = FS_TOTAL_WAVES / a.Hkv;
-    if (waves_per_head < FS_WAVES) waves_per_head = FS_WAVES;
+    // Waves per group: all that LDS holds once every wave has a dozen tiles or more (131072 cells of 8 kv heads: 94.5 -> 82 us for
+    // Q8_0, 90 -> 73 us for Q4_0); with fewer tiles, two per group spread over more compute units are quicker (32768 cells: 34 us
+    // against 39 us).
+    int nwv = fsq_waves_rt(a.type_k, a.type_v);
+    if (n_tiles * a.Hkv < (int64_t)FSQ_TOTAL_GROUPS * nwv * 12) nwv = 2;
+    int64_t waves_per_head = (int64_t)FSQ_TOTAL_GROUPS * nwv / a.Hkv;
+    if (waves_per_head < nwv) waves_per_head = nwv;
     if (waves_per_head > 256) waves_per_head = 256;   // k_fattn_combine takes up to 256 splits
     int64_t tiles_per_wave = (n_tiles + waves_per_head - 1) / waves_per_head;
-    if (tiles_per_wave > FS_MAX_TILES) return 1;
+    if (tiles_per_wave > FSQ_MAX_TILES) return 1;
     int64_t n_splits = (n_tiles + tiles_per_wave - 1) / tiles_per_wave;
-    n_splits = (n_splits + FS_WAVES - 1) / FS_WAVES * FS_WAVES;   // whole groups; a wave without tiles writes an empty partial
+    n_splits = (n_splits + nwv - 1) / nwv * nwv;   // whole groups; a wave without tiles writes an empty partial
+    if (n_splits > 256) return 1;
     if (ws_bytes < (size_t)a.Hq * (size_t)n_splits * (size_t)(FS_D + 2) * sizeof(float)) return 1;
     a.n_splits = (int)n_splits;
-    const dim3 grid((unsigned)(n_splits / FS_WAVES), (unsigned)a.Hkv), block(FS_WAVES * 64);
+    const dim3 grid((unsigned)(n_splits / nwv), (unsigned)a.Hkv), block((unsigned)nwv * 64);
 #define MI355_FSQ_LAUNCH(TK, TV) MI355_LAUNCH((k_fattn_dec_stream_q<TK, TV>), grid, block, 0, s, a, ks, vs, (int)tiles_per_wave, (int)n_tiles, (int)R)
     if (a.type_k == MI355_Q8_0 && a.type_v == MI355_Q8_0) MI355_FSQ_LAUNCH(MI355_Q8_0, MI355_Q8_0);
     else if (a.type_k == MI355_Q8_0) MI355_FSQ_LAUNCH(MI355_Q8_0, MI355_Q4_0);

@@ -20,6 +20,17 @@ import struct
 
 import numpy as np
 
+
+def _package():
+    """the mi355 package, also when this file is run as a script (python llama.cpp_amd/mi355/gguf.py ...)"""
+    import importlib
+    import os
+    import sys
+    if __package__:
+        return importlib.import_module(__package__)
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    return importlib.import_module("mi355")
+
 F32, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL = 0, 2, 3, 6, 7, 8, 12, 13, 14, 20
 BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34),
          IQ4_NL: (32, 18)}
@@ -135,7 +146,7 @@ def quantized_tensor(ttype, shape, seed, device, std=0.02):
     """bytes of a tensor of `shape` (ggml order: shape[0] = row length) drawn from N(0, std) and quantized to ttype on the device
     with the reference quantizers' arithmetic (mi355_quantize_weights); rows are quantized in slices to bound memory"""
     import torch
-    from . import quantize_weights
+    quantize_weights = _package().quantize_weights
     k = shape[0]
     nrows = int(np.prod(shape[1:])) if len(shape) > 1 else 1
     gen = torch.Generator(device=device)
@@ -198,7 +209,7 @@ def write_model(path, n_layer=32, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=
                 f.write(b"\0" * ((-len(data)) % align))
                 continue
             if quantize_on is not None:
-                from . import load
+                load = _package().load
                 if load().mi355_quantize_weights_supported(ttype):
                     f.write(quantized_tensor(ttype, shape, seed + 7919 * (1 + len(name)) + sum(map(ord, name)), quantize_on))
                     f.write(b"\0" * ((-nbytes(ttype, shape)) % align))
