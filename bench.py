@@ -307,14 +307,15 @@ def sweep(kinds):
             del ks, vs
 
     if "fattn" in kinds or "fattn_kv" in kinds:
-        # decode over a quantized cache kept as llama.cpp's cache tensors are in a plug-in buffer ([cells][Hkv * D] rows in the device row
-        # layout), filled through the quantizing store; the blocks are read where they lie
+        # decode over a quantized cache kept as llama.cpp's cache tensors are in a plug-in buffer (a 1-D tensor of all cells in the device
+        # row layout: all levels first, all scales behind them), filled through the quantizing store; the blocks are read where they lie
         H, HK, D = 32, 8, 128
         for tname, t, bb in (("Q8_0", mi355.Q8_0, 34), ("Q4_0", mi355.Q4_0, 18)):
             for Nkv in (256, 1024, 4096, 32768, 131072):
                 nrot = max(2, min(16, (1 << 29) // (Nkv * HK * D)))
-                rb = HK * D // 32
-                row_bytes = rb * bb
+                cb = HK * D // 32              # blocks per cell
+                rb = Nkv * cb                  # blocks of the one row that is the whole cache
+                row_bytes = cb * bb
                 q = torch.randn(1, H, D, device=dev, generator=gen)
                 caches = []
                 for _ in range(2 * nrot):

@@ -475,6 +475,20 @@ int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, in
  *   so results agree to the tolerance of the op (NMSE 5e-4), not to the bit.  ws: 256-byte aligned, at least
  *   mi355_flash_attn_kv_ws_bytes.  D % 32 == 0. */
 int mi355_cpy_f32_quant(void *stream, int type, const float *src, void *dst_base, int64_t dst_first_block, int64_t dst_row_blocks, int64_t n);
+/* CPY between contiguous f32 rows and a VIEW of a Q8_0 / Q4_0 tensor whose rows start on block boundaries, in either direction: what
+ * the K-shift of a quantized cache does around its ROPE (llama_kv_cache_unified::build_rope_shift, src/llama-kv-cache.cpp: ggml_cast
+ * of the [head_dim, heads, cells] view of the cache to f32, ggml_rope_ext_inplace, ggml_cpy back; ggml-cpu.c:3519-3830 with the
+ * type's to_float / from_float).  f32: ne[0] x ne[1] x ne[2] x ne[3] contiguous floats; element (i0, i1, i2, i3) lies in block
+ * q_first_block + i0 / 32 + i1 * stride_blocks[0] + i2 * stride_blocks[1] + i3 * stride_blocks[2] of the tensor that owns the
+ * memory (q_base, q_row_blocks as in mi355_cpy_f32_quant).  to_f32 = 1 dequantizes (dequantize_row_q8_0 / q4_0), 0 quantizes
+ * (quantize_row_q8_0_ref / q4_0_ref).  ne[0] % 32 == 0. */
+/* CPY of n_blocks consecutive blocks (in plain ggml addressing) of a Q8_0 / Q4_0 tensor to consecutive blocks of another tensor of
+ * the same type - the row copies of build_defrag (src/llama.cpp:1215-1300) on a quantized cache; base / first_block / row_blocks
+ * per side as in mi355_cpy_f32_quant. */
+int mi355_cpy_quant_blocks(void *stream, int type, const void *src_base, int64_t src_first_block, int64_t src_row_blocks, void *dst_base,
+                           int64_t dst_first_block, int64_t dst_row_blocks, int64_t n_blocks);
+int mi355_cpy_quant_view(void *stream, int type, int to_f32, float *f32, void *q_base, int64_t q_first_block, int64_t q_row_blocks, const int64_t *ne,
+                         const int64_t *stride_blocks);
 size_t mi355_flash_attn_kv_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, int type_k, int type_v);
 int mi355_flash_attn_ext_kv(void *stream, const float *q, const void *k, int type_k, const void *k_base, int64_t k_row_blocks, const void *v,
                             int type_v, const void *v_base, int64_t v_row_blocks, const void *mask, float *dst, int64_t D, int64_t Nq, int64_t Nkv,

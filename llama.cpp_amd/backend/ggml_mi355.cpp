@@ -706,10 +706,22 @@ bool device_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
             const ggml_type dt = op->op == GGML_OP_CPY ? op->src[1]->type : op->type;
             const bool sf = st == GGML_TYPE_F32 || st == GGML_TYPE_F16, df = dt == GGML_TYPE_F32 || dt == GGML_TYPE_F16;
             if (op->op == GGML_OP_CPY && st == GGML_TYPE_F32 && (dt == GGML_TYPE_Q8_0 || dt == GGML_TYPE_Q4_0)) {
-                // the store into a quantized KV cache: contiguous f32 rows into consecutive blocks
+                // the store into a quantized KV cache (contiguous f32 rows into consecutive blocks) and the copy back after a K-shift
+                // (contiguous f32 rows into a view whose rows start on block boundaries)
                 const ggml_tensor * a = op->src[0], * d = op->src[1];
-                return ggml_is_contiguous(a) && ggml_is_contiguous(d) && a->ne[0] % 32 == 0 && ggml_nelements(a) == ggml_nelements(d) &&
-                       kv_operand_of(d).ok && base_aligned16(a);
+                if (!ggml_is_contiguous(a) || a->ne[0] % 32 != 0 || !kv_operand_of(d).ok || !base_aligned16(a)) return false;
+                return ggml_is_contiguous(d) ? ggml_nelements(a) == ggml_nelements(d) && d->ne[0] % 32 == 0 : ggml_are_same_shape(a, d);
+            }
+            if (op->op == GGML_OP_CPY && dt == GGML_TYPE_F32 && (st == GGML_TYPE_Q8_0 || st == GGML_TYPE_Q4_0)) {
+                // ggml_cast of a quantized cache view to f32 (the first step of its K-shift)
+                const ggml_tensor * a = op->src[0], * d = op->src[1];
+                return ggml_is_contiguous(d) && ggml_are_same_shape(a, d) && a->ne[0] % 32 == 0 && kv_operand_of(a).ok && base_aligned16(d);
+            }
+            if (op->op == GGML_OP_CPY && st == dt && (st == GGML_TYPE_Q8_0 || st == GGML_TYPE_Q4_0)) {
+                // consecutive blocks of a quantized tensor to consecutive blocks of another (the row copies of a cache defragmentation)
+                const ggml_tensor * a = op->src[0], * d = op->src[1];
+                return ggml_is_contiguous(a) && ggml_is_contiguous(d) && ggml_nelements(a) == ggml_nelements(d) && a->ne[0] % 32 == 0 && d->ne[0] % 32 == 0 &&
+                       kv_operand_of(a).ok && kv_operand_of(d).ok;
             }
             return (sf && df) || (st == GGML_TYPE_I32 && dt == GGML_TYPE_I32);
         }
@@ -729,7 +741,10 @@ bool device_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
         case GGML_OP_ROPE: {
             const int mode = ((const int32_t *) op->op_params)[2];
             if (mode != 0 && mode != GGML_ROPE_TYPE_NEOX) return false;   // no mrope / vision
-            if (!f32_rows(op->src[0]) || !f32_rows(op) || op->src[1]->type != GGML_TYPE_I32) return false;
+            // f32, or f16 onto f16 (the in-place rotation of an f16 K cache when the context is shifted)
+            const bool f16 = op->src[0]->type == GGML_TYPE_F16 && op->type == GGML_TYPE_F16 && op->src[0]->nb[0] == sizeof(ggml_fp16_t) &&
+                             op->nb[0] == sizeof(ggml_fp16_t);
+            if (!(f16 || (f32_rows(op->src[0]) && f32_rows(op))) || op->src[1]->type != GGML_TYPE_I32) return false;
             if (op->src[2] && op->src[2]->type != GGML_TYPE_F32) return false;
             return op->src[0]->ne[0] % 2 == 0;
         }
@@ -840,12 +855,31 @@ void compute_node(backend_ctx * ctx, ggml_tensor * node) {
         } break;
         case GGML_OP_CPY: {
             const ggml_tensor * dt = node->src[1];
-            if (dt->type == GGML_TYPE_Q8_0 || dt->type == GGML_TYPE_Q4_0) {
-                const kv_operand o = kv_operand_of(dt);
+            const ggml_tensor * st = node->src[0];
+            if (st->type == dt->type && (st->type == GGML_TYPE_Q8_0 || st->type == GGML_TYPE_Q4_0)) {   // block ranges, each side in its owner's layout
+                const kv_operand a = kv_operand_of(st), d = kv_operand_of(dt);
+                GGML_ASSERT(a.ok && d.ok);
+                const ptrdiff_t bb = (ptrdiff_t) ggml_type_size(st->type);
+                MI355_K_OK(mi355_cpy_quant_blocks(s, to_mi355_type(st->type), a.base, (int64_t) (((const char *) a.p - (const char *) a.base) / bb), a.row_blocks,
+                                                  (void *) d.base, (int64_t) (((const char *) d.p - (const char *) d.base) / bb), d.row_blocks,
+                                                  ggml_nelements(dt) / 32));
+                break;
+            }
+            const bool to_quant = dt->type == GGML_TYPE_Q8_0 || dt->type == GGML_TYPE_Q4_0;
+            const bool from_quant = st->type == GGML_TYPE_Q8_0 || st->type == GGML_TYPE_Q4_0;
+            if (to_quant || from_quant) {
+                const ggml_tensor * qt = to_quant ? dt : st, * ft = to_quant ? st : dt;
+                const kv_operand o = kv_operand_of(qt);
                 GGML_ASSERT(o.ok);
-                const int64_t first = (int64_t) (((const char *) o.p - (const char *) o.base) / (ptrdiff_t) ggml_type_size(dt->type));
-                MI355_K_OK(mi355_cpy_f32_quant(s, to_mi355_type(dt->type), (const float *) node->src[0]->data, (void *) o.base, first, o.row_blocks,
-                                               ggml_nelements(dt)));
+                const int64_t bb = (int64_t) ggml_type_size(qt->type);
+                const int64_t first = (int64_t) (((const char *) o.p - (const char *) o.base) / (ptrdiff_t) bb);
+                if (to_quant && ggml_is_contiguous(qt)) {   // consecutive blocks, whatever the two shapes are
+                    MI355_K_OK(mi355_cpy_f32_quant(s, to_mi355_type(qt->type), (const float *) ft->data, (void *) o.base, first, o.row_blocks, ggml_nelements(qt)));
+                } else {
+                    const int64_t strides[3] = {(int64_t) qt->nb[1] / bb, (int64_t) qt->nb[2] / bb, (int64_t) qt->nb[3] / bb};
+                    MI355_K_OK(mi355_cpy_quant_view(s, to_mi355_type(qt->type), from_quant ? 1 : 0, (float *) ft->data, (void *) o.base, first, o.row_blocks,
+                                                    qt->ne, strides));
+                }
                 break;
             }
             mi355_tensor a = desc(node->src[0]), d = desc(node->src[1]);

@@ -46,11 +46,12 @@ __device__ __forceinline__ float dot8_f16(const u32x4 &a, const u32x4 &b) {
 
 
 // Where this lane's eight elements d0 .. d0 + 7 of the (cell 0, kv head hk) row of a quantized operand lie: their levels (Q4_0: the
-// eight bytes whose low or high nibbles - shift 0 or 4 - they are) and the block's f16 scale; a cell further on is nb1 bytes
-// further on in both.
+// eight bytes whose low or high nibbles - shift 0 or 4 - they are) and the block's f16 scale; a cell further on they are lv_step /
+// sc_step bytes further on.
 struct kv_lane {
     const uint8_t *lv, *sc;
     int shift;
+    int64_t lv_step, sc_step;
 };
 __device__ __forceinline__ kv_lane kv_lane_of(const kv_src &s, int type, int64_t hk, int d0) {
     const int BB = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES, LB = type == MI355_Q8_0 ? 32 : 16;
@@ -69,13 +70,15 @@ __device__ __forceinline__ kv_lane kv_lane_of(const kv_src &s, int type, int64_t
     }
     o.lv = lv + (type == MI355_Q8_0 ? j : (j & 15));
     o.shift = (type == MI355_Q4_0 && j >= 16) ? 4 : 0;
+    o.lv_step = s.cell_lv;
+    o.sc_step = s.cell_sc;
     return o;
 }
 // the raw bytes of one cell's eight elements: levels in words 0 and 1, the scale's bits in word 2 (plain blocks are 2-byte aligned)
-__device__ __forceinline__ u32x4 kv_load8(const kv_lane &p, int64_t off) {
+__device__ __forceinline__ u32x4 kv_load8(const kv_lane &p, int64_t cell) {
     u32x2 w;
-    __builtin_memcpy(&w, p.lv + off, 8);
-    return u32x4{w[0], w[1], (u32)*(const unsigned short *)(p.sc + off), 0u};
+    __builtin_memcpy(&w, p.lv + cell * p.lv_step, 8);
+    return u32x4{w[0], w[1], (u32)*(const unsigned short *)(p.sc + cell * p.sc_step), 0u};
 }
 // d * level of the eight elements (dequantize_row_q8_0 / dequantize_row_q4_0, ggml-quants.c:255-273, 365-380)
 __device__ __forceinline__ void kv_values8(int type, const u32x4 &raw, int shift, float (&f)[8]) {
@@ -167,7 +170,7 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
     // quantized operands (wave-uniform choice): this lane's place in the rows of kv head hk
     const bool k_f16 = !QUANT || a.type_k == MI355_F16, v_f16 = !QUANT || a.type_v == MI355_F16;
-    kv_lane kl = {nullptr, nullptr, 0}, vl = {nullptr, nullptr, 0};
+    kv_lane kl = {nullptr, nullptr, 0, 0, 0}, vl = {nullptr, nullptr, 0, 0, 0};
     if (!k_f16 && active) kl = kv_lane_of(a.kq, a.type_k, hk, d0);
     if (!v_f16 && active) vl = kv_lane_of(a.vq, a.type_v, hk, d0);
 
@@ -193,8 +196,8 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
             kk[j] = u32x4{0, 0, 0, 0};
             vv[j] = u32x4{0, 0, 0, 0};
             if (valid[j] && active) {   // masked cells cost no K/V traffic
-                kk[j] = k_f16 ? load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2) : kv_load8(kl, c * (int64_t)a.k_nb1);
-                vv[j] = v_f16 ? load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2) : kv_load8(vl, c * (int64_t)a.v_nb1);
+                kk[j] = k_f16 ? load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2) : kv_load8(kl, c);
+                vv[j] = v_f16 ? load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2) : kv_load8(vl, c);
             }
         }
         float kd[U];   // quantized K: the levels as exact f16 values; their dot with q takes the block's scale afterwards

@@ -5,19 +5,22 @@
 
 namespace mi355 {
 
-// A Q8_0 / Q4_0 operand of the vector kernel, read block by block where it lies (no f16 copy).  Block g of the owning tensor sits
-// at g * block bytes (row_blocks == 0: plain ggml blocks, the f16 scale in front of the levels) or, for a tensor in the device row
-// layout, in row g / row_blocks at position g % row_blocks (the levels of a row first, its scales behind them).  The (cell, head)
-// row starts at block first_block + cell * (nb1 / block bytes) + head * head_blocks; nb1 is a whole number of rows of the owner.
+// A Q8_0 / Q4_0 operand read block by block where it lies (no f16 copy).  Block g of the owning tensor sits at g * block bytes
+// (row_blocks == 0: plain ggml blocks, the f16 scale in front of the levels) or, for a tensor in the device row layout, in row
+// g / row_blocks at position g % row_blocks (the levels of a row first, its scales behind them).  The (cell 0, head) row starts at
+// block first_block + head * head_blocks; a cell further on, the levels lie cell_lv bytes and the scales cell_sc bytes further on:
+// both nb1 for plain blocks and where a cell's stride is a whole number of the owner's rows; (blocks per cell) * 32 or 16 and
+// (blocks per cell) * 2 where all cells lie in ONE row of the owner (llama.cpp's cache tensors are 1-D: one row of all cells).
 struct kv_src {
     const uint8_t *base;
     int64_t first_block, row_blocks, head_blocks;
+    int64_t cell_lv, cell_sc;
 };
 
 struct fattn_args {
     const uint8_t *q, *k, *v, *mask;
     int type_k = MI355_F16, type_v = MI355_F16;   // k_fattn_vec only: MI355_Q8_0 / MI355_Q4_0 operands are described by kq / vq
-    kv_src kq = {nullptr, 0, 0, 0}, vq = {nullptr, 0, 0, 0};
+    kv_src kq = {nullptr, 0, 0, 0, 0, 0}, vq = {nullptr, 0, 0, 0, 0, 0};
     float *dst;      // [D, Hq, Nq]
     int8_t *act_q;   // optional: Q8_1 of dst rows (Hq*D elements per query) in the split activation layout
     act_ds *act_s;

@@ -312,8 +312,9 @@ __global__ void __launch_bounds__(FS_WAVES * 64, 1) k_fattn_dec_stream(fattn_arg
 // f16 operations on exact values until the one rounding of the product - and writes them row-major into its own 16 KiB of LDS,
 // where fs_output finds what it finds for an f16 cache.
 struct fsq_src {
-    const uint8_t *lv, *sc;   // levels / scales of (cell 0, kv head 0); a cell further on is nb1 bytes further on in both
+    const uint8_t *lv, *sc;   // levels / scales of (cell 0, kv head 0)
     int64_t head_lv, head_sc; // bytes from one kv head to the next
+    int64_t cell_lv, cell_sc; // bytes from one cell to the next
 };
 template <int T>
 struct fsq_geo {
@@ -511,13 +512,13 @@ __global__ void __launch_bounds__((fsq_waves<TK, TV>() * 64), 1) k_fattn_dec_str
         const unsigned p = (unsigned)lane;
         if constexpr (TK == MI355_Q8_0) {
 #pragma unroll
-            for (int e = 0; e < 2; e++) koff[e] = (p >> 3) * (unsigned)a.k_nb1 + (((p & 7) ^ ((4 * e + (p >> 4)) & 7)) << 4);
+            for (int e = 0; e < 2; e++) koff[e] = (p >> 3) * (unsigned)ksrc.cell_lv + (((p & 7) ^ ((4 * e + (p >> 4)) & 7)) << 4);
         } else {
-            koff[0] = koff[1] = (p >> 2) * (unsigned)a.k_nb1 + (((p & 3) ^ ((p >> 4) & 3)) << 4);
+            koff[0] = koff[1] = (p >> 2) * (unsigned)ksrc.cell_lv + (((p & 3) ^ ((p >> 4) & 3)) << 4);
         }
-        voff = TV == MI355_Q8_0 ? (p >> 3) * (unsigned)a.v_nb1 + ((p & 7) << 4) : (p >> 2) * (unsigned)a.v_nb1 + ((p & 3) << 4);
-        ksoff = (p >> 1) * (unsigned)a.k_nb1 + ((p & 1) << 2);
-        vsoff = (p >> 1) * (unsigned)a.v_nb1 + ((p & 1) << 2);
+        voff = TV == MI355_Q8_0 ? (p >> 3) * (unsigned)vsrc.cell_lv + ((p & 7) << 4) : (p >> 2) * (unsigned)vsrc.cell_lv + ((p & 3) << 4);
+        ksoff = (p >> 1) * (unsigned)ksrc.cell_sc + ((p & 1) << 2);
+        vsoff = (p >> 1) * (unsigned)vsrc.cell_sc + ((p & 1) << 2);
     }
     auto dma16 = [&](const uint8_t *g, unsigned off, uint8_t *l) {   // g, l: wave-uniform
         asm volatile("" : "+v"(off));
@@ -531,18 +532,18 @@ __global__ void __launch_bounds__((fsq_waves<TK, TV>() * 64), 1) k_fattn_dec_str
     auto issue = [&](int t, int st, int which) {
         const int64_t c0 = c_begin + (int64_t)t * FS_TILE;
         uint8_t *sb = ring + st * STAGE;
-        const int64_t nb1 = which ? (int64_t)a.v_nb1 : (int64_t)a.k_nb1;
+        const int64_t nb_lv = which ? vsrc.cell_lv : ksrc.cell_lv, nb_sc = which ? vsrc.cell_sc : ksrc.cell_sc;
         const uint8_t *lvp = which ? v_lv : k_lv, *scp = which ? v_sc : k_sc;
         uint8_t *l_lv = sb + (which ? OFF_V : 0), *l_sc = sb + (which ? OFF_VS : OFF_KS);
         const int NT = which ? GV::NT : GK::NT, RPT = which ? GV::RPT : GK::RPT, CH = which ? GV::CH : GK::CH;
         if (c0 + FS_TILE <= a.Nkv) {
-            const uint8_t *g = lvp + c0 * nb1;
+            const uint8_t *g = lvp + c0 * nb_lv;
 #pragma unroll
             for (int i = 0; i < 8; i++)
-                if (i < NT) dma16(g + (int64_t)(RPT * i) * nb1, which ? voff : koff[i & 1], l_lv + i * 1024);
-            const uint8_t *gs = scp + c0 * nb1;
+                if (i < NT) dma16(g + (int64_t)(RPT * i) * nb_lv, which ? voff : koff[i & 1], l_lv + i * 1024);
+            const uint8_t *gs = scp + c0 * nb_sc;
             dma4(gs, which ? vsoff : ksoff, l_sc);
-            dma4(gs + 32 * nb1, which ? vsoff : ksoff, l_sc + 256);
+            dma4(gs + 32 * nb_sc, which ? vsoff : ksoff, l_sc + 256);
         } else {   // the cache's last, partial tile: rows past the end repeat the last cell (their scores are discarded)
 #pragma unroll
             for (int i = 0; i < 8; i++)
@@ -551,14 +552,14 @@ __global__ void __launch_bounds__((fsq_waves<TK, TV>() * 64), 1) k_fattn_dec_str
                     int64_t cell = c0 + row;
                     if (cell >= a.Nkv) cell = a.Nkv - 1;
                     const int swz = which ? 0 : (TK == MI355_Q8_0 ? (row >> 1) & 7 : (row >> 2) & 3);
-                    const uint8_t *g = lvp + cell * nb1 + ((pos ^ swz) << 4);
+                    const uint8_t *g = lvp + cell * nb_lv + ((pos ^ swz) << 4);
                     __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)g, (void __attribute__((address_space(3))) *)(l_lv + i * 1024), 16, 0, 0);
                 }
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 int64_t cell = c0 + 32 * i + (lane >> 1);
                 if (cell >= a.Nkv) cell = a.Nkv - 1;
-                const uint8_t *g = scp + cell * nb1 + ((lane & 1) << 2);
+                const uint8_t *g = scp + cell * nb_sc + ((lane & 1) << 2);
                 __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)g, (void __attribute__((address_space(3))) *)(l_sc + i * 256), 4, 0, 0);
             }
         }
@@ -826,17 +827,19 @@ int launch_fattn_dec_stream(hipStream_t s, fattn_args &a, int64_t D, size_t ws_b
 
 // fsq_src of a kv_src in the device row layout; false when the operand does not have the shape the kernel moves (whole heads of four
 // blocks inside one row of the owner, levels 16-byte and scales 4-byte aligned)
-static bool fsq_describe(int type, const kv_src &q, int64_t Hkv, size_t nb1, fsq_src &o) {
+static bool fsq_describe(int type, const kv_src &q, fsq_src &o) {
     if (q.row_blocks <= 0 || q.base == nullptr) return false;
     const int64_t BB = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES, LB = type == MI355_Q8_0 ? 32 : 16;
     const int64_t row0 = q.first_block / q.row_blocks, b0 = q.first_block % q.row_blocks, RB = q.row_blocks * BB;
-    if (q.head_blocks < FS_D / 32 || b0 + (Hkv - 1) * q.head_blocks + FS_D / 32 > q.row_blocks) return false;
+    if (q.head_blocks < FS_D / 32) return false;   // (that heads and cells stay inside their rows of the owner was checked with kv_src)
     o.lv = q.base + row0 * RB + b0 * LB;
     o.sc = q.base + row0 * RB + q.row_blocks * LB + b0 * 2;
     o.head_lv = q.head_blocks * LB;
     o.head_sc = q.head_blocks * 2;
-    if (((uintptr_t)o.lv & 15) != 0 || (o.head_lv & 15) != 0 || (nb1 & 15) != 0 || ((uintptr_t)o.sc & 3) != 0 || (o.head_sc & 3) != 0) return false;
-    if (nb1 >= ((size_t)1 << 26)) return false;   // the per-lane offsets are 32-bit
+    o.cell_lv = q.cell_lv;
+    o.cell_sc = q.cell_sc;
+    if (((uintptr_t)o.lv & 15) != 0 || (o.head_lv & 15) != 0 || (o.cell_lv & 15) != 0 || ((uintptr_t)o.sc & 3) != 0 || (o.head_sc & 3) != 0 || (o.cell_sc & 3) != 0) return false;
+    if (o.cell_lv >= ((int64_t)1 << 26) || o.cell_sc >= ((int64_t)1 << 26)) return false;   // the per-lane offsets are 32-bit
     return true;
 }
 
@@ -847,7 +850,7 @@ int launch_fattn_dec_stream_q(hipStream_t s, fattn_args &a, int64_t D, size_t ws
     if (D != FS_D || a.Nq != 1 || R > 4 || a.Hkv > 65535 || a.ws == nullptr || (a.q_nb2 % 16) != 0) return 1;
     if ((a.type_k != MI355_Q8_0 && a.type_k != MI355_Q4_0) || (a.type_v != MI355_Q8_0 && a.type_v != MI355_Q4_0)) return 1;
     fsq_src ks, vs;
-    if (!fsq_describe(a.type_k, a.kq, a.Hkv, a.k_nb1, ks) || !fsq_describe(a.type_v, a.vq, a.Hkv, a.v_nb1, vs)) return 1;
+    if (!fsq_describe(a.type_k, a.kq, ks) || !fsq_describe(a.type_v, a.vq, vs)) return 1;
     const int64_t n_tiles = (a.Nkv + FS_TILE - 1) / FS_TILE;
     // Waves per group: all that LDS holds once every wave has a dozen tiles or more (131072 cells of 8 kv heads: 94.5 -> 82 us for
     // Q8_0, 90 -> 73 us for Q4_0); with fewer tiles, two per group spread over more compute units are quicker (32768 cells: 34 us

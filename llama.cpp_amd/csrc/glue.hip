@@ -224,11 +224,14 @@ struct rope_params {
     int n_dims, mode;
     float theta_scale, freq_scale, ext_factor, attn_factor, corr0, corr1;
 };
+// T: float, or _Float16 (the rotation of an f16 K cache in place when the context is shifted, llama_kv_cache K-shift graph:
+// values are widened, rotated in f32 and rounded back, ggml_compute_forward_rope_f16, ggml-cpu.c:9530-9700)
+template <typename T>
 __global__ void k_rope(tens src, const int32_t *__restrict__ pos, const float *__restrict__ ff, tens dst, rope_params p) {
     const int64_t row = blockIdx.x;   // over ne1*ne2*ne3
     const int64_t i2 = (row / src.ne[1]) % src.ne[2];
-    const float *x = (const float *)row_ptr(src, row);
-    float *y = (float *)row_ptr(dst, row);
+    const T *x = (const T *)row_ptr(src, row);
+    T *y = (T *)row_ptr(dst, row);
     const int64_t ne0 = src.ne[0];
     const bool neox = (p.mode & 2) != 0;
     for (int64_t pair = threadIdx.x; pair < ne0 / 2; pair += blockDim.x) {
@@ -249,10 +252,10 @@ __global__ void k_rope(tens src, const int32_t *__restrict__ pos, const float *_
         }
         const float c = cosf(theta) * mscale, s = sinf(theta) * mscale;
         const int64_t ia = neox ? pair : i0, ib = neox ? pair + p.n_dims / 2 : i0 + 1;
-        const float x0 = x[ia], x1 = x[ib];
+        const float x0 = (float)x[ia], x1 = (float)x[ib];
         // separately rounded products: the fused rope + KV-store kernel rotates with the same four roundings
-        y[ia] = sub_rn(mul_rn(x0, c), mul_rn(x1, s));
-        y[ib] = add_rn(mul_rn(x0, s), mul_rn(x1, c));
+        y[ia] = (T)sub_rn(mul_rn(x0, c), mul_rn(x1, s));
+        y[ib] = (T)add_rn(mul_rn(x0, s), mul_rn(x1, c));
     }
 }
 
@@ -488,7 +491,7 @@ int mi355_soft_max(void *stream, const mi355_tensor *src, const mi355_tensor *ma
 int mi355_rope(void *stream, const mi355_tensor *src, const int32_t *pos, const float *freq_factors,
                const mi355_tensor *dst, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
-    MI355_REQUIRE(src->type == MI355_F32 && dst->type == MI355_F32, "rope: f32 only");
+    MI355_REQUIRE((src->type == MI355_F32 || src->type == MI355_F16) && dst->type == src->type, "rope: f32 -> f32 or f16 -> f16 only");
     MI355_REQUIRE(same_shape(src, dst) && rows_dense(src) && rows_dense(dst), "rope: shapes differ or rows are strided");
     MI355_REQUIRE(mode == 0 || mode == 2, "rope: mode %d not supported (0 = adjacent pairs, 2 = NeoX)", mode);
     MI355_REQUIRE(n_dims > 0 && n_dims % 2 == 0 && n_dims <= src->ne[0] && src->ne[0] % 2 == 0, "rope: bad n_dims");
@@ -508,7 +511,8 @@ int mi355_rope(void *stream, const mi355_tensor *src, const int32_t *pos, const 
     const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
     p.corr0 = c0 > 0 ? c0 : 0;
     p.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
-    MI355_LAUNCH(k_rope, dim3((unsigned)nr), dim3(64), 0, (hipStream_t)stream, to_tens(src), pos, freq_factors, to_tens(dst), p);
+    if (src->type == MI355_F32) MI355_LAUNCH(k_rope<float>, dim3((unsigned)nr), dim3(64), 0, (hipStream_t)stream, to_tens(src), pos, freq_factors, to_tens(dst), p);
+    else MI355_LAUNCH(k_rope<_Float16>, dim3((unsigned)nr), dim3(64), 0, (hipStream_t)stream, to_tens(src), pos, freq_factors, to_tens(dst), p);
     return launch_status("k_rope");
 }
 

@@ -37,8 +37,21 @@ __device__ __forceinline__ void kv_block_offsets(const kv_place &p, int64_t g, i
     }
 }
 
+// A view of a quantized tensor whose rows start on block boundaries: element (i0, i1, i2, i3) of the contiguous f32 side lies in block
+// first_block + i0 / 32 + i1 * nbb[0] + i2 * nbb[1] + i3 * nbb[2] of the owner (strides in blocks).  ne0 == 0: consecutive blocks.
+struct kv_view {
+    int64_t ne0, ne1, ne2;
+    int64_t nbb[3];
+};
+__device__ __forceinline__ int64_t kv_view_block(const kv_view &vw, int64_t e0) {
+    if (vw.ne0 == 0) return e0 >> 5;
+    const int64_t i0 = e0 % vw.ne0, r = e0 / vw.ne0;
+    const int64_t i1 = r % vw.ne1, r2 = r / vw.ne1;
+    return (i0 >> 5) + i1 * vw.nbb[0] + (r2 % vw.ne2) * vw.nbb[1] + (r2 / vw.ne2) * vw.nbb[2];
+}
+
 // Eight lanes share one 32-element block (4 consecutive elements each); n is a multiple of 32.
-__global__ void __launch_bounds__(256) k_cpy_f32_q8_0(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, kv_place pl) {
+__global__ void __launch_bounds__(256) k_cpy_f32_q8_0(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, kv_place pl, kv_view vw) {
     const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const bool live = e0 < n;   // a block is all live or all dead
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
@@ -50,7 +63,7 @@ __global__ void __launch_bounds__(256) k_cpy_f32_q8_0(const float *__restrict__ 
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     if (!live) return;
     int64_t lv, sc;
-    kv_block_offsets<MI355_Q8_0>(pl, pl.first_block + (e0 >> 5), lv, sc);
+    kv_block_offsets<MI355_Q8_0>(pl, pl.first_block + kv_view_block(vw, e0), lv, sc);
     const int sub = (int)((e0 >> 2) & 7);
     int q[4];
 #pragma unroll
@@ -62,7 +75,7 @@ __global__ void __launch_bounds__(256) k_cpy_f32_q8_0(const float *__restrict__ 
     if (sub == 0) *(unsigned short *)(y + sc) = float_to_half_bits(d);
 }
 
-__global__ void __launch_bounds__(256) k_cpy_f32_q4_0(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, kv_place pl) {
+__global__ void __launch_bounds__(256) k_cpy_f32_q4_0(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n, kv_place pl, kv_view vw) {
     const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     const bool live = e0 < n;
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
@@ -106,12 +119,55 @@ __global__ void __launch_bounds__(256) k_cpy_f32_q4_0(const float *__restrict__ 
     const unsigned hi = (unsigned)__shfl_down((int)packed, 4, 8);
     if (!live || lane8 >= 4) return;
     int64_t lv, sc;
-    kv_block_offsets<MI355_Q4_0>(pl, pl.first_block + (e0 >> 5), lv, sc);
+    kv_block_offsets<MI355_Q4_0>(pl, pl.first_block + kv_view_block(vw, e0), lv, sc);
     const unsigned bytes = packed | (hi << 4);
     unsigned short *o = (unsigned short *)(y + lv + 4 * lane8);
     o[0] = (unsigned short)(bytes & 0xFFFFu);
     o[1] = (unsigned short)(bytes >> 16);
     if (lane8 == 0) *(unsigned short *)(y + sc) = (unsigned short)(float_to_half_bits(eighth) ^ 0x8000u);
+}
+
+// the other direction (ggml_cast of a quantized cache view to f32, the first step of its K-shift): y contiguous f32, four elements
+// per lane; dequantize_row_q8_0 / dequantize_row_q4_0 (ggml-quants.c:255-273, 365-380)
+template <int TYPE>
+__global__ void __launch_bounds__(256) k_cpy_quant_f32(const uint8_t *__restrict__ src, float *__restrict__ y, int64_t n, kv_place pl, kv_view vw) {
+    const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e0 >= n) return;
+    const int j = (int)((vw.ne0 == 0 ? e0 : e0 % vw.ne0) & 31);
+    int64_t lv, sc;
+    kv_block_offsets<TYPE>(pl, pl.first_block + kv_view_block(vw, e0), lv, sc);
+    const float d = half_bits_to_float(*(const unsigned short *)(src + sc));
+    f32x4 f;
+    if constexpr (TYPE == MI355_Q8_0) {
+        const unsigned short *p = (const unsigned short *)(src + lv + j);
+        const unsigned w = (unsigned)p[0] | ((unsigned)p[1] << 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = (float)(int8_t)((w >> (8 * i)) & 0xFF) * d;
+    } else {
+        const unsigned short *p = (const unsigned short *)(src + lv + (j & 15));
+        const unsigned w = ((unsigned)p[0] | ((unsigned)p[1] << 16)) >> (j >= 16 ? 4 : 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = (float)((int)((w >> (8 * i)) & 0xF) - 8) * d;
+    }
+    *(f32x4 *)(y + e0) = f;
+}
+
+// n consecutive blocks (in plain ggml addressing) of one quantized tensor to n consecutive blocks of another of the same type: the
+// row copies of a cache defragmentation (build_defrag, src/llama.cpp:1215-1300).  One thread per block; overlapping ranges are the
+// caller's business, as with ggml_cpy.
+template <int TYPE>
+__global__ void __launch_bounds__(256) k_cpy_quant_blocks(const uint8_t *__restrict__ src, kv_place sp, uint8_t *__restrict__ dst, kv_place dp, int64_t n) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= n) return;
+    constexpr int LB = TYPE == MI355_Q8_0 ? 32 : 16;
+    int64_t slv, ssc, dlv, dsc;
+    kv_block_offsets<TYPE>(sp, sp.first_block + g, slv, ssc);
+    kv_block_offsets<TYPE>(dp, dp.first_block + g, dlv, dsc);
+    const unsigned short *a = (const unsigned short *)(src + slv);
+    unsigned short *b = (unsigned short *)(dst + dlv);
+#pragma unroll
+    for (int i = 0; i < LB / 2; i++) b[i] = a[i];
+    *(unsigned short *)(dst + dsc) = *(const unsigned short *)(src + ssc);
 }
 
 // dst f16 [cell][head][D] = dequantized rows of a typed cache whose (cell, head) row starts at block cell * cb + head * hb (+ the
@@ -157,18 +213,28 @@ static size_t kv_image_bytes(int type, int64_t D, int64_t Nkv, int64_t Hkv) {
 // shared by all rows); below it the vector kernel dequantizes in its registers.
 constexpr int64_t KV_IMAGE_MIN_ROWS = 16;
 
-// describes a quantized operand for in-place reads; false when its rows do not start on block boundaries or a cell's stride is not
-// a whole number of the owner's rows (then the image path, with its own checks, takes it)
-static bool kv_in_place(int type, const void *p, const void *base, int64_t row_blocks, size_t nb1, size_t nb2, kv_src &o) {
-    const int64_t bb = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES;
+// describes a quantized operand for in-place reads (Nkv cells of Hkv heads of D elements); false when its rows do not start on block
+// boundaries or its cells are neither whole rows of the owner apart nor all inside one row of it (then the image path, with its own
+// checks, takes it)
+static bool kv_in_place(int type, const void *p, const void *base, int64_t row_blocks, size_t nb1, size_t nb2, int64_t D, int64_t Nkv, int64_t Hkv, kv_src &o) {
+    const int64_t bb = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES, lb = type == MI355_Q8_0 ? 32 : 16;
     if (base == nullptr) base = p;
     const int64_t off = (const char *)p - (const char *)base;
     if (((uintptr_t)base & 1) != 0 || off < 0 || off % bb != 0 || nb1 % bb != 0 || nb2 % bb != 0 || row_blocks < 0) return false;
-    if (row_blocks > 0 && ((int64_t)(nb1 / bb) % row_blocks) != 0) return false;
+    const int64_t cb = (int64_t)(nb1 / bb), hb = (int64_t)(nb2 / bb), first = off / bb;
     o.base = (const uint8_t *)base;
-    o.first_block = off / bb;
+    o.first_block = first;
     o.row_blocks = row_blocks;
-    o.head_blocks = (int64_t)(nb2 / bb);
+    o.head_blocks = hb;
+    if (row_blocks == 0 || cb % row_blocks == 0) {
+        if (row_blocks > 0 && first % row_blocks + (Hkv - 1) * hb + D / 32 > row_blocks) return false;   // a cell's heads within one row
+        o.cell_lv = o.cell_sc = (int64_t)nb1;
+        return true;
+    }
+    // all cells inside one row of the owner: levels and scales advance by their own strides
+    if (first % row_blocks + (Nkv - 1) * cb + (Hkv - 1) * hb + D / 32 > row_blocks) return false;
+    o.cell_lv = cb * lb;
+    o.cell_sc = cb * 2;
     return true;
 }
 
@@ -185,10 +251,49 @@ int mi355_cpy_f32_quant(void *stream, int type, const float *src, void *dst_base
                   "cpy_f32_quant: source must be 16-byte, destination 2-byte aligned");
     if (n == 0) return MI355_OK;
     const kv_place pl = {dst_first_block, dst_row_blocks};
+    const kv_view vw = {0, 1, 1, {0, 0, 0}};
     const dim3 grid((unsigned)((n / 4 + 255) / 256));
-    if (type == MI355_Q8_0) MI355_LAUNCH(k_cpy_f32_q8_0, grid, dim3(256), 0, (hipStream_t)stream, src, (uint8_t *)dst_base, n, pl);
-    else MI355_LAUNCH(k_cpy_f32_q4_0, grid, dim3(256), 0, (hipStream_t)stream, src, (uint8_t *)dst_base, n, pl);
+    if (type == MI355_Q8_0) MI355_LAUNCH(k_cpy_f32_q8_0, grid, dim3(256), 0, (hipStream_t)stream, src, (uint8_t *)dst_base, n, pl, vw);
+    else MI355_LAUNCH(k_cpy_f32_q4_0, grid, dim3(256), 0, (hipStream_t)stream, src, (uint8_t *)dst_base, n, pl, vw);
     return launch_status("k_cpy_f32_quant");
+}
+
+int mi355_cpy_quant_view(void *stream, int type, int to_f32, float *f32, void *q_base, int64_t q_first_block, int64_t q_row_blocks, const int64_t *ne,
+                         const int64_t *stride_blocks) {
+    MI355_REQUIRE(type == MI355_Q8_0 || type == MI355_Q4_0, "cpy_quant_view: type %d is not Q8_0 or Q4_0", type);
+    MI355_REQUIRE(ne != nullptr && stride_blocks != nullptr && ne[0] > 0 && ne[0] % 32 == 0 && ne[1] > 0 && ne[2] > 0 && ne[3] > 0,
+                  "cpy_quant_view: rows must be whole blocks of 32");
+    MI355_REQUIRE(stride_blocks[0] >= 0 && stride_blocks[1] >= 0 && stride_blocks[2] >= 0 && q_first_block >= 0 && q_row_blocks >= 0,
+                  "cpy_quant_view: negative strides");
+    MI355_REQUIRE(((uintptr_t)f32 & 15) == 0 && ((uintptr_t)q_base & 1) == 0, "cpy_quant_view: f32 side must be 16-byte, quantized side 2-byte aligned");
+    const int64_t n = ne[0] * ne[1] * ne[2] * ne[3];
+    MI355_REQUIRE(n / 1024 < 0x7fffffff, "cpy_quant_view: too many elements for one launch");
+    const kv_place pl = {q_first_block, q_row_blocks};
+    const kv_view vw = {ne[0], ne[1], ne[2], {stride_blocks[0], stride_blocks[1], stride_blocks[2]}};
+    const dim3 grid((unsigned)((n / 4 + 255) / 256));
+    hipStream_t s = (hipStream_t)stream;
+    if (to_f32) {
+        if (type == MI355_Q8_0) MI355_LAUNCH(k_cpy_quant_f32<MI355_Q8_0>, grid, dim3(256), 0, s, (const uint8_t *)q_base, f32, n, pl, vw);
+        else MI355_LAUNCH(k_cpy_quant_f32<MI355_Q4_0>, grid, dim3(256), 0, s, (const uint8_t *)q_base, f32, n, pl, vw);
+    } else {
+        if (type == MI355_Q8_0) MI355_LAUNCH(k_cpy_f32_q8_0, grid, dim3(256), 0, s, (const float *)f32, (uint8_t *)q_base, n, pl, vw);
+        else MI355_LAUNCH(k_cpy_f32_q4_0, grid, dim3(256), 0, s, (const float *)f32, (uint8_t *)q_base, n, pl, vw);
+    }
+    return launch_status("k_cpy_quant_view");
+}
+
+int mi355_cpy_quant_blocks(void *stream, int type, const void *src_base, int64_t src_first_block, int64_t src_row_blocks, void *dst_base,
+                           int64_t dst_first_block, int64_t dst_row_blocks, int64_t n_blocks) {
+    MI355_REQUIRE(type == MI355_Q8_0 || type == MI355_Q4_0, "cpy_quant_blocks: type %d is not Q8_0 or Q4_0", type);
+    MI355_REQUIRE(n_blocks >= 0 && n_blocks / 256 < 0x7fffffff && src_first_block >= 0 && dst_first_block >= 0 && src_row_blocks >= 0 && dst_row_blocks >= 0,
+                  "cpy_quant_blocks: bad block range");
+    MI355_REQUIRE(((uintptr_t)src_base & 1) == 0 && ((uintptr_t)dst_base & 1) == 0, "cpy_quant_blocks: tensors must be 2-byte aligned");
+    if (n_blocks == 0) return MI355_OK;
+    const kv_place sp = {src_first_block, src_row_blocks}, dp = {dst_first_block, dst_row_blocks};
+    const dim3 grid((unsigned)((n_blocks + 255) / 256));
+    if (type == MI355_Q8_0) MI355_LAUNCH(k_cpy_quant_blocks<MI355_Q8_0>, grid, dim3(256), 0, (hipStream_t)stream, (const uint8_t *)src_base, sp, (uint8_t *)dst_base, dp, n_blocks);
+    else MI355_LAUNCH(k_cpy_quant_blocks<MI355_Q4_0>, grid, dim3(256), 0, (hipStream_t)stream, (const uint8_t *)src_base, sp, (uint8_t *)dst_base, dp, n_blocks);
+    return launch_status("k_cpy_quant_blocks");
 }
 
 size_t mi355_flash_attn_kv_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t Hq, int64_t Hkv, int type_k, int type_v) {
@@ -227,9 +332,9 @@ int mi355_flash_attn_ext_kv(void *stream, const float *q, const void *k, int typ
     hipStream_t s = (hipStream_t)stream;
     // A few query rows (decode): the vector kernel reads the blocks where they lie, each byte of the cache once.
     if (Nq < KV_IMAGE_MIN_ROWS) {
-        kv_src kq = {nullptr, 0, 0, 0}, vq = {nullptr, 0, 0, 0};
-        const bool k_ok = type_k == MI355_F16 || kv_in_place(type_k, k, k_base, k_row_blocks, k_nb1, k_nb2, kq);
-        const bool v_ok = type_v == MI355_F16 || kv_in_place(type_v, v, v_base, v_row_blocks, v_nb1, v_nb2, vq);
+        kv_src kq = {nullptr, 0, 0, 0, 0, 0}, vq = {nullptr, 0, 0, 0, 0, 0};
+        const bool k_ok = type_k == MI355_F16 || kv_in_place(type_k, k, k_base, k_row_blocks, k_nb1, k_nb2, D, Nkv, Hkv, kq);
+        const bool v_ok = type_v == MI355_F16 || kv_in_place(type_v, v, v_base, v_row_blocks, v_nb1, v_nb2, D, Nkv, Hkv, vq);
         if (k_ok && v_ok)
             return fattn_vec_kv(s, q, k, type_k, kq, v, type_v, vq, mask, dst, D, Nq, Nkv, Hq, Hkv, q_nb1, q_nb2, k_nb1, k_nb2, v_nb1, v_nb2, mask_nb1, scale,
                                 max_bias, logit_softcap, ws, ws_bytes, act);

@@ -112,6 +112,8 @@ _SIGNATURES = {
     "mi355_flash_attn_ext_quant": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _sz, _sz,
                                           _sz, _f, _f, _f, _p, _sz, _p]),
     "mi355_cpy_f32_quant": (_int, [_p, _int, _p, _p, _i64, _i64, _i64]),
+    "mi355_cpy_quant_view": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _p]),
+    "mi355_cpy_quant_blocks": (_int, [_p, _int, _p, _i64, _i64, _p, _i64, _i64, _i64]),
     "mi355_flash_attn_kv_ws_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _int, _int]),
     "mi355_flash_attn_ext_kv": (_int, [_p, _p, _p, _int, _p, _i64, _p, _int, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz,
                                        _sz, _sz, _sz, _f, _f, _f, _p, _sz, _p]),

@@ -9,6 +9,12 @@
 // LLAMA_LOGITS_NO_MMAP=1 in the environment loads the file with read() instead of mmap (llama.cpp's --no-mmap), which is the
 // path that uploads through pinned buffers, set_tensor_async and events when the device offers them.
 //
+// LLAMA_LOGITS_SHIFT=<n> drops the first n cells of the sequence after the prompt and moves the rest down by n (what llama-cli's
+// context shift does: llama_kv_cache_seq_rm + llama_kv_cache_seq_add + llama_kv_cache_update, which runs the K-shift graph -
+// ROPE in place on an f16 cache, cast to f32 / ROPE / copy back on a quantized one) before the decoded tokens.
+// LLAMA_LOGITS_DEFRAG=<n> instead removes n cells from the middle of the sequence after the prompt and asks for a defragmentation
+// (llama_kv_cache_defrag + llama_kv_cache_update: build_defrag's row copies inside the K and V caches).
+//
 // Tokens are (7 i + 3) mod n_vocab.  Output: float32 rows of n_vocab logits, one for the last prompt token and one per
 // decoded token (the token ids are fixed, the logits are not fed back).
 #include "ggml-backend.h"
@@ -56,6 +62,20 @@ int main(int argc, char ** argv) {
     for (int i = 0; i < n_prompt; i++) toks[i] = (7 * i + 3) % n_vocab;
     if (llama_decode(ctx, llama_batch_get_one(toks.data(), n_prompt)) != 0) return 1;
     fwrite(llama_get_logits_ith(ctx, -1), sizeof(float), n_vocab, f);
+    if (const char * sh = getenv("LLAMA_LOGITS_SHIFT")) {
+        const int n_discard = atoi(sh);
+        if (n_discard <= 0 || n_discard >= n_prompt) return 2;
+        llama_kv_cache_seq_rm(ctx, 0, 0, n_discard);
+        llama_kv_cache_seq_add(ctx, 0, n_discard, n_prompt, -n_discard);
+        llama_kv_cache_update(ctx);
+    }
+    if (const char * df = getenv("LLAMA_LOGITS_DEFRAG")) {
+        const int n_hole = atoi(df);
+        if (n_hole <= 0 || 2 * n_hole >= n_prompt) return 2;
+        llama_kv_cache_seq_rm(ctx, 0, n_hole, 2 * n_hole);
+        llama_kv_cache_defrag(ctx);
+        llama_kv_cache_update(ctx);
+    }
     for (int i = 0; i < n_decode; i++) {
         llama_token t = (7 * (n_prompt + i) + 3) % n_vocab;
         if (llama_decode(ctx, llama_batch_get_one(&t, 1)) != 0) return 1;

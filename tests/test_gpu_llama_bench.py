@@ -53,9 +53,13 @@ def test_llama_bench_runs_on_the_plugin(dev, tmp_path):
 LOGITS = os.path.join(ROOT, "oracle", "_ref", "llama_logits")
 
 
-def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None, cache=None, mmap=True):
+def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None, cache=None, mmap=True, shift=0, defrag=0):
     import numpy as np
     env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN, MI355_GRAPH_STATS="1")
+    if shift:
+        env["LLAMA_LOGITS_SHIFT"] = str(shift)
+    if defrag:
+        env["LLAMA_LOGITS_DEFRAG"] = str(defrag)
     if not mmap:
         env["LLAMA_LOGITS_NO_MMAP"] = "1"
     if not fusion:
@@ -198,6 +202,59 @@ def test_model_logits_quantized_kv_cache(dev, tmp_path, cache, n_prompt):
     # projections), a value on a rounding boundary lands on another level and moves by 1/8 of the block's range.  A short prompt
     # has few cells to average that over.  The op-level parity of the stores and of attention is in tests/test_gpu_kv_quant.py.
     assert orc.nmse(gpu, cpu) < (2e-2 if "q4_0" in cache else 2e-3)
+
+
+@pytest.mark.parametrize("cache", [None, ("q8_0", "q8_0"), ("q4_0", "q4_0")])
+def test_model_logits_after_context_shift(dev, tmp_path, cache):
+    """llama-cli's context shift (llama_kv_cache_seq_rm + seq_add + update): the K-shift graph of build_k_shift (src/llama.cpp:1167-1213)
+    runs on the plug-in - ROPE in place on the [head_dim, heads, cells] view of an f16 cache; for a quantized cache the cast of
+    that view to f32, ROPE, and the copy back - and the tokens decoded after the shift reproduce the reference CPU backend's logits."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / "small.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048)
+    cpu = _logits(model, 0, 60, 5, str(tmp_path / "cpu.bin"), cache=cache, shift=17)
+    gpu = _logits(model, 99, 60, 5, str(tmp_path / "gpu.bin"), cache=cache, shift=17)
+    unshifted = _logits(model, 99, 60, 5, str(tmp_path / "gpu0.bin"), cache=cache)
+    assert cpu.shape == gpu.shape and np.isfinite(gpu).all()
+    n_vocab = 2048
+    assert orc.nmse(gpu, cpu) < (2e-2 if cache and "q4_0" in cache else 2e-3)
+    # the shift changes what the decoded tokens see (the prompt's own logits, row 0, come before it)
+    assert np.array_equal(gpu[:n_vocab], unshifted[:n_vocab]) and orc.nmse(gpu[n_vocab:], unshifted[n_vocab:]) > 1e-3
+
+
+@pytest.mark.parametrize("cache", [None, ("q8_0", "q8_0"), ("q4_0", "q4_0")])
+def test_model_logits_after_defrag(dev, tmp_path, cache):
+    """cells removed from the middle of a sequence and the cache defragmented (build_defrag, src/llama.cpp:1215-1300: copies of whole
+    rows inside the K and V cache tensors - for a quantized cache copies between views of one quantized type) on the plug-in.  With
+    an f16 cache the tokens decoded afterwards reproduce the reference CPU backend's logits.  With a quantized cache the CPU backend
+    is no yardstick: its same-type contiguous copy (ggml_compute_forward_dup_same_cont, ggml-cpu.c:2875-2902) moves
+    nelements * type_size bytes, 32 times the blocks it was asked for, and overwrites the cells behind the destination; the
+    plug-in copies the blocks of the view, and is held to its own run with an f16 cache instead (same cells moved, only the cache's
+    precision differs)."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / "small.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048)
+    gpu = _logits(model, 99, 60, 5, str(tmp_path / "gpu.bin"), cache=cache, defrag=13)
+    whole = _logits(model, 99, 60, 5, str(tmp_path / "gpu0.bin"), cache=cache)
+    assert np.isfinite(gpu).all()
+    if cache is None:
+        cpu = _logits(model, 0, 60, 5, str(tmp_path / "cpu.bin"), defrag=13)
+        assert cpu.shape == gpu.shape and orc.nmse(gpu, cpu) < 2e-3
+    else:
+        f16 = _logits(model, 99, 60, 5, str(tmp_path / "gpu16.bin"), defrag=13)
+        f16_whole = _logits(model, 99, 60, 5, str(tmp_path / "gpu160.bin"))
+        assert orc.nmse(gpu, f16) < 3 * orc.nmse(whole, f16_whole) + 1e-3   # as close to the f16 cache's logits as without the defragmentation
+    assert orc.nmse(gpu[2048:], whole[2048:]) > 1e-3   # the removed cells are gone from what the decoded tokens see
 
 
 @pytest.mark.parametrize("n_prompt", [3, 48])
