@@ -392,6 +392,17 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
                         const int32_t *cells, const float *freq_factors, int64_t T, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
                         size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
                         float ext_factor, float attn_factor, float beta_fast, float beta_slow);
+/* The same launch with typed caches (what llm_build_kv_store builds with -ctk / -ctv q8_0, q4_0: CPY f32 -> Q8_0 / Q4_0,
+ * ggml_compute_forward_dup_f32, ggml-cpu.c:3519-3830, via quantize_row_q8_0_ref / quantize_row_q4_0_ref, ggml-quants.c:194-218, 39-72;
+ * bit-identical to mi355_cpy_f32_quant of the rotated rows).  For an f16 cache (type MI355_F16) kcache / k_a / k_b are the view's
+ * data, nb1 and nb2 as above; for MI355_Q8_0 / MI355_Q4_0 kcache is the data of the tensor that owns the cache memory, k_a the
+ * index (blocks of 32, plain ggml addressing) of cell 0's first block within it and k_b its blocks per row in the device row
+ * layout (0: plain ggml blocks); token t's rows go to blocks k_a + cells[t] * HK * D / 32 ...  Likewise for V.  A quantized
+ * cache takes mode 0 (adjacent pairs) and D % 32 == 0. */
+int mi355_rope_kv_store_typed(void *stream, float *q, const float *k, const float *v, int type_k, void *kcache, int64_t k_a, int64_t k_b, int type_v,
+                              void *vcache, int64_t v_a, int64_t v_b, const int32_t *pos, const int32_t *cells, const float *freq_factors, int64_t T,
+                              int64_t H, int64_t HK, int64_t D, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                              float ext_factor, float attn_factor, float beta_fast, float beta_slow);
 /* Up to three weight matrices on one quantized activation whose finished rows go through the nodes that follow the projections in
  * build_llama (src/llama.cpp:1514-1548; llm_build_kv_store :157-199): ROPE (ggml-cpu.c:9366-9549, adjacent-pair mode only) and / or
  * CPY to an f16 tensor such as a KV-cache view (ggml-cpu.c:3519-3830).  A wave owns output rows 2i and 2i+1, i.e. one rotation pair.
@@ -399,16 +410,22 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
  *   MI355_EPI_ROPE        dst f32 [B][dst_stride], rows = [head][head_dim]  rotated by pos[b]
  *   MI355_EPI_ROPE_CACHE  dst f16 at cells[b]*nb1 + head*nb2 + 2*d          rotated, then converted
  *   MI355_EPI_CACHE       dst f16 at cells[b]*nb1 + head*nb2 + 2*d          converted
+ *   MI355_EPI_ROPE_QCACHE / MI355_EPI_QCACHE   the same two with a Q8_0 / Q4_0 destination (CPY f32 -> quantized, ggml_compute_forward_dup_f32, ggml-cpu.c:3519-3830, via
+ *                         quantize_row_q8_0_ref / quantize_row_q4_0_ref, ggml-quants.c:194-218, 39-72; bit-identical to
+ *                         mi355_cpy_f32_quant of the rotated row): dst = data of the tensor that owns the cache memory, dst_stride =
+ *                         MI355_Q8_0 or MI355_Q4_0, nb1 = index (in blocks of 32, plain ggml addressing) of cell 0's first block
+ *                         within that tensor, nb2 = the owner's blocks per row when it is kept in the device row layout (0: plain
+ *                         ggml blocks); row b of the product becomes blocks nb1 + cells[b]*N/32 ... of the owner.  N % 32 == 0.
  * pos / cells: DEVICE int32 [B].  B <= 4; 16-byte aligned weight rows. */
-enum { MI355_EPI_STORE = 0, MI355_EPI_ROPE = 1, MI355_EPI_ROPE_CACHE = 2, MI355_EPI_CACHE = 3 };
+enum { MI355_EPI_STORE = 0, MI355_EPI_ROPE = 1, MI355_EPI_ROPE_CACHE = 2, MI355_EPI_CACHE = 3, MI355_EPI_ROPE_QCACHE = 4, MI355_EPI_QCACHE = 5 };
 typedef struct mi355_gemv_rope_mat {
     int          type;
     const void  *W;           /* N rows x K, device layout */
     int64_t      N;           /* a whole number of heads unless the epilogue is MI355_EPI_STORE */
     int          epilogue;
     void        *dst;
-    int64_t      dst_stride;  /* f32 elements between activation rows (STORE, ROPE) */
-    int64_t      nb1, nb2;    /* bytes per cell and per head (ROPE_CACHE, CACHE) */
+    int64_t      dst_stride;  /* f32 elements between activation rows (STORE, ROPE); the cache type (ROPE_QCACHE, QCACHE) */
+    int64_t      nb1, nb2;    /* bytes per cell and per head (ROPE_CACHE, CACHE); first block and blocks per row (ROPE_QCACHE, QCACHE) */
 } mi355_gemv_rope_mat;
 typedef struct mi355_rope_desc {
     const int32_t *pos;

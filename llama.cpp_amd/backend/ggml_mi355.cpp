@@ -1217,6 +1217,7 @@ qkv_window match_qkv_window(backend_ctx * ctx, const graph_walk & w, int first, 
         int out_index;
         mi355_gemv_rope_mat m;
         void * cache_base;          // cache stores that start at cell kv_head: the cache tensor's first byte
+        int64_t first_block0;       // ... of a quantized cache: the block index of its cell 0 within the tensor that owns the memory
     } ch[3];
     int n_ch = 0, last = first - 1;
     mi355_rope_desc rd;
@@ -1237,6 +1238,7 @@ qkv_window match_qkv_window(backend_ctx * ctx, const graph_walk & w, int first, 
             chain & c = ch[n_ch++];
             c.mm = t; c.out = t; c.out_index = k;
             c.cache_base = nullptr;
+            c.first_block0 = 0;
             c.m.type = to_mi355_type(t->src[0]->type);
             c.m.W = t->src[0]->data;
             c.m.N = t->ne[0];
@@ -1292,9 +1294,28 @@ qkv_window match_qkv_window(backend_ctx * ctx, const graph_walk & w, int first, 
             for (int q = 0; q < n_ch; q++)
                 if (t->src[0] == ch[q].out && (ch[q].m.epilogue == MI355_EPI_STORE || ch[q].m.epilogue == MI355_EPI_ROPE)) c = &ch[q];
             const ggml_tensor * d = t->src[1];
-            if (!c || !w.sole_use(c->out_index) || d->type != GGML_TYPE_F16 || !ggml_is_contiguous(d) || ggml_nelements(d) != c->m.N * B ||
+            const bool quant = d->type == GGML_TYPE_Q8_0 || d->type == GGML_TYPE_Q4_0;
+            if (!c || !w.sole_use(c->out_index) || (d->type != GGML_TYPE_F16 && !quant) || !ggml_is_contiguous(d) || ggml_nelements(d) != c->m.N * B ||
                 ((uintptr_t) d->data & 1) != 0)
                 break;
+            if (quant) {   // Q8_0 / Q4_0 cache: the launch quantizes the row's blocks where the CPY node would
+                const kv_operand o = kv_operand_of(d);
+                if (!o.ok || c->m.N % 32 != 0 || ((uintptr_t) o.base & 1) != 0) break;
+                const ptrdiff_t bb = (ptrdiff_t) ggml_type_size(d->type);
+                c->m.epilogue = c->m.epilogue == MI355_EPI_ROPE ? MI355_EPI_ROPE_QCACHE : MI355_EPI_QCACHE;
+                c->m.dst = (void *) o.base;
+                c->m.dst_stride = to_mi355_type(d->type);
+                c->m.nb1 = (int64_t) (((const char *) o.p - (const char *) o.base) / bb);   // with rd.cells = iota: row b goes b * N / 32 blocks further
+                c->m.nb2 = o.row_blocks;
+                c->out = nullptr;
+                if (ctx->kv_head >= 0 && d->view_src && d->view_src->data &&
+                    (const char *) d->data - (const char *) d->view_src->data == (ptrdiff_t) (ctx->kv_head * (c->m.N / 32) * bb)) {
+                    c->cache_base = d->view_src->data;
+                    c->first_block0 = (int64_t) (((const char *) d->view_src->data - (const char *) o.base) / bb);
+                }
+                last = k;
+                continue;
+            }
             c->m.epilogue = c->m.epilogue == MI355_EPI_ROPE ? MI355_EPI_ROPE_CACHE : MI355_EPI_CACHE;
             c->m.dst = d->data;
             c->m.dst_stride = 0;
@@ -1317,11 +1338,12 @@ qkv_window match_qkv_window(backend_ctx * ctx, const graph_walk & w, int first, 
     }
     bool heads_ok = true;
     int n_base = 0;
+    auto quant_store = [](const mi355_gemv_rope_mat & m) { return m.epilogue == MI355_EPI_ROPE_QCACHE || m.epilogue == MI355_EPI_QCACHE; };
     for (int q = 0; q < n_ch; q++) {
         win.mats[q] = ch[q].m;
         if (win.mats[q].epilogue != MI355_EPI_STORE) heads_ok = heads_ok && win.mats[q].N % rd.head_dim == 0;
-        if (win.mats[q].epilogue == MI355_EPI_ROPE_CACHE || win.mats[q].epilogue == MI355_EPI_CACHE) {
-            win.mats[q].nb2 = rd.head_dim * 2;
+        if (win.mats[q].epilogue == MI355_EPI_ROPE_CACHE || win.mats[q].epilogue == MI355_EPI_CACHE) win.mats[q].nb2 = rd.head_dim * 2;
+        if (win.mats[q].epilogue >= MI355_EPI_ROPE_CACHE) {
             win.n_store++;
             if (ch[q].cache_base) n_base++;
         }
@@ -1330,8 +1352,11 @@ qkv_window match_qkv_window(backend_ctx * ctx, const graph_walk & w, int first, 
     // Cache stores that all start at cell kv_head address the cache tensor through the device-side cell list instead
     // of through the view's own address, so the launch's arguments do not change from token to token.
     if (win.n_store > 0 && n_base == win.n_store) {
-        for (int q = 0; q < n_ch; q++)
-            if (ch[q].cache_base) win.mats[q].dst = ch[q].cache_base;
+        for (int q = 0; q < n_ch; q++) {
+            if (!ch[q].cache_base) continue;
+            if (quant_store(win.mats[q])) win.mats[q].nb1 = ch[q].first_block0;
+            else win.mats[q].dst = ch[q].cache_base;
+        }
         rd.cells = ctx->cells;
         win.redirect = true;
     }
@@ -1345,6 +1370,7 @@ qkv_window match_qkv_window(backend_ctx * ctx, const graph_walk & w, int first, 
 void note_window_writes(backend_ctx * ctx, const qkv_window & win, int64_t B) {
     if (win.redirect) ctx->kv_redirected += win.n_store;
     for (int q = 0; q < win.n_ch; q++) {
+        if (win.mats[q].epilogue >= MI355_EPI_ROPE_QCACHE) continue;   // a quantized cache is never the source of a cached activation
         const bool f32_out = win.mats[q].epilogue == MI355_EPI_STORE || win.mats[q].epilogue == MI355_EPI_ROPE;
         ctx->note_write(win.mats[q].dst, (size_t) win.mats[q].N * (size_t) B * (f32_out ? sizeof(float) : 2));
     }
@@ -1447,8 +1473,12 @@ prefill_qkv match_prefill_qkv(const graph_walk & w, int i) {
     const ggml_tensor * rq = w.nodes[j1], * mk = w.nodes[j2], * rk = w.nodes[j3], * mv = w.nodes[j4], * ck = w.nodes[j5], * cv = w.nodes[j6];
     auto store_ok = [&](const ggml_tensor * c, const ggml_tensor * src) {
         const ggml_tensor * d = c->src[1];
-        return c->op == GGML_OP_CPY && c->src[0] == src && d->type == GGML_TYPE_F16 && ggml_is_contiguous(d) && ggml_nelements(d) == ggml_nelements(src) &&
-               ((uintptr_t) d->data & 1) == 0;
+        if (c->op != GGML_OP_CPY || c->src[0] != src || !ggml_is_contiguous(d) || ggml_nelements(d) != ggml_nelements(src) || ((uintptr_t) d->data & 1) != 0)
+            return false;
+        if (d->type == GGML_TYPE_F16) return true;
+        // a Q8_0 / Q4_0 cache: whole blocks per head, adjacent-pair rotation (the launch quantizes 16 lanes x 2 elements per block)
+        const int32_t * q = (const int32_t *) rq->op_params;
+        return (d->type == GGML_TYPE_Q8_0 || d->type == GGML_TYPE_Q4_0) && kv_operand_of(d).ok && rq->ne[0] % 32 == 0 && q[2] == 0;
     };
     if (!store_ok(ck, rk) || !store_ok(cv, mv)) return p;
     // one set of rope parameters, positions and frequency factors; k and v heads of q's size
@@ -1503,10 +1533,20 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             memcpy(&beta_fast, op + 9, sizeof(float));
             memcpy(&beta_slow, op + 10, sizeof(float));
             const int64_t D = rq->ne[0], H = rq->ne[1], HK = p.rk->ne[1], T = rq->ne[2];
-            MI355_K_OK(mi355_rope_kv_store(s, (float *) rq->data, (const float *) p.rk->data, (const float *) p.mv->data, p.ck->src[1]->data, p.cv->src[1]->data,
-                                           (const int32_t *) rq->src[1]->data, ctx->iota, rq->src[2] ? (const float *) rq->src[2]->data : nullptr, T, H, HK, D,
-                                           (size_t) (HK * D * 2), (size_t) (D * 2), (size_t) (HK * D * 2), (size_t) (D * 2), op[1], op[2], op[4], freq_base,
-                                           freq_scale, ext_factor, attn_factor, beta_fast, beta_slow));
+            // an f16 cache view: its data and the byte strides of a cell and a head; a quantized one: the owning tensor's data, the
+            // view's first block within it and the owner's blocks per row
+            struct store_dest { int type; void * base; int64_t a, b; };
+            auto dest_of = [&](const ggml_tensor * d) {
+                if (d->type == GGML_TYPE_F16) return store_dest{MI355_F16, d->data, HK * D * 2, D * 2};
+                const kv_operand o = kv_operand_of(d);
+                return store_dest{to_mi355_type(d->type), (void *) o.base,
+                                  (int64_t) (((const char *) o.p - (const char *) o.base) / (ptrdiff_t) ggml_type_size(d->type)), o.row_blocks};
+            };
+            const store_dest dk = dest_of(p.ck->src[1]), dv = dest_of(p.cv->src[1]);
+            MI355_K_OK(mi355_rope_kv_store_typed(s, (float *) rq->data, (const float *) p.rk->data, (const float *) p.mv->data, dk.type, dk.base, dk.a, dk.b,
+                                                 dv.type, dv.base, dv.a, dv.b, (const int32_t *) rq->src[1]->data, ctx->iota,
+                                                 rq->src[2] ? (const float *) rq->src[2]->data : nullptr, T, H, HK, D, op[1], op[2], op[4], freq_base,
+                                                 freq_scale, ext_factor, attn_factor, beta_fast, beta_slow));
             ctx->note_write(rq->data, ggml_nbytes(rq));
             ctx->note_write(p.rk->data, ggml_nbytes(p.rk));
             ctx->note_write(p.ck->src[1]->data, ggml_nbytes(p.ck->src[1]));
@@ -1716,7 +1756,8 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     if (node->op == GGML_OP_FLASH_ATTN_EXT) {
         const ggml_tensor * q = node->src[0];
         const int64_t D = q->ne[0], Nq = q->ne[1], Hq = q->ne[2];
-        if (q->ne[3] == 1 && Nq <= 8 && D % 32 == 0 && node->src[1]->type == GGML_TYPE_F16 && node->src[2]->type == GGML_TYPE_F16 &&
+        auto cache_type = [](ggml_type t) { return t == GGML_TYPE_F16 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q4_0; };
+        if (q->ne[3] == 1 && Nq <= 8 && D % 32 == 0 && cache_type(node->src[1]->type) && cache_type(node->src[2]->type) &&
             feeds_quant_gemv(w, i, node->data, Hq * D, Nq)) {
             const ggml_tensor * k = node->src[1];
             const ggml_tensor * v = node->src[2];
@@ -1726,6 +1767,19 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
             memcpy(&softcap, (const float *) node->op_params + 2, sizeof(float));
             const int64_t Nkv = k->ne[1], Hkv = k->ne[2];
+            if (k->type != GGML_TYPE_F16 || v->type != GGML_TYPE_F16) {   // quantized cache, read in place (fewer than 16 query rows)
+                const kv_operand ko = kv_operand_of(k), vo = kv_operand_of(v);
+                GGML_ASSERT(ko.ok && vo.ok);
+                const size_t ws_bytes = mi355_flash_attn_kv_ws_bytes(D, Nq, Nkv, Hq, Hkv, to_mi355_type(k->type), to_mi355_type(v->type));
+                void * ws = ctx->workspace(ws_bytes);
+                void * act = ctx->act_slot(mi355_act_bytes(Hq * D, Nq));
+                MI355_K_OK(mi355_flash_attn_ext_kv(s, (const float *) q->data, ko.p, to_mi355_type(k->type), ko.base, ko.row_blocks, vo.p,
+                                                   to_mi355_type(v->type), vo.base, vo.row_blocks, mask ? mask->data : nullptr, (float *) node->data, D, Nq,
+                                                   Nkv, Hq, Hkv, q->nb[1], q->nb[2], k->nb[1], k->nb[2], v->nb[1], v->nb[2], mask ? mask->nb[1] : 0, scale,
+                                                   max_bias, softcap, ws, ws_bytes, act));
+                ctx->cache = act_cache{node->data, Hq * D, Nq, ACT_Q8_1, true, act};
+                return i;
+            }
             const size_t full = mi355_flash_attn_ws_bytes(D, Nq, Nkv, Hq);
             const size_t ws_bytes = full < (size_t(256) << 20) ? full : (size_t(256) << 20);
             void * ws = ctx->workspace(ws_bytes);
@@ -1957,7 +2011,8 @@ uint64_t sig_tensor(uint64_t h, const ggml_tensor * t, bool through_cache) {
 bool is_cache_store(const ggml_tensor * node) {
     if (node->op != GGML_OP_CPY) return false;
     const ggml_tensor * d = node->src[1];
-    return d && d->type == GGML_TYPE_F16 && d->view_src && d->view_src->data && ggml_is_contiguous(d);
+    return d && (d->type == GGML_TYPE_F16 || d->type == GGML_TYPE_Q8_0 || d->type == GGML_TYPE_Q4_0) && d->view_src && d->view_src->data &&
+           ggml_is_contiguous(d);
 }
 
 graph_signature sign_graph(ggml_cgraph * cgraph, std::vector<uint64_t> * trace = nullptr) {

@@ -62,11 +62,9 @@ __device__ __forceinline__ kv_lane kv_lane_of(const kv_src &s, int type, int64_t
     if (s.row_blocks == 0) {
         o.sc = s.base + g * BB;
         lv = o.sc + 2;
-    } else {
-        const int64_t row = g / s.row_blocks, b = g % s.row_blocks;
-        const uint8_t *rb = s.base + row * s.row_blocks * BB;
-        lv = rb + b * LB;
-        o.sc = rb + s.row_blocks * LB + b * 2;
+    } else {   // cell 0's blocks lie in the owner's row that starts at s.base (kv_in_place): g < row_blocks
+        lv = s.base + g * LB;
+        o.sc = s.base + s.row_blocks * LB + g * 2;
     }
     o.lv = lv + (type == MI355_Q8_0 ? j : (j & 15));
     o.shift = (type == MI355_Q4_0 && j >= 16) ? 4 : 0;
@@ -108,9 +106,14 @@ __device__ __forceinline__ float kv_levels8_f16(int type, const u32x4 &raw, int 
     return half_bits_to_float((unsigned short)raw[2]);
 }
 
-// NW: waves per group; QUANT: K and / or V may be Q8_0 / Q4_0 (a.type_k, a.type_v), read in place
-template <int D, int R, int NW = 4, bool QUANT = false>
+// NW: waves per group; KV: 0 = f16 K and V; 1 = K and / or V are Q8_0 / Q4_0 read in place, the types taken from a.type_k, a.type_v
+// (every use of a type is then a branch, uniform but in the way of the scheduler: 10.3 us at 256 cells against 7.1 us for f16);
+// 2 = both Q8_0, 3 = both Q4_0, known to the compiler
+template <int D, int R, int NW = 4, int KV = 0>
 __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
+    constexpr bool QUANT = KV != 0;
+    const int type_k = KV == 2 ? MI355_Q8_0 : KV == 3 ? MI355_Q4_0 : a.type_k;
+    const int type_v = KV == 2 ? MI355_Q8_0 : KV == 3 ? MI355_Q4_0 : a.type_v;
     constexpr int LPR = D <= 64 ? 8 : (D <= 128 ? 16 : 32);   // lanes per K/V row
     constexpr int CPW = 64 / LPR;                               // cells per wave step
     constexpr int SLOTS = NW * CPW;                             // independent softmax states per group
@@ -169,10 +172,10 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     const unsigned short *mrow = a.mask ? (const unsigned short *)(a.mask + iq * a.mask_nb1) : nullptr;
     const float scale = a.softcap != 0.0f ? a.scale / a.softcap : a.scale;
     // quantized operands (wave-uniform choice): this lane's place in the rows of kv head hk
-    const bool k_f16 = !QUANT || a.type_k == MI355_F16, v_f16 = !QUANT || a.type_v == MI355_F16;
+    const bool k_f16 = !QUANT || type_k == MI355_F16, v_f16 = !QUANT || type_v == MI355_F16;
     kv_lane kl = {nullptr, nullptr, 0, 0, 0}, vl = {nullptr, nullptr, 0, 0, 0};
-    if (!k_f16 && active) kl = kv_lane_of(a.kq, a.type_k, hk, d0);
-    if (!v_f16 && active) vl = kv_lane_of(a.vq, a.type_v, hk, d0);
+    if (!k_f16 && active) kl = kv_lane_of(a.kq, type_k, hk, d0);
+    if (!v_f16 && active) vl = kv_lane_of(a.vq, type_v, hk, d0);
 
     // U steps of SLOTS cells at a time: all mask entries, then all K/V rows of the U steps are requested before the first
     // is used, so a short context costs one round trip to memory instead of one per step.  Cells are still folded into a
@@ -206,7 +209,7 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
             kd[j] = 1.0f;
             if (!k_f16) {
                 const u32x4 raw = kk[j];
-                kd[j] = kv_levels8_f16(a.type_k, raw, kl.shift, kk[j]);
+                kd[j] = kv_levels8_f16(type_k, raw, kl.shift, kk[j]);
             }
         }
         // V rows as floats, then per head: the U scores (independent of each other), ONE new maximum and ONE rescale of the state,
@@ -223,7 +226,7 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
                     vf[j][2 * i + 1] = (float)h2[1];
                 }
             } else {
-                kv_values8(a.type_v, vv[j], vl.shift, vf[j]);
+                kv_values8(type_v, vv[j], vl.shift, vf[j]);
             }
         }
 #pragma unroll
@@ -391,14 +394,17 @@ static int launch_vec(hipStream_t s, fattn_args &a) {
     a.groups = (int)(a.Hq / a.Hkv) / R;
     const dim3 grid((unsigned)a.n_splits, (unsigned)(a.Hkv * a.groups), (unsigned)a.Nq);
     if constexpr (D % 32 == 0) {
-        if (quant) MI355_LAUNCH((k_fattn_vec<D, R, NW, true>), grid, dim3(NW * 64), 0, s, a);
-        else MI355_LAUNCH((k_fattn_vec<D, R, NW, false>), grid, dim3(NW * 64), 0, s, a);
+        const bool same = a.type_k == a.type_v && D == 128;   // the caches llama.cpp builds with -ctk / -ctv of one type
+        if (quant && same && a.type_k == MI355_Q8_0) MI355_LAUNCH((k_fattn_vec<D, R, NW, D == 128 ? 2 : 1>), grid, dim3(NW * 64), 0, s, a);
+        else if (quant && same && a.type_k == MI355_Q4_0) MI355_LAUNCH((k_fattn_vec<D, R, NW, D == 128 ? 3 : 1>), grid, dim3(NW * 64), 0, s, a);
+        else if (quant) MI355_LAUNCH((k_fattn_vec<D, R, NW, 1>), grid, dim3(NW * 64), 0, s, a);
+        else MI355_LAUNCH((k_fattn_vec<D, R, NW, 0>), grid, dim3(NW * 64), 0, s, a);
     } else {
         if (quant) {
             set_error("flash_attn: head size %d is not a whole number of quantization blocks", D);
             return MI355_ERR_ARG;
         }
-        MI355_LAUNCH((k_fattn_vec<D, R, NW, false>), grid, dim3(NW * 64), 0, s, a);
+        MI355_LAUNCH((k_fattn_vec<D, R, NW, 0>), grid, dim3(NW * 64), 0, s, a);
     }
     int rc = launch_status("k_fattn_vec");
     if (rc != MI355_OK) return rc;

@@ -8,7 +8,8 @@ namespace mi355 {
 // A Q8_0 / Q4_0 operand read block by block where it lies (no f16 copy).  Block g of the owning tensor sits at g * block bytes
 // (row_blocks == 0: plain ggml blocks, the f16 scale in front of the levels) or, for a tensor in the device row layout, in row
 // g / row_blocks at position g % row_blocks (the levels of a row first, its scales behind them).  The (cell 0, head) row starts at
-// block first_block + head * head_blocks; a cell further on, the levels lie cell_lv bytes and the scales cell_sc bytes further on:
+// block first_block + head * head_blocks, and in the device row layout base is the owner's row that holds all of cell 0's blocks
+// (first_block + head * head_blocks + D / 32 <= row_blocks for every head); a cell further on, the levels lie cell_lv bytes and the scales cell_sc bytes further on:
 // both nb1 for plain blocks and where a cell's stride is a whole number of the owner's rows; (blocks per cell) * 32 or 16 and
 // (blocks per cell) * 2 where all cells lie in ONE row of the owner (llama.cpp's cache tensors are 1-D: one row of all cells).
 struct kv_src {

@@ -10,6 +10,7 @@
 // exactly one 256-element super-block)
 //   ROPE(q), ROPE(k), CPY(k -> cache), CPY(v -> cache)   k_rope_kv_store
 #include "common.hpp"
+#include "kv_blocks.hpp"
 #include "norm_quant.hpp"
 #include "q8k.hpp"
 #include "tiles.hpp"
@@ -65,6 +66,9 @@ struct rope_kv_args {
     const float *k;         // [T][HK][D] f32
     const float *v;         // [T][HK][D] f32
     uint8_t *kcache, *vcache;   // f16; element (cell, head, d) at cell*nb1 + head*nb2 + 2*d
+                                // Q8_0 / Q4_0 (type_k / type_v): data of the tensor that owns the memory; nb1 = index of cell 0's first
+                                // block within it, nb2 = its blocks per row in the device row layout (0: plain ggml blocks)
+    int type_k, type_v;
     const int32_t *pos;     // [T] rope positions
     const int32_t *cells;   // [T] cache cell of each token
     const float *ff;        // rope frequency factors [n_dims/2] or null
@@ -91,6 +95,9 @@ __device__ __forceinline__ void rope_cos_sin(const rope_kv_args &a, int pos, int
 // One 256-thread group per token.  The rotation of a pair depends on the token's position and the pair only, so a wave works it
 // out once per pair (lane = pair) and applies it to every head it is given: the four waves share the H query heads, HK key heads
 // and HK value heads (plain f16 copies) between them, wave w taking slots w, w + 4, ...  Same roundings as k_rope: no contraction.
+// QC: K and / or V go to a Q8_0 / Q4_0 cache (adjacent-pair mode, D a multiple of 32): a lane holds two adjacent elements, 16 lanes
+// one block, quantized as quantize_row_q8_0_ref / quantize_row_q4_0_ref do.
+template <bool QC>
 __global__ void __launch_bounds__(256) k_rope_kv_store(rope_kv_args a) {
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int D = a.D, n_slots = a.H + 2 * a.HK;
@@ -130,6 +137,21 @@ __global__ void __launch_bounds__(256) k_rope_kv_store(rope_kv_args a) {
                     float *o = a.q_out + ((int64_t)t * a.H + h) * D;
                     o[ia] = y0;
                     o[ib] = y1;
+                } else if (QC && (h < a.H + a.HK ? a.type_k : a.type_v) != MI355_F16) {   // uniform over the wave
+                    const bool is_k = h < a.H + a.HK;
+                    const int type = is_k ? a.type_k : a.type_v;
+                    const int head = is_k ? h - a.H : h - a.H - a.HK;
+                    const kv_place pl = {0, is_k ? a.k_nb2 : a.v_nb2};
+                    const int64_t g = (is_k ? a.k_nb1 : a.v_nb1) + (cell * a.HK + head) * (D >> 5) + (i0 >> 5);
+                    uint8_t *base = is_k ? a.kcache : a.vcache;
+                    int64_t lv, sc;
+                    if (type == MI355_Q8_0) {
+                        kv_block_offsets<MI355_Q8_0>(pl, g, lv, sc);
+                        kv_store_q8_0_pair16(y0, y1, pair & 15, base, lv, sc);
+                    } else {
+                        kv_block_offsets<MI355_Q4_0>(pl, g, lv, sc);
+                        kv_store_q4_0_pair16(y0, y1, pair & 15, base, lv, sc);
+                    }
                 } else if (h < a.H + a.HK) {
                     _Float16 *kc = (_Float16 *)(a.kcache + cell * a.k_nb1 + (int64_t)(h - a.H) * a.k_nb2);
                     kc[ia] = (_Float16)y0;
@@ -222,17 +244,22 @@ int mi355_swiglu_quant_q8k_tiled(void *stream, const float *gate, const float *u
     return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, 2);
 }
 
-int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, void *kcache, void *vcache, const int32_t *pos,
-                        const int32_t *cells, const float *freq_factors, int64_t T, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
-                        size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
-                        float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
+static int rope_kv_store_impl(void *stream, float *q, const float *k, const float *v, int type_k, void *kcache, int64_t k_a, int64_t k_b, int type_v,
+                              void *vcache, int64_t v_a, int64_t v_b, const int32_t *pos, const int32_t *cells, const float *freq_factors, int64_t T,
+                              int64_t H, int64_t HK, int64_t D, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                              float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
     MI355_REQUIRE(T > 0 && T <= 65535 && H > 0 && HK > 0 && D > 0 && D % 2 == 0 && D <= 2048, "rope_kv_store: bad shape");
     MI355_REQUIRE(mode == 0 || mode == 2, "rope_kv_store: mode %d not supported (0 = adjacent pairs, 2 = NeoX)", mode);
     MI355_REQUIRE(n_dims > 0 && n_dims % 2 == 0 && n_dims <= D, "rope_kv_store: bad n_dims");
+    const bool qc = type_k != MI355_F16 || type_v != MI355_F16;
+    for (int t : {type_k, type_v}) MI355_REQUIRE(t == MI355_F16 || t == MI355_Q8_0 || t == MI355_Q4_0, "rope_kv_store: cache type %d (f16, Q8_0, Q4_0 are served)", t);
+    MI355_REQUIRE(!qc || (mode == 0 && D % 32 == 0 && k_a >= 0 && k_b >= 0 && v_a >= 0 && v_b >= 0 && (((uintptr_t)kcache | (uintptr_t)vcache) & 1) == 0),
+                  "rope_kv_store: a quantized cache takes the adjacent-pair mode and head sizes that are multiples of 32");
     rope_kv_args a;
     a.q = q; a.q_out = q; a.k = k; a.v = v; a.kcache = (uint8_t *)kcache; a.vcache = (uint8_t *)vcache;
+    a.type_k = type_k; a.type_v = type_v;
     a.pos = pos; a.cells = cells; a.ff = freq_factors;
-    a.k_nb1 = (int64_t)k_nb1; a.k_nb2 = (int64_t)k_nb2; a.v_nb1 = (int64_t)v_nb1; a.v_nb2 = (int64_t)v_nb2;
+    a.k_nb1 = k_a; a.k_nb2 = k_b; a.v_nb1 = v_a; a.v_nb2 = v_b;
     a.T = (int)T; a.H = (int)H; a.HK = (int)HK; a.D = (int)D; a.n_dims = n_dims; a.mode = mode;
     a.theta_scale = powf(freq_base, -2.0f / n_dims);
     a.freq_scale = freq_scale; a.ext_factor = ext_factor; a.attn_factor = attn_factor;
@@ -241,8 +268,25 @@ int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, 
     const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
     a.corr0 = c0 > 0 ? c0 : 0;
     a.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
-    MI355_LAUNCH(k_rope_kv_store, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, a);
+    if (qc) MI355_LAUNCH(k_rope_kv_store<true>, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, a);
+    else MI355_LAUNCH(k_rope_kv_store<false>, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, a);
     return launch_status("k_rope_kv_store");
+}
+
+int mi355_rope_kv_store(void *stream, float *q, const float *k, const float *v, void *kcache, void *vcache, const int32_t *pos,
+                        const int32_t *cells, const float *freq_factors, int64_t T, int64_t H, int64_t HK, int64_t D, size_t k_nb1,
+                        size_t k_nb2, size_t v_nb1, size_t v_nb2, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                        float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
+    return rope_kv_store_impl(stream, q, k, v, MI355_F16, kcache, (int64_t)k_nb1, (int64_t)k_nb2, MI355_F16, vcache, (int64_t)v_nb1, (int64_t)v_nb2, pos, cells,
+                              freq_factors, T, H, HK, D, n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+}
+
+int mi355_rope_kv_store_typed(void *stream, float *q, const float *k, const float *v, int type_k, void *kcache, int64_t k_a, int64_t k_b, int type_v,
+                              void *vcache, int64_t v_a, int64_t v_b, const int32_t *pos, const int32_t *cells, const float *freq_factors, int64_t T,
+                              int64_t H, int64_t HK, int64_t D, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
+                              float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
+    return rope_kv_store_impl(stream, q, k, v, type_k, kcache, k_a, k_b, type_v, vcache, v_a, v_b, pos, cells, freq_factors, T, H, HK, D, n_dims, mode,
+                              n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
 }
 
 }  // extern "C"

@@ -10,6 +10,7 @@
 // the groups of all matrices are laid end to end in the grid, which turns three short launches
 // into one long enough to fill the chip.  An optional residual is added in the epilogue.
 #include "common.hpp"
+#include "kv_blocks.hpp"
 #include "qdot.hpp"
 #include "norm_quant.hpp"
 #include "ffn.hpp"
@@ -29,8 +30,11 @@ struct gemv_item {
     int first_group;         // index of this matrix's first group in the launch
     int epi;                 // EPI_*: what happens to a finished row
     int64_t nb1, nb2;        // EPI_*_CACHE: byte strides of a cache cell and of a head inside it (dst = cache base)
+                             // EPI_*_QCACHE: block index of cell 0 within the tensor that owns the cache memory (dst = its data) and
+                             // that tensor's blocks per row in the device row layout (0: plain ggml blocks)
+    int ctype;               // EPI_*_QCACHE: MI355_Q8_0 or MI355_Q4_0
 };
-enum { EPI_STORE = 0, EPI_ROPE = 1, EPI_ROPE_CACHE = 2, EPI_CACHE = 3 };
+enum { EPI_STORE = 0, EPI_ROPE = 1, EPI_ROPE_CACHE = 2, EPI_CACHE = 3, EPI_ROPE_QCACHE = 4, EPI_QCACHE = 5 };
 
 // rotary embedding of the Q/K rows produced by the fused QKV launch (mode 0: adjacent pairs)
 struct gemv_rope {
@@ -199,6 +203,149 @@ __device__ __forceinline__ void gemv_body(const gemv_item &m, int group, const i
     }
 }
 
+// The Q/K/V launch when K and / or V go to a Q8_0 / Q4_0 cache: groups of EIGHT waves.  QUANT: the group's 32 rows (four per wave)
+// are one block of a cache row; the finished, rotated values meet in LDS and wave c quantizes the block of activation row c
+// (quantize_row_q8_0_ref / quantize_row_q4_0_ref, as the cache copies of kv_quant.hip do); m.N is a multiple of 32, so every wave is
+// live.  !QUANT: 16 rows per group (two per wave) with the epilogues of gemv_body.  Every row sum is formed exactly as in gemv_body.
+// (Groups of four waves that took their eight rows each in two passes of four were measured first: 14.6 us against 10.3 us for the
+// launch with f16 stores on the Llama-8B shapes - the groups of 32 rows ran twice as long as the others.)
+template <int TYPE, int NCOLS, bool NORM, bool QUANT>
+__device__ __forceinline__ void gemv_body_qc(const gemv_item &m, int group, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K,
+                                             const gemv_rope &R, uint8_t *s_act) {
+    typedef wq<TYPE> T;
+    constexpr int NW = 8, RPW = QUANT ? 4 : 2, NP = RPW / 2;
+    static_assert(NCOLS <= 4, "wave c quantizes activation row c");
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t row0 = ((int64_t)group * NW + wave) * RPW;
+    const bool wave_live = row0 < m.N;   // uniform over the wave; always true with QUANT
+    if (!NORM && !wave_live) return;     // with NORM a wave without rows still takes its share of the norm and its barriers
+    const row_layout L = make_row_layout(TYPE, K);
+    const int nchunks = K / T::CHUNK;
+    const int nblk = K >> 5;
+
+    const uint8_t *rows[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; r++) {
+        const int64_t row = row0 + r < m.N ? row0 + r : m.N - 1;   // clamp: tail rows recompute the last row, never stored
+        rows[r] = m.W + row * L.row_bytes;
+    }
+
+    float rope_c[NP], rope_s[NP];
+    bool rotate[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+        rope_c[p] = 1.0f;
+        rope_s[p] = 0.0f;
+        rotate[p] = false;
+    }
+    int cell = 0;
+    if (lane < NCOLS) {
+        const bool rope_epi = m.epi == EPI_ROPE || m.epi == EPI_ROPE_CACHE || m.epi == EPI_ROPE_QCACHE;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int d = (int)((row0 + 2 * p) % R.D);
+            rotate[p] = rope_epi && d < R.n_dims;
+            if (rotate[p]) rope_coeffs(R, R.pos[lane], d >> 1, rope_c[p], rope_s[p]);
+        }
+        if (m.epi == EPI_ROPE_CACHE || m.epi == EPI_CACHE) cell = R.cells[lane];
+    }
+#pragma unroll
+    for (int p = 0; p < NP; p++) asm volatile("" : "+v"(rope_c[p]), "+v"(rope_s[p]));
+    asm volatile("" : "+v"(cell));
+
+    typename T::chunk w_first[RPW];
+    if constexpr (NORM) {   // as in gemv_body: the first step's weights are on their way while the group normalises and quantizes the row
+        const int c = lane < nchunks ? lane : nchunks - 1;
+#pragma unroll
+        for (int r = 0; r < RPW; r++) w_first[r] = T::load_w(rows[r], L, c);
+        __shared__ float s_norm[4];
+        if (threadIdx.x < 256) rms_norm_quant_row<4, false, false>(R.nx, R.nw, nullptr, s_act, 0, K, 1, R.neps, s_norm);
+        else __syncthreads();   // the one barrier inside the norm
+        __syncthreads();
+        if (!wave_live) return;
+        aq = (const int8_t *)s_act;
+        ads = (const act_ds *)(s_act + NCOLS * K);
+    }
+
+    float acc[RPW][NCOLS];
+#pragma unroll
+    for (int r = 0; r < RPW; r++)
+#pragma unroll
+        for (int c = 0; c < NCOLS; c++) acc[r][c] = 0.0f;
+    for (int c0 = 0; c0 < nchunks; c0 += 64) {
+        const int c = c0 + lane;
+        if (c < nchunks) {
+            typename T::chunk w[RPW];
+#pragma unroll
+            for (int r = 0; r < RPW; r++) {
+                if (NORM && c0 == 0) w[r] = w_first[r];
+                else w[r] = T::load_w(rows[r], L, c);
+            }
+#pragma unroll
+            for (int col = 0; col < NCOLS; col++) {
+                const typename T::act A = T::load_a(aq + (int64_t)col * K, ads + col * nblk, c);
+#pragma unroll
+                for (int r = 0; r < RPW; r++) {
+                    const chunk_dots d = T::dots(w[r], A);
+                    acc[r][col] = T::accumulate(acc[r][col], w[r], A, d);
+                }
+            }
+        }
+    }
+    float sv[RPW];
+#pragma unroll
+    for (int r = 0; r < RPW; r++) sv[r] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RPW; r++)
+#pragma unroll
+        for (int c = 0; c < NCOLS; c++) {
+            const float a = wave_sum_dpp(acc[r][c]);
+            if (lane == c) sv[r] = a;
+        }
+    if constexpr (QUANT) {
+        __shared__ float s_blk[NCOLS][32];
+        if (lane < NCOLS) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                float y0 = sv[2 * p], y1 = sv[2 * p + 1];
+                if (rotate[p]) rope_apply(rope_c[p], rope_s[p], sv[2 * p], sv[2 * p + 1], y0, y1);
+                s_blk[lane][wave * RPW + 2 * p] = y0;
+                s_blk[lane][wave * RPW + 2 * p + 1] = y1;
+            }
+        }
+        __syncthreads();
+        if (wave < NCOLS) {
+            const int j = lane & 31;
+            const float v = s_blk[wave][j];
+            const int64_t g = m.nb1 + (int64_t)R.cells[wave] * (m.N >> 5) + group;
+            const kv_place pl = {0, m.nb2};
+            int64_t lv, sc;
+            if (m.ctype == MI355_Q8_0) {
+                kv_block_offsets<MI355_Q8_0>(pl, g, lv, sc);
+                kv_store_q8_0_lane32(v, j, (uint8_t *)m.dst, lv, sc, lane < 32);
+            } else {
+                kv_block_offsets<MI355_Q4_0>(pl, g, lv, sc);
+                kv_store_q4_0_lane32(v, j, (uint8_t *)m.dst, lv, sc, lane < 32);
+            }
+        }
+    } else if (lane < NCOLS && row0 + 1 < m.N) {
+        const int64_t head = row0 / R.D;
+        const int d = (int)(row0 % R.D);
+        float y0 = sv[0], y1 = sv[1];
+        if (rotate[0]) rope_apply(rope_c[0], rope_s[0], sv[0], sv[1], y0, y1);
+        if (m.epi == EPI_ROPE || m.epi == EPI_STORE) {
+            float *o = m.dst + lane * m.dst_stride + row0;
+            o[0] = y0;
+            o[1] = y1;
+        } else {
+            _Float16 *o = (_Float16 *)((uint8_t *)m.dst + (int64_t)cell * m.nb1 + head * m.nb2) + d;
+            o[0] = (_Float16)y0;
+            o[1] = (_Float16)y1;
+        }
+    }
+}
+
 // dynamic LDS of the launches below: the group's copy of the activation (LDSA), act_lds_bytes() bytes
 extern __shared__ __attribute__((aligned(16))) uint8_t s_act_dyn[];
 
@@ -243,6 +390,49 @@ __global__ void __launch_bounds__(256) k_gemv_qkv_norm(gemv_batch b, int K, gemv
 #define MI355_BODY(TY) gemv_body<TY, 1, 2, true, false, true, true>(m, group, nullptr, nullptr, K, &rp, s_act_dyn);
     MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)
 #undef MI355_BODY
+}
+
+// The same two launches with K and / or V going to a Q8_0 / Q4_0 cache (gemv_body_qc): 512 threads per group; the matrices with a
+// quantized destination have groups of 32 rows, one cache block per group, the others groups of 16.  The host lists the groups
+// of 32 rows first in the grid.
+__device__ __forceinline__ int qkv_item_of(const gemv_batch &b, int g) {
+    int i = 0, best = -1;
+#pragma unroll
+    for (int j = 0; j < 3; j++)
+        if (g >= b.it[j].first_group && b.it[j].first_group > best) {   // unused items start at INT_MAX
+            i = j;
+            best = b.it[j].first_group;
+        }
+    return i;
+}
+
+template <int NCOLS>
+__global__ void __launch_bounds__(512, (NCOLS == 1 ? 4 : 2)) k_gemv_qkv_qc(gemv_batch b, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int K, gemv_rope rp) {
+    const gemv_item &m = b.it[qkv_item_of(b, blockIdx.x)];
+    const int group = blockIdx.x - m.first_group;
+    if (m.epi >= EPI_ROPE_QCACHE) {   // uniform over the group
+#define MI355_BODY(TY) gemv_body_qc<TY, NCOLS, false, true>(m, group, aq, ads, K, rp, nullptr);
+        MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)
+#undef MI355_BODY
+    } else {
+#define MI355_BODY(TY) gemv_body_qc<TY, NCOLS, false, false>(m, group, aq, ads, K, rp, nullptr);
+        MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)
+#undef MI355_BODY
+    }
+}
+
+__global__ void __launch_bounds__(512, 4) k_gemv_qkv_norm_qc(gemv_batch b, int K, gemv_rope rp) {
+    const gemv_item &m = b.it[qkv_item_of(b, blockIdx.x)];
+    const int group = blockIdx.x - m.first_group;
+    if (m.epi >= EPI_ROPE_QCACHE) {
+#define MI355_BODY(TY) gemv_body_qc<TY, 1, true, true>(m, group, nullptr, nullptr, K, rp, s_act_dyn);
+        MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)
+#undef MI355_BODY
+    } else {
+#define MI355_BODY(TY) gemv_body_qc<TY, 1, true, false>(m, group, nullptr, nullptr, K, rp, s_act_dyn);
+        MI355_WEIGHT_TYPE_SWITCH(m.type, MI355_BODY)
+#undef MI355_BODY
+    }
 }
 
 // several matrices sharing one activation
@@ -583,34 +773,51 @@ static int vec_q_rope_impl(void *stream, int n_mats, const mi355_gemv_rope_mat *
     gemv_batch b;
     b.n = n_mats;
     int64_t groups = 0;
-    bool needs_pos = false, needs_cells = false;
-    for (int i = 0; i < 4; i++) {
-        const mi355_gemv_rope_mat &m = mats[i < n_mats ? i : 0];
-        if (i < n_mats) {
-            int rc = check_gemv_args("mul_mat_vec_q_rope", m.type, m.W, m.N, K, m.N);
-            if (rc != MI355_OK) return rc;
-            MI355_REQUIRE(m.epilogue >= MI355_EPI_STORE && m.epilogue <= MI355_EPI_CACHE && m.dst != nullptr && m.N % 2 == 0,
-                          "mul_mat_vec_q_rope: bad epilogue %d, missing destination or odd row count", m.epilogue);
-            if (m.epilogue == MI355_EPI_STORE || m.epilogue == MI355_EPI_ROPE)
-                MI355_REQUIRE(m.dst_stride >= m.N, "mul_mat_vec_q_rope: dst_stride < N");
-            else
-                MI355_REQUIRE(((uintptr_t)m.dst & 1) == 0 && m.nb1 % 2 == 0 && m.nb2 % 2 == 0, "mul_mat_vec_q_rope: misaligned f16 destination");
-            if (m.epilogue != MI355_EPI_STORE) MI355_REQUIRE(m.N % D == 0, "mul_mat_vec_q_rope: N=%lld is not a whole number of heads", (long long)m.N);
-            needs_pos = needs_pos || m.epilogue == MI355_EPI_ROPE || m.epilogue == MI355_EPI_ROPE_CACHE;
-            needs_cells = needs_cells || m.epilogue == MI355_EPI_ROPE_CACHE || m.epilogue == MI355_EPI_CACHE;
+    bool needs_pos = false, needs_cells = false, any_qc = false;
+    for (int i = 0; i < n_mats; i++) any_qc = any_qc || mats[i].epilogue == MI355_EPI_ROPE_QCACHE || mats[i].epilogue == MI355_EPI_QCACHE;
+    // groups of 32 rows (quantized-cache epilogues) first in the grid, then the groups of 8: pass 0 places the former
+    for (int pass = 0; pass < 2; pass++) {
+        for (int i = 0; i < 4; i++) {
+            const mi355_gemv_rope_mat &m = mats[i < n_mats ? i : 0];
+            const bool qc = m.epilogue == MI355_EPI_ROPE_QCACHE || m.epilogue == MI355_EPI_QCACHE;
+            if (i < n_mats && qc != (pass == 0)) continue;
+            if (i >= n_mats && pass == 0) continue;
+            if (i < n_mats) {
+                int rc = check_gemv_args("mul_mat_vec_q_rope", m.type, m.W, m.N, K, m.N);
+                if (rc != MI355_OK) return rc;
+                MI355_REQUIRE(m.epilogue >= MI355_EPI_STORE && m.epilogue <= MI355_EPI_QCACHE && m.dst != nullptr && m.N % 2 == 0,
+                              "mul_mat_vec_q_rope: bad epilogue %d, missing destination or odd row count", m.epilogue);
+                if (m.epilogue == MI355_EPI_STORE || m.epilogue == MI355_EPI_ROPE)
+                    MI355_REQUIRE(m.dst_stride >= m.N, "mul_mat_vec_q_rope: dst_stride < N");
+                else if (qc)
+                    MI355_REQUIRE(((uintptr_t)m.dst & 1) == 0 && (m.dst_stride == MI355_Q8_0 || m.dst_stride == MI355_Q4_0) && m.nb1 >= 0 && m.nb2 >= 0 &&
+                                      m.N % 32 == 0,
+                                  "mul_mat_vec_q_rope: a quantized cache takes whole Q8_0 / Q4_0 blocks (N a multiple of 32)");
+                else
+                    MI355_REQUIRE(((uintptr_t)m.dst & 1) == 0 && m.nb1 % 2 == 0 && m.nb2 % 2 == 0, "mul_mat_vec_q_rope: misaligned f16 destination");
+                if (m.epilogue != MI355_EPI_STORE) MI355_REQUIRE(m.N % D == 0, "mul_mat_vec_q_rope: N=%lld is not a whole number of heads", (long long)m.N);
+                needs_pos = needs_pos || m.epilogue == MI355_EPI_ROPE || m.epilogue == MI355_EPI_ROPE_CACHE || m.epilogue == MI355_EPI_ROPE_QCACHE;
+                needs_cells = needs_cells || m.epilogue == MI355_EPI_ROPE_CACHE || m.epilogue == MI355_EPI_CACHE || qc;
+            }
+            b.it[i].W = (const uint8_t *)m.W;
+            b.it[i].residual = nullptr;
+            b.it[i].N = m.N;
+            b.it[i].type = m.type;
+            b.it[i].dst = (float *)m.dst;
+            b.it[i].dst_stride = m.dst_stride;
+            b.it[i].nb1 = m.nb1;
+            b.it[i].nb2 = m.nb2;
+            b.it[i].ctype = qc ? (int)m.dst_stride : 0;
+            // the kernel's epilogue codes: plain rows take the rope path with no rotation applied to them
+            b.it[i].epi = m.epilogue == MI355_EPI_STORE        ? EPI_STORE
+                          : m.epilogue == MI355_EPI_ROPE       ? EPI_ROPE
+                          : m.epilogue == MI355_EPI_ROPE_CACHE ? EPI_ROPE_CACHE
+                          : m.epilogue == MI355_EPI_CACHE      ? EPI_CACHE
+                          : m.epilogue == MI355_EPI_ROPE_QCACHE ? EPI_ROPE_QCACHE
+                                                               : EPI_QCACHE;
+            b.it[i].first_group = i < n_mats ? (int)groups : 0x7fffffff;
+            if (i < n_mats) groups += any_qc ? (qc ? m.N / 32 : (m.N + 15) / 16) : (m.N + 7) / 8;   // 8 waves x 4 or 2 rows; without quantized stores 4 waves x 2 rows
         }
-        b.it[i].W = (const uint8_t *)m.W;
-        b.it[i].residual = nullptr;
-        b.it[i].N = m.N;
-        b.it[i].type = m.type;
-        b.it[i].dst = (float *)m.dst;
-        b.it[i].dst_stride = m.dst_stride;
-        b.it[i].nb1 = m.nb1;
-        b.it[i].nb2 = m.nb2;
-        // the kernel's epilogue codes: plain rows take the rope path with no rotation applied to them
-        b.it[i].epi = m.epilogue == MI355_EPI_STORE ? EPI_STORE : m.epilogue == MI355_EPI_ROPE ? EPI_ROPE : m.epilogue == MI355_EPI_ROPE_CACHE ? EPI_ROPE_CACHE : EPI_CACHE;
-        b.it[i].first_group = i < n_mats ? (int)groups : 0x7fffffff;
-        if (i < n_mats) groups += (m.N + 7) / 8;   // 4 waves x 2 rows
     }
     MI355_REQUIRE(!needs_pos || rope->pos != nullptr, "mul_mat_vec_q_rope: rope positions missing");
     MI355_REQUIRE(!needs_cells || rope->cells != nullptr, "mul_mat_vec_q_rope: cache cells missing");
@@ -631,10 +838,23 @@ static int vec_q_rope_impl(void *stream, int n_mats, const mi355_gemv_rope_mat *
     const size_t lds = act_lds_bytes((int)B, K, groups);
     if (nx != nullptr) {
         rp.nx = nx; rp.nw = nw; rp.neps = neps;
+        if (any_qc) {
+            MI355_LAUNCH(k_gemv_qkv_norm_qc, dim3((unsigned)groups), dim3(512), (size_t)K + K / 4, s, b, (int)K, rp);
+            return launch_status("k_gemv_qkv_norm_qc");
+        }
         MI355_LAUNCH(k_gemv_qkv_norm, dim3((unsigned)groups), dim3(256), (size_t)K + K / 4, s, b, (int)K, rp);
         return launch_status("k_gemv_qkv_norm");
     }
     rp.nx = rp.nw = nullptr; rp.neps = 0.0f;
+    if (any_qc) {   // every wave reads the activation from memory (L2): these launches have too few groups for the copy in LDS to pay
+        switch (B) {
+            case 1: MI355_LAUNCH((k_gemv_qkv_qc<1>), dim3((unsigned)groups), dim3(512), 0, s, b, aq, ads, (int)K, rp); break;
+            case 2: MI355_LAUNCH((k_gemv_qkv_qc<2>), dim3((unsigned)groups), dim3(512), 0, s, b, aq, ads, (int)K, rp); break;
+            case 3: MI355_LAUNCH((k_gemv_qkv_qc<3>), dim3((unsigned)groups), dim3(512), 0, s, b, aq, ads, (int)K, rp); break;
+            default: MI355_LAUNCH((k_gemv_qkv_qc<4>), dim3((unsigned)groups), dim3(512), 0, s, b, aq, ads, (int)K, rp); break;
+        }
+        return launch_status("k_gemv_qkv_qc");
+    }
     switch (B) {
         case 1:
             if (lds) MI355_LAUNCH((k_gemv_qkv<1, true>), dim3((unsigned)groups), dim3(256), lds, s, b, aq, ads, (int)K, rp);

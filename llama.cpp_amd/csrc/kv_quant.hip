@@ -12,30 +12,10 @@
 // row g / row_blocks of that tensor, whatever view of it (1-D for the store, [D, cells, heads] for attention) is being used.
 #include "common.hpp"
 #include "fattn.hpp"
+#include "kv_blocks.hpp"
 
 namespace mi355 {
 
-
-struct kv_place {
-    int64_t first_block;   // block index, within the owning tensor, of the first block addressed
-    int64_t row_blocks;    // blocks per row of the owning tensor in the device row layout; 0 = plain ggml blocks
-};
-
-// byte offsets (from the owning tensor's data) of the levels and of the f16 scale of block g
-template <int TYPE>
-__device__ __forceinline__ void kv_block_offsets(const kv_place &p, int64_t g, int64_t &levels, int64_t &scale) {
-    constexpr int BB = TYPE == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES;   // block bytes
-    constexpr int LB = TYPE == MI355_Q8_0 ? 32 : 16;                   // bytes of levels per block
-    if (p.row_blocks == 0) {
-        scale = g * BB;
-        levels = scale + 2;
-    } else {
-        const int64_t row = g / p.row_blocks, b = g % p.row_blocks;
-        const int64_t base = row * p.row_blocks * BB;
-        levels = base + b * LB;
-        scale = base + p.row_blocks * LB + b * 2;
-    }
-}
 
 // A view of a quantized tensor whose rows start on block boundaries: element (i0, i1, i2, i3) of the contiguous f32 side lies in block
 // first_block + i0 / 32 + i1 * nbb[0] + i2 * nbb[1] + i3 * nbb[2] of the owner (strides in blocks).  ne0 == 0: consecutive blocks.
@@ -172,11 +152,14 @@ __global__ void __launch_bounds__(256) k_cpy_quant_blocks(const uint8_t *__restr
 
 // dst f16 [cell][head][D] = dequantized rows of a typed cache whose (cell, head) row starts at block cell * cb + head * hb (+ the
 // view's first block); one lane per 4 elements
+struct kv_image {
+    const uint8_t *src;
+    int64_t cb, hb;
+    kv_place pl;
+    _Float16 *dst;
+};
 template <int TYPE>
-__global__ void __launch_bounds__(256) k_kv_dequant_f16(const uint8_t *__restrict__ src, int64_t cb, int64_t hb, kv_place pl, _Float16 *__restrict__ dst,
-                                                        int D, int HK, int64_t n_quads) {
-    const int64_t qd = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (qd >= n_quads) return;
+__device__ __forceinline__ void kv_dequant_quad(const kv_image &im, int D, int HK, int64_t qd) {
     const int per_row = D >> 2;
     const int64_t rowi = qd / per_row;
     const int e0 = (int)(qd % per_row) * 4;
@@ -184,24 +167,33 @@ __global__ void __launch_bounds__(256) k_kv_dequant_f16(const uint8_t *__restric
     const int head = (int)(rowi % HK);
     const int j = e0 & 31;
     int64_t lv, sc;
-    kv_block_offsets<TYPE>(pl, pl.first_block + cell * cb + (int64_t)head * hb + (e0 >> 5), lv, sc);
-    const float d = half_bits_to_float(*(const unsigned short *)(src + sc));
+    kv_block_offsets<TYPE>(im.pl, im.pl.first_block + cell * im.cb + (int64_t)head * im.hb + (e0 >> 5), lv, sc);
+    const float d = half_bits_to_float(*(const unsigned short *)(im.src + sc));
     float f[4];
     if constexpr (TYPE == MI355_Q8_0) {
-        const unsigned short *p = (const unsigned short *)(src + lv + j);
+        const unsigned short *p = (const unsigned short *)(im.src + lv + j);
         const unsigned w = (unsigned)p[0] | ((unsigned)p[1] << 16);
 #pragma unroll
         for (int i = 0; i < 4; i++) f[i] = (float)(int8_t)((w >> (8 * i)) & 0xFF) * d;
     } else {
-        const unsigned short *p = (const unsigned short *)(src + lv + (j & 15));
+        const unsigned short *p = (const unsigned short *)(im.src + lv + (j & 15));
         const unsigned w = ((unsigned)p[0] | ((unsigned)p[1] << 16)) >> (j >= 16 ? 4 : 0);
 #pragma unroll
         for (int i = 0; i < 4; i++) f[i] = (float)((int)((w >> (8 * i)) & 0xF) - 8) * d;
     }
-    _Float16 *o = dst + rowi * D + e0;
+    _Float16 *o = im.dst + rowi * D + e0;
     const f16x2 lo = {(_Float16)f[0], (_Float16)f[1]}, hi = {(_Float16)f[2], (_Float16)f[3]};
     *(f16x2 *)o = lo;
     *(f16x2 *)(o + 2) = hi;
+}
+// blockIdx.y: 0 = the K image, 1 = the V image (one launch for both; TV < 0: only K)
+template <int TK, int TV>
+__global__ void __launch_bounds__(256) k_kv_dequant_f16(kv_image k, kv_image v, int D, int HK, int64_t n_quads) {
+    const int64_t qd = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (qd >= n_quads) return;
+    constexpr int TV2 = TV < 0 ? TK : TV;
+    if (TV < 0 || blockIdx.y == 0) kv_dequant_quad<TK>(k, D, HK, qd);
+    else kv_dequant_quad<TV2>(v, D, HK, qd);
 }
 
 static bool kv_type_ok(int t) { return t == MI355_F16 || t == MI355_Q8_0 || t == MI355_Q4_0; }
@@ -221,7 +213,14 @@ static bool kv_in_place(int type, const void *p, const void *base, int64_t row_b
     if (base == nullptr) base = p;
     const int64_t off = (const char *)p - (const char *)base;
     if (((uintptr_t)base & 1) != 0 || off < 0 || off % bb != 0 || nb1 % bb != 0 || nb2 % bb != 0 || row_blocks < 0) return false;
-    const int64_t cb = (int64_t)(nb1 / bb), hb = (int64_t)(nb2 / bb), first = off / bb;
+    const int64_t cb = (int64_t)(nb1 / bb), hb = (int64_t)(nb2 / bb);
+    int64_t first = off / bb;
+    // every block of cell 0 lies in one row of the owner (checked below): that row becomes the base, so that the kernels find a block
+    // of cell 0 without dividing by the row length
+    if (row_blocks > 0) {
+        base = (const char *)base + (first / row_blocks) * row_blocks * bb;
+        first %= row_blocks;
+    }
     o.base = (const uint8_t *)base;
     o.first_block = first;
     o.row_blocks = row_blocks;
@@ -302,21 +301,40 @@ size_t mi355_flash_attn_kv_ws_bytes(int64_t D, int64_t Nq, int64_t Nkv, int64_t 
     return ((base + 255) & ~(size_t)255) + kv_image_bytes(type_k, D, Nkv, Hkv) + kv_image_bytes(type_v, D, Nkv, Hkv);
 }
 
-// expands one quantized operand into its f16 image; `p` points at the first row in plain ggml addressing, `base` at the data of
-// the tensor that owns the memory
-static int kv_expand(hipStream_t s, int type, const void *p, const void *base, int64_t row_blocks, size_t nb1, size_t nb2, void *img, int64_t D,
-                     int64_t Nkv, int64_t Hkv) {
+// describes one quantized operand for the expansion into its f16 image; `p` points at the first row in plain ggml addressing, `base`
+// at the data of the tensor that owns the memory
+static int kv_image_of(int type, const void *p, const void *base, int64_t row_blocks, size_t nb1, size_t nb2, void *img, kv_image &o) {
     const int64_t bb = type == MI355_Q8_0 ? Q8_0_BYTES : Q4_0_BYTES;
     if (base == nullptr) base = p;
     const int64_t off = (const char *)p - (const char *)base;
     MI355_REQUIRE(((uintptr_t)base & 1) == 0 && off >= 0 && off % bb == 0 && nb1 % bb == 0 && nb2 % bb == 0 && row_blocks >= 0,
                   "flash_attn_kv: quantized rows must start on block boundaries");
+    o.src = (const uint8_t *)base;
+    o.cb = (int64_t)nb1 / bb;
+    o.hb = (int64_t)nb2 / bb;
+    o.pl = kv_place{off / bb, row_blocks};
+    o.dst = (_Float16 *)img;
+    return MI355_OK;
+}
+
+// the f16 images of the quantized operands, K and V in one launch where both are quantized (type F16: nothing to do for that operand)
+static int kv_expand(hipStream_t s, int type_k, const kv_image &k, int type_v, const kv_image &v, int64_t D, int64_t Nkv, int64_t Hkv) {
     const int64_t n_quads = Nkv * Hkv * (D / 4);
     MI355_REQUIRE(n_quads / 256 < 0x7fffffff, "flash_attn_kv: cache too large for one launch");
-    const dim3 grid((unsigned)((n_quads + 255) / 256));
-    const kv_place pl = {off / bb, row_blocks};
-    if (type == MI355_Q8_0) MI355_LAUNCH(k_kv_dequant_f16<MI355_Q8_0>, grid, dim3(256), 0, s, (const uint8_t *)base, (int64_t)nb1 / bb, (int64_t)nb2 / bb, pl, (_Float16 *)img, (int)D, (int)Hkv, n_quads);
-    else MI355_LAUNCH(k_kv_dequant_f16<MI355_Q4_0>, grid, dim3(256), 0, s, (const uint8_t *)base, (int64_t)nb1 / bb, (int64_t)nb2 / bb, pl, (_Float16 *)img, (int)D, (int)Hkv, n_quads);
+    const unsigned gx = (unsigned)((n_quads + 255) / 256);
+    const int Di = (int)D, Hi = (int)Hkv;
+    if (type_k != MI355_F16 && type_v != MI355_F16) {
+        const dim3 grid(gx, 2);
+        if (type_k == MI355_Q8_0 && type_v == MI355_Q8_0) MI355_LAUNCH((k_kv_dequant_f16<MI355_Q8_0, MI355_Q8_0>), grid, dim3(256), 0, s, k, v, Di, Hi, n_quads);
+        else if (type_k == MI355_Q8_0) MI355_LAUNCH((k_kv_dequant_f16<MI355_Q8_0, MI355_Q4_0>), grid, dim3(256), 0, s, k, v, Di, Hi, n_quads);
+        else if (type_v == MI355_Q8_0) MI355_LAUNCH((k_kv_dequant_f16<MI355_Q4_0, MI355_Q8_0>), grid, dim3(256), 0, s, k, v, Di, Hi, n_quads);
+        else MI355_LAUNCH((k_kv_dequant_f16<MI355_Q4_0, MI355_Q4_0>), grid, dim3(256), 0, s, k, v, Di, Hi, n_quads);
+    } else {
+        const kv_image &one = type_k != MI355_F16 ? k : v;
+        const int type = type_k != MI355_F16 ? type_k : type_v;
+        if (type == MI355_Q8_0) MI355_LAUNCH((k_kv_dequant_f16<MI355_Q8_0, -1>), dim3(gx), dim3(256), 0, s, one, one, Di, Hi, n_quads);
+        else MI355_LAUNCH((k_kv_dequant_f16<MI355_Q4_0, -1>), dim3(gx), dim3(256), 0, s, one, one, Di, Hi, n_quads);
+    }
     return launch_status("k_kv_dequant_f16");
 }
 
@@ -344,16 +362,23 @@ int mi355_flash_attn_ext_kv(void *stream, const float *q, const void *k, int typ
     // the images sit at the end of the workspace; what is in front of them serves the kv splits as before
     const size_t front = (ws_bytes - kb - vb) & ~(size_t)255;
     uint8_t *kimg = (uint8_t *)ws + front, *vimg = kimg + kb;
+    kv_image ki = {nullptr, 0, 0, {0, 0}, nullptr}, vi = ki;
     if (type_k != MI355_F16) {
-        int rc = kv_expand(s, type_k, k, k_base, k_row_blocks, k_nb1, k_nb2, kimg, D, Nkv, Hkv);
+        int rc = kv_image_of(type_k, k, k_base, k_row_blocks, k_nb1, k_nb2, kimg, ki);
         if (rc != MI355_OK) return rc;
+    }
+    if (type_v != MI355_F16) {
+        int rc = kv_image_of(type_v, v, v_base, v_row_blocks, v_nb1, v_nb2, vimg, vi);
+        if (rc != MI355_OK) return rc;
+    }
+    int rc = kv_expand(s, type_k, ki, type_v, vi, D, Nkv, Hkv);
+    if (rc != MI355_OK) return rc;
+    if (type_k != MI355_F16) {
         k = kimg;
         k_nb1 = (size_t)Hkv * D * 2;
         k_nb2 = (size_t)D * 2;
     }
     if (type_v != MI355_F16) {
-        int rc = kv_expand(s, type_v, v, v_base, v_row_blocks, v_nb1, v_nb2, vimg, D, Nkv, Hkv);
-        if (rc != MI355_OK) return rc;
         v = vimg;
         v_nb1 = (size_t)Hkv * D * 2;
         v_nb2 = (size_t)D * 2;

@@ -29,6 +29,20 @@ class GemvMat(C.Structure):
     _fields_ = [("type", _int), ("W", _p), ("N", _i64), ("dst", _p), ("dst_stride", _i64), ("residual", _p)]
 
 
+class GemvRopeMat(C.Structure):
+    """struct mi355_gemv_rope_mat"""
+    _fields_ = [("type", _int), ("W", _p), ("N", _i64), ("epilogue", _int), ("dst", _p), ("dst_stride", _i64), ("nb1", _i64), ("nb2", _i64)]
+
+
+class RopeDesc(C.Structure):
+    """struct mi355_rope_desc"""
+    _fields_ = [("pos", _p), ("cells", _p), ("freq_factors", _p), ("head_dim", _i64), ("n_dims", _int), ("mode", _int), ("n_ctx_orig", _int),
+                ("freq_base", _f), ("freq_scale", _f), ("ext_factor", _f), ("attn_factor", _f), ("beta_fast", _f), ("beta_slow", _f)]
+
+
+EPI_STORE, EPI_ROPE, EPI_ROPE_CACHE, EPI_CACHE, EPI_ROPE_QCACHE, EPI_QCACHE = range(6)
+
+
 class Tensor(C.Structure):
     """struct mi355_tensor"""
     _fields_ = [("data", _p), ("type", _int), ("ne", _i64 * 4), ("nb", _sz * 4)]
@@ -90,6 +104,8 @@ _SIGNATURES = {
     "mi355_swiglu_quant_q8k_tiled": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
     "mi355_rope_kv_store": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _int, _int, _int,
                             _f, _f, _f, _f, _f, _f]),
+    "mi355_rope_kv_store_typed": (_int, [_p, _p, _p, _p, _int, _p, _i64, _i64, _int, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _int, _int, _int,
+                                  _f, _f, _f, _f, _f, _f]),
     "mi355_ffn_gate_up_swiglu": (_int, [_p, _int, _p, _int, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q_rope": (_int, [_p, _int, _p, _p, _i64, _i64, _p]),
     "mi355_rms_norm_mul_mat_vec_q_rope": (_int, [_p, _p, _p, _f, _int, _p, _i64, _p]),

@@ -97,6 +97,67 @@ def test_rope_kv_store(dev, mode):
     assert not kcn[untouched].any() and not vcn[untouched].any()
 
 
+@pytest.mark.parametrize("ck,cv,device_rows", [(orc.Q8_0, orc.Q8_0, True), (orc.Q4_0, orc.Q4_0, True), (orc.Q4_0, orc.Q8_0, False), ("f16", orc.Q4_0, True)])
+@pytest.mark.parametrize("D", [128, 64])
+def test_rope_kv_store_quantized_caches(dev, ck, cv, device_rows, D):
+    """ROPE(q), ROPE(k) and both cache stores in one launch with Q8_0 / Q4_0 caches: the blocks are those of mi355_cpy_f32_quant of the
+    rotated rows, and (plain ggml blocks) those of the oracle's quantize_row_*_ref."""
+    import torch
+    import mi355
+    lib = mi355.load()
+    rng = np.random.default_rng(11 + D)
+    T, H, HK, n_ctx = 37, 8, 2, 64
+    N = HK * D
+    q = rng.standard_normal((T, H, D)).astype(np.float32)
+    k = rng.standard_normal((T, HK, D)).astype(np.float32)
+    v = rng.standard_normal((T, HK, D)).astype(np.float32)
+    v[3, 1, 32:64] = 0.0                      # a block of zeros (Q4_0 keeps the reference's -0.0 scale)
+    k[5, 0, :32] = np.abs(k[5, 0, 7])         # ties in magnitude: the first element wins the Q4_0 scale
+    k[5, 0, 9] = -np.abs(k[5, 0, 7])
+    pos = rng.integers(0, 4000, T).astype(np.int32)
+    cells = rng.permutation(n_ctx)[:T].astype(np.int32)
+    pd, cd = _t(dev, pos), _t(dev, cells)
+    rope = (D, 0, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+    row_blocks = n_ctx * N // 32 if device_rows else 0
+
+    def cache(ct):
+        if ct == "f16":
+            return torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+        return torch.zeros(n_ctx * N // 32 * mi355.BLOCK[ct][1], dtype=torch.uint8, device=dev)
+
+    def dest(ct, c):
+        return (mi355.F16, c.data_ptr(), N * 2, D * 2) if ct == "f16" else (ct, c.data_ptr(), 0, row_blocks)
+
+    # rotated k as f32: the same launch with k in the place of q
+    kr = _t(dev, k)
+    d1, d2 = torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev), torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+    mi355.check(lib.mi355_rope_kv_store(None, kr.data_ptr(), _t(dev, k).data_ptr(), _t(dev, v).data_ptr(), d1.data_ptr(), d2.data_ptr(), pd.data_ptr(),
+                                        cd.data_ptr(), None, T, HK, HK, D, N * 2, D * 2, N * 2, D * 2, *rope))
+    vd = _t(dev, v)
+    kc0, vc0 = cache(ck), cache(cv)
+    for ct, rows, c in ((ck, kr, kc0), (cv, vd, vc0)):
+        for t in range(T):
+            if ct == "f16":
+                c[int(cells[t])] = rows[t].to(torch.float16)
+            else:
+                mi355.check(lib.mi355_cpy_f32_quant(None, ct, rows[t].data_ptr(), c.data_ptr(), int(cells[t]) * N // 32, row_blocks, N))
+    qd, kd = _t(dev, q), _t(dev, k)
+    kc1, vc1 = cache(ck), cache(cv)
+    mi355.check(lib.mi355_rope_kv_store_typed(None, qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), *dest(ck, kc1), *dest(cv, vc1), pd.data_ptr(), cd.data_ptr(),
+                                              None, T, H, HK, D, *rope))
+    torch.cuda.synchronize()
+    qr = np.zeros_like(q)
+    orc.oracle.orc_rope(orc._ptr(q), orc._ptr(pos), None, orc._ptr(qr), D, H, T, D, 0, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 8192)
+    assert orc.nmse(qd.cpu().numpy(), qr) < 1e-7
+    assert torch.equal(kc1, kc0)
+    assert torch.equal(vc1, vc0)
+    if not device_rows:   # plain blocks: the oracle's bytes
+        for ct, rows, c in ((ck, kr.cpu().numpy(), kc1), (cv, v, vc1)):
+            want = orc.quantize("oracle", ct, rows.reshape(T, N))
+            got = c.cpu().numpy().reshape(n_ctx, -1)[cells]
+            assert np.array_equal(got, want.reshape(T, -1))
+
+
 @pytest.mark.parametrize("B", [1, 3, 8])
 @pytest.mark.parametrize("specs", [[(orc.Q4_K, 1024), (orc.Q4_K, 512), (orc.Q6_K, 256), (orc.Q8_0, 130)],
                                    [(orc.Q5_0, 1024), (orc.IQ4_NL, 512), (orc.Q5_1, 256), (orc.Q4_1, 130)],
@@ -205,6 +266,80 @@ def test_qkv_rope_store_equals_three_launch_sequence(dev, B, tq, tk, tv):
     assert torch.equal(kc1, kc0)
     assert torch.equal(vc1, vc0)
     assert kc1.abs().sum().item() > 0 and vc1.abs().sum().item() > 0
+
+
+@pytest.mark.parametrize("B,norm", [(1, False), (1, True), (2, False), (4, False)])
+@pytest.mark.parametrize("ck,cv,device_rows", [(orc.Q8_0, orc.Q8_0, True), (orc.Q4_0, orc.Q4_0, True), (orc.Q8_0, orc.Q4_0, False), ("f16", orc.Q8_0, True)])
+@pytest.mark.parametrize("tq,tk,tv", [(orc.Q4_K, orc.Q4_K, orc.Q6_K), (orc.Q5_0, orc.Q8_0, orc.Q4_0)])
+def test_qkv_rope_quantized_store_equals_separate_copies(dev, B, norm, ck, cv, device_rows, tq, tk, tv):
+    """K and V leave the Q/K/V launch as Q8_0 / Q4_0 blocks of a quantized cache: bit-identical to the launch that writes f32 rows
+    followed by mi355_cpy_f32_quant of each row into its cell (plain ggml blocks, or a 1-D cache tensor in the device row layout)."""
+    import torch
+    import mi355
+    lib = mi355.load()
+    rng = np.random.default_rng(7 * B + tq + (3 if norm else 0))
+    K, H, HK, D, n_ctx = 2048, 8, 2, 128, 64
+    N = HK * D
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    nw = (1.0 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    xd, nwd = _t(dev, x), _t(dev, nw)
+    act = None if norm else mi355.quantize_act(xd)
+    Ws = []
+    for t, n in ((tq, H * D), (tk, N), (tv, N)):
+        Wq = orc.quantize("oracle", t, (rng.standard_normal((n, K)) * 0.05).astype(np.float32))
+        Ws.append(mi355.upload_weights(t, _t(dev, Wq)))
+    cell_ids = [9, 3, 33, 0][:B]
+    pos = _t(dev, np.array([5, 17, 40, 41][:B], dtype=np.int32))
+    cells = _t(dev, np.array(cell_ids, dtype=np.int32))
+    iota = _t(dev, np.arange(B, dtype=np.int32))
+    rd = mi355.RopeDesc(pos.data_ptr(), cells.data_ptr(), None, D, D, 0, 4096, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+    rd_rows = mi355.RopeDesc(pos.data_ptr(), iota.data_ptr(), None, D, D, 0, 4096, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+
+    def cache(ct):
+        if ct == "f16":
+            return torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+        return torch.zeros(n_ctx * N // 32 * mi355.BLOCK[ct][1], dtype=torch.uint8, device=dev)
+
+    row_blocks = n_ctx * N // 32 if device_rows else 0
+
+    def launch(mats, desc):
+        arr = (mi355.GemvRopeMat * 3)(*mats)
+        if norm:
+            mi355.check(lib.mi355_rms_norm_mul_mat_vec_q_rope(None, xd.data_ptr(), nwd.data_ptr(), 1e-5, 3, arr, K, C.byref(desc)))
+        else:
+            mi355.check(lib.mi355_mul_mat_vec_q_rope(None, 3, arr, act.data_ptr(), K, B, C.byref(desc)))
+
+    # separate: f32 rows (K rotated), then one copy per row into its cell
+    q0 = torch.zeros(B, H * D, device=dev)
+    k0 = torch.zeros(B, N, device=dev)
+    v0 = torch.zeros(B, N, device=dev)
+    launch([mi355.GemvRopeMat(tq, Ws[0].data_ptr(), H * D, mi355.EPI_ROPE, q0.data_ptr(), H * D, 0, 0),
+            mi355.GemvRopeMat(tk, Ws[1].data_ptr(), N, mi355.EPI_ROPE, k0.data_ptr(), N, 0, 0),
+            mi355.GemvRopeMat(tv, Ws[2].data_ptr(), N, mi355.EPI_STORE, v0.data_ptr(), N, 0, 0)], rd_rows)
+    kc0, vc0 = cache(ck), cache(cv)
+    for ct, rows, c in ((ck, k0, kc0), (cv, v0, vc0)):
+        for b, cell in enumerate(cell_ids):
+            if ct == "f16":
+                c[cell] = rows[b].view(HK, D).to(torch.float16)
+            else:
+                mi355.check(lib.mi355_cpy_f32_quant(None, ct, rows[b].data_ptr(), c.data_ptr(), cell * N // 32, row_blocks, N))
+    # one launch
+    q1 = torch.zeros(B, H * D, device=dev)
+    kc1, vc1 = cache(ck), cache(cv)
+
+    def dest(ct, c, rope):
+        if ct == "f16":
+            return (mi355.EPI_ROPE_CACHE if rope else mi355.EPI_CACHE, c.data_ptr(), 0, c.stride(0) * 2, c.stride(1) * 2)
+        return (mi355.EPI_ROPE_QCACHE if rope else mi355.EPI_QCACHE, c.data_ptr(), ct, 0, row_blocks)
+
+    launch([mi355.GemvRopeMat(tq, Ws[0].data_ptr(), H * D, mi355.EPI_ROPE, q1.data_ptr(), H * D, 0, 0),
+            mi355.GemvRopeMat(tk, Ws[1].data_ptr(), N, *dest(ck, kc1, True)),
+            mi355.GemvRopeMat(tv, Ws[2].data_ptr(), N, *dest(cv, vc1, False))], rd)
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q0)
+    assert torch.equal(kc1, kc0)
+    assert torch.equal(vc1, vc0)
+    assert kc1.float().abs().sum().item() > 0 and vc1.float().abs().sum().item() > 0
 
 
 @pytest.mark.parametrize("B", [1, 2, 3, 4])
