@@ -279,11 +279,12 @@ def test_moe_model_logits_cpu_vs_plugin(dev, tmp_path, n_prompt):
     assert orc.nmse(gpu, cpu) < 2e-3
 
 
-@pytest.mark.parametrize("moe", [False, True])
-def test_decode_graph_replay_equals_launch_by_launch(dev, tmp_path, moe):
+@pytest.mark.parametrize("moe,cache", [(False, None), (True, None), (False, ("q8_0", "q8_0")), (False, ("q4_0", "q4_0"))])
+def test_decode_graph_replay_equals_launch_by_launch(dev, tmp_path, moe, cache):
     """Decode graphs replayed as HIP graphs give the bits of the same graphs issued launch by launch, over a run that crosses a
     256-cell boundary of the attention window (the graph changes there and is recorded again), with the prompt's prefill and
-    the host's synchronizing logits reads between the replays.  Every decoded token's logits are compared."""
+    the host's synchronizing logits reads between the replays.  Every decoded token's logits are compared.  With a Q8_0 / Q4_0
+    cache the stores leave with the Q/K/V launch through the device-side cell list, like the f16 stores."""
     if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
         pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
@@ -295,14 +296,15 @@ def test_decode_graph_replay_equals_launch_by_launch(dev, tmp_path, moe):
     else:
         make_synthetic_gguf.write_model(model, n_layer=3, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048)
     st = {}
-    replayed = _logits(model, 99, 249, 14, str(tmp_path / "graph.bin"), stats=st)
-    launched = _logits(model, 99, 249, 14, str(tmp_path / "eager.bin"), graphs=False)
+    replayed = _logits(model, 99, 249, 14, str(tmp_path / "graph.bin"), stats=st, cache=cache)
+    launched = _logits(model, 99, 249, 14, str(tmp_path / "eager.bin"), graphs=False, cache=cache)
     assert st["captures"] >= 2 and st["replays"] >= 8, st
     assert replayed.shape == launched.shape and np.isfinite(replayed).all()
     assert np.array_equal(replayed, launched)
 
 
-def test_launches_per_layer(dev, tmp_path):
+@pytest.mark.parametrize("cache", [None, ("q8_0", "q8_0")])
+def test_launches_per_layer(dev, tmp_path, cache):
     """What the plug-in launches for the reference's llama graphs, counted by the kernel library itself and reported per graph
     under MI355_LOG_GRAPH (one-time copies of weights are reported apart): the difference between a 4-layer and a 2-layer
     model is two layers' worth.  One decoded token takes 6 launches per layer ([norm + Q/K/V + rope + cache stores] [attention]
@@ -310,7 +312,8 @@ def test_launches_per_layer(dev, tmp_path):
     stays within 256 cache cells) takes at most 14: norm, [Q + K (+ V where its type is theirs) in one launch], (V alone where it is
     Q6_K, with the reduction launch of a product that is cut along K because it has few tiles), [rope, rope, store, store],
     attention, quantization, wo + residual and its reduction launch, norm, [gate + up in one launch], SiLU*up, down + residual
-    and its reduction launch."""
+    and its reduction launch.  A Q8_0 cache changes neither count's structure: its stores leave with the same launches, and a prompt
+    batch adds the one launch that expands the cells it attends to into f16."""
     if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
         pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
@@ -320,7 +323,7 @@ def test_launches_per_layer(dev, tmp_path):
         model = str(tmp_path / ("l%d.gguf" % n_layer))
         make_synthetic_gguf.write_model(model, n_layer=n_layer, n_embd=4096, n_ff=14336, n_head=32, n_head_kv=8, n_vocab=2048)
         env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN, MI355_LOG_GRAPH="1", MI355_NO_GRAPH="1")
-        r = subprocess.run([LOGITS, model, "99", "200", "3", str(tmp_path / "o.bin")], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+        r = subprocess.run([LOGITS, model, "99", "200", "3", str(tmp_path / "o.bin")] + (list(cache) if cache else []), env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
                            text=True, timeout=600, cwd=os.path.dirname(LOGITS))
         assert r.returncode == 0, r.stdout[-3000:]
         per_batch = {}
@@ -332,7 +335,7 @@ def test_launches_per_layer(dev, tmp_path):
     decode = (counts[4][1] - counts[2][1]) / 2
     prefill = (counts[4][200] - counts[2][200]) / 2
     os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-    with open(os.path.join(ROOT, "gpurun_out", "launches_per_layer.txt"), "w") as f:
-        f.write("decode %g launches per layer, prefill(200) %g; totals %r\n" % (decode, prefill, counts))
+    with open(os.path.join(ROOT, "gpurun_out", "launches_per_layer.txt"), "a") as f:
+        f.write("cache %s: decode %g launches per layer, prefill(200) %g; totals %r\n" % (cache[0] if cache else "f16", decode, prefill, counts))
     assert decode == 6, counts     # norm + Q/K/V + ROPE + stores, attention, wo + residual, norm, gate + up + SiLU*up, down + residual
-    assert prefill <= 14, counts
+    assert prefill <= (15 if cache else 14), counts
