@@ -475,6 +475,19 @@ int mi355_rms_norm_qkv_rope_store(void *stream, const float *x, const float *nor
 int mi355_ffn_gate_up_swiglu(void *stream, int type_gate, const void *w_gate, int type_up, const void *w_up, const void *act, float *gate,
                              float *up, int64_t out_stride, void *act_out, unsigned *counters, int64_t N, int64_t K, int64_t B);
 
+/* The same for the experts of a mixture-of-experts layer (llm_build_moe_ffn, src/llama.cpp:417-538): MUL_MAT_ID(up experts),
+ * MUL_MAT_ID(gate experts), UNARY(SILU), MUL and the Q8_1 rows the MUL_MAT_ID of the down experts reads, in one launch
+ * (ggml_compute_forward_mul_mat_id, ggml-cpu.c:7717-7894, per slot as mi355_mul_mat_id_vec; same bits as that call twice followed by
+ * mi355_swiglu_quant).  as_gate / as_up: n_expert stacked matrices of N rows in the device layout, both of `type`; act: the
+ * mi355_quantize_act form of src1 (nb1 * T rows of K); slot t * n_used + e reads expert ids[t * ids_stride + e] and activation row
+ * t * nb1 + e % nb1.  gate / up: f32 [T * n_used][N], the raw products; act_out: mi355_quantize_act layout of T * n_used rows of N.
+ * N % 32 == 0, K % 64 == 0, 16-byte aligned weight rows. */
+int mi355_moe_gate_up_swiglu(void *stream, int type, const void *as_gate, const void *as_up, const void *act, const int32_t *ids, int64_t ids_stride,
+                             float *gate, float *up, void *act_out, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T);
+/* 1 when mi355_moe_gate_up_swiglu takes these expert stacks (the shape limits above and 16-byte aligned rows), else 0; no counterpart
+ * in the reference (a caller's pre-check, like ggml_backend_dev_supports_op for one launch form). */
+int mi355_moe_gate_up_swiglu_supported(int type, const void *as_gate, const void *as_up, int64_t N, int64_t K);
+
 
 
 /* Quantized KV cache (llama.cpp's -ctk / -ctv q8_0, q4_0).
@@ -526,6 +539,11 @@ int mi355_moe_weights(void *stream, const float *probs, const int32_t *ids, int6
                       int64_t n_expert, int64_t n_used, int64_t T);
 int mi355_moe_combine(void *stream, const float *experts, const float *weights, float *scaled, const float *residual, float *out,
                       int64_t n_embd, int64_t n_used, int64_t T);
+/* moe_weights and moe_combine in one launch (a few tokens): the same outputs with the same bits.  raw, sum and norm may be NULL (all
+ * three) when nothing else reads the weights; nothing the launch writes may overlap probs or ids. */
+int mi355_moe_weights_combine(void *stream, const float *probs, const int32_t *ids, int64_t ids_stride, float *raw, float *sum, float *norm,
+                              int64_t n_expert, const float *experts, float *scaled, const float *residual, float *out, int64_t n_embd, int64_t n_used,
+                              int64_t T);
 
 /* MUL_MAT with f32 or f16 src0 and f32 src1 (router / small dense matrices): dst[b][n] = sum_k W[n][k] x[b][k], strides honoured, ne2/ne3 broadcast */
 int mi355_mul_mat_f(void *stream, const mi355_tensor *src0, const mi355_tensor *src1, const mi355_tensor *dst);

@@ -1184,6 +1184,26 @@ bool feeds_quant_mmid(const graph_walk & w, int i, const void * data, int64_t K,
     return b->data == data && b->ne[0] == K && b->ne[1] * b->ne[2] == rows && K % 32 == 0;
 }
 
+// Is the tensor at `data` first read by an f32 MUL_MAT (the router of a mixture-of-experts layer) and, a few nodes later, by a
+// MUL_MAT_ID that takes its rows quantized to Q8_1?  Nothing in between may take the activation slots: only the router's own chain
+// (SOFT_MAX, ARGSORT, GET_ROWS, SUM_ROWS, DIV and views) is accepted there.
+bool router_then_quant_mmid(const graph_walk & w, int i, const void * data, int64_t K, int64_t rows) {
+    int j = w.next(i);
+    if (j >= w.n || w.nodes[j]->op != GGML_OP_MUL_MAT || w.nodes[j]->src[0]->type != GGML_TYPE_F32 || w.nodes[j]->src[1]->data != data) return false;
+    for (int k = 0; k < 8; k++) {
+        j = w.next(j);
+        if (j >= w.n) return false;
+        const ggml_tensor * op = w.nodes[j];
+        if (op->op == GGML_OP_MUL_MAT_ID) {
+            const ggml_tensor * b = op->src[1];
+            return !mmid_uses_tiles(op) && b->data == data && b->ne[0] == K && b->ne[1] * b->ne[2] == rows && K % 32 == 0;
+        }
+        if (op->op != GGML_OP_SOFT_MAX && op->op != GGML_OP_ARGSORT && op->op != GGML_OP_GET_ROWS && op->op != GGML_OP_SUM_ROWS && op->op != GGML_OP_DIV)
+            return false;
+    }
+    return false;
+}
+
 // Do the bytes of two tensors intersect?  A pattern that runs a node ahead of its place in the graph must check this: the
 // graph allocator reuses the memory of a tensor once its last reader, in graph order, has run, so a node that comes later may
 // write where an earlier, not yet executed node still has to read.
@@ -1497,6 +1517,114 @@ prefill_qkv match_prefill_qkv(const graph_walk & w, int i) {
     return p;
 }
 
+// SOFT_MAX (no mask, scale 1) at node i followed by ARGSORT(descending) of its result: expert probabilities and their order
+struct moe_route_match {
+    bool ok = false;
+    int j_argsort = -1;
+};
+moe_route_match match_moe_route(const graph_walk & w, int i) {
+    moe_route_match r;
+    const ggml_tensor * node = w.nodes[i];
+    const int j = w.next(i);
+    const ggml_tensor * nxt = j < w.n ? w.nodes[j] : nullptr;
+    if (node->op != GGML_OP_SOFT_MAX || node->src[1] || !nxt || nxt->op != GGML_OP_ARGSORT || nxt->src[0] != node) return r;
+    float scale, max_bias;
+    memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
+    memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
+    const ggml_tensor * x = node->src[0];
+    r.ok = scale == 1.0f && max_bias == 0.0f && x->ne[0] <= 64 && x->type == GGML_TYPE_F32 && ggml_is_contiguous(x) && ggml_is_contiguous(node) &&
+           ggml_is_contiguous(nxt) && nxt->type == GGML_TYPE_I32 && ((const int32_t *) nxt->op_params)[0] == GGML_SORT_ORDER_DESC;
+    r.j_argsort = j;
+    return r;
+}
+
+// GET_ROWS(probabilities of the selected experts) at node i -> SUM_ROWS -> DIV: normalised expert weights
+struct moe_weights_match {
+    bool ok = false;
+    int last = -1;
+    const ggml_tensor * probs = nullptr, * ids = nullptr, * raw = nullptr, * sum = nullptr, * div = nullptr;
+    int64_t n_expert = 0, n_used = 0, T = 0, ids_stride = 0;
+};
+moe_weights_match match_moe_weights(const graph_walk & w, int i) {
+    moe_weights_match m;
+    const ggml_tensor * node = w.nodes[i];
+    const int j = w.next(i);
+    const ggml_tensor * nxt = j < w.n ? w.nodes[j] : nullptr;
+    if (node->op != GGML_OP_GET_ROWS || !nxt || nxt->op != GGML_OP_SUM_ROWS) return m;
+    const ggml_tensor * probs = node->src[0];   // [1, n_expert, T]
+    const ggml_tensor * ids = node->src[1];     // [n_used, T]
+    const int jd = w.next(j);
+    const ggml_tensor * div = jd < w.n ? w.nodes[jd] : nullptr;
+    const ggml_tensor * w2d = nxt->src[0];       // [n_used, T] reshape of the GET_ROWS result
+    const int64_t n_expert = probs->ne[1], T = probs->ne[2], n_used = ids->ne[0];
+    m.ok = div && div->op == GGML_OP_DIV && div->src[0] == w2d && div->src[1] == nxt && w2d->op == GGML_OP_RESHAPE && w2d->src[0] == node &&
+           probs->type == GGML_TYPE_F32 && probs->ne[0] == 1 && probs->ne[3] == 1 && ggml_is_contiguous(probs) && ids->type == GGML_TYPE_I32 &&
+           ids->nb[0] == sizeof(int32_t) && ids->ne[1] == T && ids->ne[2] == 1 && ids->ne[3] == 1 && n_used <= 64 && n_used <= n_expert &&
+           ggml_is_contiguous(node) && node->ne[0] == 1 && node->ne[1] == n_used && node->ne[2] == T && ggml_is_contiguous(w2d) &&
+           ggml_is_contiguous(nxt) && ggml_is_contiguous(div) && w2d->ne[0] == n_used && w2d->ne[1] == T && ggml_nelements(nxt) == T;
+    m.last = jd;
+    m.probs = probs; m.ids = ids; m.raw = node; m.sum = nxt; m.div = div;
+    m.n_expert = n_expert; m.n_used = n_used; m.T = T;
+    m.ids_stride = (int64_t) (ids->nb[1] / sizeof(int32_t));
+    return m;
+}
+
+// MUL(expert outputs, weights) at node i -> ADD over the expert slots [-> ADD(residual)]: weighted sum of the selected experts
+struct moe_combine_match {
+    bool ok = false;
+    int last = -1;
+    const ggml_tensor * ex = nullptr, * wt = nullptr, * out = nullptr;
+    const float * residual = nullptr;
+    int64_t n_embd = 0, n_used = 0, T = 0;
+};
+moe_combine_match match_moe_combine(const graph_walk & w, int i) {
+    moe_combine_match c;
+    const ggml_tensor * node = w.nodes[i];
+    const int j = w.next(i);
+    const ggml_tensor * nxt = j < w.n ? w.nodes[j] : nullptr;
+    if (node->op != GGML_OP_MUL || node->ne[1] < 2 || node->ne[1] > 64 || node->ne[3] != 1 || !nxt || nxt->op != GGML_OP_ADD) return c;
+    const ggml_tensor * ex = node->src[0];
+    const ggml_tensor * wt = node->src[1];
+    const int64_t n_embd = node->ne[0], n_used = node->ne[1], T = node->ne[2];
+    auto slot_view = [&](const ggml_tensor * v, int64_t e) {
+        return v && v->op == GGML_OP_VIEW && v->view_src == node && v->view_offs == (size_t) e * node->nb[1] && v->ne[0] == n_embd && v->ne[1] == T &&
+               v->ne[2] == 1 && v->ne[3] == 1 && v->nb[1] == node->nb[2] && v->nb[0] == sizeof(float);
+    };
+    bool ok = ex->type == GGML_TYPE_F32 && wt->type == GGML_TYPE_F32 && ggml_are_same_shape(ex, node) && ggml_is_contiguous(ex) && ggml_is_contiguous(node) &&
+              ggml_is_contiguous(wt) && wt->ne[0] == 1 && wt->ne[1] == n_used && wt->ne[2] == T && wt->ne[3] == 1 && n_embd % 4 == 0 && T <= 65535 &&
+              (((uintptr_t) ex->data | (uintptr_t) node->data) & 15) == 0;
+    int k = j;   // the ADD chain: ((slot0 + slot1) + slot2) + ...
+    const ggml_tensor * sum = nullptr;
+    for (int64_t e = 1; ok && e < n_used; e++) {
+        const ggml_tensor * add = k < w.n ? w.nodes[k] : nullptr;
+        ok = add && add->op == GGML_OP_ADD && slot_view(add->src[1], e) && (e == 1 ? slot_view(add->src[0], 0) : add->src[0] == sum) &&
+             ggml_is_contiguous(add) && add->type == GGML_TYPE_F32 && ((uintptr_t) add->data & 15) == 0;
+        if (ok && e + 1 < n_used) ok = w.sole_use(k);   // intermediate sums are not materialised
+        if (ok) {
+            sum = add;
+            if (e + 1 < n_used) k = w.next(k);
+        }
+    }
+    if (!ok) return c;
+    c.last = k;
+    c.out = sum;
+    const int jr = w.next(k);
+    const ggml_tensor * radd = jr < w.n ? w.nodes[jr] : nullptr;
+    if (radd && radd->op == GGML_OP_ADD && w.sole_use(k) && (radd->src[0] == sum || radd->src[1] == sum)) {
+        const ggml_tensor * res = radd->src[0] == sum ? radd->src[1] : radd->src[0];
+        if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, sum) && ggml_is_contiguous(res) && ggml_is_contiguous(radd) &&
+            (((uintptr_t) res->data | (uintptr_t) radd->data) & 15) == 0) {
+            c.residual = (const float *) res->data;
+            c.out = radd;
+            c.last = jr;
+        }
+    }
+    c.ok = true;
+    c.ex = ex; c.wt = wt;
+    c.n_embd = n_embd; c.n_used = n_used; c.T = T;
+    return c;
+}
+
 // Runs node i and possibly a few of its successors; returns the index of the last node consumed.
 int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     hipStream_t s = ctx->stream;
@@ -1590,6 +1718,8 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 return j;
             }
             if (rows <= 32 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
+            // a mixture-of-experts layer: the f32 router product comes first, the experts' MUL_MAT_ID then reads the same rows quantized
+            else if (rows <= 8 && router_then_quant_mmid(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
             MI355_K_OK(mi355_rms_norm_mul_quant(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
             ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
             return j;
@@ -1641,6 +1771,42 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             }
         }
     }
+    // ---- MUL_MAT_ID(up) -> MUL_MAT_ID(gate) -> UNARY(SILU) -> MUL -> [MUL_MAT_ID(down) by GEMV] (llm_build_moe_ffn, one to a few tokens):
+    //      one launch for both expert products, SiLU * up and the Q8_1 rows the down experts read; the f32 product is not materialised
+    if (node->op == GGML_OP_MUL_MAT_ID && nxt && nxt->op == GGML_OP_MUL_MAT_ID && !mmid_uses_tiles(node) && w.sole_use(i) && w.sole_use(j)) {
+        const ggml_tensor * up = node, * gate = nxt;
+        const int js = w.next(j), jm = js < w.n ? w.next(js) : w.n;
+        if (jm < w.n) {
+            const ggml_tensor * silu = w.nodes[js], * mul = w.nodes[jm];
+            const ggml_tensor * as_up = up->src[0], * as_gate = gate->src[0], * b = up->src[1], * ids = up->src[2];
+            const int64_t K = as_up->ne[0], N = as_up->ne[1], n_expert = as_up->ne[2];
+            const int64_t nb1 = b->ne[1], T = b->ne[2], n_used = ids->ne[0], slots = n_used * T;
+            const bool chain = silu->op == GGML_OP_UNARY && ggml_get_unary_op(silu) == GGML_UNARY_OP_SILU && silu->src[0] == gate && w.sole_use(js) &&
+                               mul->op == GGML_OP_MUL && ((mul->src[0] == silu && mul->src[1] == up) || (mul->src[1] == silu && mul->src[0] == up)) &&
+                               w.sole_use(jm) && ggml_is_contiguous(mul) && mul->type == GGML_TYPE_F32 && ggml_are_same_shape(mul, up) &&
+                               ggml_are_same_shape(gate, up) && ggml_is_contiguous(up) && ggml_is_contiguous(gate) && ggml_is_contiguous(silu);
+            if (chain && gate->src[1]->data == b->data && ggml_are_same_shape(gate->src[1], b) && gate->src[2] == ids && as_gate->type == as_up->type &&
+                ggml_are_same_shape(as_gate, as_up) && ((uintptr_t) b->data & 15) == 0 && slots <= 8 && nb1 * T <= 8 && b->type == GGML_TYPE_F32 &&
+                ggml_is_contiguous(b) && ids->type == GGML_TYPE_I32 && !bytes_overlap(up, gate) && feeds_quant_mmid(w, jm, mul->data, N, slots) &&
+                mi355_moe_gate_up_swiglu_supported(to_mi355_type(as_up->type), as_gate->data, as_up->data, N, K)) {
+                const int64_t rows = nb1 * T;
+                const size_t in_bytes = mi355_act_bytes(K, rows), out_bytes = mi355_act_bytes(N, slots);
+                ctx->act_reserve(in_bytes > out_bytes ? in_bytes : out_bytes);
+                if (!ctx->cached(b->data, K, rows, ACT_Q8_1)) {
+                    void * fresh = ctx->act_slot(in_bytes);
+                    MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, rows, K));
+                    ctx->cache = act_cache{b->data, K, rows, ACT_Q8_1, true, fresh};
+                }
+                const void * act_in = ctx->cache.ptr;
+                void * act_out = ctx->act_slot(out_bytes, true);
+                MI355_K_OK(mi355_moe_gate_up_swiglu(s, to_mi355_type(as_up->type), as_gate->data, as_up->data, act_in, (const int32_t *) ids->data,
+                                                    (int64_t) (ids->nb[1] / sizeof(int32_t)), (float *) gate->data, (float *) up->data, act_out, N, K, n_expert,
+                                                    n_used, nb1, T));
+                ctx->cache = act_cache{mul->data, N, slots, ACT_Q8_1, true, act_out};
+                return jm;
+            }
+        }
+    }
     // ---- MUL_MAT_ID: the quantized rows of src1 are shared by consecutive products (up and gate experts read the same rows)
     if (node->op == GGML_OP_MUL_MAT_ID) {
         const ggml_tensor * as = node->src[0];
@@ -1674,82 +1840,64 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         }
     }
     // ---- SOFT_MAX -> ARGSORT(descending): expert probabilities and their order (llm_build_moe_ffn)
-    if (node->op == GGML_OP_SOFT_MAX && !node->src[1] && nxt && nxt->op == GGML_OP_ARGSORT && nxt->src[0] == node) {
-        float scale, max_bias;
-        memcpy(&scale, (const float *) node->op_params + 0, sizeof(float));
-        memcpy(&max_bias, (const float *) node->op_params + 1, sizeof(float));
-        const ggml_tensor * x = node->src[0];
-        if (scale == 1.0f && max_bias == 0.0f && x->ne[0] <= 64 && x->type == GGML_TYPE_F32 && ggml_is_contiguous(x) && ggml_is_contiguous(node) &&
-            ggml_is_contiguous(nxt) && nxt->type == GGML_TYPE_I32 && ((const int32_t *) nxt->op_params)[0] == GGML_SORT_ORDER_DESC) {
+    if (node->op == GGML_OP_SOFT_MAX) {
+        const moe_route_match r = match_moe_route(w, i);
+        if (r.ok) {
+            const ggml_tensor * x = node->src[0];
             ctx->note_write(node->data, ggml_nbytes(node));
-            MI355_K_OK(mi355_moe_route(s, (const float *) x->data, (float *) node->data, (int32_t *) nxt->data, x->ne[0], ggml_nrows(x)));
-            return j;
+            MI355_K_OK(mi355_moe_route(s, (const float *) x->data, (float *) node->data, (int32_t *) w.nodes[r.j_argsort]->data, x->ne[0], ggml_nrows(x)));
+            return r.j_argsort;
         }
     }
-    // ---- GET_ROWS(probabilities of the selected experts) -> SUM_ROWS -> DIV: normalised expert weights
-    if (node->op == GGML_OP_GET_ROWS && nxt && nxt->op == GGML_OP_SUM_ROWS) {
-        const ggml_tensor * probs = node->src[0];   // [1, n_expert, T]
-        const ggml_tensor * ids = node->src[1];     // [n_used, T]
-        const int jd = w.next(j);
-        const ggml_tensor * div = jd < w.n ? w.nodes[jd] : nullptr;
-        const ggml_tensor * w2d = nxt->src[0];       // [n_used, T] reshape of the GET_ROWS result
-        const int64_t n_expert = probs->ne[1], T = probs->ne[2], n_used = ids->ne[0];
-        if (div && div->op == GGML_OP_DIV && div->src[0] == w2d && div->src[1] == nxt && w2d->op == GGML_OP_RESHAPE && w2d->src[0] == node &&
-            probs->type == GGML_TYPE_F32 && probs->ne[0] == 1 && probs->ne[3] == 1 && ggml_is_contiguous(probs) && ids->type == GGML_TYPE_I32 &&
-            ids->nb[0] == sizeof(int32_t) && ids->ne[1] == T && ids->ne[2] == 1 && ids->ne[3] == 1 && n_used <= 64 && n_used <= n_expert &&
-            ggml_is_contiguous(node) && node->ne[0] == 1 && node->ne[1] == n_used && node->ne[2] == T && ggml_is_contiguous(w2d) &&
-            ggml_is_contiguous(nxt) && ggml_is_contiguous(div) && w2d->ne[0] == n_used && w2d->ne[1] == T && ggml_nelements(nxt) == T) {
-            ctx->note_write(node->data, ggml_nbytes(node));
-            ctx->note_write(div->data, ggml_nbytes(div));
-            MI355_K_OK(mi355_moe_weights(s, (const float *) probs->data, (const int32_t *) ids->data, (int64_t) (ids->nb[1] / sizeof(int32_t)),
-                                         (float *) node->data, (float *) nxt->data, (float *) div->data, n_expert, n_used, T));
-            return jd;
+    // ---- GET_ROWS(probabilities of the selected experts) -> SUM_ROWS -> DIV: normalised expert weights; with the weighted sum of the
+    //      experts' outputs right behind them (a few tokens), both in one launch
+    if (node->op == GGML_OP_GET_ROWS) {
+        const moe_weights_match m = match_moe_weights(w, i);
+        if (m.ok) {
+            const int jc = w.next(m.last);
+            const moe_combine_match c = jc < w.n ? match_moe_combine(w, jc) : moe_combine_match();
+            ctx->note_write(m.raw->data, ggml_nbytes(m.raw));
+            ctx->note_write(m.div->data, ggml_nbytes(m.div));
+            // One launch for both when the weighted sum is the only reader of the weights (GET_ROWS, SUM_ROWS and DIV results are then not
+            // materialised: the allocator has often lent their memory to the sum's own operands by now, e.g. SUM_ROWS' result lies on
+            // the probabilities, or the sum on SUM_ROWS' result) and the sum's outputs do not lie on the probabilities or the ids, which
+            // every group reads.
+            bool one_launch = c.ok && c.wt->data == m.div->data && c.n_used == m.n_used && c.T == m.T && m.T <= 8 && w.sole_use(i) && w.sole_use(w.next(i)) &&
+                              w.sole_use(m.last);
+            if (one_launch) {
+                const ggml_tensor * mul = w.nodes[jc];
+                for (int k = i + 1; k < jc; k++) {   // the reshapes in between: [n_used, T] read by SUM_ROWS and DIV, [1, n_used, T] read by the MUL
+                    const ggml_tensor * t = w.nodes[k];
+                    if (!is_noop(t)) continue;
+                    if (t == m.sum->src[0]) one_launch = one_launch && w.uses[k] == 2 && !(t->flags & GGML_TENSOR_FLAG_OUTPUT);
+                    else if (t == c.wt) one_launch = one_launch && w.sole_use(k);
+                }
+                for (const ggml_tensor * in : {m.probs, m.ids})
+                    for (const ggml_tensor * o : {mul, c.out}) one_launch = one_launch && !bytes_overlap(in, o);
+            }
+            if (one_launch) {
+                const ggml_tensor * mul = w.nodes[jc];
+                ctx->note_write(mul->data, ggml_nbytes(mul));
+                ctx->note_write(c.out->data, ggml_nbytes(c.out));
+                MI355_K_OK(mi355_moe_weights_combine(s, (const float *) m.probs->data, (const int32_t *) m.ids->data, m.ids_stride, nullptr, nullptr, nullptr,
+                                                     m.n_expert, (const float *) c.ex->data, (float *) mul->data, c.residual, (float *) c.out->data, c.n_embd, c.n_used,
+                                                     c.T));
+                return c.last;
+            }
+            MI355_K_OK(mi355_moe_weights(s, (const float *) m.probs->data, (const int32_t *) m.ids->data, m.ids_stride, (float *) m.raw->data,
+                                         (float *) m.sum->data, (float *) m.div->data, m.n_expert, m.n_used, m.T));
+            return m.last;
         }
     }
     // ---- MUL(expert outputs, weights) -> ADD over the expert slots [-> ADD(residual)]: weighted sum of the selected experts
-    if (node->op == GGML_OP_MUL && node->ne[1] >= 2 && node->ne[1] <= 64 && node->ne[3] == 1 && nxt && nxt->op == GGML_OP_ADD) {
-        const ggml_tensor * ex = node->src[0];
-        const ggml_tensor * wt = node->src[1];
-        const int64_t n_embd = node->ne[0], n_used = node->ne[1], T = node->ne[2];
-        auto slot_view = [&](const ggml_tensor * v, int64_t e) {
-            return v && v->op == GGML_OP_VIEW && v->view_src == node && v->view_offs == (size_t) e * node->nb[1] && v->ne[0] == n_embd && v->ne[1] == T &&
-                   v->ne[2] == 1 && v->ne[3] == 1 && v->nb[1] == node->nb[2] && v->nb[0] == sizeof(float);
-        };
-        bool ok = ex->type == GGML_TYPE_F32 && wt->type == GGML_TYPE_F32 && ggml_are_same_shape(ex, node) && ggml_is_contiguous(ex) && ggml_is_contiguous(node) &&
-                  ggml_is_contiguous(wt) && wt->ne[0] == 1 && wt->ne[1] == n_used && wt->ne[2] == T && wt->ne[3] == 1 && n_embd % 4 == 0 && T <= 65535 &&
-                  (((uintptr_t) ex->data | (uintptr_t) node->data) & 15) == 0;
-        int k = j;   // the ADD chain: ((slot0 + slot1) + slot2) + ...
-        const ggml_tensor * sum = nullptr;
-        for (int64_t e = 1; ok && e < n_used; e++) {
-            const ggml_tensor * add = k < w.n ? w.nodes[k] : nullptr;
-            ok = add && add->op == GGML_OP_ADD && slot_view(add->src[1], e) && (e == 1 ? slot_view(add->src[0], 0) : add->src[0] == sum) &&
-                 ggml_is_contiguous(add) && add->type == GGML_TYPE_F32 && ((uintptr_t) add->data & 15) == 0;
-            if (ok && e + 1 < n_used) ok = w.sole_use(k);   // intermediate sums are not materialised
-            if (ok) {
-                sum = add;
-                if (e + 1 < n_used) k = w.next(k);
-            }
-        }
-        if (ok) {
-            int last = k;
-            const ggml_tensor * out = sum;
-            const float * residual = nullptr;
-            const int jr = w.next(k);
-            const ggml_tensor * radd = jr < w.n ? w.nodes[jr] : nullptr;
-            if (radd && radd->op == GGML_OP_ADD && w.sole_use(k) && (radd->src[0] == sum || radd->src[1] == sum)) {
-                const ggml_tensor * res = radd->src[0] == sum ? radd->src[1] : radd->src[0];
-                if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, sum) && ggml_is_contiguous(res) && ggml_is_contiguous(radd) &&
-                    (((uintptr_t) res->data | (uintptr_t) radd->data) & 15) == 0) {
-                    residual = (const float *) res->data;
-                    out = radd;
-                    last = jr;
-                }
-            }
+    if (node->op == GGML_OP_MUL) {
+        const moe_combine_match c = match_moe_combine(w, i);
+        if (c.ok) {
             ctx->note_write(node->data, ggml_nbytes(node));
-            ctx->note_write(out->data, ggml_nbytes(out));
-            MI355_K_OK(mi355_moe_combine(s, (const float *) ex->data, (const float *) wt->data, (float *) node->data, residual, (float *) out->data, n_embd,
-                                         n_used, T));
-            return last;
+            ctx->note_write(c.out->data, ggml_nbytes(c.out));
+            MI355_K_OK(mi355_moe_combine(s, (const float *) c.ex->data, (const float *) c.wt->data, (float *) node->data, c.residual, (float *) c.out->data, c.n_embd,
+                                         c.n_used, c.T));
+            return c.last;
         }
     }
     // ---- FLASH_ATTN_EXT whose output feeds a quantized product

@@ -141,4 +141,39 @@ int launch_gate_up_blk(hipStream_t s, int type, const void *w_gate, const void *
     return launch_status("k_gemv_gate_up_blk");
 }
 
+// The same launch for the experts of a mixture-of-experts layer (llm_build_moe_ffn, src/llama.cpp:417-538: MUL_MAT_ID(up),
+// MUL_MAT_ID(gate), SILU, MUL): blockIdx.y = slot = t * n_used + e, the expert read on the device as k_gemv_id does, one activation
+// row per slot.  gate / up: f32 [slots][N]; the quantized product: rows of N per slot.
+template <int TYPE, int WAVES, int R>
+__global__ void __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4, 8)))
+k_gemv_gate_up_blk_id(const uint8_t *__restrict__ as_gate, const uint8_t *__restrict__ as_up, const int8_t *__restrict__ aq, const act_ds *__restrict__ ads,
+                      const int32_t *__restrict__ ids, int64_t ids_stride, int K, float *__restrict__ gate, float *__restrict__ up,
+                      int8_t *__restrict__ act_q, act_ds *__restrict__ act_s, int n, int64_t n_expert, int64_t n_used, int64_t nb1) {
+    __shared__ float s_g[1][32], s_u[1][32];
+    const int64_t slot = blockIdx.y, t = slot / n_used, e = slot % n_used;
+    int64_t ex = ids[t * ids_stride + e];
+    ex = ex < 0 ? 0 : (ex >= n_expert ? n_expert - 1 : ex);   // never index outside the expert stack
+    const int64_t arow = t * nb1 + e % nb1;
+    const row_layout L = make_row_layout(TYPE, K);
+    const int64_t expert_bytes = (int64_t)n * L.row_bytes;
+    gate_up_blk_phase<TYPE, 1, WAVES, R, false>(as_gate + ex * expert_bytes, as_up + ex * expert_bytes, aq + arow * K, ads + arow * (K >> 5), K,
+                                                gate + slot * n, up + slot * n, n, act_q + slot * n, act_s + slot * (n >> 5), n, s_ffn_dyn, s_g, s_u);
+}
+
+int launch_gate_up_blk_id(hipStream_t s, int type, const void *as_gate, const void *as_up, const int8_t *aq, const act_ds *ads, const int32_t *ids,
+                          int64_t ids_stride, int64_t K, float *gate, float *up, void *act_out, int64_t N, int64_t n_expert, int64_t n_used, int64_t nb1,
+                          int64_t T) {
+    const size_t lds = (size_t)(K + K / 4);
+    const int64_t slots = n_used * T;
+    int8_t *oq = (int8_t *)act_out;
+    act_ds *os = (act_ds *)(oq + slots * N);
+    const dim3 grid((unsigned)(N / 32), (unsigned)slots);
+#define MI355_BLK_ID_LAUNCH(TY)                                                                                                                          \
+    MI355_LAUNCH((k_gemv_gate_up_blk_id<TY, GU_WAVES, gu_rows_in_flight(TY)>), grid, dim3(64 * GU_WAVES), lds, s, (const uint8_t *)as_gate,              \
+                 (const uint8_t *)as_up, aq, ads, ids, ids_stride, (int)K, gate, up, oq, os, (int)N, n_expert, n_used, nb1);
+    MI355_WEIGHT_TYPE_SWITCH(type, MI355_BLK_ID_LAUNCH)
+#undef MI355_BLK_ID_LAUNCH
+    return launch_status("k_gemv_gate_up_blk_id");
+}
+
 }  // namespace mi355

@@ -1006,6 +1006,28 @@ int mi355_mul_mat_id_vec(void *stream, int type, const void *as, const void *act
     return launch_status("k_gemv_id");
 }
 
+int mi355_moe_gate_up_swiglu_supported(int type, const void *as_gate, const void *as_up, int64_t N, int64_t K) {
+    if (!is_weight_type(type) || N <= 0 || N % 32 != 0 || N / 32 >= 0x7fffffff || K <= 0 || K > 32768 || K % 64 != 0 || K % type_block_elems(type) != 0) return 0;
+    const row_layout L = make_row_layout(type, K);
+    return layout_aligned(as_gate, L) && layout_aligned(as_up, L) ? 1 : 0;
+}
+
+int mi355_moe_gate_up_swiglu(void *stream, int type, const void *as_gate, const void *as_up, const void *act, const int32_t *ids, int64_t ids_stride,
+                             float *gate, float *up, void *act_out, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T) {
+    MI355_REQUIRE(is_weight_type(type), "moe_gate_up_swiglu: unsupported weight type %d", type);
+    MI355_REQUIRE(N > 0 && N % 32 == 0 && N / 32 < 0x7fffffff && K > 0 && K <= 32768 && n_expert > 0 && n_used > 0 && nb1 > 0 && T > 0,
+                  "moe_gate_up_swiglu: bad shape (N must be a multiple of 32, K at most 32768)");
+    MI355_REQUIRE(K % type_block_elems(type) == 0 && K % 64 == 0, "moe_gate_up_swiglu: K=%lld must be a multiple of the block size and of 64", (long long)K);
+    MI355_REQUIRE(n_used * T <= 65535, "moe_gate_up_swiglu: too many expert slots for one launch");
+    MI355_REQUIRE(ids != nullptr && gate != nullptr && up != nullptr && ((uintptr_t)act & 15) == 0 && ((uintptr_t)act_out & 15) == 0,
+                  "moe_gate_up_swiglu: misaligned or missing operands");
+    const row_layout L = make_row_layout(type, K);
+    MI355_REQUIRE(layout_aligned(as_gate, L) && layout_aligned(as_up, L), "moe_gate_up_swiglu: expert rows must be 16-byte aligned");
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + nb1 * T * K);
+    return launch_gate_up_blk_id((hipStream_t)stream, type, as_gate, as_up, aq, ads, ids, ids_stride, K, gate, up, act_out, N, n_expert, n_used, nb1, T);
+}
+
 int mi355_block_dots_q8_1(void *stream, int type, const void *W, const void *a, int32_t *out, int64_t N, int64_t K) {
     int rc = check_gemv_args("block_dots", type, W, N, K, N);
     if (rc != MI355_OK) return rc;

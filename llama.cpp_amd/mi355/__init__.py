@@ -106,6 +106,8 @@ _SIGNATURES = {
                             _f, _f, _f, _f, _f, _f]),
     "mi355_rope_kv_store_typed": (_int, [_p, _p, _p, _p, _int, _p, _i64, _i64, _int, _p, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _int, _int, _int,
                                   _f, _f, _f, _f, _f, _f]),
+    "mi355_moe_gate_up_swiglu_supported": (_int, [_int, _p, _p, _i64, _i64]),
+    "mi355_moe_gate_up_swiglu": (_int, [_p, _int, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64]),
     "mi355_ffn_gate_up_swiglu": (_int, [_p, _int, _p, _int, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_vec_q_rope": (_int, [_p, _int, _p, _p, _i64, _i64, _p]),
     "mi355_rms_norm_mul_mat_vec_q_rope": (_int, [_p, _p, _p, _f, _int, _p, _i64, _p]),
@@ -120,6 +122,7 @@ _SIGNATURES = {
     "mi355_mul_mat_id_q8k": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_moe_route": (_int, [_p, _p, _p, _p, _i64, _i64]),
     "mi355_moe_weights": (_int, [_p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64]),
+    "mi355_moe_weights_combine": (_int, [_p, _p, _p, _i64, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64]),
     "mi355_moe_combine": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_id_vec": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64]),
     "mi355_flash_attn_ws_bytes": (_sz, [_i64, _i64, _i64, _i64]),

@@ -90,3 +90,74 @@ def test_combine_equals_separate_nodes(dev, n_embd, n_used, T, residual):
     assert torch.equal(scaled2, scaled) and torch.equal(out2, acc)
     want = (experts.double() * weights.double()).sum(1) + (res.double() if residual else 0)
     assert orc.nmse(out2.cpu().numpy(), want.cpu().numpy()) < 1e-7
+
+
+@pytest.mark.parametrize("name,t", [("q4_K", orc.Q4_K), ("q6_K", orc.Q6_K), ("q5_K", orc.Q5_K), ("q8_0", orc.Q8_0), ("q4_0", orc.Q4_0), ("iq4_nl", orc.IQ4_NL)])
+@pytest.mark.parametrize("n_expert,n_used,T,N,K", [(8, 2, 1, 512, 4096), (8, 2, 3, 256, 2048), (4, 4, 2, 96, 1024)])
+def test_expert_gate_up_swiglu_equals_separate_launches(dev, name, t, n_expert, n_used, T, N, K):
+    """MUL_MAT_ID(up), MUL_MAT_ID(gate), SILU, MUL and the Q8_1 rows for the down experts in one launch: the bits of
+    mi355_mul_mat_id_vec twice followed by mi355_swiglu_quant."""
+    import torch
+    import mi355
+    lib = mi355.load()
+    rng = np.random.default_rng(n_expert + T + N)
+    stacks = []
+    for _ in range(2):
+        Wq = orc.quantize("oracle", t, (rng.standard_normal((n_expert * N, K)) * 0.05).astype(np.float32))
+        stacks.append(mi355.upload_weights(t, torch.from_numpy(Wq).to(dev)))
+    as_gate, as_up = stacks
+    x = torch.from_numpy(rng.standard_normal((T, K)).astype(np.float32)).to(dev)
+    act = mi355.quantize_act(x)
+    ids_full = torch.from_numpy(np.stack([rng.permutation(n_expert) for _ in range(T)]).astype(np.int32)).to(dev)
+    ids = ids_full[:, :n_used]
+    slots = T * n_used
+    if t == orc.Q6_K and K % 2048 != 0:   # its rows are 16-byte aligned only when K is a multiple of 2048: the caller keeps the separate launches
+        assert lib.mi355_moe_gate_up_swiglu_supported(t, as_gate.data_ptr(), as_up.data_ptr(), N, K) == 0
+        return
+    assert lib.mi355_moe_gate_up_swiglu_supported(t, as_gate.data_ptr(), as_up.data_ptr(), N, K) == 1
+    g0, u0 = torch.zeros(slots, N, device=dev), torch.zeros(slots, N, device=dev)
+    for W, out in ((as_gate, g0), (as_up, u0)):
+        mi355.check(lib.mi355_mul_mat_id_vec(None, t, W.data_ptr(), act.data_ptr(), ids.data_ptr(), ids.stride(0), out.data_ptr(), N, K, n_expert, n_used, 1, T))
+    a0 = torch.zeros(int(lib.mi355_act_bytes(N, slots)), dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_swiglu_quant(None, g0.data_ptr(), u0.data_ptr(), N, None, 0, a0.data_ptr(), N, slots))
+    g1, u1, a1 = torch.zeros_like(g0), torch.zeros_like(u0), torch.zeros_like(a0)
+    mi355.check(lib.mi355_moe_gate_up_swiglu(None, t, as_gate.data_ptr(), as_up.data_ptr(), act.data_ptr(), ids.data_ptr(), ids.stride(0), g1.data_ptr(),
+                                             u1.data_ptr(), a1.data_ptr(), N, K, n_expert, n_used, 1, T))
+    torch.cuda.synchronize()
+    assert torch.equal(g1, g0) and torch.equal(u1, u0)
+    used = slots * N + slots * (N // 32) * 8
+    assert torch.equal(a1[:used], a0[:used])
+    assert g1.abs().sum().item() > 0 and a1[:slots * N].float().abs().sum().item() > 0
+
+
+@pytest.mark.parametrize("n_expert,n_embd,n_used,T,residual", [(8, 4096, 2, 1, True), (8, 2048, 2, 5, False), (16, 1024, 4, 8, True), (64, 4096, 6, 2, True)])
+def test_weights_combine_equals_the_two_launches(dev, n_expert, n_embd, n_used, T, residual):
+    import torch
+    import mi355
+    lib = mi355.load()
+    g = torch.Generator().manual_seed(n_embd + T + n_expert)
+    probs = torch.softmax(torch.randn(T, n_expert, generator=g) * 2, dim=1).to(dev)
+    order = torch.stack([torch.randperm(n_expert, generator=g) for _ in range(T)]).to(torch.int32).to(dev)
+    ids = order[:, :n_used]
+    experts = torch.randn(T, n_used, n_embd, generator=g).to(dev)
+    res = torch.randn(T, n_embd, generator=g).to(dev)
+    raw, tot, norm = torch.empty(T, n_used, device=dev), torch.empty(T, device=dev), torch.empty(T, n_used, device=dev)
+    mi355.check(lib.mi355_moe_weights(None, mi355._ptr(probs), mi355._ptr(ids), ids.stride(0), mi355._ptr(raw), mi355._ptr(tot), mi355._ptr(norm),
+                                      n_expert, n_used, T))
+    scaled, out = torch.empty_like(experts), torch.empty(T, n_embd, device=dev)
+    mi355.check(lib.mi355_moe_combine(None, mi355._ptr(experts), mi355._ptr(norm), mi355._ptr(scaled), mi355._ptr(res) if residual else None, mi355._ptr(out),
+                                      n_embd, n_used, T))
+    raw2, tot2, norm2 = torch.zeros_like(raw), torch.zeros_like(tot), torch.zeros_like(norm)
+    scaled2, out2 = torch.zeros_like(scaled), torch.zeros_like(out)
+    mi355.check(lib.mi355_moe_weights_combine(None, mi355._ptr(probs), mi355._ptr(ids), ids.stride(0), mi355._ptr(raw2), mi355._ptr(tot2), mi355._ptr(norm2),
+                                              n_expert, mi355._ptr(experts), mi355._ptr(scaled2), mi355._ptr(res) if residual else None, mi355._ptr(out2),
+                                              n_embd, n_used, T))
+    torch.cuda.synchronize()
+    assert torch.equal(raw2, raw) and torch.equal(tot2, tot) and torch.equal(norm2, norm)
+    assert torch.equal(scaled2, scaled) and torch.equal(out2, out)
+    # the weights not materialised, the scaled outputs in place on the experts' (what the plug-in launches)
+    ex3, out3 = experts.clone(), torch.zeros_like(out)
+    mi355.check(lib.mi355_moe_weights_combine(None, mi355._ptr(probs), mi355._ptr(ids), ids.stride(0), None, None, None, n_expert, mi355._ptr(ex3), mi355._ptr(ex3),
+                                              mi355._ptr(res) if residual else None, mi355._ptr(out3), n_embd, n_used, T))
+    torch.cuda.synchronize()
+    assert torch.equal(ex3, scaled) and torch.equal(out3, out)
