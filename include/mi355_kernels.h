@@ -371,6 +371,13 @@ int mi355_argsort(void *stream, const mi355_tensor *src, const mi355_tensor *dst
  * x f32 rows of k (row stride x_stride elements), w f32 [k] or NULL, y f32 rows (y_stride). k <= 16384. */
 int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride,
                              void *act, int64_t k, int64_t nrows, float eps);
+/* The same for the FFN norm of a mixture-of-experts layer, continued with the router of llm_build_moe_ffn (src/llama.cpp:438-468):
+ * logits f32 [nrows][n_expert] = MUL_MAT(W f32 [n_expert] rows of k, stride w_stride elements; y), probs = SOFT_MAX(logits), order i32
+ * [nrows][n_expert] = ARGSORT(descending).  Same bits as mi355_rms_norm_mul_quant, mi355_mul_mat_f and mi355_moe_route one after the
+ * other.  k <= 4096, a few rows, n_expert <= 64; W 16-byte aligned. */
+int mi355_rms_norm_mul_quant_router(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act, int64_t k,
+                                    int64_t nrows, float eps, const float *W, int64_t w_stride, float *logits, float *probs, int32_t *order,
+                                    int64_t n_expert);
 /* llm_build_ffn LLM_FFN_SILU + LLM_FFN_PAR: UNARY(SILU)(gate) then MUL by up (src/llama.cpp:280-320; ggml-cpu.c:6646-6683). */
 int mi355_swiglu_quant(void *stream, const float *gate, const float *up, int64_t in_stride, float *y, int64_t y_stride, void *act,
                        int64_t k, int64_t nrows);

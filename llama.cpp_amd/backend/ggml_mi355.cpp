@@ -1625,6 +1625,17 @@ moe_combine_match match_moe_combine(const graph_walk & w, int i) {
     return c;
 }
 
+// The norm + router launch writes y, the logits, the probabilities and the order while it reads x, the norm weights and the router:
+// the later tensors must not lie on the earlier ones' memory (the soft-max may be in place on the logits, as in separate launches).
+bool router_outputs_apart(const ggml_tensor * x, const ggml_tensor * nw, const ggml_tensor * W, const ggml_tensor * y, const ggml_tensor * logits,
+                          const ggml_tensor * probs, const ggml_tensor * order) {
+    for (const ggml_tensor * in : {x, nw, W})
+        for (const ggml_tensor * o : {logits, probs, order})
+            if (bytes_overlap(in, o)) return false;
+    if (bytes_overlap(y, logits) || bytes_overlap(y, probs) || bytes_overlap(y, order) || bytes_overlap(order, logits) || bytes_overlap(order, probs)) return false;
+    return probs->data == logits->data || !bytes_overlap(probs, logits);
+}
+
 // Runs node i and possibly a few of its successors; returns the index of the last node consumed.
 int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     hipStream_t s = ctx->stream;
@@ -1719,7 +1730,26 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             }
             if (rows <= 32 && feeds_quant_gemv(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
             // a mixture-of-experts layer: the f32 router product comes first, the experts' MUL_MAT_ID then reads the same rows quantized
-            else if (rows <= 8 && router_then_quant_mmid(w, j, nxt->data, K, rows)) act = ctx->act_slot(mi355_act_bytes(K, rows));
+            else if (rows <= 8 && router_then_quant_mmid(w, j, nxt->data, K, rows)) {
+                act = ctx->act_slot(mi355_act_bytes(K, rows));
+                // ... and the router product, its soft-max and the order go out with the norm (one group per row has the row in registers)
+                const int jr = w.next(j);
+                const ggml_tensor * rt = w.nodes[jr];   // the MUL_MAT (router_then_quant_mmid)
+                const ggml_tensor * W = rt->src[0];
+                const int js = w.next(jr);
+                const moe_route_match r = js < w.n ? match_moe_route(w, js) : moe_route_match();
+                if (r.ok && w.nodes[js]->src[0] == rt && w.sole_use(jr) && K <= 4096 && W->ne[0] == K && W->ne[1] <= 64 && W->ne[2] == 1 && W->ne[3] == 1 &&
+                    W->nb[0] == sizeof(float) && W->nb[1] % 16 == 0 && ((uintptr_t) W->data & 15) == 0 && rt->src[1]->ne[1] == rows && rt->src[1]->ne[2] == 1 &&
+                    rt->src[1]->ne[3] == 1 && ggml_is_contiguous(rt) && rt->type == GGML_TYPE_F32 && rt->ne[0] == W->ne[1] && !(nxt->flags & GGML_TENSOR_FLAG_OUTPUT) &&
+                    router_outputs_apart(x, wt, W, nxt, rt, w.nodes[js], w.nodes[r.j_argsort])) {
+                    const ggml_tensor * sm = w.nodes[js], * as = w.nodes[r.j_argsort];
+                    MI355_K_OK(mi355_rms_norm_mul_quant_router(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps,
+                                                               (const float *) W->data, (int64_t) (W->nb[1] / sizeof(float)), (float *) rt->data, (float *) sm->data,
+                                                               (int32_t *) as->data, W->ne[1]));
+                    ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, true, act};
+                    return r.j_argsort;
+                }
+            }
             MI355_K_OK(mi355_rms_norm_mul_quant(s, (const float *) x->data, K, (const float *) wt->data, (float *) nxt->data, K, act, K, rows, eps));
             ctx->cache = act_cache{nxt->data, K, rows, ACT_Q8_1, act != nullptr, act};
             return j;

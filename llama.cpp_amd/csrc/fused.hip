@@ -11,6 +11,7 @@
 //   ROPE(q), ROPE(k), CPY(k -> cache), CPY(v -> cache)   k_rope_kv_store
 #include "common.hpp"
 #include "kv_blocks.hpp"
+#include "moe.hpp"
 #include "norm_quant.hpp"
 #include "q8k.hpp"
 #include "tiles.hpp"
@@ -25,6 +26,76 @@ __global__ void __launch_bounds__(256) k_rms_norm_mul_quant(const float *__restr
     __shared__ float sh[4];
     const int64_t row = blockIdx.x;
     rms_norm_quant_row<NV, FMT, false>(x + row * x_stride, w, y ? y + row * y_stride : nullptr, act, row, k, nrows, eps, sh);
+}
+
+// The FFN norm of a mixture-of-experts layer for a few tokens, continued with the router (llm_build_moe_ffn, src/llama.cpp:438-468):
+// logits[e] = W[e] . y for the row y the group has just normalised, then soft-max and the descending order.  A thread's pieces of y
+// are the pieces k_mul_mat_f (glue.hip) gives thread t of its 256-thread group - elements 4 t + 1024 i - and the sums are formed in
+// its order (the pieces in order, the wave, then the waves in order), so the logits hold the bits of that launch; the router's rows
+// are requested before the norm's own loads are waited for.  NE8: experts in rounds of eight.
+template <int NV>
+__global__ void __launch_bounds__(256) k_rms_norm_mul_quant_router(const float *__restrict__ x, int64_t x_stride, const float *__restrict__ w,
+                                                                   float *__restrict__ y, int64_t y_stride, void *__restrict__ act, int64_t k, int64_t nrows,
+                                                                   float eps, const float *__restrict__ W, int64_t w_stride, float *__restrict__ logits,
+                                                                   float *__restrict__ probs, int32_t *__restrict__ order, int n_expert) {
+    __shared__ float sh[4];
+    __shared__ float s_part[8][4];
+    __shared__ float s_logit[64];
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the first eight experts' rows: on their way before the norm waits for anything
+    f32x4 wpre[NV][8];
+#pragma unroll
+    for (int it = 0; it < NV; it++) {
+        const int64_t k0 = ((int64_t)it * 256 + tid) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            wpre[it][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (k0 < k && i < n_expert) wpre[it][i] = *(const f32x4 *)(W + (int64_t)i * w_stride + k0);
+        }
+    }
+    f32x4 yv[NV];
+    rms_norm_quant_row<NV, 0, false>(x + row * x_stride, w, y ? y + row * y_stride : nullptr, act, row, k, nrows, eps, sh, yv);
+    for (int e0 = 0; e0 < n_expert; e0 += 8) {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = 0.0f;
+#pragma unroll
+        for (int it = 0; it < NV; it++) {
+            const int64_t k0 = ((int64_t)it * 256 + tid) * 4;
+            if (k0 < k) {
+                const f32x4 x0 = yv[it];
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    if (e0 + i < n_expert) {
+                        const f32x4 w0 = e0 == 0 ? wpre[it][i] : *(const f32x4 *)(W + (int64_t)(e0 + i) * w_stride + k0);
+                        acc[i] += w0[0] * x0[0] + w0[1] * x0[1] + w0[2] * x0[2] + w0[3] * x0[3];
+                    }
+                }
+            }
+        }
+        __syncthreads();   // s_part of the previous round has been read
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float v = wave_sum(acc[i]);
+            if (lane == 0) s_part[i][wave] = v;
+        }
+        __syncthreads();
+        if (tid < 8 && e0 + tid < n_expert) {
+            float t = 0.0f;
+            for (int q = 0; q < 4; q++) t += s_part[tid][q];
+            s_logit[e0 + tid] = t;
+            logits[row * n_expert + e0 + tid] = t;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float p;
+    const int rank = moe_route_lane(lane < n_expert ? s_logit[lane] : -INFINITY, lane, n_expert, p);
+    if (lane < n_expert) {
+        probs[row * n_expert + lane] = p;
+        order[row * n_expert + rank] = lane;
+    }
 }
 
 // h = silu(gate) * up, optional f32 output, optional Q8_1 output; one lane per 4 elements
@@ -195,6 +266,24 @@ static int rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, co
     else MI355_LAUNCH_NORM(16);
 #undef MI355_LAUNCH_NORM
     return launch_status("k_rms_norm_mul_quant");
+}
+
+int mi355_rms_norm_mul_quant_router(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act, int64_t k,
+                                    int64_t nrows, float eps, const float *W, int64_t w_stride, float *logits, float *probs, int32_t *order,
+                                    int64_t n_expert) {
+    MI355_REQUIRE(k > 0 && k % 32 == 0 && k <= 4096, "rms_norm_mul_quant_router: k=%lld must be a multiple of 32 and at most 4096", (long long)k);
+    MI355_REQUIRE(nrows >= 0 && nrows <= 64, "rms_norm_mul_quant_router: a few rows (%lld given)", (long long)nrows);
+    MI355_REQUIRE(n_expert >= 1 && n_expert <= 64 && w_stride >= k && w_stride % 4 == 0, "rms_norm_mul_quant_router: 1..64 experts, router rows of at least k");
+    MI355_REQUIRE(((uintptr_t)x & 15) == 0 && x_stride % 4 == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 15) == 0 && y_stride % 4 == 0 &&
+                  ((uintptr_t)act & 15) == 0 && ((uintptr_t)W & 15) == 0, "rms_norm_mul_quant_router: operands must be 16-byte aligned");
+    MI355_REQUIRE(W && logits && probs && order, "rms_norm_mul_quant_router: null operand");
+    if (nrows == 0) return MI355_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)nrows), block(256);
+    if (k <= 1024) MI355_LAUNCH((k_rms_norm_mul_quant_router<1>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps, W, w_stride, logits, probs, order, (int)n_expert);
+    else if (k <= 2048) MI355_LAUNCH((k_rms_norm_mul_quant_router<2>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps, W, w_stride, logits, probs, order, (int)n_expert);
+    else MI355_LAUNCH((k_rms_norm_mul_quant_router<4>), grid, block, 0, s, x, x_stride, w, y, y_stride, act, k, nrows, eps, W, w_stride, logits, probs, order, (int)n_expert);
+    return launch_status("k_rms_norm_mul_quant_router");
 }
 
 int mi355_rms_norm_mul_quant(void *stream, const float *x, int64_t x_stride, const float *w, float *y, int64_t y_stride, void *act,

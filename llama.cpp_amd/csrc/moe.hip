@@ -9,28 +9,11 @@
 // Each kernel writes every tensor the separate nodes would have written, with the same arithmetic (same reduction
 // order, no fused multiply-adds), so the fused and the node-by-node execution of a graph agree bit for bit.
 #include "common.hpp"
+#include "moe.hpp"
 
 namespace mi355 {
 
-// One wave per token; n_expert <= 64.  probs = softmax(logits) as k_soft_max computes it for a 64-thread group
-// (ggml_compute_forward_soft_max_f32, ggml-cpu.c:8959-9055); order[rank] = expert, descending by probability, ties by
-// index (ggml_compute_forward_argsort_f32, ggml-cpu.c:10857, leaves ties unspecified).  Lane e holds expert e; returns its rank.
-__device__ __forceinline__ int moe_route_lane(float x, int e, int n_expert, float &p) {
-    const bool live = e < n_expert;
-    if (!live) x = -INFINITY;
-    const float mx = wave_max(x);
-    const float ex = live ? expf(x - mx) : 0.0f;
-    const float sum = wave_sum(ex);
-    const float inv = 1.0f / sum;
-    p = ex * inv;
-    int rank = 0;
-    for (int j = 0; j < n_expert; j++) {
-        const float pj = __shfl(p, j, 64);
-        rank += (pj > p || (pj == p && j < e)) ? 1 : 0;
-    }
-    return rank;
-}
-
+// One wave per token (moe_route_lane, moe.hpp): probs = softmax(logits), order[rank] = expert.
 __global__ void __launch_bounds__(64) k_moe_route(const float *__restrict__ logits, float *__restrict__ probs, int32_t *__restrict__ order,
                                                   int n_expert) {
     const int64_t t = blockIdx.x;

@@ -79,8 +79,10 @@ __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qr
 // Called by the first 256 threads of a group; contains exactly one group barrier, which further waves of a larger group must
 // match with a barrier of their own.
 template <int NV, int FMT, bool COH>
+// keep: where the caller wants the thread's NV pieces of the normalised row (registers), or null
 __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr, const float *__restrict__ w, float *__restrict__ yr,
-                                                   void *__restrict__ act, int64_t row, int64_t k, int64_t nrows, float eps, float *sh) {
+                                                   void *__restrict__ act, int64_t row, int64_t k, int64_t nrows, float eps, float *sh,
+                                                   f32x4 *keep = nullptr) {
     const int tid = threadIdx.x;
     f32x4 v[NV], ww[NV];
     // the weight does not depend on the reduction: fetch it together with the row, one memory round trip instead of two
@@ -123,6 +125,7 @@ __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr,
             for (int i = 0; i < 4; i++) o[i] = o[i] * ww[it][i];
         }
         if (yr && live) *(f32x4 *)(yr + e0) = o;
+        if (keep) keep[it] = o;
         if constexpr (FMT == 2) {
             if (act && live) q8k_quantize_wave_tiled(o, tid & 63, (uint8_t *)act, k, nrows, row, e0 >> 8);   // whole wave: k is a multiple of 256
         } else if constexpr (FMT == 1) {

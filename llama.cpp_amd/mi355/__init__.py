@@ -96,6 +96,7 @@ _SIGNATURES = {
     "mi355_mul_mat_q8k_tiled_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled_multi": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
+    "mi355_rms_norm_mul_quant_router": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f, _p, _i64, _p, _p, _p, _i64]),
     "mi355_rms_norm_mul_quant": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),
     "mi355_swiglu_quant": (_int, [_p, _p, _p, _i64, _p, _i64, _p, _i64, _i64]),
     "mi355_rms_norm_mul_quant_q8k": (_int, [_p, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _f]),

@@ -161,3 +161,33 @@ def test_weights_combine_equals_the_two_launches(dev, n_expert, n_embd, n_used, 
                                               mi355._ptr(res) if residual else None, mi355._ptr(out3), n_embd, n_used, T))
     torch.cuda.synchronize()
     assert torch.equal(ex3, scaled) and torch.equal(out3, out)
+
+
+@pytest.mark.parametrize("n_expert,T,K", [(8, 1, 4096), (8, 3, 4096), (64, 2, 2048), (4, 8, 1024), (12, 1, 3072)])
+def test_norm_router_equals_norm_product_route(dev, n_expert, T, K):
+    """mi355_rms_norm_mul_quant_router = the FFN norm (f32 row + Q8_1 rows), the f32 router product and soft-max + order, with the
+    bits of the three launches it replaces."""
+    import torch
+    import mi355
+    lib = mi355.load()
+    g = torch.Generator().manual_seed(n_expert * 100 + T)
+    W = (torch.randn(n_expert, K, generator=g) * 0.05).to(dev)
+    x = torch.randn(T, K, generator=g).to(dev)
+    nw = (1.0 + 0.1 * torch.randn(K, generator=g)).to(dev)
+    nact = int(lib.mi355_act_bytes(K, T))
+    y, act = torch.empty(T, K, device=dev), torch.zeros(nact, dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_rms_norm_mul_quant(None, mi355._ptr(x), K, mi355._ptr(nw), mi355._ptr(y), K, mi355._ptr(act), K, T, 1e-5))
+    logits = torch.empty(T, n_expert, device=dev)
+    mi355.check(lib.mi355_mul_mat_f(None, _d(W), _d(y), _d(logits)))
+    probs, order = torch.empty_like(logits), torch.empty(T, n_expert, dtype=torch.int32, device=dev)
+    mi355.check(lib.mi355_moe_route(None, mi355._ptr(logits), mi355._ptr(probs), mi355._ptr(order), n_expert, T))
+    y2, act2 = torch.zeros_like(y), torch.zeros_like(act)
+    logits2, probs2, order2 = torch.zeros_like(logits), torch.zeros_like(probs), torch.zeros_like(order)
+    mi355.check(lib.mi355_rms_norm_mul_quant_router(None, mi355._ptr(x), K, mi355._ptr(nw), mi355._ptr(y2), K, mi355._ptr(act2), K, T, 1e-5, mi355._ptr(W), K,
+                                                    mi355._ptr(logits2), mi355._ptr(probs2), mi355._ptr(order2), n_expert))
+    torch.cuda.synchronize()
+    used = T * K + T * (K // 32) * 8
+    assert torch.equal(y2, y) and torch.equal(act2[:used], act[:used])
+    assert torch.equal(logits2, logits) and torch.equal(probs2, probs) and torch.equal(order2, order)
+    want = y.cpu().double() @ W.cpu().double().T
+    assert orc.nmse(logits2.cpu().numpy(), want.numpy().astype(np.float32)) < 1e-10
