@@ -1,7 +1,7 @@
 """Drop-in check at model level: the reference's own benchmark program, examples/llama-bench, built unmodified from the
 reference sources (oracle/Makefile, target llamabench), loads libggml-mi355.so through GGML_BACKEND_PATH, offloads every
 layer of a synthetic llama-architecture Q4_K_M model (tests/make_synthetic_gguf.py) and runs prefill and decode with flash
-attention.  The test asserts that the run completes on the plug-in's device and writes the table to gpurun_out/."""
+attention.  The test asserts that the run completes on the plug-in's device and keeps the table it printed as a log file."""
 import os
 import re
 import subprocess
