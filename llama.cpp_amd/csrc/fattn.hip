@@ -184,23 +184,64 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     for (int64_t cb = c_begin; cb < c_end; cb += U * SLOTS) {
         float mv[U];
         bool valid[U];
+        {
+            // the U mask entries are requested together, from clamped addresses and without a branch per entry (a branch per entry
+            // makes each load wait for the one before it: U round trips instead of one)
+            unsigned mraw[U];   // (32-bit each: halves packed in pairs would be merged load by load, with a wait for each)
 #pragma unroll
-        for (int j = 0; j < U; j++) {
-            const int64_t c = cb + j * SLOTS + slot;
-            const bool in_range = c < c_end;
-            mv[j] = 0.0f;
-            if (mrow && in_range) mv[j] = half_bits_to_float(mrow[c]);
-            valid[j] = in_range && mv[j] != -INFINITY;
+            for (int j = 0; j < U; j++) mraw[j] = 0;
+            if (mrow) {   // uniform
+#pragma unroll
+                for (int j = 0; j < U; j++) {
+                    const int64_t c = cb + j * SLOTS + slot;
+                    mraw[j] = mrow[c < c_end ? c : c_end - 1];
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);   // (or each load is moved down to its first use, and waited for there)
+#pragma unroll
+            for (int j = 0; j < U; j++) {
+                const int64_t c = cb + j * SLOTS + slot;
+                mv[j] = half_bits_to_float((unsigned short)mraw[j]);
+                valid[j] = c < c_end && mv[j] != -INFINITY;
+                if (c >= c_end) mv[j] = 0.0f;
+            }
         }
         u32x4 kk[U], vv[U];
+        if constexpr (!QUANT) {
 #pragma unroll
-        for (int j = 0; j < U; j++) {
-            const int64_t c = cb + j * SLOTS + slot;
-            kk[j] = u32x4{0, 0, 0, 0};
-            vv[j] = u32x4{0, 0, 0, 0};
-            if (valid[j] && active) {   // masked cells cost no K/V traffic
+            for (int j = 0; j < U; j++) {
+                const int64_t c = cb + j * SLOTS + slot;
+                kk[j] = u32x4{0, 0, 0, 0};
+                vv[j] = u32x4{0, 0, 0, 0};
+                if (valid[j] && active) {   // masked cells cost no K/V traffic
+                    kk[j] = load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2);
+                    vv[j] = load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2);
+                }
+            }
+        } else if (!active) {
+#pragma unroll
+            for (int j = 0; j < U; j++) {
+                kk[j] = u32x4{0, 0, 0, 0};
+                vv[j] = u32x4{0, 0, 0, 0};
+            }
+        } else {
+            // Quantized operands take two or three loads per row; under a branch per step the narrow ones (the scales) are waited
+            // for inside it, a round trip per step (9.1 us at 256 cells of a Q8_0 cache, 7.6 without).  So no branch: a masked cell
+            // reads the split's first cell instead - a row that is in use, not one that may never have been written and would come
+            // from memory cold - and is zeroed afterwards.
+#pragma unroll
+            for (int j = 0; j < U; j++) {
+                const int64_t c = valid[j] ? cb + j * SLOTS + slot : c_begin;
                 kk[j] = k_f16 ? load16(a.k + c * a.k_nb1 + hk * a.k_nb2 + d0 * 2) : kv_load8(kl, c);
                 vv[j] = v_f16 ? load16(a.v + c * a.v_nb1 + hk * a.v_nb2 + d0 * 2) : kv_load8(vl, c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < U; j++) {
+                if (!valid[j]) {
+                    kk[j] = u32x4{0, 0, 0, 0};
+                    vv[j] = u32x4{0, 0, 0, 0};
+                }
             }
         }
         float kd[U];   // quantized K: the levels as exact f16 values; their dot with q takes the block's scale afterwards
@@ -423,7 +464,9 @@ static int launch_vec_r(hipStream_t s, fattn_args &a, int R) {
     // Up to 1024 cells and few (token, head) pairs: one head per group, eight waves per group (32 cells of a D = 128 head per step,
     // four steps' loads in flight) and no split of the cells over groups, so no second launch.  Measured per decoded token of
     // the 8B model at 256 cells: 4 waves 1.897 ms, 8 waves 1.856 ms, 16 waves 1.875 ms; requesting K and V together with the mask
-    // instead of after it (one round trip less per step, but masked cells then cost their bytes) 1.91-1.96 ms.
+    // instead of after it (one round trip less per step, but masked cells - rows of the cache that may never have been written - then
+    // come from memory cold, and every lane waits for them) 1.91-1.96 ms; measured again with the mask entries requested together:
+    // 6.6 us for 256 cells that are all in use, but a decoded token 1.87 ms against 1.83.
     constexpr int64_t one_head_max = 1024;
     // (quantized operands cost more arithmetic per cell: from 257 cells on their cells are split over groups)
     const bool quantized = a.type_k != MI355_F16 || a.type_v != MI355_F16;
