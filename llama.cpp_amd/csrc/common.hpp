@@ -140,6 +140,33 @@ __device__ __forceinline__ float dpp_max(float v) {
     const int b = __builtin_bit_cast(int, v);
     return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(b, b, CTRL, ROWMASK, 0xF, false)));
 }
+// Maximum / integer sum over aligned groups of W lanes (4, 8, 16 or 32), every lane of the group getting the result, with DPP row
+// operations: a few cycles per step where a cross-lane move through the LDS crossbar (ds_bpermute, what __shfl_xor compiles to)
+// is a round trip of a hundred or so.  Both operations are exact whatever the order, so the result is that of a butterfly of
+// __shfl_xor steps.  W == 32 ends with one swizzle (lane ^ 16).
+template <int CTRL>
+__device__ __forceinline__ int dpp_get(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
+template <int W>
+__device__ __forceinline__ float lanes_max(float v) {
+    static_assert(W == 4 || W == 8 || W == 16 || W == 32, "aligned groups of 4, 8, 16 or 32 lanes");
+    v = fmaxf(v, __builtin_bit_cast(float, dpp_get<0xB1>(__builtin_bit_cast(int, v))));    // quad_perm [1,0,3,2]
+    v = fmaxf(v, __builtin_bit_cast(float, dpp_get<0x4E>(__builtin_bit_cast(int, v))));    // quad_perm [2,3,0,1]
+    if constexpr (W >= 8) v = fmaxf(v, __builtin_bit_cast(float, dpp_get<0x141>(__builtin_bit_cast(int, v))));    // row_half_mirror
+    if constexpr (W >= 16) v = fmaxf(v, __builtin_bit_cast(float, dpp_get<0x140>(__builtin_bit_cast(int, v))));   // row_mirror
+    if constexpr (W >= 32) v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F)));   // lane ^ 16
+    return v;
+}
+template <int W>
+__device__ __forceinline__ int lanes_sum_i(int v) {
+    static_assert(W == 4 || W == 8 || W == 16 || W == 32, "aligned groups of 4, 8, 16 or 32 lanes");
+    v += dpp_get<0xB1>(v);
+    v += dpp_get<0x4E>(v);
+    if constexpr (W >= 8) v += dpp_get<0x141>(v);
+    if constexpr (W >= 16) v += dpp_get<0x140>(v);
+    if constexpr (W >= 32) v += __builtin_amdgcn_ds_swizzle(v, 0x401F);
+    return v;
+}
+
 // x / (1 + exp(-x)) for the fused SiLU * up launches: exp as v_exp_f32 of a scaled argument and the quotient as a multiplication
 // by v_rcp_f32 (a few 1e-7 relative from the library forms, which cost ~35 instructions per element and made the 512-row
 // launch compute-bound; the reference's own SiLU is a vectorized approximation, ggml-cpu.c:1868-1911).  The unary SILU node

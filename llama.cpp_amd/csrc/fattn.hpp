@@ -41,15 +41,11 @@ struct fattn_args {
 // Q8_1 of one value per lane, 32 consecutive lanes = one block (quantize_row_q8_1_ref,
 // ggml/src/ggml-quants.c:220-253); e = element index inside the query row of k elements
 __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
-    float amax = fabsf(v);
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float amax = lanes_max<32>(fabsf(v));
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     const int q = (int)roundf(v * id);
-    int sum = q;
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const int sum = lanes_sum_i<32>(q);
     qrow[e] = (int8_t)q;
     if ((e & 31) == 0) {
         act_ds o;

@@ -13,9 +13,7 @@ namespace mi355 {
 // split activation layout.  Mirrors k_quantize_q8_1 (quantize.hip) instruction for instruction.
 __device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, int8_t *__restrict__ qplane, act_ds *__restrict__ ds,
                                                     int64_t row, int64_t k, int64_t e0) {
-    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-#pragma unroll
-    for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float amax = lanes_max<8>(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     int q[4];
@@ -25,8 +23,7 @@ __device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, i
         q[i] = (int)roundf(v[i] * id);
         sum += q[i];
     }
-#pragma unroll
-    for (int off = 4; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    sum = lanes_sum_i<8>(sum);
     if (!live) return;
     const u32 packed = (u32)(q[0] & 0xFF) | ((u32)(q[1] & 0xFF) << 8) | ((u32)(q[2] & 0xFF) << 16) | ((u32)(q[3] & 0xFF) << 24);
     *(u32 *)(qplane + row * k + e0) = packed;
@@ -43,15 +40,11 @@ __device__ __forceinline__ void quantize_block_lane(const f32x4 &v, bool live, i
 // 8-byte store), for rows that other groups of the same launch read after a grid-wide step.
 template <bool COH = false>
 __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qrow, act_ds *__restrict__ srow, int64_t e) {
-    float amax = fabsf(v);
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float amax = lanes_max<32>(fabsf(v));
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     const int q = (int)roundf(v * id);
-    int sum = q;
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const int sum = lanes_sum_i<32>(q);
     act_ds o;
     o.d = half_bits_to_float(float_to_half_bits(d));
     o.sum = sum;
@@ -106,7 +99,7 @@ __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr,
     for (int it = 0; it < NV; it++)
 #pragma unroll
         for (int i = 0; i < 4; i++) ss = __builtin_fmaf(v[it][i], v[it][i], ss);
-    ss = wave_sum(ss);
+    ss = wave_sum_dpp(ss);
     if ((tid & 63) == 0) sh[tid >> 6] = ss;
     __syncthreads();
     ss = add_rn(add_rn(add_rn(sh[0], sh[1]), sh[2]), sh[3]);

@@ -40,9 +40,7 @@ __global__ void __launch_bounds__(256) k_quantize_q8_1(const float *__restrict__
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
     if (live) v = *(const f32x4 *)(x + row * x_stride + e0);
 
-    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-#pragma unroll
-    for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float amax = lanes_max<8>(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
 
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
@@ -53,8 +51,7 @@ __global__ void __launch_bounds__(256) k_quantize_q8_1(const float *__restrict__
         q[i] = (int)roundf(v[i] * id);
         sum += q[i];
     }
-#pragma unroll
-    for (int off = 4; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    sum = lanes_sum_i<8>(sum);
 
     if (!live) return;
     const u32 packed = (u32)(q[0] & 0xFF) | ((u32)(q[1] & 0xFF) << 8) | ((u32)(q[2] & 0xFF) << 16) | ((u32)(q[3] & 0xFF) << 24);
