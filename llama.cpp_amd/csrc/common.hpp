@@ -167,6 +167,33 @@ __device__ __forceinline__ int lanes_sum_i(int v) {
     return v;
 }
 
+// The largest 64-bit key (hi, lo) of the 64 lanes, to every lane: four DPP steps inside the 16-lane rows, then the four rows' winners
+// through scalar registers.
+__device__ __forceinline__ void wave_max_key(u32 &hi, u32 &lo) {
+#define MI355_KEY_STEP(CTRL)                                                     \
+    {                                                                            \
+        const u32 oh = (u32)dpp_get<CTRL>((int)hi), ol = (u32)dpp_get<CTRL>((int)lo); \
+        const bool take = oh > hi || (oh == hi && ol > lo);                      \
+        hi = take ? oh : hi;                                                     \
+        lo = take ? ol : lo;                                                     \
+    }
+    MI355_KEY_STEP(0xB1)
+    MI355_KEY_STEP(0x4E)
+    MI355_KEY_STEP(0x141)
+    MI355_KEY_STEP(0x140)
+#undef MI355_KEY_STEP
+    u32 bh = (u32)__builtin_amdgcn_readlane((int)hi, 0), bl = (u32)__builtin_amdgcn_readlane((int)lo, 0);
+#pragma unroll
+    for (int r = 1; r < 4; r++) {
+        const u32 oh = (u32)__builtin_amdgcn_readlane((int)hi, 16 * r), ol = (u32)__builtin_amdgcn_readlane((int)lo, 16 * r);
+        const bool take = oh > bh || (oh == bh && ol > bl);
+        bh = take ? oh : bh;
+        bl = take ? ol : bl;
+    }
+    hi = bh;
+    lo = bl;
+}
+
 // x / (1 + exp(-x)) for the fused SiLU * up launches: exp as v_exp_f32 of a scaled argument and the quotient as a multiplication
 // by v_rcp_f32 (a few 1e-7 relative from the library forms, which cost ~35 instructions per element and made the 512-row
 // launch compute-bound; the reference's own SiLU is a vectorized approximation, ggml-cpu.c:1868-1911).  The unary SILU node

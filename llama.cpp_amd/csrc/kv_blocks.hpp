@@ -34,9 +34,7 @@ __device__ __forceinline__ void kv_block_offsets(const kv_place &p, int64_t g, i
 // One block by the 32 lanes j = 0..31 of a half wave, lane j holding element j (both halves of the wave must run this with their
 // own 32 values: the exchanges stay inside a half).  quantize_row_q8_0_ref (ggml/src/ggml-quants.c:194-218) bit for bit.
 __device__ __forceinline__ void kv_store_q8_0_lane32(float v, int j, uint8_t *__restrict__ y, int64_t lv, int64_t sc, bool live) {
-    float amax = fabsf(v);
-#pragma unroll
-    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float amax = lanes_max<32>(fabsf(v));
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     const int q = (int)roundf(v * id);
@@ -76,9 +74,7 @@ __device__ __forceinline__ void kv_store_q4_0_lane32(float v, int j, uint8_t *__
 // The same two quantizations with TWO adjacent elements per lane, 16 lanes per block: lane l16 of the block holds elements
 // 2 * l16 and 2 * l16 + 1 (the rotation pairs of the adjacent-pair rope mode).
 __device__ __forceinline__ void kv_store_q8_0_pair16(float y0, float y1, int l16, uint8_t *__restrict__ y, int64_t lv, int64_t sc) {
-    float amax = fmaxf(fabsf(y0), fabsf(y1));
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    const float amax = lanes_max<16>(fmaxf(fabsf(y0), fabsf(y1)));
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
     const int q0 = (int)roundf(y0 * id), q1 = (int)roundf(y1 * id);

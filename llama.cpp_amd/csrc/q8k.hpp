@@ -22,12 +22,12 @@ __device__ __forceinline__ void q8k_quantize_values(const f32x4 &v, int lane, u3
         const float ax = fabsf(v[i]);
         if (ax > amax) { amax = ax; vmax = v[i]; }
     }
-    int who = lane;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float oa = __shfl_xor(amax, off, 64), ov = __shfl_xor(vmax, off, 64);
-        const int ow = __shfl_xor(who, off, 64);
-        if (oa > amax || (oa == amax && ow < who)) { amax = oa; vmax = ov; who = ow; }
+    // over the wave: the largest magnitude, the lowest lane among equals (magnitudes order as their bit patterns), then that lane's value
+    {
+        u32 hi = __builtin_bit_cast(u32, amax), lo = 63u - (u32)lane;
+        wave_max_key(hi, lo);
+        amax = __builtin_bit_cast(float, hi);
+        vmax = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, vmax), (int)(63u - lo)));
     }
 
     int lv[4] = {0, 0, 0, 0};
@@ -41,9 +41,7 @@ __device__ __forceinline__ void q8k_quantize_values(const f32x4 &v, int lane, u3
         }
         d = 1.0f / iscale;
     }
-    sum = lv[0] + lv[1] + lv[2] + lv[3];
-#pragma unroll
-    for (int off = 1; off < 8; off <<= 1) sum += __shfl_xor(sum, off, 64);
+    sum = lanes_sum_i<8>(lv[0] + lv[1] + lv[2] + lv[3]);
     packed = (u32)(lv[0] & 0xFF) | ((u32)(lv[1] & 0xFF) << 8) | ((u32)(lv[2] & 0xFF) << 16) | ((u32)(lv[3] & 0xFF) << 24);
 }
 
