@@ -594,6 +594,9 @@ static int pick_rpw(int64_t total_rows) {
 // Measured and not adopted: splitting K over the four waves of a group (each wave reads a quarter of the activation, partial
 // sums meet in LDS at the end) - Q4_K 4096 x 4096 4.9 -> 4.3 us and 14336 x 4096 8.2 -> 7.9 us, but Q6_K slower throughout
 // (4096 x 14336 11.2 -> 14.0 us, output projection 80 -> 87 us): its 16-byte pieces per lane then form 256-byte runs.
+// Also measured and not adopted: the next step's weights requested before the current step's are used (one step of look-ahead in
+// the loop below) - Q4_K 4096 x 14336 10.9 -> 10.7 us, but norm + Q/K/V 10.0 -> 10.8, Q6_K 4096 x 14336 11.9 -> 13.9, wo 4.85 -> 5.1
+// and the output projection 70 -> 123 us (decode 557 -> 521 tokens/s).
 // Also measured and not adopted: a fixed number of groups (512..1536) that walk the matrix, activation copied to LDS once per
 // group, the next block's weights requested before the current one is contracted - bit-identical sums, but 14336 x 4096 Q4_K
 // 8.3 -> 9.9..10.9 us and the output projection 50.6 -> 61..77 us: many short-lived waves keep more loads in flight than few
