@@ -212,7 +212,6 @@ def sweep(kinds):
            mi355.Q4_1: 20 / 32, mi355.Q5_0: 22 / 32, mi355.Q5_1: 24 / 32, mi355.IQ4_NL: 18 / 32}
     names = {mi355.Q4_0: "Q4_0", mi355.Q8_0: "Q8_0", mi355.Q4_K: "Q4_K", mi355.Q5_K: "Q5_K", mi355.Q6_K: "Q6_K", mi355.Q4_1: "Q4_1", mi355.Q5_0: "Q5_0",
              mi355.Q5_1: "Q5_1", mi355.IQ4_NL: "IQ4_NL"}
-    gemv_only = (mi355.Q5_K, mi355.Q4_1, mi355.Q5_0, mi355.Q5_1, mi355.IQ4_NL)   # no weight-streaming matrix-core kernel: the GEMV serves up to eight rows
     all_types = (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q5_K, mi355.Q6_K, mi355.Q4_1, mi355.Q5_0, mi355.Q5_1, mi355.IQ4_NL)
     shapes = [(4096, 4096), (14336, 4096), (4096, 14336)]
     if "gemv" in kinds:
@@ -224,14 +223,14 @@ def sweep(kinds):
                 for B in (1, 8):
                     act = mi355.quantize_act(torch.randn(B, K, device=dev, generator=gen))
                     out = torch.empty(B, N, device=dev)
-                    if B == 1 or t in gemv_only:
+                    if B == 1:
                         us = timed(lambda i: mi355.check(lib.mi355_mul_mat_vec_q(stream.cuda_stream, t, Ws[i].data_ptr(), act.data_ptr(), out.data_ptr(), N, K, B, N)), nm, 4)
                     else:   # the weight-streaming matrix-core kernel, with the workspace that lets products with few rows split K
                         ws = torch.empty(int(lib.mi355_mul_mat_skinny_ws_bytes(N, K, B)) + 256, dtype=torch.uint8, device=dev)
                         us = timed(lambda i: mi355.check(lib.mi355_mul_mat_skinny(stream.cuda_stream, t, Ws[i].data_ptr(), act.data_ptr(), out.data_ptr(), None, N, K, B, N,
                                                                                   ws.data_ptr(), ws.numel())), nm, 4)
                     alg = wbytes + B * (4 * K + 4 * N)
-                    emit(kernel="MUL_MAT batch 1 (GEMV)" if B == 1 else ("MUL_MAT batch %d (GEMV)" % B if t in gemv_only else "MUL_MAT batch %d (k_mm_skinny)" % B), case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
+                    emit(kernel="MUL_MAT batch 1 (GEMV)" if B == 1 else "MUL_MAT batch %d (k_mm_skinny)" % B, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="hbm", achieved=round(alg / us / 1e3, 1),
                          unit="GB/s", frac=round(alg / us / 1e3 / HBM_PEAK_GBS, 4), algorithmic_bytes=alg)
                 del Ws
     if "mmq" in kinds or "mmq_wide" in kinds:

@@ -131,7 +131,7 @@ size_t mi355_mul_mat_q_ws_bytes(int64_t N, int64_t K, int64_t B);
 int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const void *act, float *dst, int64_t N, int64_t K, int64_t B,
                        int64_t dst_stride, void *ws, size_t ws_bytes);
 
-/* MUL_MAT for 1..32 activation rows as one weight-streaming launch on the int8 matrix cores (Q4_0, Q8_0, Q4_K, Q6_K; K a
+/* MUL_MAT for 1..32 activation rows as one weight-streaming launch on the int8 matrix cores (every weight type; K a
  * multiple of 256; 16-byte aligned rows: mi355_mul_mat_skinny_supported says whether a product qualifies).  Same operands
  * as mi355_mul_mat_vec_q (`act` from mi355_quantize_act) plus an optional residual added to the result (may alias dst).
  * It is what mi355_mul_mat uses between the batch-1 kernels and the tile kernels (ggml's MUL_MAT with src1->ne[1] of

@@ -50,8 +50,6 @@
 namespace {
 
 // ------------------------------------------------------------------------------- helpers
-// types whose batches of 5..32 rows have the weight-streaming matrix-core kernel; the others stay with the GEMV up to 8 rows
-bool has_skinny_kernel(ggml_type t) { return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q6_K; }
 bool is_repacked_type(ggml_type t) {
     return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K || t == GGML_TYPE_Q4_1 || t == GGML_TYPE_Q5_0 || t == GGML_TYPE_Q5_1 ||
            t == GGML_TYPE_IQ4_NL;
@@ -1117,7 +1115,6 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
     if (mm->op != GGML_OP_MUL_MAT || !is_weight_type(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
     if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
-    if (!has_skinny_kernel(a->type) && b->ne[1] > 8) return false;    // the GEMV only (up to eight rows); more rows take the generic path
     const int64_t K = a->ne[0];
     if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
     if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)

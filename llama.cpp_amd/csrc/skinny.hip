@@ -24,11 +24,21 @@ namespace mi355 {
 
 namespace {
 
-template <int TYPE> struct sk_traits;
-template <> struct sk_traits<MI355_Q4_0> { static constexpr int ROW_BYTES = 128; };    // bytes copied to LDS per step and weight row
-template <> struct sk_traits<MI355_Q8_0> { static constexpr int ROW_BYTES = 256; };
-template <> struct sk_traits<MI355_Q4_K> { static constexpr int ROW_BYTES = 128; };    // qs only; the header goes to registers
-template <> struct sk_traits<MI355_Q6_K> { static constexpr int ROW_BYTES = 128; };    // ql; qh (64 bytes) is copied beside it
+// What goes through LDS per step (256 elements) and weight row: the 4-bit (Q8_0: 8-bit) plane of the levels - 128 bytes of
+// nibbles for every type but Q8_0; Q6_K copies its 64 bytes of high bit pairs beside them.  Everything a lane needs of ITS row
+// only (block scales and minima, the K-quants' 16-byte header, the fifth bits of Q5_0 / Q5_1 / Q5_K) goes straight to registers.
+template <int TYPE> struct sk_traits {
+    static constexpr int ROW_BYTES = TYPE == MI355_Q8_0 ? 256 : 128;
+    // per-32-block types whose block is 16 bytes of nibbles, element b low and element 16 + b high in byte b
+    static constexpr bool NIB32 = TYPE == MI355_Q4_0 || TYPE == MI355_IQ4_NL || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1;
+    static constexpr bool PAIR = TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;          // {f16 d, f16 m} per block
+    static constexpr bool FIFTH32 = TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1;       // one word of fifth bits per block
+    static constexpr bool KQ = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K;            // 16-byte header + 6-bit (scale, min) pairs
+    static constexpr int STEP_BYTES = TYPE == MI355_Q8_0 ? 256 : TYPE == MI355_Q4_K ? Q4_K_BYTES : TYPE == MI355_Q5_K ? Q5_K_BYTES : 128;
+    static constexpr int QS_OFF = TYPE == MI355_Q4_K ? 16 : TYPE == MI355_Q5_K ? 48 : 0;   // where the nibbles start inside a step
+    // the activation's block sum enters as x = OFFSET * d * sum (levels stored with an offset) or as d * sum (block minimum)
+    static constexpr float OFFSET = TYPE == MI355_Q4_0 ? -8.0f : TYPE == MI355_Q5_0 ? -16.0f : 1.0f;
+};
 
 // Orders a wave's own LDS accesses around the point where its lanes exchange data through LDS: the hardware completes
 // them in program order, so all that is needed is that neither the compiler nor the instruction scheduler moves an access
@@ -55,7 +65,9 @@ template <int TYPE, int NI> struct sk_regs {
     static constexpr int NA = 2 * NI;                                   // ... for 8 NI activation rows of 256 bytes
     static constexpr int NT = (NI + 1) / 2;                             // ... for their 8 {d, sum} pairs each
     u32x4 w[NW], a[NA], t[NT], hdr;
-    u32x4 qh[TYPE == MI355_Q6_K ? 2 : 1];   // Q6_K: the high bit pairs, 32 rows x 64 bytes
+    u32x4 hdr2;                             // Q4_1 / Q5_1: the second half of the eight {d, m} pairs
+    u32x4 qh[2];                            // Q6_K: the high bit pairs, 32 rows x 64 bytes (on their way to LDS); Q5_0 / Q5_1: the
+                                            // eight fifth-bit words of the lane's row; Q5_K ([0] only): qh bytes 16 (lane / 32) .. + 16
     u32 d6;                                 // Q6_K: the f16 super-block scale of the lane's row (hdr holds its 16 int8 scales)
 };
 
@@ -102,7 +114,7 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
     for (int u = 0; u < R::NW; u++) {
         int64_t row = row0 + w_row + u * RPL;
         row = row < N ? row : N - 1;   // clamp: rows past the end repeat the last row and are not stored
-        w_src[u] = W + row * L.row_bytes + 16 * w_piece + (TYPE == MI355_Q4_K ? 16 : 0);
+        w_src[u] = W + row * L.row_bytes + 16 * w_piece + T::QS_OFF;
     }
     const uint8_t *qh_src[2];   // Q6_K: 4 lanes per row, 16 rows per load
 #pragma unroll
@@ -131,11 +143,24 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
     // loads of one step into the register set `g`
     auto fetch = [&](int step, R &g) {
         const int s = step < nsteps ? step : nsteps - 1;
-        const int w_off = s * (TYPE == MI355_Q8_0 ? 256 : TYPE == MI355_Q4_K ? Q4_K_BYTES : 128);   // < 2^31: rows are shorter than that
+        const int w_off = s * T::STEP_BYTES;   // < 2^31: rows are shorter than that
 #pragma unroll
         for (int u = 0; u < R::NW; u++) g.w[u] = load16(w_src[u] + w_off);
-        if constexpr (TYPE == MI355_Q4_K) {
+        if constexpr (T::KQ) {
             g.hdr = load16(w_mine + w_off);
+            if constexpr (TYPE == MI355_Q5_K) g.qh[0] = load16(w_mine + w_off + 16 + 16 * kh);
+        } else if constexpr (T::FIFTH32) {
+            g.qh[0] = load16(w_mine + L.off_b + s * 32);
+            g.qh[1] = load16(w_mine + L.off_b + s * 32 + 16);
+            if constexpr (T::PAIR) {
+                g.hdr = load16(w_mine + L.off_c + s * 32);
+                g.hdr2 = load16(w_mine + L.off_c + s * 32 + 16);
+            } else {
+                g.hdr = load16(w_mine + L.off_c + s * 16);
+            }
+        } else if constexpr (T::PAIR) {
+            g.hdr = load16(w_mine + L.off_b + s * 32);
+            g.hdr2 = load16(w_mine + L.off_b + s * 32 + 16);
         } else if constexpr (Q6) {
 #pragma unroll
             for (int u = 0; u < 2; u++) g.qh[u] = load16(qh_src[u] + s * 64);
@@ -158,7 +183,7 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
 
     // One set of load registers: as soon as a step's loads have been copied to LDS, the same registers take the next step's
     // loads, which are then in flight while this step is contracted.  Only the weight scales of the lane's row stay behind.
-    R cur;
+    R cur = {};
     fetch(s_lo, cur);
     for (int step = s_lo; step < s_hi; step++) {
         // ---- registers -> the wave's LDS
@@ -188,12 +213,13 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
                     const float sum = (float)(int)sum_bits;
                     float2 v;
                     v.x = d;
-                    v.y = TYPE == MI355_Q4_0 ? -8.0f * d * sum : d * sum;
+                    v.y = T::OFFSET * d * sum;
                     s_t[(2 * t_piece + h) * (8 * NI) + t_row + 16 * u] = v;
                 }
             }
         }
-        const u32x4 hdr = cur.hdr;
+        const u32x4 hdr = cur.hdr, hdr2 = cur.hdr2;
+        const u32x4 fifth[2] = {cur.qh[0], cur.qh[1]};   // (Q6_K's went to LDS above)
         const u32 d6 = cur.d6;
         wave_lds_sync();
         if (step + 1 < s_hi) fetch(step + 1, cur);
@@ -241,7 +267,7 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
         } else {
             // ---- per-block weight scales of this lane's row
             float ws[8], wm[8];
-            if constexpr (TYPE == MI355_Q4_K) {
+            if constexpr (T::KQ) {
                 const float d = half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu));
                 const float dmin = half_bits_to_float((unsigned short)(hdr[0] >> 16));
                     // all eight 6-bit (scale, min) pairs at once, as the bytes of four words (get_scale_min_k4, ggml-quants.c:631-638)
@@ -255,6 +281,13 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
                     ws[j] = d * (float)((S >> (8 * (j & 3))) & 0xFFu);
                     wm[j] = -(dmin * (float)((M >> (8 * (j & 3))) & 0xFFu));
                 }
+            } else if constexpr (T::PAIR) {
+    #pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const u32 dm = j < 4 ? hdr[j & 3] : hdr2[j & 3];
+                    ws[j] = half_bits_to_float((unsigned short)(dm & 0xFFFFu));
+                    wm[j] = half_bits_to_float((unsigned short)(dm >> 16));
+                }
             } else {
     #pragma unroll
                 for (int j = 0; j < 8; j++) ws[j] = f16_of(hdr, j);
@@ -265,14 +298,24 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
                 i32x4 wop;
                 if constexpr (TYPE == MI355_Q8_0) {
                     wop = *(const i32x4 *)(s_w + r * WPAD + 32 * j + 16 * kh);
-                } else if constexpr (TYPE == MI355_Q4_0) {   // byte b of the block's 16: level b in the low nibble, level 16 + b in the high one
+                } else if constexpr (T::NIB32) {   // byte b of the block's 16: level b in the low nibble, level 16 + b in the high one
                     const u32x4 v = *(const u32x4 *)(s_w + r * WPAD + 16 * j);
+                    const u32 fw = j < 4 ? fifth[0][j & 3] : fifth[1][j & 3];   // Q5_0 / Q5_1: bit e = fifth bit of element e
     #pragma unroll
-                    for (int i = 0; i < 4; i++) wop[i] = (int)((v[i] >> (4 * kh)) & 0x0F0F0F0Fu);
+                    for (int i = 0; i < 4; i++) {
+                        const u32 nib = (v[i] >> (4 * kh)) & 0x0F0F0F0Fu;   // elements 16 kh + 4 i .. + 4
+                        if constexpr (TYPE == MI355_IQ4_NL) wop[i] = (int)iq4nl_lookup4(nib);
+                        else if constexpr (T::FIFTH32) wop[i] = (int)(nib | spread4(fw >> (16 * kh + 4 * i)));
+                        else wop[i] = (int)nib;
+                    }
                 } else {   // chunk j / 2: byte b of its 32: level b of sub-block 2 (j / 2) in the low nibble, of the next one in the high nibble
                     const u32x4 v = *(const u32x4 *)(s_w + r * WPAD + 32 * (j >> 1) + 16 * kh);
     #pragma unroll
-                    for (int i = 0; i < 4; i++) wop[i] = (int)((v[i] >> (4 * (j & 1))) & 0x0F0F0F0Fu);
+                    for (int i = 0; i < 4; i++) {
+                        wop[i] = (int)((v[i] >> (4 * (j & 1))) & 0x0F0F0F0Fu);
+                        // Q5_K: bit j of qh byte l is the fifth bit of level l of sub-block j (dequantize_row_q5_K, ggml/src/ggml-quants.c:1482-1507)
+                        if constexpr (TYPE == MI355_Q5_K) wop[i] |= (int)(((fifth[0][i] >> j) & 0x01010101u) << 4);
+                    }
                 }
                 const i32x4 aop = *(const i32x4 *)(s_a + am * SK_APAD + 32 * j + 16 * kh);
                 i32x16 z;
@@ -288,11 +331,11 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
     #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const float Df = (float)D[4 * q + i];
-                        if constexpr (TYPE == MI355_Q4_0) {
-                            acc[q][i] = __builtin_fmaf(ws[j], __builtin_fmaf(dd[i], Df, xx[i]), acc[q][i]);   // x = -8 d sum
-                        } else if constexpr (TYPE == MI355_Q8_0) {
+                        if constexpr (TYPE == MI355_Q4_0 || TYPE == MI355_Q5_0) {
+                            acc[q][i] = __builtin_fmaf(ws[j], __builtin_fmaf(dd[i], Df, xx[i]), acc[q][i]);   // x = -8 (-16) d sum
+                        } else if constexpr (TYPE == MI355_Q8_0 || TYPE == MI355_IQ4_NL) {
                             acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);
-                        } else {
+                        } else {   // block minimum: + m (Q4_1, Q5_1), - dmin * 6-bit minimum (Q4_K, Q5_K)
                             acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);
                             acc[q][i] = __builtin_fmaf(wm[j], xx[i], acc[q][i]);                              // x = d sum
                         }
@@ -381,8 +424,7 @@ using namespace mi355;
 extern "C" {
 
 int mi355_mul_mat_skinny_supported(int type, const void *W, int64_t K, int64_t B) {
-    // the other types have no operand unpacking in this kernel: their products stay with the GEMV
-    return (type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K || type == MI355_Q6_K) && B >= 1 && B <= 32 && K > 0 && K % 256 == 0 && K < (int64_t(1) << 30) &&
+    return is_weight_type(type) && B >= 1 && B <= 32 && K > 0 && K % 256 == 0 && K < (int64_t(1) << 30) &&
            layout_aligned(W, make_row_layout(type, K));
 }
 
@@ -402,12 +444,9 @@ int mi355_mul_mat_skinny(void *stream, int type, const void *W, const void *act,
     hipStream_t s = (hipStream_t)stream;
     const int8_t *aq = (const int8_t *)act;
     const act_ds *ads = (const act_ds *)(aq + B * K);
-    switch (type) {
-        case MI355_Q4_0: launch_skinny_nt<MI355_Q4_0>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
-        case MI355_Q8_0: launch_skinny_nt<MI355_Q8_0>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
-        case MI355_Q4_K: launch_skinny_nt<MI355_Q4_K>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
-        default: launch_skinny_nt<MI355_Q6_K>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws); break;
-    }
+#define X(T) launch_skinny_nt<T>(s, W, aq, ads, dst, residual, N, (int)K, (int)B, dst_stride, slices, (float *)ws);
+    MI355_WEIGHT_TYPE_SWITCH(type, X)
+#undef X
     return launch_status("k_mm_skinny");
 }
 

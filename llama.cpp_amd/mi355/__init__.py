@@ -349,7 +349,7 @@ def mul_mat_static(t, W, x, dst):
 
 
 def mul_mat_skinny(t, W, x, residual=None, split=True):
-    """The weight-streaming matrix-core product for 1..32 activation rows (Q4_0, Q8_0, Q4_K): W device layout [N, row_bytes],
+    """The weight-streaming matrix-core product for 1..32 activation rows (every weight type): W device layout [N, row_bytes],
     x f32 [B, K] -> f32 [B, N] (+ residual [B, N]).  split: give it the workspace that lets few rows run as slices along K"""
     import torch
     B, K = x.shape
