@@ -15,6 +15,8 @@
 // LLAMA_LOGITS_DEFRAG=<n> instead removes n cells from the middle of the sequence after the prompt and asks for a defragmentation
 // (llama_kv_cache_defrag + llama_kv_cache_update: build_defrag's row copies inside the K and V caches).
 //
+// LLAMA_LOGITS_CTX=<n> sets the context size (default 1024); a prompt longer than the batch size of 512 is fed 512 tokens at a time.
+//
 // Tokens are (7 i + 3) mod n_vocab.  Output: float32 rows of n_vocab logits, one for the last prompt token and one per
 // decoded token (the token ids are fixed, the logits are not fed back).
 #include "ggml-backend.h"
@@ -43,7 +45,7 @@ int main(int argc, char ** argv) {
     llama_model * model = llama_model_load_from_file(argv[1], mp);
     if (!model) return 1;
     llama_context_params cp = llama_context_default_params();
-    cp.n_ctx = 1024;
+    cp.n_ctx = getenv("LLAMA_LOGITS_CTX") ? atoi(getenv("LLAMA_LOGITS_CTX")) : 1024;
     cp.n_batch = 512;
     cp.n_ubatch = 512;
     cp.flash_attn = true;
@@ -60,7 +62,10 @@ int main(int argc, char ** argv) {
     if (!f) return 1;
     std::vector<llama_token> toks(n_prompt);
     for (int i = 0; i < n_prompt; i++) toks[i] = (7 * i + 3) % n_vocab;
-    if (llama_decode(ctx, llama_batch_get_one(toks.data(), n_prompt)) != 0) return 1;
+    for (int i0 = 0; i0 < n_prompt; i0 += 512) {
+        const int n = n_prompt - i0 < 512 ? n_prompt - i0 : 512;
+        if (llama_decode(ctx, llama_batch_get_one(toks.data() + i0, n)) != 0) return 1;
+    }
     fwrite(llama_get_logits_ith(ctx, -1), sizeof(float), n_vocab, f);
     if (const char * sh = getenv("LLAMA_LOGITS_SHIFT")) {
         const int n_discard = atoi(sh);

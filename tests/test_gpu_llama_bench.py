@@ -53,9 +53,11 @@ def test_llama_bench_runs_on_the_plugin(dev, tmp_path):
 LOGITS = os.path.join(ROOT, "oracle", "_ref", "llama_logits")
 
 
-def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None, cache=None, mmap=True, shift=0, defrag=0):
+def _logits(model, ngl, n_prompt, n_decode, out, fusion=True, graphs=True, stats=None, cache=None, mmap=True, shift=0, defrag=0, ctx=0):
     import numpy as np
     env = dict(os.environ, GGML_BACKEND_PATH=PLUGIN, MI355_GRAPH_STATS="1")
+    if ctx:
+        env["LLAMA_LOGITS_CTX"] = str(ctx)
     if shift:
         env["LLAMA_LOGITS_SHIFT"] = str(shift)
     if defrag:
@@ -202,6 +204,31 @@ def test_model_logits_quantized_kv_cache(dev, tmp_path, cache, n_prompt):
     # projections), a value on a rounding boundary lands on another level and moves by 1/8 of the block's range.  A short prompt
     # has few cells to average that over.  The op-level parity of the stores and of attention is in tests/test_gpu_kv_quant.py.
     assert orc.nmse(gpu, cpu) < (2e-2 if "q4_0" in cache else 2e-3)
+
+
+@pytest.mark.parametrize("cache", [None, ("q8_0", "q8_0")])
+@pytest.mark.parametrize("n_prompt", [700, 3400])
+def test_model_logits_long_context(dev, tmp_path, cache, n_prompt):
+    """Contexts beyond the other model tests' 1024 cells: a prompt fed in batches of 512 (prefill attention over a growing cache,
+    through the f16 image of a quantized one), then decoded tokens at 700+ cells (the matrix-core decode kernel and its merge
+    launch) and at 3400+ cells (the streaming decode kernel, over f16 and over Q8_0 blocks read in place), replayed as HIP graphs.
+    The reference's runtime reproduces its CPU backend's logits, and graph replay reproduces launch-by-launch execution bit for bit."""
+    if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
+        pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import numpy as np
+    import make_synthetic_gguf
+    import orc
+    model = str(tmp_path / "small.gguf")
+    make_synthetic_gguf.write_model(model, n_layer=2, n_embd=2048, n_ff=4096, n_head=16, n_head_kv=4, n_vocab=2048)
+    cpu = _logits(model, 0, n_prompt, 6, str(tmp_path / "cpu.bin"), cache=cache, ctx=4096)
+    st = {}
+    gpu = _logits(model, 99, n_prompt, 6, str(tmp_path / "gpu.bin"), cache=cache, ctx=4096, stats=st)
+    eager = _logits(model, 99, n_prompt, 6, str(tmp_path / "eager.bin"), cache=cache, ctx=4096, graphs=False)
+    assert cpu.shape == gpu.shape == eager.shape and np.isfinite(gpu).all()
+    assert st["replays"] >= 3, st
+    assert np.array_equal(gpu, eager)
+    assert orc.nmse(gpu, cpu) < 2e-3
 
 
 @pytest.mark.parametrize("cache", [None, ("q8_0", "q8_0"), ("q4_0", "q4_0")])
