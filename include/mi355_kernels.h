@@ -220,6 +220,15 @@ int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, in
 size_t mi355_mul_mat_q8k_tiled_ws_bytes(int64_t N, int64_t K, int64_t B);
 int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N,
                             int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes);
+/* The same product followed by the RMS norm of its rows: dst as above, then y[b] = rms_norm(dst[b]) * norm_w and act_out = the
+ * tile image of y (mi355_act_q8k_tiled_bytes(N, B) bytes) - MUL_MAT(wo / ffn_down) -> ADD(residual) -> RMS_NORM -> MUL(norm weight)
+ * of llm_build_kv / llm_build_ffn / the next layer's llm_build_norm (src/llama.cpp:1566, :1609, :175-198), whose readers are
+ * K-quant products on tile images.  When the product is cut along K (few tiles: a 4096-row matrix at batch 512) the launch that adds
+ * the slices and the residual also normalises and quantizes the row it has just formed; otherwise the norm is a launch of its own.
+ * Same bits as mi355_mul_mat_q8k_tiled followed by mi355_rms_norm_mul_quant_q8k_tiled.  N a multiple of 256; y may be NULL. */
+int mi355_mul_mat_q8k_tiled_norm(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N,
+                                 int64_t K, int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes, const float *norm_w, float eps, float *y,
+                                 int64_t y_stride, void *act_out);
 /* One launch for up to three matrices of the same K-quant type that consume the same activation image (gate and up of llm_build_ffn,
  * src/llama.cpp:280-320; Q, K and V of a layer where their types agree): their tiles fill the compute units together (gate + up at
  * batch 512: 896 tiles = 3.5 rounds on 256 compute units instead of two launches of 2 rounds; Q + K + V: 192 tiles in one round

@@ -2133,6 +2133,35 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         if (add && add->op == GGML_OP_ADD && w.sole_use(i) && (add->src[0] == node || add->src[1] == node)) {
             const ggml_tensor * res = add->src[0] == node ? add->src[1] : add->src[0];
             if (res->type == GGML_TYPE_F32 && ggml_are_same_shape(res, node) && ggml_is_contiguous(res) && ggml_is_contiguous(add) && ggml_is_contiguous(node)) {
+                // ... -> RMS_NORM -> MUL(norm weight) whose readers are tile products again (wo -> the FFN norm, ffn_down -> the next
+                // layer's attention norm): a product that is cut along K adds its slices row by row, and the group that has formed a
+                // row normalises and quantizes it on the spot (same bits as the norm launch it replaces)
+                if (tl && split_ws) {
+                    const int jn = w.next(j);
+                    const int jm = jn < w.n ? w.next(jn) : w.n;
+                    const ggml_tensor * nrm = jn < w.n ? w.nodes[jn] : nullptr;
+                    const ggml_tensor * mul = jm < w.n ? w.nodes[jm] : nullptr;
+                    if (nrm && mul && nrm->op == GGML_OP_RMS_NORM && nrm->src[0] == add && mul->op == GGML_OP_MUL && mul->src[0] == nrm && w.sole_use(jn) &&
+                        add->ne[2] == 1 && add->ne[3] == 1 && ggml_is_contiguous(mul) && mul->type == GGML_TYPE_F32 && N % 256 == 0 && N <= 4096) {
+                        const ggml_tensor * wt = mul->src[1];
+                        if (wt->type == GGML_TYPE_F32 && ggml_is_contiguous(wt) && ggml_nelements(wt) == N &&
+                            (((uintptr_t) add->data | (uintptr_t) mul->data | (uintptr_t) wt->data | (uintptr_t) res->data) & 15) == 0 &&
+                            feeds_q8k_tiles(w, jm, mul->data, N, B) && q8k_format_for(s, w.nodes[w.next(jm)]) == ACT_Q8KT &&
+                            !bytes_overlap(mul, add) && !bytes_overlap(mul, b) &&
+                            mi355_act_q8k_tiled_bytes(N, B) <= ctx->act_size) {   // (a larger slot would move the activation the product reads)
+                            float eps;
+                            memcpy(&eps, nrm->op_params, sizeof(float));
+                            void * act_out = ctx->act_slot(mi355_act_q8k_tiled_bytes(N, B), true);   // the product still reads the other slot
+                            MI355_K_OK(mi355_mul_mat_q8k_tiled_norm(s, wtype, tl, ctx->cache.ptr, (float *) add->data, (const float *) res->data, N, K, B,
+                                                                    (int64_t) (add->nb[1] / sizeof(float)), split_ws, split_bytes, (const float *) wt->data, eps,
+                                                                    (float *) mul->data, N, act_out));
+                            ctx->note_write(add->data, ggml_nbytes(add));
+                            ctx->note_write(mul->data, ggml_nbytes(mul));
+                            ctx->cache = act_cache{mul->data, N, B, ACT_Q8KT, true, act_out};
+                            return jm;
+                        }
+                    }
+                }
                 product((float *) add->data, (const float *) res->data, (int64_t) (add->nb[1] / sizeof(float)));
                 ctx->note_write(add->data, ggml_nbytes(add));
                 return j;

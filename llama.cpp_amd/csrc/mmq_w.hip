@@ -32,6 +32,7 @@
 // MFMA operand mapping (A = activations, B = weights, D[i][j]): lane l supplies row l % 32 and k bytes [16*(l/32), +16)
 // (f16: k slots [8*(l/32), +8)); D register r of lane l is i = 8*(r/4) + 4*(l/32) + r%4, j = l % 32.
 #include "common.hpp"
+#include "norm_quant.hpp"
 #include "q8k.hpp"
 #include "qdot.hpp"
 #include "tiles.hpp"
@@ -616,6 +617,40 @@ __global__ void __launch_bounds__(256) k_wt_split_sum(const float *__restrict__ 
     for (int j = 0; j < 4; j++) dst[o + j] = acc[j];
 }
 
+// The same sum for a product whose rows are normalised next: one 256-thread group per activation row adds the row's slices and
+// the residual in k_wt_split_sum's order, stores the row, and continues with RMS_NORM -> MUL(w) -> the row of y and its part of
+// the tile image from the registers (what k_rms_norm_mul_quant<NV, 2> does after loading the row).
+template <int NV>
+__global__ void __launch_bounds__(256) k_wt_split_sum_norm(const float *__restrict__ part, float *__restrict__ dst, const float *__restrict__ residual,
+                                                           int64_t N, int64_t B, int64_t dst_stride, int n_slices, const float *__restrict__ w, float eps,
+                                                           float *__restrict__ y, int64_t y_stride, uint8_t *__restrict__ act_out) {
+    __shared__ float sh[4];
+    const int64_t b = blockIdx.x;
+    f32x4 v[NV];
+#pragma unroll
+    for (int it = 0; it < NV; it++) {
+        const int64_t n = ((int64_t)it * 256 + threadIdx.x) * 4;
+        v[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (n < N) {
+            f32x4 acc = *(const f32x4 *)(part + b * N + n);
+            for (int sl = 1; sl < n_slices; sl++) {
+                const f32x4 t = *(const f32x4 *)(part + ((int64_t)sl * B + b) * N + n);
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[j] = add_rn(acc[j], t[j]);
+            }
+            const int64_t o = b * dst_stride + n;
+            if (residual) {
+                const f32x4 t = *(const f32x4 *)(residual + o);
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[j] = add_rn(acc[j], t[j]);
+            }
+            *(f32x4 *)(dst + o) = acc;
+            v[it] = acc;
+        }
+    }
+    rms_norm_quant_row<NV, 2, false>(nullptr, w, y ? y + b * y_stride : nullptr, act_out, b, N, B, eps, sh, nullptr, v);
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -689,8 +724,25 @@ size_t mi355_mul_mat_q8k_tiled_multi_ws_bytes(int n_mats, const int64_t *Ns, int
     return wt_plan_ws_bytes(wt_make_plan(n_mats, Ns, K, B, true), Ns, B);
 }
 
+// norm: the single matrix's rows are normalised next (mi355_mul_mat_q8k_tiled_norm); taken when the product is cut along K, whose
+// sum launch then carries the norm.  *norm_done says whether it did.
+struct wt_norm {
+    const float *w;
+    float eps;
+    float *y;
+    int64_t y_stride;
+    void *act_out;
+};
+static int mul_mat_q8k_tiled_launch(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
+                                    size_t ws_bytes, const wt_norm *norm, bool *norm_done);
+
 int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
                                   void *ws, size_t ws_bytes) {
+    return mul_mat_q8k_tiled_launch(stream, type, n_mats, mats, act, K, B, ws, ws_bytes, nullptr, nullptr);
+}
+
+static int mul_mat_q8k_tiled_launch(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
+                                    size_t ws_bytes, const wt_norm *norm, bool *norm_done) {
     MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", type);
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_q8k_tiled: 1 to 3 matrices per launch, got %d", n_mats);
     MI355_REQUIRE(K > 0 && B > 0 && K % QKK == 0, "mul_mat_q8k_tiled: bad shape K=%lld B=%lld (K must be a multiple of 256)", (long long)K, (long long)B);
@@ -728,10 +780,36 @@ int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi35
     if (type == MI355_Q4_K) MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
     else if (type == MI355_Q5_K) MI355_LAUNCH(k_mmq_w<MI355_Q5_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
     else MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
-    if (p.slices > 1)
+    if (p.slices > 1 && norm && Ns[0] <= 4096 && mats[0].dst_stride % 4 == 0 && ((uintptr_t)mats[0].dst & 15) == 0 &&
+        (mats[0].residual == nullptr || ((uintptr_t)mats[0].residual & 15) == 0)) {
+        MI355_LAUNCH((k_wt_split_sum_norm<4>), dim3((unsigned)B), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B, mats[0].dst_stride,
+                     p.slices, norm->w, norm->eps, norm->y, norm->y_stride, (uint8_t *)norm->act_out);
+        *norm_done = true;
+    } else if (p.slices > 1) {
         MI355_LAUNCH(k_wt_split_sum, dim3((unsigned)((Ns[0] * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B,
                      mats[0].dst_stride, p.slices);
+    }
     return launch_status("k_mmq_w");
+}
+
+int mi355_mul_mat_q8k_tiled_norm(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
+                                 int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes, const float *norm_w, float eps, float *y, int64_t y_stride,
+                                 void *act_out) {
+    MI355_REQUIRE(N > 0 && K > 0 && B > 0 && N % QKK == 0, "mul_mat_q8k_tiled_norm: bad shape N=%lld K=%lld B=%lld (N must be a multiple of 256)", (long long)N,
+                  (long long)K, (long long)B);
+    MI355_REQUIRE(norm_w != nullptr && act_out != nullptr && ((uintptr_t)norm_w & 15) == 0 && ((uintptr_t)act_out & 15) == 0 && ((uintptr_t)y & 15) == 0 &&
+                  y_stride % 4 == 0, "mul_mat_q8k_tiled_norm: the norm's operands must be 16-byte aligned");
+    mi355_tiled_mat m;
+    m.tiles = tiles;
+    m.dst = dst;
+    m.residual = residual;
+    m.N = N;
+    m.dst_stride = dst_stride;
+    const wt_norm nm = {norm_w, eps, y, y_stride, act_out};
+    bool done = false;
+    const int rc = mul_mat_q8k_tiled_launch(stream, type, 1, &m, act, K, B, ws, ws_bytes, &nm, &done);
+    if (rc != MI355_OK || done) return rc;
+    return mi355_rms_norm_mul_quant_q8k_tiled(stream, dst, dst_stride, norm_w, y, y_stride, act_out, N, B, eps);   // an uncut product: the norm is its own launch
 }
 
 int mi355_mul_mat_q8k_tiled(void *stream, int type, const void *tiles, const void *act, float *dst, const float *residual, int64_t N,

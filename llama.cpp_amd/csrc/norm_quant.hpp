@@ -73,9 +73,10 @@ __device__ __forceinline__ void quantize_lane32(float v, int8_t *__restrict__ qr
 // match with a barrier of their own.
 template <int NV, int FMT, bool COH>
 // keep: where the caller wants the thread's NV pieces of the normalised row (registers), or null
+// given: the thread's NV pieces of the row when the caller has just formed them (xr is not read then), or null
 __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr, const float *__restrict__ w, float *__restrict__ yr,
                                                    void *__restrict__ act, int64_t row, int64_t k, int64_t nrows, float eps, float *sh,
-                                                   f32x4 *keep = nullptr) {
+                                                   f32x4 *keep = nullptr, const f32x4 *given = nullptr) {
     const int tid = threadIdx.x;
     f32x4 v[NV], ww[NV];
     // the weight does not depend on the reduction: fetch it together with the row, one memory round trip instead of two
@@ -85,7 +86,9 @@ __device__ __forceinline__ void rms_norm_quant_row(const float *__restrict__ xr,
         v[it] = f32x4{0.f, 0.f, 0.f, 0.f};
         ww[it] = f32x4{1.f, 1.f, 1.f, 1.f};
         if (e0 < k) {
-            if constexpr (COH) {
+            if (given) {
+                v[it] = given[it];
+            } else if constexpr (COH) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) v[it][i] = __hip_atomic_load(xr + e0 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             } else {

@@ -93,6 +93,7 @@ _SIGNATURES = {
     "mi355_mul_mat_id_q8k_tiled": (_int, [_p, _int, _p, _sz, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_q8k_tiled_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_q8k_tiled_norm": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz, _p, _f, _p, _i64, _p]),
     "mi355_mul_mat_q8k_tiled_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled_multi": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_vec_q_multi": (_int, [_p, _int, _p, _p, _i64, _i64]),
@@ -321,6 +322,20 @@ def mul_mat_q8k_tiled(t, tiles, act, N, K, B, residual=None, split=True, dst=Non
     check(load().mi355_mul_mat_q8k_tiled(_stream(), t, _ptr(tiles), _ptr(act), _ptr(dst), _ptr(residual) if residual is not None else None,
                                          N, K, B, dst.stride(0), _ptr(ws) if nws else None, nws))
     return dst
+
+
+def mul_mat_q8k_tiled_norm(t, tiles, act, N, K, B, norm_w, eps, residual=None, split=True, dst=None):
+    """the wide-tile K-quant GEMM (+ residual) followed by RMS_NORM * norm_w of its rows -> (dst f32 [B, N], y f32 [B, N], tile image of y)"""
+    import torch
+    if dst is None:
+        dst = torch.empty((B, N), dtype=torch.float32, device=tiles.device)
+    y = torch.empty((B, N), dtype=torch.float32, device=tiles.device)
+    img = torch.zeros(load().mi355_act_q8k_tiled_bytes(N, B), dtype=torch.uint8, device=tiles.device)
+    nws = load().mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) if split else 0
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=tiles.device)
+    check(load().mi355_mul_mat_q8k_tiled_norm(_stream(), t, _ptr(tiles), _ptr(act), _ptr(dst), _ptr(residual) if residual is not None else None,
+                                              N, K, B, dst.stride(0), _ptr(ws) if nws else None, nws, _ptr(norm_w), eps, _ptr(y), y.stride(0), _ptr(img)))
+    return dst, y, img
 
 
 def mul_mat(t, W, x, ws=None, split=True):

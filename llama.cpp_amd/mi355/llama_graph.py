@@ -123,6 +123,7 @@ class LlamaRunner:
         # that the 2 bytes per weight make the product HBM-bound and the kernel that unpacks the 4.5-bit rows wins
         self.use_tiles = True
         self.tiles = {}
+        self.fuse_sum_norm = True   # prefill: a cut product's sum launch also normalises and quantizes its rows for the next products
         self.split_ws = None    # partial sums of tile products that are split along K (grown on first use, before any graph capture)
         # decode, T <= 4: SiLU*up + Q8_1 inside the gate/up launch (True: with both matrices of one type a group owns a whole 32-row
         # block of both and quantizes it itself; otherwise the last group of each block finishes it) or as a launch of their own
@@ -239,8 +240,11 @@ class LlamaRunner:
               self.lib.mi355_rms_norm_mul_quant_q8k_tiled)[int(q8k)]
         check(fn(_stream(), _ptr(x), x.stride(0), _ptr(w), None, 0, _ptr(act), K, T, self.cfg.rms_eps))
 
-    def _mm_act(self, mats, act, K, T, residual=None, q8k=False):
-        """mats: list of ((type, W), out); all consume the quantized activation `act` (T rows of K)"""
+    def _mm_act(self, mats, act, K, T, residual=None, q8k=False, norm=None):
+        """mats: list of ((type, W), out); all consume the quantized activation `act` (T rows of K).
+        norm: (norm weight, activation buffer) - the single product's rows are normalised next and their tile image goes to the
+        buffer (wide-tile GEMM only: the launch that adds a cut product's slices carries the norm)"""
+        assert norm is None or (q8k == 2 and len(mats) == 1 and T > 8)
         if T <= 8:
             arr = (GemvMat * len(mats))()
             for i, ((t, W), out) in enumerate(mats):
@@ -277,7 +281,10 @@ class LlamaRunner:
                         self.split_ws = torch.empty(need + 256, dtype=torch.uint8, device=self.dev)
                     sw, sn = (_ptr(self.split_ws), self.split_ws.numel()) if need else (None, 0)
                     res = _ptr(residual) if residual is not None else None
-                    if q8k == 2:
+                    if q8k == 2 and norm is not None:
+                        check(self.lib.mi355_mul_mat_q8k_tiled_norm(_stream(), t, _ptr(self._tiles(t, W, N, K)), _ptr(act), _ptr(out), res, N, K, T,
+                                                                    out.stride(0), sw, sn, _ptr(norm[0]), self.cfg.rms_eps, None, 0, _ptr(norm[1])))
+                    elif q8k == 2:
                         check(self.lib.mi355_mul_mat_q8k_tiled(_stream(), t, _ptr(self._tiles(t, W, N, K)), _ptr(act), _ptr(out), res, N, K, T,
                                                                out.stride(0), sw, sn))
                     elif t == Q6_K and self.use_planes:   # Q6_K streams its int8 planes, unpacked once per matrix
@@ -298,10 +305,12 @@ class LlamaRunner:
         x = self.x[:T]
         if T <= 4 and self.fuse_qkv and (T == 1 or not last_only):
             return self._forward_decode(T, n_kv)
+        normed = False   # the previous layer's ffn_down product has left this layer's normalised input in act_a
         for il, L in enumerate(w.layers):
             qkv = [(L["wq"], self.q[:T]), (L["wk"], self.k[:T]), (L["wv"], self.v[:T])]
             kq = self._fmt(qkv, E, T)
-            self._norm_quant(x, L["attn_norm"], self.act_a, T, kq)
+            if not normed:
+                self._norm_quant(x, L["attn_norm"], self.act_a, T, kq)
             kc, vc = self.kcache[il], self.vcache[il]
             if T <= 4 and self.fuse_qkv:    # decode: projections, rope and KV store in one launch
                 (tq, Wq), (tk, Wk), (tv, Wv) = L["wq"], L["wk"], L["wv"]
@@ -320,16 +329,21 @@ class LlamaRunner:
                 self._quant(self.attn, self.act_a, H * D, T, kq)
             else:
                 self._attn(il, T, n_kv, act=self.act_a)   # attention writes its own Q8_1 output
-            self._mm_act(wo, self.act_a, H * D, T, residual=x, q8k=kq)
             gu = [(L["gate"], self.gate[:T]), (L["up"], self.up[:T])]
-            kq = self._fmt(gu, E, T)
-            self._norm_quant(x, L["ffn_norm"], self.act_a, T, kq)
-            self._mm_act(gu, self.act_a, E, T, q8k=kq)
+            kq_gu = self._fmt(gu, E, T)
+            # wide-tile products on both sides of a norm: the product's sum launch also normalises and quantizes the rows it forms
+            fuse = self.fuse_sum_norm and kq == 2 and kq_gu == 2 and E % 256 == 0
+            self._mm_act(wo, self.act_a, H * D, T, residual=x, q8k=kq, norm=(L["ffn_norm"], self.act_a) if fuse else None)
+            if not fuse:
+                self._norm_quant(x, L["ffn_norm"], self.act_a, T, kq_gu)
+            self._mm_act(gu, self.act_a, E, T, q8k=kq_gu)
             down = [(L["down"], x)]
             kq = self._fmt(down, F, T)
             fn = (lib.mi355_swiglu_quant, lib.mi355_swiglu_quant_q8k, lib.mi355_swiglu_quant_q8k_tiled, lib.mi355_swiglu_quant_q8k_tiled)[kq]
             check(fn(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
-            self._mm_act(down, self.act_b, F, T, residual=x, q8k=kq)
+            nxt = w.layers[il + 1] if il + 1 < len(w.layers) else None
+            normed = self.fuse_sum_norm and nxt is not None and kq == 2 and E % 256 == 0 and self._fmt([(nxt["wq"], self.q[:T]), (nxt["wk"], self.k[:T]), (nxt["wv"], self.v[:T])], E, T) == 2
+            self._mm_act(down, self.act_b, F, T, residual=x, q8k=kq, norm=(nxt["attn_norm"], self.act_a) if normed else None)
         To = 1 if last_only else T
         xo = self.x[T - 1:T] if last_only else x
         out = [(w.output, self.logits[:To])]

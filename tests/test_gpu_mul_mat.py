@@ -401,6 +401,43 @@ def test_fused_producers_write_tile_images(dev, name, t):
 
 
 @pytest.mark.parametrize("name,t", TILED_TYPES)
+@pytest.mark.parametrize("N,K,B,split", [(4096, 4096, 512, True),       # wo of an 8B llama: cut along K, the sum launch carries the norm
+                                         (4096, 14336, 512, True),      # ffn_down
+                                         (2048, 2048, 300, True),       # ragged batch
+                                         (4096, 4096, 512, False),      # no workspace: uncut, the norm is its own launch
+                                         (4096, 2048, 2048, True),      # enough tiles: uncut
+                                         (8192, 2048, 200, True)])      # rows longer than the fused form takes
+def test_mmq_tiled_norm_equals_product_then_norm(dev, name, t, N, K, B, split):
+    """MUL_MAT (+ residual) -> RMS_NORM -> MUL(weight) -> tile image as one call: the bits of the product followed by the norm launch,
+    in the row, in the normalised row and in every byte of the image that the norm launch writes"""
+    import torch
+    import mi355
+    lib = mi355.load()
+    rng = np.random.default_rng(N + K + B + t)
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    act = mi355.quantize_act_q8k_tiled(_to_dev(dev, x))
+    tiles = mi355.kq_unpack_tiles(t, mi355.upload_weights(t, _to_dev(dev, _weights(rng, t, N, K, "ref"))))
+    res = _to_dev(dev, rng.standard_normal((B, N)).astype(np.float32))
+    nw = _to_dev(dev, rng.standard_normal(N).astype(np.float32))
+    for residual in (res, None):
+        want_x = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B, residual=residual, split=split)
+        want_y = torch.empty((B, N), dtype=torch.float32, device=dev)
+        want_img = torch.zeros(lib.mi355_act_q8k_tiled_bytes(N, B), dtype=torch.uint8, device=dev)
+        mi355.check(lib.mi355_rms_norm_mul_quant_q8k_tiled(None, want_x.data_ptr(), N, nw.data_ptr(), want_y.data_ptr(), N, want_img.data_ptr(), N, B, 1e-5))
+        got_x, got_y, got_img = mi355.mul_mat_q8k_tiled_norm(t, tiles, act, N, K, B, nw, 1e-5, residual=residual, split=split)
+        torch.cuda.synchronize()
+        assert np.array_equal(got_x.cpu().numpy(), want_x.cpu().numpy())
+        assert np.array_equal(got_y.cpu().numpy(), want_y.cpu().numpy())
+        assert np.array_equal(got_img.cpu().numpy(), want_img.cpu().numpy())     # both start from zeros: bytes neither writes agree too
+    # in place: the residual is the destination (what the ggml graph allocator hands out for MUL_MAT -> ADD)
+    dst = res.clone()
+    got_x, got_y, got_img = mi355.mul_mat_q8k_tiled_norm(t, tiles, act, N, K, B, nw, 1e-5, residual=dst, split=split, dst=dst)
+    want_x = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B, residual=res, split=split)
+    torch.cuda.synchronize()
+    assert np.array_equal(got_x.cpu().numpy(), want_x.cpu().numpy())
+
+
+@pytest.mark.parametrize("name,t", TILED_TYPES)
 @pytest.mark.parametrize("Ns,K,B", [((14336, 14336), 4096, 512),       # gate + up of an 8B llama: 896 tiles
                                     ((4096, 1024, 1024), 4096, 512),    # Q, K, V: 192 tiles in one round
                                     ((8200, 8300, 130), 2048, 300),     # ragged rows and batch
