@@ -245,6 +245,12 @@ typedef struct mi355_tiled_mat {
 size_t mi355_mul_mat_q8k_tiled_multi_ws_bytes(int n_mats, const int64_t *Ns, int64_t K, int64_t B);
 int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
                                   void *ws, size_t ws_bytes);
+/* The same launch for matrices of different K-quant types (types[i] of mats[i]): llama-quantize's Q4_K_M mix gives attn_v and ffn_down
+ * Q6_K in half of the layers (src/llama-quant.cpp:122-340), and a lone Q6_K V product is 32 tiles at batch 512 - cut along K and
+ * summed by a second launch after the Q + K launch, or 32 more tiles inside that launch, which leaves compute units free.  The planes of
+ * the three types differ only in the radix between them (8, 16, 64), taken per matrix; Q6_K images carry zero minima.  Every matrix
+ * gets the bits of its own mi355_mul_mat_q8k_tiled launch without a workspace.  No split along K. */
+int mi355_mul_mat_q8k_tiled_mixed(void *stream, int n_mats, const int *types, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B);
 
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE

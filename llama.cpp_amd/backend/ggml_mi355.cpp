@@ -1400,40 +1400,36 @@ void note_window_writes(backend_ctx * ctx, const qkv_window & win, int64_t B) {
 // the v product, so the rotations cannot simply wait for the products: instead the q and k products write straight into the
 // memory of their ROPE nodes' results, which nothing else can occupy before those results are read (q by attention, k by its
 // cache store), and are rotated there.
-// Several K-quant products on one activation at a large batch: those of one weight type that have tile images go out as one
-// launch of the wide-tile GEMM, so that their tiles fill the compute units together (mi355_mul_mat_q8k_tiled_multi).  idx: graph
+// Several K-quant products on one activation at a large batch: those that have tile images go out as one launch of the wide-tile
+// GEMM, whatever their K-quant types, so that their tiles fill the compute units together (mi355_mul_mat_q8k_tiled_mixed).  idx: graph
 // positions of the products, all reading the same src1.  Returns the mask of the products done (0 or at least two bits).
 unsigned tiled_multi(backend_ctx * ctx, hipStream_t s, const graph_walk & w, const int * idx, int n) {
     const ggml_tensor * b = w.nodes[idx[0]]->src[1];
     const int64_t K = b->ne[0], B = b->ne[1];
     const void * tl[3] = {nullptr, nullptr, nullptr};
-    const ggml_type kinds[3] = {GGML_TYPE_Q4_K, GGML_TYPE_Q5_K, GGML_TYPE_Q6_K};
-    int n_of[3] = {0, 0, 0};
+    int n_with = 0;
     for (int k = 0; k < n && k < 3; k++) {
         const ggml_tensor * mm = w.nodes[idx[k]];
         if (!is_q8k_tile_candidate(mm) || mm->src[1]->data != b->data || mm->src[1]->ne[0] != K || mm->src[1]->ne[1] != B || mm->src[1]->nb[1] != b->nb[1] ||
             mm->type != GGML_TYPE_F32 || mm->nb[0] != sizeof(float) || mm->nb[1] % sizeof(float) != 0 || takes_mid_kernel(mm) || q8k_format_for(s, mm) != ACT_Q8KT)
             continue;
         tl[k] = tiles().get(s, mm->src[0]);
-        if (tl[k])
-            for (int t = 0; t < 3; t++) n_of[t] += mm->src[0]->type == kinds[t];
+        n_with += tl[k] != nullptr;
     }
-    int best = 0;
-    for (int t = 1; t < 3; t++)
-        if (n_of[t] > n_of[best]) best = t;
-    const ggml_type type = kinds[best];
-    if (n_of[best] < 2) return 0;
+    if (n_with < 2) return 0;
     if (!ctx->cached(b->data, K, B, ACT_Q8KT)) {
         void * fresh = ctx->act_slot(mi355_act_q8k_tiled_bytes(K, B));
         MI355_K_OK(mi355_quantize_act_q8k_tiled(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
         ctx->cache = act_cache{b->data, K, B, ACT_Q8KT, true, fresh};
     }
     mi355_tiled_mat mats[3];
+    int types[3] = {0, 0, 0};
     unsigned mask = 0;
     int m = 0;
     for (int k = 0; k < n && k < 3; k++) {
         const ggml_tensor * mm = w.nodes[idx[k]];
-        if (!tl[k] || mm->src[0]->type != type) continue;
+        if (!tl[k]) continue;
+        types[m] = to_mi355_type(mm->src[0]->type);
         mats[m].tiles = tl[k];
         mats[m].dst = (float *) ctx->out_ptr(mm);
         mats[m].residual = nullptr;
@@ -1442,7 +1438,7 @@ unsigned tiled_multi(backend_ctx * ctx, hipStream_t s, const graph_walk & w, con
         m++;
         mask |= 1u << k;
     }
-    MI355_K_OK(mi355_mul_mat_q8k_tiled_multi(s, to_mi355_type(type), m, mats, ctx->cache.ptr, K, B, nullptr, 0));
+    MI355_K_OK(mi355_mul_mat_q8k_tiled_mixed(s, m, types, mats, ctx->cache.ptr, K, B));
     for (int k = 0; k < m; k++) ctx->note_write(mats[k].dst, (size_t) mats[k].N * (size_t) B * sizeof(float));
     return mask;
 }
@@ -1653,7 +1649,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
             ctx->redirect_node[1] = p.mk;  ctx->redirect_to[1] = p.rk->data;
             ctx->n_redirect = 2;
             const int at[3] = {i, p.ik, p.iv};
-            const unsigned together = tiled_multi(ctx, s, w, at, 3);   // those of one K-quant type in one launch
+            const unsigned together = tiled_multi(ctx, s, w, at, 3);   // those with tile images in one launch
             for (int k = 0; k < 3; k++) {
                 if (together & (1u << k)) continue;
                 const int done = compute_fused(ctx, w, at[k]);

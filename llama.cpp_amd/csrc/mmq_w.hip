@@ -193,9 +193,14 @@ __global__ void __launch_bounds__(256) k_unpack_tiles(const uint8_t *__restrict_
         }
         c0 = 2 * qa + (p & 1);
         c1 = c0 + 4;
-        if (half == 0 && p == 0) {
+        if (half == 0 && p == 0) {   // the Q4_K entry with no minima
             uint8_t *e = aux + (sb * n_rb_pad + (row >> 4)) * W_AUX;
-            *(float *)(e + (row & 15) * 4) = live ? half_bits_to_float(*(const unsigned short *)(wrow + L.off_d + sb * 2)) : 0.0f;
+            const int r = (int)(row & 15);
+            const u32x4 z = {0, 0, 0, 0};
+            *(u32x4 *)(e + r * 32) = z;
+            *(u32x4 *)(e + r * 32 + 16) = z;
+            *(float *)(e + 512 + r * 4) = live ? half_bits_to_float(*(const unsigned short *)(wrow + L.off_d + sb * 2)) : 0.0f;
+            *(float *)(e + 576 + r * 4) = 0.0f;
         }
     }
     *(u32x4 *)(hi_img + wt_tile_off(row, k0 + c0 * 16, K)) = a1;
@@ -258,6 +263,7 @@ struct wt_mat {
     const float *residual;   // may be null; same shape and stride as dst; may be dst itself
     int64_t N, dst_stride;
     int first_tile;          // index of this matrix's first tile in the launch (unused entries: INT_MAX)
+    int shift;               // log2 of the radix between the matrix's two planes: 3 Q4_K, 4 Q5_K, 6 Q6_K
 };
 struct wt_launch {
     wt_mat m[3];
@@ -267,17 +273,19 @@ struct wt_launch {
 
 // ID: MUL_MAT_ID.  The "matrix" is expert 0's images, the column tiles are those of the sorted slot list (rt), B the rows of the
 // activation image (128 per column tile); a tile's rows go to the dst rows of its slots.
+// TYPE: MI355_Q4_K = the form with the min term, the radix between the planes taken from the matrix (Q4_K, Q5_K, and Q6_K images,
+// whose minima are zeros, in a launch they share with the other two); MI355_Q6_K = launches of Q6_K matrices only: no min term.
 template <int TYPE, bool ID = false>
 __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__restrict__ a_img, int64_t K, int64_t B, wt_route rt) {
-    constexpr bool Q4 = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K;   // sub-block mins: the min term and its scale records
-    constexpr int RADIX_SHIFT = TYPE == MI355_Q4_K ? 3 : (TYPE == MI355_Q5_K ? 4 : 6);
+    static_assert(TYPE == MI355_Q4_K || TYPE == MI355_Q6_K, "two forms");
+    constexpr bool Q4 = TYPE == MI355_Q4_K;   // sub-block mins: the min term and its scale records
     constexpr int NP = 2;                                                      // weight planes
     constexpr int W_AUX = wt_w_aux_bytes(TYPE);
     constexpr int STAGE = (NP * WT_BM + WT_BN) * 64;                           // bytes of one 64-element stage: plane(s), activations
     constexpr int OFF_LO = WT_BM * 64, OFF_A = NP * WT_BM * 64;
     constexpr int DPS = NP + 1;                                                // transfers per wave and stage
     constexpr int N_A_CHUNKS = (WT_A_AUX_TILE + 1023) / 1024;                  // 5, the last one half full
-    constexpr int N_W_CHUNKS = (WT_BM / 16) * W_AUX / 1024;                    // 5 or 1
+    constexpr int N_W_CHUNKS = (WT_BM / 16) * W_AUX / 1024;                    // 5
     constexpr int N_CHUNKS = N_A_CHUNKS + N_W_CHUNKS;                          // scale transfers per super-block
     constexpr int AUX_W_OFF = N_A_CHUNKS * 1024;                               // weight entries behind the (padded) activation entries
     // Ring of stage buffers: 8 (two super-blocks) where they fit, else 4; a stage's transfers are issued DIST stages ahead.
@@ -300,6 +308,7 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__r
     const float *residual = P.m[mi].residual;
     const int64_t N = P.m[mi].N;
     const int64_t dst_stride = P.m[mi].dst_stride;
+    const int radix_shift = Q4 ? __builtin_amdgcn_readfirstlane(P.m[mi].shift) : 6;
     const int n_col_tiles = P.n_col_tiles;
     const int ltile = tile - P.m[mi].first_tile;
     const int64_t row0 = (int64_t)(ltile / n_col_tiles) * WT_BM;
@@ -402,7 +411,7 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__r
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int r = 4 * q + i;
-            const float f = (float)((h[r] << RADIX_SHIFT) + l[r]);
+            const float f = (float)((h[r] << radix_shift) + l[r]);
             if constexpr (Q4) acc[tb][r] = __builtin_fmaf(d8[i], __builtin_fmaf(-dn, M[r], mul_rn(dw, f)), acc[tb][r]);
             else acc[tb][r] = __builtin_fmaf(d8[i], mul_rn(dw, f), acc[tb][r]);
         }
@@ -521,7 +530,7 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__r
                     e_dw = *(const float *)(ax_cur + (we_off + 512 + (l32 & 15) * 4));
                     e_dn = *(const float *)(ax_cur + (we_off + 576 + (l32 & 15) * 4));
                 } else {
-                    e_dw = *(const float *)(ax_cur + (we_off + (l32 & 15) * 4));
+                    e_dw = *(const float *)(ax_cur + (we_off + 512 + (l32 & 15) * 4));
                 }
             }
             if (Q4 && PREV && piece == 2) e_am = load_am(ax_prev, 1);
@@ -733,18 +742,30 @@ struct wt_norm {
     int64_t y_stride;
     void *act_out;
 };
-static int mul_mat_q8k_tiled_launch(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
+static int wt_radix_shift(int type) { return type == MI355_Q4_K ? 3 : type == MI355_Q5_K ? 4 : 6; }
+
+static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
                                     size_t ws_bytes, const wt_norm *norm, bool *norm_done);
 
 int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
                                   void *ws, size_t ws_bytes) {
-    return mul_mat_q8k_tiled_launch(stream, type, n_mats, mats, act, K, B, ws, ws_bytes, nullptr, nullptr);
+    const int types[3] = {type, type, type};
+    return mul_mat_q8k_tiled_launch(stream, types, n_mats, mats, act, K, B, ws, ws_bytes, nullptr, nullptr);
 }
 
-static int mul_mat_q8k_tiled_launch(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
+int mi355_mul_mat_q8k_tiled_mixed(void *stream, int n_mats, const int *types, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B) {
+    MI355_REQUIRE(types != nullptr, "mul_mat_q8k_tiled_mixed: no types");
+    return mul_mat_q8k_tiled_launch(stream, types, n_mats, mats, act, K, B, nullptr, 0, nullptr, nullptr);
+}
+
+static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
                                     size_t ws_bytes, const wt_norm *norm, bool *norm_done) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", type);
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_q8k_tiled: 1 to 3 matrices per launch, got %d", n_mats);
+    bool all_q6 = true;
+    for (int i = 0; i < n_mats; i++) {
+        MI355_REQUIRE(types[i] == MI355_Q4_K || types[i] == MI355_Q5_K || types[i] == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", types[i]);
+        all_q6 = all_q6 && types[i] == MI355_Q6_K;
+    }
     MI355_REQUIRE(K > 0 && B > 0 && K % QKK == 0, "mul_mat_q8k_tiled: bad shape K=%lld B=%lld (K must be a multiple of 256)", (long long)K, (long long)B);
     MI355_REQUIRE(act != nullptr && ((uintptr_t)act & 15) == 0, "mul_mat_q8k_tiled: the activation image is not 16-byte aligned");
     int64_t Ns[3] = {0, 0, 0};
@@ -767,6 +788,7 @@ static int mul_mat_q8k_tiled_launch(void *stream, int type, int n_mats, const mi
         L.m[i].N = mats[k].N;
         L.m[i].dst_stride = mats[k].dst_stride;
         L.m[i].first_tile = p.first_tile[i];
+        L.m[i].shift = wt_radix_shift(types[k]);
     }
     L.n_col_tiles = p.n_col_tiles;
     L.n_tiles = p.n_tiles;
@@ -777,9 +799,8 @@ static int mul_mat_q8k_tiled_launch(void *stream, int type, int n_mats, const mi
         L.m[0].dst_stride = Ns[0];
     }
     const dim3 grid((unsigned)L.n_tiles_padded, (unsigned)p.slices);
-    if (type == MI355_Q4_K) MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
-    else if (type == MI355_Q5_K) MI355_LAUNCH(k_mmq_w<MI355_Q5_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
-    else MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
+    if (all_q6) MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
+    else MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
     if (p.slices > 1 && norm && Ns[0] <= 4096 && mats[0].dst_stride % 4 == 0 && ((uintptr_t)mats[0].dst & 15) == 0 &&
         (mats[0].residual == nullptr || ((uintptr_t)mats[0].residual & 15) == 0)) {
         MI355_LAUNCH((k_wt_split_sum_norm<4>), dim3((unsigned)B), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B, mats[0].dst_stride,
@@ -807,7 +828,7 @@ int mi355_mul_mat_q8k_tiled_norm(void *stream, int type, const void *tiles, cons
     m.dst_stride = dst_stride;
     const wt_norm nm = {norm_w, eps, y, y_stride, act_out};
     bool done = false;
-    const int rc = mul_mat_q8k_tiled_launch(stream, type, 1, &m, act, K, B, ws, ws_bytes, &nm, &done);
+    const int rc = mul_mat_q8k_tiled_launch(stream, &type, 1, &m, act, K, B, ws, ws_bytes, &nm, &done);
     if (rc != MI355_OK || done) return rc;
     return mi355_rms_norm_mul_quant_q8k_tiled(stream, dst, dst_stride, norm_w, y, y_stride, act_out, N, B, eps);   // an uncut product: the norm is its own launch
 }
@@ -863,6 +884,7 @@ int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles,
         L.m[i].N = N;
         L.m[i].dst_stride = N;
         L.m[i].first_tile = i == 0 ? 0 : 0x7fffffff;
+        L.m[i].shift = wt_radix_shift(type);
     }
     const int64_t n_row_tiles = (N + WT_BM - 1) / WT_BM;
     MI355_REQUIRE(n_row_tiles * max_tiles + 8 < (1 << 30), "mul_mat_id_q8k_tiled: too many tiles");
@@ -871,9 +893,8 @@ int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles,
     L.n_tiles_padded = (L.n_tiles + 7) & ~7;
     const wt_route rt = {dst_row, tiles, n_tiles, (int64_t)expert_tiles_bytes};
     const dim3 grid((unsigned)L.n_tiles_padded);
-    if (type == MI355_Q4_K) MI355_LAUNCH((k_mmq_w<MI355_Q4_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
-    else if (type == MI355_Q5_K) MI355_LAUNCH((k_mmq_w<MI355_Q5_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
-    else MI355_LAUNCH((k_mmq_w<MI355_Q6_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
+    if (type == MI355_Q6_K) MI355_LAUNCH((k_mmq_w<MI355_Q6_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
+    else MI355_LAUNCH((k_mmq_w<MI355_Q4_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
     return launch_status("k_mmq_w (routed)");
 }
 

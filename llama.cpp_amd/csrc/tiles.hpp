@@ -10,9 +10,10 @@
 //                                                 bs = {bsum_j & 63 (j = 0..7), bsum_j >> 6 (j = 0..7)}; cb_pad = B16/16 rounded up to 16
 //   weights (mi355_kq_unpack_tiles):              int8 hi image [N16 x K], int8 lo image [N16 x K]   (value = R * hi + lo;
 //                                                 Q4_K: sc * n with R = 8, Q5_K: sc * n with R = 16, Q6_K: sc * (l - 32) with R = 64)
-//                                                 aux [K/256][rb_pad][W_AUX]: per 16 rows, Q4_K and Q5_K (640 bytes):
-//                                                 { fp16 m[16][16] = {min_j, 64 * min_j}; float d[16]; float dmin[16] },
-//                                                 Q6_K (128 bytes): { float d[16]; pad }; rb_pad = N16/16 rounded up to 8
+//                                                 aux [K/256][rb_pad][640]: per 16 rows
+//                                                 { fp16 m[16][16] = {min_j, 64 * min_j}; float d[16]; float dmin[16] }
+//                                                 (Q6_K has no minima: zeros there, so that its images can ride in a launch of the
+//                                                 kernel that handles them); rb_pad = N16/16 rounded up to 8
 // Levels, scales and sums are those of quantize_row_q8_K_ref (ggml/src/ggml-quants.c:2479-2516) and of the Q4_K / Q6_K
 // dequantizers (ggml/src/ggml-quants.c:1280-1302, 1690-1719).
 #pragma once
@@ -24,7 +25,7 @@ namespace mi355 {
 constexpr int WT_TILE = 1024;
 constexpr int WT_A_AUX = 576;
 
-__host__ __device__ constexpr int wt_w_aux_bytes(int type) { return type == MI355_Q6_K ? 128 : 640; }
+__host__ __device__ constexpr int wt_w_aux_bytes(int) { return 640; }
 __host__ __device__ inline int64_t wt_rb_pad(int64_t N) { return (((N + 15) >> 4) + 7) & ~(int64_t)7; }
 __host__ __device__ inline int64_t wt_cb_pad(int64_t B) { return (((B + 15) >> 4) + 15) & ~(int64_t)15; }
 

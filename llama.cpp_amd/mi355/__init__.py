@@ -93,6 +93,7 @@ _SIGNATURES = {
     "mi355_mul_mat_id_q8k_tiled": (_int, [_p, _int, _p, _sz, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_q8k_tiled_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_q8k_tiled_mixed": (_int, [_p, _int, _p, _p, _p, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled_norm": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz, _p, _f, _p, _i64, _p]),
     "mi355_mul_mat_q8k_tiled_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled_multi": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _sz]),
@@ -295,7 +296,8 @@ def kq_unpack_tiles(t, W):
 
 
 def mul_mat_q8k_tiled_multi(t, tiles_list, act, Ns, K, B, dsts=None, residuals=None):
-    """one launch of the wide-tile K-quant GEMM for up to three matrices of type t that share `act` -> list of f32 [B, N_i]"""
+    """one launch of the wide-tile K-quant GEMM for up to three matrices of type t (a list: one type per matrix) that share `act`
+    -> list of f32 [B, N_i]"""
     import torch
     n = len(tiles_list)
     dev = tiles_list[0].device
@@ -305,6 +307,9 @@ def mul_mat_q8k_tiled_multi(t, tiles_list, act, Ns, K, B, dsts=None, residuals=N
     for i in range(n):
         arr[i].tiles, arr[i].dst, arr[i].N, arr[i].dst_stride = tiles_list[i].data_ptr(), dsts[i].data_ptr(), Ns[i], dsts[i].stride(0)
         arr[i].residual = residuals[i].data_ptr() if residuals is not None and residuals[i] is not None else None
+    if isinstance(t, (list, tuple)):
+        check(load().mi355_mul_mat_q8k_tiled_mixed(_stream(), n, (C.c_int * n)(*t), arr, _ptr(act), K, B))
+        return dsts
     ns = (C.c_int64 * n)(*Ns)
     nws = load().mi355_mul_mat_q8k_tiled_multi_ws_bytes(n, ns, K, B)
     ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)

@@ -252,19 +252,14 @@ class LlamaRunner:
                 arr[i].residual = residual.data_ptr() if residual is not None else None
             check(self.lib.mi355_mul_mat_vec_q_multi(_stream(), len(mats), arr, _ptr(act), K, T))
         else:
-            if q8k == 2 and len(mats) > 1:   # matrices of one type go out as one launch of the wide-tile GEMM
-                rest = []
-                for t in sorted({m[0][0] for m in mats}):
-                    same = [m for m in mats if m[0][0] == t]
-                    if len(same) == 1:
-                        rest += same
-                        continue
-                    arr = (TiledMat * len(same))()
-                    for i, ((_, W), out) in enumerate(same):
-                        arr[i].tiles, arr[i].dst, arr[i].N, arr[i].dst_stride = self._tiles(t, W, out.shape[1], K).data_ptr(), out.data_ptr(), out.shape[1], out.stride(0)
-                        arr[i].residual = residual.data_ptr() if residual is not None else None
-                    check(self.lib.mi355_mul_mat_q8k_tiled_multi(_stream(), t, len(same), arr, _ptr(act), K, T, None, 0))
-                mats = rest
+            if q8k == 2 and 1 < len(mats) <= 3:   # one launch of the wide-tile GEMM, whatever the K-quant type of each matrix
+                arr = (TiledMat * len(mats))()
+                for i, ((t, W), out) in enumerate(mats):
+                    arr[i].tiles, arr[i].dst, arr[i].N, arr[i].dst_stride = self._tiles(t, W, out.shape[1], K).data_ptr(), out.data_ptr(), out.shape[1], out.stride(0)
+                    arr[i].residual = residual.data_ptr() if residual is not None else None
+                types = (C.c_int * len(mats))(*[t for (t, _), _ in mats])
+                check(self.lib.mi355_mul_mat_q8k_tiled_mixed(_stream(), len(mats), types, arr, _ptr(act), K, T))
+                mats = []
             for (t, W), out in mats:
                 if q8k == 3:
                     N = out.shape[1]

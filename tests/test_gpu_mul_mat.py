@@ -400,6 +400,31 @@ def test_fused_producers_write_tile_images(dev, name, t):
     assert np.array_equal(a3.cpu().numpy()[sel], a4.cpu().numpy()[sel])
 
 
+@pytest.mark.parametrize("types,Ns,K,B", [((orc.Q4_K, orc.Q4_K, orc.Q6_K), (4096, 1024, 1024), 4096, 512),   # Q, K, V of the Q4_K_M mix
+                                          ((orc.Q6_K, orc.Q5_K, orc.Q4_K), (1000, 8300, 130), 2048, 300),    # ragged rows and batch
+                                          ((orc.Q6_K, orc.Q4_K), (14336, 14336), 4096, 512),                  # 896 tiles
+                                          ((orc.Q6_K, orc.Q6_K), (520, 130), 2048, 200)])                      # Q6_K only: the form without a min term
+def test_mmq_tiled_mixed_types(dev, types, Ns, K, B):
+    """matrices of different K-quant types in one launch of the wide-tile GEMM: every matrix equals its own launch bit for bit, with
+    and without a residual, and the oracle's integer arithmetic at the corners"""
+    import mi355
+    rng = np.random.default_rng(sum(Ns) + K + B + sum(types))
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    act = mi355.quantize_act_q8k_tiled(_to_dev(dev, x))
+    Wq = [_weights(rng, t, N, K, "ref") for t, N in zip(types, Ns)]
+    tiles = [mi355.kq_unpack_tiles(t, mi355.upload_weights(t, _to_dev(dev, W))) for t, W in zip(types, Wq)]
+    res = [_to_dev(dev, rng.standard_normal((B, N)).astype(np.float32)) if i != 1 else None for i, N in enumerate(Ns)]
+    alone = [mi355.mul_mat_q8k_tiled(t, tl, act, N, K, B, split=False).cpu().numpy() for t, tl, N in zip(types, tiles, Ns)]
+    mixed = [o.cpu().numpy() for o in mi355.mul_mat_q8k_tiled_multi(list(types), tiles, act, list(Ns), K, B)]
+    with_res = [o.cpu().numpy() for o in mi355.mul_mat_q8k_tiled_multi(list(types), tiles, act, list(Ns), K, B, residuals=res)]
+    for i, (t, N) in enumerate(zip(types, Ns)):
+        assert np.array_equal(mixed[i], alone[i])
+        assert np.array_equal(with_res[i], mixed[i] + res[i].cpu().numpy() if res[i] is not None else mixed[i])
+        Nt, Bt = min(N, 40), min(B, 16)
+        assert orc.nmse(mixed[i][:Bt, :Nt], orc.mul_mat("cpu", t, Wq[i][:Nt], x[:Bt])) < 1e-9
+        assert orc.nmse(mixed[i][B - 5:, N - 7:], orc.mul_mat("cpu", t, Wq[i][N - 7:], x[B - 5:])) < 1e-9
+
+
 @pytest.mark.parametrize("name,t", TILED_TYPES)
 @pytest.mark.parametrize("N,K,B,split", [(4096, 4096, 512, True),       # wo of an 8B llama: cut along K, the sum launch carries the norm
                                          (4096, 14336, 512, True),      # ffn_down
