@@ -251,6 +251,18 @@ int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi35
  * the three types differ only in the radix between them (8, 16, 64), taken per matrix; Q6_K images carry zero minima.  Every matrix
  * gets the bits of its own mi355_mul_mat_q8k_tiled launch without a workspace.  No split along K. */
 int mi355_mul_mat_q8k_tiled_mixed(void *stream, int n_mats, const int *types, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B);
+/* Q, K and V of a prompt batch in that launch, with what llm_build_kv does to them next in its epilogue (src/llama.cpp:1514-1560:
+ * ggml_rope_ext on Q and K, ggml_cpy of K and V into the f16 cache views): mats[0] = Q, dst = the rotated q, f32 [B][N_q]; mats[1] = K
+ * and mats[2] = V, dst = base of the f16 cache, element (cell, head, d) at cells[b] * nb1 + head * nb2 + 2 * d (dst_stride unused).
+ * ROPE in its adjacent-pair mode (mode 0, ggml_compute_forward_rope_f32, ggml/src/ggml-cpu/ggml-cpu.c:9390-9470): the two elements of
+ * a pair are neighbouring rows of the matrix, hence neighbouring lanes of the result.  rope_table: {cos, sin} per (token, pair), T x D/2
+ * float pairs written by mi355_rope_table once per batch (positions and frequencies do not depend on the layer).  Same bits as
+ * mi355_mul_mat_q8k_tiled_mixed followed by mi355_rope_kv_store.  N_q, N_k = N_v multiples of D; no residual. */
+int mi355_rope_table(void *stream, const int32_t *pos, const float *freq_factors, float *table, int64_t T, int64_t D, int n_dims, int n_ctx_orig,
+                     float freq_base, float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow);
+int mi355_mul_mat_q8k_tiled_qkv_rope(void *stream, const int *types, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
+                                     const float *rope_table, const int32_t *cells, int64_t D, int n_dims, size_t k_nb1, size_t k_nb2, size_t v_nb1,
+                                     size_t v_nb2);
 
 /* Up to four weight matrices that consume the same quantized activation (the Q/K/V and the
  * gate/up projections of llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :200-330) in ONE

@@ -143,6 +143,13 @@ struct backend_ctx {
     act_cache cache;
     bool fuse = true;      // MI355_NO_FUSION=1 executes the graph node for node
     int32_t * iota = nullptr;   // device {0, 1, 2, ... IOTA_N - 1}: token t of a batch goes to row t of a KV-cache view
+    // {cos, sin} per (token, pair) of a prompt batch's rotations, written once per graph for the Q/K/V launches of all its layers
+    float * rope_tab = nullptr;
+    size_t rope_tab_floats = 0;
+    uint64_t graph_serial = 0, rope_tab_serial = 0;   // the table is that of graph rope_tab_serial ...
+    const void * rope_tab_pos = nullptr, * rope_tab_ff = nullptr;   // ... for these positions, frequency factors and parameters
+    int32_t rope_tab_params[11] = {0};
+    int64_t rope_tab_D = 0, rope_tab_T = 0;
     // products whose result is written somewhere else than into their own tensor (see match_prefill_qkv)
     const ggml_tensor * redirect_node[2] = {nullptr, nullptr};
     void * redirect_to[2] = {nullptr, nullptr};
@@ -936,6 +943,7 @@ void backend_free(ggml_backend_t backend) {
     if (ctx->ws) (void) hipFree(ctx->ws);
     if (ctx->act) (void) hipFree(ctx->act);
     if (ctx->iota) (void) hipFree(ctx->iota);
+    if (ctx->rope_tab) (void) hipFree(ctx->rope_tab);
     if (ctx->cells) (void) hipFree(ctx->cells);
     if (ctx->tickets) (void) hipFree(ctx->tickets);
     if (ctx->stage) (void) hipHostFree(ctx->stage);
@@ -1630,6 +1638,85 @@ bool router_outputs_apart(const ggml_tensor * x, const ggml_tensor * nw, const g
     return probs->data == logits->data || !bytes_overlap(probs, logits);
 }
 
+// The prefill window of match_prefill_qkv as ONE launch of the wide-tile GEMM: Q, K and V products whose epilogue rotates q and k
+// and stores k and v into the f16 cache views (mi355_mul_mat_q8k_tiled_qkv_rope).  Needs tile images of all three matrices, f16
+// caches and ROPE in its adjacent-pair mode.  The {cos, sin} table of the batch is written by the first layer's call of a graph.
+bool tiled_qkv_rope(backend_ctx * ctx, hipStream_t s, const graph_walk & w, int i, const prefill_qkv & p) {
+    const ggml_tensor * mm[3] = {w.nodes[i], p.mk, p.mv};
+    const ggml_tensor * b = mm[0]->src[1];
+    const ggml_tensor * rq = p.rq;
+    const int64_t K = b->ne[0], B = b->ne[1], D = rq->ne[0];
+    const int32_t * op = (const int32_t *) rq->op_params;
+    const ggml_tensor * dk = p.ck->src[1], * dv = p.cv->src[1];
+    if (op[2] != 0 || dk->type != GGML_TYPE_F16 || dv->type != GGML_TYPE_F16 || rq->src[1]->ne[0] != B || !ggml_is_contiguous(rq->src[1]) || B > IOTA_N) return false;
+    if (rq->src[2] && !ggml_is_contiguous(rq->src[2])) return false;
+    const void * tl[3];
+    int types[3];
+    for (int k = 0; k < 3; k++) {
+        const ggml_tensor * m = mm[k];
+        if (!is_q8k_tile_candidate(m) || m->src[1]->data != b->data || m->src[1]->nb[1] != b->nb[1] || takes_mid_kernel(m) || q8k_format_for(s, m) != ACT_Q8KT ||
+            m->src[0]->ne[1] % D != 0)
+            return false;
+        tl[k] = tiles().get(s, m->src[0]);
+        if (!tl[k]) return false;
+        types[k] = to_mi355_type(m->src[0]->type);
+    }
+    const int64_t HK = p.rk->ne[1];
+    if (mm[1]->src[0]->ne[1] != HK * D || mm[2]->src[0]->ne[1] != HK * D || ((uintptr_t) rq->data & 15) != 0) return false;
+    // the batch's rotations: once per graph (positions, frequency factors and parameters are the same in every layer)
+    const size_t tab_floats = (size_t) B * (size_t) D;
+    const bool tab_ok = ctx->rope_tab && ctx->rope_tab_serial == ctx->graph_serial && ctx->rope_tab_pos == rq->src[1]->data &&
+                        ctx->rope_tab_ff == (rq->src[2] ? rq->src[2]->data : nullptr) && ctx->rope_tab_D == D && ctx->rope_tab_T == B &&
+                        memcmp(ctx->rope_tab_params, op, sizeof(ctx->rope_tab_params)) == 0;
+    if (!tab_ok) {
+        if (tab_floats > ctx->rope_tab_floats) {
+            if (!ctx->may_allocate()) return false;
+            if (ctx->rope_tab) {
+                MI355_HIP_OK(hipStreamSynchronize(ctx->stream));
+                MI355_HIP_OK(hipFree(ctx->rope_tab));
+                ctx->rope_tab = nullptr;
+            }
+            ctx->rope_tab_floats = tab_floats;
+            MI355_HIP_OK(hipMalloc((void **) &ctx->rope_tab, tab_floats * sizeof(float)));
+        }
+        float freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
+        memcpy(&freq_base, op + 5, sizeof(float));
+        memcpy(&freq_scale, op + 6, sizeof(float));
+        memcpy(&ext_factor, op + 7, sizeof(float));
+        memcpy(&attn_factor, op + 8, sizeof(float));
+        memcpy(&beta_fast, op + 9, sizeof(float));
+        memcpy(&beta_slow, op + 10, sizeof(float));
+        MI355_K_OK(mi355_rope_table(s, (const int32_t *) rq->src[1]->data, rq->src[2] ? (const float *) rq->src[2]->data : nullptr, ctx->rope_tab, B, D, op[1], op[4],
+                                    freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow));
+        ctx->rope_tab_serial = ctx->graph_serial;
+        ctx->rope_tab_pos = rq->src[1]->data;
+        ctx->rope_tab_ff = rq->src[2] ? rq->src[2]->data : nullptr;
+        ctx->rope_tab_D = D;
+        ctx->rope_tab_T = B;
+        memcpy(ctx->rope_tab_params, op, sizeof(ctx->rope_tab_params));
+    }
+    if (!ctx->cached(b->data, K, B, ACT_Q8KT)) {
+        void * fresh = ctx->act_slot(mi355_act_q8k_tiled_bytes(K, B));
+        MI355_K_OK(mi355_quantize_act_q8k_tiled(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
+        ctx->cache = act_cache{b->data, K, B, ACT_Q8KT, true, fresh};
+    }
+    mi355_tiled_mat mats[3];
+    void * dst[3] = {rq->data, dk->data, dv->data};
+    for (int k = 0; k < 3; k++) {
+        mats[k].tiles = tl[k];
+        mats[k].dst = (float *) dst[k];
+        mats[k].residual = nullptr;
+        mats[k].N = mm[k]->src[0]->ne[1];
+        mats[k].dst_stride = mats[k].N;
+    }
+    MI355_K_OK(mi355_mul_mat_q8k_tiled_qkv_rope(s, types, mats, ctx->cache.ptr, K, B, ctx->rope_tab, ctx->iota, D, op[1], (size_t) (HK * D * 2), (size_t) (D * 2),
+                                                (size_t) (HK * D * 2), (size_t) (D * 2)));
+    ctx->note_write(rq->data, ggml_nbytes(rq));
+    ctx->note_write(dk->data, ggml_nbytes(dk));
+    ctx->note_write(dv->data, ggml_nbytes(dv));
+    return true;
+}
+
 // Runs node i and possibly a few of its successors; returns the index of the last node consumed.
 int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     hipStream_t s = ctx->stream;
@@ -1645,6 +1732,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
     if (node->op == GGML_OP_MUL_MAT && ctx->n_redirect == 0 && node->src[1]->ne[1] > 4) {
         const prefill_qkv p = match_prefill_qkv(w, i);
         if (p.ok) {
+            if (tiled_qkv_rope(ctx, s, w, i, p)) return p.last;
             ctx->redirect_node[0] = node;  ctx->redirect_to[0] = p.rq->data;
             ctx->redirect_node[1] = p.mk;  ctx->redirect_to[1] = p.rk->data;
             ctx->n_redirect = 2;
@@ -2311,6 +2399,7 @@ ggml_status backend_graph_compute(ggml_backend_t backend, ggml_cgraph * cgraph) 
     backend_ctx * ctx = (backend_ctx *) backend->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     ctx->cache.valid = false;
+    ctx->graph_serial++;
     if (!ctx->fuse) {
         const int n = ggml_graph_n_nodes(cgraph);
         for (int i = 0; i < n; i++) {

@@ -163,6 +163,18 @@ __device__ __forceinline__ void rope_cos_sin(const rope_kv_args &a, int pos, int
     s = sinf(theta) * mscale;
 }
 
+// {cos, sin} of every (token, pair), for a launch that rotates the rows it has just formed (the Q/K/V launch of the wide-tile GEMM):
+// the values k_rope_kv_store works out per pair, written once per batch and read by every layer's launch
+__global__ void __launch_bounds__(64) k_rope_table(rope_kv_args a, float2 *__restrict__ cs) {
+    const int t = blockIdx.x;
+    const int pos = a.pos[t];
+    for (int pair = threadIdx.x; 2 * pair < a.D; pair += 64) {
+        float c = 1.0f, sn = 0.0f;
+        if (2 * pair < a.n_dims) rope_cos_sin(a, pos, pair, c, sn);
+        cs[(int64_t)t * (a.D / 2) + pair] = make_float2(c, sn);
+    }
+}
+
 // One 256-thread group per token.  The rotation of a pair depends on the token's position and the pair only, so a wave works it
 // out once per pair (lane = pair) and applies it to every head it is given: the four waves share the H query heads, HK key heads
 // and HK value heads (plain f16 copies) between them, wave w taking slots w, w + 4, ...  Same roundings as k_rope: no contraction.
@@ -333,6 +345,30 @@ int mi355_swiglu_quant_q8k_tiled(void *stream, const float *gate, const float *u
     return swiglu_quant(stream, gate, up, in_stride, y, y_stride, act, k, nrows, 2);
 }
 
+static void rope_freq_args(rope_kv_args &a, int n_dims, int n_ctx_orig, float freq_base, float freq_scale, float ext_factor, float attn_factor,
+                           float beta_fast, float beta_slow) {
+    a.theta_scale = powf(freq_base, -2.0f / n_dims);
+    a.freq_scale = freq_scale; a.ext_factor = ext_factor; a.attn_factor = attn_factor;
+    const float pi = 3.14159265358979323846f;   // ggml_rope_yarn_corr_dims, ggml/src/ggml.c:3695-3707
+    const float c0 = floorf(n_dims * logf(n_ctx_orig / (beta_fast * 2 * pi)) / (2 * logf(freq_base)));
+    const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
+    a.corr0 = c0 > 0 ? c0 : 0;
+    a.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
+}
+
+int mi355_rope_table(void *stream, const int32_t *pos, const float *freq_factors, float *table, int64_t T, int64_t D, int n_dims, int n_ctx_orig,
+                     float freq_base, float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow) {
+    MI355_REQUIRE(T > 0 && T <= 65535 && D > 0 && D % 2 == 0 && D <= 2048, "rope_table: bad shape");
+    MI355_REQUIRE(n_dims > 0 && n_dims % 2 == 0 && n_dims <= D, "rope_table: bad n_dims");
+    MI355_REQUIRE(pos != nullptr && table != nullptr && ((uintptr_t)table & 7) == 0, "rope_table: null or misaligned operand");
+    rope_kv_args a = {};
+    a.pos = pos; a.ff = freq_factors;
+    a.T = (int)T; a.D = (int)D; a.n_dims = n_dims;
+    rope_freq_args(a, n_dims, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+    MI355_LAUNCH(k_rope_table, dim3((unsigned)T), dim3(64), 0, (hipStream_t)stream, a, (float2 *)table);
+    return launch_status("k_rope_table");
+}
+
 static int rope_kv_store_impl(void *stream, float *q, const float *k, const float *v, int type_k, void *kcache, int64_t k_a, int64_t k_b, int type_v,
                               void *vcache, int64_t v_a, int64_t v_b, const int32_t *pos, const int32_t *cells, const float *freq_factors, int64_t T,
                               int64_t H, int64_t HK, int64_t D, int n_dims, int mode, int n_ctx_orig, float freq_base, float freq_scale,
@@ -350,13 +386,7 @@ static int rope_kv_store_impl(void *stream, float *q, const float *k, const floa
     a.pos = pos; a.cells = cells; a.ff = freq_factors;
     a.k_nb1 = k_a; a.k_nb2 = k_b; a.v_nb1 = v_a; a.v_nb2 = v_b;
     a.T = (int)T; a.H = (int)H; a.HK = (int)HK; a.D = (int)D; a.n_dims = n_dims; a.mode = mode;
-    a.theta_scale = powf(freq_base, -2.0f / n_dims);
-    a.freq_scale = freq_scale; a.ext_factor = ext_factor; a.attn_factor = attn_factor;
-    const float pi = 3.14159265358979323846f;   // ggml_rope_yarn_corr_dims, ggml/src/ggml.c:3695-3707
-    const float c0 = floorf(n_dims * logf(n_ctx_orig / (beta_fast * 2 * pi)) / (2 * logf(freq_base)));
-    const float c1 = ceilf(n_dims * logf(n_ctx_orig / (beta_slow * 2 * pi)) / (2 * logf(freq_base)));
-    a.corr0 = c0 > 0 ? c0 : 0;
-    a.corr1 = c1 < n_dims - 1 ? c1 : (float)(n_dims - 1);
+    rope_freq_args(a, n_dims, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
     if (qc) MI355_LAUNCH(k_rope_kv_store<true>, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, a);
     else MI355_LAUNCH(k_rope_kv_store<false>, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, a);
     return launch_status("k_rope_kv_store");

@@ -264,20 +264,32 @@ struct wt_mat {
     int64_t N, dst_stride;
     int first_tile;          // index of this matrix's first tile in the launch (unused entries: INT_MAX)
     int shift;               // log2 of the radix between the matrix's two planes: 3 Q4_K, 4 Q5_K, 6 Q6_K
+    int epi;                 // EPI launches: WT_EPI_*
+    int64_t nb1, nb2;        // WT_EPI_*CACHE: dst = base of an f16 cache; byte strides of a cell and of a head inside it
+};
+// EPI launches (Q, K and V of a prompt batch): what becomes of a finished sum.  The rotation is ROPE in its adjacent-pair mode, the
+// pair (2 p, 2 p + 1) of a head being two neighbouring rows of the matrix, i.e. two neighbouring lanes.
+enum { WT_EPI_ROPE = 1, WT_EPI_ROPE_CACHE = 2, WT_EPI_CACHE = 3 };   // rotate -> f32 dst | rotate -> f16 cache | f16 cache
+struct wt_rope {
+    const float2 *cs;        // [B][D / 2] {cos, sin} of the rotation of pair p at token b's position (k_rope_table)
+    const int32_t *cells;    // [B] cache cell of token b
+    int D, n_dims;           // head size; elements of a head that are rotated
 };
 struct wt_launch {
     wt_mat m[3];
     int n_col_tiles;
     int n_tiles, n_tiles_padded;   // n_tiles_padded: rounded up to a multiple of 8
+    wt_rope rope;
 };
 
 // ID: MUL_MAT_ID.  The "matrix" is expert 0's images, the column tiles are those of the sorted slot list (rt), B the rows of the
 // activation image (128 per column tile); a tile's rows go to the dst rows of its slots.
 // TYPE: MI355_Q4_K = the form with the min term, the radix between the planes taken from the matrix (Q4_K, Q5_K, and Q6_K images,
 // whose minima are zeros, in a launch they share with the other two); MI355_Q6_K = launches of Q6_K matrices only: no min term.
-template <int TYPE, bool ID = false>
+template <int TYPE, bool ID = false, bool EPI = false>
 __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__restrict__ a_img, int64_t K, int64_t B, wt_route rt) {
     static_assert(TYPE == MI355_Q4_K || TYPE == MI355_Q6_K, "two forms");
+    static_assert(!(ID && EPI), "one or the other");
     constexpr bool Q4 = TYPE == MI355_Q4_K;   // sub-block mins: the min term and its scale records
     constexpr int NP = 2;                                                      // weight planes
     constexpr int W_AUX = wt_w_aux_bytes(TYPE);
@@ -575,6 +587,62 @@ __global__ void __launch_bounds__(512, 1) k_mmq_w(wt_launch P, const int8_t *__r
         }
     }
 
+    if constexpr (EPI) {
+        // Q, K and V of a prompt batch: the rotation and the cache stores ride in the epilogue.  A lane holds row n of the matrix =
+        // element d of head n / D; its partner in the pair is the neighbouring lane.  Same roundings as k_rope_kv_store.
+        const int kind = P.m[mi].epi;   // uniform over the group
+        const int64_t n = row0 + wrow0 + l32;
+        const int D = P.rope.D, d = (int)(n % D);
+        const int64_t head = n / D;
+        const bool rot = kind != WT_EPI_CACHE && d < P.rope.n_dims;
+        const float2 *cs = P.rope.cs + (d >> 1);
+        uint8_t *cache = (uint8_t *)dst + head * P.m[mi].nb2 + 2 * d;
+        // Every load before the first store: on this hardware a wait for a load also waits for the stores issued before it, so loads
+        // between the stores would put a store's trip to memory into the chain once per token.  The rotations of a 32-token tile
+        // are requested and applied in place, then those of the other tile, then everything is stored; the wave's 64 cache cells
+        // sit one per lane and are read across lanes.
+        const bool row_live = n < N;
+        const int64_t nb1 = P.m[mi].nb1;
+        int cell_of_lane = 0;
+        if (kind != WT_EPI_ROPE) {
+            const int64_t bl = col0 + wcol0 + lane;
+            cell_of_lane = P.rope.cells[bl < B ? bl : B - 1];
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);   // (no load ahead of this point either, where the registers are still in use)
+        if (rot) {
+#pragma unroll
+            for (int tb = 0; tb < 2; tb++) {
+                float2 t[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+                    t[r] = cs[(b < B ? b : B - 1) * (D >> 1)];
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float x = acc[tb][r];
+                    const float xp = __builtin_bit_cast(float, dpp_get<0xB1>(__builtin_bit_cast(int, x)));   // quad_perm [1, 0, 3, 2]: the other element of the pair
+                    acc[tb][r] = (d & 1) ? add_rn(mul_rn(xp, t[r].y), mul_rn(x, t[r].x)) : sub_rn(mul_rn(x, t[r].x), mul_rn(xp, t[r].y));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int tl = tb * 32 + 8 * (r >> 2) + (r & 3);   // the token's place in the wave's 64, for lhi = 0; lhi = 1: 4 further on
+                const int64_t b = col0 + wcol0 + tl + 4 * lhi;
+                if (kind == WT_EPI_ROPE) {
+                    if (row_live && b < B) dst[b * dst_stride + n] = acc[tb][r];
+                } else {
+                    const int c0 = __builtin_amdgcn_readlane(cell_of_lane, tl), c1 = __builtin_amdgcn_readlane(cell_of_lane, tl + 4);
+                    if (row_live && b < B) *(_Float16 *)(cache + (int64_t)(lhi ? c1 : c0) * nb1) = (_Float16)acc[tb][r];
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int tb = 0; tb < 2; tb++) {
         const int64_t n = row0 + wrow0 + l32;
@@ -744,8 +812,13 @@ struct wt_norm {
 };
 static int wt_radix_shift(int type) { return type == MI355_Q4_K ? 3 : type == MI355_Q5_K ? 4 : 6; }
 
+// qkv: the three matrices are Q, K and V of a prompt batch; their rows are rotated and stored as wt_mat::epi says
+struct wt_qkv {
+    wt_rope rope;
+    int64_t k_nb1, k_nb2, v_nb1, v_nb2;
+};
 static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
-                                    size_t ws_bytes, const wt_norm *norm, bool *norm_done);
+                                    size_t ws_bytes, const wt_norm *norm, bool *norm_done, const wt_qkv *qkv = nullptr);
 
 int mi355_mul_mat_q8k_tiled_multi(void *stream, int type, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B,
                                   void *ws, size_t ws_bytes) {
@@ -758,8 +831,25 @@ int mi355_mul_mat_q8k_tiled_mixed(void *stream, int n_mats, const int *types, co
     return mul_mat_q8k_tiled_launch(stream, types, n_mats, mats, act, K, B, nullptr, 0, nullptr, nullptr);
 }
 
+int mi355_mul_mat_q8k_tiled_qkv_rope(void *stream, const int *types, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, const float *rope_table,
+                                     const int32_t *cells, int64_t D, int n_dims, size_t k_nb1, size_t k_nb2, size_t v_nb1, size_t v_nb2) {
+    MI355_REQUIRE(types != nullptr && mats != nullptr && rope_table != nullptr && cells != nullptr, "mul_mat_q8k_tiled_qkv_rope: null operand");
+    MI355_REQUIRE(D > 0 && D % 2 == 0 && n_dims > 0 && n_dims % 2 == 0 && n_dims <= D, "mul_mat_q8k_tiled_qkv_rope: bad head size or n_dims");
+    for (int i = 0; i < 3; i++)
+        MI355_REQUIRE(mats[i].N > 0 && mats[i].N % D == 0 && mats[i].residual == nullptr, "mul_mat_q8k_tiled_qkv_rope: matrix %d: whole heads, no residual", i);
+    MI355_REQUIRE(mats[1].N == mats[2].N && (((uintptr_t)mats[1].dst | (uintptr_t)mats[2].dst | k_nb1 | k_nb2 | v_nb1 | v_nb2) & 1) == 0 &&
+                  ((uintptr_t)rope_table & 7) == 0, "mul_mat_q8k_tiled_qkv_rope: K and V have the same heads; caches and strides are 2-byte aligned");
+    wt_qkv q;
+    q.rope.cs = (const float2 *)rope_table;
+    q.rope.cells = cells;
+    q.rope.D = (int)D;
+    q.rope.n_dims = n_dims;
+    q.k_nb1 = (int64_t)k_nb1; q.k_nb2 = (int64_t)k_nb2; q.v_nb1 = (int64_t)v_nb1; q.v_nb2 = (int64_t)v_nb2;
+    return mul_mat_q8k_tiled_launch(stream, types, 3, mats, act, K, B, nullptr, 0, nullptr, nullptr, &q);
+}
+
 static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, const mi355_tiled_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
-                                    size_t ws_bytes, const wt_norm *norm, bool *norm_done) {
+                                    size_t ws_bytes, const wt_norm *norm, bool *norm_done, const wt_qkv *qkv) {
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_q8k_tiled: 1 to 3 matrices per launch, got %d", n_mats);
     bool all_q6 = true;
     for (int i = 0; i < n_mats; i++) {
@@ -789,6 +879,15 @@ static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, 
         L.m[i].dst_stride = mats[k].dst_stride;
         L.m[i].first_tile = p.first_tile[i];
         L.m[i].shift = wt_radix_shift(types[k]);
+        L.m[i].epi = 0;
+        L.m[i].nb1 = L.m[i].nb2 = 0;
+    }
+    L.rope = wt_rope{nullptr, nullptr, 0, 0};
+    if (qkv) {
+        L.rope = qkv->rope;
+        L.m[0].epi = WT_EPI_ROPE;
+        L.m[1].epi = WT_EPI_ROPE_CACHE; L.m[1].nb1 = qkv->k_nb1; L.m[1].nb2 = qkv->k_nb2;
+        L.m[2].epi = WT_EPI_CACHE;      L.m[2].nb1 = qkv->v_nb1; L.m[2].nb2 = qkv->v_nb2;
     }
     L.n_col_tiles = p.n_col_tiles;
     L.n_tiles = p.n_tiles;
@@ -799,6 +898,11 @@ static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, 
         L.m[0].dst_stride = Ns[0];
     }
     const dim3 grid((unsigned)L.n_tiles_padded, (unsigned)p.slices);
+    if (qkv) {
+        if (all_q6) MI355_LAUNCH((k_mmq_w<MI355_Q6_K, false, true>), grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
+        else MI355_LAUNCH((k_mmq_w<MI355_Q4_K, false, true>), grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
+        return launch_status("k_mmq_w (Q/K/V)");
+    }
     if (all_q6) MI355_LAUNCH(k_mmq_w<MI355_Q6_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
     else MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
     if (p.slices > 1 && norm && Ns[0] <= 4096 && mats[0].dst_stride % 4 == 0 && ((uintptr_t)mats[0].dst & 15) == 0 &&
@@ -877,6 +981,7 @@ int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles,
     const dim3 qgrid((unsigned)((K / QKK + 3) / 4), (unsigned)B_img);
     MI355_LAUNCH(k_quantize_q8k_tiled_routed, qgrid, dim3(256), 0, s, b, img, K, B_img, K, act_row, tiles, n_tiles);
     wt_launch L;
+    L.rope = wt_rope{nullptr, nullptr, 0, 0};
     for (int i = 0; i < 3; i++) {
         L.m[i].w_img = (const int8_t *)expert_tiles;
         L.m[i].dst = dst;
@@ -885,6 +990,8 @@ int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles,
         L.m[i].dst_stride = N;
         L.m[i].first_tile = i == 0 ? 0 : 0x7fffffff;
         L.m[i].shift = wt_radix_shift(type);
+        L.m[i].epi = 0;
+        L.m[i].nb1 = L.m[i].nb2 = 0;
     }
     const int64_t n_row_tiles = (N + WT_BM - 1) / WT_BM;
     MI355_REQUIRE(n_row_tiles * max_tiles + 8 < (1 << 30), "mul_mat_id_q8k_tiled: too many tiles");

@@ -94,6 +94,8 @@ _SIGNATURES = {
     "mi355_mul_mat_q8k_tiled_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_q8k_tiled_mixed": (_int, [_p, _int, _p, _p, _p, _i64, _i64]),
+    "mi355_rope_table": (_int, [_p, _p, _p, _p, _i64, _i64, _int, _int, _f, _f, _f, _f, _f, _f]),
+    "mi355_mul_mat_q8k_tiled_qkv_rope": (_int, [_p, _p, _p, _p, _i64, _i64, _p, _p, _i64, _int, _sz, _sz, _sz, _sz]),
     "mi355_mul_mat_q8k_tiled_norm": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz, _p, _f, _p, _i64, _p]),
     "mi355_mul_mat_q8k_tiled_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_q8k_tiled_multi": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _sz]),

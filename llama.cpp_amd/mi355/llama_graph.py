@@ -123,6 +123,8 @@ class LlamaRunner:
         # that the 2 bytes per weight make the product HBM-bound and the kernel that unpacks the 4.5-bit rows wins
         self.use_tiles = True
         self.tiles = {}
+        self.fuse_qkv_rope = True   # prefill: ROPE and the KV-cache stores in the epilogue of the Q/K/V launch of the wide-tile GEMM
+        self.rope_table = None
         self.fuse_sum_norm = True   # prefill: a cut product's sum launch also normalises and quantizes its rows for the next products
         self.split_ws = None    # partial sums of tile products that are split along K (grown on first use, before any graph capture)
         # decode, T <= 4: SiLU*up + Q8_1 inside the gate/up launch (True: with both matrices of one type a group owns a whole 32-row
@@ -312,6 +314,19 @@ class LlamaRunner:
                 check(lib.mi355_qkv_rope_store(_stream(), tq, _ptr(Wq), tk, _ptr(Wk), tv, _ptr(Wv), _ptr(self.act_a), _ptr(self.q), _ptr(kc), _ptr(vc),
                                                _ptr(self.pos), _ptr(self.pos), None, E, T, H, HK, D, kc.stride(0) * 2, kc.stride(1) * 2,
                                                vc.stride(0) * 2, vc.stride(1) * 2, D, 0, cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
+            elif kq == 2 and self.fuse_qkv_rope:
+                # wide-tile GEMM: the rotations and the cache stores ride in the epilogue of the Q/K/V launch; {cos, sin} per
+                # (token, pair) are the same for every layer and are written once per batch
+                if il == 0:
+                    if self.rope_table is None or self.rope_table.numel() < T * D:
+                        self.rope_table = torch.empty(T * D, dtype=torch.float32, device=self.dev)
+                    check(lib.mi355_rope_table(_stream(), _ptr(self.pos), None, _ptr(self.rope_table), T, D, D, cfg.n_ctx, cfg.rope_theta, 1.0, 0.0, 1.0, 32.0, 1.0))
+                arr = (TiledMat * 3)()
+                for i, ((t, W), dst, N) in enumerate(((L["wq"], self.q, H * D), (L["wk"], kc, HK * D), (L["wv"], vc, HK * D))):
+                    arr[i].tiles, arr[i].dst, arr[i].residual, arr[i].N, arr[i].dst_stride = self._tiles(t, W, N, E).data_ptr(), dst.data_ptr(), None, N, N
+                types = (C.c_int * 3)(L["wq"][0], L["wk"][0], L["wv"][0])
+                check(lib.mi355_mul_mat_q8k_tiled_qkv_rope(_stream(), types, arr, _ptr(self.act_a), E, T, _ptr(self.rope_table), _ptr(self.pos), D, D,
+                                                           kc.stride(0) * 2, kc.stride(1) * 2, vc.stride(0) * 2, vc.stride(1) * 2))
             else:
                 self._mm_act(qkv, self.act_a, E, T, q8k=kq)
                 check(lib.mi355_rope_kv_store(_stream(), _ptr(self.q), _ptr(self.k), _ptr(self.v), _ptr(kc), _ptr(vc), _ptr(self.pos), _ptr(self.pos),

@@ -535,3 +535,45 @@ def test_tile_gemm_from_planes_equals_packed(dev, name, t, N, K, B):
         again = torch.zeros(B, N + 8, device=dev)
         mi355.check(lib.mi355_mul_mat_q8k_ws(None, t, mi355._ptr(W), mi355._ptr(act), mi355._ptr(again), r, N, K, B, N + 8, mi355._ptr(ws), need - 16))
         assert torch.equal(again, want)
+
+
+@pytest.mark.parametrize("types", [(orc.Q4_K, orc.Q4_K, orc.Q6_K), (orc.Q4_K, orc.Q4_K, orc.Q4_K), (orc.Q6_K, orc.Q6_K, orc.Q6_K), (orc.Q5_K, orc.Q4_K, orc.Q6_K)])
+@pytest.mark.parametrize("T,H,HK,D,n_dims", [(512, 32, 8, 128, 128), (300, 8, 2, 64, 32), (77, 4, 4, 128, 64)])
+def test_tiled_qkv_rope_store_equals_product_then_rope_store(dev, types, T, H, HK, D, n_dims):
+    """Q, K and V of a prompt batch with ROPE and the f16 cache stores in the epilogue of the wide-tile GEMM: the rotated q and both
+    caches hold the bits of the same products followed by mi355_rope_kv_store (ragged batch, partial rotation, scattered cells)."""
+    import ctypes as C
+    import torch
+    import mi355
+    lib = mi355.load()
+    K, n_ctx = 2048, 640
+    rng = np.random.default_rng(T + H + D + sum(types))
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    act = mi355.quantize_act_q8k_tiled(_t(dev, x))
+    Ns = (H * D, HK * D, HK * D)
+    tiles = [mi355.kq_unpack_tiles(t, mi355.upload_weights(t, _t(dev, orc.quantize("ref" if orc.ref is not None else "oracle", t,
+                                   (rng.standard_normal((N, K)) * 0.05).astype(np.float32))))) for t, N in zip(types, Ns)]
+    pos = _t(dev, rng.integers(0, 5000, T).astype(np.int32))
+    cells = _t(dev, rng.permutation(n_ctx)[:T].astype(np.int32))
+    rope = (n_dims, 8192, 500000.0, 1.0, 0.0, 1.0, 32.0, 1.0)
+    # the separate launches
+    q0, k0, v0 = mi355.mul_mat_q8k_tiled_multi(list(types), tiles, act, list(Ns), K, T)
+    kc0 = torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+    vc0 = torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+    mi355.check(lib.mi355_rope_kv_store(None, q0.data_ptr(), k0.data_ptr(), v0.data_ptr(), kc0.data_ptr(), vc0.data_ptr(), pos.data_ptr(), cells.data_ptr(), None,
+                                        T, H, HK, D, HK * D * 2, D * 2, HK * D * 2, D * 2, n_dims, 0, *rope[1:]))
+    # one launch
+    table = torch.empty(T * D // 2 * 2, dtype=torch.float32, device=dev)
+    mi355.check(lib.mi355_rope_table(None, pos.data_ptr(), None, table.data_ptr(), T, D, *rope))
+    q1 = torch.zeros(T, H * D, dtype=torch.float32, device=dev)
+    kc1 = torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+    vc1 = torch.zeros(n_ctx, HK, D, dtype=torch.float16, device=dev)
+    arr = (mi355.TiledMat * 3)()
+    for i, (tl, dst, N) in enumerate(zip(tiles, (q1, kc1, vc1), Ns)):
+        arr[i].tiles, arr[i].dst, arr[i].residual, arr[i].N, arr[i].dst_stride = tl.data_ptr(), dst.data_ptr(), None, N, N
+    mi355.check(lib.mi355_mul_mat_q8k_tiled_qkv_rope(None, (C.c_int * 3)(*types), arr, act.data_ptr(), K, T, table.data_ptr(), cells.data_ptr(), D, n_dims,
+                                                     HK * D * 2, D * 2, HK * D * 2, D * 2))
+    torch.cuda.synchronize()
+    assert np.array_equal(q1.cpu().numpy(), q0.cpu().numpy())
+    assert np.array_equal(kc1.cpu().numpy().view(np.uint16), kc0.cpu().numpy().view(np.uint16))
+    assert np.array_equal(vc1.cpu().numpy().view(np.uint16), vc0.cpu().numpy().view(np.uint16))
