@@ -279,6 +279,14 @@ typedef struct mi355_gemv_mat {
     const float *residual;    /* NULL for none */
 } mi355_gemv_mat;
 int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B);
+/* mi355_mul_mat_mid for up to three matrices of the type that share the activation image (Q, K and V; gate and up of
+ * llm_build_kv / llm_build_ffn, src/llama.cpp:1514-1533, :280-320) as one launch: their 32-row tiles fill the compute units together and
+ * the small ones (1024 rows: 32 groups) do not pay a launch and a slice-sum launch of their own.  The slices along K are chosen for the
+ * launch as a whole; ws of mi355_mul_mat_mid_multi_ws_bytes(n_mats, Ns, K, B) bytes (NULL / less: one slice).  Every matrix gets the
+ * integer sums of its own mi355_mul_mat_mid call (f32 summation order follows the number of slices). */
+size_t mi355_mul_mat_mid_multi_ws_bytes(int n_mats, const int64_t *Ns, int64_t K, int64_t B);
+int mi355_mul_mat_mid_multi(void *stream, int type, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
+                            size_t ws_bytes);
 
 /* Integer sub-block dots, for parity checking the kernels' inner products bit-for-bit
  * against ggml_vec_dot_q4_0_q8_0 / q8_0_q8_0 / q4_K_q8_K / q5_K_q8_K / q6_K_q8_K

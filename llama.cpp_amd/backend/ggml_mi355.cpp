@@ -1414,6 +1414,40 @@ void note_window_writes(backend_ctx * ctx, const qkv_window & win, int64_t B) {
 unsigned tiled_multi(backend_ctx * ctx, hipStream_t s, const graph_walk & w, const int * idx, int n) {
     const ggml_tensor * b = w.nodes[idx[0]]->src[1];
     const int64_t K = b->ne[0], B = b->ne[1];
+    // 33 to 128 rows: the Q4_K ones among them as one launch of the weight-streaming kernel on packed rows (mi355_mul_mat_mid_multi)
+    {
+        mi355_gemv_mat mm_mid[3];
+        int64_t Ns[3];
+        unsigned mask = 0;
+        int m = 0;
+        for (int k = 0; k < n && k < 3; k++) {
+            const ggml_tensor * mm = w.nodes[idx[k]];
+            if (!is_q8k_tile_candidate(mm) || mm->src[1]->data != b->data || mm->src[1]->ne[0] != K || mm->src[1]->ne[1] != B || mm->src[1]->nb[1] != b->nb[1] ||
+                mm->type != GGML_TYPE_F32 || mm->nb[0] != sizeof(float) || mm->nb[1] % sizeof(float) != 0 || !takes_mid_kernel(mm))
+                continue;
+            mm_mid[m].type = MI355_Q4_K;
+            mm_mid[m].W = mm->src[0]->data;
+            mm_mid[m].N = mm->src[0]->ne[1];
+            mm_mid[m].dst = (float *) ctx->out_ptr(mm);
+            mm_mid[m].dst_stride = (int64_t) (mm->nb[1] / sizeof(float));
+            mm_mid[m].residual = nullptr;
+            Ns[m] = mm_mid[m].N;
+            m++;
+            mask |= 1u << k;
+        }
+        if (m >= 2) {
+            if (!ctx->cached(b->data, K, B, ACT_Q8KT)) {
+                void * fresh = ctx->act_slot(mi355_act_q8k_tiled_bytes(K, B));
+                MI355_K_OK(mi355_quantize_act_q8k_tiled(s, (const float *) b->data, fresh, K, B, (int64_t) (b->nb[1] / sizeof(float))));
+                ctx->cache = act_cache{b->data, K, B, ACT_Q8KT, true, fresh};
+            }
+            const size_t split_bytes = mi355_mul_mat_mid_multi_ws_bytes(m, Ns, K, B);
+            void * split_ws = split_bytes ? ctx->workspace(split_bytes) : nullptr;
+            MI355_K_OK(mi355_mul_mat_mid_multi(s, MI355_Q4_K, m, mm_mid, ctx->cache.ptr, K, B, split_ws, split_bytes));
+            for (int k = 0; k < m; k++) ctx->note_write(mm_mid[k].dst, (size_t) mm_mid[k].N * (size_t) B * sizeof(float));
+            return mask;
+        }
+    }
     const void * tl[3] = {nullptr, nullptr, nullptr};
     int n_with = 0;
     for (int k = 0; k < n && k < 3; k++) {

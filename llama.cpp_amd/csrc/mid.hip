@@ -50,10 +50,27 @@ template <int NB> struct mid_act {
 // instructions); the group's four waves are NBW such sets of tiles x 4 / NBW parts of the slice's K range: wave = part * NBW + set.
 // Waves of one part copy the same weights, each to its own LDS (no barrier; the second copy comes from cache).
 // act: tile images of B rows (mi355_quantize_act_q8k_tiled).
+// Up to three matrices that read the same activation go out in one launch, their 32-row tiles numbered one matrix after the other
+// (Q, K and V; gate and up: the small ones alone are a handful of groups each, and every launch costs its start-up).
+struct mid_mat {
+    const uint8_t *W;
+    float *dst;
+    const float *residual;   // may be null; same shape and stride as dst; may be dst itself
+    int64_t N, dst_stride;
+    int first_tile;          // index of the matrix's first 32-row tile in the launch (unused entries: INT_MAX)
+};
+struct mid_launch {
+    mid_mat m[3];
+};
 template <int NB, int NBW>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
-k_mm_mid_q4k(const uint8_t *__restrict__ W, const uint8_t *__restrict__ act, float *__restrict__ dst, const float *__restrict__ residual, int64_t N, int K,
-             int B, int64_t dst_stride, int steps_per_slice, int steps_per_wave) {
+k_mm_mid_q4k(mid_launch P, const uint8_t *__restrict__ act, int K, int B, int steps_per_slice, int steps_per_wave) {
+    const int mi = ((int)blockIdx.x >= P.m[1].first_tile ? 1 : 0) + ((int)blockIdx.x >= P.m[2].first_tile ? 1 : 0);   // uniform
+    const uint8_t *__restrict__ W = P.m[mi].W;
+    float *__restrict__ dst = P.m[mi].dst;
+    const float *__restrict__ residual = P.m[mi].residual;
+    const int64_t N = P.m[mi].N, dst_stride = P.m[mi].dst_stride;
+    const int tile_x = (int)blockIdx.x - P.m[mi].first_tile;
     constexpr int KS = 4 / NBW;
     constexpr int WAVE_BYTES = MID_STAGES * MID_STAGE;
     constexpr int RED_BYTES = 4 * NB * 16 * 64 * 4;
@@ -65,7 +82,7 @@ k_mm_mid_q4k(const uint8_t *__restrict__ W, const uint8_t *__restrict__ act, flo
     uint8_t *ring = s_mem + wave * WAVE_BYTES;
     const unsigned ring_lds = (unsigned)(uintptr_t)(void __attribute__((address_space(3))) *)ring;
 
-    const int64_t row0 = (int64_t)blockIdx.x * 32;
+    const int64_t row0 = (int64_t)tile_x * 32;
     const int nsteps = K >> 8;
     const int slice_lo = blockIdx.y * steps_per_slice;
     const int slice_hi = slice_lo + steps_per_slice < nsteps ? slice_lo + steps_per_slice : nsteps;
@@ -279,23 +296,32 @@ k_mm_mid_q4k(const uint8_t *__restrict__ W, const uint8_t *__restrict__ act, flo
     }
 }
 
-// sum of the K slices: dst[c][n] = sum_s part[s][c][n] (+ residual), slices in ascending order
-__global__ void __launch_bounds__(256) k_mid_slices(const float *__restrict__ part, float *__restrict__ dst, const float *__restrict__ residual, int64_t N,
-                                                    int B, int64_t dst_stride, int slices) {
+// sum of the K slices: dst[c][n] = sum_s part[s][c][n] (+ residual), slices in ascending order; blockIdx.z = matrix of the launch,
+// whose partial sums lie behind those of the matrices before it
+struct mid_sum {
+    const float *part[3];
+    float *dst[3];
+    const float *residual[3];
+    int64_t N[3], dst_stride[3];
+};
+__global__ void __launch_bounds__(256) k_mid_slices(mid_sum S, int B, int slices) {
+    const int mi = blockIdx.z;
+    const int64_t N = S.N[mi];
     const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int c = blockIdx.y;
     if (n >= N) return;
+    const float *__restrict__ part = S.part[mi];
     float sum = part[(int64_t)c * N + n];
     for (int s = 1; s < slices; s++) sum += part[((int64_t)s * B + c) * N + n];
-    const int64_t o = c * dst_stride + n;
-    dst[o] = residual ? sum + residual[o] : sum;
+    const int64_t o = c * S.dst_stride[mi] + n;
+    S.dst[mi][o] = S.residual[mi] ? sum + S.residual[mi][o] : sum;
 }
 
 // sets of activation tiles across the waves of a group (a wave takes 1 tile up to 32 rows, 2 beyond)
 int mid_sets(int64_t B) { return B <= 64 ? 1 : 2; }
 
 // slices of K: enough groups to cover the chip about twice, as long as a wave keeps two super-blocks
-int mid_slices(int64_t N, int64_t K, int64_t B) {
+int mid_slices(int64_t N, int64_t K, int64_t B) {   // N: rows of all matrices of the launch (each a multiple of 32, or one matrix)
     const int64_t groups = (N + 31) / 32, nsteps = K >> 8;
     const int ks = 4 / mid_sets(B);
     int s = 1;
@@ -320,32 +346,90 @@ size_t mi355_mul_mat_mid_ws_bytes(int64_t N, int64_t K, int64_t B) {
     return s > 1 ? (size_t)s * B * N * sizeof(float) : 0;
 }
 
-int mi355_mul_mat_mid(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
-                      int64_t dst_stride, void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(mi355_mul_mat_mid_supported(type, W, K, B), "mul_mat_mid: type %d, K=%lld, B=%lld or the weight alignment is not supported", type,
-                  (long long)K, (long long)B);
-    MI355_REQUIRE(N > 0 && dst_stride >= N && N < (int64_t(1) << 31), "mul_mat_mid: bad shape N=%lld dst_stride=%lld", (long long)N, (long long)dst_stride);
-    MI355_REQUIRE(N * (K / 256 * Q4_K_BYTES) < (int64_t(1) << 32), "mul_mat_mid: matrix of 4 GiB or more");
+int mi355_mul_mat_mid_multi(void *stream, int type, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B, void *ws, size_t ws_bytes) {
+    MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_mid: 1 to 3 matrices per launch, got %d", n_mats);
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_mid: activation image is not 16-byte aligned");
     MI355_REQUIRE(mi355_act_q8k_tiled_bytes(K, B) < ((size_t)1 << 32), "mul_mat_mid: activation image of 4 GiB or more");
-    int slices = mid_slices(N, K, B);
-    if (slices > 1 && (ws == nullptr || ws_bytes < (size_t)slices * B * N * sizeof(float))) slices = 1;   // no room for partial sums: one slice
+    int64_t n_sum = 0, tiles = 0;
+    mid_launch L;
+    for (int i = 0; i < 3; i++) {
+        const mi355_gemv_mat &m = mats[i < n_mats ? i : 0];
+        if (i < n_mats) {
+            MI355_REQUIRE(m.type == type && mi355_mul_mat_mid_supported(type, m.W, K, B), "mul_mat_mid: type %d, K=%lld, B=%lld or the weight alignment is not supported",
+                          m.type, (long long)K, (long long)B);
+            MI355_REQUIRE(m.N > 0 && m.dst_stride >= m.N && m.N < (int64_t(1) << 31), "mul_mat_mid: bad shape N=%lld dst_stride=%lld", (long long)m.N, (long long)m.dst_stride);
+            MI355_REQUIRE(m.N * (K / 256 * Q4_K_BYTES) < (int64_t(1) << 32), "mul_mat_mid: matrix of 4 GiB or more");
+        }
+        L.m[i].W = (const uint8_t *)m.W;
+        L.m[i].dst = m.dst;
+        L.m[i].residual = m.residual;
+        L.m[i].N = m.N;
+        L.m[i].dst_stride = m.dst_stride;
+        L.m[i].first_tile = i < n_mats ? (int)tiles : 0x7fffffff;
+        if (i < n_mats) {
+            tiles += (m.N + 31) / 32;
+            n_sum += m.N;
+        }
+    }
+    MI355_REQUIRE(tiles < (1 << 30), "mul_mat_mid: too many tiles");
+    int slices = mid_slices(tiles * 32, K, B);
+    if (slices > 1 && (ws == nullptr || ws_bytes < (size_t)slices * B * n_sum * sizeof(float))) slices = 1;   // no room for partial sums: one slice
     hipStream_t s = (hipStream_t)stream;
     const int nsteps = (int)(K >> 8);
     const int steps_per_slice = (nsteps + slices - 1) / slices;
     const int nbw = mid_sets(B);
     const int steps_per_wave = (steps_per_slice + 4 / nbw - 1) / (4 / nbw);
-    const dim3 grid((unsigned)((N + 31) / 32), (unsigned)slices);
-    float *out = slices == 1 ? dst : (float *)ws;
-    const float *res = slices == 1 ? residual : nullptr;
-    const int64_t stride = slices == 1 ? dst_stride : N;
-#define MI355_MID_ARGS grid, dim3(256), 0, s, (const uint8_t *)W, (const uint8_t *)act, out, res, N, (int)K, (int)B, stride, steps_per_slice, steps_per_wave
+    const dim3 grid((unsigned)tiles, (unsigned)slices);
+    mid_sum S;
+    int64_t n_max = 0;
+    if (slices > 1) {   // partial sums: per matrix [slice][B][N], one matrix after the other
+        float *part = (float *)ws;
+        for (int i = 0; i < 3; i++) {
+            const int k = i < n_mats ? i : 0;
+            S.part[i] = part;
+            S.dst[i] = mats[k].dst;
+            S.residual[i] = mats[k].residual;
+            S.N[i] = mats[k].N;
+            S.dst_stride[i] = mats[k].dst_stride;
+            if (i < n_mats) {
+                L.m[i].dst = part;
+                L.m[i].residual = nullptr;
+                L.m[i].dst_stride = mats[i].N;
+                part += (int64_t)slices * B * mats[i].N;
+                n_max = mats[i].N > n_max ? mats[i].N : n_max;
+            }
+        }
+    }
+#define MI355_MID_ARGS grid, dim3(256), 0, s, L, (const uint8_t *)act, (int)K, (int)B, steps_per_slice, steps_per_wave
     if (B <= 32) MI355_LAUNCH((k_mm_mid_q4k<1, 1>), MI355_MID_ARGS);
     else if (B <= 64) MI355_LAUNCH((k_mm_mid_q4k<2, 1>), MI355_MID_ARGS);
     else MI355_LAUNCH((k_mm_mid_q4k<2, 2>), MI355_MID_ARGS);
 #undef MI355_MID_ARGS
-    if (slices > 1) MI355_LAUNCH(k_mid_slices, dim3((unsigned)((N + 255) / 256), (unsigned)B), dim3(256), 0, s, (const float *)ws, dst, residual, N, (int)B, dst_stride, slices);
+    if (slices > 1) MI355_LAUNCH(k_mid_slices, dim3((unsigned)((n_max + 255) / 256), (unsigned)B, (unsigned)n_mats), dim3(256), 0, s, S, (int)B, slices);
     return launch_status("k_mm_mid");
+}
+
+size_t mi355_mul_mat_mid_multi_ws_bytes(int n_mats, const int64_t *Ns, int64_t K, int64_t B) {
+    if (n_mats < 1 || n_mats > 3 || Ns == nullptr) return 0;
+    int64_t n_sum = 0, tiles = 0;
+    for (int i = 0; i < n_mats; i++) {
+        n_sum += Ns[i];
+        tiles += (Ns[i] + 31) / 32;
+    }
+    const int s = mid_slices(tiles * 32, K, B);
+    return s > 1 ? (size_t)s * B * n_sum * sizeof(float) : 0;
+}
+
+int mi355_mul_mat_mid(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
+                      int64_t dst_stride, void *ws, size_t ws_bytes) {
+    mi355_gemv_mat m;
+    m.type = type;
+    m.W = W;
+    m.N = N;
+    m.dst = dst;
+    m.dst_stride = dst_stride;
+    m.residual = residual;
+    return mi355_mul_mat_mid_multi(stream, type, 1, &m, act, K, B, ws, ws_bytes);
 }
 
 }  // extern "C"

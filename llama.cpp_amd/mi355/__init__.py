@@ -75,6 +75,8 @@ _SIGNATURES = {
     "mi355_mul_mat_mid_supported": (_int, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_mid_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_mid": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_mid_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
+    "mi355_mul_mat_mid_multi": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _sz]),
     "mi355_act_q8k_bytes": (_sz, [_i64, _i64]),
     "mi355_quantize_act_q8k": (_int, [_p, _p, _p, _i64, _i64, _i64]),
     "mi355_mul_mat_q8k": (_int, [_p, _int, _p, _p, _p, _i64, _i64, _i64, _i64]),
@@ -398,6 +400,24 @@ def mul_mat_mid(t, W, x, residual=None, split=True):
     check(load().mi355_mul_mat_mid(_stream(), t, _ptr(W), _ptr(act), _ptr(dst), _ptr(residual) if residual is not None else None,
                                    N, K, B, N, _ptr(ws) if nws else None, nws))
     return dst
+
+
+def mul_mat_mid_multi(t, Ws, x, residuals=None, split=True):
+    """mul_mat_mid for up to three matrices on one activation in one launch -> list of f32 [B, N_i]"""
+    import torch
+    B, K = x.shape
+    n = len(Ws)
+    act = quantize_act_q8k_tiled(x)
+    Ns = [W.shape[0] for W in Ws]
+    dsts = [torch.empty((B, N), dtype=torch.float32, device=x.device) for N in Ns]
+    arr = (GemvMat * n)()
+    for i in range(n):
+        arr[i].type, arr[i].W, arr[i].N, arr[i].dst, arr[i].dst_stride = t, Ws[i].data_ptr(), Ns[i], dsts[i].data_ptr(), Ns[i]
+        arr[i].residual = residuals[i].data_ptr() if residuals is not None and residuals[i] is not None else None
+    nws = load().mi355_mul_mat_mid_multi_ws_bytes(n, (C.c_int64 * n)(*Ns), K, B) if split else 0
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=x.device)
+    check(load().mi355_mul_mat_mid_multi(_stream(), t, n, arr, _ptr(act), K, B, _ptr(ws) if nws else None, nws))
+    return dsts
 
 
 def block_dots(t, W, x_row):

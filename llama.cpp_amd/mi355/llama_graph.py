@@ -262,6 +262,17 @@ class LlamaRunner:
                 types = (C.c_int * len(mats))(*[t for (t, _), _ in mats])
                 check(self.lib.mi355_mul_mat_q8k_tiled_mixed(_stream(), len(mats), types, arr, _ptr(act), K, T))
                 mats = []
+            if q8k == 3 and 1 < len(mats) <= 3:   # 33..128 rows on Q4_K: the matrices that share the activation in one launch
+                arr = (GemvMat * len(mats))()
+                for i, ((t, W), out) in enumerate(mats):
+                    arr[i].type, arr[i].W, arr[i].N, arr[i].dst, arr[i].dst_stride = t, W.data_ptr(), out.shape[1], out.data_ptr(), out.stride(0)
+                    arr[i].residual = residual.data_ptr() if residual is not None else None
+                ns = (C.c_int64 * len(mats))(*[out.shape[1] for _, out in mats])
+                need = int(self.lib.mi355_mul_mat_mid_multi_ws_bytes(len(mats), ns, K, T))
+                if self.split_ws is None or self.split_ws.numel() < need:
+                    self.split_ws = torch.empty(need + 256, dtype=torch.uint8, device=self.dev)
+                check(self.lib.mi355_mul_mat_mid_multi(_stream(), Q4_K, len(mats), arr, _ptr(act), K, T, _ptr(self.split_ws) if need else None, need))
+                mats = []
             for (t, W), out in mats:
                 if q8k == 3:
                     N = out.shape[1]

@@ -216,6 +216,32 @@ def test_mid_matches_oracle(dev, N, K, B, split):
         assert np.array_equal(mi355.mul_mat(t, Wd, _to_dev(dev, x), split=split).cpu().numpy(), got)
 
 
+@pytest.mark.parametrize("Ns,K,B", [((4096, 1024, 1024), 4096, 128), ((14336, 14336), 4096, 64), ((100, 257, 64), 2048, 100), ((2048, 512), 1024, 40)])
+@pytest.mark.parametrize("split", [False, True])
+def test_mid_multi_equals_single_launches(dev, Ns, K, B, split):
+    """up to three Q4_K matrices on one activation in one launch of the 33..128-row kernel: without slices every matrix has the bits of
+    its own launch; with slices (chosen for the launch as a whole) the same integer sums in another f32 order; residuals per matrix"""
+    import mi355
+    t = orc.Q4_K
+    rng = np.random.default_rng(sum(Ns) + K + B)
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    Wq = [_weights(rng, t, N, K, "ref") for N in Ns]
+    Wd = [mi355.upload_weights(t, _to_dev(dev, W)) for W in Wq]
+    res = [_to_dev(dev, rng.standard_normal((B, N)).astype(np.float32)) if i != 1 else None for i, N in enumerate(Ns)]
+    xd = _to_dev(dev, x)
+    alone = [mi355.mul_mat_mid(t, W, xd, split=False).cpu().numpy() for W in Wd]
+    multi = [o.cpu().numpy() for o in mi355.mul_mat_mid_multi(t, Wd, xd, split=split)]
+    with_res = [o.cpu().numpy() for o in mi355.mul_mat_mid_multi(t, Wd, xd, residuals=res, split=split)]
+    for i, N in enumerate(Ns):
+        if not split:
+            assert np.array_equal(multi[i], alone[i])
+        assert orc.nmse(multi[i], alone[i]) < 1e-12
+        assert np.array_equal(with_res[i], multi[i] + res[i].cpu().numpy() if res[i] is not None else multi[i])
+        Nt = min(N, 40)
+        assert orc.nmse(multi[i][:, :Nt], orc.mul_mat("cpu", t, Wq[i][:Nt], x)) < 1e-9
+        assert orc.nmse(multi[i][B - 5:, N - 7:], orc.mul_mat("cpu", t, Wq[i][N - 7:], x[B - 5:])) < 1e-9
+
+
 @pytest.mark.parametrize("name,t", TYPES)
 @pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
 def test_mmq_llama8b_ffn_shapes(dev, name, t, N, K):
