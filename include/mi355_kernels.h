@@ -284,6 +284,11 @@ int mi355_mul_mat_vec_q_multi(void *stream, int n_mats, const mi355_gemv_mat *ma
  * the small ones (1024 rows: 32 groups) do not pay a launch and a slice-sum launch of their own.  The slices along K are chosen for the
  * launch as a whole; ws of mi355_mul_mat_mid_multi_ws_bytes(n_mats, Ns, K, B) bytes (NULL / less: one slice).  Every matrix gets the
  * integer sums of its own mi355_mul_mat_mid call (f32 summation order follows the number of slices). */
+/* mi355_mul_mat_mid followed by the RMS norm of its rows, as mi355_mul_mat_q8k_tiled_norm does for the wide-tile GEMM (same operands,
+ * same bits as the product followed by mi355_rms_norm_mul_quant_q8k_tiled; the launch that adds a cut product's slices carries the
+ * norm).  ws: mi355_mul_mat_mid_ws_bytes(N, K, B). */
+int mi355_mul_mat_mid_norm(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
+                           int64_t dst_stride, void *ws, size_t ws_bytes, const float *norm_w, float eps, float *y, int64_t y_stride, void *act_out);
 size_t mi355_mul_mat_mid_multi_ws_bytes(int n_mats, const int64_t *Ns, int64_t K, int64_t B);
 int mi355_mul_mat_mid_multi(void *stream, int type, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B, void *ws,
                             size_t ws_bytes);

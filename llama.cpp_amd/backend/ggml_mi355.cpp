@@ -2254,7 +2254,7 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                 // ... -> RMS_NORM -> MUL(norm weight) whose readers are tile products again (wo -> the FFN norm, ffn_down -> the next
                 // layer's attention norm): a product that is cut along K adds its slices row by row, and the group that has formed a
                 // row normalises and quantizes it on the spot (same bits as the norm launch it replaces)
-                if (tl && split_ws) {
+                if ((tl || mid) && split_ws) {
                     const int jn = w.next(j);
                     const int jm = jn < w.n ? w.next(jn) : w.n;
                     const ggml_tensor * nrm = jn < w.n ? w.nodes[jn] : nullptr;
@@ -2270,9 +2270,14 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                             float eps;
                             memcpy(&eps, nrm->op_params, sizeof(float));
                             void * act_out = ctx->act_slot(mi355_act_q8k_tiled_bytes(N, B), true);   // the product still reads the other slot
-                            MI355_K_OK(mi355_mul_mat_q8k_tiled_norm(s, wtype, tl, ctx->cache.ptr, (float *) add->data, (const float *) res->data, N, K, B,
-                                                                    (int64_t) (add->nb[1] / sizeof(float)), split_ws, split_bytes, (const float *) wt->data, eps,
-                                                                    (float *) mul->data, N, act_out));
+                            if (mid)
+                                MI355_K_OK(mi355_mul_mat_mid_norm(s, wtype, node->src[0]->data, ctx->cache.ptr, (float *) add->data, (const float *) res->data, N, K, B,
+                                                                  (int64_t) (add->nb[1] / sizeof(float)), split_ws, split_bytes, (const float *) wt->data, eps,
+                                                                  (float *) mul->data, N, act_out));
+                            else
+                                MI355_K_OK(mi355_mul_mat_q8k_tiled_norm(s, wtype, tl, ctx->cache.ptr, (float *) add->data, (const float *) res->data, N, K, B,
+                                                                        (int64_t) (add->nb[1] / sizeof(float)), split_ws, split_bytes, (const float *) wt->data, eps,
+                                                                        (float *) mul->data, N, act_out));
                             ctx->note_write(add->data, ggml_nbytes(add));
                             ctx->note_write(mul->data, ggml_nbytes(mul));
                             ctx->cache = act_cache{mul->data, N, B, ACT_Q8KT, true, act_out};

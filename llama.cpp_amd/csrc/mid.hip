@@ -346,7 +346,42 @@ size_t mi355_mul_mat_mid_ws_bytes(int64_t N, int64_t K, int64_t B) {
     return s > 1 ? (size_t)s * B * N * sizeof(float) : 0;
 }
 
+// norm: the single matrix's rows are normalised next; taken when the product is cut along K, whose sum launch then carries the norm
+struct mid_norm {
+    const float *w;
+    float eps;
+    float *y;
+    int64_t y_stride;
+    void *act_out;
+};
+static int mul_mat_mid_launch(void *stream, int type, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B, void *ws, size_t ws_bytes,
+                              const mid_norm *norm, bool *norm_done);
+
 int mi355_mul_mat_mid_multi(void *stream, int type, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B, void *ws, size_t ws_bytes) {
+    return mul_mat_mid_launch(stream, type, n_mats, mats, act, K, B, ws, ws_bytes, nullptr, nullptr);
+}
+
+int mi355_mul_mat_mid_norm(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
+                           int64_t dst_stride, void *ws, size_t ws_bytes, const float *norm_w, float eps, float *y, int64_t y_stride, void *act_out) {
+    MI355_REQUIRE(N > 0 && N % QKK == 0, "mul_mat_mid_norm: N=%lld must be a multiple of 256", (long long)N);
+    MI355_REQUIRE(norm_w != nullptr && act_out != nullptr && ((uintptr_t)norm_w & 15) == 0 && ((uintptr_t)act_out & 15) == 0 && ((uintptr_t)y & 15) == 0 &&
+                  y_stride % 4 == 0, "mul_mat_mid_norm: the norm's operands must be 16-byte aligned");
+    mi355_gemv_mat m;
+    m.type = type;
+    m.W = W;
+    m.N = N;
+    m.dst = dst;
+    m.dst_stride = dst_stride;
+    m.residual = residual;
+    const mid_norm nm = {norm_w, eps, y, y_stride, act_out};
+    bool done = false;
+    const int rc = mul_mat_mid_launch(stream, type, 1, &m, act, K, B, ws, ws_bytes, &nm, &done);
+    if (rc != MI355_OK || done) return rc;
+    return mi355_rms_norm_mul_quant_q8k_tiled(stream, dst, dst_stride, norm_w, y, y_stride, act_out, N, B, eps);   // an uncut product: the norm is its own launch
+}
+
+static int mul_mat_mid_launch(void *stream, int type, int n_mats, const mi355_gemv_mat *mats, const void *act, int64_t K, int64_t B, void *ws, size_t ws_bytes,
+                              const mid_norm *norm, bool *norm_done) {
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_mid: 1 to 3 matrices per launch, got %d", n_mats);
     MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_mid: activation image is not 16-byte aligned");
     MI355_REQUIRE(mi355_act_q8k_tiled_bytes(K, B) < ((size_t)1 << 32), "mul_mat_mid: activation image of 4 GiB or more");
@@ -405,7 +440,14 @@ int mi355_mul_mat_mid_multi(void *stream, int type, int n_mats, const mi355_gemv
     else if (B <= 64) MI355_LAUNCH((k_mm_mid_q4k<2, 1>), MI355_MID_ARGS);
     else MI355_LAUNCH((k_mm_mid_q4k<2, 2>), MI355_MID_ARGS);
 #undef MI355_MID_ARGS
-    if (slices > 1) MI355_LAUNCH(k_mid_slices, dim3((unsigned)((n_max + 255) / 256), (unsigned)B, (unsigned)n_mats), dim3(256), 0, s, S, (int)B, slices);
+    if (slices > 1 && norm && n_mats == 1 && mats[0].N <= 4096 && mats[0].N % 4 == 0 && mats[0].dst_stride % 4 == 0 && ((uintptr_t)mats[0].dst & 15) == 0 &&
+        (mats[0].residual == nullptr || ((uintptr_t)mats[0].residual & 15) == 0) && ((uintptr_t)ws & 15) == 0) {
+        launch_split_sum_norm(s, (const float *)ws, mats[0].dst, mats[0].residual, mats[0].N, B, mats[0].dst_stride, slices, norm->w, norm->eps, norm->y,
+                              norm->y_stride, norm->act_out);
+        *norm_done = true;
+    } else if (slices > 1) {
+        MI355_LAUNCH(k_mid_slices, dim3((unsigned)((n_max + 255) / 256), (unsigned)B, (unsigned)n_mats), dim3(256), 0, s, S, (int)B, slices);
+    }
     return launch_status("k_mm_mid");
 }
 

@@ -728,6 +728,12 @@ __global__ void __launch_bounds__(256) k_wt_split_sum_norm(const float *__restri
     rms_norm_quant_row<NV, 2, false>(nullptr, w, y ? y + b * y_stride : nullptr, act_out, b, N, B, eps, sh, nullptr, v);
 }
 
+void launch_split_sum_norm(hipStream_t s, const float *part, float *dst, const float *residual, int64_t N, int64_t B, int64_t dst_stride, int n_slices,
+                           const float *w, float eps, float *y, int64_t y_stride, void *act_out) {
+    MI355_LAUNCH((k_wt_split_sum_norm<4>), dim3((unsigned)B), dim3(256), 0, s, part, dst, residual, N, B, dst_stride, n_slices, w, eps, y, y_stride,
+                 (uint8_t *)act_out);
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -907,8 +913,8 @@ static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, 
     else MI355_LAUNCH(k_mmq_w<MI355_Q4_K>, grid, dim3(512), 0, s, L, (const int8_t *)act, K, B, wt_route{});
     if (p.slices > 1 && norm && Ns[0] <= 4096 && mats[0].dst_stride % 4 == 0 && ((uintptr_t)mats[0].dst & 15) == 0 &&
         (mats[0].residual == nullptr || ((uintptr_t)mats[0].residual & 15) == 0)) {
-        MI355_LAUNCH((k_wt_split_sum_norm<4>), dim3((unsigned)B), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B, mats[0].dst_stride,
-                     p.slices, norm->w, norm->eps, norm->y, norm->y_stride, (uint8_t *)norm->act_out);
+        launch_split_sum_norm(s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B, mats[0].dst_stride, p.slices, norm->w, norm->eps, norm->y,
+                              norm->y_stride, norm->act_out);
         *norm_done = true;
     } else if (p.slices > 1) {
         MI355_LAUNCH(k_wt_split_sum, dim3((unsigned)((Ns[0] * B / 4 + 255) / 256)), dim3(256), 0, s, (const float *)ws, mats[0].dst, mats[0].residual, Ns[0], B,

@@ -65,6 +65,12 @@ __device__ __forceinline__ void q8k_quantize_wave_tiled(const f32x4 &v, int lane
     }
 }
 
+// Sum of a product's K slices (partial sums [slice][B][N]) + residual -> dst rows, each row then RMS-normalised, multiplied by w and
+// written as y (optional) and as its part of the tile image act_out: one launch, the bits of the slice sum followed by the norm
+// launch (mmq_w.hip).  N <= 4096, a multiple of 256; 16-byte aligned operands.
+void launch_split_sum_norm(hipStream_t s, const float *part, float *dst, const float *residual, int64_t N, int64_t B, int64_t dst_stride, int n_slices,
+                           const float *w, float eps, float *y, int64_t y_stride, void *act_out);
+
 // MUL_MAT_ID: the (token, expert slot) pairs sorted by expert (k_route_slots, mmq_k.hip).  Column c of the sorted list reads
 // activation row act_row[c] and writes dst row dst_row[c]; tiles[4 i] = {expert, first column, end column of the expert, 0} for
 // column tiles of at most bn columns; *n_tiles tiles are in use.  At most 256 experts.

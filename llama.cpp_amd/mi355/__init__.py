@@ -75,6 +75,7 @@ _SIGNATURES = {
     "mi355_mul_mat_mid_supported": (_int, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_mid_ws_bytes": (_sz, [_i64, _i64, _i64]),
     "mi355_mul_mat_mid": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz]),
+    "mi355_mul_mat_mid_norm": (_int, [_p, _int, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz, _p, _f, _p, _i64, _p]),
     "mi355_mul_mat_mid_multi_ws_bytes": (_sz, [_int, _p, _i64, _i64]),
     "mi355_mul_mat_mid_multi": (_int, [_p, _int, _int, _p, _p, _i64, _i64, _p, _sz]),
     "mi355_act_q8k_bytes": (_sz, [_i64, _i64]),

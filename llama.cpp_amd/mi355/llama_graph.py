@@ -246,7 +246,7 @@ class LlamaRunner:
         """mats: list of ((type, W), out); all consume the quantized activation `act` (T rows of K).
         norm: (norm weight, activation buffer) - the single product's rows are normalised next and their tile image goes to the
         buffer (wide-tile GEMM only: the launch that adds a cut product's slices carries the norm)"""
-        assert norm is None or (q8k == 2 and len(mats) == 1 and T > 8)
+        assert norm is None or (q8k in (2, 3) and len(mats) == 1 and T > 8)
         if T <= 8:
             arr = (GemvMat * len(mats))()
             for i, ((t, W), out) in enumerate(mats):
@@ -279,8 +279,13 @@ class LlamaRunner:
                     need = int(self.lib.mi355_mul_mat_mid_ws_bytes(N, K, T))
                     if self.split_ws is None or self.split_ws.numel() < need:
                         self.split_ws = torch.empty(need + 256, dtype=torch.uint8, device=self.dev)
-                    check(self.lib.mi355_mul_mat_mid(_stream(), t, _ptr(W), _ptr(act), _ptr(out), _ptr(residual) if residual is not None else None, N, K, T,
-                                                     out.stride(0), _ptr(self.split_ws) if need else None, need))
+                    if norm is not None:
+                        check(self.lib.mi355_mul_mat_mid_norm(_stream(), t, _ptr(W), _ptr(act), _ptr(out), _ptr(residual) if residual is not None else None, N, K, T,
+                                                              out.stride(0), _ptr(self.split_ws) if need else None, need, _ptr(norm[0]), self.cfg.rms_eps, None, 0,
+                                                              _ptr(norm[1])))
+                    else:
+                        check(self.lib.mi355_mul_mat_mid(_stream(), t, _ptr(W), _ptr(act), _ptr(out), _ptr(residual) if residual is not None else None, N, K, T,
+                                                         out.stride(0), _ptr(self.split_ws) if need else None, need))
                     continue
                 if q8k:     # the residual add is the tile kernel's epilogue; products with few tiles are split along K through split_ws
                     N = out.shape[1]
@@ -353,7 +358,7 @@ class LlamaRunner:
             gu = [(L["gate"], self.gate[:T]), (L["up"], self.up[:T])]
             kq_gu = self._fmt(gu, E, T)
             # wide-tile products on both sides of a norm: the product's sum launch also normalises and quantizes the rows it forms
-            fuse = self.fuse_sum_norm and kq == 2 and kq_gu == 2 and E % 256 == 0
+            fuse = self.fuse_sum_norm and kq in (2, 3) and kq_gu in (2, 3) and E % 256 == 0
             self._mm_act(wo, self.act_a, H * D, T, residual=x, q8k=kq, norm=(L["ffn_norm"], self.act_a) if fuse else None)
             if not fuse:
                 self._norm_quant(x, L["ffn_norm"], self.act_a, T, kq_gu)
@@ -363,7 +368,7 @@ class LlamaRunner:
             fn = (lib.mi355_swiglu_quant, lib.mi355_swiglu_quant_q8k, lib.mi355_swiglu_quant_q8k_tiled, lib.mi355_swiglu_quant_q8k_tiled)[kq]
             check(fn(_stream(), _ptr(self.gate), _ptr(self.up), F, None, 0, _ptr(self.act_b), F, T))
             nxt = w.layers[il + 1] if il + 1 < len(w.layers) else None
-            normed = self.fuse_sum_norm and nxt is not None and kq == 2 and E % 256 == 0 and self._fmt([(nxt["wq"], self.q[:T]), (nxt["wk"], self.k[:T]), (nxt["wv"], self.v[:T])], E, T) == 2
+            normed = self.fuse_sum_norm and nxt is not None and kq in (2, 3) and E % 256 == 0 and self._fmt([(nxt["wq"], self.q[:T]), (nxt["wk"], self.k[:T]), (nxt["wv"], self.v[:T])], E, T) in (2, 3)
             self._mm_act(down, self.act_b, F, T, residual=x, q8k=kq, norm=(nxt["attn_norm"], self.act_a) if normed else None)
         To = 1 if last_only else T
         xo = self.x[T - 1:T] if last_only else x

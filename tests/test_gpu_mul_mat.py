@@ -216,6 +216,37 @@ def test_mid_matches_oracle(dev, N, K, B, split):
         assert np.array_equal(mi355.mul_mat(t, Wd, _to_dev(dev, x), split=split).cpu().numpy(), got)
 
 
+@pytest.mark.parametrize("N,K,B,split", [(4096, 4096, 128, True), (4096, 14336, 64, True), (2048, 1024, 100, True), (4096, 4096, 128, False), (8192, 2048, 50, True)])
+def test_mid_norm_equals_product_then_norm(dev, N, K, B, split):
+    """the 33..128-row product (+ residual) -> RMS_NORM -> MUL(weight) -> tile image as one call: the bits of the product followed by
+    the norm launch, in the row, in the normalised row and in the image"""
+    import torch
+    import mi355
+    lib = mi355.load()
+    t = orc.Q4_K
+    rng = np.random.default_rng(N + K + B)
+    xd = _to_dev(dev, rng.standard_normal((B, K)).astype(np.float32))
+    act = mi355.quantize_act_q8k_tiled(xd)
+    Wd = mi355.upload_weights(t, _to_dev(dev, _weights(rng, t, N, K, "ref")))
+    res = _to_dev(dev, rng.standard_normal((B, N)).astype(np.float32))
+    nw = _to_dev(dev, rng.standard_normal(N).astype(np.float32))
+    want_x = mi355.mul_mat_mid(t, Wd, xd, residual=res, split=split)
+    want_y = torch.empty((B, N), dtype=torch.float32, device=dev)
+    want_img = torch.zeros(lib.mi355_act_q8k_tiled_bytes(N, B), dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_rms_norm_mul_quant_q8k_tiled(None, want_x.data_ptr(), N, nw.data_ptr(), want_y.data_ptr(), N, want_img.data_ptr(), N, B, 1e-5))
+    got_x = torch.empty((B, N), dtype=torch.float32, device=dev)
+    got_y = torch.empty((B, N), dtype=torch.float32, device=dev)
+    got_img = torch.zeros_like(want_img)
+    nws = lib.mi355_mul_mat_mid_ws_bytes(N, K, B) if split else 0
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+    mi355.check(lib.mi355_mul_mat_mid_norm(None, t, Wd.data_ptr(), act.data_ptr(), got_x.data_ptr(), res.data_ptr(), N, K, B, N, ws.data_ptr() if nws else None, nws,
+                                           nw.data_ptr(), 1e-5, got_y.data_ptr(), N, got_img.data_ptr()))
+    torch.cuda.synchronize()
+    assert np.array_equal(got_x.cpu().numpy(), want_x.cpu().numpy())
+    assert np.array_equal(got_y.cpu().numpy(), want_y.cpu().numpy())
+    assert np.array_equal(got_img.cpu().numpy(), want_img.cpu().numpy())
+
+
 @pytest.mark.parametrize("Ns,K,B", [((4096, 1024, 1024), 4096, 128), ((14336, 14336), 4096, 64), ((100, 257, 64), 2048, 100), ((2048, 512), 1024, 40)])
 @pytest.mark.parametrize("split", [False, True])
 def test_mid_multi_equals_single_launches(dev, Ns, K, B, split):
