@@ -114,13 +114,8 @@ __device__ __forceinline__ float sub_rn(float a, float b) {
     return a - b;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-// Sum over the 64 lanes with DPP row operations (no LDS round trips), broadcast from lane 63 through a scalar register.
-// Every lane gets the same value; the summation order differs from wave_sum's butterfly.
+// Sum over the 64 lanes with DPP row operations (no LDS round trips: a __shfl_xor butterfly is six ds_bpermute of about a hundred
+// cycles each), broadcast from lane 63 through a scalar register.  Every lane gets the same value.
 template <int CTRL, int ROWMASK>
 __device__ __forceinline__ float dpp_add(float v) {
     return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xF, true));
@@ -134,6 +129,7 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     v = dpp_add<0x143, 0xC>(v);   // row_bcast31 into rows 2 and 3: lane 63 holds the total
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+__device__ __forceinline__ float wave_sum(float v) { return wave_sum_dpp(v); }
 // Maximum over the 64 lanes the same way (rows that a step does not write keep their value)
 template <int CTRL, int ROWMASK>
 __device__ __forceinline__ float dpp_max(float v) {
@@ -209,11 +205,7 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
     v = dpp_max<0x143, 0xC>(v);
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
-}
+__device__ __forceinline__ float wave_max(float v) { return wave_max_dpp(v); }   // a maximum is the same in any order
 
 // ---- host-side error plumbing
 void set_error(const char *fmt, ...);
