@@ -207,6 +207,27 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
 }
 __device__ __forceinline__ float wave_max(float v) { return wave_max_dpp(v); }   // a maximum is the same in any order
 
+// The values that a lane and the lane OFF away (lane ^ OFF; 8, 16 or 32) hold, as an unordered pair - the same pair, in the same
+// order, in both lanes: v_permlane16_swap / v_permlane32_swap hand the halves of a register to each other in a few cycles (for 8 a
+// rotation inside the 16-lane row), where __shfl_xor goes through the LDS crossbar.  For merges that are symmetric in the two.
+struct lane_pair { float a, b; };
+template <int OFF>
+__device__ __forceinline__ lane_pair lanes_pair(float x) {
+    static_assert(OFF == 8 || OFF == 16 || OFF == 32, "8, 16 or 32 lanes apart");
+    const int xi = __builtin_bit_cast(int, x);
+    if constexpr (OFF == 32) {
+        const auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+        return lane_pair{__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1])};
+    } else if constexpr (OFF == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);
+        return lane_pair{__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1])};
+    } else {
+        const float o = __builtin_bit_cast(float, dpp_get<0x128>(xi));   // row_ror:8 = lane ^ 8 inside a row of 16
+        const bool first = (threadIdx.x & 8) == 0;
+        return lane_pair{first ? x : o, first ? o : x};
+    }
+}
+
 // ---- host-side error plumbing
 void set_error(const char *fmt, ...);
 

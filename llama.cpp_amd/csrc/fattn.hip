@@ -13,6 +13,7 @@
 #include "fattn.hpp"
 
 #include <float.h>
+#include <type_traits>
 #include <stdlib.h>
 
 namespace mi355 {
@@ -300,16 +301,25 @@ __global__ void __launch_bounds__(NW * 64) k_fattn_vec(fattn_args a) {
     // merge the states: first the CPW lane groups of a wave (cross-lane), then the NW waves through LDS
 #pragma unroll
     for (int r = 0; r < R; r++) {
+        // (a lane and its partner end up with the same merged state: the pair is taken in one order by both)
+        auto merge_step = [&](auto off_c) {
+            constexpr int OFF = decltype(off_c)::value;
+            if constexpr (OFF >= LPR) {
+                const lane_pair pm = lanes_pair<OFF>(m[r]), pl = lanes_pair<OFF>(l[r]);
+                const float M = fmaxf(pm.a, pm.b);
+                const float fa = __expf(pm.a - M), fb = __expf(pm.b - M);
+                l[r] = pl.a * fa + pl.b * fb;
 #pragma unroll
-        for (int off = LPR; off < 64; off <<= 1) {
-            const float om = __shfl_xor(m[r], off, 64), ol = __shfl_xor(l[r], off, 64);
-            const float M = fmaxf(m[r], om);
-            const float fa = __expf(m[r] - M), fb = __expf(om - M);
-            l[r] = l[r] * fa + ol * fb;
-#pragma unroll
-            for (int i = 0; i < 8; i++) acc[r][i] = acc[r][i] * fa + __shfl_xor(acc[r][i], off, 64) * fb;
-            m[r] = M;
-        }
+                for (int i = 0; i < 8; i++) {
+                    const lane_pair pa = lanes_pair<OFF>(acc[r][i]);
+                    acc[r][i] = pa.a * fa + pa.b * fb;
+                }
+                m[r] = M;
+            }
+        };
+        merge_step(std::integral_constant<int, 8>{});
+        merge_step(std::integral_constant<int, 16>{});
+        merge_step(std::integral_constant<int, 32>{});
         if (lane == 0) {
             s_m[wave][r] = m[r];
             s_l[wave][r] = l[r];
