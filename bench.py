@@ -209,10 +209,10 @@ def sweep(kinds):
         print(json.dumps(kw), flush=True)
 
     bpe = {mi355.Q4_0: 18 / 32, mi355.Q8_0: 34 / 32, mi355.Q4_K: 144 / 256, mi355.Q5_K: 176 / 256, mi355.Q6_K: 210 / 256,
-           mi355.Q4_1: 20 / 32, mi355.Q5_0: 22 / 32, mi355.Q5_1: 24 / 32, mi355.IQ4_NL: 18 / 32}
+           mi355.Q4_1: 20 / 32, mi355.Q5_0: 22 / 32, mi355.Q5_1: 24 / 32, mi355.IQ4_NL: 18 / 32, mi355.IQ4_XS: 136 / 256}
     names = {mi355.Q4_0: "Q4_0", mi355.Q8_0: "Q8_0", mi355.Q4_K: "Q4_K", mi355.Q5_K: "Q5_K", mi355.Q6_K: "Q6_K", mi355.Q4_1: "Q4_1", mi355.Q5_0: "Q5_0",
-             mi355.Q5_1: "Q5_1", mi355.IQ4_NL: "IQ4_NL"}
-    all_types = (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q5_K, mi355.Q6_K, mi355.Q4_1, mi355.Q5_0, mi355.Q5_1, mi355.IQ4_NL)
+             mi355.Q5_1: "Q5_1", mi355.IQ4_NL: "IQ4_NL", mi355.IQ4_XS: "IQ4_XS"}
+    all_types = (mi355.Q4_0, mi355.Q8_0, mi355.Q4_K, mi355.Q5_K, mi355.Q6_K, mi355.Q4_1, mi355.Q5_0, mi355.Q5_1, mi355.IQ4_NL, mi355.IQ4_XS)
     shapes = [(4096, 4096), (14336, 4096), (4096, 14336)]
     if "gemv" in kinds:
         for t in all_types:

@@ -8,7 +8,7 @@
  *
  * Each entry point names the reference function it stands in for (paths relative to the
  * llama.cpp tree).  Element types use the reference's enum values
- * (ggml/include/ggml.h:351-392): F32 0, F16 1, Q4_0 2, Q4_1 3, Q5_0 6, Q5_1 7, Q8_0 8, Q8_1 9, Q4_K 12, Q5_K 13, Q6_K 14, IQ4_NL 20, I32 26.
+ * (ggml/include/ggml.h:351-392): F32 0, F16 1, Q4_0 2, Q4_1 3, Q5_0 6, Q5_1 7, Q8_0 8, Q8_1 9, Q4_K 12, Q5_K 13, Q6_K 14, IQ4_NL 20, IQ4_XS 23, I32 26.
  */
 #ifndef MI355_KERNELS_H
 #define MI355_KERNELS_H
@@ -27,7 +27,7 @@ extern "C" {
 
 enum mi355_type {
     MI355_F32 = 0, MI355_F16 = 1, MI355_Q4_0 = 2, MI355_Q4_1 = 3, MI355_Q5_0 = 6, MI355_Q5_1 = 7, MI355_Q8_0 = 8, MI355_Q8_1 = 9,
-    MI355_Q4_K = 12, MI355_Q5_K = 13, MI355_Q6_K = 14, MI355_IQ4_NL = 20, MI355_I32 = 26,
+    MI355_Q4_K = 12, MI355_Q5_K = 13, MI355_Q6_K = 14, MI355_IQ4_NL = 20, MI355_IQ4_XS = 23, MI355_I32 = 26,
 };
 
 /* Library / device ------------------------------------------------------------------ */
@@ -61,8 +61,9 @@ int mi355_quantize_weights(void *stream, int type, const float *x, void *y, int6
  *   Q5_1 : [nb x 16 B nibbles][nb x 4 B fifth bits][nb x {fp16 d, fp16 m}]
  *   Q8_0 : [nb x 32 B int8   ][nb x fp16 d]
  *   Q6_K : [nb x 128 B ql][nb x 64 B qh][nb x 16 B scales][nb x fp16 d]
+ *   IQ4_XS : [nb x 128 B nibbles][nb x {fp16 d, u16 scales_h, 4 B scales_l}]
  * A row occupies exactly the same number of bytes as in the reference's block layout
- * (ggml/src/ggml-common.h:161-208, 279-290, 314-320, 399-404); the mapping is a byte
+ * (ggml/src/ggml-common.h:161-208, 279-290, 314-320, 399-412); the mapping is a byte
  * permutation inside each row.  These two entry points apply it / undo it for the byte
  * range [offset, offset+size) of a tensor of `nrows` rows of `k` elements, so partial
  * uploads and read-back return the reference's bytes
@@ -98,7 +99,9 @@ int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64
  * Q4_1, Q5_0, Q5_1 and IQ4_NL (ggml/src/ggml-common.h:168-201, 399-404; ggml_vec_dot_q4_1_q8_1, _q5_0_q8_0, _q5_1_q8_1 and
  * _iq4_nl_q8_0, ggml/src/ggml-cpu/ggml-cpu-quants.c:2511, 2804, 3159, 11188) have the GEMV for up to 8 rows (also in the
  * launches that take several matrices or fuse an epilogue) and the per-32-block int8-MFMA tile kernel (mi355_mul_mat_q) beyond;
- * the weight-streaming kernel for 5..32 rows is built for Q4_0, Q8_0, Q4_K and Q6_K only.
+ * the weight-streaming kernel for 5..32 rows serves them too.
+ * IQ4_XS (block_iq4_xs, ggml/src/ggml-common.h:406-412; ggml_vec_dot_iq4_xs_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:11381) runs on the
+ * same three kernels as IQ4_NL, its block scales d * (ls - 32) taken from the super-block headers.
  * `ws` is scratch of at least mi355_mul_mat_ws_bytes(K, B) bytes. */
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,
@@ -387,7 +390,7 @@ int mi355_cpy(void *stream, const mi355_tensor *src, const mi355_tensor *dst);
  * emits (src/llama.cpp:157-199; ggml_compute_forward_dup_f32, ggml-cpu.c:3519-3830), with the row taken from device
  * memory so that a captured launch sequence does not change as the cache fills. */
 int mi355_set_rows(void *stream, const mi355_tensor *src, const int32_t *rows, const mi355_tensor *dst);
-/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, or whole quantized rows (Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0, Q4_K, Q5_K, Q6_K in the
+/* ggml_compute_forward_get_rows (ggml-cpu.c:8464-8590): src f32/f16 rows, or whole quantized rows (Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q8_0, Q4_K, Q5_K, Q6_K in the
  * device row layout, nb[1] = row bytes; dequantize_row_*, ggml-quants.c:255-273, 349-363, 1280-1302, 1482-1507, 1690-1719), ids i32
  * [n, b2, b3]; dst f32 */
 int mi355_get_rows(void *stream, const mi355_tensor *src, const mi355_tensor *ids, const mi355_tensor *dst);

@@ -14,7 +14,7 @@
 //  * buffer set/get_tensor synchronise the device first, because the scheduler may read a
 //    result right after an asynchronous graph_compute (ggml/src/ggml-backend.cpp:243-252).
 //
-// Quantized tensors of type Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / Q8_0 / Q6_K live in HBM in the 16-byte-aligned row layout
+// Quantized tensors of type Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / IQ4_XS / Q8_0 / Q6_K live in HBM in the 16-byte-aligned row layout
 // described in mi355_kernels.h; set_tensor applies that byte permutation and get_tensor
 // undoes it, so every caller sees the reference's bytes.
 
@@ -52,7 +52,7 @@ namespace {
 // ------------------------------------------------------------------------------- helpers
 bool is_repacked_type(ggml_type t) {
     return t == GGML_TYPE_Q4_0 || t == GGML_TYPE_Q8_0 || t == GGML_TYPE_Q6_K || t == GGML_TYPE_Q4_1 || t == GGML_TYPE_Q5_0 || t == GGML_TYPE_Q5_1 ||
-           t == GGML_TYPE_IQ4_NL;
+           t == GGML_TYPE_IQ4_NL || t == GGML_TYPE_IQ4_XS;
 }
 bool is_weight_type(ggml_type t) { return is_repacked_type(t) || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K; }
 
@@ -66,6 +66,7 @@ int to_mi355_type(ggml_type t) {
         case GGML_TYPE_Q5_0: return MI355_Q5_0;
         case GGML_TYPE_Q5_1: return MI355_Q5_1;
         case GGML_TYPE_IQ4_NL: return MI355_IQ4_NL;
+        case GGML_TYPE_IQ4_XS: return MI355_IQ4_XS;
         case GGML_TYPE_Q8_0: return MI355_Q8_0;
         case GGML_TYPE_Q4_K: return MI355_Q4_K;
         case GGML_TYPE_Q5_K: return MI355_Q5_K;
@@ -422,7 +423,7 @@ void * buffer_get_base(ggml_backend_buffer_t buffer) { return ((buffer_ctx *) bu
 // number of rows / elements per row of a tensor whose rows are contiguous blocks
 int64_t tensor_nrows(const ggml_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
 
-// Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0 and Q6_K tensors live in the device row layout, which is defined by the rows of the tensor that owns the memory: a
+// Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q8_0 and Q6_K tensors live in the device row layout, which is defined by the rows of the tensor that owns the memory: a
 // view (a slice of experts, a permuted or 1-D view of a cache) addresses bytes of that tensor, so transfers through a view go
 // through the owner's layout at the view's byte offset.
 struct repack_target {

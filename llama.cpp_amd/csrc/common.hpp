@@ -23,17 +23,17 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int WAVE = 64;
 
-// ---- block geometry (ggml/src/ggml-common.h:161-221, 279-290, 296-308, 314-320, 399-404)
+// ---- block geometry (ggml/src/ggml-common.h:161-221, 279-290, 296-308, 314-320, 399-412)
 constexpr int QK = 32;     // elements per Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / Q8_0 / Q8_1 block
 constexpr int QKK = 256;   // elements per K-quant super-block
 constexpr int Q4_0_BYTES = 18, Q8_0_BYTES = 34, Q8_1_BYTES = 36, Q4_K_BYTES = 144, Q5_K_BYTES = 176, Q6_K_BYTES = 210;
-constexpr int Q4_1_BYTES = 20, Q5_0_BYTES = 22, Q5_1_BYTES = 24, IQ4_NL_BYTES = 18;
+constexpr int Q4_1_BYTES = 20, Q5_0_BYTES = 22, Q5_1_BYTES = 24, IQ4_NL_BYTES = 18, IQ4_XS_BYTES = 136;
 
 __host__ __device__ inline int type_block_elems(int t) {
     switch (t) {
         case MI355_Q4_0: case MI355_Q8_0: case MI355_Q8_1: return QK;
         case MI355_Q4_1: case MI355_Q5_0: case MI355_Q5_1: case MI355_IQ4_NL: return QK;
-        case MI355_Q4_K: case MI355_Q5_K: case MI355_Q6_K: return QKK;
+        case MI355_Q4_K: case MI355_Q5_K: case MI355_Q6_K: case MI355_IQ4_XS: return QKK;
         case MI355_F32: case MI355_F16: case MI355_I32: return 1;
         default: return 0;
     }
@@ -45,6 +45,7 @@ __host__ __device__ inline int type_block_bytes(int t) {
         case MI355_Q5_0: return Q5_0_BYTES;
         case MI355_Q5_1: return Q5_1_BYTES;
         case MI355_IQ4_NL: return IQ4_NL_BYTES;
+        case MI355_IQ4_XS: return IQ4_XS_BYTES;
         case MI355_Q8_0: return Q8_0_BYTES;
         case MI355_Q8_1: return Q8_1_BYTES;
         case MI355_Q4_K: return Q4_K_BYTES;
@@ -57,7 +58,7 @@ __host__ __device__ inline int type_block_bytes(int t) {
 }
 __host__ __device__ inline bool is_weight_type(int t) {
     return t == MI355_Q4_0 || t == MI355_Q8_0 || t == MI355_Q4_K || t == MI355_Q5_K || t == MI355_Q6_K || t == MI355_Q4_1 || t == MI355_Q5_0 ||
-           t == MI355_Q5_1 || t == MI355_IQ4_NL;
+           t == MI355_Q5_1 || t == MI355_IQ4_NL || t == MI355_IQ4_XS;
 }
 // Expands X(TYPE) for the weight type t (checked with is_weight_type before).
 #define MI355_WEIGHT_TYPE_SWITCH(t, X)            \
@@ -70,6 +71,7 @@ __host__ __device__ inline bool is_weight_type(int t) {
         case MI355_Q8_0: X(MI355_Q8_0) break;     \
         case MI355_Q4_K: X(MI355_Q4_K) break;     \
         case MI355_Q5_K: X(MI355_Q5_K) break;     \
+        case MI355_IQ4_XS: X(MI355_IQ4_XS) break; \
         default: X(MI355_Q6_K) break;             \
     }
 

@@ -13,6 +13,7 @@
 //   Q4_0 : level - 8 as int8, scale d                    (one MFMA per block)
 //   Q8_0 : level as int8, scale d
 //   Q5_0 : level - 16 as int8, scale d;  IQ4_NL : the table value of the nibble as int8, scale d
+//   IQ4_XS : as IQ4_NL, scale d * (ls - 32) from the super-block's header
 //   Q4_1, Q5_1 : level 0..15 / 0..31 as int8, scale d; the "+ m * d_x * sum(q)" term of the stage's four blocks is added with one
 //          v_mfma_f32_32x32x16_f16 on (fp16 dx*sum(q), the reference's `s` field of block_q8_1) x (fp16 m)
 //   Q4_K, Q5_K : level 0..15 / 0..31 as int8, scale d*sc; the "- dmin*m*sum(q)" term of all blocks is
@@ -43,7 +44,8 @@ template <int TYPE> struct mmq_cfg {
     // a per-block offset rides on the sums of the activation levels: - dmin * m (Q4_K), + m (Q4_1, Q5_1)
     static constexpr bool MIN = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;
     // 16 bytes of nibbles per block with a per-block scale: one request / commit form serves them all
-    static constexpr bool NIBBLE32 = TYPE == MI355_Q4_0 || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1 || TYPE == MI355_IQ4_NL;
+    static constexpr bool NIBBLE32 = TYPE == MI355_Q4_0 || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1 || TYPE == MI355_IQ4_NL ||
+                                     TYPE == MI355_IQ4_XS;
     static constexpr bool PREFETCH = NIBBLE32 || TYPE == MI355_Q8_0;
 };
 
@@ -197,13 +199,13 @@ __device__ __forceinline__ void load_act_stage(const int8_t *__restrict__ aq, co
 // ---- the same stages split into "request" (global -> registers) and "commit" (unpack -> LDS), so that the next stage's bytes
 // travel while the current stage is contracted (Q4_0 / Q8_0, whose per-32 scales keep them on this kernel)
 template <int TYPE, bool NIB = mmq_cfg<TYPE>::NIBBLE32> struct mmq_wregs {};
-// Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL: thread t owns blocks (row, b) = (idx >> 2, idx & 3), idx = t and t + 256
+// Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS: thread t owns blocks (row, b) = (idx >> 2, idx & 3), idx = t and t + 256
 template <int TYPE> struct mmq_wregs<TYPE, true> {
     static constexpr bool HAS_QH = TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1;
     static constexpr bool HAS_MIN = TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;
     u32x4 q[2];
     u32 qh[2];
-    u32 dm[2];   // fp16 d in the low half, fp16 m above it (HAS_MIN)
+    u32 dm[2];   // fp16 d in the low half, fp16 m above it (HAS_MIN); IQ4_XS: the bits of the f32 block scale
     __device__ __forceinline__ void fetch(const uint8_t *__restrict__ W, const row_layout &L, int64_t row0, int64_t N, int64_t k0, int tid) {
 #pragma unroll
         for (int it = 0; it < 2; it++) {
@@ -215,7 +217,10 @@ template <int TYPE> struct mmq_wregs<TYPE, true> {
             q[it] = load16(wrow + blk * 16);
             if constexpr (HAS_QH) qh[it] = *(const u32 *)(wrow + L.off_b + blk * 4);
             const int so = HAS_QH ? L.off_c : L.off_b;   // the scales follow the fifth bits where there are any
-            if constexpr (HAS_MIN) dm[it] = *(const u32 *)(wrow + so + blk * 4);
+            if constexpr (TYPE == MI355_IQ4_XS) {
+                const uint2 h = *(const uint2 *)(wrow + L.off_b + (blk >> 3) * 8);
+                dm[it] = __builtin_bit_cast(u32, iq4xs_block_scale(h.x, h.y, (int)(blk & 7)));
+            } else if constexpr (HAS_MIN) dm[it] = *(const u32 *)(wrow + so + blk * 4);
             else dm[it] = *(const unsigned short *)(wrow + so + blk * 2);
         }
     }
@@ -238,7 +243,7 @@ template <int TYPE> struct mmq_wregs<TYPE, true> {
                 } else if constexpr (TYPE == MI355_Q5_0) {   // level - 16
                     a = ((a | 0x80808080u) - 0x10101010u) ^ 0x80808080u;
                     c = ((c | 0x80808080u) - 0x10101010u) ^ 0x80808080u;
-                } else if constexpr (TYPE == MI355_IQ4_NL) {
+                } else if constexpr (TYPE == MI355_IQ4_NL || TYPE == MI355_IQ4_XS) {
                     a = iq4nl_lookup4(a);
                     c = iq4nl_lookup4(c);
                 }
@@ -247,7 +252,8 @@ template <int TYPE> struct mmq_wregs<TYPE, true> {
             }
             *(u32x4 *)(sW + r * MMQ_LDK + b * 32) = lo;
             *(u32x4 *)(sW + r * MMQ_LDK + b * 32 + 16) = hi;
-            sWs[b * MMQ_BM + r] = half_bits_to_float((unsigned short)(dm[it] & 0xFFFFu));
+            if constexpr (TYPE == MI355_IQ4_XS) sWs[b * MMQ_BM + r] = __builtin_bit_cast(float, dm[it]);
+            else sWs[b * MMQ_BM + r] = half_bits_to_float((unsigned short)(dm[it] & 0xFFFFu));
             if constexpr (HAS_MIN) {
                 union { unsigned short u; _Float16 f; } m;
                 m.u = (unsigned short)(dm[it] >> 16);
@@ -567,6 +573,7 @@ extern "C" int mi355_mul_mat_q_ws(void *stream, int type, const void *W, const v
         case MI355_Q5_0: launch_mmq_tn<MI355_Q5_0>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_Q5_1: launch_mmq_tn<MI355_Q5_1>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         case MI355_IQ4_NL: launch_mmq_tn<MI355_IQ4_NL>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
+        case MI355_IQ4_XS: launch_mmq_tn<MI355_IQ4_XS>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
         default: launch_mmq_tn<MI355_Q6_K>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes); break;
     }
     return launch_status("k_mmq");

@@ -3,6 +3,7 @@
 // Work unit ("chunk"): what one lane consumes per step.  Chunk c of a row is taken by lane
 // c % 64 at step c / 64, so a wave walks a row in consecutive 16-byte, 16-byte-aligned loads.
 //   Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL : chunk = one 32-element block.
+//   IQ4_XS      : chunk = one 32-element block of its super-block; 8 chunks share the 8-byte header.
 //   Q4_K        : chunk = 32 bytes of qs = sub-blocks 2g (low nibbles) and 2g+1 (high nibbles),
 //                 64 elements; 4 chunks per super-block share its 16-byte header.
 //   Q5_K        : as Q4_K, plus the 32 bytes of qh that carry the fifth bit of all eight sub-blocks.
@@ -19,7 +20,7 @@ namespace mi355 {
 // Device layout of one weight row (see mi355_kernels.h): byte offsets of the per-row regions.
 struct row_layout {
     int64_t row_bytes;
-    int off_b;   // Q4_0/Q8_0/IQ4_NL: fp16 d array.  Q4_1: {fp16 d, fp16 m} array.  Q5_0/Q5_1: fifth-bit words.  Q6_K: qh array
+    int off_b;   // IQ4_XS: {fp16 d, scales_h, scales_l[4]} array.  Q4_0/Q8_0/IQ4_NL: fp16 d array.  Q4_1: {fp16 d, fp16 m} array.  Q5_0/Q5_1: fifth-bit words.  Q6_K: qh array
     int off_c;   // Q5_0: fp16 d array.  Q5_1: {fp16 d, fp16 m} array.  Q6_K: scales array
     int off_d;   // Q6_K: fp16 d array
 };
@@ -32,6 +33,7 @@ __host__ __device__ inline row_layout make_row_layout(int type, int64_t k) {
         case MI355_Q4_0: case MI355_IQ4_NL: case MI355_Q4_1: L.off_b = (int)(nb * 16); break;
         case MI355_Q5_0: case MI355_Q5_1: L.off_b = (int)(nb * 16); L.off_c = (int)(nb * 20); break;
         case MI355_Q8_0: L.off_b = (int)(nb * 32); break;
+        case MI355_IQ4_XS: L.off_b = (int)(nb * 128); break;
         case MI355_Q6_K: L.off_b = (int)(nb * 128); L.off_c = (int)(nb * 192); L.off_d = (int)(nb * 208); break;
         default: break;
     }
@@ -171,6 +173,33 @@ template <> struct wq<MI355_IQ4_NL> {
         chunk_dots r = {s, 0};
         return r;
     }
+    static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
+        return __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), acc);
+    }
+};
+
+// ---------------------------------------------------------------- IQ4_XS
+// block_iq4_xs (ggml/src/ggml-common.h:406-412): eight blocks of IQ4_NL levels under one fp16 d; block ib is scaled by
+// d * (ls - 32), ls = scales_l nibble ib | two bits of scales_h << 4 (dequantize_row_iq4_xs, ggml/src/ggml-quants.c:2454-2475;
+// ggml_vec_dot_iq4_xs_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:11381, scalar tail :11647-11676).
+// hdr = the header's two dwords: {d | scales_h << 16, scales_l[0..3]}
+__device__ __forceinline__ float iq4xs_block_scale(u32 h0, u32 h1, int ib) {
+    const int ls = (int)(((h1 >> (4 * ib)) & 0xFu) | (((h0 >> (16 + 2 * ib)) & 3u) << 4));
+    return mul_rn(half_bits_to_float((unsigned short)(h0 & 0xFFFFu)), (float)(ls - 32));
+}
+template <> struct wq<MI355_IQ4_XS> {
+    static constexpr int CHUNK = 32;
+    typedef wq<MI355_Q4_0>::chunk chunk;
+    typedef wq<MI355_Q8_0>::act act;
+    static __device__ __forceinline__ chunk load_w(const uint8_t *__restrict__ row, const row_layout &L, int c) {
+        chunk w;
+        w.qs = load_stream16(row + c * 16);
+        const uint2 h = *(const uint2 *)(row + L.off_b + (c >> 3) * 8);   // the same eight bytes for the eight lanes of a super-block
+        w.d = iq4xs_block_scale(h.x, h.y, c & 7);
+        return w;
+    }
+    static __device__ __forceinline__ act load_a(const int8_t *__restrict__ q, const act_ds *__restrict__ ds, int c) { return wq<MI355_Q8_0>::load_a(q, ds, c); }
+    static __device__ __forceinline__ chunk_dots dots(const chunk &w, const act &A) { return wq<MI355_IQ4_NL>::dots(w, A); }
     static __device__ __forceinline__ float accumulate(float acc, const chunk &w, const act &A, const chunk_dots &r) {
         return __builtin_fmaf(w.d, mul_rn(A.d, (float)r.i0), acc);
     }
@@ -445,7 +474,7 @@ template <> struct wq<MI355_Q6_K> {
 // Dequantized weight element e of a row stored in device layout.  Byte loads only, so it
 // works for rows that are not 16-byte aligned (K not a multiple of 256 for Q4_0/Q8_0, of
 // 2048 for Q6_K).  Semantics: dequantize_row_* of ggml/src/ggml-quants.c:255-347, 349-363,
-// 1280-1302, 1482-1507, 1690-1719, 2436-2452.
+// 1280-1302, 1482-1507, 1690-1719, 2436-2475.
 template <int TYPE>
 __device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, const row_layout &L, int64_t e) {
     if constexpr (TYPE == MI355_Q4_0) {
@@ -462,6 +491,15 @@ __device__ __forceinline__ float weight_value(const uint8_t *__restrict__ row, c
         const uint8_t byte = row[b * 16 + (j & 15)];
         const unsigned short dh = (unsigned short)(row[L.off_b + 2 * b] | (row[L.off_b + 2 * b + 1] << 8));
         return half_bits_to_float(dh) * (float)values[j < 16 ? (byte & 0x0F) : (byte >> 4)];
+    } else if constexpr (TYPE == MI355_IQ4_XS) {
+        constexpr int8_t values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+        const int64_t b = e >> 5;
+        const int j = (int)(e & 31), ib = (int)(b & 7);
+        const uint8_t byte = row[b * 16 + (j & 15)];
+        const uint8_t *h = row + L.off_b + (b >> 3) * 8;
+        const int ls = ((h[4 + ib / 2] >> (4 * (ib & 1))) & 0xF) | (((((int)h[2] | ((int)h[3] << 8)) >> (2 * ib)) & 3) << 4);
+        const float dl = half_bits_to_float((unsigned short)(h[0] | (h[1] << 8))) * (float)(ls - 32);
+        return dl * (float)values[j < 16 ? (byte & 0x0F) : (byte >> 4)];
     } else if constexpr (TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1) {
         const int64_t b = e >> 5;
         const int j = (int)(e & 31);

@@ -101,6 +101,10 @@ __device__ __forceinline__ int64_t dev_offset_in_row(int type, int64_t nb, int64
             if (o < 4) return nb * 20 + b * 4 + o;
             return o < 8 ? nb * 16 + b * 4 + (o - 4) : b * 16 + (o - 8);
         }
+        case MI355_IQ4_XS: {   // d, scales_h, scales_l[4], 128 nibble bytes
+            const int64_t b = w / IQ4_XS_BYTES, o = w % IQ4_XS_BYTES;
+            return o < 8 ? nb * 128 + b * 8 + o : b * 128 + (o - 8);
+        }
         case MI355_Q8_0: {
             const int64_t b = w / Q8_0_BYTES, o = w % Q8_0_BYTES;
             return o < 2 ? nb * 32 + b * 2 + o : b * 32 + (o - 2);

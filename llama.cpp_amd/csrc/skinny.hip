@@ -30,7 +30,9 @@ namespace {
 template <int TYPE> struct sk_traits {
     static constexpr int ROW_BYTES = TYPE == MI355_Q8_0 ? 256 : 128;
     // per-32-block types whose block is 16 bytes of nibbles, element b low and element 16 + b high in byte b
-    static constexpr bool NIB32 = TYPE == MI355_Q4_0 || TYPE == MI355_IQ4_NL || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1;
+    static constexpr bool NIB32 = TYPE == MI355_Q4_0 || TYPE == MI355_IQ4_NL || TYPE == MI355_IQ4_XS || TYPE == MI355_Q4_1 || TYPE == MI355_Q5_0 ||
+                                  TYPE == MI355_Q5_1;
+    static constexpr bool TABLE = TYPE == MI355_IQ4_NL || TYPE == MI355_IQ4_XS;     // a nibble stands for an entry of the sixteen-value table
     static constexpr bool PAIR = TYPE == MI355_Q4_1 || TYPE == MI355_Q5_1;          // {f16 d, f16 m} per block
     static constexpr bool FIFTH32 = TYPE == MI355_Q5_0 || TYPE == MI355_Q5_1;       // one word of fifth bits per block
     static constexpr bool KQ = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K;            // 16-byte header + 6-bit (scale, min) pairs
@@ -161,6 +163,10 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
         } else if constexpr (T::PAIR) {
             g.hdr = load16(w_mine + L.off_b + s * 32);
             g.hdr2 = load16(w_mine + L.off_b + s * 32 + 16);
+        } else if constexpr (TYPE == MI355_IQ4_XS) {
+            const uint2 h = *(const uint2 *)(w_mine + L.off_b + s * 8);   // the super-block's d, scales_h, scales_l
+            g.hdr[0] = h.x;
+            g.hdr[1] = h.y;
         } else if constexpr (Q6) {
 #pragma unroll
             for (int u = 0; u < 2; u++) g.qh[u] = load16(qh_src[u] + s * 64);
@@ -288,6 +294,9 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
                     ws[j] = half_bits_to_float((unsigned short)(dm & 0xFFFFu));
                     wm[j] = half_bits_to_float((unsigned short)(dm >> 16));
                 }
+            } else if constexpr (TYPE == MI355_IQ4_XS) {
+    #pragma unroll
+                for (int j = 0; j < 8; j++) ws[j] = iq4xs_block_scale(hdr[0], hdr[1], j);
             } else {
     #pragma unroll
                 for (int j = 0; j < 8; j++) ws[j] = f16_of(hdr, j);
@@ -304,7 +313,7 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
     #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const u32 nib = (v[i] >> (4 * kh)) & 0x0F0F0F0Fu;   // elements 16 kh + 4 i .. + 4
-                        if constexpr (TYPE == MI355_IQ4_NL) wop[i] = (int)iq4nl_lookup4(nib);
+                        if constexpr (T::TABLE) wop[i] = (int)iq4nl_lookup4(nib);
                         else if constexpr (T::FIFTH32) wop[i] = (int)(nib | spread4(fw >> (16 * kh + 4 * i)));
                         else wop[i] = (int)nib;
                     }
@@ -333,7 +342,7 @@ __global__ void __launch_bounds__(256) k_mm_skinny(const uint8_t *__restrict__ W
                         const float Df = (float)D[4 * q + i];
                         if constexpr (TYPE == MI355_Q4_0 || TYPE == MI355_Q5_0) {
                             acc[q][i] = __builtin_fmaf(ws[j], __builtin_fmaf(dd[i], Df, xx[i]), acc[q][i]);   // x = -8 (-16) d sum
-                        } else if constexpr (TYPE == MI355_Q8_0 || TYPE == MI355_IQ4_NL) {
+                        } else if constexpr (TYPE == MI355_Q8_0 || T::TABLE) {
                             acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);
                         } else {   // block minimum: + m (Q4_1, Q5_1), - dmin * 6-bit minimum (Q4_K, Q5_K)
                             acc[q][i] = __builtin_fmaf(ws[j], dd[i] * Df, acc[q][i]);

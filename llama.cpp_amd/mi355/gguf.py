@@ -31,12 +31,12 @@ def _package():
     sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     return importlib.import_module("mi355")
 
-F32, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL = 0, 2, 3, 6, 7, 8, 12, 13, 14, 20
+F32, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS = 0, 2, 3, 6, 7, 8, 12, 13, 14, 20, 23
 BLOCK = {Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34),
-         IQ4_NL: (32, 18)}
-# file type -> (default tensor type, LLAMA_FTYPE_MOSTLY_* of include/llama.h:146-169)
+         IQ4_NL: (32, 18), IQ4_XS: (256, 136)}
+# file type -> (default tensor type, LLAMA_FTYPE_MOSTLY_* of include/llama.h:146-174)
 FTYPES = {"q4_k_m": (Q4_K, 15), "q5_k_m": (Q5_K, 17), "q4_0": (Q4_0, 2), "q4_1": (Q4_1, 3), "q5_0": (Q5_0, 8), "q5_1": (Q5_1, 9), "q8_0": (Q8_0, 7),
-          "iq4_nl": (IQ4_NL, 25)}
+          "iq4_nl": (IQ4_NL, 25), "iq4_xs": (IQ4_XS, 30)}
 T_U32, T_F32, T_STR, T_U64 = 4, 6, 8, 10
 
 
@@ -68,14 +68,14 @@ def tensor_list(n_layer, n_embd, n_ff, n_head, n_head_kv, head_dim, n_vocab, n_e
     of `llama-quantize --pure ... Q4_K`; the router ffn_gate_inp stays f32 (src/llama-quant.cpp:749).
     base: Q4_K for the Q4_K_M mix, Q5_K for Q5_K_M (the same rules with Q5_K as the default type, src/llama-quant.cpp:122-340).
     A per-32-block base (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0) is used for every matrix, as llama-quantize does without an importance
-    matrix, with output.weight Q6_K (Q8_0 stays Q8_0, :166-168); IQ4_NL takes Q5_K for attn_v (grouped-query models, :232-234) and for
+    matrix, with output.weight Q6_K (Q8_0 stays Q8_0, :166-168); IQ4_NL and IQ4_XS take Q5_K for attn_v (grouped-query models, :232-234) and for
     ffn_down in the first eighth of the layers (:299-301)."""
     t = [("token_embd.weight", base, (n_embd, n_vocab))]
     kmix = base in (Q4_K, Q5_K)
     for il in range(n_layer):
         more = kmix and use_more_bits(il, n_layer) and n_expert == 0
-        v_type = Q6_K if more else Q5_K if (base == IQ4_NL and n_head // n_head_kv >= 4) else base
-        down_type = Q6_K if more else Q5_K if (base == IQ4_NL and il < n_layer // 8) else base
+        v_type = Q6_K if more else Q5_K if (base in (IQ4_NL, IQ4_XS) and n_head // n_head_kv >= 4) else base
+        down_type = Q6_K if more else Q5_K if (base in (IQ4_NL, IQ4_XS) and il < n_layer // 8) else base
         p = "blk.%d." % il
         if n_expert > 0:
             t += [(p + "attn_norm.weight", F32, (n_embd,)),
@@ -133,6 +133,8 @@ def random_blocks(ttype, n_blocks, rng, pool):
         put_half(2, 0.02 / (31.5 * 9.2) * 15.5)
     elif ttype == Q6_K:    # w = d*sc*(q-32), sc int8
         put_half(208, 0.02 / (74.0 * 18.5))
+    elif ttype == IQ4_XS:  # w = d * (ls - 32) * table[n], ls ~ U[0, 63]
+        put_half(0, 0.02 / (18.5 * 68.0))
     elif ttype in (Q4_0, Q8_0, Q5_0, IQ4_NL):   # w = d * level: levels of spread 4.6 / 74 / 9.2 / 68
         put_half(0, 0.02 / {Q4_0: 4.6, Q8_0: 74.0, Q5_0: 9.2, IQ4_NL: 68.0}[ttype])
     else:                  # Q4_1 / Q5_1: w = d * n + m

@@ -13,7 +13,7 @@ import math
 
 import torch
 
-from . import (F16, F32, I32, Q4_K, Q5_K, Q6_K, Q4_0, Q8_0, Q4_1, Q5_0, Q5_1, IQ4_NL, BLOCK, GemvMat, Tensor, TiledMat, check, load, row_bytes, tensor_desc,
+from . import (F16, F32, I32, Q4_K, Q5_K, Q6_K, Q4_0, Q8_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, BLOCK, GemvMat, Tensor, TiledMat, check, load, row_bytes, tensor_desc,
                upload_weights, _ptr, _stream)
 
 
@@ -56,6 +56,8 @@ def random_quantized(t, nrows, k, device, gen):
         put_half(0, 0.02 / 9.2)
     elif t == IQ4_NL:  # w = d*table[n]
         put_half(0, 0.02 / 68.0)
+    elif t == IQ4_XS:  # w = d*(ls-32)*table[n], ls ~ U[0, 63]
+        put_half(0, 0.02 / (18.5 * 68.0))
     elif t in (Q4_1, Q5_1):   # w = d*n + m
         spread, mid = (4.6, 7.5) if t == Q4_1 else (9.2, 15.5)
         put_half(0, 0.02 / spread)

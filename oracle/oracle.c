@@ -32,13 +32,14 @@
 /* ------------------------------------------------------------------ block layouts
  * ggml/src/ggml-common.h:161-166 (q4_0), 203-208 (q8_0), 210-221 (q8_1),
  * 279-290 (q4_K), 296-308 (q5_K), 314-320 (q6_K), 322-328 (q8_K), 168-179 (q4_1), 181-187 (q5_0), 189-201 (q5_1),
- * 399-404 (iq4_nl).  All packed, no padding. */
+ * 399-404 (iq4_nl), 406-412 (iq4_xs).  All packed, no padding. */
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[16]; } blk_q4_0;                       /* 18 B  */
 typedef struct { uint16_t d; uint16_t m; uint8_t qs[16]; } blk_q4_1;           /* 20 B  */
 typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_0;        /* 22 B  */
 typedef struct { uint16_t d; uint16_t m; uint8_t qh[4]; uint8_t qs[16]; } blk_q5_1; /* 24 B */
 typedef struct { uint16_t d; uint8_t qs[16]; } blk_iq4_nl;                     /* 18 B  */
+typedef struct { uint16_t d; uint16_t scales_h; uint8_t scales_l[4]; uint8_t qs[128]; } blk_iq4_xs; /* 136 B */
 typedef struct { uint16_t d; int8_t qs[32]; } blk_q8_0;                        /* 34 B  */
 typedef struct { uint16_t d; uint16_t s; int8_t qs[32]; } blk_q8_1;            /* 36 B  */
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[128]; } blk_q4_K; /* 144 B */
@@ -100,7 +101,7 @@ int orc_block_elems(int type) {
     switch (type) {
         case ORC_F32: case ORC_F16: return 1;
         case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_IQ4_NL: case ORC_Q8_0: case ORC_Q8_1: return QK;
-        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_Q8_K: return QKK;
+        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_Q8_K: case ORC_IQ4_XS: return QKK;
         default: return 0;
     }
 }
@@ -113,6 +114,7 @@ size_t orc_block_bytes(int type) {
         case ORC_Q5_0: return sizeof(blk_q5_0);
         case ORC_Q5_1: return sizeof(blk_q5_1);
         case ORC_IQ4_NL: return sizeof(blk_iq4_nl);
+        case ORC_IQ4_XS: return sizeof(blk_iq4_xs);
         case ORC_Q8_0: return sizeof(blk_q8_0);
         case ORC_Q8_1: return sizeof(blk_q8_1);
         case ORC_Q4_K: return sizeof(blk_q4_K);
@@ -311,56 +313,52 @@ static int iq4nl_best_index(float x) {   /* best_index_int8, ggml/src/ggml-quant
     }
     return x - val[mu - 1] < val[mu] - x ? mu - 1 : mu;
 }
-static void quant_iq4_nl(const float *x, blk_iq4_nl *y, int64_t k) {
+/* the scale of one 32-element block: the first guess max / -127, then the 15 candidates (itry - 127) / max, each scored by the
+ * weighted least-squares fit with weights x^2 (quantize_row_iq4_nl_impl :4588-4640 with quant_weights == NULL, ntry = 7);
+ * 0 for a block whose largest magnitude is below GROUP_MAX_EPS */
+static float iq4nl_block_scale(const float *xb) {
     const int ntry = 7;
+    float amax = 0, max = 0;
+    for (int j = 0; j < QK; j++) {
+        const float ax = fabsf(xb[j]);
+        if (ax > amax) { amax = ax; max = xb[j]; }
+    }
+    if (amax < 1e-15f) return 0;
+    float d = -max / iq4nl_values[0];
+    float id = 1 / d;
+    float sumqx = 0, sumq2 = 0;
+    for (int j = 0; j < QK; j++) {
+        const float q = iq4nl_values[iq4nl_best_index(id * xb[j])];
+        const float w = xb[j] * xb[j];
+        sumqx += w * q * xb[j];
+        sumq2 += w * q * q;
+    }
+    d = sumqx / sumq2;
+    float best = d * sumqx;
+    for (int itry = -ntry; itry <= ntry; itry++) {
+        id = (itry + iq4nl_values[0]) / max;
+        sumqx = sumq2 = 0;
+        for (int j = 0; j < QK; j++) {
+            const float q = iq4nl_values[iq4nl_best_index(id * xb[j])];
+            const float w = xb[j] * xb[j];
+            sumqx += w * q * xb[j];
+            sumq2 += w * q * q;
+        }
+        if (sumq2 > 0 && sumqx * sumqx > best * sumq2) { d = sumqx / sumq2; best = d * sumqx; }
+    }
+    return d;
+}
+static void iq4nl_pack_block(const float *xb, float id, uint8_t *qs) {   /* element j low, element 16 + j high in byte j */
+    uint8_t L[QK];
+    for (int j = 0; j < QK; j++) L[j] = (uint8_t)iq4nl_best_index(id * xb[j]);
+    for (int j = 0; j < 16; j++) qs[j] = (uint8_t)(L[j] | (L[16 + j] << 4));
+}
+static void quant_iq4_nl(const float *x, blk_iq4_nl *y, int64_t k) {
     for (int64_t b = 0; b < k / QK; b++) {
         const float *xb = x + b * QK;
-        uint8_t L[QK];
-        float weight[QK];
-        memset(y[b].qs, 0, 16);
-        y[b].d = orc_f32_to_f16(0.f);
-        for (int j = 0; j < QK; j++) weight[j] = xb[j] * xb[j];
-        float amax = 0, max = 0;
-        for (int j = 0; j < QK; j++) {
-            const float ax = fabsf(xb[j]);
-            if (ax > amax) { amax = ax; max = xb[j]; }
-        }
-        float scale = 0;
-        memset(L, 0, sizeof(L));
-        if (amax >= 1e-15f) {
-            float d = -max / iq4nl_values[0];
-            float id = 1 / d;
-            float sumqx = 0, sumq2 = 0;
-            for (int j = 0; j < QK; j++) {
-                const float al = id * xb[j];
-                const int l = iq4nl_best_index(al);
-                L[j] = (uint8_t)l;
-                const float q = iq4nl_values[l];
-                const float w = weight[j];
-                sumqx += w * q * xb[j];
-                sumq2 += w * q * q;
-            }
-            d = sumqx / sumq2;
-            float best = d * sumqx;
-            for (int itry = -ntry; itry <= ntry; itry++) {
-                id = (itry + iq4nl_values[0]) / max;
-                sumqx = sumq2 = 0;
-                for (int j = 0; j < QK; j++) {
-                    const float al = id * xb[j];
-                    const int l = iq4nl_best_index(al);
-                    const float q = iq4nl_values[l];
-                    const float w = weight[j];
-                    sumqx += w * q * xb[j];
-                    sumq2 += w * q * q;
-                }
-                if (sumq2 > 0 && sumqx * sumqx > best * sumq2) { d = sumqx / sumq2; best = d * sumqx; }
-            }
-            scale = d;
-        }
+        const float scale = iq4nl_block_scale(xb);
         y[b].d = orc_f32_to_f16(scale);
-        const float id = scale ? 1 / scale : 0;
-        for (int j = 0; j < QK; j++) L[j] = (uint8_t)iq4nl_best_index(id * xb[j]);
-        for (int j = 0; j < 16; j++) y[b].qs[j] = (uint8_t)(L[j] | (L[16 + j] << 4));
+        iq4nl_pack_block(xb, scale ? 1 / scale : 0, y[b].qs);
     }
 }
 static void dequant_iq4_nl(const blk_iq4_nl *x, float *y, int64_t k) {
@@ -369,6 +367,53 @@ static void dequant_iq4_nl(const blk_iq4_nl *x, float *y, int64_t k) {
         for (int j = 0; j < QK / 2; j++) {
             y[b * QK + j] = d * iq4nl_values[x[b].qs[j] & 0x0F];
             y[b * QK + j + QK / 2] = d * iq4nl_values[x[b].qs[j] >> 4];
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ IQ4_XS
+ * super-blocks of 256: eight 32-element blocks of IQ4_NL levels whose scales are d * (ls - 32), ls six bits (low four in scales_l,
+ * high two in scales_h).  quantize_iq4_xs without importance weights (ggml/src/ggml-quants.c:4722-4745) = quantize_row_iq4_nl_impl
+ * on the super-block (:4573-4682): the block scales as for IQ4_NL, d = -(the block scale of largest magnitude) / 32, ls = the block
+ * scale over d rounded and clamped to [-32, 31], the levels chosen again for d * ls.  dequantize_row_iq4_xs :2454-2475. */
+static int iq4xs_ls(const blk_iq4_xs *b, int ib) {
+    return ((b->scales_l[ib / 2] >> 4 * (ib % 2)) & 0xF) | (((b->scales_h >> 2 * ib) & 3) << 4);
+}
+static void quant_iq4_xs(const float *x, blk_iq4_xs *y, int64_t k) {
+    for (int64_t sb = 0; sb < k / QKK; sb++) {
+        const float *xs = x + sb * QKK;
+        float scales[8];
+        float max_scale = 0, amax_scale = 0;
+        memset(&y[sb], 0, sizeof(blk_iq4_xs));
+        for (int ib = 0; ib < 8; ib++) {
+            scales[ib] = iq4nl_block_scale(xs + ib * QK);
+            const float a = fabsf(scales[ib]);
+            if (a > amax_scale) { amax_scale = a; max_scale = scales[ib]; }
+        }
+        const float d = -max_scale / 32;
+        y[sb].d = orc_f32_to_f16(d);
+        const float id = d ? 1 / d : 0.f;
+        for (int ib = 0; ib < 8; ib++) {
+            int l = near_int(id * scales[ib]);
+            l = MAXI(-32, MINI(31, l));
+            const float dl = d * l;
+            iq4nl_pack_block(xs + ib * QK, dl ? 1 / dl : 0.f, y[sb].qs + 16 * ib);
+            l += 32;
+            y[sb].scales_l[ib / 2] |= (uint8_t)((l & 0xF) << 4 * (ib % 2));
+            y[sb].scales_h |= (uint16_t)((l >> 4) << 2 * ib);
+        }
+    }
+}
+static void dequant_iq4_xs(const blk_iq4_xs *x, float *y, int64_t k) {
+    for (int64_t sb = 0; sb < k / QKK; sb++) {
+        const float d = orc_f16_to_f32(x[sb].d);
+        for (int ib = 0; ib < 8; ib++) {
+            const float dl = d * (iq4xs_ls(&x[sb], ib) - 32);
+            const uint8_t *qs = x[sb].qs + 16 * ib;
+            for (int j = 0; j < 16; j++) {
+                y[sb * QKK + ib * QK + j] = dl * iq4nl_values[qs[j] & 0x0F];
+                y[sb * QKK + ib * QK + j + 16] = dl * iq4nl_values[qs[j] >> 4];
+            }
         }
     }
 }
@@ -759,6 +804,7 @@ static int quantize_row(int type, const float *x, void *y, int64_t k) {
         case ORC_Q5_0: quant_q5_0(x, (blk_q5_0 *)y, k); return 0;
         case ORC_Q5_1: quant_q5_1(x, (blk_q5_1 *)y, k); return 0;
         case ORC_IQ4_NL: quant_iq4_nl(x, (blk_iq4_nl *)y, k); return 0;
+        case ORC_IQ4_XS: quant_iq4_xs(x, (blk_iq4_xs *)y, k); return 0;
         case ORC_Q8_0: quant_q8_0(x, (blk_q8_0 *)y, k); return 0;
         case ORC_Q8_1: quant_q8_1(x, (blk_q8_1 *)y, k); return 0;
         case ORC_Q4_K: quant_q4_K(x, (blk_q4_K *)y, k); return 0;
@@ -777,6 +823,7 @@ static int dequantize_row(int type, const void *x, float *y, int64_t k) {
         case ORC_Q5_0: dequant_q5_0((const blk_q5_0 *)x, y, k); return 0;
         case ORC_Q5_1: dequant_q5_1((const blk_q5_1 *)x, y, k); return 0;
         case ORC_IQ4_NL: dequant_iq4_nl((const blk_iq4_nl *)x, y, k); return 0;
+        case ORC_IQ4_XS: dequant_iq4_xs((const blk_iq4_xs *)x, y, k); return 0;
         case ORC_Q8_0: dequant_q8_0((const blk_q8_0 *)x, y, k); return 0;
         case ORC_Q8_1: dequant_q8_1((const blk_q8_1 *)x, y, k); return 0;
         case ORC_Q4_K: dequant_q4_K((const blk_q4_K *)x, y, k); return 0;
@@ -826,6 +873,11 @@ static int weight_level(int type, const void *row, int64_t e) {
             const int j = (int)(e % QK);
             return iq4nl_values[j < 16 ? (b->qs[j] & 0x0F) : (b->qs[j - 16] >> 4)];
         }
+        case ORC_IQ4_XS: {
+            const blk_iq4_xs *b = (const blk_iq4_xs *)row + e / QKK;
+            const int ib = (int)(e % QKK) / QK, j = (int)(e % QK);
+            return iq4nl_values[j < 16 ? (b->qs[16 * ib + j] & 0x0F) : (b->qs[16 * ib + j - 16] >> 4)];
+        }
         case ORC_Q8_0: return ((const blk_q8_0 *)row + e / QK)->qs[e % QK];
         case ORC_Q4_K: return q4k_level((const blk_q4_K *)row + e / QKK, (int)(e % QKK));
         case ORC_Q5_K: return q5k_level((const blk_q5_K *)row + e / QKK, (int)(e % QKK));
@@ -837,7 +889,7 @@ static int granule(int type) { return type == ORC_Q6_K ? 16 : 32; }
 static int is_weight_type(int type) {
     switch (type) {
         case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_IQ4_NL: case ORC_Q8_0:
-        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 1;
+        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_IQ4_XS: return 1;
         default: return 0;
     }
 }
@@ -993,12 +1045,31 @@ static float dot_q6_K_q8_K(const blk_q6_K *w, const blk_q8_K *a, int64_t k) {   
     return sumf;
 }
 
+static float dot_iq4_xs_q8_K(const blk_iq4_xs *w, const blk_q8_K *a, int64_t k) {   /* ggml-cpu-quants.c:11381 ff., scalar tail :11647-11676 */
+    float sumf = 0;
+    for (int64_t sb = 0; sb < k / QKK; sb++) {
+        const float d4d8 = orc_f16_to_f32(w[sb].d) * a[sb].d;
+        for (int ib = 0; ib < 8; ib++) {
+            const float dl = d4d8 * (iq4xs_ls(&w[sb], ib) - 32);
+            const uint8_t *qs = w[sb].qs + 16 * ib;
+            const int8_t *q8 = a[sb].qs + 32 * ib;
+            int sumi1 = 0, sumi2 = 0;
+            for (int j = 0; j < 16; j++) {
+                sumi1 += q8[j] * iq4nl_values[qs[j] & 0x0F];
+                sumi2 += q8[j + 16] * iq4nl_values[qs[j] >> 4];
+            }
+            sumf += dl * (sumi1 + sumi2);
+        }
+    }
+    return sumf;
+}
+
 int orc_mul_mat_cpu(int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B) {
     int atype;
     switch (type) {
         case ORC_Q4_0: case ORC_Q5_0: case ORC_IQ4_NL: case ORC_Q8_0: atype = ORC_Q8_0; break;
         case ORC_Q4_1: case ORC_Q5_1: atype = ORC_Q8_1; break;    /* vec_dot_type, ggml-cpu.c:274-296, 384-389 */
-        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: atype = ORC_Q8_K; break;
+        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_IQ4_XS: atype = ORC_Q8_K; break;   /* :390-395 for IQ4_XS */
         default: return -1;
     }
     if (K % orc_block_elems(type)) return -1;
@@ -1019,6 +1090,7 @@ int orc_mul_mat_cpu(int type, const void *W, const float *x, float *dst, int64_t
                 case ORC_Q8_0: r = dot_q8_0_q8_0((const blk_q8_0 *)row, (const blk_q8_0 *)act, K); break;
                 case ORC_Q4_K: r = dot_q4_K_q8_K((const blk_q4_K *)row, (const blk_q8_K *)act, K); break;
                 case ORC_Q5_K: r = dot_q5_K_q8_K((const blk_q5_K *)row, (const blk_q8_K *)act, K); break;
+                case ORC_IQ4_XS: r = dot_iq4_xs_q8_K((const blk_iq4_xs *)row, (const blk_q8_K *)act, K); break;
                 default:       r = dot_q6_K_q8_K((const blk_q6_K *)row, (const blk_q8_K *)act, K); break;
             }
             dst[b * N + n] = r;
@@ -1051,6 +1123,11 @@ static double row_dot_q8_1(int type, const void *row, const blk_q8_1 *act, int64
                 for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
                 const uint16_t dh = type == ORC_Q5_0 ? ((const blk_q5_0 *)row)[b].d : ((const blk_iq4_nl *)row)[b].d;
                 acc += (double)orc_f16_to_f32(dh) * dx * isum;
+            } break;
+            case ORC_IQ4_XS: {
+                const blk_iq4_xs *w = (const blk_iq4_xs *)row + b / 8;
+                for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];
+                acc += (double)orc_f16_to_f32(w->d) * (iq4xs_ls(w, (int)(b % 8)) - 32) * dx * isum;
             } break;
             case ORC_Q4_1: case ORC_Q5_1: {     /* value = d * level + m */
                 for (int j = 0; j < QK; j++) isum += weight_level(type, row, b * QK + j) * act[b].qs[j];

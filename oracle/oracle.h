@@ -30,6 +30,7 @@ enum orc_type {
     ORC_Q6_K = 14,
     ORC_Q8_K = 15,
     ORC_IQ4_NL = 20,
+    ORC_IQ4_XS = 23,
 };
 
 /* IEEE binary16 <-> binary32, round to nearest even */

@@ -14,11 +14,11 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 F32, F16, Q4_0, Q8_0, Q8_1, Q4_K, Q5_K, Q6_K, Q8_K, I32 = 0, 1, 2, 8, 9, 12, 13, 14, 15, 26
-Q4_1, Q5_0, Q5_1, IQ4_NL = 3, 6, 7, 20
+Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS = 3, 6, 7, 20, 23
 WEIGHT_TYPES = {"q4_0": Q4_0, "q8_0": Q8_0, "q4_K": Q4_K, "q5_K": Q5_K, "q6_K": Q6_K, "q4_1": Q4_1, "q5_0": Q5_0, "q5_1": Q5_1,
-                "iq4_nl": IQ4_NL}
+                "iq4_nl": IQ4_NL, "iq4_xs": IQ4_XS}
 BLOCK = {F32: (1, 4), F16: (1, 2), Q4_0: (32, 18), Q8_0: (32, 34), Q8_1: (32, 36), Q4_K: (256, 144), Q5_K: (256, 176),
-         Q6_K: (256, 210), Q8_K: (256, 292), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), IQ4_NL: (32, 18)}
+         Q6_K: (256, 210), Q8_K: (256, 292), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), IQ4_NL: (32, 18), IQ4_XS: (256, 136)}
 
 _p = C.c_void_p
 _i64 = C.c_int64

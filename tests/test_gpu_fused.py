@@ -161,7 +161,9 @@ def test_rope_kv_store_quantized_caches(dev, ck, cv, device_rows, D):
 @pytest.mark.parametrize("B", [1, 3, 8])
 @pytest.mark.parametrize("specs", [[(orc.Q4_K, 1024), (orc.Q4_K, 512), (orc.Q6_K, 256), (orc.Q8_0, 130)],
                                    [(orc.Q5_0, 1024), (orc.IQ4_NL, 512), (orc.Q5_1, 256), (orc.Q4_1, 130)],
-                                   [(orc.IQ4_NL, 2048), (orc.Q5_K, 640)]], ids=["k_quants_q8_0", "per_32_block_types", "iq4_nl_q5_K"])
+                                   [(orc.IQ4_NL, 2048), (orc.Q5_K, 640)],
+                                   [(orc.IQ4_XS, 1024), (orc.IQ4_XS, 130), (orc.Q5_K, 256)]],
+                         ids=["k_quants_q8_0", "per_32_block_types", "iq4_nl_q5_K", "iq4_xs_q5_K"])
 def test_multi_matrix_gemv_with_residual(dev, B, specs):
     import torch
     import mi355
@@ -222,7 +224,7 @@ def test_fused_layer_stack_matches_node_sequence(dev):
 
 @pytest.mark.parametrize("B", [1, 3])
 @pytest.mark.parametrize("tq,tk,tv", [(orc.Q4_K, orc.Q4_K, orc.Q6_K), (orc.Q4_0, orc.Q8_0, orc.Q4_0), (orc.Q5_0, orc.Q5_0, orc.Q5_1), (orc.IQ4_NL, orc.IQ4_NL, orc.Q5_K),
-                                      (orc.Q4_1, orc.Q4_1, orc.Q4_1)])
+                                      (orc.Q4_1, orc.Q4_1, orc.Q4_1), (orc.IQ4_XS, orc.IQ4_XS, orc.Q5_K)])
 def test_qkv_rope_store_equals_three_launch_sequence(dev, B, tq, tk, tv):
     """projections + rope + KV store in one launch give bit-identical q and cache contents"""
     import torch
@@ -346,7 +348,7 @@ def test_qkv_rope_quantized_store_equals_separate_copies(dev, B, norm, ck, cv, d
 @pytest.mark.parametrize("tg,tu,K,N", [(orc.Q4_K, orc.Q6_K, 2048, 1536),       # two types: groups of 8 rows, the last group of a 32-row block finishes it
                                        (orc.Q4_K, orc.Q4_K, 2048, 1536),       # one type: a group owns a 32-row block in both matrices
                                        (orc.Q6_K, orc.Q6_K, 2048, 96), (orc.Q8_0, orc.Q8_0, 1024, 160), (orc.Q4_0, orc.Q4_0, 8192, 64),
-                                       (orc.IQ4_NL, orc.IQ4_NL, 1024, 64), (orc.Q5_K, orc.Q5_K, 768, 32), (orc.Q5_1, orc.Q5_1, 4096, 64),
+                                       (orc.IQ4_NL, orc.IQ4_NL, 1024, 64), (orc.IQ4_XS, orc.IQ4_XS, 1024, 96), (orc.Q5_K, orc.Q5_K, 768, 32), (orc.Q5_1, orc.Q5_1, 4096, 64),
                                        (orc.Q4_K, orc.Q4_K, 16384, 32)])       # K beyond what the one-type launch keeps in LDS at 3 and 4 rows
 def test_tail_fused_launches_equal_separate_kernels(dev, B, tg, tu, K, N):
     """gate/up + swiglu + Q8_1 in one launch gives the bytes of the separate launches"""

@@ -101,11 +101,11 @@ def test_model_logits_q5_k_m(dev, tmp_path, n_prompt):
     assert orc.nmse(dev_out, cpu) < 2e-3
 
 
-@pytest.mark.parametrize("ftype", ["q4_1", "q5_0", "q5_1", "iq4_nl"])
+@pytest.mark.parametrize("ftype", ["q4_1", "q5_0", "q5_1", "iq4_nl", "iq4_xs"])
 @pytest.mark.parametrize("n_prompt", [5, 40])
 def test_model_logits_per_32_block_types(dev, tmp_path, ftype, n_prompt):
-    """Files of the per-32-block types beyond Q4_0 / Q8_0 (Q4_1, Q5_0, Q5_1, IQ4_NL with the Q5_K / Q6_K tensors llama-quantize
-    mixes in): the reference's runtime on the plug-in reproduces its CPU backend's logits, so their MUL_MAT (the GEMV launches of
+    """Files of the per-32-block types beyond Q4_0 / Q8_0 (Q4_1, Q5_0, Q5_1, IQ4_NL, and IQ4_XS whose blocks sit eight to a super-block,
+    with the Q5_K / Q6_K tensors llama-quantize mixes in): the reference's runtime on the plug-in reproduces its CPU backend's logits, so their MUL_MAT (the GEMV launches of
     decode, the per-32-block tile kernel for a prompt) and GET_ROWS stay on the device with the reference's arithmetic."""
     if not (os.path.exists(LOGITS) and os.path.exists(PLUGIN)):
         pytest.skip("llama_logits or the plug-in is not built (needs the llama.cpp tree at build time)")

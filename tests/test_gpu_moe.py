@@ -92,7 +92,8 @@ def test_combine_equals_separate_nodes(dev, n_embd, n_used, T, residual):
     assert orc.nmse(out2.cpu().numpy(), want.cpu().numpy()) < 1e-7
 
 
-@pytest.mark.parametrize("name,t", [("q4_K", orc.Q4_K), ("q6_K", orc.Q6_K), ("q5_K", orc.Q5_K), ("q8_0", orc.Q8_0), ("q4_0", orc.Q4_0), ("iq4_nl", orc.IQ4_NL)])
+@pytest.mark.parametrize("name,t", [("q4_K", orc.Q4_K), ("q6_K", orc.Q6_K), ("q5_K", orc.Q5_K), ("q8_0", orc.Q8_0), ("q4_0", orc.Q4_0), ("iq4_nl", orc.IQ4_NL),
+                                    ("iq4_xs", orc.IQ4_XS)])
 @pytest.mark.parametrize("n_expert,n_used,T,N,K", [(8, 2, 1, 512, 4096), (8, 2, 3, 256, 2048), (4, 4, 2, 96, 1024)])
 def test_expert_gate_up_swiglu_equals_separate_launches(dev, name, t, n_expert, n_used, T, N, K):
     """MUL_MAT_ID(up), MUL_MAT_ID(gate), SILU, MUL and the Q8_1 rows for the down experts in one launch: the bits of

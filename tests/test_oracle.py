@@ -130,6 +130,10 @@ def _levels(t, W, K):
         bits = ((qh >> np.arange(32, dtype=np.uint32).reshape(1, 1, 32)) & 1).astype(np.int32)
         n = np.concatenate([(b & 15), (b >> 4)], axis=2).astype(np.int32) + 16 * bits
         return (n - (16 if t == orc.Q5_0 else 0)).reshape(N, K)
+    if t == orc.IQ4_XS:
+        b = W.reshape(N, K // 256, 136)[:, :, 8:].reshape(N, K // 32, 16)
+        n = np.concatenate([(b & 15), (b >> 4)], axis=2).astype(np.int32).reshape(N, K)
+        return np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.int32)[n]
     if t == orc.Q4_K:
         qs = W.reshape(N, K // 256, 144)[:, :, 16:].reshape(N, K // 256, 4, 32)
         return np.concatenate([(qs & 15), (qs >> 4)], axis=3).astype(np.int32).reshape(N, K)
