@@ -235,7 +235,7 @@ def sweep(kinds):
                 del Ws
     if "mmq" in kinds or "mmq_wide" in kinds:
         wide_only = "mmq" not in kinds    # the wide-tile GEMM alone on the gate/up shape (for counter collection)
-        for t in ((mi355.Q4_K, mi355.Q5_K, mi355.Q6_K) if wide_only else all_types):
+        for t in ((mi355.Q4_K, mi355.Q5_K, mi355.Q6_K, mi355.IQ4_XS) if wide_only else all_types):
             for N, K in ([(14336, 4096)] if wide_only else shapes):
                 for B in ((512,) if wide_only else (64, 512)):
                     nm = 4
@@ -251,7 +251,7 @@ def sweep(kinds):
                         label = "MUL_MAT batch %d (activation quantization + tile GEMM)" % B
                         emit(kernel=label, case="%s %dx%d" % (names[t], N, K), us=round(us, 2), bound="mfma",
                              achieved=round(ops / us / 1e6, 1), unit="TOP/s", frac=round(ops / us / 1e6 / INT8_PEAK_TOPS, 4), ops=ops)
-                    if t in (mi355.Q4_K, mi355.Q5_K, mi355.Q6_K):   # the wide-tile GEMM on tile images (what prefill uses for K-quants), without the quantization
+                    if t in (mi355.Q4_K, mi355.Q5_K, mi355.Q6_K, mi355.IQ4_XS):   # the wide-tile GEMM on tile images (what prefill uses for K-quants), without the quantization
                         tiles = [mi355.kq_unpack_tiles(t, W) for W in Ws]
                         a8 = mi355.quantize_act_q8k_tiled(x)
                         sws = torch.empty(int(lib.mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B)) + 256, dtype=torch.uint8, device=dev)

@@ -209,10 +209,11 @@ int mi355_mul_mat_q8k_planes_ws(void *stream, int type, const void *planes, cons
  *   weights:     mi355_kq_unpack_tiles - the two int8 planes of mi355_kq_unpack_planes (dequantize_row_q4_K / _q6_K,
  *                ggml/src/ggml-quants.c:1280-1302, 1690-1719) plus per-super-block d, dmin and mins, written once per
  *                weight matrix, mi355_kq_tiles_bytes(type, rows, K) bytes (about 2 bytes per weight).  Also Q5_K
- *                (dequantize_row_q5_K, :1482-1507): sub-block scale times level 0..31 = 16 * hi + lo.
+ *                (dequantize_row_q5_K, :1482-1507): sub-block scale times level 0..31 = 16 * hi + lo; and IQ4_XS
+ *                (dequantize_row_iq4_xs, :2454-2475): (ls - 32) times the table value = 64 * hi + lo, no minima (the Q6_K form).
  * mi355_mul_mat_q8k_tiled computes what mi355_mul_mat_q8k_add computes (same integer sums: ggml_vec_dot_q4_K_q8_K /
  * ggml_vec_dot_q6_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6817-6848, 8262-8283; f32 summation order may differ), and for
- * Q5_K the integer sums of ggml_vec_dot_q5_K_q8_K (:7539-7592).
+ * Q5_K / IQ4_XS the integer sums of ggml_vec_dot_q5_K_q8_K (:7539-7592) / ggml_vec_dot_iq4_xs_q8_K (:11381 ff.).
  * ws: optional workspace of mi355_mul_mat_q8k_tiled_ws_bytes(N, K, B) bytes for the split along K of products with few
  * tiles (NULL or too small: unsplit).  No counterpart in the reference (its CUDA backend unpacks in the tile loaders,
  * ggml/src/ggml-cuda/mmq.cuh). */

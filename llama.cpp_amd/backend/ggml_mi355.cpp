@@ -55,6 +55,12 @@ bool is_repacked_type(ggml_type t) {
            t == GGML_TYPE_IQ4_NL || t == GGML_TYPE_IQ4_XS;
 }
 bool is_weight_type(ggml_type t) { return is_repacked_type(t) || t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K; }
+// types whose matrices can get tile images for the wide-tile GEMM (mi355_kq_unpack_tiles)
+bool has_tile_images(ggml_type t) { return t == GGML_TYPE_Q4_K || t == GGML_TYPE_Q5_K || t == GGML_TYPE_Q6_K || t == GGML_TYPE_IQ4_XS; }
+// ... and those among them with no super-block tile kernel on packed rows: without images they take the per-32-block kernels
+bool tiles_or_generic(ggml_type t) { return t == GGML_TYPE_Q5_K || t == GGML_TYPE_IQ4_XS; }
+// rows of K elements are 16-byte multiples in the device layout when K is a multiple of this (256 for the other types)
+int64_t aligned_row_elems(ggml_type t) { return t == GGML_TYPE_Q6_K ? 2048 : t == GGML_TYPE_IQ4_XS ? 512 : 256; }
 
 int to_mi355_type(ggml_type t) {
     switch (t) {
@@ -363,7 +369,7 @@ struct tile_store {
     bool enabled = getenv("MI355_NO_TILES") == nullptr;
 
     const void * get(hipStream_t s, const ggml_tensor * w) {
-        if (!enabled || (w->type != GGML_TYPE_Q4_K && w->type != GGML_TYPE_Q5_K && w->type != GGML_TYPE_Q6_K) || w->buffer == nullptr ||
+        if (!enabled || !has_tile_images(w->type) || w->buffer == nullptr ||
             w->buffer->usage != GGML_BACKEND_BUFFER_USAGE_WEIGHTS)
             return nullptr;
         std::lock_guard<std::mutex> lock(mu);
@@ -451,7 +457,7 @@ void buffer_set_tensor(ggml_backend_buffer_t buffer, ggml_tensor * tensor, const
     buffer_ctx * ctx = (buffer_ctx *) buffer->context;
     MI355_HIP_OK(hipSetDevice(ctx->device));
     if (size == 0) return;
-    if (tensor->type == GGML_TYPE_Q6_K || tensor->type == GGML_TYPE_Q4_K || tensor->type == GGML_TYPE_Q5_K) {
+    if (has_tile_images(tensor->type)) {
         MI355_HIP_OK(hipDeviceSynchronize());
         planes().drop(tensor->data, ggml_nbytes(tensor));   // rebuilt from the new contents on next use
         tiles().drop(tensor->data, ggml_nbytes(tensor));
@@ -506,7 +512,7 @@ bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const ggml_tensor * src, gg
     MI355_HIP_OK(hipSetDevice(ctx->device));
     MI355_HIP_OK(hipDeviceSynchronize());
     if (dst->type == GGML_TYPE_Q6_K) planes().drop(dst->data, ggml_nbytes(dst));
-    if (dst->type == GGML_TYPE_Q6_K || dst->type == GGML_TYPE_Q4_K || dst->type == GGML_TYPE_Q5_K) tiles().drop(dst->data, ggml_nbytes(dst));
+    if (has_tile_images(dst->type)) tiles().drop(dst->data, ggml_nbytes(dst));
     MI355_HIP_OK(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyDeviceToDevice));
     MI355_HIP_OK(hipDeviceSynchronize());
     return true;
@@ -1125,19 +1131,18 @@ bool is_quant_gemv_candidate(const ggml_tensor * mm) {
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
     if (b->ne[1] > 32 || b->nb[1] != b->ne[0] * sizeof(float)) return false;
     const int64_t K = a->ne[0];
-    if (K % 256 != 0) return false;                                   // every type's rows are 16-byte multiples then ...
-    if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;     // ... except Q6_K (210-byte blocks)
+    if (K % 256 != 0 || K % aligned_row_elems(a->type) != 0) return false;   // rows that are 16-byte multiples (Q6_K: 210-byte, IQ4_XS: 136-byte blocks)
     return ((uintptr_t) a->data & 15) == 0 && ((uintptr_t) b->data & 15) == 0;
 }
 
 bool is_q8k_tile_candidate(const ggml_tensor * mm) {
     const ggml_tensor * a = mm->src[0];
     const ggml_tensor * b = mm->src[1];
-    if (mm->op != GGML_OP_MUL_MAT || (a->type != GGML_TYPE_Q4_K && a->type != GGML_TYPE_Q5_K && a->type != GGML_TYPE_Q6_K)) return false;
+    if (mm->op != GGML_OP_MUL_MAT || !has_tile_images(a->type)) return false;
     if (a->ne[2] != 1 || a->ne[3] != 1 || b->ne[2] != 1 || b->ne[3] != 1) return false;
     if (b->ne[1] <= 32 || b->nb[1] % 16 != 0) return false;
     const int64_t K = a->ne[0];
-    if (a->type == GGML_TYPE_Q6_K && K % 2048 != 0) return false;
+    if (K % aligned_row_elems(a->type) != 0) return false;
     return ((uintptr_t) a->data & 15) == 0 && ((uintptr_t) b->data & 15) == 0;
 }
 
@@ -2206,8 +2211,9 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
         return last;
     }
     // ---- runs of K-quant products on one activation (batch > 8): one per-super-block quantization
-    // (a Q5_K matrix without tile images - not in a weights buffer, or no memory for them - takes the generic path below)
-    if (is_q8k_tile_candidate(node) && !(node->src[0]->type == GGML_TYPE_Q5_K && q8k_format_for(s, node) != ACT_Q8KT)) {
+    // (a Q5_K or IQ4_XS matrix without tile images - not in a weights buffer, no memory for them, or a batch below the images'
+    // threshold - takes the generic path below)
+    if (is_q8k_tile_candidate(node) && !(tiles_or_generic(node->src[0]->type) && q8k_format_for(s, node) != ACT_Q8KT)) {
         const ggml_tensor * b = node->src[1];
         const int64_t K = b->ne[0], B = b->ne[1];
         // MUL_MAT(gate) -> UNARY(SILU) -> MUL_MAT(up) -> MUL: the up product goes out with the gate product (it reads the same

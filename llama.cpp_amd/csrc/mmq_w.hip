@@ -64,6 +64,20 @@ __device__ __forceinline__ void wt_q6k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
     lo = le | (lo_ << 8);
 }
 
+// IQ4_XS: the four table values (int8) in the bytes of `a` times the block scale -32..31 -> P = 64 * hi + lo, hi -64..63, lo 0..63:
+// the Q6_K form
+__device__ __forceinline__ void wt_iq4xs_planes(u32 a, int sc, u32 &hi, u32 &lo) {
+    const wt_i16x2 s = {(short)sc, (short)sc};
+    const wt_i16x2 eight = {8, 8}, six = {6, 6};
+    const wt_i16x2 e = (__builtin_bit_cast(wt_i16x2, a << 8) & (wt_i16x2){(short)0xFF00, (short)0xFF00}) >> eight;   // sign-extended even bytes
+    const wt_i16x2 o = (__builtin_bit_cast(wt_i16x2, a) & (wt_i16x2){(short)0xFF00, (short)0xFF00}) >> eight;        // ... odd bytes
+    const wt_i16x2 pe = e * s, po = o * s;
+    const u32 he = __builtin_bit_cast(u32, pe >> six), ho = __builtin_bit_cast(u32, po >> six);
+    const u32 le = __builtin_bit_cast(u32, pe) & 0x003F003Fu, lo_ = __builtin_bit_cast(u32, po) & 0x003F003Fu;
+    hi = (he & 0x00FF00FFu) | ((ho & 0x00FF00FFu) << 8);
+    lo = le | (lo_ << 8);
+}
+
 // Q5_K: the four levels 0..31 in the bytes of `a` times the sub-block scale 0..63 -> P = 16 * hi + lo with hi <= 122, lo <= 15
 __device__ __forceinline__ void wt_q5k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
     const wt_u16x2 s = {(unsigned short)sc, (unsigned short)sc};
@@ -76,6 +90,10 @@ __device__ __forceinline__ void wt_q5k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
     hi = (he & 0x00FF00FFu) | ((ho & 0x00FF00FFu) << 8);
     lo = le | (lo_ << 8);
 }
+
+// weight types with tile images: the K-quants of the Q4_K form (minima, radix 8 / 16) and those of the Q6_K form (signed levels
+// times signed scales, radix 64, no minima: Q6_K and IQ4_XS)
+static bool wt_has_images(int type) { return type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K || type == MI355_IQ4_XS; }
 
 template <int TYPE>
 __global__ void __launch_bounds__(256) k_unpack_tiles(const uint8_t *__restrict__ W, int8_t *__restrict__ img, int64_t N, int64_t K, row_layout L) {
@@ -172,6 +190,34 @@ __global__ void __launch_bounds__(256) k_unpack_tiles(const uint8_t *__restrict_
             *(f16x8 *)(e + r * 32 + 16) = m64;
             *(float *)(e + 512 + r * 4) = live ? half_bits_to_float((unsigned short)(hdr[0] & 0xFFFFu)) : 0.0f;
             *(float *)(e + 576 + r * 4) = live ? half_bits_to_float((unsigned short)(hdr[0] >> 16)) : 0.0f;
+        }
+    } else if constexpr (TYPE == MI355_IQ4_XS) {
+        // block ib = 4 half + p of the super-block (block_iq4_xs, ggml/src/ggml-common.h:406-412): byte l of its 16 holds the table
+        // index of element l in the low nibble and of element 16 + l in the high one; value = d * (ls - 32) * table[index]
+        const int ib = half * 4 + p;
+        const u32x4 q = load16(wrow + sb * 128 + ib * 16);
+        const uint2 h = *(const uint2 *)(wrow + L.off_b + sb * 8);
+        const int ls = (int)(((h.y >> (4 * ib)) & 0xFu) | (((h.x >> (16 + 2 * ib)) & 3u) << 4)) - 32;
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                u32 hi, lo;
+                wt_iq4xs_planes(iq4nl_lookup4(q[i] & 0x0F0F0F0Fu), ls, hi, lo);
+                a1[i] = hi; a0[i] = lo;
+                wt_iq4xs_planes(iq4nl_lookup4((q[i] >> 4) & 0x0F0F0F0Fu), ls, hi, lo);
+                b1[i] = hi; b0[i] = lo;
+            }
+        }
+        c0 = 2 * p;
+        c1 = c0 + 1;
+        if (half == 0 && p == 0) {   // the Q4_K entry with no minima
+            uint8_t *e = aux + (sb * n_rb_pad + (row >> 4)) * W_AUX;
+            const int r = (int)(row & 15);
+            const u32x4 z = {0, 0, 0, 0};
+            *(u32x4 *)(e + r * 32) = z;
+            *(u32x4 *)(e + r * 32 + 16) = z;
+            *(float *)(e + 512 + r * 4) = live ? half_bits_to_float((unsigned short)(h.x & 0xFFFFu)) : 0.0f;
+            *(float *)(e + 576 + r * 4) = 0.0f;
         }
     } else {
         const int l0 = 16 * (p & 1), qa = p >> 1;
@@ -757,12 +803,12 @@ int mi355_quantize_act_q8k_tiled(void *stream, const float *x, void *act, int64_
 }
 
 size_t mi355_kq_tiles_bytes(int type, int64_t rows, int64_t K) {
-    if (rows <= 0 || K <= 0 || K % QKK != 0 || (type != MI355_Q4_K && type != MI355_Q5_K && type != MI355_Q6_K)) return 0;
+    if (rows <= 0 || K <= 0 || K % QKK != 0 || !wt_has_images(type)) return 0;
     return wt_weight_bytes(type, rows, K);
 }
 
 int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, int64_t rows, int64_t K) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K, "kq_unpack_tiles: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(wt_has_images(type), "kq_unpack_tiles: weight type %d has no tile images", type);
     MI355_REQUIRE(rows > 0 && K > 0 && K % QKK == 0, "kq_unpack_tiles: bad shape rows=%lld K=%lld", (long long)rows, (long long)K);
     const row_layout L = make_row_layout(type, K);
     MI355_REQUIRE(layout_aligned(W, L) && ((uintptr_t)tiles & 15) == 0, "kq_unpack_tiles: rows are not 16-byte aligned (K=%lld)", (long long)K);
@@ -771,6 +817,7 @@ int mi355_kq_unpack_tiles(void *stream, int type, const void *W, void *tiles, in
     const dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
     if (type == MI355_Q4_K) MI355_LAUNCH(k_unpack_tiles<MI355_Q4_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
     else if (type == MI355_Q5_K) MI355_LAUNCH(k_unpack_tiles<MI355_Q5_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
+    else if (type == MI355_IQ4_XS) MI355_LAUNCH(k_unpack_tiles<MI355_IQ4_XS>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
     else MI355_LAUNCH(k_unpack_tiles<MI355_Q6_K>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)W, (int8_t *)tiles, rows, K, L);
     return launch_status("k_unpack_tiles");
 }
@@ -859,8 +906,8 @@ static int mul_mat_q8k_tiled_launch(void *stream, const int *types, int n_mats, 
     MI355_REQUIRE(n_mats >= 1 && n_mats <= 3 && mats != nullptr, "mul_mat_q8k_tiled: 1 to 3 matrices per launch, got %d", n_mats);
     bool all_q6 = true;
     for (int i = 0; i < n_mats; i++) {
-        MI355_REQUIRE(types[i] == MI355_Q4_K || types[i] == MI355_Q5_K || types[i] == MI355_Q6_K, "mul_mat_q8k_tiled: weight type %d is not a K-quant", types[i]);
-        all_q6 = all_q6 && types[i] == MI355_Q6_K;
+        MI355_REQUIRE(wt_has_images(types[i]), "mul_mat_q8k_tiled: weight type %d has no tile images", types[i]);
+        all_q6 = all_q6 && wt_radix_shift(types[i]) == 6;   // Q6_K, IQ4_XS: radix 64 and no minima
     }
     MI355_REQUIRE(K > 0 && B > 0 && K % QKK == 0, "mul_mat_q8k_tiled: bad shape K=%lld B=%lld (K must be a multiple of 256)", (long long)K, (long long)B);
     MI355_REQUIRE(act != nullptr && ((uintptr_t)act & 15) == 0, "mul_mat_q8k_tiled: the activation image is not 16-byte aligned");
@@ -968,7 +1015,7 @@ size_t mi355_mul_mat_id_q8k_tiled_ws_bytes(int64_t K, int64_t n_expert, int64_t 
 int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles, size_t expert_tiles_bytes, const float *b, const int32_t *ids,
                                int64_t ids_stride, float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T,
                                void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K, "mul_mat_id_q8k_tiled: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(wt_has_images(type), "mul_mat_id_q8k_tiled: weight type %d has no tile images", type);
     MI355_REQUIRE(N > 0 && K > 0 && n_expert > 0 && n_expert <= 256 && n_used > 0 && nb1 > 0 && T > 0 && K % QKK == 0, "mul_mat_id_q8k_tiled: bad shape");
     MI355_REQUIRE(ids_stride >= n_used && T * n_used < (1 << 24) && nb1 * T < (1 << 24), "mul_mat_id_q8k_tiled: bad ids stride or too many slots");
     MI355_REQUIRE(expert_tiles != nullptr && ((uintptr_t)expert_tiles & 15) == 0 && expert_tiles_bytes % 16 == 0 && expert_tiles_bytes >= wt_weight_bytes(type, N, K),
@@ -1006,7 +1053,7 @@ int mi355_mul_mat_id_q8k_tiled(void *stream, int type, const void *expert_tiles,
     L.n_tiles_padded = (L.n_tiles + 7) & ~7;
     const wt_route rt = {dst_row, tiles, n_tiles, (int64_t)expert_tiles_bytes};
     const dim3 grid((unsigned)L.n_tiles_padded);
-    if (type == MI355_Q6_K) MI355_LAUNCH((k_mmq_w<MI355_Q6_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
+    if (wt_radix_shift(type) == 6) MI355_LAUNCH((k_mmq_w<MI355_Q6_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
     else MI355_LAUNCH((k_mmq_w<MI355_Q4_K, true>), grid, dim3(512), 0, s, L, (const int8_t *)img, K, B_img, rt);
     return launch_status("k_mmq_w (routed)");
 }

@@ -291,7 +291,7 @@ def quantize_act_q8k_tiled(x):
 
 
 def kq_unpack_tiles(t, W):
-    """W: device-layout uint8 [N, row_bytes] (Q4_K / Q6_K) -> tile images of its two int8 planes + per-super-block scales"""
+    """W: device-layout uint8 [N, row_bytes] (Q4_K / Q5_K / Q6_K / IQ4_XS) -> tile images of its two int8 planes + per-super-block scales"""
     import torch
     N, rb = W.shape
     K = rb // BLOCK[t][1] * BLOCK[t][0]

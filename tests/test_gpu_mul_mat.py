@@ -347,7 +347,7 @@ def test_unaligned_rows_fallback(dev, name, t):
 
 
 KQ_TYPES = [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q6_K)]
-TILED_TYPES = [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q5_K, orc.Q6_K)]   # types with tile images for the wide-tile GEMM
+TILED_TYPES = [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q5_K, orc.Q6_K, orc.IQ4_XS)]   # types with tile images for the wide-tile GEMM
 
 
 def _tile_off(row, k, K):
@@ -411,7 +411,7 @@ def test_mmq_tiled_matches_oracle(dev, name, t, N, K, B, split):
     assert orc.nmse(got[:Bt, :Nt], orc.mul_mat("cpu", t, Wq[:Nt], x[:Bt])) < 1e-9
     # the last rows and columns (partial tiles)
     assert orc.nmse(got[B - 5:, N - 7:], orc.mul_mat("cpu", t, Wq[N - 7:], x[B - 5:])) < 1e-9
-    if t != orc.Q5_K:   # the 64 x 128 tile kernel on packed rows does not unpack Q5_K
+    if t not in (orc.Q5_K, orc.IQ4_XS):   # the 64 x 128 tile kernel on packed rows unpacks Q4_K and Q6_K only
         old = torch.empty((B, N), dtype=torch.float32, device=dev)
         a2 = mi355.quantize_act_q8k(_to_dev(dev, x))
         mi355.check(mi355.load().mi355_mul_mat_q8k(None, t, Wd.data_ptr(), a2.data_ptr(), old.data_ptr(), N, K, B, N))
@@ -462,7 +462,9 @@ def test_fused_producers_write_tile_images(dev, name, t):
 @pytest.mark.parametrize("types,Ns,K,B", [((orc.Q4_K, orc.Q4_K, orc.Q6_K), (4096, 1024, 1024), 4096, 512),   # Q, K, V of the Q4_K_M mix
                                           ((orc.Q6_K, orc.Q5_K, orc.Q4_K), (1000, 8300, 130), 2048, 300),    # ragged rows and batch
                                           ((orc.Q6_K, orc.Q4_K), (14336, 14336), 4096, 512),                  # 896 tiles
-                                          ((orc.Q6_K, orc.Q6_K), (520, 130), 2048, 200)])                      # Q6_K only: the form without a min term
+                                          ((orc.Q6_K, orc.Q6_K), (520, 130), 2048, 200),                       # Q6_K only: the form without a min term
+                                          ((orc.IQ4_XS, orc.IQ4_XS, orc.Q5_K), (1024, 260, 512), 2048, 300),  # Q, K, V of an IQ4_XS file
+                                          ((orc.IQ4_XS, orc.Q6_K), (520, 130), 2048, 200)])                    # both without minima
 def test_mmq_tiled_mixed_types(dev, types, Ns, K, B):
     """matrices of different K-quant types in one launch of the wide-tile GEMM: every matrix equals its own launch bit for bit, with
     and without a residual, and the oracle's integer arithmetic at the corners"""
