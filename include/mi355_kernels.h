@@ -156,7 +156,7 @@ size_t mi355_mul_mat_mid_ws_bytes(int64_t N, int64_t K, int64_t B);
 int mi355_mul_mat_mid(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K, int64_t B,
                       int64_t dst_stride, void *ws, size_t ws_bytes);
 
-/* K-quant (Q4_K, Q6_K) tile GEMM with the activation format ggml-cpu uses for these weight
+/* K-quant (Q4_K, Q6_K; Q5_K and IQ4_XS on the 64 x 128 form of the kernel) tile GEMM with the activation format ggml-cpu uses for these weight
  * types: one f32 scale per 256 elements (quantize_row_q8_K_ref, ggml/src/ggml-quants.c:2479-2516;
  * vec_dot_type of type_traits_cpu, ggml/src/ggml-cpu/ggml-cpu.c:252-417), so the integer
  * sub-scales fold into the int8 operands and the sums of a whole super-block stay integer
@@ -317,7 +317,7 @@ int mi355_mul_mat_id(void *stream, int type, const void *as, const float *b, con
                      float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T,
                      void *ws, size_t ws_bytes);
 
-/* mi355_mul_mat_id for many (token, expert slot) pairs and K-quant experts: the slots are sorted by expert on the
+/* mi355_mul_mat_id for many (token, expert slot) pairs and Q4_K / Q5_K / Q6_K / IQ4_XS experts: the slots are sorted by expert on the
  * device (the row grouping of ggml_compute_forward_mul_mat_id, ggml/src/ggml-cpu/ggml-cpu.c:7805-7820, mmid_row_mapping
  * :7639-7644) and one tile launch walks all experts, so every expert's matrix is read once.  `act` holds the nb1*T rows
  * of b in the mi355_quantize_act_q8k layout; route_ws: at least mi355_mul_mat_id_q8k_route_bytes(...) bytes, 16-byte

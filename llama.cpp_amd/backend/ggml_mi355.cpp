@@ -1183,7 +1183,7 @@ bool mmid_uses_tiles(const ggml_tensor * op) {
     const ggml_tensor * as = op->src[0];
     const int64_t K = as->ne[0], slots = op->src[2]->ne[0] * op->src[1]->ne[2];
     if (slots < 32 || as->ne[2] > 256 || K % 256 != 0 || ((uintptr_t) as->data & 15) != 0) return false;
-    return as->type == GGML_TYPE_Q4_K || (as->type == GGML_TYPE_Q6_K && K % 2048 == 0);
+    return has_tile_images(as->type) && K % aligned_row_elems(as->type) == 0;   // the types of the routed super-block tile kernel
 }
 
 // does the node after `i` (skipping views) route the rows of the tensor at `data` through quantized experts by GEMV?

@@ -127,6 +127,31 @@ __device__ __forceinline__ u32 mul_bytes(u32 x, u32 f) {
     return __builtin_bit_cast(u32, p);
 }
 
+// Q5_K: four levels 0..31 (bytes of a) times the sub-block scale 0..63 -> value = 16*hi + lo, hi <= 122, lo <= 15
+__device__ __forceinline__ void q5k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
+    const u16x2 s = {(unsigned short)sc, (unsigned short)sc};
+    const u16x2 e = __builtin_bit_cast(u16x2, a & 0x00FF00FFu);
+    const u16x2 o = __builtin_bit_cast(u16x2, (a >> 8) & 0x00FF00FFu);
+    const u16x2 pe = e * s, po = o * s;
+    const u16x2 four = {4, 4};
+    const u32 he = __builtin_bit_cast(u32, pe >> four), ho = __builtin_bit_cast(u32, po >> four);
+    const u32 le = __builtin_bit_cast(u32, pe) & 0x000F000Fu, lo_ = __builtin_bit_cast(u32, po) & 0x000F000Fu;
+    hi = (he & 0x00FF00FFu) | ((ho & 0x00FF00FFu) << 8);
+    lo = le | (lo_ << 8);
+}
+// IQ4_XS: four table values (int8 bytes of a) times the block scale -32..31 -> value = 64*hi + lo, hi -64..63, lo 0..63 (the Q6_K form)
+__device__ __forceinline__ void iq4xs_planes(u32 a, int sc, u32 &hi, u32 &lo) {
+    const i16x2 s = {(short)sc, (short)sc};
+    const i16x2 eight = {8, 8}, six = {6, 6};
+    const i16x2 e = __builtin_bit_cast(i16x2, a << 8) >> eight;   // sign-extended even bytes
+    const i16x2 o = __builtin_bit_cast(i16x2, a) >> eight;        // ... odd bytes
+    const i16x2 pe = e * s, po = o * s;
+    const u32 he = __builtin_bit_cast(u32, pe >> six), ho = __builtin_bit_cast(u32, po >> six);
+    const u32 le = __builtin_bit_cast(u32, pe) & 0x003F003Fu, lo_ = __builtin_bit_cast(u32, po) & 0x003F003Fu;
+    hi = (he & 0x00FF00FFu) | ((ho & 0x00FF00FFu) << 8);
+    lo = le | (lo_ << 8);
+}
+
 // Q6_K: four unsigned 6-bit levels (bytes of a) -> int8 planes of sc*(level-32): value = 64*hi + lo
 __device__ __forceinline__ void q6k_planes(u32 a, int sc, u32 &hi, u32 &lo) {
     const i16x2 s = {(short)sc, (short)sc};
@@ -387,14 +412,25 @@ __device__ __forceinline__ int kp_off(int row, int chunk) { return row * KP_ROW 
 template <int TYPE> struct kp_w;   // the 16-byte weight piece of one stage that this thread unpacks (row tid / 4, piece tid % 4)
 template <> struct kp_w<MI355_Q4_K> { u32x4 q; };
 template <> struct kp_w<MI355_Q6_K> { u32x4 ql, qh; int scA, scB; };
+template <> struct kp_w<MI355_Q5_K> { u32x4 q, qh; };
+template <> struct kp_w<MI355_IQ4_XS> { u32x4 q; int ls; };   // ls: the block's scale, -32..31
+// the two forms of the kernel: with a min term and an unsigned product (Q4_K, Q5_K) / signed products and no min term (Q6_K, IQ4_XS)
+template <int TYPE> struct kp_form {
+    static constexpr bool MIN = TYPE == MI355_Q4_K || TYPE == MI355_Q5_K;
+    static constexpr int RADIX_SHIFT = TYPE == MI355_Q4_K ? 3 : TYPE == MI355_Q5_K ? 4 : 6;
+};
 // per super-block data of this thread's weight row: the Q4_K block header (d, dmin, 12 scale bytes) / the Q6_K d
 template <int TYPE> struct kp_h;
 template <> struct kp_h<MI355_Q4_K> { u32x4 hdr; };
 template <> struct kp_h<MI355_Q6_K> { unsigned short d; };   // raw fp16 bits: converting at the load would wait for it
+template <> struct kp_h<MI355_Q5_K> { u32x4 hdr; };
+template <> struct kp_h<MI355_IQ4_XS> { unsigned short d; };
 
 template <int TYPE>
 __device__ __forceinline__ void kp_fetch_h(kp_h<TYPE> &H, const uint8_t *__restrict__ wrow, const row_layout &L, int64_t sb) {
     if constexpr (TYPE == MI355_Q4_K) H.hdr = load16(wrow + sb * Q4_K_BYTES);
+    else if constexpr (TYPE == MI355_Q5_K) H.hdr = load16(wrow + sb * Q5_K_BYTES);
+    else if constexpr (TYPE == MI355_IQ4_XS) H.d = *(const unsigned short *)(wrow + L.off_b + sb * 8);
     else H.d = *(const unsigned short *)(wrow + L.off_d + sb * 2);
 }
 
@@ -404,6 +440,15 @@ __device__ __forceinline__ void kp_fetch_w(kp_w<TYPE> &R, const uint8_t *__restr
     if constexpr (TYPE == MI355_Q4_K) {
         const uint8_t *blk = wrow + sb * Q4_K_BYTES;
         R.q = load16(blk + 16 + (half * 2 + (p >> 1)) * 32 + (p & 1) * 16);
+    } else if constexpr (TYPE == MI355_Q5_K) {   // the Q4_K geometry behind 32 bytes of fifth bits (bit j of qh[l]: sub-block j, level l)
+        const uint8_t *blk = wrow + sb * Q5_K_BYTES;
+        R.q = load16(blk + 48 + (half * 2 + (p >> 1)) * 32 + (p & 1) * 16);
+        R.qh = load16(blk + 16 + (p & 1) * 16);
+    } else if constexpr (TYPE == MI355_IQ4_XS) {   // block 4 half + p: 16 bytes of table indices, its six-bit scale from the header
+        const int ib = half * 4 + p;
+        R.q = load16(wrow + sb * 128 + ib * 16);
+        const uint2 h = *(const uint2 *)(wrow + L.off_b + sb * 8);
+        R.ls = (int)(((h.y >> (4 * ib)) & 0xFu) | (((h.x >> (16 + 2 * ib)) & 3u) << 4)) - 32;
     } else {
         const int l0 = 16 * (p & 1), qa = p >> 1;
         R.ql = load16(wrow + sb * 128 + half * 64 + p * 16);
@@ -431,6 +476,24 @@ __device__ __forceinline__ void kp_unpack(const kp_w<TYPE> &R, const kp_h<TYPE> 
         P.a0[i] = mul_bytes(nl, (u32)scl & 7u);
         P.b1[i] = mul_bytes(nh, (u32)sch >> 3);
         P.b0[i] = mul_bytes(nh, (u32)sch & 7u);
+    } else if constexpr (TYPE == MI355_Q5_K) {
+        const int g = half * 2 + (p >> 1);
+        int scl, mnl, sch, mnh;
+        q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], 2 * g, scl, mnl);
+        q4k_scale_min(H.hdr[1], H.hdr[2], H.hdr[3], 2 * g + 1, sch, mnh);
+        const u32 nl = (R.q[i] & 0x0F0F0F0Fu) | (((R.qh[i] >> (2 * g)) & 0x01010101u) << 4);
+        const u32 nh = ((R.q[i] >> 4) & 0x0F0F0F0Fu) | (((R.qh[i] >> (2 * g + 1)) & 0x01010101u) << 4);
+        u32 hi, lo;
+        q5k_planes(nl, scl, hi, lo);
+        P.a1[i] = hi; P.a0[i] = lo;
+        q5k_planes(nh, sch, hi, lo);
+        P.b1[i] = hi; P.b0[i] = lo;
+    } else if constexpr (TYPE == MI355_IQ4_XS) {
+        u32 hi, lo;
+        iq4xs_planes(iq4nl_lookup4(R.q[i] & 0x0F0F0F0Fu), R.ls, hi, lo);
+        P.a1[i] = hi; P.a0[i] = lo;
+        iq4xs_planes(iq4nl_lookup4((R.q[i] >> 4) & 0x0F0F0F0Fu), R.ls, hi, lo);
+        P.b1[i] = hi; P.b0[i] = lo;
     } else {
         const int qa = p >> 1;
         const u32 va = (R.ql[i] & 0x0F0F0F0Fu) | (((R.qh[i] >> (2 * qa)) & 0x03030303u) << 4);
@@ -447,8 +510,9 @@ template <int TYPE>
 __device__ __forceinline__ void kp_store(const kp_planes &P, int8_t *__restrict__ sW1, int8_t *__restrict__ sW0) {
     const int r = threadIdx.x >> 2, p = threadIdx.x & 3;
     // Q4_K: low nibbles are sub-block 2*gl, high nibbles sub-block 2*gl + 1 (32 bytes later); Q6_K: the second group is 64 bytes later
-    const int c0 = TYPE == MI355_Q4_K ? 4 * (p >> 1) + (p & 1) : 2 * (p >> 1) + (p & 1);
-    const int c1 = c0 + (TYPE == MI355_Q4_K ? 2 : 4);
+    // (Q5_K as Q4_K; IQ4_XS: the two halves of block p follow each other)
+    const int c0 = kp_form<TYPE>::MIN ? 4 * (p >> 1) + (p & 1) : TYPE == MI355_IQ4_XS ? 2 * p : 2 * (p >> 1) + (p & 1);
+    const int c1 = c0 + (kp_form<TYPE>::MIN ? 2 : TYPE == MI355_IQ4_XS ? 1 : 4);
     *(u32x4 *)(sW1 + kp_off(r, c0)) = P.a1;
     *(u32x4 *)(sW0 + kp_off(r, c0)) = P.a0;
     *(u32x4 *)(sW1 + kp_off(r, c1)) = P.b1;
@@ -478,8 +542,8 @@ __global__ void __launch_bounds__(256, 2) k_mmq_kp(const uint8_t *__restrict__ W
                                                    const _Float16 *__restrict__ abs_, float *dst, const float *residual,
                                                    int64_t N, int64_t K, int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles,
                                                    int n_groups, int n_groups_padded, mmq_route route) {
-    constexpr bool Q4 = TYPE == MI355_Q4_K;
-    constexpr int RADIX_SHIFT = Q4 ? 3 : 6;
+    constexpr bool Q4 = kp_form<TYPE>::MIN;   // the form with a min term (Q4_K, Q5_K)
+    constexpr int RADIX_SHIFT = kp_form<TYPE>::RADIX_SHIFT;
     constexpr int BM = 64, BN = 128;
     __shared__ __attribute__((aligned(16))) int8_t sW1a[BM * KP_ROW], sW1b[BM * KP_ROW];
     __shared__ __attribute__((aligned(16))) int8_t sW0a[BM * KP_ROW], sW0b[BM * KP_ROW];
@@ -1159,7 +1223,8 @@ template <int TYPE>
 static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int64_t act_rows, const int32_t *ids, int64_t ids_stride,
                             float *dst, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws) {
     const int64_t S = T * n_used;
-    const int bn = route_bn(n_expert, S);
+    constexpr bool BOTH = TYPE == MI355_Q4_K || TYPE == MI355_Q6_K;   // the types the 64-column kernel unpacks too
+    const int bn = BOTH ? route_bn(n_expert, S) : 128;
     const int max_tiles = (int)((S + bn - 1) / bn + n_expert);
     int32_t *act_row = (int32_t *)route_ws, *dst_row = act_row + S, *tiles = dst_row + S, *n_tiles = tiles + 4 * (int64_t)route_max_tiles(n_expert, S);
     MI355_LAUNCH(k_route_slots, dim3(1), dim3(1024), 0, s, ids, ids_stride, n_expert, n_used, nb1, T, bn, act_row, dst_row, tiles, n_tiles);
@@ -1171,11 +1236,14 @@ static void launch_mmq_k_id(hipStream_t s, const void *as, const void *act, int6
     const int n_groups = n_row_tiles * max_tiles;
     const int n_groups_padded = (n_groups + 7) & ~7;
     const mmq_route route = {act_row, dst_row, tiles, n_tiles, N * L.row_bytes};
-    if (bn == 64)
-        MI355_LAUNCH((k_mmq_k<TYPE, 1, 1, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
-                           dst, nullptr, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
-    else
-        MI355_LAUNCH((k_mmq_kp<TYPE, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_, dst, nullptr, N, K,
+    if constexpr (BOTH) {
+        if (bn == 64) {
+            MI355_LAUNCH((k_mmq_k<TYPE, 1, 1, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_,
+                               dst, nullptr, N, K, S, N, L, max_tiles, n_groups, n_groups_padded, route);
+            return;
+        }
+    }
+    MI355_LAUNCH((k_mmq_kp<TYPE, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ad8, abs_, dst, nullptr, N, K,
                            S, N, L, max_tiles, n_groups, n_groups_padded, route);
 }
 
@@ -1212,7 +1280,7 @@ size_t mi355_mul_mat_id_q8k_route_bytes(int64_t n_expert, int64_t n_used, int64_
 int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride, float *dst,
                          int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws,
                          size_t route_ws_bytes) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_id_q8k: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K || type == MI355_IQ4_XS, "mul_mat_id_q8k: weight type %d has no super-block tile kernel", type);
     MI355_REQUIRE(N > 0 && K > 0 && n_expert > 0 && n_used > 0 && nb1 > 0 && T > 0, "mul_mat_id_q8k: bad shape");
     MI355_REQUIRE(K % QKK == 0, "mul_mat_id_q8k: K=%lld is not a multiple of 256", (long long)K);
     MI355_REQUIRE(n_expert <= ROUTE_MAX_EXPERTS, "mul_mat_id_q8k: more than %d experts", ROUTE_MAX_EXPERTS);
@@ -1227,6 +1295,8 @@ int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act
     }
     hipStream_t s = (hipStream_t)stream;
     if (type == MI355_Q4_K) launch_mmq_k_id<MI355_Q4_K>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
+    else if (type == MI355_Q5_K) launch_mmq_k_id<MI355_Q5_K>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
+    else if (type == MI355_IQ4_XS) launch_mmq_k_id<MI355_IQ4_XS>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
     else launch_mmq_k_id<MI355_Q6_K>(s, as, act, nb1 * T, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws);
     return launch_status("k_mmq_k (routed)");
 }
@@ -1300,7 +1370,7 @@ int mi355_mul_mat_q8k_add(void *stream, int type, const void *W, const void *act
 
 int mi355_mul_mat_q8k_ws(void *stream, int type, const void *W, const void *act, float *dst, const float *residual, int64_t N, int64_t K,
                          int64_t B, int64_t dst_stride, void *ws, size_t ws_bytes) {
-    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q6_K, "mul_mat_q8k: weight type %d is not a K-quant", type);
+    MI355_REQUIRE(type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K || type == MI355_IQ4_XS, "mul_mat_q8k: weight type %d has no super-block tile kernel", type);
     MI355_REQUIRE(N > 0 && K > 0 && B > 0, "mul_mat_q8k: bad shape N=%lld K=%lld B=%lld", (long long)N, (long long)K, (long long)B);
     MI355_REQUIRE(K % QKK == 0, "mul_mat_q8k: K=%lld is not a multiple of 256", (long long)K);
     MI355_REQUIRE(dst_stride >= N, "mul_mat_q8k: dst_stride < N");
@@ -1311,6 +1381,8 @@ int mi355_mul_mat_q8k_ws(void *stream, int type, const void *W, const void *act,
     MI355_REQUIRE((N + 63) / 64 * ((B + 63) / 64) < (1 << 30), "mul_mat_q8k: too many tiles");
     hipStream_t s = (hipStream_t)stream;
     if (type == MI355_Q4_K) launch_mmq_k<MI355_Q4_K>(s, W, act, dst, residual, N, K, B, dst_stride, ws, ws_bytes);
+    else if (type == MI355_Q5_K) launch_mmq_k<MI355_Q5_K>(s, W, act, dst, residual, N, K, B, dst_stride, ws, ws_bytes);
+    else if (type == MI355_IQ4_XS) launch_mmq_k<MI355_IQ4_XS>(s, W, act, dst, residual, N, K, B, dst_stride, ws, ws_bytes);
     else launch_mmq_k<MI355_Q6_K>(s, W, act, dst, residual, N, K, B, dst_stride, ws, ws_bytes);
     return launch_status("k_mmq_k");
 }

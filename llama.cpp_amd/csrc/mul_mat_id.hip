@@ -13,7 +13,9 @@ extern "C" {
 static constexpr int64_t ROUTED_MIN_SLOTS = 32;   // measured cross-over on 8 experts of 14336 x 4096
 
 static bool use_routed_tiles(int type, const void *as, int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t T) {
-    if (T * n_used < ROUTED_MIN_SLOTS || n_expert > 256 || K % QKK != 0 || (type != MI355_Q4_K && type != MI355_Q6_K)) return false;
+    if (T * n_used < ROUTED_MIN_SLOTS || n_expert > 256 || K % QKK != 0 ||
+        (type != MI355_Q4_K && type != MI355_Q5_K && type != MI355_Q6_K && type != MI355_IQ4_XS))
+        return false;
     const row_layout L = make_row_layout(type, K);
     return layout_aligned(as, L) && (N * L.row_bytes) % 16 == 0;
 }

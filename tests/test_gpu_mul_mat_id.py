@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 def routed(t, n_used, T, K):
     """mi355_mul_mat_id sorts the slots by expert and uses the K-quant tile kernel (ggml-cpu's Q8_K arithmetic)"""
-    return T * n_used >= 32 and ((t == orc.Q4_K and K % 256 == 0) or (t == orc.Q6_K and K % 2048 == 0))
+    return T * n_used >= 32 and ((t in (orc.Q4_K, orc.Q5_K) and K % 256 == 0) or (t == orc.Q6_K and K % 2048 == 0) or (t == orc.IQ4_XS and K % 512 == 0))
 
 
 def expected_per_expert(kind, t, Wq, b, ids_full, n_expert, n_used, nb1, N):
@@ -57,7 +57,7 @@ def test_mul_mat_id(dev, name, t, n_expert, n_used, nb1_bcast, T, N, K):
         assert orc.nmse(got, cpu) <= 5e-4      # tests/test-backend-ops.cpp:2001
 
 
-@pytest.mark.parametrize("name,t", [("q4_k", orc.Q4_K), ("q6_k", orc.Q6_K)])
+@pytest.mark.parametrize("name,t", [("q4_k", orc.Q4_K), ("q6_k", orc.Q6_K), ("q5_k", orc.Q5_K), ("iq4_xs", orc.IQ4_XS)])
 @pytest.mark.parametrize("pattern", ["one_expert", "two_of_eight", "out_of_range"])
 def test_mul_mat_id_skewed_routing(dev, name, t, pattern):
     """experts with no slots, one expert with more slots than a column tile, ids outside [0, n_expert) clamped like the GEMV path"""
