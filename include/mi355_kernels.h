@@ -94,14 +94,15 @@ int mi355_quantize_act(void *stream, const float *x, void *act, int64_t k, int64
  * bandwidth-bound GEMV (per-block integer dots of the weights against Q8_1 activations), up to 32
  * the weight-streaming matrix-core kernel (mi355_mul_mat_skinny), larger B the int8-MFMA tile kernels.
  * Q5_K (block_q5_K, ggml/src/ggml-common.h:296-308; ggml_vec_dot_q5_K_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:6859-7592) has the
- * GEMV for up to 8 rows, the per-32-block int8-MFMA tile kernel (mi355_mul_mat_q) for batches on packed rows - what this entry
- * point runs - and the wide-tile GEMM on tile images (mi355_kq_unpack_tiles + mi355_mul_mat_q8k_tiled) for callers that keep images.
+ * GEMV for up to 8 rows, the super-block tile kernel on packed rows (mi355_mul_mat_q8k) for batches - what this entry
+ * point runs above 32 rows; the per-32-block kernel mi355_mul_mat_q takes it too - and the wide-tile GEMM on tile images (mi355_kq_unpack_tiles + mi355_mul_mat_q8k_tiled) for callers that keep images.
  * Q4_1, Q5_0, Q5_1 and IQ4_NL (ggml/src/ggml-common.h:168-201, 399-404; ggml_vec_dot_q4_1_q8_1, _q5_0_q8_0, _q5_1_q8_1 and
  * _iq4_nl_q8_0, ggml/src/ggml-cpu/ggml-cpu-quants.c:2511, 2804, 3159, 11188) have the GEMV for up to 8 rows (also in the
  * launches that take several matrices or fuse an epilogue) and the per-32-block int8-MFMA tile kernel (mi355_mul_mat_q) beyond;
  * the weight-streaming kernel for 5..32 rows serves them too.
  * IQ4_XS (block_iq4_xs, ggml/src/ggml-common.h:406-412; ggml_vec_dot_iq4_xs_q8_K, ggml/src/ggml-cpu/ggml-cpu-quants.c:11381) runs on the
- * same three kernels as IQ4_NL, its block scales d * (ls - 32) taken from the super-block headers.
+ * same three kernels as IQ4_NL, its block scales d * (ls - 32) taken from the super-block headers; from 256 rows on this entry point
+ * runs it on mi355_mul_mat_q8k, and it has tile images for mi355_mul_mat_q8k_tiled.
  * `ws` is scratch of at least mi355_mul_mat_ws_bytes(K, B) bytes. */
 size_t mi355_mul_mat_ws_bytes(int64_t K, int64_t B);
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,

@@ -91,8 +91,11 @@ static bool use_skinny(int type, const void *W, int64_t K, int64_t B) {
 // 33 to 128 activation rows on Q4_K: the weight-streaming matrix-core kernel with the sub-block scales folded into the operand (mid.hip)
 static bool use_mid(int type, const void *W, int64_t K, int64_t B) { return B > 32 && B <= 128 && mi355_mul_mat_mid_supported(type, W, K, B); }
 
+// the super-block tile kernel on packed rows and per-256 activation scales: Q4_K, Q6_K, Q5_K (its per-32-block kernel is 1.5x slower
+// at 512 rows, equal at 64), IQ4_XS from 256 rows on (below, the per-32-block kernel is ahead: 34 against 50 us at 64 rows of 14336 x 4096)
 static bool use_q8k_tiles(int type, const void *W, int64_t K, int64_t B) {
-    return B > 8 && !use_skinny(type, W, K, B) && !use_mid(type, W, K, B) && (type == MI355_Q4_K || type == MI355_Q6_K) && layout_aligned(W, make_row_layout(type, K));
+    const bool typed = type == MI355_Q4_K || type == MI355_Q6_K || type == MI355_Q5_K || (type == MI355_IQ4_XS && B >= 256);
+    return B > 8 && !use_skinny(type, W, K, B) && !use_mid(type, W, K, B) && typed && layout_aligned(W, make_row_layout(type, K));
 }
 
 int mi355_mul_mat(void *stream, int type, const void *W, const float *x, float *dst, int64_t N, int64_t K, int64_t B,

@@ -151,7 +151,8 @@ def test_mmq_matches_oracle(dev, name, t, N, K, B):
     got = mi355.mul_mat(t, Wd, _to_dev(dev, x)).cpu().numpy()
     Nt, Bt = min(N, 64), min(B, 24)
     skinny = B <= 32 and K % 256 == 0 and (t != orc.Q6_K or K % 2048 == 0)   # up to 32 activation rows: the weight-streaming kernel, Q8_1 activations
-    if B > 8 and not skinny and (t == orc.Q4_K or (t == orc.Q6_K and K % 2048 == 0)):   # Q6_K rows are 16-byte aligned only then
+    if B > 8 and not skinny and (t in (orc.Q4_K, orc.Q5_K) or (t == orc.Q6_K and K % 2048 == 0) or
+                                 (t == orc.IQ4_XS and B >= 256 and K % 512 == 0)):   # Q6_K / IQ4_XS rows are 16-byte aligned only then
         # K-quants take the activation format of the CPU path (one scale per 256): integer sums are the
         # CPU's own (ggml-cpu-quants.c:6817-6848, 8262-8283), only the f32 summation order differs
         want = orc.mul_mat("cpu", t, Wq[:Nt], x[:Bt])
@@ -285,13 +286,14 @@ def test_mmq_llama8b_ffn_shapes(dev, name, t, N, K):
     rng = np.random.default_rng(N + K + t)
     Wq = _weights(rng, t, N, K, "ref")
     Wd = mi355.upload_weights(t, _to_dev(dev, Wq))
-    kq = t in (orc.Q4_K, orc.Q6_K)
+    kq = t in (orc.Q4_K, orc.Q5_K, orc.Q6_K, orc.IQ4_XS)
     tiles = mi355.kq_unpack_tiles(t, Wd) if kq else None
     for B in (64, 512):
         x = rng.standard_normal((B, K)).astype(np.float32)
         xd = _to_dev(dev, x)
         got = mi355.mul_mat(t, Wd, xd).cpu().numpy()
-        kind = "cpu" if kq else "q8_1"          # K-quants compute in the CPU path's Q8_K format, the others in Q8_1
+        # K-quants (IQ4_XS from 256 rows on) compute in the CPU path's Q8_K format, the others in Q8_1
+        kind = "cpu" if (kq and (t != orc.IQ4_XS or B >= 256)) else "q8_1"
         corner = orc.mul_mat(kind, t, Wq[:64], x[:24])
         edge = orc.mul_mat(kind, t, Wq[N - 9:], x[B - 3:])
         tol = 1e-6 if t in (orc.Q4_1, orc.Q5_1, orc.Q5_K) else 1e-9    # the block minimum meets fp16(d_x * sum(q)), as in the reference's dot
@@ -303,10 +305,13 @@ def test_mmq_llama8b_ffn_shapes(dev, name, t, N, K):
         if kq:
             act = mi355.quantize_act_q8k_tiled(xd)
             wide = mi355.mul_mat_q8k_tiled(t, tiles, act, N, K, B).cpu().numpy()
-            assert orc.nmse(wide[:24, :64], corner) < 1e-9
-            assert orc.nmse(wide[B - 3:, N - 9:], edge) < 1e-9
             assert orc.nmse(wide, want) <= 5e-4
-            assert orc.nmse(wide, got) < 1e-12      # same integer sums in both tile kernels
+            if kind == "cpu":
+                assert orc.nmse(wide[:24, :64], corner) < 1e-9
+                assert orc.nmse(wide[B - 3:, N - 9:], edge) < 1e-9
+                assert orc.nmse(wide, got) < 1e-12      # same integer sums in both tile kernels
+            else:
+                assert orc.nmse(wide[:24, :64], orc.mul_mat("cpu", t, Wq[:64], x[:24])) < 1e-9
 
 
 @pytest.mark.parametrize("name,t", [(n, t) for n, t in TYPES if t in (orc.Q4_K, orc.Q6_K)])
@@ -341,7 +346,7 @@ def test_unaligned_rows_fallback(dev, name, t):
         got = mi355.mul_mat(t, Wd, _to_dev(dev, x)).cpu().numpy()
         # Q4_K rows are always aligned, so B > 32 takes the super-block tile kernel and the CPU's activation format
         # (5..32 rows: the weight-streaming kernel with Q8_1 activations)
-        want = orc.mul_mat("cpu" if (t == orc.Q4_K and B > 32) else "q8_1", t, Wq, x)
+        want = orc.mul_mat("cpu" if (t in (orc.Q4_K, orc.Q5_K) and B > 32) else "q8_1", t, Wq, x)
         # Q5_K rows are always aligned too: its batches run the per-32-block tile kernel, whose minimum term goes through fp16 operands
         assert orc.nmse(got, want) < (1e-6 if (t == orc.Q5_K and B > 8) else 1e-9)
 
