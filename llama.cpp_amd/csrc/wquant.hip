@@ -1,6 +1,6 @@
 // Weight quantizers on the device: f32 rows -> blocks in the reference's own byte layout, bit for bit what the reference's
 // quantize_row_*_ref functions write (ggml/src/ggml-quants.c: q4_0 :31-66, q8_0 :194-217, q4_K :1208-1278, q5_K :1395-1480,
-// q6_K :1620-1688, with make_qkx2_quants :550-629, make_qx_quants :379-446 and nearest_int :372-377) - the functions llama-quantize
+// q6_K :1620-1688, iq4_nl / iq4_xs :4573-4745, with make_qkx2_quants :550-629, make_qx_quants :379-446 and nearest_int :372-377) - the functions llama-quantize
 // runs without an importance matrix (ggml_quantize_chunk, ggml/src/ggml.c:6410).  Used to build model files and resident models
 // from f32 tensors without a host pass.
 //
@@ -379,6 +379,119 @@ __global__ void __launch_bounds__(256) k_quantize_q4_0_q8_0(const float *__restr
     }
 }
 
+// quantize_iq4_nl / quantize_iq4_xs without importance weights (ggml/src/ggml-quants.c:4684-4745) = quantize_row_iq4_nl_impl
+// (:4573-4682) with ntry = 7: thread = one 32-element block; the eight threads of an IQ4_XS super-block are neighbouring lanes.
+__device__ __forceinline__ int iq4nl_best_index(float x) {   // best_index_int8 (:4562-4571) on kvalues_iq4nl
+    MI355_EXACT
+    constexpr int8_t val[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+    if (x <= (float)val[0]) return 0;
+    if (x >= (float)val[15]) return 15;
+    int ml = 0, mu = 15;
+    while (mu - ml > 1) {
+        const int mav = (ml + mu) / 2;
+        if (x < (float)val[mav]) mu = mav; else ml = mav;
+    }
+    return x - (float)val[mu - 1] < (float)val[mu] - x ? mu - 1 : mu;
+}
+__device__ __forceinline__ float iq4nl_value(int l) {
+    constexpr int8_t val[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+    return (float)val[l];
+}
+template <bool XS>
+__global__ void __launch_bounds__(256) k_quantize_iq4(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n_blk) {
+    MI355_EXACT
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= n_blk) return;   // n_blk is a multiple of 8 for IQ4_XS: the lanes of a super-block leave together
+    float xv[32];
+    const f32x4 *p = (const f32x4 *)(x + b * 32);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const f32x4 v = p[i];
+        xv[4 * i] = v[0]; xv[4 * i + 1] = v[1]; xv[4 * i + 2] = v[2]; xv[4 * i + 3] = v[3];
+    }
+    // the block's scale: first guess max / 127 with the sign that maps max onto -127, then 15 candidates, scored by the least-squares fit
+    float amax = 0.0f, mx = 0.0f;
+    for (int j = 0; j < 32; j++) {
+        const float ax = fabsf(xv[j]);
+        if (ax > amax) { amax = ax; mx = xv[j]; }
+    }
+    float scale = 0.0f;
+    if (!(amax < 1e-15f)) {
+        float d = -mx / -127.0f;
+        float id = 1 / d;
+        float sumqx = 0, sumq2 = 0;
+        for (int j = 0; j < 32; j++) {
+            const float q = iq4nl_value(iq4nl_best_index(id * xv[j]));
+            const float w = xv[j] * xv[j];
+            sumqx += w * q * xv[j];
+            sumq2 += w * q * q;
+        }
+        d = sumqx / sumq2;
+        float best = d * sumqx;
+        for (int itry = -7; itry <= 7; itry++) {
+            id = (float)(itry - 127) / mx;
+            sumqx = sumq2 = 0;
+            for (int j = 0; j < 32; j++) {
+                const float q = iq4nl_value(iq4nl_best_index(id * xv[j]));
+                const float w = xv[j] * xv[j];
+                sumqx += w * q * xv[j];
+                sumq2 += w * q * q;
+            }
+            if (sumq2 > 0 && sumqx * sumqx > best * sumq2) { d = sumqx / sumq2; best = d * sumqx; }
+        }
+        scale = d;
+    }
+    float id_levels;   // what the levels are chosen with
+    u32 *qs;           // the block's 16 bytes of level pairs (4-byte aligned in both layouts... IQ4_NL: 2-byte, written as halves below)
+    if constexpr (XS) {
+        const int lane = threadIdx.x & 63, base = lane & ~7, ib = lane & 7;
+        float max_scale = 0, amax_scale = 0;
+        for (int i = 0; i < 8; i++) {
+            const float si = __shfl(scale, base + i, 64);
+            const float a = fabsf(si);
+            if (a > amax_scale) { amax_scale = a; max_scale = si; }
+        }
+        const float d = -max_scale / 32;
+        const float id = d != 0.0f ? 1 / d : 0.f;
+        int l = clampi(nearest_int(id * scale), -32, 31);
+        const float dl = d * (float)l;
+        id_levels = dl != 0.0f ? 1 / dl : 0.f;
+        l += 32;
+        u32 sl = 0, sh = 0;
+        for (int i = 0; i < 8; i++) {
+            const int li = __shfl(l, base + i, 64);
+            sl |= (u32)(li & 0xF) << (4 * i);
+            sh |= (u32)(li >> 4) << (2 * i);
+        }
+        uint8_t *blk = y + (b >> 3) * IQ4_XS_BYTES;
+        if (ib == 0) {
+            ((u32 *)blk)[0] = (u32)float_to_half_bits(d) | (sh << 16);
+            ((u32 *)blk)[1] = sl;
+        }
+        qs = (u32 *)(blk + 8 + 16 * ib);
+    } else {
+        id_levels = scale != 0.0f ? 1 / scale : 0.f;
+        qs = nullptr;
+    }
+    u32 packed[4] = {0, 0, 0, 0};
+    for (int j = 0; j < 16; j++) {
+        const u32 lo = (u32)iq4nl_best_index(id_levels * xv[j]), hi = (u32)iq4nl_best_index(id_levels * xv[16 + j]);
+        packed[j >> 2] |= (lo | (hi << 4)) << (8 * (j & 3));
+    }
+    if constexpr (XS) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) qs[i] = packed[i];
+    } else {
+        unsigned short *o = (unsigned short *)(y + b * IQ4_NL_BYTES);   // 18-byte blocks: 2-byte aligned
+        o[0] = float_to_half_bits(scale);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            o[1 + 2 * i] = (unsigned short)(packed[i] & 0xFFFFu);
+            o[2 + 2 * i] = (unsigned short)(packed[i] >> 16);
+        }
+    }
+}
+
 }  // namespace
 
 }  // namespace mi355
@@ -388,7 +501,8 @@ using namespace mi355;
 extern "C" {
 
 int mi355_quantize_weights_supported(int type) {
-    return type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K;
+    return type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K || type == MI355_IQ4_NL ||
+           type == MI355_IQ4_XS;
 }
 
 int mi355_quantize_weights(void *stream, int type, const float *x, void *y, int64_t k, int64_t nrows) {
@@ -411,6 +525,8 @@ int mi355_quantize_weights(void *stream, int type, const float *x, void *y, int6
         const int64_t n_blk = n / 32;
         MI355_REQUIRE((n_blk + 255) / 256 < 0x7fffffff, "quantize_weights: tensor too large for one launch");
         if (type == MI355_Q4_0) MI355_LAUNCH(k_quantize_q4_0_q8_0<MI355_Q4_0>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
+        else if (type == MI355_IQ4_NL) MI355_LAUNCH(k_quantize_iq4<false>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
+        else if (type == MI355_IQ4_XS) MI355_LAUNCH(k_quantize_iq4<true>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
         else MI355_LAUNCH(k_quantize_q4_0_q8_0<MI355_Q8_0>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
     }
     return launch_status("k_quantize_weights");
