@@ -45,7 +45,8 @@ int mi355_device_supported(int device);
 
 /* Weight quantizers on the device (what `llama-quantize` runs per tensor without an importance matrix: ggml_quantize_chunk,
  * ggml/src/ggml.c:6410 -> quantize_row_q4_0_ref / q8_0_ref / q4_K_ref / q5_K_ref / q6_K_ref, ggml/src/ggml-quants.c:31-66, 194-217,
- * 1208-1278, 1395-1480, 1620-1688; quantize_iq4_nl / quantize_iq4_xs, :4573-4745).  x: DEVICE f32 [nrows][k], contiguous; y: DEVICE blocks in the REFERENCE byte layout
+ * 1208-1278, 1395-1480, 1620-1688; q4_1 / q5_0 / q5_1 :68-192; quantize_iq4_nl / quantize_iq4_xs, :4573-4745: every weight type
+ * of enum mi355_type).  x: DEVICE f32 [nrows][k], contiguous; y: DEVICE blocks in the REFERENCE byte layout
  * (nrows * k / block elements * block bytes; what a GGUF file holds and mi355_weights_scatter takes).  Bit for bit the reference's
  * bytes.  k a multiple of the type's block size; x 16-byte, y 4-byte aligned. */
 int mi355_quantize_weights_supported(int type);

@@ -1,6 +1,6 @@
 // Weight quantizers on the device: f32 rows -> blocks in the reference's own byte layout, bit for bit what the reference's
 // quantize_row_*_ref functions write (ggml/src/ggml-quants.c: q4_0 :31-66, q8_0 :194-217, q4_K :1208-1278, q5_K :1395-1480,
-// q6_K :1620-1688, iq4_nl / iq4_xs :4573-4745, with make_qkx2_quants :550-629, make_qx_quants :379-446 and nearest_int :372-377) - the functions llama-quantize
+// q6_K :1620-1688, q4_1 / q5_0 / q5_1 :68-192, iq4_nl / iq4_xs :4573-4745, with make_qkx2_quants :550-629, make_qx_quants :379-446 and nearest_int :372-377) - the functions llama-quantize
 // runs without an importance matrix (ggml_quantize_chunk, ggml/src/ggml.c:6410).  Used to build model files and resident models
 // from f32 tensors without a host pass.
 //
@@ -379,6 +379,77 @@ __global__ void __launch_bounds__(256) k_quantize_q4_0_q8_0(const float *__restr
     }
 }
 
+// quantize_row_q4_1_ref / q5_0_ref / q5_1_ref (ggml/src/ggml-quants.c:68-103, 105-147, 149-192): thread = one 32-element block.
+// Blocks are written in 16-bit pieces (Q5_0's 22-byte blocks are only 2-byte aligned).
+template <int TYPE>
+__global__ void __launch_bounds__(256) k_quantize_q4_1_q5(const float *__restrict__ x, uint8_t *__restrict__ y, int64_t n_blk) {
+    MI355_EXACT
+    constexpr bool MIN = TYPE != MI355_Q5_0, FIVE = TYPE != MI355_Q4_1;
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= n_blk) return;
+    float xv[32];
+    const f32x4 *p = (const f32x4 *)(x + b * 32);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const f32x4 v = p[i];
+        xv[4 * i] = v[0]; xv[4 * i + 1] = v[1]; xv[4 * i + 2] = v[2]; xv[4 * i + 3] = v[3];
+    }
+    unsigned short *o = (unsigned short *)(y + b * (TYPE == MI355_Q4_1 ? Q4_1_BYTES : TYPE == MI355_Q5_0 ? Q5_0_BYTES : Q5_1_BYTES));
+    float id, vmin = 0.0f;
+    int at = 1;   // next 16-bit piece of the block
+    if constexpr (MIN) {
+        vmin = 3.402823466e+38f;
+        float vmax = -3.402823466e+38f;
+#pragma unroll
+        for (int j = 0; j < 32; j++) {
+            if (xv[j] < vmin) vmin = xv[j];
+            if (xv[j] > vmax) vmax = xv[j];
+        }
+        const float d = (vmax - vmin) / (FIVE ? 31 : 15);
+        id = d != 0.0f ? 1.0f / d : 0.0f;
+        o[0] = float_to_half_bits(d);
+        o[1] = float_to_half_bits(vmin);
+        at = 2;
+    } else {
+        float amax = 0.0f, mx = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; j++) {
+            if (amax < fabsf(xv[j])) { amax = fabsf(xv[j]); mx = xv[j]; }
+        }
+        // d = max / -16: exact as a sixteenth with the sign flipped in the half's bits (a zero block keeps the reference's -0.0)
+        const float e = mx * 0.0625f;
+        const float d = -e;
+        id = d != 0.0f ? 1.0f / d : 0.0f;
+        o[0] = (unsigned short)(float_to_half_bits(e) ^ 0x8000u);
+    }
+    int lv[32];
+#pragma unroll
+    for (int j = 0; j < 32; j++) {
+        if constexpr (TYPE == MI355_Q4_1) {
+            const int q = (int)(signed char)(int)((xv[j] - vmin) * id + 0.5f);
+            lv[j] = q < 15 ? q : 15;
+        } else if constexpr (TYPE == MI355_Q5_0) {
+            const int q = (int)(signed char)(int)(xv[j] * id + 16.5f);
+            lv[j] = q < 31 ? q : 31;
+        } else {
+            lv[j] = (int)(unsigned char)(int)((xv[j] - vmin) * id + 0.5f);   // no clamp in the reference: bits above the fifth are dropped
+        }
+    }
+    if constexpr (FIVE) {
+        u32 h = 0;
+#pragma unroll
+        for (int j = 0; j < 32; j++) h |= (u32)((lv[j] >> 4) & 1) << j;
+        o[at] = (unsigned short)(h & 0xFFFFu);
+        o[at + 1] = (unsigned short)(h >> 16);
+        at += 2;
+    }
+#pragma unroll
+    for (int j = 0; j < 16; j += 2) {
+        const u32 b0 = (u32)((lv[j] & 0xF) | ((lv[16 + j] & 0xF) << 4)), b1 = (u32)((lv[j + 1] & 0xF) | ((lv[17 + j] & 0xF) << 4));
+        o[at + (j >> 1)] = (unsigned short)(b0 | (b1 << 8));
+    }
+}
+
 // quantize_iq4_nl / quantize_iq4_xs without importance weights (ggml/src/ggml-quants.c:4684-4745) = quantize_row_iq4_nl_impl
 // (:4573-4682) with ntry = 7: thread = one 32-element block; the eight threads of an IQ4_XS super-block are neighbouring lanes.
 __device__ __forceinline__ int iq4nl_best_index(float x) {   // best_index_int8 (:4562-4571) on kvalues_iq4nl
@@ -501,8 +572,7 @@ using namespace mi355;
 extern "C" {
 
 int mi355_quantize_weights_supported(int type) {
-    return type == MI355_Q4_0 || type == MI355_Q8_0 || type == MI355_Q4_K || type == MI355_Q5_K || type == MI355_Q6_K || type == MI355_IQ4_NL ||
-           type == MI355_IQ4_XS;
+    return is_weight_type(type);   // every weight type the kernels read
 }
 
 int mi355_quantize_weights(void *stream, int type, const float *x, void *y, int64_t k, int64_t nrows) {
@@ -525,6 +595,9 @@ int mi355_quantize_weights(void *stream, int type, const float *x, void *y, int6
         const int64_t n_blk = n / 32;
         MI355_REQUIRE((n_blk + 255) / 256 < 0x7fffffff, "quantize_weights: tensor too large for one launch");
         if (type == MI355_Q4_0) MI355_LAUNCH(k_quantize_q4_0_q8_0<MI355_Q4_0>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
+        else if (type == MI355_Q4_1) MI355_LAUNCH(k_quantize_q4_1_q5<MI355_Q4_1>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
+        else if (type == MI355_Q5_0) MI355_LAUNCH(k_quantize_q4_1_q5<MI355_Q5_0>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
+        else if (type == MI355_Q5_1) MI355_LAUNCH(k_quantize_q4_1_q5<MI355_Q5_1>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
         else if (type == MI355_IQ4_NL) MI355_LAUNCH(k_quantize_iq4<false>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
         else if (type == MI355_IQ4_XS) MI355_LAUNCH(k_quantize_iq4<true>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);
         else MI355_LAUNCH(k_quantize_q4_0_q8_0<MI355_Q8_0>, dim3((unsigned)((n_blk + 255) / 256)), dim3(256), 0, s, x, (uint8_t *)y, n_blk);

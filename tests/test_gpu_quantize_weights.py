@@ -1,6 +1,6 @@
 """The weight quantizers on the device (mi355_quantize_weights) against the reference's own quantize_row_*_ref, byte for byte:
 what llama-quantize runs per tensor without an importance matrix (ggml/src/ggml-quants.c:31-66, 194-217, 1208-1278, 1395-1480,
-1620-1688; IQ4_NL / IQ4_XS: quantize_iq4_nl / quantize_iq4_xs, 4573-4745), plus the model-file driver that uses them."""
+1620-1688; Q4_1 / Q5_0 / Q5_1: 68-192; IQ4_NL / IQ4_XS: quantize_iq4_nl / quantize_iq4_xs, 4573-4745), plus the model-file driver that uses them."""
 import os
 import sys
 
@@ -11,8 +11,7 @@ import orc
 
 pytestmark = pytest.mark.gpu
 
-TYPES = [("q4_0", orc.Q4_0), ("q8_0", orc.Q8_0), ("q4_K", orc.Q4_K), ("q5_K", orc.Q5_K), ("q6_K", orc.Q6_K), ("iq4_nl", orc.IQ4_NL),
-         ("iq4_xs", orc.IQ4_XS)]
+TYPES = list(orc.WEIGHT_TYPES.items())   # every weight type has its quantizer on the device
 
 
 def _special_rows(rng, k):
