@@ -329,6 +329,15 @@ int mi355_mul_mat_id_q8k(void *stream, int type, const void *as, const void *act
                          int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws,
                          size_t route_ws_bytes);
 
+/* The same for experts of the per-32-block types (Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q8_0): the routed form of mi355_mul_mat_q's tile
+ * kernel on 128-slot column tiles.  `act` holds the nb1*T rows of b in the mi355_quantize_act (Q8_1) layout; route_ws as above.
+ * K a multiple of 128, expert rows 16-byte aligned, at most 256 experts (mi355_mul_mat_id_q_supported); mi355_mul_mat_id picks
+ * this path from 32 slots on. */
+int mi355_mul_mat_id_q_supported(int type, const void *as, int64_t N, int64_t K, int64_t n_expert);
+int mi355_mul_mat_id_q(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride, float *dst,
+                       int64_t N, int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws,
+                       size_t route_ws_bytes);
+
 /* MUL_MAT_ID with many slots on the wide-tile kernel (ggml_compute_forward_mul_mat_id, ggml-cpu.c:7717-7895; K-quants only).
  * expert_tiles: the experts' tile images (mi355_kq_unpack_tiles of each expert's N x K matrix), expert e at
  * expert_tiles + e * expert_tiles_bytes.  b: the f32 activations [T][nb1][K] (16-byte aligned, rows K apart); they are

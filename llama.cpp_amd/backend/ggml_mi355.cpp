@@ -1984,8 +1984,16 @@ int compute_fused(backend_ctx * ctx, const graph_walk & w, int i) {
                     MI355_K_OK(mi355_quantize_act(s, (const float *) b->data, fresh, K, rows, K));
                     ctx->cache = act_cache{b->data, K, rows, ACT_Q8_1, true, fresh};
                 }
-                MI355_K_OK(mi355_mul_mat_id_vec(s, to_mi355_type(as->type), as->data, ctx->cache.ptr, (const int32_t *) ids->data, ids_stride,
-                                                (float *) node->data, N, K, n_expert, n_used, nb1, T));
+                // many slots on experts of a per-32-block type: sorted by expert onto the routed form of their tile kernel
+                if (n_used * T >= 32 && mi355_mul_mat_id_q_supported(to_mi355_type(as->type), as->data, N, K, n_expert)) {
+                    const size_t route_bytes = mi355_mul_mat_id_q8k_route_bytes(n_expert, n_used, T);
+                    void * route = ctx->workspace(route_bytes);
+                    MI355_K_OK(mi355_mul_mat_id_q(s, to_mi355_type(as->type), as->data, ctx->cache.ptr, (const int32_t *) ids->data, ids_stride,
+                                                  (float *) node->data, N, K, n_expert, n_used, nb1, T, route, route_bytes));
+                } else {
+                    MI355_K_OK(mi355_mul_mat_id_vec(s, to_mi355_type(as->type), as->data, ctx->cache.ptr, (const int32_t *) ids->data, ids_stride,
+                                                    (float *) node->data, N, K, n_expert, n_used, nb1, T));
+                }
             }
             ctx->note_write(node->data, ggml_nbytes(node));
             return i;

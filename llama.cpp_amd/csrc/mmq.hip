@@ -31,6 +31,7 @@
 // (ids are dealt round-robin over the 8 XCDs) and hit its L2 instead of HBM.
 #include "common.hpp"
 #include "qdot.hpp"
+#include "tiles.hpp"
 
 namespace mi355 {
 
@@ -291,21 +292,24 @@ template <int BN, bool WITH_SUM> struct mmq_aregs {
     u32x4 q[NQ];
     float d[NS];
     int sum[NS];
+    // row_of: null, or the activation row of every column (the routed form: columns are (token, expert slot) pairs sorted by expert)
     __device__ __forceinline__ void fetch(const int8_t *__restrict__ aq, const act_ds *__restrict__ ads, int64_t col0, int64_t B, int64_t K, int64_t k0,
-                                          int tid) {
+                                          int tid, const int32_t *__restrict__ row_of = nullptr) {
         const int64_t nblk = K >> 5;
 #pragma unroll
         for (int it = 0; it < NQ; it++) {
             const int idx = tid + it * 256;
             const int r = idx >> 3, c = idx & 7;
-            const int64_t col = col0 + r < B ? col0 + r : B - 1;
+            int64_t col = col0 + r < B ? col0 + r : B - 1;
+            if (row_of) col = row_of[col];
             q[it] = load16(aq + col * K + k0 + c * 16);
         }
 #pragma unroll
         for (int it = 0; it < NS; it++) {
             const int idx = tid + it * 256;
             const int r = (idx >> 2) < BN ? (idx >> 2) : BN - 1, b = idx & 3;
-            const int64_t col = col0 + r < B ? col0 + r : B - 1;
+            int64_t col = col0 + r < B ? col0 + r : B - 1;
+            if (row_of) col = row_of[col];
             const act_ds e = ads[col * nblk + (k0 >> 5) + b];
             d[it] = e.d;
             if constexpr (WITH_SUM) sum[it] = e.sum;
@@ -329,12 +333,23 @@ template <int BN, bool WITH_SUM> struct mmq_aregs {
     }
 };
 
-template <int TYPE, int TN>
+// MUL_MAT_ID with many slots (ID): column tile ct of the slot list sorted by expert (k_route_slots) holds slots [first, end) of one
+// expert; their activation rows are gathered through act_row and their results go to the dst rows of dst_row.
+struct mmq32_route {
+    const int32_t *act_row;
+    const int32_t *dst_row;
+    const int32_t *tiles;      // per column tile: expert, first slot, end slot, -
+    const int32_t *n_tiles;    // column tiles in use (device value)
+    int64_t expert_bytes;      // from one expert's matrix to the next
+};
+
+template <int TYPE, int TN, bool ID = false>
 __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, const int8_t *__restrict__ aq,
                                              const act_ds *__restrict__ ads, float *__restrict__ dst, int64_t N,
                                              int64_t K, int64_t B, int64_t dst_stride, row_layout L, int n_col_tiles,
-                                             int n_groups, int n_groups_padded) {
+                                             int n_groups, int n_groups_padded, mmq32_route route) {
     typedef mmq_cfg<TYPE> C;
+    static_assert(!ID || C::PREFETCH, "the routed form exists for the per-32-block types");
     constexpr int BN = 64 * TN;
     __shared__ __attribute__((aligned(16))) int8_t sW[MMQ_BM * MMQ_LDK];
     __shared__ __attribute__((aligned(16))) int8_t sA[BN * MMQ_LDK];
@@ -348,7 +363,16 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
     const int lid = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
     if (lid >= n_groups) return;   // uniform for the whole group
     const int64_t row0 = (int64_t)(lid / n_col_tiles) * MMQ_BM;
-    const int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+    int64_t col0 = (int64_t)(lid % n_col_tiles) * BN;
+    const int32_t *row_of = nullptr;
+    if constexpr (ID) {
+        const int ct = lid % n_col_tiles;
+        if (ct >= *route.n_tiles) return;   // uniform for the whole group
+        W += (int64_t)route.tiles[4 * ct] * route.expert_bytes;
+        col0 = route.tiles[4 * ct + 1];
+        B = route.tiles[4 * ct + 2];
+        row_of = route.act_row;
+    }
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
@@ -374,7 +398,7 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
     mmq_aregs<BN, C::MIN> aregs;
     if constexpr (PREFETCH) {
         wregs.fetch(W, L, row0, N, k_lo, threadIdx.x);
-        aregs.fetch(aq, ads, col0, B, K, k_lo, threadIdx.x);
+        aregs.fetch(aq, ads, col0, B, K, k_lo, threadIdx.x, row_of);
     }
     for (int64_t k0 = k_lo; k0 < k_hi; k0 += MMQ_BK) {
         __syncthreads();
@@ -390,7 +414,7 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
             // past the end the last stage is requested again and never committed: no branch, the loads stay here
             const int64_t k1 = k0 + MMQ_BK < k_hi ? k0 + MMQ_BK : k0;
             wregs.fetch(W, L, row0, N, k1, threadIdx.x);
-            aregs.fetch(aq, ads, col0, B, K, k1, threadIdx.x);
+            aregs.fetch(aq, ads, col0, B, K, k1, threadIdx.x, row_of);
             __builtin_amdgcn_sched_barrier(0);   // requested now, a whole stage ahead of their commit
         }
 
@@ -479,7 +503,7 @@ __global__ void __launch_bounds__(256) k_mmq(const uint8_t *__restrict__ W, cons
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t b = col0 + wcol0 + tb * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-                if (n < N && b < B) dst[b * dst_stride + n] = acc[tb][tw][r];
+                if (n < N && b < B) dst[(ID ? (int64_t)route.dst_row[b] : b) * dst_stride + n] = acc[tb][tw][r];
             }
         }
 }
@@ -522,12 +546,12 @@ static void launch_mmq(hipStream_t s, const void *W, const void *act, float *dst
     if (n_slices > 1 && (ws == nullptr || ((uintptr_t)ws & 15) != 0 || ws_bytes < (size_t)n_slices * (size_t)N * (size_t)B * sizeof(float))) n_slices = 1;
     if (n_slices > 1) {
         MI355_LAUNCH((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded, (unsigned)n_slices), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
-                           (float *)ws, N, K, B, N, L, n_col_tiles, n_groups, n_groups_padded);
+                           (float *)ws, N, K, B, N, L, n_col_tiles, n_groups, n_groups_padded, mmq32_route{});
         MI355_LAUNCH(k_mmq_split_sum, dim3((unsigned)((N * B + 255) / 256)), dim3(256), 0, s, (const float *)ws, dst, N, B, dst_stride, n_slices);
         return;
     }
     MI355_LAUNCH((k_mmq<TYPE, TN>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)W, aq, ads,
-                       dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded);
+                       dst, N, K, B, dst_stride, L, n_col_tiles, n_groups, n_groups_padded, mmq32_route{});
 }
 
 template <int TYPE>
@@ -537,9 +561,62 @@ static void launch_mmq_tn(hipStream_t s, const void *W, const void *act, float *
     else launch_mmq<TYPE, 2>(s, W, act, dst, N, K, B, dst_stride, ws, ws_bytes);
 }
 
+// the routed launch: 128-column tiles over the slot list sorted by expert; the routing workspace is laid out as for the
+// super-block kernel's routed form (act_row[S], dst_row[S], tiles[4 x ((S + 63) / 64 + n_expert)], n_tiles)
+template <int TYPE>
+static void launch_mmq_id(hipStream_t s, const void *as, const void *act, int64_t act_rows, const int32_t *ids, int64_t ids_stride, float *dst, int64_t N,
+                          int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws) {
+    constexpr int BN = 128;
+    const int64_t S = T * n_used;
+    const int max_tiles = (int)((S + BN - 1) / BN + n_expert);
+    int32_t *act_row = (int32_t *)route_ws, *dst_row = act_row + S, *tiles = dst_row + S, *n_tiles = tiles + 4 * ((S + 63) / 64 + n_expert);
+    launch_route_slots(s, ids, ids_stride, n_expert, n_used, nb1, T, BN, act_row, dst_row, tiles, n_tiles);
+    const row_layout L = make_row_layout(TYPE, K);
+    const int8_t *aq = (const int8_t *)act;
+    const act_ds *ads = (const act_ds *)(aq + act_rows * K);
+    const int n_row_tiles = (int)((N + MMQ_BM - 1) / MMQ_BM);
+    const int n_groups = n_row_tiles * max_tiles;
+    const int n_groups_padded = (n_groups + 7) & ~7;
+    const mmq32_route route = {act_row, dst_row, tiles, n_tiles, N * L.row_bytes};
+    MI355_LAUNCH((k_mmq<TYPE, 2, true>), dim3((unsigned)n_groups_padded), dim3(256), 0, s, (const uint8_t *)as, aq, ads, dst, N, K, S, N, L, max_tiles,
+                 n_groups, n_groups_padded, route);
+}
+
 }  // namespace mi355
 
 using namespace mi355;
+
+extern "C" int mi355_mul_mat_id_q_supported(int type, const void *as, int64_t N, int64_t K, int64_t n_expert) {
+    const bool typed = type == MI355_Q4_0 || type == MI355_Q4_1 || type == MI355_Q5_0 || type == MI355_Q5_1 || type == MI355_IQ4_NL || type == MI355_Q8_0;
+    if (!typed || N <= 0 || K <= 0 || K % MMQ_BK != 0 || n_expert <= 0 || n_expert > 256) return 0;
+    const row_layout L = make_row_layout(type, K);
+    return layout_aligned(as, L) && (N * L.row_bytes) % 16 == 0 ? 1 : 0;
+}
+
+extern "C" int mi355_mul_mat_id_q(void *stream, int type, const void *as, const void *act, const int32_t *ids, int64_t ids_stride, float *dst, int64_t N,
+                                  int64_t K, int64_t n_expert, int64_t n_used, int64_t nb1, int64_t T, void *route_ws, size_t route_ws_bytes) {
+    MI355_REQUIRE(mi355_mul_mat_id_q_supported(type, as, N, K, n_expert), "mul_mat_id_q: type %d, K=%lld, %lld experts or the weight alignment is not supported",
+                  type, (long long)K, (long long)n_expert);
+    MI355_REQUIRE(n_used > 0 && nb1 > 0 && T > 0 && ids_stride >= n_used, "mul_mat_id_q: bad shape");
+    MI355_REQUIRE(T * n_used < (1 << 24) && nb1 * T < (1 << 24), "mul_mat_id_q: too many slots");
+    MI355_REQUIRE(((uintptr_t)act & 15) == 0, "mul_mat_id_q: activation workspace is not 16-byte aligned");
+    const size_t need = mi355_mul_mat_id_q8k_route_bytes(n_expert, n_used, T);
+    if (route_ws == nullptr || route_ws_bytes < need || ((uintptr_t)route_ws & 15) != 0) {
+        set_error("mul_mat_id_q: routing workspace of %zu bytes, need %zu (16-byte aligned)", route_ws_bytes, need);
+        return MI355_ERR_WORKSPACE;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t rows = nb1 * T;
+    switch (type) {
+        case MI355_Q4_0: launch_mmq_id<MI355_Q4_0>(s, as, act, rows, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws); break;
+        case MI355_Q4_1: launch_mmq_id<MI355_Q4_1>(s, as, act, rows, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws); break;
+        case MI355_Q5_0: launch_mmq_id<MI355_Q5_0>(s, as, act, rows, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws); break;
+        case MI355_Q5_1: launch_mmq_id<MI355_Q5_1>(s, as, act, rows, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws); break;
+        case MI355_IQ4_NL: launch_mmq_id<MI355_IQ4_NL>(s, as, act, rows, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws); break;
+        default: launch_mmq_id<MI355_Q8_0>(s, as, act, rows, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, route_ws); break;
+    }
+    return launch_status("k_mmq (routed)");
+}
 
 extern "C" size_t mi355_mul_mat_q_ws_bytes(int64_t N, int64_t K, int64_t B) {
     if (N <= 0 || K <= 0 || B <= 0 || K % MMQ_BK != 0) return 0;

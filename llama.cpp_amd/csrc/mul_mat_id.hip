@@ -45,6 +45,10 @@ int mi355_mul_mat_id(void *stream, int type, const void *as, const float *b, con
     }
     int rc = mi355_quantize_act(stream, b, ws, K, nb1 * T, K);
     if (rc != MI355_OK) return rc;
+    if (T * n_used >= ROUTED_MIN_SLOTS && mi355_mul_mat_id_q_supported(type, as, N, K, n_expert)) {   // per-32-block types: the routed form of their tile kernel
+        const size_t act = (mi355_act_bytes(K, nb1 * T) + 255) & ~(size_t)255;
+        return mi355_mul_mat_id_q(stream, type, as, ws, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T, (uint8_t *)ws + act, ws_bytes - act);
+    }
     return mi355_mul_mat_id_vec(stream, type, as, ws, ids, ids_stride, dst, N, K, n_expert, n_used, nb1, T);
 }
 

@@ -132,6 +132,8 @@ _SIGNATURES = {
     "mi355_moe_weights": (_int, [_p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64]),
     "mi355_moe_weights_combine": (_int, [_p, _p, _p, _i64, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64]),
     "mi355_moe_combine": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64]),
+    "mi355_mul_mat_id_q_supported": (_int, [_int, _p, _i64, _i64, _i64]),
+    "mi355_mul_mat_id_q": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _sz]),
     "mi355_mul_mat_id_vec": (_int, [_p, _int, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64, _i64, _i64]),
     "mi355_flash_attn_ws_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "mi355_flash_attn_ext": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _sz, _sz, _sz, _sz, _sz, _sz,

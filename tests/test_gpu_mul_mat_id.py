@@ -49,7 +49,9 @@ def test_mul_mat_id(dev, name, t, n_expert, n_used, nb1_bcast, T, N, K):
         want = np.zeros((T, n_used, N), dtype=np.float32)
         assert orc.oracle.orc_mul_mat_id_q8_1(t, orc._ptr(Wq), orc._ptr(b), orc._ptr(ids_full), n_expert, orc._ptr(want), N, K,
                                               n_expert, n_used, nb1, T) == 0
-    assert orc.nmse(got, want) < 1e-9
+    # per-32-block experts with 32+ slots run the routed form of their tile kernel, where the block minimum of Q4_1 / Q5_1 meets
+    # fp16(d_x * sum(q)), the `s` field the reference's own dot uses
+    assert orc.nmse(got, want) < (1e-6 if (t in (orc.Q4_1, orc.Q5_1) and T * n_used >= 32) else 1e-9)
     if orc.ref is not None:
         cpu = np.zeros_like(want)
         assert orc.ref.ref_mul_mat_id(t, orc._ptr(Wq), orc._ptr(b), orc._ptr(ids_full), orc._ptr(cpu), N, K, n_expert, n_used,
@@ -57,7 +59,8 @@ def test_mul_mat_id(dev, name, t, n_expert, n_used, nb1_bcast, T, N, K):
         assert orc.nmse(got, cpu) <= 5e-4      # tests/test-backend-ops.cpp:2001
 
 
-@pytest.mark.parametrize("name,t", [("q4_k", orc.Q4_K), ("q6_k", orc.Q6_K), ("q5_k", orc.Q5_K), ("iq4_xs", orc.IQ4_XS)])
+@pytest.mark.parametrize("name,t", [("q4_k", orc.Q4_K), ("q6_k", orc.Q6_K), ("q5_k", orc.Q5_K), ("iq4_xs", orc.IQ4_XS), ("q4_0", orc.Q4_0), ("q8_0", orc.Q8_0),
+                                    ("q5_1", orc.Q5_1)])
 @pytest.mark.parametrize("pattern", ["one_expert", "two_of_eight", "out_of_range"])
 def test_mul_mat_id_skewed_routing(dev, name, t, pattern):
     """experts with no slots, one expert with more slots than a column tile, ids outside [0, n_expert) clamped like the GEMV path"""
@@ -77,8 +80,9 @@ def test_mul_mat_id_skewed_routing(dev, name, t, pattern):
     Wd = mi355.upload_weights(t, torch.from_numpy(Wq).to(dev)).reshape(n_expert, N, -1)
     idd = torch.from_numpy(ids).to(dev)[:, :n_used]
     got = mi355.mul_mat_id(t, Wd, torch.from_numpy(b).to(dev), idd, n_used).cpu().numpy()
-    want = expected_per_expert("cpu", t, Wq, b, np.clip(ids, 0, n_expert - 1), n_expert, n_used, 1, N)
-    assert orc.nmse(got, want) < 1e-9
+    kind = "cpu" if t in (orc.Q4_K, orc.Q6_K, orc.Q5_K, orc.IQ4_XS) else "q8_1"   # the activation format of the type's routed tile kernel
+    want = expected_per_expert(kind, t, Wq, b, np.clip(ids, 0, n_expert - 1), n_expert, n_used, 1, N)
+    assert orc.nmse(got, want) < (1e-6 if t in (orc.Q4_1, orc.Q5_1) else 1e-9)   # the block minimum meets fp16(d_x * sum(q)) in the tile kernel
 
 
 @pytest.mark.parametrize("name,t", [("q4_k", orc.Q4_K), ("q5_k", orc.Q5_K), ("q6_k", orc.Q6_K)])
